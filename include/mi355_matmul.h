@@ -1,0 +1,250 @@
+/*
+ * mi355_matmul.h -- thin C ABI between the host-side oneDNN-compatible matmul
+ * primitive and the hand-written gfx950 (MI355X / CDNA4) HIP kernels.
+ *
+ * Everything that crosses this boundary is plain C: PODs, raw device pointers,
+ * sizes and an opaque stream handle.  No C++ or HIP types appear in the
+ * signatures, so the host library (plain g++), a cgo/ctypes caller or a test
+ * can bind it without HIP headers.
+ *
+ * What each piece replaces in the reference (uxlfoundation/oneDNN v3.14):
+ *   - mi355_matmul_desc_t   : the information a matmul pd_t holds after
+ *                             init(): src/common/matmul_pd.hpp:63-440 (M/N/K,
+ *                             data types, strides, qmasks, groups, post-ops).
+ *   - mi355_matmul_args_t   : the exec_ctx_t argument map of
+ *                             primitive_t::execute, src/common/primitive_exec_types.hpp:112-186
+ *                             and the brgemm_post_ops_data_t bundle of
+ *                             src/cpu/x64/matmul/brgemm_matmul.cpp:966-981.
+ *   - mi355_matmul_launch   : primitive_t::execute(const exec_ctx_t&)
+ *                             (src/common/primitive.hpp:54) of the matmul
+ *                             implementations ref_matmul_t / ref_matmul_int8_t /
+ *                             brgemm_matmul_t.
+ *   - mi355_matmul_query    : pd_t::init() dispatch predicate + name()
+ *                             (DECLARE_COMMON_PD_T, src/common/primitive_desc.hpp).
+ *   - mi355_mem_* / stream  : memory_storage_t / stream_t of an engine
+ *                             (src/common/memory_storage.hpp, src/common/stream.hpp).
+ */
+#ifndef MI355_MATMUL_H
+#define MI355_MATMUL_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* Data types: numeric values equal dnnl_data_type_t
+ * (include/oneapi/dnnl/dnnl_common_types.h:80-114). */
+enum {
+    MI355_DT_UNDEF = 0,
+    MI355_DT_F16 = 1,
+    MI355_DT_BF16 = 2,
+    MI355_DT_F32 = 3,
+    MI355_DT_S32 = 4,
+    MI355_DT_S8 = 5,
+    MI355_DT_U8 = 6,
+    MI355_DT_F64 = 7,
+    MI355_DT_BOOLEAN = 8,
+    MI355_DT_F8_E5M2 = 9,
+    MI355_DT_F8_E4M3 = 10,
+    MI355_DT_S4 = 11,
+    MI355_DT_U4 = 12,
+    MI355_DT_E8M0 = 13,
+    MI355_DT_F4_E2M1 = 14
+};
+
+/* Status codes: numeric values equal dnnl_status_t
+ * (include/oneapi/dnnl/dnnl_common_types.h:44-66). */
+enum {
+    MI355_SUCCESS = 0,
+    MI355_OUT_OF_MEMORY = 1,
+    MI355_INVALID_ARGUMENTS = 2,
+    MI355_UNIMPLEMENTED = 3,
+    MI355_LAST_IMPL_REACHED = 4,
+    MI355_RUNTIME_ERROR = 5,
+    MI355_NOT_REQUIRED = 6
+};
+
+/* Post-op kinds (the four matmul admits, src/common/matmul.cpp:610-612). */
+enum {
+    MI355_PO_SUM = 1,
+    MI355_PO_ELTWISE = 2,
+    MI355_PO_BINARY = 3,
+    MI355_PO_PRELU = 4
+};
+
+/* Algorithm kinds: numeric values equal dnnl_alg_kind_t
+ * (include/oneapi/dnnl/dnnl_types.h, eltwise 0x20.., binary 0x1fff0..). */
+enum {
+    MI355_ELTWISE_RELU = 0x20,
+    MI355_ELTWISE_TANH = 0x21,
+    MI355_ELTWISE_ELU = 0x22,
+    MI355_ELTWISE_SQUARE = 0x23,
+    MI355_ELTWISE_ABS = 0x24,
+    MI355_ELTWISE_SQRT = 0x25,
+    MI355_ELTWISE_LINEAR = 0x26,
+    MI355_ELTWISE_SOFT_RELU = 0x27,
+    MI355_ELTWISE_HARDSIGMOID = 0x28,
+    MI355_ELTWISE_LOGISTIC = 0x29,
+    MI355_ELTWISE_EXP = 0x2a,
+    MI355_ELTWISE_GELU_TANH = 0x2b,
+    MI355_ELTWISE_SWISH = 0x2c,
+    MI355_ELTWISE_LOG = 0x2d,
+    MI355_ELTWISE_CLIP = 0x2e,
+    MI355_ELTWISE_CLIP_V2 = 0x2f,
+    MI355_ELTWISE_POW = 0x30,
+    MI355_ELTWISE_GELU_ERF = 0x31,
+    MI355_ELTWISE_ROUND = 0x32,
+    MI355_ELTWISE_MISH = 0x33,
+    MI355_ELTWISE_HARDSWISH = 0x34,
+    MI355_BINARY_ADD = 0x1fff0,
+    MI355_BINARY_MUL = 0x1fff1,
+    MI355_BINARY_MAX = 0x1fff2,
+    MI355_BINARY_MIN = 0x1fff3,
+    MI355_BINARY_DIV = 0x1fff4,
+    MI355_BINARY_SUB = 0x1fff5,
+    MI355_BINARY_GE = 0x1fff6,
+    MI355_BINARY_GT = 0x1fff7,
+    MI355_BINARY_LE = 0x1fff8,
+    MI355_BINARY_LT = 0x1fff9,
+    MI355_BINARY_EQ = 0x1fffa,
+    MI355_BINARY_NE = 0x1fffb
+};
+
+/* Which arithmetic flavour of "the reference's own matmul" to reproduce where
+ * the reference's two CPU implementations differ bit-wise. */
+enum {
+    /* ref_matmul_int8_t / ref_matmul_t: d /= dst_scale
+     * (src/cpu/matmul/ref_matmul_int8.cpp:293-297). */
+    MI355_DST_SCALE_DIVIDE = 0,
+    /* brgemm_matmul_t: d *= (1.f / dst_scale)
+     * (src/cpu/x64/matmul/brgemm_matmul.cpp:703-709). */
+    MI355_DST_SCALE_RECIPROCAL = 1
+};
+
+/* Kernel families (implementation ids). 0 lets the library choose. */
+enum {
+    MI355_IMPL_AUTO = 0,
+    MI355_IMPL_REF = 1,      /* "hip:ref:any": one thread per dst element */
+    MI355_IMPL_I8_MFMA = 2,  /* "hip:mfma_i8": LDS-tiled i8 MFMA GEMM */
+    MI355_IMPL_F8_MFMA = 3,  /* "hip:mfma_f8": e4m3/e5m2 MFMA GEMM */
+    MI355_IMPL_MXF4_MFMA = 4,/* "hip:mfma_mxf4": block-scaled e2m1 MFMA GEMM */
+    MI355_IMPL_WOQ_GEMV = 5, /* "hip:woq_gemv": int4/int8 weight-only decode */
+    MI355_IMPL_COUNT = 6
+};
+
+#define MI355_MAX_POST_OPS 32 /* post_ops_t::post_ops_limit in the reference */
+
+/* A quantization parameter tensor (scales, zero points or precomputed
+ * reductions) attached to one matmul argument.  Mirrors quant_entry_t
+ * (src/common/primitive_attr_quant.hpp:40-140): a mask over the argument's
+ * dimensions, optional groups over the last two dimensions and a data type.
+ * The parameter tensor is dense row-major with dims
+ *   [ mask&1 ? batch : 1, mask&2 ? D0/group[0] : 1, mask&4 ? D1/group[1] : 1 ]
+ * where (D0, D1) are the last two dims of the argument (src: M,K; weights:
+ * K,N; dst: M,N) -- quant_entry_t::get_md + matmul_helper_t::get_quant_off
+ * (src/cpu/matmul/matmul_utils.hpp:154-173). */
+typedef struct mi355_quant {
+    int32_t dt;       /* MI355_DT_UNDEF = parameter absent */
+    int32_t mask;     /* bit0 batch, bit1 second-to-last dim, bit2 last dim */
+    int64_t group[2]; /* >= 1 */
+} mi355_quant_t;
+
+typedef struct mi355_post_op {
+    int32_t kind; /* MI355_PO_* */
+    int32_t alg;  /* eltwise / binary algorithm */
+    float alpha, beta;
+    float scale;          /* sum scale (eltwise scale is always 1 via the API) */
+    int32_t zero_point;   /* sum zero point */
+    int32_t dt;           /* binary: src1 dt; sum: dt dst is read as (0 = dst dt) */
+    int64_t stride[3];    /* binary src1 / prelu weights element strides over
+                             (batch, M, N); 0 on broadcast dims */
+} mi355_post_op_t;
+
+typedef struct mi355_matmul_desc {
+    int64_t batch, M, N, K;
+    int32_t src_dt, wei_dt, dst_dt, bias_dt; /* bias_dt UNDEF = no bias */
+    /* element strides over (batch, row, col); 4-bit types count nibbles.
+     * A batch stride of 0 broadcasts the operand. */
+    int64_t src_stride[3];  /* (b, m, k) */
+    int64_t wei_stride[3];  /* (b, k, n) */
+    int64_t dst_stride[3];  /* (b, m, n) */
+    int64_t bias_stride[3]; /* (b, m, n); 0 on broadcast dims */
+    mi355_quant_t src_scale, wei_scale, dst_scale;
+    mi355_quant_t src_zp, wei_zp, dst_zp;
+    mi355_quant_t src_pr; /* precomputed reductions over K of src */
+    int32_t fpmath_apply_to_int; /* weight decompression switch */
+    int32_t fpmath_mode;         /* dnnl_fpmath_mode_t value, informational */
+    int32_t dst_scale_mode;      /* MI355_DST_SCALE_* */
+    int32_t n_post_ops;
+    mi355_post_op_t post_ops[MI355_MAX_POST_OPS];
+    int32_t impl; /* MI355_IMPL_*; AUTO picks the fastest applicable */
+    int32_t reserved;
+} mi355_matmul_desc_t;
+
+typedef struct mi355_matmul_args {
+    const void *src, *wei, *bias;
+    void *dst;
+    const void *src_scale, *wei_scale, *dst_scale;
+    const void *src_zp, *wei_zp, *dst_zp;
+    const void *src_pr;
+    const void *po_arg[MI355_MAX_POST_OPS]; /* binary src1 / prelu weights */
+} mi355_matmul_args_t;
+
+/* ---- device, memory, stream, events (engine / stream / memory_storage) --- */
+int mi355_device_count(int *count);
+int mi355_device_set(int device);
+/* name: gcnArchName; cus: multiProcessorCount; clock_khz; hbm_bytes */
+int mi355_device_info(int device, char *name, size_t name_len, int *cus,
+        int *clock_khz, int64_t *hbm_bytes, int64_t *l2_bytes);
+int mi355_mem_alloc(void **dptr, size_t bytes);
+int mi355_mem_free(void *dptr);
+int mi355_mem_set(void *dptr, int byte, size_t bytes, void *stream);
+int mi355_mem_h2d(void *dptr, const void *hptr, size_t bytes, void *stream);
+int mi355_mem_d2h(void *hptr, const void *dptr, size_t bytes, void *stream);
+int mi355_mem_d2d(void *dst, const void *src, size_t bytes, void *stream);
+int mi355_stream_create(void **stream);
+int mi355_stream_destroy(void *stream);
+int mi355_stream_sync(void *stream); /* NULL = default stream */
+int mi355_event_create(void **event);
+int mi355_event_destroy(void *event);
+int mi355_event_record(void *event, void *stream);
+int mi355_event_sync(void *event);
+int mi355_event_elapsed_ms(float *ms, void *start, void *stop);
+const char *mi355_last_error(void); /* thread-local text of the last failure */
+
+/* ---- the matmul path ---------------------------------------------------- */
+
+/* Dispatch predicate: MI355_SUCCESS if kernel family `impl` can run `desc`
+ * exactly, MI355_UNIMPLEMENTED if not, MI355_INVALID_ARGUMENTS on nonsense.
+ * With impl == AUTO reports the family the launcher would choose in
+ * *chosen_impl (may be NULL). */
+int mi355_matmul_query(const mi355_matmul_desc_t *desc, int impl,
+        int *chosen_impl);
+
+/* Implementation name in oneDNN's "impl_info_str" style, e.g. "hip:mfma_i8". */
+const char *mi355_matmul_impl_name(int impl);
+
+/* Bytes of device scratch `mi355_matmul_launch` needs for this problem
+ * (0 for most kernels). */
+int mi355_matmul_scratch_bytes(const mi355_matmul_desc_t *desc, size_t *bytes);
+
+/* Enqueue the matmul on `stream` (a hipStream_t passed as void*, NULL =
+ * default stream).  Asynchronous.  `scratch` may be NULL when
+ * mi355_matmul_scratch_bytes reports 0. */
+int mi355_matmul_launch(const mi355_matmul_desc_t *desc,
+        const mi355_matmul_args_t *args, void *scratch, void *stream);
+
+/* Plain device-to-device copy kernel (one 16-byte load + store per lane), used
+ * to calibrate the FETCH_SIZE / WRITE_SIZE counters against a known size. */
+int mi355_copy_kernel(void *dst, const void *src, size_t bytes, void *stream);
+
+/* Evict caches between timed launches: streams `bytes` of `buf` through a
+ * read-modify-write kernel so a following launch sees cold L2/MALL. */
+int mi355_flush_kernel(void *buf, size_t bytes, void *stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* MI355_MATMUL_H */

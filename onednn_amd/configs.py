@@ -1,0 +1,169 @@
+"""Synthetic, seeded inputs for the five benchmark configurations.
+
+Each builder returns a MatmulProblem with the data types, layouts, attributes
+and value distributions the benchmark definition states; `M/N/K` can be
+overridden to get the same problem class at a test-sized shape.  Quantization
+parameter layouts follow quant_entry_t::get_md
+(src/common/primitive_attr_quant.hpp:116-140): dense row-major over the masked
+dims with the last two divided by the group sizes.
+"""
+import numpy as np
+
+from . import cabi
+from . import dtypes as dtp
+from .problem import MatmulProblem, PostOp, QuantParam, strides_for
+
+MASK_COMMON = 0
+MASK_ROW = 2   # second-to-last dim of the argument
+MASK_COL = 4   # last dim of the argument
+
+
+def _rng(seed, tensor_id):
+    return np.random.Generator(np.random.PCG64([seed, tensor_id]))
+
+
+def config1(M=256, N=1024, K=1024, dst="f32", seed=1, impl=cabi.IMPL_AUTO):
+    """u8 x s8 -> f32 (or s32): src zero point 128, src scale 0.02, per-N
+    weights scales, f32 bias.  dst='s32' drops scales and bias (accumulator
+    check)."""
+    src = _rng(seed, 1).integers(0, 256, size=(M, K), dtype=np.uint8)
+    wei = _rng(seed, 2).integers(-127, 128, size=(K, N), dtype=np.int8)
+    quant = {"src_zp": QuantParam(cabi.DT_S32, MASK_COMMON, np.array([128], np.int32))}
+    bias = None
+    bias_dt = cabi.DT_UNDEF
+    if dst == "f32":
+        quant["src_scale"] = QuantParam(cabi.DT_F32, MASK_COMMON, np.array([0.02], np.float32))
+        quant["wei_scale"] = QuantParam(
+            cabi.DT_F32, MASK_COL, _rng(seed, 3).uniform(1e-3, 1e-2, size=N).astype(np.float32))
+        bias = _rng(seed, 4).uniform(-1, 1, size=N).astype(np.float32)
+        bias_dt = cabi.DT_F32
+    return MatmulProblem(M=M, N=N, K=K, src_dt=cabi.DT_U8, wei_dt=cabi.DT_S8,
+                         dst_dt=cabi.DT_NAMES[dst], src=src, wei=wei, bias_dt=bias_dt, bias=bias,
+                         quant=quant, impl=impl, name=f"C1-{dst}")
+
+
+def config2(M=1, N=14336, K=4096, group=128, seed=2, impl=cabi.IMPL_AUTO, wtag="ab"):
+    """bf16 x u4 -> bf16 weight-only decode: per-group bf16 scales and u4 zero
+    points along K, fpmath bf16 with apply_to_int."""
+    src = dtp.f32_to_bf16(_rng(seed, 1).standard_normal((M, K)).astype(np.float32))
+    codes = _rng(seed, 2).integers(0, 16, size=(K, N), dtype=np.uint8)
+    if wtag == "ab":
+        wei = dtp.pack_nibbles(codes)            # two n per byte
+    else:
+        wei = dtp.pack_nibbles(codes.T.copy())   # two k per byte
+    G = K // group
+    scales = dtp.f32_to_bf16(_rng(seed, 3).uniform(0.005, 0.02, size=(G, N)).astype(np.float32))
+    zps = dtp.pack_nibbles(_rng(seed, 4).integers(0, 16, size=(G, N), dtype=np.uint8))
+    quant = {
+        "wei_scale": QuantParam(cabi.DT_BF16, MASK_ROW | MASK_COL, scales, (group, 1)),
+        "wei_zp": QuantParam(cabi.DT_U4, MASK_ROW | MASK_COL, zps, (group, 1)),
+    }
+    return MatmulProblem(M=M, N=N, K=K, src_dt=cabi.DT_BF16, wei_dt=cabi.DT_U4,
+                         dst_dt=cabi.DT_BF16, src=src, wei=wei,
+                         wei_stride=strides_for(wtag, 1, K, N), quant=quant, apply_to_int=True,
+                         fpmath_mode=1, impl=impl, name=f"C2-M{M}")
+
+
+def config3(M=8192, N=8192, K=8192, seed=3, impl=cabi.IMPL_AUTO, wtag="ab",
+            dst_scale_mode=cabi.DST_SCALE_DIVIDE):
+    """s8 x s8 -> s8: src scale 0.01, per-N weights scales, dst scale 0.05,
+    ReLU, round-to-nearest-even with saturation."""
+    src = _rng(seed, 1).integers(-127, 128, size=(M, K), dtype=np.int8)
+    wei = _rng(seed, 2).integers(-127, 128, size=(K, N), dtype=np.int8)
+    if wtag == "ba":
+        wei = np.ascontiguousarray(wei.T)
+    quant = {
+        "src_scale": QuantParam(cabi.DT_F32, MASK_COMMON, np.array([0.01], np.float32)),
+        "wei_scale": QuantParam(cabi.DT_F32, MASK_COL,
+                                _rng(seed, 3).uniform(1e-3, 1e-2, size=N).astype(np.float32)),
+        "dst_scale": QuantParam(cabi.DT_F32, MASK_COMMON, np.array([0.05], np.float32)),
+    }
+    po = [PostOp(kind=cabi.PO_ELTWISE, alg=cabi.ELTWISE["relu"], alpha=0.0, beta=0.0, scale=1.0)]
+    return MatmulProblem(M=M, N=N, K=K, src_dt=cabi.DT_S8, wei_dt=cabi.DT_S8, dst_dt=cabi.DT_S8,
+                         src=src, wei=wei, wei_stride=strides_for(wtag, 1, K, N), quant=quant,
+                         post_ops=po, dst_scale_mode=dst_scale_mode, impl=impl, name="C3")
+
+
+def _quant_e4m3_per_tensor(x):
+    amax = np.float32(np.max(np.abs(x)))
+    scale = np.float32(amax / np.float32(448.0))
+    return dtp.f32_to_e4m3((x / scale).astype(np.float32)), scale
+
+
+def config4(M=4096, N=28672, K=8192, seed=4, impl=cabi.IMPL_AUTO, wtag="ab"):
+    """e4m3 x e4m3 -> bf16 FFN up-projection: per-tensor scales amax/448, bf16
+    bias, GELU-tanh, then binary add of a bf16 residual."""
+    src, s_scale = _quant_e4m3_per_tensor(_rng(seed, 1).standard_normal((M, K), dtype=np.float32))
+    w = _rng(seed, 2).standard_normal((K, N), dtype=np.float32)
+    wei, w_scale = _quant_e4m3_per_tensor(w)
+    del w
+    if wtag == "ba":
+        wei = np.ascontiguousarray(wei.T)
+    bias = dtp.f32_to_bf16(_rng(seed, 3).uniform(-0.1, 0.1, size=N).astype(np.float32))
+    resid = dtp.f32_to_bf16(_rng(seed, 4).standard_normal((M, N), dtype=np.float32))
+    quant = {
+        "src_scale": QuantParam(cabi.DT_F32, MASK_COMMON, np.array([s_scale], np.float32)),
+        "wei_scale": QuantParam(cabi.DT_F32, MASK_COMMON, np.array([w_scale], np.float32)),
+    }
+    po = [
+        PostOp(kind=cabi.PO_ELTWISE, alg=cabi.ELTWISE["gelu_tanh"], scale=1.0),
+        PostOp(kind=cabi.PO_BINARY, alg=cabi.BINARY["add"], dt=cabi.DT_BF16,
+               stride=(M * N, N, 1), data=resid),
+    ]
+    return MatmulProblem(M=M, N=N, K=K, src_dt=cabi.DT_F8_E4M3, wei_dt=cabi.DT_F8_E4M3,
+                         dst_dt=cabi.DT_BF16, src=src, wei=wei,
+                         wei_stride=strides_for(wtag, 1, K, N), bias_dt=cabi.DT_BF16, bias=bias,
+                         quant=quant, post_ops=po, impl=impl, name="C4")
+
+
+def mx_quantize(x, axis):
+    """Block-quantize to e2m1 in blocks of 32 along `axis` with e8m0 scales
+    2^floor(log2(block amax / 6)); returns (codes, scale bytes)."""
+    x = np.asarray(x, dtype=np.float32)
+    xm = np.moveaxis(x, axis, -1)
+    shp = xm.shape
+    blk = xm.reshape(shp[:-1] + (shp[-1] // 32, 32))
+    amax = np.max(np.abs(blk), axis=-1)
+    with np.errstate(divide="ignore"):
+        e = np.floor(np.log2(amax / np.float32(6.0)))
+    e = np.where(amax > 0, e, -127.0)
+    sb = np.clip(e + 127, 0, 254).astype(np.int32)
+    scale = np.ldexp(np.float32(1.0), sb - 127).astype(np.float32)
+    q = dtp.f32_to_e2m1_codes((blk / scale[..., None]).astype(np.float32))
+    codes = np.moveaxis(q.reshape(shp), -1, axis)
+    scales = np.moveaxis(sb.astype(np.uint8), -1, axis) if False else sb.astype(np.uint8)
+    return codes, scales
+
+
+def config5(M=8192, N=8192, K=8192, seed=5, impl=cabi.IMPL_AUTO, wtag="ba"):
+    """MXFP4: e2m1 x e2m1 -> bf16 with e8m0 scales per block of 32 along K on
+    both operands; weights K-contiguous (tag ba) by default."""
+    xs = _rng(seed, 1).standard_normal((M, K), dtype=np.float32)
+    s_codes, s_sb = mx_quantize(xs, axis=1)          # scales [M][K/32]
+    del xs
+    xw = _rng(seed, 2).standard_normal((K, N), dtype=np.float32)
+    w_codes, w_sbT = mx_quantize(xw, axis=0)          # blocks along K: [N][K/32]
+    del xw
+    w_sb = np.ascontiguousarray(w_sbT.T)              # layout [K/32][N]
+    src = dtp.pack_nibbles(s_codes)
+    if wtag == "ba":
+        wei = dtp.pack_nibbles(np.ascontiguousarray(w_codes.T))
+    else:
+        wei = dtp.pack_nibbles(w_codes)
+    quant = {
+        "src_scale": QuantParam(cabi.DT_E8M0, MASK_ROW | MASK_COL, s_sb, (1, 32)),
+        "wei_scale": QuantParam(cabi.DT_E8M0, MASK_ROW | MASK_COL, w_sb, (32, 1)),
+    }
+    return MatmulProblem(M=M, N=N, K=K, src_dt=cabi.DT_F4_E2M1, wei_dt=cabi.DT_F4_E2M1,
+                         dst_dt=cabi.DT_BF16, src=src, wei=wei,
+                         wei_stride=strides_for(wtag, 1, K, N), quant=quant, impl=impl, name="C5")
+
+
+# algorithmic work per configuration
+def config_ops(p):
+    return 2 * p.batch * p.M * p.N * p.K
+
+
+def config2_bytes(M, N=14336, K=4096, group=128):
+    G = K // group
+    return K * N // 2 + G * N * 2 + G * N // 2 + M * K * 2 + M * N * 2

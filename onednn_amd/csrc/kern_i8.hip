@@ -1,0 +1,367 @@
+// "hip:mfma_i8" -- LDS-tiled int8 GEMM on the gfx950 matrix cores
+// (v_mfma_i32_32x32x32_i8) with the zero-point compensation folded into an
+// s32 row/column-sum correction and the reference's epilogue fused in.
+//
+// Replaces, for integer src and weights, the reference's brgemm int8 path
+// (src/cpu/x64/matmul/brgemm_matmul.cpp:658-1027: copy_B with s8s8/zp
+// compensation + AMX/VNNI microkernel + jit_brgemm_post_ops) and computes the
+// same values as ref_matmul_int8_t (src/cpu/matmul/ref_matmul_int8.cpp:174-306)
+// when there is a single group along K:
+//   acc[m,n] = sum_k (src[m,k] - zs) * (wei[k,n] - zw[n])          (s32)
+//            = sum_k s'w' + a*colsum'[n] + c[n]*rowsum'[m] + K*a*c[n]
+//     with s' = src - off_s, w' = wei - off_w the bytes re-biased to s8
+//     (off = 128 for u8, 0 for s8), a = off_s - zs, c[n] = off_w - zw[n];
+//   d = (float)acc * src_scale * wei_scale[n]  -> shared epilogue.
+#include "kernels.hpp"
+
+namespace mi355 {
+
+typedef int v4i __attribute__((ext_vector_type(4)));
+typedef int v16i __attribute__((ext_vector_type(16)));
+
+namespace {
+
+constexpr int BM = 256, BN = 256, BK = 64;
+constexpr int NT = 256;
+
+// byte offset of 16-byte chunk `chunk` (0..3) of tile row `row`; the chunk
+// index is XOR-swizzled with the row so that the 32 rows an MFMA operand read
+// touches spread over all LDS banks
+__device__ __forceinline__ int swz(int row, int chunk) {
+    return row * BK + ((chunk ^ ((row >> 1) & 3)) << 4);
+}
+
+struct i8_extra_t {
+    const int8_t *bt; // weights as [N][K] bytes, K contiguous
+    long ldb;         // bytes between consecutive n
+    long bt_bstride;  // bytes between batches (0 = broadcast)
+    const int *colsum; // [Bw][N] sum_k w'  (null when a == 0)
+    const int *rowsum; // [Bs][M] sum_k s'  (null when c == 0)
+    int src_u8, wei_u8;
+    int tiles_m, tiles_n;
+};
+
+__global__ void __launch_bounds__(NT) i8_gemm_kernel(const problem_t P_, const i8_extra_t X) {
+    const auto &P = MI355_KERNARG_PROBLEM();
+    __shared__ __attribute__((aligned(16))) char smem[2][2][BM * BK];
+
+    const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
+    const int wm = wave >> 1, wn = wave & 1;
+    const long b = blockIdx.z;
+
+    // XCD-aware tile order: consecutive workgroup ids go to different XCDs, so
+    // give each XCD a contiguous run of tiles, walked in bands of 8 tile rows.
+    int tile;
+    {
+        const int nwg = gridDim.x, id = blockIdx.x;
+        const int per = nwg / 8;
+        tile = (nwg % 8 == 0) ? (id % 8) * per + id / 8 : id;
+    }
+    constexpr int GM = 8;
+    const int band = tile / (GM * X.tiles_n);
+    const int band_rows = min(GM, X.tiles_m - band * GM);
+    const int in_band = tile - band * GM * X.tiles_n;
+    const int tm = band * GM + in_band % band_rows;
+    const int tn = in_band / band_rows;
+    const long m0 = (long)tm * BM, n0 = (long)tn * BN;
+
+    const int8_t *A = (const int8_t *)P.src + (P.ss[0] ? b * P.ss[0] : 0);
+    const long lda = P.ss[1];
+    const int8_t *Bt = X.bt + b * X.bt_bstride;
+    const long ldb = X.ldb;
+
+    // global -> register staging: 4 + 4 chunks of 16 bytes per thread
+    const int lrow = t >> 2, lchunk = t & 3;
+    const int8_t *ga[4], *gb[4];
+    int soff[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const int row = lrow + i * 64;
+        long ar = m0 + row;
+        if (ar > P.M - 1) ar = P.M - 1;
+        long br = n0 + row;
+        if (br > P.N - 1) br = P.N - 1;
+        ga[i] = A + ar * lda + lchunk * 16;
+        gb[i] = Bt + br * ldb + lchunk * 16;
+        soff[i] = swz(row, lchunk);
+    }
+
+    v16i acc[4][4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) acc[i][j][r] = 0;
+
+    const int nk = (int)(P.K / BK);
+    v4i ra[4], rb[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        ra[i] = *(const v4i *)(ga[i]);
+        rb[i] = *(const v4i *)(gb[i]);
+    }
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        *(v4i *)&smem[0][0][soff[i]] = ra[i];
+        *(v4i *)&smem[0][1][soff[i]] = rb[i];
+    }
+    __syncthreads();
+
+    const int frow = lane & 31, fch = lane >> 5;
+    const int xa = X.src_u8 ? (int)0x80808080 : 0, xb = X.wei_u8 ? (int)0x80808080 : 0;
+
+    for (int kt = 0; kt < nk; ++kt) {
+        const int cur = kt & 1;
+        if (kt + 1 < nk) {
+            const long ko = (long)(kt + 1) * BK;
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                ra[i] = *(const v4i *)(ga[i] + ko);
+                rb[i] = *(const v4i *)(gb[i] + ko);
+            }
+        }
+        const char *As = smem[cur][0], *Bs = smem[cur][1];
+#pragma unroll
+        for (int kh = 0; kh < 2; ++kh) {
+            v4i fa[4], fb[4];
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                fa[i] = *(const v4i *)&As[swz(wm * 128 + i * 32 + frow, kh * 2 + fch)];
+                fb[i] = *(const v4i *)&Bs[swz(wn * 128 + i * 32 + frow, kh * 2 + fch)];
+                fa[i] ^= xa;
+                fb[i] ^= xb;
+            }
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+#pragma unroll
+                for (int j = 0; j < 4; ++j)
+                    acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fa[i], fb[j], acc[i][j], 0, 0, 0);
+        }
+        if (kt + 1 < nk) {
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                *(v4i *)&smem[cur ^ 1][0][soff[i]] = ra[i];
+                *(v4i *)&smem[cur ^ 1][1][soff[i]] = rb[i];
+            }
+        }
+        __syncthreads();
+    }
+
+    // ---- epilogue: s32 compensation, scales, shared tail.
+    // Accumulators go through LDS one 32-row slab at a time so that each lane
+    // ends up with four consecutive n of one row: the per-element epilogue
+    // code exists once (a rolled loop) and dst leaves in wide coalesced stores.
+    const long bs = P.ss[0] ? b : 0, bw = P.ws[0] ? b : 0;
+    const int off_s = X.src_u8 ? 128 : 0, off_w = X.wei_u8 ? 128 : 0;
+    int a_c = off_s;
+    if (P.src_zp.dt != MI355_DT_UNDEF) a_c -= load_int(P.src_zp.dt, P.src_zp.p, 0);
+    const bool with_src_sc = P.src_scale.dt != MI355_DT_UNDEF;
+    const bool with_wei_sc = P.wei_scale.dt != MI355_DT_UNDEF;
+    const float ssc = with_src_sc ? load_float(P.src_scale.dt, P.src_scale.p, 0) : 1.f;
+    const int Kc = (int)P.K;
+
+    const long nbase = n0 + wn * 128 + (lane & 31) * 4;
+    int col_corr[4], c_c[4];
+    float wsc[4];
+    int nvalid = 0;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+        const long n = nbase + e;
+        col_corr[e] = 0; c_c[e] = 0; wsc[e] = 1.f;
+        if (n < P.N) {
+            nvalid = e + 1;
+            int c = off_w;
+            if (P.wei_zp.dt != MI355_DT_UNDEF)
+                c -= load_int(P.wei_zp.dt, P.wei_zp.p, quant_off(P.wei_zp, bw, 0, n, P.K, P.N));
+            c_c[e] = c;
+            col_corr[e] = (a_c != 0 ? a_c * X.colsum[bw * P.N + n] : 0) + Kc * a_c * c;
+            if (with_wei_sc)
+                wsc[e] = load_float(P.wei_scale.dt, P.wei_scale.p,
+                        quant_off(P.wei_scale, bw, 0, n, P.K, P.N));
+        }
+    }
+    const bool any_c = X.rowsum != nullptr;
+
+    int *wl = (int *)&smem[0][0][0] + wave * 4096; // 16 KB per wave
+    auto slab = [&](const v16i (&a)[4], const int i) {
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+#pragma unroll
+            for (int r = 0; r < 16; ++r)
+                wl[((r >> 2) * 8 + (lane >> 5) * 4 + (r & 3)) * 128 + j * 32 + (lane & 31)] = a[j][r];
+#pragma unroll 1
+        for (int it = 0; it < 16; ++it) {
+            const int row = it * 2 + (lane >> 5);
+            const long m = m0 + wm * 128 + i * 32 + row;
+            const v4i raw = *(const v4i *)&wl[row * 128 + (lane & 31) * 4];
+            if (m < P.M && nvalid > 0) {
+                const int rs = any_c ? X.rowsum[bs * P.M + m] : 0;
+                float f[4];
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    const int v = raw[e] + col_corr[e] + c_c[e] * rs;
+                    float x = (float)v;
+                    if (with_src_sc) x *= ssc;
+                    if (with_wei_sc) x *= wsc[e];
+                    f[e] = x;
+                }
+                epilogue_store4(P, f, b, m, nbase, nvalid);
+            }
+        }
+    };
+    slab(acc[0], 0);
+    slab(acc[1], 1);
+    slab(acc[2], 2);
+    slab(acc[3], 3);
+}
+
+// out[r] = sum_k (bytes[r][k] ^ flip) as signed bytes; one wave per row
+__global__ void __launch_bounds__(256) i8_rowsum_kernel(const int8_t *p, long rows, long K,
+        long ld, int flip, int *out) {
+    const long r = (long)blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (r >= rows) return;
+    const int lane = threadIdx.x & 63;
+    const int8_t *row = p + r * ld;
+    int s = 0;
+    const long k16 = K / 16 * 16;
+    for (long k = lane * 16; k < k16; k += 64 * 16) {
+        v4i v = *(const v4i *)(row + k);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const int w = v[i] ^ flip;
+            s += (int)(int8_t)(w & 0xff) + (int)(int8_t)((w >> 8) & 0xff)
+                    + (int)(int8_t)((w >> 16) & 0xff) + (w >> 24);
+        }
+    }
+    for (long k = k16 + lane; k < K; k += 64) s += (int)(int8_t)(row[k] ^ (flip & 0xff));
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) s += __shfl_down(s, o, 64);
+    if (lane == 0) out[r] = s;
+}
+
+// in: [R][C] bytes with row pitch ld_in  ->  out: [C][R] bytes, pitch ld_out
+__global__ void __launch_bounds__(256) transpose_bytes_kernel(const uint8_t *in, long R, long C,
+        long ld_in, long in_bstride, uint8_t *out, long ld_out, long out_bstride) {
+    __shared__ uint8_t tile[64][65];
+    in += blockIdx.z * in_bstride;
+    out += blockIdx.z * out_bstride;
+    const long r0 = (long)blockIdx.y * 64, c0 = (long)blockIdx.x * 64;
+    const int tx = threadIdx.x & 63, ty = threadIdx.x >> 6;
+    for (int i = ty; i < 64; i += 4) {
+        const long r = r0 + i, c = c0 + tx;
+        tile[i][tx] = (r < R && c < C) ? in[r * ld_in + c] : 0;
+    }
+    __syncthreads();
+    for (int i = ty; i < 64; i += 4) {
+        const long c = c0 + i, r = r0 + tx;
+        if (c < C && r < R) out[c * ld_out + r] = tile[tx][i];
+    }
+}
+
+struct i8_plan_t {
+    bool need_transpose, need_colsum, need_rowsum;
+    size_t off_bt, off_colsum, off_rowsum, total;
+    long Bw, Bs;
+};
+
+i8_plan_t make_plan(const mi355_matmul_desc_t &d) {
+    i8_plan_t p {};
+    p.Bw = d.wei_stride[0] ? d.batch : 1;
+    p.Bs = d.src_stride[0] ? d.batch : 1;
+    p.need_transpose = !(d.wei_stride[1] == 1);
+    // a = off_s - zs can be non-zero whenever src is u8 or has a zero point;
+    // c likewise for the weights
+    p.need_colsum = d.src_dt == MI355_DT_U8 || !quant_absent(d.src_zp);
+    p.need_rowsum = d.wei_dt == MI355_DT_U8 || !quant_absent(d.wei_zp);
+    size_t off = 0;
+    p.off_bt = off;
+    if (p.need_transpose) off += align_up((size_t)p.Bw * d.N * d.K, 256);
+    p.off_colsum = off;
+    if (p.need_colsum) off += align_up((size_t)p.Bw * d.N * 4, 256);
+    p.off_rowsum = off;
+    if (p.need_rowsum) off += align_up((size_t)p.Bs * d.M * 4, 256);
+    p.total = off;
+    return p;
+}
+
+} // namespace
+
+int i8_supported(const mi355_matmul_desc_t &d) {
+    if (!is_int8_dt(d.src_dt) || !is_int8_dt(d.wei_dt)) return MI355_UNIMPLEMENTED;
+    if (dt_bits(d.dst_dt) < 8) return MI355_UNIMPLEMENTED;
+    if (d.K < BK || d.K % BK != 0) return MI355_UNIMPLEMENTED;
+    if (d.src_stride[2] != 1 || d.src_stride[1] % 16 != 0) return MI355_UNIMPLEMENTED;
+    if (d.src_stride[0] % 16 != 0) return MI355_UNIMPLEMENTED;
+    const bool k_major = d.wei_stride[1] == 1 && d.wei_stride[2] % 16 == 0
+            && d.wei_stride[0] % 16 == 0;
+    const bool n_major = d.wei_stride[2] == 1;
+    if (!k_major && !n_major) return MI355_UNIMPLEMENTED;
+    // single group along K, per-tensor src parameters, per-tensor or per-N
+    // weights parameters
+    if (!quant_absent(d.src_pr)) return MI355_UNIMPLEMENTED;
+    if (!quant_absent(d.src_scale) && (d.src_scale.mask != 0)) return MI355_UNIMPLEMENTED;
+    if (!quant_absent(d.src_zp) && (d.src_zp.mask != 0)) return MI355_UNIMPLEMENTED;
+    if (!quant_absent(d.wei_scale)
+            && ((d.wei_scale.mask & 2) || d.wei_scale.group[0] > 1 || d.wei_scale.group[1] > 1))
+        return MI355_UNIMPLEMENTED;
+    if (!quant_absent(d.wei_zp)
+            && ((d.wei_zp.mask & 2) || d.wei_zp.group[0] > 1 || d.wei_zp.group[1] > 1))
+        return MI355_UNIMPLEMENTED;
+    if (d.batch > 65535) return MI355_UNIMPLEMENTED;
+    return MI355_SUCCESS;
+}
+
+size_t i8_scratch_bytes(const mi355_matmul_desc_t &d) {
+    return make_plan(d).total;
+}
+
+int i8_launch(const mi355_matmul_desc_t &d, const problem_t &P, void *scratch,
+        hipStream_t stream) {
+    const i8_plan_t plan = make_plan(d);
+    if (plan.total > 0 && !scratch) {
+        set_error("mfma_i8: %zu bytes of scratch required", plan.total);
+        return MI355_INVALID_ARGUMENTS;
+    }
+    char *sc = (char *)scratch;
+    i8_extra_t X {};
+    X.src_u8 = d.src_dt == MI355_DT_U8;
+    X.wei_u8 = d.wei_dt == MI355_DT_U8;
+    if (plan.need_transpose) {
+        uint8_t *bt = (uint8_t *)(sc + plan.off_bt);
+        dim3 grid((unsigned)((d.N + 63) / 64), (unsigned)((d.K + 63) / 64), (unsigned)plan.Bw);
+        hipLaunchKernelGGL(transpose_bytes_kernel, grid, dim3(256), 0, stream,
+                (const uint8_t *)P.wei, d.K, d.N, d.wei_stride[1], d.wei_stride[0], bt, d.K,
+                d.N * d.K);
+        X.bt = (const int8_t *)bt;
+        X.ldb = d.K;
+        X.bt_bstride = plan.Bw > 1 ? d.N * d.K : 0;
+    } else {
+        X.bt = (const int8_t *)P.wei;
+        X.ldb = d.wei_stride[2];
+        X.bt_bstride = d.wei_stride[0];
+    }
+    if (plan.need_colsum) {
+        int *cs = (int *)(sc + plan.off_colsum);
+        for (long b = 0; b < plan.Bw; ++b)
+            hipLaunchKernelGGL(i8_rowsum_kernel, dim3((unsigned)((d.N + 3) / 4)), dim3(256), 0,
+                    stream, X.bt + b * X.bt_bstride, d.N, d.K, X.ldb,
+                    X.wei_u8 ? (int)0x80808080 : 0, cs + b * d.N);
+        X.colsum = cs;
+    }
+    if (plan.need_rowsum) {
+        int *rs = (int *)(sc + plan.off_rowsum);
+        for (long b = 0; b < plan.Bs; ++b)
+            hipLaunchKernelGGL(i8_rowsum_kernel, dim3((unsigned)((d.M + 3) / 4)), dim3(256), 0,
+                    stream, (const int8_t *)P.src + b * d.src_stride[0], d.M, d.K,
+                    d.src_stride[1], X.src_u8 ? (int)0x80808080 : 0, rs + b * d.M);
+        X.rowsum = rs;
+    }
+    X.tiles_m = (int)((d.M + BM - 1) / BM);
+    X.tiles_n = (int)((d.N + BN - 1) / BN);
+    dim3 grid((unsigned)(X.tiles_m * X.tiles_n), 1, (unsigned)d.batch);
+    hipLaunchKernelGGL(i8_gemm_kernel, grid, dim3(NT), 0, stream, P, X);
+    return hipGetLastError() == hipSuccess ? MI355_SUCCESS : MI355_RUNTIME_ERROR;
+}
+
+} // namespace mi355

@@ -1,0 +1,133 @@
+// "hip:ref:any" -- one thread per dst element, every data type and attribute
+// combination the path admits.  It is the GPU-side counterpart of the
+// reference's naive implementations and computes in exactly their order:
+//   integer src:  ref_matmul_int8_t::execute_ref  src/cpu/matmul/ref_matmul_int8.cpp:174-306
+//   other src:    ref_matmul_t::execute_ref       src/cpu/matmul/ref_matmul.cpp:168-331
+// so its f32 results agree bit for bit with them wherever no libm function is
+// involved.  The tuned kernel families fall back to it for shapes and
+// attribute mixes they do not cover.
+#include "mi355_device.hpp"
+#include "kernels.hpp"
+
+namespace mi355 {
+
+template <class Q>
+__device__ __forceinline__ long ngroups_k(const Q &q, int kdim, long K) {
+    if (q.dt == MI355_DT_UNDEF) return 1;
+    const long g = kdim ? q.g1 : q.g0;
+    return g > 1 ? K / g : 1;
+}
+
+template <class PT>
+__device__ float ref_int_dot(const PT &P, long b, long m, long n) {
+    const long K = P.K, M = P.M, N = P.N;
+    const long bs = P.ss[0] ? b : 0, bw = P.ws[0] ? b : 0;
+    const bool src_zp = P.src_zp.dt != MI355_DT_UNDEF;
+    const bool wei_zp = P.wei_zp.dt != MI355_DT_UNDEF;
+    const bool src_pr = P.src_pr.dt != MI355_DT_UNDEF;
+    long ng = 1, t;
+    if ((t = ngroups_k(P.src_zp, 1, K)) > ng) ng = t;
+    if ((t = ngroups_k(P.wei_zp, 0, K)) > ng) ng = t;
+    if ((t = ngroups_k(P.src_scale, 1, K)) > ng) ng = t;
+    if ((t = ngroups_k(P.wei_scale, 0, K)) > ng) ng = t;
+    if ((t = ngroups_k(P.src_pr, 1, K)) > ng) ng = t;
+    const long gk = K / ng;
+    float res = 0.f;
+    for (long g = 0; g < ng; ++g) {
+        int acc = 0;
+        long k = g * gk;
+        for (long kk = 0; kk < gk; ++kk) {
+            k = g * gk + kk;
+            int s = load_int(P.src_dt, P.src, bs * P.ss[0] + m * P.ss[1] + k * P.ss[2]);
+            int w = load_int(P.wei_dt, P.wei, bw * P.ws[0] + k * P.ws[1] + n * P.ws[2]);
+            if (src_zp) s -= load_int(P.src_zp.dt, P.src_zp.p, quant_off(P.src_zp, bs, m, k, M, K));
+            if (wei_zp && !src_pr)
+                w -= load_int(P.wei_zp.dt, P.wei_zp.p, quant_off(P.wei_zp, bw, k, n, K, N));
+            acc += s * w;
+        }
+        if (src_pr) {
+            const int pr = load_int(P.src_pr.dt, P.src_pr.p, quant_off(P.src_pr, bs, m, k, M, K));
+            const int wzp = load_int(P.wei_zp.dt, P.wei_zp.p, quant_off(P.wei_zp, bw, k, n, K, N));
+            acc -= pr * wzp;
+            if (src_zp) {
+                const int szp = load_int(P.src_zp.dt, P.src_zp.p, quant_off(P.src_zp, bs, m, k, M, K));
+                acc += (int)(gk * wzp * szp);
+            }
+        }
+        float f = (float)acc;
+        if (P.src_scale.dt != MI355_DT_UNDEF)
+            f *= load_float(P.src_scale.dt, P.src_scale.p, quant_off(P.src_scale, bs, m, k, M, K));
+        if (P.wei_scale.dt != MI355_DT_UNDEF)
+            f *= load_float(P.wei_scale.dt, P.wei_scale.p, quant_off(P.wei_scale, bw, k, n, K, N));
+        res += f;
+    }
+    return res;
+}
+
+template <class PT>
+__device__ float ref_fp_dot(const PT &P, long b, long m, long n) {
+    const long K = P.K, M = P.M, N = P.N;
+    const long bs = P.ss[0] ? b : 0, bw = P.ws[0] ? b : 0;
+    const bool wei_int = P.wei_dt == MI355_DT_S8 || P.wei_dt == MI355_DT_U8
+            || P.wei_dt == MI355_DT_S4 || P.wei_dt == MI355_DT_U4;
+    const bool decomp = wei_int && P.apply_to_int;
+    const bool wei_zp = P.wei_zp.dt != MI355_DT_UNDEF;
+    const bool src_sc = P.src_scale.dt != MI355_DT_UNDEF;
+    const bool wei_sc = P.wei_scale.dt != MI355_DT_UNDEF;
+    const long sgk = src_sc ? P.src_scale.g1 : 1;
+    const long wgk = wei_sc ? P.wei_scale.g0 : 1;
+    const long ng = K / sgk > K / wgk ? K / sgk : K / wgk;
+    const long gk = K / ng;
+    float res = 0.f;
+    for (long g = 0; g < ng; ++g) {
+        float acc = 0.f;
+        long k = g * gk;
+        for (long kk = 0; kk < gk; ++kk) {
+            k = g * gk + kk;
+            const float s = load_float(P.src_dt, P.src, bs * P.ss[0] + m * P.ss[1] + k * P.ss[2]);
+            float w = load_float(P.wei_dt, P.wei, bw * P.ws[0] + k * P.ws[1] + n * P.ws[2]);
+            if (decomp) {
+                if (wei_zp)
+                    w -= load_float(P.wei_zp.dt, P.wei_zp.p, quant_off(P.wei_zp, bw, k, n, K, N));
+                if (wei_sc)
+                    w *= load_float(P.wei_scale.dt, P.wei_scale.p, quant_off(P.wei_scale, bw, k, n, K, N));
+            }
+            acc += s * w;
+        }
+        if (src_sc)
+            acc *= load_float(P.src_scale.dt, P.src_scale.p, quant_off(P.src_scale, bs, m, k, M, K));
+        if (wei_sc && !decomp)
+            acc *= load_float(P.wei_scale.dt, P.wei_scale.p, quant_off(P.wei_scale, bw, k, n, K, N));
+        res += acc;
+    }
+    return res;
+}
+
+__global__ void __launch_bounds__(256) ref_matmul_kernel(const problem_t P_) {
+    const auto &P = MI355_KERNARG_PROBLEM();
+    const long total = P.B * P.M * P.N;
+    for (long i = (long)blockIdx.x * blockDim.x + threadIdx.x; i < total;
+            i += (long)gridDim.x * blockDim.x) {
+        const long n = i % P.N, m = (i / P.N) % P.M, b = i / (P.N * P.M);
+        const bool int_path = P.src_dt == MI355_DT_S8 || P.src_dt == MI355_DT_U8;
+        const float v = int_path ? ref_int_dot(P, b, m, n) : ref_fp_dot(P, b, m, n);
+        epilogue_store(P, v, b, m, n);
+    }
+}
+
+int ref_supported(const mi355_matmul_desc_t &d) {
+    // 4-bit dst would need two elements per thread; not offered.
+    if (dt_bits(d.dst_dt) < 8) return MI355_UNIMPLEMENTED;
+    return MI355_SUCCESS;
+}
+
+int ref_launch(const problem_t &P, hipStream_t stream) {
+    const long total = P.B * P.M * P.N;
+    if (total == 0) return MI355_SUCCESS;
+    long blocks = (total + 255) / 256;
+    if (blocks > 1048576) blocks = 1048576;
+    hipLaunchKernelGGL(ref_matmul_kernel, dim3((unsigned)blocks), dim3(256), 0, stream, P);
+    return hipGetLastError() == hipSuccess ? MI355_SUCCESS : MI355_RUNTIME_ERROR;
+}
+
+} // namespace mi355

@@ -1,0 +1,43 @@
+// Internal interface between the C-ABI dispatcher (api.hip) and the kernel
+// families.  Each family exports a predicate (can it compute this problem
+// exactly?), its scratch need and a launcher.
+#pragma once
+#include <hip/hip_runtime.h>
+
+#include "../../include/mi355_matmul.h"
+#include "mi355_device.hpp"
+
+namespace mi355 {
+
+int ref_supported(const mi355_matmul_desc_t &d);
+int ref_launch(const problem_t &P, hipStream_t stream);
+
+int i8_supported(const mi355_matmul_desc_t &d);
+size_t i8_scratch_bytes(const mi355_matmul_desc_t &d);
+int i8_launch(const mi355_matmul_desc_t &d, const problem_t &P, void *scratch,
+        hipStream_t stream);
+
+int f8_supported(const mi355_matmul_desc_t &d);
+size_t f8_scratch_bytes(const mi355_matmul_desc_t &d);
+int f8_launch(const mi355_matmul_desc_t &d, const problem_t &P, void *scratch,
+        hipStream_t stream);
+
+int mxf4_supported(const mi355_matmul_desc_t &d);
+size_t mxf4_scratch_bytes(const mi355_matmul_desc_t &d);
+int mxf4_launch(const mi355_matmul_desc_t &d, const problem_t &P, void *scratch,
+        hipStream_t stream);
+
+int woq_supported(const mi355_matmul_desc_t &d);
+size_t woq_scratch_bytes(const mi355_matmul_desc_t &d);
+int woq_launch(const mi355_matmul_desc_t &d, const problem_t &P, void *scratch,
+        hipStream_t stream);
+
+void set_error(const char *fmt, ...);
+
+inline bool is_int8_dt(int dt) { return dt == MI355_DT_S8 || dt == MI355_DT_U8; }
+inline bool is_int4_dt(int dt) { return dt == MI355_DT_S4 || dt == MI355_DT_U4; }
+inline bool is_f8_dt(int dt) { return dt == MI355_DT_F8_E4M3 || dt == MI355_DT_F8_E5M2; }
+inline bool quant_absent(const mi355_quant_t &q) { return q.dt == MI355_DT_UNDEF; }
+inline size_t align_up(size_t v, size_t a) { return (v + a - 1) / a * a; }
+
+} // namespace mi355

@@ -1,0 +1,171 @@
+"""TEST INFRASTRUCTURE: ctypes binding of the CPU oracle (oracle/liboracle.so).
+
+Only tests/, __graft_entry__.smoke() and bench.py's cpu_baseline leg import
+this module; nothing under onednn_amd/ does.
+"""
+import ctypes as C
+import os
+import subprocess
+
+import numpy as np
+
+from onednn_amd import cabi
+from onednn_amd.problem import MatmulProblem, storage_dtype
+
+_DIR = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_DIR, "liboracle.so")
+FLAG_WEI_BF16 = 1
+FLAG_FOLD_SCALES = 2
+_lib = None
+
+
+def build():
+    subprocess.check_call(["make", "-C", _DIR, "-s"])
+
+
+def load():
+    global _lib
+    if _lib is not None:
+        return _lib
+    if not os.path.exists(LIB_PATH):
+        build()
+    lib = C.CDLL(LIB_PATH)
+    lib.oracle_matmul.argtypes = [C.POINTER(cabi.MatmulDesc), C.POINTER(cabi.MatmulArgs),
+                                  C.c_int, C.c_void_p, C.c_void_p]
+    lib.oracle_int8_acc.argtypes = [C.POINTER(cabi.MatmulDesc), C.POINTER(cabi.MatmulArgs),
+                                    C.c_void_p]
+    _lib = lib
+    return lib
+
+
+def _ptr(a):
+    return a.ctypes.data if a is not None else None
+
+
+def host_args(prob: MatmulProblem, dst):
+    """MatmulArgs over host arrays; returns (args, keepalive list)."""
+    keep = []
+    a = cabi.MatmulArgs()
+
+    def hold(x):
+        x = np.ascontiguousarray(x)
+        keep.append(x)
+        return x.ctypes.data
+
+    a.src, a.wei = hold(prob.src), hold(prob.wei)
+    if prob.bias is not None:
+        a.bias = hold(prob.bias)
+    a.dst = dst.ctypes.data
+    for name, q in prob.quant.items():
+        setattr(a, name, hold(q.data))
+    for i, po in enumerate(prob.post_ops):
+        if po.data is not None:
+            a.po_arg[i] = hold(po.data)
+    return a, keep
+
+
+def run_oracle(prob: MatmulProblem, flags=0, want_ideal=False):
+    """Returns raw dst storage (and, on request, the f64 pre-bias sum and the
+    sum of |terms| per dst element, for forward-error bounds)."""
+    lib = load()
+    dst = prob.initial_dst()
+    desc = prob.desc()
+    args, keep = host_args(prob, dst)
+    n = prob.batch * prob.M * prob.N
+    ideal = np.zeros(n, dtype=np.float64) if want_ideal else None
+    asum = np.zeros(n, dtype=np.float64) if want_ideal else None
+    st = lib.oracle_matmul(C.byref(desc), C.byref(args), flags, _ptr(ideal), _ptr(asum))
+    assert st == 0, f"oracle_matmul status {st}"
+    del keep
+    if want_ideal:
+        return dst, ideal, asum
+    return dst
+
+
+def run_int8_acc(prob: MatmulProblem):
+    lib = load()
+    dst = prob.initial_dst()
+    desc = prob.desc()
+    args, keep = host_args(prob, dst)
+    acc = np.zeros(prob.batch * prob.M * prob.N, dtype=np.int32)
+    st = lib.oracle_int8_acc(C.byref(desc), C.byref(args), acc.ctypes.data)
+    assert st == 0
+    del keep
+    return acc
+
+
+def _cvt(fn, arr, in_dt, out_dt, n_out=None):
+    lib = load()
+    arr = np.ascontiguousarray(arr, dtype=in_dt)
+    n = arr.size if n_out is None else n_out
+    out = np.zeros(n if n_out is None else n_out, dtype=out_dt)
+    getattr(lib, fn)(C.c_void_p(arr.ctypes.data), C.c_void_p(out.ctypes.data), C.c_int64(n))
+    return out
+
+
+def f32_to_bf16(x): return _cvt("oracle_f32_to_bf16", x, np.float32, np.uint16)
+def bf16_to_f32(x): return _cvt("oracle_bf16_to_f32", x, np.uint16, np.float32)
+def f32_to_f16(x): return _cvt("oracle_f32_to_f16", x, np.float32, np.uint16)
+def f16_to_f32(x): return _cvt("oracle_f16_to_f32", x, np.uint16, np.float32)
+def f16_to_e4m3(x): return _cvt("oracle_f16_to_e4m3", x, np.uint16, np.uint8)
+def f32_to_e4m3(x): return _cvt("oracle_f32_to_e4m3", x, np.float32, np.uint8)
+def e4m3_to_f32(x): return _cvt("oracle_e4m3_to_f32", x, np.uint8, np.float32)
+def f16_to_e5m2(x): return _cvt("oracle_f16_to_e5m2", x, np.uint16, np.uint8)
+def f32_to_e5m2(x): return _cvt("oracle_f32_to_e5m2", x, np.float32, np.uint8)
+def e5m2_to_f32(x): return _cvt("oracle_e5m2_to_f32", x, np.uint8, np.float32)
+def f32_to_e8m0(x): return _cvt("oracle_f32_to_e8m0", x, np.float32, np.uint8)
+def e8m0_to_f32(x): return _cvt("oracle_e8m0_to_f32", x, np.uint8, np.float32)
+
+
+def f32_to_e2m1_packed(x):
+    lib = load()
+    x = np.ascontiguousarray(x, dtype=np.float32)
+    out = np.zeros((x.size + 1) // 2, dtype=np.uint8)
+    lib.oracle_f32_to_e2m1(C.c_void_p(x.ctypes.data), C.c_void_p(out.ctypes.data), C.c_int64(x.size))
+    return out
+
+
+def nibbles_to_f32(fn, packed, n):
+    lib = load()
+    packed = np.ascontiguousarray(packed, dtype=np.uint8)
+    out = np.zeros(n, dtype=np.float32)
+    getattr(lib, fn)(C.c_void_p(packed.ctypes.data), C.c_void_p(out.ctypes.data), C.c_int64(n))
+    return out
+
+
+def store_float(dt, x):
+    lib = load()
+    x = np.ascontiguousarray(x, dtype=np.float32)
+    n_store = (x.size + 1) // 2 if cabi.DT_BITS[dt] == 4 else x.size
+    out = np.zeros(n_store, dtype=storage_dtype(dt))
+    lib.oracle_store_float(C.c_int(dt), C.c_void_p(x.ctypes.data), C.c_void_p(out.ctypes.data),
+                           C.c_int64(x.size))
+    return out
+
+
+def load_float(dt, raw, n):
+    lib = load()
+    raw = np.ascontiguousarray(raw)
+    out = np.zeros(n, dtype=np.float32)
+    lib.oracle_load_float(C.c_int(dt), C.c_void_p(raw.ctypes.data), C.c_void_p(out.ctypes.data),
+                          C.c_int64(n))
+    return out
+
+
+def eltwise(alg, x, alpha=0.0, beta=0.0):
+    lib = load()
+    x = np.ascontiguousarray(x, dtype=np.float32)
+    out = np.zeros_like(x)
+    lib.oracle_eltwise(C.c_int(alg), C.c_float(alpha), C.c_float(beta), C.c_void_p(x.ctypes.data),
+                       C.c_void_p(out.ctypes.data), C.c_int64(x.size))
+    return out
+
+
+def binary(alg, x, y):
+    lib = load()
+    x = np.ascontiguousarray(x, dtype=np.float32)
+    y = np.ascontiguousarray(y, dtype=np.float32)
+    out = np.zeros_like(x)
+    lib.oracle_binary(C.c_int(alg), C.c_void_p(x.ctypes.data), C.c_void_p(y.ctypes.data),
+                      C.c_void_p(out.ctypes.data), C.c_int64(x.size))
+    return out

@@ -1,0 +1,547 @@
+/*
+ * TEST INFRASTRUCTURE -- CPU oracle, not part of the shipped library.
+ * Only tests/, __graft_entry__.smoke() and bench.py's cpu_baseline leg may use
+ * anything in this directory; the product never links or loads it.
+ *
+ * A plain-C restatement of the two naive matmul implementations of the
+ * reference (uxlfoundation/oneDNN v3.14) and of the helpers they call:
+ *
+ *   orc_int8_dot      ref_matmul_int8_t::execute_ref, the `ker` lambda
+ *                     src/cpu/matmul/ref_matmul_int8.cpp:174-261
+ *   orc_fp_dot        ref_matmul_t::execute_ref, the `ker` lambda
+ *                     src/cpu/matmul/ref_matmul.cpp:168-236
+ *   orc_finish        bias + post-ops + dst scale + dst zero point + store
+ *                     ref_matmul_int8.cpp:275-306, ref_matmul.cpp:283-331
+ *   orc_post_ops      ref_post_ops_t::execute src/cpu/primitive_attr_postops.cpp:312-394
+ *   orc_eltwise       compute_eltwise_scalar_fwd :49-87 with the formulas of
+ *                     src/common/math_utils.hpp:120-430
+ *   orc_binary        compute_binary_scalar src/cpu/primitive_attr_postops.cpp:30-47
+ *   orc_load_int / orc_load_float / orc_store_float
+ *                     io::load_int_value / load_float_value / store_float_value
+ *                     src/cpu/ref_io_helper.hpp:34-150 and
+ *                     q10n::saturate_and_round src/cpu/simple_q10n.hpp:41-81
+ *   orc_quant_off     quant_entry_t::get_md src/common/primitive_attr_quant.hpp:116-140
+ *                     + matmul_helper_t::get_quant_off src/cpu/matmul/matmul_utils.hpp:154-173
+ *
+ * Implementation choice follows the CPU engine's list
+ * (src/cpu/matmul/cpu_matmul_list.cpp:73-109): integer src (s8/u8) takes the
+ * s32-accumulating path, every other src the f32 path.
+ *
+ * Two documented deviations of the reference's JIT path ("brg_matmul") are
+ * available as switches because they change bits:
+ *   desc->dst_scale_mode == MI355_DST_SCALE_RECIPROCAL:  d *= (1.f/dst_scale)
+ *       instead of d /= dst_scale  (src/cpu/x64/matmul/brgemm_matmul.cpp:703-709)
+ *   ORC_FLAG_WEI_BF16: decompressed weights are rounded to bf16 before the
+ *       multiply (src/cpu/x64/matmul/brgemm_matmul_copy_utils.cpp:2870-2896)
+ *
+ * Parity status: every function here is pinned by tests/test_oracle_*.py
+ * (brute-force int64 loops, closed forms, one-hot decodes, tie vectors, f64
+ * restatements with forward error bounds).  The reference cannot be compiled
+ * in this environment (its sources need a CMake-generated dnnl_config.h), so
+ * no oracle/_ref build exists; see the pinning list in the tests' docstrings.
+ * Unpinned: none of the functions used by the five benchmark configurations;
+ * the libm-dependent eltwise algorithms other than relu/gelu_tanh/linear/tanh
+ * are "parity unpinned" beyond their textbook formula.
+ */
+#include <limits.h>
+#include <math.h>
+#include <stdint.h>
+#include <stdlib.h>
+#include <string.h>
+
+#include "../include/mi355_matmul.h"
+#include "oracle_dtypes.h"
+
+#define ORC_FLAG_WEI_BF16 1 /* round decompressed weights to bf16 (JIT flavour) */
+#define ORC_FLAG_FOLD_SCALES 2 /* fp path: apply per-tensor scales once after
+                                  the K sum (what a GEMM kernel does) */
+
+/* ------------------------------------------------------------------ loads */
+static inline int orc_load_int(int dt, const void *p, int64_t off) {
+    switch (dt) {
+        case MI355_DT_S32: return ((const int32_t *)p)[off];
+        case MI355_DT_S8: return ((const int8_t *)p)[off];
+        case MI355_DT_U8: return ((const uint8_t *)p)[off];
+        case MI355_DT_S4: return orc_s4_to_int(orc_nibble_get(p, off));
+        case MI355_DT_U4: return (int)orc_nibble_get(p, off);
+        default: return INT_MAX;
+    }
+}
+
+static inline float orc_load_float(int dt, const void *p, int64_t off) {
+    switch (dt) {
+        case MI355_DT_F32: return ((const float *)p)[off];
+        case MI355_DT_BF16: return orc_bf16_to_f32(((const uint16_t *)p)[off]);
+        case MI355_DT_F16: return orc_f16_to_f32(((const uint16_t *)p)[off]);
+        case MI355_DT_F8_E4M3: return orc_e4m3_to_f32(((const uint8_t *)p)[off]);
+        case MI355_DT_F8_E5M2: return orc_e5m2_to_f32(((const uint8_t *)p)[off]);
+        case MI355_DT_E8M0: return orc_e8m0_to_f32(((const uint8_t *)p)[off]);
+        case MI355_DT_F4_E2M1: return orc_e2m1_to_f32(orc_nibble_get(p, off));
+        case MI355_DT_S32: return (float)((const int32_t *)p)[off];
+        case MI355_DT_S8: return (float)((const int8_t *)p)[off];
+        case MI355_DT_U8: return (float)((const uint8_t *)p)[off];
+        case MI355_DT_S4: return (float)orc_s4_to_int(orc_nibble_get(p, off));
+        case MI355_DT_U4: return (float)orc_nibble_get(p, off);
+        default: return NAN;
+    }
+}
+
+static inline float orc_sat(float v, float lo, float hi) {
+    if (v < lo) v = lo;
+    if (v > hi) v = hi;
+    return v;
+}
+
+static inline void orc_store_float(int dt, float v, void *p, int64_t off) {
+    switch (dt) {
+        case MI355_DT_F32: ((float *)p)[off] = v; break;
+        case MI355_DT_BF16: ((uint16_t *)p)[off] = orc_f32_to_bf16(v); break;
+        case MI355_DT_F16: ((uint16_t *)p)[off] = orc_f32_to_f16(v); break;
+        case MI355_DT_F8_E4M3: ((uint8_t *)p)[off] = orc_f32_to_e4m3(v); break;
+        case MI355_DT_F8_E5M2: ((uint8_t *)p)[off] = orc_f32_to_e5m2(v); break;
+        case MI355_DT_E8M0: ((uint8_t *)p)[off] = orc_f32_to_e8m0(v); break;
+        case MI355_DT_F4_E2M1: orc_nibble_set(p, off, orc_f32_to_e2m1(v)); break;
+        /* integers: clamp in f32 first, then round to nearest even.  The s32
+         * upper bound is the largest float below 2^31
+         * (src/common/type_helpers.hpp:232). */
+        case MI355_DT_S32:
+            ((int32_t *)p)[off]
+                    = (int32_t)nearbyintf(orc_sat(v, -2147483648.f, 2147483520.f));
+            break;
+        case MI355_DT_S8:
+            ((int8_t *)p)[off] = (int8_t)nearbyintf(orc_sat(v, -128.f, 127.f));
+            break;
+        case MI355_DT_U8:
+            ((uint8_t *)p)[off] = (uint8_t)nearbyintf(orc_sat(v, 0.f, 255.f));
+            break;
+        default: break;
+    }
+}
+
+/* --------------------------------------------------- quant parameter index */
+static inline int64_t orc_quant_off(const mi355_quant_t *q, int64_t b,
+        int64_t i0, int64_t i1, int64_t D0, int64_t D1) {
+    int64_t q1 = (q->mask & 2) ? D0 / q->group[0] : 1;
+    int64_t q2 = (q->mask & 4) ? D1 / q->group[1] : 1;
+    int64_t ib = (q->mask & 1) ? b : 0;
+    int64_t j0 = (q->mask & 2) ? i0 / q->group[0] : 0;
+    int64_t j1 = (q->mask & 4) ? i1 / q->group[1] : 0;
+    return (ib * q1 + j0) * q2 + j1;
+}
+
+/* number of groups a parameter induces along K; `kdim` = 0/1 is the position
+ * of K among the argument's last two dims */
+static inline int64_t orc_ngroups_k(const mi355_quant_t *q, int kdim, int64_t K) {
+    if (q->dt == MI355_DT_UNDEF) return 1;
+    int64_t g = q->group[kdim];
+    return g > 1 ? K / g : 1;
+}
+
+/* ----------------------------------------------------------------- eltwise */
+static float orc_logistic(float s) {
+    const float bound = 88.72283172607421875f;
+    float in = -s;
+    return in < bound ? 1.f / (1.f + expf(in)) : 0.f;
+}
+static float orc_soft_relu(float s, float alpha) {
+    const float bound = 88.72283172607421875f;
+    float in = s * alpha;
+    float v = in < bound ? log1pf(expf(in)) : in;
+    return v / alpha;
+}
+
+float orc_eltwise(int alg, float s, float alpha, float beta) {
+    switch (alg) {
+        case MI355_ELTWISE_RELU: return s > 0 ? s : s * alpha;
+        case MI355_ELTWISE_TANH: return tanhf(s);
+        case MI355_ELTWISE_ELU: return s > 0 ? s : alpha * expm1f(s);
+        case MI355_ELTWISE_SQUARE: return s * s;
+        case MI355_ELTWISE_ABS: return s > 0 ? s : -s;
+        case MI355_ELTWISE_SQRT: return sqrtf(s);
+        case MI355_ELTWISE_LINEAR: return alpha * s + beta;
+        case MI355_ELTWISE_SOFT_RELU: return orc_soft_relu(s, alpha);
+        case MI355_ELTWISE_HARDSIGMOID: {
+            float v = alpha * s + beta;
+            return v <= 0.f ? 0.f : v >= 1.f ? 1.f : v;
+        }
+        case MI355_ELTWISE_LOGISTIC: return orc_logistic(s);
+        case MI355_ELTWISE_EXP: return expf(s);
+        case MI355_ELTWISE_GELU_TANH: {
+            const float sqrt_2_over_pi = 0.79788458347320556640625f;
+            const float fit = 0.044715f;
+            float v = tanhf(sqrt_2_over_pi * s * (1 + fit * s * s));
+            return (float)(0.5 * s * (1. + v)); /* outer product in double */
+        }
+        case MI355_ELTWISE_SWISH: return s * orc_logistic(alpha * s);
+        case MI355_ELTWISE_LOG: return logf(s);
+        case MI355_ELTWISE_CLIP: {
+            s = s > alpha ? s : alpha;
+            return s > beta ? beta : s;
+        }
+        case MI355_ELTWISE_CLIP_V2: {
+            s = s > alpha ? s : alpha;
+            return s < beta ? s : beta;
+        }
+        case MI355_ELTWISE_POW: return alpha * powf(s, beta);
+        case MI355_ELTWISE_GELU_ERF: {
+            const float sqrt_2_over_2 = 0.707106769084930419921875f;
+            float v = s * sqrt_2_over_2;
+            return 0.5f * s * (1.f + erff(v));
+        }
+        case MI355_ELTWISE_ROUND: return nearbyintf(s);
+        case MI355_ELTWISE_MISH: return s * tanhf(orc_soft_relu(s, 1.f));
+        case MI355_ELTWISE_HARDSWISH: {
+            float v = alpha * s + beta;
+            float h = v <= 0.f ? 0.f : v >= 1.f ? 1.f : v;
+            return s * h;
+        }
+        default: return NAN;
+    }
+}
+
+float orc_binary(int alg, float x, float y) {
+    switch (alg) {
+        case MI355_BINARY_ADD: return x + y;
+        case MI355_BINARY_DIV: return x / y;
+        case MI355_BINARY_MAX: return x > y ? x : y; /* nstl::max: (a > b) ? a : b */
+        case MI355_BINARY_MIN: return x < y ? x : y;
+        case MI355_BINARY_MUL: return x * y;
+        case MI355_BINARY_SUB: return x - y;
+        case MI355_BINARY_GE: return x >= y;
+        case MI355_BINARY_GT: return x > y;
+        case MI355_BINARY_LE: return x <= y;
+        case MI355_BINARY_LT: return x < y;
+        case MI355_BINARY_EQ: return x == y;
+        case MI355_BINARY_NE: return x != y;
+        default: return NAN;
+    }
+}
+
+static float orc_post_ops(const mi355_matmul_desc_t *d,
+        const mi355_matmul_args_t *a, float res, float dst_old, int64_t b,
+        int64_t m, int64_t n) {
+    for (int i = 0; i < d->n_post_ops; ++i) {
+        const mi355_post_op_t *po = &d->post_ops[i];
+        switch (po->kind) {
+            case MI355_PO_SUM:
+                res += po->scale * (dst_old - (float)po->zero_point);
+                break;
+            case MI355_PO_ELTWISE:
+                res = orc_eltwise(po->alg, res, po->alpha, po->beta) * po->scale;
+                break;
+            case MI355_PO_BINARY: {
+                int64_t off = b * po->stride[0] + m * po->stride[1]
+                        + n * po->stride[2];
+                float v = orc_load_float(po->dt, a->po_arg[i], off);
+                res = orc_binary(po->alg, res, v);
+            } break;
+            case MI355_PO_PRELU: {
+                if (res >= 0) break;
+                int64_t off = b * po->stride[0] + m * po->stride[1]
+                        + n * po->stride[2];
+                res = ((const float *)a->po_arg[i])[off] * res;
+            } break;
+            default: break;
+        }
+    }
+    return res;
+}
+
+/* ------------------------------------------------------------- int8 path */
+static float orc_int8_dot(const mi355_matmul_desc_t *d,
+        const mi355_matmul_args_t *a, int64_t b, int64_t m, int64_t n,
+        int32_t *last_acc) {
+    const int64_t K = d->K, M = d->M, N = d->N;
+    const int64_t bs = d->src_stride[0] ? b : 0, bw = d->wei_stride[0] ? b : 0;
+    const int with_src_zp = d->src_zp.dt != MI355_DT_UNDEF;
+    const int with_wei_zp = d->wei_zp.dt != MI355_DT_UNDEF;
+    const int with_src_pr = d->src_pr.dt != MI355_DT_UNDEF;
+    const int with_src_sc = d->src_scale.dt != MI355_DT_UNDEF;
+    const int with_wei_sc = d->wei_scale.dt != MI355_DT_UNDEF;
+
+    int64_t ng = 1, t;
+    if ((t = orc_ngroups_k(&d->src_zp, 1, K)) > ng) ng = t;
+    if ((t = orc_ngroups_k(&d->wei_zp, 0, K)) > ng) ng = t;
+    if ((t = orc_ngroups_k(&d->src_scale, 1, K)) > ng) ng = t;
+    if ((t = orc_ngroups_k(&d->wei_scale, 0, K)) > ng) ng = t;
+    if ((t = orc_ngroups_k(&d->src_pr, 1, K)) > ng) ng = t;
+    const int64_t gk = K / ng;
+
+    float res = 0.f;
+    for (int64_t g = 0; g < ng; ++g) {
+        uint32_t acc = 0; /* s32 arithmetic with defined wrap-around */
+        int64_t k = g * gk;
+        for (int64_t kk = 0; kk < gk; ++kk) {
+            k = g * gk + kk;
+            int s = orc_load_int(d->src_dt, a->src,
+                    bs * d->src_stride[0] + m * d->src_stride[1]
+                            + k * d->src_stride[2]);
+            int w = orc_load_int(d->wei_dt, a->wei,
+                    bw * d->wei_stride[0] + k * d->wei_stride[1]
+                            + n * d->wei_stride[2]);
+            if (with_src_zp)
+                s -= orc_load_int(d->src_zp.dt, a->src_zp,
+                        orc_quant_off(&d->src_zp, bs, m, k, M, K));
+            if (with_wei_zp && !with_src_pr)
+                w -= orc_load_int(d->wei_zp.dt, a->wei_zp,
+                        orc_quant_off(&d->wei_zp, bw, k, n, K, N));
+            acc += (uint32_t)(s * w);
+        }
+        if (with_src_pr) {
+            /* k is the last index of the group, as in the reference */
+            int pr = orc_load_int(d->src_pr.dt, a->src_pr,
+                    orc_quant_off(&d->src_pr, bs, m, k, M, K));
+            int wzp = orc_load_int(d->wei_zp.dt, a->wei_zp,
+                    orc_quant_off(&d->wei_zp, bw, k, n, K, N));
+            acc -= (uint32_t)(pr * wzp);
+            if (with_src_zp) {
+                int szp = orc_load_int(d->src_zp.dt, a->src_zp,
+                        orc_quant_off(&d->src_zp, bs, m, k, M, K));
+                acc += (uint32_t)(int)(gk * wzp * szp);
+            }
+        }
+        float acc_f = (float)(int32_t)acc;
+        if (last_acc) *last_acc = (int32_t)acc;
+        if (with_src_sc)
+            acc_f *= orc_load_float(d->src_scale.dt, a->src_scale,
+                    orc_quant_off(&d->src_scale, bs, m, k, M, K));
+        if (with_wei_sc)
+            acc_f *= orc_load_float(d->wei_scale.dt, a->wei_scale,
+                    orc_quant_off(&d->wei_scale, bw, k, n, K, N));
+        res += acc_f;
+    }
+    return res;
+}
+
+/* --------------------------------------------------------------- fp path */
+static float orc_fp_dot(const mi355_matmul_desc_t *d,
+        const mi355_matmul_args_t *a, int64_t b, int64_t m, int64_t n,
+        int flags, double *ideal, double *abs_sum) {
+    const int64_t K = d->K, M = d->M, N = d->N;
+    const int64_t bs = d->src_stride[0] ? b : 0, bw = d->wei_stride[0] ? b : 0;
+    const int wei_is_int = d->wei_dt == MI355_DT_S8 || d->wei_dt == MI355_DT_U8
+            || d->wei_dt == MI355_DT_S4 || d->wei_dt == MI355_DT_U4;
+    const int decomp = wei_is_int && d->fpmath_apply_to_int;
+    const int with_wei_zp = d->wei_zp.dt != MI355_DT_UNDEF;
+    const int with_src_sc = d->src_scale.dt != MI355_DT_UNDEF;
+    const int with_wei_sc = d->wei_scale.dt != MI355_DT_UNDEF;
+
+    /* get_group() returns 1 when groups are absent, so without groups on
+     * both sides every product is its own "group" (ref_matmul.cpp:135-166) */
+    int64_t sgk = with_src_sc ? d->src_scale.group[1] : 1;
+    int64_t wgk = with_wei_sc ? d->wei_scale.group[0] : 1;
+    int64_t ng = K / sgk > K / wgk ? K / sgk : K / wgk;
+    int64_t gk = K / ng;
+    const int fold = (flags & ORC_FLAG_FOLD_SCALES) && !decomp
+            && !(d->src_scale.mask & 4) && !(d->wei_scale.mask & 2);
+    if (fold) { ng = 1; gk = K; }
+
+    float res = 0.f;
+    double id = 0., as = 0.;
+    for (int64_t g = 0; g < ng; ++g) {
+        float acc = 0.f;
+        double acc_d = 0., acc_a = 0.;
+        int64_t k = g * gk;
+        for (int64_t kk = 0; kk < gk; ++kk) {
+            k = g * gk + kk;
+            float s = orc_load_float(d->src_dt, a->src,
+                    bs * d->src_stride[0] + m * d->src_stride[1]
+                            + k * d->src_stride[2]);
+            float w = orc_load_float(d->wei_dt, a->wei,
+                    bw * d->wei_stride[0] + k * d->wei_stride[1]
+                            + n * d->wei_stride[2]);
+            if (decomp) {
+                if (with_wei_zp)
+                    w -= orc_load_float(d->wei_zp.dt, a->wei_zp,
+                            orc_quant_off(&d->wei_zp, bw, k, n, K, N));
+                if (with_wei_sc)
+                    w *= orc_load_float(d->wei_scale.dt, a->wei_scale,
+                            orc_quant_off(&d->wei_scale, bw, k, n, K, N));
+                if (flags & ORC_FLAG_WEI_BF16)
+                    w = orc_bf16_to_f32(orc_f32_to_bf16(w));
+            }
+            float p = s * w;
+            acc += p;
+            acc_d += (double)s * (double)w;
+            acc_a += fabs((double)s * (double)w);
+        }
+        double sc = 1.;
+        if (with_src_sc) {
+            float v = orc_load_float(d->src_scale.dt, a->src_scale,
+                    orc_quant_off(&d->src_scale, bs, m, k, M, K));
+            acc *= v;
+            sc *= (double)v;
+        }
+        if (with_wei_sc && !decomp) {
+            float v = orc_load_float(d->wei_scale.dt, a->wei_scale,
+                    orc_quant_off(&d->wei_scale, bw, k, n, K, N));
+            acc *= v;
+            sc *= (double)v;
+        }
+        res += acc;
+        id += acc_d * sc;
+        as += acc_a * fabs(sc);
+    }
+    if (ideal) *ideal = id;
+    if (abs_sum) *abs_sum = as;
+    return res;
+}
+
+/* ------------------------------------------------------------- epilogue */
+static void orc_finish(const mi355_matmul_desc_t *d,
+        const mi355_matmul_args_t *a, float v, int64_t b, int64_t m,
+        int64_t n) {
+    const int64_t doff
+            = b * d->dst_stride[0] + m * d->dst_stride[1] + n * d->dst_stride[2];
+    if (d->bias_dt != MI355_DT_UNDEF)
+        v += orc_load_float(d->bias_dt, a->bias,
+                b * d->bias_stride[0] + m * d->bias_stride[1]
+                        + n * d->bias_stride[2]);
+    if (d->n_post_ops > 0) {
+        float dst_old = 0.f;
+        for (int i = 0; i < d->n_post_ops; ++i)
+            if (d->post_ops[i].kind == MI355_PO_SUM) {
+                int sdt = d->post_ops[i].dt ? d->post_ops[i].dt : d->dst_dt;
+                dst_old = orc_load_float(sdt, a->dst, doff);
+                break;
+            }
+        v = orc_post_ops(d, a, v, dst_old, b, m, n);
+    }
+    if (d->dst_scale.dt != MI355_DT_UNDEF) {
+        float s = orc_load_float(d->dst_scale.dt, a->dst_scale, 0);
+        if (d->dst_scale_mode == MI355_DST_SCALE_RECIPROCAL) {
+            float r = 1.f / s;
+            v *= r;
+        } else {
+            v /= s;
+        }
+    }
+    if (d->dst_zp.dt != MI355_DT_UNDEF) {
+        int z = orc_load_int(MI355_DT_S32, a->dst_zp, (d->dst_zp.mask & 4) ? n : 0);
+        v += (float)z;
+    }
+    orc_store_float(d->dst_dt, v, a->dst, doff);
+}
+
+static int orc_src_is_int(int dt) {
+    return dt == MI355_DT_S8 || dt == MI355_DT_U8;
+}
+
+/*
+ * Run the matmul described by `d` on host pointers.
+ *   flags        ORC_FLAG_*
+ *   ideal        optional [batch*M*N] doubles: the pre-bias sum evaluated in
+ *                f64 (fp path only)
+ *   abs_sum      optional [batch*M*N] doubles: sum of |terms| of that sum, the
+ *                scale of its forward rounding error
+ */
+int oracle_matmul(const mi355_matmul_desc_t *d, const mi355_matmul_args_t *a,
+        int flags, double *ideal, double *abs_sum) {
+    if (!d || !a) return MI355_INVALID_ARGUMENTS;
+    if (d->batch == 0 || d->M == 0 || d->N == 0 || d->K == 0) return MI355_SUCCESS;
+    const int int_path = orc_src_is_int(d->src_dt);
+    const int64_t B = d->batch, M = d->M, N = d->N;
+    /* 4-bit dst: two n share a byte, so a thread owns whole rows */
+#pragma omp parallel for collapse(2) schedule(static)
+    for (int64_t b = 0; b < B; ++b)
+        for (int64_t m = 0; m < M; ++m)
+            for (int64_t n = 0; n < N; ++n) {
+                float v;
+                if (int_path) {
+                    v = orc_int8_dot(d, a, b, m, n, NULL);
+                } else {
+                    int64_t i = (b * M + m) * N + n;
+                    v = orc_fp_dot(d, a, b, m, n, flags, ideal ? ideal + i : NULL,
+                            abs_sum ? abs_sum + i : NULL);
+                }
+                orc_finish(d, a, v, b, m, n);
+            }
+    return MI355_SUCCESS;
+}
+
+/* s32 accumulator only: Sum_k (src - zp_s)(wei - zp_w), for closed-form and
+ * brute-force checks of the integer core.  Zero-point and precomputed-
+ * reduction groups along K are not meaningful here (one group is reported). */
+int oracle_int8_acc(const mi355_matmul_desc_t *d, const mi355_matmul_args_t *a,
+        int32_t *acc_out) {
+    mi355_matmul_desc_t t = *d;
+    t.src_scale.dt = t.wei_scale.dt = MI355_DT_UNDEF;
+    t.src_scale.group[0] = t.src_scale.group[1] = 1;
+    t.wei_scale.group[0] = t.wei_scale.group[1] = 1;
+    if (!orc_src_is_int(d->src_dt)) return MI355_INVALID_ARGUMENTS;
+    const int64_t B = d->batch, M = d->M, N = d->N;
+#pragma omp parallel for collapse(2) schedule(static)
+    for (int64_t b = 0; b < B; ++b)
+        for (int64_t m = 0; m < M; ++m)
+            for (int64_t n = 0; n < N; ++n)
+                (void)orc_int8_dot(&t, a, b, m, n, &acc_out[(b * M + m) * N + n]);
+    return MI355_SUCCESS;
+}
+
+/* ------------------------------------------- array conversions for tests */
+#define ORC_CVT_LOOP(expr) \
+    for (int64_t i = 0; i < n; ++i) { expr; }
+
+void oracle_f32_to_bf16(const float *in, uint16_t *out, int64_t n) {
+    ORC_CVT_LOOP(out[i] = orc_f32_to_bf16(in[i]))
+}
+void oracle_bf16_to_f32(const uint16_t *in, float *out, int64_t n) {
+    ORC_CVT_LOOP(out[i] = orc_bf16_to_f32(in[i]))
+}
+void oracle_f32_to_f16(const float *in, uint16_t *out, int64_t n) {
+    ORC_CVT_LOOP(out[i] = orc_f32_to_f16(in[i]))
+}
+void oracle_f16_to_f32(const uint16_t *in, float *out, int64_t n) {
+    ORC_CVT_LOOP(out[i] = orc_f16_to_f32(in[i]))
+}
+void oracle_f16_to_e4m3(const uint16_t *in, uint8_t *out, int64_t n) {
+    ORC_CVT_LOOP(out[i] = orc_f16_to_e4m3(in[i]))
+}
+void oracle_f32_to_e4m3(const float *in, uint8_t *out, int64_t n) {
+    ORC_CVT_LOOP(out[i] = orc_f32_to_e4m3(in[i]))
+}
+void oracle_e4m3_to_f32(const uint8_t *in, float *out, int64_t n) {
+    ORC_CVT_LOOP(out[i] = orc_e4m3_to_f32(in[i]))
+}
+void oracle_f16_to_e5m2(const uint16_t *in, uint8_t *out, int64_t n) {
+    ORC_CVT_LOOP(out[i] = orc_f16_to_e5m2(in[i]))
+}
+void oracle_f32_to_e5m2(const float *in, uint8_t *out, int64_t n) {
+    ORC_CVT_LOOP(out[i] = orc_f32_to_e5m2(in[i]))
+}
+void oracle_e5m2_to_f32(const uint8_t *in, float *out, int64_t n) {
+    ORC_CVT_LOOP(out[i] = orc_e5m2_to_f32(in[i]))
+}
+void oracle_f32_to_e8m0(const float *in, uint8_t *out, int64_t n) {
+    ORC_CVT_LOOP(out[i] = orc_f32_to_e8m0(in[i]))
+}
+void oracle_e8m0_to_f32(const uint8_t *in, float *out, int64_t n) {
+    ORC_CVT_LOOP(out[i] = orc_e8m0_to_f32(in[i]))
+}
+/* 4-bit arrays: `n` logical elements, packed two per byte, low nibble first */
+void oracle_f32_to_e2m1(const float *in, uint8_t *out, int64_t n) {
+    ORC_CVT_LOOP(orc_nibble_set(out, i, orc_f32_to_e2m1(in[i])))
+}
+void oracle_e2m1_to_f32(const uint8_t *in, float *out, int64_t n) {
+    ORC_CVT_LOOP(out[i] = orc_e2m1_to_f32(orc_nibble_get(in, i)))
+}
+void oracle_s4_to_f32(const uint8_t *in, float *out, int64_t n) {
+    ORC_CVT_LOOP(out[i] = (float)orc_s4_to_int(orc_nibble_get(in, i)))
+}
+void oracle_u4_to_f32(const uint8_t *in, float *out, int64_t n) {
+    ORC_CVT_LOOP(out[i] = (float)orc_nibble_get(in, i))
+}
+void oracle_store_float(int dt, const float *in, void *out, int64_t n) {
+    ORC_CVT_LOOP(orc_store_float(dt, in[i], out, i))
+}
+void oracle_load_float(int dt, const void *in, float *out, int64_t n) {
+    ORC_CVT_LOOP(out[i] = orc_load_float(dt, in, i))
+}
+void oracle_eltwise(int alg, float alpha, float beta, const float *in,
+        float *out, int64_t n) {
+    ORC_CVT_LOOP(out[i] = orc_eltwise(alg, in[i], alpha, beta))
+}
+void oracle_binary(int alg, const float *x, const float *y, float *out,
+        int64_t n) {
+    ORC_CVT_LOOP(out[i] = orc_binary(alg, x[i], y[i]))
+}

@@ -1,0 +1,33 @@
+import os
+import sys
+
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+
+def pytest_configure(config):
+    config.addinivalue_line("markers", "gpu: needs a real MI355X (run with -m gpu)")
+
+
+@pytest.fixture(scope="session")
+def oracle():
+    from oracle import binding
+    binding.load()
+    return binding
+
+
+@pytest.fixture(scope="session")
+def gpu():
+    """The C-ABI kernel library with a visible device; fails loudly, never
+    falls back to a CPU path."""
+    from onednn_amd import cabi
+    lib = cabi.load_kernels()
+    import ctypes as C
+    n = C.c_int(0)
+    cabi.check(lib.mi355_device_count(C.byref(n)))
+    assert n.value > 0, "no HIP device visible"
+    cabi.check(lib.mi355_device_set(0))
+    return lib
