@@ -105,11 +105,12 @@ def load_kernels():
     global _lib
     if _lib is not None:
         return _lib
-    if not os.path.exists(KERNEL_LIB_PATH):
+    path = os.environ.get("MI355_KERNEL_LIB", KERNEL_LIB_PATH)
+    if not os.path.exists(path):
         raise ImportError(
-            f"{KERNEL_LIB_PATH} is missing: build it with `make -C onednn_amd/csrc` "
+            f"{path} is missing: build it with `make -C onednn_amd/csrc` "
             "(or __graft_entry__.build()); there is no fallback path")
-    lib = C.CDLL(KERNEL_LIB_PATH)
+    lib = C.CDLL(path)
     vp = C.c_void_p
     lib.mi355_last_error.restype = C.c_char_p
     lib.mi355_matmul_impl_name.restype = C.c_char_p

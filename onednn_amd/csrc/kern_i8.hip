@@ -12,24 +12,15 @@
 //     with s' = src - off_s, w' = wei - off_w the bytes re-biased to s8
 //     (off = 128 for u8, 0 for s8), a = off_s - zs, c[n] = off_w - zw[n];
 //   d = (float)acc * src_scale * wei_scale[n]  -> shared epilogue.
-#include "kernels.hpp"
+#include "gemm_core.hpp"
 
 namespace mi355 {
 
-typedef int v4i __attribute__((ext_vector_type(4)));
-typedef int v16i __attribute__((ext_vector_type(16)));
-
 namespace {
 
-constexpr int BM = 256, BN = 256, BK = 64;
-constexpr int NT = 256;
-
-// byte offset of 16-byte chunk `chunk` (0..3) of tile row `row`; the chunk
-// index is XOR-swizzled with the row so that the 32 rows an MFMA operand read
-// touches spread over all LDS banks
-__device__ __forceinline__ int swz(int row, int chunk) {
-    return row * BK + ((chunk ^ ((row >> 1) & 3)) << 4);
-}
+using namespace gemm;
+constexpr int BK = BKB;       // int8: one byte per K element
+constexpr int NSTAGE = 4;     // 4 x 32 KB LDS ring
 
 struct i8_extra_t {
     const int8_t *bt; // weights as [N][K] bytes, K contiguous
@@ -37,54 +28,70 @@ struct i8_extra_t {
     long bt_bstride;  // bytes between batches (0 = broadcast)
     const int *colsum; // [Bw][N] sum_k w'  (null when a == 0)
     const int *rowsum; // [Bs][M] sum_k s'  (null when c == 0)
-    int src_u8, wei_u8;
     int tiles_m, tiles_n;
 };
 
+struct i8_ctx_t {};
+
+// v_mfma_i32_32x32x32_i8: lane l supplies row l%32, K bytes 16*(l/32)..+16
+template <bool SRC_U8, bool WEI_U8>
+struct i8_mma_t {
+    __device__ static __forceinline__ void stage(v16i (&acc)[4][4], const char *As, const char *Bs,
+            int wm, int wn, int lane, int, const i8_ctx_t &) {
+        const int frow = lane & 31, fch = lane >> 5;
+#pragma unroll
+        for (int kh = 0; kh < 2; ++kh) {
+            v4i fa[4], fb[4];
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                fa[i] = *(const v4i *)&As[swz(wm * 128 + i * 32 + frow, kh * 2 + fch)];
+                fb[i] = *(const v4i *)&Bs[swz(wn * 128 + i * 32 + frow, kh * 2 + fch)];
+                if (SRC_U8) fa[i] ^= (int)0x80808080;
+                if (WEI_U8) fb[i] ^= (int)0x80808080;
+            }
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+#pragma unroll
+                for (int j = 0; j < 4; ++j)
+                    acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fa[i], fb[j], acc[i][j], 0, 0, 0);
+        }
+    }
+};
+
+// raw s32 accumulator -> f32 entering the shared epilogue
+struct i8_conv_t {
+    int col_corr[4], c_c[4];
+    float wsc[4], ssc;
+    bool with_src_sc, with_wei_sc;
+    const int *rowsum; // already offset to this batch, or null
+    __device__ __forceinline__ void row(const v4i &raw, long m, float (&f)[4]) const {
+        const int rs = rowsum ? rowsum[m] : 0;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            const int v = raw[e] + col_corr[e] + c_c[e] * rs;
+            float x = (float)v;
+            if (with_src_sc) x *= ssc;
+            if (with_wei_sc) x *= wsc[e];
+            f[e] = x;
+        }
+    }
+};
+
+extern __shared__ __attribute__((aligned(16))) char i8_smem[];
+
+template <bool SRC_U8, bool WEI_U8>
 __global__ void __launch_bounds__(NT) i8_gemm_kernel(const problem_t P_, const i8_extra_t X) {
     const auto &P = MI355_KERNARG_PROBLEM();
-    __shared__ __attribute__((aligned(16))) char smem[2][2][BM * BK];
-
+    char *smem = i8_smem;
     const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
     const int wm = wave >> 1, wn = wave & 1;
     const long b = blockIdx.z;
+    const tile_pos_t tp = tile_position(X.tiles_m, X.tiles_n);
+    const long m0 = tp.m0, n0 = tp.n0;
 
-    // XCD-aware tile order: consecutive workgroup ids go to different XCDs, so
-    // give each XCD a contiguous run of tiles, walked in bands of 8 tile rows.
-    int tile;
-    {
-        const int nwg = gridDim.x, id = blockIdx.x;
-        const int per = nwg / 8;
-        tile = (nwg % 8 == 0) ? (id % 8) * per + id / 8 : id;
-    }
-    constexpr int GM = 8;
-    const int band = tile / (GM * X.tiles_n);
-    const int band_rows = min(GM, X.tiles_m - band * GM);
-    const int in_band = tile - band * GM * X.tiles_n;
-    const int tm = band * GM + in_band % band_rows;
-    const int tn = in_band / band_rows;
-    const long m0 = (long)tm * BM, n0 = (long)tn * BN;
-
-    const int8_t *A = (const int8_t *)P.src + (P.ss[0] ? b * P.ss[0] : 0);
     const long lda = P.ss[1];
-    const int8_t *Bt = X.bt + b * X.bt_bstride;
-    const long ldb = X.ldb;
-
-    // global -> register staging: 4 + 4 chunks of 16 bytes per thread
-    const int lrow = t >> 2, lchunk = t & 3;
-    const int8_t *ga[4], *gb[4];
-    int soff[4];
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-        const int row = lrow + i * 64;
-        long ar = m0 + row;
-        if (ar > P.M - 1) ar = P.M - 1;
-        long br = n0 + row;
-        if (br > P.N - 1) br = P.N - 1;
-        ga[i] = A + ar * lda + lchunk * 16;
-        gb[i] = Bt + br * ldb + lchunk * 16;
-        soff[i] = swz(row, lchunk);
-    }
+    const char *A = (const char *)P.src + (P.ss[0] ? b * P.ss[0] : 0) + m0 * lda;
+    const char *Bt = (const char *)X.bt + b * X.bt_bstride + n0 * X.ldb;
 
     v16i acc[4][4];
 #pragma unroll
@@ -94,126 +101,51 @@ __global__ void __launch_bounds__(NT) i8_gemm_kernel(const problem_t P_, const i
 #pragma unroll
             for (int r = 0; r < 16; ++r) acc[i][j][r] = 0;
 
-    const int nk = (int)(P.K / BK);
-    v4i ra[4], rb[4];
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-        ra[i] = *(const v4i *)(ga[i]);
-        rb[i] = *(const v4i *)(gb[i]);
-    }
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-        *(v4i *)&smem[0][0][soff[i]] = ra[i];
-        *(v4i *)&smem[0][1][soff[i]] = rb[i];
-    }
-    __syncthreads();
+    main_loop<NSTAGE, i8_mma_t<SRC_U8, WEI_U8>>(acc, smem, A, Bt, lda, X.ldb, P.M - m0, P.N - n0,
+            (int)(P.K / BK), i8_ctx_t {});
 
-    const int frow = lane & 31, fch = lane >> 5;
-    const int xa = X.src_u8 ? (int)0x80808080 : 0, xb = X.wei_u8 ? (int)0x80808080 : 0;
-
-    for (int kt = 0; kt < nk; ++kt) {
-        const int cur = kt & 1;
-        if (kt + 1 < nk) {
-            const long ko = (long)(kt + 1) * BK;
-#pragma unroll
-            for (int i = 0; i < 4; ++i) {
-                ra[i] = *(const v4i *)(ga[i] + ko);
-                rb[i] = *(const v4i *)(gb[i] + ko);
-            }
-        }
-        const char *As = smem[cur][0], *Bs = smem[cur][1];
-#pragma unroll
-        for (int kh = 0; kh < 2; ++kh) {
-            v4i fa[4], fb[4];
-#pragma unroll
-            for (int i = 0; i < 4; ++i) {
-                fa[i] = *(const v4i *)&As[swz(wm * 128 + i * 32 + frow, kh * 2 + fch)];
-                fb[i] = *(const v4i *)&Bs[swz(wn * 128 + i * 32 + frow, kh * 2 + fch)];
-                fa[i] ^= xa;
-                fb[i] ^= xb;
-            }
-#pragma unroll
-            for (int i = 0; i < 4; ++i)
-#pragma unroll
-                for (int j = 0; j < 4; ++j)
-                    acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fa[i], fb[j], acc[i][j], 0, 0, 0);
-        }
-        if (kt + 1 < nk) {
-#pragma unroll
-            for (int i = 0; i < 4; ++i) {
-                *(v4i *)&smem[cur ^ 1][0][soff[i]] = ra[i];
-                *(v4i *)&smem[cur ^ 1][1][soff[i]] = rb[i];
-            }
-        }
-        __syncthreads();
-    }
-
-    // ---- epilogue: s32 compensation, scales, shared tail.
-    // Accumulators go through LDS one 32-row slab at a time so that each lane
-    // ends up with four consecutive n of one row: the per-element epilogue
-    // code exists once (a rolled loop) and dst leaves in wide coalesced stores.
+    // ---- epilogue: s32 compensation, scales, shared tail
     const long bs = P.ss[0] ? b : 0, bw = P.ws[0] ? b : 0;
-    const int off_s = X.src_u8 ? 128 : 0, off_w = X.wei_u8 ? 128 : 0;
+    const int off_s = SRC_U8 ? 128 : 0, off_w = WEI_U8 ? 128 : 0;
     int a_c = off_s;
     if (P.src_zp.dt != MI355_DT_UNDEF) a_c -= load_int(P.src_zp.dt, P.src_zp.p, 0);
-    const bool with_src_sc = P.src_scale.dt != MI355_DT_UNDEF;
-    const bool with_wei_sc = P.wei_scale.dt != MI355_DT_UNDEF;
-    const float ssc = with_src_sc ? load_float(P.src_scale.dt, P.src_scale.p, 0) : 1.f;
+    i8_conv_t cv;
+    cv.with_src_sc = P.src_scale.dt != MI355_DT_UNDEF;
+    cv.with_wei_sc = P.wei_scale.dt != MI355_DT_UNDEF;
+    cv.ssc = cv.with_src_sc ? load_float(P.src_scale.dt, P.src_scale.p, 0) : 1.f;
+    cv.rowsum = X.rowsum ? X.rowsum + bs * P.M : nullptr;
     const int Kc = (int)P.K;
-
     const long nbase = n0 + wn * 128 + (lane & 31) * 4;
-    int col_corr[4], c_c[4];
-    float wsc[4];
-    int nvalid = 0;
 #pragma unroll
     for (int e = 0; e < 4; ++e) {
         const long n = nbase + e;
-        col_corr[e] = 0; c_c[e] = 0; wsc[e] = 1.f;
+        cv.col_corr[e] = 0; cv.c_c[e] = 0; cv.wsc[e] = 1.f;
         if (n < P.N) {
-            nvalid = e + 1;
             int c = off_w;
             if (P.wei_zp.dt != MI355_DT_UNDEF)
                 c -= load_int(P.wei_zp.dt, P.wei_zp.p, quant_off(P.wei_zp, bw, 0, n, P.K, P.N));
-            c_c[e] = c;
-            col_corr[e] = (a_c != 0 ? a_c * X.colsum[bw * P.N + n] : 0) + Kc * a_c * c;
-            if (with_wei_sc)
-                wsc[e] = load_float(P.wei_scale.dt, P.wei_scale.p,
+            cv.c_c[e] = c;
+            cv.col_corr[e] = (a_c != 0 ? a_c * X.colsum[bw * P.N + n] : 0) + Kc * a_c * c;
+            if (cv.with_wei_sc)
+                cv.wsc[e] = load_float(P.wei_scale.dt, P.wei_scale.p,
                         quant_off(P.wei_scale, bw, 0, n, P.K, P.N));
         }
     }
-    const bool any_c = X.rowsum != nullptr;
-
-    int *wl = (int *)&smem[0][0][0] + wave * 4096; // 16 KB per wave
-    auto slab = [&](const v16i (&a)[4], const int i) {
+    const bool interior = m0 + BM <= P.M && n0 + BN <= P.N;
+#ifndef MI355_DBG_NO_EPI
+    store_quadrant(P, smem, acc, b, m0 + wm * 128, n0 + wn * 128, interior, cv);
+#else
+    {
+        int sacc = 0;
 #pragma unroll
-        for (int j = 0; j < 4; ++j)
+        for (int i = 0; i < 4; ++i)
 #pragma unroll
-            for (int r = 0; r < 16; ++r)
-                wl[((r >> 2) * 8 + (lane >> 5) * 4 + (r & 3)) * 128 + j * 32 + (lane & 31)] = a[j][r];
-#pragma unroll 1
-        for (int it = 0; it < 16; ++it) {
-            const int row = it * 2 + (lane >> 5);
-            const long m = m0 + wm * 128 + i * 32 + row;
-            const v4i raw = *(const v4i *)&wl[row * 128 + (lane & 31) * 4];
-            if (m < P.M && nvalid > 0) {
-                const int rs = any_c ? X.rowsum[bs * P.M + m] : 0;
-                float f[4];
+            for (int j = 0; j < 4; ++j)
 #pragma unroll
-                for (int e = 0; e < 4; ++e) {
-                    const int v = raw[e] + col_corr[e] + c_c[e] * rs;
-                    float x = (float)v;
-                    if (with_src_sc) x *= ssc;
-                    if (with_wei_sc) x *= wsc[e];
-                    f[e] = x;
-                }
-                epilogue_store4(P, f, b, m, nbase, nvalid);
-            }
-        }
-    };
-    slab(acc[0], 0);
-    slab(acc[1], 1);
-    slab(acc[2], 2);
-    slab(acc[3], 3);
+                for (int r = 0; r < 16; ++r) sacc += acc[i][j][r];
+        if (sacc == 123456789) ((int *)P.dst)[0] = cv.col_corr[0] + interior;
+    }
+#endif
 }
 
 // out[r] = sum_k (bytes[r][k] ^ flip) as signed bytes; one wave per row
@@ -325,8 +257,7 @@ int i8_launch(const mi355_matmul_desc_t &d, const problem_t &P, void *scratch,
     }
     char *sc = (char *)scratch;
     i8_extra_t X {};
-    X.src_u8 = d.src_dt == MI355_DT_U8;
-    X.wei_u8 = d.wei_dt == MI355_DT_U8;
+    const bool src_u8 = d.src_dt == MI355_DT_U8, wei_u8 = d.wei_dt == MI355_DT_U8;
     if (plan.need_transpose) {
         uint8_t *bt = (uint8_t *)(sc + plan.off_bt);
         dim3 grid((unsigned)((d.N + 63) / 64), (unsigned)((d.K + 63) / 64), (unsigned)plan.Bw);
@@ -346,7 +277,7 @@ int i8_launch(const mi355_matmul_desc_t &d, const problem_t &P, void *scratch,
         for (long b = 0; b < plan.Bw; ++b)
             hipLaunchKernelGGL(i8_rowsum_kernel, dim3((unsigned)((d.N + 3) / 4)), dim3(256), 0,
                     stream, X.bt + b * X.bt_bstride, d.N, d.K, X.ldb,
-                    X.wei_u8 ? (int)0x80808080 : 0, cs + b * d.N);
+                    wei_u8 ? (int)0x80808080 : 0, cs + b * d.N);
         X.colsum = cs;
     }
     if (plan.need_rowsum) {
@@ -354,14 +285,31 @@ int i8_launch(const mi355_matmul_desc_t &d, const problem_t &P, void *scratch,
         for (long b = 0; b < plan.Bs; ++b)
             hipLaunchKernelGGL(i8_rowsum_kernel, dim3((unsigned)((d.M + 3) / 4)), dim3(256), 0,
                     stream, (const int8_t *)P.src + b * d.src_stride[0], d.M, d.K,
-                    d.src_stride[1], X.src_u8 ? (int)0x80808080 : 0, rs + b * d.M);
+                    d.src_stride[1], src_u8 ? (int)0x80808080 : 0, rs + b * d.M);
         X.rowsum = rs;
     }
     X.tiles_m = (int)((d.M + BM - 1) / BM);
     X.tiles_n = (int)((d.N + BN - 1) / BN);
     dim3 grid((unsigned)(X.tiles_m * X.tiles_n), 1, (unsigned)d.batch);
-    hipLaunchKernelGGL(i8_gemm_kernel, grid, dim3(NT), 0, stream, P, X);
-    return hipGetLastError() == hipSuccess ? MI355_SUCCESS : MI355_RUNTIME_ERROR;
+    constexpr int smem_bytes = NSTAGE * STAGE_BYTES;
+    const bool su = d.src_dt == MI355_DT_U8, wu = d.wei_dt == MI355_DT_U8;
+    auto go = [&](auto kern) {
+        static bool attr_done = false; // per instantiation
+        if (!attr_done) {
+            if (hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize,
+                        smem_bytes) != hipSuccess) {
+                set_error("mfma_i8: cannot reserve %d bytes of LDS", smem_bytes);
+                return MI355_RUNTIME_ERROR;
+            }
+            attr_done = true;
+        }
+        hipLaunchKernelGGL(kern, grid, dim3(NT), smem_bytes, stream, P, X);
+        return hipGetLastError() == hipSuccess ? MI355_SUCCESS : MI355_RUNTIME_ERROR;
+    };
+    if (su && wu) return go(i8_gemm_kernel<true, true>);
+    if (su) return go(i8_gemm_kernel<true, false>);
+    if (wu) return go(i8_gemm_kernel<false, true>);
+    return go(i8_gemm_kernel<false, false>);
 }
 
 } // namespace mi355

@@ -260,47 +260,4 @@ __device__ __forceinline__ void epilogue_store(
     store_float(P.dst_dt, v, P.dst, b * P.ds[0] + m * P.ds[1] + n * P.ds[2]);
 }
 
-// Store four consecutive-n results of one dst row.  When dst is dense along n
-// and the address is aligned the four values leave as one 4/8/16-byte store.
-template <class PT>
-__device__ __forceinline__ void epilogue_store4(const PT &P, const float (&f)[4],
-        long b, long m, long n, int nvalid) {
-    float v[4];
-#pragma unroll
-    for (int e = 0; e < 4; ++e) v[e] = (e < nvalid) ? epilogue_value(P, f[e], b, m, n + e) : 0.f;
-    const long off = b * P.ds[0] + m * P.ds[1] + n * P.ds[2];
-    const int bits = dt_bits(P.dst_dt);
-    if (nvalid == 4 && P.ds[2] == 1) {
-        uint32_t w[4];
-#pragma unroll
-        for (int e = 0; e < 4; ++e) w[e] = cvt_store_bits(P.dst_dt, v[e]);
-        if (bits == 8) {
-            uint8_t *p = (uint8_t *)P.dst + off;
-            if (((uintptr_t)p & 3) == 0) {
-                *(uint32_t *)p = w[0] | (w[1] << 8) | (w[2] << 16) | (w[3] << 24);
-                return;
-            }
-        } else if (bits == 16) {
-            uint16_t *p = (uint16_t *)P.dst + off;
-            if (((uintptr_t)p & 7) == 0) {
-                uint2 o;
-                o.x = w[0] | (w[1] << 16);
-                o.y = w[2] | (w[3] << 16);
-                *(uint2 *)p = o;
-                return;
-            }
-        } else {
-            uint32_t *p = (uint32_t *)P.dst + off;
-            if (((uintptr_t)p & 15) == 0) {
-                uint4 o;
-                o.x = w[0]; o.y = w[1]; o.z = w[2]; o.w = w[3];
-                *(uint4 *)p = o;
-                return;
-            }
-        }
-    }
-    for (int e = 0; e < nvalid; ++e)
-        store_float(P.dst_dt, v[e], P.dst, off + e * P.ds[2]);
-}
-
 } // namespace mi355

@@ -1,0 +1,467 @@
+// Epilogue of the LDS-tiled MFMA kernels.
+//
+// After the K loop every wavefront owns a 128x128 quadrant in accumulator
+// registers (16 tiles of 32x32).  It leaves through LDS in four 32-row slabs;
+// afterwards each lane owns four consecutive n of one row, so dst goes out in
+// coalesced 4/8/16-byte stores and the per-element epilogue code exists once,
+// in a rolled loop over the 16 row pairs of a slab.
+//
+// With one wavefront per SIMD nothing hides memory latency inside that loop,
+// so every operand that does not depend on the row is loaded once per lane
+// before it (dst scale, dst zero points, per-n bias, one per-n binary
+// operand), and one per-element operand stream (the src1 tensor of a binary
+// post-op, the old dst of a sum post-op, or a per-element bias) is prefetched
+// a whole slab ahead into an LDS staging area with 16 loads in flight.
+// Anything beyond that is still computed exactly, with loads inside the loop.
+//
+// Order of operations: ref_matmul_int8.cpp:275-306 / ref_matmul.cpp:283-331.
+#pragma once
+#include "mi355_device.hpp"
+
+namespace mi355 {
+namespace gemm {
+
+typedef int v4i_t __attribute__((ext_vector_type(4)));
+
+__device__ __forceinline__ int raw_bits(int x) { return x; }
+__device__ __forceinline__ int raw_bits(float x) { return __float_as_int(x); }
+
+constexpr int STG_NONE = -1, STG_BIAS = 100, STG_SUM = 101;
+
+struct po_reg_t {
+    int kind, alg;
+    float alpha, beta, scale, zpf;
+};
+
+struct epi_hoist_t {
+    float bias4[4];
+    float hv4[4];   // hoisted per-n operand of post-op `hoisted_po`
+    float dzp4[4];
+    float ds, ds_inv;
+    int bias_mode;  // 0 none, 1 hoisted, 2 per element
+    int ds_mode;    // 0 none, 1 divide, 2 multiply by reciprocal
+    int dzp_mode;   // 0 none, 1 present
+    int hoisted_po; // post-op index or -1
+    int staged;     // STG_NONE, STG_BIAS, STG_SUM or a binary post-op index
+    int staged_dt;
+    const char *staged_p;
+    long st_s0, st_s1; // element strides of the staged stream (stride along n is 1)
+    // the leading "simple" post-ops (at most three), resident in registers
+    po_reg_t pf0, pf1, pf2;
+    int nfast; // how many of them; the rest run through the generic loop
+    int n_po;
+    int dst_dt, dst_vec; // dst_vec: four consecutive n leave as one aligned store
+};
+
+__device__ __forceinline__ bool vec_ok(const void *p, long s0, long s1, int bits) {
+    // four consecutive elements must form one aligned 8- or 16-byte vector
+    const int bytes4 = bits / 2;
+    return (bits == 16 || bits == 32) && (((uintptr_t)p) % bytes4) == 0 && (s0 % 4) == 0
+            && (s1 % 4) == 0;
+}
+
+__device__ __forceinline__ bool vec_ok_store(const void *p, long s0, long s1, int bits) {
+    const int bytes4 = bits / 2; // bytes of four elements
+    const long e4 = bits == 8 ? 4 : 4; // strides are in elements: need multiples of 4
+    return (bits == 8 || bits == 16 || bits == 32) && (((uintptr_t)p) % bytes4) == 0
+            && (s0 % e4) == 0 && (s1 % e4) == 0;
+}
+
+template <class PT>
+__device__ __forceinline__ epi_hoist_t make_hoist(const PT &P, long b, long nbase, int nvalid,
+        bool interior) {
+    epi_hoist_t H;
+    H.bias_mode = 0; H.ds_mode = 0; H.dzp_mode = 0; H.hoisted_po = -1; H.staged = STG_NONE;
+    H.staged_dt = 0; H.staged_p = nullptr; H.st_s0 = H.st_s1 = 0; H.ds = 1.f; H.ds_inv = 1.f;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) { H.bias4[e] = 0.f; H.hv4[e] = 0.f; H.dzp4[e] = 0.f; }
+    if (P.bias_dt != MI355_DT_UNDEF) {
+        if (P.bs[1] == 0) {
+            H.bias_mode = 1;
+#pragma unroll
+            for (int e = 0; e < 4; ++e)
+                if (e < nvalid) H.bias4[e] = load_float(P.bias_dt, P.bias, b * P.bs[0] + (nbase + e) * P.bs[2]);
+        } else {
+            H.bias_mode = 2;
+        }
+    }
+    if (P.dst_scale.dt != MI355_DT_UNDEF) {
+        H.ds = load_float(P.dst_scale.dt, P.dst_scale.p, 0);
+        H.ds_inv = 1.f / H.ds;
+        H.ds_mode = P.dst_scale_mode == MI355_DST_SCALE_RECIPROCAL ? 2 : 1;
+    }
+    if (P.dst_zp.dt != MI355_DT_UNDEF) {
+        H.dzp_mode = 1;
+#pragma unroll
+        for (int e = 0; e < 4; ++e)
+            if (e < nvalid)
+                H.dzp4[e] = (float)((const int *)P.dst_zp.p)[(P.dst_zp.mask & 4) ? nbase + e : 0];
+    }
+    H.n_po = P.n_po;
+    H.dst_dt = P.dst_dt;
+    H.dst_vec = P.ds[2] == 1 && vec_ok_store(P.dst, P.ds[0], P.ds[1], dt_bits(P.dst_dt));
+    {
+        auto grab = [&](int i, po_reg_t &r) -> bool {
+            r.kind = 0; r.alg = 0; r.alpha = r.beta = r.zpf = 0.f; r.scale = 1.f;
+            if (i >= P.n_po) return false;
+            r.kind = P.po[i].kind; r.alg = P.po[i].alg; r.alpha = P.po[i].alpha;
+            r.beta = P.po[i].beta; r.scale = P.po[i].scale; r.zpf = (float)P.po[i].zp;
+            const bool simple_elt = r.kind == MI355_PO_ELTWISE
+                    && (r.alg == MI355_ELTWISE_RELU || r.alg == MI355_ELTWISE_LINEAR
+                            || r.alg == MI355_ELTWISE_GELU_TANH || r.alg == MI355_ELTWISE_CLIP
+                            || r.alg == MI355_ELTWISE_CLIP_V2);
+            return simple_elt || r.kind == MI355_PO_BINARY || r.kind == MI355_PO_SUM;
+        };
+        H.nfast = 0;
+        if (grab(0, H.pf0)) {
+            H.nfast = 1;
+            if (grab(1, H.pf1)) {
+                H.nfast = 2;
+                if (grab(2, H.pf2)) H.nfast = 3;
+            } else {
+                grab(3 + MI355_MAX_POST_OPS, H.pf2);
+            }
+        } else {
+            grab(3 + MI355_MAX_POST_OPS, H.pf1);
+            grab(3 + MI355_MAX_POST_OPS, H.pf2);
+        }
+    }
+    int first_sum = -1;
+    for (int i = 0; i < P.n_po; ++i) {
+        const auto &po = P.po[i];
+        if (po.kind == MI355_PO_BINARY) {
+            if (po.s1 == 0 && H.hoisted_po < 0) {
+                H.hoisted_po = i;
+#pragma unroll
+                for (int e = 0; e < 4; ++e)
+                    if (e < nvalid) H.hv4[e] = load_float(po.dt, po.p, b * po.s0 + (nbase + e) * po.s2);
+            } else if (po.s1 != 0 && po.s2 == 1 && H.staged == STG_NONE && interior
+                    && vec_ok(po.p, po.s0, po.s1, dt_bits(po.dt))) {
+                H.staged = i; H.staged_dt = po.dt; H.staged_p = (const char *)po.p;
+                H.st_s0 = po.s0; H.st_s1 = po.s1;
+            }
+        } else if (po.kind == MI355_PO_SUM && first_sum < 0) {
+            first_sum = i;
+        }
+    }
+    if (H.staged == STG_NONE && interior && first_sum >= 0 && P.ds[2] == 1
+            && vec_ok(P.dst, P.ds[0], P.ds[1], dt_bits(P.sum_dt))) {
+        H.staged = STG_SUM; H.staged_dt = P.sum_dt; H.staged_p = (const char *)P.dst;
+        H.st_s0 = P.ds[0]; H.st_s1 = P.ds[1];
+    }
+    if (H.staged == STG_NONE && interior && H.bias_mode == 2 && P.bs[2] == 1
+            && vec_ok(P.bias, P.bs[0], P.bs[1], dt_bits(P.bias_dt))) {
+        H.staged = STG_BIAS; H.staged_dt = P.bias_dt; H.staged_p = (const char *)P.bias;
+        H.st_s0 = P.bs[0]; H.st_s1 = P.bs[1];
+    }
+    return H;
+}
+
+// decode four packed 16- or 32-bit values (one dispatch for the four)
+__device__ __forceinline__ void staged4(int dt, const uint4 &raw, float (&y)[4]) {
+    const uint32_t w[4] = {raw.x, raw.y, raw.z, raw.w};
+    switch (dt) {
+        case MI355_DT_BF16:
+#pragma unroll
+            for (int e = 0; e < 4; ++e) y[e] = u2f((w[e >> 1] >> ((e & 1) * 16)) << 16);
+            break;
+        case MI355_DT_F16:
+#pragma unroll
+            for (int e = 0; e < 4; ++e) y[e] = f16_to_f32((uint16_t)(w[e >> 1] >> ((e & 1) * 16)));
+            break;
+        case MI355_DT_F32:
+#pragma unroll
+            for (int e = 0; e < 4; ++e) y[e] = u2f(w[e]);
+            break;
+        default: // s32
+#pragma unroll
+            for (int e = 0; e < 4; ++e) y[e] = (float)(int)w[e];
+            break;
+    }
+}
+
+// eltwise on four values: one dispatch, four bodies (the cheap algorithms)
+__device__ __forceinline__ void eltwise4_simple(int alg, float (&v)[4], float alpha, float beta,
+        float scale) {
+    if (alg == MI355_ELTWISE_RELU) {
+#pragma unroll
+        for (int e = 0; e < 4; ++e) v[e] = (v[e] > 0 ? v[e] : v[e] * alpha) * scale;
+    } else if (alg == MI355_ELTWISE_LINEAR) {
+#pragma unroll
+        for (int e = 0; e < 4; ++e) v[e] = (alpha * v[e] + beta) * scale;
+    } else if (alg == MI355_ELTWISE_GELU_TANH) {
+#pragma unroll
+        for (int e = 0; e < 4; ++e) v[e] = eltwise_f(MI355_ELTWISE_GELU_TANH, v[e], alpha, beta) * scale;
+    } else if (alg == MI355_ELTWISE_CLIP) {
+#pragma unroll
+        for (int e = 0; e < 4; ++e) v[e] = eltwise_f(MI355_ELTWISE_CLIP, v[e], alpha, beta) * scale;
+    } else {
+#pragma unroll
+        for (int e = 0; e < 4; ++e) v[e] = eltwise_f(MI355_ELTWISE_CLIP_V2, v[e], alpha, beta) * scale;
+    }
+}
+
+// every eltwise algorithm, one copy of the long-tail code (rolled over the
+// four values; selects of values, not of addresses)
+__device__ __forceinline__ void eltwise4_any(int alg, float (&v)[4], float alpha, float beta,
+        float scale) {
+    float v0 = v[0], v1 = v[1], v2 = v[2], v3 = v[3];
+#pragma unroll 1
+    for (int e = 0; e < 4; ++e) {
+        const float x = e == 0 ? v0 : e == 1 ? v1 : e == 2 ? v2 : v3;
+        const float y = eltwise_f(alg, x, alpha, beta) * scale;
+        if (e == 0) v0 = y;
+        else if (e == 1) v1 = y;
+        else if (e == 2) v2 = y;
+        else v3 = y;
+    }
+    v[0] = v0; v[1] = v1; v[2] = v2; v[3] = v3;
+}
+
+template <class PT>
+__device__ __forceinline__ void apply_epilogue4(const PT &P, const epi_hoist_t &H, float (&v)[4],
+        long b, long m, long nbase, int nvalid, const uint4 &stg) {
+    float sy[4] = {0.f, 0.f, 0.f, 0.f};
+    if (H.staged != STG_NONE) staged4(H.staged_dt, stg, sy);
+    if (H.bias_mode == 1) {
+#pragma unroll
+        for (int e = 0; e < 4; ++e) v[e] += H.bias4[e];
+    } else if (H.bias_mode == 2) {
+        if (H.staged == STG_BIAS) {
+#pragma unroll
+            for (int e = 0; e < 4; ++e) v[e] += sy[e];
+        } else {
+#pragma unroll
+            for (int e = 0; e < 4; ++e)
+                if (e < nvalid)
+                    v[e] += load_float(P.bias_dt, P.bias, b * P.bs[0] + m * P.bs[1] + (nbase + e) * P.bs[2]);
+        }
+    }
+    if (H.n_po > 0) {
+        float dst_old[4] = {0.f, 0.f, 0.f, 0.f};
+        if (P.sum_dt != MI355_DT_UNDEF) {
+            if (H.staged == STG_SUM) {
+#pragma unroll
+                for (int e = 0; e < 4; ++e) dst_old[e] = sy[e];
+            } else {
+#pragma unroll
+                for (int e = 0; e < 4; ++e)
+                    if (e < nvalid)
+                        dst_old[e] = load_float(P.sum_dt, P.dst,
+                                b * P.ds[0] + m * P.ds[1] + (nbase + e) * P.ds[2]);
+            }
+        }
+        auto binary_operand = [&](int i, float (&y)[4]) {
+            if (i == H.hoisted_po) {
+#pragma unroll
+                for (int e = 0; e < 4; ++e) y[e] = H.hv4[e];
+            } else if (i == H.staged) {
+#pragma unroll
+                for (int e = 0; e < 4; ++e) y[e] = sy[e];
+            } else {
+                const auto &po = P.po[i];
+#pragma unroll
+                for (int e = 0; e < 4; ++e)
+                    y[e] = e < nvalid ? load_float(po.dt, po.p, b * po.s0 + m * po.s1 + (nbase + e) * po.s2)
+                                      : 0.f;
+            }
+        };
+        auto binary4 = [&](int alg, const float (&y)[4]) {
+            if (alg == MI355_BINARY_ADD) {
+#pragma unroll
+                for (int e = 0; e < 4; ++e) v[e] = v[e] + y[e];
+            } else if (alg == MI355_BINARY_MUL) {
+#pragma unroll
+                for (int e = 0; e < 4; ++e) v[e] = v[e] * y[e];
+            } else {
+#pragma unroll
+                for (int e = 0; e < 4; ++e) v[e] = binary_f(alg, v[e], y[e]);
+            }
+        };
+        auto fast_op = [&](const po_reg_t &r, int i) {
+            if (r.kind == MI355_PO_ELTWISE) {
+                eltwise4_simple(r.alg, v, r.alpha, r.beta, r.scale);
+            } else if (r.kind == MI355_PO_BINARY) {
+                float y[4];
+                binary_operand(i, y);
+                binary4(r.alg, y);
+            } else { // sum
+#pragma unroll
+                for (int e = 0; e < 4; ++e) v[e] += r.scale * (dst_old[e] - r.zpf);
+            }
+        };
+        if (H.nfast > 0) fast_op(H.pf0, 0);
+        if (H.nfast > 1) fast_op(H.pf1, 1);
+        if (H.nfast > 2) fast_op(H.pf2, 2);
+#pragma unroll 1
+        for (int i = H.nfast; i < H.n_po; ++i) {
+            const auto &po = P.po[i];
+            const int kind = po.kind;
+            if (kind == MI355_PO_ELTWISE) {
+                eltwise4_any(po.alg, v, po.alpha, po.beta, po.scale);
+            } else if (kind == MI355_PO_BINARY) {
+                float y[4];
+                binary_operand(i, y);
+                binary4(po.alg, y);
+            } else if (kind == MI355_PO_SUM) {
+                const float sc = po.scale, zpf = (float)po.zp;
+#pragma unroll
+                for (int e = 0; e < 4; ++e) v[e] += sc * (dst_old[e] - zpf);
+            } else if (kind == MI355_PO_PRELU) {
+#pragma unroll
+                for (int e = 0; e < 4; ++e)
+                    if (e < nvalid && !(v[e] >= 0))
+                        v[e] = ((const float *)po.p)[b * po.s0 + m * po.s1 + (nbase + e) * po.s2] * v[e];
+            }
+        }
+    }
+    if (H.ds_mode == 1) {
+#pragma unroll
+        for (int e = 0; e < 4; ++e) v[e] /= H.ds;
+    } else if (H.ds_mode == 2) {
+#pragma unroll
+        for (int e = 0; e < 4; ++e) v[e] *= H.ds_inv;
+    }
+    if (H.dzp_mode) {
+#pragma unroll
+        for (int e = 0; e < 4; ++e) v[e] += H.dzp4[e];
+    }
+}
+
+// convert four values to the dst type: one dispatch for the four
+__device__ __forceinline__ void cvt4(int dt, const float (&v)[4], uint32_t (&w)[4]) {
+    switch (dt) {
+        case MI355_DT_S8:
+#pragma unroll
+            for (int e = 0; e < 4; ++e) w[e] = (uint32_t)(int)__builtin_rintf(sat(v[e], -128.f, 127.f)) & 0xffu;
+            break;
+        case MI355_DT_U8:
+#pragma unroll
+            for (int e = 0; e < 4; ++e) w[e] = (uint32_t)(int)__builtin_rintf(sat(v[e], 0.f, 255.f)) & 0xffu;
+            break;
+        case MI355_DT_BF16:
+#pragma unroll
+            for (int e = 0; e < 4; ++e) w[e] = f32_to_bf16(v[e]);
+            break;
+        case MI355_DT_F32:
+#pragma unroll
+            for (int e = 0; e < 4; ++e) w[e] = f2u(v[e]);
+            break;
+        case MI355_DT_S32:
+#pragma unroll
+            for (int e = 0; e < 4; ++e)
+                w[e] = (uint32_t)(int)__builtin_rintf(sat(v[e], -2147483648.f, 2147483520.f));
+            break;
+        default:
+#pragma unroll
+            for (int e = 0; e < 4; ++e) w[e] = cvt_store_bits(dt, v[e]);
+            break;
+    }
+}
+
+template <class PT>
+__device__ __forceinline__ void store4(const PT &P, const epi_hoist_t &H, const float (&v)[4], long b,
+        long m, long n, int nvalid) {
+    const long off = b * P.ds[0] + m * P.ds[1] + n * P.ds[2];
+    uint32_t w[4];
+    cvt4(H.dst_dt, v, w);
+    const int bits = dt_bits(H.dst_dt);
+    if (nvalid == 4 && H.dst_vec) {
+        if (bits == 8) {
+            *(uint32_t *)((uint8_t *)P.dst + off) = w[0] | (w[1] << 8) | (w[2] << 16) | (w[3] << 24);
+        } else if (bits == 16) {
+            uint2 o;
+            o.x = w[0] | (w[1] << 16);
+            o.y = w[2] | (w[3] << 16);
+            *(uint2 *)((uint16_t *)P.dst + off) = o;
+        } else {
+            uint4 o;
+            o.x = w[0]; o.y = w[1]; o.z = w[2]; o.w = w[3];
+            *(uint4 *)((uint32_t *)P.dst + off) = o;
+        }
+        return;
+    }
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+        if (e < nvalid) {
+            const long o = off + e * P.ds[2];
+            if (bits == 8) ((uint8_t *)P.dst)[o] = (uint8_t)w[e];
+            else if (bits == 16) ((uint16_t *)P.dst)[o] = (uint16_t)w[e];
+            else ((uint32_t *)P.dst)[o] = w[e];
+        }
+    }
+}
+
+// `conv.row(raw, m, f)` turns four raw accumulators of row m into the f32
+// values that enter the epilogue.  32x32 MFMA accumulator layout: register r
+// of tile (i, j) holds row 8*(r/4) + 4*(lane/32) + r%4, column lane%32.
+// smem: >= 128 KB; [0, 64K) accumulator slabs, [64K, 128K) operand staging.
+template <class PT, class Raw16, class Conv>
+__device__ __forceinline__ void store_quadrant(const PT &P, char *smem, const Raw16 (&acc)[4][4],
+        long b, long m_base, long n_base_wave, bool interior, const Conv &conv) {
+    const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
+    int *wl = (int *)smem + wave * 4096;                    // 16 KB per wavefront
+    uint4 *stg = (uint4 *)(smem + 65536) + wave * 1024;     // 16 KB per wavefront
+    const long nbase = n_base_wave + (lane & 31) * 4;
+    int nvalid = 0;
+#pragma unroll
+    for (int e = 0; e < 4; ++e)
+        if (nbase + e < P.N) nvalid = e + 1;
+    const epi_hoist_t H = make_hoist(P, b, nbase, nvalid, interior);
+    const int sbytes = dt_bits(H.staged_dt) / 8;
+
+    auto write_slab = [&](const Raw16 (&a)[4]) {
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+#pragma unroll
+            for (int r = 0; r < 16; ++r)
+                wl[((r >> 2) * 8 + (lane >> 5) * 4 + (r & 3)) * 128 + j * 32 + (lane & 31)]
+                        = raw_bits(a[j][r]);
+    };
+
+    // rolled over the four slabs: the epilogue arithmetic exists once
+#pragma unroll 1
+    for (int i = 0; i < 4; ++i) {
+        if (H.staged != STG_NONE) {
+            // 16 independent vector loads in flight, then park them in LDS
+            uint4 tmp[16];
+            const char *base = H.staged_p
+                    + (b * H.st_s0 + (m_base + i * 32 + (lane >> 5)) * H.st_s1 + nbase) * sbytes;
+            if (sbytes == 2) {
+#pragma unroll
+                for (int it = 0; it < 16; ++it) {
+                    const uint2 q = *(const uint2 *)(base + (long)it * 2 * H.st_s1 * 2);
+                    tmp[it].x = q.x; tmp[it].y = q.y; tmp[it].z = 0; tmp[it].w = 0;
+                }
+            } else {
+#pragma unroll
+                for (int it = 0; it < 16; ++it) tmp[it] = *(const uint4 *)(base + (long)it * 2 * H.st_s1 * 4);
+            }
+#pragma unroll
+            for (int it = 0; it < 16; ++it) stg[it * 64 + lane] = tmp[it];
+        }
+        switch (i) {
+            case 0: write_slab(acc[0]); break;
+            case 1: write_slab(acc[1]); break;
+            case 2: write_slab(acc[2]); break;
+            default: write_slab(acc[3]); break;
+        }
+#pragma unroll 1
+        for (int it = 0; it < 16; ++it) {
+            const int row = it * 2 + (lane >> 5);
+            const long m = m_base + i * 32 + row;
+            const v4i_t raw = *(const v4i_t *)&wl[row * 128 + (lane & 31) * 4];
+            uint4 sv = make_uint4(0, 0, 0, 0);
+            if (H.staged != STG_NONE) sv = stg[it * 64 + lane];
+            if (m < P.M && nvalid > 0) {
+                float v[4];
+                conv.row(raw, m, v);
+                apply_epilogue4(P, H, v, b, m, nbase, nvalid, sv);
+                store4(P, H, v, b, m, nbase, nvalid);
+            }
+        }
+    }
+}
+
+} // namespace gemm
+} // namespace mi355
