@@ -120,8 +120,14 @@ __device__ __forceinline__ void issue_stage(const dma_plan_t &p, const char *a_b
     for (int i = 0; i < 4; ++i) dma16(b_base, p.voff_b[i], lds_stage + p.lds_b[i]);
 }
 
-// Main loop.  `Mma::stage(acc, As, Bs, wm, wn, lane, kt, mma_ctx)` consumes
-// one stage.  a_tile / b_tile point at the first K byte of tile row 0.
+// Main loop.  Per K step kt (ring slot kt % NSTAGE):
+//   s_waitcnt vmcnt(..)   own DMAs of stage kt landed
+//   s_barrier             everybody's did, and everybody finished stage kt-1
+//   DMA stage kt+NSTAGE-1 into the slot stage kt-1 used
+//   ds_read + MFMA over stage kt
+// `Mma` supplies frag_t, load(frag, As, Bs, wm, wn, lane, ctx, kt) and
+// mma(acc, frag, ctx, kt).  a_tile / b_tile point at the first K byte of tile
+// row 0.
 template <int NSTAGE, class Mma, class Acc, class Ctx>
 __device__ __forceinline__ void main_loop(Acc &acc, char *smem, const char *a_tile,
         const char *b_tile, long lda, long ldb, long rows_a_left, long rows_b_left, int nk,
@@ -154,8 +160,10 @@ __device__ __forceinline__ void main_loop(Acc &acc, char *smem, const char *a_ti
 #endif
         }
         const char *As = smem + slot * STAGE_BYTES;
+        typename Mma::frag_t f;
+        Mma::load(f, As, As + B_OFF, wm, wn, lane, ctx, kt);
 #ifndef MI355_DBG_NO_MMA
-        Mma::stage(acc, As, As + B_OFF, wm, wn, lane, kt, ctx);
+        Mma::mma(acc, f, ctx, kt);
 #endif
         if (++slot == NSTAGE) slot = 0;
     }

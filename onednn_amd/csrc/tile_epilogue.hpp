@@ -392,12 +392,59 @@ __device__ __forceinline__ void store4(const PT &P, const epi_hoist_t &H, const 
     }
 }
 
+// Accumulator layouts: how a wavefront's 128x128 quadrant sits in registers
+// and how one 32-row slab of it is written to LDS as [32 rows][128 cols] s32.
+//
+// 32x32 MFMA tiles, acc[4][4] of 16 registers: register r of tile (i, j) holds
+// row 32i + 8*(r/4) + 4*(lane/32) + r%4, column 32j + lane%32.
+struct layout32_t {
+    template <class Acc>
+    static __device__ __forceinline__ void write_slab(const Acc &acc, int s, int *wl, int lane) {
+        auto w = [&](const auto &a) {
+#pragma unroll
+            for (int j = 0; j < 4; ++j)
+#pragma unroll
+                for (int r = 0; r < 16; ++r)
+                    wl[((r >> 2) * 8 + (lane >> 5) * 4 + (r & 3)) * 128 + j * 32 + (lane & 31)]
+                            = raw_bits(a[j][r]);
+        };
+        switch (s) {
+            case 0: w(acc[0]); break;
+            case 1: w(acc[1]); break;
+            case 2: w(acc[2]); break;
+            default: w(acc[3]); break;
+        }
+    }
+};
+
+// 16x16 MFMA tiles, acc[8][8] of 4 registers: register r of tile (i, j) holds
+// row 16i + 4*(lane/16) + r, column 16j + lane%16.
+struct layout16_t {
+    template <class Acc>
+    static __device__ __forceinline__ void write_slab(const Acc &acc, int s, int *wl, int lane) {
+        auto w = [&](const auto &a0, const auto &a1) {
+#pragma unroll
+            for (int j = 0; j < 8; ++j)
+#pragma unroll
+                for (int r = 0; r < 4; ++r) {
+                    wl[((lane >> 4) * 4 + r) * 128 + j * 16 + (lane & 15)] = raw_bits(a0[j][r]);
+                    wl[(16 + (lane >> 4) * 4 + r) * 128 + j * 16 + (lane & 15)] = raw_bits(a1[j][r]);
+                }
+        };
+        switch (s) {
+            case 0: w(acc[0], acc[1]); break;
+            case 1: w(acc[2], acc[3]); break;
+            case 2: w(acc[4], acc[5]); break;
+            default: w(acc[6], acc[7]); break;
+        }
+    }
+};
+
 // `conv.row(raw, m, f)` turns four raw accumulators of row m into the f32
-// values that enter the epilogue.  32x32 MFMA accumulator layout: register r
-// of tile (i, j) holds row 8*(r/4) + 4*(lane/32) + r%4, column lane%32.
+// values that enter the epilogue.
 // smem: >= 128 KB; [0, 64K) accumulator slabs, [64K, 128K) operand staging.
-template <class PT, class Raw16, class Conv>
-__device__ __forceinline__ void store_quadrant(const PT &P, char *smem, const Raw16 (&acc)[4][4],
+template <class Layout, class PT, class Acc, class Conv>
+__device__ __forceinline__ void store_quadrant(const PT &P, char *smem, const Acc &acc,
         long b, long m_base, long n_base_wave, bool interior, const Conv &conv) {
     const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
     int *wl = (int *)smem + wave * 4096;                    // 16 KB per wavefront
@@ -409,15 +456,6 @@ __device__ __forceinline__ void store_quadrant(const PT &P, char *smem, const Ra
         if (nbase + e < P.N) nvalid = e + 1;
     const epi_hoist_t H = make_hoist(P, b, nbase, nvalid, interior);
     const int sbytes = dt_bits(H.staged_dt) / 8;
-
-    auto write_slab = [&](const Raw16 (&a)[4]) {
-#pragma unroll
-        for (int j = 0; j < 4; ++j)
-#pragma unroll
-            for (int r = 0; r < 16; ++r)
-                wl[((r >> 2) * 8 + (lane >> 5) * 4 + (r & 3)) * 128 + j * 32 + (lane & 31)]
-                        = raw_bits(a[j][r]);
-    };
 
     // rolled over the four slabs: the epilogue arithmetic exists once
 #pragma unroll 1
@@ -440,12 +478,7 @@ __device__ __forceinline__ void store_quadrant(const PT &P, char *smem, const Ra
 #pragma unroll
             for (int it = 0; it < 16; ++it) stg[it * 64 + lane] = tmp[it];
         }
-        switch (i) {
-            case 0: write_slab(acc[0]); break;
-            case 1: write_slab(acc[1]); break;
-            case 2: write_slab(acc[2]); break;
-            default: write_slab(acc[3]); break;
-        }
+        Layout::write_slab(acc, i, wl, lane);
 #pragma unroll 1
         for (int it = 0; it < 16; ++it) {
             const int row = it * 2 + (lane >> 5);
