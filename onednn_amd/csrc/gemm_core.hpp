@@ -50,6 +50,14 @@ __device__ __forceinline__ int swz(int row, int chunk) {
     return row * BKB + ((chunk ^ swz_f(row)) << 4);
 }
 
+// 4 bytes per lane: LDS byte address lds_addr + 4*i
+__device__ __forceinline__ void dma4(const void *sbase, unsigned voff, unsigned lds_addr) {
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dword %1, %2"
+                 :
+                 : "s"(lds_addr), "v"(voff), "s"(sbase)
+                 : "memory", "m0");
+}
+
 // one wavefront-wide direct-to-LDS load: lane i brings 16 bytes from
 // sbase + voff to LDS byte address lds_addr + 16*i
 __device__ __forceinline__ void dma16(const void *sbase, unsigned voff, unsigned lds_addr) {
@@ -120,52 +128,67 @@ __device__ __forceinline__ void issue_stage(const dma_plan_t &p, const char *a_b
     for (int i = 0; i < 4; ++i) dma16(b_base, p.voff_b[i], lds_stage + p.lds_b[i]);
 }
 
-// Main loop.  Per K step kt (ring slot kt % NSTAGE):
-//   s_waitcnt vmcnt(..)   own DMAs of stage kt landed
-//   s_barrier             everybody's did, and everybody finished stage kt-1
-//   DMA stage kt+NSTAGE-1 into the slot stage kt-1 used
-//   ds_read + MFMA over stage kt
-// `Mma` supplies frag_t, load(frag, As, Bs, wm, wn, lane, ctx, kt) and
-// mma(acc, frag, ctx, kt).  a_tile / b_tile point at the first K byte of tile
-// row 0.
-template <int NSTAGE, class Mma, class Acc, class Ctx>
+// Main loop.  The ring holds NSTAGE stages; one iteration consumes KSTEP of
+// them (a "group": KSTEP * 64 bytes of K), so NSTAGE / KSTEP groups rotate.
+// Per group g:
+//   s_waitcnt vmcnt(..)   own DMAs of group g landed
+//   s_barrier             everybody's did, and everybody finished group g-1
+//   DMA group g+NG-1      into the slots group g-1 used
+//   ds_read + MFMA over group g
+// `Mma` supplies frag_t, load(frag, S, wm, wn, lane, ctx, g) with S[k] the LDS
+// address of the k-th stage of the group, and mma(acc, frag, ctx, g).
+// a_tile / b_tile point at the first K byte of tile row 0.
+template <int NSTAGE, int KSTEP, class Mma, class Acc, class Ctx>
 __device__ __forceinline__ void main_loop(Acc &acc, char *smem, const char *a_tile,
-        const char *b_tile, long lda, long ldb, long rows_a_left, long rows_b_left, int nk,
+        const char *b_tile, long lda, long ldb, long rows_a_left, long rows_b_left, int ngroups,
         const Ctx &ctx) {
-    static_assert(NSTAGE >= 3 && NSTAGE <= 5, "ring depth");
+    constexpr int NG = NSTAGE / KSTEP;           // groups in the ring
+    constexpr int GROUP_BYTES = KSTEP * STAGE_BYTES;
+    constexpr int GROUP_DMAS = KSTEP * 8 + Mma::EXTRA_DMAS;
+    static_assert(NSTAGE % KSTEP == 0 && NG >= 2 && NG <= 5, "ring depth");
+    static_assert((NG - 2) * GROUP_DMAS < 64, "vmcnt range");
     const int t = threadIdx.x, lane = t & 63;
     const int wave = __builtin_amdgcn_readfirstlane(t >> 6);
     const int wm = wave >> 1, wn = wave & 1;
     const unsigned lds0 = (unsigned)(size_t)(__attribute__((address_space(3))) char *)smem;
     const dma_plan_t plan = make_dma_plan(wave, lane, rows_a_left, rows_b_left, lda, ldb);
 
-    // prologue: stages 0 .. NSTAGE-2 in flight
+    auto issue_group = [&](int g, int slot) {
 #pragma unroll
-    for (int s = 0; s < NSTAGE - 1; ++s)
-        if (s < nk) issue_stage(plan, a_tile + (long)s * BKB, b_tile + (long)s * BKB, lds0 + s * STAGE_BYTES);
+        for (int k = 0; k < KSTEP; ++k)
+            issue_stage(plan, a_tile + ((long)g * KSTEP + k) * BKB, b_tile + ((long)g * KSTEP + k) * BKB,
+                    lds0 + slot * GROUP_BYTES + k * STAGE_BYTES);
+        Mma::issue_extra(ctx, g, slot, wave, lane);
+    };
+
+    // prologue: groups 0 .. NG-2 in flight
+#pragma unroll
+    for (int s = 0; s < NG - 1; ++s)
+        if (s < ngroups) issue_group(s, s);
 
     int slot = 0;
-    for (int kt = 0; kt < nk; ++kt) {
-        // stages kt+1 .. kt+NSTAGE-2 may stay in flight (8 DMAs each)
-        if (kt + NSTAGE - 2 < nk) wait_vmcnt<(NSTAGE - 2) * 8>();
+    for (int g = 0; g < ngroups; ++g) {
+        // groups g+1 .. g+NG-2 may stay in flight
+        if (g + NG - 2 < ngroups) wait_vmcnt<(NG - 2) * GROUP_DMAS>();
         else wait_vmcnt<0>();
         __builtin_amdgcn_s_barrier();
-        const int nxt = kt + NSTAGE - 1;
-        if (nxt < nk) {
-            int nslot = slot + NSTAGE - 1;
-            if (nslot >= NSTAGE) nslot -= NSTAGE;
+        const int nxt = g + NG - 1;
+        if (nxt < ngroups) {
+            int nslot = slot + NG - 1;
+            if (nslot >= NG) nslot -= NG;
 #ifndef MI355_DBG_NO_DMA
-            issue_stage(plan, a_tile + (long)nxt * BKB, b_tile + (long)nxt * BKB,
-                    lds0 + nslot * STAGE_BYTES);
+            issue_group(nxt, nslot);
 #endif
         }
-        const char *As = smem + slot * STAGE_BYTES;
+        const char *S[KSTEP];
+#pragma unroll
+        for (int k = 0; k < KSTEP; ++k) S[k] = smem + slot * GROUP_BYTES + k * STAGE_BYTES;
         typename Mma::frag_t f;
-        Mma::load(f, As, As + B_OFF, wm, wn, lane, ctx, kt);
+        Mma::load(f, S, wm, wn, lane, ctx, g);
 #ifndef MI355_DBG_NO_MMA
-        Mma::mma(acc, f, ctx, kt);
+        Mma::mma(acc, f, ctx, g);
 #endif
-        if (++slot == NSTAGE) slot = 0;
+        if (++slot == NG) slot = 0;
     }
     wait_vmcnt<0>();
     __builtin_amdgcn_s_barrier();

@@ -39,11 +39,14 @@ struct i8_ctx_t {};
 // shape ~3.0 POPS.)
 template <bool SRC_U8, bool WEI_U8>
 struct i8_mma_t {
+    static constexpr int EXTRA_DMAS = 0;
+    __device__ static __forceinline__ void issue_extra(const i8_ctx_t &, int, int, int, int) {}
     struct frag_t {
         v4i a[8], b[8];
     };
-    __device__ static __forceinline__ void load(frag_t &f, const char *As, const char *Bs, int wm,
-            int wn, int lane, const i8_ctx_t &, int) {
+    __device__ static __forceinline__ void load(frag_t &f, const char *const (&S)[1], int wm, int wn,
+            int lane, const i8_ctx_t &, int) {
+        const char *As = S[0], *Bs = S[0] + B_OFF;
         const int frow = lane & 15, fch = lane >> 4;
 #pragma unroll
         for (int i = 0; i < 8; ++i) {
@@ -109,7 +112,7 @@ __global__ void __launch_bounds__(NT) i8_gemm_kernel(const problem_t P_, const i
 #pragma unroll
             for (int r = 0; r < 4; ++r) acc[i][j][r] = 0;
 
-    main_loop<NSTAGE, i8_mma_t<SRC_U8, WEI_U8>>(acc, smem, A, Bt, lda, X.ldb, P.M - m0, P.N - n0,
+    main_loop<NSTAGE, 1, i8_mma_t<SRC_U8, WEI_U8>>(acc, smem, A, Bt, lda, X.ldb, P.M - m0, P.N - n0,
             (int)(P.K / BK), i8_ctx_t {});
 
     // ---- epilogue: s32 compensation, scales, shared tail
@@ -178,25 +181,6 @@ __global__ void __launch_bounds__(256) i8_rowsum_kernel(const int8_t *p, long ro
 #pragma unroll
     for (int o = 32; o > 0; o >>= 1) s += __shfl_down(s, o, 64);
     if (lane == 0) out[r] = s;
-}
-
-// in: [R][C] bytes with row pitch ld_in  ->  out: [C][R] bytes, pitch ld_out
-__global__ void __launch_bounds__(256) transpose_bytes_kernel(const uint8_t *in, long R, long C,
-        long ld_in, long in_bstride, uint8_t *out, long ld_out, long out_bstride) {
-    __shared__ uint8_t tile[64][65];
-    in += blockIdx.z * in_bstride;
-    out += blockIdx.z * out_bstride;
-    const long r0 = (long)blockIdx.y * 64, c0 = (long)blockIdx.x * 64;
-    const int tx = threadIdx.x & 63, ty = threadIdx.x >> 6;
-    for (int i = ty; i < 64; i += 4) {
-        const long r = r0 + i, c = c0 + tx;
-        tile[i][tx] = (r < R && c < C) ? in[r * ld_in + c] : 0;
-    }
-    __syncthreads();
-    for (int i = ty; i < 64; i += 4) {
-        const long c = c0 + i, r = r0 + tx;
-        if (c < C && r < R) out[c * ld_out + r] = tile[tx][i];
-    }
 }
 
 struct i8_plan_t {
@@ -268,10 +252,8 @@ int i8_launch(const mi355_matmul_desc_t &d, const problem_t &P, void *scratch,
     const bool src_u8 = d.src_dt == MI355_DT_U8, wei_u8 = d.wei_dt == MI355_DT_U8;
     if (plan.need_transpose) {
         uint8_t *bt = (uint8_t *)(sc + plan.off_bt);
-        dim3 grid((unsigned)((d.N + 63) / 64), (unsigned)((d.K + 63) / 64), (unsigned)plan.Bw);
-        hipLaunchKernelGGL(transpose_bytes_kernel, grid, dim3(256), 0, stream,
-                (const uint8_t *)P.wei, d.K, d.N, d.wei_stride[1], d.wei_stride[0], bt, d.K,
-                d.N * d.K);
+        transpose_bytes(P.wei, d.K, d.N, d.wei_stride[1], d.wei_stride[0], bt, d.K, d.N * d.K,
+                plan.Bw, stream);
         X.bt = (const int8_t *)bt;
         X.ldb = d.K;
         X.bt_bstride = plan.Bw > 1 ? d.N * d.K : 0;

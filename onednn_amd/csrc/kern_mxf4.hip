@@ -1,6 +1,254 @@
-#include "kernels.hpp"
+// "hip:mfma_mxf4" -- MXFP4 GEMM: f4_e2m1 x f4_e2m1 with e8m0 block scales over
+// 32 consecutive K on both operands, f32 accumulation, on the gfx950
+// block-scaled matrix instruction v_mfma_scale_f32_16x16x128_f8f6f4.
+//
+// Semantics: ref_matmul_t with group_k = 32 (src/cpu/matmul/ref_matmul.cpp:
+// 168-236; the Intel GPU reference kernel src/gpu/intel/matmul/ref.cl:200-262
+// is the in-tree implementation that runs it):
+//   for each block g of 32 k:  acc = sum_j src*wei  (exact in f32)
+//                              acc *= 2^(ss-127); acc *= 2^(ws-127); res += acc
+// One MFMA covers 128 k = four blocks; lane l carries row l%16 and block l/16,
+// i.e. exactly one MX block and one scale byte per operand per lane.  Only the
+// rounding of the cross-block f32 additions can differ from the reference.
+//
+// Operand bytes are K-contiguous nibble pairs; the order of the two nibbles
+// inside a byte is irrelevant as long as both operands agree, because all 32
+// elements of a block share one scale.
+//
+// Scales ride along with the tile stages: per stage and operand one extra
+// direct-to-LDS load per wavefront brings the 4 scale bytes (one dword) of
+// each of its 64 rows; weights scales [K/32][N] are transposed to [N][K/32]
+// by a pre-pass so both sides look alike.
+#include "gemm_core.hpp"
+
 namespace mi355 {
-int mxf4_supported(const mi355_matmul_desc_t &) { return MI355_UNIMPLEMENTED; }
-size_t mxf4_scratch_bytes(const mi355_matmul_desc_t &) { return 0; }
-int mxf4_launch(const mi355_matmul_desc_t &, const problem_t &, void *, hipStream_t) { return MI355_UNIMPLEMENTED; }
+namespace {
+
+using namespace gemm;
+constexpr int NSTAGE = 4;
+constexpr int SCALE_OFF = NSTAGE * STAGE_BYTES;      // scale ring after the tile ring
+constexpr int SCALE_STAGE = 2048;                    // 256 dwords A + 256 dwords B
+constexpr int SMEM_BYTES = SCALE_OFF + NSTAGE * SCALE_STAGE;
+
+struct mxf4_extra_t {
+    const char *bt;       // weights [N][K/2] bytes
+    long ldb, bt_bstride; // bytes
+    const char *sa;       // src scales [M][K/32] bytes, this batch added in-kernel
+    const char *sb;       // weights scales [N][K/32] bytes (transposed copy)
+    long sa_bstride, sb_bstride;
+    int tiles_m, tiles_n;
+};
+
+struct mxf4_ctx_t {
+    const char *sa_tile, *sb_tile; // first scale byte of tile row 0
+    unsigned voff_a, voff_b;       // this lane's row offset in the scale arrays
+    unsigned lds_scale0;           // LDS byte address of the scale ring
+    const char *smem;
+};
+
+struct mxf4_mma_t {
+    static constexpr int EXTRA_DMAS = 2;
+    // wave w brings the scale dwords of tile rows [64w, 64w+64) of both operands
+    __device__ static __forceinline__ void issue_extra(const mxf4_ctx_t &c, int g, int slot, int wave,
+            int) {
+        const unsigned dst = c.lds_scale0 + slot * SCALE_STAGE + wave * 256;
+        dma4(c.sa_tile + (long)g * 4, c.voff_a, dst);
+        dma4(c.sb_tile + (long)g * 4, c.voff_b, dst + 1024);
+    }
+    struct frag_t {
+        v4i a[8], b[8];
+        int sa[8], sb[8];
+    };
+    __device__ static __forceinline__ void load(frag_t &f, const char *const (&S)[1], int wm, int wn,
+            int lane, const mxf4_ctx_t &c, int) {
+        const char *As = S[0], *Bs = S[0] + B_OFF;
+        const int slot = (int)((S[0] - c.smem) / STAGE_BYTES);
+        const unsigned *sc = (const unsigned *)(c.smem + SCALE_OFF + slot * SCALE_STAGE);
+        const int frow = lane & 15, q = lane >> 4;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            const int ra = wm * 128 + i * 16 + frow, rb = wn * 128 + i * 16 + frow;
+            f.a[i] = *(const v4i *)&As[swz(ra, q)];
+            f.b[i] = *(const v4i *)&Bs[swz(rb, q)];
+            f.sa[i] = (int)((sc[ra] >> (q * 8)) & 0xffu);
+            f.sb[i] = (int)((sc[256 + rb] >> (q * 8)) & 0xffu);
+        }
+    }
+    __device__ static __forceinline__ void mma(v4f (&acc)[8][8], const frag_t &f, const mxf4_ctx_t &, int) {
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            const v8i a = {f.a[i][0], f.a[i][1], f.a[i][2], f.a[i][3], 0, 0, 0, 0};
+#pragma unroll
+            for (int j = 0; j < 8; ++j) {
+                const v8i bb = {f.b[j][0], f.b[j][1], f.b[j][2], f.b[j][3], 0, 0, 0, 0};
+                acc[i][j] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(
+                        a, bb, acc[i][j], 4, 4, 0, f.sa[i], 0, f.sb[j]);
+            }
+        }
+    }
+};
+
+struct mxf4_conv_t {
+    __device__ __forceinline__ void row(const v4i_t &raw, long, float (&f)[4]) const {
+#pragma unroll
+        for (int e = 0; e < 4; ++e) f[e] = __int_as_float(raw[e]);
+    }
+};
+
+extern __shared__ __attribute__((aligned(16))) char mxf4_smem[];
+
+__global__ void __launch_bounds__(NT) mxf4_gemm_kernel(const problem_t P_, const mxf4_extra_t X) {
+    const auto &P = MI355_KERNARG_PROBLEM();
+    char *smem = mxf4_smem;
+    const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
+    const int wm = wave >> 1, wn = wave & 1;
+    const long b = blockIdx.z;
+    const tile_pos_t tp = tile_position(X.tiles_m, X.tiles_n);
+    const long m0 = tp.m0, n0 = tp.n0;
+
+    const long lda = P.ss[1] / 2; // bytes per src row
+    const long kb = P.K / 32;     // scale bytes per row
+    const char *A = (const char *)P.src + (P.ss[0] ? b * (P.ss[0] / 2) : 0) + m0 * lda;
+    const char *Bt = X.bt + b * X.bt_bstride + n0 * X.ldb;
+
+    mxf4_ctx_t ctx;
+    ctx.smem = smem;
+    ctx.lds_scale0 = (unsigned)(size_t)(__attribute__((address_space(3))) char *)smem + SCALE_OFF;
+    ctx.sa_tile = X.sa + b * X.sa_bstride + m0 * kb;
+    ctx.sb_tile = X.sb + b * X.sb_bstride + n0 * kb;
+    {
+        long ra = wave * 64 + lane, rb = ra;
+        if (ra > P.M - m0 - 1) ra = P.M - m0 - 1;
+        if (rb > P.N - n0 - 1) rb = P.N - n0 - 1;
+        ctx.voff_a = (unsigned)(ra * kb);
+        ctx.voff_b = (unsigned)(rb * kb);
+    }
+
+    v4f acc[8][8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i)
+#pragma unroll
+        for (int j = 0; j < 8; ++j)
+#pragma unroll
+            for (int r = 0; r < 4; ++r) acc[i][j][r] = 0.f;
+
+    main_loop<NSTAGE, 1, mxf4_mma_t>(acc, smem, A, Bt, lda, X.ldb, P.M - m0, P.N - n0,
+            (int)(P.K / 128), ctx);
+
+    const bool interior = m0 + BM <= P.M && n0 + BN <= P.N;
+    store_quadrant<layout16_t>(P, smem, acc, b, m0 + wm * 128, n0 + wn * 128, interior,
+            mxf4_conv_t {});
 }
+
+// in: [R][C] nibbles, C contiguous (two per byte)  ->  out: [C][R] nibbles
+__global__ void __launch_bounds__(256) transpose_nibbles_kernel(const uint8_t *in, long R, long C,
+        long in_bstride, uint8_t *out, long out_bstride) {
+    in += blockIdx.z * in_bstride;
+    out += blockIdx.z * out_bstride;
+    // one thread per output byte: column c, rows 2r and 2r+1
+    const long total = C * (R / 2);
+    for (long i = (long)blockIdx.x * blockDim.x + threadIdx.x; i < total;
+            i += (long)gridDim.x * blockDim.x) {
+        const long c = i / (R / 2), r2 = i % (R / 2);
+        const uint8_t b0 = in[((2 * r2) * C + c) >> 1], b1 = in[((2 * r2 + 1) * C + c) >> 1];
+        const uint8_t lo = (c & 1) ? (b0 >> 4) : (b0 & 0xf), hi = (c & 1) ? (b1 >> 4) : (b1 & 0xf);
+        out[c * (R / 2) + r2] = (uint8_t)(lo | (hi << 4));
+    }
+}
+
+struct mxf4_plan_t {
+    bool need_transpose;
+    size_t off_bt, off_sb, total;
+    long Bw, Bsb;
+};
+
+mxf4_plan_t make_plan(const mi355_matmul_desc_t &d) {
+    mxf4_plan_t p {};
+    p.Bw = d.wei_stride[0] ? d.batch : 1;
+    p.Bsb = (d.wei_scale.mask & 1) ? p.Bw : 1;
+    p.need_transpose = !(d.wei_stride[1] == 1);
+    size_t off = 0;
+    p.off_bt = off;
+    if (p.need_transpose) off += align_up((size_t)p.Bw * d.N * d.K / 2, 256);
+    p.off_sb = off;
+    off += align_up((size_t)p.Bsb * d.N * (d.K / 32), 256);
+    p.total = off;
+    return p;
+}
+
+} // namespace
+
+int mxf4_supported(const mi355_matmul_desc_t &d) {
+    if (d.src_dt != MI355_DT_F4_E2M1 || d.wei_dt != MI355_DT_F4_E2M1) return MI355_UNIMPLEMENTED;
+    if (dt_bits(d.dst_dt) < 8) return MI355_UNIMPLEMENTED;
+    if (d.K < 128 || d.K % 128 != 0) return MI355_UNIMPLEMENTED;
+    if (d.src_stride[2] != 1 || d.src_stride[1] % 32 != 0 || d.src_stride[0] % 32 != 0)
+        return MI355_UNIMPLEMENTED;
+    const bool k_major = d.wei_stride[1] == 1 && d.wei_stride[2] % 32 == 0 && d.wei_stride[0] % 32 == 0;
+    const bool n_major = d.wei_stride[2] == 1 && d.wei_stride[1] == d.N && d.N % 2 == 0
+            && (d.wei_stride[0] == 0 || d.wei_stride[0] == d.K * d.N);
+    if (!k_major && !n_major) return MI355_UNIMPLEMENTED;
+    if (!quant_absent(d.src_zp) || !quant_absent(d.wei_zp) || !quant_absent(d.src_pr))
+        return MI355_UNIMPLEMENTED;
+    // MX scales on both operands: e8m0, one per 32 consecutive k
+    const mi355_quant_t &ss = d.src_scale, &ws = d.wei_scale;
+    if (ss.dt != MI355_DT_E8M0 || (ss.mask & 6) != 6 || ss.group[0] != 1 || ss.group[1] != 32)
+        return MI355_UNIMPLEMENTED;
+    if (ws.dt != MI355_DT_E8M0 || (ws.mask & 6) != 6 || ws.group[0] != 32 || ws.group[1] != 1)
+        return MI355_UNIMPLEMENTED;
+    if (d.batch > 65535) return MI355_UNIMPLEMENTED;
+    return MI355_SUCCESS;
+}
+
+size_t mxf4_scratch_bytes(const mi355_matmul_desc_t &d) {
+    return make_plan(d).total;
+}
+
+int mxf4_launch(const mi355_matmul_desc_t &d, const problem_t &P, void *scratch, hipStream_t stream) {
+    const mxf4_plan_t plan = make_plan(d);
+    if (!scratch) {
+        set_error("mfma_mxf4: %zu bytes of scratch required", plan.total);
+        return MI355_INVALID_ARGUMENTS;
+    }
+    char *sc = (char *)scratch;
+    mxf4_extra_t X {};
+    if (plan.need_transpose) {
+        const long total = d.N * (d.K / 2);
+        long blocks = (total + 255) / 256;
+        if (blocks > 65535) blocks = 65535;
+        hipLaunchKernelGGL(transpose_nibbles_kernel, dim3((unsigned)blocks, 1, (unsigned)plan.Bw),
+                dim3(256), 0, stream, (const uint8_t *)P.wei, d.K, d.N, d.wei_stride[0] / 2,
+                (uint8_t *)(sc + plan.off_bt), d.N * d.K / 2);
+        X.bt = sc + plan.off_bt;
+        X.ldb = d.K / 2;
+        X.bt_bstride = plan.Bw > 1 ? d.N * d.K / 2 : 0;
+    } else {
+        X.bt = (const char *)P.wei;
+        X.ldb = d.wei_stride[2] / 2;
+        X.bt_bstride = d.wei_stride[0] / 2;
+    }
+    // weights scales [K/32][N] -> [N][K/32]
+    const long kb = d.K / 32;
+    transpose_bytes(P.wei_scale.p, kb, d.N, d.N, kb * d.N, sc + plan.off_sb, kb, d.N * kb, plan.Bsb,
+            stream);
+    X.sb = sc + plan.off_sb;
+    X.sb_bstride = plan.Bsb > 1 ? d.N * kb : 0;
+    X.sa = (const char *)P.src_scale.p;
+    X.sa_bstride = ((d.src_scale.mask & 1) && d.src_stride[0]) ? d.M * kb : 0;
+    X.tiles_m = (int)((d.M + BM - 1) / BM);
+    X.tiles_n = (int)((d.N + BN - 1) / BN);
+    dim3 grid((unsigned)(X.tiles_m * X.tiles_n), 1, (unsigned)d.batch);
+    static bool attr_done = false;
+    if (!attr_done) {
+        if (hipFuncSetAttribute((const void *)mxf4_gemm_kernel,
+                    hipFuncAttributeMaxDynamicSharedMemorySize, SMEM_BYTES) != hipSuccess) {
+            set_error("mfma_mxf4: cannot reserve %d bytes of LDS", SMEM_BYTES);
+            return MI355_RUNTIME_ERROR;
+        }
+        attr_done = true;
+    }
+    hipLaunchKernelGGL(mxf4_gemm_kernel, grid, dim3(NT), SMEM_BYTES, stream, P, X);
+    return hipGetLastError() == hipSuccess ? MI355_SUCCESS : MI355_RUNTIME_ERROR;
+}
+
+} // namespace mi355

@@ -19,6 +19,33 @@ __global__ void __launch_bounds__(256) flush_kernel(v4i *buf, long n16) {
         buf[i] = v;
     }
 }
+
+// in: [R][C] bytes with row pitch ld_in  ->  out: [C][R] bytes, pitch ld_out
+__global__ void __launch_bounds__(256) transpose_bytes_kernel(const uint8_t *in, long R, long C,
+        long ld_in, long in_bstride, uint8_t *out, long ld_out, long out_bstride) {
+    __shared__ uint8_t tile[64][65];
+    in += blockIdx.z * in_bstride;
+    out += blockIdx.z * out_bstride;
+    const long r0 = (long)blockIdx.y * 64, c0 = (long)blockIdx.x * 64;
+    const int tx = threadIdx.x & 63, ty = threadIdx.x >> 6;
+    for (int i = ty; i < 64; i += 4) {
+        const long r = r0 + i, c = c0 + tx;
+        tile[i][tx] = (r < R && c < C) ? in[r * ld_in + c] : 0;
+    }
+    __syncthreads();
+    for (int i = ty; i < 64; i += 4) {
+        const long c = c0 + i, r = r0 + tx;
+        if (c < C && r < R) out[c * ld_out + r] = tile[tx][i];
+    }
+}
+
+
+void transpose_bytes(const void *in, long R, long C, long ld_in, long in_bstride, void *out,
+        long ld_out, long out_bstride, long batches, hipStream_t stream) {
+    dim3 grid((unsigned)((C + 63) / 64), (unsigned)((R + 63) / 64), (unsigned)batches);
+    hipLaunchKernelGGL(transpose_bytes_kernel, grid, dim3(256), 0, stream, (const uint8_t *)in, R, C,
+            ld_in, in_bstride, (uint8_t *)out, ld_out, out_bstride);
+}
 } // namespace mi355
 
 using namespace mi355;

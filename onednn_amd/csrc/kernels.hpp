@@ -34,6 +34,10 @@ int woq_launch(const mi355_matmul_desc_t &d, const problem_t &P, void *scratch,
 
 void set_error(const char *fmt, ...);
 
+// [R][C] bytes (row pitch ld_in) -> [C][R] bytes (row pitch ld_out), per batch
+void transpose_bytes(const void *in, long R, long C, long ld_in, long in_bstride, void *out,
+        long ld_out, long out_bstride, long batches, hipStream_t stream);
+
 inline bool is_int8_dt(int dt) { return dt == MI355_DT_S8 || dt == MI355_DT_U8; }
 inline bool is_int4_dt(int dt) { return dt == MI355_DT_S4 || dt == MI355_DT_U4; }
 inline bool is_f8_dt(int dt) { return dt == MI355_DT_F8_E4M3 || dt == MI355_DT_F8_E5M2; }

@@ -36,3 +36,54 @@ def test_config1_full_size(gpu, oracle):
     assert name.startswith("hip:mfma_i8")
     want = oracle.run_oracle(p)
     assert_bit_exact(p, got, want, name)
+
+
+@pytest.mark.parametrize("impl", [cabi.IMPL_REF, cabi.IMPL_F8_MFMA])
+@pytest.mark.parametrize("wtag", ["ab", "ba"])
+def test_config4_small(gpu, oracle, impl, wtag):
+    # fp8 x fp8 -> bf16 with bf16 bias, gelu_tanh and a bf16 residual add.
+    # f32 accumulation order and the device tanhf differ from the oracle's:
+    # thresholds are the reference checker's eltwise ladder plus the forward
+    # error bound of the K-sum (tests/helpers.py).
+    p = configs.config4(M=192, N=320, K=512, wtag=wtag)
+    got, name = run_gpu(p, impl)
+    want, _, asum = oracle.run_oracle(p, want_ideal=True)
+    assert_close(p, got, want, abs_sum=asum, transcendental=True, what=name)
+
+
+def test_config4_no_postops_f32(gpu, oracle):
+    # plain scaled fp8 GEMM into f32: only the summation order differs
+    p = configs.config4(M=256, N=256, K=1024)
+    p.post_ops = []
+    p.bias, p.bias_dt = None, cabi.DT_UNDEF
+    p.dst_dt = cabi.DT_F32
+    got, name = run_gpu(p, cabi.IMPL_F8_MFMA)
+    want, _, asum = oracle.run_oracle(p, want_ideal=True)
+    assert_close(p, got, want, abs_sum=asum, what=name)
+
+
+@pytest.mark.parametrize("impl", [cabi.IMPL_REF, cabi.IMPL_MXF4_MFMA])
+@pytest.mark.parametrize("wtag", ["ba", "ab"])
+def test_config5_small(gpu, oracle, impl, wtag):
+    # MXFP4: every 32-long block dot is exact in f32 and the e8m0 scales are
+    # powers of two, so only the order of the K/32 cross-block additions can
+    # differ: bounded by the forward error of that sum, then one bf16 rounding.
+    p = configs.config5(M=160, N=288, K=512, wtag=wtag)
+    got, name = run_gpu(p, impl)
+    want, _, asum = oracle.run_oracle(p, want_ideal=True)
+    if impl == cabi.IMPL_REF:
+        assert_bit_exact(p, got, want, name)   # same order as the reference
+    else:
+        assert_close(p, got, want, abs_sum=asum, what=name)
+
+
+def test_config5_f32_dst_single_block_exact(gpu, oracle):
+    # K = 128 is one MFMA: four blocks, f32 dst.  With all scales equal the
+    # sum of four exactly representable block sums is exact in any order.
+    p = configs.config5(M=256, N=256, K=128)
+    p.dst_dt = cabi.DT_F32
+    p.quant["src_scale"].data[:] = 127
+    p.quant["wei_scale"].data[:] = 126
+    got, name = run_gpu(p, cabi.IMPL_MXF4_MFMA)
+    want = oracle.run_oracle(p)
+    assert_bit_exact(p, got, want, name)
