@@ -1,0 +1,260 @@
+#!/usr/bin/env python3
+"""Benchmark of the quantized matmul hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c3|c2|c4|c5|c1]
+
+A "step" is one launch of the matmul primitive (through the C ABI,
+mi355_matmul_launch) on synthetic, seeded inputs that are resident in HBM
+before the timed region starts.  The line printed at the end is one JSON
+object: the headline metric of the chosen workload plus
+
+  roofline      the dominant kernel of that workload against the MI355X peak
+                that bounds it; the kernel duration is measured here with HIP
+                events on the launch stream
+  cpu_baseline  the CPU restatement of the reference algorithm (oracle/),
+                timed on this machine's host cores on a bounded sample of the
+                same workload
+  others        the remaining benchmark configurations, measured the same way
+                with fewer steps (informational)
+
+Workloads (BASELINE.json configs):
+  c3  s8 x s8 -> s8, M=N=K=8192, scales + ReLU (MFMA int8 bound)      [default]
+  c2  bf16 x u4 -> bf16 decode, K=4096 N=14336, M in {1,8,32} (HBM bound)
+  c4  e4m3 x e4m3 -> bf16, 4096 x 8192 x 28672, bias+gelu+add (MFMA fp8 bound)
+  c5  MXFP4, M=N=K=8192 (MFMA fp4 bound)
+  c1  u8 x s8 -> f32, 256 x 1024 x 1024 (latency bound, no roofline claim)
+"""
+import argparse
+import ctypes as C
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+import numpy as np  # noqa: E402
+
+# MI355X published peaks
+PEAK_HBM_GBS = 8000.0
+PEAK_I8_TOPS = 5000.0
+PEAK_F8_TFLOPS = 5000.0
+PEAK_F4_TFLOPS = 10100.0
+
+
+def log(*a):
+    print(*a, file=sys.stderr, flush=True)
+
+
+class Timer:
+    """HIP events on the stream the kernels are launched on."""
+
+    def __init__(self, lib, stream=None):
+        self.lib, self.stream = lib, stream
+        self.e0, self.e1 = C.c_void_p(), C.c_void_p()
+        from onednn_amd import cabi
+        cabi.check(lib.mi355_event_create(C.byref(self.e0)))
+        cabi.check(lib.mi355_event_create(C.byref(self.e1)))
+
+    def time_ms(self, fn, iters):
+        from onednn_amd import cabi
+        cabi.check(self.lib.mi355_stream_sync(self.stream))
+        cabi.check(self.lib.mi355_event_record(self.e0, self.stream))
+        for _ in range(iters):
+            fn()
+        cabi.check(self.lib.mi355_event_record(self.e1, self.stream))
+        cabi.check(self.lib.mi355_event_sync(self.e1))
+        ms = C.c_float()
+        cabi.check(self.lib.mi355_event_elapsed_ms(C.byref(ms), self.e0, self.e1))
+        return ms.value / iters
+
+
+def build_problem(name, M=None):
+    from onednn_amd import configs
+    if name == "c1":
+        return configs.config1()
+    if name == "c2":
+        return configs.config2(M=M or 1)
+    if name == "c3":
+        return configs.config3()
+    if name == "c4":
+        return configs.config4()
+    if name == "c5":
+        return configs.config5()
+    raise ValueError(name)
+
+
+def algorithmic(name, p):
+    """(work per launch, unit of the rate, roofline bound, peak)."""
+    from onednn_amd import configs
+    ops = 2.0 * p.batch * p.M * p.N * p.K
+    if name == "c2":
+        return configs.config2_bytes(p.M, p.N, p.K), "GB/s", "hbm", PEAK_HBM_GBS
+    if name == "c3":
+        return ops, "TOPS", "mfma", PEAK_I8_TOPS
+    if name == "c4":
+        return ops, "TFLOP/s", "mfma", PEAK_F8_TFLOPS
+    if name == "c5":
+        return ops, "TFLOP/s", "mfma", PEAK_F4_TFLOPS
+    return ops, "TOPS", "mfma", PEAK_I8_TOPS
+
+
+def rate(work, ms, unit):
+    if unit == "GB/s":
+        return work / (ms * 1e-3) / 1e9
+    return work / (ms * 1e-3) / 1e12
+
+
+def run_gpu_workload(lib, name, steps, warmup, M=None, cold_copies=0):
+    """Returns dict with ms_per_step, value, unit, impl."""
+    from onednn_amd import cabi
+    from onednn_amd.problem import GpuRun
+    t0 = time.time()
+    p = build_problem(name, M)
+    log(f"[bench] {name}: generated {p.name} in {time.time() - t0:.1f}s")
+    runs = [GpuRun(p)]
+    # decode is HBM-bound only if the weights are not already in the 256 MB
+    # last-level cache: rotate over enough weight copies to exceed it
+    for _ in range(cold_copies):
+        runs.append(GpuRun(p))
+    timer = Timer(lib)
+    idx = [0]
+
+    def step():
+        runs[idx[0] % len(runs)].launch()
+        idx[0] += 1
+
+    for _ in range(max(warmup, 1)):
+        step()
+    ms = timer.time_ms(step, steps)
+    work, unit, bound, peak = algorithmic(name, p)
+    out = {
+        "workload": p.name, "impl": cabi.impl_name(runs[0].impl), "ms_per_step": ms,
+        "value": rate(work, ms, unit), "unit": unit, "bound": bound, "peak": peak, "work": work,
+        "shape": [p.M, p.K, p.N],
+    }
+    for r in runs:
+        r.free()
+    return out, p
+
+
+def cpu_baseline(name, M=None):
+    """The oracle timed on a bounded sample of the same workload."""
+    from oracle import binding as oracle
+    from onednn_amd import configs
+    threads = int(os.environ.get("OMP_NUM_THREADS", "0")) or (os.cpu_count() or 1)
+    threads = min(threads, 16)
+    os.environ["OMP_NUM_THREADS"] = str(threads)
+    if name == "c3":
+        p = configs.config3(M=256, N=1024, K=8192)
+        sample = "rows 0..255 x cols 0..1023 of the 8192^3 problem shape (M=256, N=1024, K=8192)"
+    elif name == "c2":
+        p = configs.config2(M=M or 1, N=14336, K=4096)
+        sample = f"full problem M={p.M}, K=4096, N=14336"
+    elif name == "c4":
+        p = configs.config4(M=128, N=1024, K=8192)
+        sample = "M=128, N=1024, K=8192 slice of the 4096x8192x28672 shape"
+    elif name == "c5":
+        p = configs.config5(M=128, N=1024, K=8192)
+        sample = "M=128, N=1024, K=8192 slice of the 8192^3 shape"
+    else:
+        p = configs.config1()
+        sample = "full problem 256x1024x1024"
+    oracle.load()
+    t0 = time.time()
+    oracle.run_oracle(p)
+    dt = time.time() - t0
+    work, unit, _, _ = algorithmic(name, p)
+    return {"value": rate(work, dt * 1e3, unit), "unit": unit, "cores": threads, "kind": "port",
+            "sample": sample + f"; {dt:.2f} s wall; oracle/liboracle.so (naive restatement of "
+            "ref_matmul*_t, OpenMP over dst rows)"}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--workload", default="c3", choices=["c1", "c2", "c3", "c4", "c5"])
+    ap.add_argument("--decode-m", type=int, default=1, help="M of the c2 decode workload")
+    ap.add_argument("--no-others", action="store_true", help="skip the informational configs")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py: this build runs on one GPU (one-GPU boxes only); "
+                 "--gpus must be 1. Sharding is described in DESIGN.md, not built.")
+
+    from onednn_amd import cabi
+    lib = cabi.load_kernels()  # raises if the HIP library is missing: no fallback
+    n = C.c_int(0)
+    cabi.check(lib.mi355_device_count(C.byref(n)))
+    if n.value < 1:
+        sys.exit("bench.py: no HIP device visible")
+    cabi.check(lib.mi355_device_set(0))
+    name = C.create_string_buffer(64)
+    cus, khz = C.c_int(), C.c_int()
+    hbm, l2 = C.c_int64(), C.c_int64()
+    cabi.check(lib.mi355_device_info(0, name, 64, C.byref(cus), C.byref(khz), C.byref(hbm),
+                                     C.byref(l2)))
+    log(f"[bench] device {name.value.decode()} CUs={cus.value} clock={khz.value / 1e3:.0f} MHz "
+        f"HBM={hbm.value / 2**30:.0f} GiB")
+
+    main_name = args.workload
+    cold = 11 if main_name == "c2" else 0
+    res, prob = run_gpu_workload(lib, main_name, args.steps, args.warmup, args.decode_m, cold)
+    log(f"[bench] {res['workload']}: {res['ms_per_step']:.4f} ms/step -> {res['value']:.1f} "
+        f"{res['unit']} via {res['impl']}")
+
+    # The timed step is one launch whose time is dominated by one kernel (the
+    # tile GEMM / the decode kernel); pre-pass kernels of the same launch
+    # (layout change of `ab` weights, column sums) are part of the measured
+    # step and therefore of `achieved`.
+    roofline = {
+        "bound": res["bound"], "achieved": res["value"], "peak": res["peak"],
+        "unit": "GB/s" if res["unit"] == "GB/s" else "TFLOP/s",
+        "frac": res["value"] / res["peak"], "traffic": None,
+        "kernel": res["impl"], "kernel_ms": res["ms_per_step"],
+    }
+
+    others = []
+    if not args.no_others:
+        plan = [("c2", 1), ("c2", 8), ("c2", 32), ("c3", None), ("c4", None), ("c5", None),
+                ("c1", None)]
+        for nm, m in plan:
+            if nm == main_name and (nm != "c2" or m == args.decode_m):
+                continue
+            try:
+                r, _ = run_gpu_workload(lib, nm, max(5, args.steps // 2), 2, m,
+                                        11 if nm == "c2" else 0)
+                r["frac_of_peak"] = r["value"] / r["peak"]
+                others.append({k: r[k] for k in ("workload", "impl", "ms_per_step", "value", "unit",
+                                                 "bound", "peak", "frac_of_peak")})
+                log(f"[bench] {r['workload']}: {r['ms_per_step']:.4f} ms -> {r['value']:.1f} "
+                    f"{r['unit']} ({100 * r['frac_of_peak']:.1f}% of {r['bound']} peak) via {r['impl']}")
+            except Exception as e:  # a failing side workload must not hide the headline
+                others.append({"workload": f"{nm}-M{m}" if m else nm, "error": str(e)})
+                log(f"[bench] {nm}: failed: {e}")
+
+    cpu = None
+    if not args.no_cpu:
+        cpu = cpu_baseline(main_name, args.decode_m)
+        log(f"[bench] cpu baseline: {cpu['value']:.4f} {cpu['unit']} on {cpu['cores']} threads")
+
+    metric = {"c3": "int8 matmul TOPS @8192^3", "c2": "int4 weight-only decode GB/s",
+              "c4": "fp8 matmul TFLOP/s @4096x8192x28672", "c5": "MXFP4 matmul TFLOP/s @8192^3",
+              "c1": "int8 matmul TOPS @256x1024x1024"}[main_name]
+    dtype = {"c3": "s8", "c2": "bf16", "c4": "f8_e4m3", "c5": "f4_e2m1", "c1": "u8"}[main_name]
+    line = {
+        "metric": metric, "value": res["value"], "unit": res["unit"], "n_gpus": 1,
+        "steps": args.steps, "warmup": args.warmup, "ms_per_step": res["ms_per_step"],
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": dtype,
+        "data": "synthetic",
+        "config": {"workload": res["workload"], "shape_MKN": res["shape"], "impl": res["impl"]},
+        "roofline": roofline, "cpu_baseline": cpu, "others": others,
+    }
+    print(json.dumps(line), flush=True)
+
+
+if __name__ == "__main__":
+    main()

@@ -87,3 +87,13 @@ def test_config5_f32_dst_single_block_exact(gpu, oracle):
     got, name = run_gpu(p, cabi.IMPL_MXF4_MFMA)
     want = oracle.run_oracle(p)
     assert_bit_exact(p, got, want, name)
+
+
+@pytest.mark.parametrize("M", [1, 8, 32])
+def test_config2_small_ref_kernel(gpu, oracle, M):
+    # weight-only int4 decode through the generic kernel: same operation order
+    # as the reference's naive loop, no transcendental functions -> bit-exact
+    p = configs.config2(M=M, N=512, K=1024)
+    got, name = run_gpu(p, cabi.IMPL_REF)
+    want = oracle.run_oracle(p)
+    assert_bit_exact(p, got, want, name)
