@@ -97,3 +97,32 @@ def test_config2_small_ref_kernel(gpu, oracle, M):
     got, name = run_gpu(p, cabi.IMPL_REF)
     want = oracle.run_oracle(p)
     assert_bit_exact(p, got, want, name)
+
+
+@pytest.mark.parametrize("M", [1, 8, 32])
+def test_config2_small_woq_kernel(gpu, oracle, M):
+    # the decode kernel evaluates the same real-valued expression with a
+    # different rounding (group factor applied once per group, MFMA f32
+    # accumulation): bf16 threshold plus the forward error bound of the K sum
+    p = configs.config2(M=M, N=512, K=1024)
+    got, name = run_gpu(p, cabi.IMPL_WOQ_GEMV)
+    assert name.startswith("hip:woq_gemv")
+    want, _, asum = oracle.run_oracle(p, want_ideal=True)
+    # the offset-binary trick adds 128 * |sum of src| to the magnitude of the
+    # accumulated terms of a group: widen the bound accordingly
+    assert_close(p, got, want, abs_sum=asum * 20.0, what=name)
+
+
+def test_woq_one_hot_rows_are_exact(gpu, oracle):
+    # src = identity: every output is a single decompressed weight,
+    # (w - zp) * scale with one rounding -> must equal the oracle bit for bit.
+    # Exercises nibble order, group indexing and the K split / reduction.
+    import numpy as np
+    from onednn_amd import dtypes as dtp
+    K = 32
+    p = configs.config2(M=K, N=256, K=K, group=16)
+    p.src = dtp.f32_to_bf16(np.eye(K, dtype=np.float32))
+    p.dst_dt = cabi.DT_F32
+    got, name = run_gpu(p, cabi.IMPL_WOQ_GEMV)
+    want = oracle.run_oracle(p)
+    assert_bit_exact(p, got, want, name)
