@@ -1,0 +1,329 @@
+/*
+ * dnnl_amd.h -- the subset of oneDNN's public C API that the matmul primitive
+ * needs, exported by libdnnl_amd.so with the reference's symbol names,
+ * signatures and enum values, so that code written against oneDNN's own
+ * headers (dnnl.h / dnnl.hpp, which are header-only wrappers over these
+ * symbols) links against this library unchanged and only has to ask for a GPU
+ * engine.
+ *
+ * Each declaration cites the reference declaration it reproduces
+ * (uxlfoundation/oneDNN v3.14, paths relative to include/oneapi/dnnl/).
+ * Callers that already include oneDNN's headers do not need this file; it
+ * exists for callers (and tests) that do not have them.
+ */
+#ifndef DNNL_AMD_H
+#define DNNL_AMD_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* dnnl_common_types.h:44-66 */
+typedef enum {
+    dnnl_success = 0,
+    dnnl_out_of_memory = 1,
+    dnnl_invalid_arguments = 2,
+    dnnl_unimplemented = 3,
+    dnnl_last_impl_reached = 4,
+    dnnl_runtime_error = 5,
+    dnnl_not_required = 6,
+    dnnl_invalid_graph = 7,
+    dnnl_invalid_graph_op = 8,
+    dnnl_invalid_shape = 9,
+    dnnl_invalid_data_type = 10
+} dnnl_status_t;
+
+/* dnnl_common_types.h:80-114 */
+typedef enum {
+    dnnl_data_type_undef = 0,
+    dnnl_f16 = 1,
+    dnnl_bf16 = 2,
+    dnnl_f32 = 3,
+    dnnl_s32 = 4,
+    dnnl_s8 = 5,
+    dnnl_u8 = 6,
+    dnnl_f64 = 7,
+    dnnl_boolean = 8,
+    dnnl_f8_e5m2 = 9,
+    dnnl_f8_e4m3 = 10,
+    dnnl_s4 = 11,
+    dnnl_u4 = 12,
+    dnnl_e8m0 = 13,
+    dnnl_f4_e2m1 = 14
+} dnnl_data_type_t;
+
+#define DNNL_MAX_NDIMS 12                  /* dnnl_common_types.h:123 */
+typedef int64_t dnnl_dim_t;                /* dnnl_common_types.h:126 */
+typedef dnnl_dim_t dnnl_dims_t[DNNL_MAX_NDIMS];
+#define DNNL_RUNTIME_DIM_VAL INT64_MIN     /* dnnl_types.h:2331 */
+
+/* dnnl_common_types.h:137-148 */
+typedef enum {
+    dnnl_fpmath_mode_strict = 0,
+    dnnl_fpmath_mode_bf16,
+    dnnl_fpmath_mode_f16,
+    dnnl_fpmath_mode_any,
+    dnnl_fpmath_mode_tf32
+} dnnl_fpmath_mode_t;
+
+/* dnnl_common_types.h:157-170 */
+typedef enum {
+    dnnl_accumulation_mode_strict = 0,
+    dnnl_accumulation_mode_relaxed,
+    dnnl_accumulation_mode_any,
+    dnnl_accumulation_mode_s32,
+    dnnl_accumulation_mode_f32,
+    dnnl_accumulation_mode_f16
+} dnnl_accumulation_mode_t;
+
+/* dnnl_common_types.h:180-187 */
+typedef enum { dnnl_any_engine = 0, dnnl_cpu = 1, dnnl_gpu = 2 } dnnl_engine_kind_t;
+
+/* dnnl_common_types.h:206-213 */
+typedef enum {
+    dnnl_stream_in_order = 0x1U,
+    dnnl_stream_out_of_order = 0x2U,
+    dnnl_stream_default_flags = dnnl_stream_in_order
+} dnnl_stream_flags_t;
+
+#define DNNL_MEMORY_NONE (NULL)                    /* dnnl_common_types.h:253 */
+#define DNNL_MEMORY_ALLOCATE ((void *)(size_t)-1)  /* dnnl_common_types.h:257 */
+
+/* dnnl_types.h:45-63 */
+typedef enum {
+    dnnl_format_kind_undef = 0,
+    dnnl_format_kind_any,
+    dnnl_blocked,
+    dnnl_format_kind_opaque
+} dnnl_format_kind_t;
+
+/* dnnl_types.h:175-209: only the plain tags with at most four dimensions */
+typedef enum {
+    dnnl_format_tag_undef = 0,
+    dnnl_format_tag_any = 1,
+    dnnl_a = 2,
+    dnnl_ab = 3,
+    dnnl_abc = 4,
+    dnnl_abcd = 5,
+    dnnl_ba = 14,
+    dnnl_acb = 15,
+    dnnl_abdc = 20
+} dnnl_format_tag_t;
+
+/* dnnl_types.h:2057-2101 */
+typedef enum {
+    dnnl_undefined_primitive = 0,
+    dnnl_sum = 4,
+    dnnl_eltwise = 7,
+    dnnl_binary = 13,
+    dnnl_matmul = 14,
+    dnnl_prelu = 18
+} dnnl_primitive_kind_t;
+
+/* dnnl_types.h:2110-2230: the eltwise and binary algorithms post-ops admit */
+typedef enum {
+    dnnl_alg_kind_undef = 0,
+    dnnl_eltwise_relu = 0x20,
+    dnnl_eltwise_tanh,
+    dnnl_eltwise_elu,
+    dnnl_eltwise_square,
+    dnnl_eltwise_abs,
+    dnnl_eltwise_sqrt,
+    dnnl_eltwise_linear,
+    dnnl_eltwise_soft_relu,
+    dnnl_eltwise_hardsigmoid,
+    dnnl_eltwise_logistic,
+    dnnl_eltwise_exp,
+    dnnl_eltwise_gelu_tanh,
+    dnnl_eltwise_swish,
+    dnnl_eltwise_log,
+    dnnl_eltwise_clip,
+    dnnl_eltwise_clip_v2,
+    dnnl_eltwise_pow,
+    dnnl_eltwise_gelu_erf,
+    dnnl_eltwise_round,
+    dnnl_eltwise_mish,
+    dnnl_eltwise_hardswish,
+    dnnl_binary_add = 0x1fff0,
+    dnnl_binary_mul = 0x1fff1,
+    dnnl_binary_max = 0x1fff2,
+    dnnl_binary_min = 0x1fff3,
+    dnnl_binary_div = 0x1fff4,
+    dnnl_binary_sub = 0x1fff5,
+    dnnl_binary_ge = 0x1fff6,
+    dnnl_binary_gt = 0x1fff7,
+    dnnl_binary_le = 0x1fff8,
+    dnnl_binary_lt = 0x1fff9,
+    dnnl_binary_eq = 0x1fffa,
+    dnnl_binary_ne = 0x1fffb
+} dnnl_alg_kind_t;
+
+/* dnnl_types.h:2448-2458 */
+typedef enum { dnnl_scratchpad_mode_library = 0, dnnl_scratchpad_mode_user = 1 } dnnl_scratchpad_mode_t;
+
+/* dnnl_types.h:2846-2930 */
+typedef enum {
+    dnnl_query_undef = 0,
+    dnnl_query_engine = 1,
+    dnnl_query_primitive_kind = 2,
+    dnnl_query_num_of_inputs_s32 = 3,
+    dnnl_query_num_of_outputs_s32 = 4,
+    dnnl_query_memory_consumption_s64 = 6,
+    dnnl_query_impl_info_str = 8,
+    dnnl_query_prop_kind = 11,
+    dnnl_query_strides = 14,
+    dnnl_query_src_md = 129,
+    dnnl_query_weights_md = 131,
+    dnnl_query_dst_md = 133,
+    dnnl_query_scratchpad_md = 136,
+    dnnl_query_exec_arg_md = 255,
+    dnnl_query_ndims_s32 = 256,
+    dnnl_query_dims = 257,
+    dnnl_query_data_type = 258,
+    dnnl_query_format_kind = 262
+} dnnl_query_t;
+
+/* execute argument ids, dnnl_types.h:2544-2784 */
+#define DNNL_ARG_SRC 1
+#define DNNL_ARG_SRC_1 2
+#define DNNL_ARG_DST 17
+#define DNNL_ARG_WEIGHTS 33
+#define DNNL_ARG_BIAS 41
+#define DNNL_ARG_SCRATCHPAD 80
+#define DNNL_ARG_ATTR_PRECOMPUTED_REDUCTIONS 512
+#define DNNL_ARG_ATTR_SCALES 4096
+#define DNNL_ARG_ATTR_ZERO_POINTS 8192
+#define DNNL_ARG_ATTR_MULTIPLE_POST_OP_BASE 32768
+#define DNNL_ARG_ATTR_MULTIPLE_POST_OP(idx) (DNNL_ARG_ATTR_MULTIPLE_POST_OP_BASE * ((idx) + 1))
+
+/* opaque handles, dnnl_common_types.h / dnnl_types.h */
+typedef struct dnnl_engine *dnnl_engine_t;
+typedef struct dnnl_stream *dnnl_stream_t;
+typedef struct dnnl_memory_desc *dnnl_memory_desc_t;
+typedef const struct dnnl_memory_desc *const_dnnl_memory_desc_t;
+typedef struct dnnl_memory *dnnl_memory_t;
+typedef const struct dnnl_memory *const_dnnl_memory_t;
+typedef struct dnnl_primitive_attr *dnnl_primitive_attr_t;
+typedef const struct dnnl_primitive_attr *const_dnnl_primitive_attr_t;
+typedef struct dnnl_post_ops *dnnl_post_ops_t;
+typedef const struct dnnl_post_ops *const_dnnl_post_ops_t;
+typedef struct dnnl_primitive_desc *dnnl_primitive_desc_t;
+typedef const struct dnnl_primitive_desc *const_dnnl_primitive_desc_t;
+typedef struct dnnl_primitive *dnnl_primitive_t;
+typedef const struct dnnl_primitive *const_dnnl_primitive_t;
+
+/* dnnl_types.h:2791-2794 */
+typedef struct {
+    int arg;
+    dnnl_memory_t memory;
+} dnnl_exec_arg_t;
+
+/* ---- engine and stream: dnnl_common.h:54-109 ---- */
+dnnl_status_t dnnl_engine_create(dnnl_engine_t *engine, dnnl_engine_kind_t kind, size_t index);
+dnnl_status_t dnnl_engine_get_kind(dnnl_engine_t engine, dnnl_engine_kind_t *kind);
+dnnl_status_t dnnl_engine_destroy(dnnl_engine_t engine);
+size_t dnnl_engine_get_count(dnnl_engine_kind_t kind);
+dnnl_status_t dnnl_stream_create(dnnl_stream_t *stream, dnnl_engine_t engine, unsigned flags);
+dnnl_status_t dnnl_stream_get_engine(dnnl_stream_t stream, dnnl_engine_t *engine);
+dnnl_status_t dnnl_stream_wait(dnnl_stream_t stream);
+dnnl_status_t dnnl_stream_destroy(dnnl_stream_t stream);
+
+/* ---- memory descriptors: dnnl.h:1018-1424 ---- */
+dnnl_status_t dnnl_memory_desc_create_with_strides(dnnl_memory_desc_t *memory_desc, int ndims,
+        const dnnl_dims_t dims, dnnl_data_type_t data_type, const dnnl_dims_t strides);
+dnnl_status_t dnnl_memory_desc_create_with_tag(dnnl_memory_desc_t *memory_desc, int ndims,
+        const dnnl_dims_t dims, dnnl_data_type_t data_type, dnnl_format_tag_t tag);
+dnnl_status_t dnnl_memory_desc_clone(dnnl_memory_desc_t *memory_desc, const_dnnl_memory_desc_t existing);
+dnnl_status_t dnnl_memory_desc_destroy(dnnl_memory_desc_t memory_desc);
+dnnl_status_t dnnl_memory_desc_query(const_dnnl_memory_desc_t memory_desc, dnnl_query_t what, void *result);
+int dnnl_memory_desc_equal(const_dnnl_memory_desc_t lhs, const_dnnl_memory_desc_t rhs);
+size_t dnnl_memory_desc_get_size(const_dnnl_memory_desc_t memory_desc);
+size_t dnnl_data_type_size(dnnl_data_type_t data_type);
+
+/* ---- memory objects: dnnl.h:1482-1705 ---- */
+dnnl_status_t dnnl_memory_create(dnnl_memory_t *memory, const_dnnl_memory_desc_t memory_desc,
+        dnnl_engine_t engine, void *handle);
+dnnl_status_t dnnl_memory_get_memory_desc(const_dnnl_memory_t memory, const_dnnl_memory_desc_t *memory_desc);
+dnnl_status_t dnnl_memory_get_engine(const_dnnl_memory_t memory, dnnl_engine_t *engine);
+dnnl_status_t dnnl_memory_map_data(const_dnnl_memory_t memory, void **mapped_ptr);
+dnnl_status_t dnnl_memory_unmap_data(const_dnnl_memory_t memory, void *mapped_ptr);
+dnnl_status_t dnnl_memory_get_data_handle(const_dnnl_memory_t memory, void **handle);
+dnnl_status_t dnnl_memory_set_data_handle(dnnl_memory_t memory, void *handle);
+dnnl_status_t dnnl_memory_destroy(dnnl_memory_t memory);
+
+/* ---- attributes: dnnl.h:340-720 ---- */
+dnnl_status_t dnnl_primitive_attr_create(dnnl_primitive_attr_t *attr);
+dnnl_status_t dnnl_primitive_attr_clone(dnnl_primitive_attr_t *attr, const_dnnl_primitive_attr_t existing_attr);
+dnnl_status_t dnnl_primitive_attr_destroy(dnnl_primitive_attr_t attr);
+dnnl_status_t dnnl_primitive_attr_set_fpmath_mode(dnnl_primitive_attr_t attr, dnnl_fpmath_mode_t mode);
+dnnl_status_t dnnl_primitive_attr_set_fpmath_mode_v2(dnnl_primitive_attr_t attr, dnnl_fpmath_mode_t mode,
+        int apply_to_int);
+dnnl_status_t dnnl_primitive_attr_get_fpmath_mode_v2(const_dnnl_primitive_attr_t attr,
+        dnnl_fpmath_mode_t *mode, int *apply_to_int);
+dnnl_status_t dnnl_primitive_attr_set_accumulation_mode(dnnl_primitive_attr_t attr, dnnl_accumulation_mode_t mode);
+dnnl_status_t dnnl_primitive_attr_set_scratchpad_mode(dnnl_primitive_attr_t attr, dnnl_scratchpad_mode_t mode);
+dnnl_status_t dnnl_primitive_attr_get_scratchpad_mode(const_dnnl_primitive_attr_t attr,
+        dnnl_scratchpad_mode_t *mode);
+dnnl_status_t dnnl_primitive_attr_set_scales_mask(dnnl_primitive_attr_t attr, int arg, int mask);
+dnnl_status_t dnnl_primitive_attr_set_scales(dnnl_primitive_attr_t attr, int arg, int mask, int group_ndims,
+        const dnnl_dims_t group_dims, dnnl_data_type_t data_type);
+dnnl_status_t dnnl_primitive_attr_set_zero_points_mask(dnnl_primitive_attr_t attr, int arg, int mask);
+dnnl_status_t dnnl_primitive_attr_set_zero_points(dnnl_primitive_attr_t attr, int arg, int mask,
+        int group_ndims, const dnnl_dims_t group_dims, dnnl_data_type_t data_type);
+dnnl_status_t dnnl_primitive_attr_set_precomputed_reductions(dnnl_primitive_attr_t attr, int arg, int mask,
+        int group_ndims, const dnnl_dims_t group_dims, dnnl_data_type_t data_type);
+dnnl_status_t dnnl_primitive_attr_set_post_ops(dnnl_primitive_attr_t attr, const_dnnl_post_ops_t post_ops);
+dnnl_status_t dnnl_primitive_attr_get_post_ops(const_dnnl_primitive_attr_t attr, const_dnnl_post_ops_t *post_ops);
+
+/* ---- post-ops: dnnl.h:730-960 ---- */
+dnnl_status_t dnnl_post_ops_create(dnnl_post_ops_t *post_ops);
+dnnl_status_t dnnl_post_ops_clone(dnnl_post_ops_t *post_ops, const_dnnl_post_ops_t existing_post_ops);
+dnnl_status_t dnnl_post_ops_destroy(dnnl_post_ops_t post_ops);
+int dnnl_post_ops_len(const_dnnl_post_ops_t post_ops);
+dnnl_primitive_kind_t dnnl_post_ops_get_kind(const_dnnl_post_ops_t post_ops, int index);
+dnnl_status_t dnnl_post_ops_append_sum(dnnl_post_ops_t post_ops, float scale, int32_t zero_point,
+        dnnl_data_type_t data_type);
+dnnl_status_t dnnl_post_ops_get_params_sum(const_dnnl_post_ops_t post_ops, int index, float *scale,
+        int32_t *zero_point, dnnl_data_type_t *data_type);
+dnnl_status_t dnnl_post_ops_append_eltwise(dnnl_post_ops_t post_ops, dnnl_alg_kind_t alg_kind, float alpha,
+        float beta);
+dnnl_status_t dnnl_post_ops_get_params_eltwise(const_dnnl_post_ops_t post_ops, int index,
+        dnnl_alg_kind_t *alg_kind, float *alpha, float *beta);
+dnnl_status_t dnnl_post_ops_append_binary(dnnl_post_ops_t post_ops, dnnl_alg_kind_t alg_kind,
+        const_dnnl_memory_desc_t src1_desc);
+dnnl_status_t dnnl_post_ops_get_params_binary(const_dnnl_post_ops_t post_ops, int index,
+        dnnl_alg_kind_t *alg_kind, const_dnnl_memory_desc_t *src1_desc);
+dnnl_status_t dnnl_post_ops_append_prelu(dnnl_post_ops_t post_ops, int mask);
+dnnl_status_t dnnl_post_ops_get_params_prelu(const_dnnl_post_ops_t post_ops, int index, int *mask);
+
+/* ---- matmul primitive descriptor: dnnl.h:3774-3779 ---- */
+dnnl_status_t dnnl_matmul_primitive_desc_create(dnnl_primitive_desc_t *primitive_desc, dnnl_engine_t engine,
+        const_dnnl_memory_desc_t src_desc, const_dnnl_memory_desc_t weights_desc,
+        const_dnnl_memory_desc_t bias_desc, const_dnnl_memory_desc_t dst_desc,
+        const_dnnl_primitive_attr_t attr);
+
+/* ---- primitive descriptors and primitives: dnnl.h:60-243 ---- */
+dnnl_status_t dnnl_primitive_desc_clone(dnnl_primitive_desc_t *primitive_desc,
+        const_dnnl_primitive_desc_t existing_primitive_desc);
+dnnl_status_t dnnl_primitive_desc_next_impl(dnnl_primitive_desc_t primitive_desc);
+dnnl_status_t dnnl_primitive_desc_get_attr(const_dnnl_primitive_desc_t primitive_desc,
+        const_dnnl_primitive_attr_t *attr);
+dnnl_status_t dnnl_primitive_desc_destroy(dnnl_primitive_desc_t primitive_desc);
+dnnl_status_t dnnl_primitive_desc_query(const_dnnl_primitive_desc_t primitive_desc, dnnl_query_t what,
+        int index, void *result);
+const_dnnl_memory_desc_t dnnl_primitive_desc_query_md(const_dnnl_primitive_desc_t primitive_desc,
+        dnnl_query_t what, int index);
+dnnl_status_t dnnl_primitive_create(dnnl_primitive_t *primitive, const_dnnl_primitive_desc_t primitive_desc);
+dnnl_status_t dnnl_primitive_execute(const_dnnl_primitive_t primitive, dnnl_stream_t stream, int nargs,
+        const dnnl_exec_arg_t *args);
+dnnl_status_t dnnl_primitive_get_primitive_desc(const_dnnl_primitive_t primitive,
+        const_dnnl_primitive_desc_t *primitive_desc);
+dnnl_status_t dnnl_primitive_destroy(dnnl_primitive_t primitive);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* DNNL_AMD_H */

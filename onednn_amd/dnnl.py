@@ -1,0 +1,260 @@
+"""ctypes mirror of the dnnl_* C API subset (include/dnnl_amd.h), shaped after
+oneDNN's C++ wrappers (include/oneapi/dnnl/dnnl.hpp: engine, stream,
+memory::desc, memory, primitive_attr, post_ops, matmul::primitive_desc,
+matmul) so that tests read like the reference's.  Every status other than
+success raises `error`, as dnnl::error does.
+"""
+import ctypes as C
+import os
+
+import numpy as np
+
+from . import cabi
+
+_PKG_DIR = os.path.dirname(os.path.abspath(__file__))
+HOST_LIB_PATH = os.path.join(_PKG_DIR, "lib", "libdnnl_amd.so")
+_lib = None
+
+MAX_NDIMS = 12
+dims_t = C.c_int64 * MAX_NDIMS
+
+# enums (include/dnnl_amd.h)
+success, out_of_memory, invalid_arguments, unimplemented, last_impl_reached, runtime_error = range(6)
+cpu, gpu = 1, 2
+tag_any, tag_a, tag_ab, tag_abc, tag_abcd, tag_ba, tag_acb, tag_abdc = 1, 2, 3, 4, 5, 14, 15, 20
+kind_sum, kind_eltwise, kind_binary, kind_matmul, kind_prelu = 4, 7, 13, 14, 18
+query_impl_info_str, query_src_md, query_weights_md, query_dst_md, query_scratchpad_md = 8, 129, 131, 133, 136
+query_ndims_s32, query_dims, query_data_type, query_strides, query_memory_consumption = 256, 257, 258, 14, 6
+ARG_SRC, ARG_SRC_1, ARG_DST, ARG_WEIGHTS, ARG_BIAS, ARG_SCRATCHPAD = 1, 2, 17, 33, 41, 80
+ARG_ATTR_PRECOMPUTED_REDUCTIONS, ARG_ATTR_SCALES, ARG_ATTR_ZERO_POINTS = 512, 4096, 8192
+scratchpad_library, scratchpad_user = 0, 1
+fpmath_strict, fpmath_bf16, fpmath_f16, fpmath_any = 0, 1, 2, 3
+MEMORY_ALLOCATE = C.c_void_p(-1 & (2 ** 64 - 1))
+
+
+def ARG_ATTR_MULTIPLE_POST_OP(idx):
+    return 32768 * (idx + 1)
+
+
+class ExecArg(C.Structure):
+    _fields_ = [("arg", C.c_int), ("memory", C.c_void_p)]
+
+
+class error(RuntimeError):
+    def __init__(self, status, what):
+        super().__init__(f"{what}: status {status}")
+        self.status = status
+
+
+def lib():
+    global _lib
+    if _lib is None:
+        cabi.load_kernels()
+        if not os.path.exists(HOST_LIB_PATH):
+            raise ImportError(f"{HOST_LIB_PATH} is missing: build it with `make -C onednn_amd/host`")
+        _lib = C.CDLL(HOST_LIB_PATH)
+        _lib.dnnl_memory_desc_get_size.restype = C.c_size_t
+        _lib.dnnl_primitive_desc_query_md.restype = C.c_void_p
+        _lib.dnnl_engine_get_count.restype = C.c_size_t
+    return _lib
+
+
+def _check(st, what):
+    if st != success:
+        raise error(st, what)
+
+
+def _dims(seq):
+    a = dims_t()
+    for i, v in enumerate(seq):
+        a[i] = v
+    return a
+
+
+class engine:
+    def __init__(self, kind=gpu, index=0):
+        self.h = C.c_void_p()
+        _check(lib().dnnl_engine_create(C.byref(self.h), kind, C.c_size_t(index)), "engine_create")
+
+    def get_kind(self):
+        k = C.c_int()
+        _check(lib().dnnl_engine_get_kind(self.h, C.byref(k)), "engine_get_kind")
+        return k.value
+
+
+class stream:
+    def __init__(self, eng, flags=1):
+        self.engine = eng
+        self.h = C.c_void_p()
+        _check(lib().dnnl_stream_create(C.byref(self.h), eng.h, C.c_uint(flags)), "stream_create")
+
+    def wait(self):
+        _check(lib().dnnl_stream_wait(self.h), "stream_wait")
+
+
+class memory_desc:
+    def __init__(self, dims=None, dt=None, tag=None, strides=None, handle=None):
+        self.h = C.c_void_p()
+        self.owned = handle is None
+        if handle is not None:
+            self.h = C.c_void_p(handle)
+            return
+        nd = len(dims)
+        if strides is not None:
+            st = lib().dnnl_memory_desc_create_with_strides(C.byref(self.h), nd, _dims(dims), dt, _dims(strides))
+        else:
+            st = lib().dnnl_memory_desc_create_with_tag(C.byref(self.h), nd, _dims(dims), dt, tag)
+        _check(st, "memory_desc_create")
+
+    def get_size(self):
+        return lib().dnnl_memory_desc_get_size(self.h)
+
+    def ndims(self):
+        v = C.c_int32()
+        _check(lib().dnnl_memory_desc_query(self.h, query_ndims_s32, C.byref(v)), "md_query")
+        return v.value
+
+    def _vec(self, what):
+        p = C.POINTER(dims_t)()
+        _check(lib().dnnl_memory_desc_query(self.h, what, C.byref(p)), "md_query")
+        return list(p.contents[: self.ndims()])
+
+    def dims(self):
+        return self._vec(query_dims)
+
+    def strides(self):
+        return self._vec(query_strides)
+
+    def data_type(self):
+        v = C.c_int()
+        _check(lib().dnnl_memory_desc_query(self.h, query_data_type, C.byref(v)), "md_query")
+        return v.value
+
+
+class memory:
+    """Device memory; `data` (numpy, raw storage) is uploaded through map/unmap."""
+
+    def __init__(self, md, eng, data=None):
+        self.md, self.engine = md, eng
+        self.h = C.c_void_p()
+        _check(lib().dnnl_memory_create(C.byref(self.h), md.h, eng.h, MEMORY_ALLOCATE), "memory_create")
+        if data is not None:
+            self.write(data)
+
+    def write(self, data):
+        data = np.ascontiguousarray(data)
+        p = C.c_void_p()
+        _check(lib().dnnl_memory_map_data(self.h, C.byref(p)), "memory_map_data")
+        n = self.md.get_size()
+        assert data.nbytes <= n, (data.nbytes, n)
+        if data.nbytes:
+            C.memmove(p, data.ctypes.data, data.nbytes)
+        _check(lib().dnnl_memory_unmap_data(self.h, p), "memory_unmap_data")
+
+    def read(self, dtype):
+        p = C.c_void_p()
+        _check(lib().dnnl_memory_map_data(self.h, C.byref(p)), "memory_map_data")
+        n = self.md.get_size()
+        out = np.empty(n // np.dtype(dtype).itemsize, dtype=dtype)
+        if n:
+            C.memmove(out.ctypes.data, p, n)
+        _check(lib().dnnl_memory_unmap_data(self.h, p), "memory_unmap_data")
+        return out
+
+
+class post_ops:
+    def __init__(self):
+        self.h = C.c_void_p()
+        _check(lib().dnnl_post_ops_create(C.byref(self.h)), "post_ops_create")
+
+    def append_eltwise(self, alg, alpha=0.0, beta=0.0):
+        _check(lib().dnnl_post_ops_append_eltwise(self.h, alg, C.c_float(alpha), C.c_float(beta)), "append_eltwise")
+
+    def append_binary(self, alg, src1_md):
+        _check(lib().dnnl_post_ops_append_binary(self.h, alg, src1_md.h), "append_binary")
+
+    def append_sum(self, scale=1.0, zero_point=0, dt=0):
+        _check(lib().dnnl_post_ops_append_sum(self.h, C.c_float(scale), C.c_int32(zero_point), dt), "append_sum")
+
+    def append_prelu(self, mask):
+        _check(lib().dnnl_post_ops_append_prelu(self.h, mask), "append_prelu")
+
+    def len(self):
+        return lib().dnnl_post_ops_len(self.h)
+
+    def kind(self, i):
+        return lib().dnnl_post_ops_get_kind(self.h, i)
+
+
+class primitive_attr:
+    def __init__(self):
+        self.h = C.c_void_p()
+        _check(lib().dnnl_primitive_attr_create(C.byref(self.h)), "attr_create")
+
+    def set_scales_mask(self, arg, mask):
+        _check(lib().dnnl_primitive_attr_set_scales_mask(self.h, arg, mask), "set_scales_mask")
+
+    def set_scales(self, arg, mask, groups=(), dt=cabi.DT_F32):
+        _check(lib().dnnl_primitive_attr_set_scales(self.h, arg, mask, len(groups), _dims(groups), dt), "set_scales")
+
+    def set_zero_points_mask(self, arg, mask):
+        _check(lib().dnnl_primitive_attr_set_zero_points_mask(self.h, arg, mask), "set_zero_points_mask")
+
+    def set_zero_points(self, arg, mask, groups=(), dt=cabi.DT_S32):
+        _check(lib().dnnl_primitive_attr_set_zero_points(self.h, arg, mask, len(groups), _dims(groups), dt),
+               "set_zero_points")
+
+    def set_precomputed_reductions(self, arg, mask, groups=(), dt=cabi.DT_S32):
+        _check(lib().dnnl_primitive_attr_set_precomputed_reductions(self.h, arg, mask, len(groups), _dims(groups), dt),
+               "set_precomputed_reductions")
+
+    def set_fpmath_mode(self, mode, apply_to_int=False):
+        _check(lib().dnnl_primitive_attr_set_fpmath_mode_v2(self.h, mode, int(apply_to_int)), "set_fpmath_mode")
+
+    def set_post_ops(self, po):
+        _check(lib().dnnl_primitive_attr_set_post_ops(self.h, po.h), "set_post_ops")
+
+    def set_scratchpad_mode(self, mode):
+        _check(lib().dnnl_primitive_attr_set_scratchpad_mode(self.h, mode), "set_scratchpad_mode")
+
+
+class matmul_primitive_desc:
+    def __init__(self, eng, src_md, weights_md, dst_md, bias_md=None, attr=None):
+        self.engine = eng
+        self.h = C.c_void_p()
+        _check(lib().dnnl_matmul_primitive_desc_create(
+            C.byref(self.h), eng.h, src_md.h, weights_md.h, bias_md.h if bias_md else None, dst_md.h,
+            attr.h if attr else None), "matmul_primitive_desc_create")
+
+    def impl_info_str(self):
+        s = C.c_char_p()
+        _check(lib().dnnl_primitive_desc_query(self.h, query_impl_info_str, 0, C.byref(s)), "pd_query")
+        return s.value.decode()
+
+    def next_impl(self):
+        st = lib().dnnl_primitive_desc_next_impl(self.h)
+        if st == last_impl_reached:
+            return False
+        _check(st, "next_impl")
+        return True
+
+    def query_md(self, what, index=0):
+        p = lib().dnnl_primitive_desc_query_md(self.h, what, index)
+        return memory_desc(handle=p) if p else None
+
+    def scratchpad_desc(self):
+        return self.query_md(query_scratchpad_md)
+
+
+class matmul:
+    def __init__(self, pd):
+        self.pd = pd
+        self.h = C.c_void_p()
+        _check(lib().dnnl_primitive_create(C.byref(self.h), pd.h), "primitive_create")
+
+    def execute(self, strm, args):
+        arr = (ExecArg * len(args))()
+        for i, (k, m) in enumerate(args.items()):
+            arr[i].arg = k
+            arr[i].memory = m.h
+        _check(lib().dnnl_primitive_execute(self.h, strm.h, len(args), arr), "primitive_execute")

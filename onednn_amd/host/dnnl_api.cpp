@@ -1,0 +1,1218 @@
+// Host side of the drop-in: the subset of oneDNN's C API that the matmul
+// primitive needs (include/dnnl_amd.h), implemented over the thin C ABI of the
+// HIP kernels (include/mi355_matmul.h).  No HIP headers here: device memory,
+// streams and launches all go through mi355_* calls.
+//
+// What is restated from the reference (uxlfoundation/oneDNN v3.14):
+//   matmul_desc_init            src/common/matmul.cpp:630-744   (shape rules)
+//   matmul_attr_check           src/common/matmul.cpp:261-624   (attribute legality)
+//   matmul_pd_t::attr_*_ok      src/common/matmul_pd.hpp:209-397
+//   attribute setters' checks   src/common/primitive_attr.cpp:623-720
+//   default_accum_data_type     src/common/type_helpers.hpp:515-551
+//   pd iteration / next_impl    src/common/primitive_desc_iterator.hpp:37-95
+//   execute-argument mapping    src/common/primitive_iface.cpp:244-274,
+//                               src/common/matmul_pd.hpp:74-93
+// Validation failures return dnnl_invalid_arguments, legal-but-unsupported
+// requests dnnl_unimplemented, device failures dnnl_runtime_error, as there.
+#include <stdio.h>
+#include <stdlib.h>
+#include <string.h>
+
+#include <atomic>
+#include <chrono>
+#include <map>
+#include <memory>
+#include <mutex>
+#include <string>
+#include <vector>
+
+#include "../../include/dnnl_amd.h"
+#include "../../include/mi355_matmul.h"
+
+#define DNNL_EXPORT extern "C" __attribute__((visibility("default")))
+
+namespace {
+
+using dim_t = dnnl_dim_t;
+
+int verbose_level() {
+    static int lvl = [] {
+        const char *e = getenv("ONEDNN_VERBOSE");
+        if (!e) e = getenv("DNNL_VERBOSE");
+        if (!e) return 0;
+        if (!strcmp(e, "all") || !strcmp(e, "profile") || !strcmp(e, "profile_exec")) return 2;
+        return atoi(e);
+    }();
+    return lvl;
+}
+
+dnnl_status_t from_mi355(int st) {
+    switch (st) {
+        case MI355_SUCCESS: return dnnl_success;
+        case MI355_OUT_OF_MEMORY: return dnnl_out_of_memory;
+        case MI355_INVALID_ARGUMENTS: return dnnl_invalid_arguments;
+        case MI355_UNIMPLEMENTED: return dnnl_unimplemented;
+        default: return dnnl_runtime_error;
+    }
+}
+
+bool dt_valid(int dt) {
+    return dt >= dnnl_f16 && dt <= dnnl_f4_e2m1 && dt != dnnl_f64 && dt != dnnl_boolean;
+}
+int dt_bits(int dt) {
+    switch (dt) {
+        case dnnl_f32:
+        case dnnl_s32: return 32;
+        case dnnl_f16:
+        case dnnl_bf16: return 16;
+        case dnnl_s4:
+        case dnnl_u4:
+        case dnnl_f4_e2m1: return 4;
+        case dnnl_f64: return 64;
+        default: return 8;
+    }
+}
+bool is_int_dt(int dt) { return dt == dnnl_s8 || dt == dnnl_u8 || dt == dnnl_s4 || dt == dnnl_u4 || dt == dnnl_s32; }
+bool is_int8(int dt) { return dt == dnnl_s8 || dt == dnnl_u8; }
+bool is_fp8(int dt) { return dt == dnnl_f8_e4m3 || dt == dnnl_f8_e5m2; }
+const char *dt_name(int dt) {
+    static const char *n[] = {"undef", "f16", "bf16", "f32", "s32", "s8", "u8", "f64", "bool", "f8_e5m2",
+            "f8_e4m3", "s4", "u4", "e8m0", "f4_e2m1"};
+    return (dt >= 0 && dt <= 14) ? n[dt] : "?";
+}
+
+} // namespace
+
+// ------------------------------------------------------------------ objects
+struct dnnl_engine {
+    dnnl_engine_kind_t kind;
+    size_t index;
+};
+
+struct dnnl_stream {
+    dnnl_engine_t engine;
+    void *hip_stream;
+};
+
+struct dnnl_memory_desc {
+    int ndims = 0;
+    dnnl_dims_t dims = {};
+    dnnl_dims_t strides = {};
+    dnnl_data_type_t dt = dnnl_data_type_undef;
+    dnnl_format_kind_t kind = dnnl_format_kind_undef;
+
+    bool is_zero() const { return ndims == 0; }
+    dim_t nelems() const {
+        if (ndims == 0) return 0;
+        dim_t n = 1;
+        for (int i = 0; i < ndims; ++i) n *= dims[i];
+        return n;
+    }
+    // logical elements the buffer spans (last offset + 1)
+    dim_t span() const {
+        if (ndims == 0 || nelems() == 0) return 0;
+        dim_t off = 0;
+        for (int i = 0; i < ndims; ++i) off += (dims[i] - 1) * strides[i];
+        return off + 1;
+    }
+    size_t size_bytes() const {
+        const dim_t s = span();
+        return dt_bits(dt) == 4 ? (size_t)(s + 1) / 2 : (size_t)s * (dt_bits(dt) / 8);
+    }
+    void set_dense() {
+        dim_t s = 1;
+        for (int i = ndims - 1; i >= 0; --i) {
+            strides[i] = s;
+            s *= dims[i] == 0 ? 1 : dims[i];
+        }
+        kind = dnnl_blocked;
+    }
+    bool operator==(const dnnl_memory_desc &o) const {
+        if (ndims != o.ndims || dt != o.dt || kind != o.kind) return false;
+        for (int i = 0; i < ndims; ++i)
+            if (dims[i] != o.dims[i] || (kind == dnnl_blocked && strides[i] != o.strides[i])) return false;
+        return true;
+    }
+};
+
+struct dnnl_memory {
+    dnnl_memory_desc md;
+    dnnl_engine_t engine;
+    void *handle = nullptr;
+    bool owned = false;
+    void *mapped = nullptr; // host staging buffer while mapped
+};
+
+namespace {
+struct quant_entry_t {
+    int mask = 0;
+    dnnl_data_type_t dt = dnnl_data_type_undef;
+    int group_ndims = 0;
+    dim_t groups[2] = {1, 1};
+    dim_t group(int d) const { return group_ndims == 0 ? 1 : groups[d]; }
+};
+
+struct post_op_entry_t {
+    dnnl_primitive_kind_t kind = dnnl_undefined_primitive;
+    dnnl_alg_kind_t alg = dnnl_alg_kind_undef;
+    float alpha = 0.f, beta = 0.f, scale = 1.f;
+    int32_t zero_point = 0;
+    dnnl_data_type_t dt = dnnl_data_type_undef;
+    dnnl_memory_desc src1;
+    int mask = 0;
+};
+} // namespace
+
+struct dnnl_post_ops {
+    std::vector<post_op_entry_t> entries;
+};
+
+struct dnnl_primitive_attr {
+    std::map<int, quant_entry_t> scales, zero_points, reductions;
+    dnnl_fpmath_mode_t fpmath = dnnl_fpmath_mode_strict;
+    int apply_to_int = 0;
+    dnnl_accumulation_mode_t acc_mode = dnnl_accumulation_mode_strict;
+    dnnl_scratchpad_mode_t scratchpad_mode = dnnl_scratchpad_mode_library;
+    dnnl_post_ops post_ops;
+    const quant_entry_t *find(const std::map<int, quant_entry_t> &m, int arg) const {
+        auto it = m.find(arg);
+        return it == m.end() ? nullptr : &it->second;
+    }
+};
+
+struct dnnl_primitive_desc {
+    dnnl_engine_t engine = nullptr;
+    dnnl_memory_desc src, wei, bias, dst, scratchpad;
+    bool with_bias = false;
+    dnnl_primitive_attr attr;
+    mi355_matmul_desc_t desc;     // impl field = the chosen kernel family
+    std::vector<int> impls;       // kernel families that can run it, best first
+    size_t impl_pos = 0;
+    size_t scratch_bytes = 0;
+    std::string impl_name;
+};
+
+struct dnnl_primitive {
+    dnnl_primitive_desc pd;
+    void *scratch = nullptr; // library-mode scratchpad (device)
+    std::mutex scratch_mutex;
+};
+
+namespace {
+
+#define CHECK_ARG(cond) \
+    do { \
+        if (!(cond)) return dnnl_invalid_arguments; \
+    } while (0)
+#define CHECK_UNIMPL(cond) \
+    do { \
+        if (!(cond)) return dnnl_unimplemented; \
+    } while (0)
+#define IMPLICATION(a, b) (!(a) || (b))
+
+// ------------------------------------------------------------ validation
+// matmul_desc_init, src/common/matmul.cpp:630-744
+dnnl_status_t check_shapes(const dnnl_memory_desc &s, const dnnl_memory_desc &w, const dnnl_memory_desc *b,
+        const dnnl_memory_desc &d) {
+    const int nd = d.ndims;
+    CHECK_ARG(nd >= 2 && nd <= DNNL_MAX_NDIMS);
+    CHECK_ARG(s.ndims == nd && w.ndims == nd);
+    CHECK_ARG(IMPLICATION(b, b->ndims == nd));
+    const int mi = nd - 2, ni = nd - 1;
+    CHECK_ARG(d.dims[mi] == s.dims[mi]);
+    CHECK_ARG(d.dims[ni] == w.dims[ni]);
+    CHECK_ARG(s.dims[ni] == w.dims[mi]);
+    if (b) {
+        CHECK_ARG(b->dims[ni] == 1 || b->dims[ni] == d.dims[ni]);
+        CHECK_ARG(b->dims[mi] == 1 || b->dims[mi] == d.dims[mi]);
+    }
+    for (int i = 0; i < nd - 2; ++i) {
+        const dim_t sd = s.dims[i], wd = w.dims[i], dd = d.dims[i];
+        const bool all_eq = sd == wd && wd == dd;
+        CHECK_ARG(IMPLICATION(!all_eq, sd == 1 || wd == 1));
+        CHECK_ARG(IMPLICATION(sd == 1, dd == wd));
+        CHECK_ARG(IMPLICATION(wd == 1, dd == sd));
+        if (b) CHECK_ARG(b->dims[i] == 1 || b->dims[i] == dd);
+    }
+    return dnnl_success;
+}
+
+// default_accum_data_type, src/common/type_helpers.hpp:515-551 (forward)
+int accum_dt(int src, int wei, int dst) {
+    (void)dst;
+    if (is_int8(src) && (is_int8(wei) || wei == dnnl_s4 || wei == dnnl_u4)) return dnnl_s32;
+    if (src == dnnl_f64) return dnnl_f64;
+    return dnnl_f32;
+}
+
+// matmul_attr_check (src/common/matmul.cpp:261-624) plus the generic checks of
+// matmul_pd_t::attr_scales_ok / attr_zero_points_ok (matmul_pd.hpp:209-397)
+dnnl_status_t check_attr(const dnnl_memory_desc &s, const dnnl_memory_desc &w, const dnnl_memory_desc &d,
+        const dnnl_primitive_attr &a) {
+    const int nd = s.ndims;
+    const dim_t M = s.dims[nd - 2], K = w.dims[nd - 2], N = w.dims[nd - 1];
+    const int src_dt = s.dt, wei_dt = w.dt, dst_dt = d.dt;
+    const bool src_int8 = is_int8(src_dt), src_fp8 = is_fp8(src_dt), src_fp4 = src_dt == dnnl_f4_e2m1;
+    const bool wei_int = wei_dt == dnnl_s8 || wei_dt == dnnl_u8 || wei_dt == dnnl_s4 || wei_dt == dnnl_u4;
+    const bool wei_lowp = wei_int || is_fp8(wei_dt) || wei_dt == dnnl_f4_e2m1;
+    const int qM = 1 << (nd - 2), qK_src = 1 << (nd - 1);
+    const int qK_wei = 1 << (nd - 2), qN = 1 << (nd - 1);
+    const int full = (1 << nd) - 1;
+    auto divisible = [](dim_t g1, dim_t g2) { return IMPLICATION(g1 > 1 && g2 > 1, g1 % g2 == 0 || g2 % g1 == 0); };
+
+    // zero points and precomputed reductions only with low-precision src
+    // (weights zero points also serve weight decompression)
+    if (!a.zero_points.empty())
+        CHECK_UNIMPL(src_int8 || src_fp8 || src_fp4 || wei_int);
+    if (!a.reductions.empty()) CHECK_UNIMPL(src_int8);
+    for (auto &kv : a.scales)
+        CHECK_UNIMPL(kv.first == DNNL_ARG_SRC || kv.first == DNNL_ARG_WEIGHTS || kv.first == DNNL_ARG_DST);
+    for (auto &kv : a.zero_points)
+        CHECK_UNIMPL(kv.first == DNNL_ARG_SRC || kv.first == DNNL_ARG_WEIGHTS || kv.first == DNNL_ARG_DST);
+    for (auto &kv : a.reductions) CHECK_UNIMPL(kv.first == DNNL_ARG_SRC);
+
+    dim_t src_sg_k = 1, wei_sg_k = 1;
+    if (auto q = a.find(a.scales, DNNL_ARG_SRC)) {
+        CHECK_UNIMPL(q->mask == 0 || q->mask == qM || q->mask == qK_src || q->mask == qM + qK_src
+                || q->mask == full);
+        if (q->group_ndims && (q->mask & qK_src)) src_sg_k = q->group(1);
+        CHECK_UNIMPL(IMPLICATION(src_sg_k > 1 && src_sg_k < K, src_sg_k % 16 == 0));
+        // matmul_pd_t::attr_scales_ok
+        CHECK_UNIMPL(IMPLICATION(q->mask & qK_src, q->group_ndims != 0));
+        CHECK_UNIMPL(IMPLICATION(q->group_ndims, q->group(0) == 1));
+        CHECK_UNIMPL(IMPLICATION(q->group_ndims, K % q->group(1) == 0));
+        CHECK_UNIMPL(IMPLICATION(q->mask == qM, q->group_ndims == 0));
+        CHECK_UNIMPL(!wei_lowp ? q->group_ndims == 0 : true);
+    }
+    if (auto q = a.find(a.scales, DNNL_ARG_WEIGHTS)) {
+        dim_t gn = 1;
+        if (q->group_ndims) {
+            CHECK_UNIMPL(wei_lowp);
+            if (q->mask & qK_wei) wei_sg_k = q->group(0);
+            if (q->mask & qN) gn = q->group(1);
+            CHECK_UNIMPL(IMPLICATION(q->group(0) > 1, K % q->group(0) == 0));
+            CHECK_UNIMPL(IMPLICATION(q->group(1) > 1, N % q->group(1) == 0));
+        }
+        CHECK_UNIMPL(IMPLICATION(wei_sg_k > 1 && wei_sg_k < K, wei_sg_k % 16 == 0));
+        CHECK_UNIMPL(IMPLICATION(gn > 1 && gn < N, gn % 16 == 0));
+        // a K mask on integer weights only for weight decompression
+        if (is_int_dt(wei_dt)) {
+            const bool decomp = wei_int && IMPLICATION(!is_int_dt(src_dt), a.apply_to_int);
+            CHECK_UNIMPL(IMPLICATION(q->mask & qK_wei, decomp));
+        }
+    }
+    if (auto q = a.find(a.scales, DNNL_ARG_DST)) {
+        CHECK_UNIMPL(q->mask == 0 || q->mask == qN || q->mask == qM || q->mask == qM + qN || q->mask == full);
+        CHECK_UNIMPL(IMPLICATION(q->group_ndims, is_fp8(dst_dt) || dst_dt == dnnl_f4_e2m1));
+        CHECK_UNIMPL(IMPLICATION(q->group_ndims, M % q->group(0) == 0 && N % q->group(1) == 0));
+    }
+    CHECK_UNIMPL(IMPLICATION(src_sg_k > 1, (src_int8 || src_fp8 || src_fp4) && divisible(src_sg_k, wei_sg_k)));
+
+    dim_t src_zg_k = 1, wei_zg_k = 1;
+    if (auto q = a.find(a.zero_points, DNNL_ARG_SRC)) {
+        CHECK_UNIMPL(q->mask == 0 || q->mask == qK_src || q->mask == qM + qK_src || q->mask == full);
+        CHECK_UNIMPL(IMPLICATION(q->mask == full, nd <= 3));
+        CHECK_UNIMPL(IMPLICATION(q->mask == full && nd == 3, s.dims[0] == 1));
+        if (q->group_ndims && (q->mask & qK_src)) src_zg_k = q->group(1);
+        CHECK_UNIMPL(IMPLICATION(src_zg_k > 1 && src_zg_k < K, src_zg_k % 32 == 0));
+        CHECK_UNIMPL(IMPLICATION(q->group_ndims, q->group(0) == 1 && K % q->group(1) == 0));
+    }
+    if (auto q = a.find(a.zero_points, DNNL_ARG_WEIGHTS)) {
+        dim_t gn = 1;
+        if (q->group_ndims) {
+            CHECK_UNIMPL(wei_lowp);
+            if (q->mask & qK_wei) wei_zg_k = q->group(0);
+            if (q->mask & qN) gn = q->group(1);
+            CHECK_UNIMPL(IMPLICATION(q->group(0) > 1, K % q->group(0) == 0));
+            CHECK_UNIMPL(IMPLICATION(q->group(1) > 1, N % q->group(1) == 0));
+            CHECK_UNIMPL(q->group(0) == 1 || q->group(1) == 1); // one non-unit group
+        }
+        CHECK_UNIMPL(IMPLICATION(gn > 1, a.apply_to_int));
+        CHECK_UNIMPL(IMPLICATION(wei_zg_k > 1 && wei_zg_k < K, wei_zg_k % 16 == 0));
+        CHECK_UNIMPL(IMPLICATION(gn > 1 && gn < N, gn % 16 == 0));
+        if (q->dt == dnnl_s4 || q->dt == dnnl_u4) {
+            CHECK_UNIMPL(IMPLICATION(q->mask & qK_wei, K % 2 == 0));
+            CHECK_UNIMPL(IMPLICATION(q->mask & qN, N % 2 == 0));
+        }
+        CHECK_UNIMPL(q->dt == dnnl_s32 || wei_lowp); // non-s32 zero-point types need low-precision weights
+    }
+    if (auto q = a.find(a.zero_points, DNNL_ARG_DST)) {
+        CHECK_UNIMPL(q->mask == 0 || (d.ndims == 2 && q->mask == (1 << 1)));
+        CHECK_UNIMPL(q->group_ndims == 0);
+    }
+    CHECK_UNIMPL(IMPLICATION(src_zg_k > 1, src_int8 && divisible(src_zg_k, wei_zg_k)));
+
+    if (auto pr = a.find(a.reductions, DNNL_ARG_SRC)) {
+        CHECK_UNIMPL(a.find(a.zero_points, DNNL_ARG_WEIGHTS) != nullptr);
+        CHECK_UNIMPL(pr->mask == full);
+        CHECK_UNIMPL(pr->dt == dnnl_s32);
+        if (pr->group_ndims) {
+            const dim_t g = pr->group(1);
+            dim_t minimal = INT64_MAX;
+            dim_t wzk = 1;
+            if (auto q = a.find(a.zero_points, DNNL_ARG_WEIGHTS))
+                if (q->group_ndims) { wzk = q->group(0); minimal = std::min(minimal, wzk); }
+            if (auto q = a.find(a.zero_points, DNNL_ARG_SRC))
+                if (q->group_ndims) minimal = std::min(minimal, q->group(1));
+            if (auto q = a.find(a.scales, DNNL_ARG_WEIGHTS))
+                if (q->group_ndims) minimal = std::min(minimal, q->group(0));
+            if (auto q = a.find(a.scales, DNNL_ARG_SRC))
+                if (q->group_ndims) minimal = std::min(minimal, q->group(1));
+            CHECK_ARG(IMPLICATION(g > 1, src_int8));
+            CHECK_ARG(IMPLICATION(g > 1, divisible(g, wzk)));
+            CHECK_ARG(IMPLICATION(g > 1, g <= minimal));
+            CHECK_UNIMPL(pr->group(0) == 1 && K % g == 0);
+        }
+    }
+
+    // post-ops: binary, eltwise, prelu, sum (matmul.cpp:606-620)
+    int n_sum = 0;
+    for (auto &e : a.post_ops.entries) {
+        CHECK_UNIMPL(e.kind == dnnl_binary || e.kind == dnnl_eltwise || e.kind == dnnl_prelu || e.kind == dnnl_sum);
+        if (e.kind == dnnl_sum) {
+            ++n_sum;
+            // check_sum_consistency: same size as dst, zero point only for int8
+            CHECK_UNIMPL(IMPLICATION(e.dt != dnnl_data_type_undef, dt_bits(e.dt) == dt_bits(dst_dt)));
+            CHECK_UNIMPL(IMPLICATION(e.zero_point != 0, src_int8));
+        }
+        if (e.kind == dnnl_binary) {
+            CHECK_ARG(e.src1.ndims == d.ndims);
+            for (int i = 0; i < d.ndims; ++i) CHECK_ARG(e.src1.dims[i] == 1 || e.src1.dims[i] == d.dims[i]);
+        }
+    }
+    CHECK_UNIMPL(n_sum <= 1 || true);
+    return dnnl_success;
+}
+
+// ------------------------------------------------- lowering to the C ABI
+// Collapse the batch dims of one operand into a single stride: all broadcast
+// (stride 0) or all present and nested.
+bool collapse_batch(const dnnl_memory_desc &x, const dnnl_memory_desc &dst, int64_t *bstride) {
+    const int nb = dst.ndims - 2;
+    *bstride = 0;
+    if (nb == 0) return true;
+    bool all_one = true, all_full = true;
+    for (int i = 0; i < nb; ++i) {
+        if (x.dims[i] != 1) all_one = false;
+        if (x.dims[i] != dst.dims[i]) all_full = false;
+    }
+    dim_t total = 1;
+    for (int i = 0; i < nb; ++i) total *= dst.dims[i];
+    if (all_one && total > 1) return true; // broadcast
+    if (!all_full) return false;
+    for (int i = 0; i + 1 < nb; ++i)
+        if (x.dims[i + 1] != 1 && x.strides[i] != x.strides[i + 1] * x.dims[i + 1]) return false;
+    *bstride = x.strides[nb - 1];
+    if (total == 1) *bstride = 0;
+    return true;
+}
+
+bool lower_quant(const quant_entry_t *q, int nd, int default_dt, mi355_quant_t *out) {
+    out->dt = MI355_DT_UNDEF;
+    out->mask = 0;
+    out->group[0] = out->group[1] = 1;
+    if (!q) return true;
+    const int batch_bits = (1 << (nd - 2)) - 1;
+    const int bm = q->mask & batch_bits;
+    if (bm != 0 && bm != batch_bits) return false; // partial batch masks are not lowered
+    out->dt = q->dt == dnnl_data_type_undef ? default_dt : q->dt;
+    out->mask = (bm ? 1 : 0) | ((q->mask >> (nd - 2)) & 1) << 1 | ((q->mask >> (nd - 1)) & 1) << 2;
+    out->group[0] = q->group(0);
+    out->group[1] = q->group(1);
+    // a group on an unmasked dim carries no information
+    if (!(out->mask & 2)) out->group[0] = 1;
+    if (!(out->mask & 4)) out->group[1] = 1;
+    return true;
+}
+
+dnnl_status_t lower(dnnl_primitive_desc &pd) {
+    mi355_matmul_desc_t &D = pd.desc;
+    memset(&D, 0, sizeof(D));
+    const int nd = pd.dst.ndims;
+    dim_t batch = 1;
+    for (int i = 0; i < nd - 2; ++i) batch *= pd.dst.dims[i];
+    D.batch = batch;
+    D.M = pd.dst.dims[nd - 2];
+    D.N = pd.dst.dims[nd - 1];
+    D.K = pd.src.dims[nd - 1];
+    D.src_dt = pd.src.dt; D.wei_dt = pd.wei.dt; D.dst_dt = pd.dst.dt;
+    D.bias_dt = pd.with_bias ? (int)pd.bias.dt : (int)MI355_DT_UNDEF;
+    auto strides3 = [&](const dnnl_memory_desc &x, int64_t *out) -> bool {
+        if (!collapse_batch(x, pd.dst, &out[0])) return false;
+        out[1] = x.dims[nd - 2] == 1 && pd.dst.dims[nd - 2] != 1 && &x != &pd.src && &x != &pd.wei ? 0 : x.strides[nd - 2];
+        out[2] = x.dims[nd - 1] == 1 && pd.dst.dims[nd - 1] != 1 && &x != &pd.src && &x != &pd.wei ? 0 : x.strides[nd - 1];
+        return true;
+    };
+    CHECK_UNIMPL(strides3(pd.src, D.src_stride));
+    CHECK_UNIMPL(strides3(pd.wei, D.wei_stride));
+    CHECK_UNIMPL(strides3(pd.dst, D.dst_stride));
+    if (pd.with_bias) CHECK_UNIMPL(strides3(pd.bias, D.bias_stride));
+    const dnnl_primitive_attr &a = pd.attr;
+    CHECK_UNIMPL(lower_quant(a.find(a.scales, DNNL_ARG_SRC), nd, dnnl_f32, &D.src_scale));
+    CHECK_UNIMPL(lower_quant(a.find(a.scales, DNNL_ARG_WEIGHTS), nd, dnnl_f32, &D.wei_scale));
+    CHECK_UNIMPL(lower_quant(a.find(a.scales, DNNL_ARG_DST), nd, dnnl_f32, &D.dst_scale));
+    CHECK_UNIMPL(lower_quant(a.find(a.zero_points, DNNL_ARG_SRC), nd, dnnl_s32, &D.src_zp));
+    CHECK_UNIMPL(lower_quant(a.find(a.zero_points, DNNL_ARG_WEIGHTS), nd, dnnl_s32, &D.wei_zp));
+    CHECK_UNIMPL(lower_quant(a.find(a.zero_points, DNNL_ARG_DST), nd, dnnl_s32, &D.dst_zp));
+    CHECK_UNIMPL(lower_quant(a.find(a.reductions, DNNL_ARG_SRC), nd, dnnl_s32, &D.src_pr));
+    // dynamic (grouped) dst scales are not offered; dst scale is one value
+    CHECK_UNIMPL(D.dst_scale.dt == MI355_DT_UNDEF || D.dst_scale.mask == 0);
+    CHECK_UNIMPL(D.dst_zp.dt == MI355_DT_UNDEF || D.dst_zp.dt == MI355_DT_S32);
+    D.fpmath_apply_to_int = a.apply_to_int;
+    D.fpmath_mode = a.fpmath;
+    D.dst_scale_mode = MI355_DST_SCALE_DIVIDE;
+    if (const char *e = getenv("ONEDNN_AMD_DST_SCALE_RECIPROCAL"))
+        if (atoi(e)) D.dst_scale_mode = MI355_DST_SCALE_RECIPROCAL;
+    CHECK_UNIMPL(a.post_ops.entries.size() <= MI355_MAX_POST_OPS);
+    D.n_post_ops = (int)a.post_ops.entries.size();
+    for (int i = 0; i < D.n_post_ops; ++i) {
+        const post_op_entry_t &e = a.post_ops.entries[i];
+        mi355_post_op_t &o = D.post_ops[i];
+        o.alpha = e.alpha; o.beta = e.beta; o.scale = e.scale; o.zero_point = e.zero_point;
+        switch (e.kind) {
+            case dnnl_sum: o.kind = MI355_PO_SUM; o.dt = e.dt; break;
+            case dnnl_eltwise: o.kind = MI355_PO_ELTWISE; o.alg = e.alg; break;
+            case dnnl_binary: {
+                o.kind = MI355_PO_BINARY; o.alg = e.alg; o.dt = e.src1.dt;
+                int64_t st[3];
+                if (!collapse_batch(e.src1, pd.dst, &st[0])) return dnnl_unimplemented;
+                st[1] = e.src1.dims[nd - 2] == 1 ? 0 : e.src1.strides[nd - 2];
+                st[2] = e.src1.dims[nd - 1] == 1 ? 0 : e.src1.strides[nd - 1];
+                if (pd.dst.dims[nd - 2] == 1) st[1] = e.src1.strides[nd - 2];
+                if (pd.dst.dims[nd - 1] == 1) st[2] = e.src1.strides[nd - 1];
+                memcpy(o.stride, st, sizeof(st));
+            } break;
+            case dnnl_prelu: {
+                // weights are f32, dims = dst dims under the mask, dense row-major
+                o.kind = MI355_PO_PRELU; o.dt = dnnl_f32;
+                const int batch_bits = (1 << (nd - 2)) - 1;
+                const int bm = e.mask & batch_bits;
+                if (bm != 0 && bm != batch_bits) return dnnl_unimplemented;
+                const bool mm = (e.mask >> (nd - 2)) & 1, mn = (e.mask >> (nd - 1)) & 1;
+                const dim_t dn = mn ? D.N : 1, dm = mm ? D.M : 1;
+                o.stride[2] = mn ? 1 : 0;
+                o.stride[1] = mm ? dn : 0;
+                o.stride[0] = bm ? dm * dn : 0;
+            } break;
+            default: return dnnl_unimplemented;
+        }
+    }
+    D.impl = MI355_IMPL_AUTO;
+    return dnnl_success;
+}
+
+// implementation list of the HIP engine, best first (the role of
+// engine_t::get_implementation_list, src/common/engine.hpp:134-137)
+const int k_impl_list[] = {MI355_IMPL_WOQ_GEMV, MI355_IMPL_I8_MFMA, MI355_IMPL_F8_MFMA, MI355_IMPL_MXF4_MFMA,
+        MI355_IMPL_REF};
+
+dnnl_status_t select_impl(dnnl_primitive_desc &pd) {
+    pd.desc.impl = pd.impls[pd.impl_pos];
+    pd.impl_name = mi355_matmul_impl_name(pd.desc.impl);
+    size_t bytes = 0;
+    const int st = mi355_matmul_scratch_bytes(&pd.desc, &bytes);
+    if (st != MI355_SUCCESS) return from_mi355(st);
+    pd.scratch_bytes = bytes;
+    pd.scratchpad = dnnl_memory_desc();
+    if (pd.attr.scratchpad_mode == dnnl_scratchpad_mode_user && bytes > 0) {
+        pd.scratchpad.ndims = 1;
+        pd.scratchpad.dims[0] = (dim_t)bytes;
+        pd.scratchpad.dt = dnnl_u8;
+        pd.scratchpad.set_dense();
+    }
+    return dnnl_success;
+}
+
+} // namespace
+
+// ================================================================ C API
+DNNL_EXPORT dnnl_status_t dnnl_engine_create(dnnl_engine_t *engine, dnnl_engine_kind_t kind, size_t index) {
+    CHECK_ARG(engine);
+    // this library provides the GPU (HIP) engine only
+    CHECK_ARG(kind == dnnl_gpu);
+    int n = 0;
+    const int rc = mi355_device_count(&n);
+    // ONEDNN_AMD_ALLOW_NO_DEVICE=1: descriptor-only engine on a machine without
+    // a GPU (primitive descriptors can be created and queried, nothing executes)
+    const char *nodev = getenv("ONEDNN_AMD_ALLOW_NO_DEVICE");
+    if (!(nodev && atoi(nodev) && index == 0)) {
+        if (rc != MI355_SUCCESS) return dnnl_runtime_error;
+        CHECK_ARG((int)index < n);
+    }
+    *engine = new dnnl_engine {kind, index};
+    return dnnl_success;
+}
+DNNL_EXPORT size_t dnnl_engine_get_count(dnnl_engine_kind_t kind) {
+    if (kind != dnnl_gpu) return 0;
+    int n = 0;
+    if (mi355_device_count(&n) != MI355_SUCCESS) return 0;
+    return (size_t)n;
+}
+DNNL_EXPORT dnnl_status_t dnnl_engine_get_kind(dnnl_engine_t engine, dnnl_engine_kind_t *kind) {
+    CHECK_ARG(engine && kind);
+    *kind = engine->kind;
+    return dnnl_success;
+}
+DNNL_EXPORT dnnl_status_t dnnl_engine_destroy(dnnl_engine_t engine) {
+    delete engine;
+    return dnnl_success;
+}
+
+DNNL_EXPORT dnnl_status_t dnnl_stream_create(dnnl_stream_t *stream, dnnl_engine_t engine, unsigned flags) {
+    CHECK_ARG(stream && engine);
+    CHECK_ARG(flags & (dnnl_stream_in_order | dnnl_stream_out_of_order));
+    if (mi355_device_set((int)engine->index) != MI355_SUCCESS) return dnnl_runtime_error;
+    void *s = nullptr;
+    if (mi355_stream_create(&s) != MI355_SUCCESS) return dnnl_runtime_error;
+    *stream = new dnnl_stream {engine, s};
+    return dnnl_success;
+}
+DNNL_EXPORT dnnl_status_t dnnl_stream_get_engine(dnnl_stream_t stream, dnnl_engine_t *engine) {
+    CHECK_ARG(stream && engine);
+    *engine = stream->engine;
+    return dnnl_success;
+}
+DNNL_EXPORT dnnl_status_t dnnl_stream_wait(dnnl_stream_t stream) {
+    CHECK_ARG(stream);
+    return from_mi355(mi355_stream_sync(stream->hip_stream));
+}
+DNNL_EXPORT dnnl_status_t dnnl_stream_destroy(dnnl_stream_t stream) {
+    if (stream) {
+        mi355_stream_destroy(stream->hip_stream);
+        delete stream;
+    }
+    return dnnl_success;
+}
+
+// ---- memory descriptors
+static dnnl_status_t md_common(dnnl_memory_desc &md, int ndims, const dnnl_dims_t dims, dnnl_data_type_t dt) {
+    CHECK_ARG(ndims > 0 && ndims <= DNNL_MAX_NDIMS && dims);
+    CHECK_ARG(dt_valid(dt));
+    md.ndims = ndims;
+    md.dt = dt;
+    for (int i = 0; i < ndims; ++i) {
+        if (dims[i] == DNNL_RUNTIME_DIM_VAL) return dnnl_unimplemented; // runtime dims are not offered
+        CHECK_ARG(dims[i] >= 0);
+        md.dims[i] = dims[i];
+    }
+    return dnnl_success;
+}
+DNNL_EXPORT dnnl_status_t dnnl_memory_desc_create_with_strides(dnnl_memory_desc_t *memory_desc, int ndims,
+        const dnnl_dims_t dims, dnnl_data_type_t data_type, const dnnl_dims_t strides) {
+    CHECK_ARG(memory_desc);
+    std::unique_ptr<dnnl_memory_desc> md(new dnnl_memory_desc);
+    dnnl_status_t st = md_common(*md, ndims, dims, data_type);
+    if (st) return st;
+    if (!strides) {
+        md->set_dense();
+    } else {
+        for (int i = 0; i < ndims; ++i) {
+            CHECK_ARG(strides[i] >= 0);
+            md->strides[i] = strides[i];
+        }
+        md->kind = dnnl_blocked;
+        // sub-byte types need an innermost unit stride (memory_desc.cpp, 4-bit rule)
+        if (dt_bits(data_type) == 4) {
+            bool unit = false;
+            for (int i = 0; i < ndims; ++i)
+                if (md->strides[i] == 1) unit = true;
+            CHECK_ARG(unit);
+        }
+    }
+    *memory_desc = md.release();
+    return dnnl_success;
+}
+DNNL_EXPORT dnnl_status_t dnnl_memory_desc_create_with_tag(dnnl_memory_desc_t *memory_desc, int ndims,
+        const dnnl_dims_t dims, dnnl_data_type_t data_type, dnnl_format_tag_t tag) {
+    CHECK_ARG(memory_desc);
+    std::unique_ptr<dnnl_memory_desc> md(new dnnl_memory_desc);
+    dnnl_status_t st = md_common(*md, ndims, dims, data_type);
+    if (st) return st;
+    int perm[DNNL_MAX_NDIMS];
+    for (int i = 0; i < ndims; ++i) perm[i] = i;
+    switch (tag) {
+        case dnnl_format_tag_any: md->kind = dnnl_format_kind_any; *memory_desc = md.release(); return dnnl_success;
+        case dnnl_a: CHECK_ARG(ndims == 1); break;
+        case dnnl_ab: CHECK_ARG(ndims == 2); break;
+        case dnnl_abc: CHECK_ARG(ndims == 3); break;
+        case dnnl_abcd: CHECK_ARG(ndims == 4); break;
+        case dnnl_ba: CHECK_ARG(ndims == 2); perm[0] = 1; perm[1] = 0; break;
+        case dnnl_acb: CHECK_ARG(ndims == 3); perm[1] = 2; perm[2] = 1; break;
+        case dnnl_abdc: CHECK_ARG(ndims == 4); perm[2] = 3; perm[3] = 2; break;
+        default: return dnnl_unimplemented; // blocked layouts are not offered
+    }
+    dim_t s = 1;
+    for (int i = ndims - 1; i >= 0; --i) {
+        md->strides[perm[i]] = s;
+        s *= md->dims[perm[i]] == 0 ? 1 : md->dims[perm[i]];
+    }
+    md->kind = dnnl_blocked;
+    *memory_desc = md.release();
+    return dnnl_success;
+}
+DNNL_EXPORT dnnl_status_t dnnl_memory_desc_clone(dnnl_memory_desc_t *memory_desc, const_dnnl_memory_desc_t existing) {
+    CHECK_ARG(memory_desc && existing);
+    *memory_desc = new dnnl_memory_desc(*existing);
+    return dnnl_success;
+}
+DNNL_EXPORT dnnl_status_t dnnl_memory_desc_destroy(dnnl_memory_desc_t memory_desc) {
+    delete memory_desc;
+    return dnnl_success;
+}
+DNNL_EXPORT dnnl_status_t dnnl_memory_desc_query(const_dnnl_memory_desc_t md, dnnl_query_t what, void *result) {
+    CHECK_ARG(md && result);
+    switch (what) {
+        case dnnl_query_ndims_s32: *(int32_t *)result = md->ndims; break;
+        case dnnl_query_dims: *(const dnnl_dims_t **)result = &md->dims; break;
+        case dnnl_query_data_type: *(dnnl_data_type_t *)result = md->dt; break;
+        case dnnl_query_format_kind: *(dnnl_format_kind_t *)result = md->kind; break;
+        case dnnl_query_strides:
+            if (md->kind != dnnl_blocked) return dnnl_invalid_arguments;
+            *(const dnnl_dims_t **)result = &md->strides;
+            break;
+        default: return dnnl_unimplemented;
+    }
+    return dnnl_success;
+}
+DNNL_EXPORT int dnnl_memory_desc_equal(const_dnnl_memory_desc_t lhs, const_dnnl_memory_desc_t rhs) {
+    if (lhs == rhs) return 1;
+    if (!lhs || !rhs) return 0;
+    return *lhs == *rhs;
+}
+DNNL_EXPORT size_t dnnl_memory_desc_get_size(const_dnnl_memory_desc_t md) {
+    if (!md || md->kind != dnnl_blocked) return 0;
+    return md->size_bytes();
+}
+DNNL_EXPORT size_t dnnl_data_type_size(dnnl_data_type_t dt) {
+    return dt_bits(dt) / 8 ? dt_bits(dt) / 8 : 1;
+}
+
+// ---- memory objects
+DNNL_EXPORT dnnl_status_t dnnl_memory_create(dnnl_memory_t *memory, const_dnnl_memory_desc_t md,
+        dnnl_engine_t engine, void *handle) {
+    CHECK_ARG(memory && md && engine);
+    CHECK_ARG(md->kind != dnnl_format_kind_any);
+    std::unique_ptr<dnnl_memory> m(new dnnl_memory);
+    m->md = *md;
+    m->engine = engine;
+    if (handle == DNNL_MEMORY_ALLOCATE) {
+        if (mi355_device_set((int)engine->index) != MI355_SUCCESS) return dnnl_runtime_error;
+        const int st = mi355_mem_alloc(&m->handle, md->size_bytes());
+        if (st != MI355_SUCCESS) return from_mi355(st);
+        m->owned = true;
+    } else {
+        m->handle = handle;
+    }
+    *memory = m.release();
+    return dnnl_success;
+}
+DNNL_EXPORT dnnl_status_t dnnl_memory_get_memory_desc(const_dnnl_memory_t memory, const_dnnl_memory_desc_t *md) {
+    CHECK_ARG(memory && md);
+    *md = &memory->md;
+    return dnnl_success;
+}
+DNNL_EXPORT dnnl_status_t dnnl_memory_get_engine(const_dnnl_memory_t memory, dnnl_engine_t *engine) {
+    CHECK_ARG(memory && engine);
+    *engine = memory->engine;
+    return dnnl_success;
+}
+DNNL_EXPORT dnnl_status_t dnnl_memory_map_data(const_dnnl_memory_t cmemory, void **mapped_ptr) {
+    CHECK_ARG(cmemory && mapped_ptr);
+    dnnl_memory *memory = const_cast<dnnl_memory *>(cmemory);
+    CHECK_ARG(!memory->mapped);
+    const size_t bytes = memory->md.size_bytes();
+    if (!memory->handle || bytes == 0) {
+        *mapped_ptr = nullptr;
+        return dnnl_success;
+    }
+    void *host = malloc(bytes);
+    if (!host) return dnnl_out_of_memory;
+    const int st = mi355_mem_d2h(host, memory->handle, bytes, nullptr);
+    if (st != MI355_SUCCESS) {
+        free(host);
+        return from_mi355(st);
+    }
+    memory->mapped = host;
+    *mapped_ptr = host;
+    return dnnl_success;
+}
+DNNL_EXPORT dnnl_status_t dnnl_memory_unmap_data(const_dnnl_memory_t cmemory, void *mapped_ptr) {
+    CHECK_ARG(cmemory);
+    dnnl_memory *memory = const_cast<dnnl_memory *>(cmemory);
+    if (!memory->mapped) return mapped_ptr ? dnnl_invalid_arguments : dnnl_success;
+    CHECK_ARG(mapped_ptr == memory->mapped);
+    const int st = mi355_mem_h2d(memory->handle, memory->mapped, memory->md.size_bytes(), nullptr);
+    free(memory->mapped);
+    memory->mapped = nullptr;
+    return from_mi355(st);
+}
+DNNL_EXPORT dnnl_status_t dnnl_memory_get_data_handle(const_dnnl_memory_t memory, void **handle) {
+    CHECK_ARG(memory && handle);
+    *handle = memory->handle;
+    return dnnl_success;
+}
+DNNL_EXPORT dnnl_status_t dnnl_memory_set_data_handle(dnnl_memory_t memory, void *handle) {
+    CHECK_ARG(memory);
+    if (memory->owned) {
+        mi355_mem_free(memory->handle);
+        memory->owned = false;
+    }
+    memory->handle = handle;
+    return dnnl_success;
+}
+DNNL_EXPORT dnnl_status_t dnnl_memory_destroy(dnnl_memory_t memory) {
+    if (memory) {
+        if (memory->mapped) free(memory->mapped);
+        if (memory->owned) mi355_mem_free(memory->handle);
+        delete memory;
+    }
+    return dnnl_success;
+}
+
+// ---- attributes
+DNNL_EXPORT dnnl_status_t dnnl_primitive_attr_create(dnnl_primitive_attr_t *attr) {
+    CHECK_ARG(attr);
+    *attr = new dnnl_primitive_attr;
+    return dnnl_success;
+}
+DNNL_EXPORT dnnl_status_t dnnl_primitive_attr_clone(dnnl_primitive_attr_t *attr, const_dnnl_primitive_attr_t existing) {
+    CHECK_ARG(attr && existing);
+    *attr = new dnnl_primitive_attr(*existing);
+    return dnnl_success;
+}
+DNNL_EXPORT dnnl_status_t dnnl_primitive_attr_destroy(dnnl_primitive_attr_t attr) {
+    delete attr;
+    return dnnl_success;
+}
+DNNL_EXPORT dnnl_status_t dnnl_primitive_attr_set_fpmath_mode_v2(dnnl_primitive_attr_t attr,
+        dnnl_fpmath_mode_t mode, int apply_to_int) {
+    CHECK_ARG(attr);
+    CHECK_ARG(mode >= dnnl_fpmath_mode_strict && mode <= dnnl_fpmath_mode_tf32);
+    attr->fpmath = mode;
+    attr->apply_to_int = apply_to_int != 0;
+    return dnnl_success;
+}
+DNNL_EXPORT dnnl_status_t dnnl_primitive_attr_set_fpmath_mode(dnnl_primitive_attr_t attr, dnnl_fpmath_mode_t mode) {
+    return dnnl_primitive_attr_set_fpmath_mode_v2(attr, mode, 0);
+}
+DNNL_EXPORT dnnl_status_t dnnl_primitive_attr_get_fpmath_mode_v2(const_dnnl_primitive_attr_t attr,
+        dnnl_fpmath_mode_t *mode, int *apply_to_int) {
+    CHECK_ARG(attr);
+    if (mode) *mode = attr->fpmath;
+    if (apply_to_int) *apply_to_int = attr->apply_to_int;
+    return dnnl_success;
+}
+DNNL_EXPORT dnnl_status_t dnnl_primitive_attr_set_accumulation_mode(dnnl_primitive_attr_t attr,
+        dnnl_accumulation_mode_t mode) {
+    CHECK_ARG(attr);
+    CHECK_ARG(mode >= dnnl_accumulation_mode_strict && mode <= dnnl_accumulation_mode_f16);
+    attr->acc_mode = mode;
+    return dnnl_success;
+}
+DNNL_EXPORT dnnl_status_t dnnl_primitive_attr_set_scratchpad_mode(dnnl_primitive_attr_t attr,
+        dnnl_scratchpad_mode_t mode) {
+    CHECK_ARG(attr);
+    CHECK_ARG(mode == dnnl_scratchpad_mode_library || mode == dnnl_scratchpad_mode_user);
+    attr->scratchpad_mode = mode;
+    return dnnl_success;
+}
+DNNL_EXPORT dnnl_status_t dnnl_primitive_attr_get_scratchpad_mode(const_dnnl_primitive_attr_t attr,
+        dnnl_scratchpad_mode_t *mode) {
+    CHECK_ARG(attr && mode);
+    *mode = attr->scratchpad_mode;
+    return dnnl_success;
+}
+
+static dnnl_status_t set_quant(std::map<int, quant_entry_t> &m, int arg, int mask, int group_ndims,
+        const dnnl_dims_t group_dims, dnnl_data_type_t dt) {
+    CHECK_ARG(arg >= 0 && mask >= 0);
+    CHECK_ARG(group_ndims == 0 || group_ndims == 2);
+    quant_entry_t q;
+    q.mask = mask;
+    q.dt = dt;
+    q.group_ndims = group_ndims;
+    if (group_ndims) {
+        CHECK_ARG(group_dims && group_dims[0] > 0 && group_dims[1] > 0);
+        q.groups[0] = group_dims[0];
+        q.groups[1] = group_dims[1];
+    }
+    m[arg] = q;
+    return dnnl_success;
+}
+// checks of dnnl_primitive_attr_set_scales_v3, src/common/primitive_attr.cpp:637-663
+DNNL_EXPORT dnnl_status_t dnnl_primitive_attr_set_scales(dnnl_primitive_attr_t attr, int arg, int mask,
+        int group_ndims, const dnnl_dims_t group_dims, dnnl_data_type_t data_type) {
+    CHECK_ARG(attr);
+    CHECK_ARG(data_type == dnnl_f32 || data_type == dnnl_bf16 || data_type == dnnl_f16 || data_type == dnnl_e8m0
+            || data_type == dnnl_f8_e4m3);
+    CHECK_ARG(IMPLICATION(data_type == dnnl_e8m0 || data_type == dnnl_f8_e4m3, mask > 0));
+    return set_quant(attr->scales, arg, mask, group_ndims, group_dims, data_type);
+}
+DNNL_EXPORT dnnl_status_t dnnl_primitive_attr_set_scales_mask(dnnl_primitive_attr_t attr, int arg, int mask) {
+    return dnnl_primitive_attr_set_scales(attr, arg, mask, 0, nullptr, dnnl_f32);
+}
+// checks of dnnl_primitive_attr_set_zero_points_v2, primitive_attr.cpp:684-716
+DNNL_EXPORT dnnl_status_t dnnl_primitive_attr_set_zero_points(dnnl_primitive_attr_t attr, int arg, int mask,
+        int group_ndims, const dnnl_dims_t group_dims, dnnl_data_type_t data_type) {
+    CHECK_ARG(attr);
+    CHECK_ARG(data_type == dnnl_s32 || data_type == dnnl_s8 || data_type == dnnl_u8 || data_type == dnnl_s4
+            || data_type == dnnl_u4);
+    CHECK_ARG(IMPLICATION(data_type == dnnl_s4 || data_type == dnnl_u4, mask > 0));
+    CHECK_ARG(IMPLICATION(arg != DNNL_ARG_SRC && arg != DNNL_ARG_WEIGHTS, data_type == dnnl_s32 && group_ndims == 0));
+    CHECK_ARG(IMPLICATION(group_ndims > 0, mask > 0));
+    return set_quant(attr->zero_points, arg, mask, group_ndims, group_dims, data_type);
+}
+DNNL_EXPORT dnnl_status_t dnnl_primitive_attr_set_zero_points_mask(dnnl_primitive_attr_t attr, int arg, int mask) {
+    return dnnl_primitive_attr_set_zero_points(attr, arg, mask, 0, nullptr, dnnl_s32);
+}
+DNNL_EXPORT dnnl_status_t dnnl_primitive_attr_set_precomputed_reductions(dnnl_primitive_attr_t attr, int arg,
+        int mask, int group_ndims, const dnnl_dims_t group_dims, dnnl_data_type_t data_type) {
+    CHECK_ARG(attr);
+    CHECK_ARG(data_type == dnnl_s32);
+    CHECK_ARG(mask > 0);
+    return set_quant(attr->reductions, arg, mask, group_ndims, group_dims, data_type);
+}
+DNNL_EXPORT dnnl_status_t dnnl_primitive_attr_set_post_ops(dnnl_primitive_attr_t attr, const_dnnl_post_ops_t post_ops) {
+    CHECK_ARG(attr && post_ops);
+    attr->post_ops = *post_ops;
+    return dnnl_success;
+}
+DNNL_EXPORT dnnl_status_t dnnl_primitive_attr_get_post_ops(const_dnnl_primitive_attr_t attr, const_dnnl_post_ops_t *post_ops) {
+    CHECK_ARG(attr && post_ops);
+    *post_ops = &attr->post_ops; // borrowed, as in the reference (dnnl.h:683-694)
+    return dnnl_success;
+}
+
+// ---- post-ops
+DNNL_EXPORT dnnl_status_t dnnl_post_ops_create(dnnl_post_ops_t *post_ops) {
+    CHECK_ARG(post_ops);
+    *post_ops = new dnnl_post_ops;
+    return dnnl_success;
+}
+DNNL_EXPORT dnnl_status_t dnnl_post_ops_clone(dnnl_post_ops_t *post_ops, const_dnnl_post_ops_t existing) {
+    CHECK_ARG(post_ops && existing);
+    *post_ops = new dnnl_post_ops(*existing);
+    return dnnl_success;
+}
+DNNL_EXPORT dnnl_status_t dnnl_post_ops_destroy(dnnl_post_ops_t post_ops) {
+    delete post_ops;
+    return dnnl_success;
+}
+DNNL_EXPORT int dnnl_post_ops_len(const_dnnl_post_ops_t post_ops) {
+    return post_ops ? (int)post_ops->entries.size() : 0;
+}
+DNNL_EXPORT dnnl_primitive_kind_t dnnl_post_ops_get_kind(const_dnnl_post_ops_t post_ops, int index) {
+    if (!post_ops || index < 0 || index >= (int)post_ops->entries.size()) return dnnl_undefined_primitive;
+    return post_ops->entries[index].kind;
+}
+static bool po_full(const_dnnl_post_ops_t p) { return p->entries.size() >= MI355_MAX_POST_OPS; }
+DNNL_EXPORT dnnl_status_t dnnl_post_ops_append_sum(dnnl_post_ops_t post_ops, float scale, int32_t zero_point,
+        dnnl_data_type_t data_type) {
+    CHECK_ARG(post_ops);
+    if (po_full(post_ops)) return dnnl_out_of_memory;
+    post_op_entry_t e;
+    e.kind = dnnl_sum; e.scale = scale; e.zero_point = zero_point; e.dt = data_type;
+    post_ops->entries.push_back(e);
+    return dnnl_success;
+}
+DNNL_EXPORT dnnl_status_t dnnl_post_ops_get_params_sum(const_dnnl_post_ops_t post_ops, int index, float *scale,
+        int32_t *zero_point, dnnl_data_type_t *data_type) {
+    CHECK_ARG(post_ops && index >= 0 && index < (int)post_ops->entries.size());
+    const post_op_entry_t &e = post_ops->entries[index];
+    CHECK_ARG(e.kind == dnnl_sum);
+    if (scale) *scale = e.scale;
+    if (zero_point) *zero_point = e.zero_point;
+    if (data_type) *data_type = e.dt;
+    return dnnl_success;
+}
+DNNL_EXPORT dnnl_status_t dnnl_post_ops_append_eltwise(dnnl_post_ops_t post_ops, dnnl_alg_kind_t alg, float alpha,
+        float beta) {
+    CHECK_ARG(post_ops);
+    CHECK_ARG(alg >= dnnl_eltwise_relu && alg <= dnnl_eltwise_hardswish);
+    // is_eltwise_ok, src/common/math_utils.hpp:432-470
+    CHECK_ARG(IMPLICATION(alg == dnnl_eltwise_clip || alg == dnnl_eltwise_clip_v2, beta >= alpha));
+    if (po_full(post_ops)) return dnnl_out_of_memory;
+    post_op_entry_t e;
+    e.kind = dnnl_eltwise; e.alg = alg; e.alpha = alpha; e.beta = beta; e.scale = 1.f;
+    post_ops->entries.push_back(e);
+    return dnnl_success;
+}
+DNNL_EXPORT dnnl_status_t dnnl_post_ops_get_params_eltwise(const_dnnl_post_ops_t post_ops, int index,
+        dnnl_alg_kind_t *alg, float *alpha, float *beta) {
+    CHECK_ARG(post_ops && index >= 0 && index < (int)post_ops->entries.size());
+    const post_op_entry_t &e = post_ops->entries[index];
+    CHECK_ARG(e.kind == dnnl_eltwise);
+    if (alg) *alg = e.alg;
+    if (alpha) *alpha = e.alpha;
+    if (beta) *beta = e.beta;
+    return dnnl_success;
+}
+DNNL_EXPORT dnnl_status_t dnnl_post_ops_append_binary(dnnl_post_ops_t post_ops, dnnl_alg_kind_t alg,
+        const_dnnl_memory_desc_t src1_desc) {
+    CHECK_ARG(post_ops && src1_desc);
+    CHECK_ARG(alg >= dnnl_binary_add && alg <= dnnl_binary_ne);
+    CHECK_ARG(src1_desc->kind == dnnl_blocked || src1_desc->kind == dnnl_format_kind_any);
+    if (po_full(post_ops)) return dnnl_out_of_memory;
+    post_op_entry_t e;
+    e.kind = dnnl_binary; e.alg = alg; e.src1 = *src1_desc;
+    if (e.src1.kind == dnnl_format_kind_any) e.src1.set_dense();
+    post_ops->entries.push_back(e);
+    return dnnl_success;
+}
+DNNL_EXPORT dnnl_status_t dnnl_post_ops_get_params_binary(const_dnnl_post_ops_t post_ops, int index,
+        dnnl_alg_kind_t *alg, const_dnnl_memory_desc_t *src1_desc) {
+    CHECK_ARG(post_ops && index >= 0 && index < (int)post_ops->entries.size());
+    const post_op_entry_t &e = post_ops->entries[index];
+    CHECK_ARG(e.kind == dnnl_binary);
+    if (alg) *alg = e.alg;
+    if (src1_desc) *src1_desc = &e.src1;
+    return dnnl_success;
+}
+DNNL_EXPORT dnnl_status_t dnnl_post_ops_append_prelu(dnnl_post_ops_t post_ops, int mask) {
+    CHECK_ARG(post_ops && mask >= 0);
+    if (po_full(post_ops)) return dnnl_out_of_memory;
+    post_op_entry_t e;
+    e.kind = dnnl_prelu; e.mask = mask;
+    post_ops->entries.push_back(e);
+    return dnnl_success;
+}
+DNNL_EXPORT dnnl_status_t dnnl_post_ops_get_params_prelu(const_dnnl_post_ops_t post_ops, int index, int *mask) {
+    CHECK_ARG(post_ops && index >= 0 && index < (int)post_ops->entries.size());
+    const post_op_entry_t &e = post_ops->entries[index];
+    CHECK_ARG(e.kind == dnnl_prelu);
+    if (mask) *mask = e.mask;
+    return dnnl_success;
+}
+
+// ---- matmul primitive descriptor
+DNNL_EXPORT dnnl_status_t dnnl_matmul_primitive_desc_create(dnnl_primitive_desc_t *primitive_desc,
+        dnnl_engine_t engine, const_dnnl_memory_desc_t src_desc, const_dnnl_memory_desc_t weights_desc,
+        const_dnnl_memory_desc_t bias_desc, const_dnnl_memory_desc_t dst_desc, const_dnnl_primitive_attr_t attr) {
+    CHECK_ARG(primitive_desc && engine);
+    CHECK_ARG(src_desc && weights_desc && dst_desc);
+    const dnnl_memory_desc *bias = (bias_desc && !bias_desc->is_zero()) ? bias_desc : nullptr;
+    dnnl_status_t st = check_shapes(*src_desc, *weights_desc, bias, *dst_desc);
+    if (st) return st;
+    CHECK_ARG(accum_dt(src_desc->dt, weights_desc->dt, dst_desc->dt) != dnnl_data_type_undef);
+    std::unique_ptr<dnnl_primitive_desc> pd(new dnnl_primitive_desc);
+    if (attr) pd->attr = *attr;
+    st = check_attr(*src_desc, *weights_desc, *dst_desc, pd->attr);
+    if (st) return st;
+    pd->engine = engine;
+    pd->src = *src_desc; pd->wei = *weights_desc; pd->dst = *dst_desc;
+    pd->with_bias = bias != nullptr;
+    if (bias) pd->bias = *bias;
+    // format `any` -> plain row-major (matmul_pd_t::set_default_formats, matmul_pd.hpp:419-431)
+    for (dnnl_memory_desc *m : {&pd->src, &pd->wei, &pd->dst, &pd->bias})
+        if (m->kind == dnnl_format_kind_any) m->set_dense();
+    // data type combinations of the reference's two naive implementations
+    // (ref_matmul.hpp:44-123, ref_matmul_int8.hpp:44-92)
+    {
+        const int s = pd->src.dt, w = pd->wei.dt, d = pd->dst.dt;
+        const bool int_path = is_int8(s);
+        if (int_path) {
+            CHECK_UNIMPL(is_int8(w) || w == dnnl_s4 || w == dnnl_u4);
+            CHECK_UNIMPL(d == dnnl_f32 || d == dnnl_bf16 || d == dnnl_f16 || d == dnnl_s32 || is_int8(d));
+            if (bias) CHECK_UNIMPL(bias->dt == dnnl_f32 || bias->dt == dnnl_bf16 || bias->dt == dnnl_f16
+                    || bias->dt == dnnl_s32 || is_int8(bias->dt));
+        } else {
+            CHECK_UNIMPL(s == dnnl_f32 || s == dnnl_bf16 || s == dnnl_f16 || is_fp8(s) || s == dnnl_f4_e2m1);
+            CHECK_UNIMPL(w == dnnl_f32 || w == dnnl_bf16 || w == dnnl_f16 || is_fp8(w) || w == dnnl_f4_e2m1
+                    || is_int8(w) || w == dnnl_s4 || w == dnnl_u4);
+            CHECK_UNIMPL(s == w || w == dnnl_bf16 || w == dnnl_f16 || is_fp8(w) || is_int8(w) || w == dnnl_s4
+                    || w == dnnl_u4);
+            // integer weights under a floating-point src only as weight decompression
+            CHECK_UNIMPL(IMPLICATION(is_int8(w) || w == dnnl_s4 || w == dnnl_u4, pd->attr.apply_to_int));
+            CHECK_UNIMPL(d == dnnl_f32 || d == dnnl_bf16 || d == dnnl_f16 || is_fp8(d) || is_int8(d));
+            if (bias) CHECK_UNIMPL(bias->dt == dnnl_f32 || bias->dt == dnnl_bf16 || bias->dt == dnnl_f16 || is_fp8(bias->dt));
+        }
+    }
+    st = lower(*pd);
+    if (st) return st;
+    for (int impl : k_impl_list) {
+        int chosen = 0;
+        if (mi355_matmul_query(&pd->desc, impl, &chosen) == MI355_SUCCESS) pd->impls.push_back(impl);
+    }
+    if (pd->impls.empty()) return dnnl_unimplemented;
+    pd->impl_pos = 0;
+    st = select_impl(*pd);
+    if (st) return st;
+    if (verbose_level() >= 1)
+        fprintf(stderr, "onednn_verbose,v1,primitive,create:dispatch,gpu,matmul,%s\n", pd->impl_name.c_str());
+    *primitive_desc = pd.release();
+    return dnnl_success;
+}
+
+DNNL_EXPORT dnnl_status_t dnnl_primitive_desc_clone(dnnl_primitive_desc_t *primitive_desc,
+        const_dnnl_primitive_desc_t existing) {
+    CHECK_ARG(primitive_desc && existing);
+    *primitive_desc = new dnnl_primitive_desc(*existing);
+    return dnnl_success;
+}
+DNNL_EXPORT dnnl_status_t dnnl_primitive_desc_next_impl(dnnl_primitive_desc_t pd) {
+    CHECK_ARG(pd);
+    if (pd->impl_pos + 1 >= pd->impls.size()) return dnnl_last_impl_reached;
+    ++pd->impl_pos;
+    return select_impl(*pd);
+}
+DNNL_EXPORT dnnl_status_t dnnl_primitive_desc_get_attr(const_dnnl_primitive_desc_t pd, const_dnnl_primitive_attr_t *attr) {
+    CHECK_ARG(pd && attr);
+    *attr = &pd->attr;
+    return dnnl_success;
+}
+DNNL_EXPORT dnnl_status_t dnnl_primitive_desc_destroy(dnnl_primitive_desc_t pd) {
+    delete pd;
+    return dnnl_success;
+}
+DNNL_EXPORT const_dnnl_memory_desc_t dnnl_primitive_desc_query_md(const_dnnl_primitive_desc_t pd, dnnl_query_t what,
+        int index) {
+    if (!pd) return nullptr;
+    static const dnnl_memory_desc zero_md;
+    switch (what) {
+        case dnnl_query_src_md: return index == 0 ? &pd->src : nullptr;
+        case dnnl_query_weights_md: return index == 0 ? &pd->wei : index == 1 ? (pd->with_bias ? &pd->bias : &zero_md) : nullptr;
+        case dnnl_query_dst_md: return index == 0 ? &pd->dst : nullptr;
+        case dnnl_query_scratchpad_md: return index == 0 ? &pd->scratchpad : nullptr;
+        case dnnl_query_exec_arg_md:
+            switch (index) {
+                case DNNL_ARG_SRC: return &pd->src;
+                case DNNL_ARG_WEIGHTS: return &pd->wei;
+                case DNNL_ARG_BIAS: return pd->with_bias ? &pd->bias : &zero_md;
+                case DNNL_ARG_DST: return &pd->dst;
+                case DNNL_ARG_SCRATCHPAD: return &pd->scratchpad;
+                default: return nullptr;
+            }
+        default: return nullptr;
+    }
+}
+DNNL_EXPORT dnnl_status_t dnnl_primitive_desc_query(const_dnnl_primitive_desc_t pd, dnnl_query_t what, int index,
+        void *result) {
+    CHECK_ARG(pd && result);
+    switch (what) {
+        case dnnl_query_engine: *(dnnl_engine_t *)result = pd->engine; break;
+        case dnnl_query_primitive_kind: *(dnnl_primitive_kind_t *)result = dnnl_matmul; break;
+        case dnnl_query_num_of_inputs_s32: *(int32_t *)result = 2 + (pd->with_bias ? 1 : 0); break;
+        case dnnl_query_num_of_outputs_s32: *(int32_t *)result = 1; break;
+        case dnnl_query_memory_consumption_s64:
+            *(int64_t *)result = pd->attr.scratchpad_mode == dnnl_scratchpad_mode_library ? (int64_t)pd->scratch_bytes : 0;
+            break;
+        case dnnl_query_impl_info_str: *(const char **)result = pd->impl_name.c_str(); break;
+        case dnnl_query_prop_kind: *(int *)result = 96; break; // dnnl_forward_inference
+        case dnnl_query_src_md:
+        case dnnl_query_weights_md:
+        case dnnl_query_dst_md:
+        case dnnl_query_scratchpad_md:
+        case dnnl_query_exec_arg_md: {
+            const_dnnl_memory_desc_t md = dnnl_primitive_desc_query_md(pd, what, index);
+            if (!md) return dnnl_invalid_arguments;
+            *(const_dnnl_memory_desc_t *)result = md;
+        } break;
+        default: return dnnl_unimplemented;
+    }
+    return dnnl_success;
+}
+
+// ---- primitive
+DNNL_EXPORT dnnl_status_t dnnl_primitive_create(dnnl_primitive_t *primitive, const_dnnl_primitive_desc_t pd) {
+    CHECK_ARG(primitive && pd);
+    std::unique_ptr<dnnl_primitive> p(new dnnl_primitive);
+    p->pd = *pd;
+    if (p->pd.attr.scratchpad_mode == dnnl_scratchpad_mode_library && p->pd.scratch_bytes > 0) {
+        if (mi355_device_set((int)p->pd.engine->index) != MI355_SUCCESS) return dnnl_runtime_error;
+        const int st = mi355_mem_alloc(&p->scratch, p->pd.scratch_bytes);
+        if (st != MI355_SUCCESS) return from_mi355(st);
+    }
+    *primitive = p.release();
+    return dnnl_success;
+}
+DNNL_EXPORT dnnl_status_t dnnl_primitive_get_primitive_desc(const_dnnl_primitive_t primitive,
+        const_dnnl_primitive_desc_t *pd) {
+    CHECK_ARG(primitive && pd);
+    *pd = &primitive->pd;
+    return dnnl_success;
+}
+DNNL_EXPORT dnnl_status_t dnnl_primitive_destroy(dnnl_primitive_t primitive) {
+    if (primitive) {
+        if (primitive->scratch) mi355_mem_free(primitive->scratch);
+        delete primitive;
+    }
+    return dnnl_success;
+}
+
+DNNL_EXPORT dnnl_status_t dnnl_primitive_execute(const_dnnl_primitive_t cprimitive, dnnl_stream_t stream, int nargs,
+        const dnnl_exec_arg_t *args) {
+    CHECK_ARG(cprimitive && stream);
+    CHECK_ARG(nargs >= 0 && IMPLICATION(nargs > 0, args));
+    dnnl_primitive *prim = const_cast<dnnl_primitive *>(cprimitive);
+    const dnnl_primitive_desc &pd = prim->pd;
+    CHECK_ARG(stream->engine == pd.engine || stream->engine->index == pd.engine->index);
+    std::map<int, dnnl_memory_t> m;
+    for (int i = 0; i < nargs; ++i) {
+        CHECK_ARG(m.find(args[i].arg) == m.end()); // duplicated argument
+        m[args[i].arg] = args[i].memory;
+    }
+    auto handle = [&](int arg, bool required, void **out) -> dnnl_status_t {
+        auto it = m.find(arg);
+        if (it == m.end() || !it->second) {
+            *out = nullptr;
+            return required ? dnnl_invalid_arguments : dnnl_success;
+        }
+        *out = it->second->handle;
+        return dnnl_success;
+    };
+    mi355_matmul_args_t A;
+    memset(&A, 0, sizeof(A));
+    dnnl_status_t st;
+    const bool empty = pd.desc.batch == 0 || pd.desc.M == 0 || pd.desc.N == 0 || pd.desc.K == 0;
+    void *p = nullptr;
+#define TAKE(field, arg, required) \
+    do { \
+        if ((st = handle(arg, required, &p)) != dnnl_success) return st; \
+        A.field = p; \
+    } while (0)
+    TAKE(src, DNNL_ARG_SRC, true);
+    TAKE(wei, DNNL_ARG_WEIGHTS, true);
+    TAKE(dst, DNNL_ARG_DST, true);
+    TAKE(bias, DNNL_ARG_BIAS, pd.with_bias);
+    TAKE(src_scale, DNNL_ARG_ATTR_SCALES | DNNL_ARG_SRC, pd.desc.src_scale.dt != MI355_DT_UNDEF);
+    TAKE(wei_scale, DNNL_ARG_ATTR_SCALES | DNNL_ARG_WEIGHTS, pd.desc.wei_scale.dt != MI355_DT_UNDEF);
+    TAKE(dst_scale, DNNL_ARG_ATTR_SCALES | DNNL_ARG_DST, pd.desc.dst_scale.dt != MI355_DT_UNDEF);
+    TAKE(src_zp, DNNL_ARG_ATTR_ZERO_POINTS | DNNL_ARG_SRC, pd.desc.src_zp.dt != MI355_DT_UNDEF);
+    TAKE(wei_zp, DNNL_ARG_ATTR_ZERO_POINTS | DNNL_ARG_WEIGHTS, pd.desc.wei_zp.dt != MI355_DT_UNDEF);
+    TAKE(dst_zp, DNNL_ARG_ATTR_ZERO_POINTS | DNNL_ARG_DST, pd.desc.dst_zp.dt != MI355_DT_UNDEF);
+    TAKE(src_pr, DNNL_ARG_ATTR_PRECOMPUTED_REDUCTIONS | DNNL_ARG_SRC, pd.desc.src_pr.dt != MI355_DT_UNDEF);
+    for (int i = 0; i < pd.desc.n_post_ops; ++i) {
+        const int kind = pd.desc.post_ops[i].kind;
+        if (kind == MI355_PO_BINARY) {
+            if ((st = handle(DNNL_ARG_ATTR_MULTIPLE_POST_OP(i) | DNNL_ARG_SRC_1, true, &p))) return st;
+            A.po_arg[i] = p;
+        } else if (kind == MI355_PO_PRELU) {
+            if ((st = handle(DNNL_ARG_ATTR_MULTIPLE_POST_OP(i) | DNNL_ARG_WEIGHTS, true, &p))) return st;
+            A.po_arg[i] = p;
+        }
+    }
+#undef TAKE
+    if (empty) return dnnl_success;
+    if (!A.src || !A.wei || !A.dst) return dnnl_invalid_arguments;
+
+    void *scratch = prim->scratch;
+    std::unique_lock<std::mutex> lock(prim->scratch_mutex, std::defer_lock);
+    if (pd.attr.scratchpad_mode == dnnl_scratchpad_mode_user) {
+        if ((st = handle(DNNL_ARG_SCRATCHPAD, pd.scratch_bytes > 0, &scratch))) return st;
+    } else if (scratch) {
+        // the library-mode scratchpad belongs to the primitive: executions of
+        // one primitive object are serialised on the host while they enqueue
+        lock.lock();
+    }
+    if (mi355_device_set((int)pd.engine->index) != MI355_SUCCESS) return dnnl_runtime_error;
+    const auto t0 = std::chrono::steady_clock::now();
+    const int rc = mi355_matmul_launch(&pd.desc, &A, scratch, stream->hip_stream);
+    if (verbose_level() >= 2) {
+        mi355_stream_sync(stream->hip_stream);
+        const double ms = std::chrono::duration<double, std::milli>(std::chrono::steady_clock::now() - t0).count();
+        fprintf(stderr, "onednn_verbose,v1,primitive,exec,gpu,matmul,%s,undef,src:%s wei:%s dst:%s,,%ldx%ldx%ld:%ldx%ldx%ld,%g\n",
+                pd.impl_name.c_str(), dt_name(pd.src.dt), dt_name(pd.wei.dt), dt_name(pd.dst.dt), (long)pd.desc.batch,
+                (long)pd.desc.M, (long)pd.desc.K, (long)pd.desc.batch, (long)pd.desc.K, (long)pd.desc.N, ms);
+    }
+    return from_mi355(rc);
+}

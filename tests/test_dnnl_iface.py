@@ -1,0 +1,211 @@
+"""Interface tests of the dnnl_* C API subset (libdnnl_amd.so) that need no
+GPU: a descriptor-only engine (ONEDNN_AMD_ALLOW_NO_DEVICE=1) creates and
+queries primitive descriptors.  Modelled on the reference's interface tests
+(tests/gtests/test_matmul.cpp:392-680, test_iface_attr_quantization.cpp) and on
+the conditions of matmul_desc_init / matmul_attr_check
+(src/common/matmul.cpp:261-744): status codes, not numerics."""
+import ctypes as C
+import os
+import re
+
+import pytest
+
+os.environ["ONEDNN_AMD_ALLOW_NO_DEVICE"] = "1"
+
+from onednn_amd import cabi, dnnl  # noqa: E402
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+DT = cabi.DT_NAMES
+
+
+@pytest.fixture(scope="module")
+def eng():
+    return dnnl.engine(dnnl.gpu, 0)
+
+
+def md(dims, dt, tag=None, strides=None):
+    if tag is None and strides is None:
+        tag = {1: dnnl.tag_a, 2: dnnl.tag_ab, 3: dnnl.tag_abc, 4: dnnl.tag_abcd}[len(dims)]
+    return dnnl.memory_desc(dims, DT[dt], tag=tag, strides=strides)
+
+
+def make_pd(eng, M, K, N, sdt, wdt, ddt, attr=None, bias=None, wtag=dnnl.tag_ab):
+    return dnnl.matmul_primitive_desc(eng, md([M, K], sdt), md([K, N], wdt, tag=wtag), md([M, N], ddt),
+                                      bias_md=bias, attr=attr)
+
+
+def status_of(fn):
+    try:
+        fn()
+        return dnnl.success
+    except dnnl.error as e:
+        return e.status
+
+
+def test_every_declared_symbol_is_exported():
+    text = re.sub(r"/\*.*?\*/", "", open(os.path.join(ROOT, "include", "dnnl_amd.h")).read(), flags=re.S)
+    names = sorted(set(re.findall(r"\b(dnnl_[a-z0-9_]+)\s*\(", text)))
+    assert len(names) >= 55
+    lib = dnnl.lib()
+    for n in names:
+        assert hasattr(lib, n), f"{n} is declared in include/dnnl_amd.h but not exported"
+
+
+def test_engine_kinds(eng):
+    assert eng.get_kind() == dnnl.gpu
+    assert status_of(lambda: dnnl.engine(dnnl.cpu, 0)) == dnnl.invalid_arguments   # no CPU engine here
+
+
+def test_memory_desc_queries():
+    m = md([3, 5, 7], "bf16")
+    assert m.ndims() == 3 and m.dims() == [3, 5, 7] and m.strides() == [35, 7, 1]
+    assert m.data_type() == DT["bf16"] and m.get_size() == 3 * 5 * 7 * 2
+    t = md([4, 6], "s8", tag=dnnl.tag_ba)
+    assert t.strides() == [1, 4]
+    s = md([4, 6], "f32", strides=[16, 2])
+    assert s.get_size() == ((3 * 16 + 5 * 2) + 1) * 4
+    n4 = md([4, 6], "u4")
+    assert n4.get_size() == 12                      # two nibbles per byte
+    assert status_of(lambda: md([4, 6], "u4", strides=[12, 2])) == dnnl.invalid_arguments
+    assert status_of(lambda: dnnl.memory_desc([2, 2], 99, tag=dnnl.tag_ab)) == dnnl.invalid_arguments
+    assert status_of(lambda: dnnl.memory_desc([2, 2], DT["f32"], tag=dnnl.tag_abc)) == dnnl.invalid_arguments
+
+
+def test_shape_rules(eng):
+    # matmul_desc_init: M, N, K consistency and broadcast rules -> invalid_arguments
+    ok = lambda: dnnl.matmul_primitive_desc(eng, md([8, 16], "f32"), md([16, 4], "f32"), md([8, 4], "f32"))
+    assert status_of(ok) == dnnl.success
+    bad_k = lambda: dnnl.matmul_primitive_desc(eng, md([8, 16], "f32"), md([15, 4], "f32"), md([8, 4], "f32"))
+    bad_m = lambda: dnnl.matmul_primitive_desc(eng, md([8, 16], "f32"), md([16, 4], "f32"), md([7, 4], "f32"))
+    bad_nd = lambda: dnnl.matmul_primitive_desc(eng, md([8, 16], "f32"), md([1, 16, 4], "f32"), md([8, 4], "f32"))
+    for f in (bad_k, bad_m, bad_nd):
+        assert status_of(f) == dnnl.invalid_arguments
+    # batch broadcast: 3x1 batch dims
+    bc = lambda: dnnl.matmul_primitive_desc(eng, md([3, 8, 16], "f32"), md([1, 16, 4], "f32"), md([3, 8, 4], "f32"))
+    assert status_of(bc) == dnnl.success
+    bad_bc = lambda: dnnl.matmul_primitive_desc(eng, md([3, 8, 16], "f32"), md([2, 16, 4], "f32"), md([3, 8, 4], "f32"))
+    assert status_of(bad_bc) == dnnl.invalid_arguments
+    # bias must broadcast onto dst and have dst's ndims
+    b_ok = lambda: make_pd(eng, 8, 16, 4, "f32", "f32", "f32", bias=md([1, 4], "f32"))
+    b_bad = lambda: make_pd(eng, 8, 16, 4, "f32", "f32", "f32", bias=md([1, 3], "f32"))
+    b_nd = lambda: make_pd(eng, 8, 16, 4, "f32", "f32", "f32", bias=md([4], "f32"))
+    assert status_of(b_ok) == dnnl.success
+    assert status_of(b_bad) == dnnl.invalid_arguments and status_of(b_nd) == dnnl.invalid_arguments
+
+
+def test_attribute_setters_validate():
+    a = dnnl.primitive_attr()
+    # primitive_attr.cpp:637-716
+    assert status_of(lambda: a.set_scales(dnnl.ARG_SRC, 0, dt=DT["s8"])) == dnnl.invalid_arguments
+    assert status_of(lambda: a.set_scales(dnnl.ARG_SRC, 0, dt=DT["e8m0"])) == dnnl.invalid_arguments   # needs a mask
+    assert status_of(lambda: a.set_scales(dnnl.ARG_WEIGHTS, 3, (32,), DT["f32"])) == dnnl.invalid_arguments  # 0 or 2 group dims
+    assert status_of(lambda: a.set_zero_points(dnnl.ARG_WEIGHTS, 0, dt=DT["u4"])) == dnnl.invalid_arguments
+    assert status_of(lambda: a.set_zero_points(dnnl.ARG_DST, 2, dt=DT["s8"])) == dnnl.invalid_arguments
+    assert status_of(lambda: a.set_zero_points(dnnl.ARG_SRC, -1)) == dnnl.invalid_arguments
+    assert status_of(lambda: a.set_scales(dnnl.ARG_WEIGHTS, 3, (128, 1), DT["bf16"])) == dnnl.success
+    po = dnnl.post_ops()
+    assert status_of(lambda: po.append_eltwise(cabi.ELTWISE["clip"], 2.0, 1.0)) == dnnl.invalid_arguments
+    assert status_of(lambda: po.append_eltwise(0x7777)) == dnnl.invalid_arguments
+    po.append_eltwise(cabi.ELTWISE["relu"])
+    po.append_sum(1.0)
+    assert po.len() == 2 and po.kind(0) == dnnl.kind_eltwise and po.kind(1) == dnnl.kind_sum
+
+
+# (description, src, wei, dst, attr builder, expected status): rows follow matmul_attr_check
+def _attr(build):
+    a = dnnl.primitive_attr()
+    build(a)
+    return a
+
+
+ATTR_CASES = [
+    ("src scale common", "u8", "s8", "f32", lambda a: a.set_scales_mask(dnnl.ARG_SRC, 0), dnnl.success),
+    ("src scale per-M", "u8", "s8", "f32", lambda a: a.set_scales_mask(dnnl.ARG_SRC, 1), dnnl.success),
+    ("src scale per-K without groups", "u8", "s8", "f32", lambda a: a.set_scales_mask(dnnl.ARG_SRC, 2), dnnl.unimplemented),
+    ("wei scale per-N", "u8", "s8", "f32", lambda a: a.set_scales_mask(dnnl.ARG_WEIGHTS, 2), dnnl.success),
+    ("wei scale K mask on int8 x int8 is decompression-only... allowed for int src", "u8", "s8", "f32",
+     lambda a: a.set_scales(dnnl.ARG_WEIGHTS, 3, (32, 1)), dnnl.success),
+    ("wei scale K groups not multiple of 16", "u8", "s8", "f32",
+     lambda a: a.set_scales(dnnl.ARG_WEIGHTS, 3, (8, 1)), dnnl.unimplemented),
+    ("wei scale K mask on bf16 src without apply_to_int", "bf16", "u4", "bf16",
+     lambda a: a.set_scales(dnnl.ARG_WEIGHTS, 3, (32, 1), DT["bf16"]), dnnl.unimplemented),
+    ("decompression with K-grouped scales and u4 zero points", "bf16", "u4", "bf16",
+     lambda a: (a.set_fpmath_mode(dnnl.fpmath_bf16, True), a.set_scales(dnnl.ARG_WEIGHTS, 3, (32, 1), DT["bf16"]),
+                a.set_zero_points(dnnl.ARG_WEIGHTS, 3, (32, 1), DT["u4"])), dnnl.success),
+    ("wei zp N-groups need apply_to_int", "u8", "s8", "f32",
+     lambda a: a.set_zero_points(dnnl.ARG_WEIGHTS, 2, (1, 16), DT["s8"]), dnnl.unimplemented),
+    ("src zp per-K groups multiple of 32", "u8", "s8", "f32",
+     lambda a: a.set_zero_points(dnnl.ARG_SRC, 3, (1, 32)), dnnl.success),
+    ("src zp K group 16 rejected", "u8", "s8", "f32",
+     lambda a: a.set_zero_points(dnnl.ARG_SRC, 3, (1, 16)), dnnl.unimplemented),
+    ("src zp per-M only rejected", "u8", "s8", "f32", lambda a: a.set_zero_points_mask(dnnl.ARG_SRC, 1), dnnl.unimplemented),
+    ("zero points on f32 src", "f32", "f32", "f32", lambda a: a.set_zero_points_mask(dnnl.ARG_SRC, 0), dnnl.unimplemented),
+    ("dst zp per-N", "u8", "s8", "u8", lambda a: a.set_zero_points_mask(dnnl.ARG_DST, 2), dnnl.success),
+    ("dst zp per-M rejected", "u8", "s8", "u8", lambda a: a.set_zero_points_mask(dnnl.ARG_DST, 1), dnnl.unimplemented),
+    ("precomputed reductions need weights zero points", "u8", "s8", "f32",
+     lambda a: a.set_precomputed_reductions(dnnl.ARG_SRC, 3, (1, 32)), dnnl.unimplemented),
+    ("precomputed reductions with weights zero points", "u8", "s8", "f32",
+     lambda a: (a.set_zero_points(dnnl.ARG_WEIGHTS, 3, (32, 1), DT["s8"]),
+                a.set_precomputed_reductions(dnnl.ARG_SRC, 3, (1, 32))), dnnl.success),
+    ("mx scales on f4", "f4_e2m1", "f4_e2m1", "bf16",
+     lambda a: (a.set_scales(dnnl.ARG_SRC, 3, (1, 32), DT["e8m0"]), a.set_scales(dnnl.ARG_WEIGHTS, 3, (32, 1), DT["e8m0"])),
+     dnnl.success),
+    ("scale on an argument matmul does not have", "u8", "s8", "f32", lambda a: a.set_scales_mask(dnnl.ARG_BIAS, 0),
+     dnnl.unimplemented),
+]
+
+
+@pytest.mark.parametrize("case", ATTR_CASES, ids=[c[0] for c in ATTR_CASES])
+def test_attribute_legality(eng, case):
+    _, s, w, d, build, want = case
+    a = _attr(build)
+    got = status_of(lambda: make_pd(eng, 64, 128, 64, s, w, d, attr=a))
+    assert got == want
+
+
+def test_unsupported_data_type_mixes(eng):
+    assert status_of(lambda: make_pd(eng, 16, 32, 16, "bf16", "u4", "bf16")) == dnnl.unimplemented   # no apply_to_int
+    assert status_of(lambda: make_pd(eng, 16, 32, 16, "u8", "f32", "f32")) == dnnl.unimplemented
+    assert status_of(lambda: make_pd(eng, 16, 32, 16, "f32", "f32", "s32")) == dnnl.unimplemented
+    assert status_of(lambda: make_pd(eng, 16, 32, 16, "f32", "f32", "f32")) == dnnl.success
+    assert status_of(lambda: make_pd(eng, 16, 32, 16, "u8", "s8", "f4_e2m1")) == dnnl.unimplemented
+
+
+def test_implementation_list_and_next_impl(eng):
+    a = dnnl.primitive_attr()
+    a.set_scales_mask(dnnl.ARG_SRC, 0)
+    a.set_scales_mask(dnnl.ARG_WEIGHTS, 2)
+    a.set_zero_points_mask(dnnl.ARG_SRC, 0)
+    pd = make_pd(eng, 256, 1024, 1024, "u8", "s8", "f32", attr=a, bias=md([1, 1024], "f32"))
+    assert pd.impl_info_str().startswith("hip:mfma_i8")
+    assert pd.next_impl() and pd.impl_info_str() == "hip:ref:any"
+    assert not pd.next_impl()                                  # last_impl_reached
+    # K not a multiple of the tile: only the generic kernel applies
+    pd = make_pd(eng, 256, 1000, 1024, "u8", "s8", "f32", attr=a)
+    assert pd.impl_info_str() == "hip:ref:any"
+    # fp8, mxfp4 and int4 decode pick their kernel families
+    assert make_pd(eng, 128, 256, 128, "f8_e4m3", "f8_e4m3", "bf16").impl_info_str().startswith("hip:mfma_f8")
+    mx = _attr(lambda t: (t.set_scales(dnnl.ARG_SRC, 3, (1, 32), DT["e8m0"]), t.set_scales(dnnl.ARG_WEIGHTS, 3, (32, 1), DT["e8m0"])))
+    assert make_pd(eng, 128, 256, 128, "f4_e2m1", "f4_e2m1", "bf16", attr=mx, wtag=dnnl.tag_ba).impl_info_str().startswith("hip:mfma_mxf4")
+    wo = _attr(lambda t: (t.set_fpmath_mode(dnnl.fpmath_bf16, True), t.set_scales(dnnl.ARG_WEIGHTS, 3, (128, 1), DT["bf16"]),
+                          t.set_zero_points(dnnl.ARG_WEIGHTS, 3, (128, 1), DT["u4"])))
+    assert make_pd(eng, 8, 4096, 14336, "bf16", "u4", "bf16", attr=wo).impl_info_str().startswith("hip:woq_gemv")
+
+
+def test_format_any_becomes_plain(eng):
+    pd = dnnl.matmul_primitive_desc(eng, md([8, 16], "s8", tag=dnnl.tag_any), md([16, 4], "s8", tag=dnnl.tag_any),
+                                    md([8, 4], "s32", tag=dnnl.tag_any))
+    assert pd.query_md(dnnl.query_src_md).strides() == [16, 1]
+    assert pd.query_md(dnnl.query_weights_md).strides() == [4, 1]
+    assert pd.query_md(dnnl.query_dst_md).strides() == [4, 1]
+
+
+def test_user_scratchpad_is_reported(eng):
+    a = dnnl.primitive_attr()
+    a.set_scratchpad_mode(dnnl.scratchpad_user)
+    a.set_zero_points_mask(dnnl.ARG_SRC, 0)
+    pd = make_pd(eng, 256, 1024, 1024, "u8", "s8", "s32", attr=a)     # `ab` weights: layout pre-pass + column sums
+    sp = pd.scratchpad_desc()
+    assert sp.ndims() == 1 and sp.dims()[0] >= 1024 * 1024
+    lib_mode = make_pd(eng, 256, 1024, 1024, "u8", "s8", "s32")
+    assert lib_mode.scratchpad_desc().ndims() == 0

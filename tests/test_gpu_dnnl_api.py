@@ -1,0 +1,133 @@
+"""End to end through the oneDNN-compatible C API (libdnnl_amd.so): engine,
+stream, memory objects, attributes, primitive descriptor, primitive, execute
+with the reference's argument ids -- results against the CPU oracle."""
+import numpy as np
+import pytest
+
+from onednn_amd import cabi, configs, dnnl
+from onednn_amd.problem import storage_dtype
+from tests.helpers import assert_bit_exact, assert_close
+
+pytestmark = pytest.mark.gpu
+DT = cabi.DT_NAMES
+
+
+def run_through_api(p, scratchpad_user=False):
+    """Builds the dnnl objects that describe MatmulProblem `p` (2-D, dense)."""
+    eng = dnnl.engine(dnnl.gpu, 0)
+    strm = dnnl.stream(eng)
+    src_md = dnnl.memory_desc([p.M, p.K], p.src_dt, strides=list(p.src_stride[1:]))
+    wei_md = dnnl.memory_desc([p.K, p.N], p.wei_dt, strides=list(p.wei_stride[1:]))
+    dst_md = dnnl.memory_desc([p.M, p.N], p.dst_dt, strides=list(p.dst_stride[1:]))
+    bias_md = dnnl.memory_desc([1, p.N], p.bias_dt, tag=dnnl.tag_ab) if p.bias is not None else None
+    attr = dnnl.primitive_attr()
+    args = {}
+    name_to = {"src": dnnl.ARG_SRC, "wei": dnnl.ARG_WEIGHTS, "dst": dnnl.ARG_DST}
+    for qname, q in p.quant.items():
+        which, kind = qname.split("_")
+        arg = name_to[which]
+        mask2d = q.mask >> 1                       # (row, col) bits of the 2-D argument
+        groups = q.groups if q.groups != (1, 1) else ()
+        dims = {"src": (p.M, p.K), "wei": (p.K, p.N), "dst": (p.M, p.N)}[which]
+        g = q.groups
+        qdims = [dims[0] // g[0] if mask2d & 1 else 1, dims[1] // g[1] if mask2d & 2 else 1]
+        if kind == "scale":
+            attr.set_scales(arg, mask2d, groups, q.dt)
+            flag = dnnl.ARG_ATTR_SCALES
+        elif kind == "zp":
+            attr.set_zero_points(arg, mask2d, groups, q.dt)
+            flag = dnnl.ARG_ATTR_ZERO_POINTS
+        else:
+            attr.set_precomputed_reductions(arg, mask2d, groups, q.dt)
+            flag = dnnl.ARG_ATTR_PRECOMPUTED_REDUCTIONS
+        qmd = dnnl.memory_desc(qdims, q.dt, tag=dnnl.tag_ab)
+        args[flag | arg] = dnnl.memory(qmd, eng, q.data)
+    if p.apply_to_int:
+        attr.set_fpmath_mode(dnnl.fpmath_bf16, True)
+    po = dnnl.post_ops()
+    for i, op in enumerate(p.post_ops):
+        if op.kind == cabi.PO_ELTWISE:
+            po.append_eltwise(op.alg, op.alpha, op.beta)
+        elif op.kind == cabi.PO_BINARY:
+            dims = [p.M if op.stride[1] else 1, p.N if op.stride[2] else 1]
+            bmd = dnnl.memory_desc(dims, op.dt, tag=dnnl.tag_ab)
+            po.append_binary(op.alg, bmd)
+            args[dnnl.ARG_ATTR_MULTIPLE_POST_OP(i) | dnnl.ARG_SRC_1] = dnnl.memory(bmd, eng, op.data)
+        elif op.kind == cabi.PO_SUM:
+            po.append_sum(op.scale, op.zero_point, op.dt)
+    if p.post_ops:
+        attr.set_post_ops(po)
+    if scratchpad_user:
+        attr.set_scratchpad_mode(dnnl.scratchpad_user)
+    pd = dnnl.matmul_primitive_desc(eng, src_md, wei_md, dst_md, bias_md=bias_md, attr=attr)
+    prim = dnnl.matmul(pd)
+    args[dnnl.ARG_SRC] = dnnl.memory(src_md, eng, p.src)
+    args[dnnl.ARG_WEIGHTS] = dnnl.memory(wei_md, eng, p.wei)
+    dst = dnnl.memory(dst_md, eng, p.initial_dst())
+    args[dnnl.ARG_DST] = dst
+    if p.bias is not None:
+        args[dnnl.ARG_BIAS] = dnnl.memory(bias_md, eng, p.bias)
+    if scratchpad_user:
+        sp = pd.scratchpad_desc()
+        if sp.ndims():
+            args[dnnl.ARG_SCRATCHPAD] = dnnl.memory(sp, eng)
+    prim.execute(strm, args)
+    strm.wait()
+    return dst.read(storage_dtype(p.dst_dt)), pd.impl_info_str(), (pd, prim, strm, args)
+
+
+@pytest.mark.parametrize("dst", ["s32", "f32"])
+def test_config1_through_the_api(gpu, oracle, dst):
+    p = configs.config1(M=256, N=512, K=512, dst=dst)
+    got, impl, _ = run_through_api(p)
+    assert impl.startswith("hip:mfma_i8")
+    assert_bit_exact(p, got, oracle.run_oracle(p), impl)
+
+
+def test_config3_user_scratchpad_and_next_impl(gpu, oracle):
+    p = configs.config3(M=256, N=256, K=512)
+    got, impl, keep = run_through_api(p, scratchpad_user=True)
+    want = oracle.run_oracle(p)
+    assert_bit_exact(p, got, want, impl)
+    # the second implementation of the list (generic kernel) gives the same bits
+    pd, _, strm, args = keep
+    assert pd.next_impl() and pd.impl_info_str() == "hip:ref:any"
+    prim2 = dnnl.matmul(pd)
+    args[dnnl.ARG_DST].write(p.initial_dst())
+    prim2.execute(strm, args)
+    strm.wait()
+    assert_bit_exact(p, args[dnnl.ARG_DST].read(np.int8), want, "hip:ref:any")
+
+
+def test_config2_through_the_api(gpu, oracle):
+    p = configs.config2(M=8, N=512, K=1024)
+    got, impl, _ = run_through_api(p)
+    assert impl.startswith("hip:woq_gemv")
+    want, _, asum = oracle.run_oracle(p, want_ideal=True)
+    assert_close(p, got, want, abs_sum=asum * 20.0, what=impl)
+
+
+def test_config4_through_the_api(gpu, oracle):
+    p = configs.config4(M=256, N=256, K=512)
+    got, impl, _ = run_through_api(p)
+    assert impl.startswith("hip:mfma_f8")
+    want, _, asum = oracle.run_oracle(p, want_ideal=True)
+    assert_close(p, got, want, abs_sum=asum, transcendental=True, what=impl)
+
+
+def test_config5_through_the_api(gpu, oracle):
+    p = configs.config5(M=256, N=256, K=512)
+    got, impl, _ = run_through_api(p)
+    assert impl.startswith("hip:mfma_mxf4")
+    want, _, asum = oracle.run_oracle(p, want_ideal=True)
+    assert_close(p, got, want, abs_sum=asum, what=impl)
+
+
+def test_missing_argument_is_invalid_arguments(gpu):
+    p = configs.config1(M=64, N=64, K=64, dst="s32")
+    _, _, (pd, prim, strm, args) = run_through_api(p)
+    bad = dict(args)
+    del bad[dnnl.ARG_ATTR_ZERO_POINTS | dnnl.ARG_SRC]
+    with pytest.raises(dnnl.error) as e:
+        prim.execute(strm, bad)
+    assert e.value.status == dnnl.invalid_arguments
