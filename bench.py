@@ -70,18 +70,23 @@ class Timer:
         return ms.value / iters
 
 
-def build_problem(name, M=None):
+def build_problem(name, M=None, wtag="any"):
+    """`any` is what weights format_tag::any resolves to in the primitive
+    descriptor: K-contiguous (ba) for the MFMA operand types, row-major (ab)
+    for the int4 decode weights.  With an explicit `ab` the MFMA families run
+    a layout pre-pass inside every launch, which then is part of the step."""
     from onednn_amd import configs
     if name == "c1":
         return configs.config1()
     if name == "c2":
-        return configs.config2(M=M or 1)
+        return configs.config2(M=M or 1, wtag="ab" if wtag == "any" else wtag)
+    mfma_tag = "ba" if wtag == "any" else wtag
     if name == "c3":
-        return configs.config3()
+        return configs.config3(wtag=mfma_tag)
     if name == "c4":
-        return configs.config4()
+        return configs.config4(wtag=mfma_tag)
     if name == "c5":
-        return configs.config5()
+        return configs.config5(wtag=mfma_tag)
     raise ValueError(name)
 
 
@@ -106,12 +111,12 @@ def rate(work, ms, unit):
     return work / (ms * 1e-3) / 1e12
 
 
-def run_gpu_workload(lib, name, steps, warmup, M=None, cold_copies=0):
+def run_gpu_workload(lib, name, steps, warmup, M=None, cold_copies=0, wtag="any"):
     """Returns dict with ms_per_step, value, unit, impl."""
     from onednn_amd import cabi
     from onednn_amd.problem import GpuRun
     t0 = time.time()
-    p = build_problem(name, M)
+    p = build_problem(name, M, wtag)
     log(f"[bench] {name}: generated {p.name} in {time.time() - t0:.1f}s")
     runs = [GpuRun(p)]
     # decode is HBM-bound only if the weights are not already in the 256 MB
@@ -178,8 +183,13 @@ def main():
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--workload", default="c3", choices=["c1", "c2", "c3", "c4", "c5"])
     ap.add_argument("--decode-m", type=int, default=1, help="M of the c2 decode workload")
+    ap.add_argument("--wtag", default="any", choices=["any", "ab", "ba"],
+                    help="weights layout; any = what format_tag::any resolves to (default)")
     ap.add_argument("--no-others", action="store_true", help="skip the informational configs")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--calib-copy", action="store_true",
+                    help="also launch the plain copy kernel on 256 MiB three times: the known-size "
+                         "dispatch that FETCH_SIZE / WRITE_SIZE counter passes are scaled by")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build runs on one GPU (one-GPU boxes only); "
@@ -202,9 +212,19 @@ def main():
 
     main_name = args.workload
     cold = 11 if main_name == "c2" else 0
-    res, prob = run_gpu_workload(lib, main_name, args.steps, args.warmup, args.decode_m, cold)
+    res, prob = run_gpu_workload(lib, main_name, args.steps, args.warmup, args.decode_m, cold,
+                                 args.wtag)
     log(f"[bench] {res['workload']}: {res['ms_per_step']:.4f} ms/step -> {res['value']:.1f} "
         f"{res['unit']} via {res['impl']}")
+
+    if args.calib_copy:
+        nbytes = 256 << 20
+        a, b = cabi.DeviceBuffer(nbytes), cabi.DeviceBuffer(nbytes)
+        for _ in range(3):
+            cabi.check(lib.mi355_copy_kernel(b.ptr, a.ptr, C.c_size_t(nbytes), None))
+        cabi.check(lib.mi355_stream_sync(None))
+        a.free()
+        b.free()
 
     # The timed step is one launch whose time is dominated by one kernel (the
     # tile GEMM / the decode kernel); pre-pass kernels of the same launch

@@ -64,6 +64,46 @@ def config2(M=1, N=14336, K=4096, group=128, seed=2, impl=cabi.IMPL_AUTO, wtag="
                          fpmath_mode=1, impl=impl, name=f"C2-M{M}")
 
 
+def woq_variant(M, N, K, group, wei_dt="u4", sc_dt="bf16", zp_dt="u4", zp_kind="grouped", sc_kind="grouped",
+                dst_dt="bf16", relu_bias=False, seed=12):
+    """Weight-only int4 decode in the attribute combinations the reference admits
+    (matmul_pd.hpp:131-226): s4 / u4 weights; f32 / bf16 / f16 scales, grouped
+    along K or per column; s32 / s8 / u8 / s4 / u4 zero points, grouped, per
+    column, one common value, or none; optional f32 bias + ReLU."""
+    names = {"f32": cabi.DT_F32, "bf16": cabi.DT_BF16, "f16": cabi.DT_F16, "s32": cabi.DT_S32, "s8": cabi.DT_S8,
+             "u8": cabi.DT_U8, "s4": cabi.DT_S4, "u4": cabi.DT_U4}
+    src = dtp.f32_to_bf16(_rng(seed, 1).standard_normal((M, K)).astype(np.float32))
+    codes = _rng(seed, 2).integers(0, 16, size=(K, N), dtype=np.uint8)  # raw nibbles, s4 reads them as signed
+    wei = dtp.pack_nibbles(codes)
+    G = K // group
+
+    def shaped(kind):
+        return {"grouped": ((G, N), MASK_ROW | MASK_COL, (group, 1)), "column": ((N,), MASK_COL, (1, 1)),
+                "common": ((1,), MASK_COMMON, (1, 1))}[kind]
+
+    quant = {}
+    if sc_kind != "none":
+        shape, mask, grp = shaped(sc_kind)
+        v = _rng(seed, 3).uniform(0.005, 0.02, size=shape).astype(np.float32)
+        raw = {"f32": v, "bf16": dtp.f32_to_bf16(v), "f16": v.astype(np.float16).view(np.uint16)}[sc_dt]
+        quant["wei_scale"] = QuantParam(names[sc_dt], mask, raw, grp)
+    if zp_kind != "none":
+        shape, mask, grp = shaped(zp_kind)
+        lo, hi = {"s32": (-20, 21), "s8": (-20, 21), "u8": (0, 21), "s4": (-8, 8), "u4": (0, 16)}[zp_dt]
+        z = _rng(seed, 4).integers(lo, hi, size=shape)
+        raw = {"s32": z.astype(np.int32), "s8": z.astype(np.int8), "u8": z.astype(np.uint8),
+               "s4": dtp.pack_nibbles((z & 0xF).astype(np.uint8)), "u4": dtp.pack_nibbles(z.astype(np.uint8))}[zp_dt]
+        quant["wei_zp"] = QuantParam(names[zp_dt], mask, raw, grp)
+    kw = {}
+    if relu_bias:
+        kw["bias_dt"] = cabi.DT_F32
+        kw["bias"] = _rng(seed, 5).uniform(-1, 1, size=N).astype(np.float32)
+        kw["post_ops"] = [PostOp(kind=cabi.PO_ELTWISE, alg=cabi.ELTWISE["relu"], alpha=0.0, beta=0.0, scale=1.0)]
+    return MatmulProblem(M=M, N=N, K=K, src_dt=cabi.DT_BF16, wei_dt=names[wei_dt], dst_dt=names[dst_dt], src=src,
+                         wei=wei, wei_stride=strides_for("ab", 1, K, N), quant=quant, apply_to_int=True,
+                         fpmath_mode=1, name=f"WOQ-{wei_dt}-{sc_dt}/{sc_kind}-{zp_dt}/{zp_kind}-M{M}", **kw)
+
+
 def config3(M=8192, N=8192, K=8192, seed=3, impl=cabi.IMPL_AUTO, wtag="ab",
             dst_scale_mode=cabi.DST_SCALE_DIVIDE):
     """s8 x s8 -> s8: src scale 0.01, per-N weights scales, dst scale 0.05,

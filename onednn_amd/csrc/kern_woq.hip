@@ -23,23 +23,25 @@
 // at once), the products run on the bf16 matrix cores, and the per-weight
 // subtract/multiply of the naive formula moves to once per group and column.
 //
-// Data flow per wavefront step (16 k-rows x 16 lanes x 8*CHD columns):
-//   lane (c = lane%16, q = lane/16) loads CHD dwords of rows k0+4q .. k0+4q+3 at
+// Data flow per wavefront step (16 k-rows x 16 lanes x 16 columns):
+//   lane (c = lane%16, q = lane/16) loads two dwords of rows k0+4q .. k0+4q+3 at
 //   column chunk c; every dword yields four bf16 pairs (n, n+4) by shift+and_or;
 //   the four rows of one pair are the B operand of v_mfma_f32_16x16x32_bf16
 //   (MFMA k-slot 2t+h <-> row 4q+t, column half h); the A operand interleaves
 //   zeros, (s,0,s,0,..) or (0,s,0,s,..), so that one MFMA yields column n and a
 //   second one column n+4.  An MFMA against an all-ones B gives sum_k src[m,k].
 //
-// Work split: grid = column chunks x K splits; the 4 wavefronts of a workgroup
-// take consecutive K sub-ranges, reduce through LDS, and the workgroup writes
-// one f32 partial [M][chunk] to scratch.  The last workgroup to arrive for a
-// chunk (epoch-stamped arrival counter in scratch, so scratch needs no
-// initialisation) adds the partials in split order -- deterministic -- and runs
-// the shared epilogue.
-#include <stdlib.h>
-
+// Work split: grid = column chunks x K splits, sized to one workgroup per CU
+// (a CU sustains ~35 GB/s of misses, so every CU has to pull its share, and
+// row segments shorter than a 128-byte line are fetched whole: chunks are 256
+// columns wide).  A wavefront keeps the weight loads of four 16-row steps in
+// flight ahead of the MFMAs, and the wavefronts of a workgroup reduce through
+// LDS into one f32 partial [M][chunk] in scratch.  The last workgroup
+// to arrive for a chunk (one wrapping atomic increment on a counter that is
+// zero between launches) adds the partials in split order -- deterministic --
+// and runs the shared epilogue.
 #include <atomic>
+#include <mutex>
 
 #include "kernels.hpp"
 
@@ -48,96 +50,135 @@ namespace {
 
 typedef int v4i __attribute__((ext_vector_type(4)));
 typedef float v4f __attribute__((ext_vector_type(4)));
+typedef unsigned v2u __attribute__((ext_vector_type(2)));
 typedef __bf16 v8bf __attribute__((ext_vector_type(8)));
 
-constexpr int COUNTER_BYTES = 4096; // up to 1024 column chunks
+constexpr int NPL = 16;      // columns per lane (two dwords of nibbles)
+constexpr int NW = 16 * NPL; // columns per wavefront / workgroup: 128-byte row segments
+constexpr int NP = 8;        // bf16 pairs per lane per row
 
+// Arrival counters live in library-owned device memory: zero when the module
+// is loaded, and every launch leaves the counters it used at zero again (the
+// increment wraps at the number of splits).  A launch takes the next of
+// COUNTER_SLOTS blocks, so launches that overlap on different streams do not
+// share counters unless more than COUNTER_SLOTS are in flight.
+constexpr int COUNTER_SLOTS = 32;
+constexpr int MAX_CHUNKS = 1024;
+__device__ unsigned g_arrivals[COUNTER_SLOTS][MAX_CHUNKS];
+
+// Everything the main loop needs, gathered in one argument so that the kernel
+// starts with a single block of scalar loads: the first weight load must not
+// wait behind a chain of dependent argument fetches.
 struct woq_extra_t {
-    unsigned *counters; // [chunks] epoch-stamped arrival counters
-    float *partials;    // [ksplit][M][N]
-    unsigned epoch;     // 24-bit, never 0
-    int ksplit;         // K splits across workgroups
-    int krange;         // k per workgroup (multiple of 64)
-    int G;              // k per quantization group (multiple of 16), K if ungrouped
+    const uint8_t *wei;  // [K][N/2]
+    const uint8_t *src;  // bf16 [M][src_ld]
+    const uint8_t *sc, *zp; // weights scales / zero points (NULL when absent)
+    float *partials;     // [ksplit][M][N]
+    unsigned *counters;  // [chunks] arrival counters, zero between launches
+    int M, N, K, src_ld;
+    int row_bytes;       // N / 2
+    int krange;          // k per workgroup (multiple of 16 * wavefronts)
+    int ksplit;          // K splits across workgroups
+    int G;               // k per quantization group (multiple of 16), K if ungrouped
+    int sc_dt, zp_dt;    // MI355_DT_UNDEF when absent
     int sc_grouped, zp_grouped; // parameter has a K dimension
-    int zp_common;      // single zero point
-    int signed_w;       // s4 weights
+    int zp_common;       // single zero point
+    int signed_w;        // s4 weights
 };
 
 __device__ __forceinline__ v8bf as_bf(const v4i &x) { return __builtin_bit_cast(v8bf, x); }
 
-// NPL consecutive parameter values held as raw 32-bit words -> f32; one
-// data-type dispatch, fully unrolled bodies (static register indices)
-template <int NPL>
-__device__ __forceinline__ void decode_raw(int dt, const uint4 (&r)[NPL / 4], float (&out)[NPL]) {
-    unsigned w[NPL];
+// NPL consecutive parameter values of BITS bits each, as raw dwords
+template <int BITS>
+struct raw_t {
+    static constexpr int DW = BITS ? NPL * BITS / 32 : 1;
+    unsigned w[DW];
+};
+
+template <int BITS>
+__device__ __forceinline__ void load_raw(raw_t<BITS> &r, const uint8_t *p) {
+    if constexpr (BITS == 4) {
+        const uint2 v = *(const uint2 *)p;
+        r.w[0] = v.x; r.w[1] = v.y;
+    } else if constexpr (BITS != 0) {
 #pragma unroll
-    for (int i = 0; i < NPL / 4; ++i) {
-        w[4 * i] = r[i].x; w[4 * i + 1] = r[i].y; w[4 * i + 2] = r[i].z; w[4 * i + 3] = r[i].w;
-    }
-    switch (dt) {
-        case MI355_DT_F32:
-#pragma unroll
-            for (int i = 0; i < NPL; ++i) out[i] = u2f(w[i]);
-            break;
-        case MI355_DT_S32:
-#pragma unroll
-            for (int i = 0; i < NPL; ++i) out[i] = (float)(int)w[i];
-            break;
-        case MI355_DT_BF16:
-#pragma unroll
-            for (int i = 0; i < NPL; ++i) out[i] = u2f((w[i / 2] >> ((i & 1) * 16)) << 16);
-            break;
-        case MI355_DT_F16:
-#pragma unroll
-            for (int i = 0; i < NPL; ++i) out[i] = f16_to_f32((uint16_t)(w[i / 2] >> ((i & 1) * 16)));
-            break;
-        case MI355_DT_S8:
-#pragma unroll
-            for (int i = 0; i < NPL; ++i) out[i] = (float)(int)(int8_t)((w[i / 4] >> ((i & 3) * 8)) & 0xffu);
-            break;
-        case MI355_DT_U8:
-#pragma unroll
-            for (int i = 0; i < NPL; ++i) out[i] = (float)((w[i / 4] >> ((i & 3) * 8)) & 0xffu);
-            break;
-        case MI355_DT_S4:
-#pragma unroll
-            for (int i = 0; i < NPL; ++i) out[i] = (float)s4_to_int((uint8_t)((w[i / 8] >> ((i & 7) * 4)) & 0xfu));
-            break;
-        default: // u4
-#pragma unroll
-            for (int i = 0; i < NPL; ++i) out[i] = (float)((w[i / 8] >> ((i & 7) * 4)) & 0xfu);
-            break;
+        for (int i = 0; i < raw_t<BITS>::DW / 4; ++i) {
+            const uint4 v = *(const uint4 *)(p + 16 * i);
+            r.w[4 * i] = v.x; r.w[4 * i + 1] = v.y; r.w[4 * i + 2] = v.z; r.w[4 * i + 3] = v.w;
+        }
     }
 }
 
-// NWV wavefronts per workgroup share one column chunk and split its K range.
-template <int CHD, int MT, int NWV>
+// scales: f32 (32 bits) or bf16 / f16 (16 bits)
+template <int BITS>
+__device__ __forceinline__ void decode_scales(int dt, const raw_t<BITS> &r, float (&out)[NPL]) {
+    if constexpr (BITS == 32) {
+#pragma unroll
+        for (int i = 0; i < NPL; ++i) out[i] = u2f(r.w[i]);
+    } else if constexpr (BITS == 16) {
+        if (dt == MI355_DT_BF16) {
+#pragma unroll
+            for (int i = 0; i < NPL; ++i) out[i] = u2f((r.w[i / 2] >> ((i & 1) * 16)) << 16);
+        } else {
+#pragma unroll
+            for (int i = 0; i < NPL; ++i) out[i] = f16_to_f32((uint16_t)(r.w[i / 2] >> ((i & 1) * 16)));
+        }
+    } else {
+#pragma unroll
+        for (int i = 0; i < NPL; ++i) out[i] = 1.f;
+    }
+}
+
+// zero points: s32 (32 bits), s8 / u8 (8 bits), s4 / u4 (4 bits)
+template <int BITS>
+__device__ __forceinline__ void decode_zps(int dt, const raw_t<BITS> &r, float (&out)[NPL]) {
+    if constexpr (BITS == 32) {
+#pragma unroll
+        for (int i = 0; i < NPL; ++i) out[i] = (float)(int)r.w[i];
+    } else if constexpr (BITS == 8) {
+        if (dt == MI355_DT_U8) {
+#pragma unroll
+            for (int i = 0; i < NPL; ++i) out[i] = (float)((r.w[i / 4] >> ((i & 3) * 8)) & 0xffu);
+        } else {
+#pragma unroll
+            for (int i = 0; i < NPL; ++i) out[i] = (float)(int)(int8_t)((r.w[i / 4] >> ((i & 3) * 8)) & 0xffu);
+        }
+    } else if constexpr (BITS == 4) {
+        // s4 as offset-binary: (nibble ^ 8) - 8
+        const unsigned flip = dt == MI355_DT_S4 ? 0x88888888u : 0u;
+        const float bias = dt == MI355_DT_S4 ? -8.f : 0.f;
+#pragma unroll
+        for (int i = 0; i < NPL; ++i) out[i] = (float)(((r.w[i / 8] ^ flip) >> ((i & 7) * 4)) & 0xfu) + bias;
+    } else {
+#pragma unroll
+        for (int i = 0; i < NPL; ++i) out[i] = 0.f;
+    }
+}
+
+// MT 16-row tiles of activations; NWV wavefronts per workgroup share one column
+// chunk and split its K range; SS = 16-row steps of one super-step; SCB / ZPB =
+// bits per scale / zero point (0 = absent).
+template <int MT, int NWV, int SS, int SCB, int ZPB>
 __global__ void __launch_bounds__(NWV * 64) woq_gemv_kernel(const problem_t P_, const woq_extra_t X) {
-    const auto &P = MI355_KERNARG_PROBLEM();
-    extern __shared__ __attribute__((aligned(16))) float red[]; // [4][M][NW]
-    constexpr int NPL = CHD * 8;      // columns per lane
-    constexpr int NW = 16 * NPL;      // columns per wavefront / workgroup
-    constexpr int NP = CHD * 4;       // bf16 pairs per lane per row
+    extern __shared__ __attribute__((aligned(16))) float red[]; // [NWV][M][NW], columns permuted
+    constexpr int PF = SS < 4 ? SS : 4; // weight steps in flight ahead of the MFMAs
     constexpr int WOQ_NT = NWV * 64;
-    const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
+    const int t = threadIdx.x, lane = t & 63;
+    // uniform: addresses below split into a scalar base and one 32-bit lane offset
+    const int wave = __builtin_amdgcn_readfirstlane(t >> 6);
     const int c = lane & 15, q = lane >> 4;
     const int chunk = blockIdx.x, split = blockIdx.y;
-    const long N = P.N, K = P.K;
-    const int M = (int)P.M;
-    const long n_lane = (long)chunk * NW + c * NPL; // first column of this lane
-    const bool lane_on = n_lane < N;                // N is a multiple of NPL
+    const int N = X.N, K = X.K, M = X.M;
+    // Lanes whose columns lie beyond N (last chunk) and MFMA rows beyond M read
+    // the last valid columns / row instead: every output element depends on its
+    // own row and column only, and those results are never stored.
+    const int n_lane = chunk * NW + c * NPL;
+    const int n_ld = n_lane < N - NPL ? n_lane : N - NPL;
 
-    // K sub-range of this wavefront: quarter of the workgroup's range, in 16-row steps
-    const int kr4 = X.krange / NWV;
-    long kb = (long)split * X.krange + (long)wave * kr4;
-    long ke = kb + kr4;
-    if (ke > K) ke = K;
-
-    const uint8_t *wei = (const uint8_t *)P.wei;
-    const long row_bytes = N / 2;
-    const uint16_t *src = (const uint16_t *)P.src;
-    const long lds = P.ss[1];
+    // K sub-range of this wavefront: its share of the workgroup's range, in 16-row steps
+    const int krw = X.krange / NWV;
+    const int kb = split * X.krange + wave * krw;
+    const int ke = kb + krw < K ? kb + krw : K;
 
     v4f acc[NP][2][MT], rs[MT];
 #pragma unroll
@@ -145,41 +186,44 @@ __global__ void __launch_bounds__(NWV * 64) woq_gemv_kernel(const problem_t P_, 
 #pragma unroll
         for (int h = 0; h < 2; ++h)
 #pragma unroll
-            for (int mt = 0; mt < MT; ++mt) {
-                acc[p][h][mt] = v4f {0.f, 0.f, 0.f, 0.f};
-            }
+            for (int mt = 0; mt < MT; ++mt) acc[p][h][mt] = v4f {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt) rs[mt] = v4f {0.f, 0.f, 0.f, 0.f};
 
     struct step_t {
-        unsigned w[4][CHD]; // rows 4q+t, dwords of this lane's chunk
-        uint2 a[MT];        // src[m][k0+4q .. +3] as four bf16
+        v2u w[4];    // rows 4q+t, the two dwords of this lane's columns
+        uint2 a[MT]; // src[m][k0+4q .. +3] as four bf16
     };
-    auto load_step = [&](step_t &s, long k0) __attribute__((always_inline)) {
-        const long kr = k0 + 4 * q;
+    const unsigned wei_lane_off = (unsigned)(4 * q * X.row_bytes + n_ld / 2);
+    unsigned src_lane_off[MT];
 #pragma unroll
-        for (int tt = 0; tt < 4; ++tt) {
-            const uint8_t *p = wei + (kr + tt) * row_bytes + n_lane / 2;
-            if (CHD == 4) {
-                uint4 v = lane_on ? *(const uint4 *)p : make_uint4(0, 0, 0, 0);
-                s.w[tt][0] = v.x; s.w[tt][1 % CHD] = v.y; s.w[tt][2 % CHD] = v.z; s.w[tt][3 % CHD] = v.w;
-            } else if (CHD == 2) {
-                uint2 v = lane_on ? *(const uint2 *)p : make_uint2(0, 0);
-                s.w[tt][0] = v.x; s.w[tt][1 % CHD] = v.y;
-            } else {
-                s.w[tt][0] = lane_on ? *(const unsigned *)p : 0u;
-            }
-        }
+    for (int mt = 0; mt < MT; ++mt) {
+        const int m = mt * 16 + c < M ? mt * 16 + c : M - 1;
+        src_lane_off[mt] = (unsigned)(m * X.src_ld * 2 + 4 * q * 2);
+    }
+    auto load_src = [&](step_t &s, int k0) __attribute__((always_inline)) {
 #pragma unroll
-        for (int mt = 0; mt < MT; ++mt) {
-            const int m = mt * 16 + c;
-            s.a[mt] = m < M ? *(const uint2 *)(src + (long)m * lds + kr) : make_uint2(0, 0);
-        }
+        for (int mt = 0; mt < MT; ++mt) s.a[mt] = *(const uint2 *)(X.src + (long)k0 * 2 + src_lane_off[mt]);
+    };
+    // the weights are read once: non-temporal loads keep them from displacing
+    // the activations and parameters in the caches
+    auto load_wei = [&](step_t &s, int k0) __attribute__((always_inline)) {
+#pragma unroll
+        for (int tt = 0; tt < 4; ++tt)
+            s.w[tt] = __builtin_nontemporal_load((const v2u *)(X.wei + (long)(k0 + tt) * X.row_bytes + wei_lane_off));
     };
 
-    const unsigned sx = X.signed_w ? 0x88888888u : 0u; // s4 -> offset-binary
+    // 0x4300 | nibble = bf16(128 + nibble).  The constant is kept in a vector
+    // register: a VOP3 instruction takes one scalar operand at most, so
+    // (x & mask) | magic fuses into v_and_or_b32 only when `magic` is not scalar.
+    unsigned magic;
+    asm volatile("v_mov_b32 %0, 0x43004300" : "=v"(magic));
     const v4i ones = {0x3F803F80, 0x3F803F80, 0x3F803F80, 0x3F803F80};
-    auto compute_step = [&](const step_t &s) __attribute__((always_inline)) {
+    auto compute_step = [&](step_t &s) __attribute__((always_inline)) {
+        if (X.signed_w) { // s4 -> offset-binary
+#pragma unroll
+            for (int tt = 0; tt < 4; ++tt) s.w[tt] ^= v2u {0x88888888u, 0x88888888u};
+        }
         v4i aa[MT], ab[MT];
 #pragma unroll
         for (int mt = 0; mt < MT; ++mt) {
@@ -189,13 +233,12 @@ __global__ void __launch_bounds__(NWV * 64) woq_gemv_kernel(const problem_t P_, 
             rs[mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf(aa[mt]), as_bf(ones), rs[mt], 0, 0, 0);
         }
 #pragma unroll
-        for (int d = 0; d < CHD; ++d) {
+        for (int d = 0; d < 2; ++d) {
 #pragma unroll
             for (int sh = 0; sh < 4; ++sh) {
                 v4i b;
 #pragma unroll
-                for (int tt = 0; tt < 4; ++tt)
-                    b[tt] = (int)((((s.w[tt][d] ^ sx) >> (4 * sh)) & 0x000F000Fu) | 0x43004300u);
+                for (int tt = 0; tt < 4; ++tt) b[tt] = (int)(((s.w[tt][d] >> (4 * sh)) & 0x000F000Fu) | magic);
                 const int p = d * 4 + sh;
 #pragma unroll
                 for (int mt = 0; mt < MT; ++mt) {
@@ -206,218 +249,212 @@ __global__ void __launch_bounds__(NWV * 64) woq_gemv_kernel(const problem_t P_, 
         }
     };
 
-    // Quantization parameters of one group for this lane's NPL columns, fetched
-    // as raw vectors (no data-type dispatch between the loads, so they are all
-    // in flight together) when the group starts and decoded when it ends.
-    constexpr int RAWQ = NPL / 4; // uint4 registers for NPL 32-bit values
+    // Quantization parameters of one group for this lane's columns: raw loads
+    // when the group starts, decoded when it ends.
     struct qraw_t {
-        uint4 s[RAWQ], z[RAWQ];
+        raw_t<SCB> s;
+        raw_t<ZPB> z;
     };
-    const int sc_bits = dt_bits(P.wei_scale.dt), zp_bits = dt_bits(P.wei_zp.dt);
-    const bool with_sc = P.wei_scale.dt != MI355_DT_UNDEF, with_zp = P.wei_zp.dt != MI355_DT_UNDEF;
-    auto load_raw = [&](uint4 (&r)[RAWQ], const void *base, long elem_off, int bits) {
-        // NPL consecutive elements of `bits` bits starting at element elem_off
-        const char *p = (const char *)base + elem_off * bits / 8;
-        const int bytes = NPL * bits / 8;
-#pragma unroll
-        for (int i = 0; i < RAWQ; ++i) {
-            r[i] = make_uint4(0, 0, 0, 0);
-            if (i * 16 + 16 <= bytes) r[i] = *(const uint4 *)(p + i * 16);
-            else if (i * 16 + 8 <= bytes) {
-                const uint2 v = *(const uint2 *)(p + i * 16);
-                r[i].x = v.x; r[i].y = v.y;
-            } else if (i * 16 + 4 <= bytes) r[i].x = *(const unsigned *)(p + i * 16);
+    auto fetch_group = [&](qraw_t &qr, int g) __attribute__((always_inline)) {
+        if constexpr (SCB != 0)
+            load_raw<SCB>(qr.s, X.sc + ((long)(X.sc_grouped ? g : 0) * N * SCB / 8 + (unsigned)(n_ld * SCB / 8)));
+        if constexpr (ZPB != 0) {
+            if (X.zp_common) // element 0 for every column
+                qr.z.w[0] = ZPB == 32 ? *(const unsigned *)X.zp : (unsigned)*X.zp;
+            else
+                load_raw<ZPB>(qr.z, X.zp + ((long)(X.zp_grouped ? g : 0) * N * ZPB / 8 + (unsigned)(n_ld * ZPB / 8)));
         }
     };
-    auto fetch_group = [&](qraw_t &qr, long g) __attribute__((always_inline)) {
-        if (!lane_on) return;
-        if (with_sc) load_raw(qr.s, P.wei_scale.p, (X.sc_grouped ? g * N : 0) + n_lane, sc_bits);
-        if (with_zp && !X.zp_common) load_raw(qr.z, P.wei_zp.p, (X.zp_grouped ? g * N : 0) + n_lane, zp_bits);
-    };
-    const float zp_common_val = (with_zp && X.zp_common) ? load_float(P.wei_zp.dt, P.wei_zp.p, 0) : 0.f;
 
     // fold one finished group into this wavefront's LDS slice:
     //   red[wave][m][n] (+)= scale * (acc - (128 + zp) * rowsum)
+    // column i of lane c is kept at i * 16 + c: the 16 lanes of a row write
+    // consecutive words
     bool first_flush = true;
     auto flush_group = [&](const qraw_t &qr) __attribute__((always_inline)) {
         float sc[NPL], zc[NPL];
-        const float zbase = (X.signed_w ? 136.f : 128.f) + zp_common_val;
+        decode_scales<SCB>(X.sc_dt, qr.s, sc);
+        decode_zps<ZPB>(X.zp_dt, qr.z, zc);
+        if (ZPB != 0 && X.zp_common) {
 #pragma unroll
-        for (int i = 0; i < NPL; ++i) { sc[i] = 1.f; zc[i] = 0.f; }
-        if (with_sc && lane_on) decode_raw<NPL>(P.wei_scale.dt, qr.s, sc);
-        if (with_zp && !X.zp_common && lane_on) decode_raw<NPL>(P.wei_zp.dt, qr.z, zc);
+            for (int i = 1; i < NPL; ++i) zc[i] = zc[0];
+        }
+        const float zbase = X.signed_w ? 136.f : 128.f;
 #pragma unroll
         for (int i = 0; i < NPL; ++i) zc[i] += zbase;
 #pragma unroll
+        for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                const int m = mt * 16 + q * 4 + r;
+                if (m < M) {
+                    float *row = &red[(wave * M + m) * NW + c];
+#pragma unroll
+                    for (int p = 0; p < NP; ++p)
+#pragma unroll
+                        for (int h = 0; h < 2; ++h) {
+                            const int i = (p / 4) * 8 + h * 4 + (p % 4); // column of (pair p, half h)
+                            const float tmp = __builtin_fmaf(-zc[i], rs[mt][r], acc[p][h][mt][r]);
+                            row[i * 16] = first_flush ? sc[i] * tmp : __builtin_fmaf(sc[i], tmp, row[i * 16]);
+                        }
+                }
+            }
+#pragma unroll
         for (int p = 0; p < NP; ++p)
 #pragma unroll
-            for (int h = 0; h < 2; ++h) {
-                const int i = (p / 4) * 8 + h * 4 + (p % 4); // column of (pair p, half h)
+            for (int h = 0; h < 2; ++h)
 #pragma unroll
-                for (int mt = 0; mt < MT; ++mt)
-#pragma unroll
-                    for (int r = 0; r < 4; ++r) {
-                        const int m = mt * 16 + q * 4 + r;
-                        if (m < M) {
-                            float *slot = &red[((long)wave * M + m) * NW + c * NPL + i];
-                            const float tmp = __builtin_fmaf(-zc[i], rs[mt][r], acc[p][h][mt][r]);
-                            *slot = first_flush ? sc[i] * tmp : __builtin_fmaf(sc[i], tmp, *slot);
-                        }
-                        acc[p][h][mt][r] = 0.f;
-                    }
-            }
+                for (int mt = 0; mt < MT; ++mt) acc[p][h][mt] = v4f {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
         for (int mt = 0; mt < MT; ++mt) rs[mt] = v4f {0.f, 0.f, 0.f, 0.f};
         first_flush = false;
     };
 
-    if (kb < ke) {
-        // Super-steps of SS steps: all weight and src loads of a super-step are
-        // issued before its first MFMA, so one wavefront keeps SS * 4 row loads
-        // in flight (HBM latency is hidden by depth, not by occupancy: the
-        // accumulators leave room for one wavefront per SIMD only).
-        constexpr int SS = 4;
-        step_t sb[SS];
+    // The K range of the wavefront is walked one quantization group at a time;
+    // inside a group, super-steps of SS steps.  Issue order: the group's
+    // parameters (few bytes, needed last: loads return in order, so they must
+    // not queue behind the weights), the activations, then the weight rows PF
+    // steps ahead of the MFMAs that consume them.
+    for (int k = kb; k < ke;) {
+        const int g = k / X.G;
+        const int kend = (g + 1) * X.G < ke ? (g + 1) * X.G : ke;
         qraw_t qr;
-        long g_cur = kb / X.G;
-        fetch_group(qr, g_cur);
-        for (long k = kb; k < ke; k += 16 * SS) {
+        fetch_group(qr, g);
+        for (; k + 16 * SS <= kend; k += 16 * SS) {
+            step_t sb[SS];
 #pragma unroll
-            for (int i = 0; i < SS; ++i)
-                if (k + 16 * i < ke) load_step(sb[i], k + 16 * i);
+            for (int i = 0; i < SS; ++i) load_src(sb[i], k + 16 * i);
+#pragma unroll
+            for (int i = 0; i < PF; ++i) load_wei(sb[i], k + 16 * i);
 #pragma unroll
             for (int i = 0; i < SS; ++i) {
-                const long kk = k + 16 * i;
-                if (kk < ke) {
-                    if (kk / X.G != g_cur) {
-                        flush_group(qr);
-                        g_cur = kk / X.G;
-                        fetch_group(qr, g_cur);
-                    }
-#ifndef MI355_DBG_WOQ_NOCOMPUTE
-                    compute_step(sb[i]);
-#else
-                    acc[0][0][0][0] += __uint_as_float(sb[i].w[0][0] ^ sb[i].w[1][0] ^ sb[i].w[2][1] ^ sb[i].w[3][1] ^ sb[i].a[0].x);
-#endif
-                }
+                if (i + PF < SS) load_wei(sb[i + PF], k + 16 * (i + PF));
+                compute_step(sb[i]);
             }
+        }
+        for (; k < kend; k += 16) { // remainder of the group, one step at a time
+            step_t s1;
+            load_src(s1, k);
+            load_wei(s1, k);
+            compute_step(s1);
         }
         flush_group(qr);
     }
-    if (first_flush) flush_group(qraw_t {}); // empty K range: contribute zeros
-    // ---- reduce the wavefronts' LDS slices: red[wave][m][n_local]
+    if (first_flush) { // empty K range: contribute zeros
+        for (int idx = lane; idx < M * NW; idx += 64) red[wave * M * NW + idx] = 0.f;
+    }
+    // ---- reduce the wavefronts' LDS slices: red[wave][m][permuted column]
     __syncthreads();
-    const long n0 = (long)chunk * NW;
-    float *part = X.partials + (long)split * M * N;
+    const int n0 = chunk * NW;
     const bool direct = X.ksplit == 1;
-    for (int idx = t; idx < M * NW; idx += WOQ_NT) {
-        const int m = idx / NW, nl = idx % NW;
-        if (n0 + nl >= N) continue;
+    auto wave_sum = [&](int m, int nl) __attribute__((always_inline)) {
+        const int slot = (nl % NPL) * 16 + nl / NPL;
         float v = 0.f;
 #pragma unroll
-        for (int w = 0; w < NWV; ++w) v += red[((long)w * M + m) * NW + nl];
-        if (direct) epilogue_store(P, v, 0, m, n0 + nl);
-        else __hip_atomic_store(part + (long)m * N + n0 + nl, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    }
-    if (direct) return;
-#ifdef MI355_DBG_WOQ_NOFINAL
-    return;
-#endif
-
-    // ---- arrival counter: the last workgroup of this chunk finishes the job
-    // The partial sums were written with device-coherent (agent-scope atomic)
-    // stores; waiting for them to complete orders them before the arrival
-    // below without a device-wide cache write-back.
-    __shared__ int is_last;
-    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
-    __builtin_amdgcn_s_waitcnt(0);
-    __syncthreads();
-    if (t == 0) {
-        unsigned *ctr = X.counters + chunk;
-        unsigned old = __hip_atomic_load(ctr, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        unsigned want;
-        do {
-            // a stamp from another launch (or uninitialised memory) counts as zero arrivals
-            const unsigned cnt = (old >> 8) == X.epoch ? (old & 0xffu) : 0u;
-            want = (X.epoch << 8) | (cnt + 1u);
-        } while (!__hip_atomic_compare_exchange_strong(ctr, &old, want, __ATOMIC_RELAXED,
-                __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT));
-        is_last = (int)((want & 0xffu) == (unsigned)X.ksplit);
-    }
-    __syncthreads();
-    if (!is_last) return;
-    for (int idx = t; idx < M * NW; idx += WOQ_NT) {
-        const int m = idx / NW, nl = idx % NW;
-        if (n0 + nl >= N) continue;
-        float v = 0.f;
-        const float *pp = X.partials + (long)m * N + n0 + nl;
-        const long sstride = (long)M * N;
-        int s = 0;
-        for (; s + 8 <= X.ksplit; s += 8) {
-            float tv[8];
-#pragma unroll
-            for (int j = 0; j < 8; ++j)
-                tv[j] = __hip_atomic_load(pp + (s + j) * sstride, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-#pragma unroll
-            for (int j = 0; j < 8; ++j) v += tv[j];
+        for (int w = 0; w < NWV; ++w) v += red[(w * M + m) * NW + slot];
+        return v;
+    };
+    if (!direct) {
+        float *part = X.partials + (long)split * M * N;
+        for (int idx = t; idx < M * NW; idx += WOQ_NT) {
+            const int m = idx / NW, nl = idx % NW;
+            if (n0 + nl < N)
+                __hip_atomic_store(part + (long)m * N + n0 + nl, wave_sum(m, nl), __ATOMIC_RELAXED,
+                        __HIP_MEMORY_SCOPE_AGENT);
         }
-        for (; s < X.ksplit; ++s)
-            v += __hip_atomic_load(pp + s * sstride, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        // ---- arrival counter: the last workgroup of this chunk finishes the job.
+        // The partial sums were written with device-coherent (agent-scope atomic)
+        // stores; waiting for them to complete orders them before the arrival
+        // below without a device-wide cache write-back.
+        __shared__ int is_last;
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+        __builtin_amdgcn_s_waitcnt(0);
+        __syncthreads();
+        if (t == 0) {
+            // wrapping increment: ksplit arrivals take the counter 0 -> ... -> ksplit-1 -> 0
+            const unsigned old = __builtin_amdgcn_atomic_inc32(X.counters + chunk, (unsigned)X.ksplit - 1u,
+                    __ATOMIC_RELAXED, "agent");
+            is_last = (int)(old == (unsigned)X.ksplit - 1u);
+        }
+        __syncthreads();
+        if (!is_last) return;
+    }
+    // ---- sum over the splits in split order and finish with the shared epilogue
+    const auto &P = MI355_KERNARG_PROBLEM();
+    for (int idx = t; idx < M * NW; idx += WOQ_NT) {
+        const int m = idx / NW, nl = idx % NW;
+        if (n0 + nl >= N) continue;
+        float v = 0.f;
+        if (direct) {
+            v = wave_sum(m, nl);
+        } else {
+            const float *pp = X.partials + (long)m * N + n0 + nl;
+            const long sstride = (long)M * N;
+            int s = 0;
+            for (; s + 4 <= X.ksplit; s += 4) {
+                float tv[4];
+#pragma unroll
+                for (int j = 0; j < 4; ++j)
+                    tv[j] = __hip_atomic_load(pp + (s + j) * sstride, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+#pragma unroll
+                for (int j = 0; j < 4; ++j) v += tv[j];
+            }
+            for (; s < X.ksplit; ++s)
+                v += __hip_atomic_load(pp + s * sstride, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
         epilogue_store(P, v, 0, m, n0 + nl);
     }
 }
 
+// Launch geometry.  One workgroup per CU is the target: the grid never exceeds
+// the CU count, so every load of the problem is issued by the first and only
+// wave of workgroups.
 struct woq_plan_t {
-    int chd, mt, nwv, ksplit, krange, chunks;
+    int mt, nwv, ksplit, krange, chunks;
     size_t lds_bytes, total;
 };
 
+constexpr int TARGET_WGS = 256;
+
 woq_plan_t make_plan(const mi355_matmul_desc_t &d) {
     woq_plan_t p {};
-    p.mt = d.M > 16 ? 2 : 1;
-    // Wide-N problems: 16 lanes x 8 columns per workgroup and the whole K range
-    // inside it (16 wavefronts, or 8 for two M tiles) -- no cross-workgroup
-    // reduction at all.  Narrow-N problems: wider chunks, K split over
-    // workgroups, partial sums through scratch.
-    const long chunks1 = (d.N + 127) / 128;
-    // (measured on MI355X: the whole-K form is latency-bound, 38 us against 25 us
-    // for the split form on 4096 x 14336, so it is opt-in for now)
-    const bool whole_k = chunks1 >= 96 && d.K >= 1024 && getenv("MI355_WOQ_WHOLE_K") != nullptr;
-    long krange;
-    if (whole_k) {
-        p.chd = 1;
-        p.nwv = p.mt == 2 ? 8 : 16;
-        p.chunks = (int)chunks1;
-        krange = (d.K + 16 * p.nwv - 1) / (16 * p.nwv) * (16 * p.nwv);
-    } else {
-        p.chd = 2;
-        p.nwv = 4;
-        const int nw = 16 * p.chd * 8;
-        p.chunks = (int)((d.N + nw - 1) / nw);
-        // K range per workgroup: a power-of-two multiple of 64, the smallest that
-        // keeps the grid near two workgroups per CU; larger M gets longer ranges
-        // (each split costs M*N*4 bytes of partial-sum traffic)
-        const long min_range = d.M <= 2 ? 64 : d.M <= 8 ? 256 : 512;
-        krange = 64;
-        const long kmax = (d.K + 63) / 64 * 64;
-        while (krange < kmax && (krange < min_range || p.chunks * ((d.K + krange - 1) / krange) > 512))
-            krange *= 2;
-        if (const char *e = getenv("MI355_WOQ_KRANGE")) krange = atol(e); // tuning aid
-        if (krange > kmax) krange = kmax;
-    }
-    int ksplit = (int)((d.K + krange - 1) / krange);
-    while (ksplit > 255) {
-        krange *= 2;
-        ksplit = (int)((d.K + krange - 1) / krange);
-    }
-    p.ksplit = ksplit;
+    // M <= 16: one 16-row tile, 8 wavefronts; M <= 32: two tiles, 4 wavefronts.
+    // Both keep the LDS reduction buffer [wavefronts][M][256] within 128 KB.
+    p.mt = d.M <= 16 ? 1 : 2;
+    p.nwv = d.M <= 16 ? 8 : 4;
+    p.chunks = (int)((d.N + NW - 1) / NW);
+    // K range per workgroup: a multiple of 16 rows per wavefront
+    const long unit = 16L * p.nwv;
+    long ksplit = TARGET_WGS / p.chunks;
+    if (ksplit < 1) ksplit = 1;
+    long krange = ((d.K + ksplit - 1) / ksplit + unit - 1) / unit * unit;
+    // every split costs M*N*4 bytes of partial sums each way: keep the K range
+    // of a split at least 8 rows per row of activations
+    while (krange < d.K && krange < 8L * d.M * p.nwv) krange += unit;
+    ksplit = (d.K + krange - 1) / krange;
+    p.ksplit = (int)ksplit;
     p.krange = (int)krange;
-    p.lds_bytes = (size_t)p.nwv * d.M * (16 * p.chd * 8) * sizeof(float);
-    p.total = COUNTER_BYTES + (ksplit > 1 ? (size_t)ksplit * d.M * d.N * sizeof(float) : 0);
+    p.lds_bytes = (size_t)p.nwv * d.M * NW * sizeof(float);
+    p.total = ksplit > 1 ? (size_t)ksplit * d.M * d.N * sizeof(float) : 0;
     return p;
 }
 
-std::atomic<unsigned> g_epoch {1};
+std::atomic<unsigned> g_launch_seq {0};
+
+// device address of the arrival counters, per device
+unsigned *arrival_counters(int slot) {
+    static std::mutex mtx;
+    static unsigned *base[64] = {};
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return nullptr;
+    std::lock_guard<std::mutex> lock(mtx);
+    if (!base[dev]) {
+        void *ptr = nullptr;
+        if (hipGetSymbolAddress(&ptr, HIP_SYMBOL(g_arrivals)) != hipSuccess) return nullptr;
+        base[dev] = (unsigned *)ptr;
+    }
+    return base[dev] + (size_t)slot * MAX_CHUNKS;
+}
 
 bool param_layout_ok(const mi355_quant_t &q, long K, bool allow_common, long *G) {
     // per-n with or without groups along K, or a single common value
@@ -433,6 +470,50 @@ bool param_layout_ok(const mi355_quant_t &q, long K, bool allow_common, long *G)
     return true;
 }
 
+int scale_bits(int dt) {
+    return dt == MI355_DT_UNDEF ? 0 : dt == MI355_DT_F32 ? 32 : (dt == MI355_DT_BF16 || dt == MI355_DT_F16) ? 16 : -1;
+}
+
+int zp_bits(int dt) {
+    return dt == MI355_DT_UNDEF ? 0
+            : dt == MI355_DT_S32 ? 32
+            : (dt == MI355_DT_S8 || dt == MI355_DT_U8) ? 8
+            : (dt == MI355_DT_S4 || dt == MI355_DT_U4) ? 4 : -1;
+}
+
+template <int MT, int NWV, int SS>
+int launch_variant(int scb, int zpb, dim3 grid, size_t lds, hipStream_t stream, const problem_t &P,
+        const woq_extra_t &X) {
+    auto go = [&](auto kern) __attribute__((always_inline)) {
+        if (lds > 65536) {
+            if (hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds)
+                    != hipSuccess) {
+                set_error("woq_gemv: cannot reserve %zu bytes of LDS", lds);
+                return MI355_RUNTIME_ERROR;
+            }
+        }
+        hipLaunchKernelGGL(kern, grid, dim3(NWV * 64), lds, stream, P, X);
+        return hipGetLastError() == hipSuccess ? MI355_SUCCESS : MI355_RUNTIME_ERROR;
+    };
+#define MI355_WOQ_CASE(S, Z) \
+    if (scb == S && zpb == Z) return go(woq_gemv_kernel<MT, NWV, SS, S, Z>)
+    MI355_WOQ_CASE(16, 4);
+    MI355_WOQ_CASE(16, 8);
+    MI355_WOQ_CASE(16, 32);
+    MI355_WOQ_CASE(16, 0);
+    MI355_WOQ_CASE(32, 4);
+    MI355_WOQ_CASE(32, 8);
+    MI355_WOQ_CASE(32, 32);
+    MI355_WOQ_CASE(32, 0);
+    MI355_WOQ_CASE(0, 4);
+    MI355_WOQ_CASE(0, 8);
+    MI355_WOQ_CASE(0, 32);
+    MI355_WOQ_CASE(0, 0);
+#undef MI355_WOQ_CASE
+    set_error("woq_gemv: no kernel for %d-bit scales and %d-bit zero points", scb, zpb);
+    return MI355_UNIMPLEMENTED;
+}
+
 } // namespace
 
 int woq_supported(const mi355_matmul_desc_t &d) {
@@ -441,10 +522,12 @@ int woq_supported(const mi355_matmul_desc_t &d) {
     if (dt_bits(d.dst_dt) < 8) return MI355_UNIMPLEMENTED;
     if (d.batch != 1 || d.M < 1 || d.M > 32) return MI355_UNIMPLEMENTED;
     if (d.K % 16 != 0 || d.N % 16 != 0 || d.K < 16) return MI355_UNIMPLEMENTED;
-    if (d.src_stride[2] != 1 || d.src_stride[1] % 4 != 0) return MI355_UNIMPLEMENTED;
-    if (d.wei_stride[2] != 1 || d.wei_stride[1] != d.N) return MI355_UNIMPLEMENTED;
+    // 32-bit byte offsets into src and into a weights row
+    if (d.src_stride[2] != 1 || d.src_stride[1] % 4 != 0 || d.src_stride[1] >= (1L << 25)) return MI355_UNIMPLEMENTED;
+    if (d.wei_stride[2] != 1 || d.wei_stride[1] != d.N || d.N >= (1L << 28)) return MI355_UNIMPLEMENTED;
     if (!quant_absent(d.src_scale) || !quant_absent(d.src_zp) || !quant_absent(d.src_pr))
         return MI355_UNIMPLEMENTED;
+    if (scale_bits(d.wei_scale.dt) < 0 || zp_bits(d.wei_zp.dt) < 0) return MI355_UNIMPLEMENTED;
     long gs, gz;
     if (!param_layout_ok(d.wei_scale, d.K, false, &gs)) return MI355_UNIMPLEMENTED;
     if (!param_layout_ok(d.wei_zp, d.K, true, &gz)) return MI355_UNIMPLEMENTED;
@@ -452,7 +535,7 @@ int woq_supported(const mi355_matmul_desc_t &d) {
     const bool sg = !quant_absent(d.wei_scale) && (d.wei_scale.mask & 2);
     const bool zg = !quant_absent(d.wei_zp) && (d.wei_zp.mask & 2);
     if (sg && zg && gs != gz) return MI355_UNIMPLEMENTED;
-    if ((d.N + 127) / 128 > COUNTER_BYTES / 4) return MI355_UNIMPLEMENTED;
+    if ((d.N + NW - 1) / NW > MAX_CHUNKS) return MI355_UNIMPLEMENTED;
     return MI355_SUCCESS;
 }
 
@@ -462,39 +545,39 @@ size_t woq_scratch_bytes(const mi355_matmul_desc_t &d) {
 
 int woq_launch(const mi355_matmul_desc_t &d, const problem_t &P, void *scratch, hipStream_t stream) {
     const woq_plan_t plan = make_plan(d);
-    if (!scratch) {
+    if (plan.total && !scratch) {
         set_error("woq_gemv: %zu bytes of scratch required", plan.total);
         return MI355_INVALID_ARGUMENTS;
     }
     woq_extra_t X {};
-    X.counters = (unsigned *)scratch;
-    X.partials = (float *)((char *)scratch + COUNTER_BYTES);
-    X.epoch = (g_epoch.fetch_add(1) % 0xFFFFFEu) + 1u;
+    X.counters = arrival_counters((int)(g_launch_seq.fetch_add(1) % COUNTER_SLOTS));
+    if (!X.counters) {
+        set_error("woq_gemv: cannot resolve the arrival counters on this device");
+        return MI355_RUNTIME_ERROR;
+    }
+    X.wei = (const uint8_t *)P.wei;
+    X.src = (const uint8_t *)P.src;
+    X.partials = (float *)scratch;
+    X.M = (int)d.M; X.N = (int)d.N; X.K = (int)d.K;
+    X.src_ld = (int)d.src_stride[1];
+    X.row_bytes = (int)(d.N / 2);
     X.ksplit = plan.ksplit;
     X.krange = plan.krange;
     const bool sg = !quant_absent(d.wei_scale) && (d.wei_scale.mask & 2);
     const bool zg = !quant_absent(d.wei_zp) && (d.wei_zp.mask & 2);
     X.G = (int)(sg ? d.wei_scale.group[0] : zg ? d.wei_zp.group[0] : d.K);
+    X.sc_dt = d.wei_scale.dt;
+    X.zp_dt = d.wei_zp.dt;
+    X.sc = X.sc_dt ? (const uint8_t *)P.wei_scale.p : nullptr;
+    X.zp = X.zp_dt ? (const uint8_t *)P.wei_zp.p : nullptr;
     X.sc_grouped = sg;
     X.zp_grouped = zg;
-    X.zp_common = !quant_absent(d.wei_zp) && d.wei_zp.mask == 0;
+    X.zp_common = X.zp_dt && d.wei_zp.mask == 0;
     X.signed_w = d.wei_dt == MI355_DT_S4;
-    dim3 grid((unsigned)plan.chunks, (unsigned)plan.ksplit, 1);
-    auto go = [&](auto kern) __attribute__((always_inline)) {
-        if (plan.lds_bytes > 65536) {
-            if (hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize,
-                        (int)plan.lds_bytes) != hipSuccess) {
-                set_error("woq_gemv: cannot reserve %zu bytes of LDS", plan.lds_bytes);
-                return MI355_RUNTIME_ERROR;
-            }
-        }
-        hipLaunchKernelGGL(kern, grid, dim3(plan.nwv * 64), plan.lds_bytes, stream, P, X);
-        return hipGetLastError() == hipSuccess ? MI355_SUCCESS : MI355_RUNTIME_ERROR;
-    };
-    if (plan.nwv == 16) return go(woq_gemv_kernel<1, 1, 16>);
-    if (plan.nwv == 8) return go(woq_gemv_kernel<1, 2, 8>);
-    if (plan.mt == 2) return go(woq_gemv_kernel<2, 2, 4>);
-    return go(woq_gemv_kernel<2, 1, 4>);
+    const dim3 grid((unsigned)plan.chunks, (unsigned)plan.ksplit, 1);
+    const int scb = scale_bits(X.sc_dt), zpb = zp_bits(X.zp_dt);
+    if (plan.mt == 1) return launch_variant<1, 8, 8>(scb, zpb, grid, plan.lds_bytes, stream, P, X);
+    return launch_variant<2, 4, 8>(scb, zpb, grid, plan.lds_bytes, stream, P, X);
 }
 
 } // namespace mi355

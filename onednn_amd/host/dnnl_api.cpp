@@ -1002,8 +1002,23 @@ DNNL_EXPORT dnnl_status_t dnnl_matmul_primitive_desc_create(dnnl_primitive_desc_
     pd->src = *src_desc; pd->wei = *weights_desc; pd->dst = *dst_desc;
     pd->with_bias = bias != nullptr;
     if (bias) pd->bias = *bias;
-    // format `any` -> plain row-major (matmul_pd_t::set_default_formats, matmul_pd.hpp:419-431)
-    for (dnnl_memory_desc *m : {&pd->src, &pd->wei, &pd->dst, &pd->bias})
+    // format `any`: the implementation picks the layout and the caller asks
+    // weights_desc() for it, as with the reference's blocked weights
+    // (brgemm_matmul_utils.cpp: set_or_check_B_tag).  The MFMA GEMM families
+    // consume K-contiguous weight columns, so int8 / fp8 / fp4 weights resolve
+    // to the plain transposed tag (ba, acb, ...); everything else resolves to
+    // row-major (matmul_pd_t::set_default_formats, matmul_pd.hpp:419-431).
+    if (pd->wei.kind == dnnl_format_kind_any) {
+        dnnl_memory_desc &w = pd->wei;
+        w.set_dense();
+        const bool mfma_operands = (is_int8(pd->src.dt) && is_int8(w.dt)) || (is_fp8(pd->src.dt) && is_fp8(w.dt))
+                || (pd->src.dt == dnnl_f4_e2m1 && w.dt == dnnl_f4_e2m1);
+        if (mfma_operands && w.ndims >= 2) {
+            w.strides[w.ndims - 2] = 1;
+            w.strides[w.ndims - 1] = w.dims[w.ndims - 2] == 0 ? 1 : w.dims[w.ndims - 2];
+        }
+    }
+    for (dnnl_memory_desc *m : {&pd->src, &pd->dst, &pd->bias})
         if (m->kind == dnnl_format_kind_any) m->set_dense();
     // data type combinations of the reference's two naive implementations
     // (ref_matmul.hpp:44-123, ref_matmul_int8.hpp:44-92)

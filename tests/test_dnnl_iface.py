@@ -192,12 +192,21 @@ def test_implementation_list_and_next_impl(eng):
     assert make_pd(eng, 8, 4096, 14336, "bf16", "u4", "bf16", attr=wo).impl_info_str().startswith("hip:woq_gemv")
 
 
-def test_format_any_becomes_plain(eng):
+def test_format_any_is_resolved_by_the_implementation(eng):
+    # src / dst: plain row-major (matmul_pd.hpp:419-431); weights: the layout the
+    # kernels consume, to be read back through weights_desc() like a blocked
+    # layout of the reference -- K-contiguous for the MFMA operand types ...
     pd = dnnl.matmul_primitive_desc(eng, md([8, 16], "s8", tag=dnnl.tag_any), md([16, 4], "s8", tag=dnnl.tag_any),
                                     md([8, 4], "s32", tag=dnnl.tag_any))
     assert pd.query_md(dnnl.query_src_md).strides() == [16, 1]
-    assert pd.query_md(dnnl.query_weights_md).strides() == [4, 1]
+    assert pd.query_md(dnnl.query_weights_md).strides() == [1, 16]
     assert pd.query_md(dnnl.query_dst_md).strides() == [4, 1]
+    pd = dnnl.matmul_primitive_desc(eng, md([2, 8, 128], "f8_e4m3"), md([2, 128, 4], "f8_e4m3", tag=dnnl.tag_any),
+                                    md([2, 8, 4], "bf16"))
+    assert pd.query_md(dnnl.query_weights_md).strides() == [512, 1, 128]
+    # ... and row-major for everything else
+    pd = dnnl.matmul_primitive_desc(eng, md([8, 16], "f32"), md([16, 4], "f32", tag=dnnl.tag_any), md([8, 4], "f32"))
+    assert pd.query_md(dnnl.query_weights_md).strides() == [4, 1]
 
 
 def test_user_scratchpad_is_reported(eng):

@@ -126,3 +126,50 @@ def test_woq_one_hot_rows_are_exact(gpu, oracle):
     got, name = run_gpu(p, cabi.IMPL_WOQ_GEMV)
     want = oracle.run_oracle(p)
     assert_bit_exact(p, got, want, name)
+
+
+WOQ_VARIANTS = [
+    # M, N, K, group, weights, scales dt/kind, zero points dt/kind, dst, bias+relu
+    (1, 512, 1024, 128, "u4", "f32", "grouped", "s8", "grouped", "bf16", False),
+    (5, 272, 1040, 80, "u4", "f16", "column", "u8", "column", "f32", True),     # ragged N and K, per-column parameters
+    (16, 512, 512, 64, "s4", "bf16", "grouped", "s4", "grouped", "bf16", False),
+    (17, 256, 2048, 128, "s4", "bf16", "grouped", "s32", "common", "f32", False),
+    (32, 1024, 512, 32, "u4", "f32", "grouped", "u4", "none", "bf16", True),
+    (3, 4096, 256, 256, "u4", "bf16", "none", "u8", "grouped", "f32", False),    # no K split (wide N), no scales
+    (8, 768, 4096, 128, "u4", "bf16", "grouped", "s32", "grouped", "bf16", False),
+]
+
+
+@pytest.mark.parametrize("case", WOQ_VARIANTS, ids=lambda c: "-".join(str(x) for x in c))
+def test_woq_attribute_variants(gpu, oracle, case):
+    M, N, K, group, wdt, sdt, skind, zdt, zkind, ddt, relu_bias = case
+    p = configs.woq_variant(M, N, K, group, wei_dt=wdt, sc_dt=sdt, sc_kind=skind, zp_dt=zdt, zp_kind=zkind,
+                            dst_dt=ddt, relu_bias=relu_bias)
+    got, name = run_gpu(p, cabi.IMPL_WOQ_GEMV)
+    assert name.startswith("hip:woq_gemv")
+    want, _, asum = oracle.run_oracle(p, want_ideal=True)
+    assert_close(p, got, want, abs_sum=asum * 20.0, what=name)
+    # and the generic kernel follows the reference's operation order exactly
+    got_ref, name_ref = run_gpu(p, cabi.IMPL_REF)
+    assert_bit_exact(p, got_ref, want, name_ref)
+
+
+def test_woq_back_to_back_launches_share_nothing(gpu, oracle):
+    # the arrival counters return to zero after every launch: a second launch on
+    # the same scratch, and a different problem right after, see a clean state
+    from onednn_amd.problem import GpuRun
+    a = configs.config2(M=4, N=512, K=2048)
+    b = configs.config2(M=1, N=768, K=1024, seed=9)
+    ra, rb = GpuRun(a, cabi.IMPL_WOQ_GEMV), GpuRun(b, cabi.IMPL_WOQ_GEMV)
+    outs = []
+    for r in (ra, ra, rb, ra, rb):
+        r.reset_dst()
+        r.launch()
+        r.sync()
+        outs.append(r.result())
+    assert np.array_equal(outs[0], outs[1]) and np.array_equal(outs[0], outs[3])
+    assert np.array_equal(outs[2], outs[4])
+    want, _, asum = oracle.run_oracle(b, want_ideal=True)
+    assert_close(b, outs[4], want, abs_sum=asum * 20.0, what="second problem")
+    ra.free()
+    rb.free()
