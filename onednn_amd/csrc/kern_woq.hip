@@ -36,13 +36,12 @@
 // row segments shorter than a 128-byte line are fetched whole: chunks are 256
 // columns wide).  A wavefront keeps the weight loads of four 16-row steps in
 // flight ahead of the MFMAs, and the wavefronts of a workgroup reduce through
-// LDS into one f32 partial [M][chunk] in scratch.  The last workgroup
-// to arrive for a chunk (one wrapping atomic increment on a counter that is
-// zero between launches) adds the partials in split order -- deterministic --
-// and runs the shared epilogue.
-#include <atomic>
-#include <mutex>
-
+// LDS into one f32 partial [row quad][chunk] in scratch.  A second small
+// kernel adds the partials of all splits in split order -- deterministic -- and
+// runs the shared epilogue; measured on MI355X it costs no more than a
+// last-workgroup-finishes scheme with arrival counters for one row of
+// activations and half as much for 32 rows, and it keeps no state between
+// launches.
 #include "kernels.hpp"
 
 namespace mi355 {
@@ -53,18 +52,8 @@ typedef float v4f __attribute__((ext_vector_type(4)));
 typedef unsigned v2u __attribute__((ext_vector_type(2)));
 typedef __bf16 v8bf __attribute__((ext_vector_type(8)));
 
-constexpr int NPL = 16;      // columns per lane (two dwords of nibbles)
-constexpr int NW = 16 * NPL; // columns per wavefront / workgroup: 128-byte row segments
-constexpr int NP = 8;        // bf16 pairs per lane per row
-
-// Arrival counters live in library-owned device memory: zero when the module
-// is loaded, and every launch leaves the counters it used at zero again (the
-// increment wraps at the number of splits).  A launch takes the next of
-// COUNTER_SLOTS blocks, so launches that overlap on different streams do not
-// share counters unless more than COUNTER_SLOTS are in flight.
-constexpr int COUNTER_SLOTS = 32;
-constexpr int MAX_CHUNKS = 1024;
-__device__ unsigned g_arrivals[COUNTER_SLOTS][MAX_CHUNKS];
+// CHD = dwords of nibbles per lane and row: 2 (16 columns per lane, 256 per
+// workgroup) or 4 (32 columns per lane, 512 per workgroup)
 
 // Everything the main loop needs, gathered in one argument so that the kernel
 // starts with a single block of scalar loads: the first weight load must not
@@ -73,8 +62,7 @@ struct woq_extra_t {
     const uint8_t *wei;  // [K][N/2]
     const uint8_t *src;  // bf16 [M][src_ld]
     const uint8_t *sc, *zp; // weights scales / zero points (NULL when absent)
-    float *partials;     // [ksplit][M][N]
-    unsigned *counters;  // [chunks] arrival counters, zero between launches
+    float *partials;     // [ksplit][chunks][unit][4]: row quads in the order of the LDS reduction
     int M, N, K, src_ld;
     int row_bytes;       // N / 2
     int krange;          // k per workgroup (multiple of 16 * wavefronts)
@@ -89,20 +77,20 @@ struct woq_extra_t {
 __device__ __forceinline__ v8bf as_bf(const v4i &x) { return __builtin_bit_cast(v8bf, x); }
 
 // NPL consecutive parameter values of BITS bits each, as raw dwords
-template <int BITS>
+template <int NPL, int BITS>
 struct raw_t {
     static constexpr int DW = BITS ? NPL * BITS / 32 : 1;
     unsigned w[DW];
 };
 
-template <int BITS>
-__device__ __forceinline__ void load_raw(raw_t<BITS> &r, const uint8_t *p) {
-    if constexpr (BITS == 4) {
+template <int NPL, int BITS>
+__device__ __forceinline__ void load_raw(raw_t<NPL, BITS> &r, const uint8_t *p) {
+    if constexpr (raw_t<NPL, BITS>::DW == 2) {
         const uint2 v = *(const uint2 *)p;
         r.w[0] = v.x; r.w[1] = v.y;
     } else if constexpr (BITS != 0) {
 #pragma unroll
-        for (int i = 0; i < raw_t<BITS>::DW / 4; ++i) {
+        for (int i = 0; i < raw_t<NPL, BITS>::DW / 4; ++i) {
             const uint4 v = *(const uint4 *)(p + 16 * i);
             r.w[4 * i] = v.x; r.w[4 * i + 1] = v.y; r.w[4 * i + 2] = v.z; r.w[4 * i + 3] = v.w;
         }
@@ -110,8 +98,8 @@ __device__ __forceinline__ void load_raw(raw_t<BITS> &r, const uint8_t *p) {
 }
 
 // scales: f32 (32 bits) or bf16 / f16 (16 bits)
-template <int BITS>
-__device__ __forceinline__ void decode_scales(int dt, const raw_t<BITS> &r, float (&out)[NPL]) {
+template <int NPL, int BITS>
+__device__ __forceinline__ void decode_scales(int dt, const raw_t<NPL, BITS> &r, float (&out)[NPL]) {
     if constexpr (BITS == 32) {
 #pragma unroll
         for (int i = 0; i < NPL; ++i) out[i] = u2f(r.w[i]);
@@ -130,8 +118,8 @@ __device__ __forceinline__ void decode_scales(int dt, const raw_t<BITS> &r, floa
 }
 
 // zero points: s32 (32 bits), s8 / u8 (8 bits), s4 / u4 (4 bits)
-template <int BITS>
-__device__ __forceinline__ void decode_zps(int dt, const raw_t<BITS> &r, float (&out)[NPL]) {
+template <int NPL, int BITS>
+__device__ __forceinline__ void decode_zps(int dt, const raw_t<NPL, BITS> &r, float (&out)[NPL]) {
     if constexpr (BITS == 32) {
 #pragma unroll
         for (int i = 0; i < NPL; ++i) out[i] = (float)(int)r.w[i];
@@ -155,12 +143,16 @@ __device__ __forceinline__ void decode_zps(int dt, const raw_t<BITS> &r, float (
     }
 }
 
-// MT 16-row tiles of activations; NWV wavefronts per workgroup share one column
-// chunk and split its K range; SS = 16-row steps of one super-step; SCB / ZPB =
-// bits per scale / zero point (0 = absent).
-template <int MT, int NWV, int SS, int SCB, int ZPB>
+// CHD dwords per lane and row; MT 16-row tiles of activations; NWV wavefronts
+// per workgroup share one column chunk and split its K range; SS = 16-row steps
+// of one super-step; SCB / ZPB = bits per scale / zero point (0 = absent).
+template <int CHD, int MT, int NWV, int SS, int SCB, int ZPB>
 __global__ void __launch_bounds__(NWV * 64) woq_gemv_kernel(const problem_t P_, const woq_extra_t X) {
-    extern __shared__ __attribute__((aligned(16))) float red[]; // [NWV][M][NW], columns permuted
+    extern __shared__ __attribute__((aligned(16))) float red[]; // [NWV][row quads][NW] x 4 floats
+    constexpr int NPL = CHD * 8; // columns per lane
+    constexpr int NW = 16 * NPL; // columns per wavefront / workgroup: 128- or 256-byte row segments
+    constexpr int NP = CHD * 4;  // bf16 pairs per lane per row
+    typedef unsigned vwu __attribute__((ext_vector_type(CHD)));
     constexpr int PF = SS < 4 ? SS : 4; // weight steps in flight ahead of the MFMAs
     constexpr int WOQ_NT = NWV * 64;
     const int t = threadIdx.x, lane = t & 63;
@@ -191,7 +183,7 @@ __global__ void __launch_bounds__(NWV * 64) woq_gemv_kernel(const problem_t P_, 
     for (int mt = 0; mt < MT; ++mt) rs[mt] = v4f {0.f, 0.f, 0.f, 0.f};
 
     struct step_t {
-        v2u w[4];    // rows 4q+t, the two dwords of this lane's columns
+        vwu w[4];    // rows 4q+t, the dwords of this lane's columns
         uint2 a[MT]; // src[m][k0+4q .. +3] as four bf16
     };
     const unsigned wei_lane_off = (unsigned)(4 * q * X.row_bytes + n_ld / 2);
@@ -210,7 +202,7 @@ __global__ void __launch_bounds__(NWV * 64) woq_gemv_kernel(const problem_t P_, 
     auto load_wei = [&](step_t &s, int k0) __attribute__((always_inline)) {
 #pragma unroll
         for (int tt = 0; tt < 4; ++tt)
-            s.w[tt] = __builtin_nontemporal_load((const v2u *)(X.wei + (long)(k0 + tt) * X.row_bytes + wei_lane_off));
+            s.w[tt] = __builtin_nontemporal_load((const vwu *)(X.wei + (long)(k0 + tt) * X.row_bytes + wei_lane_off));
     };
 
     // 0x4300 | nibble = bf16(128 + nibble).  The constant is kept in a vector
@@ -222,7 +214,7 @@ __global__ void __launch_bounds__(NWV * 64) woq_gemv_kernel(const problem_t P_, 
     auto compute_step = [&](step_t &s) __attribute__((always_inline)) {
         if (X.signed_w) { // s4 -> offset-binary
 #pragma unroll
-            for (int tt = 0; tt < 4; ++tt) s.w[tt] ^= v2u {0x88888888u, 0x88888888u};
+            for (int tt = 0; tt < 4; ++tt) s.w[tt] ^= (vwu)(0x88888888u);
         }
         v4i aa[MT], ab[MT];
 #pragma unroll
@@ -233,7 +225,7 @@ __global__ void __launch_bounds__(NWV * 64) woq_gemv_kernel(const problem_t P_, 
             rs[mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf(aa[mt]), as_bf(ones), rs[mt], 0, 0, 0);
         }
 #pragma unroll
-        for (int d = 0; d < 2; ++d) {
+        for (int d = 0; d < CHD; ++d) {
 #pragma unroll
             for (int sh = 0; sh < 4; ++sh) {
                 v4i b;
@@ -252,29 +244,37 @@ __global__ void __launch_bounds__(NWV * 64) woq_gemv_kernel(const problem_t P_, 
     // Quantization parameters of one group for this lane's columns: raw loads
     // when the group starts, decoded when it ends.
     struct qraw_t {
-        raw_t<SCB> s;
-        raw_t<ZPB> z;
+        raw_t<NPL, SCB> s;
+        raw_t<NPL, ZPB> z;
     };
     auto fetch_group = [&](qraw_t &qr, int g) __attribute__((always_inline)) {
         if constexpr (SCB != 0)
-            load_raw<SCB>(qr.s, X.sc + ((long)(X.sc_grouped ? g : 0) * N * SCB / 8 + (unsigned)(n_ld * SCB / 8)));
+            load_raw<NPL, SCB>(qr.s, X.sc + ((long)(X.sc_grouped ? g : 0) * N * SCB / 8 + (unsigned)(n_ld * SCB / 8)));
         if constexpr (ZPB != 0) {
             if (X.zp_common) // element 0 for every column
                 qr.z.w[0] = ZPB == 32 ? *(const unsigned *)X.zp : (unsigned)*X.zp;
             else
-                load_raw<ZPB>(qr.z, X.zp + ((long)(X.zp_grouped ? g : 0) * N * ZPB / 8 + (unsigned)(n_ld * ZPB / 8)));
+                load_raw<NPL, ZPB>(qr.z, X.zp + ((long)(X.zp_grouped ? g : 0) * N * ZPB / 8 + (unsigned)(n_ld * ZPB / 8)));
         }
     };
 
-    // fold one finished group into this wavefront's LDS slice:
-    //   red[wave][m][n] (+)= scale * (acc - (128 + zp) * rowsum)
-    // column i of lane c is kept at i * 16 + c: the 16 lanes of a row write
-    // consecutive words
+    // Rows are handled in quads (the four rows a lane holds of one MFMA tile):
+    // MQ quads in all, MQ0 of them in the first 16-row tile.
+    const int MQ = (M + 3) / 4, MQ0 = MQ < 4 ? MQ : 4;
+    // fold one finished group into this wavefront's LDS slice, one 16-byte
+    // write per column and row quad:
+    //   red[wave][tile][slot][quad] (+)= scale * (acc - (128 + zp) * rowsum)
+    // column i of lane c sits at slot i * 16 + c, so the lanes of a write
+    // cover consecutive 16-byte words (no bank conflicts)
+    v4f *red4 = (v4f *)red;
+    int rows_used[MT]; // rows of a quad that can hold data in tile mt (4 unless M is below 4 there)
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) rows_used[mt] = M - 16 * mt < 4 ? M - 16 * mt : 4;
     bool first_flush = true;
     auto flush_group = [&](const qraw_t &qr) __attribute__((always_inline)) {
         float sc[NPL], zc[NPL];
-        decode_scales<SCB>(X.sc_dt, qr.s, sc);
-        decode_zps<ZPB>(X.zp_dt, qr.z, zc);
+        decode_scales<NPL, SCB>(X.sc_dt, qr.s, sc);
+        decode_zps<NPL, ZPB>(X.zp_dt, qr.z, zc);
         if (ZPB != 0 && X.zp_common) {
 #pragma unroll
             for (int i = 1; i < NPL; ++i) zc[i] = zc[0];
@@ -283,22 +283,28 @@ __global__ void __launch_bounds__(NWV * 64) woq_gemv_kernel(const problem_t P_, 
 #pragma unroll
         for (int i = 0; i < NPL; ++i) zc[i] += zbase;
 #pragma unroll
-        for (int mt = 0; mt < MT; ++mt)
+        for (int mt = 0; mt < MT; ++mt) {
+            const int mqt = mt ? MQ - MQ0 : MQ0; // quads of this tile
+            if (q < mqt) {
+                v4f *col = red4 + (wave * MQ + (mt ? MQ0 : 0)) * NW + c * mqt + q;
 #pragma unroll
-            for (int r = 0; r < 4; ++r) {
-                const int m = mt * 16 + q * 4 + r;
-                if (m < M) {
-                    float *row = &red[(wave * M + m) * NW + c];
+                for (int p = 0; p < NP; ++p)
 #pragma unroll
-                    for (int p = 0; p < NP; ++p)
+                    for (int h = 0; h < 2; ++h) {
+                        const int i = (p / 4) * 8 + h * 4 + (p % 4); // column of (pair p, half h)
+                        v4f val = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-                        for (int h = 0; h < 2; ++h) {
-                            const int i = (p / 4) * 8 + h * 4 + (p % 4); // column of (pair p, half h)
-                            const float tmp = __builtin_fmaf(-zc[i], rs[mt][r], acc[p][h][mt][r]);
-                            row[i * 16] = first_flush ? sc[i] * tmp : __builtin_fmaf(sc[i], tmp, row[i * 16]);
-                        }
-                }
+                        for (int r = 0; r < 4; ++r)
+                            if (r < rows_used[mt]) // uniform: skips the padding rows of small M
+                                val[r] = sc[i] * __builtin_fmaf(-zc[i], rs[mt][r], acc[p][h][mt][r]);
+                        v4f *slot = col + i * 16 * mqt;
+                        *slot = first_flush ? val : *slot + val;
+                    }
             }
+        }
+        first_flush = false;
+    };
+    auto clear_acc = [&]() __attribute__((always_inline)) {
 #pragma unroll
         for (int p = 0; p < NP; ++p)
 #pragma unroll
@@ -307,7 +313,6 @@ __global__ void __launch_bounds__(NWV * 64) woq_gemv_kernel(const problem_t P_, 
                 for (int mt = 0; mt < MT; ++mt) acc[p][h][mt] = v4f {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
         for (int mt = 0; mt < MT; ++mt) rs[mt] = v4f {0.f, 0.f, 0.f, 0.f};
-        first_flush = false;
     };
 
     // The K range of the wavefront is walked one quantization group at a time;
@@ -339,70 +344,88 @@ __global__ void __launch_bounds__(NWV * 64) woq_gemv_kernel(const problem_t P_, 
             compute_step(s1);
         }
         flush_group(qr);
+        if (k < ke) clear_acc();
     }
     if (first_flush) { // empty K range: contribute zeros
-        for (int idx = lane; idx < M * NW; idx += 64) red[wave * M * NW + idx] = 0.f;
+        for (int u = lane; u < MQ * NW; u += 64) red4[wave * MQ * NW + u] = v4f {0.f, 0.f, 0.f, 0.f};
     }
-    // ---- reduce the wavefronts' LDS slices: red[wave][m][permuted column]
+    // ---- reduce the wavefronts' LDS slices.  A unit is one 16-byte word: four
+    // rows of one column, in the order the flush wrote them; the partial sums
+    // in scratch keep that order, [split][chunk][unit].
     __syncthreads();
     const int n0 = chunk * NW;
-    const bool direct = X.ksplit == 1;
-    auto wave_sum = [&](int m, int nl) __attribute__((always_inline)) {
-        const int slot = (nl % NPL) * 16 + nl / NPL;
-        float v = 0.f;
+    const int units = MQ * NW;
+    auto wave_sum = [&](int u) __attribute__((always_inline)) {
+        v4f v = red4[u];
 #pragma unroll
-        for (int w = 0; w < NWV; ++w) v += red[(w * M + m) * NW + slot];
+        for (int w = 1; w < NWV; ++w) v += red4[w * units + u];
         return v;
     };
-    if (!direct) {
-        float *part = X.partials + (long)split * M * N;
-        for (int idx = t; idx < M * NW; idx += WOQ_NT) {
-            const int m = idx / NW, nl = idx % NW;
-            if (n0 + nl < N)
-                __hip_atomic_store(part + (long)m * N + n0 + nl, wave_sum(m, nl), __ATOMIC_RELAXED,
-                        __HIP_MEMORY_SCOPE_AGENT);
-        }
-        // ---- arrival counter: the last workgroup of this chunk finishes the job.
-        // The partial sums were written with device-coherent (agent-scope atomic)
-        // stores; waiting for them to complete orders them before the arrival
-        // below without a device-wide cache write-back.
-        __shared__ int is_last;
-        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
-        __builtin_amdgcn_s_waitcnt(0);
-        __syncthreads();
-        if (t == 0) {
-            // wrapping increment: ksplit arrivals take the counter 0 -> ... -> ksplit-1 -> 0
-            const unsigned old = __builtin_amdgcn_atomic_inc32(X.counters + chunk, (unsigned)X.ksplit - 1u,
-                    __ATOMIC_RELAXED, "agent");
-            is_last = (int)(old == (unsigned)X.ksplit - 1u);
-        }
-        __syncthreads();
-        if (!is_last) return;
-    }
-    // ---- sum over the splits in split order and finish with the shared epilogue
     const auto &P = MI355_KERNARG_PROBLEM();
-    for (int idx = t; idx < M * NW; idx += WOQ_NT) {
-        const int m = idx / NW, nl = idx % NW;
-        if (n0 + nl >= N) continue;
-        float v = 0.f;
-        if (direct) {
-            v = wave_sum(m, nl);
-        } else {
-            const float *pp = X.partials + (long)m * N + n0 + nl;
-            const long sstride = (long)M * N;
-            int s = 0;
-            for (; s + 4 <= X.ksplit; s += 4) {
-                float tv[4];
-#pragma unroll
-                for (int j = 0; j < 4; ++j)
-                    tv[j] = __hip_atomic_load(pp + (s + j) * sstride, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-#pragma unroll
-                for (int j = 0; j < 4; ++j) v += tv[j];
-            }
-            for (; s < X.ksplit; ++s)
-                v += __hip_atomic_load(pp + s * sstride, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    if (X.ksplit > 1) { // plain stores: the kernel boundary publishes them to the second pass
+        v4f *part = (v4f *)X.partials + ((long)split * gridDim.x + chunk) * units;
+        for (int u = t; u < units; u += WOQ_NT) part[u] = wave_sum(u);
+        return;
+    }
+    // a single split: finish here
+    for (int u0 = t; u0 < units; u0 += WOQ_NT) {
+        const v4f v = wave_sum(u0);
+        // unit -> (tile, slot, quad) -> column and rows
+        int u = u0, mt = 0, mqt = MQ0;
+        if (u >= MQ0 * NW) {
+            u -= MQ0 * NW;
+            mt = 1;
+            mqt = MQ - MQ0;
         }
-        epilogue_store(P, v, 0, m, n0 + nl);
+        const int slot = u / mqt, mq = u % mqt;
+        const int n = n0 + (slot % 16) * NPL + slot / 16;
+        if (n >= N) continue;
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+            const int m = mt * 16 + mq * 4 + r;
+            if (m < M) epilogue_store(P, v[r], 0, m, n);
+        }
+    }
+}
+
+// Second pass: the partial sums of all splits are added in split order, one
+// thread per row quad and column over the whole device.
+template <int CHD>
+__global__ void __launch_bounds__(256) woq_reduce_kernel(const problem_t P_, const woq_extra_t X, int chunks) {
+    const auto &P = MI355_KERNARG_PROBLEM();
+    constexpr int NPL = CHD * 8, NW = 16 * NPL;
+    const int M = X.M, N = X.N;
+    const int MQ = (M + 3) / 4, MQ0 = MQ < 4 ? MQ : 4;
+    const int units = MQ * NW;
+    const long g = (long)blockIdx.x * 256 + threadIdx.x;
+    if (g >= (long)chunks * units) return;
+    const int chunk = (int)(g / units);
+    int u = (int)(g % units);
+    const v4f *pp = (const v4f *)X.partials + g;
+    const long sstride = (long)chunks * units;
+    v4f v = {0.f, 0.f, 0.f, 0.f};
+    int s = 0;
+    for (; s + 4 <= X.ksplit; s += 4) {
+        v4f tv[4];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) tv[j] = pp[(s + j) * sstride];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) v += tv[j];
+    }
+    for (; s < X.ksplit; ++s) v += pp[s * sstride];
+    int mt = 0, mqt = MQ0;
+    if (u >= MQ0 * NW) {
+        u -= MQ0 * NW;
+        mt = 1;
+        mqt = MQ - MQ0;
+    }
+    const int slot = u / mqt, mq = u % mqt;
+    const int n = chunk * NW + (slot % 16) * NPL + slot / 16;
+    if (n >= N) return;
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+        const int m = mt * 16 + mq * 4 + r;
+        if (m < M) epilogue_store(P, v[r], 0, m, n);
     }
 }
 
@@ -410,7 +433,7 @@ __global__ void __launch_bounds__(NWV * 64) woq_gemv_kernel(const problem_t P_, 
 // the CU count, so every load of the problem is issued by the first and only
 // wave of workgroups.
 struct woq_plan_t {
-    int mt, nwv, ksplit, krange, chunks;
+    int chd, mt, nwv, ksplit, krange, chunks;
     size_t lds_bytes, total;
 };
 
@@ -420,8 +443,14 @@ woq_plan_t make_plan(const mi355_matmul_desc_t &d) {
     woq_plan_t p {};
     // M <= 16: one 16-row tile, 8 wavefronts; M <= 32: two tiles, 4 wavefronts.
     // Both keep the LDS reduction buffer [wavefronts][M][256] within 128 KB.
+    // (Measured on MI355X for M = 1 at 4096 x 14336, against 12-13 us for this
+    // shape: 512-column chunks with 16-byte loads and one wavefront per SIMD
+    // 16 us, 4 wavefronts x 16 steps 22 us, 16 wavefronts x 4 steps 19 us -- two
+    // wavefronts per SIMD overlap one's nibble unpacking with the other's MFMAs.)
+    p.chd = 2;
     p.mt = d.M <= 16 ? 1 : 2;
     p.nwv = d.M <= 16 ? 8 : 4;
+    const int NW = 16 * 8 * p.chd;
     p.chunks = (int)((d.N + NW - 1) / NW);
     // K range per workgroup: a multiple of 16 rows per wavefront
     const long unit = 16L * p.nwv;
@@ -434,26 +463,10 @@ woq_plan_t make_plan(const mi355_matmul_desc_t &d) {
     ksplit = (d.K + krange - 1) / krange;
     p.ksplit = (int)ksplit;
     p.krange = (int)krange;
-    p.lds_bytes = (size_t)p.nwv * d.M * NW * sizeof(float);
-    p.total = ksplit > 1 ? (size_t)ksplit * d.M * d.N * sizeof(float) : 0;
+    const size_t m4 = (size_t)(d.M + 3) / 4 * 4; // rows in quads
+    p.lds_bytes = (size_t)p.nwv * m4 * NW * sizeof(float);
+    p.total = ksplit > 1 ? (size_t)ksplit * p.chunks * NW * m4 * sizeof(float) : 0;
     return p;
-}
-
-std::atomic<unsigned> g_launch_seq {0};
-
-// device address of the arrival counters, per device
-unsigned *arrival_counters(int slot) {
-    static std::mutex mtx;
-    static unsigned *base[64] = {};
-    int dev = 0;
-    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return nullptr;
-    std::lock_guard<std::mutex> lock(mtx);
-    if (!base[dev]) {
-        void *ptr = nullptr;
-        if (hipGetSymbolAddress(&ptr, HIP_SYMBOL(g_arrivals)) != hipSuccess) return nullptr;
-        base[dev] = (unsigned *)ptr;
-    }
-    return base[dev] + (size_t)slot * MAX_CHUNKS;
 }
 
 bool param_layout_ok(const mi355_quant_t &q, long K, bool allow_common, long *G) {
@@ -481,7 +494,7 @@ int zp_bits(int dt) {
             : (dt == MI355_DT_S4 || dt == MI355_DT_U4) ? 4 : -1;
 }
 
-template <int MT, int NWV, int SS>
+template <int CHD, int MT, int NWV, int SS>
 int launch_variant(int scb, int zpb, dim3 grid, size_t lds, hipStream_t stream, const problem_t &P,
         const woq_extra_t &X) {
     auto go = [&](auto kern) __attribute__((always_inline)) {
@@ -493,10 +506,15 @@ int launch_variant(int scb, int zpb, dim3 grid, size_t lds, hipStream_t stream, 
             }
         }
         hipLaunchKernelGGL(kern, grid, dim3(NWV * 64), lds, stream, P, X);
+        if (X.ksplit > 1) {
+            const long total = (long)grid.x * ((X.M + 3) / 4) * (16 * 8 * CHD);
+            hipLaunchKernelGGL(woq_reduce_kernel<CHD>, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, stream,
+                    P, X, (int)grid.x);
+        }
         return hipGetLastError() == hipSuccess ? MI355_SUCCESS : MI355_RUNTIME_ERROR;
     };
 #define MI355_WOQ_CASE(S, Z) \
-    if (scb == S && zpb == Z) return go(woq_gemv_kernel<MT, NWV, SS, S, Z>)
+    if (scb == S && zpb == Z) return go(woq_gemv_kernel<CHD, MT, NWV, SS, S, Z>)
     MI355_WOQ_CASE(16, 4);
     MI355_WOQ_CASE(16, 8);
     MI355_WOQ_CASE(16, 32);
@@ -535,7 +553,6 @@ int woq_supported(const mi355_matmul_desc_t &d) {
     const bool sg = !quant_absent(d.wei_scale) && (d.wei_scale.mask & 2);
     const bool zg = !quant_absent(d.wei_zp) && (d.wei_zp.mask & 2);
     if (sg && zg && gs != gz) return MI355_UNIMPLEMENTED;
-    if ((d.N + NW - 1) / NW > MAX_CHUNKS) return MI355_UNIMPLEMENTED;
     return MI355_SUCCESS;
 }
 
@@ -550,11 +567,6 @@ int woq_launch(const mi355_matmul_desc_t &d, const problem_t &P, void *scratch, 
         return MI355_INVALID_ARGUMENTS;
     }
     woq_extra_t X {};
-    X.counters = arrival_counters((int)(g_launch_seq.fetch_add(1) % COUNTER_SLOTS));
-    if (!X.counters) {
-        set_error("woq_gemv: cannot resolve the arrival counters on this device");
-        return MI355_RUNTIME_ERROR;
-    }
     X.wei = (const uint8_t *)P.wei;
     X.src = (const uint8_t *)P.src;
     X.partials = (float *)scratch;
@@ -576,8 +588,8 @@ int woq_launch(const mi355_matmul_desc_t &d, const problem_t &P, void *scratch, 
     X.signed_w = d.wei_dt == MI355_DT_S4;
     const dim3 grid((unsigned)plan.chunks, (unsigned)plan.ksplit, 1);
     const int scb = scale_bits(X.sc_dt), zpb = zp_bits(X.zp_dt);
-    if (plan.mt == 1) return launch_variant<1, 8, 8>(scb, zpb, grid, plan.lds_bytes, stream, P, X);
-    return launch_variant<2, 4, 8>(scb, zpb, grid, plan.lds_bytes, stream, P, X);
+    if (plan.mt == 1) return launch_variant<2, 1, 8, 8>(scb, zpb, grid, plan.lds_bytes, stream, P, X);
+    return launch_variant<2, 2, 4, 8>(scb, zpb, grid, plan.lds_bytes, stream, P, X);
 }
 
 } // namespace mi355

@@ -137,6 +137,11 @@ WOQ_VARIANTS = [
     (32, 1024, 512, 32, "u4", "f32", "grouped", "u4", "none", "bf16", True),
     (3, 4096, 256, 256, "u4", "bf16", "none", "u8", "grouped", "f32", False),    # no K split (wide N), no scales
     (8, 768, 4096, 128, "u4", "bf16", "grouped", "s32", "grouped", "bf16", False),
+    # wide N: 512-column chunks, 16-byte weight loads
+    (1, 2048, 1024, 128, "u4", "bf16", "grouped", "u4", "grouped", "bf16", False),
+    (8, 2080, 528, 48, "s4", "f16", "grouped", "s8", "grouped", "f32", True),     # ragged last chunk, K not a multiple of the split
+    (16, 4096, 1024, 128, "u4", "f32", "column", "u4", "common", "bf16", False),
+    (2, 14336, 256, 128, "u4", "bf16", "grouped", "s4", "column", "f32", False),
 ]
 
 
