@@ -135,8 +135,11 @@ __device__ __forceinline__ void issue_stage(const dma_plan_t &p, const char *a_b
 //   s_barrier             everybody's did, and everybody finished group g-1
 //   DMA group g+NG-1      into the slots group g-1 used
 //   ds_read + MFMA over group g
-// `Mma` supplies frag_t, load(frag, S, wm, wn, lane, ctx, g) with S[k] the LDS
-// address of the k-th stage of the group, and mma(acc, frag, ctx, g).
+// `Mma` supplies frag_t, load_b(frag, S, wn, lane, ctx, g) for the 8 B^T
+// fragments, load_a(frag, i, S, wm, lane, ctx, g) for A fragment i (S[k] is the
+// LDS address of the k-th stage of the group), mma_row(acc, frag, i, ctx, g)
+// for the 8 MFMAs of A fragment i, and A_READS / B_READS = LDS read
+// instructions per fragment.
 // a_tile / b_tile point at the first K byte of tile row 0.
 template <int NSTAGE, int KSTEP, class Mma, class Acc, class Ctx>
 __device__ __forceinline__ void main_loop(Acc &acc, char *smem, const char *a_tile,
@@ -153,41 +156,71 @@ __device__ __forceinline__ void main_loop(Acc &acc, char *smem, const char *a_ti
     const unsigned lds0 = (unsigned)(size_t)(__attribute__((address_space(3))) char *)smem;
     const dma_plan_t plan = make_dma_plan(wave, lane, rows_a_left, rows_b_left, lda, ldb);
 
-    auto issue_group = [&](int g, int slot) {
+    // DMA number i (0..7) of every stage of group g: A row blocks first, then B^T
+    auto issue_part = [&](int g, int slot, int i) __attribute__((always_inline)) {
 #pragma unroll
-        for (int k = 0; k < KSTEP; ++k)
-            issue_stage(plan, a_tile + ((long)g * KSTEP + k) * BKB, b_tile + ((long)g * KSTEP + k) * BKB,
-                    lds0 + slot * GROUP_BYTES + k * STAGE_BYTES);
-        Mma::issue_extra(ctx, g, slot, wave, lane);
+        for (int k = 0; k < KSTEP; ++k) {
+            const long koff = ((long)g * KSTEP + k) * BKB;
+            const unsigned lds_stage = lds0 + slot * GROUP_BYTES + k * STAGE_BYTES;
+            if (i < 4) dma16(a_tile + koff, plan.voff_a[i], lds_stage + plan.lds_a[i]);
+            else dma16(b_tile + koff, plan.voff_b[i - 4], lds_stage + plan.lds_b[i - 4]);
+        }
+        if (i == 7) Mma::issue_extra(ctx, g, slot, wave, lane);
     };
 
     // prologue: groups 0 .. NG-2 in flight
 #pragma unroll
     for (int s = 0; s < NG - 1; ++s)
-        if (s < ngroups) issue_group(s, s);
+        if (s < ngroups) {
+#pragma unroll
+            for (int i = 0; i < 8; ++i) issue_part(s, s, i);
+        }
 
     int slot = 0;
+    // One group: all B fragments and the first two A fragments, then per A
+    // fragment i its 8 MFMAs, with the load of A fragment i+2 issued ahead of
+    // them.  The DMAs of group g+NG-1 go out first, in one burst (spreading
+    // them over the rows of MFMAs made the register allocator shuffle the
+    // accumulators around every inline-assembly statement).  The scheduling
+    // barriers pin the interleaving of LDS reads and MFMAs (the
+    // compiler otherwise funnels every A fragment through one register set and
+    // waits out an LDS round trip before each row of MFMAs).
+    // (The conditional around the DMA burst matters beyond its purpose: with a
+    // branch-free body the compiler rotates the loop and shuffles the 256
+    // accumulators through copies in every iteration.)
     for (int g = 0; g < ngroups; ++g) {
         // groups g+1 .. g+NG-2 may stay in flight
         if (g + NG - 2 < ngroups) wait_vmcnt<(NG - 2) * GROUP_DMAS>();
         else wait_vmcnt<0>();
         __builtin_amdgcn_s_barrier();
-        const int nxt = g + NG - 1;
-        if (nxt < ngroups) {
-            int nslot = slot + NG - 1;
-            if (nslot >= NG) nslot -= NG;
-#ifndef MI355_DBG_NO_DMA
-            issue_group(nxt, nslot);
-#endif
-        }
+        int nslot = slot + NG - 1;
+        if (nslot >= NG) nslot -= NG;
         const char *S[KSTEP];
 #pragma unroll
         for (int k = 0; k < KSTEP; ++k) S[k] = smem + slot * GROUP_BYTES + k * STAGE_BYTES;
-        typename Mma::frag_t f;
-        Mma::load(f, S, wm, wn, lane, ctx, g);
-#ifndef MI355_DBG_NO_MMA
-        Mma::mma(acc, f, ctx, g);
+#ifndef MI355_DBG_NO_DMA
+        if (g + NG - 1 < ngroups) {
+#pragma unroll
+            for (int i = 0; i < 8; ++i) issue_part(g + NG - 1, nslot, i);
+        }
 #endif
+        typename Mma::frag_t f;
+        Mma::load_b(f, S, wn, lane, ctx, g);
+        Mma::load_a(f, 0, S, wm, lane, ctx, g);
+        Mma::load_a(f, 1, S, wm, lane, ctx, g);
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            if (i + 2 < 8) Mma::load_a(f, i + 2, S, wm, lane, ctx, g);
+#ifndef MI355_DBG_NO_MMA
+            Mma::mma_row(acc, f, i, ctx, g);
+#endif
+        }
+        __builtin_amdgcn_sched_group_barrier(0x100, 8 * Mma::B_READS + 2 * Mma::A_READS, 0);
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            if (i + 2 < 8) __builtin_amdgcn_sched_group_barrier(0x100, Mma::A_READS, 0);
+            __builtin_amdgcn_sched_group_barrier(0x008, 8, 0);
+        }
         if (++slot == NG) slot = 0;
     }
     wait_vmcnt<0>();

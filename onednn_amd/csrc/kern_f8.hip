@@ -35,34 +35,36 @@ template <int FMT_A, int FMT_B>
 struct f8_mma_t {
     static constexpr int EXTRA_DMAS = 0;
     __device__ static __forceinline__ void issue_extra(const f8_ctx_t &, int, int, int, int) {}
+    static constexpr int A_READS = 2, B_READS = 2;
     struct frag_t {
         v8i a[8], b[8];
     };
     // lane l supplies row l%16 and K bytes 32*(l/16) .. +32 of the 128-byte
     // group: quarters 0,1 live in the first stage of the group, 2,3 in the
     // second
-    __device__ static __forceinline__ void load(frag_t &f, const char *const (&S)[2], int wm, int wn,
-            int lane, const f8_ctx_t &, int) {
+    __device__ static __forceinline__ v8i read32(const char *T, int row, int c0) {
+        const v4i lo = *(const v4i *)&T[swz(row, c0)], hi = *(const v4i *)&T[swz(row, c0 + 1)];
+        return v8i {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+    }
+    __device__ static __forceinline__ void load_b(frag_t &f, const char *const (&S)[2], int wn, int lane,
+            const f8_ctx_t &, int) {
+        const int frow = lane & 15, q = lane >> 4;
+        const char *Bs = ((q & 2) ? S[1] : S[0]) + B_OFF;
+#pragma unroll
+        for (int j = 0; j < 8; ++j) f.b[j] = read32(Bs, wn * 128 + j * 16 + frow, (q & 1) * 2);
+    }
+    __device__ static __forceinline__ void load_a(frag_t &f, int i, const char *const (&S)[2], int wm, int lane,
+            const f8_ctx_t &, int) {
         const int frow = lane & 15, q = lane >> 4;
         const char *As = (q & 2) ? S[1] : S[0];
-        const char *Bs = As + B_OFF;
-        const int c0 = (q & 1) * 2;
-#pragma unroll
-        for (int i = 0; i < 8; ++i) {
-            const int ra = wm * 128 + i * 16 + frow, rb = wn * 128 + i * 16 + frow;
-            const v4i alo = *(const v4i *)&As[swz(ra, c0)], ahi = *(const v4i *)&As[swz(ra, c0 + 1)];
-            const v4i blo = *(const v4i *)&Bs[swz(rb, c0)], bhi = *(const v4i *)&Bs[swz(rb, c0 + 1)];
-            f.a[i] = v8i {alo[0], alo[1], alo[2], alo[3], ahi[0], ahi[1], ahi[2], ahi[3]};
-            f.b[i] = v8i {blo[0], blo[1], blo[2], blo[3], bhi[0], bhi[1], bhi[2], bhi[3]};
-        }
+        f.a[i] = read32(As, wm * 128 + i * 16 + frow, (q & 1) * 2);
     }
-    __device__ static __forceinline__ void mma(v4f (&acc)[8][8], const frag_t &f, const f8_ctx_t &, int) {
+    __device__ static __forceinline__ void mma_row(v4f (&acc)[8][8], const frag_t &f, int i, const f8_ctx_t &,
+            int) {
 #pragma unroll
-        for (int i = 0; i < 8; ++i)
-#pragma unroll
-            for (int j = 0; j < 8; ++j)
-                acc[i][j] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(
-                        f.a[i], f.b[j], acc[i][j], FMT_A, FMT_B, 0, 0, 0, 0);
+        for (int j = 0; j < 8; ++j)
+            acc[i][j] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(
+                    f.a[i], f.b[j], acc[i][j], FMT_A, FMT_B, 0, 0, 0, 0);
     }
 };
 

@@ -41,31 +41,30 @@ template <bool SRC_U8, bool WEI_U8>
 struct i8_mma_t {
     static constexpr int EXTRA_DMAS = 0;
     __device__ static __forceinline__ void issue_extra(const i8_ctx_t &, int, int, int, int) {}
+    static constexpr int A_READS = 1, B_READS = 1;
     struct frag_t {
         v4i a[8], b[8];
     };
-    __device__ static __forceinline__ void load(frag_t &f, const char *const (&S)[1], int wm, int wn,
-            int lane, const i8_ctx_t &, int) {
-        const char *As = S[0], *Bs = S[0] + B_OFF;
+    __device__ static __forceinline__ void load_b(frag_t &f, const char *const (&S)[1], int wn, int lane,
+            const i8_ctx_t &, int) {
+        const char *Bs = S[0] + B_OFF;
         const int frow = lane & 15, fch = lane >> 4;
 #pragma unroll
-        for (int i = 0; i < 8; ++i) {
-            f.a[i] = *(const v4i *)&As[swz(wm * 128 + i * 16 + frow, fch)];
-            f.b[i] = *(const v4i *)&Bs[swz(wn * 128 + i * 16 + frow, fch)];
-        }
+        for (int j = 0; j < 8; ++j) f.b[j] = *(const v4i *)&Bs[swz(wn * 128 + j * 16 + frow, fch)];
     }
-    __device__ static __forceinline__ void mma(v4i (&acc)[8][8], const frag_t &f, const i8_ctx_t &, int) {
-        v4i a[8], b[8];
+    __device__ static __forceinline__ void load_a(frag_t &f, int i, const char *const (&S)[1], int wm, int lane,
+            const i8_ctx_t &, int) {
+        const int frow = lane & 15, fch = lane >> 4;
+        f.a[i] = *(const v4i *)&S[0][swz(wm * 128 + i * 16 + frow, fch)];
+    }
+    __device__ static __forceinline__ void mma_row(v4i (&acc)[8][8], const frag_t &f, int i, const i8_ctx_t &,
+            int) {
+        const v4i a = SRC_U8 ? (f.a[i] ^ (int)0x80808080) : f.a[i];
 #pragma unroll
-        for (int i = 0; i < 8; ++i) {
-            a[i] = SRC_U8 ? (f.a[i] ^ (int)0x80808080) : f.a[i];
-            b[i] = WEI_U8 ? (f.b[i] ^ (int)0x80808080) : f.b[i];
+        for (int j = 0; j < 8; ++j) {
+            const v4i b = WEI_U8 ? (f.b[j] ^ (int)0x80808080) : f.b[j];
+            acc[i][j] = __builtin_amdgcn_mfma_i32_16x16x64_i8(a, b, acc[i][j], 0, 0, 0);
         }
-#pragma unroll
-        for (int i = 0; i < 8; ++i)
-#pragma unroll
-            for (int j = 0; j < 8; ++j)
-                acc[i][j] = __builtin_amdgcn_mfma_i32_16x16x64_i8(a[i], b[j], acc[i][j], 0, 0, 0);
     }
 };
 

@@ -55,35 +55,43 @@ struct mxf4_mma_t {
         dma4(c.sa_tile + (long)g * 4, c.voff_a, dst);
         dma4(c.sb_tile + (long)g * 4, c.voff_b, dst + 1024);
     }
+    static constexpr int A_READS = 2, B_READS = 2; // data + scale dword
     struct frag_t {
         v4i a[8], b[8];
         int sa[8], sb[8];
     };
-    __device__ static __forceinline__ void load(frag_t &f, const char *const (&S)[1], int wm, int wn,
-            int lane, const mxf4_ctx_t &c, int) {
-        const char *As = S[0], *Bs = S[0] + B_OFF;
+    __device__ static __forceinline__ const unsigned *scales(const char *const (&S)[1], const mxf4_ctx_t &c) {
         const int slot = (int)((S[0] - c.smem) / STAGE_BYTES);
-        const unsigned *sc = (const unsigned *)(c.smem + SCALE_OFF + slot * SCALE_STAGE);
+        return (const unsigned *)(c.smem + SCALE_OFF + slot * SCALE_STAGE);
+    }
+    __device__ static __forceinline__ void load_b(frag_t &f, const char *const (&S)[1], int wn, int lane,
+            const mxf4_ctx_t &c, int) {
+        const char *Bs = S[0] + B_OFF;
+        const unsigned *sc = scales(S, c);
         const int frow = lane & 15, q = lane >> 4;
 #pragma unroll
-        for (int i = 0; i < 8; ++i) {
-            const int ra = wm * 128 + i * 16 + frow, rb = wn * 128 + i * 16 + frow;
-            f.a[i] = *(const v4i *)&As[swz(ra, q)];
-            f.b[i] = *(const v4i *)&Bs[swz(rb, q)];
-            f.sa[i] = (int)((sc[ra] >> (q * 8)) & 0xffu);
-            f.sb[i] = (int)((sc[256 + rb] >> (q * 8)) & 0xffu);
+        for (int j = 0; j < 8; ++j) {
+            const int rb = wn * 128 + j * 16 + frow;
+            f.b[j] = *(const v4i *)&Bs[swz(rb, q)];
+            f.sb[j] = (int)((sc[256 + rb] >> (q * 8)) & 0xffu);
         }
     }
-    __device__ static __forceinline__ void mma(v4f (&acc)[8][8], const frag_t &f, const mxf4_ctx_t &, int) {
+    __device__ static __forceinline__ void load_a(frag_t &f, int i, const char *const (&S)[1], int wm, int lane,
+            const mxf4_ctx_t &c, int) {
+        const unsigned *sc = scales(S, c);
+        const int frow = lane & 15, q = lane >> 4;
+        const int ra = wm * 128 + i * 16 + frow;
+        f.a[i] = *(const v4i *)&S[0][swz(ra, q)];
+        f.sa[i] = (int)((sc[ra] >> (q * 8)) & 0xffu);
+    }
+    __device__ static __forceinline__ void mma_row(v4f (&acc)[8][8], const frag_t &f, int i, const mxf4_ctx_t &,
+            int) {
+        const v8i a = {f.a[i][0], f.a[i][1], f.a[i][2], f.a[i][3], 0, 0, 0, 0};
 #pragma unroll
-        for (int i = 0; i < 8; ++i) {
-            const v8i a = {f.a[i][0], f.a[i][1], f.a[i][2], f.a[i][3], 0, 0, 0, 0};
-#pragma unroll
-            for (int j = 0; j < 8; ++j) {
-                const v8i bb = {f.b[j][0], f.b[j][1], f.b[j][2], f.b[j][3], 0, 0, 0, 0};
-                acc[i][j] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(
-                        a, bb, acc[i][j], 4, 4, 0, f.sa[i], 0, f.sb[j]);
-            }
+        for (int j = 0; j < 8; ++j) {
+            const v8i bb = {f.b[j][0], f.b[j][1], f.b[j][2], f.b[j][3], 0, 0, 0, 0};
+            acc[i][j] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(
+                    a, bb, acc[i][j], 4, 4, 0, f.sa[i], 0, f.sb[j]);
         }
     }
 };

@@ -51,6 +51,7 @@ struct epi_hoist_t {
     int nfast; // how many of them; the rest run through the generic loop
     int n_po;
     int dst_dt, dst_vec; // dst_vec: four consecutive n leave as one aligned store
+    int batchable;       // every operand is hoisted or staged and every post-op is a register-resident one
 };
 
 __device__ __forceinline__ bool vec_ok(const void *p, long s0, long s1, int bits) {
@@ -153,6 +154,23 @@ __device__ __forceinline__ epi_hoist_t make_hoist(const PT &P, long b, long nbas
             && vec_ok(P.bias, P.bs[0], P.bs[1], dt_bits(P.bias_dt))) {
         H.staged = STG_BIAS; H.staged_dt = P.bias_dt; H.staged_p = (const char *)P.bias;
         H.st_s0 = P.bs[0]; H.st_s1 = P.bs[1];
+    }
+    // The batched epilogue (several row quads per dispatch) needs every operand in
+    // registers or in the staging area: no loads inside the loop.
+    H.batchable = H.n_po == H.nfast && (H.bias_mode != 2 || H.staged == STG_BIAS) && nvalid == 4 && H.dst_vec;
+    {
+        auto operand_ready = [&](const po_reg_t &r, int i) {
+            if (r.kind == MI355_PO_BINARY)
+                return (i == H.hoisted_po || i == H.staged) && (r.alg == MI355_BINARY_ADD || r.alg == MI355_BINARY_MUL);
+            if (r.kind == MI355_PO_SUM) return H.staged == STG_SUM;
+            return true; // grab() admits the five cheap eltwise algorithms only
+        };
+        const int dd = H.dst_dt;
+        if (dd != MI355_DT_S8 && dd != MI355_DT_U8 && dd != MI355_DT_BF16 && dd != MI355_DT_F32 && dd != MI355_DT_S32)
+            H.batchable = 0;
+        if (H.nfast > 0 && !operand_ready(H.pf0, 0)) H.batchable = 0;
+        if (H.nfast > 1 && !operand_ready(H.pf1, 1)) H.batchable = 0;
+        if (H.nfast > 2 && !operand_ready(H.pf2, 2)) H.batchable = 0;
     }
     return H;
 }
@@ -392,6 +410,181 @@ __device__ __forceinline__ void store4(const PT &P, const epi_hoist_t &H, const 
     }
 }
 
+// ---- batched form: NQ row quads per dispatch.  Every data-type and post-op
+// dispatch below is uniform over the wavefront and is taken once for the NQ
+// quads, and the quads' LDS reads and stores overlap; with one wavefront per
+// SIMD a dispatch per quad leaves the SIMD idle through every branch.
+template <int NQ>
+__device__ __forceinline__ void eltwiseQ_simple(int alg, float (&v)[NQ][4], float alpha, float beta, float scale) {
+    if (alg == MI355_ELTWISE_RELU) {
+#pragma unroll
+        for (int k = 0; k < NQ; ++k)
+#pragma unroll
+            for (int e = 0; e < 4; ++e) v[k][e] = (v[k][e] > 0 ? v[k][e] : v[k][e] * alpha) * scale;
+    } else if (alg == MI355_ELTWISE_LINEAR) {
+#pragma unroll
+        for (int k = 0; k < NQ; ++k)
+#pragma unroll
+            for (int e = 0; e < 4; ++e) v[k][e] = (alpha * v[k][e] + beta) * scale;
+    } else if (alg == MI355_ELTWISE_GELU_TANH) {
+#pragma unroll
+        for (int k = 0; k < NQ; ++k)
+#pragma unroll
+            for (int e = 0; e < 4; ++e) v[k][e] = eltwise_f(MI355_ELTWISE_GELU_TANH, v[k][e], alpha, beta) * scale;
+    } else if (alg == MI355_ELTWISE_CLIP) {
+#pragma unroll
+        for (int k = 0; k < NQ; ++k)
+#pragma unroll
+            for (int e = 0; e < 4; ++e) v[k][e] = eltwise_f(MI355_ELTWISE_CLIP, v[k][e], alpha, beta) * scale;
+    } else {
+#pragma unroll
+        for (int k = 0; k < NQ; ++k)
+#pragma unroll
+            for (int e = 0; e < 4; ++e) v[k][e] = eltwise_f(MI355_ELTWISE_CLIP_V2, v[k][e], alpha, beta) * scale;
+    }
+}
+
+template <int NQ>
+__device__ __forceinline__ void apply_epilogueQ(const epi_hoist_t &H, float (&v)[NQ][4], const uint4 (&stg)[NQ]) {
+    float sy[NQ][4];
+#pragma unroll
+    for (int k = 0; k < NQ; ++k)
+#pragma unroll
+        for (int e = 0; e < 4; ++e) sy[k][e] = 0.f;
+    if (H.staged != STG_NONE) {
+        // every array index below is a compile-time constant: a rolled loop over
+        // the quads would put these arrays into private memory
+        if (H.staged_dt == MI355_DT_BF16) {
+#pragma unroll
+            for (int k = 0; k < NQ; ++k) staged4(MI355_DT_BF16, stg[k], sy[k]);
+        } else if (H.staged_dt == MI355_DT_F32) {
+#pragma unroll
+            for (int k = 0; k < NQ; ++k) staged4(MI355_DT_F32, stg[k], sy[k]);
+        } else if (H.staged_dt == MI355_DT_F16) {
+#pragma unroll
+            for (int k = 0; k < NQ; ++k) staged4(MI355_DT_F16, stg[k], sy[k]);
+        } else {
+#pragma unroll
+            for (int k = 0; k < NQ; ++k) staged4(MI355_DT_S32, stg[k], sy[k]);
+        }
+    }
+    if (H.bias_mode == 1) {
+#pragma unroll
+        for (int k = 0; k < NQ; ++k)
+#pragma unroll
+            for (int e = 0; e < 4; ++e) v[k][e] += H.bias4[e];
+    } else if (H.bias_mode == 2) { // staged
+#pragma unroll
+        for (int k = 0; k < NQ; ++k)
+#pragma unroll
+            for (int e = 0; e < 4; ++e) v[k][e] += sy[k][e];
+    }
+    auto fast_op = [&](const po_reg_t &r, int i) __attribute__((always_inline)) {
+        if (r.kind == MI355_PO_ELTWISE) {
+            eltwiseQ_simple<NQ>(r.alg, v, r.alpha, r.beta, r.scale);
+        } else if (r.kind == MI355_PO_BINARY) {
+            const bool hoisted = i == H.hoisted_po;
+            if (r.alg == MI355_BINARY_ADD) {
+#pragma unroll
+                for (int k = 0; k < NQ; ++k)
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) v[k][e] = v[k][e] + (hoisted ? H.hv4[e] : sy[k][e]);
+            } else { // mul (nothing else is batchable)
+#pragma unroll
+                for (int k = 0; k < NQ; ++k)
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) v[k][e] = v[k][e] * (hoisted ? H.hv4[e] : sy[k][e]);
+            }
+        } else { // sum: the old dst is the staged stream
+#pragma unroll
+            for (int k = 0; k < NQ; ++k)
+#pragma unroll
+                for (int e = 0; e < 4; ++e) v[k][e] += r.scale * (sy[k][e] - r.zpf);
+        }
+    };
+    if (H.nfast > 0) fast_op(H.pf0, 0);
+    if (H.nfast > 1) fast_op(H.pf1, 1);
+    if (H.nfast > 2) fast_op(H.pf2, 2);
+    if (H.ds_mode == 1) {
+#pragma unroll
+        for (int k = 0; k < NQ; ++k)
+#pragma unroll
+            for (int e = 0; e < 4; ++e) v[k][e] /= H.ds;
+    } else if (H.ds_mode == 2) {
+#pragma unroll
+        for (int k = 0; k < NQ; ++k)
+#pragma unroll
+            for (int e = 0; e < 4; ++e) v[k][e] *= H.ds_inv;
+    }
+    if (H.dzp_mode) {
+#pragma unroll
+        for (int k = 0; k < NQ; ++k)
+#pragma unroll
+            for (int e = 0; e < 4; ++e) v[k][e] += H.dzp4[e];
+    }
+}
+
+// four full quads (nvalid == 4, vector stores allowed) to dst; `ok[k]` masks rows beyond M
+template <int NQ, class PT>
+__device__ __forceinline__ void storeQ(const PT &P, const epi_hoist_t &H, const float (&v)[NQ][4], long b,
+        const long (&m)[NQ], long n, const bool (&ok)[NQ]) {
+    uint32_t w[NQ][4];
+    const int dt = H.dst_dt;
+    if (dt == MI355_DT_S8) {
+#pragma unroll
+        for (int k = 0; k < NQ; ++k)
+#pragma unroll
+            for (int e = 0; e < 4; ++e) w[k][e] = (uint32_t)(int)__builtin_rintf(sat(v[k][e], -128.f, 127.f)) & 0xffu;
+    } else if (dt == MI355_DT_U8) {
+#pragma unroll
+        for (int k = 0; k < NQ; ++k)
+#pragma unroll
+            for (int e = 0; e < 4; ++e) w[k][e] = (uint32_t)(int)__builtin_rintf(sat(v[k][e], 0.f, 255.f)) & 0xffu;
+    } else if (dt == MI355_DT_BF16) {
+#pragma unroll
+        for (int k = 0; k < NQ; ++k)
+#pragma unroll
+            for (int e = 0; e < 4; ++e) w[k][e] = f32_to_bf16(v[k][e]);
+    } else if (dt == MI355_DT_F32) {
+#pragma unroll
+        for (int k = 0; k < NQ; ++k)
+#pragma unroll
+            for (int e = 0; e < 4; ++e) w[k][e] = f2u(v[k][e]);
+    } else { // s32 (nothing else is batchable)
+#pragma unroll
+        for (int k = 0; k < NQ; ++k)
+#pragma unroll
+            for (int e = 0; e < 4; ++e)
+                w[k][e] = (uint32_t)(int)__builtin_rintf(sat(v[k][e], -2147483648.f, 2147483520.f));
+    }
+    const int bits = dt_bits(dt);
+    const long off0 = b * P.ds[0] + n;
+    if (bits == 8) {
+#pragma unroll
+        for (int k = 0; k < NQ; ++k)
+            if (ok[k])
+                *(uint32_t *)((uint8_t *)P.dst + off0 + m[k] * P.ds[1])
+                        = w[k][0] | (w[k][1] << 8) | (w[k][2] << 16) | (w[k][3] << 24);
+    } else if (bits == 16) {
+#pragma unroll
+        for (int k = 0; k < NQ; ++k)
+            if (ok[k]) {
+                uint2 o;
+                o.x = w[k][0] | (w[k][1] << 16);
+                o.y = w[k][2] | (w[k][3] << 16);
+                *(uint2 *)((uint16_t *)P.dst + off0 + m[k] * P.ds[1]) = o;
+            }
+    } else {
+#pragma unroll
+        for (int k = 0; k < NQ; ++k)
+            if (ok[k]) {
+                uint4 o;
+                o.x = w[k][0]; o.y = w[k][1]; o.z = w[k][2]; o.w = w[k][3];
+                *(uint4 *)((uint32_t *)P.dst + off0 + m[k] * P.ds[1]) = o;
+            }
+    }
+}
+
 // Accumulator layouts: how a wavefront's 128x128 quadrant sits in registers
 // and how one 32-row slab of it is written to LDS as [32 rows][128 cols] s32.
 //
@@ -479,6 +672,34 @@ __device__ __forceinline__ void store_quadrant(const PT &P, char *smem, const Ac
             for (int it = 0; it < 16; ++it) stg[it * 64 + lane] = tmp[it];
         }
         Layout::write_slab(acc, i, wl, lane);
+        if (H.batchable) {
+            constexpr int NQ = 4;
+#pragma unroll 1
+            for (int it0 = 0; it0 < 16; it0 += NQ) {
+                v4i_t raw[NQ];
+                uint4 sv[NQ];
+                long m[NQ];
+                bool ok[NQ];
+#pragma unroll
+                for (int k = 0; k < NQ; ++k) {
+                    const int row = (it0 + k) * 2 + (lane >> 5);
+                    m[k] = m_base + i * 32 + row;
+                    ok[k] = m[k] < P.M;
+                    raw[k] = *(const v4i_t *)&wl[row * 128 + (lane & 31) * 4];
+                    sv[k] = make_uint4(0, 0, 0, 0);
+                }
+                if (H.staged != STG_NONE) {
+#pragma unroll
+                    for (int k = 0; k < NQ; ++k) sv[k] = stg[(it0 + k) * 64 + lane];
+                }
+                float v[NQ][4];
+#pragma unroll
+                for (int k = 0; k < NQ; ++k) conv.row(raw[k], ok[k] ? m[k] : m_base, v[k]);
+                apply_epilogueQ<NQ>(H, v, sv);
+                storeQ<NQ>(P, H, v, b, m, nbase, ok);
+            }
+            continue;
+        }
 #pragma unroll 1
         for (int it = 0; it < 16; ++it) {
             const int row = it * 2 + (lane >> 5);
