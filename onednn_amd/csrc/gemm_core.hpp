@@ -67,6 +67,14 @@ __device__ __forceinline__ void dma16(const void *sbase, unsigned voff, unsigned
                  : "memory", "m0");
 }
 
+// LDS reads through explicit 32-bit LDS addresses: a generic pointer that the
+// compiler cannot prove to be shared memory (one selected between two stages,
+// say) turns every ds_read into a flat load through the vector memory path.
+typedef const v4i __attribute__((address_space(3))) *lds_v4i_ptr_t;
+typedef const unsigned __attribute__((address_space(3))) *lds_u32_ptr_t;
+__device__ __forceinline__ v4i lds_read16(unsigned addr) { return *(lds_v4i_ptr_t)(size_t)addr; }
+__device__ __forceinline__ unsigned lds_read4(unsigned addr) { return *(lds_u32_ptr_t)(size_t)addr; }
+
 // s_waitcnt vmcnt(n) only (expcnt / lgkmcnt left at their maxima)
 template <int N>
 __device__ __forceinline__ void wait_vmcnt() {
@@ -137,9 +145,9 @@ __device__ __forceinline__ void issue_stage(const dma_plan_t &p, const char *a_b
 //   ds_read + MFMA over group g
 // `Mma` supplies frag_t, load_b(frag, S, wn, lane, ctx, g) for the 8 B^T
 // fragments, load_a(frag, i, S, wm, lane, ctx, g) for A fragment i (S[k] is the
-// LDS address of the k-th stage of the group), mma_row(acc, frag, i, ctx, g)
-// for the 8 MFMAs of A fragment i, and A_READS / B_READS = LDS read
-// instructions per fragment.
+// LDS byte address of the k-th stage of the group), mma_row(acc, frag, i, ctx, g)
+// for the COLS MFMAs of A fragment i (ROWS x COLS MFMA tiles per quadrant),
+// and A_READS / B_READS = LDS read instructions per fragment.
 // a_tile / b_tile point at the first K byte of tile row 0.
 template <int NSTAGE, int KSTEP, class Mma, class Acc, class Ctx>
 __device__ __forceinline__ void main_loop(Acc &acc, char *smem, const char *a_tile,
@@ -178,7 +186,7 @@ __device__ __forceinline__ void main_loop(Acc &acc, char *smem, const char *a_ti
 
     int slot = 0;
     // One group: all B fragments and the first two A fragments, then per A
-    // fragment i its 8 MFMAs, with the load of A fragment i+2 issued ahead of
+    // fragment i its row of MFMAs, with the load of A fragment i+2 issued ahead of
     // them.  The DMAs of group g+NG-1 go out first, in one burst (spreading
     // them over the rows of MFMAs made the register allocator shuffle the
     // accumulators around every inline-assembly statement).  The scheduling
@@ -195,9 +203,9 @@ __device__ __forceinline__ void main_loop(Acc &acc, char *smem, const char *a_ti
         __builtin_amdgcn_s_barrier();
         int nslot = slot + NG - 1;
         if (nslot >= NG) nslot -= NG;
-        const char *S[KSTEP];
+        unsigned S[KSTEP]; // LDS byte addresses of the group's stages
 #pragma unroll
-        for (int k = 0; k < KSTEP; ++k) S[k] = smem + slot * GROUP_BYTES + k * STAGE_BYTES;
+        for (int k = 0; k < KSTEP; ++k) S[k] = lds0 + slot * GROUP_BYTES + k * STAGE_BYTES;
 #ifndef MI355_DBG_NO_DMA
         if (g + NG - 1 < ngroups) {
 #pragma unroll
@@ -205,21 +213,22 @@ __device__ __forceinline__ void main_loop(Acc &acc, char *smem, const char *a_ti
         }
 #endif
         typename Mma::frag_t f;
+        constexpr int ROWS = Mma::ROWS, COLS = Mma::COLS; // MFMA tiles of the quadrant
         Mma::load_b(f, S, wn, lane, ctx, g);
         Mma::load_a(f, 0, S, wm, lane, ctx, g);
         Mma::load_a(f, 1, S, wm, lane, ctx, g);
 #pragma unroll
-        for (int i = 0; i < 8; ++i) {
-            if (i + 2 < 8) Mma::load_a(f, i + 2, S, wm, lane, ctx, g);
+        for (int i = 0; i < ROWS; ++i) {
+            if (i + 2 < ROWS) Mma::load_a(f, i + 2, S, wm, lane, ctx, g);
 #ifndef MI355_DBG_NO_MMA
             Mma::mma_row(acc, f, i, ctx, g);
 #endif
         }
-        __builtin_amdgcn_sched_group_barrier(0x100, 8 * Mma::B_READS + 2 * Mma::A_READS, 0);
+        __builtin_amdgcn_sched_group_barrier(0x100, COLS * Mma::B_READS + 2 * Mma::A_READS, 0);
 #pragma unroll
-        for (int i = 0; i < 8; ++i) {
-            if (i + 2 < 8) __builtin_amdgcn_sched_group_barrier(0x100, Mma::A_READS, 0);
-            __builtin_amdgcn_sched_group_barrier(0x008, 8, 0);
+        for (int i = 0; i < ROWS; ++i) {
+            if (i + 2 < ROWS) __builtin_amdgcn_sched_group_barrier(0x100, Mma::A_READS, 0);
+            __builtin_amdgcn_sched_group_barrier(0x008, COLS, 0);
         }
         if (++slot == NG) slot = 0;
     }

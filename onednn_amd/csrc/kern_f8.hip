@@ -1,5 +1,5 @@
 // "hip:mfma_f8" -- LDS-tiled fp8 GEMM (OCP e4m3 / e5m2 operands, f32
-// accumulation) on the gfx950 matrix cores, v_mfma_f32_16x16x128_f8f6f4, with
+// accumulation) on the gfx950 matrix cores, v_mfma_f32_32x32x64_f8f6f4, with
 // the reference's epilogue fused in.
 //
 // Semantics: ref_matmul_t (src/cpu/matmul/ref_matmul.cpp:168-331) for f8 src
@@ -11,16 +11,21 @@
 // once, which differs only in rounding and is covered by the f32/bf16
 // comparison thresholds.
 //
-// Measured on MI355X with random operands: the 16x16x128 shape sustains
-// ~4.9 PFLOP/s, the 32x32x64 shape ~4.3 PFLOP/s, hence the choice.
+// MFMA shape: v_mfma_f32_32x32x64_f8f6f4.  Measured on MI355X with random
+// operands the 16x16x128 shape sustains ~4.9 PFLOP/s against ~4.3 for this
+// one, but it consumes 128 bytes of K per instruction: two 32 KB stages at a
+// time, which leaves room for two such groups in LDS and a prefetch distance
+// of one group, shorter than the memory latency (measured 175 us per 256x256
+// tile at K = 8192).  The 32x32x64 shape consumes one 64-byte stage like the
+// int8 kernel and keeps three stages in flight.
 #include "gemm_core.hpp"
 
 namespace mi355 {
 namespace {
 
 using namespace gemm;
-constexpr int NSTAGE = 4; // 4 x 32 KB ring, consumed two stages (K = 128) at a time
-constexpr int KSTEP = 2;
+constexpr int NSTAGE = 4; // 4 x 32 KB ring, one stage (K = 64) per step
+constexpr int KSTEP = 1;
 
 struct f8_extra_t {
     const char *bt; // weights as [N][K] bytes, K contiguous
@@ -35,35 +40,31 @@ template <int FMT_A, int FMT_B>
 struct f8_mma_t {
     static constexpr int EXTRA_DMAS = 0;
     __device__ static __forceinline__ void issue_extra(const f8_ctx_t &, int, int, int, int) {}
-    static constexpr int A_READS = 2, B_READS = 2;
+    static constexpr int ROWS = 4, COLS = 4, A_READS = 2, B_READS = 2;
     struct frag_t {
-        v8i a[8], b[8];
+        v8i a[4], b[4];
     };
-    // lane l supplies row l%16 and K bytes 32*(l/16) .. +32 of the 128-byte
-    // group: quarters 0,1 live in the first stage of the group, 2,3 in the
-    // second
-    __device__ static __forceinline__ v8i read32(const char *T, int row, int c0) {
-        const v4i lo = *(const v4i *)&T[swz(row, c0)], hi = *(const v4i *)&T[swz(row, c0 + 1)];
+    // lane l supplies row l%32 and K bytes 32*(l/32) .. +32 of the stage
+    __device__ static __forceinline__ v8i read32(unsigned T, int row, int c0) {
+        const v4i lo = lds_read16(T + swz(row, c0)), hi = lds_read16(T + swz(row, c0 + 1));
         return v8i {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
     }
-    __device__ static __forceinline__ void load_b(frag_t &f, const char *const (&S)[2], int wn, int lane,
+    __device__ static __forceinline__ void load_b(frag_t &f, const unsigned (&S)[1], int wn, int lane,
             const f8_ctx_t &, int) {
-        const int frow = lane & 15, q = lane >> 4;
-        const char *Bs = ((q & 2) ? S[1] : S[0]) + B_OFF;
+        const int frow = lane & 31, h = lane >> 5;
 #pragma unroll
-        for (int j = 0; j < 8; ++j) f.b[j] = read32(Bs, wn * 128 + j * 16 + frow, (q & 1) * 2);
+        for (int j = 0; j < 4; ++j) f.b[j] = read32(S[0] + B_OFF, wn * 128 + j * 32 + frow, h * 2);
     }
-    __device__ static __forceinline__ void load_a(frag_t &f, int i, const char *const (&S)[2], int wm, int lane,
+    __device__ static __forceinline__ void load_a(frag_t &f, int i, const unsigned (&S)[1], int wm, int lane,
             const f8_ctx_t &, int) {
-        const int frow = lane & 15, q = lane >> 4;
-        const char *As = (q & 2) ? S[1] : S[0];
-        f.a[i] = read32(As, wm * 128 + i * 16 + frow, (q & 1) * 2);
+        const int frow = lane & 31, h = lane >> 5;
+        f.a[i] = read32(S[0], wm * 128 + i * 32 + frow, h * 2);
     }
-    __device__ static __forceinline__ void mma_row(v4f (&acc)[8][8], const frag_t &f, int i, const f8_ctx_t &,
+    __device__ static __forceinline__ void mma_row(v16f (&acc)[4][4], const frag_t &f, int i, const f8_ctx_t &,
             int) {
 #pragma unroll
-        for (int j = 0; j < 8; ++j)
-            acc[i][j] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(
+        for (int j = 0; j < 4; ++j)
+            acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(
                     f.a[i], f.b[j], acc[i][j], FMT_A, FMT_B, 0, 0, 0, 0);
     }
 };
@@ -103,13 +104,13 @@ __global__ void __launch_bounds__(NT) f8_gemm_kernel(const problem_t P_, const f
     const char *A = (const char *)P.src + (P.ss[0] ? b * P.ss[0] : 0) + m0 * lda;
     const char *Bt = X.bt + b * X.bt_bstride + n0 * X.ldb;
 
-    v4f acc[8][8];
+    v16f acc[4][4];
 #pragma unroll
-    for (int i = 0; i < 8; ++i)
+    for (int i = 0; i < 4; ++i)
 #pragma unroll
-        for (int j = 0; j < 8; ++j)
+        for (int j = 0; j < 4; ++j)
 #pragma unroll
-            for (int r = 0; r < 4; ++r) acc[i][j][r] = 0.f;
+            for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
 
     main_loop<NSTAGE, KSTEP, f8_mma_t<FMT_A, FMT_B>>(acc, smem, A, Bt, lda, X.ldb, P.M - m0,
             P.N - n0, (int)(P.K / (BKB * KSTEP)), f8_ctx_t {});
@@ -137,7 +138,7 @@ __global__ void __launch_bounds__(NT) f8_gemm_kernel(const problem_t P_, const f
                     quant_off(P.wei_scale, bw, 0, nbase + e, P.K, P.N));
     }
     const bool interior = m0 + BM <= P.M && n0 + BN <= P.N;
-    store_quadrant<layout16_t>(P, smem, acc, b, m0 + wm * 128, n0 + wn * 128, interior, cv);
+    store_quadrant<layout32_t>(P, smem, acc, b, m0 + wm * 128, n0 + wn * 128, interior, cv);
 }
 
 struct f8_plan_t {

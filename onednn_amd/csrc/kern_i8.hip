@@ -41,21 +41,20 @@ template <bool SRC_U8, bool WEI_U8>
 struct i8_mma_t {
     static constexpr int EXTRA_DMAS = 0;
     __device__ static __forceinline__ void issue_extra(const i8_ctx_t &, int, int, int, int) {}
-    static constexpr int A_READS = 1, B_READS = 1;
+    static constexpr int ROWS = 8, COLS = 8, A_READS = 1, B_READS = 1;
     struct frag_t {
         v4i a[8], b[8];
     };
-    __device__ static __forceinline__ void load_b(frag_t &f, const char *const (&S)[1], int wn, int lane,
+    __device__ static __forceinline__ void load_b(frag_t &f, const unsigned (&S)[1], int wn, int lane,
             const i8_ctx_t &, int) {
-        const char *Bs = S[0] + B_OFF;
         const int frow = lane & 15, fch = lane >> 4;
 #pragma unroll
-        for (int j = 0; j < 8; ++j) f.b[j] = *(const v4i *)&Bs[swz(wn * 128 + j * 16 + frow, fch)];
+        for (int j = 0; j < 8; ++j) f.b[j] = lds_read16(S[0] + B_OFF + swz(wn * 128 + j * 16 + frow, fch));
     }
-    __device__ static __forceinline__ void load_a(frag_t &f, int i, const char *const (&S)[1], int wm, int lane,
+    __device__ static __forceinline__ void load_a(frag_t &f, int i, const unsigned (&S)[1], int wm, int lane,
             const i8_ctx_t &, int) {
         const int frow = lane & 15, fch = lane >> 4;
-        f.a[i] = *(const v4i *)&S[0][swz(wm * 128 + i * 16 + frow, fch)];
+        f.a[i] = lds_read16(S[0] + swz(wm * 128 + i * 16 + frow, fch));
     }
     __device__ static __forceinline__ void mma_row(v4i (&acc)[8][8], const frag_t &f, int i, const i8_ctx_t &,
             int) {

@@ -43,7 +43,7 @@ struct mxf4_ctx_t {
     const char *sa_tile, *sb_tile; // first scale byte of tile row 0
     unsigned voff_a, voff_b;       // this lane's row offset in the scale arrays
     unsigned lds_scale0;           // LDS byte address of the scale ring
-    const char *smem;
+    unsigned lds0;                 // LDS byte address of the tile ring
 };
 
 struct mxf4_mma_t {
@@ -55,34 +55,34 @@ struct mxf4_mma_t {
         dma4(c.sa_tile + (long)g * 4, c.voff_a, dst);
         dma4(c.sb_tile + (long)g * 4, c.voff_b, dst + 1024);
     }
-    static constexpr int A_READS = 2, B_READS = 2; // data + scale dword
+    static constexpr int ROWS = 8, COLS = 8, A_READS = 2, B_READS = 2; // data + scale dword
     struct frag_t {
         v4i a[8], b[8];
         int sa[8], sb[8];
     };
-    __device__ static __forceinline__ const unsigned *scales(const char *const (&S)[1], const mxf4_ctx_t &c) {
-        const int slot = (int)((S[0] - c.smem) / STAGE_BYTES);
-        return (const unsigned *)(c.smem + SCALE_OFF + slot * SCALE_STAGE);
+    // LDS byte address of the scale dwords that belong to the stage at S[0]
+    __device__ static __forceinline__ unsigned scales(const unsigned (&S)[1], const mxf4_ctx_t &c) {
+        const unsigned slot = (S[0] - c.lds0) / STAGE_BYTES;
+        return c.lds_scale0 + slot * SCALE_STAGE;
     }
-    __device__ static __forceinline__ void load_b(frag_t &f, const char *const (&S)[1], int wn, int lane,
+    __device__ static __forceinline__ void load_b(frag_t &f, const unsigned (&S)[1], int wn, int lane,
             const mxf4_ctx_t &c, int) {
-        const char *Bs = S[0] + B_OFF;
-        const unsigned *sc = scales(S, c);
+        const unsigned sc = scales(S, c);
         const int frow = lane & 15, q = lane >> 4;
 #pragma unroll
         for (int j = 0; j < 8; ++j) {
             const int rb = wn * 128 + j * 16 + frow;
-            f.b[j] = *(const v4i *)&Bs[swz(rb, q)];
-            f.sb[j] = (int)((sc[256 + rb] >> (q * 8)) & 0xffu);
+            f.b[j] = lds_read16(S[0] + B_OFF + swz(rb, q));
+            f.sb[j] = (int)((lds_read4(sc + (256 + rb) * 4) >> (q * 8)) & 0xffu);
         }
     }
-    __device__ static __forceinline__ void load_a(frag_t &f, int i, const char *const (&S)[1], int wm, int lane,
+    __device__ static __forceinline__ void load_a(frag_t &f, int i, const unsigned (&S)[1], int wm, int lane,
             const mxf4_ctx_t &c, int) {
-        const unsigned *sc = scales(S, c);
+        const unsigned sc = scales(S, c);
         const int frow = lane & 15, q = lane >> 4;
         const int ra = wm * 128 + i * 16 + frow;
-        f.a[i] = *(const v4i *)&S[0][swz(ra, q)];
-        f.sa[i] = (int)((sc[ra] >> (q * 8)) & 0xffu);
+        f.a[i] = lds_read16(S[0] + swz(ra, q));
+        f.sa[i] = (int)((lds_read4(sc + ra * 4) >> (q * 8)) & 0xffu);
     }
     __device__ static __forceinline__ void mma_row(v4f (&acc)[8][8], const frag_t &f, int i, const mxf4_ctx_t &,
             int) {
@@ -120,7 +120,7 @@ __global__ void __launch_bounds__(NT) mxf4_gemm_kernel(const problem_t P_, const
     const char *Bt = X.bt + b * X.bt_bstride + n0 * X.ldb;
 
     mxf4_ctx_t ctx;
-    ctx.smem = smem;
+    ctx.lds0 = (unsigned)(size_t)(__attribute__((address_space(3))) char *)smem;
     ctx.lds_scale0 = (unsigned)(size_t)(__attribute__((address_space(3))) char *)smem + SCALE_OFF;
     ctx.sa_tile = X.sa + b * X.sa_bstride + m0 * kb;
     ctx.sb_tile = X.sb + b * X.sb_bstride + n0 * kb;

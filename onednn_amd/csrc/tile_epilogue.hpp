@@ -22,11 +22,29 @@ namespace mi355 {
 namespace gemm {
 
 typedef int v4i_t __attribute__((ext_vector_type(4)));
+// The accumulator slab in LDS is written one dword at a time and read back as
+// 16-byte vectors: both accesses go through may_alias types, otherwise
+// type-based alias analysis lets the reads move above the writes.
+typedef int __attribute__((may_alias)) slab_int_t;
+typedef int __attribute__((ext_vector_type(4), may_alias)) slab_v4i_t;
+typedef uint4 __attribute__((may_alias)) stage_u4_t;
 
 __device__ __forceinline__ int raw_bits(int x) { return x; }
 __device__ __forceinline__ int raw_bits(float x) { return __float_as_int(x); }
 
 constexpr int STG_NONE = -1, STG_BIAS = 100, STG_SUM = 101;
+
+// gelu_tanh(s) = 0.5 s (1 + tanh(v)), v = sqrt(2/pi) s (1 + 0.044715 s^2)
+// (math_utils.hpp gelu_tanh_fwd), evaluated as s / (1 + exp(-2v)): the same
+// real function without the cancellation of 1 + tanh(v) for negative v, in one
+// hardware exponential and one reciprocal (a few ulp, like the polynomial
+// evaluation of the reference's JIT injector; the generic kernel keeps the
+// libm form of the reference's scalar code).
+__device__ __forceinline__ float gelu_tanh_fast(float s) {
+    const float v = 0.79788458347320556640625f * s * (1.f + 0.044715f * s * s);
+    const float e = __builtin_amdgcn_exp2f(-2.8853900817779268f * v); // exp(-2v)
+    return s * __builtin_amdgcn_rcpf(1.f + e);
+}
 
 struct po_reg_t {
     int kind, alg;
@@ -209,7 +227,7 @@ __device__ __forceinline__ void eltwise4_simple(int alg, float (&v)[4], float al
         for (int e = 0; e < 4; ++e) v[e] = (alpha * v[e] + beta) * scale;
     } else if (alg == MI355_ELTWISE_GELU_TANH) {
 #pragma unroll
-        for (int e = 0; e < 4; ++e) v[e] = eltwise_f(MI355_ELTWISE_GELU_TANH, v[e], alpha, beta) * scale;
+        for (int e = 0; e < 4; ++e) v[e] = gelu_tanh_fast(v[e]) * scale;
     } else if (alg == MI355_ELTWISE_CLIP) {
 #pragma unroll
         for (int e = 0; e < 4; ++e) v[e] = eltwise_f(MI355_ELTWISE_CLIP, v[e], alpha, beta) * scale;
@@ -430,7 +448,7 @@ __device__ __forceinline__ void eltwiseQ_simple(int alg, float (&v)[NQ][4], floa
 #pragma unroll
         for (int k = 0; k < NQ; ++k)
 #pragma unroll
-            for (int e = 0; e < 4; ++e) v[k][e] = eltwise_f(MI355_ELTWISE_GELU_TANH, v[k][e], alpha, beta) * scale;
+            for (int e = 0; e < 4; ++e) v[k][e] = gelu_tanh_fast(v[k][e]) * scale;
     } else if (alg == MI355_ELTWISE_CLIP) {
 #pragma unroll
         for (int k = 0; k < NQ; ++k)
@@ -592,14 +610,18 @@ __device__ __forceinline__ void storeQ(const PT &P, const epi_hoist_t &H, const 
 // row 32i + 8*(r/4) + 4*(lane/32) + r%4, column 32j + lane%32.
 struct layout32_t {
     template <class Acc>
-    static __device__ __forceinline__ void write_slab(const Acc &acc, int s, int *wl, int lane) {
+    static __device__ __forceinline__ void write_slab(const Acc &acc, int s, slab_int_t *wl, int lane) {
+        // volatile: the dword stores stay single ds_write_b32 instructions.  Merged
+        // into ds_write2_b32 pairs by the compiler (ROCm 7.2), two stores per tile
+        // of this layout came out with their first offset divided by four and
+        // landed in other cells of the slab; the parity tests caught it.
+        volatile slab_int_t *vw = wl;
         auto w = [&](const auto &a) {
 #pragma unroll
             for (int j = 0; j < 4; ++j)
 #pragma unroll
                 for (int r = 0; r < 16; ++r)
-                    wl[((r >> 2) * 8 + (lane >> 5) * 4 + (r & 3)) * 128 + j * 32 + (lane & 31)]
-                            = raw_bits(a[j][r]);
+                    vw[((r >> 2) * 8 + (lane >> 5) * 4 + (r & 3)) * 128 + j * 32 + (lane & 31)] = raw_bits(a[j][r]);
         };
         switch (s) {
             case 0: w(acc[0]); break;
@@ -614,14 +636,15 @@ struct layout32_t {
 // row 16i + 4*(lane/16) + r, column 16j + lane%16.
 struct layout16_t {
     template <class Acc>
-    static __device__ __forceinline__ void write_slab(const Acc &acc, int s, int *wl, int lane) {
+    static __device__ __forceinline__ void write_slab(const Acc &acc, int s, slab_int_t *wl, int lane) {
+        slab_int_t *vw = wl;
         auto w = [&](const auto &a0, const auto &a1) {
 #pragma unroll
             for (int j = 0; j < 8; ++j)
 #pragma unroll
                 for (int r = 0; r < 4; ++r) {
-                    wl[((lane >> 4) * 4 + r) * 128 + j * 16 + (lane & 15)] = raw_bits(a0[j][r]);
-                    wl[(16 + (lane >> 4) * 4 + r) * 128 + j * 16 + (lane & 15)] = raw_bits(a1[j][r]);
+                    vw[((lane >> 4) * 4 + r) * 128 + j * 16 + (lane & 15)] = raw_bits(a0[j][r]);
+                    vw[(16 + (lane >> 4) * 4 + r) * 128 + j * 16 + (lane & 15)] = raw_bits(a1[j][r]);
                 }
         };
         switch (s) {
@@ -640,8 +663,8 @@ template <class Layout, class PT, class Acc, class Conv>
 __device__ __forceinline__ void store_quadrant(const PT &P, char *smem, const Acc &acc,
         long b, long m_base, long n_base_wave, bool interior, const Conv &conv) {
     const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
-    int *wl = (int *)smem + wave * 4096;                    // 16 KB per wavefront
-    uint4 *stg = (uint4 *)(smem + 65536) + wave * 1024;     // 16 KB per wavefront
+    slab_int_t *wl = (slab_int_t *)smem + wave * 4096;      // 16 KB per wavefront
+    stage_u4_t *stg = (stage_u4_t *)(smem + 65536) + wave * 1024; // 16 KB per wavefront
     const long nbase = n_base_wave + (lane & 31) * 4;
     int nvalid = 0;
 #pragma unroll
@@ -685,7 +708,7 @@ __device__ __forceinline__ void store_quadrant(const PT &P, char *smem, const Ac
                     const int row = (it0 + k) * 2 + (lane >> 5);
                     m[k] = m_base + i * 32 + row;
                     ok[k] = m[k] < P.M;
-                    raw[k] = *(const v4i_t *)&wl[row * 128 + (lane & 31) * 4];
+                    raw[k] = *(const slab_v4i_t *)&wl[row * 128 + (lane & 31) * 4];
                     sv[k] = make_uint4(0, 0, 0, 0);
                 }
                 if (H.staged != STG_NONE) {
@@ -704,7 +727,7 @@ __device__ __forceinline__ void store_quadrant(const PT &P, char *smem, const Ac
         for (int it = 0; it < 16; ++it) {
             const int row = it * 2 + (lane >> 5);
             const long m = m_base + i * 32 + row;
-            const v4i_t raw = *(const v4i_t *)&wl[row * 128 + (lane & 31) * 4];
+            const v4i_t raw = *(const slab_v4i_t *)&wl[row * 128 + (lane & 31) * 4];
             uint4 sv = make_uint4(0, 0, 0, 0);
             if (H.staged != STG_NONE) sv = stg[it * 64 + lane];
             if (m < P.M && nvalid > 0) {
