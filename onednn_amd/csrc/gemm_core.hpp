@@ -213,16 +213,12 @@ __device__ __forceinline__ void main_loop(Acc &acc, char *smem, const char *a_ti
         Mma::load_a(f, 1, S, wm, lane, ctx, g);
 #pragma unroll
         for (int i = 0; i < ROWS; ++i) {
-#ifndef MI355_DBG_NO_DMA
             if (dma) {
 #pragma unroll
                 for (int d = 0; d < DPR; ++d) issue_part(g + NG - 1, nslot, i * DPR + d);
             }
-#endif
             if (i + 2 < ROWS) Mma::load_a(f, i + 2, S, wm, lane, ctx, g);
-#ifndef MI355_DBG_NO_MMA
             Mma::mma_row(acc, f, i, ctx, g);
-#endif
         }
         if (++slot == NG) slot = 0;
     }

@@ -141,20 +141,7 @@ __global__ void __launch_bounds__(NT) i8_gemm_kernel(const problem_t P_, const i
         }
     }
     const bool interior = m0 + BM <= P.M && n0 + BN <= P.N;
-#ifndef MI355_DBG_NO_EPI
     store_quadrant<layout16_t>(P, smem, acc, b, m0 + wm * 128, n0 + wn * 128, interior, cv);
-#else
-    {
-        int sacc = 0;
-#pragma unroll
-        for (int i = 0; i < 8; ++i)
-#pragma unroll
-            for (int j = 0; j < 8; ++j)
-#pragma unroll
-                for (int r = 0; r < 4; ++r) sacc += acc[i][j][r];
-        if (sacc == 123456789) ((int *)P.dst)[0] = cv.col_corr[0] + interior;
-    }
-#endif
 }
 
 // out[r] = sum_k (bytes[r][k] ^ flip) as signed bytes; one wave per row
