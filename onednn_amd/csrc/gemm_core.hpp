@@ -208,8 +208,10 @@ __device__ __forceinline__ void main_loop(Acc &acc, char *smem, const char *a_ti
         typename Mma::frag_t f;
         constexpr int ROWS = Mma::ROWS, COLS = Mma::COLS; // MFMA tiles of the quadrant
         constexpr int DPR = 8 / ROWS;                     // DMAs per row of MFMAs
-        Mma::load_b(f, S, wn, lane, ctx, g);
+        // A fragment 0 first: LDS reads return in order, so the first MFMA can go
+        // as soon as it and the first B fragment are in
         Mma::load_a(f, 0, S, wm, lane, ctx, g);
+        Mma::load_b(f, S, wn, lane, ctx, g);
         Mma::load_a(f, 1, S, wm, lane, ctx, g);
 #pragma unroll
         for (int i = 0; i < ROWS; ++i) {
