@@ -1,0 +1,346 @@
+#!/usr/bin/env python3
+"""A matmul driver with benchdnn's command-line vocabulary.
+
+    python tests/benchdnn_matmul.py --matmul [--mode=C|P|CP] --dt=u8:s8:f32 --wtag=ba \\
+        --bia-dt=f32 --attr-scales=src:common:0.25+wei:per_oc --attr-zero-points=src:common:1 \\
+        --attr-post-ops=relu+add:f32 256x1024:1024x1024
+
+What it mirrors of the reference's harness (tests/benchdnn/matmul/matmul.cpp,
+doc/knobs_attr.md): the knob syntax, comma lists expanding to the cartesian
+product of problems, data filled with small integers and power-of-two scales
+so that every product and partial sum is exact in f32 (fill_data :576-661,
+fill.cpp:161-199), correctness against a naive reference (here the CPU oracle
+under oracle/) and a perf mode that reports min / avg time of back-to-back
+executions.  The library is driven through its dnnl_* C API exactly like a
+user would: engine, memory descriptors, attributes, primitive descriptor,
+primitive, execute.
+
+Test infrastructure: the correctness mode needs the oracle, which the product
+package never imports.
+
+Supported knobs: --dt, --stag, --wtag, --dtag (ab | ba | any), --bia-dt,
+--attr-scales, --attr-zero-points, --attr-post-ops, --attr-fpmath, --impl,
+--mode, and 2-D problem descriptors MxK:KxN.  Policies: common, per_oc,
+per_ocic (with GxH groups), per_tensor (with GxH groups), per_dim_0, per_dim_1.
+"""
+import itertools
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+sys.path.insert(0, ROOT)
+
+import numpy as np  # noqa: E402
+
+from onednn_amd import cabi, dnnl  # noqa: E402
+from onednn_amd import dtypes as dtp  # noqa: E402
+from onednn_amd.problem import MatmulProblem, PostOp, QuantParam, storage_dtype, strides_for  # noqa: E402
+
+DT = {"f32": cabi.DT_F32, "bf16": cabi.DT_BF16, "f16": cabi.DT_F16, "s32": cabi.DT_S32, "s8": cabi.DT_S8,
+      "u8": cabi.DT_U8, "s4": cabi.DT_S4, "u4": cabi.DT_U4, "f8_e4m3": cabi.DT_F8_E4M3,
+      "f8_e5m2": cabi.DT_F8_E5M2, "f4_e2m1": cabi.DT_F4_E2M1, "e8m0": cabi.DT_E8M0}
+MASK_ROW, MASK_COL = 2, 4  # bit 0 is the batch dimension of the thin C ABI
+
+
+def encode(dt, values):
+    """Logical values (small integers, exactly representable) -> raw storage of `dt`."""
+    v = np.asarray(values, dtype=np.float32)
+    if dt == cabi.DT_F32:
+        return v
+    if dt == cabi.DT_BF16:
+        return dtp.f32_to_bf16(v)
+    if dt == cabi.DT_F16:
+        return v.astype(np.float16).view(np.uint16)
+    if dt == cabi.DT_S32:
+        return v.astype(np.int32)
+    if dt == cabi.DT_S8:
+        return v.astype(np.int8)
+    if dt == cabi.DT_U8:
+        return v.astype(np.uint8)
+    if dt in (cabi.DT_S4, cabi.DT_U4):
+        return dtp.pack_nibbles((v.astype(np.int32) & 0xF).astype(np.uint8))
+    if dt == cabi.DT_F8_E4M3:
+        return dtp.f32_to_e4m3(v)
+    if dt == cabi.DT_F8_E5M2:
+        # the fill values have at most two significant bits: e5m2 is the top byte of their f16 form
+        return (v.astype(np.float16).view(np.uint16) >> 8).astype(np.uint8)
+    if dt == cabi.DT_F4_E2M1:
+        return dtp.pack_nibbles(dtp.f32_to_e2m1_codes(v))
+    if dt == cabi.DT_E8M0:
+        return dtp.f32_to_e8m0(v)
+    raise ValueError(dt)
+
+
+def value_range(dt):
+    """Fill range per data type: small integers every type represents exactly."""
+    if dt in (cabi.DT_U8, cabi.DT_U4):
+        return 0, 8
+    if dt == cabi.DT_F4_E2M1:
+        return -2, 2
+    return -4, 4
+
+
+class Spec:
+    """One fully specified problem (one element of the cartesian product)."""
+
+    def __init__(self, **kw):
+        self.__dict__.update(kw)
+
+    def repro(self):
+        parts = ["--matmul", f"--dt={self.dt}", f"--stag={self.stag}", f"--wtag={self.wtag}", f"--dtag={self.dtag}"]
+        if self.bia_dt != "undef":
+            parts.append(f"--bia-dt={self.bia_dt}")
+        for knob in ("attr_scales", "attr_zero_points", "attr_post_ops", "attr_fpmath"):
+            if getattr(self, knob):
+                parts.append(f"--{knob.replace('_', '-')}={getattr(self, knob)}")
+        if self.impl:
+            parts.append(f"--impl={self.impl}")
+        parts.append(self.desc)
+        return " ".join(parts)
+
+
+def parse(argv):
+    """benchdnn-style arguments -> (mode, [Spec, ...])."""
+    knobs = {"dt": ["f32"], "stag": ["ab"], "wtag": ["ab"], "dtag": ["ab"], "bia_dt": ["undef"],
+             "attr_scales": [""], "attr_zero_points": [""], "attr_post_ops": [""], "attr_fpmath": [""],
+             "impl": [""]}
+    mode, specs = "C", []
+    for a in argv:
+        if a in ("--matmul", "--reset"):
+            continue
+        if a.startswith("--mode="):
+            mode = a.split("=", 1)[1].upper()
+            continue
+        if a.startswith("--"):
+            k, _, v = a[2:].partition("=")
+            k = k.replace("-", "_")
+            if k == "bia_mask":
+                if v not in ("2", ""):
+                    raise ValueError("only --bia_mask=2 (1 x N bias) is supported")
+                continue
+            if k not in knobs:
+                raise ValueError(f"unknown knob --{k}")
+            knobs[k] = v.split(",") if v else [""]
+            continue
+        for combo in itertools.product(*knobs.values()):
+            specs.append(Spec(desc=a, **dict(zip(knobs.keys(), combo))))
+    return mode, specs
+
+
+def _tag_strides(tag, rows, cols):
+    return strides_for("ab" if tag == "any" else tag, 1, rows, cols)
+
+
+def build_problem(sp, seed=7):
+    """Spec -> MatmulProblem with benchdnn-like data."""
+    lhs, rhs = sp.desc.split(":")
+    M, K = (int(x) for x in lhs.split("x"))
+    K2, N = (int(x) for x in rhs.split("x"))
+    if K != K2:
+        raise ValueError(f"inconsistent K in {sp.desc}")
+    dts = sp.dt.split(":")
+    if len(dts) == 1:
+        dts = dts * 3
+    sdt, wdt, ddt = (DT[x] for x in dts)
+    rng = np.random.default_rng(seed)
+
+    def ints(dt, shape):
+        lo, hi = value_range(dt)
+        return rng.integers(lo, hi + 1, size=shape).astype(np.float32)
+
+    wtag = sp.wtag
+    if wtag == "any":  # what the primitive descriptor resolves `any` weights to
+        mfma = (sdt in (cabi.DT_S8, cabi.DT_U8) and wdt in (cabi.DT_S8, cabi.DT_U8)) or (
+            sdt in (cabi.DT_F8_E4M3, cabi.DT_F8_E5M2) and wdt in (cabi.DT_F8_E4M3, cabi.DT_F8_E5M2)) or (
+            sdt == wdt == cabi.DT_F4_E2M1)
+        wtag = "ba" if mfma else "ab"
+    src_v, wei_v = ints(sdt, (M, K)), ints(wdt, (K, N))
+    src = encode(sdt, src_v if sp.stag != "ba" else src_v.T.copy())
+    wei = encode(wdt, wei_v if wtag != "ba" else wei_v.T.copy())
+    kw = dict(src_stride=_tag_strides(sp.stag, M, K), wei_stride=strides_for(wtag, 1, K, N),
+              dst_stride=_tag_strides(sp.dtag, M, N))
+    if sp.bia_dt != "undef":
+        kw["bias_dt"] = DT[sp.bia_dt]
+        kw["bias"] = encode(DT[sp.bia_dt], rng.integers(-8, 9, size=N))
+    dims = {"src": (M, K), "wei": (K, N), "dst": (M, N)}
+
+    def quant_entry(arg, policy, rest, is_scale):
+        value, dt, groups = None, (cabi.DT_F32 if is_scale else cabi.DT_S32), (1, 1)
+        for tok in rest:
+            if tok in DT:
+                dt = DT[tok]
+            elif "x" in tok and tok.replace("x", "").isdigit():
+                groups = tuple(int(x) for x in tok.split("x"))
+            elif tok:
+                value = float(tok)
+        r, c = dims[arg]
+        if policy == "common":
+            mask, shape = 0, (1,)
+        elif policy in ("per_oc", "per_dim_1"):
+            mask, shape = MASK_COL, (c,)
+        elif policy == "per_dim_0":
+            mask, shape = MASK_ROW, (r,)
+        elif policy in ("per_ocic", "per_tensor", "per_dim_01"):
+            mask, shape = MASK_ROW | MASK_COL, (r // groups[0], c // groups[1])
+        else:
+            raise ValueError(f"policy {policy}")
+        if value is not None and policy == "common":
+            vals = np.full(shape, value, np.float32)
+        elif is_scale:
+            vals = rng.choice(np.array([0.125, 0.25, 0.5], np.float32), size=shape)
+        else:
+            lo = 0 if dt in (cabi.DT_U8, cabi.DT_U4) else -2
+            vals = rng.integers(lo, 3, size=shape).astype(np.float32)
+        return QuantParam(dt, mask, encode(dt, vals), groups)
+
+    quant = {}
+    for knob, is_scale, suffix in ((sp.attr_scales, True, "scale"), (sp.attr_zero_points, False, "zp")):
+        for ent in filter(None, knob.split("+")):
+            arg, policy, *rest = ent.split(":")
+            quant[f"{arg}_{suffix}"] = quant_entry(arg, policy, rest, is_scale)
+    post_ops, dst_init = [], None
+    for ent in filter(None, sp.attr_post_ops.split("+")):
+        name, *rest = ent.split(":")
+        if name in cabi.ELTWISE:
+            alpha = float(rest[0]) if len(rest) > 0 else 0.0
+            beta = float(rest[1]) if len(rest) > 1 else 0.0
+            post_ops.append(PostOp(kind=cabi.PO_ELTWISE, alg=cabi.ELTWISE[name], alpha=alpha, beta=beta, scale=1.0))
+        elif name in cabi.BINARY:
+            bdt = DT[rest[0]] if rest else cabi.DT_F32
+            policy = rest[1] if len(rest) > 1 else "per_tensor"
+            shape, stride = {"per_tensor": ((M, N), (0, N, 1)), "per_oc": ((1, N), (0, 0, 1)),
+                             "common": ((1, 1), (0, 0, 0))}[policy]
+            post_ops.append(PostOp(kind=cabi.PO_BINARY, alg=cabi.BINARY[name], dt=bdt, stride=stride,
+                                   data=encode(bdt, ints(bdt, shape))))
+        elif name == "sum":
+            post_ops.append(PostOp(kind=cabi.PO_SUM, scale=float(rest[0]) if rest else 1.0))
+            dst_init = encode(ddt, ints(ddt, (M, N)))
+        else:
+            raise ValueError(f"post-op {name}")
+    apply_to_int, fpmath = False, 0
+    if sp.attr_fpmath:
+        mode, _, flag = sp.attr_fpmath.partition(":")
+        fpmath = {"strict": 0, "bf16": 1, "f16": 2, "any": 3}[mode]
+        apply_to_int = flag == "true"
+    impl = {"": cabi.IMPL_AUTO, "ref": cabi.IMPL_REF}.get(sp.impl, cabi.IMPL_AUTO)
+    return MatmulProblem(M=M, N=N, K=K, src_dt=sdt, wei_dt=wdt, dst_dt=ddt, src=src, wei=wei, quant=quant,
+                         post_ops=post_ops, apply_to_int=apply_to_int, fpmath_mode=fpmath, dst_init=dst_init,
+                         impl=impl, name=sp.desc, **kw)
+
+
+def api_objects(p, want_ref_impl=False):
+    """MatmulProblem -> dnnl engine, primitive and execute arguments (2-D, dense)."""
+    eng = dnnl.engine(dnnl.gpu, 0)
+    strm = dnnl.stream(eng)
+    src_md = dnnl.memory_desc([p.M, p.K], p.src_dt, strides=list(p.src_stride[1:]))
+    wei_md = dnnl.memory_desc([p.K, p.N], p.wei_dt, strides=list(p.wei_stride[1:]))
+    dst_md = dnnl.memory_desc([p.M, p.N], p.dst_dt, strides=list(p.dst_stride[1:]))
+    bias_md = dnnl.memory_desc([1, p.N], p.bias_dt, tag=dnnl.tag_ab) if p.bias is not None else None
+    attr = dnnl.primitive_attr()
+    args = {}
+    name_to = {"src": dnnl.ARG_SRC, "wei": dnnl.ARG_WEIGHTS, "dst": dnnl.ARG_DST}
+    for qname, q in p.quant.items():
+        which, kind = qname.split("_")
+        arg, mask2d = name_to[which], q.mask >> 1
+        groups = q.groups if q.groups != (1, 1) else ()
+        dims = {"src": (p.M, p.K), "wei": (p.K, p.N), "dst": (p.M, p.N)}[which]
+        qdims = [dims[0] // q.groups[0] if mask2d & 1 else 1, dims[1] // q.groups[1] if mask2d & 2 else 1]
+        if kind == "scale":
+            attr.set_scales(arg, mask2d, groups, q.dt)
+            flag = dnnl.ARG_ATTR_SCALES
+        else:
+            attr.set_zero_points(arg, mask2d, groups, q.dt)
+            flag = dnnl.ARG_ATTR_ZERO_POINTS
+        args[flag | arg] = dnnl.memory(dnnl.memory_desc(qdims, q.dt, tag=dnnl.tag_ab), eng, q.data)
+    if p.fpmath_mode or p.apply_to_int:
+        attr.set_fpmath_mode(p.fpmath_mode, p.apply_to_int)
+    po = dnnl.post_ops()
+    for i, op in enumerate(p.post_ops):
+        if op.kind == cabi.PO_ELTWISE:
+            po.append_eltwise(op.alg, op.alpha, op.beta)
+        elif op.kind == cabi.PO_BINARY:
+            bmd = dnnl.memory_desc([p.M if op.stride[1] else 1, p.N if op.stride[2] else 1], op.dt, tag=dnnl.tag_ab)
+            po.append_binary(op.alg, bmd)
+            args[dnnl.ARG_ATTR_MULTIPLE_POST_OP(i) | dnnl.ARG_SRC_1] = dnnl.memory(bmd, eng, op.data)
+        elif op.kind == cabi.PO_SUM:
+            po.append_sum(op.scale, op.zero_point, op.dt)
+    if p.post_ops:
+        attr.set_post_ops(po)
+    pd = dnnl.matmul_primitive_desc(eng, src_md, wei_md, dst_md, bias_md=bias_md, attr=attr)
+    if want_ref_impl:
+        while pd.impl_info_str() != "hip:ref:any":
+            if not pd.next_impl():
+                raise RuntimeError("no hip:ref:any implementation in the list")
+    prim = dnnl.matmul(pd)
+    args[dnnl.ARG_SRC] = dnnl.memory(src_md, eng, p.src)
+    args[dnnl.ARG_WEIGHTS] = dnnl.memory(wei_md, eng, p.wei)
+    dst = dnnl.memory(dst_md, eng, p.initial_dst())
+    args[dnnl.ARG_DST] = dst
+    if p.bias is not None:
+        args[dnnl.ARG_BIAS] = dnnl.memory(bias_md, eng, p.bias)
+    return pd, prim, strm, args, dst
+
+
+def run_spec(sp, mode="C", min_times=5, max_ms=300.0):
+    """Returns (status, impl, details): status PASSED / FAILED / SKIPPED (unimplemented)."""
+    p = build_problem(sp)
+    try:
+        pd, prim, strm, args, dst = api_objects(p, want_ref_impl=sp.impl == "ref")
+    except dnnl.error as e:
+        if e.status == dnnl.unimplemented:
+            return "SKIPPED", "", "unimplemented"
+        return "FAILED", "", f"primitive descriptor: {e}"
+    impl = pd.impl_info_str()
+    details = {}
+    if "C" in mode:
+        from oracle import binding as oracle
+        from tests.helpers import compare
+        oracle.load()
+        prim.execute(strm, args)
+        strm.wait()
+        got = dst.read(storage_dtype(p.dst_dt))
+        want, _, asum = oracle.run_oracle(p, want_ideal=True)
+        transcendental = any(op.kind == cabi.PO_ELTWISE and op.alg not in (
+            cabi.ELTWISE["relu"], cabi.ELTWISE["linear"], cabi.ELTWISE["clip"]) for op in p.post_ops)
+        nbad, msg = compare(p, got, want, abs_sum=asum, transcendental=transcendental)
+        details["errors"] = nbad
+        if nbad:
+            return "FAILED", impl, msg
+    if "P" in mode:
+        prim.execute(strm, args)
+        strm.wait()
+        times, t_all = [], time.perf_counter()
+        while len(times) < min_times or (time.perf_counter() - t_all) * 1e3 < max_ms:
+            t0 = time.perf_counter()
+            for _ in range(10):
+                prim.execute(strm, args)
+            strm.wait()
+            times.append((time.perf_counter() - t0) * 1e3 / 10)
+            if len(times) >= 1000:
+                break
+        details["min_ms"], details["avg_ms"] = min(times), sum(times) / len(times)
+        details["gops"] = 2.0 * p.M * p.N * p.K / (min(times) * 1e-3) / 1e9
+    return "PASSED", impl, details
+
+
+def main(argv):
+    mode, specs = parse(argv)
+    failed = 0
+    for i, sp in enumerate(specs):
+        t0 = time.perf_counter()
+        status, impl, det = run_spec(sp, mode)
+        ms = (time.perf_counter() - t0) * 1e3
+        if status == "FAILED":
+            failed += 1
+            print(f"{i}:FAILED ({det}) ({ms:.0f} ms) __REPRO: {sp.repro()}")
+            continue
+        print(f"{i}:{status} ({ms:.0f} ms) __REPRO: {sp.repro()}")
+        if status == "PASSED" and "P" in mode:
+            print(f"perf,gpu,{impl},{sp.repro()},{det['min_ms']:.4f},{det['avg_ms']:.4f},{det['gops']:.1f}")
+    print(f"tests:{len(specs)} passed:{len(specs) - failed} failed:{failed}")
+    return 1 if failed else 0
+
+
+if __name__ == "__main__":
+    sys.exit(main(sys.argv[1:]))

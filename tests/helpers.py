@@ -40,26 +40,38 @@ def assert_bit_exact(prob, got_raw, want_raw, what=""):
             f"got {g[first] if first else '?'} want {w[first] if first else '?'}")
 
 
-def assert_close(prob, got_raw, want_raw, *, abs_sum=None, transcendental=False, what="",
-                 extra_rel=0.0):
+def compare(prob, got_raw, want_raw, *, abs_sum=None, transcendental=False, extra_rel=0.0):
+    """The comparison ladder: returns (number of elements outside tolerance,
+    description of the first one).  Integer dst types compare exactly."""
     g = logical(prob, got_raw).astype(np.float64)
     w = logical(prob, want_raw).astype(np.float64)
-    eps = EPS[prob.dst_dt]
-    diff = np.abs(g - w)
-    rdiff = diff / np.maximum(np.abs(w), 1e-30)
-    ok = (g == w) | (np.isnan(g) & np.isnan(w))
-    ok |= (np.abs(w) <= 1e-5) & (diff < 2.0 ** -23)
-    trh = max(eps, 1e-5) + extra_rel
-    ok |= rdiff <= trh
-    if transcendental:
-        ok |= (diff <= max(eps, 2e-5)) | (rdiff <= max(eps, 8e-6))
-    if abs_sum is not None:
-        bound = prob.K * 2.0 ** -24 * np.asarray(abs_sum).reshape(g.shape)
-        # one ulp of the dst type on top of the accumulation bound
-        ok |= diff <= bound + eps * np.abs(w)
-    if not ok.all():
-        bad = np.argwhere(~ok)
-        i = tuple(bad[0])
-        raise AssertionError(
-            f"{prob.name} {what}: {len(bad)} of {g.size} outside tolerance; first at {i}: "
-            f"got {g[i]} want {w[i]} diff {diff[i]:.3e} rdiff {rdiff[i]:.3e}")
+    if prob.dst_dt in (cabi.DT_S32, cabi.DT_S8, cabi.DT_U8):
+        ok = g == w
+    else:
+        eps = EPS[prob.dst_dt]
+        diff = np.abs(g - w)
+        rdiff = diff / np.maximum(np.abs(w), 1e-30)
+        ok = (g == w) | (np.isnan(g) & np.isnan(w))
+        ok |= (np.abs(w) <= 1e-5) & (diff < 2.0 ** -23)
+        trh = max(eps, 1e-5) + extra_rel
+        ok |= rdiff <= trh
+        if transcendental:
+            ok |= (diff <= max(eps, 2e-5)) | (rdiff <= max(eps, 8e-6))
+        if abs_sum is not None:
+            bound = prob.K * 2.0 ** -24 * np.asarray(abs_sum).reshape(g.shape)
+            # one ulp of the dst type on top of the accumulation bound
+            ok |= diff <= bound + eps * np.abs(w)
+    if ok.all():
+        return 0, ""
+    bad = np.argwhere(~ok)
+    i = tuple(bad[0])
+    return len(bad), (f"{len(bad)} of {g.size} outside tolerance; first at {tuple(int(x) for x in i)}: "
+                      f"got {g[i]} want {w[i]} diff {abs(g[i] - w[i]):.3e}")
+
+
+def assert_close(prob, got_raw, want_raw, *, abs_sum=None, transcendental=False, what="",
+                 extra_rel=0.0):
+    nbad, msg = compare(prob, got_raw, want_raw, abs_sum=abs_sum, transcendental=transcendental,
+                        extra_rel=extra_rel)
+    if nbad:
+        raise AssertionError(f"{prob.name} {what}: {msg}")
