@@ -1,7 +1,9 @@
 // LDS-tiled MFMA GEMM core shared by the int8, fp8 and MXFP4 kernel families.
 //
-// Shape of the computation (one workgroup = 4 wavefronts = one 256x256 dst
-// tile, each wavefront a 128x128 quadrant held in 256 accumulator registers):
+// Shape of the computation: one workgroup = one 256x256 dst tile, split over
+// either 4 wavefronts (a 128x128 part each, 256 accumulator registers, one
+// wavefront per SIMD) or 8 wavefronts (128x64 each, 128 accumulator registers,
+// two wavefronts per SIMD that fill each other's LDS and barrier waits):
 //
 //   HBM/L2 --global_load_lds_dwordx4--> LDS ring of NSTAGE stages
 //       stage = A[256 rows][64 B of K] + B^T[256 rows][64 B of K]  (32 KB)
@@ -38,11 +40,37 @@ typedef float v16f __attribute__((ext_vector_type(16)));
 
 namespace gemm {
 
-constexpr int BM = 256, BN = 256;
+constexpr int BM = 256;               // rows of a workgroup's dst tile
 constexpr int BKB = 64;               // bytes of K per row per stage
-constexpr int NT = 256;               // threads per workgroup
-constexpr int STAGE_BYTES = (BM + BN) * BKB; // 32 KB
 constexpr int B_OFF = BM * BKB;       // B^T tile offset inside a stage
+
+// Tile geometry: a workgroup of NW wavefronts computes a 256 x BN dst tile, two
+// wavefronts along m (128 rows each) and NW/2 along n.
+//   geo_t<4, 256>  128x128 per wavefront (256 accumulators), one wavefront per
+//                  SIMD: the fewest LDS bytes per MFMA (64 KB of fragment reads
+//                  per K step and CU), nothing to hide LDS latency behind
+//   geo_t<8, 256>  128x64 per wavefront, two wavefronts per SIMD in two groups
+//                  that alternate between reading and multiplying (96 KB of
+//                  fragment reads per K step)
+// Each kernel family uses the one measured faster on its headline shape.  (A
+// 256x128 tile with two independent workgroups per CU, geo_t<4, 128>, also runs
+// through this code; it measured 10-30 % slower than either and is not built.)
+template <int NW_, int BN_>
+struct geo_t {
+    static constexpr int NW = NW_, NT = 64 * NW_, BN = BN_;
+    static constexpr int WN = NW_ / 2;        // wavefronts along n
+    static constexpr int WCOLS = BN_ / WN;    // columns of a wavefront's part
+    static constexpr int DPA = (BM / 16) / NW_;  // A DMAs per stage and wavefront
+    static constexpr int DPB = (BN_ / 16) / NW_; // B^T DMAs per stage and wavefront
+    static constexpr int DPS = DPA + DPB;
+    static constexpr int STAGE_BYTES = (BM + BN_) * BKB;
+    static constexpr int NSTAGE = BN_ == 256 ? 4 : 3; // ring depth: 128 KB or 72 KB
+    static constexpr int WG_PER_CU = BN_ == 256 ? 1 : 2;
+    // the epilogue needs the ring's memory: accumulator slabs + operand staging
+    static_assert(NSTAGE * STAGE_BYTES >= 2 * NW_ * 32 * WCOLS * 4, "epilogue LDS");
+    __device__ static __forceinline__ int wm(int wave) { return wave / WN; }
+    __device__ static __forceinline__ int wn(int wave) { return wave % WN; }
+};
 
 // chunk swizzle: conflict-free for ds_read_b128 over 8 or 16 consecutive rows
 __device__ __forceinline__ int swz_f(int row) { return ((row >> 1) & 3) ^ ((row >> 3) & 1); }
@@ -89,6 +117,7 @@ struct tile_pos_t {
 // (8 of them, each with a private L2); give every XCD one contiguous run of
 // tiles, walked in bands of GM tile rows so that concurrently resident tiles
 // share A rows and B columns in that L2.
+template <class G>
 __device__ __forceinline__ tile_pos_t tile_position(int tiles_m, int tiles_n) {
     const int nwg = gridDim.x, id = blockIdx.x;
     const int per = nwg / 8;
@@ -99,41 +128,164 @@ __device__ __forceinline__ tile_pos_t tile_position(int tiles_m, int tiles_n) {
     const int in_band = tile - band * GM * tiles_n;
     tile_pos_t p;
     p.m0 = (long)(band * GM + in_band % band_rows) * BM;
-    p.n0 = (long)(in_band / band_rows) * BN;
+    p.n0 = (long)(in_band / band_rows) * G::BN;
     return p;
 }
 
-// Per-thread DMA plan: wave w owns tile rows [64w, 64w+64) of A and of B^T,
-// four DMAs each per stage.
+// Per-thread DMA plan: wave w owns DPA blocks of 16 tile rows of A and DPB of
+// B^T, one DMA each per stage.
+template <int DPA, int DPB>
 struct dma_plan_t {
-    unsigned voff_a[4], voff_b[4]; // byte offsets from the scalar tile base
-    unsigned lds_a[4], lds_b[4];   // LDS byte offsets inside a stage
+    unsigned voff_a[DPA], voff_b[DPB]; // byte offsets from the scalar tile base
+    unsigned lds_a[DPA], lds_b[DPB];   // LDS byte offsets inside a stage
 };
 
-__device__ __forceinline__ dma_plan_t make_dma_plan(int wave, int lane, long rows_a_left,
+template <int DPA, int DPB>
+__device__ __forceinline__ dma_plan_t<DPA, DPB> make_dma_plan(int wave, int lane, long rows_a_left,
         long rows_b_left, long lda, long ldb) {
-    dma_plan_t p;
+    dma_plan_t<DPA, DPB> p;
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-        const int row = (wave * 4 + i) * 16 + (lane >> 2);
+    for (int i = 0; i < DPA; ++i) {
+        const int row = (wave * DPA + i) * 16 + (lane >> 2);
         const int chunk = (lane & 3) ^ swz_f(row);
-        long ra = row, rb = row;
+        long ra = row;
         if (ra > rows_a_left - 1) ra = rows_a_left - 1;
-        if (rb > rows_b_left - 1) rb = rows_b_left - 1;
         p.voff_a[i] = (unsigned)(ra * lda + chunk * 16);
+        p.lds_a[i] = (unsigned)((wave * DPA + i) * 1024);
+    }
+#pragma unroll
+    for (int i = 0; i < DPB; ++i) {
+        const int row = (wave * DPB + i) * 16 + (lane >> 2);
+        const int chunk = (lane & 3) ^ swz_f(row);
+        long rb = row;
+        if (rb > rows_b_left - 1) rb = rows_b_left - 1;
         p.voff_b[i] = (unsigned)(rb * ldb + chunk * 16);
-        p.lds_a[i] = (unsigned)((wave * 4 + i) * 1024);
-        p.lds_b[i] = (unsigned)(B_OFF + (wave * 4 + i) * 1024);
+        p.lds_b[i] = (unsigned)(B_OFF + (wave * DPB + i) * 1024);
     }
     return p;
 }
 
-__device__ __forceinline__ void issue_stage(const dma_plan_t &p, const char *a_base,
-        const char *b_base, unsigned lds_stage) {
+// s_waitcnt lgkmcnt(0) only
+__device__ __forceinline__ void wait_lds_reads() {
+    __builtin_amdgcn_s_waitcnt(0xC07F);
+}
+
+// workgroup barrier that neither memory accesses nor MFMAs are scheduled across
+__device__ __forceinline__ void phase_barrier() {
+    asm volatile("" ::: "memory");
+    __builtin_amdgcn_sched_barrier(0);
+    __builtin_amdgcn_s_barrier();
+    __builtin_amdgcn_sched_barrier(0);
+    asm volatile("" ::: "memory");
+}
+
+// Main loop for eight wavefronts, two per SIMD, in two groups of four that run
+// half a K step apart.  Both groups meet at one workgroup barrier per step; in
+// the interval after barrier g
+//   group 0:  reads stage g from LDS, then its MFMAs of stage g
+//   group 1:  its MFMAs of stage g-1 (fragments read in the previous interval),
+//             then reads stage g
+// so on every SIMD one wavefront has MFMAs to issue while the other one waits
+// for LDS, with every wavefront's instruction stream in plain program order:
+// nothing depends on how the compiler interleaves reads with MFMAs.  Both
+// groups read stage g in the same interval, so one barrier per step covers
+// both conditions: every wavefront waits for its own DMAs of stage g before
+// barrier g (then all of stage g is in LDS), and has its reads of stage g-1
+// back before it (then that slot may be overwritten by the DMAs of stage
+// g+NG-1, which are issued after the barrier).  Group 1 runs one more
+// iteration for its last MFMAs.
+template <int NSTAGE, int KSTEP, class Mma, class Acc, class Ctx>
+__device__ __forceinline__ void main_loop_two_groups(Acc &acc, char *smem, const char *a_tile,
+        const char *b_tile, long lda, long ldb, long rows_a_left, long rows_b_left, int ngroups,
+        const Ctx &ctx) {
+    using G = typename Mma::G;
+    static_assert(G::NW == 8, "two groups of four wavefronts");
+    constexpr int NG = NSTAGE / KSTEP;
+    constexpr int STAGE_BYTES = G::STAGE_BYTES, GROUP_BYTES = KSTEP * STAGE_BYTES;
+    constexpr int DPA = G::DPA, DPB = G::DPB, DPS = G::DPS;
+    constexpr int GROUP_DMAS = KSTEP * DPS + Mma::EXTRA_DMAS;
+    static_assert(NSTAGE % KSTEP == 0 && NG >= 3 && NG <= 5, "ring depth");
+    static_assert((NG - 2) * GROUP_DMAS < 64, "vmcnt range");
+    const int t = threadIdx.x, lane = t & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(t >> 6);
+    const int wm = G::wm(wave), wn = G::wn(wave);
+    const bool late = wave >= 4; // group 1
+    const unsigned lds0 = (unsigned)(size_t)(__attribute__((address_space(3))) char *)smem;
+    const dma_plan_t<DPA, DPB> plan = make_dma_plan<DPA, DPB>(wave, lane, rows_a_left, rows_b_left, lda, ldb);
+
+    auto issue_part = [&](int g, int slot, int i) __attribute__((always_inline)) {
 #pragma unroll
-    for (int i = 0; i < 4; ++i) dma16(a_base, p.voff_a[i], lds_stage + p.lds_a[i]);
+        for (int k = 0; k < KSTEP; ++k) {
+            const long koff = ((long)g * KSTEP + k) * BKB;
+            const unsigned lds_stage = lds0 + slot * GROUP_BYTES + k * STAGE_BYTES;
+            if (i < DPA) dma16(a_tile + koff, plan.voff_a[i], lds_stage + plan.lds_a[i]);
+            else dma16(b_tile + koff, plan.voff_b[i - DPA], lds_stage + plan.lds_b[i - DPA]);
+        }
+        if (i == DPS - 1) Mma::issue_extra(ctx, g, slot, wave, lane);
+    };
+    // the MFMAs of one stage with the DMAs of stage gd spread between the rows:
+    // a DMA instruction can wait tens of cycles for the address unit, which
+    // passes unnoticed behind a row of MFMAs
+    // Past the last stage the DMAs are issued all the same, clamped to the last
+    // stage and into a slot nobody reads again: the MFMA sequence stays one
+    // basic block (conditional blocks between the rows make the register
+    // allocator spill accumulators), and every stage is followed by the same
+    // number of loads, so one outstanding-load count fits every iteration.
+    auto mma_stage = [&](const typename Mma::frag_t &f, int gm, int gd, int dslot) __attribute__((always_inline)) {
+        const int gdc = gd < ngroups ? gd : ngroups - 1;
 #pragma unroll
-    for (int i = 0; i < 4; ++i) dma16(b_base, p.voff_b[i], lds_stage + p.lds_b[i]);
+        for (int i = 0; i < Mma::ROWS; ++i) {
+            Mma::mma_row(acc, f, i, ctx, gm);
+#pragma unroll
+            for (int d = 0; d < DPS; ++d)
+                if (d * Mma::ROWS / DPS == i) issue_part(gdc, dslot, d);
+            __builtin_amdgcn_sched_barrier(0); // or the DMAs all move to the front
+        }
+    };
+
+#pragma unroll
+    for (int s = 0; s < NG - 1; ++s) {
+        const int sc = s < ngroups ? s : ngroups - 1;
+#pragma unroll
+        for (int i = 0; i < DPS; ++i) issue_part(sc, s, i);
+    }
+
+    int slot = 0;
+    // Group 1 carries the fragments from one iteration to the next; they start
+    // as zeros, so that its first iteration, which has no stage to multiply
+    // yet, adds zero products instead of branching around the MFMAs (one MFMA
+    // sequence on every path keeps the accumulators where they are).
+    typename Mma::frag_t f = {};
+    const int niter = ngroups + (late ? 1 : 0);
+    auto read_stage = [&](int g) __attribute__((always_inline)) {
+        unsigned S[KSTEP];
+#pragma unroll
+        for (int k = 0; k < KSTEP; ++k) S[k] = lds0 + slot * GROUP_BYTES + k * STAGE_BYTES;
+        Mma::load_a(f, 0, S, wm, lane, ctx, g);
+        Mma::load_b(f, S, wn, lane, ctx, g);
+#pragma unroll
+        for (int i = 1; i < Mma::ROWS; ++i) Mma::load_a(f, i, S, wm, lane, ctx, g);
+    };
+#pragma nounroll
+    for (int g = 0; g < niter; ++g) {
+        // own DMAs of stage g landed; those of NG-2 later stages may stay in flight
+        wait_vmcnt<(NG - 2) * GROUP_DMAS>();
+        if (late) wait_lds_reads();
+        phase_barrier();
+        int nslot = slot + NG - 1; // the slot stage g-1 used: free after this barrier
+        if (nslot >= NG) nslot -= NG;
+        if (!late) read_stage(g);
+        __builtin_amdgcn_sched_barrier(0);
+        mma_stage(f, g, g + NG - 1, nslot); // group 0: stage g; group 1: stage g-1
+        __builtin_amdgcn_sched_barrier(0);
+        if (late && g < ngroups) read_stage(g);
+        if (++slot == NG) slot = 0;
+    }
+    if (!late) phase_barrier(); // the barrier of group 1's last iteration
+    // every DMA has landed (the clamped ones included) before the ring's memory
+    // is used for something else
+    wait_vmcnt<0>();
+    phase_barrier();
 }
 
 // Main loop.  The ring holds NSTAGE stages; one iteration consumes KSTEP of
@@ -143,8 +295,8 @@ __device__ __forceinline__ void issue_stage(const dma_plan_t &p, const char *a_b
 //   s_barrier             everybody's did, and everybody finished group g-1
 //   DMA group g+NG-1      into the slots group g-1 used
 //   ds_read + MFMA over group g
-// `Mma` supplies frag_t, load_b(frag, S, wn, lane, ctx, g) for the 8 B^T
-// fragments, load_a(frag, i, S, wm, lane, ctx, g) for A fragment i (S[k] is the
+// `Mma` supplies the geometry G = the tile geometry, frag_t, load_b(frag, S, wn, lane,
+// ctx, g) for the B^T fragments, load_a(frag, i, S, wm, lane, ctx, g) for A fragment i (S[k] is the
 // LDS byte address of the k-th stage of the group), mma_row(acc, frag, i, ctx, g)
 // for the COLS MFMAs of A fragment i (ROWS x COLS MFMA tiles per quadrant),
 // and A_READS / B_READS = LDS read instructions per fragment.
@@ -153,27 +305,34 @@ template <int NSTAGE, int KSTEP, class Mma, class Acc, class Ctx>
 __device__ __forceinline__ void main_loop(Acc &acc, char *smem, const char *a_tile,
         const char *b_tile, long lda, long ldb, long rows_a_left, long rows_b_left, int ngroups,
         const Ctx &ctx) {
+    using G = typename Mma::G;
     constexpr int NG = NSTAGE / KSTEP;           // groups in the ring
-    constexpr int GROUP_BYTES = KSTEP * STAGE_BYTES;
-    constexpr int GROUP_DMAS = KSTEP * 8 + Mma::EXTRA_DMAS;
+    constexpr int STAGE_BYTES = G::STAGE_BYTES, GROUP_BYTES = KSTEP * STAGE_BYTES;
+    if constexpr (G::NW == 8) {
+        main_loop_two_groups<NSTAGE, KSTEP, Mma>(acc, smem, a_tile, b_tile, lda, ldb, rows_a_left,
+                rows_b_left, ngroups, ctx);
+        return;
+    }
+    constexpr int DPA = G::DPA, DPB = G::DPB, DPS = G::DPS;
+    constexpr int GROUP_DMAS = KSTEP * DPS + Mma::EXTRA_DMAS;
     static_assert(NSTAGE % KSTEP == 0 && NG >= 2 && NG <= 5, "ring depth");
     static_assert((NG - 2) * GROUP_DMAS < 64, "vmcnt range");
     const int t = threadIdx.x, lane = t & 63;
     const int wave = __builtin_amdgcn_readfirstlane(t >> 6);
-    const int wm = wave >> 1, wn = wave & 1;
+    const int wm = G::wm(wave), wn = G::wn(wave);
     const unsigned lds0 = (unsigned)(size_t)(__attribute__((address_space(3))) char *)smem;
-    const dma_plan_t plan = make_dma_plan(wave, lane, rows_a_left, rows_b_left, lda, ldb);
+    const dma_plan_t<DPA, DPB> plan = make_dma_plan<DPA, DPB>(wave, lane, rows_a_left, rows_b_left, lda, ldb);
 
-    // DMA number i (0..7) of every stage of group g: A row blocks first, then B^T
+    // DMA number i (0..DPS-1) of every stage of group g: A row blocks first, then B^T
     auto issue_part = [&](int g, int slot, int i) __attribute__((always_inline)) {
 #pragma unroll
         for (int k = 0; k < KSTEP; ++k) {
             const long koff = ((long)g * KSTEP + k) * BKB;
             const unsigned lds_stage = lds0 + slot * GROUP_BYTES + k * STAGE_BYTES;
-            if (i < 4) dma16(a_tile + koff, plan.voff_a[i], lds_stage + plan.lds_a[i]);
-            else dma16(b_tile + koff, plan.voff_b[i - 4], lds_stage + plan.lds_b[i - 4]);
+            if (i < DPA) dma16(a_tile + koff, plan.voff_a[i], lds_stage + plan.lds_a[i]);
+            else dma16(b_tile + koff, plan.voff_b[i - DPA], lds_stage + plan.lds_b[i - DPA]);
         }
-        if (i == 7) Mma::issue_extra(ctx, g, slot, wave, lane);
+        if (i == DPS - 1) Mma::issue_extra(ctx, g, slot, wave, lane);
     };
 
     // prologue: groups 0 .. NG-2 in flight
@@ -181,7 +340,7 @@ __device__ __forceinline__ void main_loop(Acc &acc, char *smem, const char *a_ti
     for (int s = 0; s < NG - 1; ++s)
         if (s < ngroups) {
 #pragma unroll
-            for (int i = 0; i < 8; ++i) issue_part(s, s, i);
+            for (int i = 0; i < DPS; ++i) issue_part(s, s, i);
         }
 
     int slot = 0;
@@ -207,7 +366,6 @@ __device__ __forceinline__ void main_loop(Acc &acc, char *smem, const char *a_ti
         const bool dma = g + NG - 1 < ngroups;
         typename Mma::frag_t f;
         constexpr int ROWS = Mma::ROWS, COLS = Mma::COLS; // MFMA tiles of the quadrant
-        constexpr int DPR = 8 / ROWS;                     // DMAs per row of MFMAs
         // A fragment 0 first: LDS reads return in order, so the first MFMA can go
         // as soon as it and the first B fragment are in
         Mma::load_a(f, 0, S, wm, lane, ctx, g);
@@ -217,7 +375,8 @@ __device__ __forceinline__ void main_loop(Acc &acc, char *smem, const char *a_ti
         for (int i = 0; i < ROWS; ++i) {
             if (dma) {
 #pragma unroll
-                for (int d = 0; d < DPR; ++d) issue_part(g + NG - 1, nslot, i * DPR + d);
+                for (int d = 0; d < DPS; ++d) // spread evenly over the rows
+                    if (d * ROWS / DPS == i) issue_part(g + NG - 1, nslot, d);
             }
             if (i + 2 < ROWS) Mma::load_a(f, i + 2, S, wm, lane, ctx, g);
             Mma::mma_row(acc, f, i, ctx, g);

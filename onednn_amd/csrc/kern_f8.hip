@@ -24,8 +24,9 @@ namespace mi355 {
 namespace {
 
 using namespace gemm;
-constexpr int NSTAGE = 4; // 4 x 32 KB ring, one stage (K = 64) per step
 constexpr int KSTEP = 1;
+using f8_geo_t = geo_t<8, 256>;
+constexpr int NSTAGE = f8_geo_t::NSTAGE; // one stage (K = 64) per step
 
 struct f8_extra_t {
     const char *bt; // weights as [N][K] bytes, K contiguous
@@ -36,13 +37,14 @@ struct f8_extra_t {
 struct f8_ctx_t {};
 
 // cbsz / blgp operand format codes of the f8f6f4 MFMA: 0 = e4m3, 1 = e5m2
-template <int FMT_A, int FMT_B>
+template <int FMT_A, int FMT_B, class G_>
 struct f8_mma_t {
+    using G = G_;
     static constexpr int EXTRA_DMAS = 0;
     __device__ static __forceinline__ void issue_extra(const f8_ctx_t &, int, int, int, int) {}
-    static constexpr int ROWS = 4, COLS = 4, A_READS = 2, B_READS = 2;
+    static constexpr int ROWS = 4, COLS = G::WCOLS / 32, A_READS = 2, B_READS = 2;
     struct frag_t {
-        v8i a[4], b[4];
+        v8i a[ROWS], b[COLS];
     };
     // lane l supplies row l%32 and K bytes 32*(l/32) .. +32 of the stage
     __device__ static __forceinline__ v8i read32(unsigned T, int row, int c0) {
@@ -53,17 +55,17 @@ struct f8_mma_t {
             const f8_ctx_t &, int) {
         const int frow = lane & 31, h = lane >> 5;
 #pragma unroll
-        for (int j = 0; j < 4; ++j) f.b[j] = read32(S[0] + B_OFF, wn * 128 + j * 32 + frow, h * 2);
+        for (int j = 0; j < COLS; ++j) f.b[j] = read32(S[0] + B_OFF, wn * G::WCOLS + j * 32 + frow, h * 2);
     }
     __device__ static __forceinline__ void load_a(frag_t &f, int i, const unsigned (&S)[1], int wm, int lane,
             const f8_ctx_t &, int) {
         const int frow = lane & 31, h = lane >> 5;
         f.a[i] = read32(S[0], wm * 128 + i * 32 + frow, h * 2);
     }
-    __device__ static __forceinline__ void mma_row(v16f (&acc)[4][4], const frag_t &f, int i, const f8_ctx_t &,
-            int) {
+    __device__ static __forceinline__ void mma_row(v16f (&acc)[ROWS][COLS], const frag_t &f, int i,
+            const f8_ctx_t &, int) {
 #pragma unroll
-        for (int j = 0; j < 4; ++j)
+        for (int j = 0; j < COLS; ++j)
             acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(
                     f.a[i], f.b[j], acc[i][j], FMT_A, FMT_B, 0, 0, 0, 0);
     }
@@ -90,29 +92,30 @@ struct f8_conv_t {
 
 extern __shared__ __attribute__((aligned(16))) char f8_smem[];
 
-template <int FMT_A, int FMT_B>
-__global__ void __launch_bounds__(NT) f8_gemm_kernel(const problem_t P_, const f8_extra_t X) {
+template <int FMT_A, int FMT_B, class G>
+__global__ void __launch_bounds__(G::NT) __attribute__((amdgpu_waves_per_eu(G::NW * G::WG_PER_CU / 4))) f8_gemm_kernel(const problem_t P_, const f8_extra_t X) {
+    using Mma = f8_mma_t<FMT_A, FMT_B, G>;
     const auto &P = MI355_KERNARG_PROBLEM();
     char *smem = f8_smem;
     const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
-    const int wm = wave >> 1, wn = wave & 1;
+    const int wm = G::wm(wave), wn = G::wn(wave);
     const long b = blockIdx.z;
-    const tile_pos_t tp = tile_position(X.tiles_m, X.tiles_n);
+    const tile_pos_t tp = tile_position<G>(X.tiles_m, X.tiles_n);
     const long m0 = tp.m0, n0 = tp.n0;
 
     const long lda = P.ss[1];
     const char *A = (const char *)P.src + (P.ss[0] ? b * P.ss[0] : 0) + m0 * lda;
     const char *Bt = X.bt + b * X.bt_bstride + n0 * X.ldb;
 
-    v16f acc[4][4];
+    v16f acc[Mma::ROWS][Mma::COLS];
 #pragma unroll
-    for (int i = 0; i < 4; ++i)
+    for (int i = 0; i < Mma::ROWS; ++i)
 #pragma unroll
-        for (int j = 0; j < 4; ++j)
+        for (int j = 0; j < Mma::COLS; ++j)
 #pragma unroll
             for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
 
-    main_loop<NSTAGE, KSTEP, f8_mma_t<FMT_A, FMT_B>>(acc, smem, A, Bt, lda, X.ldb, P.M - m0,
+    main_loop<NSTAGE, KSTEP, Mma>(acc, smem, A, Bt, lda, X.ldb, P.M - m0,
             P.N - n0, (int)(P.K / (BKB * KSTEP)), f8_ctx_t {});
 
     const long bs = P.ss[0] ? b : 0, bw = P.ws[0] ? b : 0;
@@ -129,7 +132,7 @@ __global__ void __launch_bounds__(NT) f8_gemm_kernel(const problem_t P_, const f
         else
             cv.ssc_common = load_float(P.src_scale.dt, P.src_scale.p, (P.src_scale.mask & 1) ? bs : 0);
     }
-    const long nbase = n0 + wn * 128 + (lane & 31) * 4;
+    const long nbase = n0 + wn * G::WCOLS + (lane % (G::WCOLS / 4)) * 4;
 #pragma unroll
     for (int e = 0; e < 4; ++e) {
         cv.wsc[e] = 1.f;
@@ -137,8 +140,8 @@ __global__ void __launch_bounds__(NT) f8_gemm_kernel(const problem_t P_, const f
             cv.wsc[e] = load_float(P.wei_scale.dt, P.wei_scale.p,
                     quant_off(P.wei_scale, bw, 0, nbase + e, P.K, P.N));
     }
-    const bool interior = m0 + BM <= P.M && n0 + BN <= P.N;
-    store_quadrant<layout32_t>(P, smem, acc, b, m0 + wm * 128, n0 + wn * 128, interior, cv);
+    const bool interior = m0 + BM <= P.M && n0 + G::BN <= P.N;
+    store_quadrant<layout32_t, G::WCOLS, G::NW>(P, smem, acc, b, m0 + wm * 128, n0 + wn * G::WCOLS, interior, cv);
 }
 
 struct f8_plan_t {
@@ -202,9 +205,9 @@ int f8_launch(const mi355_matmul_desc_t &d, const problem_t &P, void *scratch, h
         X.bt_bstride = d.wei_stride[0];
     }
     X.tiles_m = (int)((d.M + BM - 1) / BM);
-    X.tiles_n = (int)((d.N + BN - 1) / BN);
+    X.tiles_n = (int)((d.N + f8_geo_t::BN - 1) / f8_geo_t::BN);
     dim3 grid((unsigned)(X.tiles_m * X.tiles_n), 1, (unsigned)d.batch);
-    constexpr int smem_bytes = NSTAGE * STAGE_BYTES;
+    constexpr int smem_bytes = NSTAGE * f8_geo_t::STAGE_BYTES;
     auto go = [&](auto kern) {
         static bool attr_done = false; // per instantiation
         if (!attr_done) {
@@ -215,14 +218,14 @@ int f8_launch(const mi355_matmul_desc_t &d, const problem_t &P, void *scratch, h
             }
             attr_done = true;
         }
-        hipLaunchKernelGGL(kern, grid, dim3(NT), smem_bytes, stream, P, X);
+        hipLaunchKernelGGL(kern, grid, dim3(f8_geo_t::NT), smem_bytes, stream, P, X);
         return hipGetLastError() == hipSuccess ? MI355_SUCCESS : MI355_RUNTIME_ERROR;
     };
     const int fa = d.src_dt == MI355_DT_F8_E5M2, fb = d.wei_dt == MI355_DT_F8_E5M2;
-    if (fa && fb) return go(f8_gemm_kernel<1, 1>);
-    if (fa) return go(f8_gemm_kernel<1, 0>);
-    if (fb) return go(f8_gemm_kernel<0, 1>);
-    return go(f8_gemm_kernel<0, 0>);
+    if (fa && fb) return go(f8_gemm_kernel<1, 1, f8_geo_t>);
+    if (fa) return go(f8_gemm_kernel<1, 0, f8_geo_t>);
+    if (fb) return go(f8_gemm_kernel<0, 1, f8_geo_t>);
+    return go(f8_gemm_kernel<0, 0, f8_geo_t>);
 }
 
 } // namespace mi355

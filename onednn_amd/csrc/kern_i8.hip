@@ -20,7 +20,8 @@ namespace {
 
 using namespace gemm;
 constexpr int BK = BKB;       // int8: one byte per K element
-constexpr int NSTAGE = 4;     // 4 x 32 KB LDS ring
+using i8_geo_t = geo_t<8, 256>;
+constexpr int NSTAGE = i8_geo_t::NSTAGE;
 
 struct i8_extra_t {
     const int8_t *bt; // weights as [N][K] bytes, K contiguous
@@ -37,30 +38,32 @@ struct i8_ctx_t {};
 // one instruction consumes the whole 64-byte K extent of a stage for a 16x16
 // tile.  (Measured on MI355X: this shape sustains ~4.0 POPS, the 32x32x32
 // shape ~3.0 POPS.)
-template <bool SRC_U8, bool WEI_U8>
+template <bool SRC_U8, bool WEI_U8, class G_>
 struct i8_mma_t {
+    using G = G_;
     static constexpr int EXTRA_DMAS = 0;
     __device__ static __forceinline__ void issue_extra(const i8_ctx_t &, int, int, int, int) {}
-    static constexpr int ROWS = 8, COLS = 8, A_READS = 1, B_READS = 1;
+    static constexpr int ROWS = 8, COLS = G::WCOLS / 16, A_READS = 1, B_READS = 1;
     struct frag_t {
-        v4i a[8], b[8];
+        v4i a[ROWS], b[COLS];
     };
     __device__ static __forceinline__ void load_b(frag_t &f, const unsigned (&S)[1], int wn, int lane,
             const i8_ctx_t &, int) {
         const int frow = lane & 15, fch = lane >> 4;
 #pragma unroll
-        for (int j = 0; j < 8; ++j) f.b[j] = lds_read16(S[0] + B_OFF + swz(wn * 128 + j * 16 + frow, fch));
+        for (int j = 0; j < COLS; ++j)
+            f.b[j] = lds_read16(S[0] + B_OFF + swz(wn * G::WCOLS + j * 16 + frow, fch));
     }
     __device__ static __forceinline__ void load_a(frag_t &f, int i, const unsigned (&S)[1], int wm, int lane,
             const i8_ctx_t &, int) {
         const int frow = lane & 15, fch = lane >> 4;
         f.a[i] = lds_read16(S[0] + swz(wm * 128 + i * 16 + frow, fch));
     }
-    __device__ static __forceinline__ void mma_row(v4i (&acc)[8][8], const frag_t &f, int i, const i8_ctx_t &,
-            int) {
+    __device__ static __forceinline__ void mma_row(v4i (&acc)[ROWS][COLS], const frag_t &f, int i,
+            const i8_ctx_t &, int) {
         const v4i a = SRC_U8 ? (f.a[i] ^ (int)0x80808080) : f.a[i];
 #pragma unroll
-        for (int j = 0; j < 8; ++j) {
+        for (int j = 0; j < COLS; ++j) {
             const v4i b = WEI_U8 ? (f.b[j] ^ (int)0x80808080) : f.b[j];
             acc[i][j] = __builtin_amdgcn_mfma_i32_16x16x64_i8(a, b, acc[i][j], 0, 0, 0);
         }
@@ -88,29 +91,30 @@ struct i8_conv_t {
 
 extern __shared__ __attribute__((aligned(16))) char i8_smem[];
 
-template <bool SRC_U8, bool WEI_U8>
-__global__ void __launch_bounds__(NT) i8_gemm_kernel(const problem_t P_, const i8_extra_t X) {
+template <bool SRC_U8, bool WEI_U8, class G>
+__global__ void __launch_bounds__(G::NT) __attribute__((amdgpu_waves_per_eu(G::NW * G::WG_PER_CU / 4))) i8_gemm_kernel(const problem_t P_, const i8_extra_t X) {
+    using Mma = i8_mma_t<SRC_U8, WEI_U8, G>;
     const auto &P = MI355_KERNARG_PROBLEM();
     char *smem = i8_smem;
     const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
-    const int wm = wave >> 1, wn = wave & 1;
+    const int wm = G::wm(wave), wn = G::wn(wave);
     const long b = blockIdx.z;
-    const tile_pos_t tp = tile_position(X.tiles_m, X.tiles_n);
+    const tile_pos_t tp = tile_position<G>(X.tiles_m, X.tiles_n);
     const long m0 = tp.m0, n0 = tp.n0;
 
     const long lda = P.ss[1];
     const char *A = (const char *)P.src + (P.ss[0] ? b * P.ss[0] : 0) + m0 * lda;
     const char *Bt = (const char *)X.bt + b * X.bt_bstride + n0 * X.ldb;
 
-    v4i acc[8][8];
+    v4i acc[Mma::ROWS][Mma::COLS];
 #pragma unroll
-    for (int i = 0; i < 8; ++i)
+    for (int i = 0; i < Mma::ROWS; ++i)
 #pragma unroll
-        for (int j = 0; j < 8; ++j)
+        for (int j = 0; j < Mma::COLS; ++j)
 #pragma unroll
             for (int r = 0; r < 4; ++r) acc[i][j][r] = 0;
 
-    main_loop<NSTAGE, 1, i8_mma_t<SRC_U8, WEI_U8>>(acc, smem, A, Bt, lda, X.ldb, P.M - m0, P.N - n0,
+    main_loop<NSTAGE, 1, Mma>(acc, smem, A, Bt, lda, X.ldb, P.M - m0, P.N - n0,
             (int)(P.K / BK), i8_ctx_t {});
 
     // ---- epilogue: s32 compensation, scales, shared tail
@@ -124,7 +128,7 @@ __global__ void __launch_bounds__(NT) i8_gemm_kernel(const problem_t P_, const i
     cv.ssc = cv.with_src_sc ? load_float(P.src_scale.dt, P.src_scale.p, 0) : 1.f;
     cv.rowsum = X.rowsum ? X.rowsum + bs * P.M : nullptr;
     const int Kc = (int)P.K;
-    const long nbase = n0 + wn * 128 + (lane & 31) * 4;
+    const long nbase = n0 + wn * G::WCOLS + (lane % (G::WCOLS / 4)) * 4;
 #pragma unroll
     for (int e = 0; e < 4; ++e) {
         const long n = nbase + e;
@@ -140,8 +144,8 @@ __global__ void __launch_bounds__(NT) i8_gemm_kernel(const problem_t P_, const i
                         quant_off(P.wei_scale, bw, 0, n, P.K, P.N));
         }
     }
-    const bool interior = m0 + BM <= P.M && n0 + BN <= P.N;
-    store_quadrant<layout16_t>(P, smem, acc, b, m0 + wm * 128, n0 + wn * 128, interior, cv);
+    const bool interior = m0 + BM <= P.M && n0 + G::BN <= P.N;
+    store_quadrant<layout16_t, G::WCOLS, G::NW>(P, smem, acc, b, m0 + wm * 128, n0 + wn * G::WCOLS, interior, cv);
 }
 
 // out[r] = sum_k (bytes[r][k] ^ flip) as signed bytes; one wave per row
@@ -264,9 +268,9 @@ int i8_launch(const mi355_matmul_desc_t &d, const problem_t &P, void *scratch,
         X.rowsum = rs;
     }
     X.tiles_m = (int)((d.M + BM - 1) / BM);
-    X.tiles_n = (int)((d.N + BN - 1) / BN);
+    X.tiles_n = (int)((d.N + i8_geo_t::BN - 1) / i8_geo_t::BN);
     dim3 grid((unsigned)(X.tiles_m * X.tiles_n), 1, (unsigned)d.batch);
-    constexpr int smem_bytes = NSTAGE * STAGE_BYTES;
+    constexpr int smem_bytes = NSTAGE * i8_geo_t::STAGE_BYTES;
     const bool su = d.src_dt == MI355_DT_U8, wu = d.wei_dt == MI355_DT_U8;
     auto go = [&](auto kern) {
         static bool attr_done = false; // per instantiation
@@ -278,13 +282,13 @@ int i8_launch(const mi355_matmul_desc_t &d, const problem_t &P, void *scratch,
             }
             attr_done = true;
         }
-        hipLaunchKernelGGL(kern, grid, dim3(NT), smem_bytes, stream, P, X);
+        hipLaunchKernelGGL(kern, grid, dim3(i8_geo_t::NT), smem_bytes, stream, P, X);
         return hipGetLastError() == hipSuccess ? MI355_SUCCESS : MI355_RUNTIME_ERROR;
     };
-    if (su && wu) return go(i8_gemm_kernel<true, true>);
-    if (su) return go(i8_gemm_kernel<true, false>);
-    if (wu) return go(i8_gemm_kernel<false, true>);
-    return go(i8_gemm_kernel<false, false>);
+    if (su && wu) return go(i8_gemm_kernel<true, true, i8_geo_t>);
+    if (su) return go(i8_gemm_kernel<true, false, i8_geo_t>);
+    if (wu) return go(i8_gemm_kernel<false, true, i8_geo_t>);
+    return go(i8_gemm_kernel<false, false, i8_geo_t>);
 }
 
 } // namespace mi355

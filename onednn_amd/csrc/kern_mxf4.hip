@@ -25,9 +25,10 @@ namespace mi355 {
 namespace {
 
 using namespace gemm;
-constexpr int NSTAGE = 4;
-constexpr int SCALE_OFF = NSTAGE * STAGE_BYTES;      // scale ring after the tile ring
-constexpr int SCALE_STAGE = 2048;                    // 256 dwords A + 256 dwords B
+using mx_geo_t = geo_t<4, 256>;
+constexpr int NSTAGE = mx_geo_t::NSTAGE;
+constexpr int SCALE_OFF = NSTAGE * mx_geo_t::STAGE_BYTES; // scale ring after the tile ring
+constexpr int SCALE_STAGE = (BM + mx_geo_t::BN) * 4;      // 256 dwords A + BN dwords B
 constexpr int SMEM_BYTES = SCALE_OFF + NSTAGE * SCALE_STAGE;
 
 struct mxf4_extra_t {
@@ -42,27 +43,41 @@ struct mxf4_extra_t {
 struct mxf4_ctx_t {
     const char *sa_tile, *sb_tile; // first scale byte of tile row 0
     unsigned voff_a, voff_b;       // this lane's row offset in the scale arrays
+    const char *s_tile;            // eight wavefronts: the one operand this wavefront brings
+    unsigned voff_s;
     unsigned lds_scale0;           // LDS byte address of the scale ring
     unsigned lds0;                 // LDS byte address of the tile ring
 };
 
+template <class G_>
 struct mxf4_mma_t {
-    static constexpr int EXTRA_DMAS = 2;
-    // wave w brings the scale dwords of tile rows [64w, 64w+64) of both operands
+    using G = G_;
+    static constexpr int EXTRA_DMAS = G::NW == 4 ? 2 : 1;
+    static constexpr int BBLK = G::BN / 64; // 64-row blocks of B^T scales
+    // four wavefronts: wave w brings the scale dwords of tile rows [64w, 64w+64)
+    // of A and those of block w % BBLK of B^T (with BN = 128 two wavefronts
+    // bring the same block: every wavefront issues the same number of loads,
+    // which the outstanding-load accounting relies on); eight wavefronts:
+    // waves 0-3 bring those of A, waves 4-7 those of B^T
     __device__ static __forceinline__ void issue_extra(const mxf4_ctx_t &c, int g, int slot, int wave,
             int) {
         const unsigned dst = c.lds_scale0 + slot * SCALE_STAGE + wave * 256;
-        dma4(c.sa_tile + (long)g * 4, c.voff_a, dst);
-        dma4(c.sb_tile + (long)g * 4, c.voff_b, dst + 1024);
+        if (G::NW == 4) {
+            dma4(c.sa_tile + (long)g * 4, c.voff_a, dst);
+            dma4(c.sb_tile + (long)g * 4, c.voff_b,
+                    c.lds_scale0 + slot * SCALE_STAGE + 1024 + (wave % BBLK) * 256);
+        } else {
+            dma4(c.s_tile + (long)g * 4, c.voff_s, dst);
+        }
     }
-    static constexpr int ROWS = 8, COLS = 8, A_READS = 2, B_READS = 2; // data + scale dword
+    static constexpr int ROWS = 8, COLS = G::WCOLS / 16, A_READS = 2, B_READS = 2; // data + scale dword
     struct frag_t {
-        v4i a[8], b[8];
-        int sa[8], sb[8];
+        v4i a[ROWS], b[COLS];
+        int sa[ROWS], sb[COLS];
     };
     // LDS byte address of the scale dwords that belong to the stage at S[0]
     __device__ static __forceinline__ unsigned scales(const unsigned (&S)[1], const mxf4_ctx_t &c) {
-        const unsigned slot = (S[0] - c.lds0) / STAGE_BYTES;
+        const unsigned slot = (S[0] - c.lds0) / G::STAGE_BYTES;
         return c.lds_scale0 + slot * SCALE_STAGE;
     }
     __device__ static __forceinline__ void load_b(frag_t &f, const unsigned (&S)[1], int wn, int lane,
@@ -70,8 +85,8 @@ struct mxf4_mma_t {
         const unsigned sc = scales(S, c);
         const int frow = lane & 15, q = lane >> 4;
 #pragma unroll
-        for (int j = 0; j < 8; ++j) {
-            const int rb = wn * 128 + j * 16 + frow;
+        for (int j = 0; j < COLS; ++j) {
+            const int rb = wn * G::WCOLS + j * 16 + frow;
             f.b[j] = lds_read16(S[0] + B_OFF + swz(rb, q));
             f.sb[j] = (int)((lds_read4(sc + (256 + rb) * 4) >> (q * 8)) & 0xffu);
         }
@@ -84,11 +99,11 @@ struct mxf4_mma_t {
         f.a[i] = lds_read16(S[0] + swz(ra, q));
         f.sa[i] = (int)((lds_read4(sc + ra * 4) >> (q * 8)) & 0xffu);
     }
-    __device__ static __forceinline__ void mma_row(v4f (&acc)[8][8], const frag_t &f, int i, const mxf4_ctx_t &,
-            int) {
+    __device__ static __forceinline__ void mma_row(v4f (&acc)[ROWS][COLS], const frag_t &f, int i,
+            const mxf4_ctx_t &, int) {
         const v8i a = {f.a[i][0], f.a[i][1], f.a[i][2], f.a[i][3], 0, 0, 0, 0};
 #pragma unroll
-        for (int j = 0; j < 8; ++j) {
+        for (int j = 0; j < COLS; ++j) {
             const v8i bb = {f.b[j][0], f.b[j][1], f.b[j][2], f.b[j][3], 0, 0, 0, 0};
             acc[i][j] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(
                     a, bb, acc[i][j], 4, 4, 0, f.sa[i], 0, f.sb[j]);
@@ -105,13 +120,15 @@ struct mxf4_conv_t {
 
 extern __shared__ __attribute__((aligned(16))) char mxf4_smem[];
 
-__global__ void __launch_bounds__(NT) mxf4_gemm_kernel(const problem_t P_, const mxf4_extra_t X) {
+template <class G>
+__global__ void __launch_bounds__(G::NT) __attribute__((amdgpu_waves_per_eu(G::NW * G::WG_PER_CU / 4))) mxf4_gemm_kernel(const problem_t P_, const mxf4_extra_t X) {
+    using Mma = mxf4_mma_t<G>;
     const auto &P = MI355_KERNARG_PROBLEM();
     char *smem = mxf4_smem;
     const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
-    const int wm = wave >> 1, wn = wave & 1;
+    const int wm = G::wm(wave), wn = G::wn(wave);
     const long b = blockIdx.z;
-    const tile_pos_t tp = tile_position(X.tiles_m, X.tiles_n);
+    const tile_pos_t tp = tile_position<G>(X.tiles_m, X.tiles_n);
     const long m0 = tp.m0, n0 = tp.n0;
 
     const long lda = P.ss[1] / 2; // bytes per src row
@@ -125,26 +142,29 @@ __global__ void __launch_bounds__(NT) mxf4_gemm_kernel(const problem_t P_, const
     ctx.sa_tile = X.sa + b * X.sa_bstride + m0 * kb;
     ctx.sb_tile = X.sb + b * X.sb_bstride + n0 * kb;
     {
-        long ra = wave * 64 + lane, rb = ra;
+        long ra = (wave & 3) * 64 + lane, rb = ((wave & 3) % (G::BN / 64)) * 64 + lane;
         if (ra > P.M - m0 - 1) ra = P.M - m0 - 1;
         if (rb > P.N - n0 - 1) rb = P.N - n0 - 1;
         ctx.voff_a = (unsigned)(ra * kb);
         ctx.voff_b = (unsigned)(rb * kb);
+        const bool brings_a = __builtin_amdgcn_readfirstlane(wave) < 4; // uniform: the base stays scalar
+        ctx.s_tile = brings_a ? ctx.sa_tile : ctx.sb_tile;
+        ctx.voff_s = brings_a ? ctx.voff_a : ctx.voff_b;
     }
 
-    v4f acc[8][8];
+    v4f acc[Mma::ROWS][Mma::COLS];
 #pragma unroll
-    for (int i = 0; i < 8; ++i)
+    for (int i = 0; i < Mma::ROWS; ++i)
 #pragma unroll
-        for (int j = 0; j < 8; ++j)
+        for (int j = 0; j < Mma::COLS; ++j)
 #pragma unroll
             for (int r = 0; r < 4; ++r) acc[i][j][r] = 0.f;
 
-    main_loop<NSTAGE, 1, mxf4_mma_t>(acc, smem, A, Bt, lda, X.ldb, P.M - m0, P.N - n0,
+    main_loop<NSTAGE, 1, Mma>(acc, smem, A, Bt, lda, X.ldb, P.M - m0, P.N - n0,
             (int)(P.K / 128), ctx);
 
-    const bool interior = m0 + BM <= P.M && n0 + BN <= P.N;
-    store_quadrant<layout16_t>(P, smem, acc, b, m0 + wm * 128, n0 + wn * 128, interior,
+    const bool interior = m0 + BM <= P.M && n0 + G::BN <= P.N;
+    store_quadrant<layout16_t, G::WCOLS, G::NW>(P, smem, acc, b, m0 + wm * 128, n0 + wn * G::WCOLS, interior,
             mxf4_conv_t {});
 }
 
@@ -244,18 +264,18 @@ int mxf4_launch(const mi355_matmul_desc_t &d, const problem_t &P, void *scratch,
     X.sa = (const char *)P.src_scale.p;
     X.sa_bstride = ((d.src_scale.mask & 1) && d.src_stride[0]) ? d.M * kb : 0;
     X.tiles_m = (int)((d.M + BM - 1) / BM);
-    X.tiles_n = (int)((d.N + BN - 1) / BN);
+    X.tiles_n = (int)((d.N + mx_geo_t::BN - 1) / mx_geo_t::BN);
     dim3 grid((unsigned)(X.tiles_m * X.tiles_n), 1, (unsigned)d.batch);
     static bool attr_done = false;
     if (!attr_done) {
-        if (hipFuncSetAttribute((const void *)mxf4_gemm_kernel,
+        if (hipFuncSetAttribute((const void *)mxf4_gemm_kernel<mx_geo_t>,
                     hipFuncAttributeMaxDynamicSharedMemorySize, SMEM_BYTES) != hipSuccess) {
             set_error("mfma_mxf4: cannot reserve %d bytes of LDS", SMEM_BYTES);
             return MI355_RUNTIME_ERROR;
         }
         attr_done = true;
     }
-    hipLaunchKernelGGL(mxf4_gemm_kernel, grid, dim3(NT), SMEM_BYTES, stream, P, X);
+    hipLaunchKernelGGL(mxf4_gemm_kernel<mx_geo_t>, grid, dim3(mx_geo_t::NT), SMEM_BYTES, stream, P, X);
     return hipGetLastError() == hipSuccess ? MI355_SUCCESS : MI355_RUNTIME_ERROR;
 }
 

@@ -1,10 +1,11 @@
 // Epilogue of the LDS-tiled MFMA kernels.
 //
-// After the K loop every wavefront owns a 128x128 quadrant in accumulator
-// registers (16 tiles of 32x32).  It leaves through LDS in four 32-row slabs;
-// afterwards each lane owns four consecutive n of one row, so dst goes out in
-// coalesced 4/8/16-byte stores and the per-element epilogue code exists once,
-// in a rolled loop over the 16 row pairs of a slab.
+// After the K loop every wavefront owns a 128 x WCOLS part of the tile in
+// accumulator registers (WCOLS = 128 with four wavefronts per workgroup, 64
+// with eight).  It leaves through LDS in four 32-row slabs; afterwards each
+// lane owns four consecutive n of one row, so dst goes out in coalesced
+// 4/8/16-byte stores and the per-element epilogue code exists once, in a
+// rolled loop over the row groups of a slab.
 //
 // With one wavefront per SIMD nothing hides memory latency inside that loop,
 // so every operand that does not depend on the row is loaded once per lane
@@ -603,31 +604,51 @@ __device__ __forceinline__ void storeQ(const PT &P, const epi_hoist_t &H, const 
     }
 }
 
+// One row of accumulator tiles copied by value.  The slab writers pick their rows
+// with a switch over the run-time slab number; were the cases identical code on
+// different addresses, the compiler would merge them into one copy that indexes
+// `acc` with a run-time offset, and all accumulators would live in private memory
+// from the first K step on.  The empty asm statements keep the cases apart
+// (statements of inline assembly are never merged).
+template <class T, int C>
+__device__ __forceinline__ void copy_row(const T (&src)[C], T (&dst)[C]) {
+#pragma unroll
+    for (int j = 0; j < C; ++j) {
+        T v = src[j];
+        asm volatile("" : "+v"(v));
+        dst[j] = v;
+    }
+}
+
 // Accumulator layouts: how a wavefront's 128x128 quadrant sits in registers
 // and how one 32-row slab of it is written to LDS as [32 rows][128 cols] s32.
 //
 // 32x32 MFMA tiles, acc[4][4] of 16 registers: register r of tile (i, j) holds
 // row 32i + 8*(r/4) + 4*(lane/32) + r%4, column 32j + lane%32.
 struct layout32_t {
-    template <class Acc>
-    static __device__ __forceinline__ void write_slab(const Acc &acc, int s, slab_int_t *wl, int lane) {
+    template <class T, int R, int C>
+    static __device__ __forceinline__ void write_slab(const T (&acc)[R][C], int s, slab_int_t *wl, int lane) {
+        constexpr int WCOLS = C * 32;
         // volatile: the dword stores stay single ds_write_b32 instructions.  Merged
         // into ds_write2_b32 pairs by the compiler (ROCm 7.2), two stores per tile
         // of this layout came out with their first offset divided by four and
         // landed in other cells of the slab; the parity tests caught it.
         volatile slab_int_t *vw = wl;
-        auto w = [&](const auto &a) {
+        T a[C];
+        pick_rows(acc, s, a);
 #pragma unroll
-            for (int j = 0; j < 4; ++j)
+        for (int j = 0; j < C; ++j)
 #pragma unroll
-                for (int r = 0; r < 16; ++r)
-                    vw[((r >> 2) * 8 + (lane >> 5) * 4 + (r & 3)) * 128 + j * 32 + (lane & 31)] = raw_bits(a[j][r]);
-        };
+            for (int r = 0; r < 16; ++r)
+                vw[((r >> 2) * 8 + (lane >> 5) * 4 + (r & 3)) * WCOLS + j * 32 + (lane & 31)] = raw_bits(a[j][r]);
+    }
+    template <class T, int R, int C>
+    static __device__ __forceinline__ void pick_rows(const T (&acc)[R][C], int s, T (&a)[C]) {
         switch (s) {
-            case 0: w(acc[0]); break;
-            case 1: w(acc[1]); break;
-            case 2: w(acc[2]); break;
-            default: w(acc[3]); break;
+            case 0: copy_row(acc[0], a); break;
+            case 1: copy_row(acc[1], a); break;
+            case 2: copy_row(acc[2], a); break;
+            default: copy_row(acc[3], a); break;
         }
     }
 };
@@ -635,37 +656,44 @@ struct layout32_t {
 // 16x16 MFMA tiles, acc[8][8] of 4 registers: register r of tile (i, j) holds
 // row 16i + 4*(lane/16) + r, column 16j + lane%16.
 struct layout16_t {
-    template <class Acc>
-    static __device__ __forceinline__ void write_slab(const Acc &acc, int s, slab_int_t *wl, int lane) {
+    template <class T, int R, int C>
+    static __device__ __forceinline__ void write_slab(const T (&acc)[R][C], int s, slab_int_t *wl, int lane) {
+        constexpr int WCOLS = C * 16;
         slab_int_t *vw = wl;
-        auto w = [&](const auto &a0, const auto &a1) {
-#pragma unroll
-            for (int j = 0; j < 8; ++j)
-#pragma unroll
-                for (int r = 0; r < 4; ++r) {
-                    vw[((lane >> 4) * 4 + r) * 128 + j * 16 + (lane & 15)] = raw_bits(a0[j][r]);
-                    vw[(16 + (lane >> 4) * 4 + r) * 128 + j * 16 + (lane & 15)] = raw_bits(a1[j][r]);
-                }
-        };
+        T a0[C], a1[C];
         switch (s) {
-            case 0: w(acc[0], acc[1]); break;
-            case 1: w(acc[2], acc[3]); break;
-            case 2: w(acc[4], acc[5]); break;
-            default: w(acc[6], acc[7]); break;
+            case 0: copy_row(acc[0], a0); copy_row(acc[1], a1); break;
+            case 1: copy_row(acc[2], a0); copy_row(acc[3], a1); break;
+            case 2: copy_row(acc[4], a0); copy_row(acc[5], a1); break;
+            default: copy_row(acc[6], a0); copy_row(acc[7], a1); break;
         }
+#pragma unroll
+        for (int j = 0; j < C; ++j)
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                vw[((lane >> 4) * 4 + r) * WCOLS + j * 16 + (lane & 15)] = raw_bits(a0[j][r]);
+                vw[(16 + (lane >> 4) * 4 + r) * WCOLS + j * 16 + (lane & 15)] = raw_bits(a1[j][r]);
+            }
     }
 };
 
 // `conv.row(raw, m, f)` turns four raw accumulators of row m into the f32
 // values that enter the epilogue.
-// smem: >= 128 KB; [0, 64K) accumulator slabs, [64K, 128K) operand staging.
-template <class Layout, class PT, class Acc, class Conv>
+// smem: one accumulator slab per wavefront (32 rows x WCOLS x 4 bytes), then
+// as much again for operand staging.
+// WCOLS: columns of the wavefront's part; NW: wavefronts of the workgroup.
+template <class Layout, int WCOLS, int NW, class PT, class Acc, class Conv>
 __device__ __forceinline__ void store_quadrant(const PT &P, char *smem, const Acc &acc,
         long b, long m_base, long n_base_wave, bool interior, const Conv &conv) {
+    constexpr int LPR = WCOLS / 4;     // lanes per row: four consecutive n each
+    constexpr int RPP = 64 / LPR;      // rows per pass of the wavefront
+    constexpr int PASSES = 32 / RPP;   // passes per 32-row slab
+    constexpr int SLAB_INTS = 32 * WCOLS;
     const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
-    slab_int_t *wl = (slab_int_t *)smem + wave * 4096;      // 16 KB per wavefront
-    stage_u4_t *stg = (stage_u4_t *)(smem + 65536) + wave * 1024; // 16 KB per wavefront
-    const long nbase = n_base_wave + (lane & 31) * 4;
+    const int lrow = lane / LPR, lcol = lane % LPR;
+    slab_int_t *wl = (slab_int_t *)smem + wave * SLAB_INTS;
+    stage_u4_t *stg = (stage_u4_t *)(smem + NW * SLAB_INTS * 4) + wave * (PASSES * 64);
+    const long nbase = n_base_wave + lcol * 4;
     int nvalid = 0;
 #pragma unroll
     for (int e = 0; e < 4; ++e)
@@ -677,38 +705,39 @@ __device__ __forceinline__ void store_quadrant(const PT &P, char *smem, const Ac
 #pragma unroll 1
     for (int i = 0; i < 4; ++i) {
         if (H.staged != STG_NONE) {
-            // 16 independent vector loads in flight, then park them in LDS
-            uint4 tmp[16];
+            // PASSES independent vector loads in flight, then park them in LDS
+            uint4 tmp[PASSES];
             const char *base = H.staged_p
-                    + (b * H.st_s0 + (m_base + i * 32 + (lane >> 5)) * H.st_s1 + nbase) * sbytes;
+                    + (b * H.st_s0 + (m_base + i * 32 + lrow) * H.st_s1 + nbase) * sbytes;
             if (sbytes == 2) {
 #pragma unroll
-                for (int it = 0; it < 16; ++it) {
-                    const uint2 q = *(const uint2 *)(base + (long)it * 2 * H.st_s1 * 2);
+                for (int it = 0; it < PASSES; ++it) {
+                    const uint2 q = *(const uint2 *)(base + (long)it * RPP * H.st_s1 * 2);
                     tmp[it].x = q.x; tmp[it].y = q.y; tmp[it].z = 0; tmp[it].w = 0;
                 }
             } else {
 #pragma unroll
-                for (int it = 0; it < 16; ++it) tmp[it] = *(const uint4 *)(base + (long)it * 2 * H.st_s1 * 4);
+                for (int it = 0; it < PASSES; ++it)
+                    tmp[it] = *(const uint4 *)(base + (long)it * RPP * H.st_s1 * 4);
             }
 #pragma unroll
-            for (int it = 0; it < 16; ++it) stg[it * 64 + lane] = tmp[it];
+            for (int it = 0; it < PASSES; ++it) stg[it * 64 + lane] = tmp[it];
         }
         Layout::write_slab(acc, i, wl, lane);
         if (H.batchable) {
             constexpr int NQ = 4;
 #pragma unroll 1
-            for (int it0 = 0; it0 < 16; it0 += NQ) {
+            for (int it0 = 0; it0 < PASSES; it0 += NQ) {
                 v4i_t raw[NQ];
                 uint4 sv[NQ];
                 long m[NQ];
                 bool ok[NQ];
 #pragma unroll
                 for (int k = 0; k < NQ; ++k) {
-                    const int row = (it0 + k) * 2 + (lane >> 5);
+                    const int row = (it0 + k) * RPP + lrow;
                     m[k] = m_base + i * 32 + row;
                     ok[k] = m[k] < P.M;
-                    raw[k] = *(const slab_v4i_t *)&wl[row * 128 + (lane & 31) * 4];
+                    raw[k] = *(const slab_v4i_t *)&wl[row * WCOLS + lcol * 4];
                     sv[k] = make_uint4(0, 0, 0, 0);
                 }
                 if (H.staged != STG_NONE) {
@@ -724,10 +753,10 @@ __device__ __forceinline__ void store_quadrant(const PT &P, char *smem, const Ac
             continue;
         }
 #pragma unroll 1
-        for (int it = 0; it < 16; ++it) {
-            const int row = it * 2 + (lane >> 5);
+        for (int it = 0; it < PASSES; ++it) {
+            const int row = it * RPP + lrow;
             const long m = m_base + i * 32 + row;
-            const v4i_t raw = *(const slab_v4i_t *)&wl[row * 128 + (lane & 31) * 4];
+            const v4i_t raw = *(const slab_v4i_t *)&wl[row * WCOLS + lcol * 4];
             uint4 sv = make_uint4(0, 0, 0, 0);
             if (H.staged != STG_NONE) sv = stg[it * 64 + lane];
             if (m < P.M && nvalid > 0) {
