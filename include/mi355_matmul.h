@@ -21,6 +21,10 @@
  *                             brgemm_matmul_t.
  *   - mi355_matmul_query    : pd_t::init() dispatch predicate + name()
  *                             (DECLARE_COMMON_PD_T, src/common/primitive_desc.hpp).
+ *   - mi355_reorder_*       : the reorder primitive that brings user tensors
+ *                             into the layouts / data types the matmul wants
+ *                             (src/common/reorder.cpp:67-170,
+ *                             src/cpu/reorder/simple_reorder.hpp).
  *   - mi355_mem_* / stream  : memory_storage_t / stream_t of an engine
  *                             (src/common/memory_storage.hpp, src/common/stream.hpp).
  */
@@ -235,6 +239,49 @@ int mi355_matmul_scratch_bytes(const mi355_matmul_desc_t *desc, size_t *bytes);
  * mi355_matmul_scratch_bytes reports 0. */
 int mi355_matmul_launch(const mi355_matmul_desc_t *desc,
         const mi355_matmul_args_t *args, void *scratch, void *stream);
+
+/* ---- reorder: layout and data-type conversion of one tensor -------------- */
+
+#define MI355_REORDER_MAX_DIMS 6
+
+/* What a reorder pd_t holds (src/common/reorder_pd.hpp) for plain strided
+ * tensors, with the attributes the reference's generic reorder honours
+ * (simple_reorder_impl_t<..., spec::reference>::execute,
+ * src/cpu/reorder/simple_reorder.hpp:2579-2661, and its 4-bit variants
+ * :2168-2425):
+ *   d = src_scale * (src - src_zp);  d += beta * dst_old;
+ *   d = d / dst_scale + dst_zp;      dst = saturate_and_round<dst_dt>(d)
+ * Scales / zero points are dense row-major tensors over the masked dims with
+ * the last two dims divided by the groups (quant_entry_t::get_md), mask bit i
+ * = dim i.  Strides are in elements (nibbles for 4-bit types). */
+typedef struct mi355_reorder_desc {
+    int32_t ndims;
+    int32_t src_dt, dst_dt;
+    int32_t reserved;
+    int64_t dims[MI355_REORDER_MAX_DIMS];
+    int64_t src_stride[MI355_REORDER_MAX_DIMS];
+    int64_t dst_stride[MI355_REORDER_MAX_DIMS];
+    mi355_quant_t src_scale, dst_scale; /* dst_scale: f32, no groups */
+    mi355_quant_t src_zp, dst_zp;       /* dst_zp: common s32 */
+    float beta;                         /* sum post-op scale, 0 = none */
+    int32_t reserved2;
+} mi355_reorder_desc_t;
+
+typedef struct mi355_reorder_args {
+    const void *src;
+    void *dst;
+    const void *src_scale, *dst_scale;
+    const void *src_zp, *dst_zp;
+} mi355_reorder_args_t;
+
+/* MI355_SUCCESS if the reorder kernels compute `desc` exactly,
+ * MI355_UNIMPLEMENTED / MI355_INVALID_ARGUMENTS otherwise. */
+int mi355_reorder_query(const mi355_reorder_desc_t *desc);
+
+/* Enqueue the reorder on `stream` (primitive_t::execute of the reorder
+ * implementations, DNNL_ARG_FROM -> DNNL_ARG_TO).  Asynchronous. */
+int mi355_reorder_launch(const mi355_reorder_desc_t *desc,
+        const mi355_reorder_args_t *args, void *stream);
 
 /* Plain device-to-device copy kernel (one 16-byte load + store per lane), used
  * to calibrate the FETCH_SIZE / WRITE_SIZE counters against a known size. */

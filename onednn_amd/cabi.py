@@ -78,6 +78,28 @@ class MatmulArgs(C.Structure):
     ]
 
 
+REORDER_MAX_DIMS = 6
+
+
+class ReorderDesc(C.Structure):
+    """mi355_reorder_desc_t"""
+    _fields_ = [
+        ("ndims", C.c_int32), ("src_dt", C.c_int32), ("dst_dt", C.c_int32), ("reserved", C.c_int32),
+        ("dims", C.c_int64 * REORDER_MAX_DIMS), ("src_stride", C.c_int64 * REORDER_MAX_DIMS),
+        ("dst_stride", C.c_int64 * REORDER_MAX_DIMS),
+        ("src_scale", Quant), ("dst_scale", Quant), ("src_zp", Quant), ("dst_zp", Quant),
+        ("beta", C.c_float), ("reserved2", C.c_int32),
+    ]
+
+
+class ReorderArgs(C.Structure):
+    """mi355_reorder_args_t"""
+    _fields_ = [
+        ("src", C.c_void_p), ("dst", C.c_void_p), ("src_scale", C.c_void_p), ("dst_scale", C.c_void_p),
+        ("src_zp", C.c_void_p), ("dst_zp", C.c_void_p),
+    ]
+
+
 # every symbol include/mi355_matmul.h declares
 KERNEL_SYMBOLS = [
     "mi355_device_count", "mi355_device_set", "mi355_device_info", "mi355_mem_alloc",
@@ -85,8 +107,8 @@ KERNEL_SYMBOLS = [
     "mi355_stream_create", "mi355_stream_destroy", "mi355_stream_sync", "mi355_event_create",
     "mi355_event_destroy", "mi355_event_record", "mi355_event_sync", "mi355_event_elapsed_ms",
     "mi355_last_error", "mi355_matmul_query", "mi355_matmul_impl_name",
-    "mi355_matmul_scratch_bytes", "mi355_matmul_launch", "mi355_copy_kernel",
-    "mi355_flush_kernel",
+    "mi355_matmul_scratch_bytes", "mi355_matmul_launch", "mi355_reorder_query",
+    "mi355_reorder_launch", "mi355_copy_kernel", "mi355_flush_kernel",
 ]
 
 _PKG_DIR = os.path.dirname(os.path.abspath(__file__))
@@ -137,6 +159,8 @@ def load_kernels():
     lib.mi355_matmul_query.argtypes = [C.POINTER(MatmulDesc), C.c_int, C.POINTER(C.c_int)]
     lib.mi355_matmul_scratch_bytes.argtypes = [C.POINTER(MatmulDesc), C.POINTER(C.c_size_t)]
     lib.mi355_matmul_launch.argtypes = [C.POINTER(MatmulDesc), C.POINTER(MatmulArgs), vp, vp]
+    lib.mi355_reorder_query.argtypes = [C.POINTER(ReorderDesc)]
+    lib.mi355_reorder_launch.argtypes = [C.POINTER(ReorderDesc), C.POINTER(ReorderArgs), vp]
     lib.mi355_copy_kernel.argtypes = [vp, vp, C.c_size_t, vp]
     lib.mi355_flush_kernel.argtypes = [vp, C.c_size_t, vp]
     _lib = lib

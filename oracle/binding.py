@@ -34,6 +34,7 @@ def load():
                                   C.c_int, C.c_void_p, C.c_void_p]
     lib.oracle_int8_acc.argtypes = [C.POINTER(cabi.MatmulDesc), C.POINTER(cabi.MatmulArgs),
                                     C.c_void_p]
+    lib.oracle_reorder.argtypes = [C.POINTER(cabi.ReorderDesc), C.POINTER(cabi.ReorderArgs)]
     _lib = lib
     return lib
 
@@ -169,3 +170,20 @@ def binary(alg, x, y):
     lib.oracle_binary(C.c_int(alg), C.c_void_p(x.ctypes.data), C.c_void_p(y.ctypes.data),
                       C.c_void_p(out.ctypes.data), C.c_int64(x.size))
     return out
+
+
+def reorder(prob):
+    """CPU oracle result of a onednn_amd.reorder.ReorderProblem (raw dst storage)."""
+    lib = load()
+    d = prob.desc()
+    a = cabi.ReorderArgs()
+    keep = [np.ascontiguousarray(prob.src)]
+    a.src = keep[0].ctypes.data
+    dst = prob.new_dst()
+    a.dst = dst.ctypes.data
+    for name, q in prob.quant.items():
+        keep.append(np.ascontiguousarray(q.data))
+        setattr(a, name, keep[-1].ctypes.data)
+    st = lib.oracle_reorder(C.byref(d), C.byref(a))
+    assert st == 0
+    return dst

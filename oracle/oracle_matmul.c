@@ -20,6 +20,10 @@
  *                     io::load_int_value / load_float_value / store_float_value
  *                     src/cpu/ref_io_helper.hpp:34-150 and
  *                     q10n::saturate_and_round src/cpu/simple_q10n.hpp:41-81
+ *   oracle_reorder    the generic reorder, simple_reorder_impl_t<..., spec::reference>
+ *                     ::execute src/cpu/reorder/simple_reorder.hpp:2579-2661 and
+ *                     its 4-bit variants :2168-2288 (f32 -> s4/u4/f4) and
+ *                     :2291-2425 (s4/u4/f4 -> f32/bf16/f16)
  *   orc_quant_off     quant_entry_t::get_md src/common/primitive_attr_quant.hpp:116-140
  *                     + matmul_helper_t::get_quant_off src/cpu/matmul/matmul_utils.hpp:154-173
  *
@@ -113,6 +117,14 @@ static inline void orc_store_float(int dt, float v, void *p, int64_t off) {
             break;
         case MI355_DT_U8:
             ((uint8_t *)p)[off] = (uint8_t)nearbyintf(orc_sat(v, 0.f, 255.f));
+            break;
+        /* int4_t / uint4_t: the same clamp-then-round with the 4-bit limits
+         * (src/common/int4.hpp:28-84, type_helpers.hpp max_value/lowest_value) */
+        case MI355_DT_S4:
+            orc_nibble_set(p, off, (uint8_t)((int)nearbyintf(orc_sat(v, -8.f, 7.f)) & 0xf));
+            break;
+        case MI355_DT_U4:
+            orc_nibble_set(p, off, (uint8_t)((int)nearbyintf(orc_sat(v, 0.f, 15.f)) & 0xf));
             break;
         default: break;
     }
@@ -544,4 +556,81 @@ void oracle_eltwise(int alg, float alpha, float beta, const float *in,
 void oracle_binary(int alg, const float *x, const float *y, float *out,
         int64_t n) {
     ORC_CVT_LOOP(out[i] = orc_binary(alg, x[i], y[i]))
+}
+
+/* ------------------------------------------------------------------ reorder
+ * One logical element at a time, in the reference's order of operations:
+ *   d = src_scale * (src - src_zp)     (integer sources subtract as integers:
+ *                                        `input[i_off] - src_zp_val` with
+ *                                        data_t<type_i> promoted to int, :2656;
+ *                                        4-bit sources go through float, :2421)
+ *   d += beta * dst_old                 (:2657)
+ *   d = d / dst_scale + dst_zp          (:2658; skipped when neither is set, as
+ *                                        the plain-copy implementations that
+ *                                        the reference lists first do)
+ *   dst = _qz_a1b0<f32, type_o>()(d)    (:2659) = saturate + nearbyintf for
+ *                                        integers, a conversion otherwise
+ * e8m0 sources are converted without arithmetic (:2645-2655).
+ * Scale / zero-point offsets: get_quant_off over the logical index with the
+ * groups on the last two dims (:2606-2640). */
+static int64_t orc_rq_off(const mi355_quant_t *q, const int64_t *idx, int ndims,
+        const int64_t *dims) {
+    int64_t off = 0, stride = 1;
+    for (int d = ndims - 1; d >= 0; --d) {
+        int64_t g = 1;
+        if (d == ndims - 2) g = q->group[0];
+        if (d == ndims - 1) g = q->group[1];
+        if (q->mask & (1 << d)) {
+            off += (idx[d] / g) * stride;
+            stride *= dims[d] / g;
+        }
+    }
+    return off;
+}
+
+static int orc_is_int_dt(int dt) {
+    return dt == MI355_DT_S32 || dt == MI355_DT_S8 || dt == MI355_DT_U8;
+}
+
+int oracle_reorder(const mi355_reorder_desc_t *d, const mi355_reorder_args_t *a) {
+    const int nd = d->ndims;
+    int64_t total = 1;
+    for (int i = 0; i < nd; ++i) total *= d->dims[i];
+    for (int64_t l = 0; l < total; ++l) {
+        int64_t idx[MI355_REORDER_MAX_DIMS] = {0};
+        int64_t rem = l, so = 0, dof = 0;
+        for (int i = nd - 1; i >= 0; --i) {
+            idx[i] = rem % d->dims[i];
+            rem /= d->dims[i];
+            so += idx[i] * d->src_stride[i];
+            dof += idx[i] * d->dst_stride[i];
+        }
+        float x;
+        if (d->src_dt == MI355_DT_E8M0) {
+            x = orc_load_float(MI355_DT_E8M0, a->src, so);
+        } else {
+            int zp = 0;
+            if (d->src_zp.dt != MI355_DT_UNDEF)
+                zp = (int)orc_load_float(d->src_zp.dt, a->src_zp,
+                        orc_rq_off(&d->src_zp, idx, nd, d->dims));
+            if (orc_is_int_dt(d->src_dt)) x = (float)(orc_load_int(d->src_dt, a->src, so) - zp);
+            else x = orc_load_float(d->src_dt, a->src, so) - (float)zp;
+            if (d->src_scale.dt != MI355_DT_UNDEF)
+                x = orc_load_float(d->src_scale.dt, a->src_scale,
+                            orc_rq_off(&d->src_scale, idx, nd, d->dims))
+                        * x;
+            if (d->beta != 0.f) x += d->beta * orc_load_float(d->dst_dt, a->dst, dof);
+            if (d->dst_scale.dt != MI355_DT_UNDEF || d->dst_zp.dt != MI355_DT_UNDEF) {
+                float dsc = 1.f;
+                int dzp = 0;
+                if (d->dst_scale.dt != MI355_DT_UNDEF)
+                    dsc = orc_load_float(d->dst_scale.dt, a->dst_scale,
+                            orc_rq_off(&d->dst_scale, idx, nd, d->dims));
+                if (d->dst_zp.dt != MI355_DT_UNDEF) dzp = orc_load_int(d->dst_zp.dt, a->dst_zp, 0);
+                x = x / dsc + (float)dzp;
+            }
+        }
+        orc_store_float(d->dst_dt, x, a->dst, dof);
+    }
+    return 0;
 }
