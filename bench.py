@@ -153,6 +153,43 @@ def run_gpu_workload(lib, name, steps, warmup, M=None, cold_copies=0, wtag="any"
     return out, p
 
 
+def run_reorder_workloads(lib, steps, which=("r1", "r2")):
+    """Informational: the reorder primitive on the tensors of the headline
+    shape (HBM-bound; bytes = src + dst + parameter tensors)."""
+    import numpy as np
+    from onednn_amd import cabi
+    from onednn_amd.problem import QuantParam
+    from onednn_amd.reorder import GpuReorder, ReorderProblem
+    N = 8192
+    rng = np.random.default_rng(7)
+    x8 = rng.integers(-128, 128, size=(N, N), dtype=np.int8)
+    xf = rng.standard_normal((N, N)).astype(np.float32)
+    sc = rng.uniform(0.5, 2, size=N).astype(np.float32)
+    plan = {
+        "r1": (ReorderProblem(dims=(N, N), src_dt=cabi.DT_F32, dst_dt=cabi.DT_S8, src=xf,
+                              quant={"dst_scale": QuantParam(cabi.DT_F32, 2, sc)},
+                              name="R1 f32->s8 8192x8192, per-column dst scales"), 5 * N * N + 4 * N),
+        "r2": (ReorderProblem(dims=(N, N), src_dt=cabi.DT_S8, dst_dt=cabi.DT_S8, src=x8, dst_stride=(1, N),
+                              name="R2 s8 8192x8192 ab->ba (weights into the layout format_tag::any resolves to)"),
+               2 * N * N),
+    }
+    out = []
+    timer = Timer(lib)
+    for key in which:
+        p, nbytes = plan[key]
+        r = GpuReorder(p)
+        r.launch()
+        ms = timer.time_ms(r.launch, steps)
+        gbs = nbytes / (ms * 1e-3) / 1e9
+        out.append({"workload": p.name, "impl": "hip:reorder:any", "ms_per_step": ms, "value": gbs, "unit": "GB/s",
+                    "bound": "hbm", "peak": PEAK_HBM_GBS, "frac_of_peak": gbs / PEAK_HBM_GBS, "work": nbytes})
+        log(f"[bench] {p.name}: {ms:.4f} ms -> {gbs:.1f} GB/s ({100 * gbs / PEAK_HBM_GBS:.1f}% of hbm peak) "
+            "via hip:reorder:any")
+        for b in r.bufs.values():
+            b.free()
+    return out
+
+
 def cpu_baseline(name, M=None):
     """The oracle timed on a bounded sample of the same workload."""
     from oracle import binding as oracle
@@ -196,7 +233,9 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=3)
-    ap.add_argument("--workload", default="c3", choices=["c1", "c2", "c3", "c4", "c5"])
+    ap.add_argument("--workload", default="c3", choices=["c1", "c2", "c3", "c4", "c5", "r1", "r2"],
+                    help="c1..c5: the matmul configurations (c3 is the headline); r1, r2: the reorder "
+                         "primitive on the headline shape's tensors (informational)")
     ap.add_argument("--decode-m", type=int, default=1, help="M of the c2 decode workload")
     ap.add_argument("--wtag", default="any", choices=["any", "ab", "ba"],
                     help="weights layout; any = what format_tag::any resolves to (default)")
@@ -226,13 +265,7 @@ def main():
         f"HBM={hbm.value / 2**30:.0f} GiB")
 
     main_name = args.workload
-    cold = 11 if main_name == "c2" else 0
-    res, prob = run_gpu_workload(lib, main_name, args.steps, args.warmup, args.decode_m, cold,
-                                 args.wtag)
-    log(f"[bench] {res['workload']}: {res['ms_per_step']:.4f} ms/step -> {res['value']:.1f} "
-        f"{res['unit']} via {res['impl']}")
-
-    if args.calib_copy:
+    def calib_copy():
         nbytes = 256 << 20
         a, b = cabi.DeviceBuffer(nbytes), cabi.DeviceBuffer(nbytes)
         for _ in range(3):
@@ -240,6 +273,29 @@ def main():
         cabi.check(lib.mi355_stream_sync(None))
         a.free()
         b.free()
+
+    if main_name in ("r1", "r2"):
+        r = run_reorder_workloads(lib, args.steps, (main_name,))[0]
+        if args.calib_copy:
+            calib_copy()
+        print(json.dumps({
+            "metric": "reorder GB/s", "value": r["value"], "unit": "GB/s", "n_gpus": 1, "steps": args.steps,
+            "warmup": args.warmup, "ms_per_step": r["ms_per_step"], "higher_is_better": True, "scaling": "weak",
+            "vs_baseline": None, "dtype": "f32" if main_name == "r1" else "s8", "data": "synthetic",
+            "config": {"workload": r["workload"], "impl": r["impl"]},
+            "roofline": {"bound": "hbm", "achieved": r["value"], "peak": PEAK_HBM_GBS, "unit": "GB/s",
+                         "frac": r["frac_of_peak"], "traffic": None, "algorithmic": r["work"],
+                         "kernel": r["impl"], "kernel_ms": r["ms_per_step"]},
+            "cpu_baseline": None, "others": []}), flush=True)
+        return
+    cold = 11 if main_name == "c2" else 0
+    res, prob = run_gpu_workload(lib, main_name, args.steps, args.warmup, args.decode_m, cold,
+                                 args.wtag)
+    log(f"[bench] {res['workload']}: {res['ms_per_step']:.4f} ms/step -> {res['value']:.1f} "
+        f"{res['unit']} via {res['impl']}")
+
+    if args.calib_copy:
+        calib_copy()
 
     # The timed step is one launch whose time is dominated by one kernel (the
     # tile GEMM / the decode kernel); the small kernels of the same launch (the
@@ -271,6 +327,12 @@ def main():
             except Exception as e:  # a failing side workload must not hide the headline
                 others.append({"workload": f"{nm}-M{m}" if m else nm, "error": str(e)})
                 log(f"[bench] {nm}: failed: {e}")
+
+        try:
+            others += run_reorder_workloads(lib, max(5, args.steps // 2))
+        except Exception as e:
+            others.append({"workload": "reorder", "error": str(e)})
+            log(f"[bench] reorder: failed: {e}")
 
     cpu = None
     if not args.no_cpu:

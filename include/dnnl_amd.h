@@ -116,6 +116,7 @@ typedef enum {
 /* dnnl_types.h:2057-2101 */
 typedef enum {
     dnnl_undefined_primitive = 0,
+    dnnl_reorder = 1,
     dnnl_sum = 4,
     dnnl_eltwise = 7,
     dnnl_binary = 13,
@@ -304,6 +305,15 @@ dnnl_status_t dnnl_matmul_primitive_desc_create(dnnl_primitive_desc_t *primitive
         const_dnnl_memory_desc_t src_desc, const_dnnl_memory_desc_t weights_desc,
         const_dnnl_memory_desc_t bias_desc, const_dnnl_memory_desc_t dst_desc,
         const_dnnl_primitive_attr_t attr);
+
+/* ---- reorder primitive descriptor: dnnl.h:1727-1731.  Execute arguments are
+ * DNNL_ARG_FROM / DNNL_ARG_TO (dnnl_types.h:2553,2580) plus the scales and zero
+ * points of DNNL_ARG_SRC / DNNL_ARG_DST. ---- */
+#define DNNL_ARG_FROM DNNL_ARG_SRC
+#define DNNL_ARG_TO DNNL_ARG_DST
+dnnl_status_t dnnl_reorder_primitive_desc_create(dnnl_primitive_desc_t *reorder_primitive_desc,
+        const_dnnl_memory_desc_t src_desc, dnnl_engine_t src_engine, const_dnnl_memory_desc_t dst_desc,
+        dnnl_engine_t dst_engine, const_dnnl_primitive_attr_t attr);
 
 /* ---- primitive descriptors and primitives: dnnl.h:60-243 ---- */
 dnnl_status_t dnnl_primitive_desc_clone(dnnl_primitive_desc_t *primitive_desc,

@@ -26,29 +26,36 @@ namespace mi355 {
 namespace {
 
 constexpr int RD = MI355_REORDER_MAX_DIMS;
+constexpr int NQ = 3; // src scales, dst scales, src zero points (dst zero point is one value)
 
-struct rq_t { // one quantization parameter tensor
-    const void *p;
-    int dt;
-    int present;
-    long stride[RD]; // element stride of the parameter tensor per dim, 0 = broadcast
-    long group[RD];  // logical indices per parameter along the dim
+// One logical dim as the kernels see it: extent, element strides of both
+// tensors and, per quantization parameter tensor, its stride along this dim
+// (0 = broadcast) and the group size (logical indices per parameter).
+struct rdim_t {
+    unsigned n;
+    unsigned qg[NQ];
+    long ss, ds;
+    long qs[NQ];
 };
 
 struct reorder_t {
-    int ndims, src_dt, dst_dt;
+    int src_dt, dst_dt;
     float beta;
+    int n_outer;        // dims besides `a` (and `b` in the tiled kernel)
     const void *src;
     void *dst;
-    long dims[RD], ss[RD], ds[RD];
-    // walk order: dims sorted by ascending dst stride; order[0] is the inner dim
-    int order[RD];
-    rq_t src_scale, dst_scale, src_zp, dst_zp;
-    long total;     // logical elements
-    int inner_elems; // elements per lane along order[0] (direct kernel)
-    // tiled kernel: the two tile dims and the number of tiles along each
-    int dim_s, dim_d;
-    long tiles_s, tiles_d, outer;
+    const void *qp[NQ]; // parameter tensors, null = absent
+    const void *dst_zp; // one s32, null = absent
+    int qdt[NQ];
+    int elems;          // elements per lane along `a`: 1, 2 or 4
+    int src_vec;        // the `elems` src elements of a lane are one aligned vector load
+    int packed;         // ... and the dst elements one aligned vector store
+    int plain_copy;     // same data type, no attributes
+    rdim_t a;           // the dim lanes walk: smallest dst stride
+    rdim_t b;           // tiled kernel: the dim with src stride 1
+    rdim_t outer[RD];   // the remaining dims, any order
+    unsigned outer_total;
+    unsigned tiles_a, tiles_b;
 };
 
 __device__ __forceinline__ bool is_int_dt(int dt) {
@@ -56,75 +63,209 @@ __device__ __forceinline__ bool is_int_dt(int dt) {
             || dt == MI355_DT_U4;
 }
 
-// idx[dim] = v / idx[dim] += v without a run-time array index (which would move
-// the index vector to private memory)
-__device__ __forceinline__ void idx_set(long (&idx)[RD], int dim, long v) {
-#pragma unroll
-    for (int d = 0; d < RD; ++d)
-        if (d == dim) idx[d] = v;
-}
-__device__ __forceinline__ void idx_add(long (&idx)[RD], int dim, long v) {
-#pragma unroll
-    for (int d = 0; d < RD; ++d)
-        if (d == dim) idx[d] += v;
-}
+struct rbase_t { // offsets contributed by the outer dims
+    long so, dof;
+    long q[NQ];
+};
 
-// (RT / QT: the structures are read in place from the kernel argument segment)
-template <class QT>
-__device__ __forceinline__ long rq_off(const QT &q, const long (&idx)[RD], int ndims) {
-    long off = 0;
-#pragma unroll
-    for (int d = 0; d < RD; ++d)
-        if (d < ndims && q.stride[d]) off += (idx[d] / q.group[d]) * q.stride[d];
-    return off;
-}
-
-// the converted element at logical index idx, as the raw bits of the dst type
+// (RT: the structure is read in place from the kernel argument segment)
 template <class RT>
-__device__ __forceinline__ uint32_t reorder_value(const RT &R, const long (&idx)[RD]) {
-    long so = 0, dof = 0;
+__device__ __forceinline__ rbase_t outer_base(const RT &R, unsigned o) {
+    rbase_t B;
+    B.so = 0; B.dof = 0;
 #pragma unroll
-    for (int d = 0; d < RD; ++d)
-        if (d < R.ndims) {
-            so += idx[d] * R.ss[d];
-            dof += idx[d] * R.ds[d];
-        }
-    float x;
-    if (R.src_dt == MI355_DT_E8M0) {
-        x = load_float(MI355_DT_E8M0, R.src, so);
-    } else {
-        int zp = 0;
-        if (R.src_zp.present)
-            zp = (int)load_float(R.src_zp.dt, R.src_zp.p, rq_off(R.src_zp, idx, R.ndims));
-        if (is_int_dt(R.src_dt)) x = (float)(load_int(R.src_dt, R.src, so) - zp);
-        else x = load_float(R.src_dt, R.src, so) - (float)zp;
-        if (R.src_scale.present)
-            x = load_float(R.src_scale.dt, R.src_scale.p, rq_off(R.src_scale, idx, R.ndims)) * x;
-        if (R.beta != 0.f) x += R.beta * load_float(R.dst_dt, R.dst, dof);
-        if (R.dst_scale.present || R.dst_zp.present) {
-            float dsc = 1.f;
-            int dzp = 0;
-            if (R.dst_scale.present)
-                dsc = load_float(R.dst_scale.dt, R.dst_scale.p, rq_off(R.dst_scale, idx, R.ndims));
-            if (R.dst_zp.present) dzp = load_int(R.dst_zp.dt, R.dst_zp.p, 0);
-            x = x / dsc + (float)dzp;
-        }
+    for (int k = 0; k < NQ; ++k) B.q[k] = 0;
+    for (int i = 0; i < R.n_outer; ++i) {
+        const unsigned n = R.outer[i].n;
+        const unsigned q = o / n, r = o - q * n;
+        o = q;
+        B.so += (long)r * R.outer[i].ss;
+        B.dof += (long)r * R.outer[i].ds;
+#pragma unroll
+        for (int k = 0; k < NQ; ++k)
+            if (R.outer[i].qs[k]) B.q[k] += (long)(r / R.outer[i].qg[k]) * R.outer[i].qs[k];
     }
-    switch (R.dst_dt) {
-        case MI355_DT_S4: return (uint32_t)(int)__builtin_rintf(sat(x, -8.f, 7.f)) & 0xfu;
-        case MI355_DT_U4: return (uint32_t)(int)__builtin_rintf(sat(x, 0.f, 15.f)) & 0xfu;
-        case MI355_DT_F4_E2M1: return f32_to_e2m1(x);
-        default: return cvt_store_bits(R.dst_dt, x);
+    return B;
+}
+
+template <class DT_>
+__device__ __forceinline__ void add_dim(rbase_t &B, const DT_ &d, unsigned i) {
+    B.so += (long)i * d.ss;
+    B.dof += (long)i * d.ds;
+#pragma unroll
+    for (int k = 0; k < NQ; ++k)
+        if (d.qs[k]) B.q[k] += (long)(d.qg[k] == 1 ? i : i / d.qg[k]) * d.qs[k];
+}
+
+// offsets of the N consecutive indices i .. i+N-1 along dim d
+template <int N, class DT_>
+__device__ __forceinline__ void add_dim_run(rbase_t (&B)[N], const rbase_t &B0, const DT_ &d, unsigned i) {
+    B[0] = B0;
+    add_dim(B[0], d, i);
+#pragma unroll
+    for (int e = 1; e < N; ++e) {
+        B[e].so = B[e - 1].so + d.ss;
+        B[e].dof = B[e - 1].dof + d.ds;
+#pragma unroll
+        for (int k = 0; k < NQ; ++k) {
+            B[e].q[k] = B[e - 1].q[k];
+            if (d.qs[k]) {
+                if (d.qg[k] == 1) B[e].q[k] += d.qs[k];
+                else B[e].q[k] = B0.q[k] + (long)((i + e) / d.qg[k]) * d.qs[k];
+            }
+        }
     }
 }
 
-// store n (1, 2 or 4) consecutive dst elements starting at element offset off
+// raw storage bits of one element -> its value (8-bit and wider types)
+__device__ __forceinline__ float raw_to_float(int dt, uint32_t w) {
+    switch (dt) {
+        case MI355_DT_F32: return u2f(w);
+        case MI355_DT_BF16: return bf16_to_f32((uint16_t)w);
+        case MI355_DT_F16: return f16_to_f32((uint16_t)w);
+        case MI355_DT_F8_E4M3: return e4m3_to_f32((uint8_t)w);
+        case MI355_DT_F8_E5M2: return e5m2_to_f32((uint8_t)w);
+        case MI355_DT_E8M0: return e8m0_to_f32((uint8_t)w);
+        case MI355_DT_F4_E2M1: return e2m1_to_f32((uint8_t)(w & 0xf));
+        default: return 0.f;
+    }
+}
+__device__ __forceinline__ int raw_to_int(int dt, uint32_t w) {
+    switch (dt) {
+        case MI355_DT_S32: return (int)w;
+        case MI355_DT_S8: return (int)(int8_t)w;
+        case MI355_DT_U8: return (int)(uint8_t)w;
+        case MI355_DT_S4: return s4_to_int((uint8_t)(w & 0xf));
+        default: return (int)(w & 0xf); // u4
+    }
+}
+
+__device__ __forceinline__ uint32_t load_raw(int dt, const void *p, long off) {
+    const int bits = dt_bits(dt);
+    if (bits == 32) return ((const uint32_t *)p)[off];
+    if (bits == 16) return ((const uint16_t *)p)[off];
+    if (bits == 8) return ((const uint8_t *)p)[off];
+    return nibble_get(p, off);
+}
+
+// The reference's arithmetic (see the head of this file) on N elements at once:
+// raw[e] holds the src storage bits, B[e] the offsets of element e in every
+// tensor.  Every data-type dispatch is uniform over the wavefront and is taken
+// once for the N elements.
+template <int N, class RT>
+__device__ __forceinline__ void convert(const RT &R, const uint32_t (&raw)[N], const rbase_t (&B)[N], uint32_t (&w)[N]) {
+    if (R.plain_copy) { // same type, no attributes: the bits move unchanged
+#pragma unroll
+        for (int e = 0; e < N; ++e) w[e] = raw[e];
+        return;
+    }
+    float x[N];
+    const int sdt = R.src_dt;
+    if (is_int_dt(sdt)) {
+        int v[N];
+        if (sdt == MI355_DT_S8) {
+#pragma unroll
+            for (int e = 0; e < N; ++e) v[e] = (int)(int8_t)raw[e];
+        } else if (sdt == MI355_DT_U8) {
+#pragma unroll
+            for (int e = 0; e < N; ++e) v[e] = (int)(uint8_t)raw[e];
+        } else if (sdt == MI355_DT_S32) {
+#pragma unroll
+            for (int e = 0; e < N; ++e) v[e] = (int)raw[e];
+        } else if (sdt == MI355_DT_S4) {
+#pragma unroll
+            for (int e = 0; e < N; ++e) v[e] = s4_to_int((uint8_t)(raw[e] & 0xf));
+        } else {
+#pragma unroll
+            for (int e = 0; e < N; ++e) v[e] = (int)(raw[e] & 0xf);
+        }
+        if (R.qp[2]) {
+#pragma unroll
+            for (int e = 0; e < N; ++e) v[e] -= (int)load_float(R.qdt[2], R.qp[2], B[e].q[2]);
+        }
+#pragma unroll
+        for (int e = 0; e < N; ++e) x[e] = (float)v[e];
+    } else if (sdt == MI355_DT_F32) {
+#pragma unroll
+        for (int e = 0; e < N; ++e) x[e] = u2f(raw[e]);
+    } else if (sdt == MI355_DT_BF16) {
+#pragma unroll
+        for (int e = 0; e < N; ++e) x[e] = bf16_to_f32((uint16_t)raw[e]);
+    } else if (sdt == MI355_DT_F16) {
+#pragma unroll
+        for (int e = 0; e < N; ++e) x[e] = f16_to_f32((uint16_t)raw[e]);
+    } else {
+#pragma unroll
+        for (int e = 0; e < N; ++e) x[e] = raw_to_float(sdt, raw[e]);
+    }
+    if (sdt != MI355_DT_E8M0) { // e8m0 sources are converted without arithmetic
+        if (R.qp[0]) {
+            const int qdt = R.qdt[0];
+            if (qdt == MI355_DT_F32) {
+#pragma unroll
+                for (int e = 0; e < N; ++e) x[e] = ((const float *)R.qp[0])[B[e].q[0]] * x[e];
+            } else {
+#pragma unroll
+                for (int e = 0; e < N; ++e) x[e] = load_float(qdt, R.qp[0], B[e].q[0]) * x[e];
+            }
+        }
+        if (R.beta != 0.f) {
+#pragma unroll
+            for (int e = 0; e < N; ++e) x[e] += R.beta * load_float(R.dst_dt, R.dst, B[e].dof);
+        }
+        if (R.qp[1] || R.dst_zp) {
+            const float dzp = R.dst_zp ? (float)*(const int *)R.dst_zp : 0.f;
+            if (R.qp[1]) {
+#pragma unroll
+                for (int e = 0; e < N; ++e) x[e] = x[e] / load_float(R.qdt[1], R.qp[1], B[e].q[1]) + dzp;
+            } else {
+#pragma unroll
+                for (int e = 0; e < N; ++e) x[e] = x[e] / 1.f + dzp;
+            }
+        }
+    }
+    const int ddt = R.dst_dt;
+    if (ddt == MI355_DT_S8) {
+#pragma unroll
+        for (int e = 0; e < N; ++e) w[e] = (uint32_t)(int)__builtin_rintf(sat(x[e], -128.f, 127.f)) & 0xffu;
+    } else if (ddt == MI355_DT_U8) {
+#pragma unroll
+        for (int e = 0; e < N; ++e) w[e] = (uint32_t)(int)__builtin_rintf(sat(x[e], 0.f, 255.f)) & 0xffu;
+    } else if (ddt == MI355_DT_F32) {
+#pragma unroll
+        for (int e = 0; e < N; ++e) w[e] = f2u(x[e]);
+    } else if (ddt == MI355_DT_BF16) {
+#pragma unroll
+        for (int e = 0; e < N; ++e) w[e] = f32_to_bf16(x[e]);
+    } else if (ddt == MI355_DT_F16) {
+#pragma unroll
+        for (int e = 0; e < N; ++e) w[e] = f32_to_f16(x[e]);
+    } else if (ddt == MI355_DT_S4) {
+#pragma unroll
+        for (int e = 0; e < N; ++e) w[e] = (uint32_t)(int)__builtin_rintf(sat(x[e], -8.f, 7.f)) & 0xfu;
+    } else if (ddt == MI355_DT_U4) {
+#pragma unroll
+        for (int e = 0; e < N; ++e) w[e] = (uint32_t)(int)__builtin_rintf(sat(x[e], 0.f, 15.f)) & 0xfu;
+    } else if (ddt == MI355_DT_F4_E2M1) {
+#pragma unroll
+        for (int e = 0; e < N; ++e) w[e] = f32_to_e2m1(x[e]);
+    } else {
+#pragma unroll
+        for (int e = 0; e < N; ++e) w[e] = cvt_store_bits(ddt, x[e]);
+    }
+}
+
+// store N (1, 2 or 4) consecutive dst elements starting at element offset off
 template <int N>
 __device__ __forceinline__ void store_bits(int dt, void *dst, long off, const uint32_t (&w)[N], bool packed) {
     const int bits = dt_bits(dt);
     if (bits == 4) {
         // off is even and the N nibbles fill whole bytes
         uint8_t *p = (uint8_t *)dst + (off >> 1);
+        if (N == 4 && packed) {
+            *(uint16_t *)p = (uint16_t)(w[0] | (w[1] << 4) | (w[2] << 8) | (w[3] << 12));
+            return;
+        }
 #pragma unroll
         for (int e = 0; e + 1 < N; e += 2) p[e >> 1] = (uint8_t)(w[e] | (w[e + 1] << 4));
         return;
@@ -152,99 +293,114 @@ __device__ __forceinline__ void store_bits(int dt, void *dst, long off, const ui
     }
 }
 
-// E elements per lane along the inner dim (dst stride 1 when E > 1)
-template <int E>
-__global__ void __launch_bounds__(256) reorder_direct_kernel(const reorder_t R_) {
-    const auto &R = *(const __attribute__((address_space(4))) reorder_t *)__builtin_amdgcn_kernarg_segment_ptr();
-    const long units = R.total / E;
-    for (long u = (long)blockIdx.x * blockDim.x + threadIdx.x; u < units; u += (long)gridDim.x * blockDim.x) {
-        long idx[RD] = {0, 0, 0, 0, 0, 0};
-        long rem = u;
-#pragma unroll
-        for (int k = 0; k < RD; ++k)
-            if (k < R.ndims) {
-                const int d = R.order[k];
-                const long n = k == 0 ? R.dims[d] / E : R.dims[d];
-                const long q = rem / n;
-                idx_set(idx, d, (rem - q * n) * (k == 0 ? E : 1));
-                rem = q;
-            }
-        const int di = R.order[0];
-        long dof = 0;
-#pragma unroll
-        for (int d = 0; d < RD; ++d)
-            if (d < R.ndims) dof += idx[d] * R.ds[d];
-        uint32_t w[E];
-#pragma unroll
-        for (int e = 0; e < E; ++e) {
-            w[e] = reorder_value(R, idx);
-            idx_add(idx, di, 1);
-        }
-        store_bits<E>(R.dst_dt, R.dst, dof, w, true);
+// four consecutive src elements as one vector load (off is a multiple of four)
+__device__ __forceinline__ void load_raw4(int dt, const void *p, long off, uint32_t (&w)[4]) {
+    const int bits = dt_bits(dt);
+    if (bits == 32) {
+        const uint4 v = *(const uint4 *)((const uint32_t *)p + off);
+        w[0] = v.x; w[1] = v.y; w[2] = v.z; w[3] = v.w;
+    } else if (bits == 16) {
+        const uint2 v = *(const uint2 *)((const uint16_t *)p + off);
+        w[0] = v.x & 0xffffu; w[1] = v.x >> 16; w[2] = v.y & 0xffffu; w[3] = v.y >> 16;
+    } else if (bits == 8) {
+        const uint32_t v = *(const uint32_t *)((const uint8_t *)p + off);
+        w[0] = v & 0xffu; w[1] = (v >> 8) & 0xffu; w[2] = (v >> 16) & 0xffu; w[3] = v >> 24;
+    } else {
+        const uint32_t v = *(const uint16_t *)((const uint8_t *)p + (off >> 1));
+        w[0] = v & 0xfu; w[1] = (v >> 4) & 0xfu; w[2] = (v >> 8) & 0xfu; w[3] = (v >> 12) & 0xfu;
     }
 }
 
-// 64 x 64 tile over (dim_s, dim_d); one workgroup per tile and outer index
+// grid: x over chunks of the dim `a`, y over the outer index.  E elements per
+// lane along `a` (dst stride 1 when E > 1).
+template <int E>
+__global__ void __launch_bounds__(256) reorder_direct_kernel(const reorder_t R_) {
+    const auto &R = *(const __attribute__((address_space(4))) reorder_t *)__builtin_amdgcn_kernarg_segment_ptr();
+    const unsigned units = R.a.n / E;
+    for (unsigned o = blockIdx.y; o < R.outer_total; o += gridDim.y) {
+        const rbase_t B0 = outer_base(R, o);
+        for (unsigned u = blockIdx.x * 256 + threadIdx.x; u < units; u += gridDim.x * 256) {
+            rbase_t B[E];
+            add_dim_run<E>(B, B0, R.a, u * E);
+            uint32_t raw[E], w[E];
+            bool loaded = false;
+            if constexpr (E == 4) {
+                if (R.src_vec) {
+                    load_raw4(R.src_dt, R.src, B[0].so, raw);
+                    loaded = true;
+                }
+            }
+            if (!loaded) {
+#pragma unroll
+                for (int e = 0; e < E; ++e) raw[e] = load_raw(R.src_dt, R.src, B[e].so);
+            }
+            convert<E>(R, raw, B, w);
+            store_bits<E>(R.dst_dt, R.dst, B[0].dof, w, R.packed);
+        }
+    }
+}
+
+// 64 x 64 tile over (b, a): b has src stride 1, a has dst stride 1.  grid: x
+// over the tiles, y over the outer index.
 __global__ void __launch_bounds__(256) reorder_tiled_kernel(const reorder_t R_) {
     const auto &R = *(const __attribute__((address_space(4))) reorder_t *)__builtin_amdgcn_kernarg_segment_ptr();
     __shared__ uint32_t tile[64][65];
-    const long per_outer = R.tiles_s * R.tiles_d;
-    const long ntiles = per_outer * R.outer;
+    const unsigned ntiles = R.tiles_a * R.tiles_b;
     const int tx = threadIdx.x & 63, ty = threadIdx.x >> 6;
-    for (long t = blockIdx.x; t < ntiles; t += gridDim.x) {
-        long idx[RD] = {0, 0, 0, 0, 0, 0};
-        long rem = t / per_outer;
-        const long in_outer = t - rem * per_outer;
-        // the other dims, fastest first in dst order
+    for (unsigned o = blockIdx.y; o < R.outer_total; o += gridDim.y) {
+        const rbase_t B0 = outer_base(R, o);
+        for (unsigned t = blockIdx.x; t < ntiles; t += gridDim.x) {
+            const unsigned tb = t % R.tiles_b, ta = t / R.tiles_b;
+            const unsigned b0 = tb * 64, a0 = ta * 64;
+            // read: lanes along b (src unit stride)
+            // (four rows per pass: four loads in flight, one dispatch for the four)
+            for (int i0 = ty * 4; i0 < 64; i0 += 16) {
+                rbase_t B[4];
+                uint32_t raw[4], v[4];
+                rbase_t Bb = B0;
+                const unsigned ib = b0 + tx < R.b.n ? b0 + tx : R.b.n - 1; // clamped, masked below
+                add_dim(Bb, R.b, ib);
+                if (a0 + i0 + 4 <= R.a.n) {
+                    add_dim_run<4>(B, Bb, R.a, a0 + i0);
+                } else { // ragged last tile along a: clamped, masked below
 #pragma unroll
-        for (int k = 0; k < RD; ++k)
-            if (k < R.ndims) {
-                const int d = R.order[k];
-                if (d != R.dim_s && d != R.dim_d) {
-                    const long q = rem / R.dims[d];
-                    idx_set(idx, d, rem - q * R.dims[d]);
-                    rem = q;
+                    for (int k = 0; k < 4; ++k) {
+                        B[k] = Bb;
+                        add_dim(B[k], R.a, a0 + i0 + k < R.a.n ? a0 + i0 + k : R.a.n - 1);
+                    }
                 }
-            }
-        const long s0 = (in_outer % R.tiles_s) * 64, d0 = (in_outer / R.tiles_s) * 64;
-        // read: lanes along the src unit-stride dim
-        for (int i = ty; i < 64; i += 4) {
-            idx_set(idx, R.dim_s, s0 + tx);
-            idx_set(idx, R.dim_d, d0 + i);
-            uint32_t v = 0;
-            if (s0 + tx < R.dims[R.dim_s] && d0 + i < R.dims[R.dim_d]) v = reorder_value(R, idx);
-            tile[i][tx] = v;
-        }
-        __syncthreads();
-        // write: lanes along the dst unit-stride dim, four elements each
-        const int lx = (threadIdx.x & 15) * 4, ly = threadIdx.x >> 4;
-        for (int i = ly; i < 64; i += 16) {
-            const long is = s0 + i, id = d0 + lx;
-            if (is < R.dims[R.dim_s] && id < R.dims[R.dim_d]) {
-                idx_set(idx, R.dim_s, is);
-                idx_set(idx, R.dim_d, id);
-                long dof = 0;
 #pragma unroll
-                for (int d = 0; d < RD; ++d)
-                    if (d < R.ndims) dof += idx[d] * R.ds[d];
-                const uint32_t w[4] = {tile[lx][i], tile[lx + 1][i], tile[lx + 2][i], tile[lx + 3][i]};
-                if (id + 4 <= R.dims[R.dim_d]) {
-                    store_bits<4>(R.dst_dt, R.dst, dof, w, R.inner_elems == 4);
-                } else { // ragged edge of the dst dim: dims[dim_d] is even for 4-bit types
-                    const int left = (int)(R.dims[R.dim_d] - id);
-                    if (dt_bits(R.dst_dt) == 4) {
-                        const uint32_t w2[2] = {w[0], w[1]};
-                        if (left >= 2) store_bits<2>(R.dst_dt, R.dst, dof, w2, false);
-                    } else {
-                        for (int e = 0; e < left; ++e) {
-                            const uint32_t w1[1] = {w[e]};
-                            store_bits<1>(R.dst_dt, R.dst, dof + e, w1, false);
+                for (int k = 0; k < 4; ++k) raw[k] = load_raw(R.src_dt, R.src, B[k].so);
+                convert<4>(R, raw, B, v);
+#pragma unroll
+                for (int k = 0; k < 4; ++k) tile[i0 + k][tx] = v[k];
+            }
+            __syncthreads();
+            // write: lanes along a (dst unit stride), four elements each
+            const int lx = (threadIdx.x & 15) * 4, ly = threadIdx.x >> 4;
+            for (int i = ly; i < 64; i += 16) {
+                const unsigned ib = b0 + i, ia = a0 + lx;
+                if (ib < R.b.n && ia < R.a.n) {
+                    const long dof = B0.dof + (long)ib * R.b.ds + (long)ia * R.a.ds;
+                    const uint32_t w[4] = {tile[lx][i], tile[lx + 1][i], tile[lx + 2][i], tile[lx + 3][i]};
+                    if (ia + 4 <= R.a.n) {
+                        store_bits<4>(R.dst_dt, R.dst, dof, w, R.packed);
+                    } else { // ragged edge: the extent is even for 4-bit types
+                        const int left = (int)(R.a.n - ia);
+                        if (dt_bits(R.dst_dt) == 4) {
+                            const uint32_t w2[2] = {w[0], w[1]};
+                            if (left >= 2) store_bits<2>(R.dst_dt, R.dst, dof, w2, false);
+                        } else {
+                            for (int e = 0; e < left; ++e) {
+                                const uint32_t w1[1] = {w[e]};
+                                store_bits<1>(R.dst_dt, R.dst, dof + e, w1, false);
+                            }
                         }
                     }
                 }
             }
+            __syncthreads();
         }
-        __syncthreads();
     }
 }
 
@@ -257,22 +413,20 @@ bool dt_ok(int dt) {
     }
 }
 
-// quantization parameter tensor strides over the tensor's dims
+// strides of a quantization parameter tensor along the tensor's dims: dense
+// row-major over the masked dims, the last two divided by the groups
 // (quant_entry_t::get_md, src/common/primitive_attr_quant.hpp:116-140)
-void fill_rq(rq_t &q, const mi355_quant_t &m, const void *p, int ndims, const int64_t *dims) {
-    q.p = p;
-    q.dt = m.dt;
-    q.present = m.dt != MI355_DT_UNDEF;
-    long stride = 1;
+void quant_strides(const mi355_quant_t &m, int ndims, const int64_t *dims, long (&stride)[RD], long (&group)[RD]) {
+    long st = 1;
     for (int d = RD - 1; d >= 0; --d) {
-        q.stride[d] = 0;
-        q.group[d] = 1;
-        if (d >= ndims || !q.present) continue;
-        if (d == ndims - 2) q.group[d] = m.group[0];
-        if (d == ndims - 1) q.group[d] = m.group[1];
+        stride[d] = 0;
+        group[d] = 1;
+        if (d >= ndims || m.dt == MI355_DT_UNDEF) continue;
+        if (d == ndims - 2) group[d] = m.group[0];
+        if (d == ndims - 1) group[d] = m.group[1];
         if (m.mask & (1 << d)) {
-            q.stride[d] = stride;
-            stride *= dims[d] / q.group[d];
+            stride[d] = st;
+            st *= dims[d] / group[d];
         }
     }
 }
@@ -350,40 +504,13 @@ extern "C" int mi355_reorder_launch(const mi355_reorder_desc_t *desc, const mi35
         return MI355_INVALID_ARGUMENTS;
     }
     const mi355_reorder_desc_t &d = *desc;
-    reorder_t R {};
-    R.ndims = d.ndims;
-    R.src_dt = d.src_dt;
-    R.dst_dt = d.dst_dt;
-    R.beta = d.beta;
-    R.src = args->src;
-    R.dst = args->dst;
-    R.total = 1;
-    for (int i = 0; i < RD; ++i) {
-        R.dims[i] = i < d.ndims ? d.dims[i] : 1;
-        R.ss[i] = i < d.ndims ? d.src_stride[i] : 0;
-        R.ds[i] = i < d.ndims ? d.dst_stride[i] : 0;
-        R.order[i] = i;
-        R.total *= R.dims[i];
-    }
-    if (R.total == 0) return MI355_SUCCESS;
+    long total = 1;
+    for (int i = 0; i < d.ndims; ++i) total *= d.dims[i];
+    if (total == 0) return MI355_SUCCESS;
     if (!args->src || !args->dst) {
         set_error("reorder: null tensor");
         return MI355_INVALID_ARGUMENTS;
     }
-    // walk order: ascending dst stride, dims of size 1 last
-    for (int a = 0; a < d.ndims; ++a)
-        for (int b = a + 1; b < d.ndims; ++b) {
-            const int x = R.order[a], y = R.order[b];
-            const bool x_one = R.dims[x] == 1, y_one = R.dims[y] == 1;
-            if ((x_one && !y_one) || (x_one == y_one && R.ds[y] < R.ds[x])) {
-                R.order[a] = y;
-                R.order[b] = x;
-            }
-        }
-    fill_rq(R.src_scale, d.src_scale, args->src_scale, d.ndims, d.dims);
-    fill_rq(R.dst_scale, d.dst_scale, args->dst_scale, d.ndims, d.dims);
-    fill_rq(R.src_zp, d.src_zp, args->src_zp, d.ndims, d.dims);
-    fill_rq(R.dst_zp, d.dst_zp, args->dst_zp, d.ndims, d.dims);
     const mi355_quant_t *qs[4] = {&d.src_scale, &d.dst_scale, &d.src_zp, &d.dst_zp};
     const void *qp[4] = {args->src_scale, args->dst_scale, args->src_zp, args->dst_zp};
     for (int i = 0; i < 4; ++i)
@@ -391,49 +518,121 @@ extern "C" int mi355_reorder_launch(const mi355_reorder_desc_t *desc, const mi35
             set_error("reorder: a declared scale or zero point tensor is null");
             return MI355_INVALID_ARGUMENTS;
         }
+    for (int i = 0; i < d.ndims; ++i)
+        if (d.dims[i] >= (1L << 31)) return MI355_UNIMPLEMENTED;
 
-    const int di = R.order[0];
-    const bool dst_unit = R.ds[di] == 1;
-    const int dbits = dt_bits(d.dst_dt);
-    // packed stores of four need the pointer and every other stride aligned
-    auto packable = [&](int dim) {
-        if (R.ds[dim] != 1 || R.dims[dim] % 4) return false;
-        const long bytes4 = dbits / 2; // bytes of four elements
-        if (dbits != 4 && ((uintptr_t)R.dst % (bytes4 ? bytes4 : 1))) return false;
-        for (int i = 0; i < d.ndims; ++i)
-            if (i != dim && R.dims[i] > 1 && R.ds[i] % 4) return false;
+    reorder_t R {};
+    R.src_dt = d.src_dt;
+    R.dst_dt = d.dst_dt;
+    R.beta = d.beta;
+    R.src = args->src;
+    R.dst = args->dst;
+    long qstride[NQ][RD], qgroup[NQ][RD];
+    for (int k = 0; k < NQ; ++k) {
+        quant_strides(*qs[k], d.ndims, d.dims, qstride[k], qgroup[k]);
+        R.qp[k] = qs[k]->dt != MI355_DT_UNDEF ? qp[k] : nullptr;
+        R.qdt[k] = qs[k]->dt;
+    }
+    R.dst_zp = d.dst_zp.dt != MI355_DT_UNDEF ? args->dst_zp : nullptr;
+    auto make_dim = [&](int i) {
+        rdim_t r {};
+        r.n = (unsigned)d.dims[i];
+        r.ss = d.src_stride[i];
+        r.ds = d.dst_stride[i];
+        for (int k = 0; k < NQ; ++k) {
+            r.qs[k] = qstride[k][i];
+            r.qg[k] = (unsigned)qgroup[k][i];
+        }
+        return r;
+    };
+    // dims of extent > 1, ordered by dst stride; neighbours that are contiguous
+    // in both tensors (and in every parameter tensor) merge into one dim, so a
+    // plain conversion of a dense tensor becomes one long row
+    rdim_t v[RD];
+    int nv = 0;
+    for (int i = 0; i < d.ndims; ++i)
+        if (d.dims[i] > 1) v[nv++] = make_dim(i);
+    for (int x = 0; x < nv; ++x)
+        for (int y = x + 1; y < nv; ++y)
+            if (v[y].ds < v[x].ds) {
+                const rdim_t t = v[x];
+                v[x] = v[y];
+                v[y] = t;
+            }
+    for (int x = 0; x + 1 < nv;) {
+        const rdim_t &in = v[x], &out = v[x + 1];
+        bool ok = out.ss == in.ss * (long)in.n && out.ds == in.ds * (long)in.n
+                && (long)in.n * (long)out.n < (1L << 31);
+        for (int k = 0; k < NQ && ok; ++k)
+            ok = (in.qs[k] == 0 && out.qs[k] == 0)
+                    || (in.qg[k] == 1 && out.qg[k] == 1 && in.qs[k] != 0 && out.qs[k] == in.qs[k] * (long)in.n);
+        if (!ok) {
+            ++x;
+            continue;
+        }
+        v[x].n = in.n * out.n;
+        for (int y = x + 1; y + 1 < nv; ++y) v[y] = v[y + 1];
+        --nv;
+    }
+    if (nv == 0) { // a single element
+        v[0] = make_dim(d.ndims - 1);
+        nv = 1;
+    }
+    // v[0] has the smallest dst stride: the dim lanes walk.  A transposition:
+    // src is unit-stride along another dim.
+    const int da = 0;
+    int db = -1;
+    for (int i = 1; i < nv; ++i)
+        if (v[i].ss == 1) db = i;
+    const bool tiled = v[da].ds == 1 && db > 0 && v[da].n >= 16 && v[db].n >= 16;
+    if (!tiled) db = -1;
+    R.a = v[da];
+    if (tiled) R.b = v[db];
+    long outer = 1;
+    for (int i = 1; i < nv; ++i)
+        if (i != db) {
+            R.outer[R.n_outer++] = v[i];
+            outer *= v[i].n;
+        }
+    if (outer >= (1L << 31)) return MI355_UNIMPLEMENTED;
+    R.outer_total = (unsigned)outer;
+
+    const int dbits = dt_bits(d.dst_dt), sbits = dt_bits(d.src_dt);
+    // four elements per lane along `a` as one aligned vector: unit stride, an
+    // extent that divides, every other stride and the pointer aligned to it
+    auto vec4_ok = [&](const void *p, bool src_side, int bits) {
+        const long sa = src_side ? v[da].ss : v[da].ds;
+        if (sa != 1 || v[da].n % 4) return false;
+        const long bytes4 = bits / 2 ? bits / 2 : 1;
+        if ((uintptr_t)p % (size_t)bytes4) return false;
+        for (int i = 1; i < nv; ++i)
+            if ((src_side ? v[i].ss : v[i].ds) % 4) return false;
         return true;
     };
-    // a transposition: src is unit-stride along another dim than dst
-    int dim_s = -1;
-    for (int i = 0; i < d.ndims; ++i)
-        if (R.ss[i] == 1 && R.dims[i] > 1) dim_s = i;
+    R.plain_copy = d.src_dt == d.dst_dt && d.beta == 0.f && d.src_scale.dt == MI355_DT_UNDEF
+            && d.dst_scale.dt == MI355_DT_UNDEF && d.src_zp.dt == MI355_DT_UNDEF && d.dst_zp.dt == MI355_DT_UNDEF;
+    R.packed = vec4_ok(R.dst, false, dbits);
+    R.src_vec = vec4_ok(R.src, true, sbits);
     hipStream_t hs = (hipStream_t)stream;
-    if (dst_unit && dim_s >= 0 && dim_s != di && R.dims[di] >= 16 && R.dims[dim_s] >= 16) {
-        R.dim_s = dim_s;
-        R.dim_d = di;
-        R.tiles_s = (R.dims[dim_s] + 63) / 64;
-        R.tiles_d = (R.dims[di] + 63) / 64;
-        R.outer = R.total / (R.dims[dim_s] * R.dims[di]);
-        R.inner_elems = packable(di) ? 4 : 1;
-        if (dbits == 4 && R.inner_elems != 4) {
-            // nibble pairs are stored as bytes: needs even offsets, which check() ensured
-            R.inner_elems = 2;
-        }
-        long blocks = R.tiles_s * R.tiles_d * R.outer;
-        if (blocks > (1 << 20)) blocks = 1 << 20;
-        hipLaunchKernelGGL(reorder_tiled_kernel, dim3((unsigned)blocks), dim3(256), 0, hs, R);
+    const unsigned gy = (unsigned)(outer < 65535 ? outer : 65535);
+    if (tiled) {
+        R.tiles_a = (R.a.n + 63) / 64;
+        R.tiles_b = (R.b.n + 63) / 64;
+        R.elems = 4;
+        long gx = (long)R.tiles_a * R.tiles_b;
+        if (gx > (1 << 20)) gx = 1 << 20;
+        hipLaunchKernelGGL(reorder_tiled_kernel, dim3((unsigned)gx, gy), dim3(256), 0, hs, R);
     } else {
         int E = 1;
-        if (dst_unit && packable(di)) E = 4;
+        if (R.packed) E = 4;
         else if (dbits == 4) E = 2;
-        R.inner_elems = E;
-        const long units = R.total / E;
-        long blocks = (units + 255) / 256;
-        if (blocks > (1 << 20)) blocks = 1 << 20;
-        if (E == 4) hipLaunchKernelGGL(reorder_direct_kernel<4>, dim3((unsigned)blocks), dim3(256), 0, hs, R);
-        else if (E == 2) hipLaunchKernelGGL(reorder_direct_kernel<2>, dim3((unsigned)blocks), dim3(256), 0, hs, R);
-        else hipLaunchKernelGGL(reorder_direct_kernel<1>, dim3((unsigned)blocks), dim3(256), 0, hs, R);
+        R.elems = E;
+        long gx = ((long)R.a.n / E + 255) / 256;
+        if (gx > (1 << 20)) gx = 1 << 20;
+        if (gx < 1) gx = 1;
+        if (E == 4) hipLaunchKernelGGL(reorder_direct_kernel<4>, dim3((unsigned)gx, gy), dim3(256), 0, hs, R);
+        else if (E == 2) hipLaunchKernelGGL(reorder_direct_kernel<2>, dim3((unsigned)gx, gy), dim3(256), 0, hs, R);
+        else hipLaunchKernelGGL(reorder_direct_kernel<1>, dim3((unsigned)gx, gy), dim3(256), 0, hs, R);
     }
     if (hipGetLastError() != hipSuccess) {
         set_error("reorder: launch failed");

@@ -26,6 +26,7 @@ kind_sum, kind_eltwise, kind_binary, kind_matmul, kind_prelu = 4, 7, 13, 14, 18
 query_impl_info_str, query_src_md, query_weights_md, query_dst_md, query_scratchpad_md = 8, 129, 131, 133, 136
 query_ndims_s32, query_dims, query_data_type, query_strides, query_memory_consumption = 256, 257, 258, 14, 6
 ARG_SRC, ARG_SRC_1, ARG_DST, ARG_WEIGHTS, ARG_BIAS, ARG_SCRATCHPAD = 1, 2, 17, 33, 41, 80
+ARG_FROM, ARG_TO = ARG_SRC, ARG_DST
 ARG_ATTR_PRECOMPUTED_REDUCTIONS, ARG_ATTR_SCALES, ARG_ATTR_ZERO_POINTS = 512, 4096, 8192
 scratchpad_library, scratchpad_user = 0, 1
 fpmath_strict, fpmath_bf16, fpmath_f16, fpmath_any = 0, 1, 2, 3
@@ -246,6 +247,17 @@ class matmul_primitive_desc:
         return self.query_md(query_scratchpad_md)
 
 
+class reorder_primitive_desc(matmul_primitive_desc):
+    """dnnl::reorder::primitive_desc(src_engine, src_md, dst_engine, dst_md, attr)"""
+
+    def __init__(self, src_eng, src_md, dst_eng, dst_md, attr=None):
+        self.engine = dst_eng
+        self.h = C.c_void_p()
+        _check(lib().dnnl_reorder_primitive_desc_create(
+            C.byref(self.h), src_md.h, src_eng.h, dst_md.h, dst_eng.h, attr.h if attr else None),
+            "reorder_primitive_desc_create")
+
+
 class matmul:
     def __init__(self, pd):
         self.pd = pd
@@ -258,3 +270,7 @@ class matmul:
             arr[i].arg = k
             arr[i].memory = m.h
         _check(lib().dnnl_primitive_execute(self.h, strm.h, len(args), arr), "primitive_execute")
+
+
+class reorder(matmul):
+    """dnnl::reorder(pd); execute(stream, {ARG_FROM: src, ARG_TO: dst, ...})"""

@@ -181,6 +181,8 @@ struct dnnl_primitive_attr {
 };
 
 struct dnnl_primitive_desc {
+    dnnl_primitive_kind_t kind = dnnl_matmul;
+    mi355_reorder_desc_t rdesc; // kind == dnnl_reorder (src / dst hold the two tensors)
     dnnl_engine_t engine = nullptr;
     dnnl_memory_desc src, wei, bias, dst, scratchpad;
     bool with_bias = false;
@@ -1058,6 +1060,84 @@ DNNL_EXPORT dnnl_status_t dnnl_matmul_primitive_desc_create(dnnl_primitive_desc_
     return dnnl_success;
 }
 
+// ---- reorder primitive descriptor (src/common/reorder.cpp:67-170)
+DNNL_EXPORT dnnl_status_t dnnl_reorder_primitive_desc_create(dnnl_primitive_desc_t *reorder_primitive_desc,
+        const_dnnl_memory_desc_t src_desc, dnnl_engine_t src_engine, const_dnnl_memory_desc_t dst_desc,
+        dnnl_engine_t dst_engine, const_dnnl_primitive_attr_t attr) {
+    CHECK_ARG(reorder_primitive_desc && src_desc && dst_desc && src_engine && dst_engine);
+    // one device: no cross-engine copies
+    CHECK_UNIMPL(src_engine->kind == dnnl_gpu && dst_engine->kind == dnnl_gpu && src_engine->index == dst_engine->index);
+    CHECK_ARG(src_desc->kind != dnnl_format_kind_any && dst_desc->kind != dnnl_format_kind_any); // :81-84
+    // consistent_with: same logical dims (:91-92)
+    CHECK_ARG(src_desc->ndims == dst_desc->ndims && src_desc->ndims >= 1);
+    for (int i = 0; i < src_desc->ndims; ++i) CHECK_ARG(src_desc->dims[i] == dst_desc->dims[i]);
+    CHECK_UNIMPL(src_desc->ndims <= MI355_REORDER_MAX_DIMS);
+    std::unique_ptr<dnnl_primitive_desc> pd(new dnnl_primitive_desc);
+    if (attr) pd->attr = *attr;
+    pd->kind = dnnl_reorder;
+    pd->engine = dst_engine;
+    pd->src = *src_desc;
+    pd->dst = *dst_desc;
+    const dnnl_primitive_attr &a = pd->attr;
+    const int nd = src_desc->ndims;
+    // scales / zero points on src and dst only (:106-111); everything else is not a reorder attribute
+    for (const auto *m : {&a.scales, &a.zero_points})
+        for (const auto &kv : *m) CHECK_UNIMPL(kv.first == DNNL_ARG_SRC || kv.first == DNNL_ARG_DST);
+    CHECK_UNIMPL(a.reductions.empty());
+    mi355_reorder_desc_t &r = pd->rdesc;
+    memset(&r, 0, sizeof(r));
+    r.ndims = nd;
+    r.src_dt = (int)src_desc->dt;
+    r.dst_dt = (int)dst_desc->dt;
+    for (int i = 0; i < nd; ++i) {
+        r.dims[i] = src_desc->dims[i];
+        r.src_stride[i] = src_desc->strides[i];
+        r.dst_stride[i] = dst_desc->strides[i];
+    }
+    auto lower_q = [&](const quant_entry_t *q, mi355_quant_t &out, dnnl_data_type_t default_dt) -> dnnl_status_t {
+        out.dt = MI355_DT_UNDEF;
+        out.mask = 0;
+        out.group[0] = out.group[1] = 1;
+        if (!q) return dnnl_success;
+        CHECK_ARG(q->mask >= 0 && (q->mask >> nd) == 0);
+        out.dt = (int)(q->dt == dnnl_data_type_undef ? default_dt : q->dt);
+        out.mask = q->mask;
+        if (q->group_ndims == 2) {
+            CHECK_ARG(nd >= 2);
+            // groups divide the last two dims and the mask covers both (:118-140)
+            CHECK_ARG(IMPLICATION(q->groups[0] > 1, src_desc->dims[nd - 2] % q->groups[0] == 0));
+            CHECK_ARG(IMPLICATION(q->groups[1] > 1, src_desc->dims[nd - 1] % q->groups[1] == 0));
+            CHECK_ARG((q->mask & (1 << (nd - 1))) && (q->mask & (1 << (nd - 2))));
+            out.group[0] = q->groups[0];
+            out.group[1] = q->groups[1];
+        }
+        return dnnl_success;
+    };
+    dnnl_status_t st;
+    if ((st = lower_q(a.find(a.scales, DNNL_ARG_SRC), r.src_scale, dnnl_f32))) return st;
+    if ((st = lower_q(a.find(a.scales, DNNL_ARG_DST), r.dst_scale, dnnl_f32))) return st;
+    if ((st = lower_q(a.find(a.zero_points, DNNL_ARG_SRC), r.src_zp, dnnl_s32))) return st;
+    if ((st = lower_q(a.find(a.zero_points, DNNL_ARG_DST), r.dst_zp, dnnl_s32))) return st;
+    // 4-bit sources need a mask for their scales (:113-116)
+    if (r.src_scale.dt != MI355_DT_UNDEF && (src_desc->dt == dnnl_s4 || src_desc->dt == dnnl_u4))
+        CHECK_ARG(r.src_scale.mask > 0);
+    // post-ops: a single sum (simple_po_check, src/cpu/reorder/cpu_reorder_pd.hpp)
+    const auto &po = a.post_ops.entries;
+    CHECK_UNIMPL(po.size() <= 1);
+    if (po.size() == 1) {
+        CHECK_UNIMPL(po[0].kind == dnnl_sum && po[0].zero_point == 0);
+        r.beta = po[0].scale;
+    }
+    const int rc = mi355_reorder_query(&r);
+    if (rc != MI355_SUCCESS) return from_mi355(rc);
+    pd->impl_name = "hip:reorder:any";
+    pd->impls.assign(1, 0);
+    if (verbose_level() >= 1)
+        fprintf(stderr, "onednn_verbose,v1,primitive,create:dispatch,gpu,reorder,%s\n", pd->impl_name.c_str());
+    *reorder_primitive_desc = pd.release();
+    return dnnl_success;
+}
+
 DNNL_EXPORT dnnl_status_t dnnl_primitive_desc_clone(dnnl_primitive_desc_t *primitive_desc,
         const_dnnl_primitive_desc_t existing) {
     CHECK_ARG(primitive_desc && existing);
@@ -1068,6 +1148,7 @@ DNNL_EXPORT dnnl_status_t dnnl_primitive_desc_next_impl(dnnl_primitive_desc_t pd
     CHECK_ARG(pd);
     if (pd->impl_pos + 1 >= pd->impls.size()) return dnnl_last_impl_reached;
     ++pd->impl_pos;
+    if (pd->kind == dnnl_reorder) return dnnl_success;
     return select_impl(*pd);
 }
 DNNL_EXPORT dnnl_status_t dnnl_primitive_desc_get_attr(const_dnnl_primitive_desc_t pd, const_dnnl_primitive_attr_t *attr) {
@@ -1083,6 +1164,17 @@ DNNL_EXPORT const_dnnl_memory_desc_t dnnl_primitive_desc_query_md(const_dnnl_pri
         int index) {
     if (!pd) return nullptr;
     static const dnnl_memory_desc zero_md;
+    if (pd->kind == dnnl_reorder) {
+        switch (what) {
+            case dnnl_query_src_md: return index == 0 ? &pd->src : nullptr;
+            case dnnl_query_dst_md: return index == 0 ? &pd->dst : nullptr;
+            case dnnl_query_scratchpad_md: return index == 0 ? &pd->scratchpad : nullptr;
+            case dnnl_query_exec_arg_md:
+                return index == DNNL_ARG_FROM ? &pd->src : index == DNNL_ARG_TO ? &pd->dst
+                        : index == DNNL_ARG_SCRATCHPAD ? &pd->scratchpad : nullptr;
+            default: return nullptr;
+        }
+    }
     switch (what) {
         case dnnl_query_src_md: return index == 0 ? &pd->src : nullptr;
         case dnnl_query_weights_md: return index == 0 ? &pd->wei : index == 1 ? (pd->with_bias ? &pd->bias : &zero_md) : nullptr;
@@ -1105,8 +1197,10 @@ DNNL_EXPORT dnnl_status_t dnnl_primitive_desc_query(const_dnnl_primitive_desc_t 
     CHECK_ARG(pd && result);
     switch (what) {
         case dnnl_query_engine: *(dnnl_engine_t *)result = pd->engine; break;
-        case dnnl_query_primitive_kind: *(dnnl_primitive_kind_t *)result = dnnl_matmul; break;
-        case dnnl_query_num_of_inputs_s32: *(int32_t *)result = 2 + (pd->with_bias ? 1 : 0); break;
+        case dnnl_query_primitive_kind: *(dnnl_primitive_kind_t *)result = pd->kind; break;
+        case dnnl_query_num_of_inputs_s32:
+            *(int32_t *)result = pd->kind == dnnl_reorder ? 1 : 2 + (pd->with_bias ? 1 : 0);
+            break;
         case dnnl_query_num_of_outputs_s32: *(int32_t *)result = 1; break;
         case dnnl_query_memory_consumption_s64:
             *(int64_t *)result = pd->attr.scratchpad_mode == dnnl_scratchpad_mode_library ? (int64_t)pd->scratch_bytes : 0;
@@ -1175,6 +1269,34 @@ DNNL_EXPORT dnnl_status_t dnnl_primitive_execute(const_dnnl_primitive_t cprimiti
         *out = it->second->handle;
         return dnnl_success;
     };
+    if (pd.kind == dnnl_reorder) {
+        mi355_reorder_args_t R;
+        memset(&R, 0, sizeof(R));
+        dnnl_status_t rs;
+        void *q = nullptr;
+        if ((rs = handle(DNNL_ARG_FROM, true, &q))) return rs;
+        R.src = q;
+        if ((rs = handle(DNNL_ARG_TO, true, &q))) return rs;
+        R.dst = q;
+        if ((rs = handle(DNNL_ARG_ATTR_SCALES | DNNL_ARG_SRC, pd.rdesc.src_scale.dt != MI355_DT_UNDEF, &q))) return rs;
+        R.src_scale = q;
+        if ((rs = handle(DNNL_ARG_ATTR_SCALES | DNNL_ARG_DST, pd.rdesc.dst_scale.dt != MI355_DT_UNDEF, &q))) return rs;
+        R.dst_scale = q;
+        if ((rs = handle(DNNL_ARG_ATTR_ZERO_POINTS | DNNL_ARG_SRC, pd.rdesc.src_zp.dt != MI355_DT_UNDEF, &q))) return rs;
+        R.src_zp = q;
+        if ((rs = handle(DNNL_ARG_ATTR_ZERO_POINTS | DNNL_ARG_DST, pd.rdesc.dst_zp.dt != MI355_DT_UNDEF, &q))) return rs;
+        R.dst_zp = q;
+        if (mi355_device_set((int)pd.engine->index) != MI355_SUCCESS) return dnnl_runtime_error;
+        const auto t0 = std::chrono::steady_clock::now();
+        const int rc = mi355_reorder_launch(&pd.rdesc, &R, stream->hip_stream);
+        if (verbose_level() >= 2) {
+            mi355_stream_sync(stream->hip_stream);
+            const double ms = std::chrono::duration<double, std::milli>(std::chrono::steady_clock::now() - t0).count();
+            fprintf(stderr, "onednn_verbose,v1,primitive,exec,gpu,reorder,%s,undef,src:%s dst:%s,,,%g\n",
+                    pd.impl_name.c_str(), dt_name(pd.src.dt), dt_name(pd.dst.dt), ms);
+        }
+        return from_mi355(rc);
+    }
     mi355_matmul_args_t A;
     memset(&A, 0, sizeof(A));
     dnnl_status_t st;

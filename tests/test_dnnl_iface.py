@@ -218,3 +218,40 @@ def test_user_scratchpad_is_reported(eng):
     assert sp.ndims() == 1 and sp.dims()[0] >= 1024 * 1024
     lib_mode = make_pd(eng, 256, 1024, 1024, "u8", "s8", "s32")
     assert lib_mode.scratchpad_desc().ndims() == 0
+
+
+def test_reorder_primitive_desc_rules(eng):
+    """reorder_primitive_desc_create (src/common/reorder.cpp:67-170): status codes."""
+    f32 = md([8, 16], "f32")
+    s8t = md([8, 16], "s8", tag=dnnl.tag_ba)
+    pd = dnnl.reorder_primitive_desc(eng, f32, eng, s8t)
+    assert pd.impl_info_str() == "hip:reorder:any"
+    assert pd.query_md(dnnl.query_src_md).data_type() == DT["f32"]
+    assert pd.query_md(dnnl.query_dst_md).strides() == [1, 8]
+    assert not pd.next_impl()
+    # inconsistent dims
+    assert status_of(lambda: dnnl.reorder_primitive_desc(eng, f32, eng, md([16, 8], "s8"))) == dnnl.invalid_arguments
+    # format any is not a reorder input
+    any_md = dnnl.memory_desc([8, 16], DT["s8"], tag=dnnl.tag_any)
+    assert status_of(lambda: dnnl.reorder_primitive_desc(eng, f32, eng, any_md)) == dnnl.invalid_arguments
+    # zero points only with integer data
+    a = dnnl.primitive_attr()
+    a.set_zero_points(dnnl.ARG_SRC, 0)
+    assert status_of(lambda: dnnl.reorder_primitive_desc(eng, f32, eng, s8t, attr=a)) == dnnl.invalid_arguments
+    # scales on src and dst only
+    a = dnnl.primitive_attr()
+    a.set_scales(dnnl.ARG_WEIGHTS, 0)
+    assert status_of(lambda: dnnl.reorder_primitive_desc(eng, f32, eng, s8t, attr=a)) == dnnl.unimplemented
+    # groups must divide the dims and the mask must cover the last two dims
+    a = dnnl.primitive_attr()
+    a.set_scales(dnnl.ARG_SRC, 3, (3, 1))
+    u4 = md([8, 16], "u4")
+    assert status_of(lambda: dnnl.reorder_primitive_desc(eng, u4, eng, f32, attr=a)) == dnnl.invalid_arguments
+    a = dnnl.primitive_attr()
+    a.set_scales(dnnl.ARG_SRC, 3, (4, 1), DT["bf16"])
+    a.set_zero_points(dnnl.ARG_SRC, 3, (4, 1), DT["u4"])
+    assert dnnl.reorder_primitive_desc(eng, u4, eng, f32, attr=a).impl_info_str() == "hip:reorder:any"
+    # 4-bit sources need a mask for their scales
+    a = dnnl.primitive_attr()
+    a.set_scales(dnnl.ARG_SRC, 0)
+    assert status_of(lambda: dnnl.reorder_primitive_desc(eng, u4, eng, f32, attr=a)) == dnnl.invalid_arguments

@@ -131,3 +131,53 @@ def test_missing_argument_is_invalid_arguments(gpu):
     with pytest.raises(dnnl.error) as e:
         prim.execute(strm, bad)
     assert e.value.status == dnnl.invalid_arguments
+
+
+def test_quantize_and_prepack_weights_with_reorder_then_matmul(gpu, oracle):
+    """The flow of the reference's examples (examples/tutorials/matmul/
+    inference_int8_matmul.cpp, matmul_with_weight_only_quantization.cpp:181-189):
+    weights md with format `any`, ask the matmul pd which layout it wants,
+    bring the user's f32 row-major weights there with a reorder that also
+    quantizes them, then run the matmul on the reordered memory."""
+    from onednn_amd.reorder import ReorderProblem
+    from onednn_amd.problem import MatmulProblem, QuantParam
+    from oracle import binding as orc
+    M, K, N = 256, 512, 384
+    r = np.random.default_rng(77)
+    w_f32 = r.uniform(-1, 1, size=(K, N)).astype(np.float32)
+    wsc = (np.abs(w_f32).max(axis=0) / 127).astype(np.float32)            # per-N scales
+    src = r.integers(-100, 100, size=(M, K)).astype(np.int8)
+    eng = dnnl.engine(dnnl.gpu, 0)
+    strm = dnnl.stream(eng)
+    src_md = dnnl.memory_desc([M, K], DT["s8"], tag=dnnl.tag_ab)
+    wei_any = dnnl.memory_desc([K, N], DT["s8"], tag=dnnl.tag_any)
+    dst_md = dnnl.memory_desc([M, N], DT["f32"], tag=dnnl.tag_ab)
+    attr = dnnl.primitive_attr()
+    attr.set_scales(dnnl.ARG_WEIGHTS, 2)
+    pd = dnnl.matmul_primitive_desc(eng, src_md, wei_any, dst_md, attr=attr)
+    wei_md = pd.query_md(dnnl.query_weights_md)
+    assert wei_md.strides() == [1, K]                                    # K-contiguous for the MFMA kernels
+    # reorder: f32 ab -> s8 in the queried layout, dst = src / scale[n]
+    user_md = dnnl.memory_desc([K, N], DT["f32"], tag=dnnl.tag_ab)
+    rattr = dnnl.primitive_attr()
+    rattr.set_scales(dnnl.ARG_DST, 2)
+    rpd = dnnl.reorder_primitive_desc(eng, user_md, eng, wei_md, attr=rattr)
+    wsc_mem = dnnl.memory(dnnl.memory_desc([1, N], DT["f32"], tag=dnnl.tag_ab), eng, wsc)
+    wei_mem = dnnl.memory(wei_md, eng)
+    dnnl.reorder(rpd).execute(strm, {dnnl.ARG_FROM: dnnl.memory(user_md, eng, w_f32), dnnl.ARG_TO: wei_mem,
+                                     dnnl.ARG_ATTR_SCALES | dnnl.ARG_DST: wsc_mem})
+    dst = dnnl.memory(dst_md, eng)
+    dnnl.matmul(pd).execute(strm, {dnnl.ARG_SRC: dnnl.memory(src_md, eng, src), dnnl.ARG_WEIGHTS: wei_mem,
+                                   dnnl.ARG_DST: dst, dnnl.ARG_ATTR_SCALES | dnnl.ARG_WEIGHTS: wsc_mem})
+    strm.wait()
+    assert pd.impl_info_str().startswith("hip:mfma_i8")
+    # oracle: the same two steps on the CPU
+    rp = ReorderProblem(dims=(K, N), src_dt=cabi.DT_F32, dst_dt=cabi.DT_S8, src=w_f32, dst_stride=(1, K),
+                        quant={"dst_scale": QuantParam(cabi.DT_F32, 2, wsc)})
+    w_q = orc.reorder(rp)
+    assert np.array_equal(wei_mem.read(np.int8), w_q)
+    assert np.array_equal(w_q.reshape(N, K).T, np.rint(np.clip(w_f32 / wsc[None, :], -128, 127)).astype(np.int8))
+    mp = MatmulProblem(M=M, N=N, K=K, src_dt=cabi.DT_S8, wei_dt=cabi.DT_S8, dst_dt=cabi.DT_F32, src=src, wei=w_q,
+                       wei_stride=(K * N, 1, K), quant={"wei_scale": QuantParam(cabi.DT_F32, 4, wsc)})
+    want = oracle.run_oracle(mp)
+    assert_close(mp, dst.read(np.float32), want)
