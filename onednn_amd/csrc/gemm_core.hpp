@@ -124,9 +124,12 @@ struct tile_pos_t {
 // (8 of them, each with a private L2); give every XCD one contiguous run of
 // tiles, walked in bands of GM tile rows so that concurrently resident tiles
 // share A rows and B columns in that L2.
+// (A persistent form, one workgroup per CU walking ids blockIdx.x + k * gridDim.x,
+// measured the same as one workgroup per tile: the turnover between tiles is
+// ~6 us of 130.)
 template <class G>
-__device__ __forceinline__ tile_pos_t tile_position(int tiles_m, int tiles_n) {
-    const int nwg = gridDim.x, id = blockIdx.x;
+__device__ __forceinline__ tile_pos_t tile_position(int id, int tiles_m, int tiles_n) {
+    const int nwg = tiles_m * tiles_n;
     const int per = nwg / 8;
     const int tile = (nwg % 8 == 0) ? (id % 8) * per + id / 8 : id;
     constexpr int GM = 8;
@@ -215,7 +218,7 @@ __device__ __forceinline__ void main_loop_two_groups(Acc &acc, char *smem, const
     static_assert((NG - 2) * GROUP_DMAS < 64, "vmcnt range");
     const int t = threadIdx.x, lane = t & 63;
     const int wave = __builtin_amdgcn_readfirstlane(t >> 6);
-    const int wm = G::wm(wave), wn = G::wn(wave);
+    const typename Mma::addr_t AD = Mma::lane_addr(G::wm(wave), G::wn(wave), lane);
     const bool late = wave >= 4; // group 1
     const unsigned lds0 = (unsigned)(size_t)(__attribute__((address_space(3))) char *)smem;
     const dma_plan_t<DPA, DPB> plan = make_dma_plan<DPA, DPB>(wave, lane, rows_a_left, rows_b_left, lda, ldb);
@@ -268,10 +271,10 @@ __device__ __forceinline__ void main_loop_two_groups(Acc &acc, char *smem, const
         unsigned S[KSTEP];
 #pragma unroll
         for (int k = 0; k < KSTEP; ++k) S[k] = lds0 + slot * GROUP_BYTES + k * STAGE_BYTES;
-        Mma::load_a(f, 0, S, wm, lane, ctx, g);
-        Mma::load_b(f, S, wn, lane, ctx, g);
+        Mma::load_a(f, 0, S, AD, ctx, g);
+        Mma::load_b(f, S, AD, ctx, g);
 #pragma unroll
-        for (int i = 1; i < Mma::ROWS; ++i) Mma::load_a(f, i, S, wm, lane, ctx, g);
+        for (int i = 1; i < Mma::ROWS; ++i) Mma::load_a(f, i, S, AD, ctx, g);
     };
 #pragma nounroll
     for (int g = 0; g < niter; ++g) {
@@ -283,7 +286,15 @@ __device__ __forceinline__ void main_loop_two_groups(Acc &acc, char *smem, const
         if (nslot >= NG) nslot -= NG;
         if (!late) read_stage(g);
         __builtin_amdgcn_sched_barrier(0);
+        // Group 1 gets the matrix core first: its MFMAs were ready at the barrier,
+        // and its reads for the next interval come after them.  At equal priority
+        // group 0, which starts ~125 ns later, is served first all the same and
+        // group 1's reads end up after all MFMAs of the step, with the matrix core
+        // idle (time stamps: 545 ns for group 1's block against 285 ns for group 0's;
+        // with the priority 300 against 480, and 1.5-2 % less time per launch).
+        if (late) __builtin_amdgcn_s_setprio(3);
         mma_stage(f, g, g + NG - 1, nslot); // group 0: stage g; group 1: stage g-1
+        if (late) __builtin_amdgcn_s_setprio(0);
         __builtin_amdgcn_sched_barrier(0);
         if (late && g < ngroups) read_stage(g);
         if (++slot == NG) slot = 0;
@@ -302,11 +313,15 @@ __device__ __forceinline__ void main_loop_two_groups(Acc &acc, char *smem, const
 //   s_barrier             everybody's did, and everybody finished group g-1
 //   DMA group g+NG-1      into the slots group g-1 used
 //   ds_read + MFMA over group g
-// `Mma` supplies the geometry G = the tile geometry, frag_t, load_b(frag, S, wn, lane,
-// ctx, g) for the B^T fragments, load_a(frag, i, S, wm, lane, ctx, g) for A fragment i (S[k] is the
-// LDS byte address of the k-th stage of the group), mma_row(acc, frag, i, ctx, g)
-// for the COLS MFMAs of A fragment i (ROWS x COLS MFMA tiles per quadrant),
-// and A_READS / B_READS = LDS read instructions per fragment.
+// `Mma` supplies the tile geometry G, frag_t, addr_t lane_addr(wm, wn, lane)
+// (this lane's LDS offsets of fragment 0 of both operands inside a stage; the
+// other fragments are constant offsets from it, which ride in the offset field
+// of the reads instead of one address register per fragment), load_b(frag, S,
+// addr, ctx, g) for the B^T fragments, load_a(frag, i, S, addr, ctx, g) for A
+// fragment i (S[k] is the LDS byte address of the k-th stage of the group),
+// mma_row(acc, frag, i, ctx, g) for the COLS MFMAs of A fragment i (ROWS x COLS
+// MFMA tiles per wavefront), and A_READS / B_READS = LDS read instructions per
+// fragment.
 // a_tile / b_tile point at the first K byte of tile row 0.
 template <int NSTAGE, int KSTEP, class Mma, class Acc, class Ctx>
 __device__ __forceinline__ void main_loop(Acc &acc, char *smem, const char *a_tile,
@@ -326,7 +341,7 @@ __device__ __forceinline__ void main_loop(Acc &acc, char *smem, const char *a_ti
     static_assert((NG - 2) * GROUP_DMAS < 64, "vmcnt range");
     const int t = threadIdx.x, lane = t & 63;
     const int wave = __builtin_amdgcn_readfirstlane(t >> 6);
-    const int wm = G::wm(wave), wn = G::wn(wave);
+    const typename Mma::addr_t AD = Mma::lane_addr(G::wm(wave), G::wn(wave), lane);
     const unsigned lds0 = (unsigned)(size_t)(__attribute__((address_space(3))) char *)smem;
     const dma_plan_t<DPA, DPB> plan = make_dma_plan<DPA, DPB>(wave, lane, rows_a_left, rows_b_left, lda, ldb);
 
@@ -375,9 +390,9 @@ __device__ __forceinline__ void main_loop(Acc &acc, char *smem, const char *a_ti
         constexpr int ROWS = Mma::ROWS, COLS = Mma::COLS; // MFMA tiles of the quadrant
         // A fragment 0 first: LDS reads return in order, so the first MFMA can go
         // as soon as it and the first B fragment are in
-        Mma::load_a(f, 0, S, wm, lane, ctx, g);
-        Mma::load_b(f, S, wn, lane, ctx, g);
-        Mma::load_a(f, 1, S, wm, lane, ctx, g);
+        Mma::load_a(f, 0, S, AD, ctx, g);
+        Mma::load_b(f, S, AD, ctx, g);
+        Mma::load_a(f, 1, S, AD, ctx, g);
 #pragma unroll
         for (int i = 0; i < ROWS; ++i) {
             if (dma) {
@@ -385,7 +400,7 @@ __device__ __forceinline__ void main_loop(Acc &acc, char *smem, const char *a_ti
                 for (int d = 0; d < DPS; ++d) // spread evenly over the rows
                     if (d * ROWS / DPS == i) issue_part(g + NG - 1, nslot, d);
             }
-            if (i + 2 < ROWS) Mma::load_a(f, i + 2, S, wm, lane, ctx, g);
+            if (i + 2 < ROWS) Mma::load_a(f, i + 2, S, AD, ctx, g);
             Mma::mma_row(acc, f, i, ctx, g);
         }
         if (++slot == NG) slot = 0;

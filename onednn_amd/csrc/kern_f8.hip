@@ -46,21 +46,30 @@ struct f8_mma_t {
     struct frag_t {
         v8i a[ROWS], b[COLS];
     };
-    // lane l supplies row l%32 and K bytes 32*(l/32) .. +32 of the stage
-    __device__ static __forceinline__ v8i read32(unsigned T, int row, int c0) {
-        const v4i lo = lds_read16(T + swz(row, c0)), hi = lds_read16(T + swz(row, c0 + 1));
+    // lane l supplies row l%32 and K bytes 32*(l/32) .. +32 of the stage: two
+    // 16-byte chunks.  Per-lane LDS offsets of fragment 0; fragment i is 32 rows
+    // (2 KB) further with the same swizzle.
+    struct addr_t {
+        unsigned a0, a1, b0, b1;
+    };
+    __device__ static __forceinline__ addr_t lane_addr(int wm, int wn, int lane) {
+        const int frow = lane & 31, c0 = (lane >> 5) * 2;
+        const int ra = wm * 128 + frow, rb = wn * G::WCOLS + frow;
+        return addr_t {(unsigned)swz(ra, c0), (unsigned)swz(ra, c0 + 1), (unsigned)(B_OFF + swz(rb, c0)),
+                (unsigned)(B_OFF + swz(rb, c0 + 1))};
+    }
+    __device__ static __forceinline__ v8i read32(unsigned lo_addr, unsigned hi_addr) {
+        const v4i lo = lds_read16(lo_addr), hi = lds_read16(hi_addr);
         return v8i {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
     }
-    __device__ static __forceinline__ void load_b(frag_t &f, const unsigned (&S)[1], int wn, int lane,
+    __device__ static __forceinline__ void load_b(frag_t &f, const unsigned (&S)[1], const addr_t &ad,
             const f8_ctx_t &, int) {
-        const int frow = lane & 31, h = lane >> 5;
 #pragma unroll
-        for (int j = 0; j < COLS; ++j) f.b[j] = read32(S[0] + B_OFF, wn * G::WCOLS + j * 32 + frow, h * 2);
+        for (int j = 0; j < COLS; ++j) f.b[j] = read32(S[0] + ad.b0 + j * 2048, S[0] + ad.b1 + j * 2048);
     }
-    __device__ static __forceinline__ void load_a(frag_t &f, int i, const unsigned (&S)[1], int wm, int lane,
+    __device__ static __forceinline__ void load_a(frag_t &f, int i, const unsigned (&S)[1], const addr_t &ad,
             const f8_ctx_t &, int) {
-        const int frow = lane & 31, h = lane >> 5;
-        f.a[i] = read32(S[0], wm * 128 + i * 32 + frow, h * 2);
+        f.a[i] = read32(S[0] + ad.a0 + i * 2048, S[0] + ad.a1 + i * 2048);
     }
     __device__ static __forceinline__ void mma_row(v16f (&acc)[ROWS][COLS], const frag_t &f, int i,
             const f8_ctx_t &, int) {
@@ -100,7 +109,7 @@ __global__ void __launch_bounds__(G::NT) __attribute__((amdgpu_waves_per_eu(G::N
     const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
     const int wm = G::wm(wave), wn = G::wn(wave);
     const long b = blockIdx.z;
-    const tile_pos_t tp = tile_position<G>(X.tiles_m, X.tiles_n);
+    const tile_pos_t tp = tile_position<G>((int)blockIdx.x, X.tiles_m, X.tiles_n);
     const long m0 = tp.m0, n0 = tp.n0;
 
     const long lda = P.ss[1];

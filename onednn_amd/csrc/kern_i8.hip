@@ -47,17 +47,24 @@ struct i8_mma_t {
     struct frag_t {
         v4i a[ROWS], b[COLS];
     };
-    __device__ static __forceinline__ void load_b(frag_t &f, const unsigned (&S)[1], int wn, int lane,
-            const i8_ctx_t &, int) {
+    // Per-lane LDS offsets of fragment 0 of both operands.  Fragment i is 16 rows
+    // further: the swizzle depends on the row modulo 16 only, so it is the same
+    // address plus i KB, which goes into the offset field of the read.
+    struct addr_t {
+        unsigned a, b;
+    };
+    __device__ static __forceinline__ addr_t lane_addr(int wm, int wn, int lane) {
         const int frow = lane & 15, fch = lane >> 4;
-#pragma unroll
-        for (int j = 0; j < COLS; ++j)
-            f.b[j] = lds_read16(S[0] + B_OFF + swz(wn * G::WCOLS + j * 16 + frow, fch));
+        return addr_t {(unsigned)swz(wm * 128 + frow, fch), (unsigned)(B_OFF + swz(wn * G::WCOLS + frow, fch))};
     }
-    __device__ static __forceinline__ void load_a(frag_t &f, int i, const unsigned (&S)[1], int wm, int lane,
+    __device__ static __forceinline__ void load_b(frag_t &f, const unsigned (&S)[1], const addr_t &ad,
             const i8_ctx_t &, int) {
-        const int frow = lane & 15, fch = lane >> 4;
-        f.a[i] = lds_read16(S[0] + swz(wm * 128 + i * 16 + frow, fch));
+#pragma unroll
+        for (int j = 0; j < COLS; ++j) f.b[j] = lds_read16(S[0] + ad.b + j * 1024);
+    }
+    __device__ static __forceinline__ void load_a(frag_t &f, int i, const unsigned (&S)[1], const addr_t &ad,
+            const i8_ctx_t &, int) {
+        f.a[i] = lds_read16(S[0] + ad.a + i * 1024);
     }
     __device__ static __forceinline__ void mma_row(v4i (&acc)[ROWS][COLS], const frag_t &f, int i,
             const i8_ctx_t &, int) {
@@ -99,7 +106,7 @@ __global__ void __launch_bounds__(G::NT) __attribute__((amdgpu_waves_per_eu(G::N
     const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
     const int wm = G::wm(wave), wn = G::wn(wave);
     const long b = blockIdx.z;
-    const tile_pos_t tp = tile_position<G>(X.tiles_m, X.tiles_n);
+    const tile_pos_t tp = tile_position<G>((int)blockIdx.x, X.tiles_m, X.tiles_n);
     const long m0 = tp.m0, n0 = tp.n0;
 
     const long lda = P.ss[1];

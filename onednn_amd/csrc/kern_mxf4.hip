@@ -80,24 +80,31 @@ struct mxf4_mma_t {
         const unsigned slot = (S[0] - c.lds0) / G::STAGE_BYTES;
         return c.lds_scale0 + slot * SCALE_STAGE;
     }
-    __device__ static __forceinline__ void load_b(frag_t &f, const unsigned (&S)[1], int wn, int lane,
+    // Per-lane LDS offsets of fragment 0 (data) and of its scale dword, and the
+    // bit position of this lane's scale byte; fragment i is 16 rows further.
+    struct addr_t {
+        unsigned a, b, sa, sb, shift;
+    };
+    __device__ static __forceinline__ addr_t lane_addr(int wm, int wn, int lane) {
+        const int frow = lane & 15, q = lane >> 4;
+        const int ra = wm * 128 + frow, rb = wn * G::WCOLS + frow;
+        return addr_t {(unsigned)swz(ra, q), (unsigned)(B_OFF + swz(rb, q)), (unsigned)(ra * 4),
+                (unsigned)((256 + rb) * 4), (unsigned)(q * 8)};
+    }
+    __device__ static __forceinline__ void load_b(frag_t &f, const unsigned (&S)[1], const addr_t &ad,
             const mxf4_ctx_t &c, int) {
         const unsigned sc = scales(S, c);
-        const int frow = lane & 15, q = lane >> 4;
 #pragma unroll
         for (int j = 0; j < COLS; ++j) {
-            const int rb = wn * G::WCOLS + j * 16 + frow;
-            f.b[j] = lds_read16(S[0] + B_OFF + swz(rb, q));
-            f.sb[j] = (int)((lds_read4(sc + (256 + rb) * 4) >> (q * 8)) & 0xffu);
+            f.b[j] = lds_read16(S[0] + ad.b + j * 1024);
+            f.sb[j] = (int)((lds_read4(sc + ad.sb + j * 64) >> ad.shift) & 0xffu);
         }
     }
-    __device__ static __forceinline__ void load_a(frag_t &f, int i, const unsigned (&S)[1], int wm, int lane,
+    __device__ static __forceinline__ void load_a(frag_t &f, int i, const unsigned (&S)[1], const addr_t &ad,
             const mxf4_ctx_t &c, int) {
         const unsigned sc = scales(S, c);
-        const int frow = lane & 15, q = lane >> 4;
-        const int ra = wm * 128 + i * 16 + frow;
-        f.a[i] = lds_read16(S[0] + swz(ra, q));
-        f.sa[i] = (int)((lds_read4(sc + ra * 4) >> (q * 8)) & 0xffu);
+        f.a[i] = lds_read16(S[0] + ad.a + i * 1024);
+        f.sa[i] = (int)((lds_read4(sc + ad.sa + i * 64) >> ad.shift) & 0xffu);
     }
     __device__ static __forceinline__ void mma_row(v4f (&acc)[ROWS][COLS], const frag_t &f, int i,
             const mxf4_ctx_t &, int) {
@@ -128,7 +135,7 @@ __global__ void __launch_bounds__(G::NT) __attribute__((amdgpu_waves_per_eu(G::N
     const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
     const int wm = G::wm(wave), wn = G::wn(wave);
     const long b = blockIdx.z;
-    const tile_pos_t tp = tile_position<G>(X.tiles_m, X.tiles_n);
+    const tile_pos_t tp = tile_position<G>((int)blockIdx.x, X.tiles_m, X.tiles_n);
     const long m0 = tp.m0, n0 = tp.n0;
 
     const long lda = P.ss[1] / 2; // bytes per src row
