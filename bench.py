@@ -41,8 +41,8 @@ import numpy as np  # noqa: E402
 # known 256 MiB (factors 2.0 and 1.0); the summaries with the commands are in
 # profiles/<kernel>_<workload>.md.  Keyed by (workload, M).
 MEASURED_TRAFFIC = {
-    ("c3", 8192): 1020938813, ("c4", 4096): 2939206486, ("c5", 8192): 715169018,
-    ("c2", 1): 32839650, ("c2", 8): 35736443, ("c2", 32): 51670790, ("c1", 256): 8286638,
+    ("c3", 8192): 1008038840, ("c4", 4096): 2597323049, ("c5", 8192): 569589287,
+    ("c2", 1): 32839918, ("c2", 8): 35736510, ("c2", 32): 51670432, ("c1", 256): 8357752,
 }
 
 # MI355X published peaks
