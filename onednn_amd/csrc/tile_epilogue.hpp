@@ -560,6 +560,30 @@ __device__ __forceinline__ void storeQ(const PT &P, const epi_hoist_t &H, const 
 #pragma unroll
             for (int e = 0; e < 4; ++e) w[k][e] = (uint32_t)(int)__builtin_rintf(sat(v[k][e], 0.f, 255.f)) & 0xffu;
     } else if (dt == MI355_DT_BF16) {
+        // v_cvt_pk_bf16_f32 rounds to nearest even like the reference's conversion
+        // (src/common/bfloat16.cpp:29-49) for normal numbers, zeros and infinities;
+        // the reference flushes f32 subnormals to zero and quiets NaNs by setting
+        // one bit, so a wavefront that holds any of those (class mask: s/q NaN,
+        // +-subnormal) takes the software conversion.  One class test per value
+        // and half a conversion instead of a dozen integer operations.
+        bool special = false;
+#pragma unroll
+        for (int k = 0; k < NQ; ++k)
+#pragma unroll
+            for (int e = 0; e < 4; ++e) special |= __builtin_amdgcn_classf(v[k][e], 0x93);
+        if (__builtin_amdgcn_ballot_w64(special) == 0) {
+            typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
+            typedef float f32x2_t __attribute__((ext_vector_type(2)));
+            const long off0b = b * P.ds[0] + n;
+#pragma unroll
+            for (int k = 0; k < NQ; ++k) {
+                uint2 o;
+                o.x = __builtin_bit_cast(unsigned, __builtin_convertvector(f32x2_t {v[k][0], v[k][1]}, bf16x2_t));
+                o.y = __builtin_bit_cast(unsigned, __builtin_convertvector(f32x2_t {v[k][2], v[k][3]}, bf16x2_t));
+                if (ok[k]) *(uint2 *)((uint16_t *)P.dst + off0b + m[k] * P.ds[1]) = o;
+            }
+            return;
+        }
 #pragma unroll
         for (int k = 0; k < NQ; ++k)
 #pragma unroll
