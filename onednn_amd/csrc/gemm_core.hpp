@@ -132,7 +132,7 @@ __device__ __forceinline__ tile_pos_t tile_position(int id, int tiles_m, int til
     const int nwg = tiles_m * tiles_n;
     const int per = nwg / 8;
     const int tile = (nwg % 8 == 0) ? (id % 8) * per + id / 8 : id;
-    constexpr int GM = 8;
+    constexpr int GM = 8; // measured: 4 and 8 alike, 16 is 2 % and 32 is 7 % slower on the int8 headline shape
     const int band = tile / (GM * tiles_n);
     const int band_rows = min(GM, tiles_m - band * GM);
     const int in_band = tile - band * GM * tiles_n;

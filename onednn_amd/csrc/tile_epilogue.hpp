@@ -549,16 +549,27 @@ __device__ __forceinline__ void storeQ(const PT &P, const epi_hoist_t &H, const 
         const long (&m)[NQ], long n, const bool (&ok)[NQ]) {
     uint32_t w[NQ][4];
     const int dt = H.dst_dt;
-    if (dt == MI355_DT_S8) {
+    if (dt == MI355_DT_S8 || dt == MI355_DT_U8) {
+        // Round first (v_rndne + the saturating v_cvt_i32_f32, NaN -> 0), clamp as
+        // integers, pack the four low bytes with byte permutes: the same values as
+        // the reference's clamp-then-round (rounding is monotonic and the bounds
+        // are integers) in 3 + 3/4 instructions per value instead of 7 + 7/4.
+        const int lo = dt == MI355_DT_S8 ? -128 : 0, hi = dt == MI355_DT_S8 ? 127 : 255;
+        const long off0b = b * P.ds[0] + n;
 #pragma unroll
-        for (int k = 0; k < NQ; ++k)
+        for (int k = 0; k < NQ; ++k) {
+            int q[4];
 #pragma unroll
-            for (int e = 0; e < 4; ++e) w[k][e] = (uint32_t)(int)__builtin_rintf(sat(v[k][e], -128.f, 127.f)) & 0xffu;
-    } else if (dt == MI355_DT_U8) {
-#pragma unroll
-        for (int k = 0; k < NQ; ++k)
-#pragma unroll
-            for (int e = 0; e < 4; ++e) w[k][e] = (uint32_t)(int)__builtin_rintf(sat(v[k][e], 0.f, 255.f)) & 0xffu;
+            for (int e = 0; e < 4; ++e) {
+                const int r = (int)__builtin_rintf(v[k][e]);
+                q[e] = r < lo ? lo : (r > hi ? hi : r);
+            }
+            const unsigned lo16 = __builtin_amdgcn_perm((unsigned)q[1], (unsigned)q[0], 0x0c0c0400u);
+            const unsigned hi16 = __builtin_amdgcn_perm((unsigned)q[3], (unsigned)q[2], 0x0c0c0400u);
+            const unsigned word = __builtin_amdgcn_perm(hi16, lo16, 0x05040100u);
+            if (ok[k]) *(uint32_t *)((uint8_t *)P.dst + off0b + m[k] * P.ds[1]) = word;
+        }
+        return;
     } else if (dt == MI355_DT_BF16) {
         // v_cvt_pk_bf16_f32 rounds to nearest even like the reference's conversion
         // (src/common/bfloat16.cpp:29-49) for normal numbers, zeros and infinities;

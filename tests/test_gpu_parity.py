@@ -178,3 +178,25 @@ def test_woq_back_to_back_launches_share_nothing(gpu, oracle):
     assert_close(b, outs[4], want, abs_sum=asum * 20.0, what="second problem")
     ra.free()
     rb.free()
+
+
+@pytest.mark.parametrize("scale", [1.0, 1.4e-45, 1e-43])
+def test_bf16_dst_of_integer_gemm_is_bit_exact_including_flushed_subnormals(gpu, oracle, scale):
+    """s8 x s8 -> bf16: integer accumulation, so the only rounding is the dst
+    conversion.  The reference's bf16 conversion flushes f32 subnormals to a
+    signed zero (src/common/bfloat16.cpp:29-49); the MFMA epilogue converts in
+    hardware and must take its software path for those (scale 1.4e-45 makes every
+    result subnormal, 1e-43 a mix of subnormal and normal values)."""
+    from onednn_amd.problem import MatmulProblem, QuantParam
+    r = np.random.default_rng(123)
+    M, N, K = 256, 256, 128
+    src = r.integers(-127, 128, size=(M, K), dtype=np.int8)
+    wei = r.integers(-127, 128, size=(K, N), dtype=np.int8)
+    p = MatmulProblem(M=M, N=N, K=K, src_dt=cabi.DT_S8, wei_dt=cabi.DT_S8, dst_dt=cabi.DT_BF16, src=src, wei=wei,
+                      wei_stride=(K * N, N, 1),
+                      quant={"src_scale": QuantParam(cabi.DT_F32, 0, np.array([scale], np.float32))})
+    got, name = run_gpu(p, cabi.IMPL_I8_MFMA)
+    want = oracle.run_oracle(p)
+    assert_bit_exact(p, got, want, name)
+    if scale == 1.4e-45:
+        assert np.all((want.view(np.uint16) & 0x7fff) == 0)
