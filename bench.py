@@ -84,11 +84,14 @@ def build_problem(name, M=None, wtag="any"):
     descriptor: K-contiguous (ba) for the MFMA operand types, row-major (ab)
     for the int4 decode weights.  With an explicit `ab` the MFMA families run
     a layout pre-pass inside every launch, which then is part of the step."""
-    from onednn_amd import configs
+    from onednn_amd import cabi, configs
     if name == "c1":
         return configs.config1()
     if name == "c2":
-        return configs.config2(M=M or 1, wtag="ab" if wtag == "any" else wtag)
+        p = configs.config2(M=M or 1, wtag="ab" if wtag == "any" else wtag)
+        if wtag == "any":  # what format_tag::any resolves to for decode weights
+            p.wei_packing = cabi.WEI_PACK_WOQ64
+        return p
     mfma_tag = "ba" if wtag == "any" else wtag
     if name == "c3":
         return configs.config3(wtag=mfma_tag)

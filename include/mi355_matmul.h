@@ -135,7 +135,31 @@ enum {
     MI355_IMPL_F8_MFMA = 3,  /* "hip:mfma_f8": e4m3/e5m2 MFMA GEMM */
     MI355_IMPL_MXF4_MFMA = 4,/* "hip:mfma_mxf4": block-scaled e2m1 MFMA GEMM */
     MI355_IMPL_WOQ_GEMV = 5, /* "hip:woq_gemv": int4/int8 weight-only decode */
-    MI355_IMPL_COUNT = 6
+    MI355_IMPL_WOQ_PACKED = 6, /* "hip:woq_packed": decode over MI355_WEI_PACK_WOQ64 weights */
+    MI355_IMPL_COUNT = 7
+};
+
+/* Weights packing (mi355_matmul_desc_t.wei_packing): the counterpart of an
+ * opaque blocked memory descriptor that dnnl_format_tag_any resolves to
+ * (src/common/memory_desc.hpp: format_kind blocked with inner blocks; the
+ * reference's brgemm matmul asks for such weights,
+ * src/cpu/x64/matmul/brgemm_matmul_utils.cpp:203-330).
+ *
+ * MI355_WEI_PACK_WOQ64 -- 4-bit weights [K][N], batch 1, K % 32 == 0,
+ * N % 64 == 0, K * N / 2 bytes, wei_stride ignored.  Element (k, n) is the
+ * nibble (low nibble first within a byte) at nibble offset
+ *     (n / 64) * (K * 64)        64-column chunk, all of K contiguous
+ *   + (k / 8) * 512              8 rows of the chunk: 256 bytes
+ *   + (n % 16) * 32              column within a 16-column block: 16 bytes
+ *   + ((n % 64) / 16) * 8        16-column block of the chunk: one dword
+ *   + (k % 2) * 4 + (k % 8) / 2  the 8 rows of one column in one dword
+ * so that a wavefront reads 32 rows x 64 columns as one 1 KB run, 16 bytes
+ * per lane, and every dword unpacks into a matrix-core operand with three
+ * shifts.  mi355_reorder_launch writes the layout as a six-dim strided dst
+ * (see mi355_wei_pack_reorder_dims). */
+enum {
+    MI355_WEI_PACK_NONE = 0,
+    MI355_WEI_PACK_WOQ64 = 1
 };
 
 #define MI355_MAX_POST_OPS 32 /* post_ops_t::post_ops_limit in the reference */
@@ -184,7 +208,7 @@ typedef struct mi355_matmul_desc {
     int32_t n_post_ops;
     mi355_post_op_t post_ops[MI355_MAX_POST_OPS];
     int32_t impl; /* MI355_IMPL_*; AUTO picks the fastest applicable */
-    int32_t reserved;
+    int32_t wei_packing; /* MI355_WEI_PACK_* */
 } mi355_matmul_desc_t;
 
 typedef struct mi355_matmul_args {
@@ -282,6 +306,16 @@ int mi355_reorder_query(const mi355_reorder_desc_t *desc);
  * implementations, DNNL_ARG_FROM -> DNNL_ARG_TO).  Asynchronous. */
 int mi355_reorder_launch(const mi355_reorder_desc_t *desc,
         const mi355_reorder_args_t *args, void *stream);
+
+/* Writes into desc->ndims / dims / src_stride / dst_stride the six-dim view
+ * under which a reorder moves weights [K][N] with element strides
+ * (src_stride_k, src_stride_n) into the packed layout `packing`
+ * (MI355_WEI_PACK_*); the other fields of `desc` are the caller's.  It is what
+ * a reorder into an opaque blocked memory descriptor does in the reference
+ * (simple_reorder.hpp, plain -> blocked specializations).
+ * MI355_INVALID_ARGUMENTS if K, N do not fit the layout. */
+int mi355_wei_pack_reorder_dims(int packing, int64_t K, int64_t N,
+        int64_t src_stride_k, int64_t src_stride_n, mi355_reorder_desc_t *desc);
 
 /* Plain device-to-device copy kernel (one 16-byte load + store per lane), used
  * to calibrate the FETCH_SIZE / WRITE_SIZE counters against a known size. */

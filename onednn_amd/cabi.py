@@ -40,7 +40,8 @@ BINARY = {
 }
 
 DST_SCALE_DIVIDE, DST_SCALE_RECIPROCAL = 0, 1
-IMPL_AUTO, IMPL_REF, IMPL_I8_MFMA, IMPL_F8_MFMA, IMPL_MXF4_MFMA, IMPL_WOQ_GEMV = range(6)
+IMPL_AUTO, IMPL_REF, IMPL_I8_MFMA, IMPL_F8_MFMA, IMPL_MXF4_MFMA, IMPL_WOQ_GEMV, IMPL_WOQ_PACKED = range(7)
+WEI_PACK_NONE, WEI_PACK_WOQ64 = 0, 1
 
 
 class Quant(C.Structure):
@@ -64,7 +65,7 @@ class MatmulDesc(C.Structure):
         ("fpmath_apply_to_int", C.c_int32), ("fpmath_mode", C.c_int32),
         ("dst_scale_mode", C.c_int32), ("n_post_ops", C.c_int32),
         ("post_ops", PostOp * MAX_POST_OPS),
-        ("impl", C.c_int32), ("reserved", C.c_int32),
+        ("impl", C.c_int32), ("wei_packing", C.c_int32),
     ]
 
 
@@ -108,7 +109,7 @@ KERNEL_SYMBOLS = [
     "mi355_event_destroy", "mi355_event_record", "mi355_event_sync", "mi355_event_elapsed_ms",
     "mi355_last_error", "mi355_matmul_query", "mi355_matmul_impl_name",
     "mi355_matmul_scratch_bytes", "mi355_matmul_launch", "mi355_reorder_query",
-    "mi355_reorder_launch", "mi355_copy_kernel", "mi355_flush_kernel",
+    "mi355_reorder_launch", "mi355_wei_pack_reorder_dims", "mi355_copy_kernel", "mi355_flush_kernel",
 ]
 
 _PKG_DIR = os.path.dirname(os.path.abspath(__file__))
@@ -161,6 +162,8 @@ def load_kernels():
     lib.mi355_matmul_launch.argtypes = [C.POINTER(MatmulDesc), C.POINTER(MatmulArgs), vp, vp]
     lib.mi355_reorder_query.argtypes = [C.POINTER(ReorderDesc)]
     lib.mi355_reorder_launch.argtypes = [C.POINTER(ReorderDesc), C.POINTER(ReorderArgs), vp]
+    lib.mi355_wei_pack_reorder_dims.argtypes = [C.c_int, C.c_int64, C.c_int64, C.c_int64, C.c_int64,
+                                                C.POINTER(ReorderDesc)]
     lib.mi355_copy_kernel.argtypes = [vp, vp, C.c_size_t, vp]
     lib.mi355_flush_kernel.argtypes = [vp, C.c_size_t, vp]
     _lib = lib

@@ -63,6 +63,10 @@ static int validate(const mi355_matmul_desc_t *d) {
             return MI355_INVALID_ARGUMENTS;
         }
     }
+    if (d->wei_packing != MI355_WEI_PACK_NONE && !woq64_layout_ok(*d)) {
+        set_error("weights packing %d needs 4-bit weights, batch 1, K %% 32 == 0 and N %% 64 == 0", d->wei_packing);
+        return MI355_INVALID_ARGUMENTS;
+    }
     int st;
     if ((st = check_quant(d->src_scale, "src scale"))) return st;
     if ((st = check_quant(d->wei_scale, "weights scale"))) return st;
@@ -98,13 +102,14 @@ static int impl_supported(const mi355_matmul_desc_t &d, int impl) {
         case MI355_IMPL_F8_MFMA: return f8_supported(d);
         case MI355_IMPL_MXF4_MFMA: return mxf4_supported(d);
         case MI355_IMPL_WOQ_GEMV: return woq_supported(d);
+        case MI355_IMPL_WOQ_PACKED: return woqp_supported(d);
         default: return MI355_INVALID_ARGUMENTS;
     }
 }
 
 // priority order of the implementation list (fastest first, generic last),
 // the role of an engine's impl_list_item_t[] in the reference
-static const int g_impl_order[] = {MI355_IMPL_WOQ_GEMV, MI355_IMPL_I8_MFMA, MI355_IMPL_F8_MFMA,
+static const int g_impl_order[] = {MI355_IMPL_WOQ_PACKED, MI355_IMPL_WOQ_GEMV, MI355_IMPL_I8_MFMA, MI355_IMPL_F8_MFMA,
         MI355_IMPL_MXF4_MFMA, MI355_IMPL_REF};
 
 static int choose_impl(const mi355_matmul_desc_t &d, int *chosen) {
@@ -149,6 +154,7 @@ static int build_problem(const mi355_matmul_desc_t &d, const mi355_matmul_args_t
     P.dst_scale_mode = d.dst_scale_mode;
     P.n_po = d.n_post_ops;
     P.sum_dt = MI355_DT_UNDEF;
+    P.wei_packing = d.wei_packing;
     P.src = a.src; P.wei = a.wei; P.bias = a.bias; P.dst = a.dst;
     const struct { const mi355_quant_t *q; const void *p; const char *n; } need[] = {
             {&d.src_scale, a.src_scale, "src scale"}, {&d.wei_scale, a.wei_scale, "weights scale"},
@@ -286,6 +292,7 @@ const char *mi355_matmul_impl_name(int impl) {
         case MI355_IMPL_F8_MFMA: return "hip:mfma_f8:gfx950";
         case MI355_IMPL_MXF4_MFMA: return "hip:mfma_mxf4:gfx950";
         case MI355_IMPL_WOQ_GEMV: return "hip:woq_gemv:gfx950";
+        case MI355_IMPL_WOQ_PACKED: return "hip:woq_packed:gfx950";
         default: return "undef";
     }
 }
@@ -343,6 +350,7 @@ int mi355_matmul_launch(const mi355_matmul_desc_t *desc, const mi355_matmul_args
         case MI355_IMPL_F8_MFMA: return f8_launch(*desc, P, scratch, s);
         case MI355_IMPL_MXF4_MFMA: return mxf4_launch(*desc, P, scratch, s);
         case MI355_IMPL_WOQ_GEMV: return woq_launch(*desc, P, scratch, s);
+        case MI355_IMPL_WOQ_PACKED: return woqp_launch(*desc, P, s);
         default: return MI355_UNIMPLEMENTED;
     }
 }

@@ -18,6 +18,16 @@ __device__ __forceinline__ long ngroups_k(const Q &q, int kdim, long K) {
     return g > 1 ? K / g : 1;
 }
 
+// element offset of weights (b, k, n): strided, or the nibble offset of the
+// 64-column decode packing (MI355_WEI_PACK_WOQ64)
+template <class PT>
+__device__ __forceinline__ long wei_off(const PT &P, long bw, long k, long n) {
+    if (P.wei_packing == MI355_WEI_PACK_WOQ64)
+        return (n / 64) * (P.K * 64) + (k / 8) * 512 + (n % 16) * 32 + ((n % 64) / 16) * 8 + (k % 2) * 4
+                + (k % 8) / 2;
+    return bw * P.ws[0] + k * P.ws[1] + n * P.ws[2];
+}
+
 template <class PT>
 __device__ float ref_int_dot(const PT &P, long b, long m, long n) {
     const long K = P.K, M = P.M, N = P.N;
@@ -39,7 +49,7 @@ __device__ float ref_int_dot(const PT &P, long b, long m, long n) {
         for (long kk = 0; kk < gk; ++kk) {
             k = g * gk + kk;
             int s = load_int(P.src_dt, P.src, bs * P.ss[0] + m * P.ss[1] + k * P.ss[2]);
-            int w = load_int(P.wei_dt, P.wei, bw * P.ws[0] + k * P.ws[1] + n * P.ws[2]);
+            int w = load_int(P.wei_dt, P.wei, wei_off(P, bw, k, n));
             if (src_zp) s -= load_int(P.src_zp.dt, P.src_zp.p, quant_off(P.src_zp, bs, m, k, M, K));
             if (wei_zp && !src_pr)
                 w -= load_int(P.wei_zp.dt, P.wei_zp.p, quant_off(P.wei_zp, bw, k, n, K, N));
@@ -85,7 +95,7 @@ __device__ float ref_fp_dot(const PT &P, long b, long m, long n) {
         for (long kk = 0; kk < gk; ++kk) {
             k = g * gk + kk;
             const float s = load_float(P.src_dt, P.src, bs * P.ss[0] + m * P.ss[1] + k * P.ss[2]);
-            float w = load_float(P.wei_dt, P.wei, bw * P.ws[0] + k * P.ws[1] + n * P.ws[2]);
+            float w = load_float(P.wei_dt, P.wei, wei_off(P, bw, k, n));
             if (decomp) {
                 if (wei_zp)
                     w -= load_float(P.wei_zp.dt, P.wei_zp.p, quant_off(P.wei_zp, bw, k, n, K, N));
@@ -118,6 +128,7 @@ __global__ void __launch_bounds__(256) ref_matmul_kernel(const problem_t P_) {
 int ref_supported(const mi355_matmul_desc_t &d) {
     // 4-bit dst would need two elements per thread; not offered.
     if (dt_bits(d.dst_dt) < 8) return MI355_UNIMPLEMENTED;
+    if (d.wei_packing != MI355_WEI_PACK_NONE && !woq64_layout_ok(d)) return MI355_UNIMPLEMENTED;
     return MI355_SUCCESS;
 }
 

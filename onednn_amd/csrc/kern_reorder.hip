@@ -640,3 +640,25 @@ extern "C" int mi355_reorder_launch(const mi355_reorder_desc_t *desc, const mi35
     }
     return MI355_SUCCESS;
 }
+
+extern "C" int mi355_wei_pack_reorder_dims(int packing, int64_t K, int64_t N, int64_t src_stride_k,
+        int64_t src_stride_n, mi355_reorder_desc_t *desc) {
+    using namespace mi355;
+    if (!desc || packing != MI355_WEI_PACK_WOQ64 || K <= 0 || N <= 0 || K % 32 || N % 64) {
+        set_error("weights packing %d does not fit K = %ld, N = %ld", packing, (long)K, (long)N);
+        return MI355_INVALID_ARGUMENTS;
+    }
+    // k = 8 * kq + 2 * r_hi + r_lo, n = 64 * c + 16 * t + j; dims in the order
+    // (kq, r_hi, r_lo, c, t, j)
+    const int64_t dims[6] = {K / 8, 4, 2, N / 64, 4, 16};
+    const int64_t ss[6] = {8 * src_stride_k, 2 * src_stride_k, src_stride_k, 64 * src_stride_n, 16 * src_stride_n,
+            src_stride_n};
+    const int64_t ds[6] = {512, 1, 4, K * 64, 8, 32};
+    desc->ndims = 6;
+    for (int i = 0; i < 6; ++i) {
+        desc->dims[i] = dims[i];
+        desc->src_stride[i] = ss[i];
+        desc->dst_stride[i] = ds[i];
+    }
+    return MI355_SUCCESS;
+}

@@ -537,6 +537,7 @@ int launch_variant(int scb, int zpb, dim3 grid, size_t lds, hipStream_t stream, 
 int woq_supported(const mi355_matmul_desc_t &d) {
     if (d.src_dt != MI355_DT_BF16 || !is_int4_dt(d.wei_dt) || !d.fpmath_apply_to_int)
         return MI355_UNIMPLEMENTED;
+    if (d.wei_packing != MI355_WEI_PACK_NONE) return MI355_UNIMPLEMENTED;
     if (dt_bits(d.dst_dt) < 8) return MI355_UNIMPLEMENTED;
     if (d.batch != 1 || d.M < 1 || d.M > 32) return MI355_UNIMPLEMENTED;
     if (d.K % 16 != 0 || d.N % 16 != 0 || d.K < 16) return MI355_UNIMPLEMENTED;

@@ -32,6 +32,10 @@ size_t woq_scratch_bytes(const mi355_matmul_desc_t &d);
 int woq_launch(const mi355_matmul_desc_t &d, const problem_t &P, void *scratch,
         hipStream_t stream);
 
+// the same decode over weights in the 64-column packing
+int woqp_supported(const mi355_matmul_desc_t &d);
+int woqp_launch(const mi355_matmul_desc_t &d, const problem_t &P, hipStream_t stream);
+
 void set_error(const char *fmt, ...);
 
 // [R][C] bytes (row pitch ld_in) -> [C][R] bytes (row pitch ld_out), per batch
@@ -42,6 +46,11 @@ inline bool is_int8_dt(int dt) { return dt == MI355_DT_S8 || dt == MI355_DT_U8; 
 inline bool is_int4_dt(int dt) { return dt == MI355_DT_S4 || dt == MI355_DT_U4; }
 inline bool is_f8_dt(int dt) { return dt == MI355_DT_F8_E4M3 || dt == MI355_DT_F8_E5M2; }
 inline bool quant_absent(const mi355_quant_t &q) { return q.dt == MI355_DT_UNDEF; }
+// a problem whose weights can be in the MI355_WEI_PACK_WOQ64 layout
+inline bool woq64_layout_ok(const mi355_matmul_desc_t &d) {
+    return d.wei_packing == MI355_WEI_PACK_WOQ64 && is_int4_dt(d.wei_dt) && d.batch == 1 && d.K % 32 == 0
+            && d.N % 64 == 0 && d.K > 0 && d.N > 0;
+}
 inline size_t align_up(size_t v, size_t a) { return (v + a - 1) / a * a; }
 
 } // namespace mi355

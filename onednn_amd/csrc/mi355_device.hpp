@@ -35,6 +35,7 @@ struct problem_t {
     long ss[3], ws[3], ds[3], bs[3];
     quant_dev_t src_scale, wei_scale, dst_scale, src_zp, wei_zp, dst_zp, src_pr;
     int apply_to_int, dst_scale_mode, n_po, sum_dt;
+    int wei_packing, pad_;
     const void *src, *wei, *bias;
     void *dst;
     po_dev_t po[MI355_MAX_POST_OPS];

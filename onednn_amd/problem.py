@@ -92,6 +92,22 @@ class PostOp:
     data: Optional[np.ndarray] = None
 
 
+def pack_woq64(wei, K, N, stride_k=None, stride_n=1):
+    """4-bit weights [K][N] (raw bytes, two elements per byte, low nibble first,
+    element strides (stride_k, stride_n)) in the MI355_WEI_PACK_WOQ64 layout:
+    memory order [n / 64][k / 8][n % 16][(n % 64) / 16][k % 2][(k % 8) / 2]."""
+    assert K % 32 == 0 and N % 64 == 0
+    stride_k = N if stride_k is None else stride_k
+    raw = np.ascontiguousarray(wei).view(np.uint8).reshape(-1)
+    nib = np.empty(raw.size * 2, np.uint8)
+    nib[0::2] = raw & 15
+    nib[1::2] = raw >> 4
+    kn = np.lib.stride_tricks.as_strided(nib, (K, N), (stride_k, stride_n))
+    # (kq, r_hi, r_lo, c, t, j) -> (c, kq, j, t, r_lo, r_hi)
+    v = kn.reshape(K // 8, 4, 2, N // 64, 4, 16).transpose(3, 0, 5, 4, 2, 1).reshape(-1)
+    return (v[0::2] | (v[1::2] << 4)).astype(np.uint8)
+
+
 @dataclass
 class MatmulProblem:
     M: int
@@ -115,6 +131,7 @@ class MatmulProblem:
     fpmath_mode: int = 0
     dst_scale_mode: int = cabi.DST_SCALE_DIVIDE
     impl: int = cabi.IMPL_AUTO
+    wei_packing: int = cabi.WEI_PACK_NONE  # `wei` stays plain here; GpuRun uploads it packed
     dst_init: Optional[np.ndarray] = None   # prior dst content (sum post-op)
     name: str = ""
 
@@ -162,6 +179,7 @@ class MatmulProblem:
             for j in range(3):
                 o.stride[j] = po.stride[j]
         d.impl = self.impl
+        d.wei_packing = self.wei_packing
         return d
 
     def initial_dst(self):
@@ -186,7 +204,12 @@ class GpuRun:
         self.bufs = {}
         a = cabi.MatmulArgs()
         self.bufs["src"] = cabi.DeviceBuffer.from_numpy(prob.src)
-        self.bufs["wei"] = cabi.DeviceBuffer.from_numpy(prob.wei)
+        wei = prob.wei
+        if prob.wei_packing == cabi.WEI_PACK_WOQ64:
+            if getattr(prob, "_packed_wei", None) is None:  # several runs may share one problem
+                prob._packed_wei = pack_woq64(prob.wei, prob.K, prob.N, prob.wei_stride[1], prob.wei_stride[2])
+            wei = prob._packed_wei
+        self.bufs["wei"] = cabi.DeviceBuffer.from_numpy(wei)
         a.src, a.wei = self.bufs["src"].ptr, self.bufs["wei"].ptr
         if prob.bias is not None:
             self.bufs["bias"] = cabi.DeviceBuffer.from_numpy(prob.bias)

@@ -1,0 +1,221 @@
+"""Packed decode weights (MI355_WEI_PACK_WOQ64): the layout itself (CPU), and
+the decode kernel that reads it against the CPU oracle, which always sees the
+plain weights (GPU).
+
+What pins the layout without a GPU: the nibble offset formula of the header is
+evaluated element by element in plain Python, the numpy packer and the
+six-dim reorder view (run by the oracle's reorder) must both reproduce it.
+"""
+import ctypes as C
+
+import numpy as np
+import pytest
+
+from onednn_amd import cabi, configs
+from onednn_amd import dtypes as dtp
+from onednn_amd.problem import pack_woq64, run_gpu
+from onednn_amd.reorder import ReorderProblem
+from onednn_amd import reorder as reorder_host
+from oracle import binding as oracle_binding
+from tests.helpers import assert_bit_exact, assert_close
+
+
+def nibble_offset(k, n, K):
+    return ((n // 64) * (K * 64) + (k // 8) * 512 + (n % 16) * 32 + ((n % 64) // 16) * 8
+            + (k % 2) * 4 + (k % 8) // 2)
+
+
+def random_u4(K, N, seed):
+    r = np.random.default_rng(seed)
+    nib = r.integers(0, 16, size=(K, N), dtype=np.uint8)
+    return nib, dtp.pack_nibbles(nib.reshape(-1))
+
+
+def woq64_view(K, N, stride_k, stride_n):
+    d = cabi.ReorderDesc()
+    lib = cabi.load_kernels()
+    cabi.check(lib.mi355_wei_pack_reorder_dims(cabi.WEI_PACK_WOQ64, K, N, stride_k, stride_n, C.byref(d)))
+    return (tuple(d.dims[i] for i in range(d.ndims)), tuple(d.src_stride[i] for i in range(d.ndims)),
+            tuple(d.dst_stride[i] for i in range(d.ndims)))
+
+
+# ------------------------------------------------------------------ CPU
+@pytest.mark.parametrize("K,N", [(32, 64), (64, 128), (96, 192)])
+def test_numpy_packer_follows_the_offset_formula(K, N):
+    nib, raw = random_u4(K, N, 7)
+    packed = dtp.unpack_nibbles(pack_woq64(raw, K, N), K * N)
+    want = np.empty(K * N, np.uint8)
+    for k in range(K):
+        for n in range(N):
+            want[nibble_offset(k, n, K)] = nib[k, n]
+    assert np.array_equal(packed, want)
+    # the formula is a bijection onto [0, K * N)
+    offs = sorted(nibble_offset(k, n, K) for k in range(K) for n in range(N))
+    assert offs == list(range(K * N))
+
+
+@pytest.mark.parametrize("transposed", [False, True])
+def test_reorder_view_packs_like_the_numpy_packer(transposed):
+    K, N = 64, 128
+    nib, raw = random_u4(K, N, 11)
+    if transposed:  # weights stored [N][K]
+        src = dtp.pack_nibbles(np.ascontiguousarray(nib.T).reshape(-1))
+        sk, sn = 1, K
+    else:
+        src, sk, sn = raw, N, 1
+    dims, ss, ds = woq64_view(K, N, sk, sn)
+    assert int(np.prod(dims)) == K * N
+    p = ReorderProblem(dims=dims, src_dt=cabi.DT_U4, dst_dt=cabi.DT_U4, src=src, src_stride=ss, dst_stride=ds)
+    got = oracle_binding.reorder(p)
+    assert np.array_equal(np.asarray(got).view(np.uint8).reshape(-1), pack_woq64(raw, K, N))
+    assert np.array_equal(pack_woq64(src, K, N, sk, sn), pack_woq64(raw, K, N))
+
+
+def test_packing_rules_of_the_matmul_descriptor():
+    p = configs.config2(M=1, N=512, K=1024)
+    p.wei_packing = cabi.WEI_PACK_WOQ64
+    st, impl = cabi.query(p.desc())
+    assert st == cabi.SUCCESS and cabi.impl_name(impl).startswith("hip:woq_packed")
+    # the generic kernel reads the layout too, the plain decode kernel and the GEMM families do not
+    assert cabi.query(p.desc(), cabi.IMPL_REF)[0] == cabi.SUCCESS
+    assert cabi.query(p.desc(), cabi.IMPL_WOQ_GEMV)[0] == cabi.UNIMPLEMENTED
+    # plain weights are not for the packed kernel
+    q = configs.config2(M=1, N=512, K=1024)
+    assert cabi.query(q.desc(), cabi.IMPL_WOQ_PACKED)[0] == cabi.UNIMPLEMENTED
+    # shapes the layout does not tile, and other weight types, are invalid
+    for M, N, K in [(1, 512 + 16, 1024), (1, 512, 1024 + 16)]:
+        b = configs.config2(M=M, N=N, K=K, group=16)
+        b.wei_packing = cabi.WEI_PACK_WOQ64
+        assert cabi.query(b.desc())[0] == cabi.INVALID_ARGUMENTS
+    c = configs.config1(M=32, N=64, K=64)
+    c.wei_packing = cabi.WEI_PACK_WOQ64
+    assert cabi.query(c.desc())[0] == cabi.INVALID_ARGUMENTS
+    # group sizes the packed kernel does not cover fall to the generic kernel
+    g = configs.config2(M=1, N=512, K=960, group=96)
+    g.wei_packing = cabi.WEI_PACK_WOQ64
+    st, impl = cabi.query(g.desc())
+    assert st == cabi.SUCCESS and cabi.impl_name(impl).startswith("hip:ref")
+    # more rows than the decode kernels take
+    m = configs.config2(M=33, N=512, K=1024)
+    m.wei_packing = cabi.WEI_PACK_WOQ64
+    assert cabi.impl_name(cabi.query(m.desc())[1]).startswith("hip:ref")
+
+
+# ------------------------------------------------------------------ GPU
+def packed(p):
+    p.wei_packing = cabi.WEI_PACK_WOQ64
+    return p
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("M", [1, 8, 32])
+def test_config2_small_packed_kernel(gpu, oracle, M):
+    # same bound as the plain decode kernel: bf16 threshold plus the forward
+    # error bound of the K sum, widened for the offset-binary form
+    p = packed(configs.config2(M=M, N=512, K=1024))
+    got, name = run_gpu(p, cabi.IMPL_WOQ_PACKED)
+    assert name.startswith("hip:woq_packed")
+    want, _, asum = oracle.run_oracle(p, want_ideal=True)
+    assert_close(p, got, want, abs_sum=asum * 20.0, what=name)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("K,group", [(32, 32), (64, 32), (256, 64), (512, 128), (1024, 1024), (2080 - 32, 2048)])
+def test_packed_one_hot_rows_are_exact(gpu, oracle, K, group):
+    # src rows are unit vectors: every output is a single decompressed weight,
+    # (w - zp) * scale with one rounding -> must equal the oracle bit for bit.
+    # Exercises the nibble order, the k order of both MFMA operands, group
+    # indexing and the split of K over wavefronts.
+    M = 32
+    p = packed(configs.config2(M=M, N=128, K=K, group=group))
+    hot = np.zeros((M, K), np.float32)
+    r = np.random.default_rng(K)
+    hot[np.arange(M), r.choice(K, size=M, replace=K < M)] = 1.0
+    p.src = dtp.f32_to_bf16(hot)
+    p.dst_dt = cabi.DT_F32
+    got, name = run_gpu(p, cabi.IMPL_WOQ_PACKED)
+    want = oracle.run_oracle(p)
+    assert_bit_exact(p, got, want, name)
+
+
+PACKED_VARIANTS = [
+    # M, N, K, group, weights, scales dt/kind, zero points dt/kind, dst, bias+relu
+    (1, 512, 1024, 128, "u4", "f32", "grouped", "s8", "grouped", "bf16", False),
+    (5, 320, 1056, 1056, "u4", "f16", "column", "u8", "column", "f32", True),   # per-column parameters, ragged K split
+    (16, 512, 512, 64, "s4", "bf16", "grouped", "s4", "grouped", "bf16", False),
+    (17, 256, 2048, 128, "s4", "bf16", "grouped", "s32", "common", "f32", False),
+    (32, 1024, 512, 32, "u4", "f32", "grouped", "u4", "none", "bf16", True),
+    (3, 4096, 256, 256, "u4", "bf16", "none", "u8", "grouped", "f32", False),
+    (8, 768, 4096, 128, "u4", "bf16", "grouped", "s32", "grouped", "bf16", False),
+    (8, 128, 4096, 512, "s4", "f16", "grouped", "s8", "grouped", "f32", True),   # a group holds several super-steps
+    (24, 192, 3072, 1024, "u4", "bf16", "grouped", "u4", "grouped", "f32", False),
+    (16, 4096, 1024, 128, "u4", "f32", "column", "u4", "common", "bf16", False),
+    (2, 14336, 256, 128, "u4", "bf16", "grouped", "s4", "column", "f32", False),
+    (20, 64, 96, 32, "u4", "bf16", "grouped", "u4", "grouped", "f32", False),    # fewer blocks than wavefronts
+    (9, 64, 2304, 256, "u4", "bf16", "grouped", "u8", "grouped", "bf16", False), # uneven K ranges
+]
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("case", PACKED_VARIANTS, ids=lambda c: "-".join(str(x) for x in c))
+def test_packed_attribute_variants(gpu, oracle, case):
+    M, N, K, group, wdt, sdt, skind, zdt, zkind, ddt, relu_bias = case
+    p = packed(configs.woq_variant(M, N, K, group, wei_dt=wdt, sc_dt=sdt, sc_kind=skind, zp_dt=zdt, zp_kind=zkind,
+                                   dst_dt=ddt, relu_bias=relu_bias))
+    got, name = run_gpu(p, cabi.IMPL_AUTO)
+    assert name.startswith("hip:woq_packed")
+    want, _, asum = oracle.run_oracle(p, want_ideal=True)
+    assert_close(p, got, want, abs_sum=asum * 20.0, what=name)
+    # and the generic kernel, reading the same packed weights, follows the
+    # reference's operation order exactly
+    got_ref, name_ref = run_gpu(p, cabi.IMPL_REF)
+    assert_bit_exact(p, got_ref, want, name_ref)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("transposed", [False, True])
+def test_gpu_reorder_writes_the_packed_layout(gpu, transposed):
+    K, N = 256, 192
+    nib, raw = random_u4(K, N, 13)
+    if transposed:
+        src = dtp.pack_nibbles(np.ascontiguousarray(nib.T).reshape(-1))
+        sk, sn = 1, K
+    else:
+        src, sk, sn = raw, N, 1
+    dims, ss, ds = woq64_view(K, N, sk, sn)
+    p = ReorderProblem(dims=dims, src_dt=cabi.DT_U4, dst_dt=cabi.DT_U4, src=src, src_stride=ss, dst_stride=ds)
+    got = reorder_host.run_gpu(p)
+    assert np.array_equal(np.asarray(got).view(np.uint8).reshape(-1), pack_woq64(raw, K, N))
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("M", [1, 32])
+def test_config2_full_size_packed_agrees_with_plain_kernel_and_sampled_oracle(gpu, oracle, M):
+    # full decode shape: the packed kernel against the plain-layout kernel
+    # (same expression, different summation order -> bf16 threshold on the
+    # decoded outputs), and both against exact f64 sums on sampled columns
+    p = configs.config2(M=M)
+    plain, name_plain = run_gpu(p, cabi.IMPL_WOQ_GEMV)
+    got, name = run_gpu(packed(p), cabi.IMPL_WOQ_PACKED)
+    assert name.startswith("hip:woq_packed") and name_plain.startswith("hip:woq_gemv")
+    a = dtp.bf16_to_f32(np.asarray(got).view(np.uint16).reshape(-1)).astype(np.float64)
+    b = dtp.bf16_to_f32(np.asarray(plain).view(np.uint16).reshape(-1)).astype(np.float64)
+    K, N, G = p.K, p.N, 128
+    src = dtp.bf16_to_f32(np.asarray(p.src).view(np.uint16).reshape(-1)).astype(np.float64).reshape(M, K)
+    w = dtp.unpack_nibbles(p.wei, K * N).reshape(K, N).astype(np.float64)
+    sc = dtp.bf16_to_f32(np.asarray(p.quant["wei_scale"].data).view(np.uint16).reshape(-1)).astype(np.float64)
+    sc = sc.reshape(K // G, N)
+    zp = dtp.unpack_nibbles(p.quant["wei_zp"].data, (K // G) * N).reshape(K // G, N).astype(np.float64)
+    cols = np.random.default_rng(5).choice(N, size=256, replace=False)
+    wd = (w[:, cols] - np.repeat(zp[:, cols], G, axis=0)) * np.repeat(sc[:, cols], G, axis=0)
+    exact = src @ wd
+    mag = np.abs(src) @ np.abs(wd)
+    # one bf16 rounding of the result plus the forward error bound of the f32
+    # K sum, widened for the offset-binary form as in the small cases
+    tol = np.abs(exact) * 2.0 ** -7 + 20.0 * mag * (K * 2.0 ** -24) + 1e-30
+    for out in (a, b):
+        o = out.reshape(M, N)[:, cols]
+        assert np.all(np.abs(o - exact) <= tol), float(np.max(np.abs(o - exact) / tol))
+    # the two kernels agree everywhere up to rounding (outputs are O(1): a
+    # misplaced column or group would be off by that much)
+    assert np.all(np.abs(a - b) <= np.maximum(np.abs(a), np.abs(b)) * 2.0 ** -6 + 0.02)
