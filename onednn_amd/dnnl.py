@@ -25,6 +25,8 @@ tag_any, tag_a, tag_ab, tag_abc, tag_abcd, tag_ba, tag_acb, tag_abdc = 1, 2, 3, 
 kind_sum, kind_eltwise, kind_binary, kind_matmul, kind_prelu = 4, 7, 13, 14, 18
 query_impl_info_str, query_src_md, query_weights_md, query_dst_md, query_scratchpad_md = 8, 129, 131, 133, 136
 query_ndims_s32, query_dims, query_data_type, query_strides, query_memory_consumption = 256, 257, 258, 14, 6
+query_format_kind = 262
+format_kind_undef, format_kind_any, format_kind_blocked, format_kind_opaque = 0, 1, 2, 3
 ARG_SRC, ARG_SRC_1, ARG_DST, ARG_WEIGHTS, ARG_BIAS, ARG_SCRATCHPAD = 1, 2, 17, 33, 41, 80
 ARG_FROM, ARG_TO = ARG_SRC, ARG_DST
 ARG_ATTR_PRECOMPUTED_REDUCTIONS, ARG_ATTR_SCALES, ARG_ATTR_ZERO_POINTS = 512, 4096, 8192
@@ -129,6 +131,11 @@ class memory_desc:
     def data_type(self):
         v = C.c_int()
         _check(lib().dnnl_memory_desc_query(self.h, query_data_type, C.byref(v)), "md_query")
+        return v.value
+
+    def format_kind(self):
+        v = C.c_int()
+        _check(lib().dnnl_memory_desc_query(self.h, query_format_kind, C.byref(v)), "md_query")
         return v.value
 
 

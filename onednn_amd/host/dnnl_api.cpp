@@ -100,6 +100,9 @@ struct dnnl_memory_desc {
     dnnl_dims_t strides = {};
     dnnl_data_type_t dt = dnnl_data_type_undef;
     dnnl_format_kind_t kind = dnnl_format_kind_undef;
+    // kind == dnnl_format_kind_opaque: the weights packing (MI355_WEI_PACK_*)
+    // that format_tag::any resolved to; strides are meaningless then
+    int packing = 0;
 
     bool is_zero() const { return ndims == 0; }
     dim_t nelems() const {
@@ -116,6 +119,7 @@ struct dnnl_memory_desc {
         return off + 1;
     }
     size_t size_bytes() const {
+        if (kind == dnnl_format_kind_opaque) return (size_t)nelems() * dt_bits(dt) / 8; // dense, no padding
         const dim_t s = span();
         return dt_bits(dt) == 4 ? (size_t)(s + 1) / 2 : (size_t)s * (dt_bits(dt) / 8);
     }
@@ -128,7 +132,7 @@ struct dnnl_memory_desc {
         kind = dnnl_blocked;
     }
     bool operator==(const dnnl_memory_desc &o) const {
-        if (ndims != o.ndims || dt != o.dt || kind != o.kind) return false;
+        if (ndims != o.ndims || dt != o.dt || kind != o.kind || packing != o.packing) return false;
         for (int i = 0; i < ndims; ++i)
             if (dims[i] != o.dims[i] || (kind == dnnl_blocked && strides[i] != o.strides[i])) return false;
         return true;
@@ -446,7 +450,13 @@ dnnl_status_t lower(dnnl_primitive_desc &pd) {
         return true;
     };
     CHECK_UNIMPL(strides3(pd.src, D.src_stride));
-    CHECK_UNIMPL(strides3(pd.wei, D.wei_stride));
+    if (pd.wei.kind == dnnl_format_kind_opaque) {
+        CHECK_UNIMPL(nd == 2);
+        D.wei_packing = pd.wei.packing;
+        D.wei_stride[0] = 0; D.wei_stride[1] = D.N; D.wei_stride[2] = 1; // not read
+    } else {
+        CHECK_UNIMPL(strides3(pd.wei, D.wei_stride));
+    }
     CHECK_UNIMPL(strides3(pd.dst, D.dst_stride));
     if (pd.with_bias) CHECK_UNIMPL(strides3(pd.bias, D.bias_stride));
     const dnnl_primitive_attr &a = pd.attr;
@@ -505,7 +515,7 @@ dnnl_status_t lower(dnnl_primitive_desc &pd) {
 
 // implementation list of the HIP engine, best first (the role of
 // engine_t::get_implementation_list, src/common/engine.hpp:134-137)
-const int k_impl_list[] = {MI355_IMPL_WOQ_GEMV, MI355_IMPL_I8_MFMA, MI355_IMPL_F8_MFMA, MI355_IMPL_MXF4_MFMA,
+const int k_impl_list[] = {MI355_IMPL_WOQ_PACKED, MI355_IMPL_WOQ_GEMV, MI355_IMPL_I8_MFMA, MI355_IMPL_F8_MFMA, MI355_IMPL_MXF4_MFMA,
         MI355_IMPL_REF};
 
 dnnl_status_t select_impl(dnnl_primitive_desc &pd) {
@@ -682,7 +692,7 @@ DNNL_EXPORT int dnnl_memory_desc_equal(const_dnnl_memory_desc_t lhs, const_dnnl_
     return *lhs == *rhs;
 }
 DNNL_EXPORT size_t dnnl_memory_desc_get_size(const_dnnl_memory_desc_t md) {
-    if (!md || md->kind != dnnl_blocked) return 0;
+    if (!md || (md->kind != dnnl_blocked && md->kind != dnnl_format_kind_opaque)) return 0;
     return md->size_bytes();
 }
 DNNL_EXPORT size_t dnnl_data_type_size(dnnl_data_type_t dt) {
@@ -1010,9 +1020,15 @@ DNNL_EXPORT dnnl_status_t dnnl_matmul_primitive_desc_create(dnnl_primitive_desc_
     // consume K-contiguous weight columns, so int8 / fp8 / fp4 weights resolve
     // to the plain transposed tag (ba, acb, ...); everything else resolves to
     // row-major (matmul_pd_t::set_default_formats, matmul_pd.hpp:419-431).
+    bool try_packed = false;
     if (pd->wei.kind == dnnl_format_kind_any) {
         dnnl_memory_desc &w = pd->wei;
         w.set_dense();
+        // 4-bit decode weights: the 64-column packing, if the packed decode
+        // kernel takes the problem and N gives it enough workgroups to fill
+        // the device (decided below, once the descriptor is lowered)
+        try_packed = pd->src.dt == dnnl_bf16 && (w.dt == dnnl_s4 || w.dt == dnnl_u4) && pd->attr.apply_to_int
+                && w.ndims == 2 && w.dims[1] >= 64 * 128;
         const bool mfma_operands = (is_int8(pd->src.dt) && is_int8(w.dt)) || (is_fp8(pd->src.dt) && is_fp8(w.dt))
                 || (pd->src.dt == dnnl_f4_e2m1 && w.dt == dnnl_f4_e2m1);
         if (mfma_operands && w.ndims >= 2) {
@@ -1044,6 +1060,16 @@ DNNL_EXPORT dnnl_status_t dnnl_matmul_primitive_desc_create(dnnl_primitive_desc_
             if (bias) CHECK_UNIMPL(bias->dt == dnnl_f32 || bias->dt == dnnl_bf16 || bias->dt == dnnl_f16 || is_fp8(bias->dt));
         }
     }
+    if (try_packed) {
+        const dnnl_memory_desc plain = pd->wei;
+        pd->wei.kind = dnnl_format_kind_opaque;
+        pd->wei.packing = MI355_WEI_PACK_WOQ64;
+        for (int i = 0; i < pd->wei.ndims; ++i) pd->wei.strides[i] = 0;
+        int chosen = 0;
+        if (lower(*pd) != dnnl_success
+                || mi355_matmul_query(&pd->desc, MI355_IMPL_WOQ_PACKED, &chosen) != MI355_SUCCESS)
+            pd->wei = plain;
+    }
     st = lower(*pd);
     if (st) return st;
     for (int impl : k_impl_list) {
@@ -1072,8 +1098,16 @@ DNNL_EXPORT dnnl_status_t dnnl_reorder_primitive_desc_create(dnnl_primitive_desc
     CHECK_ARG(src_desc->ndims == dst_desc->ndims && src_desc->ndims >= 1);
     for (int i = 0; i < src_desc->ndims; ++i) CHECK_ARG(src_desc->dims[i] == dst_desc->dims[i]);
     CHECK_UNIMPL(src_desc->ndims <= MI355_REORDER_MAX_DIMS);
+    // opaque (packed) weights: written by a reorder from plain weights of the
+    // same data type; reading them back is not offered
+    CHECK_UNIMPL(src_desc->kind == dnnl_blocked);
+    const bool to_packed = dst_desc->kind == dnnl_format_kind_opaque;
+    CHECK_UNIMPL(dst_desc->kind == dnnl_blocked || to_packed);
+    if (to_packed) CHECK_UNIMPL(src_desc->ndims == 2 && src_desc->dt == dst_desc->dt);
     std::unique_ptr<dnnl_primitive_desc> pd(new dnnl_primitive_desc);
     if (attr) pd->attr = *attr;
+    if (to_packed)
+        CHECK_UNIMPL(pd->attr.scales.empty() && pd->attr.zero_points.empty() && pd->attr.post_ops.entries.empty());
     pd->kind = dnnl_reorder;
     pd->engine = dst_engine;
     pd->src = *src_desc;
@@ -1127,6 +1161,11 @@ DNNL_EXPORT dnnl_status_t dnnl_reorder_primitive_desc_create(dnnl_primitive_desc
     if (po.size() == 1) {
         CHECK_UNIMPL(po[0].kind == dnnl_sum && po[0].zero_point == 0);
         r.beta = po[0].scale;
+    }
+    if (to_packed) {
+        const int prc = mi355_wei_pack_reorder_dims(dst_desc->packing, src_desc->dims[0], src_desc->dims[1],
+                src_desc->strides[0], src_desc->strides[1], &r);
+        if (prc != MI355_SUCCESS) return from_mi355(prc);
     }
     const int rc = mi355_reorder_query(&r);
     if (rc != MI355_SUCCESS) return from_mi355(rc);

@@ -209,6 +209,41 @@ def test_format_any_is_resolved_by_the_implementation(eng):
     assert pd.query_md(dnnl.query_weights_md).strides() == [4, 1]
 
 
+def test_format_any_decode_weights_resolve_to_the_packed_layout(eng):
+    # 4-bit weights of a decode problem wide enough to fill the device: an
+    # opaque descriptor (no strides), dense size, written by a reorder from
+    # plain weights of the same type -- the role of a blocked weights layout
+    # in the reference (brgemm_matmul_utils.cpp:203-330)
+    wo = _attr(lambda t: (t.set_fpmath_mode(dnnl.fpmath_bf16, True), t.set_scales(dnnl.ARG_WEIGHTS, 3, (128, 1), DT["bf16"]),
+                          t.set_zero_points(dnnl.ARG_WEIGHTS, 3, (128, 1), DT["u4"])))
+    K, N = 4096, 14336
+    pd = make_pd(eng, 8, K, N, "bf16", "u4", "bf16", attr=wo, wtag=dnnl.tag_any)
+    assert pd.impl_info_str().startswith("hip:woq_packed")
+    wmd = pd.query_md(dnnl.query_weights_md)
+    assert wmd.format_kind() == dnnl.format_kind_opaque and wmd.get_size() == K * N // 2 and wmd.dims() == [K, N]
+    assert status_of(lambda: wmd.strides()) == dnnl.invalid_arguments
+    assert pd.next_impl() and pd.impl_info_str() == "hip:ref:any"       # the generic kernel reads the layout too
+    # a primitive descriptor built on the queried descriptor is the same problem
+    pd2 = dnnl.matmul_primitive_desc(eng, md([8, K], "bf16"), wmd, md([8, N], "bf16"), attr=wo)
+    assert pd2.impl_info_str().startswith("hip:woq_packed")
+    # the reorder into it: same data type, no attributes
+    plain = md([K, N], "u4")
+    assert dnnl.reorder_primitive_desc(eng, plain, eng, wmd).impl_info_str() == "hip:reorder:any"
+    assert dnnl.reorder_primitive_desc(eng, md([K, N], "u4", tag=dnnl.tag_ba), eng, wmd).impl_info_str() == "hip:reorder:any"
+    assert status_of(lambda: dnnl.reorder_primitive_desc(eng, md([K, N], "f32"), eng, wmd)) == dnnl.unimplemented
+    assert status_of(lambda: dnnl.reorder_primitive_desc(eng, wmd, eng, plain)) == dnnl.unimplemented
+    ra = dnnl.primitive_attr()
+    ra.set_scales(dnnl.ARG_DST, 2)
+    assert status_of(lambda: dnnl.reorder_primitive_desc(eng, plain, eng, wmd, attr=ra)) == dnnl.unimplemented
+    # narrow N, more rows than a decode, or a group size the packed kernel does not take: plain row-major
+    assert make_pd(eng, 8, K, 4096, "bf16", "u4", "bf16", attr=wo, wtag=dnnl.tag_any).query_md(dnnl.query_weights_md).strides() == [4096, 1]
+    assert make_pd(eng, 64, K, N, "bf16", "u4", "bf16", attr=wo, wtag=dnnl.tag_any).query_md(dnnl.query_weights_md).strides() == [N, 1]
+    odd = _attr(lambda t: (t.set_fpmath_mode(dnnl.fpmath_bf16, True), t.set_scales(dnnl.ARG_WEIGHTS, 3, (96, 1), DT["bf16"])))
+    assert make_pd(eng, 8, 960, N, "bf16", "u4", "bf16", attr=odd, wtag=dnnl.tag_any).query_md(dnnl.query_weights_md).strides() == [N, 1]
+    # explicit row-major weights keep the plain decode kernel
+    assert make_pd(eng, 8, K, N, "bf16", "u4", "bf16", attr=wo).impl_info_str().startswith("hip:woq_gemv")
+
+
 def test_user_scratchpad_is_reported(eng):
     a = dnnl.primitive_attr()
     a.set_scratchpad_mode(dnnl.scratchpad_user)

@@ -181,3 +181,40 @@ def test_quantize_and_prepack_weights_with_reorder_then_matmul(gpu, oracle):
                        wei_stride=(K * N, 1, K), quant={"wei_scale": QuantParam(cabi.DT_F32, 4, wsc)})
     want = oracle.run_oracle(mp)
     assert_close(mp, dst.read(np.float32), want)
+
+
+def test_prepack_decode_weights_with_reorder_then_matmul(gpu, oracle):
+    """format `any` for 4-bit decode weights: the matmul pd answers with an
+    opaque packed descriptor, a reorder brings the plain u4 weights there, the
+    matmul runs on the packed memory (the flow of the reference's
+    matmul_with_weight_only_quantization.cpp:181-189 with blocked weights)."""
+    from onednn_amd.problem import pack_woq64
+    p = configs.config2(M=8, N=8192, K=512)
+    M, K, N = p.M, p.K, p.N
+    eng = dnnl.engine(dnnl.gpu, 0)
+    strm = dnnl.stream(eng)
+    src_md = dnnl.memory_desc([M, K], DT["bf16"], tag=dnnl.tag_ab)
+    dst_md = dnnl.memory_desc([M, N], DT["bf16"], tag=dnnl.tag_ab)
+    attr = dnnl.primitive_attr()
+    attr.set_fpmath_mode(dnnl.fpmath_bf16, True)
+    attr.set_scales(dnnl.ARG_WEIGHTS, 3, (128, 1), DT["bf16"])
+    attr.set_zero_points(dnnl.ARG_WEIGHTS, 3, (128, 1), DT["u4"])
+    pd = dnnl.matmul_primitive_desc(eng, src_md, dnnl.memory_desc([K, N], DT["u4"], tag=dnnl.tag_any), dst_md, attr=attr)
+    assert pd.impl_info_str().startswith("hip:woq_packed")
+    wei_md = pd.query_md(dnnl.query_weights_md)
+    assert wei_md.format_kind() == dnnl.format_kind_opaque
+    user_md = dnnl.memory_desc([K, N], DT["u4"], tag=dnnl.tag_ab)
+    wei_mem = dnnl.memory(wei_md, eng)
+    dnnl.reorder(dnnl.reorder_primitive_desc(eng, user_md, eng, wei_md)).execute(
+        strm, {dnnl.ARG_FROM: dnnl.memory(user_md, eng, p.wei), dnnl.ARG_TO: wei_mem})
+    G = K // 128
+    sc_mem = dnnl.memory(dnnl.memory_desc([G, N], DT["bf16"], tag=dnnl.tag_ab), eng, p.quant["wei_scale"].data)
+    zp_mem = dnnl.memory(dnnl.memory_desc([G, N], DT["u4"], tag=dnnl.tag_ab), eng, p.quant["wei_zp"].data)
+    dst = dnnl.memory(dst_md, eng)
+    dnnl.matmul(pd).execute(strm, {dnnl.ARG_SRC: dnnl.memory(src_md, eng, p.src), dnnl.ARG_WEIGHTS: wei_mem,
+                                   dnnl.ARG_DST: dst, dnnl.ARG_ATTR_SCALES | dnnl.ARG_WEIGHTS: sc_mem,
+                                   dnnl.ARG_ATTR_ZERO_POINTS | dnnl.ARG_WEIGHTS: zp_mem})
+    strm.wait()
+    assert np.array_equal(wei_mem.read(np.uint8), pack_woq64(p.wei, K, N))
+    want, _, asum = oracle.run_oracle(p, want_ideal=True)
+    assert_close(p, dst.read(np.uint16), want, abs_sum=asum * 20.0, what=pd.impl_info_str())
