@@ -27,6 +27,7 @@
 // across quantization groups and add them through LDS at the end, in wavefront
 // order: results do not depend on timing.
 #include "kernels.hpp"
+#include "tile_epilogue.hpp"
 
 #include <type_traits>
 
@@ -239,26 +240,46 @@ __global__ void __launch_bounds__(NWV * 64) woqp_kernel(const problem_t P_, cons
             super_step(kb, ns, std::false_type {});
     }
 
-    // ---- add the wavefronts' sums in wavefront order and store
+    // ---- add the wavefronts' sums in wavefront order and store.  LDS holds
+    // [wavefront][row][column] floats; a thread then owns four consecutive
+    // columns of one row and runs the four-wide epilogue of the GEMM tiles.
+    float *red = (float *)red4;
+    constexpr int WSTRIDE = MT * 16 * CHUNK; // floats per wavefront
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt)
 #pragma unroll
-        for (int tt = 0; tt < 4; ++tt) red4[((wave * MT + mt) * 4 + tt) * 64 + lane] = tot[mt][tt];
+        for (int tt = 0; tt < 4; ++tt)
+#pragma unroll
+            for (int r = 0; r < 4; ++r)
+                red[wave * WSTRIDE + (mt * 16 + 4 * q + r) * CHUNK + tt * 16 + j] = tot[mt][tt][r];
     __syncthreads();
     const auto &P = MI355_KERNARG_PROBLEM();
-    // one dst element per thread and pass, 64 consecutive columns per wavefront
-    const float *red = (const float *)red4;
-    constexpr int WSTRIDE = MT * 4 * 64 * 4; // floats per wavefront
-#pragma unroll 1
-    for (int e = t; e < MT * 16 * CHUNK; e += NWV * 64) {
-        const int m = e >> 6; // uniform in a wavefront
-        if (m >= M) break;
-        const int nl = e & 63, mt = m >> 4, mq = (m >> 2) & 3, r = m & 3;
-        const float *cell = red + (((mt * 4 + (nl >> 4)) * 64 + mq * 16 + (nl & 15)) * 4 + r);
+    if (M <= 8) {
+        // few rows: one element per thread, 64 consecutive columns per
+        // wavefront (the four-wide path below starts later: it gathers the
+        // epilogue's operands first, which a single pass does not win back)
+        const int m = t >> 6, nl = t & 63;
+        if (m >= M) return;
+        const float *cell = red + m * CHUNK + nl;
         float v = cell[0];
 #pragma unroll
         for (int wv = 1; wv < NWV; ++wv) v += cell[wv * WSTRIDE];
         epilogue_store(P, v, 0, m, chunk * CHUNK + nl);
+        return;
+    }
+#pragma unroll 1
+    for (int e = t; e < MT * 16 * (CHUNK / 4); e += NWV * 64) {
+        const int m = e >> 4, nq = e & 15;
+        if (m >= M) continue;
+        const v4f *cell = (const v4f *)(red + m * CHUNK + nq * 4);
+        v4f sum = cell[0];
+#pragma unroll
+        for (int wv = 1; wv < NWV; ++wv) sum += cell[wv * (WSTRIDE / 4)];
+        float v[4] = {sum[0], sum[1], sum[2], sum[3]};
+        const long n = (long)chunk * CHUNK + nq * 4;
+        const gemm::epi_hoist_t H = gemm::make_hoist(P, 0, n, 4, false);
+        gemm::apply_epilogue4(P, H, v, 0, m, n, 4, make_uint4(0, 0, 0, 0));
+        gemm::store4(P, H, v, 0, m, n, 4);
     }
 }
 
