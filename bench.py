@@ -42,7 +42,9 @@ import numpy as np  # noqa: E402
 # profiles/<kernel>_<workload>.md.  Keyed by (workload, M).
 MEASURED_TRAFFIC = {
     ("c3", 8192): 1008038840, ("c4", 4096): 2597323049, ("c5", 8192): 569589287,
-    ("c2", 1): 32839918, ("c2", 8): 35736510, ("c2", 32): 51670432, ("c1", 256): 8357752,
+    ("c2", 1): 31612633, ("c2", 8): 32271601, ("c2", 32): 34542741,        # packed weights (format any)
+    ("c2ab", 1): 32839597, ("c2ab", 8): 35736697, ("c2ab", 32): 51670775,  # plain ab weights (--wtag ab)
+    ("c1", 256): 8357752,
 }
 
 # MI355X published peaks
@@ -156,7 +158,7 @@ def run_gpu_workload(lib, name, steps, warmup, M=None, cold_copies=0, wtag="any"
     return out, p
 
 
-def run_reorder_workloads(lib, steps, which=("r1", "r2")):
+def run_reorder_workloads(lib, steps, which=("r1", "r2", "r3")):
     """Informational: the reorder primitive on the tensors of the headline
     shape (HBM-bound; bytes = src + dst + parameter tensors)."""
     import numpy as np
@@ -176,6 +178,17 @@ def run_reorder_workloads(lib, steps, which=("r1", "r2")):
                               name="R2 s8 8192x8192 ab->ba (weights into the layout format_tag::any resolves to)"),
                2 * N * N),
     }
+    if "r3" in which:
+        import ctypes as C
+        K3, N3 = 4096, 14336
+        d = cabi.ReorderDesc()
+        cabi.check(lib.mi355_wei_pack_reorder_dims(cabi.WEI_PACK_WOQ64, K3, N3, N3, 1, C.byref(d)))
+        w4 = rng.integers(0, 256, size=K3 * N3 // 2, dtype=np.uint8)
+        plan["r3"] = (ReorderProblem(dims=tuple(d.dims[i] for i in range(6)), src_dt=cabi.DT_U4, dst_dt=cabi.DT_U4,
+                                     src=w4, src_stride=tuple(d.src_stride[i] for i in range(6)),
+                                     dst_stride=tuple(d.dst_stride[i] for i in range(6)),
+                                     name="R3 u4 4096x14336 ab -> packed decode layout (what format_tag::any resolves to)"),
+                      K3 * N3)
     out = []
     timer = Timer(lib)
     for key in which:
@@ -236,7 +249,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=3)
-    ap.add_argument("--workload", default="c3", choices=["c1", "c2", "c3", "c4", "c5", "r1", "r2"],
+    ap.add_argument("--workload", default="c3", choices=["c1", "c2", "c3", "c4", "c5", "r1", "r2", "r3"],
                     help="c1..c5: the matmul configurations (c3 is the headline); r1, r2: the reorder "
                          "primitive on the headline shape's tensors (informational)")
     ap.add_argument("--decode-m", type=int, default=1, help="M of the c2 decode workload")
@@ -277,14 +290,14 @@ def main():
         a.free()
         b.free()
 
-    if main_name in ("r1", "r2"):
+    if main_name in ("r1", "r2", "r3"):
         r = run_reorder_workloads(lib, args.steps, (main_name,))[0]
         if args.calib_copy:
             calib_copy()
         print(json.dumps({
             "metric": "reorder GB/s", "value": r["value"], "unit": "GB/s", "n_gpus": 1, "steps": args.steps,
             "warmup": args.warmup, "ms_per_step": r["ms_per_step"], "higher_is_better": True, "scaling": "weak",
-            "vs_baseline": None, "dtype": "f32" if main_name == "r1" else "s8", "data": "synthetic",
+            "vs_baseline": None, "dtype": {"r1": "f32", "r2": "s8", "r3": "u4"}[main_name], "data": "synthetic",
             "config": {"workload": r["workload"], "impl": r["impl"]},
             "roofline": {"bound": "hbm", "achieved": r["value"], "peak": PEAK_HBM_GBS, "unit": "GB/s",
                          "frac": r["frac_of_peak"], "traffic": None, "algorithmic": r["work"],
@@ -308,7 +321,8 @@ def main():
     roofline = {
         "bound": res["bound"], "achieved": res["value"], "peak": res["peak"],
         "unit": "GB/s" if res["unit"] == "GB/s" else "TFLOP/s",
-        "frac": res["value"] / res["peak"], "traffic": MEASURED_TRAFFIC.get((main_name, prob.M)),
+        "frac": res["value"] / res["peak"], "traffic": MEASURED_TRAFFIC.get(
+            ("c2ab" if main_name == "c2" and args.wtag != "any" else main_name, prob.M)),
         "algorithmic": res["work"], "kernel": res["impl"], "kernel_ms": res["ms_per_step"],
     }
 

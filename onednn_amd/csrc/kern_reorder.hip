@@ -486,6 +486,85 @@ int check(const mi355_reorder_desc_t *d) {
     return MI355_SUCCESS;
 }
 
+// ---- plain 4-bit weights -> MI355_WEI_PACK_WOQ64, the one reorder whose dst
+// is not a plain strided tensor at heart: the generic kernels above handle its
+// six-dim view correctly but four nibbles at a time.  One thread writes the 16
+// bytes one lane of the decode kernel reads: rows 8kq .. 8kq+7 of the columns
+// 64c + 16t + j, t = 0..3.
+//   ROW_MAJOR: src [K][N], row pitch `pitch` bytes: the thread reads the 32
+//     bytes of its chunk in each of the 8 rows (shared by the 16 threads of
+//     the same (c, kq): cache hits) and picks nibble j of every 8-byte block.
+//   else: src [N][K], column pitch `pitch` bytes: the 8 rows of a column are
+//     one dword, its even nibbles go to the low half, the odd ones to the high.
+template <bool ROW_MAJOR>
+__global__ void __launch_bounds__(256) pack_woq64_kernel(const uint8_t *src, uint8_t *dst, int K, int N, long pitch) {
+    const long g = (long)blockIdx.x * 256 + threadIdx.x; // (c, kq, j), j fastest: 16 bytes of dst each
+    const long total = (long)(N / 64) * (K / 8) * 16;
+    if (g >= total) return;
+    const int j = (int)(g & 15);
+    const long ckq = g >> 4;
+    const int kq = (int)(ckq % (K / 8));
+    const int c = (int)(ckq / (K / 8));
+    unsigned out[4] = {0u, 0u, 0u, 0u};
+    if (ROW_MAJOR) {
+#pragma unroll
+        for (int r = 0; r < 8; ++r) {
+            const uint4 *row = (const uint4 *)(src + (long)(kq * 8 + r) * pitch + c * 32);
+            const uint4 lo = row[0], hi = row[1];
+            const unsigned long long blk[4] = {lo.x | ((unsigned long long)lo.y << 32), lo.z | ((unsigned long long)lo.w << 32),
+                    hi.x | ((unsigned long long)hi.y << 32), hi.z | ((unsigned long long)hi.w << 32)};
+            const int pos = (r & 1) * 4 + (r >> 1);
+#pragma unroll
+            for (int t = 0; t < 4; ++t) out[t] |= (unsigned)((blk[t] >> (4 * j)) & 0xfull) << (4 * pos);
+        }
+    } else {
+#pragma unroll
+        for (int t = 0; t < 4; ++t) {
+            const unsigned w = *(const unsigned *)(src + (long)(c * 64 + t * 16 + j) * pitch + kq * 4);
+            unsigned even = w & 0x0f0f0f0fu, odd = (w >> 4) & 0x0f0f0f0fu; // nibbles k = 0,2,4,6 / 1,3,5,7, one per byte
+            // compact four byte-spaced nibbles into 16 bits
+            even = (even | (even >> 4)) & 0x00ff00ffu;
+            even = (even | (even >> 8)) & 0x0000ffffu;
+            odd = (odd | (odd >> 4)) & 0x00ff00ffu;
+            odd = (odd | (odd >> 8)) & 0x0000ffffu;
+            out[t] = even | (odd << 16);
+        }
+    }
+    uint4 o;
+    o.x = out[0]; o.y = out[1]; o.z = out[2]; o.w = out[3];
+    *(uint4 *)(dst + g * 16) = o;
+}
+
+// the six-dim view mi355_wei_pack_reorder_dims writes, with a src the kernel
+// above can read: returns 1 (row-major src), 2 (column-major src) or 0
+int woq64_fast_path(const mi355_reorder_desc_t &d, const mi355_reorder_args_t &a, long *K, long *N, long *pitch) {
+    if (d.ndims != 6 || d.src_dt != d.dst_dt || dt_bits(d.src_dt) != 4 || d.beta != 0.f) return 0;
+    if (d.src_scale.dt != MI355_DT_UNDEF || d.dst_scale.dt != MI355_DT_UNDEF || d.src_zp.dt != MI355_DT_UNDEF
+            || d.dst_zp.dt != MI355_DT_UNDEF)
+        return 0;
+    if (d.dims[1] != 4 || d.dims[2] != 2 || d.dims[4] != 4 || d.dims[5] != 16) return 0;
+    *K = d.dims[0] * 8;
+    *N = d.dims[3] * 64;
+    if (*K % 32 || *K >= (1L << 31) || *N >= (1L << 31)) return 0;
+    const int64_t ds[6] = {512, 1, 4, *K * 64, 8, 32};
+    for (int i = 0; i < 6; ++i)
+        if (d.dst_stride[i] != ds[i]) return 0;
+    const int64_t sk = d.src_stride[2], sn = d.src_stride[5];
+    const int64_t ss[6] = {8 * sk, 2 * sk, sk, 64 * sn, 16 * sn, sn};
+    for (int i = 0; i < 6; ++i)
+        if (d.src_stride[i] != ss[i]) return 0;
+    if (((uintptr_t)a.dst & 15) != 0) return 0;
+    if (sn == 1 && sk >= *N && sk % 32 == 0 && ((uintptr_t)a.src & 15) == 0) {
+        *pitch = sk / 2;
+        return 1;
+    }
+    if (sk == 1 && sn >= *K && sn % 8 == 0 && ((uintptr_t)a.src & 3) == 0) {
+        *pitch = sn / 2;
+        return 2;
+    }
+    return 0;
+}
+
 } // namespace
 } // namespace mi355
 
@@ -520,6 +599,25 @@ extern "C" int mi355_reorder_launch(const mi355_reorder_desc_t *desc, const mi35
         }
     for (int i = 0; i < d.ndims; ++i)
         if (d.dims[i] >= (1L << 31)) return MI355_UNIMPLEMENTED;
+    {
+        long K = 0, N = 0, pitch = 0;
+        const int fast = woq64_fast_path(d, *args, &K, &N, &pitch);
+        if (fast) {
+            const long threads = (N / 64) * (K / 8) * 16;
+            const dim3 grid((unsigned)((threads + 255) / 256)), block(256);
+            if (fast == 1)
+                hipLaunchKernelGGL(pack_woq64_kernel<true>, grid, block, 0, (hipStream_t)stream,
+                        (const uint8_t *)args->src, (uint8_t *)args->dst, (int)K, (int)N, pitch);
+            else
+                hipLaunchKernelGGL(pack_woq64_kernel<false>, grid, block, 0, (hipStream_t)stream,
+                        (const uint8_t *)args->src, (uint8_t *)args->dst, (int)K, (int)N, pitch);
+            if (hipGetLastError() != hipSuccess) {
+                set_error("reorder: launch failed");
+                return MI355_RUNTIME_ERROR;
+            }
+            return MI355_SUCCESS;
+        }
+    }
 
     reorder_t R {};
     R.src_dt = d.src_dt;

@@ -173,15 +173,22 @@ def test_packed_attribute_variants(gpu, oracle, case):
 
 
 @pytest.mark.gpu
+@pytest.mark.parametrize("pad", [0, 2, 64])
 @pytest.mark.parametrize("transposed", [False, True])
-def test_gpu_reorder_writes_the_packed_layout(gpu, transposed):
+def test_gpu_reorder_writes_the_packed_layout(gpu, transposed, pad):
+    # pad = 0 / 64: pitches the dedicated packing kernel takes (16-byte rows,
+    # 4-byte columns); pad = 2: the generic strided kernels on the six-dim view
     K, N = 256, 192
     nib, raw = random_u4(K, N, 13)
     if transposed:
-        src = dtp.pack_nibbles(np.ascontiguousarray(nib.T).reshape(-1))
-        sk, sn = 1, K
+        wide = np.zeros((N, K + pad), np.uint8)
+        wide[:, :K] = nib.T
+        sk, sn = 1, K + pad
     else:
-        src, sk, sn = raw, N, 1
+        wide = np.zeros((K, N + pad), np.uint8)
+        wide[:, :N] = nib
+        sk, sn = N + pad, 1
+    src = dtp.pack_nibbles(wide.reshape(-1))
     dims, ss, ds = woq64_view(K, N, sk, sn)
     p = ReorderProblem(dims=dims, src_dt=cabi.DT_U4, dst_dt=cabi.DT_U4, src=src, src_stride=ss, dst_stride=ds)
     got = reorder_host.run_gpu(p)
