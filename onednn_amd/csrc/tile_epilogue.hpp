@@ -664,18 +664,27 @@ struct layout32_t {
     template <class T, int R, int C>
     static __device__ __forceinline__ void write_slab(const T (&acc)[R][C], int s, slab_int_t *wl, int lane) {
         constexpr int WCOLS = C * 32;
-        // volatile: the dword stores stay single ds_write_b32 instructions.  Merged
-        // into ds_write2_b32 pairs by the compiler (ROCm 7.2), two stores per tile
-        // of this layout came out with their first offset divided by four and
-        // landed in other cells of the slab; the parity tests caught it.
-        volatile slab_int_t *vw = wl;
+        // The stores are written as ds_write_b32 instructions by hand.  Left to
+        // the compiler (ROCm 7.2) they were merged into ds_write2_b32 pairs, and
+        // two stores per tile of this layout came out with their first offset
+        // divided by four and landed in other cells of the slab (the parity
+        // tests caught it); as volatile stores they stayed single but each one
+        // was followed by a wait for the LDS queue to drain, 11-12 us per slab.
+        const unsigned base = (unsigned)(size_t)(__attribute__((address_space(3))) char *)(char *)wl
+                + (unsigned)(((lane >> 5) * 4 * WCOLS + (lane & 31)) * 4);
         T a[C];
         pick_rows(acc, s, a);
 #pragma unroll
         for (int j = 0; j < C; ++j)
 #pragma unroll
-            for (int r = 0; r < 16; ++r)
-                vw[((r >> 2) * 8 + (lane >> 5) * 4 + (r & 3)) * WCOLS + j * 32 + (lane & 31)] = raw_bits(a[j][r]);
+            for (int r = 0; r < 16; ++r) {
+                const unsigned addr = base + (unsigned)((((r >> 2) * 8 + (r & 3)) * WCOLS + j * 32) * 4);
+                asm volatile("ds_write_b32 %0, %1" : : "v"(addr), "v"(raw_bits(a[j][r])) : "memory");
+            }
+        // the wavefront reads its own slab next: LDS operations of one
+        // wavefront complete in order, the wait only keeps the compiler's own
+        // counter bookkeeping (which does not see these stores) conservative
+        asm volatile("s_waitcnt lgkmcnt(0)" : : : "memory");
     }
     template <class T, int R, int C>
     static __device__ __forceinline__ void pick_rows(const T (&acc)[R][C], int s, T (&a)[C]) {
