@@ -127,6 +127,21 @@ enum {
     MI355_DST_SCALE_RECIPROCAL = 1
 };
 
+/* Dynamic quantization of dst (quantization_mode::dynamic_mx): the scales of
+ * DNNL_ARG_DST are an OUTPUT of the primitive.  For every group of 32
+ * consecutive n of one dst row (ref_matmul.cpp:338-423; rules
+ * src/common/matmul.cpp:407-424: full mask, groups 1 x 32, e8m0 scales)
+ *     amax  = max |d| over the group, d after bias and post-ops
+ *     scale = e8m0(e8m0(amax) / e8m0(max of dst type)), e8m0(x) = 2^floor(log2 x)
+ *             (the exponent byte of x; 2^-127 for a zero exponent)
+ *     args->dst_scale[(b, m, n / 32)] = scale       (written, despite the const)
+ *     dst = convert(clamp(d * (1 / scale), -max, +max))
+ * dst is f8_e4m3 or f8_e5m2, N % 32 == 0, no dst zero point. */
+enum {
+    MI355_DST_DYNAMIC_NONE = 0,
+    MI355_DST_DYNAMIC_MX = 1
+};
+
 /* Kernel families (implementation ids). 0 lets the library choose. */
 enum {
     MI355_IMPL_AUTO = 0,
@@ -209,6 +224,8 @@ typedef struct mi355_matmul_desc {
     mi355_post_op_t post_ops[MI355_MAX_POST_OPS];
     int32_t impl; /* MI355_IMPL_*; AUTO picks the fastest applicable */
     int32_t wei_packing; /* MI355_WEI_PACK_* */
+    int32_t dst_scale_dynamic; /* MI355_DST_DYNAMIC_* */
+    int32_t reserved;
 } mi355_matmul_desc_t;
 
 typedef struct mi355_matmul_args {

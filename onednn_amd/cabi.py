@@ -42,6 +42,7 @@ BINARY = {
 DST_SCALE_DIVIDE, DST_SCALE_RECIPROCAL = 0, 1
 IMPL_AUTO, IMPL_REF, IMPL_I8_MFMA, IMPL_F8_MFMA, IMPL_MXF4_MFMA, IMPL_WOQ_GEMV, IMPL_WOQ_PACKED = range(7)
 WEI_PACK_NONE, WEI_PACK_WOQ64 = 0, 1
+DST_DYNAMIC_NONE, DST_DYNAMIC_MX = 0, 1
 
 
 class Quant(C.Structure):
@@ -66,6 +67,7 @@ class MatmulDesc(C.Structure):
         ("dst_scale_mode", C.c_int32), ("n_post_ops", C.c_int32),
         ("post_ops", PostOp * MAX_POST_OPS),
         ("impl", C.c_int32), ("wei_packing", C.c_int32),
+        ("dst_scale_dynamic", C.c_int32), ("reserved", C.c_int32),
     ]
 
 

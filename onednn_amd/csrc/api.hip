@@ -67,6 +67,17 @@ static int validate(const mi355_matmul_desc_t *d) {
         set_error("weights packing %d needs 4-bit weights, batch 1, K %% 32 == 0 and N %% 64 == 0", d->wei_packing);
         return MI355_INVALID_ARGUMENTS;
     }
+    if (d->dst_scale_dynamic != MI355_DST_DYNAMIC_NONE) {
+        // src/common/matmul.cpp:407-424
+        const mi355_quant_t &q = d->dst_scale;
+        const bool ok = d->dst_scale_dynamic == MI355_DST_DYNAMIC_MX && q.dt == MI355_DT_E8M0
+                && (q.mask & 6) == 6 && (d->batch == 1 || (q.mask & 1)) && q.group[0] == 1 && q.group[1] == 32
+                && d->N % 32 == 0 && is_f8_dt(d->dst_dt) && quant_absent(d->dst_zp);
+        if (!ok) {
+            set_error("dynamic dst scales: e8m0, full mask, groups 1 x 32, N %% 32 == 0, f8 dst, no dst zero point");
+            return MI355_INVALID_ARGUMENTS;
+        }
+    }
     int st;
     if ((st = check_quant(d->src_scale, "src scale"))) return st;
     if ((st = check_quant(d->wei_scale, "weights scale"))) return st;
@@ -96,6 +107,8 @@ static int validate(const mi355_matmul_desc_t *d) {
 typedef int (*supported_fn)(const mi355_matmul_desc_t &);
 
 static int impl_supported(const mi355_matmul_desc_t &d, int impl) {
+    // dynamic dst quantization: the generic kernel only
+    if (d.dst_scale_dynamic != MI355_DST_DYNAMIC_NONE && impl != MI355_IMPL_REF) return MI355_UNIMPLEMENTED;
     switch (impl) {
         case MI355_IMPL_REF: return ref_supported(d);
         case MI355_IMPL_I8_MFMA: return i8_supported(d);
@@ -155,6 +168,7 @@ static int build_problem(const mi355_matmul_desc_t &d, const mi355_matmul_args_t
     P.n_po = d.n_post_ops;
     P.sum_dt = MI355_DT_UNDEF;
     P.wei_packing = d.wei_packing;
+    P.dst_dynamic = d.dst_scale_dynamic;
     P.src = a.src; P.wei = a.wei; P.bias = a.bias; P.dst = a.dst;
     const struct { const mi355_quant_t *q; const void *p; const char *n; } need[] = {
             {&d.src_scale, a.src_scale, "src scale"}, {&d.wei_scale, a.wei_scale, "weights scale"},

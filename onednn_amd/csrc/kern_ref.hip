@@ -125,16 +125,62 @@ __global__ void __launch_bounds__(256) ref_matmul_kernel(const problem_t P_) {
     }
 }
 
+// Dynamic (MX) quantization of dst, ref_matmul.cpp:268-423: one thread per
+// group of 32 consecutive n of a dst row.  The values of the group are
+// computed exactly as above, their largest magnitude gives the group's e8m0
+// scale, which is written to the scales tensor and applied by a multiplication
+// with its (exact, power of two) inverse.
+__global__ void __launch_bounds__(64) ref_matmul_dynamic_kernel(const problem_t P_) {
+    const auto &P = MI355_KERNARG_PROBLEM();
+    constexpr int G = 32;
+    const long groups_n = P.N / G;
+    const long total = P.B * P.M * groups_n;
+    const float dt_max = P.dst_dt == MI355_DT_F8_E4M3 ? 448.f : 57344.f;
+    const bool int_path = P.src_dt == MI355_DT_S8 || P.src_dt == MI355_DT_U8;
+    for (long i = (long)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += (long)gridDim.x * blockDim.x) {
+        const long ng = i % groups_n, m = (i / groups_n) % P.M, b = i / (groups_n * P.M);
+        float d[G];
+        float amax = 0.f;
+#pragma unroll 1
+        for (int e = 0; e < G; ++e) {
+            const long n = ng * G + e;
+            const float v = int_path ? ref_int_dot(P, b, m, n) : ref_fp_dot(P, b, m, n);
+            d[e] = epilogue_value(P, v, b, m, n);
+        }
+#pragma unroll
+        for (int e = 0; e < G; ++e) amax = fmaxf(amax, fabsf(d[e]));
+        // e8m0(x): the exponent byte of x
+        const float r = e8m0_to_f32(f32_to_e8m0(amax)) / e8m0_to_f32(f32_to_e8m0(dt_max));
+        const uint8_t sbyte = f32_to_e8m0(r);
+        ((uint8_t *)P.dst_scale.p)[quant_off(P.dst_scale, b, m, ng * G, P.M, P.N)] = sbyte;
+        const float inv = 1.f / e8m0_to_f32(sbyte);
+#pragma unroll
+        for (int e = 0; e < G; ++e) {
+            float v = d[e] * inv;
+            v = fminf(fmaxf(v, -dt_max), dt_max);
+            store_float(P.dst_dt, v, P.dst, b * P.ds[0] + m * P.ds[1] + (ng * G + e) * P.ds[2]);
+        }
+    }
+}
+
 int ref_supported(const mi355_matmul_desc_t &d) {
     // 4-bit dst would need two elements per thread; not offered.
     if (dt_bits(d.dst_dt) < 8) return MI355_UNIMPLEMENTED;
     if (d.wei_packing != MI355_WEI_PACK_NONE && !woq64_layout_ok(d)) return MI355_UNIMPLEMENTED;
+    // dynamic dst quantization exists in ref_matmul_t only, not in the integer implementation
+    if (d.dst_scale_dynamic != MI355_DST_DYNAMIC_NONE && is_int8_dt(d.src_dt)) return MI355_UNIMPLEMENTED;
     return MI355_SUCCESS;
 }
 
 int ref_launch(const problem_t &P, hipStream_t stream) {
     const long total = P.B * P.M * P.N;
     if (total == 0) return MI355_SUCCESS;
+    if (P.dst_dynamic) {
+        long groups = total / 32, gblocks = (groups + 63) / 64;
+        if (gblocks > 1048576) gblocks = 1048576;
+        hipLaunchKernelGGL(ref_matmul_dynamic_kernel, dim3((unsigned)gblocks), dim3(64), 0, stream, P);
+        return hipGetLastError() == hipSuccess ? MI355_SUCCESS : MI355_RUNTIME_ERROR;
+    }
     long blocks = (total + 255) / 256;
     if (blocks > 1048576) blocks = 1048576;
     hipLaunchKernelGGL(ref_matmul_kernel, dim3((unsigned)blocks), dim3(256), 0, stream, P);

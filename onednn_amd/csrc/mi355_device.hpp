@@ -35,7 +35,7 @@ struct problem_t {
     long ss[3], ws[3], ds[3], bs[3];
     quant_dev_t src_scale, wei_scale, dst_scale, src_zp, wei_zp, dst_zp, src_pr;
     int apply_to_int, dst_scale_mode, n_po, sum_dt;
-    int wei_packing, pad_;
+    int wei_packing, dst_dynamic;
     const void *src, *wei, *bias;
     void *dst;
     po_dev_t po[MI355_MAX_POST_OPS];
@@ -240,6 +240,7 @@ __device__ __forceinline__ float epilogue_value(
             }
         }
     }
+    if (P.dst_dynamic) return v; // the group's scale is computed from these values
     if (P.dst_scale.dt != MI355_DT_UNDEF) {
         const float s = load_float(P.dst_scale.dt, P.dst_scale.p, 0);
         if (P.dst_scale_mode == MI355_DST_SCALE_RECIPROCAL) {

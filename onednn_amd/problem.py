@@ -132,6 +132,7 @@ class MatmulProblem:
     dst_scale_mode: int = cabi.DST_SCALE_DIVIDE
     impl: int = cabi.IMPL_AUTO
     wei_packing: int = cabi.WEI_PACK_NONE  # `wei` stays plain here; GpuRun uploads it packed
+    dst_dynamic: int = cabi.DST_DYNAMIC_NONE  # quant["dst_scale"].data is then an output (its content is ignored)
     dst_init: Optional[np.ndarray] = None   # prior dst content (sum post-op)
     name: str = ""
 
@@ -180,6 +181,7 @@ class MatmulProblem:
                 o.stride[j] = po.stride[j]
         d.impl = self.impl
         d.wei_packing = self.wei_packing
+        d.dst_scale_dynamic = self.dst_dynamic
         return d
 
     def initial_dst(self):
@@ -245,6 +247,12 @@ class GpuRun:
     def result(self):
         self.sync()
         return self.bufs["dst"].to_numpy(storage_dtype(self.prob.dst_dt), self.dst_host_shape)
+
+    def dynamic_scales(self):
+        """The dst scales a dynamic-quantization launch wrote (raw storage)."""
+        self.sync()
+        q = self.prob.quant["dst_scale"]
+        return self.bufs["dst_scale"].to_numpy(q.data.dtype, q.data.shape)
 
     def free(self):
         for b in self.bufs.values():

@@ -83,6 +83,24 @@ def run_oracle(prob: MatmulProblem, flags=0, want_ideal=False):
     return dst
 
 
+def run_oracle_dynamic(prob: MatmulProblem, flags=0):
+    """Dynamic dst quantization: returns (raw dst storage, raw dst scales)."""
+    lib = load()
+    dst = prob.initial_dst()
+    desc = prob.desc()
+    saved = prob.quant["dst_scale"].data
+    scales = np.zeros_like(np.ascontiguousarray(saved))
+    prob.quant["dst_scale"].data = scales
+    try:
+        args, keep = host_args(prob, dst)
+        st = lib.oracle_matmul(C.byref(desc), C.byref(args), flags, None, None)
+    finally:
+        prob.quant["dst_scale"].data = saved
+    assert st == 0, f"oracle_matmul status {st}"
+    del keep
+    return dst, scales
+
+
 def run_int8_acc(prob: MatmulProblem):
     lib = load()
     dst = prob.initial_dst()

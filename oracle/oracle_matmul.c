@@ -43,6 +43,11 @@
  * restatements with forward error bounds).  The reference cannot be compiled
  * in this environment (its sources need a CMake-generated dnnl_config.h), so
  * no oracle/_ref build exists; see the pinning list in the tests' docstrings.
+ * The dynamic (MX) dst quantization (orc_finish_dynamic_group) is pinned by
+ * tests/test_dynamic_dst.py: its scale is a pure function of the group's
+ * largest magnitude through exponent bytes, restated there with numpy integer
+ * arithmetic on the f32 bit patterns and checked on constructed groups
+ * (powers of two, just below / above one, zeros, values beyond the dst range).
  * Unpinned: none of the functions used by the five benchmark configurations;
  * the libm-dependent eltwise algorithms other than relu/gelu_tanh/linear/tanh
  * are "parity unpinned" beyond their textbook formula.
@@ -400,7 +405,8 @@ static float orc_fp_dot(const mi355_matmul_desc_t *d,
 }
 
 /* ------------------------------------------------------------- epilogue */
-static void orc_finish(const mi355_matmul_desc_t *d,
+/* bias and post-ops: the value the dst quantization (static or dynamic) sees */
+static float orc_pre_quant(const mi355_matmul_desc_t *d,
         const mi355_matmul_args_t *a, float v, int64_t b, int64_t m,
         int64_t n) {
     const int64_t doff
@@ -419,6 +425,15 @@ static void orc_finish(const mi355_matmul_desc_t *d,
             }
         v = orc_post_ops(d, a, v, dst_old, b, m, n);
     }
+    return v;
+}
+
+static void orc_finish(const mi355_matmul_desc_t *d,
+        const mi355_matmul_args_t *a, float v, int64_t b, int64_t m,
+        int64_t n) {
+    const int64_t doff
+            = b * d->dst_stride[0] + m * d->dst_stride[1] + n * d->dst_stride[2];
+    v = orc_pre_quant(d, a, v, b, m, n);
     if (d->dst_scale.dt != MI355_DT_UNDEF) {
         float s = orc_load_float(d->dst_scale.dt, a->dst_scale, 0);
         if (d->dst_scale_mode == MI355_DST_SCALE_RECIPROCAL) {
@@ -433,6 +448,44 @@ static void orc_finish(const mi355_matmul_desc_t *d,
         v += (float)z;
     }
     orc_store_float(d->dst_dt, v, a->dst, doff);
+}
+
+/* types::round_to_dt(e8m0, x): through the e8m0 type and back
+ * (src/common/type_helpers.hpp:328-350, float8.cpp:29-45) */
+static float orc_round_e8m0(float x) {
+    return orc_e8m0_to_f32(orc_f32_to_e8m0(x));
+}
+
+/* types::max_value<float>(dst type) (type_helpers.hpp:204-221) */
+static float orc_dt_max(int dt) {
+    switch (dt) {
+        case MI355_DT_F8_E4M3: return 448.f;
+        case MI355_DT_F8_E5M2: return 57344.f;
+        case MI355_DT_F4_E2M1: return 6.f;
+        default: return 0.f;
+    }
+}
+
+/* One group of dynamic (MX) dst quantization, ref_matmul.cpp:268-423: the
+ * values `v[0..g)` of columns n0.. of row (b, m), after bias and post-ops. */
+static void orc_finish_dynamic_group(const mi355_matmul_desc_t *d,
+        const mi355_matmul_args_t *a, const float *v, int g, int64_t b,
+        int64_t m, int64_t n0) {
+    float max_dst_group = 0.f;
+    for (int e = 0; e < g; ++e) max_dst_group = fmaxf(max_dst_group, fabsf(v[e]));
+    const float dst_max = orc_dt_max(d->dst_dt);
+    /* :343-351, the rounding to a power of two happens before the division */
+    float scale = orc_round_e8m0(max_dst_group) / orc_round_e8m0(dst_max);
+    scale = orc_round_e8m0(scale);
+    const int64_t soff = orc_quant_off(&d->dst_scale, b, m, n0, d->M, d->N);
+    orc_store_float(d->dst_scale.dt, scale, (void *)a->dst_scale, soff); /* :377-378 */
+    const float inv = 1.f / scale; /* :381 */
+    for (int e = 0; e < g; ++e) {
+        float x = v[e] * inv;
+        x = fminf(fmaxf(x, -dst_max), dst_max); /* :405-407 */
+        orc_store_float(d->dst_dt, x, a->dst,
+                b * d->dst_stride[0] + m * d->dst_stride[1] + (n0 + e) * d->dst_stride[2]);
+    }
 }
 
 static int orc_src_is_int(int dt) {
@@ -453,6 +506,30 @@ int oracle_matmul(const mi355_matmul_desc_t *d, const mi355_matmul_args_t *a,
     if (d->batch == 0 || d->M == 0 || d->N == 0 || d->K == 0) return MI355_SUCCESS;
     const int int_path = orc_src_is_int(d->src_dt);
     const int64_t B = d->batch, M = d->M, N = d->N;
+    if (d->dst_scale_dynamic == MI355_DST_DYNAMIC_MX) {
+        const int g = (int)d->dst_scale.group[1];
+        if (g < 1 || g > 64 || N % g) return MI355_INVALID_ARGUMENTS;
+#pragma omp parallel for collapse(2) schedule(static)
+        for (int64_t b = 0; b < B; ++b)
+            for (int64_t m = 0; m < M; ++m)
+                for (int64_t n0 = 0; n0 < N; n0 += g) {
+                    float v[64];
+                    for (int e = 0; e < g; ++e) {
+                        const int64_t n = n0 + e;
+                        float x;
+                        if (int_path) {
+                            x = orc_int8_dot(d, a, b, m, n, NULL);
+                        } else {
+                            int64_t i = (b * M + m) * N + n;
+                            x = orc_fp_dot(d, a, b, m, n, flags, ideal ? ideal + i : NULL,
+                                    abs_sum ? abs_sum + i : NULL);
+                        }
+                        v[e] = orc_pre_quant(d, a, x, b, m, n);
+                    }
+                    orc_finish_dynamic_group(d, a, v, g, b, m, n0);
+                }
+        return MI355_SUCCESS;
+    }
     /* 4-bit dst: two n share a byte, so a thread owns whole rows */
 #pragma omp parallel for collapse(2) schedule(static)
     for (int64_t b = 0; b < B; ++b)

@@ -29,7 +29,7 @@ def test_struct_layout_matches_header_sizes():
     # sizes implied by the header's field lists (LP64): catches a drifting mirror
     assert C.sizeof(cabi.Quant) == 24
     assert C.sizeof(cabi.PostOp) == 56
-    assert C.sizeof(cabi.MatmulDesc) == 32 + 16 + 4 * 24 + 7 * 24 + 16 + 32 * 56 + 8
+    assert C.sizeof(cabi.MatmulDesc) == 32 + 16 + 4 * 24 + 7 * 24 + 16 + 32 * 56 + 16
     assert C.sizeof(cabi.MatmulArgs) == 8 * (11 + 32)
 
 

@@ -1,0 +1,170 @@
+"""Dynamic (MX) quantization of dst: `quantization_mode::dynamic_mx` scales on
+DNNL_ARG_DST are an output of the matmul (ref_matmul.cpp:268-423, rules
+src/common/matmul.cpp:407-424).
+
+What pins the oracle without running the reference: the group scale is a pure
+function of the group's largest magnitude through exponent bytes
+(float8.cpp:29-45: e8m0(x) keeps the exponent byte of x), so
+  * constructed groups have known answers (amax 448 -> scale 1; amax 1 ->
+    2^-8; amax just below 2 -> the scale of 1, and its largest values then
+    saturate at the dst maximum; an all-zero group -> scale byte 0, zeros),
+  * random problems are restated with numpy integer arithmetic on the f32 bit
+    patterns of the pre-quantization values, which come from the oracle's own
+    static path with an f32 dst (pinned elsewhere).
+GPU: the generic kernel follows the same operations in the same order and
+must reproduce dst and scales bit for bit.
+"""
+import numpy as np
+import pytest
+
+from onednn_amd import cabi, configs
+from onednn_amd import dtypes as dtp
+from onednn_amd.problem import GpuRun, MatmulProblem, PostOp, QuantParam
+from oracle import binding as orc
+
+DT_MAX = {cabi.DT_F8_E4M3: 448.0, cabi.DT_F8_E5M2: 57344.0}
+
+
+def f32_problem(d, dst_dt):
+    """dst = I x d: every pre-quantization value is exactly d[m, n]."""
+    M, N = d.shape
+    p = MatmulProblem(M=M, N=N, K=M, src_dt=cabi.DT_F32, wei_dt=cabi.DT_F32, dst_dt=dst_dt,
+                      src=np.eye(M, dtype=np.float32), wei=np.ascontiguousarray(d, dtype=np.float32), name="dyn-f32")
+    return dynamic(p)
+
+
+def dynamic(p):
+    p.quant["dst_scale"] = QuantParam(cabi.DT_E8M0, configs.MASK_ROW | configs.MASK_COL,
+                                      np.zeros((p.batch, p.M, p.N // 32), np.uint8), (1, 32))
+    p.dst_dynamic = cabi.DST_DYNAMIC_MX
+    return p
+
+
+def exponent_byte(x):
+    return ((np.asarray(x, np.float32).view(np.uint32) >> 23) & 0xff).astype(np.uint8)
+
+
+def from_exponent_byte(b):
+    b = np.asarray(b, np.uint32)
+    bits = np.where(b == 0, np.uint32(0x00400000), b << 23).astype(np.uint32)
+    return bits.view(np.float32)
+
+
+def numpy_dynamic(d, dst_dt):
+    """The reference's steps on pre-quantization values d [rows, N]."""
+    rows, N = d.shape
+    g = d.reshape(rows, N // 32, 32)
+    amax = np.abs(g).max(axis=2)
+    dmax = np.float32(DT_MAX[dst_dt])
+    ratio = from_exponent_byte(exponent_byte(amax)) / from_exponent_byte(exponent_byte(dmax))
+    sbyte = exponent_byte(ratio.astype(np.float32))
+    inv = np.float32(1.0) / from_exponent_byte(sbyte)
+    x = np.clip(g * inv[:, :, None], -dmax, dmax).astype(np.float32).reshape(rows, N)
+    to = dtp.f32_to_e4m3 if dst_dt == cabi.DT_F8_E4M3 else orc.f32_to_e5m2
+    return to(x.reshape(-1)).reshape(rows, N), sbyte
+
+
+# ------------------------------------------------------------------ CPU
+def test_known_answers_of_the_group_scale():
+    d = np.zeros((4, 64), np.float32)
+    d[0, :32] = np.linspace(-448, 448, 32)            # amax 448 -> 256 / 256 = 1
+    d[0, 32:] = 1.0                                   # amax 1 -> 1 / 256
+    d[1, :32] = np.float32(1.9999999)                 # e8m0 rounds down to 1: x * 256 = 511.99 saturates at 448
+    d[1, 0] = 0.5
+    d[1, 32:] = 0.0                                   # all-zero group
+    d[2, :32] = 3e-39                                 # subnormal amax: exponent byte 0 -> 2^-127 / 2^8 underflows to byte 0
+    d[2, 32:] = 1e30                                  # 2^99 / 2^8 = 2^91
+    d[3, :] = -np.arange(64, dtype=np.float32)
+    p = f32_problem(d, cabi.DT_F8_E4M3)
+    dst, sc = orc.run_oracle_dynamic(p)
+    sc = sc.reshape(4, 2)
+    val = dtp.e4m3_to_f32(dst).reshape(4, 64)
+    assert sc[0, 0] == 127 and np.array_equal(val[0, :32], dtp.e4m3_to_f32(dtp.f32_to_e4m3(d[0, :32])))
+    assert sc[0, 1] == 127 - 8 and np.all(val[0, 32:] == 256.0)
+    assert sc[1, 0] == 127 - 8 and np.all(val[1, 1:32] == 448.0) and val[1, 0] == 128.0
+    assert sc[1, 1] == 0 and np.all(val[1, 32:] == 0.0)
+    assert sc[2, 0] == 0
+    assert sc[2, 1] == 127 + 99 - 8
+    # -63 .. -32: amax 63 -> 32 / 256 = 2^-3; -31 .. 0: 16 / 256 = 2^-4
+    assert sc[3, 1] == 127 - 3 and sc[3, 0] == 127 - 4
+    # 2^3 * 63 = 504 lies beyond the e4m3 range: saturated, not NaN
+    assert np.array_equal(val[3, 32:], dtp.e4m3_to_f32(dtp.f32_to_e4m3(np.clip(d[3, 32:] * 8, -448, 448))))
+
+
+@pytest.mark.parametrize("dst", ["f8_e4m3", "f8_e5m2"])
+def test_oracle_follows_the_numpy_restatement(dst):
+    dst_dt = cabi.DT_F8_E4M3 if dst == "f8_e4m3" else cabi.DT_F8_E5M2
+    p = configs.config4(M=48, N=128, K=64)
+    p.post_ops = [PostOp(kind=cabi.PO_ELTWISE, alg=cabi.ELTWISE["relu"], alpha=0.25, scale=3.0), p.post_ops[1]]
+    # pre-quantization values: the static path with an f32 dst
+    p.dst_dt = cabi.DT_F32
+    pre = np.asarray(orc.run_oracle(p)).view(np.float32).reshape(p.M, p.N)
+    p.dst_dt = dst_dt
+    got, sc = orc.run_oracle_dynamic(dynamic(p))
+    want, want_sc = numpy_dynamic(pre, dst_dt)
+    assert np.array_equal(sc.reshape(p.M, p.N // 32), want_sc)
+    assert np.array_equal(np.asarray(got).view(np.uint8).reshape(p.M, p.N), want)
+
+
+def test_rules_of_the_descriptor():
+    p = dynamic(configs.config4(M=32, N=64, K=64))
+    p.dst_dt = cabi.DT_F8_E4M3
+    st, impl = cabi.query(p.desc())
+    assert st == cabi.SUCCESS and cabi.impl_name(impl) == "hip:ref:any"      # the generic kernel only
+    assert cabi.query(p.desc(), cabi.IMPL_F8_MFMA)[0] == cabi.UNIMPLEMENTED
+    for change in ("dt", "group", "mask", "dst", "n"):
+        q = dynamic(configs.config4(M=32, N=64 if change != "n" else 80, K=64))
+        q.dst_dt = cabi.DT_F8_E4M3 if change != "dst" else cabi.DT_BF16
+        s = q.quant["dst_scale"]
+        if change == "dt":
+            s.dt = cabi.DT_F32
+        if change == "group":
+            s.groups = (1, 16)
+        if change == "mask":
+            s.mask = configs.MASK_COL
+        assert cabi.query(q.desc())[0] == cabi.INVALID_ARGUMENTS, change
+    # integer src: the reference's integer implementation has no dynamic quantization
+    c = dynamic(configs.config1(M=32, N=64, K=64))
+    c.dst_dt = cabi.DT_F8_E4M3
+    assert cabi.query(c.desc())[0] == cabi.UNIMPLEMENTED
+
+
+# ------------------------------------------------------------------ GPU
+def run_gpu_dynamic(p):
+    run = GpuRun(p)
+    try:
+        run.launch()
+        return run.result(), run.dynamic_scales(), cabi.impl_name(run.impl)
+    finally:
+        run.free()
+
+
+@pytest.mark.gpu
+def test_gpu_known_answer_groups(gpu, oracle):
+    r = np.random.default_rng(3)
+    d = (r.standard_normal((16, 128)) * np.exp2(r.integers(-140, 120, size=(16, 4)).repeat(32, axis=1))).astype(np.float32)
+    d[0, :32] = 0.0
+    d[1, :32] = np.float32(1.9999999)
+    for dst_dt in (cabi.DT_F8_E4M3, cabi.DT_F8_E5M2):
+        p = f32_problem(d, dst_dt)
+        got, sc, name = run_gpu_dynamic(p)
+        want, want_sc = orc.run_oracle_dynamic(p)
+        assert name == "hip:ref:any"
+        assert np.array_equal(np.asarray(sc).reshape(-1), np.asarray(want_sc).reshape(-1))
+        assert np.array_equal(np.asarray(got).view(np.uint8), np.asarray(want).view(np.uint8))
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dst", ["f8_e4m3", "f8_e5m2"])
+def test_gpu_fp8_matmul_with_dynamic_dst_is_bit_exact(gpu, oracle, dst):
+    # bias, leaky relu and a residual add before the quantization: no libm
+    # function involved, so the generic kernel must match the oracle bit for bit
+    p = configs.config4(M=80, N=192, K=128)
+    p.post_ops = [PostOp(kind=cabi.PO_ELTWISE, alg=cabi.ELTWISE["relu"], alpha=0.25, scale=3.0), p.post_ops[1]]
+    p.dst_dt = cabi.DT_F8_E4M3 if dst == "f8_e4m3" else cabi.DT_F8_E5M2
+    p = dynamic(p)
+    got, sc, name = run_gpu_dynamic(p)
+    want, want_sc = orc.run_oracle_dynamic(p)
+    assert name == "hip:ref:any"
+    assert np.array_equal(np.asarray(sc).reshape(-1), np.asarray(want_sc).reshape(-1))
+    assert np.array_equal(np.asarray(got).view(np.uint8), np.asarray(want).view(np.uint8))
