@@ -69,6 +69,14 @@ typedef enum {
     dnnl_fpmath_mode_tf32
 } dnnl_fpmath_mode_t;
 
+/* dnnl_types.h:2470-2486 */
+typedef enum {
+    dnnl_quantization_mode_undef = 0,
+    dnnl_quantization_mode_static_sazp,
+    dnnl_quantization_mode_dynamic_mx,
+    dnnl_quantization_mode_dynamic_fp
+} dnnl_quantization_mode_t;
+
 /* dnnl_common_types.h:157-170 */
 typedef enum {
     dnnl_accumulation_mode_strict = 0,
@@ -269,6 +277,13 @@ dnnl_status_t dnnl_primitive_attr_set_scratchpad_mode(dnnl_primitive_attr_t attr
 dnnl_status_t dnnl_primitive_attr_get_scratchpad_mode(const_dnnl_primitive_attr_t attr,
         dnnl_scratchpad_mode_t *mode);
 dnnl_status_t dnnl_primitive_attr_set_scales_mask(dnnl_primitive_attr_t attr, int arg, int mask);
+/* dnnl.h:520-553.  With dnnl_quantization_mode_dynamic_mx on DNNL_ARG_DST the
+ * scales memory passed at execution is an output (dnnl.h:546-547); host-side
+ * scalars (is_on_host) and dnnl_quantization_mode_dynamic_fp are not offered. */
+dnnl_status_t dnnl_primitive_attr_set_scales_v2(dnnl_primitive_attr_t attr, int arg, int mask, int group_ndims,
+        const dnnl_dims_t group_dims, dnnl_data_type_t data_type, int is_on_host);
+dnnl_status_t dnnl_primitive_attr_set_scales_v3(dnnl_primitive_attr_t attr, int arg, int mask, int group_ndims,
+        const dnnl_dims_t group_dims, dnnl_data_type_t data_type, int is_on_host, dnnl_quantization_mode_t qmode);
 dnnl_status_t dnnl_primitive_attr_set_scales(dnnl_primitive_attr_t attr, int arg, int mask, int group_ndims,
         const dnnl_dims_t group_dims, dnnl_data_type_t data_type);
 dnnl_status_t dnnl_primitive_attr_set_zero_points_mask(dnnl_primitive_attr_t attr, int arg, int mask);

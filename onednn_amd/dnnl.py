@@ -26,6 +26,7 @@ kind_sum, kind_eltwise, kind_binary, kind_matmul, kind_prelu = 4, 7, 13, 14, 18
 query_impl_info_str, query_src_md, query_weights_md, query_dst_md, query_scratchpad_md = 8, 129, 131, 133, 136
 query_ndims_s32, query_dims, query_data_type, query_strides, query_memory_consumption = 256, 257, 258, 14, 6
 query_format_kind = 262
+quantization_mode_undef, quantization_mode_static_sazp, quantization_mode_dynamic_mx, quantization_mode_dynamic_fp = 0, 1, 2, 3
 format_kind_undef, format_kind_any, format_kind_blocked, format_kind_opaque = 0, 1, 2, 3
 ARG_SRC, ARG_SRC_1, ARG_DST, ARG_WEIGHTS, ARG_BIAS, ARG_SCRATCHPAD = 1, 2, 17, 33, 41, 80
 ARG_FROM, ARG_TO = ARG_SRC, ARG_DST
@@ -202,8 +203,13 @@ class primitive_attr:
     def set_scales_mask(self, arg, mask):
         _check(lib().dnnl_primitive_attr_set_scales_mask(self.h, arg, mask), "set_scales_mask")
 
-    def set_scales(self, arg, mask, groups=(), dt=cabi.DT_F32):
-        _check(lib().dnnl_primitive_attr_set_scales(self.h, arg, mask, len(groups), _dims(groups), dt), "set_scales")
+    def set_scales(self, arg, mask, groups=(), dt=cabi.DT_F32, qmode=None, is_on_host=0):
+        if qmode is None and not is_on_host:
+            _check(lib().dnnl_primitive_attr_set_scales(self.h, arg, mask, len(groups), _dims(groups), dt), "set_scales")
+        else:
+            _check(lib().dnnl_primitive_attr_set_scales_v3(
+                self.h, arg, mask, len(groups), _dims(groups), dt, is_on_host,
+                quantization_mode_static_sazp if qmode is None else qmode), "set_scales_v3")
 
     def set_zero_points_mask(self, arg, mask):
         _check(lib().dnnl_primitive_attr_set_zero_points_mask(self.h, arg, mask), "set_zero_points_mask")

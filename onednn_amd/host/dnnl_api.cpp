@@ -154,6 +154,8 @@ struct quant_entry_t {
     int group_ndims = 0;
     dim_t groups[2] = {1, 1};
     dim_t group(int d) const { return group_ndims == 0 ? 1 : groups[d]; }
+    dnnl_quantization_mode_t qmode = dnnl_quantization_mode_static_sazp;
+    bool is_mx() const { return qmode == dnnl_quantization_mode_dynamic_mx; }
 };
 
 struct post_op_entry_t {
@@ -311,7 +313,16 @@ dnnl_status_t check_attr(const dnnl_memory_desc &s, const dnnl_memory_desc &w, c
         CHECK_UNIMPL(q->mask == 0 || q->mask == qN || q->mask == qM || q->mask == qM + qN || q->mask == full);
         CHECK_UNIMPL(IMPLICATION(q->group_ndims, is_fp8(dst_dt) || dst_dt == dnnl_f4_e2m1));
         CHECK_UNIMPL(IMPLICATION(q->group_ndims, M % q->group(0) == 0 && N % q->group(1) == 0));
+        // dynamic_mx: OCP MX flavour only (matmul.cpp:407-424)
+        if (q->is_mx()) {
+            CHECK_UNIMPL(q->mask == full);
+            CHECK_UNIMPL(q->group_ndims == 2 && q->group(1) == 32 && q->group(0) == 1);
+            CHECK_UNIMPL(q->dt == dnnl_e8m0);
+        }
     }
+    // dynamic quantization is a dst scale mode
+    for (int arg : {DNNL_ARG_SRC, DNNL_ARG_WEIGHTS})
+        if (auto q = a.find(a.scales, arg)) CHECK_UNIMPL(!q->is_mx());
     CHECK_UNIMPL(IMPLICATION(src_sg_k > 1, (src_int8 || src_fp8 || src_fp4) && divisible(src_sg_k, wei_sg_k)));
 
     dim_t src_zg_k = 1, wei_zg_k = 1;
@@ -467,8 +478,16 @@ dnnl_status_t lower(dnnl_primitive_desc &pd) {
     CHECK_UNIMPL(lower_quant(a.find(a.zero_points, DNNL_ARG_WEIGHTS), nd, dnnl_s32, &D.wei_zp));
     CHECK_UNIMPL(lower_quant(a.find(a.zero_points, DNNL_ARG_DST), nd, dnnl_s32, &D.dst_zp));
     CHECK_UNIMPL(lower_quant(a.find(a.reductions, DNNL_ARG_SRC), nd, dnnl_s32, &D.src_pr));
-    // dynamic (grouped) dst scales are not offered; dst scale is one value
-    CHECK_UNIMPL(D.dst_scale.dt == MI355_DT_UNDEF || D.dst_scale.mask == 0);
+    // a static dst scale is one value; a grouped one is the dynamic (MX) mode
+    {
+        const quant_entry_t *dq = a.find(a.scales, DNNL_ARG_DST);
+        if (dq && dq->is_mx()) {
+            D.dst_scale_dynamic = MI355_DST_DYNAMIC_MX;
+            CHECK_UNIMPL(is_fp8(pd.dst.dt) && D.dst_zp.dt == MI355_DT_UNDEF && D.N % 32 == 0);
+        } else {
+            CHECK_UNIMPL(D.dst_scale.dt == MI355_DT_UNDEF || D.dst_scale.mask == 0);
+        }
+    }
     CHECK_UNIMPL(D.dst_zp.dt == MI355_DT_UNDEF || D.dst_zp.dt == MI355_DT_S32);
     D.fpmath_apply_to_int = a.apply_to_int;
     D.fpmath_mode = a.fpmath;
@@ -859,6 +878,24 @@ DNNL_EXPORT dnnl_status_t dnnl_primitive_attr_set_scales(dnnl_primitive_attr_t a
             || data_type == dnnl_f8_e4m3);
     CHECK_ARG(IMPLICATION(data_type == dnnl_e8m0 || data_type == dnnl_f8_e4m3, mask > 0));
     return set_quant(attr->scales, arg, mask, group_ndims, group_dims, data_type);
+}
+DNNL_EXPORT dnnl_status_t dnnl_primitive_attr_set_scales_v3(dnnl_primitive_attr_t attr, int arg, int mask,
+        int group_ndims, const dnnl_dims_t group_dims, dnnl_data_type_t data_type, int is_on_host,
+        dnnl_quantization_mode_t qmode) {
+    CHECK_ARG(attr);
+    CHECK_ARG(qmode == dnnl_quantization_mode_static_sazp || qmode == dnnl_quantization_mode_dynamic_mx
+            || qmode == dnnl_quantization_mode_dynamic_fp);
+    CHECK_ARG(IMPLICATION(is_on_host, mask == 0 && group_ndims == 0));
+    CHECK_UNIMPL(!is_on_host);
+    CHECK_UNIMPL(qmode != dnnl_quantization_mode_dynamic_fp);
+    const dnnl_status_t st = dnnl_primitive_attr_set_scales(attr, arg, mask, group_ndims, group_dims, data_type);
+    if (st == dnnl_success) attr->scales[arg].qmode = qmode;
+    return st;
+}
+DNNL_EXPORT dnnl_status_t dnnl_primitive_attr_set_scales_v2(dnnl_primitive_attr_t attr, int arg, int mask,
+        int group_ndims, const dnnl_dims_t group_dims, dnnl_data_type_t data_type, int is_on_host) {
+    return dnnl_primitive_attr_set_scales_v3(
+            attr, arg, mask, group_ndims, group_dims, data_type, is_on_host, dnnl_quantization_mode_static_sazp);
 }
 DNNL_EXPORT dnnl_status_t dnnl_primitive_attr_set_scales_mask(dnnl_primitive_attr_t attr, int arg, int mask) {
     return dnnl_primitive_attr_set_scales(attr, arg, mask, 0, nullptr, dnnl_f32);

@@ -244,6 +244,26 @@ def test_format_any_decode_weights_resolve_to_the_packed_layout(eng):
     assert make_pd(eng, 8, K, N, "bf16", "u4", "bf16", attr=wo).impl_info_str().startswith("hip:woq_gemv")
 
 
+def test_dynamic_mx_dst_scales_rules(eng):
+    # dnnl_primitive_attr_set_scales_v3 (primitive_attr.cpp:637-669) and the matmul rules for
+    # quantization_mode::dynamic_mx (matmul.cpp:407-424): full mask, groups 1 x 32, e8m0
+    def mx(mask=3, groups=(1, 32), dt=DT["e8m0"], arg=dnnl.ARG_DST):
+        return _attr(lambda t: t.set_scales(arg, mask, groups, dt, qmode=dnnl.quantization_mode_dynamic_mx))
+    pd = make_pd(eng, 64, 128, 256, "f8_e4m3", "f8_e4m3", "f8_e4m3", attr=mx())
+    assert pd.impl_info_str() == "hip:ref:any"
+    assert status_of(lambda: make_pd(eng, 64, 128, 256, "f8_e4m3", "f8_e4m3", "f8_e5m2", attr=mx())) == dnnl.success
+    assert status_of(lambda: make_pd(eng, 64, 128, 256, "f8_e4m3", "f8_e4m3", "f8_e4m3", attr=mx(groups=(1, 16)))) == dnnl.unimplemented
+    assert status_of(lambda: make_pd(eng, 64, 128, 256, "f8_e4m3", "f8_e4m3", "f8_e4m3", attr=mx(mask=2))) == dnnl.unimplemented
+    assert status_of(lambda: make_pd(eng, 64, 128, 256, "f8_e4m3", "f8_e4m3", "f8_e4m3", attr=mx(dt=DT["f32"]))) == dnnl.unimplemented
+    assert status_of(lambda: make_pd(eng, 64, 128, 256, "f8_e4m3", "f8_e4m3", "bf16", attr=mx())) == dnnl.unimplemented
+    assert status_of(lambda: make_pd(eng, 64, 128, 256, "f8_e4m3", "f8_e4m3", "f8_e4m3", attr=mx(arg=dnnl.ARG_SRC, groups=(1, 32)))) == dnnl.unimplemented
+    a = dnnl.primitive_attr()
+    assert status_of(lambda: a.set_scales(dnnl.ARG_DST, 3, (1, 32), DT["e8m0"], qmode=7)) == dnnl.invalid_arguments
+    assert status_of(lambda: a.set_scales(dnnl.ARG_DST, 3, (1, 16), DT["f8_e4m3"], qmode=dnnl.quantization_mode_dynamic_fp)) == dnnl.unimplemented
+    assert status_of(lambda: a.set_scales(dnnl.ARG_DST, 1, (), DT["f32"], is_on_host=1)) == dnnl.invalid_arguments
+    assert status_of(lambda: a.set_scales(dnnl.ARG_DST, 0, (), DT["f32"], is_on_host=1)) == dnnl.unimplemented
+
+
 def test_user_scratchpad_is_reported(eng):
     a = dnnl.primitive_attr()
     a.set_scratchpad_mode(dnnl.scratchpad_user)

@@ -218,3 +218,45 @@ def test_prepack_decode_weights_with_reorder_then_matmul(gpu, oracle):
     assert np.array_equal(wei_mem.read(np.uint8), pack_woq64(p.wei, K, N))
     want, _, asum = oracle.run_oracle(p, want_ideal=True)
     assert_close(p, dst.read(np.uint16), want, abs_sum=asum * 20.0, what=pd.impl_info_str())
+
+
+def test_dynamic_mx_dst_through_the_api(gpu, oracle):
+    """quantization_mode::dynamic_mx on DNNL_ARG_DST: the scales memory is an
+    output of execute (ref_matmul.cpp:338-423)."""
+    from onednn_amd.problem import PostOp, QuantParam
+    from oracle import binding as orc
+    p = configs.config4(M=64, N=256, K=128)
+    p.post_ops = [PostOp(kind=cabi.PO_ELTWISE, alg=cabi.ELTWISE["relu"], alpha=0.0, scale=1.0)]
+    p.dst_dt = cabi.DT_F8_E4M3
+    p.quant["dst_scale"] = QuantParam(cabi.DT_E8M0, 6, np.zeros((1, p.M, p.N // 32), np.uint8), (1, 32))
+    p.dst_dynamic = cabi.DST_DYNAMIC_MX
+    M, K, N = p.M, p.K, p.N
+    eng = dnnl.engine(dnnl.gpu, 0)
+    strm = dnnl.stream(eng)
+    src_md = dnnl.memory_desc([M, K], DT["f8_e4m3"], tag=dnnl.tag_ab)
+    wei_md = dnnl.memory_desc([K, N], DT["f8_e4m3"], tag=dnnl.tag_ab)
+    dst_md = dnnl.memory_desc([M, N], DT["f8_e4m3"], tag=dnnl.tag_ab)
+    bias_md = dnnl.memory_desc([1, N], DT["bf16"], tag=dnnl.tag_ab)
+    attr = dnnl.primitive_attr()
+    attr.set_scales_mask(dnnl.ARG_SRC, 0)
+    attr.set_scales_mask(dnnl.ARG_WEIGHTS, 0)
+    attr.set_scales(dnnl.ARG_DST, 3, (1, 32), DT["e8m0"], qmode=dnnl.quantization_mode_dynamic_mx)
+    po = dnnl.post_ops()
+    po.append_eltwise(cabi.ELTWISE["relu"], 0.0, 0.0)
+    attr.set_post_ops(po)
+    pd = dnnl.matmul_primitive_desc(eng, src_md, wei_md, dst_md, bias_md=bias_md, attr=attr)
+    assert pd.impl_info_str() == "hip:ref:any"
+    one = dnnl.memory_desc([1], DT["f32"], tag=dnnl.tag_a)
+    sc_md = dnnl.memory_desc([M, N // 32], DT["e8m0"], tag=dnnl.tag_ab)
+    sc_mem = dnnl.memory(sc_md, eng)
+    dst = dnnl.memory(dst_md, eng)
+    dnnl.matmul(pd).execute(strm, {
+        dnnl.ARG_SRC: dnnl.memory(src_md, eng, p.src), dnnl.ARG_WEIGHTS: dnnl.memory(wei_md, eng, p.wei),
+        dnnl.ARG_BIAS: dnnl.memory(bias_md, eng, p.bias), dnnl.ARG_DST: dst,
+        dnnl.ARG_ATTR_SCALES | dnnl.ARG_SRC: dnnl.memory(one, eng, p.quant["src_scale"].data),
+        dnnl.ARG_ATTR_SCALES | dnnl.ARG_WEIGHTS: dnnl.memory(one, eng, p.quant["wei_scale"].data),
+        dnnl.ARG_ATTR_SCALES | dnnl.ARG_DST: sc_mem})
+    strm.wait()
+    want, want_sc = orc.run_oracle_dynamic(p)
+    assert np.array_equal(sc_mem.read(np.uint8).reshape(-1), np.asarray(want_sc).reshape(-1))
+    assert np.array_equal(dst.read(np.uint8).reshape(-1), np.asarray(want).view(np.uint8).reshape(-1))
