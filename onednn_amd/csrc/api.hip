@@ -107,8 +107,10 @@ static int validate(const mi355_matmul_desc_t *d) {
 typedef int (*supported_fn)(const mi355_matmul_desc_t &);
 
 static int impl_supported(const mi355_matmul_desc_t &d, int impl) {
-    // dynamic dst quantization: the generic kernel only
-    if (d.dst_scale_dynamic != MI355_DST_DYNAMIC_NONE && impl != MI355_IMPL_REF) return MI355_UNIMPLEMENTED;
+    // dynamic dst quantization: the generic kernel and the floating-point GEMM tiles
+    if (d.dst_scale_dynamic != MI355_DST_DYNAMIC_NONE && impl != MI355_IMPL_REF && impl != MI355_IMPL_F8_MFMA
+            && impl != MI355_IMPL_MXF4_MFMA)
+        return MI355_UNIMPLEMENTED;
     switch (impl) {
         case MI355_IMPL_REF: return ref_supported(d);
         case MI355_IMPL_I8_MFMA: return i8_supported(d);

@@ -71,6 +71,7 @@ struct epi_hoist_t {
     int n_po;
     int dst_dt, dst_vec; // dst_vec: four consecutive n leave as one aligned store
     int batchable;       // every operand is hoisted or staged and every post-op is a register-resident one
+    int dynamic;         // MI355_DST_DYNAMIC_*: the dst scale is an output, computed per 32 columns of a row
 };
 
 __device__ __forceinline__ bool vec_ok(const void *p, long s0, long s1, int bits) {
@@ -105,7 +106,8 @@ __device__ __forceinline__ epi_hoist_t make_hoist(const PT &P, long b, long nbas
             H.bias_mode = 2;
         }
     }
-    if (P.dst_scale.dt != MI355_DT_UNDEF) {
+    H.dynamic = P.dst_dynamic;
+    if (P.dst_scale.dt != MI355_DT_UNDEF && !P.dst_dynamic) {
         H.ds = load_float(P.dst_scale.dt, P.dst_scale.p, 0);
         H.ds_inv = 1.f / H.ds;
         H.ds_mode = P.dst_scale_mode == MI355_DST_SCALE_RECIPROCAL ? 2 : 1;
@@ -176,7 +178,7 @@ __device__ __forceinline__ epi_hoist_t make_hoist(const PT &P, long b, long nbas
     }
     // The batched epilogue (several row quads per dispatch) needs every operand in
     // registers or in the staging area: no loads inside the loop.
-    H.batchable = H.n_po == H.nfast && (H.bias_mode != 2 || H.staged == STG_BIAS) && nvalid == 4 && H.dst_vec;
+    H.batchable = !H.dynamic && H.n_po == H.nfast && (H.bias_mode != 2 || H.staged == STG_BIAS) && nvalid == 4 && H.dst_vec;
     {
         auto operand_ready = [&](const po_reg_t &r, int i) {
             if (r.kind == MI355_PO_BINARY)
@@ -793,6 +795,45 @@ __device__ __forceinline__ void store_quadrant(const PT &P, char *smem, const Ac
                 for (int k = 0; k < NQ; ++k) conv.row(raw[k], ok[k] ? m[k] : m_base, v[k]);
                 apply_epilogueQ<NQ>(H, v, sv);
                 storeQ<NQ>(P, H, v, b, m, nbase, ok);
+            }
+            continue;
+        }
+        if (H.dynamic) {
+            // Dynamic (MX) quantization of dst, ref_matmul.cpp:338-423: a group is
+            // 32 consecutive n of one row = 8 consecutive lanes of this layout
+            // (four n each; a wavefront's columns start at a multiple of 64 and
+            // N % 32 == 0, so a group is whole or absent).  All lanes run the
+            // arithmetic and the cross-lane maximum, rows beyond M on the data of
+            // a valid row; only the stores are masked.
+            const float dt_max = H.dst_dt == MI355_DT_F8_E4M3 ? 448.f : 57344.f;
+            const float emax = e8m0_to_f32(f32_to_e8m0(dt_max));
+#pragma unroll 1
+            for (int it = 0; it < PASSES; ++it) {
+                const int row = it * RPP + lrow;
+                const long m = m_base + i * 32 + row;
+                const bool ok = m < P.M && nvalid > 0;
+                const long mv = m < P.M ? m : P.M - 1;
+                const v4i_t raw = *(const slab_v4i_t *)&wl[row * WCOLS + lcol * 4];
+                uint4 sv = make_uint4(0, 0, 0, 0);
+                if (H.staged != STG_NONE) sv = stg[it * 64 + lane];
+                float v[4] = {0.f, 0.f, 0.f, 0.f};
+                if (nvalid > 0) {
+                    conv.row(raw, mv, v);
+                    apply_epilogue4(P, H, v, b, mv, nbase, nvalid, sv);
+                }
+                float amax = fmaxf(fmaxf(fabsf(v[0]), fabsf(v[1])), fmaxf(fabsf(v[2]), fabsf(v[3])));
+                amax = fmaxf(amax, __shfl_xor(amax, 1, 64));
+                amax = fmaxf(amax, __shfl_xor(amax, 2, 64));
+                amax = fmaxf(amax, __shfl_xor(amax, 4, 64));
+                const uint8_t sbyte = f32_to_e8m0(e8m0_to_f32(f32_to_e8m0(amax)) / emax);
+                const float inv = 1.f / e8m0_to_f32(sbyte);
+#pragma unroll
+                for (int e = 0; e < 4; ++e) v[e] = fminf(fmaxf(v[e] * inv, -dt_max), dt_max);
+                if (ok) {
+                    if ((lcol & 7) == 0)
+                        ((uint8_t *)P.dst_scale.p)[quant_off(P.dst_scale, b, m, nbase, P.M, P.N)] = sbyte;
+                    store4(P, H, v, b, m, nbase, nvalid);
+                }
             }
             continue;
         }

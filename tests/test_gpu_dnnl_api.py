@@ -245,7 +245,9 @@ def test_dynamic_mx_dst_through_the_api(gpu, oracle):
     po.append_eltwise(cabi.ELTWISE["relu"], 0.0, 0.0)
     attr.set_post_ops(po)
     pd = dnnl.matmul_primitive_desc(eng, src_md, wei_md, dst_md, bias_md=bias_md, attr=attr)
-    assert pd.impl_info_str() == "hip:ref:any"
+    # the generic kernel is the one that matches the oracle bit for bit
+    while pd.impl_info_str() != "hip:ref:any":
+        assert pd.next_impl()
     one = dnnl.memory_desc([1], DT["f32"], tag=dnnl.tag_a)
     sc_md = dnnl.memory_desc([M, N // 32], DT["e8m0"], tag=dnnl.tag_ab)
     sc_mem = dnnl.memory(sc_md, eng)
