@@ -152,8 +152,53 @@ __device__ __forceinline__ uint32_t load_raw(int dt, const void *p, long off) {
 // raw[e] holds the src storage bits, B[e] the offsets of element e in every
 // tensor.  Every data-type dispatch is uniform over the wavefront and is taken
 // once for the N elements.
-template <int N, class RT>
+template <int N>
+__device__ __forceinline__ void load_raw_vec(int dt, const void *p, long off, uint32_t (&w)[N]);
+
+// How a unit finds its quantization parameters:
+//   GENERIC  every element has its own offsets B[e] into every tensor;
+//   SIMPLE   no scales, zero points or sum (a pure change of type and layout):
+//            B is not read;
+//   QVEC     no sum, and every parameter tensor is either constant along the
+//            unit or holds its N values consecutively and aligned: B[0] only,
+//            one (vector) load per parameter.
+enum { MODE_GENERIC = 0, MODE_SIMPLE = 1, MODE_QVEC = 2 };
+
+// the N values of parameter k (0 src scale, 1 dst scale, 2 src zero point)
+template <int N, int MODE, class RT>
+__device__ __forceinline__ void param_values(const RT &R, int k, const rbase_t (&B)[N], float (&out)[N]) {
+    const int dt = R.qdt[k];
+    if constexpr (MODE == MODE_QVEC) {
+        if (R.a.qs[k] == 0) {
+            const float v = load_float(dt, R.qp[k], B[0].q[k]);
+#pragma unroll
+            for (int e = 0; e < N; ++e) out[e] = v;
+        } else {
+            uint32_t pr[N];
+            load_raw_vec<N>(dt, R.qp[k], B[0].q[k], pr);
+            if (is_int_dt(dt)) {
+#pragma unroll
+                for (int e = 0; e < N; ++e) out[e] = (float)raw_to_int(dt, pr[e]);
+            } else if (dt == MI355_DT_F32) {
+#pragma unroll
+                for (int e = 0; e < N; ++e) out[e] = u2f(pr[e]);
+            } else {
+#pragma unroll
+                for (int e = 0; e < N; ++e) out[e] = raw_to_float(dt, pr[e]);
+            }
+        }
+    } else if (dt == MI355_DT_F32) {
+#pragma unroll
+        for (int e = 0; e < N; ++e) out[e] = ((const float *)R.qp[k])[B[e].q[k]];
+    } else {
+#pragma unroll
+        for (int e = 0; e < N; ++e) out[e] = load_float(dt, R.qp[k], B[e].q[k]);
+    }
+}
+
+template <int N, int MODE = MODE_GENERIC, class RT>
 __device__ __forceinline__ void convert(const RT &R, const uint32_t (&raw)[N], const rbase_t (&B)[N], uint32_t (&w)[N]) {
+    constexpr bool SIMPLE = MODE == MODE_SIMPLE;
     if (R.plain_copy) { // same type, no attributes: the bits move unchanged
 #pragma unroll
         for (int e = 0; e < N; ++e) w[e] = raw[e];
@@ -179,9 +224,13 @@ __device__ __forceinline__ void convert(const RT &R, const uint32_t (&raw)[N], c
 #pragma unroll
             for (int e = 0; e < N; ++e) v[e] = (int)(raw[e] & 0xf);
         }
-        if (R.qp[2]) {
+        if constexpr (!SIMPLE) {
+            if (R.qp[2]) {
+                float zp[N];
+                param_values<N, MODE>(R, 2, B, zp);
 #pragma unroll
-            for (int e = 0; e < N; ++e) v[e] -= (int)load_float(R.qdt[2], R.qp[2], B[e].q[2]);
+                for (int e = 0; e < N; ++e) v[e] -= (int)zp[e];
+            }
         }
 #pragma unroll
         for (int e = 0; e < N; ++e) x[e] = (float)v[e];
@@ -198,26 +247,26 @@ __device__ __forceinline__ void convert(const RT &R, const uint32_t (&raw)[N], c
 #pragma unroll
         for (int e = 0; e < N; ++e) x[e] = raw_to_float(sdt, raw[e]);
     }
-    if (sdt != MI355_DT_E8M0) { // e8m0 sources are converted without arithmetic
+    if (!SIMPLE && sdt != MI355_DT_E8M0) { // e8m0 sources are converted without arithmetic
         if (R.qp[0]) {
-            const int qdt = R.qdt[0];
-            if (qdt == MI355_DT_F32) {
+            float sc[N];
+            param_values<N, MODE>(R, 0, B, sc);
 #pragma unroll
-                for (int e = 0; e < N; ++e) x[e] = ((const float *)R.qp[0])[B[e].q[0]] * x[e];
-            } else {
-#pragma unroll
-                for (int e = 0; e < N; ++e) x[e] = load_float(qdt, R.qp[0], B[e].q[0]) * x[e];
-            }
+            for (int e = 0; e < N; ++e) x[e] = sc[e] * x[e];
         }
-        if (R.beta != 0.f) {
+        if constexpr (MODE == MODE_GENERIC) {
+            if (R.beta != 0.f) {
 #pragma unroll
-            for (int e = 0; e < N; ++e) x[e] += R.beta * load_float(R.dst_dt, R.dst, B[e].dof);
+                for (int e = 0; e < N; ++e) x[e] += R.beta * load_float(R.dst_dt, R.dst, B[e].dof);
+            }
         }
         if (R.qp[1] || R.dst_zp) {
             const float dzp = R.dst_zp ? (float)*(const int *)R.dst_zp : 0.f;
             if (R.qp[1]) {
+                float sc[N];
+                param_values<N, MODE>(R, 1, B, sc);
 #pragma unroll
-                for (int e = 0; e < N; ++e) x[e] = x[e] / load_float(R.qdt[1], R.qp[1], B[e].q[1]) + dzp;
+                for (int e = 0; e < N; ++e) x[e] = x[e] / sc[e] + dzp;
             } else {
 #pragma unroll
                 for (int e = 0; e < N; ++e) x[e] = x[e] / 1.f + dzp;
@@ -255,34 +304,79 @@ __device__ __forceinline__ void convert(const RT &R, const uint32_t (&raw)[N], c
     }
 }
 
-// store N (1, 2 or 4) consecutive dst elements starting at element offset off
+// N consecutive elements of BITS bits each as raw dwords: one access of
+// N * BITS / 8 bytes when that is at most 16 bytes, several 16-byte ones
+// otherwise.  The address is a multiple of the access size.
+template <int N, int BITS>
+struct vec_io_t {
+    static constexpr int TOTAL = N * BITS;            // bits
+    static constexpr int D = TOTAL >= 32 ? TOTAL / 32 : 1; // dwords
+    static __device__ __forceinline__ void load(const void *p, long off, uint32_t (&w)[N]) {
+        const char *q = (const char *)p + off * BITS / 8;
+        uint32_t dw[D];
+        if constexpr (TOTAL >= 128) {
+#pragma unroll
+            for (int c = 0; c < D / 4; ++c) {
+                const uint4 v = ((const uint4 *)q)[c];
+                dw[4 * c] = v.x; dw[4 * c + 1] = v.y; dw[4 * c + 2] = v.z; dw[4 * c + 3] = v.w;
+            }
+        } else if constexpr (TOTAL == 64) {
+            const uint2 v = *(const uint2 *)q;
+            dw[0] = v.x; dw[1] = v.y;
+        } else if constexpr (TOTAL == 32) {
+            dw[0] = *(const uint32_t *)q;
+        } else {
+            dw[0] = *(const uint16_t *)q;
+        }
+#pragma unroll
+        for (int e = 0; e < N; ++e)
+            w[e] = BITS == 32 ? dw[e] : (dw[e * BITS / 32] >> (e * BITS % 32)) & (0xffffffffu >> (32 - BITS));
+    }
+    static __device__ __forceinline__ void store(void *p, long off, const uint32_t (&w)[N]) {
+        char *q = (char *)p + off * BITS / 8;
+        uint32_t dw[D];
+#pragma unroll
+        for (int c = 0; c < D; ++c) dw[c] = 0;
+#pragma unroll
+        for (int e = 0; e < N; ++e) dw[e * BITS / 32] |= BITS == 32 ? w[e] : w[e] << (e * BITS % 32);
+        if constexpr (TOTAL >= 128) {
+#pragma unroll
+            for (int c = 0; c < D / 4; ++c) {
+                uint4 v;
+                v.x = dw[4 * c]; v.y = dw[4 * c + 1]; v.z = dw[4 * c + 2]; v.w = dw[4 * c + 3];
+                ((uint4 *)q)[c] = v;
+            }
+        } else if constexpr (TOTAL == 64) {
+            uint2 v;
+            v.x = dw[0]; v.y = dw[1];
+            *(uint2 *)q = v;
+        } else if constexpr (TOTAL == 32) {
+            *(uint32_t *)q = dw[0];
+        } else {
+            *(uint16_t *)q = (uint16_t)dw[0];
+        }
+    }
+};
+
+// store N consecutive dst elements starting at element offset off; `packed`:
+// they may leave as one aligned vector (N >= 4)
 template <int N>
 __device__ __forceinline__ void store_bits(int dt, void *dst, long off, const uint32_t (&w)[N], bool packed) {
     const int bits = dt_bits(dt);
+    if constexpr (N >= 4) {
+        if (packed) {
+            if (bits == 4) vec_io_t<N, 4>::store(dst, off, w);
+            else if (bits == 8) vec_io_t<N, 8>::store(dst, off, w);
+            else if (bits == 16) vec_io_t<N, 16>::store(dst, off, w);
+            else vec_io_t<N, 32>::store(dst, off, w);
+            return;
+        }
+    }
     if (bits == 4) {
         // off is even and the N nibbles fill whole bytes
         uint8_t *p = (uint8_t *)dst + (off >> 1);
-        if (N == 4 && packed) {
-            *(uint16_t *)p = (uint16_t)(w[0] | (w[1] << 4) | (w[2] << 8) | (w[3] << 12));
-            return;
-        }
 #pragma unroll
         for (int e = 0; e + 1 < N; e += 2) p[e >> 1] = (uint8_t)(w[e] | (w[e + 1] << 4));
-        return;
-    }
-    if (packed && N == 4) {
-        if (bits == 8) {
-            *(uint32_t *)((uint8_t *)dst + off) = w[0] | (w[1] << 8) | (w[2] << 16) | (w[3] << 24);
-        } else if (bits == 16) {
-            uint2 o;
-            o.x = w[0] | (w[1] << 16);
-            o.y = w[2] | (w[3] << 16);
-            *(uint2 *)((uint16_t *)dst + off) = o;
-        } else {
-            uint4 o;
-            o.x = w[0]; o.y = w[1]; o.z = w[2]; o.w = w[3];
-            *(uint4 *)((uint32_t *)dst + off) = o;
-        }
         return;
     }
 #pragma unroll
@@ -293,50 +387,95 @@ __device__ __forceinline__ void store_bits(int dt, void *dst, long off, const ui
     }
 }
 
-// four consecutive src elements as one vector load (off is a multiple of four)
-__device__ __forceinline__ void load_raw4(int dt, const void *p, long off, uint32_t (&w)[4]) {
+// N consecutive src elements as vector loads (off is a multiple of N)
+template <int N>
+__device__ __forceinline__ void load_raw_vec(int dt, const void *p, long off, uint32_t (&w)[N]) {
     const int bits = dt_bits(dt);
-    if (bits == 32) {
-        const uint4 v = *(const uint4 *)((const uint32_t *)p + off);
-        w[0] = v.x; w[1] = v.y; w[2] = v.z; w[3] = v.w;
-    } else if (bits == 16) {
-        const uint2 v = *(const uint2 *)((const uint16_t *)p + off);
-        w[0] = v.x & 0xffffu; w[1] = v.x >> 16; w[2] = v.y & 0xffffu; w[3] = v.y >> 16;
-    } else if (bits == 8) {
-        const uint32_t v = *(const uint32_t *)((const uint8_t *)p + off);
-        w[0] = v & 0xffu; w[1] = (v >> 8) & 0xffu; w[2] = (v >> 16) & 0xffu; w[3] = v >> 24;
-    } else {
-        const uint32_t v = *(const uint16_t *)((const uint8_t *)p + (off >> 1));
-        w[0] = v & 0xfu; w[1] = (v >> 4) & 0xfu; w[2] = (v >> 8) & 0xfu; w[3] = (v >> 12) & 0xfu;
-    }
+    if (bits == 32) vec_io_t<N, 32>::load(p, off, w);
+    else if (bits == 16) vec_io_t<N, 16>::load(p, off, w);
+    else if (bits == 8) vec_io_t<N, 8>::load(p, off, w);
+    else vec_io_t<N, 4>::load(p, off, w);
 }
 
-// grid: x over chunks of the dim `a`, y over the outer index.  E elements per
-// lane along `a` (dst stride 1 when E > 1).
-template <int E>
+// One unit = E consecutive elements along the dim `a` (dst stride 1 when
+// E > 1) of one outer index; units are numbered (outer, chunk of a) and walked
+// with a grid stride.  A lane issues the loads of its next unit before it
+// converts and stores the current one: with a single unit in flight per lane a
+// plain s8 copy ran at 1.7 TB/s.
+template <int E, int MODE>
 __global__ void __launch_bounds__(256) reorder_direct_kernel(const reorder_t R_) {
     const auto &R = *(const __attribute__((address_space(4))) reorder_t *)__builtin_amdgcn_kernarg_segment_ptr();
+    constexpr bool SIMPLE = MODE == MODE_SIMPLE;
     const unsigned units = R.a.n / E;
-    for (unsigned o = blockIdx.y; o < R.outer_total; o += gridDim.y) {
-        const rbase_t B0 = outer_base(R, o);
-        for (unsigned u = blockIdx.x * 256 + threadIdx.x; u < units; u += gridDim.x * 256) {
-            rbase_t B[E];
-            add_dim_run<E>(B, B0, R.a, u * E);
-            uint32_t raw[E], w[E];
-            bool loaded = false;
-            if constexpr (E == 4) {
-                if (R.src_vec) {
-                    load_raw4(R.src_dt, R.src, B[0].so, raw);
-                    loaded = true;
-                }
-            }
-            if (!loaded) {
-#pragma unroll
-                for (int e = 0; e < E; ++e) raw[e] = load_raw(R.src_dt, R.src, B[e].so);
-            }
-            convert<E>(R, raw, B, w);
-            store_bits<E>(R.dst_dt, R.dst, B[0].dof, w, R.packed);
+    const unsigned long total = (unsigned long)R.outer_total * units;
+    const unsigned long stride = (unsigned long)gridDim.x * 256;
+    // offsets of unit f (recomputed where needed rather than kept across the
+    // loads).  SIMPLE: only the src and dst offsets of the unit's first element;
+    // the per-element offsets into the parameter tensors are most of the
+    // integer work of a unit otherwise.
+    auto bases = [&](unsigned long f, rbase_t (&B)[E]) __attribute__((always_inline)) {
+        unsigned o, u;
+        if (total >> 32) {
+            o = (unsigned)(f / units);
+            u = (unsigned)(f - (unsigned long)o * units);
+        } else {
+            o = (unsigned)f / units;
+            u = (unsigned)f - o * units;
         }
+        if constexpr (SIMPLE) {
+            long so = (long)(u * E) * R.a.ss, dof = (long)(u * E) * R.a.ds;
+            for (int i = 0; i < R.n_outer; ++i) {
+                const unsigned n = R.outer[i].n;
+                const unsigned q = o / n, r = o - q * n;
+                o = q;
+                so += (long)r * R.outer[i].ss;
+                dof += (long)r * R.outer[i].ds;
+            }
+            B[0].so = so;
+            B[0].dof = dof;
+        } else if constexpr (MODE == MODE_QVEC) {
+            B[0] = outer_base(R, o);
+            add_dim(B[0], R.a, u * E);
+        } else {
+            const rbase_t B0 = outer_base(R, o);
+            add_dim_run<E>(B, B0, R.a, u * E);
+        }
+    };
+    auto fetch = [&](unsigned long f, uint32_t (&raw)[E]) __attribute__((always_inline)) {
+        rbase_t B[E];
+        bases(f, B);
+        bool loaded = false;
+        if constexpr (E >= 4) {
+            if (R.src_vec) {
+                load_raw_vec<E>(R.src_dt, R.src, B[0].so, raw);
+                loaded = true;
+            }
+        }
+        if (!loaded) {
+#pragma unroll
+            for (int e = 0; e < E; ++e)
+                raw[e] = load_raw(R.src_dt, R.src, MODE != MODE_GENERIC ? B[0].so + (long)e * R.a.ss : B[e].so);
+        }
+    };
+    unsigned long f = (unsigned long)blockIdx.x * 256 + threadIdx.x;
+    if (f >= total) return;
+    uint32_t raw[E];
+    fetch(f, raw);
+    while (true) {
+        const unsigned long fn = f + stride;
+        uint32_t next[E];
+#pragma unroll
+        for (int e = 0; e < E; ++e) next[e] = 0;
+        if (fn < total) fetch(fn, next);
+        rbase_t B[E];
+        bases(f, B);
+        uint32_t w[E];
+        convert<E, MODE>(R, raw, B, w);
+        store_bits<E>(R.dst_dt, R.dst, B[0].dof, w, R.packed);
+        if (fn >= total) break;
+#pragma unroll
+        for (int e = 0; e < E; ++e) raw[e] = next[e];
+        f = fn;
     }
 }
 
@@ -696,21 +835,35 @@ extern "C" int mi355_reorder_launch(const mi355_reorder_desc_t *desc, const mi35
     R.outer_total = (unsigned)outer;
 
     const int dbits = dt_bits(d.dst_dt), sbits = dt_bits(d.src_dt);
-    // four elements per lane along `a` as one aligned vector: unit stride, an
-    // extent that divides, every other stride and the pointer aligned to it
-    auto vec4_ok = [&](const void *p, bool src_side, int bits) {
+    // E elements per lane along `a` as one aligned vector (several 16-byte ones
+    // beyond 16 bytes): unit stride, an extent that divides, every other stride
+    // and the pointer aligned to it
+    auto vec_ok = [&](const void *p, bool src_side, int bits, int E) {
         const long sa = src_side ? v[da].ss : v[da].ds;
-        if (sa != 1 || v[da].n % 4) return false;
-        const long bytes4 = bits / 2 ? bits / 2 : 1;
-        if ((uintptr_t)p % (size_t)bytes4) return false;
+        if (sa != 1 || v[da].n % E) return false;
+        long bytes = (long)E * bits / 8;
+        if (bytes > 16) bytes = 16;
+        if (bytes < 1) bytes = 1;
+        if ((uintptr_t)p % (size_t)bytes) return false;
         for (int i = 1; i < nv; ++i)
-            if ((src_side ? v[i].ss : v[i].ds) % 4) return false;
+            if ((src_side ? v[i].ss : v[i].ds) % E) return false;
         return true;
     };
     R.plain_copy = d.src_dt == d.dst_dt && d.beta == 0.f && d.src_scale.dt == MI355_DT_UNDEF
             && d.dst_scale.dt == MI355_DT_UNDEF && d.src_zp.dt == MI355_DT_UNDEF && d.dst_zp.dt == MI355_DT_UNDEF;
-    R.packed = vec4_ok(R.dst, false, dbits);
-    R.src_vec = vec4_ok(R.src, true, sbits);
+    // direct kernel: the widest E in {16, 8, 4} whose narrower side is at most
+    // 16 bytes and whose wider side at most 64 bytes per lane
+    int E = 1;
+    if (!tiled) {
+        const int narrow = dbits < sbits ? dbits : sbits, wide = dbits < sbits ? sbits : dbits;
+        for (int cand = 16; cand >= 4 && E == 1; cand /= 2)
+            if (cand * narrow <= 128 && cand * wide <= 256 && vec_ok(R.dst, false, dbits, cand)) E = cand;
+        if (E == 1 && dbits == 4) E = 2;
+    } else {
+        E = 4;
+    }
+    R.packed = E >= 4 && vec_ok(R.dst, false, dbits, E);
+    R.src_vec = E >= 4 && vec_ok(R.src, true, sbits, E);
     hipStream_t hs = (hipStream_t)stream;
     const unsigned gy = (unsigned)(outer < 65535 ? outer : 65535);
     if (tiled) {
@@ -721,16 +874,41 @@ extern "C" int mi355_reorder_launch(const mi355_reorder_desc_t *desc, const mi35
         if (gx > (1 << 20)) gx = 1 << 20;
         hipLaunchKernelGGL(reorder_tiled_kernel, dim3((unsigned)gx, gy), dim3(256), 0, hs, R);
     } else {
-        int E = 1;
-        if (R.packed) E = 4;
-        else if (dbits == 4) E = 2;
         R.elems = E;
-        long gx = ((long)R.a.n / E + 255) / 256;
-        if (gx > (1 << 20)) gx = 1 << 20;
+        // units of all outer indices in one grid-stride walk; enough workgroups
+        // to fill the device a few times over, each lane several units
+        const long total_units = outer * ((long)R.a.n / E);
+        long gx = (total_units + 255) / 256;
+        if (gx > 256 * 16) gx = 256 * 16;
         if (gx < 1) gx = 1;
-        if (E == 4) hipLaunchKernelGGL(reorder_direct_kernel<4>, dim3((unsigned)gx, gy), dim3(256), 0, hs, R);
-        else if (E == 2) hipLaunchKernelGGL(reorder_direct_kernel<2>, dim3((unsigned)gx, gy), dim3(256), 0, hs, R);
-        else hipLaunchKernelGGL(reorder_direct_kernel<1>, dim3((unsigned)gx, gy), dim3(256), 0, hs, R);
+        const dim3 grid((unsigned)gx), block(256);
+        const bool simple = d.beta == 0.f && d.src_scale.dt == MI355_DT_UNDEF && d.dst_scale.dt == MI355_DT_UNDEF
+                && d.src_zp.dt == MI355_DT_UNDEF && d.dst_zp.dt == MI355_DT_UNDEF;
+        // every parameter tensor constant along a unit, or its E values consecutive and aligned
+        bool qvec = !simple && d.beta == 0.f && E >= 4;
+        for (int k = 0; k < 3 && qvec; ++k) {
+            if (!R.qp[k] || R.a.qs[k] == 0) continue;
+            const int pbits = dt_bits(R.qdt[k]);
+            long bytes = (long)E * pbits / 8;
+            if (bytes > 16) bytes = 16;
+            if (bytes < 1) bytes = 1;
+            if (R.a.qs[k] != 1 || R.a.qg[k] != 1 || (uintptr_t)R.qp[k] % (size_t)bytes) qvec = false;
+            for (int i = 0; i < R.n_outer && qvec; ++i)
+                if (R.outer[i].qs[k] % E) qvec = false;
+        }
+        const int mode = simple ? MODE_SIMPLE : qvec ? MODE_QVEC : MODE_GENERIC;
+#define MI355_REORDER_CASE(E_) \
+    if (E == E_) { \
+        if (mode == MODE_SIMPLE) hipLaunchKernelGGL((reorder_direct_kernel<E_, MODE_SIMPLE>), grid, block, 0, hs, R); \
+        else if (mode == MODE_QVEC) hipLaunchKernelGGL((reorder_direct_kernel<E_, MODE_QVEC>), grid, block, 0, hs, R); \
+        else hipLaunchKernelGGL((reorder_direct_kernel<E_, MODE_GENERIC>), grid, block, 0, hs, R); \
+    }
+        MI355_REORDER_CASE(16)
+        MI355_REORDER_CASE(8)
+        MI355_REORDER_CASE(4)
+        MI355_REORDER_CASE(2)
+        MI355_REORDER_CASE(1)
+#undef MI355_REORDER_CASE
     }
     if (hipGetLastError() != hipSuccess) {
         set_error("reorder: launch failed");

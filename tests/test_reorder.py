@@ -199,6 +199,24 @@ def _qp(seed, dt, mask, shape, groups=(1, 1), lo=0.05, hi=2.0):
 
 
 CASES = [
+    # direct kernel, 16 / 8 elements per lane: attribute-free (one base per unit) ...
+    lambda: _case("s8 copy 16 per lane", (24, 512), cabi.DT_S8, cabi.DT_S8, 40),
+    lambda: _case("u8->f32 16 per lane, rows strided", (3, 40, 64), cabi.DT_U8, cabi.DT_F32, 41, src_perm=(1, 0, 2)),
+    lambda: _case("f32->bf16 8 per lane", (37, 72), cabi.DT_F32, cabi.DT_BF16, 42),
+    lambda: _case("u4->s8 16 per lane", (20, 96), cabi.DT_U4, cabi.DT_S8, 43),
+    lambda: _case("s8 copy, extent only a multiple of 8", (9, 40), cabi.DT_S8, cabi.DT_S8, 44),
+    # ... and with parameters that are consecutive along the unit (vector loads) or constant along it
+    lambda: _case("f32->s8 per-column scale, 8 per lane", (33, 128), cabi.DT_F32, cabi.DT_S8, 45,
+                  quant={"dst_scale": _qp(60, cabi.DT_F32, 2, (128,))}),
+    lambda: _case("s8->bf16 per-column bf16 scale + u4 zp", (17, 64), cabi.DT_S8, cabi.DT_BF16, 46,
+                  quant={"src_scale": _qp(61, cabi.DT_BF16, 2, (64,)), "src_zp": _qp(62, cabi.DT_U4, 2, (64,))}),
+    lambda: _case("s8->f32 per-row scale, per-column zp", (48, 64), cabi.DT_S8, cabi.DT_F32, 47,
+                  quant={"src_scale": _qp(63, cabi.DT_F32, 1, (48,)), "src_zp": _qp(64, cabi.DT_S8, 2, (64,)),
+                         "dst_scale": _qp(65, cabi.DT_F32, 3, (48, 64))}),
+    lambda: _case("u8->s8 grouped along the unit (per-element offsets)", (16, 128), cabi.DT_U8, cabi.DT_S8, 48,
+                  quant={"src_scale": _qp(66, cabi.DT_F32, 3, (16, 4), (1, 32))}),
+    lambda: _case("f32->f32 per-column scale with sum (per-element offsets)", (12, 64), cabi.DT_F32, cabi.DT_F32, 49,
+                  quant={"dst_scale": _qp(67, cabi.DT_F32, 2, (64,))}, beta=0.5),
     # direct kernel: same unit-stride dim on both sides
     lambda: _case("copy f32 ragged", (7, 33), cabi.DT_F32, cabi.DT_F32, 1),
     lambda: _case("f32->s8 packed stores", (64, 256), cabi.DT_F32, cabi.DT_S8, 2,
