@@ -543,6 +543,56 @@ __global__ void __launch_bounds__(256) reorder_tiled_kernel(const reorder_t R_) 
     }
 }
 
+// Transposition of 8-bit elements without attributes (the layout change of
+// int8 / fp8 weights that format_tag::any asks for): 64 x 64 tile over (a, b),
+// b has src stride 1, a has dst stride 1, both extents multiples of 64.  A
+// thread loads a 4 x 4 block as four dwords, transposes it in registers with
+// eight byte permutes and parks the four result dwords in LDS; the tile then
+// leaves as 16-byte stores along a.
+__global__ void __launch_bounds__(256) transpose8_kernel(const reorder_t R_) {
+    const auto &R = *(const __attribute__((address_space(4))) reorder_t *)__builtin_amdgcn_kernarg_segment_ptr();
+    constexpr int PITCH = 17; // dwords per LDS row (16 + 1: spreads the banks)
+    __shared__ uint32_t tile[64 * PITCH];
+    const unsigned ntiles = R.tiles_a * R.tiles_b;
+    const int bi = threadIdx.x & 15, ai = threadIdx.x >> 4; // read: block (4 ai .. +3, 4 bi .. +3)
+    const int wb = threadIdx.x >> 2, wq = threadIdx.x & 3;  // write: row b, 16 bytes of a
+    const uint8_t *src = (const uint8_t *)R.src;
+    uint8_t *dst = (uint8_t *)R.dst;
+    for (unsigned o = blockIdx.y; o < R.outer_total; o += gridDim.y) {
+        long so = 0, dof = 0;
+        {
+            unsigned oo = o;
+            for (int i = 0; i < R.n_outer; ++i) {
+                const unsigned n = R.outer[i].n;
+                const unsigned q = oo / n, r = oo - q * n;
+                oo = q;
+                so += (long)r * R.outer[i].ss;
+                dof += (long)r * R.outer[i].ds;
+            }
+        }
+        for (unsigned t = blockIdx.x; t < ntiles; t += gridDim.x) {
+            const unsigned tb = t % R.tiles_b, ta = t / R.tiles_b;
+            const long a0 = (long)ta * 64, b0 = (long)tb * 64;
+            const uint8_t *p = src + so + (a0 + 4 * ai) * R.a.ss + b0 + 4 * bi;
+            const uint32_t r0 = *(const uint32_t *)p, r1 = *(const uint32_t *)(p + R.a.ss),
+                           r2 = *(const uint32_t *)(p + 2 * R.a.ss), r3 = *(const uint32_t *)(p + 3 * R.a.ss);
+            // byte k of r_i is element (a + i, b + k); T_k collects byte k of the four rows
+            const uint32_t x0 = __builtin_amdgcn_perm(r1, r0, 0x05010400u), x1 = __builtin_amdgcn_perm(r1, r0, 0x07030602u);
+            const uint32_t y0 = __builtin_amdgcn_perm(r3, r2, 0x05010400u), y1 = __builtin_amdgcn_perm(r3, r2, 0x07030602u);
+            tile[(4 * bi + 0) * PITCH + ai] = __builtin_amdgcn_perm(y0, x0, 0x05040100u);
+            tile[(4 * bi + 1) * PITCH + ai] = __builtin_amdgcn_perm(y0, x0, 0x07060302u);
+            tile[(4 * bi + 2) * PITCH + ai] = __builtin_amdgcn_perm(y1, x1, 0x05040100u);
+            tile[(4 * bi + 3) * PITCH + ai] = __builtin_amdgcn_perm(y1, x1, 0x07060302u);
+            __syncthreads();
+            uint4 v;
+            v.x = tile[wb * PITCH + 4 * wq]; v.y = tile[wb * PITCH + 4 * wq + 1];
+            v.z = tile[wb * PITCH + 4 * wq + 2]; v.w = tile[wb * PITCH + 4 * wq + 3];
+            *(uint4 *)(dst + dof + (b0 + wb) * R.b.ds + a0 + 16 * wq) = v;
+            __syncthreads();
+        }
+    }
+}
+
 bool dt_ok(int dt) {
     switch (dt) {
         case MI355_DT_F16: case MI355_DT_BF16: case MI355_DT_F32: case MI355_DT_S32: case MI355_DT_S8:
@@ -872,7 +922,13 @@ extern "C" int mi355_reorder_launch(const mi355_reorder_desc_t *desc, const mi35
         R.elems = 4;
         long gx = (long)R.tiles_a * R.tiles_b;
         if (gx > (1 << 20)) gx = 1 << 20;
-        hipLaunchKernelGGL(reorder_tiled_kernel, dim3((unsigned)gx, gy), dim3(256), 0, hs, R);
+        // 8-bit transposition without attributes: whole tiles, dword loads along b, 16-byte stores along a
+        bool t8 = R.plain_copy && dbits == 8 && R.a.n % 64 == 0 && R.b.n % 64 == 0 && R.a.ss % 4 == 0
+                && R.b.ds % 16 == 0 && (uintptr_t)R.src % 4 == 0 && (uintptr_t)R.dst % 16 == 0;
+        for (int i = 0; i < R.n_outer && t8; ++i)
+            if (R.outer[i].ss % 4 || R.outer[i].ds % 16) t8 = false;
+        if (t8) hipLaunchKernelGGL(transpose8_kernel, dim3((unsigned)gx, gy), dim3(256), 0, hs, R);
+        else hipLaunchKernelGGL(reorder_tiled_kernel, dim3((unsigned)gx, gy), dim3(256), 0, hs, R);
     } else {
         R.elems = E;
         // units of all outer indices in one grid-stride walk; enough workgroups

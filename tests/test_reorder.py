@@ -217,6 +217,11 @@ CASES = [
                   quant={"src_scale": _qp(66, cabi.DT_F32, 3, (16, 4), (1, 32))}),
     lambda: _case("f32->f32 per-column scale with sum (per-element offsets)", (12, 64), cabi.DT_F32, cabi.DT_F32, 49,
                   quant={"dst_scale": _qp(67, cabi.DT_F32, 2, (64,))}, beta=0.5),
+    # 8-bit transposition in registers (whole 64 x 64 tiles) and its fallback for ragged extents
+    lambda: _case("s8 ab->ba whole tiles", (128, 192), cabi.DT_S8, cabi.DT_S8, 50, dst_perm=(1, 0)),
+    lambda: _case("u8 batched acb whole tiles", (3, 64, 128), cabi.DT_U8, cabi.DT_U8, 51, dst_perm=(0, 2, 1)),
+    lambda: _case("e4m3 ba->ab whole tiles", (192, 64), cabi.DT_F8_E4M3, cabi.DT_F8_E4M3, 52, src_perm=(1, 0)),
+    lambda: _case("s8 ab->ba ragged", (130, 192), cabi.DT_S8, cabi.DT_S8, 53, dst_perm=(1, 0)),
     # direct kernel: same unit-stride dim on both sides
     lambda: _case("copy f32 ragged", (7, 33), cabi.DT_F32, cabi.DT_F32, 1),
     lambda: _case("f32->s8 packed stores", (64, 256), cabi.DT_F32, cabi.DT_S8, 2,
