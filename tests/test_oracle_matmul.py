@@ -296,3 +296,20 @@ def test_batched_broadcast_weights(oracle):
                       src=src, wei=wei, wei_stride=(0, N, 1))
     got = oracle.run_oracle(p).reshape(B, M, N)
     assert np.array_equal(got, np.einsum("bmk,kn->bmn", src.astype(np.int64), wei.astype(np.int64)))
+
+
+def test_row_sampling_of_the_full_size_checks_is_consistent():
+    """The full-size GPU checks compare sampled dst rows with the oracle run on
+    the sub-problem made of those rows: here the same construction against the
+    oracle's own full result, for the three GEMM configurations."""
+    from oracle import binding as orc
+    from tests.test_gpu_full_size import row_slice, rows_of, sample_rows
+    for make in (lambda: configs.config3(M=512, N=128, K=256, wtag="ba"),
+                 lambda: configs.config4(M=512, N=128, K=256, wtag="ba"),
+                 lambda: configs.config5(M=512, N=128, K=256, wtag="ba")):
+        p = make()
+        full = orc.run_oracle(p)
+        rows = sample_rows(p.M, 2, 1)
+        want = orc.run_oracle(row_slice(p, rows))
+        assert np.array_equal(np.asarray(rows_of(p, full, rows)).view(np.uint8),
+                              np.asarray(want).view(np.uint8).reshape(-1)), p.name
