@@ -480,7 +480,10 @@ __global__ void __launch_bounds__(256) reorder_direct_kernel(const reorder_t R_)
 }
 
 // 64 x 64 tile over (b, a): b has src stride 1, a has dst stride 1.  grid: x
-// over the tiles, y over the outer index.
+// over the tiles, y over the outer index.  MODE as in the direct kernel; the
+// modes other than MODE_GENERIC want the extent of a to be a multiple of four
+// (a lane's four rows are then all inside or all outside the tensor).
+template <int MODE>
 __global__ void __launch_bounds__(256) reorder_tiled_kernel(const reorder_t R_) {
     const auto &R = *(const __attribute__((address_space(4))) reorder_t *)__builtin_amdgcn_kernarg_segment_ptr();
     __shared__ uint32_t tile[64][65];
@@ -496,21 +499,34 @@ __global__ void __launch_bounds__(256) reorder_tiled_kernel(const reorder_t R_) 
             for (int i0 = ty * 4; i0 < 64; i0 += 16) {
                 rbase_t B[4];
                 uint32_t raw[4], v[4];
-                rbase_t Bb = B0;
                 const unsigned ib = b0 + tx < R.b.n ? b0 + tx : R.b.n - 1; // clamped, masked below
-                add_dim(Bb, R.b, ib);
-                if (a0 + i0 + 4 <= R.a.n) {
-                    add_dim_run<4>(B, Bb, R.a, a0 + i0);
-                } else { // ragged last tile along a: clamped, masked below
+                if constexpr (MODE == MODE_GENERIC) {
+                    rbase_t Bb = B0;
+                    add_dim(Bb, R.b, ib);
+                    if (a0 + i0 + 4 <= R.a.n) {
+                        add_dim_run<4>(B, Bb, R.a, a0 + i0);
+                    } else { // ragged last tile along a: clamped, masked below
 #pragma unroll
-                    for (int k = 0; k < 4; ++k) {
-                        B[k] = Bb;
-                        add_dim(B[k], R.a, a0 + i0 + k < R.a.n ? a0 + i0 + k : R.a.n - 1);
+                        for (int k = 0; k < 4; ++k) {
+                            B[k] = Bb;
+                            add_dim(B[k], R.a, a0 + i0 + k < R.a.n ? a0 + i0 + k : R.a.n - 1);
+                        }
                     }
-                }
 #pragma unroll
-                for (int k = 0; k < 4; ++k) raw[k] = load_raw(R.src_dt, R.src, B[k].so);
-                convert<4>(R, raw, B, v);
+                    for (int k = 0; k < 4; ++k) raw[k] = load_raw(R.src_dt, R.src, B[k].so);
+                } else {
+                    const unsigned ia = a0 + i0 < R.a.n ? a0 + i0 : R.a.n - 4; // clamped, masked below
+                    if constexpr (MODE == MODE_SIMPLE) {
+                        B[0].so = B0.so + (long)ib * R.b.ss + (long)ia * R.a.ss;
+                    } else {
+                        B[0] = B0;
+                        add_dim(B[0], R.b, ib);
+                        add_dim(B[0], R.a, ia);
+                    }
+#pragma unroll
+                    for (int k = 0; k < 4; ++k) raw[k] = load_raw(R.src_dt, R.src, B[0].so + (long)k * R.a.ss);
+                }
+                convert<4, MODE>(R, raw, B, v);
 #pragma unroll
                 for (int k = 0; k < 4; ++k) tile[i0 + k][tx] = v[k];
             }
@@ -927,8 +943,23 @@ extern "C" int mi355_reorder_launch(const mi355_reorder_desc_t *desc, const mi35
                 && R.b.ds % 16 == 0 && (uintptr_t)R.src % 4 == 0 && (uintptr_t)R.dst % 16 == 0;
         for (int i = 0; i < R.n_outer && t8; ++i)
             if (R.outer[i].ss % 4 || R.outer[i].ds % 16) t8 = false;
-        if (t8) hipLaunchKernelGGL(transpose8_kernel, dim3((unsigned)gx, gy), dim3(256), 0, hs, R);
-        else hipLaunchKernelGGL(reorder_tiled_kernel, dim3((unsigned)gx, gy), dim3(256), 0, hs, R);
+        const bool simple = d.beta == 0.f && d.src_scale.dt == MI355_DT_UNDEF && d.dst_scale.dt == MI355_DT_UNDEF
+                && d.src_zp.dt == MI355_DT_UNDEF && d.dst_zp.dt == MI355_DT_UNDEF;
+        // a lane converts four consecutive a at one b: every parameter tensor constant
+        // along a, or its four values consecutive and aligned
+        bool qvec = !simple && d.beta == 0.f;
+        for (int k = 0; k < 3 && qvec; ++k) {
+            if (!R.qp[k] || R.a.qs[k] == 0) continue;
+            const long bytes = 4L * dt_bits(R.qdt[k]) / 8;
+            if (R.a.qs[k] != 1 || R.a.qg[k] != 1 || (uintptr_t)R.qp[k] % (size_t)bytes || R.b.qs[k] % 4) qvec = false;
+            for (int i = 0; i < R.n_outer && qvec; ++i)
+                if (R.outer[i].qs[k] % 4) qvec = false;
+        }
+        const dim3 grid((unsigned)gx, gy), block(256);
+        if (t8) hipLaunchKernelGGL(transpose8_kernel, grid, block, 0, hs, R);
+        else if (R.a.n % 4 == 0 && simple) hipLaunchKernelGGL(reorder_tiled_kernel<MODE_SIMPLE>, grid, block, 0, hs, R);
+        else if (R.a.n % 4 == 0 && qvec) hipLaunchKernelGGL(reorder_tiled_kernel<MODE_QVEC>, grid, block, 0, hs, R);
+        else hipLaunchKernelGGL(reorder_tiled_kernel<MODE_GENERIC>, grid, block, 0, hs, R);
     } else {
         R.elems = E;
         // units of all outer indices in one grid-stride walk; enough workgroups

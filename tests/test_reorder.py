@@ -222,6 +222,17 @@ CASES = [
     lambda: _case("u8 batched acb whole tiles", (3, 64, 128), cabi.DT_U8, cabi.DT_U8, 51, dst_perm=(0, 2, 1)),
     lambda: _case("e4m3 ba->ab whole tiles", (192, 64), cabi.DT_F8_E4M3, cabi.DT_F8_E4M3, 52, src_perm=(1, 0)),
     lambda: _case("s8 ab->ba ragged", (130, 192), cabi.DT_S8, cabi.DT_S8, 53, dst_perm=(1, 0)),
+    # tiled kernel: attribute-free, parameters constant along / consecutive along the dst-contiguous dim, generic
+    lambda: _case("bf16->f32 transposed", (96, 80), cabi.DT_BF16, cabi.DT_F32, 54, dst_perm=(1, 0)),
+    lambda: _case("u4 transposed", (64, 96), cabi.DT_U4, cabi.DT_U4, 55, dst_perm=(1, 0)),
+    lambda: _case("f32->s8 transposed, scale per src-contiguous dim", (72, 128), cabi.DT_F32, cabi.DT_S8, 56,
+                  dst_perm=(1, 0), quant={"dst_scale": _qp(70, cabi.DT_F32, 2, (128,))}),
+    lambda: _case("s8->f32 transposed, scale and zp per dst-contiguous dim", (64, 48), cabi.DT_S8, cabi.DT_F32, 57,
+                  dst_perm=(1, 0), quant={"src_scale": _qp(71, cabi.DT_BF16, 1, (64,)), "src_zp": _qp(72, cabi.DT_S8, 1, (64,))}),
+    lambda: _case("f32->s8 transposed, ragged dst-contiguous extent", (70, 64), cabi.DT_F32, cabi.DT_S8, 58,
+                  dst_perm=(1, 0), quant={"dst_scale": _qp(73, cabi.DT_F32, 2, (64,))}),
+    lambda: _case("u8->s8 transposed, groups on both dims", (64, 64), cabi.DT_U8, cabi.DT_S8, 59,
+                  dst_perm=(1, 0), quant={"src_scale": _qp(74, cabi.DT_F32, 3, (2, 4), (32, 16))}),
     # direct kernel: same unit-stride dim on both sides
     lambda: _case("copy f32 ragged", (7, 33), cabi.DT_F32, cabi.DT_F32, 1),
     lambda: _case("f32->s8 packed stores", (64, 256), cabi.DT_F32, cabi.DT_S8, 2,
