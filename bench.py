@@ -44,7 +44,7 @@ MEASURED_TRAFFIC = {
     ("c3", 8192): 1024824874, ("c4", 4096): 2124622179, ("c5", 8192): 569439623,
     ("c2", 1): 31612633, ("c2", 8): 32271601, ("c2", 32): 34542741,        # packed weights (format any)
     ("c2ab", 1): 32839597, ("c2ab", 8): 35736697, ("c2ab", 32): 51670775,  # plain ab weights (--wtag ab)
-    ("c1", 256): 8413792,
+    ("c1", 256): 8645444,
 }
 
 # MI355X published peaks
