@@ -178,7 +178,7 @@ __device__ __forceinline__ epi_hoist_t make_hoist(const PT &P, long b, long nbas
     }
     // The batched epilogue (several row quads per dispatch) needs every operand in
     // registers or in the staging area: no loads inside the loop.
-    H.batchable = !H.dynamic && H.n_po == H.nfast && (H.bias_mode != 2 || H.staged == STG_BIAS) && nvalid == 4 && H.dst_vec;
+    H.batchable = H.n_po == H.nfast && (H.bias_mode != 2 || H.staged == STG_BIAS) && nvalid == 4 && H.dst_vec;
     {
         auto operand_ready = [&](const po_reg_t &r, int i) {
             if (r.kind == MI355_PO_BINARY)
@@ -187,7 +187,8 @@ __device__ __forceinline__ epi_hoist_t make_hoist(const PT &P, long b, long nbas
             return true; // grab() admits the five cheap eltwise algorithms only
         };
         const int dd = H.dst_dt;
-        if (dd != MI355_DT_S8 && dd != MI355_DT_U8 && dd != MI355_DT_BF16 && dd != MI355_DT_F32 && dd != MI355_DT_S32)
+        if (dd != MI355_DT_S8 && dd != MI355_DT_U8 && dd != MI355_DT_BF16 && dd != MI355_DT_F32 && dd != MI355_DT_S32
+                && dd != MI355_DT_F8_E4M3 && dd != MI355_DT_F8_E5M2)
             H.batchable = 0;
         if (H.nfast > 0 && !operand_ready(H.pf0, 0)) H.batchable = 0;
         if (H.nfast > 1 && !operand_ready(H.pf1, 1)) H.batchable = 0;
@@ -545,6 +546,46 @@ __device__ __forceinline__ void apply_epilogueQ(const epi_hoist_t &H, float (&v)
     }
 }
 
+// The e8m0 scale of a group with largest magnitude amax, and the bits of its
+// inverse, by exponent arithmetic: e8m0(x) keeps the exponent byte of x, so
+//     scale = e8m0(e8m0(amax) / e8m0(dt_max))  has the byte  ea - em + 127
+// (0 when that is below 1: the quotient is subnormal or zero; 255 for a NaN /
+// infinite amax), and 1 / scale = 2^(127 - byte), subnormal for byte 254.  The
+// same bytes and bits as the reference's two divisions
+// (ref_matmul.cpp:343-351, :381).
+__device__ __forceinline__ uint8_t mx_scale_byte(float amax, int em, float &inv) {
+    const int ea = (int)f32_to_e8m0(amax);
+    int sb = ea - em + 127;
+    sb = sb < 0 ? 0 : sb;
+    if (ea == 255) sb = 255;
+    const unsigned ib = sb == 255 ? 0x7fc00000u : sb == 254 ? 0x00400000u : (unsigned)(254 - sb) << 23;
+    inv = u2f(ib);
+    return (uint8_t)sb;
+}
+
+// Dynamic (MX) quantization of dst for NQ quads (ref_matmul.cpp:338-423): a
+// group is 32 consecutive n of one row = the quads of 8 consecutive lanes
+// (`lcol` is the lane's quad number in its row).  Writes the e8m0 scale of
+// every group and leaves v scaled and saturated, ready for the fp8 conversion.
+template <int NQ, class PT>
+__device__ __forceinline__ void dynamic_quantQ(const PT &P, const epi_hoist_t &H, float (&v)[NQ][4], long b,
+        const long (&m)[NQ], long n, const bool (&ok)[NQ], int lcol) {
+    const float dt_max = H.dst_dt == MI355_DT_F8_E4M3 ? 448.f : 57344.f;
+    const int em = (int)f32_to_e8m0(dt_max);
+#pragma unroll
+    for (int k = 0; k < NQ; ++k) {
+        float amax = fmaxf(fmaxf(fabsf(v[k][0]), fabsf(v[k][1])), fmaxf(fabsf(v[k][2]), fabsf(v[k][3])));
+        amax = fmaxf(amax, __shfl_xor(amax, 1, 64));
+        amax = fmaxf(amax, __shfl_xor(amax, 2, 64));
+        amax = fmaxf(amax, __shfl_xor(amax, 4, 64));
+        float inv;
+        const uint8_t sbyte = mx_scale_byte(amax, em, inv);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) v[k][e] = fminf(fmaxf(v[k][e] * inv, -dt_max), dt_max);
+        if (ok[k] && (lcol & 7) == 0) ((uint8_t *)P.dst_scale.p)[quant_off(P.dst_scale, b, m[k], n, P.M, P.N)] = sbyte;
+    }
+}
+
 // four full quads (nvalid == 4, vector stores allowed) to dst; `ok[k]` masks rows beyond M
 template <int NQ, class PT>
 __device__ __forceinline__ void storeQ(const PT &P, const epi_hoist_t &H, const float (&v)[NQ][4], long b,
@@ -606,6 +647,49 @@ __device__ __forceinline__ void storeQ(const PT &P, const epi_hoist_t &H, const 
         for (int k = 0; k < NQ; ++k)
 #pragma unroll
             for (int e = 0; e < 4; ++e) w[k][e] = f2u(v[k][e]);
+    } else if (dt == MI355_DT_F8_E4M3 || dt == MI355_DT_F8_E5M2) {
+        // The reference converts f32 -> f16 -> fp8, two roundings to nearest even
+        // (src/common/float8.cpp:47-126, :216-281).  v_cvt_f16_f32 followed by
+        // v_cvt_scalef32_pk_{fp8,bf8}_f16 with scale 1 does the same: checked on
+        // the device against the software conversions for every f16 bit pattern
+        // and 4 M f32 patterns, the results differ for NaN inputs only (the
+        // hardware returns one canonical NaN).  A wavefront that holds a NaN
+        // takes the software conversion.
+        bool special = false;
+#pragma unroll
+        for (int k = 0; k < NQ; ++k)
+#pragma unroll
+            for (int e = 0; e < 4; ++e) special |= __builtin_amdgcn_classf(v[k][e], 0x3);
+        if (__builtin_amdgcn_ballot_w64(special) == 0) {
+            typedef _Float16 f16x2_t __attribute__((ext_vector_type(2)));
+            typedef short s16x2_t __attribute__((ext_vector_type(2)));
+            const long off0b = b * P.ds[0] + n;
+#pragma unroll
+            for (int k = 0; k < NQ; ++k) {
+                const f16x2_t lo = {(_Float16)v[k][0], (_Float16)v[k][1]}, hi = {(_Float16)v[k][2], (_Float16)v[k][3]};
+                s16x2_t r = {0, 0};
+                if (dt == MI355_DT_F8_E4M3) {
+                    r = __builtin_amdgcn_cvt_scalef32_pk_fp8_f16(r, lo, 1.f, false);
+                    r = __builtin_amdgcn_cvt_scalef32_pk_fp8_f16(r, hi, 1.f, true);
+                } else {
+                    r = __builtin_amdgcn_cvt_scalef32_pk_bf8_f16(r, lo, 1.f, false);
+                    r = __builtin_amdgcn_cvt_scalef32_pk_bf8_f16(r, hi, 1.f, true);
+                }
+                if (ok[k]) *(uint32_t *)((uint8_t *)P.dst + off0b + m[k] * P.ds[1]) = __builtin_bit_cast(uint32_t, r);
+            }
+            return;
+        }
+        if (dt == MI355_DT_F8_E4M3) {
+#pragma unroll
+            for (int k = 0; k < NQ; ++k)
+#pragma unroll
+                for (int e = 0; e < 4; ++e) w[k][e] = f32_to_e4m3(v[k][e]);
+        } else {
+#pragma unroll
+            for (int k = 0; k < NQ; ++k)
+#pragma unroll
+                for (int e = 0; e < 4; ++e) w[k][e] = f32_to_e5m2(v[k][e]);
+        }
     } else { // s32 (nothing else is batchable)
 #pragma unroll
         for (int k = 0; k < NQ; ++k)
@@ -794,6 +878,7 @@ __device__ __forceinline__ void store_quadrant(const PT &P, char *smem, const Ac
 #pragma unroll
                 for (int k = 0; k < NQ; ++k) conv.row(raw[k], ok[k] ? m[k] : m_base, v[k]);
                 apply_epilogueQ<NQ>(H, v, sv);
+                if (H.dynamic) dynamic_quantQ<NQ>(P, H, v, b, m, nbase, ok, lcol);
                 storeQ<NQ>(P, H, v, b, m, nbase, ok);
             }
             continue;
@@ -806,7 +891,7 @@ __device__ __forceinline__ void store_quadrant(const PT &P, char *smem, const Ac
             // arithmetic and the cross-lane maximum, rows beyond M on the data of
             // a valid row; only the stores are masked.
             const float dt_max = H.dst_dt == MI355_DT_F8_E4M3 ? 448.f : 57344.f;
-            const float emax = e8m0_to_f32(f32_to_e8m0(dt_max));
+            const int em = (int)f32_to_e8m0(dt_max);
 #pragma unroll 1
             for (int it = 0; it < PASSES; ++it) {
                 const int row = it * RPP + lrow;
@@ -825,8 +910,8 @@ __device__ __forceinline__ void store_quadrant(const PT &P, char *smem, const Ac
                 amax = fmaxf(amax, __shfl_xor(amax, 1, 64));
                 amax = fmaxf(amax, __shfl_xor(amax, 2, 64));
                 amax = fmaxf(amax, __shfl_xor(amax, 4, 64));
-                const uint8_t sbyte = f32_to_e8m0(e8m0_to_f32(f32_to_e8m0(amax)) / emax);
-                const float inv = 1.f / e8m0_to_f32(sbyte);
+                float inv;
+                const uint8_t sbyte = mx_scale_byte(amax, em, inv);
 #pragma unroll
                 for (int e = 0; e < 4; ++e) v[e] = fminf(fmaxf(v[e] * inv, -dt_max), dt_max);
                 if (ok) {

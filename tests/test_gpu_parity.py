@@ -200,3 +200,52 @@ def test_bf16_dst_of_integer_gemm_is_bit_exact_including_flushed_subnormals(gpu,
     assert_bit_exact(p, got, want, name)
     if scale == 1.4e-45:
         assert np.all((want.view(np.uint16) & 0x7fff) == 0)
+
+
+@pytest.mark.parametrize("dst", ["f8_e4m3", "f8_e5m2"])
+@pytest.mark.parametrize("with_nan", [False, True])
+@pytest.mark.parametrize("dynamic", [False, True])
+def test_fp8_dst_of_the_fp8_gemm_is_bit_exact_on_exact_sums(gpu, oracle, dst, with_nan, dynamic):
+    # small-integer operands: every product and partial sum is exact in f32, so
+    # the GEMM's summation order does not matter and the fp8 conversion of the
+    # epilogue (hardware f32 -> f16 -> fp8 for wavefronts without NaNs, the
+    # software one otherwise) must reproduce the oracle bit for bit, including
+    # values beyond the range of the type (dst scale 4: |d| up to 576 > 448)
+    import numpy as np
+    from onednn_amd import dtypes as dtp
+    from onednn_amd.problem import MatmulProblem, QuantParam
+    M, N, K = 300, 320, 256
+    r = np.random.default_rng(9)
+    src = dtp.f32_to_e4m3(r.integers(-3, 4, size=(M, K)).astype(np.float32).reshape(-1))
+    wei = dtp.f32_to_e4m3(r.integers(-3, 4, size=(N, K)).astype(np.float32).reshape(-1))   # K-contiguous (ba)
+    bias = (r.integers(-64, 65, size=N) / 16.0).astype(np.float32)
+    if with_nan:
+        bias[5] = np.nan
+    dst_dt = cabi.DT_F8_E4M3 if dst == "f8_e4m3" else cabi.DT_F8_E5M2
+    p = MatmulProblem(M=M, N=N, K=K, src_dt=cabi.DT_F8_E4M3, wei_dt=cabi.DT_F8_E4M3, dst_dt=dst_dt, src=src, wei=wei,
+                      wei_stride=(K * N, 1, K), bias_dt=cabi.DT_F32, bias=bias,
+                      quant={"dst_scale": QuantParam(cabi.DT_F32, 0, np.array([4.0 if dst == "f8_e4m3" else 0.03125], np.float32))},
+                      name=f"f8-exact-{dst}")
+    if dynamic:
+        # the same values through the dynamic (MX) quantization: exact sums give the
+        # GEMM tile and the oracle the same group maxima, so scales and dst agree
+        # bit for bit (rows with the NaN column have a NaN maximum: scale byte 255)
+        from onednn_amd.problem import GpuRun
+        from oracle import binding as orc
+        p.quant["dst_scale"] = QuantParam(cabi.DT_E8M0, 6, np.zeros((1, M, N // 32), np.uint8), (1, 32))
+        p.dst_dynamic = cabi.DST_DYNAMIC_MX
+        run = GpuRun(p, cabi.IMPL_F8_MFMA)
+        try:
+            run.launch()
+            got, sc = run.result(), run.dynamic_scales()
+        finally:
+            run.free()
+        want, want_sc = orc.run_oracle_dynamic(p)
+        assert np.array_equal(np.asarray(sc).reshape(-1), np.asarray(want_sc).reshape(-1))
+        assert np.array_equal(np.asarray(got).view(np.uint8), np.asarray(want).view(np.uint8))
+        return
+    got, name = run_gpu(p, cabi.IMPL_F8_MFMA)
+    want = oracle.run_oracle(p)
+    assert_bit_exact(p, got, want, name)
+    codes = np.asarray(got).view(np.uint8)
+    assert len(np.unique(codes)) > 60           # the conversion is exercised over a large part of the code space
