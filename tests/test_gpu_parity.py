@@ -249,3 +249,15 @@ def test_fp8_dst_of_the_fp8_gemm_is_bit_exact_on_exact_sums(gpu, oracle, dst, wi
     assert_bit_exact(p, got, want, name)
     codes = np.asarray(got).view(np.uint8)
     assert len(np.unique(codes)) > 60           # the conversion is exercised over a large part of the code space
+
+
+def test_hardware_fp8_conversions_match_the_software_ones_except_for_nans(gpu):
+    # the calibration tool walks every f16 bit pattern through the hardware
+    # f16 -> e4m3 / e5m2 conversions and 4 M f32 patterns through f32 -> f16 and
+    # compares with the software conversions the oracle's restatement is pinned to
+    import os
+    import subprocess
+    tool = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "onednn_amd", "lib", "cvt_fp8_check")
+    out = subprocess.run([tool], capture_output=True, text=True, timeout=120)
+    assert out.returncode == 0, out.stderr
+    assert out.stdout.strip().splitlines()[-1] == "nan-only", out.stdout[-2000:]
