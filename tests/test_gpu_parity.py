@@ -229,7 +229,8 @@ def test_fp8_dst_of_the_fp8_gemm_is_bit_exact_on_exact_sums(gpu, oracle, dst, wi
     if dynamic:
         # the same values through the dynamic (MX) quantization: exact sums give the
         # GEMM tile and the oracle the same group maxima, so scales and dst agree
-        # bit for bit (rows with the NaN column have a NaN maximum: scale byte 255)
+        # bit for bit (a NaN does not enter the group maximum, as with the reference's
+        # std::max, and converts to the NaN code of the type)
         from onednn_amd.problem import GpuRun
         from oracle import binding as orc
         p.quant["dst_scale"] = QuantParam(cabi.DT_E8M0, 6, np.zeros((1, M, N // 32), np.uint8), (1, 32))
