@@ -99,6 +99,16 @@ def build_problem(name, M=None, wtag="any"):
         return configs.config3(wtag=mfma_tag)
     if name == "c4":
         return configs.config4(wtag=mfma_tag)
+    if name == "c4mx":
+        # C4 with an MXFP8 dst: e4m3 values and e8m0 scales per 32 columns, computed and written by the matmul
+        import numpy as np
+        from onednn_amd.problem import QuantParam
+        p = configs.config4(wtag=mfma_tag)
+        p.dst_dt = cabi.DT_F8_E4M3
+        p.quant["dst_scale"] = QuantParam(cabi.DT_E8M0, 6, np.zeros((1, p.M, p.N // 32), np.uint8), (1, 32))
+        p.dst_dynamic = cabi.DST_DYNAMIC_MX
+        p.name = "C4-dynamic-mx-dst"
+        return p
     if name == "c5":
         return configs.config5(wtag=mfma_tag)
     raise ValueError(name)
@@ -112,7 +122,7 @@ def algorithmic(name, p):
         return configs.config2_bytes(p.M, p.N, p.K), "GB/s", "hbm", PEAK_HBM_GBS
     if name == "c3":
         return ops, "TOPS", "mfma", PEAK_I8_TOPS
-    if name == "c4":
+    if name in ("c4", "c4mx"):
         return ops, "TFLOP/s", "mfma", PEAK_F8_TFLOPS
     if name == "c5":
         return ops, "TFLOP/s", "mfma", PEAK_F4_TFLOPS
@@ -328,7 +338,7 @@ def main():
 
     others = []
     if not args.no_others:
-        plan = [("c2", 1), ("c2", 8), ("c2", 32), ("c3", None), ("c4", None), ("c5", None),
+        plan = [("c2", 1), ("c2", 8), ("c2", 32), ("c3", None), ("c4", None), ("c4mx", None), ("c5", None),
                 ("c1", None)]
         for nm, m in plan:
             if nm == main_name and (nm != "c2" or m == args.decode_m):
