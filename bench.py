@@ -45,6 +45,7 @@ MEASURED_TRAFFIC = {
     ("c2", 1): 31612633, ("c2", 8): 32271601, ("c2", 32): 34542741,        # packed weights (format any)
     ("c2ab", 1): 32839597, ("c2ab", 8): 35736697, ("c2ab", 32): 51670775,  # plain ab weights (--wtag ab)
     ("c1", 256): 8645444,
+    ("r1", 0): 335981182, ("r2", 0): 212392274, ("r3", 0): 58765379,
 }
 
 # MI355X published peaks
@@ -310,7 +311,8 @@ def main():
             "vs_baseline": None, "dtype": {"r1": "f32", "r2": "s8", "r3": "u4"}[main_name], "data": "synthetic",
             "config": {"workload": r["workload"], "impl": r["impl"]},
             "roofline": {"bound": "hbm", "achieved": r["value"], "peak": PEAK_HBM_GBS, "unit": "GB/s",
-                         "frac": r["frac_of_peak"], "traffic": None, "algorithmic": r["work"],
+                         "frac": r["frac_of_peak"], "traffic": MEASURED_TRAFFIC.get((main_name, 0)),
+                         "algorithmic": r["work"],
                          "kernel": r["impl"], "kernel_ms": r["ms_per_step"]},
             "cpu_baseline": None, "others": []}), flush=True)
         return
