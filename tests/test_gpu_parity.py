@@ -262,3 +262,31 @@ def test_hardware_fp8_conversions_match_the_software_ones_except_for_nans(gpu):
     out = subprocess.run([tool], capture_output=True, text=True, timeout=120)
     assert out.returncode == 0, out.stderr
     assert out.stdout.strip().splitlines()[-1] == "nan-only", out.stdout[-2000:]
+
+
+@pytest.mark.parametrize("with_nan_inf", [False, True])
+def test_f16_dst_of_integer_gemm_is_bit_exact(gpu, oracle, with_nan_inf):
+    # integer accumulation is exact, so the f16 conversion of the batched tile
+    # epilogue (hardware v_cvt_f16_f32) must equal the oracle's software
+    # conversion bit for bit: normal values, f16 subnormals (tiny dst scale
+    # inverse), overflow to infinity, and NaN / infinite inputs through the bias
+    import numpy as np
+    from onednn_amd.problem import QuantParam
+    p = configs.config3(M=300, N=320, K=512, wtag="ba")
+    p.dst_dt = cabi.DT_F16
+    p.post_ops = []
+    N = p.N
+    # per-column scales spread over 40 binades: columns land in f16's subnormal, normal and overflow ranges
+    sc = np.exp2(np.random.default_rng(3).uniform(-34, 6, size=N)).astype(np.float32)
+    p.quant["wei_scale"] = QuantParam(cabi.DT_F32, configs.MASK_COL, sc)
+    p.quant.pop("dst_scale")
+    if with_nan_inf:
+        bias = np.zeros(N, np.float32)
+        bias[3], bias[40], bias[77] = np.nan, np.inf, -np.inf
+        p.bias_dt, p.bias = cabi.DT_F32, bias
+    got, name = run_gpu(p, cabi.IMPL_I8_MFMA)
+    want = oracle.run_oracle(p)
+    assert_bit_exact(p, got, want, name)
+    h = np.asarray(got).view(np.uint16)
+    e = (h >> 10) & 0x1f
+    assert np.any((e == 0) & ((h & 0x3ff) != 0)) and np.any(e == 0x1f) and np.any((e > 0) & (e < 0x1f))
