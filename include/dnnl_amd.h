@@ -59,6 +59,7 @@ typedef enum {
 typedef int64_t dnnl_dim_t;                /* dnnl_common_types.h:126 */
 typedef dnnl_dim_t dnnl_dims_t[DNNL_MAX_NDIMS];
 #define DNNL_RUNTIME_DIM_VAL INT64_MIN     /* dnnl_types.h:2331 */
+#define DNNL_RUNTIME_SIZE_VAL ((size_t)DNNL_RUNTIME_DIM_VAL) /* dnnl_types.h:2336 */
 
 /* dnnl_common_types.h:137-148 */
 typedef enum {

@@ -34,6 +34,8 @@ ARG_ATTR_PRECOMPUTED_REDUCTIONS, ARG_ATTR_SCALES, ARG_ATTR_ZERO_POINTS = 512, 40
 scratchpad_library, scratchpad_user = 0, 1
 fpmath_strict, fpmath_bf16, fpmath_f16, fpmath_any = 0, 1, 2, 3
 MEMORY_ALLOCATE = C.c_void_p(-1 & (2 ** 64 - 1))
+RUNTIME_DIM_VAL = -(2 ** 63)           # DNNL_RUNTIME_DIM_VAL, dnnl_types.h:2331
+RUNTIME_SIZE_VAL = 2 ** 63             # DNNL_RUNTIME_SIZE_VAL, dnnl_types.h:2336
 
 
 def ARG_ATTR_MULTIPLE_POST_OP(idx):

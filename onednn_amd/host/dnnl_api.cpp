@@ -105,6 +105,12 @@ struct dnnl_memory_desc {
     int packing = 0;
 
     bool is_zero() const { return ndims == 0; }
+    // a dim or a stride left open until execution (memory_desc_wrapper::has_runtime_dims_or_strides)
+    bool has_runtime() const {
+        for (int i = 0; i < ndims; ++i)
+            if (dims[i] == DNNL_RUNTIME_DIM_VAL || (kind == dnnl_blocked && strides[i] == DNNL_RUNTIME_DIM_VAL)) return true;
+        return false;
+    }
     dim_t nelems() const {
         if (ndims == 0) return 0;
         dim_t n = 1;
@@ -119,15 +125,23 @@ struct dnnl_memory_desc {
         return off + 1;
     }
     size_t size_bytes() const {
+        if (has_runtime()) return DNNL_RUNTIME_SIZE_VAL; // memory_desc_wrapper::size, src/common/memory.cpp:62
         if (kind == dnnl_format_kind_opaque) return (size_t)nelems() * dt_bits(dt) / 8; // dense, no padding
         const dim_t s = span();
         return dt_bits(dt) == 4 ? (size_t)(s + 1) / 2 : (size_t)s * (dt_bits(dt) / 8);
     }
-    void set_dense() {
+    // dense strides in the given order of dims (perm[ndims-1] innermost); a
+    // stride outside a runtime dim is a runtime value itself
+    // (memory_desc_init_by_strides, src/common/memory_desc.cpp:298-308, :838-845)
+    void set_dense(const int *perm = nullptr) {
         dim_t s = 1;
         for (int i = ndims - 1; i >= 0; --i) {
-            strides[i] = s;
-            s *= dims[i] == 0 ? 1 : dims[i];
+            const int d = perm ? perm[i] : i;
+            strides[d] = s;
+            if (s == DNNL_RUNTIME_DIM_VAL || dims[d] == DNNL_RUNTIME_DIM_VAL)
+                s = DNNL_RUNTIME_DIM_VAL;
+            else
+                s *= dims[d] == 0 ? 1 : dims[d];
         }
         kind = dnnl_blocked;
     }
@@ -198,12 +212,23 @@ struct dnnl_primitive_desc {
     size_t impl_pos = 0;
     size_t scratch_bytes = 0;
     std::string impl_name;
+    // some dim or stride is DNNL_RUNTIME_DIM_VAL: the descriptor is validated
+    // as far as the known values allow, and lowered and dispatched at each
+    // execution from the descriptors of the memory objects
+    // (exec_ctx_t::memory_mdw, src/common/primitive_exec_types.hpp:112-186)
+    bool runtime = false;
 };
 
 struct dnnl_primitive {
     dnnl_primitive_desc pd;
     void *scratch = nullptr; // library-mode scratchpad (device)
     std::mutex scratch_mutex;
+    // runtime dims: the lowering of the last executed shapes, and the scratch
+    // buffers allocated for executions so far (kept until the primitive is
+    // destroyed: earlier launches may still be running on their stream)
+    std::unique_ptr<dnnl_primitive_desc> rt_pd;
+    std::vector<void *> rt_scratch;
+    size_t rt_scratch_bytes = 0;
 };
 
 namespace {
@@ -236,6 +261,13 @@ dnnl_status_t check_shapes(const dnnl_memory_desc &s, const dnnl_memory_desc &w,
     }
     for (int i = 0; i < nd - 2; ++i) {
         const dim_t sd = s.dims[i], wd = w.dims[i], dd = d.dims[i];
+        const dim_t R = DNNL_RUNTIME_DIM_VAL;
+        if (sd == R || wd == R || dd == R || (b && b->dims[i] == R)) {
+            // a runtime batch dim is runtime in every tensor that has it (matmul.cpp:716-721)
+            CHECK_ARG(sd == R && wd == R && dd == R);
+            if (b) CHECK_ARG(b->dims[i] == 1 || b->dims[i] == R);
+            continue;
+        }
         const bool all_eq = sd == wd && wd == dd;
         CHECK_ARG(IMPLICATION(!all_eq, sd == 1 || wd == 1));
         CHECK_ARG(IMPLICATION(sd == 1, dd == wd));
@@ -252,6 +284,12 @@ int accum_dt(int src, int wei, int dst) {
     if (src == dnnl_f64) return dnnl_f64;
     return dnnl_f32;
 }
+
+// Stand-in for a runtime dim while the attributes of a descriptor with runtime
+// dims are checked at creation: divisible by every power-of-two group, like
+// DNNL_RUNTIME_DIM_VAL itself in the reference's checks.  The checks run again
+// on the real dims at execution.
+const dim_t k_probe_dim = (dim_t)1 << 40;
 
 // matmul_attr_check (src/common/matmul.cpp:261-624) plus the generic checks of
 // matmul_pd_t::attr_scales_ok / attr_zero_points_ok (matmul_pd.hpp:209-397)
@@ -394,7 +432,8 @@ dnnl_status_t check_attr(const dnnl_memory_desc &s, const dnnl_memory_desc &w, c
         }
         if (e.kind == dnnl_binary) {
             CHECK_ARG(e.src1.ndims == d.ndims);
-            for (int i = 0; i < d.ndims; ++i) CHECK_ARG(e.src1.dims[i] == 1 || e.src1.dims[i] == d.dims[i]);
+            for (int i = 0; i < d.ndims; ++i)
+                CHECK_ARG(e.src1.dims[i] == 1 || e.src1.dims[i] == d.dims[i] || d.dims[i] == k_probe_dim);
         }
     }
     CHECK_UNIMPL(n_sum <= 1 || true);
@@ -554,6 +593,100 @@ dnnl_status_t select_impl(dnnl_primitive_desc &pd) {
     return dnnl_success;
 }
 
+// data type combinations of the reference's two naive implementations
+// (ref_matmul.hpp:44-123, ref_matmul_int8.hpp:44-92)
+dnnl_status_t check_dtypes(const dnnl_primitive_desc &pd) {
+    {
+        const int s = pd.src.dt, w = pd.wei.dt, d = pd.dst.dt;
+        const bool int_path = is_int8(s);
+        if (int_path) {
+            CHECK_UNIMPL(is_int8(w) || w == dnnl_s4 || w == dnnl_u4);
+            CHECK_UNIMPL(d == dnnl_f32 || d == dnnl_bf16 || d == dnnl_f16 || d == dnnl_s32 || is_int8(d));
+            if (pd.with_bias) CHECK_UNIMPL(pd.bias.dt == dnnl_f32 || pd.bias.dt == dnnl_bf16 || pd.bias.dt == dnnl_f16
+                    || pd.bias.dt == dnnl_s32 || is_int8(pd.bias.dt));
+        } else {
+            CHECK_UNIMPL(s == dnnl_f32 || s == dnnl_bf16 || s == dnnl_f16 || is_fp8(s) || s == dnnl_f4_e2m1);
+            CHECK_UNIMPL(w == dnnl_f32 || w == dnnl_bf16 || w == dnnl_f16 || is_fp8(w) || w == dnnl_f4_e2m1
+                    || is_int8(w) || w == dnnl_s4 || w == dnnl_u4);
+            CHECK_UNIMPL(s == w || w == dnnl_bf16 || w == dnnl_f16 || is_fp8(w) || is_int8(w) || w == dnnl_s4
+                    || w == dnnl_u4);
+            // integer weights under a floating-point src only as weight decompression
+            CHECK_UNIMPL(IMPLICATION(is_int8(w) || w == dnnl_s4 || w == dnnl_u4, pd.attr.apply_to_int));
+            CHECK_UNIMPL(d == dnnl_f32 || d == dnnl_bf16 || d == dnnl_f16 || is_fp8(d) || is_int8(d));
+            if (pd.with_bias) CHECK_UNIMPL(pd.bias.dt == dnnl_f32 || pd.bias.dt == dnnl_bf16 || pd.bias.dt == dnnl_f16 || is_fp8(pd.bias.dt));
+        }
+    }
+    return dnnl_success;
+}
+
+// lowers the descriptor and lists the kernel families that take it, best first
+dnnl_status_t dispatch(dnnl_primitive_desc &pd) {
+    dnnl_status_t st = lower(pd);
+    if (st) return st;
+    pd.impls.clear();
+    for (int impl : k_impl_list) {
+        int chosen = 0;
+        if (mi355_matmul_query(&pd.desc, impl, &chosen) == MI355_SUCCESS) pd.impls.push_back(impl);
+    }
+    if (pd.impls.empty()) return dnnl_unimplemented;
+    pd.impl_pos = 0;
+    return select_impl(pd);
+}
+
+// Runtime dims: the descriptor of this execution.  A tensor whose descriptor
+// was created with runtime values takes the descriptor of its memory object
+// (exec_ctx_t::memory_mdw, src/common/primitive_exec_types.hpp:112-186), which
+// has to agree with every value that was known; then the checks that were
+// left open at creation run, the descriptor is lowered and the kernel family
+// is chosen.  The result is kept for the next execution with the same shapes.
+dnnl_status_t concretize(dnnl_primitive &prim, const std::map<int, dnnl_memory_t> &m, void **scratch) {
+    const dnnl_primitive_desc &pd0 = prim.pd;
+    std::unique_ptr<dnnl_primitive_desc> c(new dnnl_primitive_desc(pd0));
+    c->runtime = false;
+    struct slot_t {
+        int arg;
+        const dnnl_memory_desc *from;
+        dnnl_memory_desc *to;
+        bool present;
+    } slots[] = {{DNNL_ARG_SRC, &pd0.src, &c->src, true}, {DNNL_ARG_WEIGHTS, &pd0.wei, &c->wei, true},
+            {DNNL_ARG_DST, &pd0.dst, &c->dst, true}, {DNNL_ARG_BIAS, &pd0.bias, &c->bias, pd0.with_bias}};
+    for (const slot_t &sl : slots) {
+        if (!sl.present || !sl.from->has_runtime()) continue;
+        auto it = m.find(sl.arg);
+        CHECK_ARG(it != m.end() && it->second);
+        const dnnl_memory_desc &mm = it->second->md;
+        CHECK_ARG(mm.kind == dnnl_blocked && mm.ndims == sl.from->ndims && mm.dt == sl.from->dt);
+        for (int i = 0; i < mm.ndims; ++i) {
+            CHECK_ARG(sl.from->dims[i] == DNNL_RUNTIME_DIM_VAL || sl.from->dims[i] == mm.dims[i]);
+            CHECK_ARG(sl.from->strides[i] == DNNL_RUNTIME_DIM_VAL || sl.from->strides[i] == mm.strides[i]
+                    || mm.dims[i] <= 1);
+        }
+        *sl.to = mm;
+    }
+    const bool same = prim.rt_pd && prim.rt_pd->src == c->src && prim.rt_pd->wei == c->wei && prim.rt_pd->dst == c->dst
+            && (!pd0.with_bias || prim.rt_pd->bias == c->bias);
+    if (!same) {
+        dnnl_status_t st = check_shapes(c->src, c->wei, pd0.with_bias ? &c->bias : nullptr, c->dst);
+        if (st) return st;
+        st = check_attr(c->src, c->wei, c->dst, c->attr);
+        if (st) return st;
+        st = dispatch(*c);
+        if (st) return st;
+        prim.rt_pd = std::move(c);
+    }
+    const size_t need = prim.rt_pd->scratch_bytes;
+    if (need > prim.rt_scratch_bytes) {
+        if (mi355_device_set((int)pd0.engine->index) != MI355_SUCCESS) return dnnl_runtime_error;
+        void *q = nullptr;
+        const int st = mi355_mem_alloc(&q, need);
+        if (st != MI355_SUCCESS) return from_mi355(st);
+        prim.rt_scratch.push_back(q);
+        prim.rt_scratch_bytes = need;
+    }
+    *scratch = prim.rt_scratch.empty() ? nullptr : prim.rt_scratch.back();
+    return dnnl_success;
+}
+
 } // namespace
 
 // ================================================================ C API
@@ -622,8 +755,7 @@ static dnnl_status_t md_common(dnnl_memory_desc &md, int ndims, const dnnl_dims_
     md.ndims = ndims;
     md.dt = dt;
     for (int i = 0; i < ndims; ++i) {
-        if (dims[i] == DNNL_RUNTIME_DIM_VAL) return dnnl_unimplemented; // runtime dims are not offered
-        CHECK_ARG(dims[i] >= 0);
+        CHECK_ARG(dims[i] >= 0 || dims[i] == DNNL_RUNTIME_DIM_VAL);
         md.dims[i] = dims[i];
     }
     return dnnl_success;
@@ -638,7 +770,7 @@ DNNL_EXPORT dnnl_status_t dnnl_memory_desc_create_with_strides(dnnl_memory_desc_
         md->set_dense();
     } else {
         for (int i = 0; i < ndims; ++i) {
-            CHECK_ARG(strides[i] >= 0);
+            CHECK_ARG(strides[i] >= 0 || strides[i] == DNNL_RUNTIME_DIM_VAL);
             md->strides[i] = strides[i];
         }
         md->kind = dnnl_blocked;
@@ -662,7 +794,12 @@ DNNL_EXPORT dnnl_status_t dnnl_memory_desc_create_with_tag(dnnl_memory_desc_t *m
     int perm[DNNL_MAX_NDIMS];
     for (int i = 0; i < ndims; ++i) perm[i] = i;
     switch (tag) {
-        case dnnl_format_tag_any: md->kind = dnnl_format_kind_any; *memory_desc = md.release(); return dnnl_success;
+        case dnnl_format_tag_any:
+            // no layout can be picked for dims that are not known (memory_desc.cpp:70-72)
+            for (int i = 0; i < ndims; ++i) CHECK_ARG(dims[i] != DNNL_RUNTIME_DIM_VAL);
+            md->kind = dnnl_format_kind_any;
+            *memory_desc = md.release();
+            return dnnl_success;
         case dnnl_a: CHECK_ARG(ndims == 1); break;
         case dnnl_ab: CHECK_ARG(ndims == 2); break;
         case dnnl_abc: CHECK_ARG(ndims == 3); break;
@@ -672,12 +809,7 @@ DNNL_EXPORT dnnl_status_t dnnl_memory_desc_create_with_tag(dnnl_memory_desc_t *m
         case dnnl_abdc: CHECK_ARG(ndims == 4); perm[2] = 3; perm[3] = 2; break;
         default: return dnnl_unimplemented; // blocked layouts are not offered
     }
-    dim_t s = 1;
-    for (int i = ndims - 1; i >= 0; --i) {
-        md->strides[perm[i]] = s;
-        s *= md->dims[perm[i]] == 0 ? 1 : md->dims[perm[i]];
-    }
-    md->kind = dnnl_blocked;
+    md->set_dense(perm);
     *memory_desc = md.release();
     return dnnl_success;
 }
@@ -723,6 +855,7 @@ DNNL_EXPORT dnnl_status_t dnnl_memory_create(dnnl_memory_t *memory, const_dnnl_m
         dnnl_engine_t engine, void *handle) {
     CHECK_ARG(memory && md && engine);
     CHECK_ARG(md->kind != dnnl_format_kind_any);
+    CHECK_ARG(!md->has_runtime()); // src/common/memory.cpp:155
     std::unique_ptr<dnnl_memory> m(new dnnl_memory);
     m->md = *md;
     m->engine = engine;
@@ -1045,7 +1178,20 @@ DNNL_EXPORT dnnl_status_t dnnl_matmul_primitive_desc_create(dnnl_primitive_desc_
     CHECK_ARG(accum_dt(src_desc->dt, weights_desc->dt, dst_desc->dt) != dnnl_data_type_undef);
     std::unique_ptr<dnnl_primitive_desc> pd(new dnnl_primitive_desc);
     if (attr) pd->attr = *attr;
-    st = check_attr(*src_desc, *weights_desc, *dst_desc, pd->attr);
+    pd->runtime = src_desc->has_runtime() || weights_desc->has_runtime() || dst_desc->has_runtime()
+            || (bias && bias->has_runtime());
+    if (pd->runtime) {
+        // attribute rules that involve an unknown dim are checked at execution
+        dnnl_memory_desc ps = *src_desc, pw = *weights_desc, pdst = *dst_desc;
+        for (dnnl_memory_desc *m : {&ps, &pw, &pdst})
+            for (int i = 0; i < m->ndims; ++i)
+                if (m->dims[i] == DNNL_RUNTIME_DIM_VAL) m->dims[i] = k_probe_dim;
+        st = check_attr(ps, pw, pdst, pd->attr);
+        for (const post_op_entry_t &e : pd->attr.post_ops.entries)
+            if (e.kind == dnnl_binary) CHECK_UNIMPL(!e.src1.has_runtime());
+    } else {
+        st = check_attr(*src_desc, *weights_desc, *dst_desc, pd->attr);
+    }
     if (st) return st;
     pd->engine = engine;
     pd->src = *src_desc; pd->wei = *weights_desc; pd->dst = *dst_desc;
@@ -1075,27 +1221,18 @@ DNNL_EXPORT dnnl_status_t dnnl_matmul_primitive_desc_create(dnnl_primitive_desc_
     }
     for (dnnl_memory_desc *m : {&pd->src, &pd->dst, &pd->bias})
         if (m->kind == dnnl_format_kind_any) m->set_dense();
-    // data type combinations of the reference's two naive implementations
-    // (ref_matmul.hpp:44-123, ref_matmul_int8.hpp:44-92)
-    {
-        const int s = pd->src.dt, w = pd->wei.dt, d = pd->dst.dt;
-        const bool int_path = is_int8(s);
-        if (int_path) {
-            CHECK_UNIMPL(is_int8(w) || w == dnnl_s4 || w == dnnl_u4);
-            CHECK_UNIMPL(d == dnnl_f32 || d == dnnl_bf16 || d == dnnl_f16 || d == dnnl_s32 || is_int8(d));
-            if (bias) CHECK_UNIMPL(bias->dt == dnnl_f32 || bias->dt == dnnl_bf16 || bias->dt == dnnl_f16
-                    || bias->dt == dnnl_s32 || is_int8(bias->dt));
-        } else {
-            CHECK_UNIMPL(s == dnnl_f32 || s == dnnl_bf16 || s == dnnl_f16 || is_fp8(s) || s == dnnl_f4_e2m1);
-            CHECK_UNIMPL(w == dnnl_f32 || w == dnnl_bf16 || w == dnnl_f16 || is_fp8(w) || w == dnnl_f4_e2m1
-                    || is_int8(w) || w == dnnl_s4 || w == dnnl_u4);
-            CHECK_UNIMPL(s == w || w == dnnl_bf16 || w == dnnl_f16 || is_fp8(w) || is_int8(w) || w == dnnl_s4
-                    || w == dnnl_u4);
-            // integer weights under a floating-point src only as weight decompression
-            CHECK_UNIMPL(IMPLICATION(is_int8(w) || w == dnnl_s4 || w == dnnl_u4, pd->attr.apply_to_int));
-            CHECK_UNIMPL(d == dnnl_f32 || d == dnnl_bf16 || d == dnnl_f16 || is_fp8(d) || is_int8(d));
-            if (bias) CHECK_UNIMPL(bias->dt == dnnl_f32 || bias->dt == dnnl_bf16 || bias->dt == dnnl_f16 || is_fp8(bias->dt));
-        }
+    st = check_dtypes(*pd);
+    if (st) return st;
+    if (pd->runtime) {
+        // the kernel family is chosen per execution, from the real shapes
+        pd->impls.assign(1, MI355_IMPL_AUTO);
+        pd->impl_pos = 0;
+        pd->impl_name = "hip:runtime_dims:any";
+        pd->desc.impl = MI355_IMPL_AUTO;
+        if (verbose_level() >= 1)
+            fprintf(stderr, "onednn_verbose,v1,primitive,create:dispatch,gpu,matmul,%s\n", pd->impl_name.c_str());
+        *primitive_desc = pd.release();
+        return dnnl_success;
     }
     if (try_packed) {
         const dnnl_memory_desc plain = pd->wei;
@@ -1107,15 +1244,7 @@ DNNL_EXPORT dnnl_status_t dnnl_matmul_primitive_desc_create(dnnl_primitive_desc_
                 || mi355_matmul_query(&pd->desc, MI355_IMPL_WOQ_PACKED, &chosen) != MI355_SUCCESS)
             pd->wei = plain;
     }
-    st = lower(*pd);
-    if (st) return st;
-    for (int impl : k_impl_list) {
-        int chosen = 0;
-        if (mi355_matmul_query(&pd->desc, impl, &chosen) == MI355_SUCCESS) pd->impls.push_back(impl);
-    }
-    if (pd->impls.empty()) return dnnl_unimplemented;
-    pd->impl_pos = 0;
-    st = select_impl(*pd);
+    st = dispatch(*pd);
     if (st) return st;
     if (verbose_level() >= 1)
         fprintf(stderr, "onednn_verbose,v1,primitive,create:dispatch,gpu,matmul,%s\n", pd->impl_name.c_str());
@@ -1135,6 +1264,7 @@ DNNL_EXPORT dnnl_status_t dnnl_reorder_primitive_desc_create(dnnl_primitive_desc
     CHECK_ARG(src_desc->ndims == dst_desc->ndims && src_desc->ndims >= 1);
     for (int i = 0; i < src_desc->ndims; ++i) CHECK_ARG(src_desc->dims[i] == dst_desc->dims[i]);
     CHECK_UNIMPL(src_desc->ndims <= MI355_REORDER_MAX_DIMS);
+    CHECK_UNIMPL(!src_desc->has_runtime() && !dst_desc->has_runtime()); // runtime dims: matmul only
     // opaque (packed) weights: written by a reorder from plain weights of the
     // same data type; reading them back is not offered
     CHECK_UNIMPL(src_desc->kind == dnnl_blocked);
@@ -1319,6 +1449,7 @@ DNNL_EXPORT dnnl_status_t dnnl_primitive_get_primitive_desc(const_dnnl_primitive
 DNNL_EXPORT dnnl_status_t dnnl_primitive_destroy(dnnl_primitive_t primitive) {
     if (primitive) {
         if (primitive->scratch) mi355_mem_free(primitive->scratch);
+        for (void *q : primitive->rt_scratch) mi355_mem_free(q);
         delete primitive;
     }
     return dnnl_success;
@@ -1329,13 +1460,23 @@ DNNL_EXPORT dnnl_status_t dnnl_primitive_execute(const_dnnl_primitive_t cprimiti
     CHECK_ARG(cprimitive && stream);
     CHECK_ARG(nargs >= 0 && IMPLICATION(nargs > 0, args));
     dnnl_primitive *prim = const_cast<dnnl_primitive *>(cprimitive);
-    const dnnl_primitive_desc &pd = prim->pd;
-    CHECK_ARG(stream->engine == pd.engine || stream->engine->index == pd.engine->index);
+    const dnnl_primitive_desc &pd0 = prim->pd;
+    CHECK_ARG(stream->engine == pd0.engine || stream->engine->index == pd0.engine->index);
     std::map<int, dnnl_memory_t> m;
     for (int i = 0; i < nargs; ++i) {
         CHECK_ARG(m.find(args[i].arg) == m.end()); // duplicated argument
         m[args[i].arg] = args[i].memory;
     }
+    std::unique_lock<std::mutex> lock(prim->scratch_mutex, std::defer_lock);
+    void *rt_scratch = nullptr;
+    if (pd0.runtime) {
+        // executions of one primitive with runtime dims are serialised on the
+        // host while they enqueue: they share the cached lowering and scratch
+        lock.lock();
+        dnnl_status_t rs = concretize(*prim, m, &rt_scratch);
+        if (rs) return rs;
+    }
+    const dnnl_primitive_desc &pd = pd0.runtime ? *prim->rt_pd : pd0;
     auto handle = [&](int arg, bool required, void **out) -> dnnl_status_t {
         auto it = m.find(arg);
         if (it == m.end() || !it->second) {
@@ -1409,8 +1550,9 @@ DNNL_EXPORT dnnl_status_t dnnl_primitive_execute(const_dnnl_primitive_t cprimiti
     if (!A.src || !A.wei || !A.dst) return dnnl_invalid_arguments;
 
     void *scratch = prim->scratch;
-    std::unique_lock<std::mutex> lock(prim->scratch_mutex, std::defer_lock);
-    if (pd.attr.scratchpad_mode == dnnl_scratchpad_mode_user) {
+    if (pd0.runtime) {
+        scratch = rt_scratch;
+    } else if (pd.attr.scratchpad_mode == dnnl_scratchpad_mode_user) {
         if ((st = handle(DNNL_ARG_SCRATCHPAD, pd.scratch_bytes > 0, &scratch))) return st;
     } else if (scratch) {
         // the library-mode scratchpad belongs to the primitive: executions of

@@ -94,6 +94,8 @@ class Spec:
         for knob in ("attr_scales", "attr_zero_points", "attr_post_ops", "attr_fpmath"):
             if getattr(self, knob):
                 parts.append(f"--{knob.replace('_', '-')}={getattr(self, knob)}")
+        if self.runtime_dims_masks:
+            parts.append(f"--runtime_dims_masks={self.runtime_dims_masks}")
         if self.impl:
             parts.append(f"--impl={self.impl}")
         parts.append(self.desc)
@@ -104,7 +106,7 @@ def parse(argv):
     """benchdnn-style arguments -> (mode, [Spec, ...])."""
     knobs = {"dt": ["f32"], "stag": ["ab"], "wtag": ["ab"], "dtag": ["ab"], "bia_dt": ["undef"],
              "attr_scales": [""], "attr_zero_points": [""], "attr_post_ops": [""], "attr_fpmath": [""],
-             "impl": [""]}
+             "runtime_dims_masks": [""], "impl": [""]}
     mode, specs = "C", []
     for a in argv:
         if a in ("--matmul", "--reset"):
@@ -229,10 +231,35 @@ def build_problem(sp, seed=7):
                          impl=impl, name=sp.desc, **kw)
 
 
-def api_objects(p, want_ref_impl=False):
+def runtime_masks(text):
+    """--runtime_dims_masks=[SRC][:WEI] -> (src, wei, dst) bit masks over (rows, cols);
+    the dst mask follows: M from src, N from weights."""
+    if not text:
+        return 0, 0, 0
+    a, _, b = text.partition(":")
+    sm, wm = int(a or 0), int(b or 0)
+    if (sm >> 1) & 1 != wm & 1:
+        raise ValueError("K is a runtime dim in one of src / weights only")
+    return sm, wm, (sm & 1) | (wm & 2)
+
+
+def _pd_md(dims, dt, strides, mask):
+    """The descriptor handed to the primitive descriptor: dims under `mask`
+    are DNNL_RUNTIME_DIM_VAL, and so is every stride that is a product of one."""
+    if not mask:
+        return dnnl.memory_desc(list(dims), dt, strides=list(strides))
+    R = dnnl.RUNTIME_DIM_VAL
+    rt = [bool(mask >> i & 1) for i in range(len(dims))]
+    st = [R if any(rt[j] and j != i and strides[j] < strides[i] for j in range(len(dims))) else strides[i]
+          for i in range(len(dims))]
+    return dnnl.memory_desc([R if rt[i] else dims[i] for i in range(len(dims))], dt, strides=st)
+
+
+def api_objects(p, want_ref_impl=False, runtime_dims_masks=""):
     """MatmulProblem -> dnnl engine, primitive and execute arguments (2-D, dense)."""
     eng = dnnl.engine(dnnl.gpu, 0)
     strm = dnnl.stream(eng)
+    smask, wmask, dmask = runtime_masks(runtime_dims_masks)
     src_md = dnnl.memory_desc([p.M, p.K], p.src_dt, strides=list(p.src_stride[1:]))
     wei_md = dnnl.memory_desc([p.K, p.N], p.wei_dt, strides=list(p.wei_stride[1:]))
     dst_md = dnnl.memory_desc([p.M, p.N], p.dst_dt, strides=list(p.dst_stride[1:]))
@@ -267,8 +294,11 @@ def api_objects(p, want_ref_impl=False):
             po.append_sum(op.scale, op.zero_point, op.dt)
     if p.post_ops:
         attr.set_post_ops(po)
-    pd = dnnl.matmul_primitive_desc(eng, src_md, wei_md, dst_md, bias_md=bias_md, attr=attr)
-    if want_ref_impl:
+    pd = dnnl.matmul_primitive_desc(
+        eng, _pd_md([p.M, p.K], p.src_dt, p.src_stride[1:], smask), _pd_md([p.K, p.N], p.wei_dt, p.wei_stride[1:], wmask),
+        _pd_md([p.M, p.N], p.dst_dt, p.dst_stride[1:], dmask),
+        bias_md=_pd_md([1, p.N], p.bias_dt, (p.N, 1), dmask & 2) if bias_md else None, attr=attr)
+    if want_ref_impl and not (smask or wmask):
         while pd.impl_info_str() != "hip:ref:any":
             if not pd.next_impl():
                 raise RuntimeError("no hip:ref:any implementation in the list")
@@ -286,7 +316,8 @@ def run_spec(sp, mode="C", min_times=5, max_ms=300.0):
     """Returns (status, impl, details): status PASSED / FAILED / SKIPPED (unimplemented)."""
     p = build_problem(sp)
     try:
-        pd, prim, strm, args, dst = api_objects(p, want_ref_impl=sp.impl == "ref")
+        pd, prim, strm, args, dst = api_objects(p, want_ref_impl=sp.impl == "ref",
+                                                runtime_dims_masks=sp.runtime_dims_masks)
     except dnnl.error as e:
         if e.status == dnnl.unimplemented:
             return "SKIPPED", "", "unimplemented"

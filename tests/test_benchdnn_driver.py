@@ -66,6 +66,19 @@ LINES = [
     "--attr-scales=src:common:0.5+wei:common:0.25 --attr-post-ops=,relu+add:bf16 48x128:128x80 256x512:512x256",
     "--dt=f4_e2m1:f4_e2m1:bf16 --wtag=ba --attr-scales=src:per_tensor:e8m0:1x32+wei:per_tensor:e8m0:32x1 "
     "64x256:256x96 256x512:512x256",
+    # runtime dims: tests/benchdnn/inputs/matmul/test_matmul_all:4-25 and the int8 / decompression analogues
+    "--dt=f32 --wtag=ab,ba --runtime_dims_masks=0,2:1,1:0,3:1 --bia-dt=undef,f32 "
+    "--attr-scales=src:common:0.25+wei:per_oc+dst:common:4 --attr-post-ops=relu 10x30:30x20",
+    "--dt=f32 --stag=ba --wtag=ab,ba --runtime_dims_masks=3:1,3:3 --bia-dt=f32 "
+    "--attr-scales=src:common:0.25+wei:common:0.5+dst:common:4 --attr-post-ops=add:f32,sum+mul:s32:per_oc+linear:2:-1 "
+    "10x30:30x20",
+    "--dt=u8:s8:s8,s8:s8:f32 --wtag=ab,ba --runtime_dims_masks=1:0,3:3 --bia-dt=undef,f32 "
+    "--attr-scales=src:common:0.25+wei:per_oc+dst:common:4 --attr-zero-points=,src:common:1+dst:common:2 "
+    "10x30:30x20 300x128:128x260",
+    "--dt=bf16:u4:bf16 --runtime_dims_masks=1:0 --attr-scales=wei:per_ocic:bf16:32x1 --attr-zero-points=wei:per_ocic:u4:32x1 "
+    "--attr-fpmath=bf16:true 1x4096:4096x512 8x1024:1024x768",
+    "--dt=f8_e4m3:f8_e4m3:bf16 --wtag=ba --runtime_dims_masks=3:3 --bia-dt=bf16 --attr-scales=src:common:0.5+wei:common:0.25 "
+    "--attr-post-ops=relu+add:bf16 256x512:512x256",
 ]
 
 

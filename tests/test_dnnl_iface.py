@@ -311,3 +311,81 @@ def test_reorder_primitive_desc_rules(eng):
     a = dnnl.primitive_attr()
     a.set_scales(dnnl.ARG_SRC, 0)
     assert status_of(lambda: dnnl.reorder_primitive_desc(eng, u4, eng, f32, attr=a)) == dnnl.invalid_arguments
+
+
+# ---- runtime dims (DNNL_RUNTIME_DIM_VAL): tests/gtests/test_matmul.cpp:128-160,
+# :422-427, src/common/memory_desc.cpp:52-72,:298-308, src/common/memory.cpp:62,:155,
+# src/common/matmul.cpp:709-736
+R = dnnl.RUNTIME_DIM_VAL
+
+
+def test_memory_desc_with_runtime_dims(eng):
+    m = md([R, 7], "f32", tag=dnnl.tag_ab)
+    assert m.dims() == [R, 7] and m.strides() == [7, 1]
+    m = md([5, R], "f32", tag=dnnl.tag_ab)
+    assert m.strides() == [R, 1]                    # a stride outside a runtime dim is a runtime value
+    m = md([5, R], "f32", tag=dnnl.tag_ba)
+    assert m.strides() == [1, 5]
+    m = md([R, R], "s8", tag=dnnl.tag_ba)
+    assert m.strides() == [1, R]
+    m = md([2, R, 5], "bf16", tag=dnnl.tag_abc)
+    assert m.strides() == [R, 5, 1]
+    assert m.get_size() == dnnl.RUNTIME_SIZE_VAL
+    assert md([R, 4], "f32", strides=[R, 1]).strides() == [R, 1]
+    # no layout can be chosen for unknown dims, and no memory object can be made of them
+    assert status_of(lambda: md([R, 7], "f32", tag=dnnl.tag_any)) == dnnl.invalid_arguments
+    assert status_of(lambda: dnnl.memory(md([R, 7], "f32"), eng)) == dnnl.invalid_arguments
+    assert status_of(lambda: md([-3, 7], "f32")) == dnnl.invalid_arguments
+
+
+def test_matmul_pd_with_runtime_dims(eng):
+    pd = dnnl.matmul_primitive_desc(eng, md([R, R], "u8"), md([R, R], "s8", tag=dnnl.tag_ba), md([R, R], "s32"))
+    assert pd.impl_info_str() == "hip:runtime_dims:any"
+    assert pd.next_impl() is False
+    assert pd.query_md(dnnl.query_src_md).dims() == [R, R]
+    assert pd.query_md(dnnl.query_weights_md).strides() == [1, R]
+    assert pd.scratchpad_desc().ndims() == 0
+    dnnl.matmul(pd)                                   # a primitive can be created; it executes on a device only
+    # only M unknown (a decode loop): weights known
+    pd = dnnl.matmul_primitive_desc(eng, md([R, 256], "bf16"), md([256, 128], "bf16"), md([R, 128], "bf16"))
+    assert pd.impl_info_str() == "hip:runtime_dims:any"
+    # M, N, K agree as values, runtime included (matmul.cpp:683-688)
+    bad = [(md([R, 256], "f32"), md([256, 128], "f32"), md([4, 128], "f32")),
+           (md([4, R], "f32"), md([256, 128], "f32"), md([4, 128], "f32")),
+           (md([4, 256], "f32"), md([256, R], "f32"), md([4, 128], "f32"))]
+    for s, w, d in bad:
+        assert status_of(lambda: dnnl.matmul_primitive_desc(eng, s, w, d)) == dnnl.invalid_arguments
+    # a runtime batch dim is runtime in src, weights and dst alike (test_matmul.cpp:422-427)
+    assert status_of(lambda: dnnl.matmul_primitive_desc(
+        eng, md([3, 10, 10], "f32"), md([R, 10, 10], "f32"), md([R, 10, 10], "f32"))) == dnnl.invalid_arguments
+    dnnl.matmul_primitive_desc(eng, md([R, 10, 10], "f32"), md([R, 10, 10], "f32"), md([R, 10, 10], "f32"))
+    # bias over a runtime batch dim: 1 or runtime
+    dnnl.matmul_primitive_desc(eng, md([R, 10, 10], "f32"), md([R, 10, 10], "f32"), md([R, 10, 10], "f32"),
+                               bias_md=md([1, 1, 10], "f32"))
+    assert status_of(lambda: dnnl.matmul_primitive_desc(
+        eng, md([R, 10, 10], "f32"), md([R, 10, 10], "f32"), md([R, 10, 10], "f32"),
+        bias_md=md([3, 1, 10], "f32"))) == dnnl.invalid_arguments
+
+
+def test_attributes_are_checked_with_runtime_dims_too(eng):
+    # rules that need no dim value still hold at creation
+    a = dnnl.primitive_attr()
+    a.set_zero_points(dnnl.ARG_SRC, 0, (), DT["s32"])
+    assert status_of(lambda: dnnl.matmul_primitive_desc(            # zero points with a floating-point src
+        eng, md([R, R], "f32"), md([R, R], "f32"), md([R, R], "f32"), attr=a)) != dnnl.success
+    a = dnnl.primitive_attr()
+    a.set_scales(dnnl.ARG_WEIGHTS, 2, (), DT["f32"])
+    po = dnnl.post_ops()
+    po.append_eltwise(cabi.ELTWISE["relu"], 0.0, 0.0)
+    po.append_binary(cabi.BINARY["add"], md([1, 64], "f32"))       # a known src1 under an unknown dst
+    a.set_post_ops(po)
+    pd = dnnl.matmul_primitive_desc(eng, md([R, R], "s8"), md([R, R], "s8", tag=dnnl.tag_ba), md([R, R], "f32"), attr=a)
+    assert pd.impl_info_str() == "hip:runtime_dims:any"
+    # data type combinations are known at creation
+    assert status_of(lambda: dnnl.matmul_primitive_desc(
+        eng, md([R, R], "s8"), md([R, R], "f32"), md([R, R], "f32"))) == dnnl.unimplemented
+
+
+def test_reorder_with_runtime_dims_is_unimplemented(eng):
+    assert status_of(lambda: dnnl.reorder_primitive_desc(
+        eng, md([R, 8], "f32"), eng, md([R, 8], "f32"))) == dnnl.unimplemented

@@ -12,8 +12,25 @@ pytestmark = pytest.mark.gpu
 DT = cabi.DT_NAMES
 
 
-def run_through_api(p, scratchpad_user=False):
-    """Builds the dnnl objects that describe MatmulProblem `p` (2-D, dense)."""
+def runtime_md(dims, dt, strides, runtime):
+    """The descriptor given to the primitive descriptor: with `runtime` "all"
+    every dim is DNNL_RUNTIME_DIM_VAL and the layout is a tag, as in
+    tests/gtests/test_matmul.cpp:128-137; with "m" only the row count of src and
+    dst is (`dims[0]` is None for those)."""
+    R = dnnl.RUNTIME_DIM_VAL
+    tag = dnnl.tag_ab if strides[1] == 1 else dnnl.tag_ba
+    if runtime == "all":
+        return dnnl.memory_desc([R, R], dt, tag=tag)
+    if runtime == "m" and dims[0] is None:
+        assert tag == dnnl.tag_ab
+        return dnnl.memory_desc([R, dims[1]], dt, tag=tag)
+    return dnnl.memory_desc([d for d in dims], dt, strides=list(strides))
+
+
+def run_through_api(p, scratchpad_user=False, runtime=None, reuse=None):
+    """Builds the dnnl objects that describe MatmulProblem `p` (2-D, dense).
+    `runtime`: see runtime_md; `reuse` = (pd, prim) of an earlier call executes
+    that primitive on this problem's shapes."""
     eng = dnnl.engine(dnnl.gpu, 0)
     strm = dnnl.stream(eng)
     src_md = dnnl.memory_desc([p.M, p.K], p.src_dt, strides=list(p.src_stride[1:]))
@@ -59,8 +76,18 @@ def run_through_api(p, scratchpad_user=False):
         attr.set_post_ops(po)
     if scratchpad_user:
         attr.set_scratchpad_mode(dnnl.scratchpad_user)
-    pd = dnnl.matmul_primitive_desc(eng, src_md, wei_md, dst_md, bias_md=bias_md, attr=attr)
-    prim = dnnl.matmul(pd)
+    if reuse is not None:
+        pd, prim = reuse
+    elif runtime:
+        pd = dnnl.matmul_primitive_desc(
+            eng, runtime_md([None, p.K], p.src_dt, p.src_stride[1:], runtime),
+            runtime_md([p.K, p.N], p.wei_dt, p.wei_stride[1:], runtime),
+            runtime_md([None, p.N], p.dst_dt, p.dst_stride[1:], runtime),
+            bias_md=runtime_md([1, p.N], p.bias_dt, (p.N, 1), runtime) if bias_md else None, attr=attr)
+        prim = dnnl.matmul(pd)
+    else:
+        pd = dnnl.matmul_primitive_desc(eng, src_md, wei_md, dst_md, bias_md=bias_md, attr=attr)
+        prim = dnnl.matmul(pd)
     args[dnnl.ARG_SRC] = dnnl.memory(src_md, eng, p.src)
     args[dnnl.ARG_WEIGHTS] = dnnl.memory(wei_md, eng, p.wei)
     dst = dnnl.memory(dst_md, eng, p.initial_dst())
@@ -262,3 +289,71 @@ def test_dynamic_mx_dst_through_the_api(gpu, oracle):
     want, want_sc = orc.run_oracle_dynamic(p)
     assert np.array_equal(sc_mem.read(np.uint8).reshape(-1), np.asarray(want_sc).reshape(-1))
     assert np.array_equal(dst.read(np.uint8).reshape(-1), np.asarray(want).view(np.uint8).reshape(-1))
+
+
+# ---- runtime dims: one primitive, shapes known at execution only
+# (tests/gtests/test_matmul.cpp:544-576,599-660; benchdnn --runtime_dims_masks)
+def test_all_runtime_dims_int8_one_primitive_two_shapes(gpu, oracle):
+    # the src zero point makes the integer GEMM ask for a scratch buffer (column
+    # sums), which a primitive with runtime dims allocates when it executes
+    p = configs.config1()
+    got, name, (pd, prim, _, _) = run_through_api(p, runtime="all")
+    assert name == "hip:runtime_dims:any"
+    assert_bit_exact(p, got, oracle.run_oracle(p), name)
+    # the same primitive on other shapes
+    q = configs.config1(M=37, N=p.N * 2, K=p.K // 2)
+    got, _, _ = run_through_api(q, reuse=(pd, prim))
+    assert_bit_exact(q, got, oracle.run_oracle(q), name)
+    # and back: the cached lowering is replaced, not mixed up
+    got, _, _ = run_through_api(p, reuse=(pd, prim))
+    assert_bit_exact(p, got, oracle.run_oracle(p), name)
+
+
+def test_all_runtime_dims_per_column_scales_and_post_ops(gpu, oracle):
+    p = configs.config3(M=160, N=288, K=512, wtag="ba")
+    got, name, (pd, prim, _, _) = run_through_api(p, runtime="all")
+    assert name == "hip:runtime_dims:any"
+    assert_bit_exact(p, got, oracle.run_oracle(p), name)
+    q = configs.config3(M=512, N=1024, K=1024, wtag="ba")
+    got, _, _ = run_through_api(q, reuse=(pd, prim))
+    assert_bit_exact(q, got, oracle.run_oracle(q), name)
+
+
+def test_all_runtime_dims_fp8_with_binary_post_op(gpu, oracle):
+    p = configs.config4(M=96, N=256, K=512, wtag="ba")
+    got, name, _ = run_through_api(p, runtime="all")
+    want, _, asum = oracle.run_oracle(p, want_ideal=True)
+    assert_close(p, got, want, abs_sum=asum, transcendental=True, what=name)
+
+
+def test_runtime_row_count_of_the_decode_matmul(gpu, oracle):
+    p = configs.config2(M=1, N=512, K=1024)
+    got, name, (pd, prim, _, _) = run_through_api(p, runtime="m")
+    assert name == "hip:runtime_dims:any"
+    want, _, asum = oracle.run_oracle(p, want_ideal=True)
+    assert_close(p, got, want, abs_sum=asum, what=name)
+    for M in (8, 33):
+        q = configs.config2(M=M, N=512, K=1024)
+        got, _, _ = run_through_api(q, reuse=(pd, prim))
+        want, _, asum = oracle.run_oracle(q, want_ideal=True)
+        assert_close(q, got, want, abs_sum=asum, what=name)
+
+
+def test_runtime_dims_memory_that_contradicts_the_descriptor(gpu):
+    p = configs.config2(M=4, N=512, K=1024)
+    _, _, (pd, prim, strm, args) = run_through_api(p, runtime="m")
+    eng = dnnl.engine(dnnl.gpu, 0)
+    bad = dict(args)
+    # K of src differs from the K the descriptor was created with
+    bad[dnnl.ARG_SRC] = dnnl.memory(dnnl.memory_desc([4, 512], p.src_dt, tag=dnnl.tag_ab), eng)
+    with pytest.raises(dnnl.error) as e:
+        prim.execute(strm, bad)
+    assert e.value.status == dnnl.invalid_arguments
+    # row counts of src and dst disagree
+    bad = dict(args)
+    bad[dnnl.ARG_SRC] = dnnl.memory(dnnl.memory_desc([5, 1024], p.src_dt, tag=dnnl.tag_ab), eng)
+    with pytest.raises(dnnl.error) as e:
+        prim.execute(strm, bad)
+    assert e.value.status == dnnl.invalid_arguments
+    prim.execute(strm, args)                          # the primitive stays usable
+    strm.wait()
