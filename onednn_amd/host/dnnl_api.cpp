@@ -641,31 +641,28 @@ dnnl_status_t dispatch(dnnl_primitive_desc &pd) {
 // is chosen.  The result is kept for the next execution with the same shapes.
 dnnl_status_t concretize(dnnl_primitive &prim, const std::map<int, dnnl_memory_t> &m, void **scratch) {
     const dnnl_primitive_desc &pd0 = prim.pd;
-    std::unique_ptr<dnnl_primitive_desc> c(new dnnl_primitive_desc(pd0));
-    c->runtime = false;
-    struct slot_t {
-        int arg;
-        const dnnl_memory_desc *from;
-        dnnl_memory_desc *to;
-        bool present;
-    } slots[] = {{DNNL_ARG_SRC, &pd0.src, &c->src, true}, {DNNL_ARG_WEIGHTS, &pd0.wei, &c->wei, true},
-            {DNNL_ARG_DST, &pd0.dst, &c->dst, true}, {DNNL_ARG_BIAS, &pd0.bias, &c->bias, pd0.with_bias}};
-    for (const slot_t &sl : slots) {
-        if (!sl.present || !sl.from->has_runtime()) continue;
-        auto it = m.find(sl.arg);
+    // src, weights, dst, bias of this execution
+    dnnl_memory_desc now[4] = {pd0.src, pd0.wei, pd0.dst, pd0.bias};
+    const int arg_of[4] = {DNNL_ARG_SRC, DNNL_ARG_WEIGHTS, DNNL_ARG_DST, DNNL_ARG_BIAS};
+    for (int t = 0; t < 4; ++t) {
+        if ((t == 3 && !pd0.with_bias) || !now[t].has_runtime()) continue;
+        const dnnl_memory_desc &from = now[t];
+        auto it = m.find(arg_of[t]);
         CHECK_ARG(it != m.end() && it->second);
         const dnnl_memory_desc &mm = it->second->md;
-        CHECK_ARG(mm.kind == dnnl_blocked && mm.ndims == sl.from->ndims && mm.dt == sl.from->dt);
+        CHECK_ARG(mm.kind == dnnl_blocked && mm.ndims == from.ndims && mm.dt == from.dt);
         for (int i = 0; i < mm.ndims; ++i) {
-            CHECK_ARG(sl.from->dims[i] == DNNL_RUNTIME_DIM_VAL || sl.from->dims[i] == mm.dims[i]);
-            CHECK_ARG(sl.from->strides[i] == DNNL_RUNTIME_DIM_VAL || sl.from->strides[i] == mm.strides[i]
-                    || mm.dims[i] <= 1);
+            CHECK_ARG(from.dims[i] == DNNL_RUNTIME_DIM_VAL || from.dims[i] == mm.dims[i]);
+            CHECK_ARG(from.strides[i] == DNNL_RUNTIME_DIM_VAL || from.strides[i] == mm.strides[i] || mm.dims[i] <= 1);
         }
-        *sl.to = mm;
+        now[t] = mm;
     }
-    const bool same = prim.rt_pd && prim.rt_pd->src == c->src && prim.rt_pd->wei == c->wei && prim.rt_pd->dst == c->dst
-            && (!pd0.with_bias || prim.rt_pd->bias == c->bias);
+    const bool same = prim.rt_pd && prim.rt_pd->src == now[0] && prim.rt_pd->wei == now[1] && prim.rt_pd->dst == now[2]
+            && (!pd0.with_bias || prim.rt_pd->bias == now[3]);
     if (!same) {
+        std::unique_ptr<dnnl_primitive_desc> c(new dnnl_primitive_desc(pd0));
+        c->runtime = false;
+        c->src = now[0]; c->wei = now[1]; c->dst = now[2]; c->bias = now[3];
         dnnl_status_t st = check_shapes(c->src, c->wei, pd0.with_bias ? &c->bias : nullptr, c->dst);
         if (st) return st;
         st = check_attr(c->src, c->wei, c->dst, c->attr);

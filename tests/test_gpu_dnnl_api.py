@@ -357,3 +357,26 @@ def test_runtime_dims_memory_that_contradicts_the_descriptor(gpu):
     assert e.value.status == dnnl.invalid_arguments
     prim.execute(strm, args)                          # the primitive stays usable
     strm.wait()
+
+
+def test_runtime_batch_dims_and_broadcast_weights(gpu):
+    # 3-D: every dim unknown at creation; small integers in f32 are exact, numpy is the check.
+    # Second execution: weights with a batch of one, broadcast over src's batch.
+    R = dnnl.RUNTIME_DIM_VAL
+    eng = dnnl.engine(dnnl.gpu, 0)
+    strm = dnnl.stream(eng)
+    f32 = DT["f32"]
+    rt = lambda tag: dnnl.memory_desc([R, R, R], f32, tag=tag)
+    pd = dnnl.matmul_primitive_desc(eng, rt(dnnl.tag_abc), rt(dnnl.tag_acb), rt(dnnl.tag_abc))
+    prim = dnnl.matmul(pd)
+    r = np.random.default_rng(11)
+    for B, Bw, M, K, N in ((3, 3, 17, 40, 24), (4, 1, 5, 64, 130)):
+        s = r.integers(-4, 5, size=(B, M, K)).astype(np.float32)
+        w = r.integers(-4, 5, size=(Bw, K, N)).astype(np.float32)
+        dst = dnnl.memory(dnnl.memory_desc([B, M, N], f32, tag=dnnl.tag_abc), eng)
+        prim.execute(strm, {dnnl.ARG_SRC: dnnl.memory(dnnl.memory_desc([B, M, K], f32, tag=dnnl.tag_abc), eng, s),
+                            dnnl.ARG_WEIGHTS: dnnl.memory(dnnl.memory_desc([Bw, K, N], f32, tag=dnnl.tag_acb), eng,
+                                                          np.ascontiguousarray(w.transpose(0, 2, 1))),
+                            dnnl.ARG_DST: dst})
+        strm.wait()
+        assert np.array_equal(dst.read(np.float32).reshape(B, M, N), s @ w)
