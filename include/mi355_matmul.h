@@ -136,10 +136,21 @@ enum {
  *             (the exponent byte of x; 2^-127 for a zero exponent)
  *     args->dst_scale[(b, m, n / 32)] = scale       (written, despite the const)
  *     dst = convert(clamp(d * (1 / scale), -max, +max))
- * dst is f8_e4m3 or f8_e5m2, N % 32 == 0, no dst zero point. */
+ * dst is f8_e4m3, f8_e5m2 or f4_e2m1, N % 32 == 0, no dst zero point.
+ *
+ * MI355_DST_DYNAMIC_FP (quantization_mode::dynamic_fp, the NVFP4 flavour;
+ * ref_matmul.cpp:352-365, rules src/common/matmul.cpp:423-440): groups of 16
+ * consecutive n, f8_e4m3 scales
+ *     scale = e4m3(min(max(amax / max of dst type, 2^-3), 448))
+ *             (2^-3 = epsilon of e4m3, src/common/nstl.hpp:189-191)
+ * and the rest as above; N % 16 == 0.
+ *
+ * A 4-bit dst (f4_e2m1) is offered with dynamic scales only (generic kernel):
+ * unit n stride and even m / batch strides, so that a group is whole bytes. */
 enum {
     MI355_DST_DYNAMIC_NONE = 0,
-    MI355_DST_DYNAMIC_MX = 1
+    MI355_DST_DYNAMIC_MX = 1,
+    MI355_DST_DYNAMIC_FP = 2
 };
 
 /* Kernel families (implementation ids). 0 lets the library choose. */

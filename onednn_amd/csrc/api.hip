@@ -70,11 +70,14 @@ static int validate(const mi355_matmul_desc_t *d) {
     if (d->dst_scale_dynamic != MI355_DST_DYNAMIC_NONE) {
         // src/common/matmul.cpp:407-424
         const mi355_quant_t &q = d->dst_scale;
-        const bool ok = d->dst_scale_dynamic == MI355_DST_DYNAMIC_MX && q.dt == MI355_DT_E8M0
-                && (q.mask & 6) == 6 && (d->batch == 1 || (q.mask & 1)) && q.group[0] == 1 && q.group[1] == 32
-                && d->N % 32 == 0 && is_f8_dt(d->dst_dt) && quant_absent(d->dst_zp);
+        const bool mx = d->dst_scale_dynamic == MI355_DST_DYNAMIC_MX, fp = d->dst_scale_dynamic == MI355_DST_DYNAMIC_FP;
+        const int g = mx ? 32 : 16;
+        const bool ok = (mx || fp) && q.dt == (mx ? MI355_DT_E8M0 : MI355_DT_F8_E4M3)
+                && (q.mask & 6) == 6 && (d->batch == 1 || (q.mask & 1)) && q.group[0] == 1 && q.group[1] == g
+                && d->N % g == 0 && (is_f8_dt(d->dst_dt) || d->dst_dt == MI355_DT_F4_E2M1) && quant_absent(d->dst_zp);
         if (!ok) {
-            set_error("dynamic dst scales: e8m0, full mask, groups 1 x 32, N %% 32 == 0, f8 dst, no dst zero point");
+            set_error("dynamic dst scales: e8m0 with groups 1 x 32 (MX) or f8_e4m3 with groups 1 x 16 (FP), full mask, "
+                      "N a multiple of the group, f8 or f4 dst, no dst zero point");
             return MI355_INVALID_ARGUMENTS;
         }
     }
@@ -110,6 +113,10 @@ static int impl_supported(const mi355_matmul_desc_t &d, int impl) {
     // dynamic dst quantization: the generic kernel and the floating-point GEMM tiles
     if (d.dst_scale_dynamic != MI355_DST_DYNAMIC_NONE && impl != MI355_IMPL_REF && impl != MI355_IMPL_F8_MFMA
             && impl != MI355_IMPL_MXF4_MFMA)
+        return MI355_UNIMPLEMENTED;
+    // the tiles' group reduction is the MX one (32 columns, fp8 dst)
+    if ((d.dst_scale_dynamic == MI355_DST_DYNAMIC_FP || (d.dst_scale_dynamic && !is_f8_dt(d.dst_dt)))
+            && impl != MI355_IMPL_REF)
         return MI355_UNIMPLEMENTED;
     switch (impl) {
         case MI355_IMPL_REF: return ref_supported(d);

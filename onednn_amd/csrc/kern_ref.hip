@@ -130,12 +130,16 @@ __global__ void __launch_bounds__(256) ref_matmul_kernel(const problem_t P_) {
 // computed exactly as above, their largest magnitude gives the group's e8m0
 // scale, which is written to the scales tensor and applied by a multiplication
 // with its (exact, power of two) inverse.
+//
+// G == 16: the dynamic_fp (NVFP4) flavour, ref_matmul.cpp:352-365: the scale
+// is amax / max(dst type), clamped to [epsilon, max] of f8_e4m3 and rounded to
+// it.  A 4-bit dst is written a byte (two consecutive n) at a time.
+template <int G>
 __global__ void __launch_bounds__(64) ref_matmul_dynamic_kernel(const problem_t P_) {
     const auto &P = MI355_KERNARG_PROBLEM();
-    constexpr int G = 32;
     const long groups_n = P.N / G;
     const long total = P.B * P.M * groups_n;
-    const float dt_max = P.dst_dt == MI355_DT_F8_E4M3 ? 448.f : 57344.f;
+    const float dt_max = P.dst_dt == MI355_DT_F8_E4M3 ? 448.f : P.dst_dt == MI355_DT_F4_E2M1 ? 6.f : 57344.f;
     const bool int_path = P.src_dt == MI355_DT_S8 || P.src_dt == MI355_DT_U8;
     for (long i = (long)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += (long)gridDim.x * blockDim.x) {
         const long ng = i % groups_n, m = (i / groups_n) % P.M, b = i / (groups_n * P.M);
@@ -149,23 +153,46 @@ __global__ void __launch_bounds__(64) ref_matmul_dynamic_kernel(const problem_t 
         }
 #pragma unroll
         for (int e = 0; e < G; ++e) amax = fmaxf(amax, fabsf(d[e]));
-        // e8m0(x): the exponent byte of x
-        const float r = e8m0_to_f32(f32_to_e8m0(amax)) / e8m0_to_f32(f32_to_e8m0(dt_max));
-        const uint8_t sbyte = f32_to_e8m0(r);
+        uint8_t sbyte;
+        float inv;
+        if (G == 32) {
+            // e8m0(x): the exponent byte of x
+            const float r = e8m0_to_f32(f32_to_e8m0(amax)) / e8m0_to_f32(f32_to_e8m0(dt_max));
+            sbyte = f32_to_e8m0(r);
+            inv = 1.f / e8m0_to_f32(sbyte);
+        } else {
+            float r = amax / dt_max;
+            r = fmaxf(fminf(r, 448.f), 0.125f);
+            sbyte = f32_to_e4m3(r);
+            inv = 1.f / e4m3_to_f32(sbyte);
+        }
         ((uint8_t *)P.dst_scale.p)[quant_off(P.dst_scale, b, m, ng * G, P.M, P.N)] = sbyte;
-        const float inv = 1.f / e8m0_to_f32(sbyte);
+        const long off0 = b * P.ds[0] + m * P.ds[1] + ng * G * P.ds[2];
+        if (P.dst_dt == MI355_DT_F4_E2M1) {
+            // unit n stride, even row offsets (checked by the host): the group is G / 2 whole bytes
+#pragma unroll
+            for (int e = 0; e < G; e += 2) {
+                const float lo = fminf(fmaxf(d[e] * inv, -dt_max), dt_max), hi = fminf(fmaxf(d[e + 1] * inv, -dt_max), dt_max);
+                ((uint8_t *)P.dst)[(off0 + e) >> 1] = (uint8_t)(f32_to_e2m1(lo) | (f32_to_e2m1(hi) << 4));
+            }
+            continue;
+        }
 #pragma unroll
         for (int e = 0; e < G; ++e) {
             float v = d[e] * inv;
             v = fminf(fmaxf(v, -dt_max), dt_max);
-            store_float(P.dst_dt, v, P.dst, b * P.ds[0] + m * P.ds[1] + (ng * G + e) * P.ds[2]);
+            store_float(P.dst_dt, v, P.dst, off0 + e * P.ds[2]);
         }
     }
 }
 
 int ref_supported(const mi355_matmul_desc_t &d) {
-    // 4-bit dst would need two elements per thread; not offered.
-    if (dt_bits(d.dst_dt) < 8) return MI355_UNIMPLEMENTED;
+    // 4-bit dst: two elements share a byte.  Offered where one thread owns both:
+    // f4_e2m1 with dynamic scales (a thread per group of whole bytes).
+    if (dt_bits(d.dst_dt) < 8) {
+        if (d.dst_dt != MI355_DT_F4_E2M1 || d.dst_scale_dynamic == MI355_DST_DYNAMIC_NONE) return MI355_UNIMPLEMENTED;
+        if (d.dst_stride[2] != 1 || (d.dst_stride[1] & 1) || (d.dst_stride[0] & 1)) return MI355_UNIMPLEMENTED;
+    }
     if (d.wei_packing != MI355_WEI_PACK_NONE && !woq64_layout_ok(d)) return MI355_UNIMPLEMENTED;
     // dynamic dst quantization exists in ref_matmul_t only, not in the integer implementation
     if (d.dst_scale_dynamic != MI355_DST_DYNAMIC_NONE && is_int8_dt(d.src_dt)) return MI355_UNIMPLEMENTED;
@@ -176,9 +203,13 @@ int ref_launch(const problem_t &P, hipStream_t stream) {
     const long total = P.B * P.M * P.N;
     if (total == 0) return MI355_SUCCESS;
     if (P.dst_dynamic) {
-        long groups = total / 32, gblocks = (groups + 63) / 64;
+        const int G = P.dst_dynamic == MI355_DST_DYNAMIC_MX ? 32 : 16;
+        long groups = total / G, gblocks = (groups + 63) / 64;
         if (gblocks > 1048576) gblocks = 1048576;
-        hipLaunchKernelGGL(ref_matmul_dynamic_kernel, dim3((unsigned)gblocks), dim3(64), 0, stream, P);
+        if (G == 32)
+            hipLaunchKernelGGL(ref_matmul_dynamic_kernel<32>, dim3((unsigned)gblocks), dim3(64), 0, stream, P);
+        else
+            hipLaunchKernelGGL(ref_matmul_dynamic_kernel<16>, dim3((unsigned)gblocks), dim3(64), 0, stream, P);
         return hipGetLastError() == hipSuccess ? MI355_SUCCESS : MI355_RUNTIME_ERROR;
     }
     long blocks = (total + 255) / 256;

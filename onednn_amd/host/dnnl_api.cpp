@@ -170,6 +170,8 @@ struct quant_entry_t {
     dim_t group(int d) const { return group_ndims == 0 ? 1 : groups[d]; }
     dnnl_quantization_mode_t qmode = dnnl_quantization_mode_static_sazp;
     bool is_mx() const { return qmode == dnnl_quantization_mode_dynamic_mx; }
+    bool is_dynamic_fp() const { return qmode == dnnl_quantization_mode_dynamic_fp; }
+    bool is_dynamic() const { return is_mx() || is_dynamic_fp(); }
 };
 
 struct post_op_entry_t {
@@ -357,10 +359,16 @@ dnnl_status_t check_attr(const dnnl_memory_desc &s, const dnnl_memory_desc &w, c
             CHECK_UNIMPL(q->group_ndims == 2 && q->group(1) == 32 && q->group(0) == 1);
             CHECK_UNIMPL(q->dt == dnnl_e8m0);
         }
+        // dynamic_fp: the NVFP4 flavour only, f8_e4m3 scales per 16 (matmul.cpp:423-440)
+        if (q->is_dynamic_fp()) {
+            CHECK_UNIMPL(q->mask == full);
+            CHECK_UNIMPL(q->dt == dnnl_f8_e4m3);
+            CHECK_UNIMPL(q->group_ndims == 2 && q->group(1) == 16 && q->group(0) == 1);
+        }
     }
     // dynamic quantization is a dst scale mode
     for (int arg : {DNNL_ARG_SRC, DNNL_ARG_WEIGHTS})
-        if (auto q = a.find(a.scales, arg)) CHECK_UNIMPL(!q->is_mx());
+        if (auto q = a.find(a.scales, arg)) CHECK_UNIMPL(!q->is_dynamic());
     CHECK_UNIMPL(IMPLICATION(src_sg_k > 1, (src_int8 || src_fp8 || src_fp4) && divisible(src_sg_k, wei_sg_k)));
 
     dim_t src_zg_k = 1, wei_zg_k = 1;
@@ -520,9 +528,10 @@ dnnl_status_t lower(dnnl_primitive_desc &pd) {
     // a static dst scale is one value; a grouped one is the dynamic (MX) mode
     {
         const quant_entry_t *dq = a.find(a.scales, DNNL_ARG_DST);
-        if (dq && dq->is_mx()) {
-            D.dst_scale_dynamic = MI355_DST_DYNAMIC_MX;
-            CHECK_UNIMPL(is_fp8(pd.dst.dt) && D.dst_zp.dt == MI355_DT_UNDEF && D.N % 32 == 0);
+        if (dq && dq->is_dynamic()) {
+            D.dst_scale_dynamic = dq->is_mx() ? MI355_DST_DYNAMIC_MX : MI355_DST_DYNAMIC_FP;
+            CHECK_UNIMPL((is_fp8(pd.dst.dt) || pd.dst.dt == dnnl_f4_e2m1) && D.dst_zp.dt == MI355_DT_UNDEF
+                    && D.N % dq->group(1) == 0);
         } else {
             CHECK_UNIMPL(D.dst_scale.dt == MI355_DT_UNDEF || D.dst_scale.mask == 0);
         }
@@ -612,7 +621,7 @@ dnnl_status_t check_dtypes(const dnnl_primitive_desc &pd) {
                     || w == dnnl_u4);
             // integer weights under a floating-point src only as weight decompression
             CHECK_UNIMPL(IMPLICATION(is_int8(w) || w == dnnl_s4 || w == dnnl_u4, pd.attr.apply_to_int));
-            CHECK_UNIMPL(d == dnnl_f32 || d == dnnl_bf16 || d == dnnl_f16 || is_fp8(d) || is_int8(d));
+            CHECK_UNIMPL(d == dnnl_f32 || d == dnnl_bf16 || d == dnnl_f16 || is_fp8(d) || is_int8(d) || d == dnnl_f4_e2m1);
             if (pd.with_bias) CHECK_UNIMPL(pd.bias.dt == dnnl_f32 || pd.bias.dt == dnnl_bf16 || pd.bias.dt == dnnl_f16 || is_fp8(pd.bias.dt));
         }
     }
@@ -1017,7 +1026,6 @@ DNNL_EXPORT dnnl_status_t dnnl_primitive_attr_set_scales_v3(dnnl_primitive_attr_
             || qmode == dnnl_quantization_mode_dynamic_fp);
     CHECK_ARG(IMPLICATION(is_on_host, mask == 0 && group_ndims == 0));
     CHECK_UNIMPL(!is_on_host);
-    CHECK_UNIMPL(qmode != dnnl_quantization_mode_dynamic_fp);
     const dnnl_status_t st = dnnl_primitive_attr_set_scales(attr, arg, mask, group_ndims, group_dims, data_type);
     if (st == dnnl_success) attr->scales[arg].qmode = qmode;
     return st;

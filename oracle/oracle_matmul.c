@@ -48,6 +48,10 @@
  * largest magnitude through exponent bytes, restated there with numpy integer
  * arithmetic on the f32 bit patterns and checked on constructed groups
  * (powers of two, just below / above one, zeros, values beyond the dst range).
+ * The dynamic_fp branch (f8_e4m3 scales per 16, f4_e2m1 / fp8 dst) is pinned
+ * there too: the scale against an exhaustive nearest-value search over the 127
+ * positive e4m3 codes on constructed maxima (ties to even, both clamps), the
+ * dst codes against a nearest-value search over the type's codes.
  * Unpinned: none of the functions used by the five benchmark configurations;
  * the libm-dependent eltwise algorithms other than relu/gelu_tanh/linear/tanh
  * are "parity unpinned" beyond their textbook formula.
@@ -466,7 +470,7 @@ static float orc_dt_max(int dt) {
     }
 }
 
-/* One group of dynamic (MX) dst quantization, ref_matmul.cpp:268-423: the
+/* One group of dynamic (MX or FP) dst quantization, ref_matmul.cpp:268-423: the
  * values `v[0..g)` of columns n0.. of row (b, m), after bias and post-ops. */
 static void orc_finish_dynamic_group(const mi355_matmul_desc_t *d,
         const mi355_matmul_args_t *a, const float *v, int g, int64_t b,
@@ -474,9 +478,19 @@ static void orc_finish_dynamic_group(const mi355_matmul_desc_t *d,
     float max_dst_group = 0.f;
     for (int e = 0; e < g; ++e) max_dst_group = fmaxf(max_dst_group, fabsf(v[e]));
     const float dst_max = orc_dt_max(d->dst_dt);
-    /* :343-351, the rounding to a power of two happens before the division */
-    float scale = orc_round_e8m0(max_dst_group) / orc_round_e8m0(dst_max);
-    scale = orc_round_e8m0(scale);
+    float scale;
+    if (d->dst_scale_dynamic == MI355_DST_DYNAMIC_FP) {
+        /* :352-365: clamped to [epsilon, max] of the scale type f8_e4m3
+         * (epsilon = 2^-3, src/common/nstl.hpp:189-191), then rounded to it */
+        scale = max_dst_group / dst_max;
+        scale = fminf(scale, 448.f);
+        scale = fmaxf(scale, 0.125f);
+        scale = orc_e4m3_to_f32(orc_f32_to_e4m3(scale));
+    } else {
+        /* :343-351, the rounding to a power of two happens before the division */
+        scale = orc_round_e8m0(max_dst_group) / orc_round_e8m0(dst_max);
+        scale = orc_round_e8m0(scale);
+    }
     const int64_t soff = orc_quant_off(&d->dst_scale, b, m, n0, d->M, d->N);
     orc_store_float(d->dst_scale.dt, scale, (void *)a->dst_scale, soff); /* :377-378 */
     const float inv = 1.f / scale; /* :381 */
@@ -506,7 +520,7 @@ int oracle_matmul(const mi355_matmul_desc_t *d, const mi355_matmul_args_t *a,
     if (d->batch == 0 || d->M == 0 || d->N == 0 || d->K == 0) return MI355_SUCCESS;
     const int int_path = orc_src_is_int(d->src_dt);
     const int64_t B = d->batch, M = d->M, N = d->N;
-    if (d->dst_scale_dynamic == MI355_DST_DYNAMIC_MX) {
+    if (d->dst_scale_dynamic != MI355_DST_DYNAMIC_NONE) {
         const int g = (int)d->dst_scale.group[1];
         if (g < 1 || g > 64 || N % g) return MI355_INVALID_ARGUMENTS;
 #pragma omp parallel for collapse(2) schedule(static)

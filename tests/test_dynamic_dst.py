@@ -208,3 +208,154 @@ def test_gpu_gemm_tiles_quantize_dst_dynamically(gpu, oracle, family):
     # are 2^-9 of the scaled range
     tol = 0.14 * np.abs(pre) + amax * 2.0 ** -8 + 1e-6
     assert np.all(np.abs(deq - pre) <= tol), float(np.max(np.abs(deq - pre) / tol))
+
+
+# ---- quantization_mode::dynamic_fp (NVFP4 flavour): f8_e4m3 scales per 16
+# columns, f4_e2m1 or fp8 dst (ref_matmul.cpp:352-365, matmul.cpp:423-440)
+E2M1 = np.array([0.0, 0.5, 1.0, 1.5, 2.0, 3.0, 4.0, 6.0], np.float64)
+FP_MAX = {cabi.DT_F4_E2M1: 6.0, cabi.DT_F8_E4M3: 448.0, cabi.DT_F8_E5M2: 57344.0}
+
+
+def dynamic_fp(p):
+    p.quant["dst_scale"] = QuantParam(cabi.DT_F8_E4M3, configs.MASK_ROW | configs.MASK_COL,
+                                      np.zeros((p.batch, p.M, p.N // 16), np.uint8), (1, 16))
+    p.dst_dynamic = cabi.DST_DYNAMIC_FP
+    return p
+
+
+def nearest_even(x, grid):
+    """Index of the value of the ascending `grid` nearest to each x >= 0; ties go to the even index
+    (codes of e4m3 / e2m1 ascend with the value, and an even code has an even mantissa)."""
+    x = np.asarray(x, np.float64)
+    hi = np.clip(np.searchsorted(grid, x, side="left"), 1, len(grid) - 1)
+    lo = hi - 1
+    dl, dh = x - grid[lo], grid[hi] - x
+    return np.where(dl < dh, lo, np.where(dh < dl, hi, np.where(lo % 2 == 0, lo, hi)))
+
+
+def search_dynamic_fp(d, dst_dt):
+    """The reference's steps, with every conversion done as a search for the nearest representable value."""
+    rows, N = d.shape
+    g = d.reshape(rows, N // 16, 16)
+    amax = np.abs(g).max(axis=2)
+    r = (amax / np.float32(FP_MAX[dst_dt])).astype(np.float32)
+    r = np.maximum(np.minimum(r, np.float32(448.0)), np.float32(0.125))
+    e4m3_pos = dtp.e4m3_to_f32(np.arange(0x7f, dtype=np.uint8)).astype(np.float64)     # codes 0 .. 0x7e, ascending
+    # f32 -> e4m3 goes through f16 in the reference (float8.cpp:269-274): two roundings, the first one numpy's
+    sbyte = nearest_even(r.astype(np.float16).astype(np.float64), e4m3_pos).astype(np.uint8)
+    inv = (np.float32(1.0) / e4m3_pos[sbyte].astype(np.float32)).astype(np.float32)
+    x = np.clip(g * inv[:, :, None], -FP_MAX[dst_dt], FP_MAX[dst_dt]).astype(np.float32).reshape(rows, N)
+    if dst_dt == cabi.DT_F4_E2M1:
+        codes = nearest_even(np.abs(x), E2M1).astype(np.uint8) | (np.signbit(x).astype(np.uint8) << 3)
+    else:
+        codes = nearest_even(np.abs(x).astype(np.float16).astype(np.float64), e4m3_pos).astype(np.uint8) \
+            | (np.signbit(x).astype(np.uint8) << 7)
+    return codes, sbyte
+
+
+def unpack_dst(raw, dst_dt, M, N):
+    raw = np.asarray(raw).view(np.uint8).reshape(-1)
+    if dst_dt == cabi.DT_F4_E2M1:
+        return np.stack([raw & 0xf, raw >> 4], axis=1).reshape(M, N)
+    return raw.reshape(M, N)
+
+
+def test_dynamic_fp_known_answers():
+    d = np.zeros((3, 32), np.float32)
+    d[0, :16] = np.linspace(-6, 6, 16)                # amax 6 -> scale 1
+    d[0, 16:] = 0.0                                   # zero group: the scale is clamped to 2^-3 from below
+    d[1, :16] = 6 * 448 * 4                           # beyond the scale range: 448, and the values saturate at 6
+    d[1, 16:] = 6 * 1.0625                            # 1.0625 lies halfway between the e4m3 values 1 and 1.125: even -> 1
+    d[2, :16] = 6 * 1.1875                            # halfway between 1.125 (odd code) and 1.25 (even code) -> 1.25
+    d[2, 16:] = [3.0, -1.5, 0.25, 0.75, 1.25, 1.75, 2.5, 3.5, 5.0, -0.25, -5.0, 0.0, 6.0, -6.0, 0.1, 0.3]
+    p = dynamic_fp(f32_problem_plain(d, cabi.DT_F4_E2M1))
+    dst, sc = orc.run_oracle_dynamic(p)
+    sc = dtp.e4m3_to_f32(np.asarray(sc).reshape(3, 2))
+    codes = unpack_dst(dst, cabi.DT_F4_E2M1, 3, 32)
+    val = E2M1[codes & 7] * np.where(codes & 8, -1.0, 1.0)
+    assert sc[0, 0] == 1.0 and sc[0, 1] == 0.125 and np.all(val[0, 16:] == 0)
+    assert sc[1, 0] == 448.0 and np.all(val[1, :16] == 6.0)
+    assert sc[1, 1] == 1.0 and np.all(val[1, 16:] == 6.0)
+    assert sc[2, 0] == 1.25
+    # scale 1: halfway values go to the even code (0.25 -> 0, 0.75 -> 1, 1.25 -> 1, 1.75 -> 2, 2.5 -> 2, 3.5 -> 4, 5 -> 4)
+    assert sc[2, 1] == 1.0
+    assert np.array_equal(val[2, 16:], [3.0, -1.5, 0.0, 1.0, 1.0, 2.0, 2.0, 4.0, 4.0, -0.0, -4.0, 0.0, 6.0, -6.0, 0.0, 0.5])
+
+
+def f32_problem_plain(d, dst_dt):
+    M, N = d.shape
+    return MatmulProblem(M=M, N=N, K=M, src_dt=cabi.DT_F32, wei_dt=cabi.DT_F32, dst_dt=dst_dt,
+                         src=np.eye(M, dtype=np.float32), wei=np.ascontiguousarray(d, dtype=np.float32), name="dyn-fp")
+
+
+@pytest.mark.parametrize("dst", ["f4_e2m1", "f8_e4m3"])
+def test_dynamic_fp_oracle_follows_the_search_restatement(dst):
+    dst_dt = cabi.DT_F4_E2M1 if dst == "f4_e2m1" else cabi.DT_F8_E4M3
+    p = configs.config4(M=48, N=128, K=64)
+    p.post_ops = [PostOp(kind=cabi.PO_ELTWISE, alg=cabi.ELTWISE["relu"], alpha=0.25, scale=3.0), p.post_ops[1]]
+    p.dst_dt = cabi.DT_F32
+    pre = np.asarray(orc.run_oracle(p)).view(np.float32).reshape(p.M, p.N)
+    p.dst_dt = dst_dt
+    got, sc = orc.run_oracle_dynamic(dynamic_fp(p))
+    want, want_sc = search_dynamic_fp(pre, dst_dt)
+    assert np.array_equal(np.asarray(sc).reshape(p.M, p.N // 16), want_sc)
+    got = unpack_dst(got, dst_dt, p.M, p.N)
+    # -0 and +0 are one value for the search
+    zero = (want & (7 if dst_dt == cabi.DT_F4_E2M1 else 0x7f)) == 0
+    assert np.array_equal(np.where(zero, got & (7 if dst_dt == cabi.DT_F4_E2M1 else 0x7f), got), np.where(zero, 0, want))
+
+
+def test_dynamic_fp_rules_of_the_descriptor():
+    p = dynamic_fp(configs.config4(M=32, N=64, K=256))
+    p.dst_dt = cabi.DT_F4_E2M1
+    st, impl = cabi.query(p.desc())
+    assert st == cabi.SUCCESS and cabi.impl_name(impl) == "hip:ref:any"        # generic kernel only
+    assert cabi.query(p.desc(), cabi.IMPL_F8_MFMA)[0] == cabi.UNIMPLEMENTED
+    q = dynamic_fp(configs.config4(M=32, N=64, K=256))
+    q.dst_dt = cabi.DT_F4_E2M1
+    q.quant["dst_scale"].groups = (1, 32)
+    assert cabi.query(q.desc())[0] == cabi.INVALID_ARGUMENTS
+    q = dynamic_fp(configs.config4(M=32, N=64, K=256))
+    q.dst_dt = cabi.DT_F4_E2M1
+    q.quant["dst_scale"].dt = cabi.DT_E8M0
+    assert cabi.query(q.desc())[0] == cabi.INVALID_ARGUMENTS
+    # a 4-bit dst with static scales has no kernel
+    s = configs.config4(M=32, N=64, K=256)
+    s.dst_dt = cabi.DT_F4_E2M1
+    assert cabi.query(s.desc())[0] == cabi.UNIMPLEMENTED
+    # MX scales over a 4-bit dst (an MXFP4 output): generic kernel
+    m = dynamic(configs.config4(M=32, N=64, K=256))
+    m.dst_dt = cabi.DT_F4_E2M1
+    st, impl = cabi.query(m.desc())
+    assert st == cabi.SUCCESS and cabi.impl_name(impl) == "hip:ref:any"
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("mode", ["fp", "mx"])
+@pytest.mark.parametrize("dst", ["f4_e2m1", "f8_e4m3", "f8_e5m2"])
+def test_gpu_dynamic_fp_and_4bit_dst_are_bit_exact(gpu, oracle, dst, mode):
+    if mode == "mx" and dst != "f4_e2m1":
+        pytest.skip("covered above")
+    dst_dt = {"f4_e2m1": cabi.DT_F4_E2M1, "f8_e4m3": cabi.DT_F8_E4M3, "f8_e5m2": cabi.DT_F8_E5M2}[dst]
+    make = dynamic_fp if mode == "fp" else dynamic
+    # constructed groups over many binades, zero groups, huge groups
+    r = np.random.default_rng(5)
+    d = (r.standard_normal((16, 128)) * np.exp2(r.integers(-20, 24, size=(16, 8)).repeat(16, axis=1))).astype(np.float32)
+    d[0, :32] = 0.0
+    d[1, :16] = 1e30
+    p = make(f32_problem_plain(d, dst_dt))
+    got, sc, name = run_gpu_dynamic(p, cabi.IMPL_REF)
+    want, want_sc = orc.run_oracle_dynamic(p)
+    assert name == "hip:ref:any"
+    assert np.array_equal(np.asarray(sc).reshape(-1), np.asarray(want_sc).reshape(-1))
+    assert np.array_equal(np.asarray(got).view(np.uint8), np.asarray(want).view(np.uint8))
+    # a matmul with bias, leaky relu and a residual add before the quantization
+    p = configs.config4(M=80, N=192, K=128)
+    p.post_ops = [PostOp(kind=cabi.PO_ELTWISE, alg=cabi.ELTWISE["relu"], alpha=0.25, scale=3.0), p.post_ops[1]]
+    p.dst_dt = dst_dt
+    p = make(p)
+    got, sc, name = run_gpu_dynamic(p)
+    want, want_sc = orc.run_oracle_dynamic(p)
+    assert name == "hip:ref:any"
+    assert np.array_equal(np.asarray(sc).reshape(-1), np.asarray(want_sc).reshape(-1))
+    assert np.array_equal(np.asarray(got).view(np.uint8), np.asarray(want).view(np.uint8))

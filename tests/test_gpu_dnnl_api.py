@@ -247,27 +247,35 @@ def test_prepack_decode_weights_with_reorder_then_matmul(gpu, oracle):
     assert_close(p, dst.read(np.uint16), want, abs_sum=asum * 20.0, what=pd.impl_info_str())
 
 
-def test_dynamic_mx_dst_through_the_api(gpu, oracle):
-    """quantization_mode::dynamic_mx on DNNL_ARG_DST: the scales memory is an
-    output of execute (ref_matmul.cpp:338-423)."""
+@pytest.mark.parametrize("flavour", ["mx", "nvfp4"])
+def test_dynamic_dst_scales_through_the_api(gpu, oracle, flavour):
+    """quantization_mode::dynamic_mx (e8m0 per 32, e4m3 dst) and ::dynamic_fp
+    (f8_e4m3 per 16, f4_e2m1 dst: NVFP4) on DNNL_ARG_DST: the scales memory is
+    an output of execute (ref_matmul.cpp:338-423)."""
+    mx = flavour == "mx"
+    G = 32 if mx else 16
+    sdt = "e8m0" if mx else "f8_e4m3"
+    ddt = "f8_e4m3" if mx else "f4_e2m1"
     from onednn_amd.problem import PostOp, QuantParam
     from oracle import binding as orc
     p = configs.config4(M=64, N=256, K=128)
     p.post_ops = [PostOp(kind=cabi.PO_ELTWISE, alg=cabi.ELTWISE["relu"], alpha=0.0, scale=1.0)]
-    p.dst_dt = cabi.DT_F8_E4M3
-    p.quant["dst_scale"] = QuantParam(cabi.DT_E8M0, 6, np.zeros((1, p.M, p.N // 32), np.uint8), (1, 32))
-    p.dst_dynamic = cabi.DST_DYNAMIC_MX
+    p.dst_dt = DT[ddt]
+    p.quant["dst_scale"] = QuantParam(DT[sdt], 6, np.zeros((1, p.M, p.N // G), np.uint8), (1, G))
+    p.dst_dynamic = cabi.DST_DYNAMIC_MX if mx else cabi.DST_DYNAMIC_FP
     M, K, N = p.M, p.K, p.N
     eng = dnnl.engine(dnnl.gpu, 0)
     strm = dnnl.stream(eng)
     src_md = dnnl.memory_desc([M, K], DT["f8_e4m3"], tag=dnnl.tag_ab)
     wei_md = dnnl.memory_desc([K, N], DT["f8_e4m3"], tag=dnnl.tag_ab)
-    dst_md = dnnl.memory_desc([M, N], DT["f8_e4m3"], tag=dnnl.tag_ab)
+    dst_md = dnnl.memory_desc([M, N], DT[ddt], tag=dnnl.tag_ab)
+    assert dst_md.get_size() == (M * N if mx else M * N // 2)
     bias_md = dnnl.memory_desc([1, N], DT["bf16"], tag=dnnl.tag_ab)
     attr = dnnl.primitive_attr()
     attr.set_scales_mask(dnnl.ARG_SRC, 0)
     attr.set_scales_mask(dnnl.ARG_WEIGHTS, 0)
-    attr.set_scales(dnnl.ARG_DST, 3, (1, 32), DT["e8m0"], qmode=dnnl.quantization_mode_dynamic_mx)
+    attr.set_scales(dnnl.ARG_DST, 3, (1, G), DT[sdt],
+                    qmode=dnnl.quantization_mode_dynamic_mx if mx else dnnl.quantization_mode_dynamic_fp)
     po = dnnl.post_ops()
     po.append_eltwise(cabi.ELTWISE["relu"], 0.0, 0.0)
     attr.set_post_ops(po)
@@ -276,7 +284,7 @@ def test_dynamic_mx_dst_through_the_api(gpu, oracle):
     while pd.impl_info_str() != "hip:ref:any":
         assert pd.next_impl()
     one = dnnl.memory_desc([1], DT["f32"], tag=dnnl.tag_a)
-    sc_md = dnnl.memory_desc([M, N // 32], DT["e8m0"], tag=dnnl.tag_ab)
+    sc_md = dnnl.memory_desc([M, N // G], DT[sdt], tag=dnnl.tag_ab)
     sc_mem = dnnl.memory(sc_md, eng)
     dst = dnnl.memory(dst_md, eng)
     dnnl.matmul(pd).execute(strm, {
