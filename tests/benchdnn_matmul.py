@@ -185,6 +185,12 @@ def build_problem(sp, seed=7):
             mask, shape = MASK_ROW, (r,)
         elif policy in ("per_ocic", "per_tensor", "per_dim_01"):
             mask, shape = MASK_ROW | MASK_COL, (r // groups[0], c // groups[1])
+        elif policy in ("dynamic_mx", "dynamic_fp"):
+            # dst:dynamic_fp:f8_e4m3:1x16 -- the scales are an output of the matmul
+            if arg != "dst" or not is_scale:
+                raise ValueError("dynamic quantization is a dst scale mode")
+            kw["dst_dynamic"] = cabi.DST_DYNAMIC_MX if policy == "dynamic_mx" else cabi.DST_DYNAMIC_FP
+            return QuantParam(dt, MASK_ROW | MASK_COL, np.zeros((r // groups[0], c // groups[1]), np.uint8), groups)
         else:
             raise ValueError(f"policy {policy}")
         if value is not None and policy == "common":
@@ -273,7 +279,12 @@ def api_objects(p, want_ref_impl=False, runtime_dims_masks=""):
         groups = q.groups if q.groups != (1, 1) else ()
         dims = {"src": (p.M, p.K), "wei": (p.K, p.N), "dst": (p.M, p.N)}[which]
         qdims = [dims[0] // q.groups[0] if mask2d & 1 else 1, dims[1] // q.groups[1] if mask2d & 2 else 1]
-        if kind == "scale":
+        if kind == "scale" and which == "dst" and p.dst_dynamic:
+            attr.set_scales(arg, mask2d, groups, q.dt, qmode={
+                cabi.DST_DYNAMIC_MX: dnnl.quantization_mode_dynamic_mx,
+                cabi.DST_DYNAMIC_FP: dnnl.quantization_mode_dynamic_fp}[p.dst_dynamic])
+            flag = dnnl.ARG_ATTR_SCALES
+        elif kind == "scale":
             attr.set_scales(arg, mask2d, groups, q.dt)
             flag = dnnl.ARG_ATTR_SCALES
         else:
@@ -331,6 +342,15 @@ def run_spec(sp, mode="C", min_times=5, max_ms=300.0):
         prim.execute(strm, args)
         strm.wait()
         got = dst.read(storage_dtype(p.dst_dt))
+        if p.dst_dynamic:
+            # exact fills: the K sums are exact, so dst and the scales the matmul wrote compare as bytes
+            want, want_sc = oracle.run_oracle_dynamic(p)
+            got_sc = args[dnnl.ARG_ATTR_SCALES | dnnl.ARG_DST].read(np.uint8)
+            nbad = int(np.count_nonzero(got_sc.reshape(-1) != np.asarray(want_sc).reshape(-1)))
+            nbad += int(np.count_nonzero(np.asarray(got).view(np.uint8).reshape(-1)
+                                         != np.asarray(want).view(np.uint8).reshape(-1)))
+            details["errors"] = nbad
+            return ("FAILED", impl, f"{nbad} bytes of dst / dst scales differ") if nbad else ("PASSED", impl, details)
         want, _, asum = oracle.run_oracle(p, want_ideal=True)
         transcendental = any(op.kind == cabi.PO_ELTWISE and op.alg not in (
             cabi.ELTWISE["relu"], cabi.ELTWISE["linear"], cabi.ELTWISE["clip"]) for op in p.post_ops)

@@ -77,6 +77,12 @@ LINES = [
     "10x30:30x20 300x128:128x260",
     "--dt=bf16:u4:bf16 --runtime_dims_masks=1:0 --attr-scales=wei:per_ocic:bf16:32x1 --attr-zero-points=wei:per_ocic:u4:32x1 "
     "--attr-fpmath=bf16:true 1x4096:4096x512 8x1024:1024x768",
+    # dynamic dst quantization: harness_matmul_generated_ci:17,186,344,397 (2-D analogues)
+    "--dt=f8_e5m2:f8_e5m2:f4_e2m1,f4_e2m1:f4_e2m1:f4_e2m1 --wtag=ab,ba "
+    "--attr-scales=src:per_tensor:e8m0:1x32+wei:per_oc:f32+dst:dynamic_fp:f8_e4m3:1x16 --attr-post-ops=,clip:-0.25:1.0 "
+    "76x288:288x352 1x64:64x2032",
+    "--dt=f8_e4m3:f8_e4m3:f8_e4m3,f8_e4m3:f8_e4m3:f4_e2m1 --bia-dt=f32 "
+    "--attr-scales=src:common:0.5+wei:common:0.25+dst:dynamic_mx:e8m0:1x32 --attr-post-ops=,relu 48x128:128x96",
     "--dt=f8_e4m3:f8_e4m3:bf16 --wtag=ba --runtime_dims_masks=3:3 --bia-dt=bf16 --attr-scales=src:common:0.5+wei:common:0.25 "
     "--attr-post-ops=relu+add:bf16 256x512:512x256",
 ]
