@@ -219,6 +219,15 @@ struct dnnl_primitive_desc {
     // execution from the descriptors of the memory objects
     // (exec_ctx_t::memory_mdw, src/common/primitive_exec_types.hpp:112-186)
     bool runtime = false;
+    // Batch dims that do not collapse into one stride per tensor (a tensor
+    // broadcast over some batch dims only): the leading `outer_n` batch dims
+    // are walked on the host, one launch per index, with these element
+    // strides; the remaining ones form the batch of a launch.
+    int outer_n = 0;
+    dim_t outer_dims[DNNL_MAX_NDIMS] = {};
+    dim_t outer_src[DNNL_MAX_NDIMS] = {}, outer_wei[DNNL_MAX_NDIMS] = {}, outer_dst[DNNL_MAX_NDIMS] = {},
+          outer_bias[DNNL_MAX_NDIMS] = {};
+    dim_t outer_po[MI355_MAX_POST_OPS][DNNL_MAX_NDIMS] = {};
 };
 
 struct dnnl_primitive {
@@ -451,20 +460,20 @@ dnnl_status_t check_attr(const dnnl_memory_desc &s, const dnnl_memory_desc &w, c
 // ------------------------------------------------- lowering to the C ABI
 // Collapse the batch dims of one operand into a single stride: all broadcast
 // (stride 0) or all present and nested.
-bool collapse_batch(const dnnl_memory_desc &x, const dnnl_memory_desc &dst, int64_t *bstride) {
+bool collapse_batch(const dnnl_memory_desc &x, const dnnl_memory_desc &dst, int64_t *bstride, int first = 0) {
     const int nb = dst.ndims - 2;
     *bstride = 0;
-    if (nb == 0) return true;
+    if (nb - first <= 0) return true;
     bool all_one = true, all_full = true;
-    for (int i = 0; i < nb; ++i) {
+    for (int i = first; i < nb; ++i) {
         if (x.dims[i] != 1) all_one = false;
         if (x.dims[i] != dst.dims[i]) all_full = false;
     }
     dim_t total = 1;
-    for (int i = 0; i < nb; ++i) total *= dst.dims[i];
+    for (int i = first; i < nb; ++i) total *= dst.dims[i];
     if (all_one && total > 1) return true; // broadcast
     if (!all_full) return false;
-    for (int i = 0; i + 1 < nb; ++i)
+    for (int i = first; i + 1 < nb; ++i)
         if (x.dims[i + 1] != 1 && x.strides[i] != x.strides[i + 1] * x.dims[i + 1]) return false;
     *bstride = x.strides[nb - 1];
     if (total == 1) *bstride = 0;
@@ -493,8 +502,43 @@ dnnl_status_t lower(dnnl_primitive_desc &pd) {
     mi355_matmul_desc_t &D = pd.desc;
     memset(&D, 0, sizeof(D));
     const int nd = pd.dst.ndims;
+    // the fewest leading batch dims to walk on the host so that the rest collapse in every tensor
+    int first = 0;
+    {
+        auto collapses = [&](int f) {
+            int64_t t;
+            if (!collapse_batch(pd.src, pd.dst, &t, f) || !collapse_batch(pd.dst, pd.dst, &t, f)) return false;
+            if (pd.wei.kind != dnnl_format_kind_opaque && !collapse_batch(pd.wei, pd.dst, &t, f)) return false;
+            if (pd.with_bias && !collapse_batch(pd.bias, pd.dst, &t, f)) return false;
+            for (const post_op_entry_t &e : pd.attr.post_ops.entries)
+                if (e.kind == dnnl_binary && !collapse_batch(e.src1, pd.dst, &t, f)) return false;
+            return true;
+        };
+        while (first < nd - 2 && !collapses(first)) ++first;
+    }
+    pd.outer_n = first;
+    if (first > 0) {
+        // parameters indexed by the batch would need the same walk: not offered
+        for (const auto *mp : {&pd.attr.scales, &pd.attr.zero_points, &pd.attr.reductions})
+            for (const auto &kv : *mp) CHECK_UNIMPL((kv.second.mask & ((1 << (nd - 2)) - 1)) == 0);
+        for (const post_op_entry_t &e : pd.attr.post_ops.entries)
+            CHECK_UNIMPL(e.kind != dnnl_prelu || (e.mask & ((1 << (nd - 2)) - 1)) == 0);
+        bool whole_bytes = true; // a 4-bit tensor is stepped by whole bytes
+        auto outer = [&](const dnnl_memory_desc &x, dim_t *out) {
+            for (int i = 0; i < first; ++i) {
+                out[i] = x.dims[i] == 1 ? 0 : x.strides[i];
+                if (dt_bits(x.dt) == 4 && (out[i] & 1)) whole_bytes = false;
+            }
+        };
+        for (int i = 0; i < first; ++i) pd.outer_dims[i] = pd.dst.dims[i];
+        outer(pd.src, pd.outer_src); outer(pd.wei, pd.outer_wei); outer(pd.dst, pd.outer_dst);
+        if (pd.with_bias) outer(pd.bias, pd.outer_bias);
+        for (size_t i = 0; i < pd.attr.post_ops.entries.size(); ++i)
+            if (pd.attr.post_ops.entries[i].kind == dnnl_binary) outer(pd.attr.post_ops.entries[i].src1, pd.outer_po[i]);
+        CHECK_UNIMPL(whole_bytes);
+    }
     dim_t batch = 1;
-    for (int i = 0; i < nd - 2; ++i) batch *= pd.dst.dims[i];
+    for (int i = first; i < nd - 2; ++i) batch *= pd.dst.dims[i];
     D.batch = batch;
     D.M = pd.dst.dims[nd - 2];
     D.N = pd.dst.dims[nd - 1];
@@ -502,7 +546,7 @@ dnnl_status_t lower(dnnl_primitive_desc &pd) {
     D.src_dt = pd.src.dt; D.wei_dt = pd.wei.dt; D.dst_dt = pd.dst.dt;
     D.bias_dt = pd.with_bias ? (int)pd.bias.dt : (int)MI355_DT_UNDEF;
     auto strides3 = [&](const dnnl_memory_desc &x, int64_t *out) -> bool {
-        if (!collapse_batch(x, pd.dst, &out[0])) return false;
+        if (!collapse_batch(x, pd.dst, &out[0], first)) return false;
         out[1] = x.dims[nd - 2] == 1 && pd.dst.dims[nd - 2] != 1 && &x != &pd.src && &x != &pd.wei ? 0 : x.strides[nd - 2];
         out[2] = x.dims[nd - 1] == 1 && pd.dst.dims[nd - 1] != 1 && &x != &pd.src && &x != &pd.wei ? 0 : x.strides[nd - 1];
         return true;
@@ -554,7 +598,7 @@ dnnl_status_t lower(dnnl_primitive_desc &pd) {
             case dnnl_binary: {
                 o.kind = MI355_PO_BINARY; o.alg = e.alg; o.dt = e.src1.dt;
                 int64_t st[3];
-                if (!collapse_batch(e.src1, pd.dst, &st[0])) return dnnl_unimplemented;
+                if (!collapse_batch(e.src1, pd.dst, &st[0], first)) return dnnl_unimplemented;
                 st[1] = e.src1.dims[nd - 2] == 1 ? 0 : e.src1.strides[nd - 2];
                 st[2] = e.src1.dims[nd - 1] == 1 ? 0 : e.src1.strides[nd - 1];
                 if (pd.dst.dims[nd - 2] == 1) st[1] = e.src1.strides[nd - 2];
@@ -1566,7 +1610,34 @@ DNNL_EXPORT dnnl_status_t dnnl_primitive_execute(const_dnnl_primitive_t cprimiti
     }
     if (mi355_device_set((int)pd.engine->index) != MI355_SUCCESS) return dnnl_runtime_error;
     const auto t0 = std::chrono::steady_clock::now();
-    const int rc = mi355_matmul_launch(&pd.desc, &A, scratch, stream->hip_stream);
+    int rc = MI355_SUCCESS;
+    if (pd.outer_n == 0) {
+        rc = mi355_matmul_launch(&pd.desc, &A, scratch, stream->hip_stream);
+    } else {
+        // one launch per index of the batch dims that are walked on the host (in stream order: they share the scratch)
+        dim_t count = 1;
+        for (int i = 0; i < pd.outer_n; ++i) count *= pd.outer_dims[i];
+        auto shifted = [](const void *base, dim_t elems, int dt) -> const void * {
+            return base ? (const char *)base + elems * dt_bits(dt) / 8 : nullptr;
+        };
+        for (dim_t it = 0; it < count && rc == MI355_SUCCESS; ++it) {
+            dim_t idx = it, os = 0, ow = 0, od = 0, ob = 0, op[MI355_MAX_POST_OPS] = {};
+            for (int i = pd.outer_n - 1; i >= 0; --i) {
+                const dim_t c = idx % pd.outer_dims[i];
+                idx /= pd.outer_dims[i];
+                os += c * pd.outer_src[i]; ow += c * pd.outer_wei[i]; od += c * pd.outer_dst[i]; ob += c * pd.outer_bias[i];
+                for (int k = 0; k < pd.desc.n_post_ops; ++k) op[k] += c * pd.outer_po[k][i];
+            }
+            mi355_matmul_args_t B = A;
+            B.src = shifted(A.src, os, pd.src.dt);
+            B.wei = shifted(A.wei, ow, pd.wei.dt);
+            B.dst = const_cast<void *>(shifted(A.dst, od, pd.dst.dt));
+            if (pd.with_bias) B.bias = shifted(A.bias, ob, pd.bias.dt);
+            for (int k = 0; k < pd.desc.n_post_ops; ++k)
+                if (pd.desc.post_ops[k].kind == MI355_PO_BINARY) B.po_arg[k] = shifted(A.po_arg[k], op[k], pd.desc.post_ops[k].dt);
+            rc = mi355_matmul_launch(&pd.desc, &B, scratch, stream->hip_stream);
+        }
+    }
     if (verbose_level() >= 2) {
         mi355_stream_sync(stream->hip_stream);
         const double ms = std::chrono::duration<double, std::milli>(std::chrono::steady_clock::now() - t0).count();

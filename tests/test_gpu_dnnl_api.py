@@ -388,3 +388,34 @@ def test_runtime_batch_dims_and_broadcast_weights(gpu):
                             dnnl.ARG_DST: dst})
         strm.wait()
         assert np.array_equal(dst.read(np.float32).reshape(B, M, N), s @ w)
+
+
+def test_batch_dims_broadcast_in_part(gpu):
+    # numpy broadcasting over the batch dims (matmul.cpp:722-735): src has one of the two batch dims, weights
+    # the other; bias and a binary operand broadcast in their own ways.  Small integers in f32: numpy is exact.
+    eng = dnnl.engine(dnnl.gpu, 0)
+    strm = dnnl.stream(eng)
+    f32 = DT["f32"]
+    r = np.random.default_rng(12)
+    M, K, N = 9, 24, 40
+    for sb, wb in (((2, 3), (2, 1)), ((1, 3), (2, 1)), ((2, 1), (1, 3)), ((2, 3), (1, 3))):
+        B = (max(sb[0], wb[0]), max(sb[1], wb[1]))
+        s = r.integers(-4, 5, size=sb + (M, K)).astype(np.float32)
+        w = r.integers(-4, 5, size=wb + (K, N)).astype(np.float32)
+        bias = r.integers(-4, 5, size=(1, B[1], 1, N)).astype(np.float32)
+        other = r.integers(-4, 5, size=(B[0], 1, M, 1)).astype(np.float32)
+        mds = [dnnl.memory_desc(list(x.shape), f32, tag=dnnl.tag_abcd) for x in (s, w, bias, other)]
+        dst_md = dnnl.memory_desc(list(B) + [M, N], f32, tag=dnnl.tag_abcd)
+        attr = dnnl.primitive_attr()
+        po = dnnl.post_ops()
+        po.append_binary(cabi.BINARY["mul"], mds[3])
+        attr.set_post_ops(po)
+        pd = dnnl.matmul_primitive_desc(eng, mds[0], mds[1], dst_md, bias_md=mds[2], attr=attr)
+        dst = dnnl.memory(dst_md, eng)
+        dnnl.matmul(pd).execute(strm, {
+            dnnl.ARG_SRC: dnnl.memory(mds[0], eng, s), dnnl.ARG_WEIGHTS: dnnl.memory(mds[1], eng, w),
+            dnnl.ARG_BIAS: dnnl.memory(mds[2], eng, bias), dnnl.ARG_DST: dst,
+            dnnl.ARG_ATTR_MULTIPLE_POST_OP(0) | dnnl.ARG_SRC_1: dnnl.memory(mds[3], eng, other)})
+        strm.wait()
+        want = ((s @ w) + bias) * other
+        assert np.array_equal(dst.read(np.float32).reshape(want.shape), want), (sb, wb)
