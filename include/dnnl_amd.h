@@ -106,7 +106,9 @@ typedef enum {
     dnnl_format_kind_undef = 0,
     dnnl_format_kind_any,
     dnnl_blocked,
-    dnnl_format_kind_opaque
+    dnnl_format_kind_opaque,
+    dnnl_format_kind_sparse,     /* declared for the enum values only: not offered */
+    dnnl_format_kind_host_scalar /* one value that lives in the memory object itself, on the host */
 } dnnl_format_kind_t;
 
 /* dnnl_types.h:175-209: only the plain tags with at most four dimensions */
@@ -256,6 +258,12 @@ size_t dnnl_data_type_size(dnnl_data_type_t data_type);
 /* ---- memory objects: dnnl.h:1482-1705 ---- */
 dnnl_status_t dnnl_memory_create(dnnl_memory_t *memory, const_dnnl_memory_desc_t memory_desc,
         dnnl_engine_t engine, void *handle);
+/* host-side scalars (dnnl.h:1196-1203, :1506-1520, :1676-1698): the value is copied into the memory object; a scale
+ * or zero point set with is_on_host = 1 takes such a memory at execution */
+dnnl_status_t dnnl_memory_desc_create_host_scalar(dnnl_memory_desc_t *memory_desc, dnnl_data_type_t data_type);
+dnnl_status_t dnnl_memory_create_host_scalar(dnnl_memory_t *memory, const_dnnl_memory_desc_t memory_desc, void *scalar_ptr);
+dnnl_status_t dnnl_memory_get_host_scalar_value(const_dnnl_memory_t memory, void *value);
+dnnl_status_t dnnl_memory_set_host_scalar_value(dnnl_memory_t memory, const void *value);
 dnnl_status_t dnnl_memory_get_memory_desc(const_dnnl_memory_t memory, const_dnnl_memory_desc_t *memory_desc);
 dnnl_status_t dnnl_memory_get_engine(const_dnnl_memory_t memory, dnnl_engine_t *engine);
 dnnl_status_t dnnl_memory_map_data(const_dnnl_memory_t memory, void **mapped_ptr);
@@ -288,6 +296,9 @@ dnnl_status_t dnnl_primitive_attr_set_scales_v3(dnnl_primitive_attr_t attr, int 
 dnnl_status_t dnnl_primitive_attr_set_scales(dnnl_primitive_attr_t attr, int arg, int mask, int group_ndims,
         const dnnl_dims_t group_dims, dnnl_data_type_t data_type);
 dnnl_status_t dnnl_primitive_attr_set_zero_points_mask(dnnl_primitive_attr_t attr, int arg, int mask);
+/* dnnl.h:654-659: is_on_host = 1 makes the (single, mask 0) zero point a host-side scalar */
+dnnl_status_t dnnl_primitive_attr_set_zero_points_v2(dnnl_primitive_attr_t attr, int arg, int mask, int group_ndims,
+        const dnnl_dims_t group_dims, dnnl_data_type_t data_type, int is_on_host);
 dnnl_status_t dnnl_primitive_attr_set_zero_points(dnnl_primitive_attr_t attr, int arg, int mask,
         int group_ndims, const dnnl_dims_t group_dims, dnnl_data_type_t data_type);
 dnnl_status_t dnnl_primitive_attr_set_precomputed_reductions(dnnl_primitive_attr_t attr, int arg, int mask,

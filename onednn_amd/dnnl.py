@@ -142,6 +142,29 @@ class memory_desc:
         return v.value
 
 
+class host_scalar:
+    """dnnl::memory of a host-side scalar (dnnl_memory_create_host_scalar): the
+    value lives in the object; `value` is a numpy scalar of the storage type."""
+
+    def __init__(self, dt, value):
+        self.mdh = C.c_void_p()
+        _check(lib().dnnl_memory_desc_create_host_scalar(C.byref(self.mdh), dt), "memory_desc_create_host_scalar")
+        self.md = memory_desc(handle=self.mdh.value)
+        self.h = C.c_void_p()
+        v = np.ascontiguousarray(value).reshape(1)
+        _check(lib().dnnl_memory_create_host_scalar(C.byref(self.h), self.mdh, C.c_void_p(v.ctypes.data)),
+               "memory_create_host_scalar")
+
+    def set(self, value):
+        v = np.ascontiguousarray(value).reshape(1)
+        _check(lib().dnnl_memory_set_host_scalar_value(self.h, C.c_void_p(v.ctypes.data)), "set_host_scalar_value")
+
+    def get(self, dtype):
+        out = np.zeros(1, dtype)
+        _check(lib().dnnl_memory_get_host_scalar_value(self.h, C.c_void_p(out.ctypes.data)), "get_host_scalar_value")
+        return out[0]
+
+
 class memory:
     """Device memory; `data` (numpy, raw storage) is uploaded through map/unmap."""
 
@@ -216,7 +239,11 @@ class primitive_attr:
     def set_zero_points_mask(self, arg, mask):
         _check(lib().dnnl_primitive_attr_set_zero_points_mask(self.h, arg, mask), "set_zero_points_mask")
 
-    def set_zero_points(self, arg, mask, groups=(), dt=cabi.DT_S32):
+    def set_zero_points(self, arg, mask, groups=(), dt=cabi.DT_S32, is_on_host=0):
+        if is_on_host:
+            _check(lib().dnnl_primitive_attr_set_zero_points_v2(
+                self.h, arg, mask, len(groups), _dims(groups), dt, is_on_host), "set_zero_points_v2")
+            return
         _check(lib().dnnl_primitive_attr_set_zero_points(self.h, arg, mask, len(groups), _dims(groups), dt),
                "set_zero_points")
 

@@ -159,6 +159,7 @@ struct dnnl_memory {
     void *handle = nullptr;
     bool owned = false;
     void *mapped = nullptr; // host staging buffer while mapped
+    unsigned char scalar[8] = {}; // md.kind == dnnl_format_kind_host_scalar: the value
 };
 
 namespace {
@@ -169,6 +170,7 @@ struct quant_entry_t {
     dim_t groups[2] = {1, 1};
     dim_t group(int d) const { return group_ndims == 0 ? 1 : groups[d]; }
     dnnl_quantization_mode_t qmode = dnnl_quantization_mode_static_sazp;
+    bool on_host = false; // the single value is handed over in a host-scalar memory object
     bool is_mx() const { return qmode == dnnl_quantization_mode_dynamic_mx; }
     bool is_dynamic_fp() const { return qmode == dnnl_quantization_mode_dynamic_fp; }
     bool is_dynamic() const { return is_mx() || is_dynamic_fp(); }
@@ -237,6 +239,8 @@ struct dnnl_primitive {
     // runtime dims: the lowering of the last executed shapes, and the scratch
     // buffers allocated for executions so far (kept until the primitive is
     // destroyed: earlier launches may still be running on their stream)
+    // device copies of host-side scalar scales / zero points, refreshed in stream order at each execution
+    void *host_scalars = nullptr;
     std::unique_ptr<dnnl_primitive_desc> rt_pd;
     std::vector<void *> rt_scratch;
     size_t rt_scratch_bytes = 0;
@@ -893,6 +897,7 @@ DNNL_EXPORT int dnnl_memory_desc_equal(const_dnnl_memory_desc_t lhs, const_dnnl_
     return *lhs == *rhs;
 }
 DNNL_EXPORT size_t dnnl_memory_desc_get_size(const_dnnl_memory_desc_t md) {
+    if (md && md->kind == dnnl_format_kind_host_scalar) return dt_bits(md->dt) / 8;
     if (!md || (md->kind != dnnl_blocked && md->kind != dnnl_format_kind_opaque)) return 0;
     return md->size_bytes();
 }
@@ -906,6 +911,7 @@ DNNL_EXPORT dnnl_status_t dnnl_memory_create(dnnl_memory_t *memory, const_dnnl_m
     CHECK_ARG(memory && md && engine);
     CHECK_ARG(md->kind != dnnl_format_kind_any);
     CHECK_ARG(!md->has_runtime()); // src/common/memory.cpp:155
+    CHECK_ARG(md->kind != dnnl_format_kind_host_scalar); // :157, dnnl_memory_create_host_scalar makes those
     std::unique_ptr<dnnl_memory> m(new dnnl_memory);
     m->md = *md;
     m->engine = engine;
@@ -918,6 +924,42 @@ DNNL_EXPORT dnnl_status_t dnnl_memory_create(dnnl_memory_t *memory, const_dnnl_m
         m->handle = handle;
     }
     *memory = m.release();
+    return dnnl_success;
+}
+// src/common/memory.cpp:219-241, :303-333
+DNNL_EXPORT dnnl_status_t dnnl_memory_desc_create_host_scalar(dnnl_memory_desc_t *memory_desc, dnnl_data_type_t data_type) {
+    CHECK_ARG(memory_desc);
+    CHECK_ARG(dt_valid(data_type) && dt_bits(data_type) >= 8);
+    std::unique_ptr<dnnl_memory_desc> md(new dnnl_memory_desc);
+    md->ndims = 1;
+    md->dims[0] = 1;
+    md->strides[0] = 1;
+    md->dt = data_type;
+    md->kind = dnnl_format_kind_host_scalar;
+    *memory_desc = md.release();
+    return dnnl_success;
+}
+DNNL_EXPORT dnnl_status_t dnnl_memory_create_host_scalar(dnnl_memory_t *memory, const_dnnl_memory_desc_t md,
+        void *scalar_ptr) {
+    CHECK_ARG(memory && md && scalar_ptr);
+    CHECK_ARG(md->kind == dnnl_format_kind_host_scalar);
+    std::unique_ptr<dnnl_memory> m(new dnnl_memory);
+    m->md = *md;
+    m->engine = nullptr;
+    memcpy(m->scalar, scalar_ptr, dt_bits(md->dt) / 8);
+    *memory = m.release();
+    return dnnl_success;
+}
+DNNL_EXPORT dnnl_status_t dnnl_memory_get_host_scalar_value(const_dnnl_memory_t memory, void *value) {
+    CHECK_ARG(memory && value);
+    CHECK_ARG(memory->md.kind == dnnl_format_kind_host_scalar);
+    memcpy(value, memory->scalar, dt_bits(memory->md.dt) / 8);
+    return dnnl_success;
+}
+DNNL_EXPORT dnnl_status_t dnnl_memory_set_host_scalar_value(dnnl_memory_t memory, const void *value) {
+    CHECK_ARG(memory && value);
+    CHECK_ARG(memory->md.kind == dnnl_format_kind_host_scalar);
+    memcpy(memory->scalar, value, dt_bits(memory->md.dt) / 8);
     return dnnl_success;
 }
 DNNL_EXPORT dnnl_status_t dnnl_memory_get_memory_desc(const_dnnl_memory_t memory, const_dnnl_memory_desc_t *md) {
@@ -934,6 +976,7 @@ DNNL_EXPORT dnnl_status_t dnnl_memory_map_data(const_dnnl_memory_t cmemory, void
     CHECK_ARG(cmemory && mapped_ptr);
     dnnl_memory *memory = const_cast<dnnl_memory *>(cmemory);
     CHECK_ARG(!memory->mapped);
+    CHECK_ARG(memory->md.kind != dnnl_format_kind_host_scalar); // src/common/memory.cpp:265-297: value accessors only
     const size_t bytes = memory->md.size_bytes();
     if (!memory->handle || bytes == 0) {
         *mapped_ptr = nullptr;
@@ -962,11 +1005,13 @@ DNNL_EXPORT dnnl_status_t dnnl_memory_unmap_data(const_dnnl_memory_t cmemory, vo
 }
 DNNL_EXPORT dnnl_status_t dnnl_memory_get_data_handle(const_dnnl_memory_t memory, void **handle) {
     CHECK_ARG(memory && handle);
+    CHECK_ARG(memory->md.kind != dnnl_format_kind_host_scalar);
     *handle = memory->handle;
     return dnnl_success;
 }
 DNNL_EXPORT dnnl_status_t dnnl_memory_set_data_handle(dnnl_memory_t memory, void *handle) {
     CHECK_ARG(memory);
+    CHECK_ARG(memory->md.kind != dnnl_format_kind_host_scalar);
     if (memory->owned) {
         mi355_mem_free(memory->handle);
         memory->owned = false;
@@ -1069,9 +1114,11 @@ DNNL_EXPORT dnnl_status_t dnnl_primitive_attr_set_scales_v3(dnnl_primitive_attr_
     CHECK_ARG(qmode == dnnl_quantization_mode_static_sazp || qmode == dnnl_quantization_mode_dynamic_mx
             || qmode == dnnl_quantization_mode_dynamic_fp);
     CHECK_ARG(IMPLICATION(is_on_host, mask == 0 && group_ndims == 0));
-    CHECK_UNIMPL(!is_on_host);
     const dnnl_status_t st = dnnl_primitive_attr_set_scales(attr, arg, mask, group_ndims, group_dims, data_type);
-    if (st == dnnl_success) attr->scales[arg].qmode = qmode;
+    if (st == dnnl_success) {
+        attr->scales[arg].qmode = qmode;
+        attr->scales[arg].on_host = is_on_host != 0;
+    }
     return st;
 }
 DNNL_EXPORT dnnl_status_t dnnl_primitive_attr_set_scales_v2(dnnl_primitive_attr_t attr, int arg, int mask,
@@ -1092,6 +1139,14 @@ DNNL_EXPORT dnnl_status_t dnnl_primitive_attr_set_zero_points(dnnl_primitive_att
     CHECK_ARG(IMPLICATION(arg != DNNL_ARG_SRC && arg != DNNL_ARG_WEIGHTS, data_type == dnnl_s32 && group_ndims == 0));
     CHECK_ARG(IMPLICATION(group_ndims > 0, mask > 0));
     return set_quant(attr->zero_points, arg, mask, group_ndims, group_dims, data_type);
+}
+DNNL_EXPORT dnnl_status_t dnnl_primitive_attr_set_zero_points_v2(dnnl_primitive_attr_t attr, int arg, int mask,
+        int group_ndims, const dnnl_dims_t group_dims, dnnl_data_type_t data_type, int is_on_host) {
+    CHECK_ARG(attr);
+    CHECK_ARG(IMPLICATION(is_on_host, mask == 0 && group_ndims == 0)); // primitive_attr.cpp:700-702
+    const dnnl_status_t st = dnnl_primitive_attr_set_zero_points(attr, arg, mask, group_ndims, group_dims, data_type);
+    if (st == dnnl_success) attr->zero_points[arg].on_host = is_on_host != 0;
+    return st;
 }
 DNNL_EXPORT dnnl_status_t dnnl_primitive_attr_set_zero_points_mask(dnnl_primitive_attr_t attr, int arg, int mask) {
     return dnnl_primitive_attr_set_zero_points(attr, arg, mask, 0, nullptr, dnnl_s32);
@@ -1332,7 +1387,8 @@ DNNL_EXPORT dnnl_status_t dnnl_reorder_primitive_desc_create(dnnl_primitive_desc
     const int nd = src_desc->ndims;
     // scales / zero points on src and dst only (:106-111); everything else is not a reorder attribute
     for (const auto *m : {&a.scales, &a.zero_points})
-        for (const auto &kv : *m) CHECK_UNIMPL(kv.first == DNNL_ARG_SRC || kv.first == DNNL_ARG_DST);
+        for (const auto &kv : *m)
+            CHECK_UNIMPL((kv.first == DNNL_ARG_SRC || kv.first == DNNL_ARG_DST) && !kv.second.on_host);
     CHECK_UNIMPL(a.reductions.empty());
     mi355_reorder_desc_t &r = pd->rdesc;
     memset(&r, 0, sizeof(r));
@@ -1486,6 +1542,14 @@ DNNL_EXPORT dnnl_status_t dnnl_primitive_create(dnnl_primitive_t *primitive, con
         const int st = mi355_mem_alloc(&p->scratch, p->pd.scratch_bytes);
         if (st != MI355_SUCCESS) return from_mi355(st);
     }
+    bool any_on_host = false;
+    for (const auto *mp : {&p->pd.attr.scales, &p->pd.attr.zero_points})
+        for (const auto &kv : *mp) any_on_host |= kv.second.on_host;
+    if (any_on_host && p->pd.kind == dnnl_matmul) {
+        if (mi355_device_set((int)p->pd.engine->index) != MI355_SUCCESS) return dnnl_runtime_error;
+        const int st = mi355_mem_alloc(&p->host_scalars, 64);
+        if (st != MI355_SUCCESS) return from_mi355(st);
+    }
     *primitive = p.release();
     return dnnl_success;
 }
@@ -1499,6 +1563,7 @@ DNNL_EXPORT dnnl_status_t dnnl_primitive_destroy(dnnl_primitive_t primitive) {
     if (primitive) {
         if (primitive->scratch) mi355_mem_free(primitive->scratch);
         for (void *q : primitive->rt_scratch) mi355_mem_free(q);
+        if (primitive->host_scalars) mi355_mem_free(primitive->host_scalars);
         delete primitive;
     }
     return dnnl_success;
@@ -1577,12 +1642,38 @@ DNNL_EXPORT dnnl_status_t dnnl_primitive_execute(const_dnnl_primitive_t cprimiti
     TAKE(wei, DNNL_ARG_WEIGHTS, true);
     TAKE(dst, DNNL_ARG_DST, true);
     TAKE(bias, DNNL_ARG_BIAS, pd.with_bias);
-    TAKE(src_scale, DNNL_ARG_ATTR_SCALES | DNNL_ARG_SRC, pd.desc.src_scale.dt != MI355_DT_UNDEF);
-    TAKE(wei_scale, DNNL_ARG_ATTR_SCALES | DNNL_ARG_WEIGHTS, pd.desc.wei_scale.dt != MI355_DT_UNDEF);
-    TAKE(dst_scale, DNNL_ARG_ATTR_SCALES | DNNL_ARG_DST, pd.desc.dst_scale.dt != MI355_DT_UNDEF);
-    TAKE(src_zp, DNNL_ARG_ATTR_ZERO_POINTS | DNNL_ARG_SRC, pd.desc.src_zp.dt != MI355_DT_UNDEF);
-    TAKE(wei_zp, DNNL_ARG_ATTR_ZERO_POINTS | DNNL_ARG_WEIGHTS, pd.desc.wei_zp.dt != MI355_DT_UNDEF);
-    TAKE(dst_zp, DNNL_ARG_ATTR_ZERO_POINTS | DNNL_ARG_DST, pd.desc.dst_zp.dt != MI355_DT_UNDEF);
+    // a scale / zero point set with is_on_host takes a host-scalar memory object: its value goes to the primitive's
+    // device slot in stream order; any other one takes device memory
+    int slot = 0;
+    auto take_q = [&](const std::map<int, quant_entry_t> &mp, int arg, int flag, const mi355_quant_t &lowered,
+                          const void **field) -> dnnl_status_t {
+        const quant_entry_t *q = pd.attr.find(mp, arg);
+        auto it = m.find(flag | arg);
+        dnnl_memory_t mem = it == m.end() ? nullptr : it->second;
+        const int my_slot = slot++;
+        if (q && q->on_host) {
+            CHECK_ARG(mem && mem->md.kind == dnnl_format_kind_host_scalar && (int)mem->md.dt == lowered.dt);
+            if (!prim->host_scalars) return dnnl_runtime_error;
+            void *dev = (char *)prim->host_scalars + 8 * my_slot;
+            const int rc = mi355_mem_h2d(dev, mem->scalar, dt_bits(mem->md.dt) / 8, stream->hip_stream);
+            if (rc != MI355_SUCCESS) return from_mi355(rc);
+            *field = dev;
+            return dnnl_success;
+        }
+        CHECK_ARG(!mem || mem->md.kind != dnnl_format_kind_host_scalar);
+        void *h = nullptr;
+        const dnnl_status_t hs = handle(flag | arg, lowered.dt != MI355_DT_UNDEF, &h);
+        *field = h;
+        return hs;
+    };
+    if (mi355_device_set((int)pd.engine->index) != MI355_SUCCESS) return dnnl_runtime_error;
+    const dnnl_primitive_attr &at = pd.attr;
+    if ((st = take_q(at.scales, DNNL_ARG_SRC, DNNL_ARG_ATTR_SCALES, pd.desc.src_scale, &A.src_scale))) return st;
+    if ((st = take_q(at.scales, DNNL_ARG_WEIGHTS, DNNL_ARG_ATTR_SCALES, pd.desc.wei_scale, &A.wei_scale))) return st;
+    if ((st = take_q(at.scales, DNNL_ARG_DST, DNNL_ARG_ATTR_SCALES, pd.desc.dst_scale, &A.dst_scale))) return st;
+    if ((st = take_q(at.zero_points, DNNL_ARG_SRC, DNNL_ARG_ATTR_ZERO_POINTS, pd.desc.src_zp, &A.src_zp))) return st;
+    if ((st = take_q(at.zero_points, DNNL_ARG_WEIGHTS, DNNL_ARG_ATTR_ZERO_POINTS, pd.desc.wei_zp, &A.wei_zp))) return st;
+    if ((st = take_q(at.zero_points, DNNL_ARG_DST, DNNL_ARG_ATTR_ZERO_POINTS, pd.desc.dst_zp, &A.dst_zp))) return st;
     TAKE(src_pr, DNNL_ARG_ATTR_PRECOMPUTED_REDUCTIONS | DNNL_ARG_SRC, pd.desc.src_pr.dt != MI355_DT_UNDEF);
     for (int i = 0; i < pd.desc.n_post_ops; ++i) {
         const int kind = pd.desc.post_ops[i].kind;

@@ -274,7 +274,7 @@ def test_dynamic_mx_dst_scales_rules(eng):
     # a 4-bit dst without dynamic scales has no implementation here
     assert status_of(lambda: make_pd(eng, 64, 128, 256, "f8_e4m3", "f8_e4m3", "f4_e2m1")) == dnnl.unimplemented
     assert status_of(lambda: a.set_scales(dnnl.ARG_DST, 1, (), DT["f32"], is_on_host=1)) == dnnl.invalid_arguments
-    assert status_of(lambda: a.set_scales(dnnl.ARG_DST, 0, (), DT["f32"], is_on_host=1)) == dnnl.unimplemented
+    assert status_of(lambda: a.set_scales(dnnl.ARG_DST, 0, (), DT["f32"], is_on_host=1)) == dnnl.success
 
 
 def test_user_scratchpad_is_reported(eng):
@@ -401,3 +401,31 @@ def test_attributes_are_checked_with_runtime_dims_too(eng):
 def test_reorder_with_runtime_dims_is_unimplemented(eng):
     assert status_of(lambda: dnnl.reorder_primitive_desc(
         eng, md([R, 8], "f32"), eng, md([R, 8], "f32"))) == dnnl.unimplemented
+
+
+def test_host_scalar_memory_and_attributes(eng):
+    # dnnl.h:1196-1203,1506-1520,1676-1698; src/common/memory.cpp:157,219-241,265-333; primitive_attr.cpp:655-658,700-702
+    import numpy as np
+    hs = dnnl.host_scalar(DT["f32"], np.float32(0.25))
+    assert hs.md.format_kind() == 5 and hs.md.get_size() == 4           # dnnl_format_kind_host_scalar
+    assert hs.get(np.float32) == np.float32(0.25)
+    hs.set(np.float32(3.5))
+    assert hs.get(np.float32) == np.float32(3.5)
+    zp = dnnl.host_scalar(DT["s32"], np.int32(-7))
+    assert zp.get(np.int32) == -7
+    # an ordinary memory object cannot be made of the descriptor, and the value has no handle and no mapping
+    assert status_of(lambda: dnnl.memory(hs.md, eng)) == dnnl.invalid_arguments
+    p = C.c_void_p()
+    assert dnnl.lib().dnnl_memory_get_data_handle(hs.h, C.byref(p)) == dnnl.invalid_arguments
+    assert dnnl.lib().dnnl_memory_map_data(hs.h, C.byref(p)) == dnnl.invalid_arguments
+    # only a single value can live on the host
+    a = dnnl.primitive_attr()
+    assert status_of(lambda: a.set_scales(dnnl.ARG_WEIGHTS, 2, (), DT["f32"], is_on_host=1)) == dnnl.invalid_arguments
+    assert status_of(lambda: a.set_zero_points(dnnl.ARG_SRC, 1, (), DT["s32"], is_on_host=1)) == dnnl.invalid_arguments
+    a.set_scales(dnnl.ARG_SRC, 0, (), DT["f32"], is_on_host=1)
+    a.set_zero_points(dnnl.ARG_SRC, 0, (), DT["s32"], is_on_host=1)
+    assert make_pd(eng, 64, 128, 256, "u8", "s8", "f32", attr=a).impl_info_str().startswith("hip:mfma_i8")
+    # reorder: device-side parameters only
+    r = dnnl.primitive_attr()
+    r.set_scales(dnnl.ARG_DST, 0, (), DT["f32"], is_on_host=1)
+    assert status_of(lambda: dnnl.reorder_primitive_desc(eng, md([8, 8], "f32"), eng, md([8, 8], "s8"), attr=r)) == dnnl.unimplemented

@@ -419,3 +419,67 @@ def test_batch_dims_broadcast_in_part(gpu):
         strm.wait()
         want = ((s @ w) + bias) * other
         assert np.array_equal(dst.read(np.float32).reshape(want.shape), want), (sb, wb)
+
+
+def test_host_side_scalar_scales_and_zero_points(gpu, oracle):
+    """Scales / zero points set with is_on_host take host-scalar memory objects
+    (dnnl.h:494-553,631-659): C3-like int8 problem with a src zero point, all
+    four single-valued parameters on the host, per-column weights scales on the
+    device.  The value is read at each execution: changing it changes the result."""
+    from onednn_amd.problem import QuantParam
+    p = configs.config3(M=96, N=160, K=256, wtag="ba")
+    p.src_dt = cabi.DT_U8
+    p.src = (np.asarray(p.src).view(np.uint8) ^ 0x80).astype(np.uint8)
+    p.quant["src_zp"] = QuantParam(cabi.DT_S32, 0, np.array([128], np.int32))
+    p.quant["dst_zp"] = QuantParam(cabi.DT_S32, 0, np.array([3], np.int32))
+    eng = dnnl.engine(dnnl.gpu, 0)
+    strm = dnnl.stream(eng)
+    mds = {"src": dnnl.memory_desc([p.M, p.K], p.src_dt, strides=list(p.src_stride[1:])),
+           "wei": dnnl.memory_desc([p.K, p.N], p.wei_dt, strides=list(p.wei_stride[1:])),
+           "dst": dnnl.memory_desc([p.M, p.N], p.dst_dt, strides=list(p.dst_stride[1:]))}
+    attr = dnnl.primitive_attr()
+    attr.set_scales(dnnl.ARG_SRC, 0, (), DT["f32"], is_on_host=1)
+    attr.set_scales(dnnl.ARG_DST, 0, (), DT["f32"], is_on_host=1)
+    attr.set_scales(dnnl.ARG_WEIGHTS, 2, (), DT["f32"])
+    attr.set_zero_points(dnnl.ARG_SRC, 0, (), DT["s32"], is_on_host=1)
+    attr.set_zero_points(dnnl.ARG_DST, 0, (), DT["s32"], is_on_host=1)
+    po = dnnl.post_ops()
+    for op in p.post_ops:
+        po.append_eltwise(op.alg, op.alpha, op.beta)
+    attr.set_post_ops(po)
+    pd = dnnl.matmul_primitive_desc(eng, mds["src"], mds["wei"], mds["dst"], attr=attr)
+    prim = dnnl.matmul(pd)
+    scal = {"src_scale": dnnl.host_scalar(DT["f32"], p.quant["src_scale"].data.reshape(-1)[0]),
+            "dst_scale": dnnl.host_scalar(DT["f32"], p.quant["dst_scale"].data.reshape(-1)[0]),
+            "src_zp": dnnl.host_scalar(DT["s32"], np.int32(128)), "dst_zp": dnnl.host_scalar(DT["s32"], np.int32(3))}
+    dst = dnnl.memory(mds["dst"], eng)
+    args = {dnnl.ARG_SRC: dnnl.memory(mds["src"], eng, p.src), dnnl.ARG_WEIGHTS: dnnl.memory(mds["wei"], eng, p.wei),
+            dnnl.ARG_DST: dst,
+            dnnl.ARG_ATTR_SCALES | dnnl.ARG_SRC: scal["src_scale"], dnnl.ARG_ATTR_SCALES | dnnl.ARG_DST: scal["dst_scale"],
+            dnnl.ARG_ATTR_SCALES | dnnl.ARG_WEIGHTS: dnnl.memory(dnnl.memory_desc([1, p.N], DT["f32"], tag=dnnl.tag_ab), eng,
+                                                                 p.quant["wei_scale"].data),
+            dnnl.ARG_ATTR_ZERO_POINTS | dnnl.ARG_SRC: scal["src_zp"], dnnl.ARG_ATTR_ZERO_POINTS | dnnl.ARG_DST: scal["dst_zp"]}
+    prim.execute(strm, args)
+    strm.wait()
+    assert_bit_exact(p, dst.read(np.int8), oracle.run_oracle(p), pd.impl_info_str())
+    # new values in the same memory objects, same primitive
+    scal["dst_scale"].set(np.float32(0.125))
+    scal["dst_zp"].set(np.int32(-5))
+    scal["src_zp"].set(np.int32(120))
+    p.quant["dst_scale"].data = np.array([0.125], np.float32)
+    p.quant["dst_zp"].data = np.array([-5], np.int32)
+    p.quant["src_zp"].data = np.array([120], np.int32)
+    prim.execute(strm, args)
+    strm.wait()
+    assert_bit_exact(p, dst.read(np.int8), oracle.run_oracle(p), pd.impl_info_str())
+    # a device memory where a host scalar is expected, and the other way round
+    bad = dict(args)
+    bad[dnnl.ARG_ATTR_SCALES | dnnl.ARG_SRC] = dnnl.memory(dnnl.memory_desc([1], DT["f32"], tag=dnnl.tag_a), eng)
+    with pytest.raises(dnnl.error) as e:
+        prim.execute(strm, bad)
+    assert e.value.status == dnnl.invalid_arguments
+    bad = dict(args)
+    bad[dnnl.ARG_ATTR_SCALES | dnnl.ARG_WEIGHTS] = dnnl.host_scalar(DT["f32"], np.float32(1))
+    with pytest.raises(dnnl.error) as e:
+        prim.execute(strm, bad)
+    assert e.value.status == dnnl.invalid_arguments
