@@ -159,6 +159,14 @@ typedef enum {
     dnnl_eltwise_round,
     dnnl_eltwise_mish,
     dnnl_eltwise_hardswish,
+    /* the forward computation of the base algorithm (primitive_attr_postops.cpp:74-82) */
+    dnnl_eltwise_relu_use_dst_for_bwd = 0x100,
+    dnnl_eltwise_tanh_use_dst_for_bwd,
+    dnnl_eltwise_elu_use_dst_for_bwd,
+    dnnl_eltwise_sqrt_use_dst_for_bwd,
+    dnnl_eltwise_logistic_use_dst_for_bwd,
+    dnnl_eltwise_exp_use_dst_for_bwd,
+    dnnl_eltwise_clip_v2_use_dst_for_bwd,
     dnnl_binary_add = 0x1fff0,
     dnnl_binary_mul = 0x1fff1,
     dnnl_binary_max = 0x1fff2,

@@ -598,7 +598,20 @@ dnnl_status_t lower(dnnl_primitive_desc &pd) {
         o.alpha = e.alpha; o.beta = e.beta; o.scale = e.scale; o.zero_point = e.zero_point;
         switch (e.kind) {
             case dnnl_sum: o.kind = MI355_PO_SUM; o.dt = e.dt; break;
-            case dnnl_eltwise: o.kind = MI355_PO_ELTWISE; o.alg = e.alg; break;
+            case dnnl_eltwise:
+                o.kind = MI355_PO_ELTWISE;
+                // forward: a *_use_dst_for_bwd algorithm computes what its base one does (primitive_attr_postops.cpp:74-82)
+                switch (e.alg) {
+                    case dnnl_eltwise_relu_use_dst_for_bwd: o.alg = dnnl_eltwise_relu; break;
+                    case dnnl_eltwise_tanh_use_dst_for_bwd: o.alg = dnnl_eltwise_tanh; break;
+                    case dnnl_eltwise_elu_use_dst_for_bwd: o.alg = dnnl_eltwise_elu; break;
+                    case dnnl_eltwise_sqrt_use_dst_for_bwd: o.alg = dnnl_eltwise_sqrt; break;
+                    case dnnl_eltwise_logistic_use_dst_for_bwd: o.alg = dnnl_eltwise_logistic; break;
+                    case dnnl_eltwise_exp_use_dst_for_bwd: o.alg = dnnl_eltwise_exp; break;
+                    case dnnl_eltwise_clip_v2_use_dst_for_bwd: o.alg = dnnl_eltwise_clip_v2; break;
+                    default: o.alg = e.alg; break;
+                }
+                break;
             case dnnl_binary: {
                 o.kind = MI355_PO_BINARY; o.alg = e.alg; o.dt = e.src1.dt;
                 int64_t st[3];
@@ -1214,9 +1227,12 @@ DNNL_EXPORT dnnl_status_t dnnl_post_ops_get_params_sum(const_dnnl_post_ops_t pos
 DNNL_EXPORT dnnl_status_t dnnl_post_ops_append_eltwise(dnnl_post_ops_t post_ops, dnnl_alg_kind_t alg, float alpha,
         float beta) {
     CHECK_ARG(post_ops);
-    CHECK_ARG(alg >= dnnl_eltwise_relu && alg <= dnnl_eltwise_hardswish);
-    // is_eltwise_ok, src/common/math_utils.hpp:432-470
-    CHECK_ARG(IMPLICATION(alg == dnnl_eltwise_clip || alg == dnnl_eltwise_clip_v2, beta >= alpha));
+    const bool use_dst = alg >= dnnl_eltwise_relu_use_dst_for_bwd && alg <= dnnl_eltwise_clip_v2_use_dst_for_bwd;
+    CHECK_ARG((alg >= dnnl_eltwise_relu && alg <= dnnl_eltwise_hardswish) || use_dst);
+    // is_eltwise_ok, src/common/math_utils.hpp:432-456
+    CHECK_ARG(IMPLICATION(alg == dnnl_eltwise_clip || alg == dnnl_eltwise_clip_v2
+                    || alg == dnnl_eltwise_clip_v2_use_dst_for_bwd, beta >= alpha));
+    CHECK_ARG(IMPLICATION(alg == dnnl_eltwise_relu_use_dst_for_bwd || alg == dnnl_eltwise_elu_use_dst_for_bwd, alpha >= 0));
     if (po_full(post_ops)) return dnnl_out_of_memory;
     post_op_entry_t e;
     e.kind = dnnl_eltwise; e.alg = alg; e.alpha = alpha; e.beta = beta; e.scale = 1.f;

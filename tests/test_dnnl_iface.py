@@ -429,3 +429,21 @@ def test_host_scalar_memory_and_attributes(eng):
     r = dnnl.primitive_attr()
     r.set_scales(dnnl.ARG_DST, 0, (), DT["f32"], is_on_host=1)
     assert status_of(lambda: dnnl.reorder_primitive_desc(eng, md([8, 8], "f32"), eng, md([8, 8], "s8"), attr=r)) == dnnl.unimplemented
+
+
+def test_use_dst_for_bwd_eltwise_post_ops(eng):
+    # forward inference computes the base algorithm (primitive_attr_postops.cpp:74-82); the value rules of
+    # is_eltwise_ok (math_utils.hpp:442-453) hold at append time
+    po = dnnl.post_ops()
+    for alg in range(0x100, 0x107):
+        po2 = dnnl.post_ops()
+        po2.append_eltwise(alg, 0.5, 1.0)
+    assert status_of(lambda: po.append_eltwise(0x100, -1.0, 0.0)) == dnnl.invalid_arguments     # relu: alpha >= 0
+    assert status_of(lambda: po.append_eltwise(0x102, -1.0, 0.0)) == dnnl.invalid_arguments     # elu
+    assert status_of(lambda: po.append_eltwise(0x106, 2.0, 1.0)) == dnnl.invalid_arguments      # clip_v2: beta >= alpha
+    assert status_of(lambda: po.append_eltwise(0x107, 0.0, 0.0)) == dnnl.invalid_arguments
+    po.append_eltwise(0x100, 0.25, 0.0)
+    a = dnnl.primitive_attr()
+    a.set_post_ops(po)
+    pd = make_pd(eng, 64, 128, 256, "s8", "s8", "f32", attr=a)
+    assert pd.impl_info_str().startswith("hip:mfma_i8")           # lowered to plain relu: the fast epilogue takes it

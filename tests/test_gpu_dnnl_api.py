@@ -483,3 +483,16 @@ def test_host_side_scalar_scales_and_zero_points(gpu, oracle):
     with pytest.raises(dnnl.error) as e:
         prim.execute(strm, bad)
     assert e.value.status == dnnl.invalid_arguments
+
+
+def test_use_dst_for_bwd_eltwise_equals_its_base_algorithm(gpu):
+    from onednn_amd.problem import PostOp
+    base = {"relu": 0x100, "tanh": 0x101, "elu": 0x102, "sqrt": 0x103, "logistic": 0x104, "exp": 0x105, "clip_v2": 0x106}
+    for name, alias in base.items():
+        outs = []
+        for alg in (cabi.ELTWISE[name], alias):
+            p = configs.config1(M=64, N=128, K=128)
+            p.post_ops = [PostOp(kind=cabi.PO_ELTWISE, alg=alg, alpha=0.5, beta=2.0, scale=1.0)]
+            got, _, _ = run_through_api(p)
+            outs.append(np.asarray(got).view(np.uint32))
+        assert np.array_equal(outs[0], outs[1]), name
