@@ -145,8 +145,9 @@ enum {
  *             (2^-3 = epsilon of e4m3, src/common/nstl.hpp:189-191)
  * and the rest as above; N % 16 == 0.
  *
- * A 4-bit dst (f4_e2m1) is offered with dynamic scales only (generic kernel):
- * unit n stride and even m / batch strides, so that a group is whole bytes. */
+ * A 4-bit dst (f4_e2m1 with static or dynamic scales; s4 / u4 with static ones)
+ * is served by the generic kernel: even N, unit n stride and even m / batch
+ * strides, so that a thread writes whole bytes (low nibble = even n). */
 enum {
     MI355_DST_DYNAMIC_NONE = 0,
     MI355_DST_DYNAMIC_MX = 1,

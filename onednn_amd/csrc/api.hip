@@ -114,6 +114,8 @@ static int impl_supported(const mi355_matmul_desc_t &d, int impl) {
     if (d.dst_scale_dynamic != MI355_DST_DYNAMIC_NONE && impl != MI355_IMPL_REF && impl != MI355_IMPL_F8_MFMA
             && impl != MI355_IMPL_MXF4_MFMA)
         return MI355_UNIMPLEMENTED;
+    // a 4-bit dst: generic kernel only
+    if (dt_bits(d.dst_dt) < 8 && impl != MI355_IMPL_REF) return MI355_UNIMPLEMENTED;
     // the tiles' group reduction is the MX one (32 columns, fp8 dst)
     if ((d.dst_scale_dynamic == MI355_DST_DYNAMIC_FP || (d.dst_scale_dynamic && !is_f8_dt(d.dst_dt)))
             && impl != MI355_IMPL_REF)

@@ -125,6 +125,33 @@ __global__ void __launch_bounds__(256) ref_matmul_kernel(const problem_t P_) {
     }
 }
 
+// 4-bit dst (f4_e2m1, s4, u4) with static scales: two consecutive n share a
+// byte (low nibble first), so one thread computes both and writes the byte.
+// The host has checked: N even, unit n stride, even m / batch strides.
+__device__ __forceinline__ uint32_t nibble_code(int dt, float v) {
+    switch (dt) {
+        case MI355_DT_F4_E2M1: return f32_to_e2m1(v);
+        case MI355_DT_S4: return (uint32_t)(int)__builtin_rintf(sat(v, -8.f, 7.f)) & 0xfu;
+        default: return (uint32_t)(int)__builtin_rintf(sat(v, 0.f, 15.f)) & 0xfu;
+    }
+}
+
+__global__ void __launch_bounds__(256) ref_matmul_nibble_dst_kernel(const problem_t P_) {
+    const auto &P = MI355_KERNARG_PROBLEM();
+    const long half = P.N / 2, total = P.B * P.M * half;
+    const bool int_path = P.src_dt == MI355_DT_S8 || P.src_dt == MI355_DT_U8;
+    for (long i = (long)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += (long)gridDim.x * blockDim.x) {
+        const long n = (i % half) * 2, m = (i / half) % P.M, b = i / (half * P.M);
+        uint32_t byte = 0;
+#pragma unroll 1
+        for (int e = 0; e < 2; ++e) {
+            const float v = int_path ? ref_int_dot(P, b, m, n + e) : ref_fp_dot(P, b, m, n + e);
+            byte |= nibble_code(P.dst_dt, epilogue_value(P, v, b, m, n + e)) << (4 * e);
+        }
+        ((uint8_t *)P.dst)[(b * P.ds[0] + m * P.ds[1] + n) >> 1] = (uint8_t)byte;
+    }
+}
+
 // Dynamic (MX) quantization of dst, ref_matmul.cpp:268-423: one thread per
 // group of 32 consecutive n of a dst row.  The values of the group are
 // computed exactly as above, their largest magnitude gives the group's e8m0
@@ -187,11 +214,11 @@ __global__ void __launch_bounds__(64) ref_matmul_dynamic_kernel(const problem_t 
 }
 
 int ref_supported(const mi355_matmul_desc_t &d) {
-    // 4-bit dst: two elements share a byte.  Offered where one thread owns both:
-    // f4_e2m1 with dynamic scales (a thread per group of whole bytes).
+    // 4-bit dst: two elements share a byte, and one thread owns both (a thread
+    // per byte, or per group under dynamic scales): whole bytes per row needed
     if (dt_bits(d.dst_dt) < 8) {
-        if (d.dst_dt != MI355_DT_F4_E2M1 || d.dst_scale_dynamic == MI355_DST_DYNAMIC_NONE) return MI355_UNIMPLEMENTED;
-        if (d.dst_stride[2] != 1 || (d.dst_stride[1] & 1) || (d.dst_stride[0] & 1)) return MI355_UNIMPLEMENTED;
+        if (d.dst_scale_dynamic != MI355_DST_DYNAMIC_NONE && d.dst_dt != MI355_DT_F4_E2M1) return MI355_UNIMPLEMENTED;
+        if ((d.N & 1) || d.dst_stride[2] != 1 || (d.dst_stride[1] & 1) || (d.dst_stride[0] & 1)) return MI355_UNIMPLEMENTED;
     }
     if (d.wei_packing != MI355_WEI_PACK_NONE && !woq64_layout_ok(d)) return MI355_UNIMPLEMENTED;
     // dynamic dst quantization exists in ref_matmul_t only, not in the integer implementation
@@ -210,6 +237,12 @@ int ref_launch(const problem_t &P, hipStream_t stream) {
             hipLaunchKernelGGL(ref_matmul_dynamic_kernel<32>, dim3((unsigned)gblocks), dim3(64), 0, stream, P);
         else
             hipLaunchKernelGGL(ref_matmul_dynamic_kernel<16>, dim3((unsigned)gblocks), dim3(64), 0, stream, P);
+        return hipGetLastError() == hipSuccess ? MI355_SUCCESS : MI355_RUNTIME_ERROR;
+    }
+    if (dt_bits(P.dst_dt) < 8) {
+        long nblocks = (total / 2 + 255) / 256;
+        if (nblocks > 1048576) nblocks = 1048576;
+        hipLaunchKernelGGL(ref_matmul_nibble_dst_kernel, dim3((unsigned)nblocks), dim3(256), 0, stream, P);
         return hipGetLastError() == hipSuccess ? MI355_SUCCESS : MI355_RUNTIME_ERROR;
     }
     long blocks = (total + 255) / 256;

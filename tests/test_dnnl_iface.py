@@ -271,8 +271,8 @@ def test_dynamic_mx_dst_scales_rules(eng):
     assert status_of(lambda: make_pd(eng, 64, 128, 256, "f8_e4m3", "f8_e4m3", "f4_e2m1", attr=fp(dt=DT["e8m0"]))) == dnnl.unimplemented
     assert status_of(lambda: make_pd(eng, 64, 128, 256, "f8_e4m3", "f8_e4m3", "f4_e2m1", attr=fp(mask=2, groups=()))) == dnnl.unimplemented
     assert status_of(lambda: make_pd(eng, 64, 128, 256, "f8_e4m3", "f8_e4m3", "bf16", attr=fp())) == dnnl.unimplemented
-    # a 4-bit dst without dynamic scales has no implementation here
-    assert status_of(lambda: make_pd(eng, 64, 128, 256, "f8_e4m3", "f8_e4m3", "f4_e2m1")) == dnnl.unimplemented
+    # a 4-bit dst without dynamic scales: generic kernel
+    assert make_pd(eng, 64, 128, 256, "f8_e4m3", "f8_e4m3", "f4_e2m1").impl_info_str() == "hip:ref:any"
     assert status_of(lambda: a.set_scales(dnnl.ARG_DST, 1, (), DT["f32"], is_on_host=1)) == dnnl.invalid_arguments
     assert status_of(lambda: a.set_scales(dnnl.ARG_DST, 0, (), DT["f32"], is_on_host=1)) == dnnl.success
 
