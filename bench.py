@@ -41,10 +41,10 @@ import numpy as np  # noqa: E402
 # known 256 MiB (factors 2.0 and 1.0); the summaries with the commands are in
 # profiles/<kernel>_<workload>.md.  Keyed by (workload, M).
 MEASURED_TRAFFIC = {
-    ("c3", 8192): 1024824874, ("c4", 4096): 2124622179, ("c5", 8192): 569439623,
+    ("c3", 8192): 1078997046, ("c4", 4096): 2178641942, ("c5", 8192): 569460235,
     ("c2", 1): 31612633, ("c2", 8): 32271601, ("c2", 32): 34542741,        # packed weights (format any)
     ("c2ab", 1): 32839597, ("c2ab", 8): 35736697, ("c2ab", 32): 51670775,  # plain ab weights (--wtag ab)
-    ("c1", 256): 8645444,
+    ("c1", 256): 8657878,
     ("r1", 0): 335981182, ("r2", 0): 212392274, ("r3", 0): 58765379,
 }
 
