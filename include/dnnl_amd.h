@@ -178,7 +178,8 @@ typedef enum {
     dnnl_binary_le = 0x1fff8,
     dnnl_binary_lt = 0x1fff9,
     dnnl_binary_eq = 0x1fffa,
-    dnnl_binary_ne = 0x1fffb
+    dnnl_binary_ne = 0x1fffb,
+    dnnl_binary_select = 0x1fffc /* ternary: dst = src2 ? dst : src1 (dnnl_post_ops_append_binary_v2) */
 } dnnl_alg_kind_t;
 
 /* dnnl_types.h:2448-2458 */
@@ -209,6 +210,7 @@ typedef enum {
 /* execute argument ids, dnnl_types.h:2544-2784 */
 #define DNNL_ARG_SRC 1
 #define DNNL_ARG_SRC_1 2
+#define DNNL_ARG_SRC_2 3 /* dnnl_types.h:2562: the condition of a binary select post-op */
 #define DNNL_ARG_DST 17
 #define DNNL_ARG_WEIGHTS 33
 #define DNNL_ARG_BIAS 41
@@ -332,6 +334,11 @@ dnnl_status_t dnnl_post_ops_append_binary(dnnl_post_ops_t post_ops, dnnl_alg_kin
         const_dnnl_memory_desc_t src1_desc);
 dnnl_status_t dnnl_post_ops_get_params_binary(const_dnnl_post_ops_t post_ops, int index,
         dnnl_alg_kind_t *alg_kind, const_dnnl_memory_desc_t *src1_desc);
+/* dnnl.h: ternary binary post-op (select); src2_desc is NULL for every other algorithm */
+dnnl_status_t dnnl_post_ops_append_binary_v2(dnnl_post_ops_t post_ops, dnnl_alg_kind_t alg_kind,
+        const_dnnl_memory_desc_t src1_desc, const_dnnl_memory_desc_t src2_desc);
+dnnl_status_t dnnl_post_ops_get_params_binary_v2(const_dnnl_post_ops_t post_ops, int index,
+        dnnl_alg_kind_t *alg_kind, const_dnnl_memory_desc_t *src1_desc, const_dnnl_memory_desc_t *src2_desc);
 dnnl_status_t dnnl_post_ops_append_prelu(dnnl_post_ops_t post_ops, int mask);
 dnnl_status_t dnnl_post_ops_get_params_prelu(const_dnnl_post_ops_t post_ops, int index, int *mask);
 

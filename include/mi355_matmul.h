@@ -75,7 +75,13 @@ enum {
     MI355_PO_SUM = 1,
     MI355_PO_ELTWISE = 2,
     MI355_PO_BINARY = 3,
-    MI355_PO_PRELU = 4
+    MI355_PO_PRELU = 4,
+    /* The condition operand (src2) of the ternary binary post-op
+     * MI355_BINARY_SELECT, which must be the entry right before it:
+     * v = cond != 0 ? v : src1 (primitive_attr_postops.cpp:44,345-360; the
+     * condition is loaded as an integer).  This entry carries dt, stride and
+     * po_arg of the condition and computes nothing by itself. */
+    MI355_PO_SELECT_COND = 5
 };
 
 /* Algorithm kinds: numeric values equal dnnl_alg_kind_t
@@ -113,7 +119,8 @@ enum {
     MI355_BINARY_LE = 0x1fff8,
     MI355_BINARY_LT = 0x1fff9,
     MI355_BINARY_EQ = 0x1fffa,
-    MI355_BINARY_NE = 0x1fffb
+    MI355_BINARY_NE = 0x1fffb,
+    MI355_BINARY_SELECT = 0x1fffc /* generic kernel only; see MI355_PO_SELECT_COND */
 };
 
 /* Which arithmetic flavour of "the reference's own matmul" to reproduce where

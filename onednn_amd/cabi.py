@@ -25,7 +25,7 @@ DT_BITS = {DT_F16: 16, DT_BF16: 16, DT_F32: 32, DT_S32: 32, DT_S8: 8, DT_U8: 8,
 
 SUCCESS, OUT_OF_MEMORY, INVALID_ARGUMENTS, UNIMPLEMENTED, LAST_IMPL_REACHED, RUNTIME_ERROR, NOT_REQUIRED = range(7)
 
-PO_SUM, PO_ELTWISE, PO_BINARY, PO_PRELU = 1, 2, 3, 4
+PO_SUM, PO_ELTWISE, PO_BINARY, PO_PRELU, PO_SELECT_COND = 1, 2, 3, 4, 5
 
 ELTWISE = {
     "relu": 0x20, "tanh": 0x21, "elu": 0x22, "square": 0x23, "abs": 0x24, "sqrt": 0x25,
@@ -36,7 +36,7 @@ ELTWISE = {
 BINARY = {
     "add": 0x1fff0, "mul": 0x1fff1, "max": 0x1fff2, "min": 0x1fff3, "div": 0x1fff4,
     "sub": 0x1fff5, "ge": 0x1fff6, "gt": 0x1fff7, "le": 0x1fff8, "lt": 0x1fff9,
-    "eq": 0x1fffa, "ne": 0x1fffb,
+    "eq": 0x1fffa, "ne": 0x1fffb, "select": 0x1fffc,
 }
 
 DST_SCALE_DIVIDE, DST_SCALE_RECIPROCAL = 0, 1

@@ -58,8 +58,17 @@ static int validate(const mi355_matmul_desc_t *d) {
     }
     for (int i = 0; i < d->n_post_ops; ++i) {
         const int k = d->post_ops[i].kind;
-        if (k < MI355_PO_SUM || k > MI355_PO_PRELU) {
+        if (k < MI355_PO_SUM || k > MI355_PO_SELECT_COND) {
             set_error("bad post-op kind at %d", i);
+            return MI355_INVALID_ARGUMENTS;
+        }
+        // a select and its condition come as a pair
+        const bool is_select = k == MI355_PO_BINARY && d->post_ops[i].alg == MI355_BINARY_SELECT;
+        const bool next_is_cond = i + 1 < d->n_post_ops && d->post_ops[i + 1].kind == MI355_PO_SELECT_COND;
+        const bool prev_is_select = i > 0 && d->post_ops[i - 1].kind == MI355_PO_BINARY
+                && d->post_ops[i - 1].alg == MI355_BINARY_SELECT;
+        if (is_select != next_is_cond || (k == MI355_PO_SELECT_COND) != prev_is_select) {
+            set_error("post-op %d: a binary select is followed by its condition entry, which follows nothing else", i);
             return MI355_INVALID_ARGUMENTS;
         }
     }
@@ -114,6 +123,9 @@ static int impl_supported(const mi355_matmul_desc_t &d, int impl) {
     if (d.dst_scale_dynamic != MI355_DST_DYNAMIC_NONE && impl != MI355_IMPL_REF && impl != MI355_IMPL_F8_MFMA
             && impl != MI355_IMPL_MXF4_MFMA)
         return MI355_UNIMPLEMENTED;
+    // the ternary select post-op: generic kernel only
+    for (int i = 0; i < d.n_post_ops; ++i)
+        if (d.post_ops[i].kind == MI355_PO_SELECT_COND && impl != MI355_IMPL_REF) return MI355_UNIMPLEMENTED;
     // a 4-bit dst: generic kernel only
     if (dt_bits(d.dst_dt) < 8 && impl != MI355_IMPL_REF) return MI355_UNIMPLEMENTED;
     // the tiles' group reduction is the MX one (32 columns, fp8 dst)
@@ -202,7 +214,7 @@ static int build_problem(const mi355_matmul_desc_t &d, const mi355_matmul_args_t
         o.zp = s.zero_point; o.dt = s.dt;
         o.s0 = s.stride[0]; o.s1 = s.stride[1]; o.s2 = s.stride[2];
         o.p = a.po_arg[i];
-        if ((s.kind == MI355_PO_BINARY || s.kind == MI355_PO_PRELU) && !o.p) {
+        if ((s.kind == MI355_PO_BINARY || s.kind == MI355_PO_PRELU || s.kind == MI355_PO_SELECT_COND) && !o.p) {
             set_error("missing post-op argument %d", i);
             return MI355_INVALID_ARGUMENTS;
         }

@@ -232,7 +232,13 @@ __device__ __forceinline__ float epilogue_value(
                 v = eltwise_f(po.alg, v, po.alpha, po.beta) * po.scale;
             } else if (po.kind == MI355_PO_BINARY) {
                 const float y = load_float(po.dt, po.p, b * po.s0 + m * po.s1 + n * po.s2);
-                v = binary_f(po.alg, v, y);
+                if (po.alg == MI355_BINARY_SELECT) {
+                    // the next entry holds the condition (checked by the host)
+                    const auto &c = P.po[i + 1];
+                    v = load_int(c.dt, c.p, b * c.s0 + m * c.s1 + n * c.s2) != 0 ? v : y;
+                } else {
+                    v = binary_f(po.alg, v, y);
+                }
             } else if (po.kind == MI355_PO_SUM) {
                 v += po.scale * (dst_old - (float)po.zp);
             } else if (po.kind == MI355_PO_PRELU) {

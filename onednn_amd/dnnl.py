@@ -29,6 +29,7 @@ query_format_kind = 262
 quantization_mode_undef, quantization_mode_static_sazp, quantization_mode_dynamic_mx, quantization_mode_dynamic_fp = 0, 1, 2, 3
 format_kind_undef, format_kind_any, format_kind_blocked, format_kind_opaque = 0, 1, 2, 3
 ARG_SRC, ARG_SRC_1, ARG_DST, ARG_WEIGHTS, ARG_BIAS, ARG_SCRATCHPAD = 1, 2, 17, 33, 41, 80
+ARG_SRC_2 = 3
 ARG_FROM, ARG_TO = ARG_SRC, ARG_DST
 ARG_ATTR_PRECOMPUTED_REDUCTIONS, ARG_ATTR_SCALES, ARG_ATTR_ZERO_POINTS = 512, 4096, 8192
 scratchpad_library, scratchpad_user = 0, 1
@@ -204,7 +205,10 @@ class post_ops:
     def append_eltwise(self, alg, alpha=0.0, beta=0.0):
         _check(lib().dnnl_post_ops_append_eltwise(self.h, alg, C.c_float(alpha), C.c_float(beta)), "append_eltwise")
 
-    def append_binary(self, alg, src1_md):
+    def append_binary(self, alg, src1_md, src2_md=None):
+        if src2_md is not None:
+            _check(lib().dnnl_post_ops_append_binary_v2(self.h, alg, src1_md.h, src2_md.h), "append_binary_v2")
+            return
         _check(lib().dnnl_post_ops_append_binary(self.h, alg, src1_md.h), "append_binary")
 
     def append_sum(self, scale=1.0, zero_point=0, dt=0):

@@ -183,6 +183,7 @@ struct post_op_entry_t {
     int32_t zero_point = 0;
     dnnl_data_type_t dt = dnnl_data_type_undef;
     dnnl_memory_desc src1;
+    dnnl_memory_desc src2; // binary select: the condition
     int mask = 0;
 };
 } // namespace
@@ -225,6 +226,10 @@ struct dnnl_primitive_desc {
     // broadcast over some batch dims only): the leading `outer_n` batch dims
     // are walked on the host, one launch per index, with these element
     // strides; the remaining ones form the batch of a launch.
+    // post-op slot of the lowered descriptor -> index of the attribute's post-op and the execute argument it
+    // takes (a binary select lowers to two slots: the select with src1, then its condition with src2)
+    int po_entry[MI355_MAX_POST_OPS] = {};
+    int po_arg_id[MI355_MAX_POST_OPS] = {};
     int outer_n = 0;
     dim_t outer_dims[DNNL_MAX_NDIMS] = {};
     dim_t outer_src[DNNL_MAX_NDIMS] = {}, outer_wei[DNNL_MAX_NDIMS] = {}, outer_dst[DNNL_MAX_NDIMS] = {},
@@ -455,6 +460,12 @@ dnnl_status_t check_attr(const dnnl_memory_desc &s, const dnnl_memory_desc &w, c
             CHECK_ARG(e.src1.ndims == d.ndims);
             for (int i = 0; i < d.ndims; ++i)
                 CHECK_ARG(e.src1.dims[i] == 1 || e.src1.dims[i] == d.dims[i] || d.dims[i] == k_probe_dim);
+            if (e.alg == dnnl_binary_select) {
+                CHECK_ARG(e.src2.ndims == d.ndims);
+                for (int i = 0; i < d.ndims; ++i)
+                    CHECK_ARG(e.src2.dims[i] == 1 || e.src2.dims[i] == d.dims[i] || d.dims[i] == k_probe_dim);
+                CHECK_UNIMPL(e.src2.dt == dnnl_s8 || e.src2.dt == dnnl_u8 || e.src2.dt == dnnl_s32);
+            }
         }
     }
     CHECK_UNIMPL(n_sum <= 1 || true);
@@ -515,7 +526,10 @@ dnnl_status_t lower(dnnl_primitive_desc &pd) {
             if (pd.wei.kind != dnnl_format_kind_opaque && !collapse_batch(pd.wei, pd.dst, &t, f)) return false;
             if (pd.with_bias && !collapse_batch(pd.bias, pd.dst, &t, f)) return false;
             for (const post_op_entry_t &e : pd.attr.post_ops.entries)
-                if (e.kind == dnnl_binary && !collapse_batch(e.src1, pd.dst, &t, f)) return false;
+                if (e.kind == dnnl_binary
+                        && (!collapse_batch(e.src1, pd.dst, &t, f)
+                                || (e.alg == dnnl_binary_select && !collapse_batch(e.src2, pd.dst, &t, f))))
+                    return false;
             return true;
         };
         while (first < nd - 2 && !collapses(first)) ++first;
@@ -537,6 +551,7 @@ dnnl_status_t lower(dnnl_primitive_desc &pd) {
         for (int i = 0; i < first; ++i) pd.outer_dims[i] = pd.dst.dims[i];
         outer(pd.src, pd.outer_src); outer(pd.wei, pd.outer_wei); outer(pd.dst, pd.outer_dst);
         if (pd.with_bias) outer(pd.bias, pd.outer_bias);
+        for (const post_op_entry_t &e : pd.attr.post_ops.entries) CHECK_UNIMPL(e.alg != dnnl_binary_select || e.kind != dnnl_binary);
         for (size_t i = 0; i < pd.attr.post_ops.entries.size(); ++i)
             if (pd.attr.post_ops.entries[i].kind == dnnl_binary) outer(pd.attr.post_ops.entries[i].src1, pd.outer_po[i]);
         CHECK_UNIMPL(whole_bytes);
@@ -590,11 +605,23 @@ dnnl_status_t lower(dnnl_primitive_desc &pd) {
     D.dst_scale_mode = MI355_DST_SCALE_DIVIDE;
     if (const char *e = getenv("ONEDNN_AMD_DST_SCALE_RECIPROCAL"))
         if (atoi(e)) D.dst_scale_mode = MI355_DST_SCALE_RECIPROCAL;
-    CHECK_UNIMPL(a.post_ops.entries.size() <= MI355_MAX_POST_OPS);
-    D.n_post_ops = (int)a.post_ops.entries.size();
-    for (int i = 0; i < D.n_post_ops; ++i) {
-        const post_op_entry_t &e = a.post_ops.entries[i];
+    int n_slots = (int)a.post_ops.entries.size();
+    for (const post_op_entry_t &e : a.post_ops.entries) n_slots += e.kind == dnnl_binary && e.alg == dnnl_binary_select;
+    CHECK_UNIMPL(n_slots <= MI355_MAX_POST_OPS);
+    D.n_post_ops = n_slots;
+    auto operand_strides = [&](const dnnl_memory_desc &x, int64_t *st) -> bool {
+        if (!collapse_batch(x, pd.dst, &st[0], first)) return false;
+        st[1] = x.dims[nd - 2] == 1 ? 0 : x.strides[nd - 2];
+        st[2] = x.dims[nd - 1] == 1 ? 0 : x.strides[nd - 1];
+        if (pd.dst.dims[nd - 2] == 1) st[1] = x.strides[nd - 2];
+        if (pd.dst.dims[nd - 1] == 1) st[2] = x.strides[nd - 1];
+        return true;
+    };
+    for (int i = 0, ei = 0; i < D.n_post_ops; ++i, ++ei) {
+        const post_op_entry_t &e = a.post_ops.entries[ei];
         mi355_post_op_t &o = D.post_ops[i];
+        pd.po_entry[i] = ei;
+        pd.po_arg_id[i] = e.kind == dnnl_binary ? DNNL_ARG_SRC_1 : e.kind == dnnl_prelu ? DNNL_ARG_WEIGHTS : 0;
         o.alpha = e.alpha; o.beta = e.beta; o.scale = e.scale; o.zero_point = e.zero_point;
         switch (e.kind) {
             case dnnl_sum: o.kind = MI355_PO_SUM; o.dt = e.dt; break;
@@ -614,13 +641,15 @@ dnnl_status_t lower(dnnl_primitive_desc &pd) {
                 break;
             case dnnl_binary: {
                 o.kind = MI355_PO_BINARY; o.alg = e.alg; o.dt = e.src1.dt;
-                int64_t st[3];
-                if (!collapse_batch(e.src1, pd.dst, &st[0], first)) return dnnl_unimplemented;
-                st[1] = e.src1.dims[nd - 2] == 1 ? 0 : e.src1.strides[nd - 2];
-                st[2] = e.src1.dims[nd - 1] == 1 ? 0 : e.src1.strides[nd - 1];
-                if (pd.dst.dims[nd - 2] == 1) st[1] = e.src1.strides[nd - 2];
-                if (pd.dst.dims[nd - 1] == 1) st[2] = e.src1.strides[nd - 1];
-                memcpy(o.stride, st, sizeof(st));
+                if (!operand_strides(e.src1, o.stride)) return dnnl_unimplemented;
+                if (e.alg == dnnl_binary_select) {
+                    // the condition takes the next slot
+                    mi355_post_op_t &c = D.post_ops[++i];
+                    c.kind = MI355_PO_SELECT_COND; c.dt = e.src2.dt;
+                    if (!operand_strides(e.src2, c.stride)) return dnnl_unimplemented;
+                    pd.po_entry[i] = ei;
+                    pd.po_arg_id[i] = DNNL_ARG_SRC_2;
+                }
             } break;
             case dnnl_prelu: {
                 // weights are f32, dims = dst dims under the mask, dense row-major
@@ -1261,6 +1290,34 @@ DNNL_EXPORT dnnl_status_t dnnl_post_ops_append_binary(dnnl_post_ops_t post_ops, 
     post_ops->entries.push_back(e);
     return dnnl_success;
 }
+// post_ops_t::append_binary with a ternary algorithm, src/common/primitive_attr.cpp:888-894
+DNNL_EXPORT dnnl_status_t dnnl_post_ops_append_binary_v2(dnnl_post_ops_t post_ops, dnnl_alg_kind_t alg,
+        const_dnnl_memory_desc_t src1_desc, const_dnnl_memory_desc_t src2_desc) {
+    if (alg != dnnl_binary_select) {
+        CHECK_ARG(!src2_desc);
+        return dnnl_post_ops_append_binary(post_ops, alg, src1_desc);
+    }
+    CHECK_ARG(post_ops && src1_desc && src2_desc);
+    CHECK_ARG(src1_desc->kind == dnnl_blocked || src1_desc->kind == dnnl_format_kind_any);
+    CHECK_ARG(src2_desc->kind == dnnl_blocked || src2_desc->kind == dnnl_format_kind_any);
+    if (po_full(post_ops)) return dnnl_out_of_memory;
+    post_op_entry_t e;
+    e.kind = dnnl_binary; e.alg = alg; e.src1 = *src1_desc; e.src2 = *src2_desc;
+    if (e.src1.kind == dnnl_format_kind_any) e.src1.set_dense();
+    if (e.src2.kind == dnnl_format_kind_any) e.src2.set_dense();
+    post_ops->entries.push_back(e);
+    return dnnl_success;
+}
+DNNL_EXPORT dnnl_status_t dnnl_post_ops_get_params_binary_v2(const_dnnl_post_ops_t post_ops, int index,
+        dnnl_alg_kind_t *alg, const_dnnl_memory_desc_t *src1_desc, const_dnnl_memory_desc_t *src2_desc) {
+    CHECK_ARG(post_ops && index >= 0 && index < (int)post_ops->entries.size());
+    const post_op_entry_t &e = post_ops->entries[index];
+    CHECK_ARG(e.kind == dnnl_binary);
+    if (alg) *alg = e.alg;
+    if (src1_desc) *src1_desc = &e.src1;
+    if (src2_desc) *src2_desc = e.alg == dnnl_binary_select ? &e.src2 : nullptr;
+    return dnnl_success;
+}
 DNNL_EXPORT dnnl_status_t dnnl_post_ops_get_params_binary(const_dnnl_post_ops_t post_ops, int index,
         dnnl_alg_kind_t *alg, const_dnnl_memory_desc_t *src1_desc) {
     CHECK_ARG(post_ops && index >= 0 && index < (int)post_ops->entries.size());
@@ -1692,12 +1749,8 @@ DNNL_EXPORT dnnl_status_t dnnl_primitive_execute(const_dnnl_primitive_t cprimiti
     if ((st = take_q(at.zero_points, DNNL_ARG_DST, DNNL_ARG_ATTR_ZERO_POINTS, pd.desc.dst_zp, &A.dst_zp))) return st;
     TAKE(src_pr, DNNL_ARG_ATTR_PRECOMPUTED_REDUCTIONS | DNNL_ARG_SRC, pd.desc.src_pr.dt != MI355_DT_UNDEF);
     for (int i = 0; i < pd.desc.n_post_ops; ++i) {
-        const int kind = pd.desc.post_ops[i].kind;
-        if (kind == MI355_PO_BINARY) {
-            if ((st = handle(DNNL_ARG_ATTR_MULTIPLE_POST_OP(i) | DNNL_ARG_SRC_1, true, &p))) return st;
-            A.po_arg[i] = p;
-        } else if (kind == MI355_PO_PRELU) {
-            if ((st = handle(DNNL_ARG_ATTR_MULTIPLE_POST_OP(i) | DNNL_ARG_WEIGHTS, true, &p))) return st;
+        if (pd.po_arg_id[i]) {
+            if ((st = handle(DNNL_ARG_ATTR_MULTIPLE_POST_OP(pd.po_entry[i]) | pd.po_arg_id[i], true, &p))) return st;
             A.po_arg[i] = p;
         }
     }

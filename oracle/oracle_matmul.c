@@ -254,7 +254,15 @@ static float orc_post_ops(const mi355_matmul_desc_t *d,
                 int64_t off = b * po->stride[0] + m * po->stride[1]
                         + n * po->stride[2];
                 float v = orc_load_float(po->dt, a->po_arg[i], off);
-                res = orc_binary(po->alg, res, v);
+                if (po->alg == MI355_BINARY_SELECT) {
+                    /* primitive_attr_postops.cpp:44,345-360: src2 (the entry
+                     * that follows) is loaded as an integer; true keeps res */
+                    const mi355_post_op_t *c = &d->post_ops[i + 1];
+                    int64_t coff = b * c->stride[0] + m * c->stride[1] + n * c->stride[2];
+                    res = orc_load_int(c->dt, a->po_arg[i + 1], coff) != 0 ? res : v;
+                } else {
+                    res = orc_binary(po->alg, res, v);
+                }
             } break;
             case MI355_PO_PRELU: {
                 if (res >= 0) break;

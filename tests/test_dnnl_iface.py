@@ -447,3 +447,26 @@ def test_use_dst_for_bwd_eltwise_post_ops(eng):
     a.set_post_ops(po)
     pd = make_pd(eng, 64, 128, 256, "s8", "s8", "f32", attr=a)
     assert pd.impl_info_str().startswith("hip:mfma_i8")           # lowered to plain relu: the fast epilogue takes it
+
+
+def test_binary_select_post_op_rules(eng):
+    # the ternary binary post-op: dnnl_post_ops_append_binary_v2 (primitive_attr.cpp:888-894), dst = src2 ? dst : src1
+    sel = cabi.BINARY["select"]
+    po = dnnl.post_ops()
+    assert status_of(lambda: po.append_binary(sel, md([1, 256], "f32"))) == dnnl.invalid_arguments      # needs src2
+    assert status_of(lambda: po.append_binary(cabi.BINARY["add"], md([1, 256], "f32"), md([64, 1], "s8"))) == dnnl.invalid_arguments
+    po.append_binary(sel, md([1, 256], "f32"), md([64, 1], "s8"))
+    a = dnnl.primitive_attr()
+    a.set_post_ops(po)
+    assert make_pd(eng, 64, 128, 256, "s8", "s8", "f32", attr=a).impl_info_str() == "hip:ref:any"
+    # the condition broadcasts like any binary operand, and is an integer tensor
+    po = dnnl.post_ops()
+    po.append_binary(sel, md([1, 256], "f32"), md([64, 7], "s8"))
+    a = dnnl.primitive_attr()
+    a.set_post_ops(po)
+    assert status_of(lambda: make_pd(eng, 64, 128, 256, "s8", "s8", "f32", attr=a)) == dnnl.invalid_arguments
+    po = dnnl.post_ops()
+    po.append_binary(sel, md([1, 256], "f32"), md([64, 256], "f32"))
+    a = dnnl.primitive_attr()
+    a.set_post_ops(po)
+    assert status_of(lambda: make_pd(eng, 64, 128, 256, "s8", "s8", "f32", attr=a)) == dnnl.unimplemented

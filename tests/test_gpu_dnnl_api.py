@@ -496,3 +496,56 @@ def test_use_dst_for_bwd_eltwise_equals_its_base_algorithm(gpu):
             got, _, _ = run_through_api(p)
             outs.append(np.asarray(got).view(np.uint32))
         assert np.array_equal(outs[0], outs[1]), name
+
+
+def test_binary_select_post_op(gpu, oracle):
+    """dst = cond ? dst : src1 (primitive_attr_postops.cpp:44,345-360): through the C ABI against the oracle, against
+    numpy on exact values, and through dnnl_post_ops_append_binary_v2 with DNNL_ARG_SRC_2."""
+    from onednn_amd.problem import GpuRun, PostOp
+    r = np.random.default_rng(21)
+    p = configs.config1(M=48, N=96, K=64, dst="s32")            # exact integer sums
+    M, N = p.M, p.N
+    other = r.integers(-9, 10, size=(1, N)).astype(np.float32)
+    cond = r.integers(-1, 2, size=(M, 1)).astype(np.int8)        # negative values are true as well
+    p.post_ops = [PostOp(kind=cabi.PO_ELTWISE, alg=cabi.ELTWISE["linear"], alpha=2.0, beta=1.0, scale=1.0),
+                  PostOp(kind=cabi.PO_BINARY, alg=cabi.BINARY["select"], dt=cabi.DT_F32, stride=(0, 0, 1), data=other),
+                  PostOp(kind=cabi.PO_SELECT_COND, dt=cabi.DT_S8, stride=(0, 1, 0), data=cond)]
+    plain = configs.config1(M=48, N=96, K=64, dst="s32")
+    acc = np.asarray(oracle.run_oracle(plain)).view(np.int32).reshape(M, N)
+    want_np = np.where(cond != 0, 2 * acc + 1, other.astype(np.int32))
+    want = np.asarray(oracle.run_oracle(p)).view(np.int32).reshape(M, N)
+    assert np.array_equal(want, want_np)                          # pins the oracle's branch
+    run = GpuRun(p, None)
+    try:
+        run.launch()
+        got, name = np.asarray(run.result()).view(np.int32).reshape(M, N), cabi.impl_name(run.impl)
+    finally:
+        run.free()
+    assert name == "hip:ref:any" and np.array_equal(got, want)
+    # a select without its condition entry is refused
+    bad = configs.config1(M=48, N=96, K=64, dst="s32")
+    bad.post_ops = p.post_ops[:2]
+    assert cabi.query(bad.desc())[0] == cabi.INVALID_ARGUMENTS
+    # the same through the API
+    eng = dnnl.engine(dnnl.gpu, 0)
+    strm = dnnl.stream(eng)
+    mds = [dnnl.memory_desc([M, p.K], p.src_dt, tag=dnnl.tag_ab), dnnl.memory_desc([p.K, N], p.wei_dt, strides=list(p.wei_stride[1:])),
+           dnnl.memory_desc([M, N], p.dst_dt, tag=dnnl.tag_ab)]
+    o_md, c_md = dnnl.memory_desc([1, N], DT["f32"], tag=dnnl.tag_ab), dnnl.memory_desc([M, 1], DT["s8"], tag=dnnl.tag_ab)
+    attr = dnnl.primitive_attr()
+    attr.set_zero_points_mask(dnnl.ARG_SRC, 0)
+    po = dnnl.post_ops()
+    po.append_eltwise(cabi.ELTWISE["linear"], 2.0, 1.0)
+    po.append_binary(cabi.BINARY["select"], o_md, c_md)
+    attr.set_post_ops(po)
+    pd = dnnl.matmul_primitive_desc(eng, mds[0], mds[1], mds[2], attr=attr)
+    assert pd.impl_info_str() == "hip:ref:any"
+    dst = dnnl.memory(mds[2], eng)
+    dnnl.matmul(pd).execute(strm, {
+        dnnl.ARG_SRC: dnnl.memory(mds[0], eng, p.src), dnnl.ARG_WEIGHTS: dnnl.memory(mds[1], eng, p.wei), dnnl.ARG_DST: dst,
+        dnnl.ARG_ATTR_ZERO_POINTS | dnnl.ARG_SRC: dnnl.memory(dnnl.memory_desc([1], DT["s32"], tag=dnnl.tag_a), eng,
+                                                             p.quant["src_zp"].data),
+        dnnl.ARG_ATTR_MULTIPLE_POST_OP(1) | dnnl.ARG_SRC_1: dnnl.memory(o_md, eng, other),
+        dnnl.ARG_ATTR_MULTIPLE_POST_OP(1) | dnnl.ARG_SRC_2: dnnl.memory(c_md, eng, cond)})
+    strm.wait()
+    assert np.array_equal(dst.read(np.int32).reshape(M, N), want)
