@@ -52,6 +52,8 @@
  * there too: the scale against an exhaustive nearest-value search over the 127
  * positive e4m3 codes on constructed maxima (ties to even, both clamps), the
  * dst codes against a nearest-value search over the type's codes.
+ * The ternary select post-op is pinned by tests/test_oracle_matmul.py (numpy
+ * `where` on exact integer sums, three condition types).
  * Unpinned: none of the functions used by the five benchmark configurations;
  * the libm-dependent eltwise algorithms other than relu/gelu_tanh/linear/tanh
  * are "parity unpinned" beyond their textbook formula.

@@ -313,3 +313,19 @@ def test_row_sampling_of_the_full_size_checks_is_consistent():
         want = orc.run_oracle(row_slice(p, rows))
         assert np.array_equal(np.asarray(rows_of(p, full, rows)).view(np.uint8),
                               np.asarray(want).view(np.uint8).reshape(-1)), p.name
+
+
+def test_binary_select_keeps_the_value_where_the_condition_is_nonzero(oracle):
+    # primitive_attr_postops.cpp:44,345-360: res = src2 ? res : src1, the condition loaded as an integer
+    # (negative values are true); exact integer sums, numpy `where` is the check
+    r = np.random.default_rng(21)
+    for cdt, cnp in ((cabi.DT_S8, np.int8), (cabi.DT_U8, np.uint8), (cabi.DT_S32, np.int32)):
+        p = configs.config1(M=24, N=40, K=64, dst="s32")
+        acc = np.asarray(oracle.run_oracle(p)).view(np.int32).reshape(p.M, p.N)
+        other = r.integers(-9, 10, size=(p.M, p.N)).astype(np.float32)
+        cond = r.integers(0 if cnp is np.uint8 else -1, 2, size=(1, p.N)).astype(cnp)
+        p.post_ops = [PostOp(kind=cabi.PO_BINARY, alg=cabi.BINARY["select"], dt=cabi.DT_F32, stride=(0, p.N, 1), data=other),
+                      PostOp(kind=cabi.PO_SELECT_COND, dt=cdt, stride=(0, 0, 1), data=cond),
+                      PostOp(kind=cabi.PO_ELTWISE, alg=cabi.ELTWISE["linear"], alpha=3.0, beta=-1.0, scale=1.0)]
+        got = np.asarray(oracle.run_oracle(p)).view(np.int32).reshape(p.M, p.N)
+        assert np.array_equal(got, 3 * np.where(cond != 0, acc, other.astype(np.int32)) - 1)
