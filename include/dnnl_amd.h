@@ -297,8 +297,9 @@ dnnl_status_t dnnl_primitive_attr_get_scratchpad_mode(const_dnnl_primitive_attr_
         dnnl_scratchpad_mode_t *mode);
 dnnl_status_t dnnl_primitive_attr_set_scales_mask(dnnl_primitive_attr_t attr, int arg, int mask);
 /* dnnl.h:520-553.  With dnnl_quantization_mode_dynamic_mx on DNNL_ARG_DST the
- * scales memory passed at execution is an output (dnnl.h:546-547); host-side
- * scalars (is_on_host) and dnnl_quantization_mode_dynamic_fp are not offered. */
+ * (or dnnl_quantization_mode_dynamic_fp, the NVFP4 flavour) the scales memory
+ * passed at execution is an output (dnnl.h:546-547); is_on_host = 1 makes the
+ * single (mask 0) scale a host-side scalar. */
 dnnl_status_t dnnl_primitive_attr_set_scales_v2(dnnl_primitive_attr_t attr, int arg, int mask, int group_ndims,
         const dnnl_dims_t group_dims, dnnl_data_type_t data_type, int is_on_host);
 dnnl_status_t dnnl_primitive_attr_set_scales_v3(dnnl_primitive_attr_t attr, int arg, int mask, int group_ndims,
@@ -374,6 +375,16 @@ dnnl_status_t dnnl_primitive_execute(const_dnnl_primitive_t primitive, dnnl_stre
 dnnl_status_t dnnl_primitive_get_primitive_desc(const_dnnl_primitive_t primitive,
         const_dnnl_primitive_desc_t *primitive_desc);
 dnnl_status_t dnnl_primitive_destroy(dnnl_primitive_t primitive);
+
+/* ---- extension (no counterpart in dnnl.h): the thin-C-ABI problem description
+ * (struct mi355_matmul_desc_t of mi355_matmul.h, passed as void * so that this
+ * header stays self-contained) a matmul primitive descriptor without runtime
+ * dims lowered to -- shapes, collapsed batch strides, quantization parameter
+ * layouts, post-op operand strides.  For tools and tests that inspect what the
+ * kernels are given; dnnl_invalid_arguments for a reorder or runtime-dims
+ * descriptor. ---- */
+dnnl_status_t dnnl_amd_primitive_desc_get_lowered(const_dnnl_primitive_desc_t primitive_desc,
+        void *mi355_matmul_desc_out);
 
 #ifdef __cplusplus
 }

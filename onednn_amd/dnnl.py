@@ -292,6 +292,13 @@ class matmul_primitive_desc:
     def scratchpad_desc(self):
         return self.query_md(query_scratchpad_md)
 
+    def lowered_desc(self):
+        """The thin-C-ABI problem description the descriptor lowered to
+        (dnnl_amd_primitive_desc_get_lowered, an extension of this library)."""
+        d = cabi.MatmulDesc()
+        _check(lib().dnnl_amd_primitive_desc_get_lowered(self.h, C.byref(d)), "get_lowered")
+        return d
+
 
 class reorder_primitive_desc(matmul_primitive_desc):
     """dnnl::reorder::primitive_desc(src_engine, src_md, dst_engine, dst_md, attr)"""

@@ -447,11 +447,9 @@ dnnl_status_t check_attr(const dnnl_memory_desc &s, const dnnl_memory_desc &w, c
     }
 
     // post-ops: binary, eltwise, prelu, sum (matmul.cpp:606-620)
-    int n_sum = 0;
     for (auto &e : a.post_ops.entries) {
         CHECK_UNIMPL(e.kind == dnnl_binary || e.kind == dnnl_eltwise || e.kind == dnnl_prelu || e.kind == dnnl_sum);
         if (e.kind == dnnl_sum) {
-            ++n_sum;
             // check_sum_consistency: same size as dst, zero point only for int8
             CHECK_UNIMPL(IMPLICATION(e.dt != dnnl_data_type_undef, dt_bits(e.dt) == dt_bits(dst_dt)));
             CHECK_UNIMPL(IMPLICATION(e.zero_point != 0, src_int8));
@@ -468,7 +466,6 @@ dnnl_status_t check_attr(const dnnl_memory_desc &s, const dnnl_memory_desc &w, c
             }
         }
     }
-    CHECK_UNIMPL(n_sum <= 1 || true);
     return dnnl_success;
 }
 
@@ -488,9 +485,23 @@ bool collapse_batch(const dnnl_memory_desc &x, const dnnl_memory_desc &dst, int6
     for (int i = first; i < nb; ++i) total *= dst.dims[i];
     if (all_one && total > 1) return true; // broadcast
     if (!all_full) return false;
-    for (int i = first; i + 1 < nb; ++i)
-        if (x.dims[i + 1] != 1 && x.strides[i] != x.strides[i + 1] * x.dims[i + 1]) return false;
-    *bstride = x.strides[nb - 1];
+    // offset = sum b_i * stride_i must equal S * (collapsed batch index): every
+    // non-unit dim's stride is S times the extent of the dims after it
+    // (a dim of extent 1 may carry any stride)
+    dim_t inner = 1;
+    bool have = false;
+    for (int i = nb - 1; i >= first; --i) {
+        if (x.dims[i] != 1) {
+            if (!have) {
+                if (x.strides[i] % inner) return false;
+                *bstride = x.strides[i] / inner;
+                have = true;
+            } else if (x.strides[i] != *bstride * inner) {
+                return false;
+            }
+        }
+        inner *= dst.dims[i];
+    }
     if (total == 1) *bstride = 0;
     return true;
 }
@@ -652,16 +663,23 @@ dnnl_status_t lower(dnnl_primitive_desc &pd) {
                 }
             } break;
             case dnnl_prelu: {
-                // weights are f32, dims = dst dims under the mask, dense row-major
+                // weights are f32, dims = dst dims under the mask, in the layout
+                // the reference gives them (get_prelu_weights_format,
+                // src/cpu/primitive_attr_postops.cpp:218-241): ab, acb, acdb,
+                // acdeb -- from three dims on, dim 1 is the innermost one
                 o.kind = MI355_PO_PRELU; o.dt = dnnl_f32;
-                const int batch_bits = (1 << (nd - 2)) - 1;
-                const int bm = e.mask & batch_bits;
-                if (bm != 0 && bm != batch_bits) return dnnl_unimplemented;
-                const bool mm = (e.mask >> (nd - 2)) & 1, mn = (e.mask >> (nd - 1)) & 1;
-                const dim_t dn = mn ? D.N : 1, dm = mm ? D.M : 1;
-                o.stride[2] = mn ? 1 : 0;
-                o.stride[1] = mm ? dn : 0;
-                o.stride[0] = bm ? dm * dn : 0;
+                CHECK_UNIMPL(nd <= 5);
+                dnnl_memory_desc w;
+                w.ndims = nd; w.dt = dnnl_f32;
+                for (int d = 0; d < nd; ++d) w.dims[d] = ((e.mask >> d) & 1) ? pd.dst.dims[d] : 1;
+                int perm[DNNL_MAX_NDIMS];
+                for (int d = 0; d < nd; ++d) perm[d] = d;
+                if (nd >= 3) {
+                    for (int d = 1; d + 1 < nd; ++d) perm[d] = d + 1;
+                    perm[nd - 1] = 1;
+                }
+                w.set_dense(perm);
+                if (!operand_strides(w, o.stride)) return dnnl_unimplemented;
             } break;
             default: return dnnl_unimplemented;
         }
@@ -1538,6 +1556,11 @@ DNNL_EXPORT dnnl_status_t dnnl_primitive_desc_next_impl(dnnl_primitive_desc_t pd
 DNNL_EXPORT dnnl_status_t dnnl_primitive_desc_get_attr(const_dnnl_primitive_desc_t pd, const_dnnl_primitive_attr_t *attr) {
     CHECK_ARG(pd && attr);
     *attr = &pd->attr;
+    return dnnl_success;
+}
+DNNL_EXPORT dnnl_status_t dnnl_amd_primitive_desc_get_lowered(const_dnnl_primitive_desc_t pd, void *out) {
+    CHECK_ARG(pd && out && pd->kind == dnnl_matmul && !pd->runtime);
+    memcpy(out, &pd->desc, sizeof(mi355_matmul_desc_t));
     return dnnl_success;
 }
 DNNL_EXPORT dnnl_status_t dnnl_primitive_desc_destroy(dnnl_primitive_desc_t pd) {

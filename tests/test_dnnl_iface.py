@@ -470,3 +470,65 @@ def test_binary_select_post_op_rules(eng):
     a = dnnl.primitive_attr()
     a.set_post_ops(po)
     assert status_of(lambda: make_pd(eng, 64, 128, 256, "s8", "s8", "f32", attr=a)) == dnnl.unimplemented
+
+
+# ------------------------------------------------- prelu weights layout
+def _prelu_pd(eng, dims_dst, K, mask):
+    nd = len(dims_dst)
+    tags = {2: dnnl.tag_ab, 3: dnnl.tag_abc, 4: dnnl.tag_abcd}
+    sdims = list(dims_dst[:-1]) + [K]
+    wdims = list(dims_dst[:-2]) + [K, dims_dst[-1]]
+    po = dnnl.post_ops()
+    po.append_prelu(mask)
+    attr = dnnl.primitive_attr()
+    attr.set_post_ops(po)
+    return dnnl.matmul_primitive_desc(eng, dnnl.memory_desc(sdims, DT["f32"], tag=tags[nd]),
+                                      dnnl.memory_desc(wdims, DT["f32"], tag=tags[nd]),
+                                      dnnl.memory_desc(list(dims_dst), DT["f32"], tag=tags[nd]), attr=attr)
+
+
+def test_prelu_weights_follow_the_reference_layout(eng, oracle):
+    """get_prelu_weights_format (src/cpu/primitive_attr_postops.cpp:218-241): the
+    weights are dims-under-the-mask in ab / acb / acdb -- from three dims on, dim 1
+    is innermost.  The lowered strides index an array laid out that way: checked
+    by running the oracle on the lowered description against numpy indexing."""
+    import numpy as np
+    from onednn_amd.problem import MatmulProblem, PostOp
+    r = np.random.default_rng(5)
+    B, M, N, K = 3, 5, 6, 8
+    for mask in (1, 2, 4, 3, 5, 6, 7):                 # bit 0 batch, bit 1 M, bit 2 N
+        d = _prelu_pd(eng, (B, M, N), K, mask).lowered_desc()
+        db, dm, dn = (B if mask & 1 else 1), (M if mask & 2 else 1), (N if mask & 4 else 1)
+        w = r.uniform(-2, 2, size=(db, dn, dm)).astype(np.float32)      # acb: batch, N, M in memory order
+        st = tuple(d.post_ops[0].stride)
+        assert d.post_ops[0].kind == cabi.PO_PRELU
+        src = r.integers(-4, 5, size=(B, M, K)).astype(np.float32)
+        wei = r.integers(-4, 5, size=(B, K, N)).astype(np.float32)
+        p = MatmulProblem(batch=B, M=M, N=N, K=K, src_dt=cabi.DT_F32, wei_dt=cabi.DT_F32, dst_dt=cabi.DT_F32,
+                          src=src, wei=wei, post_ops=[PostOp(kind=cabi.PO_PRELU, dt=cabi.DT_F32, stride=st, data=w)])
+        got = oracle.run_oracle(p).reshape(B, M, N)
+        v = np.einsum("bmk,bkn->bmn", src, wei)
+        wfull = np.broadcast_to(w.transpose(0, 2, 1), (B, M, N))        # logical (b, m, n) view of the acb array
+        assert np.array_equal(got, np.where(v >= 0, v, wfull * v)), mask
+    # two dims: ab
+    d = _prelu_pd(eng, (M, N), K, 3).lowered_desc()
+    assert tuple(d.post_ops[0].stride)[1:] == (N, 1)
+    # four dims (acdb, dim 1 innermost): the collapsed batch index cannot express a mask over both
+    # batch dims together with M or N; masks within what one stride per tensor expresses lower
+    assert status_of(lambda: _prelu_pd(eng, (2, 3, M, N), K, 0b1111)) == dnnl.unimplemented
+    assert status_of(lambda: _prelu_pd(eng, (2, 3, M, N), K, 0b0111)) == dnnl.unimplemented
+    d = _prelu_pd(eng, (2, 3, M, N), K, 0b1100).lowered_desc()          # M and N only: N-major, as acdb says
+    assert tuple(d.post_ops[0].stride) == (0, N, 1)
+    d = _prelu_pd(eng, (2, 3, M, N), K, 0b0011).lowered_desc()          # both batch dims: memory order a, b
+    assert tuple(d.post_ops[0].stride) == (1, 0, 0)
+    d = _prelu_pd(eng, (1, 3, M, N), K, 0b1111).lowered_desc()          # one real batch dim, innermost
+    assert tuple(d.post_ops[0].stride) == (1, N * 3, 3)
+
+
+def test_batch_dims_of_extent_one_may_carry_any_stride(eng):
+    # [2, 1, M, K] with a stride on the unit dim that does not nest: still one batch stride
+    src = dnnl.memory_desc([2, 1, 4, 8], DT["f32"], strides=[32, 7, 8, 1])
+    wei = dnnl.memory_desc([2, 1, 8, 6], DT["f32"], strides=[48, 1000, 6, 1])
+    dst = dnnl.memory_desc([2, 1, 4, 6], DT["f32"], strides=[24, 24, 6, 1])
+    d = dnnl.matmul_primitive_desc(eng, src, wei, dst).lowered_desc()
+    assert (d.batch, d.src_stride[0], d.wei_stride[0], d.dst_stride[0]) == (2, 32, 48, 24)
