@@ -6,7 +6,7 @@ import pytest
 
 from onednn_amd import cabi, configs, dnnl
 from onednn_amd.problem import storage_dtype
-from tests.helpers import assert_bit_exact, assert_close
+from tests.helpers import assert_bit_exact, assert_close, assert_decode_close, assert_gemm_close
 
 pytestmark = pytest.mark.gpu
 DT = cabi.DT_NAMES
@@ -130,8 +130,8 @@ def test_config2_through_the_api(gpu, oracle):
     p = configs.config2(M=8, N=512, K=1024)
     got, impl, _ = run_through_api(p)
     assert impl.startswith("hip:woq_gemv")
-    want, _, asum = oracle.run_oracle(p, want_ideal=True)
-    assert_close(p, got, want, abs_sum=asum * 20.0, what=impl)
+    want, ideal, asum = oracle.run_oracle(p, want_ideal=True)
+    assert_decode_close(p, got, ideal, asum, what=impl)
 
 
 def test_config4_through_the_api(gpu, oracle):
@@ -243,8 +243,8 @@ def test_prepack_decode_weights_with_reorder_then_matmul(gpu, oracle):
                                    dnnl.ARG_ATTR_ZERO_POINTS | dnnl.ARG_WEIGHTS: zp_mem})
     strm.wait()
     assert np.array_equal(wei_mem.read(np.uint8), pack_woq64(p.wei, K, N))
-    want, _, asum = oracle.run_oracle(p, want_ideal=True)
-    assert_close(p, dst.read(np.uint16), want, abs_sum=asum * 20.0, what=pd.impl_info_str())
+    want, ideal, asum = oracle.run_oracle(p, want_ideal=True)
+    assert_decode_close(p, dst.read(np.uint16), ideal, asum, what=pd.impl_info_str())
 
 
 @pytest.mark.parametrize("flavour", ["mx", "nvfp4"])

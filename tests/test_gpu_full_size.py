@@ -7,8 +7,10 @@ rows: a matmul row depends on its own src row (and its own per-row parameters
 and post-op operands) only, so the sub-problem made of the sampled rows and all
 of the weights has exactly those rows as its result.  Rows are drawn from every
 256-row tile band, first and last rows included.  Bars as at the small sizes:
-bit-exact for the s8 dst of the integer GEMM, the reference checker's ladder
-plus the forward error bound of the K sum for the floating-point ones.
+bit-exact for the s8 dst of the integer GEMM; the floating-point ones against
+the oracle's float64 sums under the sqrt(K)-type bound of tests/helpers.py, with
+an f32 dst as well as the configuration's bf16 so that the dst rounding does not
+hide an error of the sum or the epilogue.
 """
 import dataclasses
 
@@ -17,7 +19,7 @@ import pytest
 
 from onednn_amd import cabi, configs
 from onednn_amd.problem import PostOp, QuantParam, run_gpu
-from tests.helpers import assert_bit_exact, assert_close
+from tests.helpers import assert_bit_exact, assert_gemm_close, fp8_mfma_bound
 
 pytestmark = pytest.mark.gpu
 
@@ -71,21 +73,30 @@ def test_config3_full_size_sampled_rows_are_bit_exact(gpu, oracle):
     assert np.mean((g > 0) & (g < 127)) > 0.05
 
 
-def test_config4_full_size_sampled_rows(gpu, oracle):
+@pytest.mark.parametrize("dst", ["bf16", "f32"])
+def test_config4_full_size_sampled_rows(gpu, oracle, dst):
+    # against the oracle's float64 K-sums with bias, gelu_tanh and the residual in float64 on top:
+    # bound = 4 standard deviations of the float32 summation error model (tests/helpers.py gemm_bound)
+    # plus the matrix cores' fp8 alignment loss (fp8_mfma_bound), together about 0.1 on pre-activations
+    # of standard deviation 90, carried through the chain; with the f32 dst nothing else is inside it,
+    # the bf16 dst adds half a unit in its last place
     p = configs.config4(wtag="ba")
+    p.dst_dt = cabi.DT_NAMES[dst]
     got, name = run_gpu(p)
     assert name.startswith("hip:mfma_f8")
     rows = sample_rows(p.M, 1, 4)
     sub = row_slice(p, rows)
-    want, _, asum = oracle.run_oracle(sub, want_ideal=True)
-    assert_close(sub, rows_of(p, got, rows), want, abs_sum=asum, transcendental=True, what=name)
+    _, ideal, asum = oracle.run_oracle(sub, want_ideal=True)
+    assert assert_gemm_close(sub, rows_of(p, got, rows), ideal, asum, what=name, hw=fp8_mfma_bound(sub)) < 1.0
 
 
-def test_config5_full_size_sampled_rows(gpu, oracle):
+@pytest.mark.parametrize("dst", ["bf16", "f32"])
+def test_config5_full_size_sampled_rows(gpu, oracle, dst):
     p = configs.config5(wtag="ba")
+    p.dst_dt = cabi.DT_NAMES[dst]
     got, name = run_gpu(p)
     assert name.startswith("hip:mfma_mxf4")
     rows = sample_rows(p.M, 1, 5)
     sub = row_slice(p, rows)
-    want, _, asum = oracle.run_oracle(sub, want_ideal=True)
-    assert_close(sub, rows_of(p, got, rows), want, abs_sum=asum, what=name)
+    _, ideal, asum = oracle.run_oracle(sub, want_ideal=True)
+    assert assert_gemm_close(sub, rows_of(p, got, rows), ideal, asum, what=name) < 1.0

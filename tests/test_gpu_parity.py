@@ -5,7 +5,7 @@ import pytest
 
 from onednn_amd import cabi, configs
 from onednn_amd.problem import run_gpu
-from tests.helpers import assert_bit_exact, assert_close
+from tests.helpers import assert_bit_exact, assert_close, assert_decode_close, assert_gemm_close, fp8_mfma_bound
 
 pytestmark = pytest.mark.gpu
 
@@ -43,12 +43,15 @@ def test_config1_full_size(gpu, oracle):
 def test_config4_small(gpu, oracle, impl, wtag):
     # fp8 x fp8 -> bf16 with bf16 bias, gelu_tanh and a bf16 residual add.
     # f32 accumulation order and the device tanhf differ from the oracle's:
-    # thresholds are the reference checker's eltwise ladder plus the forward
-    # error bound of the K-sum (tests/helpers.py).
-    p = configs.config4(M=192, N=320, K=512, wtag=wtag)
-    got, name = run_gpu(p, impl)
-    want, _, asum = oracle.run_oracle(p, want_ideal=True)
-    assert_close(p, got, want, abs_sum=asum, transcendental=True, what=name)
+    # against the oracle's float64 sum with the chain in float64 on top, under the
+    # sqrt(K)-type bound of the float32 summation (tests/helpers.py gemm_bound),
+    # for the configuration's bf16 dst and for an f32 dst
+    for dst in (cabi.DT_BF16, cabi.DT_F32):
+        p = configs.config4(M=192, N=320, K=512, wtag=wtag)
+        p.dst_dt = dst
+        got, name = run_gpu(p, impl)
+        _, ideal, asum = oracle.run_oracle(p, want_ideal=True)
+        assert_gemm_close(p, got, ideal, asum, what=name, hw=fp8_mfma_bound(p) if impl == cabi.IMPL_F8_MFMA else None)
 
 
 def test_config4_no_postops_f32(gpu, oracle):
@@ -58,8 +61,8 @@ def test_config4_no_postops_f32(gpu, oracle):
     p.bias, p.bias_dt = None, cabi.DT_UNDEF
     p.dst_dt = cabi.DT_F32
     got, name = run_gpu(p, cabi.IMPL_F8_MFMA)
-    want, _, asum = oracle.run_oracle(p, want_ideal=True)
-    assert_close(p, got, want, abs_sum=asum, what=name)
+    _, ideal, asum = oracle.run_oracle(p, want_ideal=True)
+    assert_gemm_close(p, got, ideal, asum, what=name, hw=fp8_mfma_bound(p))
 
 
 @pytest.mark.parametrize("impl", [cabi.IMPL_REF, cabi.IMPL_MXF4_MFMA])
@@ -70,11 +73,15 @@ def test_config5_small(gpu, oracle, impl, wtag):
     # differ: bounded by the forward error of that sum, then one bf16 rounding.
     p = configs.config5(M=160, N=288, K=512, wtag=wtag)
     got, name = run_gpu(p, impl)
-    want, _, asum = oracle.run_oracle(p, want_ideal=True)
+    want, ideal, asum = oracle.run_oracle(p, want_ideal=True)
     if impl == cabi.IMPL_REF:
         assert_bit_exact(p, got, want, name)   # same order as the reference
     else:
-        assert_close(p, got, want, abs_sum=asum, what=name)
+        assert_gemm_close(p, got, ideal, asum, what=name)
+        q = configs.config5(M=160, N=288, K=512, wtag=wtag)
+        q.dst_dt = cabi.DT_F32
+        got, name = run_gpu(q, impl)
+        assert_gemm_close(q, got, ideal, asum, what=name)
 
 
 def test_config5_f32_dst_single_block_exact(gpu, oracle):
@@ -107,10 +114,8 @@ def test_config2_small_woq_kernel(gpu, oracle, M):
     p = configs.config2(M=M, N=512, K=1024)
     got, name = run_gpu(p, cabi.IMPL_WOQ_GEMV)
     assert name.startswith("hip:woq_gemv")
-    want, _, asum = oracle.run_oracle(p, want_ideal=True)
-    # the offset-binary trick adds 128 * |sum of src| to the magnitude of the
-    # accumulated terms of a group: widen the bound accordingly
-    assert_close(p, got, want, abs_sum=asum * 20.0, what=name)
+    _, ideal, asum = oracle.run_oracle(p, want_ideal=True)
+    assert_decode_close(p, got, ideal, asum, what=name)
 
 
 def test_woq_one_hot_rows_are_exact(gpu, oracle):
@@ -152,8 +157,8 @@ def test_woq_attribute_variants(gpu, oracle, case):
                             dst_dt=ddt, relu_bias=relu_bias)
     got, name = run_gpu(p, cabi.IMPL_WOQ_GEMV)
     assert name.startswith("hip:woq_gemv")
-    want, _, asum = oracle.run_oracle(p, want_ideal=True)
-    assert_close(p, got, want, abs_sum=asum * 20.0, what=name)
+    want, ideal, asum = oracle.run_oracle(p, want_ideal=True)
+    assert_decode_close(p, got, ideal, asum, what=name)
     # and the generic kernel follows the reference's operation order exactly
     got_ref, name_ref = run_gpu(p, cabi.IMPL_REF)
     assert_bit_exact(p, got_ref, want, name_ref)
@@ -174,8 +179,8 @@ def test_woq_back_to_back_launches_share_nothing(gpu, oracle):
         outs.append(r.result())
     assert np.array_equal(outs[0], outs[1]) and np.array_equal(outs[0], outs[3])
     assert np.array_equal(outs[2], outs[4])
-    want, _, asum = oracle.run_oracle(b, want_ideal=True)
-    assert_close(b, outs[4], want, abs_sum=asum * 20.0, what="second problem")
+    want, ideal, asum = oracle.run_oracle(b, want_ideal=True)
+    assert_decode_close(b, outs[4], ideal, asum, what="second problem")
     ra.free()
     rb.free()
 
