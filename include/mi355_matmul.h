@@ -300,6 +300,20 @@ int mi355_matmul_scratch_bytes(const mi355_matmul_desc_t *desc, size_t *bytes);
 int mi355_matmul_launch(const mi355_matmul_desc_t *desc,
         const mi355_matmul_args_t *args, void *scratch, void *stream);
 
+/* The same launch for callers that cannot allocate device memory (code under
+ * HIP graph capture, tight serving loops, harnesses that forbid hipMalloc): no
+ * counterpart in the reference.  The scratch is a static device array of
+ * MI355_NOALLOC_SCRATCH_BYTES inside the library, one per GPU, held until the
+ * process ends; the call allocates and frees nothing.  A problem whose
+ * mi355_matmul_scratch_bytes exceeds it is refused with
+ * MI355_INVALID_ARGUMENTS (mi355_last_error names both sizes).  All calls on
+ * one GPU share that array: calls that overlap on one GPU (different streams,
+ * or threads) race on it -- order them, or use mi355_matmul_launch with a
+ * buffer per stream. */
+#define MI355_NOALLOC_SCRATCH_BYTES (8u << 20)
+int mi355_matmul_launch_noalloc(const mi355_matmul_desc_t *desc,
+        const mi355_matmul_args_t *args, void *stream);
+
 /* ---- reorder: layout and data-type conversion of one tensor -------------- */
 
 #define MI355_REORDER_MAX_DIMS 6

@@ -41,6 +41,7 @@ BINARY = {
 
 DST_SCALE_DIVIDE, DST_SCALE_RECIPROCAL = 0, 1
 IMPL_AUTO, IMPL_REF, IMPL_I8_MFMA, IMPL_F8_MFMA, IMPL_MXF4_MFMA, IMPL_WOQ_GEMV, IMPL_WOQ_PACKED = range(7)
+NOALLOC_SCRATCH_BYTES = 8 << 20
 WEI_PACK_NONE, WEI_PACK_WOQ64 = 0, 1
 DST_DYNAMIC_NONE, DST_DYNAMIC_MX, DST_DYNAMIC_FP = 0, 1, 2
 
@@ -110,7 +111,7 @@ KERNEL_SYMBOLS = [
     "mi355_stream_create", "mi355_stream_destroy", "mi355_stream_sync", "mi355_event_create",
     "mi355_event_destroy", "mi355_event_record", "mi355_event_sync", "mi355_event_elapsed_ms",
     "mi355_last_error", "mi355_matmul_query", "mi355_matmul_impl_name",
-    "mi355_matmul_scratch_bytes", "mi355_matmul_launch", "mi355_reorder_query",
+    "mi355_matmul_scratch_bytes", "mi355_matmul_launch", "mi355_matmul_launch_noalloc", "mi355_reorder_query",
     "mi355_reorder_launch", "mi355_wei_pack_reorder_dims", "mi355_copy_kernel", "mi355_flush_kernel",
 ]
 
@@ -162,6 +163,7 @@ def load_kernels():
     lib.mi355_matmul_query.argtypes = [C.POINTER(MatmulDesc), C.c_int, C.POINTER(C.c_int)]
     lib.mi355_matmul_scratch_bytes.argtypes = [C.POINTER(MatmulDesc), C.POINTER(C.c_size_t)]
     lib.mi355_matmul_launch.argtypes = [C.POINTER(MatmulDesc), C.POINTER(MatmulArgs), vp, vp]
+    lib.mi355_matmul_launch_noalloc.argtypes = [C.POINTER(MatmulDesc), C.POINTER(MatmulArgs), vp]
     lib.mi355_reorder_query.argtypes = [C.POINTER(ReorderDesc)]
     lib.mi355_reorder_launch.argtypes = [C.POINTER(ReorderDesc), C.POINTER(ReorderArgs), vp]
     lib.mi355_wei_pack_reorder_dims.argtypes = [C.c_int, C.c_int64, C.c_int64, C.c_int64, C.c_int64,

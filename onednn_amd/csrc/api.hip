@@ -5,6 +5,8 @@
 #include <stdio.h>
 #include <string.h>
 
+#include <mutex>
+
 #include "kernels.hpp"
 
 namespace mi355 {
@@ -224,6 +226,34 @@ static int build_problem(const mi355_matmul_desc_t &d, const mi355_matmul_args_t
     return MI355_SUCCESS;
 }
 
+// Scratch memory of mi355_matmul_launch_noalloc: one array per GPU, part of the
+// loaded code object, held until the process ends.  In host code the array's
+// name is only a handle for hipGetSymbolAddress; the device address it yields
+// (different on every GPU) is what kernels and copies are given.
+static __device__ __align__(256) unsigned char g_static_scratch[MI355_NOALLOC_SCRATCH_BYTES];
+
+static int static_scratch_address(void **out) {
+    constexpr int MAX_DEVICES = 64;
+    static std::mutex mu;
+    static void *addr[MAX_DEVICES] = {};
+    int dev = 0;
+    int st = hip_status(hipGetDevice(&dev), "hipGetDevice");
+    if (st) return st;
+    if (dev < 0 || dev >= MAX_DEVICES) {
+        set_error("device ordinal %d beyond the %d the static scratch table holds", dev, MAX_DEVICES);
+        return MI355_RUNTIME_ERROR;
+    }
+    std::lock_guard<std::mutex> lock(mu);
+    if (!addr[dev]) {
+        void *p = nullptr;
+        st = hip_status(hipGetSymbolAddress(&p, HIP_SYMBOL(g_static_scratch)), "hipGetSymbolAddress");
+        if (st) return st;
+        addr[dev] = p;
+    }
+    *out = addr[dev];
+    return MI355_SUCCESS;
+}
+
 } // namespace mi355
 
 using namespace mi355;
@@ -390,6 +420,25 @@ int mi355_matmul_launch(const mi355_matmul_desc_t *desc, const mi355_matmul_args
         case MI355_IMPL_WOQ_PACKED: return woqp_launch(*desc, P, s);
         default: return MI355_UNIMPLEMENTED;
     }
+}
+
+int mi355_matmul_launch_noalloc(const mi355_matmul_desc_t *desc, const mi355_matmul_args_t *args,
+        void *stream) {
+    size_t bytes = 0;
+    int st = mi355_matmul_scratch_bytes(desc, &bytes);
+    if (st) return st;
+    if (bytes > (size_t)MI355_NOALLOC_SCRATCH_BYTES) {
+        set_error("mi355_matmul_launch_noalloc: the problem needs %zu bytes of scratch, the static buffer holds %zu "
+                  "(use mi355_matmul_launch with a caller-owned buffer, or K-contiguous weights)",
+                bytes, (size_t)MI355_NOALLOC_SCRATCH_BYTES);
+        return MI355_INVALID_ARGUMENTS;
+    }
+    void *scratch = nullptr;
+    if (bytes > 0 && (st = static_scratch_address(&scratch))) return st;
+    // every kernel family writes the part of its scratch it reads within the same
+    // launch (transposed weights, row / column sums, split-K partial sums): nothing
+    // has to start at zero
+    return mi355_matmul_launch(desc, args, scratch, stream);
 }
 
 } // extern "C"
