@@ -276,6 +276,13 @@ int mi355_event_destroy(void *event);
 int mi355_event_record(void *event, void *stream);
 int mi355_event_sync(void *event);
 int mi355_event_elapsed_ms(float *ms, void *start, void *stop);
+/* work enqueued on `stream` after this call starts when `event` has completed
+ * (the in-order guarantee of a stream, extended across two streams) */
+int mi355_stream_wait_event(void *stream, void *event);
+/* writes the low `nbytes` (1, 2, 4 or 8) of `bits` to device memory in stream
+ * order, without a host copy: the value travels as a kernel argument, so the
+ * call never waits for the stream (a host-side scalar of the attributes) */
+int mi355_mem_store_scalar(void *dptr, uint64_t bits, int nbytes, void *stream);
 const char *mi355_last_error(void); /* thread-local text of the last failure */
 
 /* ---- the matmul path ---------------------------------------------------- */

@@ -110,6 +110,7 @@ KERNEL_SYMBOLS = [
     "mi355_mem_free", "mi355_mem_set", "mi355_mem_h2d", "mi355_mem_d2h", "mi355_mem_d2d",
     "mi355_stream_create", "mi355_stream_destroy", "mi355_stream_sync", "mi355_event_create",
     "mi355_event_destroy", "mi355_event_record", "mi355_event_sync", "mi355_event_elapsed_ms",
+    "mi355_stream_wait_event", "mi355_mem_store_scalar",
     "mi355_last_error", "mi355_matmul_query", "mi355_matmul_impl_name",
     "mi355_matmul_scratch_bytes", "mi355_matmul_launch", "mi355_matmul_launch_noalloc", "mi355_reorder_query",
     "mi355_reorder_launch", "mi355_wei_pack_reorder_dims", "mi355_copy_kernel", "mi355_flush_kernel",
@@ -160,6 +161,8 @@ def load_kernels():
     lib.mi355_event_record.argtypes = [vp, vp]
     lib.mi355_event_sync.argtypes = [vp]
     lib.mi355_event_elapsed_ms.argtypes = [C.POINTER(C.c_float), vp, vp]
+    lib.mi355_stream_wait_event.argtypes = [vp, vp]
+    lib.mi355_mem_store_scalar.argtypes = [vp, C.c_uint64, C.c_int, vp]
     lib.mi355_matmul_query.argtypes = [C.POINTER(MatmulDesc), C.c_int, C.POINTER(C.c_int)]
     lib.mi355_matmul_scratch_bytes.argtypes = [C.POINTER(MatmulDesc), C.POINTER(C.c_size_t)]
     lib.mi355_matmul_launch.argtypes = [C.POINTER(MatmulDesc), C.POINTER(MatmulArgs), vp, vp]

@@ -5,7 +5,9 @@
 #include <stdio.h>
 #include <string.h>
 
+#include <map>
 #include <mutex>
+#include <utility>
 
 #include "kernels.hpp"
 
@@ -18,6 +20,25 @@ void set_error(const char *fmt, ...) {
     va_start(ap, fmt);
     vsnprintf(g_err, sizeof(g_err), fmt, ap);
     va_end(ap);
+}
+
+int ensure_dynamic_lds(const void *kernel, int bytes, const char *who) {
+    static std::mutex mu;
+    static std::map<std::pair<const void *, int>, int> done; // (kernel, device) -> bytes reserved
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess) {
+        set_error("%s: no current device", who);
+        return MI355_RUNTIME_ERROR;
+    }
+    std::lock_guard<std::mutex> lock(mu);
+    auto it = done.find({kernel, dev});
+    if (it != done.end() && it->second >= bytes) return MI355_SUCCESS;
+    if (hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, bytes) != hipSuccess) {
+        set_error("%s: cannot reserve %d bytes of LDS", who, bytes);
+        return MI355_RUNTIME_ERROR;
+    }
+    done[{kernel, dev}] = bytes;
+    return MI355_SUCCESS;
 }
 
 static int hip_status(hipError_t e, const char *what) {
@@ -346,6 +367,9 @@ int mi355_event_record(void *event, void *stream) {
 }
 int mi355_event_sync(void *event) {
     return hip_status(hipEventSynchronize((hipEvent_t)event), "hipEventSynchronize");
+}
+int mi355_stream_wait_event(void *stream, void *event) {
+    return hip_status(hipStreamWaitEvent((hipStream_t)stream, (hipEvent_t)event, 0), "hipStreamWaitEvent");
 }
 int mi355_event_elapsed_ms(float *ms, void *start, void *stop) {
     if (!ms) return MI355_INVALID_ARGUMENTS;

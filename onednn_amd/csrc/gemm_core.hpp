@@ -110,6 +110,32 @@ typedef const unsigned __attribute__((address_space(3))) *lds_u32_ptr_t;
 __device__ __forceinline__ v4i lds_read16(unsigned addr) { return *(lds_v4i_ptr_t)(size_t)addr; }
 __device__ __forceinline__ unsigned lds_read4(unsigned addr) { return *(lds_u32_ptr_t)(size_t)addr; }
 
+// A workgroup-uniform value pinned to scalar registers: the DMA's base operand
+// must be an SGPR pair, and a uniform value that merges at the join of divergent
+// code ahead of the K loop counts as divergent from there on.  The value passes
+// through an empty asm statement as a vector register, which hides from the
+// compiler that it is uniform (it would fold a readfirstlane of a known-uniform
+// value away, wherever it keeps it); the readfirstlane itself is the builtin, so
+// that the compiler places the wait states the instruction needs after a VALU
+// write of its source and before a memory instruction reads its result (an
+// inline-assembly v_readfirstlane gets none of them: it read a stale register
+// right behind the v_mov that fed it).
+__device__ __forceinline__ int scalar_int(int x) {
+    asm volatile("" : "+v"(x));
+    int r = __builtin_amdgcn_readfirstlane(x);
+    // the result may go straight into the base operand of a DMA written in inline
+    // assembly, whose wait states after a VALU write of an SGPR (five before a
+    // memory instruction reads it) the compiler cannot place either
+    asm volatile("s_nop 4" : "+s"(r));
+    return r;
+}
+__device__ __forceinline__ const char *scalar_ptr(const char *p) {
+    const uint64_t v = (uint64_t)(uintptr_t)p;
+    const uint32_t lo = (uint32_t)scalar_int((int)(uint32_t)v);
+    const uint32_t hi = (uint32_t)scalar_int((int)(uint32_t)(v >> 32));
+    return (const char *)(uintptr_t)(((uint64_t)hi << 32) | lo);
+}
+
 // s_waitcnt vmcnt(n) only (expcnt / lgkmcnt left at their maxima)
 template <int N>
 __device__ __forceinline__ void wait_vmcnt() {
@@ -205,10 +231,14 @@ __device__ __forceinline__ void phase_barrier() {
 // g+NG-1, which are issued after the barrier).  Group 1 runs one more
 // iteration for its last MFMAs.
 template <int NSTAGE, int KSTEP, class Mma, class Acc, class Ctx>
-__device__ __forceinline__ void main_loop_two_groups(Acc &acc, char *smem, const char *a_tile,
-        const char *b_tile, long lda, long ldb, long rows_a_left, long rows_b_left, int ngroups,
+__device__ __forceinline__ void main_loop_two_groups(Acc &acc, char *smem, const char *a_tile_,
+        const char *b_tile_, long lda, long ldb, long rows_a_left, long rows_b_left, int ngroups_,
         const Ctx &ctx) {
     using G = typename Mma::G;
+    const char *a_tile = scalar_ptr(a_tile_), *b_tile = scalar_ptr(b_tile_);
+    // (a uniform value merged from two loads at the join of divergent code ahead of
+    // the loop counts as divergent, and the stage offsets derive from it)
+    const int ngroups = scalar_int(ngroups_);
     static_assert(G::NW == 8, "two groups of four wavefronts");
     constexpr int NG = NSTAGE / KSTEP;
     constexpr int STAGE_BYTES = G::STAGE_BYTES, GROUP_BYTES = KSTEP * STAGE_BYTES;
@@ -324,15 +354,19 @@ __device__ __forceinline__ void main_loop_two_groups(Acc &acc, char *smem, const
 // fragment.
 // a_tile / b_tile point at the first K byte of tile row 0.
 template <int NSTAGE, int KSTEP, class Mma, class Acc, class Ctx>
-__device__ __forceinline__ void main_loop(Acc &acc, char *smem, const char *a_tile,
-        const char *b_tile, long lda, long ldb, long rows_a_left, long rows_b_left, int ngroups,
+__device__ __forceinline__ void main_loop(Acc &acc, char *smem, const char *a_tile_,
+        const char *b_tile_, long lda, long ldb, long rows_a_left, long rows_b_left, int ngroups_,
         const Ctx &ctx) {
     using G = typename Mma::G;
+    const char *a_tile = scalar_ptr(a_tile_), *b_tile = scalar_ptr(b_tile_);
+    // (a uniform value merged from two loads at the join of divergent code ahead of
+    // the loop counts as divergent, and the stage offsets derive from it)
+    const int ngroups = scalar_int(ngroups_);
     constexpr int NG = NSTAGE / KSTEP;           // groups in the ring
     constexpr int STAGE_BYTES = G::STAGE_BYTES, GROUP_BYTES = KSTEP * STAGE_BYTES;
     if constexpr (G::NW == 8) {
-        main_loop_two_groups<NSTAGE, KSTEP, Mma>(acc, smem, a_tile, b_tile, lda, ldb, rows_a_left,
-                rows_b_left, ngroups, ctx);
+        main_loop_two_groups<NSTAGE, KSTEP, Mma>(acc, smem, a_tile_, b_tile_, lda, ldb, rows_a_left,
+                rows_b_left, ngroups_, ctx);
         return;
     }
     constexpr int DPA = G::DPA, DPB = G::DPB, DPS = G::DPS;

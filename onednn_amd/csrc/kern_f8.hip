@@ -75,26 +75,39 @@ struct f8_mma_t {
             const f8_ctx_t &, int) {
 #pragma unroll
         for (int j = 0; j < COLS; ++j)
+            // operands exchanged: the tile comes out transposed, a lane holds four
+            // consecutive n of one row per accumulator quad (tile_epilogue.hpp)
             acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(
-                    f.a[i], f.b[j], acc[i][j], FMT_A, FMT_B, 0, 0, 0, 0);
+                    f.b[j], f.a[i], acc[i][j], FMT_B, FMT_A, 0, 0, 0, 0);
     }
 };
 
 struct f8_conv_t {
-    float wsc[4];
+    typedef float row_t;
     float ssc_common;
     const void *ssc_p; // per-row src scales (already offset to this batch) or null
     int ssc_dt;
     bool with_src_sc, with_wei_sc;
-    __device__ __forceinline__ void row(const v4i_t &raw, long m, float (&f)[4]) const {
-        float ssc = ssc_common;
-        if (ssc_p) ssc = load_float(ssc_dt, ssc_p, m);
+    long bw;
+    template <class PT>
+    __device__ __forceinline__ void per_n(const PT &P, long, long n, float &wsc, int &, int &) const {
+        if (with_wei_sc)
+            wsc = load_float(P.wei_scale.dt, P.wei_scale.p, quant_off(P.wei_scale, bw, 0, n, P.K, P.N));
+    }
+    __device__ __forceinline__ float row_data(long m) const {
+        return ssc_p ? load_float(ssc_dt, ssc_p, m) : ssc_common;
+    }
+    __device__ __forceinline__ void quad(const v4i_t &raw, float ssc, unsigned ntab, int col, float (&f)[4]) const {
 #pragma unroll
-        for (int e = 0; e < 4; ++e) {
-            float x = __int_as_float(raw[e]);
-            if (with_src_sc) x *= ssc;
-            if (with_wei_sc) x *= wsc[e];
-            f[e] = x;
+        for (int e = 0; e < 4; ++e) f[e] = __int_as_float(raw[e]);
+        if (with_src_sc) {
+#pragma unroll
+            for (int e = 0; e < 4; ++e) f[e] *= ssc;
+        }
+        if (with_wei_sc) {
+            const v4f_t w = nt4f(ntab, NT_WSC, col);
+#pragma unroll
+            for (int e = 0; e < 4; ++e) f[e] *= w[e];
         }
     }
 };
@@ -116,6 +129,26 @@ __global__ void __launch_bounds__(G::NT) __attribute__((amdgpu_waves_per_eu(G::N
     const char *A = (const char *)P.src + (P.ss[0] ? b * P.ss[0] : 0) + m0 * lda;
     const char *Bt = X.bt + b * X.bt_bstride + n0 * X.ldb;
 
+    const long bs = P.ss[0] ? b : 0, bw = P.ws[0] ? b : 0;
+    f8_conv_t cv;
+    cv.with_src_sc = P.src_scale.dt != MI355_DT_UNDEF;
+    cv.with_wei_sc = P.wei_scale.dt != MI355_DT_UNDEF;
+    cv.ssc_common = 1.f;
+    cv.ssc_p = nullptr;
+    cv.ssc_dt = P.src_scale.dt;
+    cv.bw = bw;
+    if (cv.with_src_sc) {
+        if (P.src_scale.mask & 2)
+            cv.ssc_p = (const char *)P.src_scale.p
+                    + ((P.src_scale.mask & 1) ? bs * P.M : 0) * (dt_bits(P.src_scale.dt) / 8);
+        else
+            cv.ssc_common = load_float(P.src_scale.dt, P.src_scale.p, (P.src_scale.mask & 1) ? bs : 0);
+    }
+    // the epilogue's per-column operands go into their LDS table now: the loads
+    // hide behind the pipeline prologue
+    const unsigned ntab = (unsigned)(size_t)(__attribute__((address_space(3))) char *)smem + NSTAGE * G::STAGE_BYTES;
+    fill_ntab<G::NT>(P, cv, ntab, b, n0);
+
     v16f acc[Mma::ROWS][Mma::COLS];
 #pragma unroll
     for (int i = 0; i < Mma::ROWS; ++i)
@@ -127,30 +160,7 @@ __global__ void __launch_bounds__(G::NT) __attribute__((amdgpu_waves_per_eu(G::N
     main_loop<NSTAGE, KSTEP, Mma>(acc, smem, A, Bt, lda, X.ldb, P.M - m0,
             P.N - n0, (int)(P.K / (BKB * KSTEP)), f8_ctx_t {});
 
-    const long bs = P.ss[0] ? b : 0, bw = P.ws[0] ? b : 0;
-    f8_conv_t cv;
-    cv.with_src_sc = P.src_scale.dt != MI355_DT_UNDEF;
-    cv.with_wei_sc = P.wei_scale.dt != MI355_DT_UNDEF;
-    cv.ssc_common = 1.f;
-    cv.ssc_p = nullptr;
-    cv.ssc_dt = P.src_scale.dt;
-    if (cv.with_src_sc) {
-        if (P.src_scale.mask & 2)
-            cv.ssc_p = (const char *)P.src_scale.p
-                    + ((P.src_scale.mask & 1) ? bs * P.M : 0) * (dt_bits(P.src_scale.dt) / 8);
-        else
-            cv.ssc_common = load_float(P.src_scale.dt, P.src_scale.p, (P.src_scale.mask & 1) ? bs : 0);
-    }
-    const long nbase = n0 + wn * G::WCOLS + (lane % (G::WCOLS / 4)) * 4;
-#pragma unroll
-    for (int e = 0; e < 4; ++e) {
-        cv.wsc[e] = 1.f;
-        if (cv.with_wei_sc && nbase + e < P.N)
-            cv.wsc[e] = load_float(P.wei_scale.dt, P.wei_scale.p,
-                    quant_off(P.wei_scale, bw, 0, nbase + e, P.K, P.N));
-    }
-    const bool interior = m0 + BM <= P.M && n0 + G::BN <= P.N;
-    store_quadrant<layout32_t, G::WCOLS, G::NW>(P, smem, acc, b, m0 + wm * 128, n0 + wn * G::WCOLS, interior, cv);
+    store_quadrant<layout32_t, G::WCOLS>(P, smem, ntab, acc, b, m0 + wm * 128, n0 + wn * G::WCOLS, wn * G::WCOLS, cv);
 }
 
 struct f8_plan_t {
@@ -216,17 +226,9 @@ int f8_launch(const mi355_matmul_desc_t &d, const problem_t &P, void *scratch, h
     X.tiles_m = (int)((d.M + BM - 1) / BM);
     X.tiles_n = (int)((d.N + f8_geo_t::BN - 1) / f8_geo_t::BN);
     dim3 grid((unsigned)(X.tiles_m * X.tiles_n), 1, (unsigned)d.batch);
-    constexpr int smem_bytes = NSTAGE * f8_geo_t::STAGE_BYTES;
-    auto go = [&](auto kern) {
-        static bool attr_done = false; // per instantiation
-        if (!attr_done) {
-            if (hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize,
-                        smem_bytes) != hipSuccess) {
-                set_error("mfma_f8: cannot reserve %d bytes of LDS", smem_bytes);
-                return MI355_RUNTIME_ERROR;
-            }
-            attr_done = true;
-        }
+    constexpr int smem_bytes = NSTAGE * f8_geo_t::STAGE_BYTES + NTAB_BYTES;
+    auto go = [&](auto kern) -> int {
+        if (const int st = ensure_dynamic_lds((const void *)kern, smem_bytes, "mfma_f8")) return st;
         hipLaunchKernelGGL(kern, grid, dim3(f8_geo_t::NT), smem_bytes, stream, P, X);
         return hipGetLastError() == hipSuccess ? MI355_SUCCESS : MI355_RUNTIME_ERROR;
     };

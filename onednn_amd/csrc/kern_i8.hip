@@ -1,5 +1,5 @@
 // "hip:mfma_i8" -- LDS-tiled int8 GEMM on the gfx950 matrix cores
-// (v_mfma_i32_32x32x32_i8) with the zero-point compensation folded into an
+// (v_mfma_i32_16x16x64_i8) with the zero-point compensation folded into an
 // s32 row/column-sum correction and the reference's epilogue fused in.
 //
 // Replaces, for integer src and weights, the reference's brgemm int8 path
@@ -72,26 +72,50 @@ struct i8_mma_t {
 #pragma unroll
         for (int j = 0; j < COLS; ++j) {
             const v4i b = WEI_U8 ? (f.b[j] ^ (int)0x80808080) : f.b[j];
-            acc[i][j] = __builtin_amdgcn_mfma_i32_16x16x64_i8(a, b, acc[i][j], 0, 0, 0);
+            // operands exchanged: the tile comes out transposed, a lane holds four
+            // consecutive n of one row (tile_epilogue.hpp)
+            acc[i][j] = __builtin_amdgcn_mfma_i32_16x16x64_i8(b, a, acc[i][j], 0, 0, 0);
         }
     }
 };
 
 // raw s32 accumulator -> f32 entering the shared epilogue
 struct i8_conv_t {
-    int col_corr[4], c_c[4];
-    float wsc[4], ssc;
-    bool with_src_sc, with_wei_sc;
+    typedef int row_t;
+    float ssc;
+    bool with_src_sc, with_wei_sc, has_comp;
     const int *rowsum; // already offset to this batch, or null
-    __device__ __forceinline__ void row(const v4i &raw, long m, float (&f)[4]) const {
-        const int rs = rowsum ? rowsum[m] : 0;
+    const int *colsum; // already offset to this batch, or null
+    int a_c, off_w, Kc;
+    long bw;
+    // the per-column operands of the table: weights scale, a * colsum'[n] + K a c[n], c[n]
+    template <class PT>
+    __device__ __forceinline__ void per_n(const PT &P, long, long n, float &wsc, int &cc, int &c) const {
+        c = off_w;
+        if (P.wei_zp.dt != MI355_DT_UNDEF)
+            c -= load_int(P.wei_zp.dt, P.wei_zp.p, quant_off(P.wei_zp, bw, 0, n, P.K, P.N));
+        cc = (a_c != 0 ? a_c * colsum[n] : 0) + Kc * a_c * c;
+        if (with_wei_sc)
+            wsc = load_float(P.wei_scale.dt, P.wei_scale.p, quant_off(P.wei_scale, bw, 0, n, P.K, P.N));
+    }
+    __device__ __forceinline__ int row_data(long m) const { return rowsum ? rowsum[m] : 0; }
+    __device__ __forceinline__ void quad(const v4i_t &raw, int rs, unsigned ntab, int col, float (&f)[4]) const {
+        int v[4] = {raw[0], raw[1], raw[2], raw[3]};
+        if (has_comp) {
+            const v4i_t cc = nt4i(ntab, NT_CC, col), c = nt4i(ntab, NT_C, col);
 #pragma unroll
-        for (int e = 0; e < 4; ++e) {
-            const int v = raw[e] + col_corr[e] + c_c[e] * rs;
-            float x = (float)v;
-            if (with_src_sc) x *= ssc;
-            if (with_wei_sc) x *= wsc[e];
-            f[e] = x;
+            for (int e = 0; e < 4; ++e) v[e] += cc[e] + c[e] * rs;
+        }
+#pragma unroll
+        for (int e = 0; e < 4; ++e) f[e] = (float)v[e];
+        if (with_src_sc) {
+#pragma unroll
+            for (int e = 0; e < 4; ++e) f[e] *= ssc;
+        }
+        if (with_wei_sc) {
+            const v4f_t w = nt4f(ntab, NT_WSC, col);
+#pragma unroll
+            for (int e = 0; e < 4; ++e) f[e] *= w[e];
         }
     }
 };
@@ -113,6 +137,25 @@ __global__ void __launch_bounds__(G::NT) __attribute__((amdgpu_waves_per_eu(G::N
     const char *A = (const char *)P.src + (P.ss[0] ? b * P.ss[0] : 0) + m0 * lda;
     const char *Bt = (const char *)X.bt + b * X.bt_bstride + n0 * X.ldb;
 
+    // ---- the epilogue's per-column operands go into their LDS table now: the
+    // loads hide behind the pipeline prologue
+    const long bs = P.ss[0] ? b : 0, bw = P.ws[0] ? b : 0;
+    const int off_s = SRC_U8 ? 128 : 0, off_w = WEI_U8 ? 128 : 0;
+    i8_conv_t cv;
+    cv.a_c = off_s;
+    if (P.src_zp.dt != MI355_DT_UNDEF) cv.a_c -= load_int(P.src_zp.dt, P.src_zp.p, 0);
+    cv.off_w = off_w;
+    cv.Kc = (int)P.K;
+    cv.bw = bw;
+    cv.with_src_sc = P.src_scale.dt != MI355_DT_UNDEF;
+    cv.with_wei_sc = P.wei_scale.dt != MI355_DT_UNDEF;
+    cv.ssc = cv.with_src_sc ? load_float(P.src_scale.dt, P.src_scale.p, 0) : 1.f;
+    cv.rowsum = X.rowsum ? X.rowsum + bs * P.M : nullptr;
+    cv.colsum = X.colsum ? X.colsum + bw * P.N : nullptr;
+    cv.has_comp = X.rowsum != nullptr || X.colsum != nullptr || cv.a_c != 0 || WEI_U8 || P.wei_zp.dt != MI355_DT_UNDEF;
+    const unsigned ntab = (unsigned)(size_t)(__attribute__((address_space(3))) char *)smem + NSTAGE * G::STAGE_BYTES;
+    fill_ntab<G::NT>(P, cv, ntab, b, n0);
+
     v4i acc[Mma::ROWS][Mma::COLS];
 #pragma unroll
     for (int i = 0; i < Mma::ROWS; ++i)
@@ -124,35 +167,7 @@ __global__ void __launch_bounds__(G::NT) __attribute__((amdgpu_waves_per_eu(G::N
     main_loop<NSTAGE, 1, Mma>(acc, smem, A, Bt, lda, X.ldb, P.M - m0, P.N - n0,
             (int)(P.K / BK), i8_ctx_t {});
 
-    // ---- epilogue: s32 compensation, scales, shared tail
-    const long bs = P.ss[0] ? b : 0, bw = P.ws[0] ? b : 0;
-    const int off_s = SRC_U8 ? 128 : 0, off_w = WEI_U8 ? 128 : 0;
-    int a_c = off_s;
-    if (P.src_zp.dt != MI355_DT_UNDEF) a_c -= load_int(P.src_zp.dt, P.src_zp.p, 0);
-    i8_conv_t cv;
-    cv.with_src_sc = P.src_scale.dt != MI355_DT_UNDEF;
-    cv.with_wei_sc = P.wei_scale.dt != MI355_DT_UNDEF;
-    cv.ssc = cv.with_src_sc ? load_float(P.src_scale.dt, P.src_scale.p, 0) : 1.f;
-    cv.rowsum = X.rowsum ? X.rowsum + bs * P.M : nullptr;
-    const int Kc = (int)P.K;
-    const long nbase = n0 + wn * G::WCOLS + (lane % (G::WCOLS / 4)) * 4;
-#pragma unroll
-    for (int e = 0; e < 4; ++e) {
-        const long n = nbase + e;
-        cv.col_corr[e] = 0; cv.c_c[e] = 0; cv.wsc[e] = 1.f;
-        if (n < P.N) {
-            int c = off_w;
-            if (P.wei_zp.dt != MI355_DT_UNDEF)
-                c -= load_int(P.wei_zp.dt, P.wei_zp.p, quant_off(P.wei_zp, bw, 0, n, P.K, P.N));
-            cv.c_c[e] = c;
-            cv.col_corr[e] = (a_c != 0 ? a_c * X.colsum[bw * P.N + n] : 0) + Kc * a_c * c;
-            if (cv.with_wei_sc)
-                cv.wsc[e] = load_float(P.wei_scale.dt, P.wei_scale.p,
-                        quant_off(P.wei_scale, bw, 0, n, P.K, P.N));
-        }
-    }
-    const bool interior = m0 + BM <= P.M && n0 + G::BN <= P.N;
-    store_quadrant<layout16_t, G::WCOLS, G::NW>(P, smem, acc, b, m0 + wm * 128, n0 + wn * G::WCOLS, interior, cv);
+    store_quadrant<layout16_t, G::WCOLS>(P, smem, ntab, acc, b, m0 + wm * 128, n0 + wn * G::WCOLS, wn * G::WCOLS, cv);
 }
 
 // out[r] = sum_k (bytes[r][k] ^ flip) as signed bytes; one wave per row
@@ -277,18 +292,10 @@ int i8_launch(const mi355_matmul_desc_t &d, const problem_t &P, void *scratch,
     X.tiles_m = (int)((d.M + BM - 1) / BM);
     X.tiles_n = (int)((d.N + i8_geo_t::BN - 1) / i8_geo_t::BN);
     dim3 grid((unsigned)(X.tiles_m * X.tiles_n), 1, (unsigned)d.batch);
-    constexpr int smem_bytes = NSTAGE * i8_geo_t::STAGE_BYTES;
+    constexpr int smem_bytes = NSTAGE * i8_geo_t::STAGE_BYTES + NTAB_BYTES;
     const bool su = d.src_dt == MI355_DT_U8, wu = d.wei_dt == MI355_DT_U8;
-    auto go = [&](auto kern) {
-        static bool attr_done = false; // per instantiation
-        if (!attr_done) {
-            if (hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize,
-                        smem_bytes) != hipSuccess) {
-                set_error("mfma_i8: cannot reserve %d bytes of LDS", smem_bytes);
-                return MI355_RUNTIME_ERROR;
-            }
-            attr_done = true;
-        }
+    auto go = [&](auto kern) -> int {
+        if (const int st = ensure_dynamic_lds((const void *)kern, smem_bytes, "mfma_i8")) return st;
         hipLaunchKernelGGL(kern, grid, dim3(i8_geo_t::NT), smem_bytes, stream, P, X);
         return hipGetLastError() == hipSuccess ? MI355_SUCCESS : MI355_RUNTIME_ERROR;
     };

@@ -29,7 +29,8 @@ using mx_geo_t = geo_t<4, 256>;
 constexpr int NSTAGE = mx_geo_t::NSTAGE;
 constexpr int SCALE_OFF = NSTAGE * mx_geo_t::STAGE_BYTES; // scale ring after the tile ring
 constexpr int SCALE_STAGE = (BM + mx_geo_t::BN) * 4;      // 256 dwords A + BN dwords B
-constexpr int SMEM_BYTES = SCALE_OFF + NSTAGE * SCALE_STAGE;
+constexpr int SMEM_RING_BYTES = SCALE_OFF + NSTAGE * SCALE_STAGE;
+constexpr int SMEM_BYTES = SMEM_RING_BYTES + NTAB_BYTES;
 
 struct mxf4_extra_t {
     const char *bt;       // weights [N][K/2] bytes
@@ -112,14 +113,20 @@ struct mxf4_mma_t {
 #pragma unroll
         for (int j = 0; j < COLS; ++j) {
             const v8i bb = {f.b[j][0], f.b[j][1], f.b[j][2], f.b[j][3], 0, 0, 0, 0};
+            // operands exchanged: the tile comes out transposed, a lane holds four
+            // consecutive n of one row (tile_epilogue.hpp)
             acc[i][j] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(
-                    a, bb, acc[i][j], 4, 4, 0, f.sa[i], 0, f.sb[j]);
+                    bb, a, acc[i][j], 4, 4, 0, f.sb[j], 0, f.sa[i]);
         }
     }
 };
 
 struct mxf4_conv_t {
-    __device__ __forceinline__ void row(const v4i_t &raw, long, float (&f)[4]) const {
+    typedef int row_t;
+    template <class PT>
+    __device__ __forceinline__ void per_n(const PT &, long, long, float &, int &, int &) const {}
+    __device__ __forceinline__ int row_data(long) const { return 0; }
+    __device__ __forceinline__ void quad(const v4i_t &raw, int, unsigned, int, float (&f)[4]) const {
 #pragma unroll
         for (int e = 0; e < 4; ++e) f[e] = __int_as_float(raw[e]);
     }
@@ -159,6 +166,10 @@ __global__ void __launch_bounds__(G::NT) __attribute__((amdgpu_waves_per_eu(G::N
         ctx.voff_s = brings_a ? ctx.voff_a : ctx.voff_b;
     }
 
+    // the epilogue's per-column operands go into their LDS table now
+    const unsigned ntab = (unsigned)(size_t)(__attribute__((address_space(3))) char *)smem + SMEM_RING_BYTES;
+    fill_ntab<G::NT>(P, mxf4_conv_t {}, ntab, b, n0);
+
     v4f acc[Mma::ROWS][Mma::COLS];
 #pragma unroll
     for (int i = 0; i < Mma::ROWS; ++i)
@@ -170,8 +181,7 @@ __global__ void __launch_bounds__(G::NT) __attribute__((amdgpu_waves_per_eu(G::N
     main_loop<NSTAGE, 1, Mma>(acc, smem, A, Bt, lda, X.ldb, P.M - m0, P.N - n0,
             (int)(P.K / 128), ctx);
 
-    const bool interior = m0 + BM <= P.M && n0 + G::BN <= P.N;
-    store_quadrant<layout16_t, G::WCOLS, G::NW>(P, smem, acc, b, m0 + wm * 128, n0 + wn * G::WCOLS, interior,
+    store_quadrant<layout16_t, G::WCOLS>(P, smem, ntab, acc, b, m0 + wm * 128, n0 + wn * G::WCOLS, wn * G::WCOLS,
             mxf4_conv_t {});
 }
 
@@ -273,15 +283,7 @@ int mxf4_launch(const mi355_matmul_desc_t &d, const problem_t &P, void *scratch,
     X.tiles_m = (int)((d.M + BM - 1) / BM);
     X.tiles_n = (int)((d.N + mx_geo_t::BN - 1) / mx_geo_t::BN);
     dim3 grid((unsigned)(X.tiles_m * X.tiles_n), 1, (unsigned)d.batch);
-    static bool attr_done = false;
-    if (!attr_done) {
-        if (hipFuncSetAttribute((const void *)mxf4_gemm_kernel<mx_geo_t>,
-                    hipFuncAttributeMaxDynamicSharedMemorySize, SMEM_BYTES) != hipSuccess) {
-            set_error("mfma_mxf4: cannot reserve %d bytes of LDS", SMEM_BYTES);
-            return MI355_RUNTIME_ERROR;
-        }
-        attr_done = true;
-    }
+    if (const int st = ensure_dynamic_lds((const void *)mxf4_gemm_kernel<mx_geo_t>, SMEM_BYTES, "mfma_mxf4")) return st;
     hipLaunchKernelGGL(mxf4_gemm_kernel<mx_geo_t>, grid, dim3(mx_geo_t::NT), SMEM_BYTES, stream, P, X);
     return hipGetLastError() == hipSuccess ? MI355_SUCCESS : MI355_RUNTIME_ERROR;
 }

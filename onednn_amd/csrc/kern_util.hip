@@ -100,6 +100,22 @@ extern "C" int mi355_copy_kernel(void *dst, const void *src, size_t bytes, void 
     return hipGetLastError() == hipSuccess ? MI355_SUCCESS : MI355_RUNTIME_ERROR;
 }
 
+namespace mi355 {
+__global__ void store_scalar_kernel(unsigned char *dst, uint64_t bits, int nbytes) {
+    if (threadIdx.x < (unsigned)nbytes) dst[threadIdx.x] = (unsigned char)(bits >> (8 * threadIdx.x));
+}
+} // namespace mi355
+
+extern "C" int mi355_mem_store_scalar(void *dptr, uint64_t bits, int nbytes, void *stream) {
+    if (!dptr || (nbytes != 1 && nbytes != 2 && nbytes != 4 && nbytes != 8)) {
+        set_error("store_scalar: 1, 2, 4 or 8 bytes to a device pointer");
+        return MI355_INVALID_ARGUMENTS;
+    }
+    hipLaunchKernelGGL(store_scalar_kernel, dim3(1), dim3(64), 0, (hipStream_t)stream, (unsigned char *)dptr, bits,
+            nbytes);
+    return hipGetLastError() == hipSuccess ? MI355_SUCCESS : MI355_RUNTIME_ERROR;
+}
+
 extern "C" int mi355_flush_kernel(void *buf, size_t bytes, void *stream) {
     if (bytes % 16 || ((uintptr_t)buf & 15)) {
         set_error("flush kernel needs a 16-byte aligned pointer and size");

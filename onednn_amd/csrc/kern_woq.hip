@@ -497,13 +497,9 @@ int zp_bits(int dt) {
 template <int CHD, int MT, int NWV, int SS>
 int launch_variant(int scb, int zpb, dim3 grid, size_t lds, hipStream_t stream, const problem_t &P,
         const woq_extra_t &X) {
-    auto go = [&](auto kern) __attribute__((always_inline)) {
+    auto go = [&](auto kern) __attribute__((always_inline)) -> int {
         if (lds > 65536) {
-            if (hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds)
-                    != hipSuccess) {
-                set_error("woq_gemv: cannot reserve %zu bytes of LDS", lds);
-                return MI355_RUNTIME_ERROR;
-            }
+            if (const int st = ensure_dynamic_lds((const void *)kern, (int)lds, "woq_gemv")) return st;
         }
         hipLaunchKernelGGL(kern, grid, dim3(NWV * 64), lds, stream, P, X);
         if (X.ksplit > 1) {

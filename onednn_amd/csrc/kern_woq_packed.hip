@@ -277,9 +277,8 @@ __global__ void __launch_bounds__(NWV * 64) woqp_kernel(const problem_t P_, cons
         for (int wv = 1; wv < NWV; ++wv) sum += cell[wv * (WSTRIDE / 4)];
         float v[4] = {sum[0], sum[1], sum[2], sum[3]};
         const long n = (long)chunk * CHUNK + nq * 4;
-        const gemm::epi_hoist_t H = gemm::make_hoist(P, 0, n, 4, false);
-        gemm::apply_epilogue4(P, H, v, 0, m, n, 4, make_uint4(0, 0, 0, 0));
-        gemm::store4(P, H, v, 0, m, n, 4);
+        gemm::apply_epilogue4(P, v, 0, m, n, 4);
+        gemm::store4(P, P.ds[2] == 1 && gemm::vec_ok_store(P.dst, P.ds[0], P.ds[1], dt_bits(P.dst_dt)), v, 0, m, n, 4);
     }
 }
 

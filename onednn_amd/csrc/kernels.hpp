@@ -38,6 +38,11 @@ int woqp_launch(const mi355_matmul_desc_t &d, const problem_t &P, hipStream_t st
 
 void set_error(const char *fmt, ...);
 
+// hipFuncSetAttribute(MaxDynamicSharedMemorySize) for a kernel, once per
+// (kernel, device, size) of this process.  Safe to call from several host
+// threads.
+int ensure_dynamic_lds(const void *kernel, int bytes, const char *who);
+
 // [R][C] bytes (row pitch ld_in) -> [C][R] bytes (row pitch ld_out), per batch
 void transpose_bytes(const void *in, long R, long C, long ld_in, long in_bstride, void *out,
         long ld_out, long out_bstride, long batches, hipStream_t stream);

@@ -1,19 +1,33 @@
 // Epilogue of the LDS-tiled MFMA kernels.
 //
-// After the K loop every wavefront owns a 128 x WCOLS part of the tile in
-// accumulator registers (WCOLS = 128 with four wavefronts per workgroup, 64
-// with eight).  It leaves through LDS in four 32-row slabs; afterwards each
-// lane owns four consecutive n of one row, so dst goes out in coalesced
-// 4/8/16-byte stores and the per-element epilogue code exists once, in a
-// rolled loop over the row groups of a slab.
+// The kernels issue their MFMAs with the operands exchanged (weights columns as
+// the instruction's A operand, src rows as its B operand), so that the
+// accumulators hold the dst tile transposed inside every MFMA tile: a lane owns
+// FOUR CONSECUTIVE n OF ONE ROW m per accumulator quad,
+//   16x16 tiles: acc[i][j][r]  = dst(m = 16 i + lane % 16, n = 16 j + 4 (lane / 16) + r)
+//   32x32 tiles: acc[i][j][r]  = dst(m = 32 i + lane % 32, n = 32 j + 8 (r / 4) + 4 (lane / 32) + r % 4)
+// which is exactly the unit the epilogue arithmetic and the dst stores want
+// (4 / 8 / 16 bytes of one dst row per lane).  Nothing is transposed through
+// LDS and no wavefront waits for another one after the K loop.
 //
-// With one wavefront per SIMD nothing hides memory latency inside that loop,
-// so every operand that does not depend on the row is loaded once per lane
-// before it (dst scale, dst zero points, per-n bias, one per-n binary
-// operand), and one per-element operand stream (the src1 tensor of a binary
-// post-op, the old dst of a sum post-op, or a per-element bias) is prefetched
-// a whole slab ahead into an LDS staging area with 16 loads in flight.
-// Anything beyond that is still computed exactly, with loads inside the loop.
+// Operands of the epilogue:
+//   * per column n (weights scales, zero-point compensation terms, per-n bias,
+//     one per-n binary post-op operand, dst zero points): converted to f32 / s32
+//     once per workgroup into a small LDS table at kernel start -- the loads
+//     hide behind the pipeline prologue -- and read back 16 bytes per quad;
+//   * per row m (row sums for the weights zero points, per-row src scales):
+//     one value per lane and row block, loaded a row block ahead;
+//   * one per-element stream (binary post-op src1, the old dst of a sum
+//     post-op, a per-element bias; 16- or 32-bit elements): loaded straight
+//     into registers a row block ahead, 8 / 16 bytes per lane and quad;
+//   * everything else: loaded where it is used, by the general path.
+//
+// Two paths per wavefront: the fast one (all of the above covers every
+// operand, the post-ops are among relu / linear / clip / gelu_tanh / binary
+// add|mul / sum, the wavefront's columns lie inside N, dst takes vector stores)
+// works on the Q quads of a row block at once with every array index a
+// compile-time constant; the general one parks the quads in lane-private LDS and
+// interprets any post-op chain quad by quad.
 //
 // Order of operations: ref_matmul_int8.cpp:275-306 / ref_matmul.cpp:283-331.
 #pragma once
@@ -23,17 +37,27 @@ namespace mi355 {
 namespace gemm {
 
 typedef int v4i_t __attribute__((ext_vector_type(4)));
-// The accumulator slab in LDS is written one dword at a time and read back as
-// 16-byte vectors: both accesses go through may_alias types, otherwise
-// type-based alias analysis lets the reads move above the writes.
-typedef int __attribute__((may_alias)) slab_int_t;
-typedef int __attribute__((ext_vector_type(4), may_alias)) slab_v4i_t;
-typedef uint4 __attribute__((may_alias)) stage_u4_t;
+typedef float v4f_t __attribute__((ext_vector_type(4)));
+typedef uint4 __attribute__((may_alias)) park_u4_t;
 
 __device__ __forceinline__ int raw_bits(int x) { return x; }
 __device__ __forceinline__ int raw_bits(float x) { return __float_as_int(x); }
 
 constexpr int STG_NONE = -1, STG_BIAS = 100, STG_SUM = 101;
+
+// ---- the per-column operand table in LDS: NTAB_SLOTS rows of 256 dwords
+constexpr int NT_WSC = 0, NT_CC = 1, NT_C = 2, NT_BIAS = 3, NT_HV = 4, NT_DZP = 5, NTAB_SLOTS = 6;
+constexpr int NTAB_COLS = 256;
+constexpr int NTAB_BYTES = NTAB_SLOTS * NTAB_COLS * 4;
+
+typedef const v4i_t __attribute__((address_space(3))) *lds_q_ptr_t;
+__device__ __forceinline__ v4i_t nt4i(unsigned ntab, int slot, int col) {
+    return *(lds_q_ptr_t)(size_t)(ntab + (unsigned)((slot * NTAB_COLS + col) * 4));
+}
+__device__ __forceinline__ v4f_t nt4f(unsigned ntab, int slot, int col) {
+    const v4i_t v = nt4i(ntab, slot, col);
+    return v4f_t {__int_as_float(v[0]), __int_as_float(v[1]), __int_as_float(v[2]), __int_as_float(v[3])};
+}
 
 // gelu_tanh(s) = 0.5 s (1 + tanh(v)), v = sqrt(2/pi) s (1 + 0.044715 s^2)
 // (math_utils.hpp gelu_tanh_fwd), evaluated as s / (1 + exp(-2v)): the same
@@ -47,31 +71,51 @@ __device__ __forceinline__ float gelu_tanh_fast(float s) {
     return s * __builtin_amdgcn_rcpf(1.f + e);
 }
 
+// x / s by two Newton corrections of x * (1 / s):
+//   q0 = x y, r0 = x - s q0 (one fma, exact), q1 = q0 + r0 y, r1 = x - s q1, q = q1 + r1 y
+// with y = 1 / s correctly rounded (one IEEE division per lane, outside the
+// loop).  q1 is within an ulp of x / s, and then the last step returns the
+// correctly rounded quotient (Markstein's theorem for division by fma
+// correction: y correctly rounded, q1 faithful, the remainder exact) -- five
+// instructions instead of the dozen of an IEEE division.  The remainders are
+// exact only while nothing under- or overflows: callers take this path when
+// 2^-20 <= |s| <= 2^20 and every x of the wavefront is zero or has
+// 2^-60 <= |x| <= 2^60, and divide otherwise.  The sign of a zero quotient is
+// not preserved (x = -0 gives +0): integer dst types only.
+__device__ __forceinline__ float div_by_fma(float x, float s, float y) {
+    const float q0 = x * y;
+    const float r0 = __builtin_fmaf(-s, q0, x);
+    const float q1 = __builtin_fmaf(r0, y, q0);
+    const float r1 = __builtin_fmaf(-s, q1, x);
+    return __builtin_fmaf(r1, y, q1);
+}
+__device__ __forceinline__ bool div_by_fma_ok_x(float x) {
+    const unsigned e = (__float_as_uint(x) >> 23) & 0xffu;
+    return x == 0.f || (e >= 127 - 60 && e <= 127 + 60);
+}
+
 struct po_reg_t {
     int kind, alg;
     float alpha, beta, scale, zpf;
 };
 
-struct epi_hoist_t {
-    float bias4[4];
-    float hv4[4];   // hoisted per-n operand of post-op `hoisted_po`
-    float dzp4[4];
+// Wavefront-uniform description of the epilogue (lives in scalar registers).
+struct epi_uniform_t {
     float ds, ds_inv;
-    int bias_mode;  // 0 none, 1 hoisted, 2 per element
-    int ds_mode;    // 0 none, 1 divide, 2 multiply by reciprocal
-    int dzp_mode;   // 0 none, 1 present
-    int hoisted_po; // post-op index or -1
+    int bias_mode;  // 0 none, 1 per n (table), 2 per element
+    int ds_mode;    // 0 none, 1 divide, 2 multiply by reciprocal, 3 divide by fma correction (integer dst)
+    int dzp_mode;   // 0 none, 1 present (table)
+    int hoisted_po; // post-op whose per-n operand sits in the table, or -1
     int staged;     // STG_NONE, STG_BIAS, STG_SUM or a binary post-op index
     int staged_dt;
     const char *staged_p;
     long st_s0, st_s1; // element strides of the staged stream (stride along n is 1)
-    // the leading "simple" post-ops (at most three), resident in registers
-    po_reg_t pf0, pf1, pf2;
-    int nfast; // how many of them; the rest run through the generic loop
+    po_reg_t pf0, pf1, pf2; // the leading "simple" post-ops (at most three)
+    int nfast;      // how many of them
     int n_po;
     int dst_dt, dst_vec; // dst_vec: four consecutive n leave as one aligned store
-    int batchable;       // every operand is hoisted or staged and every post-op is a register-resident one
-    int dynamic;         // MI355_DST_DYNAMIC_*: the dst scale is an output, computed per 32 columns of a row
+    int fast;       // every operand is in the table or staged and every post-op is a register-resident one
+    int dynamic;    // MI355_DST_DYNAMIC_*
 };
 
 __device__ __forceinline__ bool vec_ok(const void *p, long s0, long s1, int bits) {
@@ -83,44 +127,70 @@ __device__ __forceinline__ bool vec_ok(const void *p, long s0, long s1, int bits
 
 __device__ __forceinline__ bool vec_ok_store(const void *p, long s0, long s1, int bits) {
     const int bytes4 = bits / 2; // bytes of four elements
-    const long e4 = bits == 8 ? 4 : 4; // strides are in elements: need multiples of 4
     return (bits == 8 || bits == 16 || bits == 32) && (((uintptr_t)p) % bytes4) == 0
-            && (s0 % e4) == 0 && (s1 % e4) == 0;
+            && (s0 % 4) == 0 && (s1 % 4) == 0;
 }
 
+// the binary post-op whose operand does not depend on the row: first one with
+// a zero row stride
 template <class PT>
-__device__ __forceinline__ epi_hoist_t make_hoist(const PT &P, long b, long nbase, int nvalid,
-        bool interior) {
-    epi_hoist_t H;
-    H.bias_mode = 0; H.ds_mode = 0; H.dzp_mode = 0; H.hoisted_po = -1; H.staged = STG_NONE;
+__device__ __forceinline__ int find_hoisted_po(const PT &P) {
+    for (int i = 0; i < P.n_po; ++i)
+        if (P.po[i].kind == MI355_PO_BINARY && P.po[i].s1 == 0 && P.po[i].alg != MI355_BINARY_SELECT) return i;
+    return -1;
+}
+
+// Fills the epilogue's rows of the table (bias, per-n binary operand, dst zero
+// points) for the tile's 256 columns starting at n0; the kernel's conversion
+// fills its own rows with `conv.per_n`.  Called by every thread of the
+// workgroup before the K loop; the loop's barriers order it before the reads.
+template <int NT, class PT, class Conv>
+__device__ __forceinline__ void fill_ntab(const PT &P, const Conv &conv, unsigned ntab, long b, long n0) {
+    typedef int __attribute__((address_space(3))) *lds_i_ptr_t;
+    static_assert(NT % NTAB_COLS == 0, "every column has a thread");
+    const int hp = find_hoisted_po(P);
+    // No branch below depends on the thread: thread t fills column t % 256 (with
+    // 512 threads two threads store the same values), columns beyond N load from
+    // column N - 1 and store neutral values.  (Values that are uniform but merge
+    // at the join of a divergent branch would count as divergent from there on.)
+    const int col = (int)threadIdx.x & (NTAB_COLS - 1);
+    const bool valid = n0 + col < P.N;
+    const long n = valid ? n0 + col : P.N - 1;
+    lds_i_ptr_t t = (lds_i_ptr_t)(size_t)(ntab + (unsigned)(col * 4));
+    float wsc = 1.f, bias = 0.f, hv = 0.f, dzp = 0.f;
+    int cc = 0, c = 0;
+    conv.per_n(P, b, n, wsc, cc, c);
+    if (P.bias_dt != MI355_DT_UNDEF && P.bs[1] == 0) bias = load_float(P.bias_dt, P.bias, b * P.bs[0] + n * P.bs[2]);
+    if (hp >= 0) hv = load_float(P.po[hp].dt, P.po[hp].p, b * P.po[hp].s0 + n * P.po[hp].s2);
+    if (P.dst_zp.dt != MI355_DT_UNDEF) dzp = (float)((const int *)P.dst_zp.p)[(P.dst_zp.mask & 4) ? n : 0];
+    t[NT_WSC * NTAB_COLS] = __float_as_int(valid ? wsc : 1.f);
+    t[NT_CC * NTAB_COLS] = valid ? cc : 0;
+    t[NT_C * NTAB_COLS] = valid ? c : 0;
+    t[NT_BIAS * NTAB_COLS] = __float_as_int(valid ? bias : 0.f);
+    t[NT_HV * NTAB_COLS] = __float_as_int(valid ? hv : 0.f);
+    t[NT_DZP * NTAB_COLS] = __float_as_int(valid ? dzp : 0.f);
+}
+
+// `cols_inside`: the wavefront's columns all lie inside N (operand streams are
+// then loaded without column masks)
+template <class PT>
+__device__ __forceinline__ epi_uniform_t make_uniform(const PT &P, bool cols_inside) {
+    epi_uniform_t H;
+    H.bias_mode = 0; H.ds_mode = 0; H.dzp_mode = 0; H.staged = STG_NONE;
     H.staged_dt = 0; H.staged_p = nullptr; H.st_s0 = H.st_s1 = 0; H.ds = 1.f; H.ds_inv = 1.f;
-#pragma unroll
-    for (int e = 0; e < 4; ++e) { H.bias4[e] = 0.f; H.hv4[e] = 0.f; H.dzp4[e] = 0.f; }
-    if (P.bias_dt != MI355_DT_UNDEF) {
-        if (P.bs[1] == 0) {
-            H.bias_mode = 1;
-#pragma unroll
-            for (int e = 0; e < 4; ++e)
-                if (e < nvalid) H.bias4[e] = load_float(P.bias_dt, P.bias, b * P.bs[0] + (nbase + e) * P.bs[2]);
-        } else {
-            H.bias_mode = 2;
-        }
-    }
+    if (P.bias_dt != MI355_DT_UNDEF) H.bias_mode = P.bs[1] == 0 ? 1 : 2;
     H.dynamic = P.dst_dynamic;
+    H.dst_dt = P.dst_dt;
     if (P.dst_scale.dt != MI355_DT_UNDEF && !P.dst_dynamic) {
         H.ds = load_float(P.dst_scale.dt, P.dst_scale.p, 0);
         H.ds_inv = 1.f / H.ds;
         H.ds_mode = P.dst_scale_mode == MI355_DST_SCALE_RECIPROCAL ? 2 : 1;
+        const bool int_dst = H.dst_dt == MI355_DT_S8 || H.dst_dt == MI355_DT_U8 || H.dst_dt == MI355_DT_S32;
+        const float as = fabsf(H.ds);
+        if (H.ds_mode == 1 && int_dst && as >= 0x1p-20f && as <= 0x1p20f) H.ds_mode = 3;
     }
-    if (P.dst_zp.dt != MI355_DT_UNDEF) {
-        H.dzp_mode = 1;
-#pragma unroll
-        for (int e = 0; e < 4; ++e)
-            if (e < nvalid)
-                H.dzp4[e] = (float)((const int *)P.dst_zp.p)[(P.dst_zp.mask & 4) ? nbase + e : 0];
-    }
+    if (P.dst_zp.dt != MI355_DT_UNDEF) H.dzp_mode = 1;
     H.n_po = P.n_po;
-    H.dst_dt = P.dst_dt;
     H.dst_vec = P.ds[2] == 1 && vec_ok_store(P.dst, P.ds[0], P.ds[1], dt_bits(P.dst_dt));
     {
         auto grab = [&](int i, po_reg_t &r) -> bool {
@@ -148,16 +218,12 @@ __device__ __forceinline__ epi_hoist_t make_hoist(const PT &P, long b, long nbas
             grab(3 + MI355_MAX_POST_OPS, H.pf2);
         }
     }
+    H.hoisted_po = find_hoisted_po(P);
     int first_sum = -1;
     for (int i = 0; i < P.n_po; ++i) {
         const auto &po = P.po[i];
         if (po.kind == MI355_PO_BINARY) {
-            if (po.s1 == 0 && H.hoisted_po < 0) {
-                H.hoisted_po = i;
-#pragma unroll
-                for (int e = 0; e < 4; ++e)
-                    if (e < nvalid) H.hv4[e] = load_float(po.dt, po.p, b * po.s0 + (nbase + e) * po.s2);
-            } else if (po.s1 != 0 && po.s2 == 1 && H.staged == STG_NONE && interior
+            if (i != H.hoisted_po && po.s1 != 0 && po.s2 == 1 && H.staged == STG_NONE && cols_inside
                     && vec_ok(po.p, po.s0, po.s1, dt_bits(po.dt))) {
                 H.staged = i; H.staged_dt = po.dt; H.staged_p = (const char *)po.p;
                 H.st_s0 = po.s0; H.st_s1 = po.s1;
@@ -166,19 +232,17 @@ __device__ __forceinline__ epi_hoist_t make_hoist(const PT &P, long b, long nbas
             first_sum = i;
         }
     }
-    if (H.staged == STG_NONE && interior && first_sum >= 0 && P.ds[2] == 1
+    if (H.staged == STG_NONE && cols_inside && first_sum >= 0 && P.ds[2] == 1
             && vec_ok(P.dst, P.ds[0], P.ds[1], dt_bits(P.sum_dt))) {
         H.staged = STG_SUM; H.staged_dt = P.sum_dt; H.staged_p = (const char *)P.dst;
         H.st_s0 = P.ds[0]; H.st_s1 = P.ds[1];
     }
-    if (H.staged == STG_NONE && interior && H.bias_mode == 2 && P.bs[2] == 1
+    if (H.staged == STG_NONE && cols_inside && H.bias_mode == 2 && P.bs[2] == 1
             && vec_ok(P.bias, P.bs[0], P.bs[1], dt_bits(P.bias_dt))) {
         H.staged = STG_BIAS; H.staged_dt = P.bias_dt; H.staged_p = (const char *)P.bias;
         H.st_s0 = P.bs[0]; H.st_s1 = P.bs[1];
     }
-    // The batched epilogue (several row quads per dispatch) needs every operand in
-    // registers or in the staging area: no loads inside the loop.
-    H.batchable = H.n_po == H.nfast && (H.bias_mode != 2 || H.staged == STG_BIAS) && nvalid == 4 && H.dst_vec;
+    H.fast = H.n_po == H.nfast && (H.bias_mode != 2 || H.staged == STG_BIAS) && cols_inside && H.dst_vec;
     {
         auto operand_ready = [&](const po_reg_t &r, int i) {
             if (r.kind == MI355_PO_BINARY)
@@ -189,15 +253,15 @@ __device__ __forceinline__ epi_hoist_t make_hoist(const PT &P, long b, long nbas
         const int dd = H.dst_dt;
         if (dd != MI355_DT_S8 && dd != MI355_DT_U8 && dd != MI355_DT_BF16 && dd != MI355_DT_F32 && dd != MI355_DT_S32
                 && dd != MI355_DT_F8_E4M3 && dd != MI355_DT_F8_E5M2 && dd != MI355_DT_F16)
-            H.batchable = 0;
-        if (H.nfast > 0 && !operand_ready(H.pf0, 0)) H.batchable = 0;
-        if (H.nfast > 1 && !operand_ready(H.pf1, 1)) H.batchable = 0;
-        if (H.nfast > 2 && !operand_ready(H.pf2, 2)) H.batchable = 0;
+            H.fast = 0;
+        if (H.nfast > 0 && !operand_ready(H.pf0, 0)) H.fast = 0;
+        if (H.nfast > 1 && !operand_ready(H.pf1, 1)) H.fast = 0;
+        if (H.nfast > 2 && !operand_ready(H.pf2, 2)) H.fast = 0;
     }
     return H;
 }
 
-// decode four packed 16- or 32-bit values (one dispatch for the four)
+// decode four packed 16- or 32-bit values
 __device__ __forceinline__ void staged4(int dt, const uint4 &raw, float (&y)[4]) {
     const uint32_t w[4] = {raw.x, raw.y, raw.z, raw.w};
     switch (dt) {
@@ -220,27 +284,6 @@ __device__ __forceinline__ void staged4(int dt, const uint4 &raw, float (&y)[4])
     }
 }
 
-// eltwise on four values: one dispatch, four bodies (the cheap algorithms)
-__device__ __forceinline__ void eltwise4_simple(int alg, float (&v)[4], float alpha, float beta,
-        float scale) {
-    if (alg == MI355_ELTWISE_RELU) {
-#pragma unroll
-        for (int e = 0; e < 4; ++e) v[e] = (v[e] > 0 ? v[e] : v[e] * alpha) * scale;
-    } else if (alg == MI355_ELTWISE_LINEAR) {
-#pragma unroll
-        for (int e = 0; e < 4; ++e) v[e] = (alpha * v[e] + beta) * scale;
-    } else if (alg == MI355_ELTWISE_GELU_TANH) {
-#pragma unroll
-        for (int e = 0; e < 4; ++e) v[e] = gelu_tanh_fast(v[e]) * scale;
-    } else if (alg == MI355_ELTWISE_CLIP) {
-#pragma unroll
-        for (int e = 0; e < 4; ++e) v[e] = eltwise_f(MI355_ELTWISE_CLIP, v[e], alpha, beta) * scale;
-    } else {
-#pragma unroll
-        for (int e = 0; e < 4; ++e) v[e] = eltwise_f(MI355_ELTWISE_CLIP_V2, v[e], alpha, beta) * scale;
-    }
-}
-
 // every eltwise algorithm, one copy of the long-tail code (rolled over the
 // four values; selects of values, not of addresses)
 __device__ __forceinline__ void eltwise4_any(int alg, float (&v)[4], float alpha, float beta,
@@ -258,91 +301,38 @@ __device__ __forceinline__ void eltwise4_any(int alg, float (&v)[4], float alpha
     v[0] = v0; v[1] = v1; v[2] = v2; v[3] = v3;
 }
 
+// The general path for one quad: bias, any post-op chain, dst scale and zero
+// point, every operand loaded where it is used.
 template <class PT>
-__device__ __forceinline__ void apply_epilogue4(const PT &P, const epi_hoist_t &H, float (&v)[4],
-        long b, long m, long nbase, int nvalid, const uint4 &stg) {
-    float sy[4] = {0.f, 0.f, 0.f, 0.f};
-    if (H.staged != STG_NONE) staged4(H.staged_dt, stg, sy);
-    if (H.bias_mode == 1) {
+__device__ __forceinline__ void apply_epilogue4(const PT &P, float (&v)[4], long b, long m, long nbase,
+        int nvalid) {
+    if (P.bias_dt != MI355_DT_UNDEF) {
 #pragma unroll
-        for (int e = 0; e < 4; ++e) v[e] += H.bias4[e];
-    } else if (H.bias_mode == 2) {
-        if (H.staged == STG_BIAS) {
-#pragma unroll
-            for (int e = 0; e < 4; ++e) v[e] += sy[e];
-        } else {
+        for (int e = 0; e < 4; ++e)
+            if (e < nvalid)
+                v[e] += load_float(P.bias_dt, P.bias, b * P.bs[0] + m * P.bs[1] + (nbase + e) * P.bs[2]);
+    }
+    if (P.n_po > 0) {
+        float dst_old[4] = {0.f, 0.f, 0.f, 0.f};
+        if (P.sum_dt != MI355_DT_UNDEF) {
 #pragma unroll
             for (int e = 0; e < 4; ++e)
                 if (e < nvalid)
-                    v[e] += load_float(P.bias_dt, P.bias, b * P.bs[0] + m * P.bs[1] + (nbase + e) * P.bs[2]);
+                    dst_old[e] = load_float(P.sum_dt, P.dst, b * P.ds[0] + m * P.ds[1] + (nbase + e) * P.ds[2]);
         }
-    }
-    if (H.n_po > 0) {
-        float dst_old[4] = {0.f, 0.f, 0.f, 0.f};
-        if (P.sum_dt != MI355_DT_UNDEF) {
-            if (H.staged == STG_SUM) {
-#pragma unroll
-                for (int e = 0; e < 4; ++e) dst_old[e] = sy[e];
-            } else {
-#pragma unroll
-                for (int e = 0; e < 4; ++e)
-                    if (e < nvalid)
-                        dst_old[e] = load_float(P.sum_dt, P.dst,
-                                b * P.ds[0] + m * P.ds[1] + (nbase + e) * P.ds[2]);
-            }
-        }
-        auto binary_operand = [&](int i, float (&y)[4]) {
-            if (i == H.hoisted_po) {
-#pragma unroll
-                for (int e = 0; e < 4; ++e) y[e] = H.hv4[e];
-            } else if (i == H.staged) {
-#pragma unroll
-                for (int e = 0; e < 4; ++e) y[e] = sy[e];
-            } else {
-                const auto &po = P.po[i];
-#pragma unroll
-                for (int e = 0; e < 4; ++e)
-                    y[e] = e < nvalid ? load_float(po.dt, po.p, b * po.s0 + m * po.s1 + (nbase + e) * po.s2)
-                                      : 0.f;
-            }
-        };
-        auto binary4 = [&](int alg, const float (&y)[4]) {
-            if (alg == MI355_BINARY_ADD) {
-#pragma unroll
-                for (int e = 0; e < 4; ++e) v[e] = v[e] + y[e];
-            } else if (alg == MI355_BINARY_MUL) {
-#pragma unroll
-                for (int e = 0; e < 4; ++e) v[e] = v[e] * y[e];
-            } else {
-#pragma unroll
-                for (int e = 0; e < 4; ++e) v[e] = binary_f(alg, v[e], y[e]);
-            }
-        };
-        auto fast_op = [&](const po_reg_t &r, int i) {
-            if (r.kind == MI355_PO_ELTWISE) {
-                eltwise4_simple(r.alg, v, r.alpha, r.beta, r.scale);
-            } else if (r.kind == MI355_PO_BINARY) {
-                float y[4];
-                binary_operand(i, y);
-                binary4(r.alg, y);
-            } else { // sum
-#pragma unroll
-                for (int e = 0; e < 4; ++e) v[e] += r.scale * (dst_old[e] - r.zpf);
-            }
-        };
-        if (H.nfast > 0) fast_op(H.pf0, 0);
-        if (H.nfast > 1) fast_op(H.pf1, 1);
-        if (H.nfast > 2) fast_op(H.pf2, 2);
 #pragma unroll 1
-        for (int i = H.nfast; i < H.n_po; ++i) {
+        for (int i = 0; i < P.n_po; ++i) {
             const auto &po = P.po[i];
             const int kind = po.kind;
             if (kind == MI355_PO_ELTWISE) {
                 eltwise4_any(po.alg, v, po.alpha, po.beta, po.scale);
             } else if (kind == MI355_PO_BINARY) {
-                float y[4];
-                binary_operand(i, y);
-                binary4(po.alg, y);
+                const int alg = po.alg;
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    const float y = e < nvalid ? load_float(po.dt, po.p, b * po.s0 + m * po.s1 + (nbase + e) * po.s2) : 0.f;
+                    v[e] = alg == MI355_BINARY_ADD ? v[e] + y : alg == MI355_BINARY_MUL ? v[e] * y : binary_f(alg, v[e], y);
+                }
             } else if (kind == MI355_PO_SUM) {
                 const float sc = po.scale, zpf = (float)po.zp;
 #pragma unroll
@@ -355,16 +345,22 @@ __device__ __forceinline__ void apply_epilogue4(const PT &P, const epi_hoist_t &
             }
         }
     }
-    if (H.ds_mode == 1) {
+    if (P.dst_dynamic) return; // the group's scale is computed from these values
+    if (P.dst_scale.dt != MI355_DT_UNDEF) {
+        const float s = load_float(P.dst_scale.dt, P.dst_scale.p, 0);
+        if (P.dst_scale_mode == MI355_DST_SCALE_RECIPROCAL) {
+            const float r = 1.f / s;
 #pragma unroll
-        for (int e = 0; e < 4; ++e) v[e] /= H.ds;
-    } else if (H.ds_mode == 2) {
+            for (int e = 0; e < 4; ++e) v[e] *= r;
+        } else {
 #pragma unroll
-        for (int e = 0; e < 4; ++e) v[e] *= H.ds_inv;
+            for (int e = 0; e < 4; ++e) v[e] /= s;
+        }
     }
-    if (H.dzp_mode) {
+    if (P.dst_zp.dt != MI355_DT_UNDEF) {
 #pragma unroll
-        for (int e = 0; e < 4; ++e) v[e] += H.dzp4[e];
+        for (int e = 0; e < 4; ++e)
+            if (e < nvalid) v[e] += (float)((const int *)P.dst_zp.p)[(P.dst_zp.mask & 4) ? nbase + e : 0];
     }
 }
 
@@ -399,14 +395,15 @@ __device__ __forceinline__ void cvt4(int dt, const float (&v)[4], uint32_t (&w)[
     }
 }
 
+// one quad to dst, `dst_vec`: as one aligned vector store
 template <class PT>
-__device__ __forceinline__ void store4(const PT &P, const epi_hoist_t &H, const float (&v)[4], long b,
+__device__ __forceinline__ void store4(const PT &P, int dst_vec, const float (&v)[4], long b,
         long m, long n, int nvalid) {
     const long off = b * P.ds[0] + m * P.ds[1] + n * P.ds[2];
     uint32_t w[4];
-    cvt4(H.dst_dt, v, w);
-    const int bits = dt_bits(H.dst_dt);
-    if (nvalid == 4 && H.dst_vec) {
+    cvt4(P.dst_dt, v, w);
+    const int bits = dt_bits(P.dst_dt);
+    if (nvalid == 4 && dst_vec) {
         if (bits == 8) {
             *(uint32_t *)((uint8_t *)P.dst + off) = w[0] | (w[1] << 8) | (w[2] << 16) | (w[3] << 24);
         } else if (bits == 16) {
@@ -432,94 +429,88 @@ __device__ __forceinline__ void store4(const PT &P, const epi_hoist_t &H, const 
     }
 }
 
-// ---- batched form: NQ row quads per dispatch.  Every data-type and post-op
-// dispatch below is uniform over the wavefront and is taken once for the NQ
-// quads, and the quads' LDS reads and stores overlap; with one wavefront per
-// SIMD a dispatch per quad leaves the SIMD idle through every branch.
-template <int NQ>
-__device__ __forceinline__ void eltwiseQ_simple(int alg, float (&v)[NQ][4], float alpha, float beta, float scale) {
+// ---- fast path: the Q quads of a row block per dispatch.  Every data-type and
+// post-op dispatch below is uniform over the wavefront and is taken once for the
+// Q quads.
+template <int Q>
+__device__ __forceinline__ void eltwiseQ_simple(int alg, float (&v)[Q][4], float alpha, float beta, float scale,
+        bool int_dst) {
     if (alg == MI355_ELTWISE_RELU) {
+        if (alpha == 0.f && scale == 1.f && int_dst) {
+            // an integer dst turns NaN and -0 into 0 either way: one maximum
 #pragma unroll
-        for (int k = 0; k < NQ; ++k)
+            for (int k = 0; k < Q; ++k)
 #pragma unroll
-            for (int e = 0; e < 4; ++e) v[k][e] = (v[k][e] > 0 ? v[k][e] : v[k][e] * alpha) * scale;
+                for (int e = 0; e < 4; ++e) v[k][e] = fmaxf(v[k][e], 0.f);
+        } else {
+#pragma unroll
+            for (int k = 0; k < Q; ++k)
+#pragma unroll
+                for (int e = 0; e < 4; ++e) v[k][e] = (v[k][e] > 0 ? v[k][e] : v[k][e] * alpha) * scale;
+        }
     } else if (alg == MI355_ELTWISE_LINEAR) {
 #pragma unroll
-        for (int k = 0; k < NQ; ++k)
+        for (int k = 0; k < Q; ++k)
 #pragma unroll
             for (int e = 0; e < 4; ++e) v[k][e] = (alpha * v[k][e] + beta) * scale;
     } else if (alg == MI355_ELTWISE_GELU_TANH) {
 #pragma unroll
-        for (int k = 0; k < NQ; ++k)
+        for (int k = 0; k < Q; ++k)
 #pragma unroll
             for (int e = 0; e < 4; ++e) v[k][e] = gelu_tanh_fast(v[k][e]) * scale;
     } else if (alg == MI355_ELTWISE_CLIP) {
 #pragma unroll
-        for (int k = 0; k < NQ; ++k)
+        for (int k = 0; k < Q; ++k)
 #pragma unroll
             for (int e = 0; e < 4; ++e) v[k][e] = eltwise_f(MI355_ELTWISE_CLIP, v[k][e], alpha, beta) * scale;
     } else {
 #pragma unroll
-        for (int k = 0; k < NQ; ++k)
+        for (int k = 0; k < Q; ++k)
 #pragma unroll
             for (int e = 0; e < 4; ++e) v[k][e] = eltwise_f(MI355_ELTWISE_CLIP_V2, v[k][e], alpha, beta) * scale;
     }
 }
 
-template <int NQ>
-__device__ __forceinline__ void apply_epilogueQ(const epi_hoist_t &H, float (&v)[NQ][4], const uint4 (&stg)[NQ]) {
-    float sy[NQ][4];
-#pragma unroll
-    for (int k = 0; k < NQ; ++k)
-#pragma unroll
-        for (int e = 0; e < 4; ++e) sy[k][e] = 0.f;
-    if (H.staged != STG_NONE) {
-        // every array index below is a compile-time constant: a rolled loop over
-        // the quads would put these arrays into private memory
-        if (H.staged_dt == MI355_DT_BF16) {
-#pragma unroll
-            for (int k = 0; k < NQ; ++k) staged4(MI355_DT_BF16, stg[k], sy[k]);
-        } else if (H.staged_dt == MI355_DT_F32) {
-#pragma unroll
-            for (int k = 0; k < NQ; ++k) staged4(MI355_DT_F32, stg[k], sy[k]);
-        } else if (H.staged_dt == MI355_DT_F16) {
-#pragma unroll
-            for (int k = 0; k < NQ; ++k) staged4(MI355_DT_F16, stg[k], sy[k]);
-        } else {
-#pragma unroll
-            for (int k = 0; k < NQ; ++k) staged4(MI355_DT_S32, stg[k], sy[k]);
-        }
-    }
+// `col[k]`: the quad's first column inside the tile (index into the table);
+// `sy`: the staged stream's values for the quads
+template <int Q>
+__device__ __forceinline__ void apply_epilogueQ(const epi_uniform_t &H, unsigned ntab, const int (&col)[Q],
+        float (&v)[Q][4], const float (&sy)[Q][4]) {
+    const bool int_dst = H.dst_dt == MI355_DT_S8 || H.dst_dt == MI355_DT_U8 || H.dst_dt == MI355_DT_S32;
     if (H.bias_mode == 1) {
 #pragma unroll
-        for (int k = 0; k < NQ; ++k)
+        for (int k = 0; k < Q; ++k) {
+            const v4f_t bb = nt4f(ntab, NT_BIAS, col[k]);
 #pragma unroll
-            for (int e = 0; e < 4; ++e) v[k][e] += H.bias4[e];
+            for (int e = 0; e < 4; ++e) v[k][e] += bb[e];
+        }
     } else if (H.bias_mode == 2) { // staged
 #pragma unroll
-        for (int k = 0; k < NQ; ++k)
+        for (int k = 0; k < Q; ++k)
 #pragma unroll
             for (int e = 0; e < 4; ++e) v[k][e] += sy[k][e];
     }
     auto fast_op = [&](const po_reg_t &r, int i) __attribute__((always_inline)) {
         if (r.kind == MI355_PO_ELTWISE) {
-            eltwiseQ_simple<NQ>(r.alg, v, r.alpha, r.beta, r.scale);
+            eltwiseQ_simple<Q>(r.alg, v, r.alpha, r.beta, r.scale, int_dst);
         } else if (r.kind == MI355_PO_BINARY) {
-            const bool hoisted = i == H.hoisted_po;
-            if (r.alg == MI355_BINARY_ADD) {
+            const bool add = r.alg == MI355_BINARY_ADD; // else mul: nothing else is on this path
+            if (i == H.hoisted_po) {
 #pragma unroll
-                for (int k = 0; k < NQ; ++k)
+                for (int k = 0; k < Q; ++k) {
+                    const v4f_t y = nt4f(ntab, NT_HV, col[k]);
 #pragma unroll
-                    for (int e = 0; e < 4; ++e) v[k][e] = v[k][e] + (hoisted ? H.hv4[e] : sy[k][e]);
-            } else { // mul (nothing else is batchable)
+                    for (int e = 0; e < 4; ++e) v[k][e] = add ? v[k][e] + y[e] : v[k][e] * y[e];
+                }
+            } else {
 #pragma unroll
-                for (int k = 0; k < NQ; ++k)
+                for (int k = 0; k < Q; ++k)
 #pragma unroll
-                    for (int e = 0; e < 4; ++e) v[k][e] = v[k][e] * (hoisted ? H.hv4[e] : sy[k][e]);
+                    for (int e = 0; e < 4; ++e) v[k][e] = add ? v[k][e] + sy[k][e] : v[k][e] * sy[k][e];
             }
         } else { // sum: the old dst is the staged stream
 #pragma unroll
-            for (int k = 0; k < NQ; ++k)
+            for (int k = 0; k < Q; ++k)
 #pragma unroll
                 for (int e = 0; e < 4; ++e) v[k][e] += r.scale * (sy[k][e] - r.zpf);
         }
@@ -527,22 +518,41 @@ __device__ __forceinline__ void apply_epilogueQ(const epi_hoist_t &H, float (&v)
     if (H.nfast > 0) fast_op(H.pf0, 0);
     if (H.nfast > 1) fast_op(H.pf1, 1);
     if (H.nfast > 2) fast_op(H.pf2, 2);
-    if (H.ds_mode == 1) {
+    if (H.ds_mode == 3) {
+        bool okx = true;
 #pragma unroll
-        for (int k = 0; k < NQ; ++k)
+        for (int k = 0; k < Q; ++k)
+#pragma unroll
+            for (int e = 0; e < 4; ++e) okx &= div_by_fma_ok_x(v[k][e]);
+        if (__builtin_amdgcn_ballot_w64(!okx) == 0) {
+#pragma unroll
+            for (int k = 0; k < Q; ++k)
+#pragma unroll
+                for (int e = 0; e < 4; ++e) v[k][e] = div_by_fma(v[k][e], H.ds, H.ds_inv);
+        } else {
+#pragma unroll
+            for (int k = 0; k < Q; ++k)
+#pragma unroll
+                for (int e = 0; e < 4; ++e) v[k][e] /= H.ds;
+        }
+    } else if (H.ds_mode == 1) {
+#pragma unroll
+        for (int k = 0; k < Q; ++k)
 #pragma unroll
             for (int e = 0; e < 4; ++e) v[k][e] /= H.ds;
     } else if (H.ds_mode == 2) {
 #pragma unroll
-        for (int k = 0; k < NQ; ++k)
+        for (int k = 0; k < Q; ++k)
 #pragma unroll
             for (int e = 0; e < 4; ++e) v[k][e] *= H.ds_inv;
     }
     if (H.dzp_mode) {
 #pragma unroll
-        for (int k = 0; k < NQ; ++k)
+        for (int k = 0; k < Q; ++k) {
+            const v4f_t z = nt4f(ntab, NT_DZP, col[k]);
 #pragma unroll
-            for (int e = 0; e < 4; ++e) v[k][e] += H.dzp4[e];
+            for (int e = 0; e < 4; ++e) v[k][e] += z[e];
+        }
     }
 }
 
@@ -563,44 +573,104 @@ __device__ __forceinline__ uint8_t mx_scale_byte(float amax, int em, float &inv)
     return (uint8_t)sb;
 }
 
-// Dynamic (MX) quantization of dst for NQ quads (ref_matmul.cpp:338-423): a
-// group is 32 consecutive n of one row = the quads of 8 consecutive lanes
-// (`lcol` is the lane's quad number in its row).  Writes the e8m0 scale of
-// every group and leaves v scaled and saturated, ready for the fp8 conversion.
-template <int NQ, class PT>
-__device__ __forceinline__ void dynamic_quantQ(const PT &P, const epi_hoist_t &H, float (&v)[NQ][4], long b,
-        const long (&m)[NQ], long n, const bool (&ok)[NQ], int lcol) {
-    const float dt_max = H.dst_dt == MI355_DT_F8_E4M3 ? 448.f : 57344.f;
-    const int em = (int)f32_to_e8m0(dt_max);
+__device__ __forceinline__ float amax4(const float (&v)[4]) {
+    return fmaxf(fmaxf(fabsf(v[0]), fabsf(v[1])), fmaxf(fabsf(v[2]), fabsf(v[3])));
+}
+
+// One row of accumulator tiles copied by value.  The row-block pickers select
+// their rows with a switch over the run-time block number; were the cases
+// identical code on different registers, the compiler would merge them into one
+// copy that indexes `acc` with a run-time offset, and all accumulators would
+// live in private memory from the first K step on.  The empty asm statements
+// keep the cases apart (statements of inline assembly are never merged).
+template <class T, int C>
+__device__ __forceinline__ void copy_row(const T (&src)[C], T (&dst)[C]) {
 #pragma unroll
-    for (int k = 0; k < NQ; ++k) {
-        float amax = fmaxf(fmaxf(fabsf(v[k][0]), fabsf(v[k][1])), fmaxf(fabsf(v[k][2]), fabsf(v[k][3])));
-        amax = fmaxf(amax, __shfl_xor(amax, 1, 64));
-        amax = fmaxf(amax, __shfl_xor(amax, 2, 64));
-        amax = fmaxf(amax, __shfl_xor(amax, 4, 64));
-        float inv;
-        const uint8_t sbyte = mx_scale_byte(amax, em, inv);
-#pragma unroll
-        for (int e = 0; e < 4; ++e) v[k][e] = fminf(fmaxf(v[k][e] * inv, -dt_max), dt_max);
-        if (ok[k] && (lcol & 7) == 0) ((uint8_t *)P.dst_scale.p)[quant_off(P.dst_scale, b, m[k], n, P.M, P.N)] = sbyte;
+    for (int j = 0; j < C; ++j) {
+        T v = src[j];
+        asm volatile("" : "+v"(v));
+        dst[j] = v;
     }
 }
 
-// four full quads (nvalid == 4, vector stores allowed) to dst; `ok[k]` masks rows beyond M
-template <int NQ, class PT>
-__device__ __forceinline__ void storeQ(const PT &P, const epi_hoist_t &H, const float (&v)[NQ][4], long b,
-        const long (&m)[NQ], long n, const bool (&ok)[NQ]) {
-    uint32_t w[NQ][4];
+// Accumulator layouts (operands exchanged, see the top of the file).
+//   RB          rows of a row block (one MFMA tile row)
+//   NB          row blocks of a wavefront's 128 rows
+//   QPG         quads of one lane inside a group of 32 consecutive columns
+//   nq<C>()     quads of a lane per row block (C MFMA tiles along n)
+//   qcol(k)     first column of quad k inside the wavefront's part
+//   quad(a, k)  the four raw accumulators of quad k of row block `a`
+//   group_max   maximum over the lanes that share a row and a 32-column group
+struct layout16_t {
+    static constexpr int RB = 16, NB = 8, QPG = 2;
+    template <int C> static constexpr int nq() { return C; }
+    static __device__ __forceinline__ int lrow(int lane) { return lane & 15; }
+    static __device__ __forceinline__ int qcol(int k, int lane) { return 16 * k + 4 * (lane >> 4); }
+    template <class T, int C>
+    static __device__ __forceinline__ v4i_t quad(const T (&a)[C], int k) {
+        return v4i_t {raw_bits(a[k][0]), raw_bits(a[k][1]), raw_bits(a[k][2]), raw_bits(a[k][3])};
+    }
+    static __device__ __forceinline__ float group_max(float x) {
+        x = fmaxf(x, __shfl_xor(x, 16, 64));
+        return fmaxf(x, __shfl_xor(x, 32, 64));
+    }
+    // the lane that writes the group's scale byte
+    static __device__ __forceinline__ bool group_leader(int lane) { return (lane >> 4) == 0; }
+    template <class T, int R, int C>
+    static __device__ __forceinline__ void pick_rows(const T (&acc)[R][C], int i, T (&a)[C]) {
+        static_assert(R == 8, "eight row blocks");
+        switch (i) {
+            case 0: copy_row(acc[0], a); break;
+            case 1: copy_row(acc[1], a); break;
+            case 2: copy_row(acc[2], a); break;
+            case 3: copy_row(acc[3], a); break;
+            case 4: copy_row(acc[4], a); break;
+            case 5: copy_row(acc[5], a); break;
+            case 6: copy_row(acc[6], a); break;
+            default: copy_row(acc[7], a); break;
+        }
+    }
+};
+
+struct layout32_t {
+    static constexpr int RB = 32, NB = 4, QPG = 4;
+    template <int C> static constexpr int nq() { return 4 * C; }
+    static __device__ __forceinline__ int lrow(int lane) { return lane & 31; }
+    static __device__ __forceinline__ int qcol(int k, int lane) { return 32 * (k >> 2) + 8 * (k & 3) + 4 * (lane >> 5); }
+    template <class T, int C>
+    static __device__ __forceinline__ v4i_t quad(const T (&a)[C], int k) {
+        const int j = k >> 2, g = k & 3;
+        return v4i_t {raw_bits(a[j][4 * g]), raw_bits(a[j][4 * g + 1]), raw_bits(a[j][4 * g + 2]), raw_bits(a[j][4 * g + 3])};
+    }
+    static __device__ __forceinline__ float group_max(float x) { return fmaxf(x, __shfl_xor(x, 32, 64)); }
+    static __device__ __forceinline__ bool group_leader(int lane) { return (lane >> 5) == 0; }
+    template <class T, int R, int C>
+    static __device__ __forceinline__ void pick_rows(const T (&acc)[R][C], int i, T (&a)[C]) {
+        static_assert(R == 4, "four row blocks");
+        switch (i) {
+            case 0: copy_row(acc[0], a); break;
+            case 1: copy_row(acc[1], a); break;
+            case 2: copy_row(acc[2], a); break;
+            default: copy_row(acc[3], a); break;
+        }
+    }
+};
+
+// Q quads of one row to dst (fast path: vector stores, columns inside N)
+template <int Q, class PT>
+__device__ __forceinline__ void storeQ(const PT &P, const epi_uniform_t &H, const float (&v)[Q][4], long b,
+        long m, bool ok, const long (&n)[Q]) {
+    uint32_t w[Q][4];
     const int dt = H.dst_dt;
+    const long rowoff = b * P.ds[0] + m * P.ds[1];
     if (dt == MI355_DT_S8 || dt == MI355_DT_U8) {
         // Round first (v_rndne + the saturating v_cvt_i32_f32, NaN -> 0), clamp as
         // integers, pack the four low bytes with byte permutes: the same values as
         // the reference's clamp-then-round (rounding is monotonic and the bounds
         // are integers) in 3 + 3/4 instructions per value instead of 7 + 7/4.
         const int lo = dt == MI355_DT_S8 ? -128 : 0, hi = dt == MI355_DT_S8 ? 127 : 255;
-        const long off0b = b * P.ds[0] + n;
 #pragma unroll
-        for (int k = 0; k < NQ; ++k) {
+        for (int k = 0; k < Q; ++k) {
             int q[4];
 #pragma unroll
             for (int e = 0; e < 4; ++e) {
@@ -610,7 +680,7 @@ __device__ __forceinline__ void storeQ(const PT &P, const epi_hoist_t &H, const 
             const unsigned lo16 = __builtin_amdgcn_perm((unsigned)q[1], (unsigned)q[0], 0x0c0c0400u);
             const unsigned hi16 = __builtin_amdgcn_perm((unsigned)q[3], (unsigned)q[2], 0x0c0c0400u);
             const unsigned word = __builtin_amdgcn_perm(hi16, lo16, 0x05040100u);
-            if (ok[k]) *(uint32_t *)((uint8_t *)P.dst + off0b + m[k] * P.ds[1]) = word;
+            if (ok) *(uint32_t *)((uint8_t *)P.dst + rowoff + n[k]) = word;
         }
         return;
     } else if (dt == MI355_DT_BF16) {
@@ -622,29 +692,28 @@ __device__ __forceinline__ void storeQ(const PT &P, const epi_hoist_t &H, const 
         // and half a conversion instead of a dozen integer operations.
         bool special = false;
 #pragma unroll
-        for (int k = 0; k < NQ; ++k)
+        for (int k = 0; k < Q; ++k)
 #pragma unroll
             for (int e = 0; e < 4; ++e) special |= __builtin_amdgcn_classf(v[k][e], 0x93);
         if (__builtin_amdgcn_ballot_w64(special) == 0) {
             typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
             typedef float f32x2_t __attribute__((ext_vector_type(2)));
-            const long off0b = b * P.ds[0] + n;
 #pragma unroll
-            for (int k = 0; k < NQ; ++k) {
+            for (int k = 0; k < Q; ++k) {
                 uint2 o;
                 o.x = __builtin_bit_cast(unsigned, __builtin_convertvector(f32x2_t {v[k][0], v[k][1]}, bf16x2_t));
                 o.y = __builtin_bit_cast(unsigned, __builtin_convertvector(f32x2_t {v[k][2], v[k][3]}, bf16x2_t));
-                if (ok[k]) *(uint2 *)((uint16_t *)P.dst + off0b + m[k] * P.ds[1]) = o;
+                if (ok) *(uint2 *)((uint16_t *)P.dst + rowoff + n[k]) = o;
             }
             return;
         }
 #pragma unroll
-        for (int k = 0; k < NQ; ++k)
+        for (int k = 0; k < Q; ++k)
 #pragma unroll
             for (int e = 0; e < 4; ++e) w[k][e] = f32_to_bf16(v[k][e]);
     } else if (dt == MI355_DT_F32) {
 #pragma unroll
-        for (int k = 0; k < NQ; ++k)
+        for (int k = 0; k < Q; ++k)
 #pragma unroll
             for (int e = 0; e < 4; ++e) w[k][e] = f2u(v[k][e]);
     } else if (dt == MI355_DT_F16) {
@@ -652,7 +721,7 @@ __device__ __forceinline__ void storeQ(const PT &P, const epi_hoist_t &H, const 
         // input, NaN payloads included: checked on the device over 4 M f32
         // bit patterns and every exponent's special mantissas
 #pragma unroll
-        for (int k = 0; k < NQ; ++k)
+        for (int k = 0; k < Q; ++k)
 #pragma unroll
             for (int e = 0; e < 4; ++e) w[k][e] = __builtin_bit_cast(uint16_t, (_Float16)v[k][e]);
     } else if (dt == MI355_DT_F8_E4M3 || dt == MI355_DT_F8_E5M2) {
@@ -665,15 +734,14 @@ __device__ __forceinline__ void storeQ(const PT &P, const epi_hoist_t &H, const 
         // takes the software conversion.
         bool special = false;
 #pragma unroll
-        for (int k = 0; k < NQ; ++k)
+        for (int k = 0; k < Q; ++k)
 #pragma unroll
             for (int e = 0; e < 4; ++e) special |= __builtin_amdgcn_classf(v[k][e], 0x3);
         if (__builtin_amdgcn_ballot_w64(special) == 0) {
             typedef _Float16 f16x2_t __attribute__((ext_vector_type(2)));
             typedef short s16x2_t __attribute__((ext_vector_type(2)));
-            const long off0b = b * P.ds[0] + n;
 #pragma unroll
-            for (int k = 0; k < NQ; ++k) {
+            for (int k = 0; k < Q; ++k) {
                 const f16x2_t lo = {(_Float16)v[k][0], (_Float16)v[k][1]}, hi = {(_Float16)v[k][2], (_Float16)v[k][3]};
                 s16x2_t r = {0, 0};
                 if (dt == MI355_DT_F8_E4M3) {
@@ -683,266 +751,232 @@ __device__ __forceinline__ void storeQ(const PT &P, const epi_hoist_t &H, const 
                     r = __builtin_amdgcn_cvt_scalef32_pk_bf8_f16(r, lo, 1.f, false);
                     r = __builtin_amdgcn_cvt_scalef32_pk_bf8_f16(r, hi, 1.f, true);
                 }
-                if (ok[k]) *(uint32_t *)((uint8_t *)P.dst + off0b + m[k] * P.ds[1]) = __builtin_bit_cast(uint32_t, r);
+                if (ok) *(uint32_t *)((uint8_t *)P.dst + rowoff + n[k]) = __builtin_bit_cast(uint32_t, r);
             }
             return;
         }
         if (dt == MI355_DT_F8_E4M3) {
 #pragma unroll
-            for (int k = 0; k < NQ; ++k)
+            for (int k = 0; k < Q; ++k)
 #pragma unroll
                 for (int e = 0; e < 4; ++e) w[k][e] = f32_to_e4m3(v[k][e]);
         } else {
 #pragma unroll
-            for (int k = 0; k < NQ; ++k)
+            for (int k = 0; k < Q; ++k)
 #pragma unroll
                 for (int e = 0; e < 4; ++e) w[k][e] = f32_to_e5m2(v[k][e]);
         }
-    } else { // s32 (nothing else is batchable)
+    } else { // s32 (nothing else is on the fast path)
 #pragma unroll
-        for (int k = 0; k < NQ; ++k)
+        for (int k = 0; k < Q; ++k)
 #pragma unroll
             for (int e = 0; e < 4; ++e)
                 w[k][e] = (uint32_t)(int)__builtin_rintf(sat(v[k][e], -2147483648.f, 2147483520.f));
     }
     const int bits = dt_bits(dt);
-    const long off0 = b * P.ds[0] + n;
+    if (!ok) return;
     if (bits == 8) {
 #pragma unroll
-        for (int k = 0; k < NQ; ++k)
-            if (ok[k])
-                *(uint32_t *)((uint8_t *)P.dst + off0 + m[k] * P.ds[1])
-                        = w[k][0] | (w[k][1] << 8) | (w[k][2] << 16) | (w[k][3] << 24);
+        for (int k = 0; k < Q; ++k)
+            *(uint32_t *)((uint8_t *)P.dst + rowoff + n[k]) = w[k][0] | (w[k][1] << 8) | (w[k][2] << 16) | (w[k][3] << 24);
     } else if (bits == 16) {
 #pragma unroll
-        for (int k = 0; k < NQ; ++k)
-            if (ok[k]) {
-                uint2 o;
-                o.x = w[k][0] | (w[k][1] << 16);
-                o.y = w[k][2] | (w[k][3] << 16);
-                *(uint2 *)((uint16_t *)P.dst + off0 + m[k] * P.ds[1]) = o;
-            }
+        for (int k = 0; k < Q; ++k) {
+            uint2 o;
+            o.x = w[k][0] | (w[k][1] << 16);
+            o.y = w[k][2] | (w[k][3] << 16);
+            *(uint2 *)((uint16_t *)P.dst + rowoff + n[k]) = o;
+        }
     } else {
 #pragma unroll
-        for (int k = 0; k < NQ; ++k)
-            if (ok[k]) {
-                uint4 o;
-                o.x = w[k][0]; o.y = w[k][1]; o.z = w[k][2]; o.w = w[k][3];
-                *(uint4 *)((uint32_t *)P.dst + off0 + m[k] * P.ds[1]) = o;
-            }
+        for (int k = 0; k < Q; ++k) {
+            uint4 o;
+            o.x = w[k][0]; o.y = w[k][1]; o.z = w[k][2]; o.w = w[k][3];
+            *(uint4 *)((uint32_t *)P.dst + rowoff + n[k]) = o;
+        }
     }
 }
 
-// One row of accumulator tiles copied by value.  The slab writers pick their rows
-// with a switch over the run-time slab number; were the cases identical code on
-// different addresses, the compiler would merge them into one copy that indexes
-// `acc` with a run-time offset, and all accumulators would live in private memory
-// from the first K step on.  The empty asm statements keep the cases apart
-// (statements of inline assembly are never merged).
-template <class T, int C>
-__device__ __forceinline__ void copy_row(const T (&src)[C], T (&dst)[C]) {
+// Dynamic (MX) quantization of dst for the quads of one row
+// (ref_matmul.cpp:338-423): a group is 32 consecutive n of the row = QPG quads
+// of this lane and the same quads of its partner lanes.  Writes the e8m0 scale
+// of every group and leaves v scaled and saturated, ready for the fp8
+// conversion.  All lanes take part in the cross-lane maximum, rows beyond M on
+// the data of a valid row; only the stores are masked.
+template <class Layout, int Q, class PT>
+__device__ __forceinline__ void dynamic_quantQ(const PT &P, int dst_dt, float (&v)[Q][4], long b, long m, bool ok,
+        const long (&n)[Q], int lane) {
+    constexpr int QPG = Layout::QPG;
+    const float dt_max = dst_dt == MI355_DT_F8_E4M3 ? 448.f : 57344.f;
+    const int em = (int)f32_to_e8m0(dt_max);
 #pragma unroll
-    for (int j = 0; j < C; ++j) {
-        T v = src[j];
-        asm volatile("" : "+v"(v));
-        dst[j] = v;
+    for (int g = 0; g < Q / QPG; ++g) {
+        float amax = 0.f;
+#pragma unroll
+        for (int kk = 0; kk < QPG; ++kk) amax = fmaxf(amax, amax4(v[g * QPG + kk]));
+        amax = Layout::group_max(amax);
+        float inv;
+        const uint8_t sbyte = mx_scale_byte(amax, em, inv);
+#pragma unroll
+        for (int kk = 0; kk < QPG; ++kk)
+#pragma unroll
+            for (int e = 0; e < 4; ++e) v[g * QPG + kk][e] = fminf(fmaxf(v[g * QPG + kk][e] * inv, -dt_max), dt_max);
+        if (ok && Layout::group_leader(lane))
+            ((uint8_t *)P.dst_scale.p)[quant_off(P.dst_scale, b, m, n[g * QPG] & ~31L, P.M, P.N)] = sbyte;
     }
 }
 
-// Accumulator layouts: how a wavefront's 128x128 quadrant sits in registers
-// and how one 32-row slab of it is written to LDS as [32 rows][128 cols] s32.
-//
-// 32x32 MFMA tiles, acc[4][4] of 16 registers: register r of tile (i, j) holds
-// row 32i + 8*(r/4) + 4*(lane/32) + r%4, column 32j + lane%32.
-struct layout32_t {
-    template <class T, int R, int C>
-    static __device__ __forceinline__ void write_slab(const T (&acc)[R][C], int s, slab_int_t *wl, int lane) {
-        constexpr int WCOLS = C * 32;
-        // The stores are written as ds_write_b32 instructions by hand.  Left to
-        // the compiler (ROCm 7.2) they were merged into ds_write2_b32 pairs, and
-        // two stores per tile of this layout came out with their first offset
-        // divided by four and landed in other cells of the slab (the parity
-        // tests caught it); as volatile stores they stayed single but each one
-        // was followed by a wait for the LDS queue to drain, 11-12 us per slab.
-        const unsigned base = (unsigned)(size_t)(__attribute__((address_space(3))) char *)(char *)wl
-                + (unsigned)(((lane >> 5) * 4 * WCOLS + (lane & 31)) * 4);
-        T a[C];
-        pick_rows(acc, s, a);
-#pragma unroll
-        for (int j = 0; j < C; ++j)
-#pragma unroll
-            for (int r = 0; r < 16; ++r) {
-                const unsigned addr = base + (unsigned)((((r >> 2) * 8 + (r & 3)) * WCOLS + j * 32) * 4);
-                asm volatile("ds_write_b32 %0, %1" : : "v"(addr), "v"(raw_bits(a[j][r])) : "memory");
-            }
-        // the wavefront reads its own slab next: LDS operations of one
-        // wavefront complete in order, the wait only keeps the compiler's own
-        // counter bookkeeping (which does not see these stores) conservative
-        asm volatile("s_waitcnt lgkmcnt(0)" : : : "memory");
-    }
-    template <class T, int R, int C>
-    static __device__ __forceinline__ void pick_rows(const T (&acc)[R][C], int s, T (&a)[C]) {
-        switch (s) {
-            case 0: copy_row(acc[0], a); break;
-            case 1: copy_row(acc[1], a); break;
-            case 2: copy_row(acc[2], a); break;
-            default: copy_row(acc[3], a); break;
-        }
-    }
-};
-
-// 16x16 MFMA tiles, acc[8][8] of 4 registers: register r of tile (i, j) holds
-// row 16i + 4*(lane/16) + r, column 16j + lane%16.
-struct layout16_t {
-    template <class T, int R, int C>
-    static __device__ __forceinline__ void write_slab(const T (&acc)[R][C], int s, slab_int_t *wl, int lane) {
-        constexpr int WCOLS = C * 16;
-        slab_int_t *vw = wl;
-        T a0[C], a1[C];
-        switch (s) {
-            case 0: copy_row(acc[0], a0); copy_row(acc[1], a1); break;
-            case 1: copy_row(acc[2], a0); copy_row(acc[3], a1); break;
-            case 2: copy_row(acc[4], a0); copy_row(acc[5], a1); break;
-            default: copy_row(acc[6], a0); copy_row(acc[7], a1); break;
-        }
-#pragma unroll
-        for (int j = 0; j < C; ++j)
-#pragma unroll
-            for (int r = 0; r < 4; ++r) {
-                vw[((lane >> 4) * 4 + r) * WCOLS + j * 16 + (lane & 15)] = raw_bits(a0[j][r]);
-                vw[(16 + (lane >> 4) * 4 + r) * WCOLS + j * 16 + (lane & 15)] = raw_bits(a1[j][r]);
-            }
-    }
-};
-
-// `conv.row(raw, m, f)` turns four raw accumulators of row m into the f32
-// values that enter the epilogue.
-// smem: one accumulator slab per wavefront (32 rows x WCOLS x 4 bytes), then
-// as much again for operand staging.
-// WCOLS: columns of the wavefront's part; NW: wavefronts of the workgroup.
-template <class Layout, int WCOLS, int NW, class PT, class Acc, class Conv>
-__device__ __forceinline__ void store_quadrant(const PT &P, char *smem, const Acc &acc,
-        long b, long m_base, long n_base_wave, bool interior, const Conv &conv) {
-    constexpr int LPR = WCOLS / 4;     // lanes per row: four consecutive n each
-    constexpr int RPP = 64 / LPR;      // rows per pass of the wavefront
-    constexpr int PASSES = 32 / RPP;   // passes per 32-row slab
-    constexpr int SLAB_INTS = 32 * WCOLS;
+// The epilogue of one wavefront's 128 x WCOLS part.
+//   park      lane-private LDS of the general path: Q x 64 x 16 bytes per wavefront
+//   ntab      LDS byte address of the per-column table (filled before the K loop)
+//   m_base    first row of the wavefront's part, n_base its first column, col0 =
+//             that column's index inside the tile (the table's index)
+//   conv      the kernel's conversion of raw accumulators:
+//                 row_t row_data(m)                         per-row operand
+//                 quad(raw, row_t, ntab, col, float (&f)[4])
+template <class Layout, int WCOLS, class PT, class T, int R, int C, class Conv>
+__device__ __forceinline__ void store_quadrant(const PT &P, char *park, unsigned ntab, const T (&acc)[R][C],
+        long b, long m_base, long n_base, int col0, const Conv &conv) {
+    constexpr int Q = Layout::template nq<C>();
+    constexpr int RB = Layout::RB, NB = Layout::NB, QPG = Layout::QPG;
+    static_assert(R == NB, "row blocks");
     const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
-    const int lrow = lane / LPR, lcol = lane % LPR;
-    slab_int_t *wl = (slab_int_t *)smem + wave * SLAB_INTS;
-    stage_u4_t *stg = (stage_u4_t *)(smem + NW * SLAB_INTS * 4) + wave * (PASSES * 64);
-    const long nbase = n_base_wave + lcol * 4;
-    int nvalid = 0;
-#pragma unroll
-    for (int e = 0; e < 4; ++e)
-        if (nbase + e < P.N) nvalid = e + 1;
-    const epi_hoist_t H = make_hoist(P, b, nbase, nvalid, interior);
-    const int sbytes = dt_bits(H.staged_dt) / 8;
+    const int lrow = Layout::lrow(lane);
+    const bool cols_inside = n_base + WCOLS <= P.N;
+    const epi_uniform_t H = make_uniform(P, cols_inside);
+    typedef typename Conv::row_t row_t;
 
-    // rolled over the four slabs: the epilogue arithmetic exists once
-#pragma unroll 1
-    for (int i = 0; i < 4; ++i) {
-        if (H.staged != STG_NONE) {
-            // PASSES independent vector loads in flight, then park them in LDS
-            uint4 tmp[PASSES];
-            const char *base = H.staged_p
-                    + (b * H.st_s0 + (m_base + i * 32 + lrow) * H.st_s1 + nbase) * sbytes;
+    if (H.fast) {
+        int col[Q];
+        long n[Q];
+#pragma unroll
+        for (int k = 0; k < Q; ++k) {
+            col[k] = col0 + Layout::qcol(k, lane);
+            n[k] = n_base + Layout::qcol(k, lane);
+        }
+        const int sbytes = H.staged != STG_NONE ? dt_bits(H.staged_dt) / 8 : 0;
+        // the staged stream's quads of a row, as raw 8 or 16 bytes
+        auto load_staged = [&](long m, uint4 (&s)[Q]) __attribute__((always_inline)) {
+            const char *base = H.staged_p + (b * H.st_s0 + m * H.st_s1 + n_base) * sbytes;
             if (sbytes == 2) {
 #pragma unroll
-                for (int it = 0; it < PASSES; ++it) {
-                    const uint2 q = *(const uint2 *)(base + (long)it * RPP * H.st_s1 * 2);
-                    tmp[it].x = q.x; tmp[it].y = q.y; tmp[it].z = 0; tmp[it].w = 0;
+                for (int k = 0; k < Q; ++k) {
+                    const uint2 q = *(const uint2 *)(base + Layout::qcol(k, lane) * 2);
+                    s[k].x = q.x; s[k].y = q.y; s[k].z = 0; s[k].w = 0;
                 }
             } else {
 #pragma unroll
-                for (int it = 0; it < PASSES; ++it)
-                    tmp[it] = *(const uint4 *)(base + (long)it * RPP * H.st_s1 * 4);
+                for (int k = 0; k < Q; ++k) s[k] = *(const uint4 *)(base + Layout::qcol(k, lane) * 4);
             }
+        };
+        auto row_of = [&](int i) { return m_base + i * RB + lrow; };
+        auto clamp_row = [&](long m) { return m < P.M ? m : P.M - 1; };
+        uint4 snext[Q];
 #pragma unroll
-            for (int it = 0; it < PASSES; ++it) stg[it * 64 + lane] = tmp[it];
-        }
-        Layout::write_slab(acc, i, wl, lane);
-        if (H.batchable) {
-            constexpr int NQ = 4;
+        for (int k = 0; k < Q; ++k) snext[k] = make_uint4(0, 0, 0, 0);
+        row_t rnext = conv.row_data(clamp_row(row_of(0)));
+        if (H.staged != STG_NONE) load_staged(clamp_row(row_of(0)), snext);
 #pragma unroll 1
-            for (int it0 = 0; it0 < PASSES; it0 += NQ) {
-                v4i_t raw[NQ];
-                uint4 sv[NQ];
-                long m[NQ];
-                bool ok[NQ];
+        for (int i = 0; i < NB; ++i) {
+            T a[C];
+            Layout::pick_rows(acc, i, a);
+            const long m = row_of(i);
+            const bool ok = m < P.M;
+            const row_t rd = rnext;
+            uint4 scur[Q];
 #pragma unroll
-                for (int k = 0; k < NQ; ++k) {
-                    const int row = (it0 + k) * RPP + lrow;
-                    m[k] = m_base + i * 32 + row;
-                    ok[k] = m[k] < P.M;
-                    raw[k] = *(const slab_v4i_t *)&wl[row * WCOLS + lcol * 4];
-                    sv[k] = make_uint4(0, 0, 0, 0);
-                }
-                if (H.staged != STG_NONE) {
-#pragma unroll
-                    for (int k = 0; k < NQ; ++k) sv[k] = stg[(it0 + k) * 64 + lane];
-                }
-                float v[NQ][4];
-#pragma unroll
-                for (int k = 0; k < NQ; ++k) conv.row(raw[k], ok[k] ? m[k] : m_base, v[k]);
-                apply_epilogueQ<NQ>(H, v, sv);
-                if (H.dynamic) dynamic_quantQ<NQ>(P, H, v, b, m, nbase, ok, lcol);
-                storeQ<NQ>(P, H, v, b, m, nbase, ok);
+            for (int k = 0; k < Q; ++k) scur[k] = snext[k];
+            if (i + 1 < NB) {
+                const long mn = clamp_row(row_of(i + 1));
+                rnext = conv.row_data(mn);
+                if (H.staged != STG_NONE) load_staged(mn, snext);
             }
-            continue;
-        }
-        if (H.dynamic) {
-            // Dynamic (MX) quantization of dst, ref_matmul.cpp:338-423: a group is
-            // 32 consecutive n of one row = 8 consecutive lanes of this layout
-            // (four n each; a wavefront's columns start at a multiple of 64 and
-            // N % 32 == 0, so a group is whole or absent).  All lanes run the
-            // arithmetic and the cross-lane maximum, rows beyond M on the data of
-            // a valid row; only the stores are masked.
-            const float dt_max = H.dst_dt == MI355_DT_F8_E4M3 ? 448.f : 57344.f;
-            const int em = (int)f32_to_e8m0(dt_max);
-#pragma unroll 1
-            for (int it = 0; it < PASSES; ++it) {
-                const int row = it * RPP + lrow;
-                const long m = m_base + i * 32 + row;
-                const bool ok = m < P.M && nvalid > 0;
-                const long mv = m < P.M ? m : P.M - 1;
-                const v4i_t raw = *(const slab_v4i_t *)&wl[row * WCOLS + lcol * 4];
-                uint4 sv = make_uint4(0, 0, 0, 0);
-                if (H.staged != STG_NONE) sv = stg[it * 64 + lane];
-                float v[4] = {0.f, 0.f, 0.f, 0.f};
-                if (nvalid > 0) {
-                    conv.row(raw, mv, v);
-                    apply_epilogue4(P, H, v, b, mv, nbase, nvalid, sv);
+            float v[Q][4], sy[Q][4];
+#pragma unroll
+            for (int k = 0; k < Q; ++k) conv.quad(Layout::quad(a, k), rd, ntab, col[k], v[k]);
+#pragma unroll
+            for (int k = 0; k < Q; ++k)
+#pragma unroll
+                for (int e = 0; e < 4; ++e) sy[k][e] = 0.f;
+            if (H.staged != STG_NONE) {
+                // one dispatch on the data type for the Q quads
+                if (H.staged_dt == MI355_DT_BF16) {
+#pragma unroll
+                    for (int k = 0; k < Q; ++k) staged4(MI355_DT_BF16, scur[k], sy[k]);
+                } else if (H.staged_dt == MI355_DT_F32) {
+#pragma unroll
+                    for (int k = 0; k < Q; ++k) staged4(MI355_DT_F32, scur[k], sy[k]);
+                } else if (H.staged_dt == MI355_DT_F16) {
+#pragma unroll
+                    for (int k = 0; k < Q; ++k) staged4(MI355_DT_F16, scur[k], sy[k]);
+                } else {
+#pragma unroll
+                    for (int k = 0; k < Q; ++k) staged4(MI355_DT_S32, scur[k], sy[k]);
                 }
-                float amax = fmaxf(fmaxf(fabsf(v[0]), fabsf(v[1])), fmaxf(fabsf(v[2]), fabsf(v[3])));
-                amax = fmaxf(amax, __shfl_xor(amax, 1, 64));
-                amax = fmaxf(amax, __shfl_xor(amax, 2, 64));
-                amax = fmaxf(amax, __shfl_xor(amax, 4, 64));
+            }
+            apply_epilogueQ<Q>(H, ntab, col, v, sy);
+            if (H.dynamic) dynamic_quantQ<Layout, Q>(P, H.dst_dt, v, b, ok ? m : P.M - 1, ok, n, lane);
+            storeQ<Q>(P, H, v, b, m, ok, n);
+        }
+        return;
+    }
+
+    // ---- general path: the quads of a row block parked in lane-private LDS, then
+    // one group of 32 columns at a time through the interpreter
+    park_u4_t *pk = (park_u4_t *)park + wave * (Q * 64);
+#pragma unroll 1
+    for (int i = 0; i < NB; ++i) {
+        {
+            T a[C];
+            Layout::pick_rows(acc, i, a);
+#pragma unroll
+            for (int k = 0; k < Q; ++k) {
+                const v4i_t q = Layout::quad(a, k);
+                pk[k * 64 + lane] = make_uint4((unsigned)q[0], (unsigned)q[1], (unsigned)q[2], (unsigned)q[3]);
+            }
+        }
+        const long m = m_base + i * RB + lrow;
+        const bool okm = m < P.M;
+        const long mv = okm ? m : P.M - 1;
+        const row_t rd = conv.row_data(mv);
+        const float dt_max = P.dst_dt == MI355_DT_F8_E4M3 ? 448.f : 57344.f;
+        const int em = (int)f32_to_e8m0(dt_max);
+#pragma unroll 1
+        for (int g = 0; g < Q / QPG; ++g) {
+            float v[QPG][4];
+            long nq[QPG];
+            int nvalid[QPG];
+            float amax = 0.f;
+#pragma unroll
+            for (int kk = 0; kk < QPG; ++kk) {
+                const int k = g * QPG + kk;
+                const int qc = Layout::qcol(k, lane);
+                nq[kk] = n_base + qc;
+                const long left = P.N - nq[kk];
+                nvalid[kk] = left >= 4 ? 4 : left > 0 ? (int)left : 0;
+                const uint4 raw = pk[k * 64 + lane];
+                conv.quad(v4i_t {(int)raw.x, (int)raw.y, (int)raw.z, (int)raw.w}, rd, ntab, col0 + qc, v[kk]);
+                if (nvalid[kk] > 0) apply_epilogue4(P, v[kk], b, mv, nq[kk], nvalid[kk]);
+#pragma unroll
+                for (int e = 0; e < 4; ++e)
+                    if (e >= nvalid[kk]) v[kk][e] = 0.f;
+                amax = fmaxf(amax, amax4(v[kk]));
+            }
+            if (H.dynamic) {
+                // N is a multiple of 32: a group is whole or absent
+                amax = Layout::group_max(amax);
                 float inv;
                 const uint8_t sbyte = mx_scale_byte(amax, em, inv);
 #pragma unroll
-                for (int e = 0; e < 4; ++e) v[e] = fminf(fmaxf(v[e] * inv, -dt_max), dt_max);
-                if (ok) {
-                    if ((lcol & 7) == 0)
-                        ((uint8_t *)P.dst_scale.p)[quant_off(P.dst_scale, b, m, nbase, P.M, P.N)] = sbyte;
-                    store4(P, H, v, b, m, nbase, nvalid);
-                }
+                for (int kk = 0; kk < QPG; ++kk)
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) v[kk][e] = fminf(fmaxf(v[kk][e] * inv, -dt_max), dt_max);
+                if (okm && nvalid[0] > 0 && Layout::group_leader(lane))
+                    ((uint8_t *)P.dst_scale.p)[quant_off(P.dst_scale, b, m, nq[0] & ~31L, P.M, P.N)] = sbyte;
             }
-            continue;
-        }
-#pragma unroll 1
-        for (int it = 0; it < PASSES; ++it) {
-            const int row = it * RPP + lrow;
-            const long m = m_base + i * 32 + row;
-            const v4i_t raw = *(const slab_v4i_t *)&wl[row * WCOLS + lcol * 4];
-            uint4 sv = make_uint4(0, 0, 0, 0);
-            if (H.staged != STG_NONE) sv = stg[it * 64 + lane];
-            if (m < P.M && nvalid > 0) {
-                float v[4];
-                conv.row(raw, m, v);
-                apply_epilogue4(P, H, v, b, m, nbase, nvalid, sv);
-                store4(P, H, v, b, m, nbase, nvalid);
-            }
+#pragma unroll
+            for (int kk = 0; kk < QPG; ++kk)
+                if (okm && nvalid[kk] > 0) store4(P, H.dst_vec, v[kk], b, m, nq[kk], nvalid[kk]);
         }
     }
 }

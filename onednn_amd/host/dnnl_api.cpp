@@ -249,6 +249,19 @@ struct dnnl_primitive {
     std::unique_ptr<dnnl_primitive_desc> rt_pd;
     std::vector<void *> rt_scratch;
     size_t rt_scratch_bytes = 0;
+    // Executions that use the primitive's own device memory (library-mode
+    // scratchpad, host-scalar slots, runtime-dims scratch) are ordered on the
+    // device as well as on the host: each records `order_event` behind its
+    // launches, and the next one on another stream makes its stream wait for it.
+    void *order_event = nullptr;
+    void *last_stream = nullptr;
+    bool event_recorded = false;
+    ~dnnl_primitive() {
+        if (scratch) mi355_mem_free(scratch);
+        for (void *q : rt_scratch) mi355_mem_free(q);
+        if (host_scalars) mi355_mem_free(host_scalars);
+        if (order_event) mi355_event_destroy(order_event);
+    }
 };
 
 namespace {
@@ -1656,12 +1669,7 @@ DNNL_EXPORT dnnl_status_t dnnl_primitive_get_primitive_desc(const_dnnl_primitive
     return dnnl_success;
 }
 DNNL_EXPORT dnnl_status_t dnnl_primitive_destroy(dnnl_primitive_t primitive) {
-    if (primitive) {
-        if (primitive->scratch) mi355_mem_free(primitive->scratch);
-        for (void *q : primitive->rt_scratch) mi355_mem_free(q);
-        if (primitive->host_scalars) mi355_mem_free(primitive->host_scalars);
-        delete primitive;
-    }
+    delete primitive; // the destructor frees the device memory and the event
     return dnnl_success;
 }
 
@@ -1678,11 +1686,24 @@ DNNL_EXPORT dnnl_status_t dnnl_primitive_execute(const_dnnl_primitive_t cprimiti
         m[args[i].arg] = args[i].memory;
     }
     std::unique_lock<std::mutex> lock(prim->scratch_mutex, std::defer_lock);
+    // Called before the first use of the primitive's own device memory in this
+    // execution: takes the host lock and, if the previous such execution ran on
+    // another stream, makes this stream wait for it.
+    bool ordered = false;
+    auto order_on_device = [&]() {
+        if (ordered) return;
+        ordered = true;
+        if (!lock.owns_lock()) lock.lock();
+        if (!prim->order_event) mi355_event_create(&prim->order_event); // the device is current here
+        if (prim->order_event && prim->event_recorded && prim->last_stream != stream->hip_stream)
+            mi355_stream_wait_event(stream->hip_stream, prim->order_event);
+    };
     void *rt_scratch = nullptr;
     if (pd0.runtime) {
         // executions of one primitive with runtime dims are serialised on the
         // host while they enqueue: they share the cached lowering and scratch
-        lock.lock();
+        if (mi355_device_set((int)pd0.engine->index) != MI355_SUCCESS) return dnnl_runtime_error;
+        order_on_device();
         dnnl_status_t rs = concretize(*prim, m, &rt_scratch);
         if (rs) return rs;
     }
@@ -1751,7 +1772,10 @@ DNNL_EXPORT dnnl_status_t dnnl_primitive_execute(const_dnnl_primitive_t cprimiti
             CHECK_ARG(mem && mem->md.kind == dnnl_format_kind_host_scalar && (int)mem->md.dt == lowered.dt);
             if (!prim->host_scalars) return dnnl_runtime_error;
             void *dev = (char *)prim->host_scalars + 8 * my_slot;
-            const int rc = mi355_mem_h2d(dev, mem->scalar, dt_bits(mem->md.dt) / 8, stream->hip_stream);
+            order_on_device();
+            uint64_t bits = 0;
+            memcpy(&bits, mem->scalar, dt_bits(mem->md.dt) / 8);
+            const int rc = mi355_mem_store_scalar(dev, bits, dt_bits(mem->md.dt) / 8, stream->hip_stream);
             if (rc != MI355_SUCCESS) return from_mi355(rc);
             *field = dev;
             return dnnl_success;
@@ -1789,7 +1813,8 @@ DNNL_EXPORT dnnl_status_t dnnl_primitive_execute(const_dnnl_primitive_t cprimiti
     } else if (scratch) {
         // the library-mode scratchpad belongs to the primitive: executions of
         // one primitive object are serialised on the host while they enqueue
-        lock.lock();
+        // and, across streams, on the device
+        order_on_device();
     }
     if (mi355_device_set((int)pd.engine->index) != MI355_SUCCESS) return dnnl_runtime_error;
     const auto t0 = std::chrono::steady_clock::now();
@@ -1819,6 +1844,12 @@ DNNL_EXPORT dnnl_status_t dnnl_primitive_execute(const_dnnl_primitive_t cprimiti
             for (int k = 0; k < pd.desc.n_post_ops; ++k)
                 if (pd.desc.post_ops[k].kind == MI355_PO_BINARY) B.po_arg[k] = shifted(A.po_arg[k], op[k], pd.desc.post_ops[k].dt);
             rc = mi355_matmul_launch(&pd.desc, &B, scratch, stream->hip_stream);
+        }
+    }
+    if (ordered && prim->order_event) {
+        if (mi355_event_record(prim->order_event, stream->hip_stream) == MI355_SUCCESS) {
+            prim->event_recorded = true;
+            prim->last_stream = stream->hip_stream;
         }
     }
     if (verbose_level() >= 2) {

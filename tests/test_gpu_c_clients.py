@@ -1,0 +1,46 @@
+"""The boundary through a compiler: two small C programs that include only
+include/dnnl_amd.h / include/mi355_matmul.h, built with gcc against the two
+shared libraries and run on the device (a u8 x s8 -> s32 matmul checked against
+an integer loop inside the program).  Struct layouts, enum values and calling
+conventions of the headers are what a compiled caller sees; the ctypes tests
+only check names."""
+import os
+import shutil
+import subprocess
+import tempfile
+
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+INC = os.path.join(ROOT, "include")
+LIB = os.path.join(ROOT, "onednn_amd", "lib")
+
+
+def build(name, lib):
+    if shutil.which("gcc") is None:
+        pytest.skip("no host compiler")
+    d = tempfile.mkdtemp(prefix="cclient")
+    exe = os.path.join(d, name)
+    subprocess.check_call(["gcc", "-std=c11", "-Wall", "-Wextra", "-Werror", "-I", INC, "-o", exe,
+                           os.path.join(ROOT, "tests", "c_clients", name + ".c"), "-L", LIB, "-l" + lib,
+                           "-Wl,-rpath," + LIB])
+    return d, exe
+
+
+def test_headers_compile_as_c_and_link():
+    # no device needed: the programs build against the headers and libraries
+    for name, lib in (("dnnl_client", "dnnl_amd"), ("mi355_client", "mi355_matmul")):
+        d, exe = build(name, lib)
+        assert os.path.exists(exe)
+        shutil.rmtree(d, ignore_errors=True)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("name,lib", [("dnnl_client", "dnnl_amd"), ("mi355_client", "mi355_matmul")])
+def test_c_client_runs_on_the_device(gpu, name, lib):
+    d, exe = build(name, lib)
+    try:
+        out = subprocess.run([exe], capture_output=True, text=True, timeout=120)
+        assert out.returncode == 0 and out.stdout.startswith("ok hip:mfma_i8"), (out.stdout, out.stderr)
+    finally:
+        shutil.rmtree(d, ignore_errors=True)

@@ -549,3 +549,45 @@ def test_binary_select_post_op(gpu, oracle):
         dnnl.ARG_ATTR_MULTIPLE_POST_OP(1) | dnnl.ARG_SRC_2: dnnl.memory(c_md, eng, cond)})
     strm.wait()
     assert np.array_equal(dst.read(np.int32).reshape(M, N), want)
+
+
+def test_one_primitive_two_threads_two_streams(gpu, oracle):
+    """primitive_t::execute is const and may run concurrently from several host threads on different streams
+    (src/common/primitive.hpp:54).  u8 src + row-major weights: the transposed weights and the column sums live in the
+    primitive's own scratchpad, which both executions use -- the second stream waits for the first one's launches."""
+    import threading
+    p = configs.config1(M=256, N=512, K=512, dst="s32")
+    want = np.asarray(oracle.run_oracle(p)).view(np.int32).reshape(p.M, p.N)
+    eng = dnnl.engine(dnnl.gpu, 0)
+    mds = [dnnl.memory_desc([p.M, p.K], p.src_dt, tag=dnnl.tag_ab), dnnl.memory_desc([p.K, p.N], p.wei_dt, tag=dnnl.tag_ab),
+           dnnl.memory_desc([p.M, p.N], p.dst_dt, tag=dnnl.tag_ab)]
+    attr = dnnl.primitive_attr()
+    attr.set_zero_points_mask(dnnl.ARG_SRC, 0)
+    pd = dnnl.matmul_primitive_desc(eng, mds[0], mds[1], mds[2], attr=attr)
+    assert pd.impl_info_str().startswith("hip:mfma_i8")
+    prim = dnnl.matmul(pd)
+    wei = dnnl.memory(mds[1], eng, p.wei)
+    zp = dnnl.memory(dnnl.memory_desc([1], DT["s32"], tag=dnnl.tag_a), eng, p.quant["src_zp"].data)
+    # each thread multiplies its own src (a row permutation of the problem's) into its own dst
+    perms = [np.arange(p.M), np.arange(p.M)[::-1].copy()]
+    errors = []
+
+    def worker(t):
+        strm = dnnl.stream(eng)
+        src = dnnl.memory(mds[0], eng, np.ascontiguousarray(p.src[perms[t]]))
+        dst = dnnl.memory(mds[2], eng)
+        for it in range(50):
+            prim.execute(strm, {dnnl.ARG_SRC: src, dnnl.ARG_WEIGHTS: wei, dnnl.ARG_DST: dst,
+                                dnnl.ARG_ATTR_ZERO_POINTS | dnnl.ARG_SRC: zp})
+            strm.wait()
+            got = dst.read(np.int32).reshape(p.M, p.N)
+            if not np.array_equal(got, want[perms[t]]):
+                errors.append((t, it, int(np.count_nonzero(got != want[perms[t]]))))
+                return
+
+    threads = [threading.Thread(target=worker, args=(t,)) for t in range(2)]
+    for th in threads:
+        th.start()
+    for th in threads:
+        th.join()
+    assert not errors, errors
