@@ -82,6 +82,9 @@ struct f8_mma_t {
     }
 };
 
+// HOT: whether the kernel instantiation carries the compile-time specialised
+// chains (e4m3 x e4m3 only: each one multiplies the code of the epilogue)
+template <bool HOT>
 struct f8_conv_t {
     typedef float row_t;
     float ssc_common;
@@ -96,6 +99,123 @@ struct f8_conv_t {
     }
     __device__ __forceinline__ float row_data(long m) const {
         return ssc_p ? load_float(ssc_dt, ssc_p, m) : ssc_common;
+    }
+
+    // The chain of the fp8 up-projection configuration and its subsets, fully
+    // unrolled over the wavefront's 4 x C accumulator tiles with every choice a
+    // template parameter:
+    //   acc * src_scale * wei_scale[n]  [+ bias[n]]  [-> gelu_tanh]  [+ bf16 residual]  -> bf16
+    // The residual quads (8 bytes per lane) are loaded four tiles ahead of their use.
+    template <bool BIAS, bool GELU, bool ADD, class PT, int C>
+    __device__ __forceinline__ void hot_store(const PT &P, const epi_uniform_t &H, unsigned ntab,
+            const v16f (&acc)[4][C], long b, long m_base, long n_base, int col0) const {
+        constexpr int NU = 4 * C, PF = 4; // units (tiles) of the wavefront; prefetch distance
+        const int lane = threadIdx.x & 63, lrow = lane & 31, ch = 4 * (lane >> 5);
+        uint16_t *dcol = (uint16_t *)P.dst + b * P.ds[0] + n_base + ch;
+        const uint16_t *rcol = ADD ? (const uint16_t *)H.staged_p + b * H.st_s0 + n_base + ch : nullptr;
+        auto row_of = [&](int u) { return m_base + 32 * (u / C) + lrow; };
+        auto load_res = [&](int u, uint2 (&r)[4]) __attribute__((always_inline)) {
+            long m = row_of(u);
+            m = m < P.M ? m : P.M - 1;
+            const uint16_t *p = rcol + m * H.st_s1 + 32 * (u % C);
+#pragma unroll
+            for (int g = 0; g < 4; ++g) r[g] = *(const uint2 *)(p + 8 * g);
+        };
+        uint2 res[PF + 1][4];
+        if (ADD) {
+#pragma unroll
+            for (int u = 0; u < PF; ++u) load_res(u, res[u]);
+        }
+#pragma unroll
+        for (int u = 0; u < NU; ++u) {
+            const int i = u / C, j = u % C;
+            if (ADD && u + PF < NU) load_res(u + PF, res[(u + PF) % (PF + 1)]);
+            const long m = row_of(u);
+            float x[4][4];
+            bool special = false;
+#pragma unroll
+            for (int g = 0; g < 4; ++g) {
+                // keeps the table reads of every tile apart: merged, the 32 columns'
+                // operands of all tiles would stay in registers
+                int col = col0 + 32 * j + 8 * g + ch;
+                asm volatile("" : "+v"(col));
+                v4f_t w = {1.f, 1.f, 1.f, 1.f}, bb = {0.f, 0.f, 0.f, 0.f};
+                if (with_wei_sc) w = nt4f(ntab, NT_WSC, col);
+                if (BIAS) bb = nt4f(ntab, NT_BIAS, col);
+                float y[4] = {0.f, 0.f, 0.f, 0.f};
+                if (ADD) {
+                    const uint2 r = res[u % (PF + 1)][g];
+                    y[0] = u2f(r.x << 16); y[1] = u2f(r.x & 0xffff0000u);
+                    y[2] = u2f(r.y << 16); y[3] = u2f(r.y & 0xffff0000u);
+                }
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    float t = acc[i][j][4 * g + e];
+                    if (with_src_sc) t *= ssc_common;
+                    if (with_wei_sc) t *= w[e];
+                    if (BIAS) t += bb[e];
+                    if (GELU) t = gelu_tanh_fast(t);
+                    if (ADD) t += y[e];
+                    special |= __builtin_amdgcn_classf(t, 0x93); // NaN or subnormal: software conversion
+                    x[g][e] = t;
+                }
+            }
+            typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
+            typedef float f32x2_t __attribute__((ext_vector_type(2)));
+            uint2 o[4];
+            if (__builtin_amdgcn_ballot_w64(special) == 0) {
+#pragma unroll
+                for (int g = 0; g < 4; ++g) {
+                    o[g].x = __builtin_bit_cast(unsigned, __builtin_convertvector(f32x2_t {x[g][0], x[g][1]}, bf16x2_t));
+                    o[g].y = __builtin_bit_cast(unsigned, __builtin_convertvector(f32x2_t {x[g][2], x[g][3]}, bf16x2_t));
+                }
+            } else {
+#pragma unroll
+                for (int g = 0; g < 4; ++g) {
+                    o[g].x = f32_to_bf16(x[g][0]) | ((unsigned)f32_to_bf16(x[g][1]) << 16);
+                    o[g].y = f32_to_bf16(x[g][2]) | ((unsigned)f32_to_bf16(x[g][3]) << 16);
+                }
+            }
+            if (m < P.M) {
+                uint16_t *d = dcol + m * P.ds[1] + 32 * j;
+#pragma unroll
+                for (int g = 0; g < 4; ++g) *(uint2 *)(d + 8 * g) = o[g];
+            }
+        }
+    }
+    template <class PT, int C>
+    __device__ __forceinline__ bool hot_chain(const PT &P, const epi_uniform_t &H, unsigned ntab,
+            const v16f (&acc)[4][C], long b, long m_base, long n_base, int col0) const {
+        if (!HOT || ssc_p || H.bias_mode == 2 || H.ds_mode != 0 || H.dzp_mode != 0 || H.dynamic || H.dst_dt != MI355_DT_BF16
+                || H.n_po > 2)
+            return false;
+        auto is_gelu = [](const po_reg_t &r) {
+            return r.kind == MI355_PO_ELTWISE && r.alg == MI355_ELTWISE_GELU_TANH && r.scale == 1.f;
+        };
+        auto is_res = [&](const po_reg_t &r, int i) {
+            return r.kind == MI355_PO_BINARY && r.alg == MI355_BINARY_ADD && i == H.staged && H.staged_dt == MI355_DT_BF16;
+        };
+        bool gelu = false, add = false;
+        if (H.n_po == 1) {
+            gelu = is_gelu(H.pf0);
+            add = is_res(H.pf0, 0);
+            if (!gelu && !add) return false;
+        } else if (H.n_po == 2) {
+            gelu = is_gelu(H.pf0);
+            add = is_res(H.pf1, 1);
+            if (!gelu || !add) return false;
+        }
+        const bool bias = H.bias_mode == 1;
+#define MI355_F8_HOT(B, G, A) hot_store<B, G, A>(P, H, ntab, acc, b, m_base, n_base, col0)
+        if (bias) {
+            if (gelu) { if (add) MI355_F8_HOT(true, true, true); else MI355_F8_HOT(true, true, false); }
+            else { if (add) MI355_F8_HOT(true, false, true); else MI355_F8_HOT(true, false, false); }
+        } else {
+            if (gelu) { if (add) MI355_F8_HOT(false, true, true); else MI355_F8_HOT(false, true, false); }
+            else { if (add) MI355_F8_HOT(false, false, true); else MI355_F8_HOT(false, false, false); }
+        }
+#undef MI355_F8_HOT
+        return true;
     }
     __device__ __forceinline__ void quad(const v4i_t &raw, float ssc, unsigned ntab, int col, float (&f)[4]) const {
 #pragma unroll
@@ -130,7 +250,7 @@ __global__ void __launch_bounds__(G::NT) __attribute__((amdgpu_waves_per_eu(G::N
     const char *Bt = X.bt + b * X.bt_bstride + n0 * X.ldb;
 
     const long bs = P.ss[0] ? b : 0, bw = P.ws[0] ? b : 0;
-    f8_conv_t cv;
+    f8_conv_t<FMT_A == 0 && FMT_B == 0> cv;
     cv.with_src_sc = P.src_scale.dt != MI355_DT_UNDEF;
     cv.with_wei_sc = P.wei_scale.dt != MI355_DT_UNDEF;
     cv.ssc_common = 1.f;

@@ -99,6 +99,81 @@ struct i8_conv_t {
             wsc = load_float(P.wei_scale.dt, P.wei_scale.p, quant_off(P.wei_scale, bw, 0, n, P.K, P.N));
     }
     __device__ __forceinline__ int row_data(long m) const { return rowsum ? rowsum[m] : 0; }
+
+    // The chain of the compute-bound int8 configuration and its neighbours, fully
+    // unrolled over the wavefront's 8 x 4 accumulator tiles with every choice a
+    // template parameter:
+    //   f32(acc) * src_scale * wei_scale[n]  [-> max(., 0)]  [-> / dst_scale]  -> s8 / u8
+    // (no compensation terms, no bias, no zero points).  Per element: convert, two
+    // multiplications, maximum, five operations of the fma-corrected division,
+    // round, convert, clamp, 3/4 of a byte permute.
+    template <bool RELU, int DS, class PT>
+    __device__ __forceinline__ void hot_store(const PT &P, const epi_uniform_t &H, unsigned ntab,
+            const v4i (&acc)[8][4], long b, long m_base, long n_base, int col0) const {
+        const int lane = threadIdx.x & 63, lrow = lane & 15, cq = 4 * (lane >> 4);
+        v4f_t w[4];
+#pragma unroll
+        for (int k = 0; k < 4; ++k) w[k] = nt4f(ntab, NT_WSC, col0 + 16 * k + cq);
+        const int lo = H.dst_dt == MI355_DT_S8 ? -128 : 0, hi = H.dst_dt == MI355_DT_S8 ? 127 : 255;
+        uint8_t *dcol = (uint8_t *)P.dst + b * P.ds[0] + n_base + cq;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            const long m = m_base + 16 * i + lrow;
+            float x[4][4];
+            unsigned mx = 0;
+#pragma unroll
+            for (int k = 0; k < 4; ++k)
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    float t = (float)acc[i][k][e] * ssc;
+                    t *= w[k][e];
+                    if (RELU) t = fmaxf(t, 0.f); // an integer dst turns NaN and -0 into 0 either way
+                    if (DS == 2) t *= H.ds_inv;
+                    if (DS == 3) mx = max(mx, mag_bits(t));
+                    x[k][e] = t;
+                }
+            if (DS == 3) {
+                if (__builtin_amdgcn_ballot_w64(mx >= DIV_BY_FMA_LIMIT) == 0) {
+#pragma unroll
+                    for (int k = 0; k < 4; ++k)
+#pragma unroll
+                        for (int e = 0; e < 4; ++e) x[k][e] = div_by_fma(x[k][e], H.ds, H.ds_inv);
+                } else {
+#pragma unroll
+                    for (int k = 0; k < 4; ++k)
+#pragma unroll
+                        for (int e = 0; e < 4; ++e) x[k][e] /= H.ds;
+                }
+            }
+            unsigned word[4];
+#pragma unroll
+            for (int k = 0; k < 4; ++k) word[k] = pack4_i8(x[k], lo, hi);
+            if (m < P.M) {
+                uint8_t *d = dcol + m * P.ds[1];
+#pragma unroll
+                for (int k = 0; k < 4; ++k) *(uint32_t *)(d + 16 * k) = word[k];
+            }
+        }
+    }
+    template <class PT>
+    __device__ __forceinline__ bool hot_chain(const PT &P, const epi_uniform_t &H, unsigned ntab,
+            const v4i (&acc)[8][4], long b, long m_base, long n_base, int col0) const {
+        const bool relu0 = H.n_po == 1 && H.pf0.kind == MI355_PO_ELTWISE && H.pf0.alg == MI355_ELTWISE_RELU
+                && H.pf0.alpha == 0.f && H.pf0.scale == 1.f;
+        if (has_comp || !with_src_sc || !with_wei_sc || H.bias_mode != 0 || H.dzp_mode != 0 || H.dynamic
+                || (H.n_po != 0 && !relu0) || H.ds_mode == 1 || (H.dst_dt != MI355_DT_S8 && H.dst_dt != MI355_DT_U8))
+            return false;
+        if (relu0) {
+            if (H.ds_mode == 0) hot_store<true, 0>(P, H, ntab, acc, b, m_base, n_base, col0);
+            else if (H.ds_mode == 2) hot_store<true, 2>(P, H, ntab, acc, b, m_base, n_base, col0);
+            else hot_store<true, 3>(P, H, ntab, acc, b, m_base, n_base, col0);
+        } else {
+            if (H.ds_mode == 0) hot_store<false, 0>(P, H, ntab, acc, b, m_base, n_base, col0);
+            else if (H.ds_mode == 2) hot_store<false, 2>(P, H, ntab, acc, b, m_base, n_base, col0);
+            else hot_store<false, 3>(P, H, ntab, acc, b, m_base, n_base, col0);
+        }
+        return true;
+    }
     __device__ __forceinline__ void quad(const v4i_t &raw, int rs, unsigned ntab, int col, float (&f)[4]) const {
         int v[4] = {raw[0], raw[1], raw[2], raw[3]};
         if (has_comp) {

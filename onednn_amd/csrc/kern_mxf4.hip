@@ -126,6 +126,11 @@ struct mxf4_conv_t {
     template <class PT>
     __device__ __forceinline__ void per_n(const PT &, long, long, float &, int &, int &) const {}
     __device__ __forceinline__ int row_data(long) const { return 0; }
+    template <class PT, class Acc>
+    __device__ __forceinline__ bool hot_chain(const PT &, const epi_uniform_t &, unsigned, const Acc &, long, long,
+            long, int) const {
+        return false;
+    }
     __device__ __forceinline__ void quad(const v4i_t &raw, int, unsigned, int, float (&f)[4]) const {
 #pragma unroll
         for (int e = 0; e < 4; ++e) f[e] = __int_as_float(raw[e]);
