@@ -102,51 +102,74 @@ struct f8_conv_t {
     }
 
     // The chain of the fp8 up-projection configuration and its subsets, fully
-    // unrolled over the wavefront's 4 x C accumulator tiles with every choice a
+    // unrolled over the wavefront's 4 x 2 accumulator tiles with every choice a
     // template parameter:
     //   acc * src_scale * wei_scale[n]  [+ bias[n]]  [-> gelu_tanh]  [+ bf16 residual]  -> bf16
-    // The residual quads (8 bytes per lane) are loaded four tiles ahead of their use.
+    //
+    // Global memory sees whole 128-byte rows only.  In the accumulator layout a
+    // lane owns 8 bytes of a dst row and a wavefront-wide access touches 32 rows,
+    // 16 bytes each: the memory pipeline takes a cycle per row touched, and 512
+    // such loads plus 512 such stores per tile cost ~10 us each.  Instead the
+    // wavefront's 128 x 64 part of the residual (16 KB) comes into its own share
+    // of the (now idle) tile ring by 16 direct-to-LDS DMAs of 8 whole rows, all in
+    // flight at once; every quad is read from there, and the bf16 result is
+    // written back over it (same lane, same address); at the end the part leaves
+    // LDS as 16 stores of 8 whole rows.  LDS rows are 128 bytes with the eight
+    // 16-byte chunks XOR-swizzled by the row number (on the global-address side of
+    // the DMA and of the final stores), which keeps both access patterns free of
+    // bank conflicts.
     template <bool BIAS, bool GELU, bool ADD, class PT, int C>
-    __device__ __forceinline__ void hot_store(const PT &P, const epi_uniform_t &H, unsigned ntab,
+    __device__ __forceinline__ void hot_store(const PT &P, const epi_uniform_t &H, unsigned ntab, unsigned lds_part,
             const v16f (&acc)[4][C], long b, long m_base, long n_base, int col0) const {
-        constexpr int NU = 4 * C, PF = 4; // units (tiles) of the wavefront; prefetch distance
-        const int lane = threadIdx.x & 63, lrow = lane & 31, ch = 4 * (lane >> 5);
-        uint16_t *dcol = (uint16_t *)P.dst + b * P.ds[0] + n_base + ch;
-        const uint16_t *rcol = ADD ? (const uint16_t *)H.staged_p + b * H.st_s0 + n_base + ch : nullptr;
-        auto row_of = [&](int u) { return m_base + 32 * (u / C) + lrow; };
-        auto load_res = [&](int u, uint2 (&r)[4]) __attribute__((always_inline)) {
-            long m = row_of(u);
-            m = m < P.M ? m : P.M - 1;
-            const uint16_t *p = rcol + m * H.st_s1 + 32 * (u % C);
-#pragma unroll
-            for (int g = 0; g < 4; ++g) r[g] = *(const uint2 *)(p + 8 * g);
-        };
-        uint2 res[PF + 1][4];
+        static_assert(C == 2, "a wavefront's part is 128 rows of 128 bytes");
+        typedef unsigned v2u_t __attribute__((ext_vector_type(2)));
+        typedef unsigned v4u_t __attribute__((ext_vector_type(4)));
+        typedef v2u_t __attribute__((address_space(3), may_alias)) *lds_u2_ptr_t;
+        typedef v4u_t __attribute__((address_space(3), may_alias)) *lds_u4_ptr_t;
+        const int lane = threadIdx.x & 63, lrow = lane & 31, half = lane >> 5;
+        const long rows_left = P.M - m_base; // > 0, checked by the caller
+        // whole-row accesses: lane -> (row d * 8 + lane / 8, chunk slot lane % 8); the slot holds
+        // the row's chunk slot ^ (row & 7)
+        const int wr = lane >> 3, wslot = lane & 7;
         if (ADD) {
+            const char *rbase = scalar_ptr(H.staged_p + (b * H.st_s0 + m_base * H.st_s1 + n_base) * 2);
 #pragma unroll
-            for (int u = 0; u < PF; ++u) load_res(u, res[u]);
+            for (int d = 0; d < 16; ++d) {
+                long r = d * 8 + wr;
+                const int chunk = wslot ^ (int)(r & 7);
+                r = r < rows_left ? r : rows_left - 1;
+                dma16(rbase, (unsigned)(r * H.st_s1 * 2 + chunk * 16), lds_part + d * 1024);
+            }
         }
 #pragma unroll
-        for (int u = 0; u < NU; ++u) {
-            const int i = u / C, j = u % C;
-            if (ADD && u + PF < NU) load_res(u + PF, res[(u + PF) % (PF + 1)]);
-            const long m = row_of(u);
+        for (int u = 0; u < 8; ++u) {
+            const int i = u / 2, j = u % 2;
+            if (ADD && j == 0) { // the four DMAs of this row block have landed
+                if (i == 0) wait_vmcnt<12>();
+                else if (i == 1) wait_vmcnt<8>();
+                else if (i == 2) wait_vmcnt<4>();
+                else wait_vmcnt<0>();
+                asm volatile("" ::: "memory"); // no LDS read moves above the wait
+            }
+            const int r = 32 * i + lrow;
             float x[4][4];
             bool special = false;
+            unsigned cell[4];
 #pragma unroll
             for (int g = 0; g < 4; ++g) {
+                cell[g] = lds_part + (unsigned)(r * 128 + (((4 * j + g) ^ (r & 7)) << 4) + 8 * half);
                 // keeps the table reads of every tile apart: merged, the 32 columns'
                 // operands of all tiles would stay in registers
-                int col = col0 + 32 * j + 8 * g + ch;
+                int col = col0 + 32 * j + 8 * g + 4 * half;
                 asm volatile("" : "+v"(col));
                 v4f_t w = {1.f, 1.f, 1.f, 1.f}, bb = {0.f, 0.f, 0.f, 0.f};
                 if (with_wei_sc) w = nt4f(ntab, NT_WSC, col);
                 if (BIAS) bb = nt4f(ntab, NT_BIAS, col);
                 float y[4] = {0.f, 0.f, 0.f, 0.f};
                 if (ADD) {
-                    const uint2 r = res[u % (PF + 1)][g];
-                    y[0] = u2f(r.x << 16); y[1] = u2f(r.x & 0xffff0000u);
-                    y[2] = u2f(r.y << 16); y[3] = u2f(r.y & 0xffff0000u);
+                    const v2u_t q = *(lds_u2_ptr_t)(size_t)cell[g];
+                    y[0] = u2f(q.x << 16); y[1] = u2f(q.x & 0xffff0000u);
+                    y[2] = u2f(q.y << 16); y[3] = u2f(q.y & 0xffff0000u);
                 }
 #pragma unroll
                 for (int e = 0; e < 4; ++e) {
@@ -162,7 +185,7 @@ struct f8_conv_t {
             }
             typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
             typedef float f32x2_t __attribute__((ext_vector_type(2)));
-            uint2 o[4];
+            v2u_t o[4];
             if (__builtin_amdgcn_ballot_w64(special) == 0) {
 #pragma unroll
                 for (int g = 0; g < 4; ++g) {
@@ -176,16 +199,26 @@ struct f8_conv_t {
                     o[g].y = f32_to_bf16(x[g][2]) | ((unsigned)f32_to_bf16(x[g][3]) << 16);
                 }
             }
-            if (m < P.M) {
-                uint16_t *d = dcol + m * P.ds[1] + 32 * j;
 #pragma unroll
-                for (int g = 0; g < 4; ++g) *(uint2 *)(d + 8 * g) = o[g];
-            }
+            for (int g = 0; g < 4; ++g) *(lds_u2_ptr_t)(size_t)cell[g] = o[g];
+        }
+        // the finished part, 8 whole rows per store
+        char *dbase = (char *)P.dst + (b * P.ds[0] + m_base * P.ds[1] + n_base) * 2;
+#pragma unroll
+        for (int d = 0; d < 16; ++d) {
+            const long r = d * 8 + wr;
+            const int chunk = wslot ^ (int)(r & 7);
+            const v4u_t q = *(lds_u4_ptr_t)(size_t)(lds_part + (unsigned)(d * 1024 + lane * 16));
+            if (r < rows_left) *(v4u_t *)(dbase + r * P.ds[1] * 2 + chunk * 16) = q;
         }
     }
     template <class PT, int C>
-    __device__ __forceinline__ bool hot_chain(const PT &P, const epi_uniform_t &H, unsigned ntab,
+    __device__ __forceinline__ bool hot_chain(const PT &P, const epi_uniform_t &H, unsigned ntab, unsigned lds_part,
             const v16f (&acc)[4][C], long b, long m_base, long n_base, int col0) const {
+        if (m_base >= P.M) return true; // nothing of this wavefront's part is inside dst
+        // 16-byte row pieces of dst and of the residual
+        if (((uintptr_t)P.dst & 15) || (P.ds[0] % 8) || (P.ds[1] % 8)) return false;
+        if (H.staged != STG_NONE && (((uintptr_t)H.staged_p & 15) || (H.st_s0 % 8) || (H.st_s1 % 8))) return false;
         if (!HOT || ssc_p || H.bias_mode == 2 || H.ds_mode != 0 || H.dzp_mode != 0 || H.dynamic || H.dst_dt != MI355_DT_BF16
                 || H.n_po > 2)
             return false;
@@ -206,7 +239,7 @@ struct f8_conv_t {
             if (!gelu || !add) return false;
         }
         const bool bias = H.bias_mode == 1;
-#define MI355_F8_HOT(B, G, A) hot_store<B, G, A>(P, H, ntab, acc, b, m_base, n_base, col0)
+#define MI355_F8_HOT(B, G, A) hot_store<B, G, A>(P, H, ntab, lds_part, acc, b, m_base, n_base, col0)
         if (bias) {
             if (gelu) { if (add) MI355_F8_HOT(true, true, true); else MI355_F8_HOT(true, true, false); }
             else { if (add) MI355_F8_HOT(true, false, true); else MI355_F8_HOT(true, false, false); }

@@ -156,7 +156,7 @@ struct i8_conv_t {
         }
     }
     template <class PT>
-    __device__ __forceinline__ bool hot_chain(const PT &P, const epi_uniform_t &H, unsigned ntab,
+    __device__ __forceinline__ bool hot_chain(const PT &P, const epi_uniform_t &H, unsigned ntab, unsigned,
             const v4i (&acc)[8][4], long b, long m_base, long n_base, int col0) const {
         const bool relu0 = H.n_po == 1 && H.pf0.kind == MI355_PO_ELTWISE && H.pf0.alg == MI355_ELTWISE_RELU
                 && H.pf0.alpha == 0.f && H.pf0.scale == 1.f;

@@ -127,8 +127,8 @@ struct mxf4_conv_t {
     __device__ __forceinline__ void per_n(const PT &, long, long, float &, int &, int &) const {}
     __device__ __forceinline__ int row_data(long) const { return 0; }
     template <class PT, class Acc>
-    __device__ __forceinline__ bool hot_chain(const PT &, const epi_uniform_t &, unsigned, const Acc &, long, long,
-            long, int) const {
+    __device__ __forceinline__ bool hot_chain(const PT &, const epi_uniform_t &, unsigned, unsigned, const Acc &, long,
+            long, long, int) const {
         return false;
     }
     __device__ __forceinline__ void quad(const v4i_t &raw, int, unsigned, int, float (&f)[4]) const {

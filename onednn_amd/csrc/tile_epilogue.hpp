@@ -848,14 +848,15 @@ __device__ __forceinline__ void dynamic_quantQ(const PT &P, int dst_dt, float (&
 }
 
 // The epilogue of one wavefront's 128 x WCOLS part.
-//   park      lane-private LDS of the general path: Q x 64 x 16 bytes per wavefront
+//   park      the idle tile ring: every wavefront owns 16 KB of it (the general path parks
+//             Q x 64 x 16 bytes there, the specialised chains stage their part of dst)
 //   ntab      LDS byte address of the per-column table (filled before the K loop)
 //   m_base    first row of the wavefront's part, n_base its first column, col0 =
 //             that column's index inside the tile (the table's index)
 //   conv      the kernel's conversion of raw accumulators:
 //                 row_t row_data(m)                         per-row operand
 //                 quad(raw, row_t, ntab, col, float (&f)[4])
-//                 bool hot_chain(P, H, ntab, acc, b, m_base, n_base, col0)
+//                 bool hot_chain(P, H, ntab, lds_part, acc, b, m_base, n_base, col0)
 //                     the whole epilogue of the wavefront for the chains the kernel
 //                     specialises at compile time (false: not one of them)
 template <class Layout, int WCOLS, class PT, class T, int R, int C, class Conv>
@@ -871,7 +872,12 @@ __device__ __forceinline__ void store_quadrant(const PT &P, char *park, unsigned
     typedef typename Conv::row_t row_t;
 
     // the benchmark configurations' chains, specialised at compile time by the kernel
-    if (H.fast && conv.hot_chain(P, H, ntab, acc, b, m_base, n_base, col0)) return;
+    {
+        // the wavefront's share of the idle tile ring: 16 KB
+        const unsigned lds_part = (unsigned)(size_t)(__attribute__((address_space(3))) char *)park
+                + (unsigned)__builtin_amdgcn_readfirstlane(wave) * 16384u;
+        if (H.fast && conv.hot_chain(P, H, ntab, lds_part, acc, b, m_base, n_base, col0)) return;
+    }
 
     if (H.fast) {
         int col[Q];
@@ -950,7 +956,8 @@ __device__ __forceinline__ void store_quadrant(const PT &P, char *park, unsigned
 
     // ---- general path: the quads of a row block parked in lane-private LDS, then
     // one group of 32 columns at a time through the interpreter
-    park_u4_t *pk = (park_u4_t *)park + wave * (Q * 64);
+    static_assert(Q * 64 * 16 <= 16384, "a wavefront's share of the ring");
+    park_u4_t *pk = (park_u4_t *)(park + wave * 16384); // the same 16 KB share the specialised chains use
 #pragma unroll 1
     for (int i = 0; i < NB; ++i) {
         {
