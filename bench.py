@@ -36,17 +36,36 @@ sys.path.insert(0, ROOT)
 
 import numpy as np  # noqa: E402
 
-# HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, each
-# scaled by what the same counter reads for the plain copy kernel moving a
-# known 256 MiB (factors 2.0 and 1.0); the summaries with the commands are in
-# profiles/<kernel>_<workload>.md.  Keyed by (workload, M).
-MEASURED_TRAFFIC = {
-    ("c3", 8192): 1078997046, ("c4", 4096): 2178641942, ("c5", 8192): 569460235,
-    ("c2", 1): 31612633, ("c2", 8): 32271601, ("c2", 32): 34542741,        # packed weights (format any)
-    ("c2ab", 1): 32839597, ("c2ab", 8): 35736697, ("c2ab", 32): 51670775,  # plain ab weights (--wtag ab)
-    ("c1", 256): 8657878,
-    ("r1", 0): 335981182, ("r2", 0): 212392274, ("r3", 0): 58765379,
+# HBM bytes per launch come from the rocprofv3 summaries under profiles/ (two
+# --pmc passes, FETCH_SIZE and WRITE_SIZE, each scaled by what the same counter
+# reads for the plain copy kernel moving a known 256 MiB): every summary carries
+# the line "HBM bytes per launch ...: N", which is read here, so that the figure
+# in the JSON line can only be as old as the committed profile it names.
+PROFILE_OF = {
+    ("c3", "any"): "i8_gemm_kernel_c3_8192.md", ("c4", "any"): "f8_gemm_kernel_c4_4096x8192x28672.md",
+    ("c5", "any"): "mxf4_gemm_kernel_c5_8192.md", ("c1", "any"): "i8_gemm_kernel_c1_256x1024x1024.md",
+    ("c2", "any", 1): "woqp_kernel_c2_m1.md", ("c2", "any", 8): "woqp_kernel_c2_m8.md",
+    ("c2", "any", 32): "woqp_kernel_c2_m32.md", ("c2", "ab", 1): "woq_gemv_kernel_c2_m1_plain_ab.md",
+    ("c2", "ab", 8): "woq_gemv_kernel_c2_m8_plain_ab.md", ("c2", "ab", 32): "woq_gemv_kernel_c2_m32_plain_ab.md",
+    ("r1", "any"): "reorder_direct_kernel_r1_f32_s8_8192.md", ("r2", "any"): "transpose8_kernel_r2_s8_transpose_8192.md",
+    ("r3", "any"): "pack_woq64_kernel_r3_u4_4096x14336.md",
 }
+
+
+def measured_traffic(name, wtag="any", M=None):
+    """(bytes per launch, profile file) from the committed summary, or (None, None)."""
+    import re
+    key = (name, wtag, M) if name == "c2" else (name, "any")
+    fn = PROFILE_OF.get(key)
+    if not fn:
+        return None, None
+    path = os.path.join(ROOT, "profiles", fn)
+    try:
+        m = re.search(r"HBM bytes per launch[^:\n]*:\s*([0-9,]+)", open(path).read())
+    except OSError:
+        return None, None
+    return (int(m.group(1).replace(",", "")), "profiles/" + fn) if m else (None, "profiles/" + fn)
+
 
 # MI355X published peaks
 PEAK_HBM_GBS = 8000.0
@@ -136,8 +155,17 @@ def rate(work, ms, unit):
     return work / (ms * 1e-3) / 1e12
 
 
-def run_gpu_workload(lib, name, steps, warmup, M=None, cold_copies=0, wtag="any"):
-    """Returns dict with ms_per_step, value, unit, impl."""
+def run_gpu_workload(lib, name, steps, warmup, M=None, cold_copies=0, wtag="any", sustained_s=0.0):
+    """Returns dict with ms_per_step, value, unit, impl.
+
+    Before the warm-up steps the workload is launched back to back for about
+    0.4 s, untimed: after an idle period the device needs a few hundred
+    milliseconds of load before its clocks settle, and a timed region of a few
+    milliseconds taken right after start-up measures that ramp rather than the
+    kernel (the same launches measured 0.56 ms each in the first 10, 0.51 over
+    30 and 0.46 over 300).  With sustained_s > 0 the workload is afterwards
+    launched back to back for at least that many seconds, timed in chunks:
+    `sustained` = average and best chunk."""
     from onednn_amd import cabi
     from onednn_amd.problem import GpuRun
     t0 = time.time()
@@ -155,14 +183,29 @@ def run_gpu_workload(lib, name, steps, warmup, M=None, cold_copies=0, wtag="any"
         runs[idx[0] % len(runs)].launch()
         idx[0] += 1
 
+    t_pre = time.time()
+    while time.time() - t_pre < 0.4:     # settle the clocks (untimed)
+        for _ in range(20):
+            step()
+        cabi.check(lib.mi355_stream_sync(None))
     for _ in range(max(warmup, 1)):
         step()
     ms = timer.time_ms(step, steps)
     work, unit, bound, peak = algorithmic(name, p)
+    sustained = None
+    if sustained_s > 0:
+        chunk = max(20, int(0.1 / max(ms * 1e-3, 1e-6)))      # ~0.1 s of launches per chunk
+        chunks, t_s = [], time.time()
+        while time.time() - t_s < sustained_s or len(chunks) < 3:
+            chunks.append(timer.time_ms(step, chunk))
+        sustained = {"seconds": round(time.time() - t_s, 2), "launches": chunk * len(chunks),
+                     "ms_per_step_avg": sum(chunks) / len(chunks), "ms_per_step_min": min(chunks),
+                     "value_avg": rate(work, sum(chunks) / len(chunks), unit), "value_best": rate(work, min(chunks), unit),
+                     "unit": unit}
     out = {
         "workload": p.name, "impl": cabi.impl_name(runs[0].impl), "ms_per_step": ms,
         "value": rate(work, ms, unit), "unit": unit, "bound": bound, "peak": peak, "work": work,
-        "shape": [p.M, p.K, p.N],
+        "shape": [p.M, p.K, p.N], "sustained": sustained,
     }
     for r in runs:
         r.free()
@@ -249,7 +292,16 @@ def cpu_baseline(name, M=None):
         if dt >= 10.0 or reps >= 200:
             break
     work, unit, _, _ = algorithmic(name, p)
+    # the reference's own optimized CPU path (brg_matmul, JIT) cannot be built on this machine; what it measured
+    # where it could be built is quoted so that the port's number is not read as the reference's speed
+    probe = {"c3": "4.97 TOPS (221 ms)", "c1": "6.37 TOPS (0.084 ms)",
+             "c2": {1: "4.17 GB/s (7.05 ms)", 8: "4.64 GB/s (6.39 ms)", 32: "3.16 GB/s (9.67 ms)"}.get(M or 1),
+             "c4": "no JIT implementation on that host (ref:any only)", "c5": "no CPU implementation (skipped)"}[name]
     return {"value": rate(work * reps, dt * 1e3, unit), "unit": unit, "cores": threads, "kind": "port",
+            "reference_probe": {"what": "benchdnn --matmul --mode=P on the reference built with its own CMake, "
+                                        "impl brg_matmul:avx10_1_512_amx, this configuration at full size",
+                                "value": probe, "hardware": "8 vCPU Intel Xeon (Sapphire Rapids class, AMX), "
+                                                            "OMP_NUM_THREADS=8; another machine, not this run"},
             "sample": sample + f"; {reps} pass(es), {dt:.2f} s wall; oracle/liboracle.so (plain C restatement of "
             "ref_matmul_t / ref_matmul_int8_t, OpenMP over dst rows; the reference itself needs CMake-generated "
             "headers and is not built here)"}
@@ -266,6 +318,9 @@ def main():
     ap.add_argument("--decode-m", type=int, default=1, help="M of the c2 decode workload")
     ap.add_argument("--wtag", default="any", choices=["any", "ab", "ba"],
                     help="weights layout; any = what format_tag::any resolves to (default)")
+    ap.add_argument("--sustained", type=float, default=1.5,
+                    help="seconds of back-to-back launches of the headline workload after the timed steps "
+                         "(reported as `sustained`; 0 = skip)")
     ap.add_argument("--no-others", action="store_true", help="skip the informational configs")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--calib-copy", action="store_true",
@@ -311,14 +366,14 @@ def main():
             "vs_baseline": None, "dtype": {"r1": "f32", "r2": "s8", "r3": "u4"}[main_name], "data": "synthetic",
             "config": {"workload": r["workload"], "impl": r["impl"]},
             "roofline": {"bound": "hbm", "achieved": r["value"], "peak": PEAK_HBM_GBS, "unit": "GB/s",
-                         "frac": r["frac_of_peak"], "traffic": MEASURED_TRAFFIC.get((main_name, 0)),
-                         "algorithmic": r["work"],
+                         "frac": r["frac_of_peak"], "traffic": measured_traffic(main_name)[0],
+                         "traffic_source": measured_traffic(main_name)[1], "algorithmic": r["work"],
                          "kernel": r["impl"], "kernel_ms": r["ms_per_step"]},
             "cpu_baseline": None, "others": []}), flush=True)
         return
     cold = 11 if main_name == "c2" else 0
     res, prob = run_gpu_workload(lib, main_name, args.steps, args.warmup, args.decode_m, cold,
-                                 args.wtag)
+                                 args.wtag, sustained_s=args.sustained)
     log(f"[bench] {res['workload']}: {res['ms_per_step']:.4f} ms/step -> {res['value']:.1f} "
         f"{res['unit']} via {res['impl']}")
 
@@ -330,25 +385,29 @@ def main():
     # split-K reduction of the decode path, column sums, the layout change of
     # `ab` weights when --wtag ab is forced) are part of the measured step and
     # therefore of `achieved`: it never flatters the dominant kernel.
+    traffic, traffic_source = measured_traffic(main_name, "any" if args.wtag == "any" else "ab", prob.M)
     roofline = {
         "bound": res["bound"], "achieved": res["value"], "peak": res["peak"],
         "unit": "GB/s" if res["unit"] == "GB/s" else "TFLOP/s",
-        "frac": res["value"] / res["peak"], "traffic": MEASURED_TRAFFIC.get(
-            ("c2ab" if main_name == "c2" and args.wtag != "any" else main_name, prob.M)),
+        "frac": res["value"] / res["peak"], "traffic": traffic, "traffic_source": traffic_source,
         "algorithmic": res["work"], "kernel": res["impl"], "kernel_ms": res["ms_per_step"],
     }
 
     others = []
     if not args.no_others:
-        plan = [("c2", 1), ("c2", 8), ("c2", 32), ("c3", None), ("c4", None), ("c4mx", None), ("c5", None),
-                ("c1", None)]
-        for nm, m in plan:
-            if nm == main_name and (nm != "c2" or m == args.decode_m):
+        # (workload, M, weights tag); "ab" = row-major weights as in the reference's benchdnn line for C3: the
+        # layout change then runs inside every launch
+        plan = [("c2", 1, "any"), ("c2", 8, "any"), ("c2", 32, "any"), ("c3", None, "any"), ("c3", None, "ab"),
+                ("c4", None, "any"), ("c4mx", None, "any"), ("c5", None, "any"), ("c1", None, "any")]
+        for nm, m, wt in plan:
+            if nm == main_name and wt == args.wtag and (nm != "c2" or m == args.decode_m):
                 continue
             try:
                 r, _ = run_gpu_workload(lib, nm, max(5, args.steps // 2), 2, m,
-                                        11 if nm == "c2" else 0)
+                                        11 if nm == "c2" else 0, wt)
                 r["frac_of_peak"] = r["value"] / r["peak"]
+                if wt != "any":
+                    r["workload"] += f" (weights tag {wt})"
                 others.append({k: r[k] for k in ("workload", "impl", "ms_per_step", "value", "unit",
                                                  "bound", "peak", "frac_of_peak")})
                 log(f"[bench] {r['workload']}: {r['ms_per_step']:.4f} ms -> {r['value']:.1f} "
@@ -379,7 +438,7 @@ def main():
         "data": "synthetic",
         "config": {"workload": res["workload"], "shape_MKN": res["shape"], "impl": res["impl"],
                    "weights_layout": args.wtag},
-        "roofline": roofline, "cpu_baseline": cpu, "others": others,
+        "roofline": roofline, "sustained": res["sustained"], "cpu_baseline": cpu, "others": others,
     }
     print(json.dumps(line), flush=True)
 
