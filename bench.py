@@ -323,6 +323,9 @@ def main():
                          "(reported as `sustained`; 0 = skip)")
     ap.add_argument("--no-others", action="store_true", help="skip the informational configs")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--calib-read", action="store_true",
+                    help="time a read-only kernel with the decode kernel's access shape over the C2 weights "
+                         "(12 rotating copies, nothing cached) and exit: the floor of the weight stream")
     ap.add_argument("--calib-copy", action="store_true",
                     help="also launch the plain copy kernel on 256 MiB three times: the known-size "
                          "dispatch that FETCH_SIZE / WRITE_SIZE counter passes are scaled by")
@@ -347,6 +350,31 @@ def main():
         f"HBM={hbm.value / 2**30:.0f} GiB")
 
     main_name = args.workload
+    if args.calib_read:
+        nbytes = 4096 * 14336 // 2
+        bufs = [cabi.DeviceBuffer(nbytes) for _ in range(12)]
+        sink = cabi.DeviceBuffer(4096)
+        timer, idx = Timer(lib), [0]
+
+        def step():
+            cabi.check(lib.mi355_read_stream_kernel(bufs[idx[0] % 12].ptr, C.c_size_t(nbytes), sink.ptr, None))
+            idx[0] += 1
+
+        t_pre = time.time()
+        while time.time() - t_pre < 0.4:
+            for _ in range(50):
+                step()
+            cabi.check(lib.mi355_stream_sync(None))
+        runs = [timer.time_ms(step, max(args.steps, 200)) for _ in range(5)]
+        ms = sum(runs) / len(runs)
+        log(f"[bench] read_stream_kernel over {nbytes} bytes (C2 weights), 12 rotating copies: "
+            f"{ms * 1e3:.2f} us/launch avg of 5 x {max(args.steps, 200)}, best {min(runs) * 1e3:.2f} us -> "
+            f"{nbytes / (ms * 1e-3) / 1e9:.0f} GB/s")
+        print(json.dumps({"metric": "read floor of the C2 weight stream", "value": nbytes / (ms * 1e-3) / 1e9,
+                          "unit": "GB/s", "us_per_launch": ms * 1e3, "us_best": min(runs) * 1e3, "bytes": nbytes}),
+              flush=True)
+        return
+
     def calib_copy():
         nbytes = 256 << 20
         a, b = cabi.DeviceBuffer(nbytes), cabi.DeviceBuffer(nbytes)

@@ -378,6 +378,12 @@ int mi355_wei_pack_reorder_dims(int packing, int64_t K, int64_t N,
  * to calibrate the FETCH_SIZE / WRITE_SIZE counters against a known size. */
 int mi355_copy_kernel(void *dst, const void *src, size_t bytes, void *stream);
 
+/* Read-only kernel with the access shape of the weight-only decode kernel
+ * (128 KiB per workgroup, 16 wavefronts of eight 1 KiB non-temporal runs):
+ * times what streaming `bytes` (a multiple of 128 KiB) of weights costs by
+ * itself.  `sink` holds 4 bytes per 128 KiB and is not written in practice. */
+int mi355_read_stream_kernel(const void *src, size_t bytes, void *sink, void *stream);
+
 /* Evict caches between timed launches: streams `bytes` of `buf` through a
  * read-modify-write kernel so a following launch sees cold L2/MALL. */
 int mi355_flush_kernel(void *buf, size_t bytes, void *stream);

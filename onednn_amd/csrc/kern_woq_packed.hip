@@ -23,9 +23,25 @@
 // zero-interleaved A operand (half the matrix-core work of the plain layout).
 // The A operand is 16 bytes of a src row, the same k order by construction.
 //
-// The eight wavefronts of a workgroup split K, keep their sums in registers
-// across quantization groups and add them through LDS at the end, in wavefront
-// order: results do not depend on timing.
+// The wavefronts of a workgroup (16 for M <= 16, 8 above) split K, keep their
+// sums in registers across quantization groups and add them through LDS at the
+// end, in wavefront order: results do not depend on timing.
+//
+// The launch lasts a few microseconds, so what a wavefront does before its
+// loads are in flight and after its last data arrive is as visible as the
+// stream itself:
+//  - the loop's operands are the first 112 bytes of the kernel arguments and
+//    are fetched with one burst of scalar loads; the problem description is
+//    read only by the general epilogue;
+//  - a problem with nothing after the K sum but the conversion to f32 / bf16 /
+//    f16 (no bias, post-ops, dst scale or zero point) runs a kernel whose end
+//    is a sum over the wavefronts and one store: no further argument fetch, no
+//    instruction-cache misses on an epilogue interpreter;
+//  - a wavefront's loads return as one burst, late ones last, and its whole
+//    unpack + MFMA work then follows that burst: more wavefronts with fewer
+//    steps each keep this tail short;
+//  - the parameter decode at a group's end is straight-line code (candidate
+//    conversions selected by uniform masks), no data-type switch.
 #include "kernels.hpp"
 #include "tile_epilogue.hpp"
 
@@ -37,9 +53,9 @@ namespace {
 typedef int v4i __attribute__((ext_vector_type(4)));
 typedef unsigned v4u __attribute__((ext_vector_type(4)));
 typedef float v4f __attribute__((ext_vector_type(4)));
+typedef unsigned v16u __attribute__((ext_vector_type(16)));
 typedef __bf16 v8bf __attribute__((ext_vector_type(8)));
 
-constexpr int NWV = 8;         // wavefronts per workgroup
 constexpr int CHUNK = 64;      // columns per workgroup
 constexpr int KBLK = 32;       // rows per step (one MFMA depth)
 constexpr int NO_GROUPS = 1 << 30;
@@ -48,6 +64,8 @@ struct woqp_extra_t {
     const uint8_t *wei;  // packed, K * N / 2 bytes
     const uint8_t *src;  // bf16 [M][src_ld]
     const uint8_t *sc, *zp; // weights scales / zero points (NULL when absent)
+    uint8_t *dst;        // the plain store: dst_dt in {f32, bf16, f16}, rows dst_ld elements apart
+    int dst_dt, dst_ld;
     int M, N, K, src_ld;
     int kbw;             // 32-row blocks per wavefront
     int spg;             // 32-row blocks per quantization group, NO_GROUPS without groups
@@ -56,52 +74,87 @@ struct woqp_extra_t {
     int sc_grouped, zp_grouped; // parameter has a K dimension
     int zp_common;       // single zero point
     int signed_w;        // s4 weights
+    int pad[6];
 };
+static_assert(sizeof(woqp_extra_t) == 128, "fetched as two 64-byte scalar loads");
+
+// the one kernel argument: the loop's operands first
+struct woqp_args_t {
+    woqp_extra_t X;
+    problem_t P;
+};
+typedef const __attribute__((address_space(4))) woqp_args_t kernarg_woqp_t;
 
 __device__ __forceinline__ v8bf as_bf(const v4i &x) { return __builtin_bit_cast(v8bf, x); }
 
 // Quantization parameters are fetched as the aligned dword that holds the
 // element (no branch on the data type next to the load, so a fetch never waits
-// for its own data); the element is cut out when the group is flushed.
-__device__ __forceinline__ unsigned param_word(const uint8_t *p, int bits, long idx) {
-    // (pointer arithmetic on p, not an address rebuilt from an integer: the
-    // load stays a global one)
-    const long off = (idx * bits) >> 3;
-    return *(const unsigned *)(p + (off - (long)(((uintptr_t)p + (size_t)off) & 3)));
+// for its own data); the element is cut out when the group is flushed.  A row
+// of parameters (one group, N elements) is a multiple of four bytes, so a
+// lane's offset inside the row, the shift and the mask are the same for every
+// group and a fetch costs one scalar multiply-add and the load.
+struct param_lane_t {
+    const uint8_t *base; // aligned down to four bytes
+    long pitch;          // bytes between groups, 0 without groups
+    unsigned voff, sh, mask;
+};
+
+__device__ __forceinline__ param_lane_t param_setup(const uint8_t *p, int bits, long n, bool grouped, long N) {
+    param_lane_t L;
+    const unsigned mis = (unsigned)((uintptr_t)p & 3);
+    const long bitoff = n * bits;
+    const unsigned byte = (unsigned)(bitoff >> 3) + mis;
+    L.base = p - mis;
+    L.pitch = grouped ? N * bits / 8 : 0;
+    L.voff = byte & ~3u;
+    L.sh = (byte & 3) * 8u + ((unsigned)bitoff & 4u);
+    L.mask = 0xffffffffu >> ((32 - bits) & 31);
+    return L;
 }
 
-__device__ __forceinline__ unsigned param_cut(const uint8_t *p, int bits, long idx, unsigned word) {
-    const uintptr_t addr = (uintptr_t)p + (size_t)((idx * bits) >> 3);
-    const unsigned sh = (unsigned)(addr & 3) * 8u + (unsigned)((idx * bits) & 4);
-    return (word >> sh) & (0xffffffffu >> ((32 - bits) & 31));
+__device__ __forceinline__ unsigned param_word(const param_lane_t &L, int g) {
+    return *(const unsigned *)(L.base + g * L.pitch + L.voff);
 }
 
+__device__ __forceinline__ unsigned param_cut(const param_lane_t &L, unsigned word) { return (word >> L.sh) & L.mask; }
+
+// Straight-line decodes: every candidate is a couple of instructions and the
+// data type is uniform, so selects cost less than branches.
 __device__ __forceinline__ float decode_scale(int dt, unsigned raw) {
-    switch (dt) {
-        case MI355_DT_F32: return u2f(raw);
-        case MI355_DT_BF16: return u2f(raw << 16);
-        case MI355_DT_F16: return f16_to_f32((uint16_t)raw);
-        default: return 1.f;
-    }
+    const float h = (float)__builtin_bit_cast(_Float16, (unsigned short)raw);
+    float r = u2f(raw << (dt == MI355_DT_BF16 ? 16 : 0));
+    r = dt == MI355_DT_F16 ? h : r;
+    return dt == MI355_DT_UNDEF ? 1.f : r;
 }
 
-__device__ __forceinline__ float decode_zp(int dt, unsigned raw) {
-    switch (dt) {
-        case MI355_DT_S32: return (float)(int)raw;
-        case MI355_DT_U8: return (float)raw;
-        case MI355_DT_S8: return (float)(int)(int8_t)raw;
-        case MI355_DT_U4: return (float)raw;
-        case MI355_DT_S4: return (float)((int)(raw ^ 8u) - 8);
-        default: return 0.f;
-    }
+// raw holds `bits` bits, zero-extended
+__device__ __forceinline__ float decode_zp(int dt, int bits, unsigned raw) {
+    const int sh = (32 - bits) & 31;
+    const unsigned x = raw << sh;
+    const bool sgn = dt == MI355_DT_S32 || dt == MI355_DT_S8 || dt == MI355_DT_S4;
+    const int v = sgn ? (int)x >> sh : (int)(x >> sh);
+    return dt == MI355_DT_UNDEF ? 0.f : (float)v;
 }
 
 // MT 16-row tiles of activations; SS steps per super-step (all of its loads
 // are issued before its first MFMA); SPG steps per quantization group when a
 // super-step holds whole groups, 0 when a group holds whole super-steps.
-template <int MT, int SS, int SPG>
-__global__ void __launch_bounds__(NWV * 64) woqp_kernel(const problem_t P_, const woqp_extra_t X) {
+// NWV wavefronts per workgroup.  PLAIN: nothing follows the K sum but the
+// conversion to the dst type.
+template <int NWV, int MT, int SS, int SPG, bool PLAIN>
+__global__ void __launch_bounds__(NWV * 64)
+        woqp_kernel(const std::conditional_t<PLAIN, woqp_extra_t, woqp_args_t> A_) {
     __shared__ v4f red4[NWV * MT * 4 * 64];
+    // the loop's operands in one burst of scalar loads (left to itself the
+    // compiler fetches each field where it is first used, a round trip through
+    // the scalar cache each)
+    struct raw_args_t {
+        v16u lo, hi;
+    } raw;
+    asm volatile("s_load_dwordx16 %0, %2, 0x0\n\ts_load_dwordx16 %1, %2, 0x40\n\ts_waitcnt lgkmcnt(0)"
+                 : "=&s"(raw.lo), "=&s"(raw.hi)
+                 : "s"(__builtin_amdgcn_kernarg_segment_ptr()));
+    const woqp_extra_t X = __builtin_bit_cast(woqp_extra_t, raw);
     constexpr int NGS = SPG ? SS / SPG : 1; // groups per super-step
     const int t = threadIdx.x, lane = t & 63;
     const int wave = __builtin_amdgcn_readfirstlane(t >> 6);
@@ -121,6 +174,25 @@ __global__ void __launch_bounds__(NWV * 64) woqp_kernel(const problem_t P_, cons
         const int m = mt * 16 + j < M ? mt * 16 + j : M - 1;
         src_lane_off[mt] = (unsigned)(m * X.src_ld * 2 + q * 16);
     }
+    // the super-step's loader: lane = row + 8 * slot over eight rows and two steps
+    static_assert(SS % 2 == 0, "activations are loaded for pairs of steps");
+    const int lr = lane & 7, lc = lane >> 3;
+    unsigned src_row_off[MT][2];
+    int wr_idx[2], rd_idx[2];
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+            const int m = mt * 16 + 8 * h + lr < M ? mt * 16 + 8 * h + lr : M - 1;
+            src_row_off[mt][h] = (unsigned)(m * X.src_ld * 2 + lc * 16);
+        }
+#pragma unroll
+    for (int h = 0; h < 2; ++h) {
+        wr_idx[h] = (8 * h + lr) * 8 + (lc ^ lr);
+        rd_idx[h] = j * 8 + ((4 * h + q) ^ (j & 7));
+    }
+    v4u *stage = (v4u *)red4 + wave * (MT * 128);
+    constexpr bool ALDS = MT == 2;
     // quantization parameters: lane l fetches column l of the chunk, the
     // columns a lane accumulates (16t + j) come from lanes 16t + j at the flush
     const long n_param = (long)chunk * CHUNK + lane;
@@ -132,10 +204,6 @@ __global__ void __launch_bounds__(NWV * 64) woqp_kernel(const problem_t P_, cons
 #pragma unroll
         for (int tt = 0; tt < 4; ++tt) acc[mt][tt] = tot[mt][tt] = v4f {0.f, 0.f, 0.f, 0.f};
     }
-    int rows_used[MT]; // rows of a quad that can hold data in tile mt (uniform: 4 unless M is below 4 there)
-#pragma unroll
-    for (int mt = 0; mt < MT; ++mt) rows_used[mt] = M - 16 * mt;
-
     // 0x4300 | nibble = bf16(128 + nibble).  The constant is kept in a vector
     // register: a VOP3 instruction takes one scalar operand at most, so
     // (x & mask) | magic fuses into v_and_or_b32 only when `magic` is not scalar.
@@ -145,12 +213,14 @@ __global__ void __launch_bounds__(NWV * 64) woqp_kernel(const problem_t P_, cons
     const unsigned flip = X.signed_w ? 0x88888888u : 0u; // s4 -> offset-binary
     const float zbase = X.signed_w ? 136.f : 128.f;
 
-    auto compute_step = [&](const v4u &w, const v4u (&a)[MT]) __attribute__((always_inline)) {
+    // `first`: the step opens a quantization group (sums start from zero)
+    auto compute_step = [&](const v4u &w, const v4u (&a)[MT], bool first) __attribute__((always_inline)) {
         v4i av[MT];
+        const v4f zero = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
         for (int mt = 0; mt < MT; ++mt) {
             av[mt] = v4i {(int)a[mt][0], (int)a[mt][1], (int)a[mt][2], (int)a[mt][3]};
-            rsum[mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf(av[mt]), as_bf(ones), rsum[mt], 0, 0, 0);
+            rsum[mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf(av[mt]), as_bf(ones), first ? zero : rsum[mt], 0, 0, 0);
         }
 #pragma unroll
         for (int tt = 0; tt < 4; ++tt) {
@@ -160,24 +230,23 @@ __global__ void __launch_bounds__(NWV * 64) woqp_kernel(const problem_t P_, cons
             for (int u = 0; u < 4; ++u) b[u] = (int)(((d >> (4 * u)) & 0x000F000Fu) | magic);
 #pragma unroll
             for (int mt = 0; mt < MT; ++mt)
-                acc[mt][tt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf(av[mt]), as_bf(b), acc[mt][tt], 0, 0, 0);
+                acc[mt][tt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf(av[mt]), as_bf(b), first ? zero : acc[mt][tt], 0, 0, 0);
         }
     };
 
-    // element index of this lane's parameters of group g
-    auto sc_index = [&](int g) __attribute__((always_inline)) { return (X.sc_grouped ? (long)g * N : 0) + n_param; };
-    auto zp_index = [&](int g) __attribute__((always_inline)) {
-        return X.zp_common ? 0 : (X.zp_grouped ? (long)g * N : 0) + n_param;
-    };
+    const param_lane_t Lsc = param_setup(X.sc, X.sc_bits, n_param, X.sc_grouped, N);
+    const param_lane_t Lzp = param_setup(X.zp, X.zp_bits, X.zp_common ? 0 : n_param, X.zp_grouped, N);
     auto fetch_params = [&](unsigned &word_s, unsigned &word_z, int g) __attribute__((always_inline)) {
-        word_s = param_word(X.sc, X.sc_bits, sc_index(g));
-        word_z = param_word(X.zp, X.zp_bits, zp_index(g));
+        word_s = param_word(Lsc, g);
+        word_z = param_word(Lzp, g);
     };
 
-    // tot += scale * (acc - (128 + zp) * rowsum) for one finished group
-    auto flush_group = [&](unsigned word_s, unsigned word_z, int g) __attribute__((always_inline)) {
-        const float s = decode_scale(X.sc_dt, param_cut(X.sc, X.sc_bits, sc_index(g), word_s));
-        const float z = decode_zp(X.zp_dt, param_cut(X.zp, X.zp_bits, zp_index(g), word_z)) + zbase;
+    // tot += scale * (acc - (128 + zp) * rowsum) for one finished group (rows
+    // beyond M hold the sums of row M - 1: finite, never stored).  ZERO: the
+    // next step does not start the sums from zero by itself.
+    auto flush_group = [&](unsigned word_s, unsigned word_z, bool zero_sums) __attribute__((always_inline)) {
+        const float s = decode_scale(X.sc_dt, param_cut(Lsc, word_s));
+        const float z = decode_zp(X.zp_dt, X.zp_bits, param_cut(Lzp, word_z)) + zbase;
 #pragma unroll
         for (int tt = 0; tt < 4; ++tt) {
             const float st = __shfl(s, tt * 16 + j, 64);
@@ -186,63 +255,122 @@ __global__ void __launch_bounds__(NWV * 64) woqp_kernel(const problem_t P_, cons
             for (int mt = 0; mt < MT; ++mt) {
 #pragma unroll
                 for (int r = 0; r < 4; ++r)
-                    if (r < rows_used[mt]) tot[mt][tt][r] += st * __builtin_fmaf(-zt, rsum[mt][r], acc[mt][tt][r]);
-                acc[mt][tt] = v4f {0.f, 0.f, 0.f, 0.f};
+                    tot[mt][tt][r] = __builtin_fmaf(st, __builtin_fmaf(-zt, rsum[mt][r], acc[mt][tt][r]), tot[mt][tt][r]);
+                if (zero_sums) acc[mt][tt] = v4f {0.f, 0.f, 0.f, 0.f};
             }
         }
+        if (zero_sums) {
 #pragma unroll
-        for (int mt = 0; mt < MT; ++mt) rsum[mt] = v4f {0.f, 0.f, 0.f, 0.f};
+            for (int mt = 0; mt < MT; ++mt) rsum[mt] = v4f {0.f, 0.f, 0.f, 0.f};
+        }
     };
 
     // One super-step.  Issue order: the groups' parameters (few bytes, needed
     // last -- loads return in order, so they must not queue behind the weights),
     // the activations, the weights; then the MFMAs step by step as their loads
-    // arrive.  FULL = all SS steps present (no guards in the common case).
-    auto super_step = [&](int kb, int ns, auto full) __attribute__((always_inline)) {
-        constexpr bool FULL = decltype(full)::value;
+    // arrive.
+    //
+    // Activations.  The MFMA operand of a step is 16 rows x 64 bytes; loaded
+    // that way every instruction touches 16 half lines, the other halves are
+    // fetched again for the next step, and the launch time grows by 0.35 us per
+    // row of src.  With two tiles (ALDS) a load covers two steps of eight rows
+    // instead, whole 128-byte lines (lane = row + 8 * slot), and a pair of
+    // steps is brought into operand order through 2 KB of LDS per tile and
+    // wavefront when its turn comes: slot c of row r is stored at c ^ (r & 7),
+    // so the eight lanes that write or read together fall into eight different
+    // slots.  The detour costs 0.8 us per launch and halves the growth per row:
+    // it pays above 16 rows.
+    auto super_step = [&](int kb) __attribute__((always_inline)) {
         unsigned raw_s[NGS], raw_z[NGS];
+        // (whole groups inside the super-step: the group size is SPG)
+        const int g0 = SPG ? kb / (SPG ? SPG : 1) : kb / X.spg;
 #pragma unroll
-        for (int gi = 0; gi < NGS; ++gi)
-            if (FULL || gi * (SPG ? SPG : SS) < ns) fetch_params(raw_s[gi], raw_z[gi], (kb + gi * SPG) / X.spg);
-        v4u a[SS][MT], w[SS];
+        for (int gi = 0; gi < NGS; ++gi) fetch_params(raw_s[gi], raw_z[gi], g0 + gi);
+        // a[p][mt][h]: ALDS: pair p, rows 8h .. 8h + 7; else step 2p + h in operand order
+        v4u a[SS / 2][MT][2], w[SS];
 #pragma unroll
-        for (int i = 0; i < SS; ++i)
-            if (FULL || i < ns) {
+        for (int p = 0; p < SS / 2; ++p)
 #pragma unroll
-                for (int mt = 0; mt < MT; ++mt)
-                    a[i][mt] = *(const v4u *)(X.src + (long)(kb + i) * (KBLK * 2) + src_lane_off[mt]);
-            }
+            for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+                for (int h = 0; h < 2; ++h)
+                    a[p][mt][h] = ALDS
+                            ? *(const v4u *)(X.src + (long)(kb + 2 * p) * (KBLK * 2) + src_row_off[mt][h])
+                            : *(const v4u *)(X.src + (long)(kb + 2 * p + h) * (KBLK * 2) + src_lane_off[mt]);
         // the weights are read once: non-temporal loads keep them from
         // displacing the activations and parameters in the caches
 #pragma unroll
         for (int i = 0; i < SS; ++i)
-            if (FULL || i < ns) w[i] = __builtin_nontemporal_load((const v4u *)(wlane + (long)(kb + i) * (KBLK * CHUNK / 2)));
+            w[i] = __builtin_nontemporal_load((const v4u *)(wlane + (long)(kb + i) * (KBLK * CHUNK / 2)));
         // every load of the super-step is in flight before its first MFMA
         __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-        for (int i = 0; i < SS; ++i)
-            if (FULL || i < ns) {
-                compute_step(w[i], a[i]);
+        for (int p = 0; p < SS / 2; ++p) {
+            v4u as[2][MT];
+            if constexpr (ALDS) {
+#pragma unroll
+                for (int mt = 0; mt < MT; ++mt) {
+#pragma unroll
+                    for (int h = 0; h < 2; ++h) stage[mt * 128 + wr_idx[h]] = a[p][mt][h];
+                }
+#pragma unroll
+                for (int sx = 0; sx < 2; ++sx)
+#pragma unroll
+                    for (int mt = 0; mt < MT; ++mt) as[sx][mt] = stage[mt * 128 + rd_idx[sx]];
+            } else {
+#pragma unroll
+                for (int sx = 0; sx < 2; ++sx)
+#pragma unroll
+                    for (int mt = 0; mt < MT; ++mt) as[sx][mt] = a[p][mt][sx];
+            }
+#pragma unroll
+            for (int sx = 0; sx < 2; ++sx) {
+                const int i = 2 * p + sx;
+                // with whole groups inside the super-step a group's first step
+                // is known at compile time and starts from a zero operand
+                compute_step(w[i], as[sx], SPG != 0 && i % (SPG ? SPG : 1) == 0);
                 if constexpr (SPG != 0) {
-                    if ((i + 1) % SPG == 0) flush_group(raw_s[i / SPG], raw_z[i / SPG], (kb + i) / X.spg);
+                    if ((i + 1) % SPG == 0) flush_group(raw_s[i / SPG], raw_z[i / SPG], false);
                 }
             }
+        }
         if constexpr (SPG == 0) {
-            if ((kb + ns) % X.spg == 0 || kb + ns >= kb1) flush_group(raw_s[0], raw_z[0], kb / X.spg);
+            if ((kb + SS) % X.spg == 0 || kb + SS >= kb1) flush_group(raw_s[0], raw_z[0], true);
         }
     };
 
-    for (int kb = kb0; kb < kb1; kb += SS) {
-        const int ns = kb1 - kb < SS ? kb1 - kb : SS;
-        if (ns == SS)
-            super_step(kb, ns, std::true_type {});
-        else
-            super_step(kb, ns, std::false_type {});
+    int kb = kb0;
+    for (; kb + SS <= kb1; kb += SS) super_step(kb);
+    if (kb < kb1) {
+        // ragged end of K: one step at a time, parameters fetched when the
+        // group ends
+        if constexpr (SPG != 0) {
+#pragma unroll
+            for (int mt = 0; mt < MT; ++mt) {
+                rsum[mt] = v4f {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+                for (int tt = 0; tt < 4; ++tt) acc[mt][tt] = v4f {0.f, 0.f, 0.f, 0.f};
+            }
+        }
+#pragma unroll 1
+        for (; kb < kb1; ++kb) {
+            v4u a1[MT];
+#pragma unroll
+            for (int mt = 0; mt < MT; ++mt) a1[mt] = *(const v4u *)(X.src + (long)kb * (KBLK * 2) + src_lane_off[mt]);
+            const v4u w1 = __builtin_nontemporal_load((const v4u *)(wlane + (long)kb * (KBLK * CHUNK / 2)));
+            compute_step(w1, a1, false);
+            if ((kb + 1) % X.spg == 0 || kb + 1 == kb1) {
+                unsigned word_s, word_z;
+                fetch_params(word_s, word_z, kb / X.spg);
+                flush_group(word_s, word_z, true);
+            }
+        }
     }
 
     // ---- add the wavefronts' sums in wavefront order and store.  LDS holds
     // [wavefront][row][column] floats; a thread then owns four consecutive
     // columns of one row and runs the four-wide epilogue of the GEMM tiles.
+    if constexpr (ALDS) __syncthreads(); // the sums take the memory the activations were staged in
     float *red = (float *)red4;
     constexpr int WSTRIDE = MT * 16 * CHUNK; // floats per wavefront
 #pragma unroll
@@ -253,18 +381,38 @@ __global__ void __launch_bounds__(NWV * 64) woqp_kernel(const problem_t P_, cons
             for (int r = 0; r < 4; ++r)
                 red[wave * WSTRIDE + (mt * 16 + 4 * q + r) * CHUNK + tt * 16 + j] = tot[mt][tt][r];
     __syncthreads();
-    const auto &P = MI355_KERNARG_PROBLEM();
-    if (M <= 8) {
-        // few rows: one element per thread, 64 consecutive columns per
-        // wavefront (the four-wide path below starts later: it gathers the
-        // epilogue's operands first, which a single pass does not win back)
-        const int m = t >> 6, nl = t & 63;
-        if (m >= M) return;
-        const float *cell = red + m * CHUNK + nl;
-        float v = cell[0];
+    if constexpr (PLAIN) {
+        // one element per thread, 64 consecutive columns per wavefront
+#pragma unroll 1
+        for (int e = t; e < M * CHUNK; e += NWV * 64) {
+            const int m = e >> 6, nl = e & 63;
+            const float *cell = red + m * CHUNK + nl;
+            float v = cell[0];
 #pragma unroll
-        for (int wv = 1; wv < NWV; ++wv) v += cell[wv * WSTRIDE];
-        epilogue_store(P, v, 0, m, chunk * CHUNK + nl);
+            for (int wv = 1; wv < NWV; ++wv) v += cell[wv * WSTRIDE];
+            const unsigned bits = X.dst_dt == MI355_DT_F32 ? f2u(v)
+                    : X.dst_dt == MI355_DT_BF16 ? (unsigned)f32_to_bf16(v) : (unsigned)f32_to_f16(v);
+            const long off = (long)m * X.dst_ld + chunk * CHUNK + nl;
+            if (X.dst_dt == MI355_DT_F32)
+                ((unsigned *)X.dst)[off] = bits;
+            else
+                ((uint16_t *)X.dst)[off] = (uint16_t)bits;
+        }
+        return;
+    } else {
+    const auto &P = (*(kernarg_woqp_t *)__builtin_amdgcn_kernarg_segment_ptr()).P;
+    if (M <= 8) {
+        // few rows: one element per thread (the four-wide path below gathers
+        // the epilogue's operands first, which a single pass does not win back)
+#pragma unroll 1
+        for (int e = t; e < M * CHUNK; e += NWV * 64) {
+            const int m = e >> 6, nl = e & 63;
+            const float *cell = red + m * CHUNK + nl;
+            float v = cell[0];
+#pragma unroll
+            for (int wv = 1; wv < NWV; ++wv) v += cell[wv * WSTRIDE];
+            epilogue_store(P, v, 0, m, chunk * CHUNK + nl);
+        }
         return;
     }
 #pragma unroll 1
@@ -279,6 +427,7 @@ __global__ void __launch_bounds__(NWV * 64) woqp_kernel(const problem_t P_, cons
         const long n = (long)chunk * CHUNK + nq * 4;
         gemm::apply_epilogue4(P, v, 0, m, n, 4);
         gemm::store4(P, P.ds[2] == 1 && gemm::vec_ok_store(P.dst, P.ds[0], P.ds[1], dt_bits(P.dst_dt)), v, 0, m, n, 4);
+    }
     }
 }
 
@@ -319,8 +468,14 @@ struct woqp_geo_t {
     int ss, spg; // template arguments; ss == 0: not covered
 };
 
+// Wavefronts per workgroup.  One tile of rows: 16 wavefronts of 8 steps each
+// at K = 4096 (a wavefront's work after its last data arrive is what ends the
+// launch); two tiles, or groups of fewer than 128 rows (more parameter words in
+// flight): 8 wavefronts, the register budget of two per SIMD.
+int wavefronts(int mt, long G, long K) { return mt == 1 && (G == K || G >= 4 * KBLK) ? 16 : 8; }
+
 woqp_geo_t pick_geo(int mt, long G, long K) {
-    const int ss_max = mt == 1 ? 16 : 8;
+    const int ss_max = mt == 1 && wavefronts(mt, G, K) == 8 ? 16 : 8;
     if (G == K) return {ss_max, 0};
     if (G % KBLK != 0) return {0, 0};
     const long spg = G / KBLK;
@@ -360,7 +515,19 @@ int woqp_launch(const mi355_matmul_desc_t &d, const problem_t &P, hipStream_t st
     const int mt = d.M <= 16 ? 1 : 2;
     const long G = group_rows(d);
     const woqp_geo_t geo = pick_geo(mt, G, d.K);
-    woqp_extra_t X {};
+    const int nw = wavefronts(mt, G, d.K);
+    // nothing after the K sum but the conversion?
+    const bool plain = P.bias_dt == MI355_DT_UNDEF && P.n_po == 0 && !P.dst_dynamic
+            && P.dst_scale.dt == MI355_DT_UNDEF && P.dst_zp.dt == MI355_DT_UNDEF && P.ds[2] == 1
+            && (P.dst_dt == MI355_DT_F32 || P.dst_dt == MI355_DT_BF16 || P.dst_dt == MI355_DT_F16)
+            && P.ds[1] < (1L << 31);
+    woqp_args_t A;
+    A.P = P;
+    woqp_extra_t &X = A.X;
+    X = woqp_extra_t {};
+    X.dst = (uint8_t *)P.dst;
+    X.dst_dt = P.dst_dt;
+    X.dst_ld = (int)P.ds[1];
     X.wei = (const uint8_t *)P.wei;
     X.src = (const uint8_t *)P.src;
     X.M = (int)d.M; X.N = (int)d.N; X.K = (int)d.K;
@@ -370,7 +537,7 @@ int woqp_launch(const mi355_matmul_desc_t &d, const problem_t &P, hipStream_t st
     // whole super-steps when a group holds super-steps
     const long unit = geo.spg ? geo.spg : (G == d.K ? 1 : geo.ss);
     const long KB = d.K / KBLK;
-    X.kbw = (int)(((KB + NWV - 1) / NWV + unit - 1) / unit * unit);
+    X.kbw = (int)(((KB + nw - 1) / nw + unit - 1) / unit * unit);
     X.sc_dt = d.wei_scale.dt;
     X.zp_dt = d.wei_zp.dt;
     // an absent parameter is fetched from src (any readable memory) and ignored
@@ -382,21 +549,23 @@ int woqp_launch(const mi355_matmul_desc_t &d, const problem_t &P, hipStream_t st
     X.zp_grouped = X.zp_dt && (d.wei_zp.mask & 2);
     X.zp_common = X.zp_dt && d.wei_zp.mask == 0;
     X.signed_w = d.wei_dt == MI355_DT_S4;
-    const dim3 grid((unsigned)(d.N / CHUNK)), block(NWV * 64);
-#define MI355_WOQP_CASE(MT_, SS_, SPG_) \
-    if (mt == MT_ && geo.ss == SS_ && geo.spg == SPG_) { \
-        hipLaunchKernelGGL((woqp_kernel<MT_, SS_, SPG_>), grid, block, 0, stream, P, X); \
+    const dim3 grid((unsigned)(d.N / CHUNK)), block(nw * 64);
+#define MI355_WOQP_CASE(NW_, MT_, SS_, SPG_) \
+    if (nw == NW_ && mt == MT_ && geo.ss == SS_ && geo.spg == SPG_) { \
+        if (plain) \
+            hipLaunchKernelGGL((woqp_kernel<NW_, MT_, SS_, SPG_, true>), grid, block, 0, stream, A.X); \
+        else \
+            hipLaunchKernelGGL((woqp_kernel<NW_, MT_, SS_, SPG_, false>), grid, block, 0, stream, A); \
         return hipGetLastError() == hipSuccess ? MI355_SUCCESS : MI355_RUNTIME_ERROR; \
     }
-    MI355_WOQP_CASE(1, 4, 1)
-    MI355_WOQP_CASE(1, 8, 2)
-    MI355_WOQP_CASE(1, 16, 4)
-    MI355_WOQP_CASE(1, 16, 8)
-    MI355_WOQP_CASE(1, 16, 0)
-    MI355_WOQP_CASE(2, 4, 1)
-    MI355_WOQP_CASE(2, 8, 2)
-    MI355_WOQP_CASE(2, 8, 4)
-    MI355_WOQP_CASE(2, 8, 0)
+    MI355_WOQP_CASE(16, 1, 8, 4)
+    MI355_WOQP_CASE(16, 1, 8, 0)
+    MI355_WOQP_CASE(8, 1, 4, 1)
+    MI355_WOQP_CASE(8, 1, 8, 2)
+    MI355_WOQP_CASE(8, 2, 4, 1)
+    MI355_WOQP_CASE(8, 2, 8, 2)
+    MI355_WOQP_CASE(8, 2, 8, 4)
+    MI355_WOQP_CASE(8, 2, 8, 0)
 #undef MI355_WOQP_CASE
     set_error("woq_packed: no kernel for %d tiles, super-step %d, group %d", mt, geo.ss, geo.spg);
     return MI355_UNIMPLEMENTED;
