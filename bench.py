@@ -108,7 +108,7 @@ def build_problem(name, M=None, wtag="any"):
     a layout pre-pass inside every launch, which then is part of the step."""
     from onednn_amd import cabi, configs
     if name == "c1":
-        return configs.config1()
+        return configs.config1(wtag="ba" if wtag == "any" else wtag)
     if name == "c2":
         p = configs.config2(M=M or 1, wtag="ab" if wtag == "any" else wtag)
         if wtag == "any":  # what format_tag::any resolves to for decode weights

@@ -22,12 +22,14 @@ def _rng(seed, tensor_id):
     return np.random.Generator(np.random.PCG64([seed, tensor_id]))
 
 
-def config1(M=256, N=1024, K=1024, dst="f32", seed=1, impl=cabi.IMPL_AUTO):
+def config1(M=256, N=1024, K=1024, dst="f32", seed=1, impl=cabi.IMPL_AUTO, wtag="ab"):
     """u8 x s8 -> f32 (or s32): src zero point 128, src scale 0.02, per-N
     weights scales, f32 bias.  dst='s32' drops scales and bias (accumulator
     check)."""
     src = _rng(seed, 1).integers(0, 256, size=(M, K), dtype=np.uint8)
     wei = _rng(seed, 2).integers(-127, 128, size=(K, N), dtype=np.int8)
+    if wtag == "ba":
+        wei = np.ascontiguousarray(wei.T)
     quant = {"src_zp": QuantParam(cabi.DT_S32, MASK_COMMON, np.array([128], np.int32))}
     bias = None
     bias_dt = cabi.DT_UNDEF
@@ -39,7 +41,7 @@ def config1(M=256, N=1024, K=1024, dst="f32", seed=1, impl=cabi.IMPL_AUTO):
         bias_dt = cabi.DT_F32
     return MatmulProblem(M=M, N=N, K=K, src_dt=cabi.DT_U8, wei_dt=cabi.DT_S8,
                          dst_dt=cabi.DT_NAMES[dst], src=src, wei=wei, bias_dt=bias_dt, bias=bias,
-                         quant=quant, impl=impl, name=f"C1-{dst}")
+                         wei_stride=strides_for(wtag, 1, K, N), quant=quant, impl=impl, name=f"C1-{dst}")
 
 
 def config2(M=1, N=14336, K=4096, group=128, seed=2, impl=cabi.IMPL_AUTO, wtag="ab"):

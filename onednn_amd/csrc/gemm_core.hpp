@@ -292,10 +292,12 @@ __device__ __forceinline__ void main_loop_two_groups(Acc &acc, char *smem, const
 
     int slot = 0;
     // Group 1 carries the fragments from one iteration to the next; they start
-    // as zeros, so that its first iteration, which has no stage to multiply
-    // yet, adds zero products instead of branching around the MFMAs (one MFMA
-    // sequence on every path keeps the accumulators where they are).
-    typename Mma::frag_t f = {};
+    // as the operands' zero (Mma::zero_frag: bytes the MFMA row reads as 0 --
+    // not all-zero bits for an operand type whose bytes are re-biased at use), so
+    // that its first iteration, which has no stage to multiply yet, adds zero
+    // products instead of branching around the MFMAs (one MFMA sequence on every
+    // path keeps the accumulators where they are).
+    typename Mma::frag_t f = Mma::zero_frag();
     const int niter = ngroups + (late ? 1 : 0);
     auto read_stage = [&](int g) __attribute__((always_inline)) {
         unsigned S[KSTEP];

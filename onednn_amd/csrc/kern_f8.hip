@@ -46,6 +46,7 @@ struct f8_mma_t {
     struct frag_t {
         v8i a[ROWS], b[COLS];
     };
+    __device__ static __forceinline__ frag_t zero_frag() { return frag_t {}; } // fp8 zero is all-zero bits
     // lane l supplies row l%32 and K bytes 32*(l/32) .. +32 of the stage: two
     // 16-byte chunks.  Per-lane LDS offsets of fragment 0; fragment i is 32 rows
     // (2 KB) further with the same swizzle.

@@ -14,6 +14,9 @@
 //   d = (float)acc * src_scale * wei_scale[n]  -> shared epilogue.
 #include "gemm_core.hpp"
 
+#include <cstdlib>
+#include <cstring>
+
 namespace mi355 {
 
 namespace {
@@ -47,6 +50,17 @@ struct i8_mma_t {
     struct frag_t {
         v4i a[ROWS], b[COLS];
     };
+    // fragments whose products are zero: a u8 operand is re-biased by 128 where
+    // it is used, so its zero is the byte 0x80
+    __device__ static __forceinline__ frag_t zero_frag() {
+        frag_t f;
+        const int za = SRC_U8 ? (int)0x80808080 : 0, zb = WEI_U8 ? (int)0x80808080 : 0;
+#pragma unroll
+        for (int i = 0; i < ROWS; ++i) f.a[i] = v4i {za, za, za, za};
+#pragma unroll
+        for (int j = 0; j < COLS; ++j) f.b[j] = v4i {zb, zb, zb, zb};
+        return f;
+    }
     // Per-lane LDS offsets of fragment 0 of both operands.  Fragment i is 16 rows
     // further: the swizzle depends on the row modulo 16 only, so it is the same
     // address plus i KB, which goes into the offset field of the read.
@@ -245,6 +259,151 @@ __global__ void __launch_bounds__(G::NT) __attribute__((amdgpu_waves_per_eu(G::N
     store_quadrant<layout16_t, G::WCOLS>(P, smem, ntab, acc, b, m0 + wm * 128, n0 + wn * G::WCOLS, wn * G::WCOLS, cv);
 }
 
+
+// ---- few tiles or a K that is not a multiple of the stage: 32 x 32 dst tiles
+// without LDS staging.  The 256 x 256 tiles above leave the device idle when
+// M x N holds only a handful of them (4 workgroups for 256 x 1024), and their
+// stage loads want K in units of 64.  Here a workgroup of four wavefronts owns a
+// 32 x 32 tile, the wavefronts take every fourth 64-byte step of K, each lane
+// loads its MFMA operands (16 bytes of a src row, 16 bytes of a weights
+// column, K contiguous in both) straight from memory, one step ahead of the
+// matrix cores, and a step beyond K's last 16 bytes is filled with the
+// operand's zero.  The column sums of the weights and the row sums of src that
+// the zero-point correction needs come out of two more MFMAs per operand tile
+// against all-ones bytes, in the accumulators' own lane layout: no pre-pass
+// kernels.  The four wavefronts' sums are added through LDS in wavefront order
+// (integer: exact in any order), converted like the large tiles' and finished
+// by the general epilogue.
+constexpr int ST = 32;     // rows and columns of a small tile
+constexpr int SNW = 4;     // wavefronts of its workgroup
+
+template <bool SRC_U8, bool WEI_U8>
+__global__ void __launch_bounds__(SNW * 64) i8_small_kernel(const problem_t P_, const i8_extra_t X) {
+    // [wavefront][slot][lane]; slots: 16 accumulators, 8 column sums, 8 row sums
+    __shared__ int part[SNW][32][64];
+    const auto &P = MI355_KERNARG_PROBLEM();
+    const int t = threadIdx.x, lane = t & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(t >> 6);
+    const int j = lane & 15, q = lane >> 4;
+    const long b = blockIdx.z;
+    const long m0 = (long)(blockIdx.x / X.tiles_n) * ST, n0 = (long)(blockIdx.x % X.tiles_n) * ST;
+    const long M = P.M, N = P.N, K = P.K;
+    const long lda = P.ss[1];
+    const char *A = (const char *)P.src + (P.ss[0] ? b * P.ss[0] : 0);
+    const char *Bt = (const char *)X.bt + b * X.bt_bstride;
+    // rows and columns beyond the edge read the last valid one (never stored)
+    const char *arow[2], *bcol[2];
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+        const long m = m0 + 16 * i + j < M ? m0 + 16 * i + j : M - 1;
+        const long n = n0 + 16 * i + j < N ? n0 + 16 * i + j : N - 1;
+        arow[i] = A + m * lda + 16 * q;
+        bcol[i] = Bt + n * X.ldb + 16 * q;
+    }
+    const int a_fill = SRC_U8 ? (int)0x80808080 : 0, b_fill = WEI_U8 ? (int)0x80808080 : 0;
+    struct frag_t {
+        v4i a[2], b[2];
+    };
+    // K is a multiple of 16: a lane's 16 bytes are inside K or beyond it
+    auto load = [&](long step) __attribute__((always_inline)) {
+        frag_t f;
+        const long k = step * 64;
+        const bool in = k + 16 * q < K;
+#pragma unroll
+        for (int i = 0; i < 2; ++i) {
+            f.a[i] = v4i {a_fill, a_fill, a_fill, a_fill};
+            f.b[i] = v4i {b_fill, b_fill, b_fill, b_fill};
+            if (in) {
+                f.a[i] = *(const v4i *)(arow[i] + k);
+                f.b[i] = *(const v4i *)(bcol[i] + k);
+            }
+        }
+        return f;
+    };
+    v4i acc[2][2], cs[2], rs[2];
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+        cs[i] = rs[i] = v4i {0, 0, 0, 0};
+#pragma unroll
+        for (int jn = 0; jn < 2; ++jn) acc[i][jn] = v4i {0, 0, 0, 0};
+    }
+    const v4i ones = {0x01010101, 0x01010101, 0x01010101, 0x01010101};
+    const long nsteps = (K + 63) / 64;
+    long step = wave;
+    frag_t cur = load(step < nsteps ? step : 0);
+    for (; step < nsteps; step += SNW) {
+        const frag_t nxt = load(step + SNW < nsteps ? step + SNW : step);
+        v4i a[2], w[2];
+#pragma unroll
+        for (int i = 0; i < 2; ++i) {
+            a[i] = SRC_U8 ? (cur.a[i] ^ (int)0x80808080) : cur.a[i];
+            w[i] = WEI_U8 ? (cur.b[i] ^ (int)0x80808080) : cur.b[i];
+        }
+        // operands exchanged as in the large tiles: a lane holds four
+        // consecutive n (4 * (lane / 16) + e) of row lane % 16
+#pragma unroll
+        for (int i = 0; i < 2; ++i) {
+#pragma unroll
+            for (int jn = 0; jn < 2; ++jn)
+                acc[i][jn] = __builtin_amdgcn_mfma_i32_16x16x64_i8(w[jn], a[i], acc[i][jn], 0, 0, 0);
+            cs[i] = __builtin_amdgcn_mfma_i32_16x16x64_i8(w[i], ones, cs[i], 0, 0, 0); // [e]: column 4 * (lane / 16) + e
+            rs[i] = __builtin_amdgcn_mfma_i32_16x16x64_i8(ones, a[i], rs[i], 0, 0, 0); // every e: row lane % 16
+        }
+        cur = nxt;
+    }
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+#pragma unroll
+            for (int jn = 0; jn < 2; ++jn) part[wave][i * 8 + jn * 4 + e][lane] = acc[i][jn][e];
+            part[wave][16 + i * 4 + e][lane] = cs[i][e];
+            part[wave][24 + i * 4 + e][lane] = rs[i][e];
+        }
+    }
+    __syncthreads();
+    // thread (unit = i, jn; lane): the quad of row m0 + 16 i + lane % 16,
+    // columns n0 + 16 jn + 4 (lane / 16) ..
+    const int unit = t >> 6, ui = unit >> 1, ujn = unit & 1;
+    int sum[4] = {0, 0, 0, 0}, csum[4] = {0, 0, 0, 0}, rsum = 0;
+#pragma unroll
+    for (int wv = 0; wv < SNW; ++wv) {
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            sum[e] += part[wv][ui * 8 + ujn * 4 + e][lane];
+            csum[e] += part[wv][16 + ujn * 4 + e][lane];
+        }
+        rsum += part[wv][24 + ui * 4][lane];
+    }
+    const long m = m0 + 16 * ui + j, nbase = n0 + 16 * ujn + 4 * q;
+    if (m >= M || nbase >= N) return;
+    const int nvalid = N - nbase < 4 ? (int)(N - nbase) : 4;
+    const long bw = P.ws[0] ? b : 0;
+    int a_c = SRC_U8 ? 128 : 0;
+    if (P.src_zp.dt != MI355_DT_UNDEF) a_c -= load_int(P.src_zp.dt, P.src_zp.p, 0);
+    const bool with_src_sc = P.src_scale.dt != MI355_DT_UNDEF, with_wei_sc = P.wei_scale.dt != MI355_DT_UNDEF;
+    const float ssc = with_src_sc ? load_float(P.src_scale.dt, P.src_scale.p, 0) : 1.f;
+    float v[4] = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+        if (e < nvalid) {
+            const long n = nbase + e;
+            int c = WEI_U8 ? 128 : 0;
+            if (P.wei_zp.dt != MI355_DT_UNDEF)
+                c -= load_int(P.wei_zp.dt, P.wei_zp.p, quant_off(P.wei_zp, bw, 0, n, P.K, P.N));
+            // the large tiles' order: a * colsum + K * a * c, then + c * rowsum
+            const int cc = a_c * csum[e] + (int)K * a_c * c;
+            float f = (float)(sum[e] + (cc + c * rsum));
+            if (with_src_sc) f *= ssc;
+            if (with_wei_sc)
+                f *= load_float(P.wei_scale.dt, P.wei_scale.p, quant_off(P.wei_scale, bw, 0, n, P.K, P.N));
+            v[e] = f;
+        }
+    }
+    apply_epilogue4(P, v, b, m, nbase, nvalid);
+    store4(P, P.ds[2] == 1 && vec_ok_store(P.dst, P.ds[0], P.ds[1], dt_bits(P.dst_dt)), v, b, m, nbase, nvalid);
+}
+
 // out[r] = sum_k (bytes[r][k] ^ flip) as signed bytes; one wave per row
 __global__ void __launch_bounds__(256) i8_rowsum_kernel(const int8_t *p, long rows, long K,
         long ld, int flip, int *out) {
@@ -270,6 +429,7 @@ __global__ void __launch_bounds__(256) i8_rowsum_kernel(const int8_t *p, long ro
 }
 
 struct i8_plan_t {
+    bool small; // 32 x 32 tiles
     bool need_transpose, need_colsum, need_rowsum;
     size_t off_bt, off_colsum, off_rowsum, total;
     long Bw, Bs;
@@ -280,10 +440,21 @@ i8_plan_t make_plan(const mi355_matmul_desc_t &d) {
     p.Bw = d.wei_stride[0] ? d.batch : 1;
     p.Bs = d.src_stride[0] ? d.batch : 1;
     p.need_transpose = !(d.wei_stride[1] == 1);
+    // the small tiles when the large ones would occupy less than a quarter of
+    // the device, or cannot step through K (they compute their own sums and
+    // have no dynamic dst quantization)
+    const long big_tiles = ((d.M + BM - 1) / BM) * ((d.N + i8_geo_t::BN - 1) / i8_geo_t::BN) * d.batch;
+    p.small = !d.dst_scale_dynamic && (big_tiles < 64 || d.K % BK != 0);
+    // MI355_I8_TILES=large|small overrides the choice where both can run (for
+    // tests and tuning; read at every call)
+    if (const char *force = getenv("MI355_I8_TILES")) {
+        if (!strcmp(force, "large") && d.K % BK == 0) p.small = false;
+        if (!strcmp(force, "small") && !d.dst_scale_dynamic) p.small = true;
+    }
     // a = off_s - zs can be non-zero whenever src is u8 or has a zero point;
     // c likewise for the weights
-    p.need_colsum = d.src_dt == MI355_DT_U8 || !quant_absent(d.src_zp);
-    p.need_rowsum = d.wei_dt == MI355_DT_U8 || !quant_absent(d.wei_zp);
+    p.need_colsum = !p.small && (d.src_dt == MI355_DT_U8 || !quant_absent(d.src_zp));
+    p.need_rowsum = !p.small && (d.wei_dt == MI355_DT_U8 || !quant_absent(d.wei_zp));
     size_t off = 0;
     p.off_bt = off;
     if (p.need_transpose) off += align_up((size_t)p.Bw * d.N * d.K, 256);
@@ -300,7 +471,10 @@ i8_plan_t make_plan(const mi355_matmul_desc_t &d) {
 int i8_supported(const mi355_matmul_desc_t &d) {
     if (!is_int8_dt(d.src_dt) || !is_int8_dt(d.wei_dt)) return MI355_UNIMPLEMENTED;
     if (dt_bits(d.dst_dt) < 8) return MI355_UNIMPLEMENTED;
-    if (d.K < BK || d.K % BK != 0) return MI355_UNIMPLEMENTED;
+    // (a K that is not a multiple of the large tiles' stage runs on the small
+    // tiles, whose 16-byte operand loads are whole inside K or beyond it)
+    if (d.K < 16 || d.K % 16 != 0) return MI355_UNIMPLEMENTED;
+    if (d.K % BK != 0 && d.dst_scale_dynamic) return MI355_UNIMPLEMENTED;
     if (d.src_stride[2] != 1 || d.src_stride[1] % 16 != 0) return MI355_UNIMPLEMENTED;
     if (d.src_stride[0] % 16 != 0) return MI355_UNIMPLEMENTED;
     const bool k_major = d.wei_stride[1] == 1 && d.wei_stride[2] % 16 == 0
@@ -364,11 +538,29 @@ int i8_launch(const mi355_matmul_desc_t &d, const problem_t &P, void *scratch,
                     d.src_stride[1], src_u8 ? (int)0x80808080 : 0, rs + b * d.M);
         X.rowsum = rs;
     }
+    const bool su = d.src_dt == MI355_DT_U8, wu = d.wei_dt == MI355_DT_U8;
+    if (plan.small) {
+        X.tiles_m = (int)((d.M + ST - 1) / ST);
+        X.tiles_n = (int)((d.N + ST - 1) / ST);
+        const long tiles = (long)X.tiles_m * X.tiles_n;
+        if (tiles >= (1L << 31)) {
+            set_error("mfma_i8: %ld small tiles exceed the grid", tiles);
+            return MI355_UNIMPLEMENTED;
+        }
+        const dim3 sgrid((unsigned)tiles, 1, (unsigned)d.batch);
+        auto go_small = [&](auto kern) -> int {
+            hipLaunchKernelGGL(kern, sgrid, dim3(SNW * 64), 0, stream, P, X);
+            return hipGetLastError() == hipSuccess ? MI355_SUCCESS : MI355_RUNTIME_ERROR;
+        };
+        if (su && wu) return go_small(i8_small_kernel<true, true>);
+        if (su) return go_small(i8_small_kernel<true, false>);
+        if (wu) return go_small(i8_small_kernel<false, true>);
+        return go_small(i8_small_kernel<false, false>);
+    }
     X.tiles_m = (int)((d.M + BM - 1) / BM);
     X.tiles_n = (int)((d.N + i8_geo_t::BN - 1) / i8_geo_t::BN);
     dim3 grid((unsigned)(X.tiles_m * X.tiles_n), 1, (unsigned)d.batch);
     constexpr int smem_bytes = NSTAGE * i8_geo_t::STAGE_BYTES + NTAB_BYTES;
-    const bool su = d.src_dt == MI355_DT_U8, wu = d.wei_dt == MI355_DT_U8;
     auto go = [&](auto kern) -> int {
         if (const int st = ensure_dynamic_lds((const void *)kern, smem_bytes, "mfma_i8")) return st;
         hipLaunchKernelGGL(kern, grid, dim3(i8_geo_t::NT), smem_bytes, stream, P, X);

@@ -76,6 +76,7 @@ struct mxf4_mma_t {
         v4i a[ROWS], b[COLS];
         int sa[ROWS], sb[COLS];
     };
+    __device__ static __forceinline__ frag_t zero_frag() { return frag_t {}; } // e2m1 zero is all-zero bits
     // LDS byte address of the scale dwords that belong to the stage at S[0]
     __device__ static __forceinline__ unsigned scales(const unsigned (&S)[1], const mxf4_ctx_t &c) {
         const unsigned slot = (S[0] - c.lds0) / G::STAGE_BYTES;

@@ -31,3 +31,12 @@ def gpu():
     assert n.value > 0, "no HIP device visible"
     cabi.check(lib.mi355_device_set(0))
     return lib
+
+
+@pytest.fixture(params=["large", "small"])
+def i8_tiles(request, monkeypatch):
+    """Runs a test once per tile geometry of hip:mfma_i8 (the 256 x 256 LDS
+    tiles and the 32 x 32 direct ones) wherever both can take the problem; by
+    itself the dispatcher would give every small test shape to the small tiles."""
+    monkeypatch.setenv("MI355_I8_TILES", request.param)
+    return request.param

@@ -7,7 +7,7 @@ from onednn_amd import cabi, configs
 from onednn_amd.problem import run_gpu
 from tests.helpers import assert_bit_exact, assert_close, assert_decode_close, assert_gemm_close, fp8_mfma_bound
 
-pytestmark = pytest.mark.gpu
+pytestmark = [pytest.mark.gpu, pytest.mark.usefixtures("i8_tiles")]
 
 
 @pytest.mark.parametrize("dst", ["s32", "f32"])

@@ -13,7 +13,7 @@ from tests import tail_cases as tc
 from tests.helpers import assert_bit_exact, logical
 from tests.test_oracle_pins import PR_VARIANTS
 
-pytestmark = pytest.mark.gpu
+pytestmark = [pytest.mark.gpu, pytest.mark.usefixtures("i8_tiles")]
 F = np.float32
 IMPLS = [cabi.IMPL_REF, cabi.IMPL_AUTO]
 
