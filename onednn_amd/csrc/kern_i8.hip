@@ -440,11 +440,13 @@ i8_plan_t make_plan(const mi355_matmul_desc_t &d) {
     p.Bw = d.wei_stride[0] ? d.batch : 1;
     p.Bs = d.src_stride[0] ? d.batch : 1;
     p.need_transpose = !(d.wei_stride[1] == 1);
-    // the small tiles when the large ones would occupy less than a quarter of
-    // the device, or cannot step through K (they compute their own sums and
-    // have no dynamic dst quantization)
+    // the small tiles when the large ones would occupy less than a tenth of the
+    // device (measured with K = 1024 and 4096: 16 large tiles take 24 / 52 us
+    // against 18 / 40 us, 32 large tiles 55 us against 74), or cannot step
+    // through K (the small tiles compute their own sums and have no dynamic dst
+    // quantization)
     const long big_tiles = ((d.M + BM - 1) / BM) * ((d.N + i8_geo_t::BN - 1) / i8_geo_t::BN) * d.batch;
-    p.small = !d.dst_scale_dynamic && (big_tiles < 64 || d.K % BK != 0);
+    p.small = !d.dst_scale_dynamic && (big_tiles < 24 || d.K % BK != 0);
     // MI355_I8_TILES=large|small overrides the choice where both can run (for
     // tests and tuning; read at every call)
     if (const char *force = getenv("MI355_I8_TILES")) {
