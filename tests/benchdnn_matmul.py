@@ -18,13 +18,31 @@ primitive, execute.
 Test infrastructure: the correctness mode needs the oracle, which the product
 package never imports.
 
+Buffers from files (tests/benchdnn/utils/fill.cpp:489-543, doc/knobs_common.md
+"--buffer-prefix"): --buffer-prefix=PREFIX fills every buffer for which the
+file PREFIX.<execution argument id>.bin exists with that file's bytes instead
+of generated data (a file whose size differs from the buffer's fails the
+case, as in the reference); --export-buffers=PREFIX writes the generated
+buffers under those names, so that the reference's benchdnn can be run on the
+bytes this driver ran on.  Ids: src 1, weights 33, bias 41, dst 17 (the sum
+post-op's input), scales 4096 + arg, zero points 8192 + arg, the tensor of
+binary post-op i 32768 * (i + 1) + 2.
+
+Performance report (doc/knobs_perf_report.md): --perf-template=def | csv |
+CUSTOM with the %engine% %impl% %name% %prb% %desc% %driver% %idx% %attr%
+%stag% %wtag% %dtag% %bia_dt% fields and the measured %time% %ops% %flops%
+%ibytes% %obytes% %iobytes% %bw% %ctime% %cpdtime% %cptime% (%clocks% and
+%freq% print 0) with the time modifiers - 0 + and the unit modifiers K M G.
+
 Supported knobs: --dt, --stag, --wtag, --dtag (ab | ba | any), --bia-dt,
 --attr-scales, --attr-zero-points, --attr-post-ops, --attr-fpmath, --impl,
---mode, and 2-D problem descriptors MxK:KxN.  Policies: common, per_oc,
+--mode, --buffer-prefix, --export-buffers, --perf-template, --max-ms-per-prb,
+and 2-D problem descriptors MxK:KxN.  Policies: common, per_oc,
 per_ocic (with GxH groups), per_tensor (with GxH groups), per_dim_0, per_dim_1.
 """
 import itertools
 import os
+import re
 import sys
 import time
 
@@ -102,8 +120,13 @@ class Spec:
         return " ".join(parts)
 
 
-def parse(argv):
-    """benchdnn-style arguments -> (mode, [Spec, ...])."""
+# settings of the run, not of a problem (they do not multiply the problem list)
+SETTINGS = {"buffer_prefix": "", "export_buffers": "", "perf_template": "def", "max_ms_per_prb": "300"}
+
+
+def parse(argv, settings=None):
+    """benchdnn-style arguments -> (mode, [Spec, ...]); run-wide knobs go into
+    `settings` (a dict like SETTINGS) when one is given."""
     knobs = {"dt": ["f32"], "stag": ["ab"], "wtag": ["ab"], "dtag": ["ab"], "bia_dt": ["undef"],
              "attr_scales": [""], "attr_zero_points": [""], "attr_post_ops": [""], "attr_fpmath": [""],
              "runtime_dims_masks": [""], "impl": [""]}
@@ -113,6 +136,11 @@ def parse(argv):
             continue
         if a.startswith("--mode="):
             mode = a.split("=", 1)[1].upper()
+            continue
+        if a.startswith("--") and a[2:].partition("=")[0].replace("-", "_") in SETTINGS:
+            k, _, v = a[2:].partition("=")
+            if settings is not None:
+                settings[k.replace("-", "_")] = v
             continue
         if a.startswith("--"):
             k, _, v = a[2:].partition("=")
@@ -323,9 +351,113 @@ def api_objects(p, want_ref_impl=False, runtime_dims_masks=""):
     return pd, prim, strm, args, dst
 
 
-def run_spec(sp, mode="C", min_times=5, max_ms=300.0):
+def buffer_ids(p):
+    """{execution argument id: (holder object, attribute name)} of the buffers of a
+    problem that benchdnn fills (dnnl_types.h: DNNL_ARG_*)."""
+    ids = {dnnl.ARG_SRC: (p, "src"), dnnl.ARG_WEIGHTS: (p, "wei")}
+    if p.bias is not None:
+        ids[dnnl.ARG_BIAS] = (p, "bias")
+    if p.dst_init is not None:
+        ids[dnnl.ARG_DST] = (p, "dst_init")
+    arg_of = {"src": dnnl.ARG_SRC, "wei": dnnl.ARG_WEIGHTS, "dst": dnnl.ARG_DST}
+    for qname, q in p.quant.items():
+        which, kind = qname.split("_")
+        if which == "dst" and kind == "scale" and p.dst_dynamic:
+            continue  # an output
+        ids[(dnnl.ARG_ATTR_SCALES if kind == "scale" else dnnl.ARG_ATTR_ZERO_POINTS) | arg_of[which]] = (q, "data")
+    for i, op in enumerate(p.post_ops):
+        if op.kind == cabi.PO_BINARY:
+            ids[dnnl.ARG_ATTR_MULTIPLE_POST_OP(i) | dnnl.ARG_SRC_1] = (op, "data")
+    return ids
+
+
+def export_buffers(p, prefix):
+    """PREFIX.<id>.bin for every filled buffer, the bytes the library is handed."""
+    names = []
+    os.makedirs(os.path.dirname(os.path.abspath(prefix)), exist_ok=True)
+    for arg, (holder, attr) in sorted(buffer_ids(p).items()):
+        name = f"{prefix}.{arg}.bin"
+        np.ascontiguousarray(getattr(holder, attr)).view(np.uint8).reshape(-1).tofile(name)
+        names.append(name)
+    return names
+
+
+def import_buffers(p, prefix):
+    """Fills the buffers whose files exist; returns (imported ids, error or None).
+    A size mismatch is an error (fill.cpp:514-523)."""
+    done = []
+    for arg, (holder, attr) in sorted(buffer_ids(p).items()):
+        name = f"{prefix}.{arg}.bin"
+        if not os.path.exists(name):
+            continue
+        cur = np.ascontiguousarray(getattr(holder, attr))
+        raw = np.fromfile(name, dtype=np.uint8)
+        if raw.size != cur.nbytes:
+            return done, (f"file '{name}' differs in size from the buffer's memory descriptor: "
+                          f"actual {raw.size}, needed {cur.nbytes}")
+        setattr(holder, attr, raw.view(cur.dtype).reshape(cur.shape))
+        done.append(arg)
+    return done, None
+
+
+PERF_TEMPLATES = {
+    "def": "perf,%engine%,%impl%,%name%,%prb%,%Gops%,%+ctime%,%-time%,%-Gflops%,%0time%,%0Gflops%",
+    "csv": "perf,%engine%,%impl%,%name%,%driver%,%stag%,%wtag%,%dtag%,%bia_dt%,%attr%,%desc%,%Gops%,%+ctime%,"
+           "%-time%,%-Gflops%,%0time%,%0Gflops%",
+}
+
+
+def perf_line(template, sp, impl, det, idx=0):
+    """One report line: `template` with its %...% fields replaced
+    (doc/knobs_perf_report.md; parser of tests/benchdnn/utils/perf_report.cpp)."""
+    template = PERF_TEMPLATES.get(template, template)
+    attr = " ".join(f"--{k.replace('_', '-')}={getattr(sp, k)}" for k in
+                    ("attr_scales", "attr_zero_points", "attr_post_ops", "attr_fpmath") if getattr(sp, k))
+    plain = {"engine": "gpu", "impl": impl, "name": "", "prb": sp.repro(), "desc": sp.desc, "driver": "matmul",
+             "idx": str(idx), "attr": attr, "stag": sp.stag, "wtag": sp.wtag, "dtag": sp.dtag, "bia_dt": sp.bia_dt,
+             "cfg": "", "dt": sp.dt, "dir": "", "mb": "0"}
+    times = {"-": det["min_ms"], "0": det["avg_ms"], "+": det["max_ms"]}
+    units = {"": 1.0, "K": 1e3, "M": 1e6, "G": 1e9}
+
+    def field(m):
+        tok = m.group(1)
+        if tok in plain:
+            return plain[tok]
+        mm = re.fullmatch(r"([-0+]?)([KMG]?)(time|clocks|freq|ibytes|obytes|iobytes|bw|ops|flops|cpdtime|cptime|ctime)", tok)
+        if not mm:
+            return m.group(0)
+        mod, unit, what = mm.groups()
+        t_ms = times[mod or "-"]
+        if what == "time":
+            v = t_ms
+        elif what in ("clocks", "freq"):
+            v = 0.0
+        elif what in ("ibytes", "obytes", "iobytes"):
+            v = {"ibytes": det["ibytes"], "obytes": det["obytes"], "iobytes": det["ibytes"] + det["obytes"]}[what]
+        elif what == "bw":
+            v = (det["ibytes"] + det["obytes"]) / (t_ms * 1e-3)
+        elif what == "ops":
+            v = det["ops"]
+        elif what == "flops":
+            v = det["ops"] / (t_ms * 1e-3)
+        else:  # creation times: one creation is measured, every modifier reports it
+            v = {"cpdtime": det["cpd_ms"], "cptime": det["cp_ms"], "ctime": det["cpd_ms"] + det["cp_ms"]}[what]
+        return f"{v / units[unit]:g}"
+
+    return re.sub(r"%([^%]*)%", field, template)
+
+
+def run_spec(sp, mode="C", min_times=5, max_ms=300.0, settings=None):
     """Returns (status, impl, details): status PASSED / FAILED / SKIPPED (unimplemented)."""
+    settings = settings or SETTINGS
     p = build_problem(sp)
+    if settings["export_buffers"]:
+        export_buffers(p, settings["export_buffers"])
+    if settings["buffer_prefix"]:
+        _, err = import_buffers(p, settings["buffer_prefix"])
+        if err:
+            return "FAILED", "", err
+    t_c0 = time.perf_counter()
     try:
         pd, prim, strm, args, dst = api_objects(p, want_ref_impl=sp.impl == "ref",
                                                 runtime_dims_masks=sp.runtime_dims_masks)
@@ -334,7 +466,8 @@ def run_spec(sp, mode="C", min_times=5, max_ms=300.0):
             return "SKIPPED", "", "unimplemented"
         return "FAILED", "", f"primitive descriptor: {e}"
     impl = pd.impl_info_str()
-    details = {}
+    # (the primitive descriptor and the primitive are created in one helper: their sum is what is timed)
+    details = {"cpd_ms": 0.0, "cp_ms": (time.perf_counter() - t_c0) * 1e3}
     if "C" in mode:
         from oracle import binding as oracle
         from tests.helpers import compare
@@ -370,17 +503,24 @@ def run_spec(sp, mode="C", min_times=5, max_ms=300.0):
             times.append((time.perf_counter() - t0) * 1e3 / 10)
             if len(times) >= 1000:
                 break
-        details["min_ms"], details["avg_ms"] = min(times), sum(times) / len(times)
-        details["gops"] = 2.0 * p.M * p.N * p.K / (min(times) * 1e-3) / 1e9
+        details["min_ms"], details["avg_ms"], details["max_ms"] = min(times), sum(times) / len(times), max(times)
+        details["ops"] = 2.0 * p.M * p.N * p.K
+        details["gops"] = details["ops"] / (min(times) * 1e-3) / 1e9
+        details["ibytes"] = float(sum(np.ascontiguousarray(getattr(h, a)).nbytes for h, a in buffer_ids(p).values()))
+        details["obytes"] = float(p.M * p.N * cabi.DT_BITS[p.dst_dt] // 8)
     return "PASSED", impl, details
 
 
 def main(argv):
-    mode, specs = parse(argv)
+    settings = dict(SETTINGS)
+    mode, specs = parse(argv, settings)
+    if (settings["buffer_prefix"] or settings["export_buffers"]) and len(specs) > 1:
+        print("--buffer-prefix / --export-buffers work with one test case at a time")
+        return 2
     failed = 0
     for i, sp in enumerate(specs):
         t0 = time.perf_counter()
-        status, impl, det = run_spec(sp, mode)
+        status, impl, det = run_spec(sp, mode, max_ms=float(settings["max_ms_per_prb"]), settings=settings)
         ms = (time.perf_counter() - t0) * 1e3
         if status == "FAILED":
             failed += 1
@@ -388,7 +528,7 @@ def main(argv):
             continue
         print(f"{i}:{status} ({ms:.0f} ms) __REPRO: {sp.repro()}")
         if status == "PASSED" and "P" in mode:
-            print(f"perf,gpu,{impl},{sp.repro()},{det['min_ms']:.4f},{det['avg_ms']:.4f},{det['gops']:.1f}")
+            print(perf_line(settings["perf_template"], sp, impl, det, i))
     print(f"tests:{len(specs)} passed:{len(specs) - failed} failed:{failed}")
     return 1 if failed else 0
 

@@ -1,6 +1,8 @@
 """The benchdnn-style driver: parsing and problem construction on the CPU, the
 reference's own input lines (tests/benchdnn/inputs/matmul/*, adapted to the
 supported knobs and shapes) on the GPU."""
+import os
+
 import numpy as np
 import pytest
 
@@ -116,3 +118,110 @@ def test_every_fast_family_is_reached_and_agrees_with_the_generic_kernel(gpu, or
         status, impl_ref, det = bd.run_spec(sp, "C")
         assert status == "PASSED" and impl_ref == "hip:ref:any", (sp.repro(), det)
     assert seen == {"mfma_i8", "mfma_f8", "woq_gemv"}
+
+
+# ---- buffers from files and the performance report (CPU: parsing, files, the oracle)
+C1_LINE = ("--matmul --dt=u8:s8:f32 --stag=ab --wtag=ab --dtag=ab --bia-dt=f32 --bia_mask=2 "
+           "--attr-scales=src:common:0.02+wei:per_oc --attr-zero-points=src:common:128 256x1024:1024x1024")
+
+
+def test_buffer_prefix_round_trip_reproduces_dst(tmp_path, oracle):
+    """--export-buffers writes PREFIX.<execution argument id>.bin for every filled
+    buffer of BASELINE's C1 line; --buffer-prefix on a problem generated from
+    another seed brings back the same bytes and the same dst (fill.cpp:489-543)."""
+    _, specs = bd.parse(C1_LINE.split())
+    assert len(specs) == 1
+    p = bd.build_problem(specs[0], seed=7)
+    prefix = str(tmp_path / "bufs" / "cfg1")
+    names = bd.export_buffers(p, prefix)
+    # src, weights, bias, src scale, weights scale, src zero point
+    assert sorted(int(n.split(".")[-2]) for n in names) == [1, 33, 41, 4097, 4129, 8193]
+    sizes = {int(n.split(".")[-2]): os.path.getsize(n) for n in names}
+    assert sizes == {1: 256 * 1024, 33: 1024 * 1024, 41: 4096, 4097: 4, 4129: 4096, 8193: 4}
+    want = oracle.run_oracle(p)
+
+    q = bd.build_problem(specs[0], seed=99)
+    assert not np.array_equal(q.src, p.src) and not np.array_equal(q.wei, p.wei)
+    done, err = bd.import_buffers(q, prefix)
+    assert err is None and done == [1, 33, 41, 4097, 4129, 8193]
+    for arg, (holder, attr) in bd.buffer_ids(q).items():
+        h0, a0 = bd.buffer_ids(p)[arg]
+        assert np.array_equal(np.asarray(getattr(holder, attr)).view(np.uint8).reshape(-1),
+                              np.asarray(getattr(h0, a0)).view(np.uint8).reshape(-1)), arg
+    got = oracle.run_oracle(q)
+    assert np.array_equal(np.asarray(got).view(np.uint32), np.asarray(want).view(np.uint32))
+
+
+def test_buffer_prefix_partial_and_mismatched_files(tmp_path):
+    _, specs = bd.parse("--dt=s8:s8:s32 --attr-post-ops=add:f32+sum 10x30:30x20".split())
+    p = bd.build_problem(specs[0])
+    prefix = str(tmp_path / "x")
+    names = bd.export_buffers(p, prefix)
+    # src, weights, dst (the sum's input), the tensor of binary post-op 0
+    assert sorted(int(n.split(".")[-2]) for n in names) == [1, 17, 33, 32770]
+    # only src present: the rest keeps the generated data
+    for n in names:
+        if not n.endswith(".1.bin"):
+            os.remove(n)
+    q = bd.build_problem(specs[0], seed=3)
+    wei_before = q.wei.copy()
+    done, err = bd.import_buffers(q, prefix)
+    assert err is None and done == [1]
+    assert np.array_equal(q.src, p.src) and np.array_equal(q.wei, wei_before)
+    # a file of the wrong size fails the case
+    with open(f"{prefix}.33.bin", "wb") as f:
+        f.write(b"\0" * 7)
+    done, err = bd.import_buffers(bd.build_problem(specs[0]), prefix)
+    assert err is not None and "differs in size" in err
+
+
+def test_run_wide_knobs_do_not_multiply_the_problem_list():
+    settings = dict(bd.SETTINGS)
+    mode, specs = bd.parse(("--mode=P --perf-template=perf,%engine%,%impl%,%prb%,%-time% --buffer-prefix=/tmp/a/b "
+                            "--max-ms-per-prb=50 --dt=u8:s8:f32,s8:s8:s32 10x30:30x20").split(), settings)
+    assert mode == "P" and len(specs) == 2
+    assert settings["buffer_prefix"] == "/tmp/a/b" and settings["max_ms_per_prb"] == "50"
+    assert settings["perf_template"] == "perf,%engine%,%impl%,%prb%,%-time%"
+
+
+def test_perf_template_fields_and_modifiers():
+    """doc/knobs_perf_report.md: BASELINE's template, the default one, time and unit modifiers."""
+    _, specs = bd.parse(C1_LINE.split())
+    sp = specs[0]
+    det = {"min_ms": 0.5, "avg_ms": 1.0, "max_ms": 2.0, "ops": 2.0 * 256 * 1024 * 1024, "ibytes": 3e6, "obytes": 1e6,
+           "cpd_ms": 1.5, "cp_ms": 2.5}
+    T = "perf,%engine%,%impl%,%prb%,%-time%,%0time%,%-Gflops%,%0Gflops%,%-Gbw%"
+    line = bd.perf_line(T, sp, "hip:mfma_i8:gfx950", det)
+    f = line.split(",")
+    assert f[:3] == ["perf", "gpu", "hip:mfma_i8:gfx950"]
+    assert f[3] == sp.repro() and "256x1024:1024x1024" in f[3]
+    assert [float(x) for x in f[4:]] == pytest.approx([0.5, 1.0, det["ops"] / 0.5e-3 / 1e9, det["ops"] / 1e-3 / 1e9,
+                                                       4e6 / 0.5e-3 / 1e9], rel=1e-5)
+    d = bd.perf_line("def", sp, "impl", det).split(",")
+    assert d[0] == "perf" and d[3] == "" and float(d[5]) == pytest.approx(det["ops"] / 1e9, rel=1e-5)
+    assert float(d[6]) == 4.0                                     # %+ctime%
+    assert bd.perf_line("%+time%|%Kops%|%Miobytes%|%driver%|%idx%|%wtag%|%unknown%", sp, "i", det, idx=4) == \
+        f"2|{det['ops'] / 1e3:g}|4|matmul|4|ab|%unknown%"
+
+
+@pytest.mark.gpu
+def test_main_with_buffer_files_and_a_custom_perf_template(gpu, oracle, tmp_path, capsys):
+    """BASELINE's C1 line end to end: export, then correctness + performance on
+    the imported bytes with BASELINE's report template."""
+    prefix = str(tmp_path / "cfg1")
+    assert bd.main(C1_LINE.split() + [f"--export-buffers={prefix}", "--mode=C"]) == 0
+    capsys.readouterr()
+    T = "--perf-template=perf,%engine%,%impl%,%prb%,%-time%,%0time%,%-Gflops%,%0Gflops%,%-Gbw%"
+    assert bd.main(C1_LINE.split() + [f"--buffer-prefix={prefix}", "--mode=CP", "--max-ms-per-prb=50", T]) == 0
+    out = capsys.readouterr().out.splitlines()
+    perf = [ln for ln in out if ln.startswith("perf,")]
+    assert len(perf) == 1
+    f = perf[0].split(",")
+    assert f[1] == "gpu" and f[2].startswith("hip:mfma_i8") and "256x1024:1024x1024" in f[3]
+    tmin, tavg, gmin, gavg, bw = (float(x) for x in f[-5:])
+    assert 0 < tmin <= tavg and gmin >= gavg > 0 and bw > 0
+    # a file of the wrong size fails the case
+    with open(f"{prefix}.1.bin", "ab") as fh:
+        fh.write(b"\0")
+    assert bd.main(C1_LINE.split() + [f"--buffer-prefix={prefix}", "--mode=C"]) == 1
+    assert "differs in size" in capsys.readouterr().out
