@@ -263,7 +263,8 @@ def test_hardware_fp8_conversions_match_the_software_ones_except_for_nans(gpu):
     # compares with the software conversions the oracle's restatement is pinned to
     import os
     import subprocess
-    tool = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "onednn_amd", "lib", "cvt_fp8_check")
+    tool = os.path.join(os.path.dirname(os.path.abspath(__file__)), "bin", "cvt_fp8_check")  # built by tests/Makefile
+    assert os.path.exists(tool), "build tests/bin/cvt_fp8_check first (make -C tests, or __graft_entry__.build())"
     out = subprocess.run([tool], capture_output=True, text=True, timeout=120)
     assert out.returncode == 0, out.stderr
     assert out.stdout.strip().splitlines()[-1] == "nan-only", out.stdout[-2000:]
