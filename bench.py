@@ -43,7 +43,7 @@ import numpy as np  # noqa: E402
 # in the JSON line can only be as old as the committed profile it names.
 PROFILE_OF = {
     ("c3", "any"): "i8_gemm_kernel_c3_8192.md", ("c4", "any"): "f8_gemm_kernel_c4_4096x8192x28672.md",
-    ("c5", "any"): "mxf4_gemm_kernel_c5_8192.md", ("c1", "any"): "i8_gemm_kernel_c1_256x1024x1024.md",
+    ("c5", "any"): "mxf4_gemm_kernel_c5_8192.md", ("c1", "any"): "i8_small_kernel_c1_256x1024x1024.md",
     ("c2", "any", 1): "woqp_kernel_c2_m1.md", ("c2", "any", 8): "woqp_kernel_c2_m8.md",
     ("c2", "any", 32): "woqp_kernel_c2_m32.md", ("c2", "ab", 1): "woq_gemv_kernel_c2_m1_plain_ab.md",
     ("c2", "ab", 8): "woq_gemv_kernel_c2_m8_plain_ab.md", ("c2", "ab", 32): "woq_gemv_kernel_c2_m32_plain_ab.md",
@@ -326,6 +326,9 @@ def main():
     ap.add_argument("--calib-read", action="store_true",
                     help="time a read-only kernel with the decode kernel's access shape over the C2 weights "
                          "(12 rotating copies, nothing cached) and exit: the floor of the weight stream")
+    ap.add_argument("--calib-mfma", action="store_true",
+                    help="time the MFMA instructions of the GEMM kernels by themselves (registers only), with random "
+                         "and with constant operand bits, and exit: the ceiling the power manager leaves")
     ap.add_argument("--calib-copy", action="store_true",
                     help="also launch the plain copy kernel on 256 MiB three times: the known-size "
                          "dispatch that FETCH_SIZE / WRITE_SIZE counter passes are scaled by")
@@ -373,6 +376,38 @@ def main():
         print(json.dumps({"metric": "read floor of the C2 weight stream", "value": nbytes / (ms * 1e-3) / 1e9,
                           "unit": "GB/s", "us_per_launch": ms * 1e3, "us_best": min(runs) * 1e3, "bytes": nbytes}),
               flush=True)
+        return
+
+    if args.calib_mfma:
+        names = ["v_mfma_i32_32x32x32_i8", "v_mfma_i32_16x16x64_i8", "v_mfma_f32_32x32x64_f8f6f4 (fp8)",
+                 "v_mfma_f32_16x16x128_f8f6f4 (fp8)", "v_mfma_scale_f32_32x32x64_f8f6f4 (fp4)",
+                 "v_mfma_scale_f32_16x16x128_f8f6f4 (fp4)"]
+        out = cabi.DeviceBuffer(1 << 20)
+        rng = np.random.default_rng(1)
+        rows = []
+        for instr, name in enumerate(names):
+            row = {"instruction": name}
+            for kind in ("random", "constant"):
+                h = rng.integers(0, 2**32, size=4096, dtype=np.uint64).astype(np.uint32) if kind == "random" \
+                    else np.full(4096, 0x01010101, np.uint32)
+                if "fp8" in name:     # finite, moderate values: clear sign and top exponent bit
+                    h &= np.uint32(0x3f3f3f3f)
+                bits = cabi.DeviceBuffer.from_numpy(h)
+                ops = C.c_double(0)
+                timer = Timer(lib)
+
+                def step():
+                    cabi.check(lib.mi355_mfma_rate_kernel(instr, 20000, out.ptr, bits.ptr, C.byref(ops), None))
+
+                step()
+                cabi.check(lib.mi355_stream_sync(None))
+                ms = min(timer.time_ms(step, 1) for _ in range(3))
+                row[kind] = ops.value / (ms * 1e-3) / 1e12
+                bits.free()
+            rows.append(row)
+            log(f"[bench] {name}: {row['random']:.0f} T(FL)OP/s with random operand bits, {row['constant']:.0f} with "
+                "constant ones")
+        print(json.dumps({"metric": "MFMA rate, registers only", "unit": "TOPS", "rows": rows}), flush=True)
         return
 
     def calib_copy():

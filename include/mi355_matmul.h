@@ -384,6 +384,15 @@ int mi355_copy_kernel(void *dst, const void *src, size_t bytes, void *stream);
  * itself.  `sink` holds 4 bytes per 128 KiB and is not written in practice. */
 int mi355_read_stream_kernel(const void *src, size_t bytes, void *sink, void *stream);
 
+/* Measures what an MFMA instruction of the GEMM kernels sustains by itself:
+ * 1024 workgroups x 4 wavefronts, operands and accumulators in registers, 8 or
+ * 16 independent accumulator chains, `iters` rounds.  instr: 0 i32_32x32x32_i8,
+ * 1 i32_16x16x64_i8, 2 f32_32x32x64 fp8, 3 f32_16x16x128 fp8, 4 f32_32x32x64
+ * fp4, 5 f32_16x16x128 fp4.  `bits`: 16 KiB of operand bits (their toggling
+ * decides the clock the power manager grants), `out`: 1 MiB.  *ops_per_launch
+ * receives the operation count to divide by the measured time. */
+int mi355_mfma_rate_kernel(int instr, int iters, void *out, const void *bits, double *ops_per_launch, void *stream);
+
 /* Evict caches between timed launches: streams `bytes` of `buf` through a
  * read-modify-write kernel so a following launch sees cold L2/MALL. */
 int mi355_flush_kernel(void *buf, size_t bytes, void *stream);

@@ -146,6 +146,82 @@ extern "C" int mi355_read_stream_kernel(const void *src, size_t bytes, void *sin
     return hipGetLastError() == hipSuccess ? MI355_SUCCESS : MI355_RUNTIME_ERROR;
 }
 
+namespace mi355 {
+// What the MFMA instructions of the GEMM kernels sustain when nothing else
+// limits them: operands and accumulators stay in registers, 4 wavefronts per
+// SIMD, 8 or 16 independent accumulator chains per wavefront.  The operand bits
+// come from memory once, so the caller decides how much they toggle (the clock
+// the power manager grants depends on it).
+enum { RATE_I8_32, RATE_I8_16, RATE_F8_32, RATE_F8_16, RATE_F4_32, RATE_F4_16, RATE_COUNT };
+
+template <int MODE>
+__global__ void __launch_bounds__(256) mfma_rate_kernel(int iters, int *out, const int *bits) {
+    typedef int v8i __attribute__((ext_vector_type(8)));
+    typedef int v16i __attribute__((ext_vector_type(16)));
+    typedef float v4f __attribute__((ext_vector_type(4)));
+    typedef float v16f __attribute__((ext_vector_type(16)));
+    const v8i *r8 = (const v8i *)bits;
+    const v8i a8 = r8[threadIdx.x * 2], b8 = r8[threadIdx.x * 2 + 1];
+    const v4i a = {a8[0], a8[1], a8[2], a8[3]}, b = {b8[0], b8[1], b8[2], b8[3]};
+    int result = 0;
+    if (MODE == RATE_I8_32) {
+        v16i c[8] = {};
+        for (int i = 0; i < iters; ++i)
+#pragma unroll
+            for (int j = 0; j < 8; ++j) c[j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a, b, c[j], 0, 0, 0);
+        for (int j = 0; j < 8; ++j) result += c[j][0];
+    } else if (MODE == RATE_I8_16) {
+        v4i c[16] = {};
+        for (int i = 0; i < iters; ++i)
+#pragma unroll
+            for (int j = 0; j < 16; ++j) c[j] = __builtin_amdgcn_mfma_i32_16x16x64_i8(a, b, c[j], 0, 0, 0);
+        for (int j = 0; j < 16; ++j) result += c[j][0];
+    } else if (MODE == RATE_F8_32 || MODE == RATE_F4_32) {
+        constexpr int fmt = MODE == RATE_F4_32 ? 4 : 0, sc = MODE == RATE_F4_32 ? 127 : 0;
+        v16f c[8] = {};
+        for (int i = 0; i < iters; ++i)
+#pragma unroll
+            for (int j = 0; j < 8; ++j)
+                c[j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(a8, b8, c[j], fmt, fmt, 0, sc, 0, sc);
+        for (int j = 0; j < 8; ++j) result += (int)c[j][0];
+    } else {
+        constexpr int fmt = MODE == RATE_F4_16 ? 4 : 0, sc = MODE == RATE_F4_16 ? 127 : 0;
+        v4f c[16] = {};
+        for (int i = 0; i < iters; ++i)
+#pragma unroll
+            for (int j = 0; j < 16; ++j)
+                c[j] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(a8, b8, c[j], fmt, fmt, 0, sc, 0, sc);
+        for (int j = 0; j < 16; ++j) result += (int)c[j][0];
+    }
+    out[blockIdx.x * 256 + threadIdx.x] = result;
+}
+} // namespace mi355
+
+extern "C" int mi355_mfma_rate_kernel(int instr, int iters, void *out, const void *bits, double *ops_per_launch,
+        void *stream) {
+    constexpr int blocks = 1024;
+    if (instr < 0 || instr >= RATE_COUNT || iters < 1 || !out || !bits) {
+        set_error("mfma rate kernel: instruction 0..5, out of 1 MiB, 16 KiB of operand bits");
+        return MI355_INVALID_ARGUMENTS;
+    }
+    static const double inst_ops[RATE_COUNT] = {2.0 * 32 * 32 * 32, 2.0 * 16 * 16 * 64, 2.0 * 32 * 32 * 64,
+            2.0 * 16 * 16 * 128, 2.0 * 32 * 32 * 64, 2.0 * 16 * 16 * 128};
+    static const int chains[RATE_COUNT] = {8, 16, 8, 16, 8, 16};
+    if (ops_per_launch) *ops_per_launch = (double)blocks * 4 * iters * chains[instr] * inst_ops[instr];
+    hipStream_t s = (hipStream_t)stream;
+    int *o = (int *)out;
+    const int *bp = (const int *)bits;
+    switch (instr) {
+        case RATE_I8_32: hipLaunchKernelGGL(mfma_rate_kernel<RATE_I8_32>, dim3(blocks), dim3(256), 0, s, iters, o, bp); break;
+        case RATE_I8_16: hipLaunchKernelGGL(mfma_rate_kernel<RATE_I8_16>, dim3(blocks), dim3(256), 0, s, iters, o, bp); break;
+        case RATE_F8_32: hipLaunchKernelGGL(mfma_rate_kernel<RATE_F8_32>, dim3(blocks), dim3(256), 0, s, iters, o, bp); break;
+        case RATE_F8_16: hipLaunchKernelGGL(mfma_rate_kernel<RATE_F8_16>, dim3(blocks), dim3(256), 0, s, iters, o, bp); break;
+        case RATE_F4_32: hipLaunchKernelGGL(mfma_rate_kernel<RATE_F4_32>, dim3(blocks), dim3(256), 0, s, iters, o, bp); break;
+        default: hipLaunchKernelGGL(mfma_rate_kernel<RATE_F4_16>, dim3(blocks), dim3(256), 0, s, iters, o, bp); break;
+    }
+    return hipGetLastError() == hipSuccess ? MI355_SUCCESS : MI355_RUNTIME_ERROR;
+}
+
 extern "C" int mi355_flush_kernel(void *buf, size_t bytes, void *stream) {
     if (bytes % 16 || ((uintptr_t)buf & 15)) {
         set_error("flush kernel needs a 16-byte aligned pointer and size");

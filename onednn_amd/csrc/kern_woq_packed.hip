@@ -352,12 +352,17 @@ __global__ void __launch_bounds__(NWV * 64)
                 for (int tt = 0; tt < 4; ++tt) acc[mt][tt] = v4f {0.f, 0.f, 0.f, 0.f};
             }
         }
+        // (the lane's weights address is rebuilt here: kept from the prologue it
+        // is spilled to scratch memory across the main loop)
+        int lane_again = lane;
+        asm volatile("" : "+v"(lane_again));
+        const uint8_t *wlane_tail = X.wei + (long)chunk * K * (CHUNK / 2) + lane_again * 16;
 #pragma unroll 1
         for (; kb < kb1; ++kb) {
             v4u a1[MT];
 #pragma unroll
             for (int mt = 0; mt < MT; ++mt) a1[mt] = *(const v4u *)(X.src + (long)kb * (KBLK * 2) + src_lane_off[mt]);
-            const v4u w1 = __builtin_nontemporal_load((const v4u *)(wlane + (long)kb * (KBLK * CHUNK / 2)));
+            const v4u w1 = __builtin_nontemporal_load((const v4u *)(wlane_tail + (long)kb * (KBLK * CHUNK / 2)));
             compute_step(w1, a1, false);
             if ((kb + 1) % X.spg == 0 || kb + 1 == kb1) {
                 unsigned word_s, word_z;
