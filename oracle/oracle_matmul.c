@@ -54,9 +54,17 @@
  * dst codes against a nearest-value search over the type's codes.
  * The ternary select post-op is pinned by tests/test_oracle_matmul.py (numpy
  * `where` on exact integer sums, three condition types).
- * Unpinned: none of the functions used by the five benchmark configurations;
- * the libm-dependent eltwise algorithms other than relu/gelu_tanh/linear/tanh
- * are "parity unpinned" beyond their textbook formula.
+ * Precomputed reductions (orc_int8_dot with src_pr, grouped / per-tensor src
+ * zero points, true and arbitrary sums), prelu with every weights layout the
+ * reference derives, every eltwise and every binary algorithm are pinned by
+ * tests/test_oracle_pins.py against closed-form numpy expectations (the
+ * formula in f32 with the reference's intermediate roundings; nstl::max / min
+ * NaN semantics).
+ * Unpinned: none of the functions used by the five benchmark configurations.
+ * "Parity unpinned" beyond the textbook formula: the last bits of the
+ * libm-dependent eltwise algorithms (tanh, elu, exp, log, pow, gelu_erf,
+ * soft_relu, mish, swish, logistic): they agree with float64 evaluations to a
+ * few ulp, the reference's own libm bits cannot be pinned without running it.
  */
 #include <limits.h>
 #include <math.h>
