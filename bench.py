@@ -17,7 +17,7 @@ object: the headline metric of the chosen workload plus
   others        the remaining benchmark configurations, measured the same way
                 with fewer steps (informational)
 
-Workloads (BASELINE.json configs):
+Workloads (the benchmark configurations):
   c3  s8 x s8 -> s8, M=N=K=8192, scales + ReLU (MFMA int8 bound)      [default]
   c2  bf16 x u4 -> bf16 decode, K=4096 N=14336, M in {1,8,32} (HBM bound)
   c4  e4m3 x e4m3 -> bf16, 4096 x 8192 x 28672, bias+gelu+add (MFMA fp8 bound)

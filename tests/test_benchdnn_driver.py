@@ -127,7 +127,7 @@ C1_LINE = ("--matmul --dt=u8:s8:f32 --stag=ab --wtag=ab --dtag=ab --bia-dt=f32 -
 
 def test_buffer_prefix_round_trip_reproduces_dst(tmp_path, oracle):
     """--export-buffers writes PREFIX.<execution argument id>.bin for every filled
-    buffer of BASELINE's C1 line; --buffer-prefix on a problem generated from
+    buffer of the u8 x s8 -> f32 benchmark line (256x1024:1024x1024); --buffer-prefix on a problem generated from
     another seed brings back the same bytes and the same dst (fill.cpp:489-543)."""
     _, specs = bd.parse(C1_LINE.split())
     assert len(specs) == 1
@@ -185,7 +185,7 @@ def test_run_wide_knobs_do_not_multiply_the_problem_list():
 
 
 def test_perf_template_fields_and_modifiers():
-    """doc/knobs_perf_report.md: BASELINE's template, the default one, time and unit modifiers."""
+    """doc/knobs_perf_report.md: a custom template, the default one, time and unit modifiers."""
     _, specs = bd.parse(C1_LINE.split())
     sp = specs[0]
     det = {"min_ms": 0.5, "avg_ms": 1.0, "max_ms": 2.0, "ops": 2.0 * 256 * 1024 * 1024, "ibytes": 3e6, "obytes": 1e6,
@@ -206,8 +206,8 @@ def test_perf_template_fields_and_modifiers():
 
 @pytest.mark.gpu
 def test_main_with_buffer_files_and_a_custom_perf_template(gpu, oracle, tmp_path, capsys):
-    """BASELINE's C1 line end to end: export, then correctness + performance on
-    the imported bytes with BASELINE's report template."""
+    """The 256x1024:1024x1024 benchmark line end to end: export, then correctness + performance on
+    the imported bytes with a custom report template."""
     prefix = str(tmp_path / "cfg1")
     assert bd.main(C1_LINE.split() + [f"--export-buffers={prefix}", "--mode=C"]) == 0
     capsys.readouterr()
