@@ -374,6 +374,72 @@ int mi355_reorder_launch(const mi355_reorder_desc_t *desc,
 int mi355_wei_pack_reorder_dims(int packing, int64_t K, int64_t N,
         int64_t src_stride_k, int64_t src_stride_n, mi355_reorder_desc_t *desc);
 
+/* ---- grouped matmul (mixture-of-experts): one matmul per group over tensors
+ * that concatenate the groups along one dimension, the group boundaries being
+ * run-time data on the device.  Replaces ref_grouped_t
+ * (src/cpu/matmul/ref_grouped_gemm.cpp:39-440; descriptor rules
+ * src/common/matmul.cpp:43-259, ref_grouped_gemm.hpp:60-270):
+ *   MI355_GROUPED_2DX3D  src [total_M][K] row-major, grouped along M;
+ *                        weights dense [G][K][N] (any strides); dst
+ *                        [total_M][N] row-major, grouped like src; optional
+ *                        bias [G][N]; scales / zero points / post-ops below
+ *   MI355_GROUPED_2DX2D  src [M][total_K] column-major, grouped along K;
+ *                        weights [total_K][N] row-major, grouped like src; dst
+ *                        dense [G][M][N] (any strides); same floating-point
+ *                        type everywhere, nothing else
+ * offsets[g] = end of group g along the variable dimension (cumulative, s32,
+ * device memory); group g starts at offsets[g - 1] (0 for g = 0).
+ * Quantization parameters (2DX3D): src scales / zero points per row,
+ * [total_M] or [total_M][K / gk]; weights scales / zero points per group and
+ * column, [G][N] or [G][K / gk][N]; gk = 0: no groups along K. */
+#define MI355_GROUPED_2DX3D 0
+#define MI355_GROUPED_2DX2D 1
+
+typedef struct mi355_grouped_post_op {
+    int32_t kind;  /* MI355_PO_ELTWISE or MI355_PO_BINARY (multiplication only) */
+    int32_t alg;
+    float alpha, beta, scale;
+    int32_t dt;          /* binary: data type of the operand */
+    int64_t bin_m, bin_n; /* binary: operand dims, [G][1], [total_M][1] or [total_M][N], dense row-major */
+    int32_t grouped;     /* binary: the operand is a grouped tensor with offsets of its own */
+} mi355_grouped_post_op_t;
+
+typedef struct mi355_grouped_desc {
+    int32_t pattern; /* MI355_GROUPED_* */
+    int64_t group_count;
+    int64_t total;   /* total_M (2DX3D) or total_K (2DX2D) */
+    int64_t M;       /* 2DX2D: rows of every group; 2DX3D: unused */
+    int64_t K;       /* 2DX3D: depth of every group; 2DX2D: unused */
+    int64_t N;
+    int32_t src_dt, wei_dt, dst_dt, bias_dt; /* bias_dt UNDEF = no bias */
+    int64_t wei_stride[3]; /* 2DX3D: element strides of [G][K][N] */
+    int64_t dst_stride[3]; /* 2DX2D: element strides of [G][M][N] */
+    int32_t src_scale_dt, wei_scale_dt, src_zp_dt, wei_zp_dt; /* UNDEF = absent */
+    int64_t src_scale_gk, wei_scale_gk, src_zp_gk, wei_zp_gk;
+    int32_t fpmath_apply_to_int;
+    int32_t n_post_ops;
+    mi355_grouped_post_op_t post_ops[MI355_MAX_POST_OPS];
+} mi355_grouped_desc_t;
+
+typedef struct mi355_grouped_args {
+    const void *src, *wei, *bias;
+    void *dst;
+    const int32_t *src_offsets, *wei_offsets, *dst_offsets; /* wei: 2DX2D; dst: 2DX3D */
+    const void *src_scale, *wei_scale, *src_zp, *wei_zp;
+    const void *po_arg[MI355_MAX_POST_OPS];
+    const int32_t *po_offsets[MI355_MAX_POST_OPS]; /* grouped binary operands */
+} mi355_grouped_args_t;
+
+/* MI355_SUCCESS if the one implementation ("hip:ref_grouped:any", a thread per
+ * dst element in the reference's operation order) takes the problem. */
+int mi355_grouped_matmul_query(const mi355_grouped_desc_t *desc);
+
+/* Asynchronous on `stream`; no scratch.  The offsets are not validated (they
+ * live on the device): rows outside every group are left untouched, a group
+ * whose src and dst ranges differ in length computes the rows both have, and
+ * no access leaves the tensors whatever the offsets hold. */
+int mi355_grouped_matmul_launch(const mi355_grouped_desc_t *desc, const mi355_grouped_args_t *args, void *stream);
+
 /* Plain device-to-device copy kernel (one 16-byte load + store per lane), used
  * to calibrate the FETCH_SIZE / WRITE_SIZE counters against a known size. */
 int mi355_copy_kernel(void *dst, const void *src, size_t bytes, void *stream);

@@ -82,6 +82,38 @@ class MatmulArgs(C.Structure):
     ]
 
 
+class GroupedPostOp(C.Structure):
+    """mi355_grouped_post_op_t"""
+    _fields_ = [("kind", C.c_int32), ("alg", C.c_int32), ("alpha", C.c_float), ("beta", C.c_float),
+                ("scale", C.c_float), ("dt", C.c_int32), ("bin_m", C.c_int64), ("bin_n", C.c_int64),
+                ("grouped", C.c_int32)]
+
+
+class GroupedDesc(C.Structure):
+    """mi355_grouped_desc_t"""
+    _fields_ = [
+        ("pattern", C.c_int32), ("group_count", C.c_int64), ("total", C.c_int64), ("M", C.c_int64),
+        ("K", C.c_int64), ("N", C.c_int64),
+        ("src_dt", C.c_int32), ("wei_dt", C.c_int32), ("dst_dt", C.c_int32), ("bias_dt", C.c_int32),
+        ("wei_stride", C.c_int64 * 3), ("dst_stride", C.c_int64 * 3),
+        ("src_scale_dt", C.c_int32), ("wei_scale_dt", C.c_int32), ("src_zp_dt", C.c_int32), ("wei_zp_dt", C.c_int32),
+        ("src_scale_gk", C.c_int64), ("wei_scale_gk", C.c_int64), ("src_zp_gk", C.c_int64), ("wei_zp_gk", C.c_int64),
+        ("fpmath_apply_to_int", C.c_int32), ("n_post_ops", C.c_int32),
+        ("post_ops", GroupedPostOp * MAX_POST_OPS),
+    ]
+
+
+class GroupedArgs(C.Structure):
+    """mi355_grouped_args_t"""
+    _fields_ = [
+        ("src", C.c_void_p), ("wei", C.c_void_p), ("bias", C.c_void_p), ("dst", C.c_void_p),
+        ("src_offsets", C.c_void_p), ("wei_offsets", C.c_void_p), ("dst_offsets", C.c_void_p),
+        ("src_scale", C.c_void_p), ("wei_scale", C.c_void_p), ("src_zp", C.c_void_p), ("wei_zp", C.c_void_p),
+        ("po_arg", C.c_void_p * MAX_POST_OPS), ("po_offsets", C.c_void_p * MAX_POST_OPS),
+    ]
+
+
+GROUPED_2DX3D, GROUPED_2DX2D = 0, 1
 REORDER_MAX_DIMS = 6
 
 
@@ -113,7 +145,8 @@ KERNEL_SYMBOLS = [
     "mi355_stream_wait_event", "mi355_mem_store_scalar",
     "mi355_last_error", "mi355_matmul_query", "mi355_matmul_impl_name",
     "mi355_matmul_scratch_bytes", "mi355_matmul_launch", "mi355_matmul_launch_noalloc", "mi355_reorder_query",
-    "mi355_reorder_launch", "mi355_wei_pack_reorder_dims", "mi355_copy_kernel", "mi355_flush_kernel", "mi355_read_stream_kernel", "mi355_mfma_rate_kernel",
+    "mi355_reorder_launch", "mi355_wei_pack_reorder_dims", "mi355_copy_kernel", "mi355_flush_kernel", "mi355_read_stream_kernel", "mi355_mfma_rate_kernel", "mi355_grouped_matmul_query",
+    "mi355_grouped_matmul_launch",
 ]
 
 _PKG_DIR = os.path.dirname(os.path.abspath(__file__))
@@ -172,6 +205,8 @@ def load_kernels():
     lib.mi355_wei_pack_reorder_dims.argtypes = [C.c_int, C.c_int64, C.c_int64, C.c_int64, C.c_int64,
                                                 C.POINTER(ReorderDesc)]
     lib.mi355_copy_kernel.argtypes = [vp, vp, C.c_size_t, vp]
+    lib.mi355_grouped_matmul_query.argtypes = [C.POINTER(GroupedDesc)]
+    lib.mi355_grouped_matmul_launch.argtypes = [C.POINTER(GroupedDesc), C.POINTER(GroupedArgs), vp]
     lib.mi355_read_stream_kernel.argtypes = [vp, C.c_size_t, vp, vp]
     lib.mi355_mfma_rate_kernel.argtypes = [C.c_int, C.c_int, vp, vp, C.POINTER(C.c_double), vp]
     lib.mi355_flush_kernel.argtypes = [vp, C.c_size_t, vp]

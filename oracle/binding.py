@@ -205,3 +205,27 @@ def reorder(prob):
     st = lib.oracle_reorder(C.byref(d), C.byref(a))
     assert st == 0
     return dst
+
+
+def run_oracle_grouped(prob):
+    """Grouped matmul (onednn_amd.grouped.GroupedProblem) on the CPU: returns
+    (status, raw dst bytes); the status is the reference's verdict on the
+    offsets (ref_grouped_gemm.cpp:169-212)."""
+    from onednn_amd import grouped
+    lib = load()
+    lib.oracle_grouped_matmul.argtypes = [C.POINTER(cabi.GroupedDesc), C.POINTER(cabi.GroupedArgs)]
+    lib.oracle_grouped_matmul.restype = C.c_int
+    keep = []
+
+    def place(arr):
+        arr = np.ascontiguousarray(arr)
+        keep.append(arr)
+        return arr.ctypes.data
+
+    d = prob.desc()
+    a = grouped.fill_args(prob, place)
+    dst = prob.initial_dst()
+    a.dst = dst.ctypes.data
+    st = lib.oracle_grouped_matmul(C.byref(d), C.byref(a))
+    del keep
+    return st, dst

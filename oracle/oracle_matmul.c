@@ -743,3 +743,123 @@ int oracle_reorder(const mi355_reorder_desc_t *d, const mi355_reorder_args_t *a)
     }
     return 0;
 }
+
+/* ------------------------------------------------------------- grouped matmul
+ * ref_grouped_t::execute, src/cpu/matmul/ref_grouped_gemm.cpp:39-440 -- the
+ * offsets validation (:169-212, MI355_INVALID_ARGUMENTS) and the per-group
+ * loops (:215-440) in the reference's operation order.  All pointers are host
+ * pointers.  Pinned by tests/test_grouped_matmul.py: per-group numpy matmuls on
+ * exact data (integer, decompression, fp with power-of-two scales), empty
+ * groups, an empty K range that still writes zeros, every binary operand
+ * shape, and the offsets the reference refuses. */
+int oracle_grouped_matmul(const mi355_grouped_desc_t *d, const mi355_grouped_args_t *a) {
+    const int64_t G = d->group_count, N = d->N;
+    const int x2 = d->pattern == MI355_GROUPED_2DX2D;
+    for (int64_t g = 0; g < G; ++g) {
+        if (x2) {
+            const int64_t k0 = g == 0 ? 0 : a->src_offsets[g - 1], k1 = a->src_offsets[g];
+            if (a->wei_offsets[g] != k1 || (g > 0 && a->wei_offsets[g - 1] != k0) || k0 < 0 || k1 > d->total || k1 < k0)
+                return MI355_INVALID_ARGUMENTS;
+        } else {
+            const int64_t s0 = g == 0 ? 0 : a->src_offsets[g - 1], s1 = a->src_offsets[g];
+            const int64_t d0 = g == 0 ? 0 : a->dst_offsets[g - 1], d1 = a->dst_offsets[g];
+            if (s0 < 0 || s1 > d->total || s1 < s0 || d0 < 0 || d1 > d->total || d1 < d0) return MI355_INVALID_ARGUMENTS;
+            for (int i = 0; i < d->n_post_ops; ++i) {
+                const mi355_grouped_post_op_t *po = &d->post_ops[i];
+                if (po->kind != MI355_PO_BINARY || !po->grouped) continue;
+                const int64_t b0 = g > 0 ? a->po_offsets[i][g - 1] : 0, b1 = a->po_offsets[i][g];
+                if (b0 < 0 || b1 > po->bin_m || b1 < b0 || b0 != d0 || b1 != d1) return MI355_INVALID_ARGUMENTS;
+            }
+        }
+    }
+    const int int_src = d->src_dt == MI355_DT_S8 || d->src_dt == MI355_DT_U8;
+    const int int_wei = d->wei_dt == MI355_DT_S8 || d->wei_dt == MI355_DT_U8 || d->wei_dt == MI355_DT_S4
+            || d->wei_dt == MI355_DT_U4;
+    const int woq = !int_src && int_wei && d->fpmath_apply_to_int;
+    const int64_t Kf = x2 ? 0 : d->K;
+#define ORC_NG(dt, gk) ((dt) != MI355_DT_UNDEF && (gk) > 1 ? Kf / (gk) : 1)
+    const int64_t ss_ng = ORC_NG(d->src_scale_dt, d->src_scale_gk), ws_ng = ORC_NG(d->wei_scale_dt, d->wei_scale_gk);
+    const int64_t sz_ng = ORC_NG(d->src_zp_dt, d->src_zp_gk), wz_ng = ORC_NG(d->wei_zp_dt, d->wei_zp_gk);
+#undef ORC_NG
+    int64_t nkg = 1;
+    if (!x2) {
+        nkg = ss_ng > ws_ng ? ss_ng : ws_ng;
+        nkg = sz_ng > nkg ? sz_ng : nkg;
+        nkg = wz_ng > nkg ? wz_ng : nkg;
+    }
+#pragma omp parallel for schedule(dynamic)
+    for (int64_t g = 0; g < G; ++g) {
+        int64_t Mg, Kg, src_start, dst_row0 = 0;
+        /* element strides of the inner matmul and the groups' bases (:58-88) */
+        int64_t s_sm, s_sk, w_sk, w_sn, d_sm, d_sn, src_base, wei_base, dst_base;
+        if (x2) {
+            const int64_t k0 = g == 0 ? 0 : a->src_offsets[g - 1];
+            Mg = d->M; Kg = a->src_offsets[g] - k0; src_start = k0;
+            s_sm = 1; s_sk = d->M; w_sk = N; w_sn = 1; d_sm = d->dst_stride[1]; d_sn = d->dst_stride[2];
+            src_base = k0 * d->M; wei_base = k0 * N; dst_base = g * d->dst_stride[0];
+        } else {
+            const int64_t s0 = g == 0 ? 0 : a->src_offsets[g - 1];
+            dst_row0 = g == 0 ? 0 : a->dst_offsets[g - 1];
+            Mg = a->src_offsets[g] - s0; Kg = d->K; src_start = s0;
+            s_sm = d->K; s_sk = 1; w_sk = d->wei_stride[1]; w_sn = d->wei_stride[2]; d_sm = N; d_sn = 1;
+            src_base = s0 * d->K; wei_base = g * d->wei_stride[0]; dst_base = dst_row0 * N;
+        }
+        if (Mg == 0) continue;
+        const int64_t kgs = Kg / nkg;
+        for (int64_t m = 0; m < Mg; ++m)
+            for (int64_t n = 0; n < N; ++n) {
+                float result = 0.0f;
+                for (int64_t ig = 0; ig < nkg; ++ig) {
+                    float acc = 0.0f;
+                    if (int_src || woq) {
+                        int zs = 0, zw = 0;
+                        float wsc = 1.0f;
+                        if (d->src_zp_dt != MI355_DT_UNDEF)
+                            zs = orc_load_int(d->src_zp_dt, a->src_zp, (src_start + m) * sz_ng + ig * sz_ng / nkg);
+                        if (d->wei_scale_dt != MI355_DT_UNDEF)
+                            wsc = orc_load_float(d->wei_scale_dt, a->wei_scale, g * ws_ng * N + (ig * ws_ng / nkg) * N + n);
+                        if (d->wei_zp_dt != MI355_DT_UNDEF)
+                            zw = orc_load_int(d->wei_zp_dt, a->wei_zp, g * wz_ng * N + (ig * wz_ng / nkg) * N + n);
+                        if (int_src) {
+                            int acc_int = 0;
+                            for (int64_t k = ig * kgs; k < (ig + 1) * kgs; ++k)
+                                acc_int += (orc_load_int(d->src_dt, a->src, src_base + m * s_sm + k * s_sk) - zs)
+                                        * (orc_load_int(d->wei_dt, a->wei, wei_base + k * w_sk + n * w_sn) - zw);
+                            acc = (float)acc_int;
+                        } else {
+                            for (int64_t k = ig * kgs; k < (ig + 1) * kgs; ++k)
+                                acc += orc_load_float(d->src_dt, a->src, src_base + m * s_sm + k * s_sk)
+                                        * (float)(orc_load_int(d->wei_dt, a->wei, wei_base + k * w_sk + n * w_sn) - zw);
+                        }
+                        if (d->src_scale_dt != MI355_DT_UNDEF)
+                            acc *= orc_load_float(d->src_scale_dt, a->src_scale, (src_start + m) * ss_ng + ig * ss_ng / nkg);
+                        result += acc * wsc;
+                    } else {
+                        for (int64_t k = ig * kgs; k < (ig + 1) * kgs; ++k)
+                            acc += orc_load_float(d->src_dt, a->src, src_base + m * s_sm + k * s_sk)
+                                    * orc_load_float(d->wei_dt, a->wei, wei_base + k * w_sk + n * w_sn);
+                        if (d->src_scale_dt != MI355_DT_UNDEF)
+                            acc *= orc_load_float(d->src_scale_dt, a->src_scale, (src_start + m) * ss_ng + ig * ss_ng / nkg);
+                        if (d->wei_scale_dt != MI355_DT_UNDEF)
+                            acc *= orc_load_float(d->wei_scale_dt, a->wei_scale, g * ws_ng * N + (ig * ws_ng / nkg) * N + n);
+                        result += acc;
+                    }
+                }
+                if (d->bias_dt != MI355_DT_UNDEF) result += orc_load_float(d->bias_dt, a->bias, g * N + n);
+                for (int i = 0; i < d->n_post_ops; ++i) {
+                    const mi355_grouped_post_op_t *po = &d->post_ops[i];
+                    if (po->kind == MI355_PO_ELTWISE) {
+                        result = orc_eltwise(po->alg, result, po->alpha, po->beta) * po->scale;
+                    } else {
+                        int64_t row_base = dst_row0;
+                        if (po->grouped) row_base = g > 0 ? a->po_offsets[i][g - 1] : 0;
+                        const int per_group = po->bin_m == G && po->bin_n == 1;
+                        const int64_t em = per_group ? g : row_base + m, en = po->bin_n > 1 ? n : 0;
+                        result = orc_binary(po->alg, result, orc_load_float(po->dt, a->po_arg[i], em * po->bin_n + en));
+                    }
+                }
+                orc_store_float(d->dst_dt, result, a->dst, dst_base + m * d_sm + n * d_sn);
+            }
+    }
+    return MI355_SUCCESS;
+}
