@@ -107,7 +107,7 @@ typedef enum {
     dnnl_format_kind_any,
     dnnl_blocked,
     dnnl_format_kind_opaque,
-    dnnl_format_kind_sparse,     /* declared for the enum values only: not offered */
+    dnnl_format_kind_sparse,     /* the grouped encoding only (dnnl_memory_desc_create_with_grouped_encoding) */
     dnnl_format_kind_host_scalar /* one value that lives in the memory object itself, on the host */
 } dnnl_format_kind_t;
 
@@ -204,8 +204,21 @@ typedef enum {
     dnnl_query_ndims_s32 = 256,
     dnnl_query_dims = 257,
     dnnl_query_data_type = 258,
-    dnnl_query_format_kind = 262
+    dnnl_query_format_kind = 262,
+    dnnl_query_sparse_encoding = 266,
+    dnnl_query_nnz_s64 = 267,
+    dnnl_query_num_handles_s32 = 268
 } dnnl_query_t;
+
+/* dnnl_sparse_encoding_t of include/oneapi/dnnl/dnnl_types.h:67-88 with
+ * DNNL_EXPERIMENTAL_GROUPED_MEMORY; only dnnl_grouped is offered. */
+typedef enum {
+    dnnl_sparse_encoding_undef = 0,
+    dnnl_csr,
+    dnnl_packed,
+    dnnl_coo,
+    dnnl_grouped
+} dnnl_sparse_encoding_t;
 
 /* execute argument ids, dnnl_types.h:2544-2784 */
 #define DNNL_ARG_SRC 1
@@ -261,6 +274,20 @@ dnnl_status_t dnnl_memory_desc_create_with_tag(dnnl_memory_desc_t *memory_desc, 
 dnnl_status_t dnnl_memory_desc_clone(dnnl_memory_desc_t *memory_desc, const_dnnl_memory_desc_t existing);
 dnnl_status_t dnnl_memory_desc_destroy(dnnl_memory_desc_t memory_desc);
 dnnl_status_t dnnl_memory_desc_query(const_dnnl_memory_desc_t memory_desc, dnnl_query_t what, void *result);
+
+/* Grouped memory (mixture-of-experts): a 2-D tensor that concatenates
+ * `group_count` sub-tensors along dims[variable_dim_idx] (index 0: row-major
+ * storage, index 1: column-major), with a second buffer of s32 cumulative
+ * group ends.  include/oneapi/dnnl/dnnl.h:1155-1193 (experimental in the
+ * reference, always present here); src/common/memory_desc.cpp:417-472.
+ * A matmul takes grouped src + dense 3-D weights + grouped dst (variable M) or
+ * grouped src + grouped weights + dense 3-D dst (variable K):
+ * src/common/matmul.cpp:43-259. */
+dnnl_status_t dnnl_memory_desc_create_with_grouped_encoding(dnnl_memory_desc_t *memory_desc, int ndims,
+        const dnnl_dims_t dims, dnnl_data_type_t data_type, int variable_dim_idx, dnnl_dim_t group_count,
+        dnnl_data_type_t offsets_dt);
+/* size of buffer `index` (0 values, 1 offsets); dnnl.h:1453 */
+size_t dnnl_memory_desc_get_size_v2(const_dnnl_memory_desc_t memory_desc, int index);
 int dnnl_memory_desc_equal(const_dnnl_memory_desc_t lhs, const_dnnl_memory_desc_t rhs);
 size_t dnnl_memory_desc_get_size(const_dnnl_memory_desc_t memory_desc);
 size_t dnnl_data_type_size(dnnl_data_type_t data_type);
@@ -280,6 +307,14 @@ dnnl_status_t dnnl_memory_map_data(const_dnnl_memory_t memory, void **mapped_ptr
 dnnl_status_t dnnl_memory_unmap_data(const_dnnl_memory_t memory, void *mapped_ptr);
 dnnl_status_t dnnl_memory_get_data_handle(const_dnnl_memory_t memory, void **handle);
 dnnl_status_t dnnl_memory_set_data_handle(dnnl_memory_t memory, void *handle);
+/* Memory objects over several buffers (dnnl.h:1503, :1591, :1627, :1660, :1672):
+ * a grouped tensor has two, the values (index 0) and the s32 offsets (index 1). */
+dnnl_status_t dnnl_memory_create_v2(dnnl_memory_t *memory, const_dnnl_memory_desc_t memory_desc, dnnl_engine_t engine,
+        int nhandles, void **handles);
+dnnl_status_t dnnl_memory_map_data_v2(const_dnnl_memory_t memory, void **mapped_ptr, int index);
+dnnl_status_t dnnl_memory_unmap_data_v2(const_dnnl_memory_t memory, void *mapped_ptr, int index);
+dnnl_status_t dnnl_memory_get_data_handle_v2(const_dnnl_memory_t memory, void **handle, int index);
+dnnl_status_t dnnl_memory_set_data_handle_v2(dnnl_memory_t memory, void *handle, int index);
 dnnl_status_t dnnl_memory_destroy(dnnl_memory_t memory);
 
 /* ---- attributes: dnnl.h:340-720 ---- */

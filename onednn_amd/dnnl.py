@@ -143,6 +143,61 @@ class memory_desc:
         return v.value
 
 
+class grouped_memory_desc(memory_desc):
+    """dnnl_memory_desc_create_with_grouped_encoding: dims [total_M][K] with
+    variable_dim_idx 0 (row-major) or [M][total_K] with 1 (column-major)."""
+
+    def __init__(self, dims, dt, variable_dim_idx, group_count, offsets_dt=None):
+        self.h = C.c_void_p()
+        self.owned = True
+        st = lib().dnnl_memory_desc_create_with_grouped_encoding(
+            C.byref(self.h), len(dims), _dims(dims), dt, variable_dim_idx, C.c_int64(group_count),
+            cabi.DT_S32 if offsets_dt is None else offsets_dt)
+        _check(st, "memory_desc_create_with_grouped_encoding")
+
+    def get_size(self, index=0):
+        lib().dnnl_memory_desc_get_size_v2.restype = C.c_size_t
+        return lib().dnnl_memory_desc_get_size_v2(self.h, index)
+
+    def num_handles(self):
+        v = C.c_int32()
+        _check(lib().dnnl_memory_desc_query(self.h, 268, C.byref(v)), "md_query")
+        return v.value
+
+
+class grouped_memory:
+    """A grouped tensor on the device: values and the groups' cumulative ends (s32)."""
+
+    def __init__(self, md, eng, values=None, offsets=None):
+        self.md, self.engine = md, eng
+        self.h = C.c_void_p()
+        handles = (C.c_void_p * 2)(MEMORY_ALLOCATE, MEMORY_ALLOCATE)
+        _check(lib().dnnl_memory_create_v2(C.byref(self.h), md.h, eng.h, 2, handles), "memory_create_v2")
+        if values is not None:
+            self.write(values, 0)
+        if offsets is not None:
+            self.write(np.asarray(offsets, np.int32), 1)
+
+    def write(self, data, index=0):
+        data = np.ascontiguousarray(data)
+        p = C.c_void_p()
+        _check(lib().dnnl_memory_map_data_v2(self.h, C.byref(p), index), "memory_map_data_v2")
+        assert data.nbytes <= self.md.get_size(index), (data.nbytes, self.md.get_size(index))
+        if data.nbytes:
+            C.memmove(p, data.ctypes.data, data.nbytes)
+        _check(lib().dnnl_memory_unmap_data_v2(self.h, p, index), "memory_unmap_data_v2")
+
+    def read(self, dtype, index=0):
+        p = C.c_void_p()
+        _check(lib().dnnl_memory_map_data_v2(self.h, C.byref(p), index), "memory_map_data_v2")
+        n = self.md.get_size(index)
+        out = np.empty(n // np.dtype(dtype).itemsize, dtype=dtype)
+        if n:
+            C.memmove(out.ctypes.data, p, n)
+        _check(lib().dnnl_memory_unmap_data_v2(self.h, p, index), "memory_unmap_data_v2")
+        return out
+
+
 class host_scalar:
     """dnnl::memory of a host-side scalar (dnnl_memory_create_host_scalar): the
     value lives in the object; `value` is a numpy scalar of the storage type."""

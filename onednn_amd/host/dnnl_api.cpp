@@ -103,6 +103,12 @@ struct dnnl_memory_desc {
     // kind == dnnl_format_kind_opaque: the weights packing (MI355_WEI_PACK_*)
     // that format_tag::any resolved to; strides are meaningless then
     int packing = 0;
+    // kind == dnnl_format_kind_sparse: the grouped encoding (memory_desc.cpp:417-472) -- a 2-D tensor that
+    // concatenates `group_count` sub-tensors along dims[var_dim], the variable dim outermost in memory
+    // (strides say so); a second buffer holds the groups' cumulative ends (s32)
+    bool grouped = false;
+    int var_dim = 0;
+    dim_t group_count = 0;
 
     bool is_zero() const { return ndims == 0; }
     // a dim or a stride left open until execution (memory_desc_wrapper::has_runtime_dims_or_strides)
@@ -127,6 +133,7 @@ struct dnnl_memory_desc {
     size_t size_bytes() const {
         if (has_runtime()) return DNNL_RUNTIME_SIZE_VAL; // memory_desc_wrapper::size, src/common/memory.cpp:62
         if (kind == dnnl_format_kind_opaque) return (size_t)nelems() * dt_bits(dt) / 8; // dense, no padding
+        if (grouped) return ((size_t)nelems() * dt_bits(dt) + 7) / 8;                  // the values buffer
         const dim_t s = span();
         return dt_bits(dt) == 4 ? (size_t)(s + 1) / 2 : (size_t)s * (dt_bits(dt) / 8);
     }
@@ -147,6 +154,7 @@ struct dnnl_memory_desc {
     }
     bool operator==(const dnnl_memory_desc &o) const {
         if (ndims != o.ndims || dt != o.dt || kind != o.kind || packing != o.packing) return false;
+        if (grouped != o.grouped || (grouped && (var_dim != o.var_dim || group_count != o.group_count))) return false;
         for (int i = 0; i < ndims; ++i)
             if (dims[i] != o.dims[i] || (kind == dnnl_blocked && strides[i] != o.strides[i])) return false;
         return true;
@@ -159,6 +167,10 @@ struct dnnl_memory {
     void *handle = nullptr;
     bool owned = false;
     void *mapped = nullptr; // host staging buffer while mapped
+    // grouped encoding: buffer 1, the offsets
+    void *handle2 = nullptr;
+    bool owned2 = false;
+    void *mapped2 = nullptr;
     unsigned char scalar[8] = {}; // md.kind == dnnl_format_kind_host_scalar: the value
 };
 
@@ -213,6 +225,8 @@ struct dnnl_primitive_desc {
     bool with_bias = false;
     dnnl_primitive_attr attr;
     mi355_matmul_desc_t desc;     // impl field = the chosen kernel family
+    bool grouped = false;         // grouped (mixture-of-experts) matmul: `gdesc` instead of `desc`
+    mi355_grouped_desc_t gdesc;
     std::vector<int> impls;       // kernel families that can run it, best first
     size_t impl_pos = 0;
     size_t scratch_bytes = 0;
@@ -467,6 +481,7 @@ dnnl_status_t check_attr(const dnnl_memory_desc &s, const dnnl_memory_desc &w, c
             CHECK_UNIMPL(IMPLICATION(e.dt != dnnl_data_type_undef, dt_bits(e.dt) == dt_bits(dst_dt)));
             CHECK_UNIMPL(IMPLICATION(e.zero_point != 0, src_int8));
         }
+        if (e.kind == dnnl_binary) CHECK_UNIMPL(!e.src1.grouped); // grouped operands: grouped matmul only
         if (e.kind == dnnl_binary) {
             CHECK_ARG(e.src1.ndims == d.ndims);
             for (int i = 0; i < d.ndims; ++i)
@@ -940,6 +955,35 @@ DNNL_EXPORT dnnl_status_t dnnl_memory_desc_create_with_tag(dnnl_memory_desc_t *m
     *memory_desc = md.release();
     return dnnl_success;
 }
+// memory_desc_init_with_grouped_encoding, src/common/memory_desc.cpp:417-472
+DNNL_EXPORT dnnl_status_t dnnl_memory_desc_create_with_grouped_encoding(dnnl_memory_desc_t *memory_desc, int ndims,
+        const dnnl_dims_t dims, dnnl_data_type_t data_type, int variable_dim_idx, dnnl_dim_t group_count,
+        dnnl_data_type_t offsets_dt) {
+    CHECK_ARG(memory_desc);
+    std::unique_ptr<dnnl_memory_desc> md(new dnnl_memory_desc);
+    if (ndims == 0) {
+        *memory_desc = md.release();
+        return dnnl_success;
+    }
+    CHECK_UNIMPL(ndims == 2);
+    CHECK_ARG(dims && dt_valid(data_type));
+    CHECK_ARG(group_count > 0);
+    CHECK_ARG(offsets_dt == dnnl_s32);
+    CHECK_ARG(variable_dim_idx >= 0 && variable_dim_idx < ndims);
+    for (int d = 0; d < ndims; ++d) CHECK_ARG(dims[d] != DNNL_RUNTIME_DIM_VAL && dims[d] > 0);
+    md->ndims = ndims;
+    md->dt = data_type;
+    for (int d = 0; d < ndims; ++d) md->dims[d] = dims[d];
+    md->kind = dnnl_format_kind_sparse;
+    md->grouped = true;
+    md->var_dim = variable_dim_idx;
+    md->group_count = group_count;
+    // the variable dim is the outermost one: idx 0 -> row-major, idx 1 -> column-major
+    md->strides[variable_dim_idx] = dims[1 - variable_dim_idx];
+    md->strides[1 - variable_dim_idx] = 1;
+    *memory_desc = md.release();
+    return dnnl_success;
+}
 DNNL_EXPORT dnnl_status_t dnnl_memory_desc_clone(dnnl_memory_desc_t *memory_desc, const_dnnl_memory_desc_t existing) {
     CHECK_ARG(memory_desc && existing);
     *memory_desc = new dnnl_memory_desc(*existing);
@@ -960,6 +1004,11 @@ DNNL_EXPORT dnnl_status_t dnnl_memory_desc_query(const_dnnl_memory_desc_t md, dn
             if (md->kind != dnnl_blocked) return dnnl_invalid_arguments;
             *(const dnnl_dims_t **)result = &md->strides;
             break;
+        case dnnl_query_sparse_encoding:
+            *(dnnl_sparse_encoding_t *)result = md->grouped ? dnnl_grouped : dnnl_sparse_encoding_undef;
+            break;
+        case dnnl_query_nnz_s64: *(int64_t *)result = md->grouped ? md->nelems() : 0; break;
+        case dnnl_query_num_handles_s32: *(int32_t *)result = md->grouped ? 2 : 1; break; // memory_desc.cpp:1096
         default: return dnnl_unimplemented;
     }
     return dnnl_success;
@@ -971,8 +1020,16 @@ DNNL_EXPORT int dnnl_memory_desc_equal(const_dnnl_memory_desc_t lhs, const_dnnl_
 }
 DNNL_EXPORT size_t dnnl_memory_desc_get_size(const_dnnl_memory_desc_t md) {
     if (md && md->kind == dnnl_format_kind_host_scalar) return dt_bits(md->dt) / 8;
+    if (md && md->grouped) return md->size_bytes();
     if (!md || (md->kind != dnnl_blocked && md->kind != dnnl_format_kind_opaque)) return 0;
     return md->size_bytes();
+}
+// buffer `index` of a descriptor: a grouped tensor has the values (0) and the s32 offsets (1)
+DNNL_EXPORT size_t dnnl_memory_desc_get_size_v2(const_dnnl_memory_desc_t md, int index) {
+    if (!md || index < 0) return 0;
+    if (index == 0) return dnnl_memory_desc_get_size(md);
+    if (md->grouped && index == 1) return (size_t)md->group_count * sizeof(int32_t);
+    return 0;
 }
 DNNL_EXPORT size_t dnnl_data_type_size(dnnl_data_type_t dt) {
     return dt_bits(dt) / 8 ? dt_bits(dt) / 8 : 1;
@@ -985,6 +1042,7 @@ DNNL_EXPORT dnnl_status_t dnnl_memory_create(dnnl_memory_t *memory, const_dnnl_m
     CHECK_ARG(md->kind != dnnl_format_kind_any);
     CHECK_ARG(!md->has_runtime()); // src/common/memory.cpp:155
     CHECK_ARG(md->kind != dnnl_format_kind_host_scalar); // :157, dnnl_memory_create_host_scalar makes those
+    CHECK_ARG(md->kind != dnnl_format_kind_sparse || md->grouped);
     std::unique_ptr<dnnl_memory> m(new dnnl_memory);
     m->md = *md;
     m->engine = engine;
@@ -998,6 +1056,80 @@ DNNL_EXPORT dnnl_status_t dnnl_memory_create(dnnl_memory_t *memory, const_dnnl_m
     }
     *memory = m.release();
     return dnnl_success;
+}
+// A memory object over several buffers (src/common/memory.cpp: dnnl_memory_create_v2): only the grouped encoding
+// has more than one here.  DNNL_MEMORY_ALLOCATE in a slot lets the library own that buffer.
+DNNL_EXPORT dnnl_status_t dnnl_memory_create_v2(dnnl_memory_t *memory, const_dnnl_memory_desc_t md, dnnl_engine_t engine,
+        int nhandles, void **handles) {
+    CHECK_ARG(memory && md && engine && handles);
+    const int need = md->grouped ? 2 : 1;
+    CHECK_ARG(nhandles == need);
+    dnnl_status_t st = dnnl_memory_create(memory, md, engine, handles[0]);
+    if (st != dnnl_success || need == 1) return st;
+    dnnl_memory *m = *memory;
+    if (handles[1] == DNNL_MEMORY_ALLOCATE) {
+        const int rc = mi355_mem_alloc(&m->handle2, dnnl_memory_desc_get_size_v2(md, 1));
+        if (rc != MI355_SUCCESS) {
+            dnnl_memory_destroy(m);
+            *memory = nullptr;
+            return from_mi355(rc);
+        }
+        m->owned2 = true;
+    } else {
+        m->handle2 = handles[1];
+    }
+    return dnnl_success;
+}
+DNNL_EXPORT dnnl_status_t dnnl_memory_get_data_handle_v2(const_dnnl_memory_t memory, void **handle, int index) {
+    CHECK_ARG(memory && handle);
+    if (index == 0) return dnnl_memory_get_data_handle(memory, handle);
+    CHECK_ARG(memory->md.grouped && index == 1);
+    *handle = memory->handle2;
+    return dnnl_success;
+}
+DNNL_EXPORT dnnl_status_t dnnl_memory_set_data_handle_v2(dnnl_memory_t memory, void *handle, int index) {
+    CHECK_ARG(memory);
+    if (index == 0) return dnnl_memory_set_data_handle(memory, handle);
+    CHECK_ARG(memory->md.grouped && index == 1);
+    if (memory->owned2) {
+        mi355_mem_free(memory->handle2);
+        memory->owned2 = false;
+    }
+    memory->handle2 = handle;
+    return dnnl_success;
+}
+DNNL_EXPORT dnnl_status_t dnnl_memory_map_data_v2(const_dnnl_memory_t cmemory, void **mapped_ptr, int index) {
+    if (index == 0) return dnnl_memory_map_data(cmemory, mapped_ptr);
+    CHECK_ARG(cmemory && mapped_ptr);
+    dnnl_memory *memory = const_cast<dnnl_memory *>(cmemory);
+    CHECK_ARG(memory->md.grouped && index == 1 && !memory->mapped2);
+    const size_t bytes = dnnl_memory_desc_get_size_v2(&memory->md, 1);
+    if (!memory->handle2) {
+        *mapped_ptr = nullptr;
+        return dnnl_success;
+    }
+    void *host = malloc(bytes);
+    if (!host) return dnnl_out_of_memory;
+    const int st = mi355_mem_d2h(host, memory->handle2, bytes, nullptr);
+    if (st != MI355_SUCCESS) {
+        free(host);
+        return from_mi355(st);
+    }
+    memory->mapped2 = host;
+    *mapped_ptr = host;
+    return dnnl_success;
+}
+DNNL_EXPORT dnnl_status_t dnnl_memory_unmap_data_v2(const_dnnl_memory_t cmemory, void *mapped_ptr, int index) {
+    if (index == 0) return dnnl_memory_unmap_data(cmemory, mapped_ptr);
+    CHECK_ARG(cmemory);
+    dnnl_memory *memory = const_cast<dnnl_memory *>(cmemory);
+    CHECK_ARG(memory->md.grouped && index == 1);
+    if (!memory->mapped2) return mapped_ptr ? dnnl_invalid_arguments : dnnl_success;
+    CHECK_ARG(mapped_ptr == memory->mapped2);
+    const int st = mi355_mem_h2d(memory->handle2, memory->mapped2, dnnl_memory_desc_get_size_v2(&memory->md, 1), nullptr);
+    free(memory->mapped2);
+    memory->mapped2 = nullptr;
+    return from_mi355(st);
 }
 // src/common/memory.cpp:219-241, :303-333
 DNNL_EXPORT dnnl_status_t dnnl_memory_desc_create_host_scalar(dnnl_memory_desc_t *memory_desc, dnnl_data_type_t data_type) {
@@ -1096,6 +1228,8 @@ DNNL_EXPORT dnnl_status_t dnnl_memory_destroy(dnnl_memory_t memory) {
     if (memory) {
         if (memory->mapped) free(memory->mapped);
         if (memory->owned) mi355_mem_free(memory->handle);
+        if (memory->mapped2) free(memory->mapped2);
+        if (memory->owned2) mi355_mem_free(memory->handle2);
         delete memory;
     }
     return dnnl_success;
@@ -1313,7 +1447,8 @@ DNNL_EXPORT dnnl_status_t dnnl_post_ops_append_binary(dnnl_post_ops_t post_ops, 
         const_dnnl_memory_desc_t src1_desc) {
     CHECK_ARG(post_ops && src1_desc);
     CHECK_ARG(alg >= dnnl_binary_add && alg <= dnnl_binary_ne);
-    CHECK_ARG(src1_desc->kind == dnnl_blocked || src1_desc->kind == dnnl_format_kind_any);
+    // (a grouped operand belongs to a grouped matmul: matmul.cpp:221-231)
+    CHECK_ARG(src1_desc->kind == dnnl_blocked || src1_desc->kind == dnnl_format_kind_any || src1_desc->grouped);
     if (po_full(post_ops)) return dnnl_out_of_memory;
     post_op_entry_t e;
     e.kind = dnnl_binary; e.alg = alg; e.src1 = *src1_desc;
@@ -1375,12 +1510,193 @@ DNNL_EXPORT dnnl_status_t dnnl_post_ops_get_params_prelu(const_dnnl_post_ops_t p
 }
 
 // ---- matmul primitive descriptor
+// ---- grouped (mixture-of-experts) matmul: descriptor rules of grouped_matmul_desc_init and
+// grouped_matmul_attr_check (src/common/matmul.cpp:43-259) and the dispatch rules of ref_grouped_t::pd_t::init
+// (src/cpu/matmul/ref_grouped_gemm.hpp:60-270), lowered to mi355_grouped_desc_t.
+namespace {
+bool is_tag_3d(const dnnl_memory_desc &m, bool acb) {
+    if (m.kind != dnnl_blocked || m.ndims != 3) return false;
+    const dim_t G = m.dims[0], K = m.dims[1], N = m.dims[2];
+    (void)G;
+    return acb ? (m.strides[0] == K * N && m.strides[1] == 1 && m.strides[2] == K)
+               : (m.strides[0] == K * N && m.strides[1] == N && m.strides[2] == 1);
+}
+
+dnnl_status_t grouped_pd_init(dnnl_primitive_desc &pd, const dnnl_memory_desc &src, const dnnl_memory_desc &wei,
+        const dnnl_memory_desc *bias, const dnnl_memory_desc &dst_in) {
+    for (const dnnl_memory_desc *m : {&src, &wei, &dst_in}) CHECK_ARG(m->kind != dnnl_format_kind_host_scalar);
+    if (bias) CHECK_ARG(bias->kind != dnnl_format_kind_host_scalar);
+    CHECK_UNIMPL(src.grouped);
+    const bool x3 = dst_in.grouped && !wei.grouped, x2 = wei.grouped && !dst_in.grouped;
+    CHECK_UNIMPL(x3 || x2);
+    const dnnl_memory_desc &variant = x3 ? dst_in : wei;
+    CHECK_UNIMPL(src.var_dim == (x3 ? 0 : 1) && variant.var_dim == 0);
+    CHECK_UNIMPL(src.group_count == variant.group_count);
+    const dim_t G = src.group_count;
+    CHECK_UNIMPL(src.ndims == 2);
+    CHECK_UNIMPL(wei.ndims == (x3 ? 3 : 2));
+    CHECK_UNIMPL(dst_in.ndims == (x3 ? 2 : 3));
+    CHECK_UNIMPL((x3 ? wei.dims[0] : dst_in.dims[0]) == G);
+    CHECK_UNIMPL(src.dims[0] == dst_in.dims[dst_in.ndims - 2]);
+    CHECK_UNIMPL(src.dims[1] == wei.dims[wei.ndims - 2]);
+    CHECK_UNIMPL(dst_in.dims[dst_in.ndims - 1] == wei.dims[wei.ndims - 1]);
+    const dim_t N = wei.dims[wei.ndims - 1];
+    dnnl_memory_desc dst = dst_in;
+    if (x3) {
+        CHECK_UNIMPL(is_tag_3d(wei, false) || is_tag_3d(wei, true)); // dense abc or acb
+        if (bias) {
+            CHECK_UNIMPL(!bias->grouped && bias->kind == dnnl_blocked && bias->ndims == 2);
+            CHECK_UNIMPL(bias->dims[0] == G && bias->dims[1] == N);
+            CHECK_UNIMPL(bias->strides[0] == N && bias->strides[1] == 1);
+        }
+    } else {
+        CHECK_UNIMPL(!bias);
+        if (dst.kind == dnnl_format_kind_any) dst.set_dense();
+        CHECK_UNIMPL(dst.kind == dnnl_blocked);
+    }
+    CHECK_UNIMPL(accum_dt(src.dt, wei.dt, dst.dt) != dnnl_data_type_undef);
+
+    mi355_grouped_desc_t &D = pd.gdesc;
+    memset(&D, 0, sizeof(D));
+    D.pattern = x3 ? MI355_GROUPED_2DX3D : MI355_GROUPED_2DX2D;
+    D.group_count = G;
+    D.total = x3 ? src.dims[0] : src.dims[1];
+    D.M = x3 ? 0 : src.dims[0];
+    D.K = x3 ? src.dims[1] : 0;
+    D.N = N;
+    D.src_dt = src.dt; D.wei_dt = wei.dt; D.dst_dt = dst.dt;
+    D.bias_dt = bias ? (int)bias->dt : MI355_DT_UNDEF;
+    if (x3) for (int i = 0; i < 3; ++i) D.wei_stride[i] = wei.strides[i];
+    else for (int i = 0; i < 3; ++i) D.dst_stride[i] = dst.strides[i];
+
+    // ---- attributes (grouped_matmul_attr_check, then the implementation's own rules)
+    const dnnl_primitive_attr &a = pd.attr;
+    const bool defaults = a.scales.empty() && a.zero_points.empty() && a.reductions.empty() && a.post_ops.entries.empty()
+            && a.fpmath == dnnl_fpmath_mode_strict && !a.apply_to_int && a.acc_mode == dnnl_accumulation_mode_strict;
+    if (!defaults) {
+        CHECK_UNIMPL(x3); // the variable-K pattern takes default attributes only
+        CHECK_UNIMPL(a.reductions.empty() && a.acc_mode == dnnl_accumulation_mode_strict);
+        auto fp_plain = [](int dt) { return dt == dnnl_f32 || dt == dnnl_bf16 || dt == dnnl_f16; };
+        const quant_entry_t *ss = a.find(a.scales, DNNL_ARG_SRC), *ws = a.find(a.scales, DNNL_ARG_WEIGHTS);
+        const quant_entry_t *sz = a.find(a.zero_points, DNNL_ARG_SRC), *wz = a.find(a.zero_points, DNNL_ARG_WEIGHTS);
+        CHECK_UNIMPL(IMPLICATION(fp_plain(src.dt), !ss));
+        CHECK_UNIMPL(IMPLICATION(fp_plain(wei.dt), !ws));
+        CHECK_UNIMPL(!a.find(a.scales, DNNL_ARG_DST) && !a.find(a.zero_points, DNNL_ARG_DST));
+        for (const auto &kv : a.scales) CHECK_UNIMPL(!kv.second.is_dynamic() && !kv.second.on_host);
+        for (const auto &kv : a.zero_points) CHECK_UNIMPL(!kv.second.on_host);
+        const dim_t K = D.K;
+        auto scale_dt_ok = [](int dt) {
+            return dt == dnnl_f32 || dt == dnnl_bf16 || dt == dnnl_f16 || dt == dnnl_e8m0 || dt == dnnl_f8_e4m3
+                    || dt == dnnl_f8_e5m2;
+        };
+        // src: per row (mask M) or per row and K group (mask M|K, groups {1, gK}); weights [G][K][N]: per group and
+        // column (mask G|N) or with K groups (mask G|K|N, groups {gK, 1})
+        auto src_entry = [&](const quant_entry_t *q, int64_t *gk) -> dnnl_status_t {
+            *gk = 0;
+            if (!q) return dnnl_success;
+            CHECK_UNIMPL(q->mask == 1 || q->mask == 3);
+            if (q->group_ndims != 0) {
+                CHECK_UNIMPL(q->group(0) == 1 && q->group(1) > 1 && K % q->group(1) == 0);
+                *gk = q->group(1);
+            }
+            CHECK_UNIMPL((q->mask == 3) == (*gk > 1));
+            return dnnl_success;
+        };
+        auto wei_entry = [&](const quant_entry_t *q, int64_t *gk) -> dnnl_status_t {
+            *gk = 0;
+            if (!q) return dnnl_success;
+            CHECK_UNIMPL(q->mask == 5 || q->mask == 7);
+            if (q->group_ndims != 0) {
+                CHECK_UNIMPL(q->group(0) > 1 && K % q->group(0) == 0 && q->group(1) == 1);
+                *gk = q->group(0);
+            }
+            CHECK_UNIMPL((q->mask == 7) == (*gk > 1));
+            return dnnl_success;
+        };
+        dnnl_status_t st;
+        if ((st = src_entry(ss, &D.src_scale_gk)) || (st = wei_entry(ws, &D.wei_scale_gk))
+                || (st = src_entry(sz, &D.src_zp_gk)) || (st = wei_entry(wz, &D.wei_zp_gk)))
+            return st;
+        if (ss) CHECK_UNIMPL(scale_dt_ok(ss->dt));
+        if (ws) CHECK_UNIMPL(scale_dt_ok(ws->dt));
+        if (sz) CHECK_UNIMPL(is_int8(src.dt) && (sz->dt == dnnl_u8 || sz->dt == dnnl_s8 || sz->dt == dnnl_s32));
+        if (wz)
+            CHECK_UNIMPL((is_int8(wei.dt) || wei.dt == dnnl_s4 || wei.dt == dnnl_u4)
+                    && (wz->dt == dnnl_u8 || wz->dt == dnnl_s8 || wz->dt == dnnl_u4 || wz->dt == dnnl_s4
+                            || wz->dt == dnnl_s32));
+        if (D.src_scale_gk > 1 && D.wei_scale_gk > 1)
+            CHECK_UNIMPL(D.src_scale_gk % D.wei_scale_gk == 0 || D.wei_scale_gk % D.src_scale_gk == 0);
+        if (ws && wz) CHECK_UNIMPL((ws->group_ndims ? ws->group(0) : 1) == (wz->group_ndims ? wz->group(0) : 1));
+        D.src_scale_dt = ss ? (int)ss->dt : MI355_DT_UNDEF;
+        D.wei_scale_dt = ws ? (int)ws->dt : MI355_DT_UNDEF;
+        D.src_zp_dt = sz ? (int)sz->dt : MI355_DT_UNDEF;
+        D.wei_zp_dt = wz ? (int)wz->dt : MI355_DT_UNDEF;
+        D.fpmath_apply_to_int = a.apply_to_int;
+        // post-ops: eltwise, and multiplication by a per-group, per-row or per-element operand
+        CHECK_UNIMPL(a.post_ops.entries.size() <= MI355_MAX_POST_OPS);
+        const dim_t total_M = dst.dims[0];
+        for (size_t i = 0; i < a.post_ops.entries.size(); ++i) {
+            const post_op_entry_t &e = a.post_ops.entries[i];
+            mi355_grouped_post_op_t &po = D.post_ops[i];
+            CHECK_UNIMPL(e.kind == dnnl_eltwise || e.kind == dnnl_binary);
+            if (e.kind == dnnl_eltwise) {
+                po.kind = MI355_PO_ELTWISE;
+                po.alg = e.alg; po.alpha = e.alpha; po.beta = e.beta; po.scale = e.scale;
+                continue;
+            }
+            CHECK_UNIMPL(e.alg == dnnl_binary_mul);
+            CHECK_ARG(e.src1.ndims == dst.ndims);
+            po.kind = MI355_PO_BINARY;
+            po.alg = e.alg;
+            po.dt = e.src1.dt;
+            po.bin_m = e.src1.dims[0];
+            po.bin_n = e.src1.dims[1];
+            if (e.src1.grouped) {
+                CHECK_UNIMPL(e.src1.group_count == dst.group_count && e.src1.var_dim == dst.var_dim);
+                CHECK_UNIMPL(po.bin_m == total_M && (po.bin_n == N || po.bin_n == 1));
+                po.grouped = 1;
+            } else {
+                dnnl_memory_desc b = e.src1;
+                if (b.kind == dnnl_format_kind_any) b.set_dense();
+                CHECK_UNIMPL(b.kind == dnnl_blocked);
+                CHECK_UNIMPL(po.bin_n == 1 || (b.strides[0] == po.bin_n && b.strides[1] == 1));
+                CHECK_UNIMPL((po.bin_m == G || po.bin_m == total_M) && IMPLICATION(po.bin_m == G, po.bin_n == 1));
+                CHECK_UNIMPL(po.bin_n == 1 || po.bin_n == N);
+            }
+        }
+        D.n_post_ops = (int)a.post_ops.entries.size();
+    }
+    CHECK_UNIMPL(mi355_grouped_matmul_query(&D) == MI355_SUCCESS);
+    pd.grouped = true;
+    pd.src = src; pd.wei = wei; pd.dst = dst;
+    pd.with_bias = bias != nullptr;
+    if (bias) pd.bias = *bias;
+    pd.impl_name = "hip:ref_grouped:any";
+    pd.impls.assign(1, MI355_IMPL_REF);
+    pd.impl_pos = 0;
+    pd.scratch_bytes = 0;
+    return dnnl_success;
+}
+} // namespace
+
 DNNL_EXPORT dnnl_status_t dnnl_matmul_primitive_desc_create(dnnl_primitive_desc_t *primitive_desc,
         dnnl_engine_t engine, const_dnnl_memory_desc_t src_desc, const_dnnl_memory_desc_t weights_desc,
         const_dnnl_memory_desc_t bias_desc, const_dnnl_memory_desc_t dst_desc, const_dnnl_primitive_attr_t attr) {
     CHECK_ARG(primitive_desc && engine);
     CHECK_ARG(src_desc && weights_desc && dst_desc);
     const dnnl_memory_desc *bias = (bias_desc && !bias_desc->is_zero()) ? bias_desc : nullptr;
+    if (src_desc->kind == dnnl_format_kind_sparse || weights_desc->kind == dnnl_format_kind_sparse
+            || dst_desc->kind == dnnl_format_kind_sparse) {
+        std::unique_ptr<dnnl_primitive_desc> gpd(new dnnl_primitive_desc);
+        if (attr) gpd->attr = *attr;
+        gpd->engine = engine;
+        const dnnl_status_t gs = grouped_pd_init(*gpd, *src_desc, *weights_desc, bias, *dst_desc);
+        if (gs) return gs;
+        if (verbose_level() >= 1)
+            fprintf(stderr, "onednn_verbose,v1,primitive,create:dispatch,gpu,matmul,%s\n", gpd->impl_name.c_str());
+        *primitive_desc = gpd.release();
+        return dnnl_success;
+    }
     dnnl_status_t st = check_shapes(*src_desc, *weights_desc, bias, *dst_desc);
     if (st) return st;
     CHECK_ARG(accum_dt(src_desc->dt, weights_desc->dt, dst_desc->dt) != dnnl_data_type_undef);
@@ -1742,6 +2058,56 @@ DNNL_EXPORT dnnl_status_t dnnl_primitive_execute(const_dnnl_primitive_t cprimiti
             const double ms = std::chrono::duration<double, std::milli>(std::chrono::steady_clock::now() - t0).count();
             fprintf(stderr, "onednn_verbose,v1,primitive,exec,gpu,reorder,%s,undef,src:%s dst:%s,,,%g\n",
                     pd.impl_name.c_str(), dt_name(pd.src.dt), dt_name(pd.dst.dt), ms);
+        }
+        return from_mi355(rc);
+    }
+    if (pd.grouped) {
+        // values in buffer 0, the groups' cumulative ends in buffer 1 of the grouped memory objects
+        mi355_grouped_args_t GA;
+        memset(&GA, 0, sizeof(GA));
+        auto mem_of = [&](int arg) -> dnnl_memory_t {
+            auto it = m.find(arg);
+            return it == m.end() ? nullptr : it->second;
+        };
+        dnnl_memory_t ms = mem_of(DNNL_ARG_SRC), mw = mem_of(DNNL_ARG_WEIGHTS), md = mem_of(DNNL_ARG_DST);
+        CHECK_ARG(ms && mw && md && ms->md.grouped);
+        const bool x3 = pd.gdesc.pattern == MI355_GROUPED_2DX3D;
+        CHECK_ARG(x3 ? md->md.grouped : mw->md.grouped);
+        GA.src = ms->handle; GA.wei = mw->handle; GA.dst = md->handle;
+        GA.src_offsets = (const int32_t *)ms->handle2;
+        if (x3) GA.dst_offsets = (const int32_t *)md->handle2;
+        else GA.wei_offsets = (const int32_t *)mw->handle2;
+        void *q = nullptr;
+        dnnl_status_t gs;
+        if ((gs = handle(DNNL_ARG_BIAS, pd.with_bias, &q))) return gs;
+        GA.bias = q;
+        if ((gs = handle(DNNL_ARG_ATTR_SCALES | DNNL_ARG_SRC, pd.gdesc.src_scale_dt != MI355_DT_UNDEF, &q))) return gs;
+        GA.src_scale = q;
+        if ((gs = handle(DNNL_ARG_ATTR_SCALES | DNNL_ARG_WEIGHTS, pd.gdesc.wei_scale_dt != MI355_DT_UNDEF, &q))) return gs;
+        GA.wei_scale = q;
+        if ((gs = handle(DNNL_ARG_ATTR_ZERO_POINTS | DNNL_ARG_SRC, pd.gdesc.src_zp_dt != MI355_DT_UNDEF, &q))) return gs;
+        GA.src_zp = q;
+        if ((gs = handle(DNNL_ARG_ATTR_ZERO_POINTS | DNNL_ARG_WEIGHTS, pd.gdesc.wei_zp_dt != MI355_DT_UNDEF, &q))) return gs;
+        GA.wei_zp = q;
+        for (int i = 0; i < pd.gdesc.n_post_ops; ++i) {
+            if (pd.gdesc.post_ops[i].kind != MI355_PO_BINARY) continue;
+            dnnl_memory_t mb = mem_of(DNNL_ARG_ATTR_MULTIPLE_POST_OP(i) | DNNL_ARG_SRC_1);
+            CHECK_ARG(mb && mb->handle);
+            GA.po_arg[i] = mb->handle;
+            if (pd.gdesc.post_ops[i].grouped) {
+                CHECK_ARG(mb->md.grouped && mb->handle2);
+                GA.po_offsets[i] = (const int32_t *)mb->handle2;
+            }
+        }
+        if (mi355_device_set((int)pd.engine->index) != MI355_SUCCESS) return dnnl_runtime_error;
+        const auto t0 = std::chrono::steady_clock::now();
+        const int rc = mi355_grouped_matmul_launch(&pd.gdesc, &GA, stream->hip_stream);
+        if (verbose_level() >= 2) {
+            mi355_stream_sync(stream->hip_stream);
+            const double ms_ = std::chrono::duration<double, std::milli>(std::chrono::steady_clock::now() - t0).count();
+            fprintf(stderr, "onednn_verbose,v1,primitive,exec,gpu,matmul,%s,undef,src:%s wei:%s dst:%s,,grouped:%ld,%g\n",
+                    pd.impl_name.c_str(), dt_name(pd.src.dt), dt_name(pd.wei.dt), dt_name(pd.dst.dt),
+                    (long)pd.gdesc.group_count, ms_);
         }
         return from_mi355(rc);
     }
