@@ -430,14 +430,28 @@ typedef struct mi355_grouped_args {
     const int32_t *po_offsets[MI355_MAX_POST_OPS]; /* grouped binary operands */
 } mi355_grouped_args_t;
 
-/* MI355_SUCCESS if the one implementation ("hip:ref_grouped:any", a thread per
- * dst element in the reference's operation order) takes the problem. */
+/* MI355_SUCCESS if an implementation takes the problem:
+ *   "hip:mfma_grouped"     2DX3D on the matrix cores: fp8 x fp8 (e4m3 / e5m2 in
+ *                          any pairing), bf16 x bf16 or f16 x f16 with
+ *                          K-contiguous weights ([G][N][K], wei_stride[1] == 1,
+ *                          16-byte aligned rows, K a multiple of 32 bytes),
+ *                          scales without groups along K, no zero points; bias
+ *                          and every post-op of the list.  f32 accumulation in
+ *                          the order of the hardware.
+ *   "hip:ref_grouped:any"  everything else the descriptor rules allow: a thread
+ *                          per dst element in the reference's operation order.
+ * The environment variable MI355_GROUPED_IMPL=ref keeps every problem on the
+ * second one (short / tall pick the matrix-core kernel's tile shape). */
 int mi355_grouped_matmul_query(const mi355_grouped_desc_t *desc);
+
+/* Name of the implementation a launch of `desc` uses ("" if none does). */
+const char *mi355_grouped_matmul_impl(const mi355_grouped_desc_t *desc);
 
 /* Asynchronous on `stream`; no scratch.  The offsets are not validated (they
  * live on the device): rows outside every group are left untouched, a group
  * whose src and dst ranges differ in length computes the rows both have, and
- * no access leaves the tensors whatever the offsets hold. */
+ * no access leaves the tensors whatever the offsets hold.  Buffers that are
+ * not 16-byte aligned run on "hip:ref_grouped:any". */
 int mi355_grouped_matmul_launch(const mi355_grouped_desc_t *desc, const mi355_grouped_args_t *args, void *stream);
 
 /* Plain device-to-device copy kernel (one 16-byte load + store per lane), used

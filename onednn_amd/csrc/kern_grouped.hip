@@ -15,6 +15,8 @@
 // finds its group by bisection; nothing is assumed about the offsets beyond
 // what keeps every access inside the tensors.
 #include "kernels.hpp"
+#include <cstdlib>
+#include <cstring>
 
 namespace mi355 {
 namespace {
@@ -142,9 +144,308 @@ __global__ void __launch_bounds__(256) grouped_2dx2d_kernel(const grouped_dev_t 
     store_float(D.dst_dt, acc, P.a.dst, g * D.dst_stride[0] + m * D.dst_stride[1] + n * D.dst_stride[2]);
 }
 
+// ---- "hip:mfma_grouped" -- the 2Dx3D pattern on the matrix cores for fp8,
+// bf16 and f16 operands with K-contiguous weights ([G][N][K], tag acb), no
+// groups along K in the scales, no zero points.
+//
+// Mixture-of-experts groups are short (tens of rows against weights of K x N
+// per group), so the work is streaming every active group's weights once: HBM
+// bound.  A workgroup owns one (group, BM rows, BN columns) tile and walks K:
+//   * four wavefronts, WN along N x WK along K (K steps of 128 bytes per row,
+//     interleaved between the WK wavefronts; the accumulators meet in LDS);
+//   * operands go from global memory straight to registers: lane (j, q) of a
+//     fragment holds bytes 32 q .. 32 q + 31 of row j's 128-byte step, for src
+//     and weights alike, so any fixed assignment of those bytes to the K slots
+//     of the instruction gives the same dot product: one
+//     v_mfma_f32_16x16x128_f8f6f4 per fragment pair for fp8, two
+//     v_mfma_f32_16x16x32_{bf16,f16} for the 16-bit types;
+//   * D steps are in flight per wavefront (registers); weights are loaded
+//     non-temporally, src rows stay in the caches for the group's other tiles.
+// The grid is (column tiles, tile slots): slot s is the s-th (group, row
+// block) in group order.  A workgroup finds its slot by a block-wide prefix
+// sum over the groups' row-block counts (the offsets live on the device); the
+// host sizes the grid by the upper bound total_M / BM + min(G, total_M).
+typedef int g4i __attribute__((ext_vector_type(4)));
+typedef int g8i __attribute__((ext_vector_type(8)));
+typedef unsigned g2u __attribute__((ext_vector_type(2)));
+typedef unsigned g4u __attribute__((ext_vector_type(4)));
+typedef float g4f __attribute__((ext_vector_type(4)));
+typedef __bf16 g8bf __attribute__((ext_vector_type(8)));
+typedef _Float16 g8h __attribute__((ext_vector_type(8)));
+
+enum { GM_F8 = 0, GM_BF16 = 1, GM_F16 = 2 };
+
+// weights fragment first: the tile comes out transposed, a lane holds four
+// consecutive n (4 * (lane / 16) + e) of row lane % 16
+template <int MODE, int FA, int FB>
+__device__ __forceinline__ g4f grouped_mma(const g8i &w, const g8i &a, g4f c) {
+    if constexpr (MODE == GM_F8) {
+        return __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(w, a, c, FB, FA, 0, 0, 0, 0);
+    } else {
+        const g4i wl = {w[0], w[1], w[2], w[3]}, wh = {w[4], w[5], w[6], w[7]};
+        const g4i al = {a[0], a[1], a[2], a[3]}, ah = {a[4], a[5], a[6], a[7]};
+        if constexpr (MODE == GM_BF16) {
+            c = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
+                    __builtin_bit_cast(g8bf, wl), __builtin_bit_cast(g8bf, al), c, 0, 0, 0);
+            return __builtin_amdgcn_mfma_f32_16x16x32_bf16(
+                    __builtin_bit_cast(g8bf, wh), __builtin_bit_cast(g8bf, ah), c, 0, 0, 0);
+        } else {
+            c = __builtin_amdgcn_mfma_f32_16x16x32_f16(
+                    __builtin_bit_cast(g8h, wl), __builtin_bit_cast(g8h, al), c, 0, 0, 0);
+            return __builtin_amdgcn_mfma_f32_16x16x32_f16(
+                    __builtin_bit_cast(g8h, wh), __builtin_bit_cast(g8h, ah), c, 0, 0, 0);
+        }
+    }
+}
+
+// rows of group g that both src and dst hold, and where they start; offsets
+// that leave [0, total] or run backwards give fewer rows, never an access
+// outside the tensors
+__device__ __forceinline__ long grouped_rows(const grouped_dev_t &P, long g, long &dst0, long &src0) {
+    const long total = P.d.total;
+    auto clamp = [&](long v) { return v < 0 ? 0 : (v > total ? total : v); };
+    dst0 = g > 0 ? clamp(P.a.dst_offsets[g - 1]) : 0;
+    src0 = g > 0 ? clamp(P.a.src_offsets[g - 1]) : 0;
+    const long nd = clamp(P.a.dst_offsets[g]) - dst0, ns = clamp(P.a.src_offsets[g]) - src0;
+    const long n = nd < ns ? nd : ns;
+    return n > 0 ? n : 0;
+}
+
+template <int MODE, int FA, int FB, int MT, int NT, int WN, int WK, int D>
+__global__ void __launch_bounds__(256) grouped_tile_kernel(const grouped_dev_t P) {
+    static_assert(WN * WK == 4, "four wavefronts");
+    constexpr int BM = 16 * MT, BN = 16 * NT * WN;
+    constexpr int ES = MODE == GM_F8 ? 1 : 2; // bytes per element
+    __shared__ int pick[2];
+    __shared__ int wave_tot[4];
+    __shared__ g4f part[4 * MT * NT * 64]; // [wk][wn][unit][lane]
+    const mi355_grouped_desc_t &Dd = P.d;
+    const int t = threadIdx.x, lane = t & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(t >> 6);
+    const long G = Dd.group_count, K = Dd.K, N = Dd.N;
+
+    // ---- which (group, row block) is slot blockIdx.y
+    const int slot = blockIdx.y;
+    const long per = (G + 255) / 256; // groups per thread
+    auto blocks_of = [&](long g) {
+        long d0, s0;
+        return (int)((grouped_rows(P, g, d0, s0) + BM - 1) / BM);
+    };
+    int local = 0;
+    for (long i = 0; i < per; ++i) {
+        const long g = (long)t * per + i;
+        if (g < G) local += blocks_of(g);
+    }
+    int x = local;
+#pragma unroll
+    for (int o = 1; o < 64; o <<= 1) {
+        const int y = __shfl_up(x, o, 64);
+        if (lane >= o) x += y;
+    }
+    if (t == 0) pick[0] = -1;
+    if (lane == 63) wave_tot[wave] = x;
+    __syncthreads();
+    int before = x - local;
+    for (int w = 0; w < wave; ++w) before += wave_tot[w];
+    for (long i = 0; i < per; ++i) {
+        const long g = (long)t * per + i;
+        if (g < G) {
+            const int nb = blocks_of(g);
+            if (slot >= before && slot < before + nb) {
+                pick[0] = (int)g;
+                pick[1] = slot - before;
+            }
+            before += nb;
+        }
+    }
+    __syncthreads();
+    const int g = __builtin_amdgcn_readfirstlane(pick[0]);
+    if (g < 0) return; // beyond the last tile
+    const long m_base = (long)__builtin_amdgcn_readfirstlane(pick[1]) * BM;
+    long dst0, src0;
+    const long rows = grouped_rows(P, g, dst0, src0); // > m_base
+
+    // ---- operands
+    const int wn = wave % WN, wk = wave / WN;
+    const int j = lane & 15, q = lane >> 4;
+    const long row_bytes = K * ES;
+    const long n_wave = (long)blockIdx.x * BN + wn * (16 * NT);
+    const char *arow[MT], *bcol[NT];
+#pragma unroll
+    for (int i = 0; i < MT; ++i) {
+        long m = m_base + 16 * i + j;
+        m = m < rows ? m : rows - 1; // rows beyond the group read its last one (never stored)
+        arow[i] = (const char *)P.a.src + (src0 + m) * row_bytes + 32 * q;
+    }
+#pragma unroll
+    for (int jn = 0; jn < NT; ++jn) {
+        long n = n_wave + 16 * jn + j;
+        n = n < N ? n : N - 1;
+        bcol[jn] = (const char *)P.a.wei + ((long)g * Dd.wei_stride[0] + n * Dd.wei_stride[2]) * ES + 32 * q;
+    }
+    struct stage_t {
+        g8i a[MT], b[NT];
+    };
+    auto join = [](const g4i &lo, const g4i &hi) { return g8i {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]}; };
+    auto load = [&](long byte_off) __attribute__((always_inline)) {
+        stage_t f;
+#pragma unroll
+        for (int jn = 0; jn < NT; ++jn) {
+            const g4i *p = (const g4i *)(bcol[jn] + byte_off);
+            f.b[jn] = join(__builtin_nontemporal_load(p), __builtin_nontemporal_load(p + 1));
+        }
+#pragma unroll
+        for (int i = 0; i < MT; ++i) {
+            const g4i *p = (const g4i *)(arow[i] + byte_off);
+            f.a[i] = join(p[0], p[1]);
+        }
+        return f;
+    };
+    g4f acc[MT][NT];
+#pragma unroll
+    for (int i = 0; i < MT; ++i)
+#pragma unroll
+        for (int jn = 0; jn < NT; ++jn) acc[i][jn] = g4f {0.f, 0.f, 0.f, 0.f};
+    auto compute = [&](const stage_t &f) __attribute__((always_inline)) {
+#pragma unroll
+        for (int i = 0; i < MT; ++i)
+#pragma unroll
+            for (int jn = 0; jn < NT; ++jn) acc[i][jn] = grouped_mma<MODE, FA, FB>(f.b[jn], f.a[i], acc[i][jn]);
+    };
+
+    // ---- K: whole 128-byte steps wk, wk + WK, .. with D of them in flight
+    const long nfull = row_bytes / 128;
+    const int tail = (int)(row_bytes % 128); // a multiple of 32
+    if (nfull > wk) {
+        // this wavefront's steps: wk + WK * c, c < count; whole rounds of D run
+        // without a condition (loads beyond the end repeat the last step)
+        const long count = (nfull - wk + WK - 1) / WK;
+        auto step_off = [&](long c) { return (wk + WK * (c < count ? c : count - 1)) * 128; };
+        stage_t st[D];
+#pragma unroll
+        for (int d = 0; d < D; ++d) st[d] = load(step_off(d));
+        long c = 0;
+        for (; c + D <= count; c += D) {
+#pragma unroll
+            for (int d = 0; d < D; ++d) {
+                compute(st[d]);
+                st[d] = load(step_off(c + D + d));
+            }
+        }
+#pragma unroll
+        for (int d = 0; d < D; ++d)
+            if (c + d < count) compute(st[d]);
+    }
+    if (tail != 0 && wk == (int)(nfull % WK)) {
+        // lanes beyond K read the step's first 32 bytes instead and contribute zeros
+        const bool in = 32 * q < tail;
+        stage_t f = load(nfull * 128 - (in ? 0 : 32 * q));
+        if (!in) {
+#pragma unroll
+            for (int i = 0; i < MT; ++i) f.a[i] = g8i {0, 0, 0, 0, 0, 0, 0, 0};
+#pragma unroll
+            for (int jn = 0; jn < NT; ++jn) f.b[jn] = g8i {0, 0, 0, 0, 0, 0, 0, 0};
+        }
+        compute(f);
+    }
+
+    // ---- every wavefront leaves its accumulators in LDS; the 16 x 16 units of
+    // the tile are then finished by the four wavefronts in turn (one copy of the
+    // scales / bias / post-op / conversion code): lane (j, q) holds row j,
+    // columns 4 q .. 4 q + 3 of a unit
+#pragma unroll
+    for (int i = 0; i < MT; ++i)
+#pragma unroll
+        for (int jn = 0; jn < NT; ++jn) part[((wk * WN + wn) * MT * NT + i * NT + jn) * 64 + lane] = acc[i][jn];
+    __syncthreads();
+    const bool with_ss = Dd.src_scale_dt != MI355_DT_UNDEF, with_ws = Dd.wei_scale_dt != MI355_DT_UNDEF;
+    const int dbits = dt_bits(Dd.dst_dt);
+    const bool vec_ok = N % 4 == 0 && ((uintptr_t)P.a.dst % 16) == 0;
+#pragma nounroll
+    for (int u = wave; u < WN * MT * NT; u += 4) {
+        const int un = u / (MT * NT), i = (u / NT) % MT, jn = u % NT;
+        g4f sum = part[(un * MT * NT + i * NT + jn) * 64 + lane];
+#pragma unroll
+        for (int w = 1; w < WK; ++w) sum += part[((w * WN + un) * MT * NT + i * NT + jn) * 64 + lane];
+        const long m = m_base + 16 * i + j;
+        const long nb = (long)blockIdx.x * BN + un * (16 * NT) + 16 * jn + 4 * q;
+        if (m >= rows || nb >= N) continue;
+        const float ss = with_ss ? load_float(Dd.src_scale_dt, P.a.src_scale, src0 + m) : 1.f;
+        const int nvalid = N - nb < 4 ? (int)(N - nb) : 4;
+        uint32_t bits[4] = {0, 0, 0, 0};
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            if (e < nvalid) {
+                float v = sum[e];
+                if (with_ss) v *= ss;
+                if (with_ws) v *= load_float(Dd.wei_scale_dt, P.a.wei_scale, (long)g * N + nb + e);
+                v = grouped_finish(P, v, g, m, nb + e, dst0);
+                bits[e] = cvt_store_bits(Dd.dst_dt, v);
+            }
+        }
+        const long off = (dst0 + m) * N + nb;
+        if (vec_ok && nvalid == 4) {
+            if (dbits == 32)
+                *(g4u *)((char *)P.a.dst + off * 4) = g4u {bits[0], bits[1], bits[2], bits[3]};
+            else
+                *(g2u *)((char *)P.a.dst + off * 2) = g2u {bits[0] | (bits[1] << 16), bits[2] | (bits[3] << 16)};
+        } else {
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                if (e < nvalid) {
+                    if (dbits == 32) ((uint32_t *)P.a.dst)[off + e] = bits[e];
+                    else ((uint16_t *)P.a.dst)[off + e] = (uint16_t)bits[e];
+                }
+            }
+        }
+    }
+}
+
 bool fp_plain(int dt) { return dt == MI355_DT_F32 || dt == MI355_DT_BF16 || dt == MI355_DT_F16; }
 bool fp_any(int dt) {
     return fp_plain(dt) || dt == MI355_DT_F8_E4M3 || dt == MI355_DT_F8_E5M2 || dt == MI355_DT_F4_E2M1;
+}
+
+bool f8_dt(int dt) { return dt == MI355_DT_F8_E4M3 || dt == MI355_DT_F8_E5M2; }
+
+// 0: the thread-per-element kernel; 1: short groups (16 x 32 tiles, K split
+// between the wavefronts); 2: 64 x 128 tiles.  Decided on the descriptor alone.
+int tile_plan(const mi355_grouped_desc_t &d) {
+    if (d.pattern != MI355_GROUPED_2DX3D) return 0;
+    if (const char *e = getenv("MI355_GROUPED_IMPL")) {
+        if (!strcmp(e, "ref")) return 0;
+    }
+    const bool f8 = f8_dt(d.src_dt) && f8_dt(d.wei_dt);
+    const bool h16 = d.src_dt == d.wei_dt && (d.src_dt == MI355_DT_BF16 || d.src_dt == MI355_DT_F16);
+    if (!f8 && !h16) return 0;
+    const long es = f8 ? 1 : 2;
+    if (d.wei_stride[1] != 1 || d.wei_stride[2] < d.K) return 0; // K-contiguous weights only
+    if ((d.wei_stride[2] * es) % 16 != 0 || (d.wei_stride[0] * es) % 16 != 0 || (d.K * es) % 32 != 0) return 0;
+    auto k_groups = [&](int dt, long gk) { return dt != MI355_DT_UNDEF && gk > 1 && gk != d.K; };
+    if (k_groups(d.src_scale_dt, d.src_scale_gk) || k_groups(d.wei_scale_dt, d.wei_scale_gk)) return 0;
+    if (d.src_zp_dt != MI355_DT_UNDEF || d.wei_zp_dt != MI355_DT_UNDEF) return 0;
+    const long active = d.group_count < d.total ? d.group_count : d.total;
+    const int plan = d.total <= 2 * d.group_count ? 1 : 2;
+    const long slots = d.total / (plan == 1 ? 16 : 64) + active;
+    if (slots > 65535) return 0;
+    if (const char *e = getenv("MI355_GROUPED_IMPL")) {
+        if (!strcmp(e, "short")) return 1;
+        if (!strcmp(e, "tall")) return 2;
+    }
+    return plan;
+}
+
+template <int MODE, int FA, int FB>
+int launch_tiles(int plan, const grouped_dev_t &P, hipStream_t stream) {
+    const mi355_grouped_desc_t &d = P.d;
+    const long active = d.group_count < d.total ? d.group_count : d.total;
+    const int bm = plan == 1 ? 16 : 64, bn = plan == 1 ? 32 : 128;
+    dim3 grid((unsigned)((d.N + bn - 1) / bn), (unsigned)(d.total / bm + active));
+    if (plan == 1)
+        hipLaunchKernelGGL((grouped_tile_kernel<MODE, FA, FB, 1, 2, 1, 4, 4>), grid, dim3(256), 0, stream, P);
+    else
+        hipLaunchKernelGGL((grouped_tile_kernel<MODE, FA, FB, 4, 2, 4, 1, 2>), grid, dim3(256), 0, stream, P);
+    return hipGetLastError() == hipSuccess ? MI355_SUCCESS : MI355_RUNTIME_ERROR;
 }
 
 } // namespace
@@ -197,6 +498,11 @@ extern "C" int mi355_grouped_matmul_query(const mi355_grouped_desc_t *d) {
     return MI355_SUCCESS;
 }
 
+extern "C" const char *mi355_grouped_matmul_impl(const mi355_grouped_desc_t *d) {
+    if (!d || mi355_grouped_matmul_query(d) != MI355_SUCCESS) return "";
+    return tile_plan(*d) != 0 ? "hip:mfma_grouped" : "hip:ref_grouped:any";
+}
+
 extern "C" int mi355_grouped_matmul_launch(const mi355_grouped_desc_t *d, const mi355_grouped_args_t *a, void *stream) {
     if (!d || !a) return MI355_INVALID_ARGUMENTS;
     if (const int st = mi355_grouped_matmul_query(d)) {
@@ -223,6 +529,18 @@ extern "C" int mi355_grouped_matmul_launch(const mi355_grouped_desc_t *d, const 
     if (blocks >= (1L << 31)) {
         set_error("grouped matmul: %ld dst elements exceed the grid", elems);
         return MI355_UNIMPLEMENTED;
+    }
+    // the tiles read 16 bytes at a time
+    const int plan = ((uintptr_t)a->src % 16 == 0 && (uintptr_t)a->wei % 16 == 0) ? tile_plan(*d) : 0;
+    if (plan != 0) {
+        hipStream_t s = (hipStream_t)stream;
+        const int fa = d->src_dt == MI355_DT_F8_E5M2, fb = d->wei_dt == MI355_DT_F8_E5M2;
+        if (d->src_dt == MI355_DT_BF16) return launch_tiles<GM_BF16, 0, 0>(plan, P, s);
+        if (d->src_dt == MI355_DT_F16) return launch_tiles<GM_F16, 0, 0>(plan, P, s);
+        if (!fa && !fb) return launch_tiles<GM_F8, 0, 0>(plan, P, s);
+        if (fa && fb) return launch_tiles<GM_F8, 1, 1>(plan, P, s);
+        if (fa) return launch_tiles<GM_F8, 1, 0>(plan, P, s);
+        return launch_tiles<GM_F8, 0, 1>(plan, P, s);
     }
     if (x3)
         hipLaunchKernelGGL(grouped_2dx3d_kernel, dim3((unsigned)blocks), dim3(256), 0, (hipStream_t)stream, P);

@@ -1671,7 +1671,7 @@ dnnl_status_t grouped_pd_init(dnnl_primitive_desc &pd, const dnnl_memory_desc &s
     pd.src = src; pd.wei = wei; pd.dst = dst;
     pd.with_bias = bias != nullptr;
     if (bias) pd.bias = *bias;
-    pd.impl_name = "hip:ref_grouped:any";
+    pd.impl_name = mi355_grouped_matmul_impl(&D);
     pd.impls.assign(1, MI355_IMPL_REF);
     pd.impl_pos = 0;
     pd.scratch_bytes = 0;

@@ -1,0 +1,244 @@
+"""Grouped matmul on the matrix cores ("hip:mfma_grouped"): fp8 / bf16 / f16
+operands with K-contiguous weights.
+
+  * data every type holds exactly, where any summation order gives the same
+    bits: against the oracle (ref_grouped_t's order) bit for bit, both tile
+    shapes, ragged / empty / long groups, K tails, column tails, more groups
+    than threads;
+  * random data: against per-group float64 matmuls within a derived bound
+    (below);
+  * mixture-of-experts shapes of tests/benchdnn/inputs/matmul/shapes_grouped_moe
+    at full size: against the thread-per-element kernel (itself bit-exact
+    against the oracle at small sizes) within the same bound.
+
+Bound on |kernel - float64| for a dst element before bias: the products of fp8
+(or bf16 / f16) operands are exact in float32; the kernel adds them in float32
+in the hardware's order -- tests.helpers.gemm_bound -- and the fp8 instruction
+additionally aligns the eight products of a group to the largest and drops what
+falls below 2^-13 of it: per group at most seven losses of 2^-13 max|product|,
+taken as independent and uniform, over K / 8 groups, max|product| bounded by
+max|src| max|wei| of the row and column.  Four standard deviations of that, and
+one rounding of the result by each scale."""
+import ctypes as C
+import os
+
+import numpy as np
+import pytest
+
+from onednn_amd import cabi
+from onednn_amd import dtypes as dtp
+from onednn_amd.grouped import GroupedProblem, GroupedQuant
+from tests import grouped_cases as gc
+from tests.helpers import U, gemm_bound
+
+F32, BF16, F16 = cabi.DT_F32, cabi.DT_BF16, cabi.DT_F16
+E4M3, E5M2 = cabi.DT_F8_E4M3, cabi.DT_F8_E5M2
+
+SHAPES = [
+    ([8, 8, 8, 8], 64, 32),
+    ([2] * 16, 128, 96),
+    ([2, 6, 8], 32, 24),
+    ([10, 20, 30, 40], 160, 36),          # K tail of 32, N not a multiple of the tiles
+    ([1, 2, 4, 8, 16], 96, 130),          # K below one step
+    ([0, 1, 2, 0, 3, 0], 32, 20),
+    ([70, 3, 129], 256, 40),              # groups longer than a tile
+    ([1] + [0] * 299 + [2], 64, 16),      # more groups than threads in a workgroup
+    ([8], 384, 12),
+]
+TYPES = [("e4m3", E4M3, E4M3), ("e5m2", E5M2, E5M2), ("e4m3 x e5m2", E4M3, E5M2), ("e5m2 x e4m3", E5M2, E4M3),
+         ("bf16", BF16, BF16), ("f16", F16, F16)]
+EXTRAS = [
+    ("plain", {}),
+    ("row and column scales + bias", dict(src_scale="row", wei_scale="col", bias=True)),
+    ("relu after a per-group factor", dict(wei_scale="col", post_ops=("mul_group", "relu"))),
+    ("gate: linear then a grouped factor", dict(src_scale="row", post_ops=("linear", "mul_grouped"), bias=True)),
+    ("per-row factor", dict(post_ops=("mul_row",))),
+]
+
+
+@pytest.fixture(params=["short", "tall"])
+def tile_shape(request):
+    """Forces one of the two tile shapes of the matrix-core kernel."""
+    old = os.environ.get("MI355_GROUPED_IMPL")
+    os.environ["MI355_GROUPED_IMPL"] = request.param
+    yield request.param
+    if old is None:
+        del os.environ["MI355_GROUPED_IMPL"]
+    else:
+        os.environ["MI355_GROUPED_IMPL"] = old
+
+
+def impl_of(p):
+    d = p.desc()
+    return cabi.load_kernels().mi355_grouped_matmul_impl(C.byref(d)).decode()
+
+
+def test_dispatch_rules():
+    """What goes to the matrix cores is decided on the descriptor."""
+    p, _ = gc.case_2dx3d([4, 4], 64, 32, src_dt=E4M3, wei_dt=E4M3, wtag="acb")
+    assert impl_of(p) == "hip:mfma_grouped"
+    p, _ = gc.case_2dx3d([4, 4], 64, 32, src_dt=BF16, wei_dt=BF16, wtag="acb", src_scale="row", wei_scale="col")
+    assert impl_of(p) == "hip:mfma_grouped"
+    p, _ = gc.case_2dx3d([4, 4], 64, 32, src_dt=BF16, wei_dt=BF16)                   # N-contiguous weights
+    assert impl_of(p) == "hip:ref_grouped:any"
+    p, _ = gc.case_2dx3d([4, 4], 64, 32, src_dt=E4M3, wei_dt=E4M3, wtag="acb", wei_scale=32)   # groups along K
+    assert impl_of(p) == "hip:ref_grouped:any"
+    p, _ = gc.case_2dx3d([4, 4], 48, 32, src_dt=E4M3, wei_dt=E4M3, wtag="acb")       # K not a multiple of 32 bytes
+    assert impl_of(p) == "hip:ref_grouped:any"
+    p, _ = gc.case_2dx3d([4, 4], 48, 32, src_dt=F16, wei_dt=F16, wtag="acb")         # 96 bytes: fine
+    assert impl_of(p) == "hip:mfma_grouped"
+    p, _ = gc.case_2dx3d([4, 4], 64, 32, wtag="acb")                                 # f32
+    assert impl_of(p) == "hip:ref_grouped:any"
+    p, _ = gc.case_2dx3d([4, 4], 64, 32, src_dt=F16, wei_dt=cabi.DT_U4, wei_scale=16, wei_zp=16)
+    assert impl_of(p) == "hip:ref_grouped:any"
+    os.environ["MI355_GROUPED_IMPL"] = "ref"
+    try:
+        p, _ = gc.case_2dx3d([4, 4], 64, 32, src_dt=E4M3, wei_dt=E4M3, wtag="acb")
+        assert impl_of(p) == "hip:ref_grouped:any"
+    finally:
+        del os.environ["MI355_GROUPED_IMPL"]
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("shape", SHAPES, ids=lambda s: f"G{len(s[0])}x{sum(s[0])}x{s[1]}x{s[2]}")
+@pytest.mark.parametrize("tname,sdt,wdt", TYPES, ids=[t[0] for t in TYPES])
+def test_exact_data_matches_the_oracle(gpu, oracle, tile_shape, shape, tname, sdt, wdt):
+    from onednn_amd import grouped
+    sizes, K, N = shape
+    for label, kw in EXTRAS:
+        for dst_dt in (F32, BF16):
+            p, want = gc.case_2dx3d(sizes, K, N, src_dt=sdt, wei_dt=wdt, dst_dt=dst_dt, wtag="acb", **kw)
+            assert impl_of(p) == "hip:mfma_grouped"
+            st, ref = oracle.run_oracle_grouped(p)
+            assert st == cabi.SUCCESS
+            got = grouped.run_gpu(p)
+            assert np.array_equal(got, ref), f"{p.name} {tname} {label} dst {dst_dt} ({tile_shape})"
+            if dst_dt == F32:
+                assert np.array_equal(gc.logical_dst(p, got), want)
+
+
+def random_case(rng, sizes, K, N, dt, scales=True, dst_dt=F32, active=None):
+    """Random operands (fp8: random finite bytes with exponents in a band of 2^8;
+    16-bit types: normal), weights [G][N][K].  Returns (problem, S, W, ss, ws) with
+    the float64 values.  `active`: groups whose weights are filled (the others
+    keep zeros; they have no rows)."""
+    G, total = len(sizes), int(sum(sizes))
+
+    def draw(shape):
+        if dt == E4M3:
+            raw = (rng.integers(0, 2, shape, dtype=np.uint8) << 7) | rng.integers(0x20, 0x60, shape, dtype=np.uint8)
+            return raw, dtp.e4m3_to_f32(raw.reshape(-1)).reshape(shape)
+        v = rng.standard_normal(shape, dtype=np.float32)
+        if dt == BF16:
+            raw = dtp.f32_to_bf16(v)
+            return raw, dtp.bf16_to_f32(raw.reshape(-1)).reshape(shape)
+        raw = v.astype(np.float16)
+        return raw.view(np.uint16), raw.astype(np.float32)
+
+    sraw, S = draw((total, K))
+    if active is None:
+        wraw, W = draw((G, N, K))
+    else:
+        wraw = np.zeros((G, N, K), sraw.dtype)
+        W = np.zeros((G, N, K), np.float32)
+        for g in active:
+            wraw[g], W[g] = draw((N, K))
+    quant = {}
+    ss, ws = np.ones(total, np.float32), np.ones((G, N), np.float32)
+    if scales:
+        ss = rng.uniform(0.5, 2.0, total).astype(np.float32)
+        ws = rng.uniform(0.5, 2.0, (G, N)).astype(np.float32)
+        quant = {"src_scale": GroupedQuant(F32, ss, 0), "wei_scale": GroupedQuant(F32, ws, 0)}
+    p = GroupedProblem(pattern=cabi.GROUPED_2DX3D, sizes=list(sizes), K=K, N=N, src_dt=dt, wei_dt=dt, dst_dt=dst_dt,
+                       src=sraw, wei=wraw, wei_stride=(K * N, 1, K), quant=quant, name=f"random {len(sizes)} groups")
+    return p, S, W, ss, ws
+
+
+def expectation(p, S, W, ss, ws, fp8):
+    """(float64 value, bound) per dst element."""
+    want = np.zeros((p.total, p.N))
+    tol = np.zeros((p.total, p.N))
+    start = 0
+    for g, mg in enumerate(p.sizes):
+        if mg == 0:
+            continue
+        s = S[start:start + mg].astype(np.float64)
+        w = W[g].astype(np.float64)
+        sc = ss[start:start + mg, None].astype(np.float64) * ws[g][None, :]
+        v = s @ w.T
+        abs_sum = np.abs(s) @ np.abs(w).T
+        t = gemm_bound(p.K, abs_sum)
+        if fp8:
+            big = np.abs(s).max(1)[:, None] * np.abs(w).max(1)[None, :]
+            t = t + 4.0 * np.sqrt(7.0 / 3.0 * (p.K / 8.0)) * 2.0 ** -13 * big
+        want[start:start + mg] = v * sc
+        tol[start:start + mg] = (t + 3 * U * np.abs(v)) * sc
+        start += mg
+    return want, tol
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dt", [E4M3, BF16, F16], ids=["e4m3", "bf16", "f16"])
+def test_random_data_within_the_derived_bound(gpu, tile_shape, dt):
+    from onednn_amd import grouped
+    rng = np.random.default_rng(21)
+    sizes = [33, 0, 5, 64, 17, 1, 90, 2]
+    p, S, W, ss, ws = random_case(rng, sizes, 1120, 200, dt)       # K tail of 96 / 64 bytes
+    assert impl_of(p) == "hip:mfma_grouped"
+    want, tol = expectation(p, S, W, ss, ws, dt == E4M3)
+    got = gc.logical_dst(p, grouped.run_gpu(p))
+    err = np.abs(got - want)
+    assert np.all(err <= tol), f"worst {np.max(err / np.maximum(tol, 1e-30)):.2f} of the bound"
+    assert err.max() > 0          # the data is not of the exact kind
+
+
+def _ref_kernel(p):
+    from onednn_amd import grouped
+    old = os.environ.get("MI355_GROUPED_IMPL")
+    os.environ["MI355_GROUPED_IMPL"] = "ref"
+    try:
+        return grouped.run_gpu(p)
+    finally:
+        if old is None:
+            del os.environ["MI355_GROUPED_IMPL"]
+        else:
+            os.environ["MI355_GROUPED_IMPL"] = old
+
+
+MOE = {
+    # name: (sizes, K, N)  -- shapes_grouped_moe
+    "Qwen3-30B-A3B gate/up prefill": (
+        [13, 12, 11, 11, 14, 11, 15, 14, 13, 15, 16, 21, 16, 17, 12, 20, 14, 21, 19, 16, 24, 12, 8, 23, 11, 17, 13, 19, 14,
+         21, 14, 16, 17, 17, 14, 23, 14, 14, 17, 24, 19, 13, 11, 9, 17, 11, 13, 11, 18, 16, 11, 11, 13, 10, 17, 17, 17, 18,
+         14, 16, 20, 22, 20, 19, 16, 13, 10, 22, 15, 16, 19, 16, 17, 24, 13, 17, 19, 20, 14, 18, 19, 14, 17, 18, 20, 15, 20,
+         12, 17, 13, 18, 9, 18, 13, 23, 15, 10, 27, 15, 8, 6, 18, 19, 14, 17, 17, 21, 16, 19, 14, 15, 12, 17, 20, 16, 18, 25,
+         17, 19, 18, 20, 19, 16, 13, 13, 16, 13, 14], 2048, 768),
+    "GPT-OSS-20b gate/up prefill": (
+        [29, 28, 31, 28, 39, 32, 36, 34, 32, 28, 28, 22, 29, 28, 36, 45, 36, 38, 31, 31, 31, 32, 24, 28, 34, 27, 33, 35, 32,
+         43, 31, 33], 2880, 2880),
+    "Qwen2-57B-A14B gate/up decode": (
+        [0, 1, 0, 0, 0, 0, 0, 0, 1, 0, 0, 0, 0, 0, 1, 1, 0, 1, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0,
+         0, 0, 0, 0, 0, 0, 0, 0, 0, 1, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 1, 0, 1], 3584, 2560),
+}
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("name", list(MOE), ids=lambda n: n.split()[0])
+def test_moe_shapes_at_full_size_against_the_reference_order_kernel(gpu, name):
+    """fp8 e4m3 with row-wise / column-wise f32 scales and bf16 -> f32 dst checked
+    twice: against the thread-per-element kernel (the reference's order) within
+    the bound both carry, and against float64 on a sample of rows."""
+    from onednn_amd import grouped
+    sizes, K, N = MOE[name]
+    assert sum(sizes) in (2048, 1024, 8)
+    rng = np.random.default_rng(5)
+    active = [g for g, m in enumerate(sizes) if m]
+    p, S, W, ss, ws = random_case(rng, sizes, K, N, E4M3, active=active)
+    assert impl_of(p) == "hip:mfma_grouped"
+    got = gc.logical_dst(p, grouped.run_gpu(p))
+    ref = gc.logical_dst(p, _ref_kernel(p))
+    want, tol = expectation(p, S, W, ss, ws, True)
+    assert np.all(np.abs(got - want) <= tol)
+    # the sequential float32 sum of the reference's order carries gemm_bound alone
+    assert np.all(np.abs(ref - want) <= tol)
+    assert np.abs(got - ref).max() > 0
