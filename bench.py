@@ -49,6 +49,9 @@ PROFILE_OF = {
     ("c2", "ab", 8): "woq_gemv_kernel_c2_m8_plain_ab.md", ("c2", "ab", 32): "woq_gemv_kernel_c2_m32_plain_ab.md",
     ("r1", "any"): "reorder_direct_kernel_r1_f32_s8_8192.md", ("r2", "any"): "transpose8_kernel_r2_s8_transpose_8192.md",
     ("r3", "any"): "pack_woq64_kernel_r3_u4_4096x14336.md",
+    ("g1", "any"): "grouped_tile_kernel_g1_deepseek_v3_prefill.md",
+    ("g2", "any"): "grouped_tile_kernel_g2_llama4_scout_prefill.md",
+    ("g3", "any"): "grouped_tile_kernel_g3_deepseek_v3_decode.md",
 }
 
 
@@ -260,6 +263,78 @@ def run_reorder_workloads(lib, steps, which=("r1", "r2", "r3")):
     return out
 
 
+def run_grouped_workloads(lib, steps, which=("g1", "g2", "g3")):
+    """The grouped (mixture-of-experts) matmul on shapes of the reference's
+    shapes_grouped_moe files: fp8 e4m3 operands, a scale per src row and per
+    group and column, bf16 dst.  HBM-bound: the weights of every group with
+    rows are read once.  Two copies of every tensor alternate between launches
+    so that the smaller shapes do not run out of the 256 MB last-level cache."""
+    import numpy as np
+    from onednn_amd import cabi, configs
+    from onednn_amd.grouped import fill_args
+    out = []
+    timer = Timer(lib)
+    for key in which:
+        t0 = time.time()
+        p = configs.grouped_config(key)
+        d = p.desc()
+        cabi.check(lib.mi355_grouped_matmul_query(C.byref(d)))
+        copies = 1 if p.wei.nbytes > (1 << 30) else 3
+        sets, bufs = [], []
+        for _ in range(copies):
+            def place(arr):
+                b = cabi.DeviceBuffer.from_numpy(np.ascontiguousarray(arr))
+                bufs.append(b)
+                return b.ptr
+            a = fill_args(p, place)
+            dst = cabi.DeviceBuffer(p.initial_dst().nbytes)
+            bufs.append(dst)
+            a.dst = dst.ptr
+            sets.append(a)
+        log(f"[bench] {key}: generated and uploaded {p.name} in {time.time() - t0:.1f}s")
+        idx = [0]
+
+        def step():
+            cabi.check(lib.mi355_grouped_matmul_launch(C.byref(d), C.byref(sets[idx[0] % copies]), None))
+            idx[0] += 1
+
+        for _ in range(3):
+            step()
+        ms = timer.time_ms(step, steps)
+        nbytes = configs.grouped_bytes(p)
+        gbs = nbytes / (ms * 1e-3) / 1e9
+        impl = lib.mi355_grouped_matmul_impl(C.byref(d)).decode()
+        out.append({"workload": p.name, "impl": impl, "ms_per_step": ms, "value": gbs, "unit": "GB/s", "bound": "hbm",
+                    "peak": PEAK_HBM_GBS, "frac_of_peak": gbs / PEAK_HBM_GBS, "work": nbytes,
+                    "tflops": 2.0 * p.total * p.K * p.N / (ms * 1e-3) / 1e12})
+        log(f"[bench] {p.name}: {ms:.4f} ms -> {gbs:.1f} GB/s ({100 * gbs / PEAK_HBM_GBS:.1f}% of hbm peak) via {impl}")
+        for b in bufs:
+            b.free()
+    return out
+
+
+def grouped_cpu_baseline(name):
+    """The oracle's restatement of ref_grouped_t on the first groups and columns of the workload."""
+    from oracle import binding as oracle
+    from onednn_amd import configs
+    groups, N = {"g1": (16, 256), "g2": (2, 256), "g3": (64, 256)}[name]
+    p = configs.grouped_config(name, groups=groups, N=N)
+    oracle.load()
+    reps, t0 = 0, time.time()
+    while True:
+        st, _ = oracle.run_oracle_grouped(p)
+        assert st == 0
+        reps += 1
+        dt = time.time() - t0
+        if dt >= 10.0 or reps >= 200:
+            break
+    from onednn_amd import configs as cf
+    return {"value": cf.grouped_bytes(p) * reps / dt / 1e9, "unit": "GB/s", "cores": 1, "kind": "port",
+            "sample": f"the first {groups} groups and {N} columns of the workload ({p.total} rows); {reps} pass(es), "
+                      f"{dt:.2f} s wall; oracle/liboracle.so, oracle_grouped_matmul (plain C restatement of "
+                      "ref_grouped_t, one thread)"}
+
+
 def cpu_baseline(name, M=None):
     """The oracle timed on a bounded sample of the same workload."""
     from oracle import binding as oracle
@@ -312,9 +387,10 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=3)
-    ap.add_argument("--workload", default="c3", choices=["c1", "c2", "c3", "c4", "c5", "r1", "r2", "r3"],
-                    help="c1..c5: the matmul configurations (c3 is the headline); r1, r2: the reorder "
-                         "primitive on the headline shape's tensors (informational)")
+    ap.add_argument("--workload", default="c3", choices=["c1", "c2", "c3", "c4", "c5", "r1", "r2", "r3", "g1", "g2", "g3"],
+                    help="c1..c5: the matmul configurations (c3 is the headline); r1..r3: the reorder "
+                         "primitive on the headline shape's tensors; g1..g3: the grouped (mixture-of-experts) "
+                         "matmul on shapes of the reference's shapes_grouped_moe files (informational)")
     ap.add_argument("--decode-m", type=int, default=1, help="M of the c2 decode workload")
     ap.add_argument("--wtag", default="any", choices=["any", "ab", "ba"],
                     help="weights layout; any = what format_tag::any resolves to (default)")
@@ -434,6 +510,22 @@ def main():
                          "kernel": r["impl"], "kernel_ms": r["ms_per_step"]},
             "cpu_baseline": None, "others": []}), flush=True)
         return
+    if main_name in ("g1", "g2", "g3"):
+        r = run_grouped_workloads(lib, args.steps, (main_name,))[0]
+        if args.calib_copy:
+            calib_copy()
+        cpu = None if args.no_cpu else grouped_cpu_baseline(main_name)
+        print(json.dumps({
+            "metric": "grouped fp8 matmul GB/s", "value": r["value"], "unit": "GB/s", "n_gpus": 1, "steps": args.steps,
+            "warmup": args.warmup, "ms_per_step": r["ms_per_step"], "higher_is_better": True, "scaling": "weak",
+            "vs_baseline": None, "dtype": "f8_e4m3", "data": "synthetic",
+            "config": {"workload": r["workload"], "impl": r["impl"], "tflops": r["tflops"]},
+            "roofline": {"bound": "hbm", "achieved": r["value"], "peak": PEAK_HBM_GBS, "unit": "GB/s",
+                         "frac": r["frac_of_peak"], "traffic": measured_traffic(main_name)[0],
+                         "traffic_source": measured_traffic(main_name)[1], "algorithmic": r["work"],
+                         "kernel": r["impl"], "kernel_ms": r["ms_per_step"]},
+            "cpu_baseline": cpu, "others": []}), flush=True)
+        return
     cold = 11 if main_name == "c2" else 0
     res, prob = run_gpu_workload(lib, main_name, args.steps, args.warmup, args.decode_m, cold,
                                  args.wtag, sustained_s=args.sustained)
@@ -484,6 +576,11 @@ def main():
         except Exception as e:
             others.append({"workload": "reorder", "error": str(e)})
             log(f"[bench] reorder: failed: {e}")
+        try:
+            others += run_grouped_workloads(lib, max(5, args.steps // 2))
+        except Exception as e:
+            others.append({"workload": "grouped", "error": str(e)})
+            log(f"[bench] grouped: failed: {e}")
 
     cpu = None
     if not args.no_cpu:

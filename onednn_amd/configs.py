@@ -209,3 +209,58 @@ def config_ops(p):
 def config2_bytes(M, N=14336, K=4096, group=128):
     G = K // group
     return K * N // 2 + G * N * 2 + G * N // 2 + M * K * 2 + M * N * 2
+
+
+# ---- grouped (mixture-of-experts) matmul: shapes of the reference's
+# tests/benchdnn/inputs/matmul/shapes_grouped_moe{,_large}, run there (GPU
+# test_matmul_grouped_gpu) as f8_e4m3 x f8_e4m3 -> bf16 with
+# --attr-scales=src:1:f32+wei:5:f32 (a scale per src row and per group and
+# column) and K-contiguous weights (--wtag=acb).
+GROUPED_SHAPES = {
+    # DeepSeek-v3 gate/up projection, prefill: 2048x7168 : 256x7168x2048
+    "g1": ("DeepSeek-v3-gate/up-proj-prefill", 7168, 2048, [
+        5, 8, 3, 7, 7, 3, 2, 8, 7, 6, 7, 4, 5, 10, 8, 6, 9, 3, 7, 9, 9, 8, 10, 11, 6, 10, 13, 5, 7, 7, 8, 10, 8, 6, 8, 13,
+        6, 12, 8, 7, 11, 14, 3, 9, 5, 3, 13, 11, 4, 7, 9, 10, 9, 4, 8, 10, 7, 7, 14, 7, 7, 6, 9, 7, 10, 8, 8, 9, 8, 6, 12,
+        9, 5, 10, 7, 8, 9, 6, 14, 10, 10, 10, 6, 7, 8, 4, 4, 5, 5, 12, 5, 5, 8, 5, 4, 6, 5, 13, 9, 5, 3, 8, 9, 3, 9, 4, 5,
+        5, 9, 8, 8, 8, 10, 9, 7, 12, 6, 7, 5, 9, 11, 9, 11, 11, 12, 9, 10, 9, 9, 6, 6, 7, 2, 8, 5, 18, 10, 4, 4, 13, 10, 8,
+        12, 3, 8, 9, 11, 13, 9, 4, 7, 11, 8, 9, 12, 8, 5, 9, 12, 7, 12, 8, 5, 9, 9, 8, 7, 11, 9, 11, 10, 5, 9, 11, 9, 3, 12,
+        5, 6, 8, 9, 7, 2, 7, 5, 14, 7, 6, 12, 11, 5, 9, 7, 4, 17, 10, 9, 7, 5, 5, 1, 5, 9, 10, 7, 11, 6, 8, 8, 9, 9, 8, 13,
+        9, 10, 6, 12, 7, 7, 7, 11, 4, 5, 9, 8, 9, 13, 7, 9, 8, 13, 5, 17, 8, 7, 9, 10, 9, 10, 8, 13, 7, 11, 8, 7, 9, 4, 8,
+        8, 5, 10, 7, 6, 7, 7, 7]),
+    # Llama4-Scout gate/up projection, prefill: 512x5120 : 16x5120x8192
+    "g2": ("Llama4-Scout-gate/up-proj-prefill", 5120, 8192,
+           [28, 31, 37, 31, 30, 27, 34, 45, 40, 25, 33, 22, 34, 39, 34, 22]),
+    # DeepSeek-v3 gate/up projection, decode: 8x7168 : 256x7168x2048 (eight groups of one row)
+    "g3": ("DeepSeek-v3-gate/up-proj-decode", 7168, 2048,
+           [1 if g in (12, 44, 52, 57, 71, 114, 125, 140) else 0 for g in range(256)]),
+}
+
+
+def grouped_config(name, seed=9, groups=None, N=None):
+    """One of GROUPED_SHAPES as a GroupedProblem with random fp8 operands
+    (finite e4m3 bytes over eight binades), f32 scales in [0.5, 2) and a bf16
+    dst.  `groups` / `N`: only the first groups / columns (CPU samples)."""
+    from .grouped import GroupedProblem, GroupedQuant
+    label, K, n_full, sizes = GROUPED_SHAPES[name]
+    sizes = list(sizes[:groups] if groups else sizes)
+    N = N or n_full
+    G, total = len(sizes), int(sum(sizes))
+    rng = _rng(seed, 1)
+
+    def fp8(shape):
+        return (rng.integers(0, 2, shape, dtype=np.uint8) << 7) | rng.integers(0x20, 0x60, shape, dtype=np.uint8)
+
+    quant = {"src_scale": GroupedQuant(cabi.DT_F32, rng.uniform(0.5, 2.0, total).astype(np.float32), 0),
+             "wei_scale": GroupedQuant(cabi.DT_F32, rng.uniform(0.5, 2.0, (G, N)).astype(np.float32), 0)}
+    return GroupedProblem(pattern=cabi.GROUPED_2DX3D, sizes=sizes, K=K, N=N, src_dt=cabi.DT_F8_E4M3,
+                          wei_dt=cabi.DT_F8_E4M3, dst_dt=cabi.DT_BF16, src=fp8((total, K)), wei=fp8((G, N, K)),
+                          wei_stride=(K * N, 1, K), quant=quant, name=f"{name.upper()} {label} {total}x{K}:{G}x{K}x{N}")
+
+
+def grouped_bytes(p):
+    """Algorithmic HBM bytes of a grouped fp8 launch: the weights of every group
+    that has rows, src, dst, scales and offsets, each once."""
+    active = sum(1 for m in p.sizes if m)
+    es = cabi.DT_BITS[p.wei_dt] // 8
+    return (active * p.K * p.N * es + p.total * p.K * es + p.total * p.N * cabi.DT_BITS[p.dst_dt] // 8
+            + 4 * p.total + 4 * active * p.N + 8 * p.G)

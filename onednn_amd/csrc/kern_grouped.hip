@@ -151,12 +151,20 @@ __global__ void __launch_bounds__(256) grouped_2dx2d_kernel(const grouped_dev_t 
 // Mixture-of-experts groups are short (tens of rows against weights of K x N
 // per group), so the work is streaming every active group's weights once: HBM
 // bound.  A workgroup owns one (group, BM rows, BN columns) tile and walks K:
-//   * four wavefronts, WN along N x WK along K (K steps of 128 bytes per row,
-//     interleaved between the WK wavefronts; the accumulators meet in LDS);
-//   * operands go from global memory straight to registers: lane (j, q) of a
-//     fragment holds bytes 32 q .. 32 q + 31 of row j's 128-byte step, for src
-//     and weights alike, so any fixed assignment of those bytes to the K slots
-//     of the instruction gives the same dot product: one
+//   * the four wavefronts take the K steps (128 bytes per row) in turn, each
+//     over the whole tile, so src and weights are both read once per
+//     workgroup; the accumulators meet in LDS (eight wavefronts measured
+//     slower on every shape);
+//   * a tile holds up to MTMAX fragments of 16 rows; the walk is compiled per
+//     fragment count and the tile's own count picks one, so a group of 20 rows
+//     loads and multiplies two fragments, not MTMAX;
+//   * operands go from global memory straight to registers, a load instruction
+//     fetching the whole 128-byte lines of 8 rows (what a compute unit can keep
+//     in flight is counted in line requests: half lines halve it); after an
+//     exchange between lanes j and j +- 8, lane (j, q) of a fragment holds
+//     bytes 16 q .. 16 q + 15 and 64 + 16 q .. 64 + 16 q + 15 of row j's step,
+//     for src and weights alike, so whichever K slots of the instruction those
+//     bytes land in, the dot product is the same: one
 //     v_mfma_f32_16x16x128_f8f6f4 per fragment pair for fp8, two
 //     v_mfma_f32_16x16x32_{bf16,f16} for the 16-bit types;
 //   * D steps are in flight per wavefront (registers); weights are loaded
@@ -211,22 +219,153 @@ __device__ __forceinline__ long grouped_rows(const grouped_dev_t &P, long g, lon
     return n > 0 ? n : 0;
 }
 
-template <int MODE, int FA, int FB, int MT, int NT, int WN, int WK, int D>
-__global__ void __launch_bounds__(256) grouped_tile_kernel(const grouped_dev_t P) {
-    static_assert(WN * WK == 4, "four wavefronts");
-    constexpr int BM = 16 * MT, BN = 16 * NT * WN;
+// what a workgroup knows about its tile (uniform over the workgroup)
+struct gtile_t {
+    long g, m_base, rows; // group, first row of the tile inside the group, rows of the group
+    long dst0, src0;      // first row of the group in dst / src
+    long n0;              // first column of the tile
+};
+
+// One wavefront's share of a tile's K walk: steps wk, wk + WK, .. of 128 bytes per
+// row for MF fragments of 16 src rows against NT fragments of 16 weights rows,
+// D steps in flight.  Leaves the MF x NT accumulators in `part`.
+template <int MODE, int FA, int FB, int MF, int NT, int D, int WK>
+__device__ __forceinline__ void grouped_walk(const grouped_dev_t &P, const gtile_t &T, g4f *part, int wk, int lane) {
     constexpr int ES = MODE == GM_F8 ? 1 : 2; // bytes per element
+    const mi355_grouped_desc_t &Dd = P.d;
+    const int j = lane & 15, q = lane >> 4;
+    const long row_bytes = Dd.K * ES;
+    // A load instruction fetches whole 128-byte lines: 8 rows x 8 chunks of 16
+    // bytes.  Lane (j, q) fetches chunk q + 4 (j / 8) of rows j % 8 and 8 + j % 8
+    // of a fragment; lanes j and j +- 8 then exchange one of the two so that
+    // lane (j, q) holds chunks q and 4 + q of row j.
+    const int half = j >> 3;
+    const uint32_t chunk = 16 * (q + 4 * half);
+    const long pitch_b = Dd.wei_stride[2] * ES;
+    const char *abase = (const char *)P.a.src + (T.src0 + T.m_base) * row_bytes;
+    const char *bbase = (const char *)P.a.wei + (T.g * Dd.wei_stride[0] + T.n0 * Dd.wei_stride[2]) * ES;
+    uint32_t aoff[MF][2], boff[NT][2];
+#pragma unroll
+    for (int i = 0; i < MF; ++i)
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+            long m = T.m_base + 16 * i + 8 * h + (j & 7);
+            m = m < T.rows ? m : T.rows - 1; // rows beyond the group read its last one (never stored)
+            aoff[i][h] = (uint32_t)((m - T.m_base) * row_bytes) + chunk;
+        }
+#pragma unroll
+    for (int jn = 0; jn < NT; ++jn)
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+            long n = T.n0 + 16 * jn + 8 * h + (j & 7);
+            n = n < Dd.N ? n : Dd.N - 1;
+            boff[jn][h] = (uint32_t)((n - T.n0) * pitch_b) + chunk;
+        }
+    struct stage_t {
+        g4i a[MF][2], b[NT][2];
+    };
+    // step_off: byte offset of the step in a row (uniform)
+    auto load = [&](long step_off, uint32_t back) __attribute__((always_inline)) {
+        stage_t f;
+#pragma unroll
+        for (int jn = 0; jn < NT; ++jn)
+#pragma unroll
+            for (int h = 0; h < 2; ++h) f.b[jn][h] = *(const g4i *)(bbase + step_off + (boff[jn][h] - back));
+#pragma unroll
+        for (int i = 0; i < MF; ++i)
+#pragma unroll
+            for (int h = 0; h < 2; ++h) f.a[i][h] = *(const g4i *)(abase + step_off + (aoff[i][h] - back));
+        return f;
+    };
+    // the exchange between lanes j and j +- 8 (a rotation by 8 inside each row of 16 lanes)
+    auto settle = [&](const g4i (&r)[2]) __attribute__((always_inline)) {
+        g8i out;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            const int send = half ? r[0][e] : r[1][e];
+            const int recv = __builtin_amdgcn_update_dpp(0, send, 0x128 /* row_ror:8 */, 0xf, 0xf, false);
+            out[e] = half ? recv : r[0][e];
+            out[4 + e] = half ? r[1][e] : recv;
+        }
+        return out;
+    };
+    g4f acc[MF][NT];
+#pragma unroll
+    for (int i = 0; i < MF; ++i)
+#pragma unroll
+        for (int jn = 0; jn < NT; ++jn) acc[i][jn] = g4f {0.f, 0.f, 0.f, 0.f};
+    auto compute = [&](const stage_t &f) __attribute__((always_inline)) {
+        g8i a[MF];
+#pragma unroll
+        for (int i = 0; i < MF; ++i) a[i] = settle(f.a[i]);
+#pragma unroll
+        for (int jn = 0; jn < NT; ++jn) {
+            const g8i w = settle(f.b[jn]);
+#pragma unroll
+            for (int i = 0; i < MF; ++i) acc[i][jn] = grouped_mma<MODE, FA, FB>(w, a[i], acc[i][jn]);
+        }
+    };
+
+    const long nfull = row_bytes / 128;
+    const int tail = (int)(row_bytes % 128); // a multiple of 32
+    if (nfull > wk) {
+        // this wavefront's steps: wk + WK * c, c < count; whole rounds of D run
+        // without a condition (loads beyond the end repeat the last step)
+        const long count = (nfull - wk + WK - 1) / WK;
+        auto step_off = [&](long c) { return (wk + WK * (c < count ? c : count - 1)) * 128; };
+        stage_t st[D];
+#pragma unroll
+        for (int d = 0; d < D; ++d) st[d] = load(step_off(d), 0);
+        long c = 0;
+        for (; c + D <= count; c += D) {
+#pragma unroll
+            for (int d = 0; d < D; ++d) {
+                compute(st[d]);
+                st[d] = load(step_off(c + D + d), 0);
+                // keep the rounds apart: the scheduler would otherwise start the next
+                // stage's products early and wait for every load in flight
+                __builtin_amdgcn_sched_barrier(0);
+            }
+        }
+#pragma unroll
+        for (int d = 0; d < D; ++d)
+            if (c + d < count) compute(st[d]);
+    }
+    if (tail != 0 && wk == (int)(nfull % WK)) {
+        // a chunk beyond K: the lane reads the step's first chunk instead and hands on zeros
+        const bool in = chunk + 16 <= (uint32_t)tail;
+        stage_t f = load(nfull * 128, in ? 0 : chunk);
+        if (!in) {
+#pragma unroll
+            for (int h = 0; h < 2; ++h) {
+#pragma unroll
+                for (int i = 0; i < MF; ++i) f.a[i][h] = g4i {0, 0, 0, 0};
+#pragma unroll
+                for (int jn = 0; jn < NT; ++jn) f.b[jn][h] = g4i {0, 0, 0, 0};
+            }
+        }
+        compute(f);
+    }
+#pragma unroll
+    for (int i = 0; i < MF; ++i)
+#pragma unroll
+        for (int jn = 0; jn < NT; ++jn) part[((wk * MF + i) * NT + jn) * 64 + lane] = acc[i][jn];
+}
+
+template <int MODE, int FA, int FB, int MTMAX, int NT, int D, int NW, int OCC>
+__global__ void __launch_bounds__(64 * NW, OCC) grouped_tile_kernel(const grouped_dev_t P) {
+    constexpr int BM = 16 * MTMAX, BN = 16 * NT;
+    extern __shared__ g4f part[]; // [wavefront][fragment row][fragment column][lane]
     __shared__ int pick[2];
-    __shared__ int wave_tot[4];
-    __shared__ g4f part[4 * MT * NT * 64]; // [wk][wn][unit][lane]
+    __shared__ int wave_tot[NW];
     const mi355_grouped_desc_t &Dd = P.d;
     const int t = threadIdx.x, lane = t & 63;
     const int wave = __builtin_amdgcn_readfirstlane(t >> 6);
-    const long G = Dd.group_count, K = Dd.K, N = Dd.N;
+    const long G = Dd.group_count, N = Dd.N;
 
     // ---- which (group, row block) is slot blockIdx.y
     const int slot = blockIdx.y;
-    const long per = (G + 255) / 256; // groups per thread
+    const long per = (G + 64 * NW - 1) / (64 * NW); // groups per thread
     auto blocks_of = [&](long g) {
         long d0, s0;
         return (int)((grouped_rows(P, g, d0, s0) + BM - 1) / BM);
@@ -259,118 +398,47 @@ __global__ void __launch_bounds__(256) grouped_tile_kernel(const grouped_dev_t P
         }
     }
     __syncthreads();
-    const int g = __builtin_amdgcn_readfirstlane(pick[0]);
-    if (g < 0) return; // beyond the last tile
-    const long m_base = (long)__builtin_amdgcn_readfirstlane(pick[1]) * BM;
-    long dst0, src0;
-    const long rows = grouped_rows(P, g, dst0, src0); // > m_base
+    gtile_t T;
+    T.g = __builtin_amdgcn_readfirstlane(pick[0]);
+    if (T.g < 0) return; // beyond the last tile
+    T.m_base = (long)__builtin_amdgcn_readfirstlane(pick[1]) * BM;
+    T.rows = grouped_rows(P, T.g, T.dst0, T.src0); // > m_base
+    T.n0 = (long)blockIdx.x * BN;
+    const long here = T.rows - T.m_base < BM ? T.rows - T.m_base : BM;
+    const int mf = __builtin_amdgcn_readfirstlane((int)((here + 15) / 16)); // fragments of 16 rows the tile holds
 
-    // ---- operands
-    const int wn = wave % WN, wk = wave / WN;
-    const int j = lane & 15, q = lane >> 4;
-    const long row_bytes = K * ES;
-    const long n_wave = (long)blockIdx.x * BN + wn * (16 * NT);
-    const char *arow[MT], *bcol[NT];
-#pragma unroll
-    for (int i = 0; i < MT; ++i) {
-        long m = m_base + 16 * i + j;
-        m = m < rows ? m : rows - 1; // rows beyond the group read its last one (never stored)
-        arow[i] = (const char *)P.a.src + (src0 + m) * row_bytes + 32 * q;
+    // ---- K: the wavefronts take the 128-byte steps in turn, each over the whole tile
+    switch (mf) {
+        case 1: grouped_walk<MODE, FA, FB, 1, NT, D, NW>(P, T, part, wave, lane); break;
+        case 2:
+            if constexpr (MTMAX >= 2) grouped_walk<MODE, FA, FB, 2, NT, D, NW>(P, T, part, wave, lane);
+            break;
+        case 3:
+            if constexpr (MTMAX >= 3) grouped_walk<MODE, FA, FB, 3, NT, D, NW>(P, T, part, wave, lane);
+            break;
+        default:
+            if constexpr (MTMAX >= 4) grouped_walk<MODE, FA, FB, 4, NT, D, NW>(P, T, part, wave, lane);
+            break;
     }
-#pragma unroll
-    for (int jn = 0; jn < NT; ++jn) {
-        long n = n_wave + 16 * jn + j;
-        n = n < N ? n : N - 1;
-        bcol[jn] = (const char *)P.a.wei + ((long)g * Dd.wei_stride[0] + n * Dd.wei_stride[2]) * ES + 32 * q;
-    }
-    struct stage_t {
-        g8i a[MT], b[NT];
-    };
-    auto join = [](const g4i &lo, const g4i &hi) { return g8i {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]}; };
-    auto load = [&](long byte_off) __attribute__((always_inline)) {
-        stage_t f;
-#pragma unroll
-        for (int jn = 0; jn < NT; ++jn) {
-            const g4i *p = (const g4i *)(bcol[jn] + byte_off);
-            f.b[jn] = join(__builtin_nontemporal_load(p), __builtin_nontemporal_load(p + 1));
-        }
-#pragma unroll
-        for (int i = 0; i < MT; ++i) {
-            const g4i *p = (const g4i *)(arow[i] + byte_off);
-            f.a[i] = join(p[0], p[1]);
-        }
-        return f;
-    };
-    g4f acc[MT][NT];
-#pragma unroll
-    for (int i = 0; i < MT; ++i)
-#pragma unroll
-        for (int jn = 0; jn < NT; ++jn) acc[i][jn] = g4f {0.f, 0.f, 0.f, 0.f};
-    auto compute = [&](const stage_t &f) __attribute__((always_inline)) {
-#pragma unroll
-        for (int i = 0; i < MT; ++i)
-#pragma unroll
-            for (int jn = 0; jn < NT; ++jn) acc[i][jn] = grouped_mma<MODE, FA, FB>(f.b[jn], f.a[i], acc[i][jn]);
-    };
-
-    // ---- K: whole 128-byte steps wk, wk + WK, .. with D of them in flight
-    const long nfull = row_bytes / 128;
-    const int tail = (int)(row_bytes % 128); // a multiple of 32
-    if (nfull > wk) {
-        // this wavefront's steps: wk + WK * c, c < count; whole rounds of D run
-        // without a condition (loads beyond the end repeat the last step)
-        const long count = (nfull - wk + WK - 1) / WK;
-        auto step_off = [&](long c) { return (wk + WK * (c < count ? c : count - 1)) * 128; };
-        stage_t st[D];
-#pragma unroll
-        for (int d = 0; d < D; ++d) st[d] = load(step_off(d));
-        long c = 0;
-        for (; c + D <= count; c += D) {
-#pragma unroll
-            for (int d = 0; d < D; ++d) {
-                compute(st[d]);
-                st[d] = load(step_off(c + D + d));
-            }
-        }
-#pragma unroll
-        for (int d = 0; d < D; ++d)
-            if (c + d < count) compute(st[d]);
-    }
-    if (tail != 0 && wk == (int)(nfull % WK)) {
-        // lanes beyond K read the step's first 32 bytes instead and contribute zeros
-        const bool in = 32 * q < tail;
-        stage_t f = load(nfull * 128 - (in ? 0 : 32 * q));
-        if (!in) {
-#pragma unroll
-            for (int i = 0; i < MT; ++i) f.a[i] = g8i {0, 0, 0, 0, 0, 0, 0, 0};
-#pragma unroll
-            for (int jn = 0; jn < NT; ++jn) f.b[jn] = g8i {0, 0, 0, 0, 0, 0, 0, 0};
-        }
-        compute(f);
-    }
-
-    // ---- every wavefront leaves its accumulators in LDS; the 16 x 16 units of
-    // the tile are then finished by the four wavefronts in turn (one copy of the
-    // scales / bias / post-op / conversion code): lane (j, q) holds row j,
-    // columns 4 q .. 4 q + 3 of a unit
-#pragma unroll
-    for (int i = 0; i < MT; ++i)
-#pragma unroll
-        for (int jn = 0; jn < NT; ++jn) part[((wk * WN + wn) * MT * NT + i * NT + jn) * 64 + lane] = acc[i][jn];
     __syncthreads();
+
+    // ---- the 16 x 16 units of the tile are finished by the wavefronts in
+    // turn (one copy of the scales / bias / post-op / conversion code): lane
+    // (j, q) holds row j, columns 4 q .. 4 q + 3 of a unit
+    const int j = lane & 15, q = lane >> 4;
     const bool with_ss = Dd.src_scale_dt != MI355_DT_UNDEF, with_ws = Dd.wei_scale_dt != MI355_DT_UNDEF;
     const int dbits = dt_bits(Dd.dst_dt);
     const bool vec_ok = N % 4 == 0 && ((uintptr_t)P.a.dst % 16) == 0;
 #pragma nounroll
-    for (int u = wave; u < WN * MT * NT; u += 4) {
-        const int un = u / (MT * NT), i = (u / NT) % MT, jn = u % NT;
-        g4f sum = part[(un * MT * NT + i * NT + jn) * 64 + lane];
+    for (int u = wave; u < mf * NT; u += NW) {
+        const int i = u / NT, jn = u % NT;
+        g4f sum = part[u * 64 + lane];
 #pragma unroll
-        for (int w = 1; w < WK; ++w) sum += part[((w * WN + un) * MT * NT + i * NT + jn) * 64 + lane];
-        const long m = m_base + 16 * i + j;
-        const long nb = (long)blockIdx.x * BN + un * (16 * NT) + 16 * jn + 4 * q;
-        if (m >= rows || nb >= N) continue;
-        const float ss = with_ss ? load_float(Dd.src_scale_dt, P.a.src_scale, src0 + m) : 1.f;
+        for (int w = 1; w < NW; ++w) sum += part[(w * mf * NT + u) * 64 + lane];
+        const long m = T.m_base + 16 * i + j;
+        const long nb = T.n0 + 16 * jn + 4 * q;
+        if (m >= T.rows || nb >= N) continue;
+        const float ss = with_ss ? load_float(Dd.src_scale_dt, P.a.src_scale, T.src0 + m) : 1.f;
         const int nvalid = N - nb < 4 ? (int)(N - nb) : 4;
         uint32_t bits[4] = {0, 0, 0, 0};
 #pragma unroll
@@ -378,12 +446,12 @@ __global__ void __launch_bounds__(256) grouped_tile_kernel(const grouped_dev_t P
             if (e < nvalid) {
                 float v = sum[e];
                 if (with_ss) v *= ss;
-                if (with_ws) v *= load_float(Dd.wei_scale_dt, P.a.wei_scale, (long)g * N + nb + e);
-                v = grouped_finish(P, v, g, m, nb + e, dst0);
+                if (with_ws) v *= load_float(Dd.wei_scale_dt, P.a.wei_scale, T.g * N + nb + e);
+                v = grouped_finish(P, v, T.g, m, nb + e, T.dst0);
                 bits[e] = cvt_store_bits(Dd.dst_dt, v);
             }
         }
-        const long off = (dst0 + m) * N + nb;
+        const long off = (T.dst0 + m) * N + nb;
         if (vec_ok && nvalid == 4) {
             if (dbits == 32)
                 *(g4u *)((char *)P.a.dst + off * 4) = g4u {bits[0], bits[1], bits[2], bits[3]};
@@ -408,30 +476,36 @@ bool fp_any(int dt) {
 
 bool f8_dt(int dt) { return dt == MI355_DT_F8_E4M3 || dt == MI355_DT_F8_E5M2; }
 
-// 0: the thread-per-element kernel; 1: short groups (16 x 32 tiles, K split
-// between the wavefronts); 2: 64 x 128 tiles.  Decided on the descriptor alone.
+// the tile shapes of the matrix-core kernel: rows (16 * MTMAX) x columns (16 * NT)
+struct gshape_t {
+    int bm, bn;
+};
+constexpr gshape_t GSHAPES[4] = {{0, 0}, {16, 32}, {48, 64}, {64, 128}};
+
+// 0: the thread-per-element kernel; 1: 16 x 32 tiles (groups of a row or two:
+// many small workgroups); 2: 48 x 64, two workgroups per compute unit; 3: 64 x 128
+// for longer groups.  Decided on the descriptor.
 int tile_plan(const mi355_grouped_desc_t &d) {
     if (d.pattern != MI355_GROUPED_2DX3D) return 0;
-    if (const char *e = getenv("MI355_GROUPED_IMPL")) {
-        if (!strcmp(e, "ref")) return 0;
-    }
+    const char *env = getenv("MI355_GROUPED_IMPL");
+    if (env && !strcmp(env, "ref")) return 0;
     const bool f8 = f8_dt(d.src_dt) && f8_dt(d.wei_dt);
     const bool h16 = d.src_dt == d.wei_dt && (d.src_dt == MI355_DT_BF16 || d.src_dt == MI355_DT_F16);
     if (!f8 && !h16) return 0;
     const long es = f8 ? 1 : 2;
     if (d.wei_stride[1] != 1 || d.wei_stride[2] < d.K) return 0; // K-contiguous weights only
     if ((d.wei_stride[2] * es) % 16 != 0 || (d.wei_stride[0] * es) % 16 != 0 || (d.K * es) % 32 != 0) return 0;
+    if (d.wei_stride[2] * es > (1L << 24)) return 0; // 32-bit offsets inside a tile
     auto k_groups = [&](int dt, long gk) { return dt != MI355_DT_UNDEF && gk > 1 && gk != d.K; };
     if (k_groups(d.src_scale_dt, d.src_scale_gk) || k_groups(d.wei_scale_dt, d.wei_scale_gk)) return 0;
     if (d.src_zp_dt != MI355_DT_UNDEF || d.wei_zp_dt != MI355_DT_UNDEF) return 0;
     const long active = d.group_count < d.total ? d.group_count : d.total;
-    const int plan = d.total <= 2 * d.group_count ? 1 : 2;
-    const long slots = d.total / (plan == 1 ? 16 : 64) + active;
-    if (slots > 65535) return 0;
-    if (const char *e = getenv("MI355_GROUPED_IMPL")) {
-        if (!strcmp(e, "short")) return 1;
-        if (!strcmp(e, "tall")) return 2;
-    }
+    // by the average group: the row blocks of a longer group read its weights again
+    int plan = d.total <= 2 * d.group_count ? 1 : (d.total <= 48 * d.group_count ? 2 : 3);
+    if (env && !strcmp(env, "short")) plan = 1;
+    if (env && !strcmp(env, "tall")) plan = 2;
+    if (env && !strcmp(env, "wide")) plan = 3;
+    if (d.total / GSHAPES[plan].bm + active > 65535) return 0;
     return plan;
 }
 
@@ -439,13 +513,17 @@ template <int MODE, int FA, int FB>
 int launch_tiles(int plan, const grouped_dev_t &P, hipStream_t stream) {
     const mi355_grouped_desc_t &d = P.d;
     const long active = d.group_count < d.total ? d.group_count : d.total;
-    const int bm = plan == 1 ? 16 : 64, bn = plan == 1 ? 32 : 128;
-    dim3 grid((unsigned)((d.N + bn - 1) / bn), (unsigned)(d.total / bm + active));
-    if (plan == 1)
-        hipLaunchKernelGGL((grouped_tile_kernel<MODE, FA, FB, 1, 2, 1, 4, 4>), grid, dim3(256), 0, stream, P);
-    else
-        hipLaunchKernelGGL((grouped_tile_kernel<MODE, FA, FB, 4, 2, 4, 1, 2>), grid, dim3(256), 0, stream, P);
-    return hipGetLastError() == hipSuccess ? MI355_SUCCESS : MI355_RUNTIME_ERROR;
+    const gshape_t sh = GSHAPES[plan];
+    dim3 grid((unsigned)((d.N + sh.bn - 1) / sh.bn), (unsigned)(d.total / sh.bm + active));
+    auto go = [&](auto kern, int mtmax, int nt, int nw) -> int {
+        const int lds = nw * mtmax * nt * 64 * 16;
+        if (const int st = ensure_dynamic_lds((const void *)kern, lds, "mfma_grouped")) return st;
+        hipLaunchKernelGGL(kern, grid, dim3(64 * nw), lds, stream, P);
+        return hipGetLastError() == hipSuccess ? MI355_SUCCESS : MI355_RUNTIME_ERROR;
+    };
+    if (plan == 1) return go(grouped_tile_kernel<MODE, FA, FB, 1, 2, 4, 4, 1>, 1, 2, 4);
+    if (plan == 2) return go(grouped_tile_kernel<MODE, FA, FB, 3, 4, 2, 4, 2>, 3, 4, 4);
+    return go(grouped_tile_kernel<MODE, FA, FB, 4, 8, 2, 4, 1>, 4, 8, 4);
 }
 
 } // namespace

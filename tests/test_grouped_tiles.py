@@ -56,9 +56,9 @@ EXTRAS = [
 ]
 
 
-@pytest.fixture(params=["short", "tall"])
+@pytest.fixture(params=["short", "tall", "wide"])
 def tile_shape(request):
-    """Forces one of the two tile shapes of the matrix-core kernel."""
+    """Forces one of the three tile shapes of the matrix-core kernel."""
     old = os.environ.get("MI355_GROUPED_IMPL")
     os.environ["MI355_GROUPED_IMPL"] = request.param
     yield request.param
