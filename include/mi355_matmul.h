@@ -441,7 +441,7 @@ typedef struct mi355_grouped_args {
  *   "hip:ref_grouped:any"  everything else the descriptor rules allow: a thread
  *                          per dst element in the reference's operation order.
  * The environment variable MI355_GROUPED_IMPL=ref keeps every problem on the
- * second one (short / tall pick the matrix-core kernel's tile shape). */
+ * second one (short / tall / wide force one of the matrix-core kernel's tile shapes). */
 int mi355_grouped_matmul_query(const mi355_grouped_desc_t *desc);
 
 /* Name of the implementation a launch of `desc` uses ("" if none does). */

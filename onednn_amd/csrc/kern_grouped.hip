@@ -312,7 +312,14 @@ __device__ __forceinline__ void grouped_walk(const grouped_dev_t &P, const gtile
         // this wavefront's steps: wk + WK * c, c < count; whole rounds of D run
         // without a condition (loads beyond the end repeat the last step)
         const long count = (nfull - wk + WK - 1) / WK;
-        auto step_off = [&](long c) { return (wk + WK * (c < count ? c : count - 1)) * 128; };
+        // workgroups start at different places of K and wrap around: walking in step, they
+        // would all ask the same few memory channels at a time when K is a power of two
+        const long c0 = (long)((blockIdx.x * 5u + blockIdx.y * 3u) % (unsigned long)count);
+        auto step_off = [&](long c) {
+            long cr = (c < count ? c : count - 1) + c0;
+            cr = cr >= count ? cr - count : cr;
+            return (wk + WK * cr) * 128;
+        };
         stage_t st[D];
 #pragma unroll
         for (int d = 0; d < D; ++d) st[d] = load(step_off(d), 0);
@@ -352,19 +359,15 @@ __device__ __forceinline__ void grouped_walk(const grouped_dev_t &P, const gtile
         for (int jn = 0; jn < NT; ++jn) part[((wk * MF + i) * NT + jn) * 64 + lane] = acc[i][jn];
 }
 
-template <int MODE, int FA, int FB, int MTMAX, int NT, int D, int NW, int OCC>
-__global__ void __launch_bounds__(64 * NW, OCC) grouped_tile_kernel(const grouped_dev_t P) {
-    constexpr int BM = 16 * MTMAX, BN = 16 * NT;
-    extern __shared__ g4f part[]; // [wavefront][fragment row][fragment column][lane]
+// Which (group, row block) is slot `slot`: a block-wide prefix sum over the
+// groups' row-block counts.  False (for the whole workgroup) beyond the last tile.
+template <int BM, int NW>
+__device__ __forceinline__ bool grouped_find_tile(const grouped_dev_t &P, int slot, gtile_t &T) {
     __shared__ int pick[2];
     __shared__ int wave_tot[NW];
-    const mi355_grouped_desc_t &Dd = P.d;
     const int t = threadIdx.x, lane = t & 63;
     const int wave = __builtin_amdgcn_readfirstlane(t >> 6);
-    const long G = Dd.group_count, N = Dd.N;
-
-    // ---- which (group, row block) is slot blockIdx.y
-    const int slot = blockIdx.y;
+    const long G = P.d.group_count;
     const long per = (G + 64 * NW - 1) / (64 * NW); // groups per thread
     auto blocks_of = [&](long g) {
         long d0, s0;
@@ -398,11 +401,60 @@ __global__ void __launch_bounds__(64 * NW, OCC) grouped_tile_kernel(const groupe
         }
     }
     __syncthreads();
-    gtile_t T;
     T.g = __builtin_amdgcn_readfirstlane(pick[0]);
-    if (T.g < 0) return; // beyond the last tile
+    if (T.g < 0) return false;
     T.m_base = (long)__builtin_amdgcn_readfirstlane(pick[1]) * BM;
     T.rows = grouped_rows(P, T.g, T.dst0, T.src0); // > m_base
+    return true;
+}
+
+// Scales, bias, post-ops, conversion and store of four consecutive columns nb .. nb + 3 of row m
+// (a lane's share of a 16 x 16 unit).
+__device__ __forceinline__ void grouped_store_quad(const grouped_dev_t &P, const gtile_t &T, g4f sum, long m, long nb) {
+    const mi355_grouped_desc_t &Dd = P.d;
+    const long N = Dd.N;
+    if (m >= T.rows || nb >= N) return;
+    const bool with_ss = Dd.src_scale_dt != MI355_DT_UNDEF, with_ws = Dd.wei_scale_dt != MI355_DT_UNDEF;
+    const int dbits = dt_bits(Dd.dst_dt);
+    const bool vec_ok = N % 4 == 0 && ((uintptr_t)P.a.dst % 16) == 0;
+    const float ss = with_ss ? load_float(Dd.src_scale_dt, P.a.src_scale, T.src0 + m) : 1.f;
+    const int nvalid = N - nb < 4 ? (int)(N - nb) : 4;
+    uint32_t bits[4] = {0, 0, 0, 0};
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+        if (e < nvalid) {
+            float v = sum[e];
+            if (with_ss) v *= ss;
+            if (with_ws) v *= load_float(Dd.wei_scale_dt, P.a.wei_scale, T.g * N + nb + e);
+            v = grouped_finish(P, v, T.g, m, nb + e, T.dst0);
+            bits[e] = cvt_store_bits(Dd.dst_dt, v);
+        }
+    }
+    const long off = (T.dst0 + m) * N + nb;
+    if (vec_ok && nvalid == 4) {
+        if (dbits == 32)
+            *(g4u *)((char *)P.a.dst + off * 4) = g4u {bits[0], bits[1], bits[2], bits[3]};
+        else
+            *(g2u *)((char *)P.a.dst + off * 2) = g2u {bits[0] | (bits[1] << 16), bits[2] | (bits[3] << 16)};
+    } else {
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            if (e < nvalid) {
+                if (dbits == 32) ((uint32_t *)P.a.dst)[off + e] = bits[e];
+                else ((uint16_t *)P.a.dst)[off + e] = (uint16_t)bits[e];
+            }
+        }
+    }
+}
+
+template <int MODE, int FA, int FB, int MTMAX, int NT, int D, int NW, int OCC>
+__global__ void __launch_bounds__(64 * NW, OCC) grouped_tile_kernel(const grouped_dev_t P) {
+    constexpr int BM = 16 * MTMAX, BN = 16 * NT;
+    extern __shared__ g4f part[]; // [wavefront][fragment row][fragment column][lane]
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    gtile_t T;
+    if (!grouped_find_tile<BM, NW>(P, blockIdx.y, T)) return;
     T.n0 = (long)blockIdx.x * BN;
     const long here = T.rows - T.m_base < BM ? T.rows - T.m_base : BM;
     const int mf = __builtin_amdgcn_readfirstlane((int)((here + 15) / 16)); // fragments of 16 rows the tile holds
@@ -426,46 +478,244 @@ __global__ void __launch_bounds__(64 * NW, OCC) grouped_tile_kernel(const groupe
     // turn (one copy of the scales / bias / post-op / conversion code): lane
     // (j, q) holds row j, columns 4 q .. 4 q + 3 of a unit
     const int j = lane & 15, q = lane >> 4;
-    const bool with_ss = Dd.src_scale_dt != MI355_DT_UNDEF, with_ws = Dd.wei_scale_dt != MI355_DT_UNDEF;
-    const int dbits = dt_bits(Dd.dst_dt);
-    const bool vec_ok = N % 4 == 0 && ((uintptr_t)P.a.dst % 16) == 0;
 #pragma nounroll
     for (int u = wave; u < mf * NT; u += NW) {
         const int i = u / NT, jn = u % NT;
         g4f sum = part[u * 64 + lane];
 #pragma unroll
         for (int w = 1; w < NW; ++w) sum += part[(w * mf * NT + u) * 64 + lane];
-        const long m = T.m_base + 16 * i + j;
-        const long nb = T.n0 + 16 * jn + 4 * q;
-        if (m >= T.rows || nb >= N) continue;
-        const float ss = with_ss ? load_float(Dd.src_scale_dt, P.a.src_scale, T.src0 + m) : 1.f;
-        const int nvalid = N - nb < 4 ? (int)(N - nb) : 4;
-        uint32_t bits[4] = {0, 0, 0, 0};
+        grouped_store_quad(P, T, sum, T.m_base + 16 * i + j, T.n0 + 16 * jn + 4 * q);
+    }
+}
+
+// ---- the second tile shape of "hip:mfma_grouped": columns split between the
+// wavefronts, src rows shared through LDS.
+//
+// A workgroup owns (group, up to 16 * MTMAX rows, 256 columns); each of its four
+// wavefronts owns 64 columns (four fragments) and walks all of K with D steps
+// of its weights in flight in registers (whole-line loads + lane exchange as
+// above).  The src rows of the tile are needed by all four wavefronts: they
+// are brought to LDS once per workgroup, 512 bytes of K (four steps) per row at
+// a time, by direct-to-LDS loads that fetch whole lines (8 rows x 128 bytes per
+// instruction), double buffered, one barrier per four steps.  Per byte of
+// weights a quarter of the src traffic of the 64-column tiles goes through the
+// vector memory path, which is what bounds these kernels.
+//
+// LDS layout of one (fragment, step) block of 16 rows x 128 bytes: the 16-byte
+// chunk c of row r sits in slot 8 r + (c ^ (r / 2)); a direct-to-LDS
+// instruction fills 64 consecutive slots, so its lane L fetches row L / 8 (of
+// the block's lower or upper half), chunk (L % 8) ^ (row / 2); the fragment
+// read of lanes (j, q) -- slots 8 j + (q ^ (j / 2)) -- touches every bank once
+// per 16 lanes.
+typedef const g4i __attribute__((address_space(3))) *lds_g4i_ptr_t;
+typedef g4f __attribute__((address_space(3))) *lds_g4f_ptr_t;
+
+// lane i brings 16 bytes from sbase + voff to LDS byte address lds_addr + 16 i
+__device__ __forceinline__ void grouped_dma16(const void *sbase, unsigned voff, unsigned lds_addr) {
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
+                 :
+                 : "s"(lds_addr), "v"(voff), "s"(sbase)
+                 : "memory", "m0");
+}
+
+// NT: fragments of 16 columns per wavefront.  Leaves the wavefront's MF x NT accumulators in LDS at
+// lds0 + (wave * MF * NT + unit) * 1024.
+template <int MODE, int FA, int FB, int MF, int NT, int D>
+__device__ __forceinline__ void grouped_walk_nsplit(const grouped_dev_t &P, const gtile_t &T, unsigned lds0, int wave,
+        int lane) {
+    constexpr int CH = 4; // steps per src chunk in LDS
+    static_assert(CH % D == 0, "a step's register stage must not depend on the chunk");
+    constexpr int ES = MODE == GM_F8 ? 1 : 2;
+    constexpr unsigned ABUF = MF * CH * 2048; // bytes of one src buffer
+    const mi355_grouped_desc_t &Dd = P.d;
+    const int j = lane & 15, q = lane >> 4;
+    const long row_bytes = Dd.K * ES;
+    const long nfull = row_bytes / 128;
+    const int tail = (int)(row_bytes % 128); // a multiple of 32
+    const long nsteps = nfull + (tail != 0);
+    const long nchunks = (nsteps + CH - 1) / CH;
+
+    // ---- weights: as in grouped_walk, for this wavefront's 64 columns
+    const int half = j >> 3;
+    const uint32_t chunk = 16 * (q + 4 * half);
+    const long pitch_b = Dd.wei_stride[2] * ES;
+    const char *bbase = (const char *)P.a.wei + (T.g * Dd.wei_stride[0] + T.n0 * Dd.wei_stride[2]) * ES;
+    uint32_t boff[NT][2];
+#pragma unroll
+    for (int jn = 0; jn < NT; ++jn)
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+            long n = T.n0 + 16 * NT * wave + 16 * jn + 8 * h + (j & 7);
+            n = n < Dd.N ? n : Dd.N - 1;
+            boff[jn][h] = (uint32_t)((n - T.n0) * pitch_b) + chunk;
+        }
+    struct stage_t {
+        g4i b[NT][2];
+    };
+    // A lane whose chunk lies beyond K in the tail step fetches the step's first chunk
+    // instead (the tail holds at least 32 bytes); steps beyond the last repeat it.
+    const uint32_t b_back = chunk + 16 <= (uint32_t)tail ? 0 : chunk;
+    auto load_b = [&](long s) __attribute__((always_inline)) {
+        stage_t f;
+        s = s < nsteps ? s : nsteps - 1;
+        const uint32_t back = s >= nfull ? b_back : 0;
+#pragma unroll
+        for (int jn = 0; jn < NT; ++jn)
+#pragma unroll
+            for (int h = 0; h < 2; ++h) f.b[jn][h] = *(const g4i *)(bbase + s * 128 + (boff[jn][h] - back));
+        return f;
+    };
+    auto settle = [&](const g4i (&r)[2]) __attribute__((always_inline)) {
+        g8i out;
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
-            if (e < nvalid) {
-                float v = sum[e];
-                if (with_ss) v *= ss;
-                if (with_ws) v *= load_float(Dd.wei_scale_dt, P.a.wei_scale, T.g * N + nb + e);
-                v = grouped_finish(P, v, T.g, m, nb + e, T.dst0);
-                bits[e] = cvt_store_bits(Dd.dst_dt, v);
-            }
+            const int send = half ? r[0][e] : r[1][e];
+            const int recv = __builtin_amdgcn_update_dpp(0, send, 0x128 /* row_ror:8 */, 0xf, 0xf, false);
+            out[e] = half ? recv : r[0][e];
+            out[4 + e] = half ? r[1][e] : recv;
         }
-        const long off = (T.dst0 + m) * N + nb;
-        if (vec_ok && nvalid == 4) {
-            if (dbits == 32)
-                *(g4u *)((char *)P.a.dst + off * 4) = g4u {bits[0], bits[1], bits[2], bits[3]};
-            else
-                *(g2u *)((char *)P.a.dst + off * 2) = g2u {bits[0] | (bits[1] << 16), bits[2] | (bits[3] << 16)};
-        } else {
+        return out;
+    };
+
+    // ---- src: this wavefront's share of a chunk's direct-to-LDS loads.  Instruction
+    // wave + 4 x of the chunk's 2 * MF * CH fills half (wave % 2) of block (wave + 4 x) / 2
+    // = (fragment, step); the row and chunk a lane fetches are the same in all of them.
+    constexpr int NDMA = 2 * MF * CH / 4;
+    const char *abase = (const char *)P.a.src + (T.src0 + T.m_base) * row_bytes;
+    const int a_r = 8 * (wave & 1) + (lane >> 3);
+    const uint32_t a_chunk = 16 * ((lane & 7) ^ (a_r >> 1));
+    const uint32_t a_back = a_chunk + 16 <= (uint32_t)tail ? 0 : a_chunk;
+    uint32_t a_row[NDMA]; // byte offset of the lane's row, per instruction (the fragment differs)
 #pragma unroll
-            for (int e = 0; e < 4; ++e) {
-                if (e < nvalid) {
-                    if (dbits == 32) ((uint32_t *)P.a.dst)[off + e] = bits[e];
-                    else ((uint16_t *)P.a.dst)[off + e] = (uint16_t)bits[e];
+    for (int x = 0; x < NDMA; ++x) {
+        const int i = ((wave + 4 * x) >> 1) / CH;
+        long m = T.m_base + 16 * i + a_r;
+        m = m < T.rows ? m : T.rows - 1; // rows beyond the group read its last one (never stored)
+        a_row[x] = (uint32_t)((m - T.m_base) * row_bytes);
+    }
+    auto issue_a = [&](long c, int which) __attribute__((always_inline)) {
+        const unsigned buf = lds0 + (unsigned)which * ABUF;
+#pragma unroll
+        for (int x = 0; x < NDMA; ++x) {
+            const int inst = wave + 4 * x, blk = inst >> 1;
+            long s = c * CH + blk % CH;
+            s = s < nsteps ? s : nsteps - 1;
+            const uint32_t voff = a_row[x] + a_chunk - (s >= nfull ? a_back : 0);
+            grouped_dma16(abase + s * 128, voff, buf + (unsigned)blk * 2048 + (unsigned)(inst & 1) * 1024);
+        }
+    };
+    const unsigned a_lo = 16 * (8 * j + (q ^ (j >> 1))), a_hi = 16 * (8 * j + ((4 + q) ^ (j >> 1)));
+    const bool lo_in = 16 * q + 16 <= tail, hi_in = 64 + 16 * q + 16 <= tail; // the lane's chunks in the tail step
+
+    g4f acc[MF][NT];
+#pragma unroll
+    for (int i = 0; i < MF; ++i)
+#pragma unroll
+        for (int jn = 0; jn < NT; ++jn) acc[i][jn] = g4f {0.f, 0.f, 0.f, 0.f};
+
+    // chunks are walked from a place of K that differs between workgroups, wrapping around
+    // (see grouped_walk); x counts chunks in walking order, p steps
+    const long c0 = (long)((blockIdx.x * 5u + blockIdx.y * 3u) % (unsigned long)nchunks);
+    auto chunk_at = [&](long x) {
+        const long cr = x + c0;
+        return cr >= nchunks ? cr - nchunks : cr;
+    };
+    auto step_at = [&](long p) {
+        p = p < nchunks * CH ? p : nchunks * CH - 1;
+        return chunk_at(p / CH) * CH + p % CH;
+    };
+    stage_t st[D];
+    issue_a(chunk_at(0), 0);
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int d = 0; d < D; ++d) st[d] = load_b(step_at(d));
+    for (long x = 0; x < nchunks; ++x) {
+        // memory operations return in order: once at most the D stages of weights issued
+        // after this wavefront's part of the chunk are in flight, that part has landed
+        asm volatile("s_waitcnt vmcnt(%0)" ::"n"(D * NT * 2) : "memory");
+        __syncthreads();
+        if (x + 1 < nchunks) issue_a(chunk_at(x + 1), (x + 1) & 1); // into the buffer whose readers passed the barrier
+        __builtin_amdgcn_sched_barrier(0);
+        const unsigned buf = lds0 + (unsigned)(x & 1) * ABUF;
+        const long c = chunk_at(x);
+#pragma unroll
+        for (int t = 0; t < CH; ++t) {
+            const long s = c * CH + t;
+            if (s < nsteps) {
+                g8i a[MF];
+#pragma unroll
+                for (int i = 0; i < MF; ++i) {
+                    const unsigned blk = buf + (unsigned)(i * CH + t) * 2048;
+                    const g4i lo = *(lds_g4i_ptr_t)(size_t)(blk + a_lo), hi = *(lds_g4i_ptr_t)(size_t)(blk + a_hi);
+                    a[i] = g8i {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+                }
+                const bool is_tail = s >= nfull;
+                if (is_tail) {
+#pragma unroll
+                    for (int i = 0; i < MF; ++i)
+#pragma unroll
+                        for (int e = 0; e < 4; ++e) {
+                            if (!lo_in) a[i][e] = 0;
+                            if (!hi_in) a[i][4 + e] = 0;
+                        }
+                }
+#pragma unroll
+                for (int jn = 0; jn < NT; ++jn) {
+                    g8i w = settle(st[t % D].b[jn]);
+                    if (is_tail) {
+#pragma unroll
+                        for (int e = 0; e < 4; ++e) {
+                            if (!lo_in) w[e] = 0;
+                            if (!hi_in) w[4 + e] = 0;
+                        }
+                    }
+#pragma unroll
+                    for (int i = 0; i < MF; ++i) acc[i][jn] = grouped_mma<MODE, FA, FB>(w, a[i], acc[i][jn]);
                 }
             }
+            st[t % D] = load_b(step_at(x * CH + t + D));
+            __builtin_amdgcn_sched_barrier(0);
         }
+    }
+    __syncthreads(); // every wavefront is done with the src buffers
+#pragma unroll
+    for (int i = 0; i < MF; ++i)
+#pragma unroll
+        for (int jn = 0; jn < NT; ++jn)
+            *(lds_g4f_ptr_t)(size_t)(lds0 + (unsigned)((wave * MF * NT + i * NT + jn) * 64 + lane) * 16) = acc[i][jn];
+}
+
+template <int MODE, int FA, int FB, int MTMAX, int NT, int D>
+__global__ void __launch_bounds__(256, 2) grouped_nsplit_kernel(const grouped_dev_t P) {
+    constexpr int BM = 16 * MTMAX, BN = 64 * NT;
+    extern __shared__ g4f part[]; // two src buffers of MTMAX * 8 KB; afterwards the accumulators
+    const unsigned lds0 = (unsigned)(size_t)(__attribute__((address_space(3))) char *)part;
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    gtile_t T;
+    if (!grouped_find_tile<BM, 4>(P, blockIdx.y, T)) return;
+    T.n0 = (long)blockIdx.x * BN;
+    const long here = T.rows - T.m_base < BM ? T.rows - T.m_base : BM;
+    const int mf = __builtin_amdgcn_readfirstlane((int)((here + 15) / 16));
+    switch (mf) {
+        case 1: grouped_walk_nsplit<MODE, FA, FB, 1, NT, D>(P, T, lds0, wave, lane); break;
+        case 2:
+            if constexpr (MTMAX >= 2) grouped_walk_nsplit<MODE, FA, FB, 2, NT, D>(P, T, lds0, wave, lane);
+            break;
+        case 3:
+            if constexpr (MTMAX >= 3) grouped_walk_nsplit<MODE, FA, FB, 3, NT, D>(P, T, lds0, wave, lane);
+            break;
+        default:
+            if constexpr (MTMAX >= 4) grouped_walk_nsplit<MODE, FA, FB, 4, NT, D>(P, T, lds0, wave, lane);
+            break;
+    }
+    // a wavefront finishes its own columns, one 16 x 16 unit at a time (one copy of the code)
+    const int j = lane & 15, q = lane >> 4;
+#pragma nounroll
+    for (int u = 0; u < mf * NT; ++u) {
+        const int i = u / NT, jn = u % NT;
+        const g4f sum = *(lds_g4f_ptr_t)(size_t)(lds0 + (unsigned)((wave * mf * NT + u) * 64 + lane) * 16);
+        grouped_store_quad(P, T, sum, T.m_base + 16 * i + j, T.n0 + 16 * NT * wave + 16 * jn + 4 * q);
     }
 }
 
@@ -480,11 +730,12 @@ bool f8_dt(int dt) { return dt == MI355_DT_F8_E4M3 || dt == MI355_DT_F8_E5M2; }
 struct gshape_t {
     int bm, bn;
 };
-constexpr gshape_t GSHAPES[4] = {{0, 0}, {16, 32}, {48, 64}, {64, 128}};
+constexpr gshape_t GSHAPES[4] = {{0, 0}, {16, 32}, {48, 64}, {64, 256}};
 
-// 0: the thread-per-element kernel; 1: 16 x 32 tiles (groups of a row or two:
-// many small workgroups); 2: 48 x 64, two workgroups per compute unit; 3: 64 x 128
-// for longer groups.  Decided on the descriptor.
+// 0: the thread-per-element kernel; 1: 16 x 32 tiles, K split between the
+// wavefronts (groups of a row or two: many small workgroups); 2: 48 x 64, K
+// split, two workgroups per compute unit; 3: 64 x 256, columns split, src rows
+// through LDS.  Decided on the descriptor.
 int tile_plan(const mi355_grouped_desc_t &d) {
     if (d.pattern != MI355_GROUPED_2DX3D) return 0;
     const char *env = getenv("MI355_GROUPED_IMPL");
@@ -500,8 +751,12 @@ int tile_plan(const mi355_grouped_desc_t &d) {
     if (k_groups(d.src_scale_dt, d.src_scale_gk) || k_groups(d.wei_scale_dt, d.wei_scale_gk)) return 0;
     if (d.src_zp_dt != MI355_DT_UNDEF || d.wei_zp_dt != MI355_DT_UNDEF) return 0;
     const long active = d.group_count < d.total ? d.group_count : d.total;
-    // by the average group: the row blocks of a longer group read its weights again
-    int plan = d.total <= 2 * d.group_count ? 1 : (d.total <= 48 * d.group_count ? 2 : 3);
+    // Groups of a row or two: the small tiles.  Otherwise the 256-column tiles (a quarter of
+    // the src traffic per byte of weights), unless they are too few to fill the device or
+    // the rows are not whole lines (K not a multiple of 128 bytes: measured slower there).
+    int plan = 3;
+    if (d.total <= 2 * d.group_count) plan = 1;
+    else if ((d.K * es) % 128 != 0 || (d.N + 255) / 256 * active < 256) plan = 2;
     if (env && !strcmp(env, "short")) plan = 1;
     if (env && !strcmp(env, "tall")) plan = 2;
     if (env && !strcmp(env, "wide")) plan = 3;
@@ -523,7 +778,8 @@ int launch_tiles(int plan, const grouped_dev_t &P, hipStream_t stream) {
     };
     if (plan == 1) return go(grouped_tile_kernel<MODE, FA, FB, 1, 2, 4, 4, 1>, 1, 2, 4);
     if (plan == 2) return go(grouped_tile_kernel<MODE, FA, FB, 3, 4, 2, 4, 2>, 3, 4, 4);
-    return go(grouped_tile_kernel<MODE, FA, FB, 4, 8, 2, 4, 1>, 4, 8, 4);
+    // two src buffers of 4 fragments x 4 steps; the accumulators fit the same space
+    return go(grouped_nsplit_kernel<MODE, FA, FB, 4, 4, 2>, 4, 4, 4);
 }
 
 } // namespace

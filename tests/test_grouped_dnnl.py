@@ -211,3 +211,30 @@ def test_execute_2dx2d(gpu, oracle, dtag):
                         dnnl.ARG_WEIGHTS: dnnl.grouped_memory(wmd, eng, p.wei, p.other_offsets), dnnl.ARG_DST: dst})
     strm.wait()
     assert np.array_equal(dst.read(np.uint8), want)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("sdt,wdt", [(cabi.DT_F8_E4M3, cabi.DT_F8_E4M3), (BF16, BF16)], ids=["e4m3", "bf16"])
+def test_execute_2dx3d_on_the_matrix_cores(gpu, oracle, sdt, wdt):
+    """The layout of the reference's GPU grouped tests (--wtag=acb, --attr-scales=src:1:f32+wei:5:f32 for fp8) goes
+    to hip:mfma_grouped; exact data, so the oracle's bits are the expectation."""
+    kw = dict(src_scale="row", wei_scale="col") if sdt != BF16 else {}
+    p, _ = gc.case_2dx3d([10, 20, 30, 40], 160, 36, src_dt=sdt, wei_dt=wdt, dst_dt=BF16, wtag="acb", bias=True,
+                         post_ops=("relu",), **kw)
+    st, want = oracle.run_oracle_grouped(p)
+    assert st == cabi.SUCCESS
+    eng = dnnl.engine(dnnl.gpu, 0)
+    strm = dnnl.stream(eng)
+    smd, wmd, dmd, bmd = mds(p)
+    attr, extra = attr_of(p)
+    pd = dnnl.matmul_primitive_desc(eng, smd, wmd, dmd, bias_md=bmd, attr=attr)
+    assert pd.impl_info_str() == "hip:mfma_grouped"
+    prim = dnnl.matmul(pd)
+    dst = dnnl.grouped_memory(dmd, eng, p.initial_dst(), p.other_offsets)
+    args = {dnnl.ARG_SRC: dnnl.grouped_memory(smd, eng, p.src, p.src_offsets),
+            dnnl.ARG_WEIGHTS: dnnl.memory(wmd, eng, p.wei), dnnl.ARG_DST: dst, dnnl.ARG_BIAS: dnnl.memory(bmd, eng, p.bias)}
+    for arg, (md, data, offsets) in extra.items():
+        args[arg] = dnnl.memory(md, eng, data)
+    prim.execute(strm, args)
+    strm.wait()
+    assert np.array_equal(dst.read(np.uint8), want)
