@@ -52,7 +52,9 @@ typedef enum {
     dnnl_s4 = 11,
     dnnl_u4 = 12,
     dnnl_e8m0 = 13,
-    dnnl_f4_e2m1 = 14
+    dnnl_f4_e2m1 = 14,
+    dnnl_f4_e3m0 = 15, /* not offered */
+    dnnl_s64 = 16      /* the dropout seed and offset only */
 } dnnl_data_type_t;
 
 #define DNNL_MAX_NDIMS 12                  /* dnnl_common_types.h:123 */
@@ -185,6 +187,9 @@ typedef enum {
 /* dnnl_types.h:2448-2458 */
 typedef enum { dnnl_scratchpad_mode_library = 0, dnnl_scratchpad_mode_user = 1 } dnnl_scratchpad_mode_t;
 
+/* dnnl_types.h:2460-2467 */
+typedef enum { dnnl_rounding_mode_environment = 0, dnnl_rounding_mode_stochastic = 1 } dnnl_rounding_mode_t;
+
 /* dnnl_types.h:2846-2930 */
 typedef enum {
     dnnl_query_undef = 0,
@@ -225,9 +230,17 @@ typedef enum {
 #define DNNL_ARG_SRC_1 2
 #define DNNL_ARG_SRC_2 3 /* dnnl_types.h:2562: the condition of a binary select post-op */
 #define DNNL_ARG_DST 17
+#define DNNL_ARG_DIFF_SRC 129     /* dnnl_types.h:2649-2652; named by the rounding-mode rule only */
+#define DNNL_ARG_DIFF_WEIGHTS 161 /* dnnl_types.h:2697-2700 */
 #define DNNL_ARG_WEIGHTS 33
 #define DNNL_ARG_BIAS 41
 #define DNNL_ARG_SCRATCHPAD 80
+/* dnnl_types.h:2737-2750 */
+#define DNNL_ARG_ATTR_DROPOUT_OFFSET 507
+#define DNNL_ARG_ATTR_ROUNDING_SEED 508 /* accepted and not read: ref_matmul_t seeds the rounding with the dropout seed */
+#define DNNL_ARG_ATTR_DROPOUT_MASK 509
+#define DNNL_ARG_ATTR_DROPOUT_PROBABILITY 510
+#define DNNL_ARG_ATTR_DROPOUT_SEED 511
 #define DNNL_ARG_ATTR_PRECOMPUTED_REDUCTIONS 512
 #define DNNL_ARG_ATTR_SCALES 4096
 #define DNNL_ARG_ATTR_ZERO_POINTS 8192
@@ -328,6 +341,20 @@ dnnl_status_t dnnl_primitive_attr_get_fpmath_mode_v2(const_dnnl_primitive_attr_t
         dnnl_fpmath_mode_t *mode, int *apply_to_int);
 dnnl_status_t dnnl_primitive_attr_set_accumulation_mode(dnnl_primitive_attr_t attr, dnnl_accumulation_mode_t mode);
 dnnl_status_t dnnl_primitive_attr_set_scratchpad_mode(dnnl_primitive_attr_t attr, dnnl_scratchpad_mode_t mode);
+/* dnnl.h:276-329: dropout applied to the matmul result after the bias and before the post-ops
+ * (ref_matmul_t, floating-point src, plain row-major dst).  mask_desc: u8 and laid out like dst, or a zero
+ * descriptor (no mask is written).  Execute arguments: DNNL_ARG_ATTR_DROPOUT_PROBABILITY (f32),
+ * _SEED (seed_dt: s32 or s64), _OFFSET (s64, with use_offset), _MASK; with use_host_scalars the first
+ * three are host-scalar memory objects. */
+dnnl_status_t dnnl_primitive_attr_get_dropout(const_dnnl_primitive_attr_t attr, const_dnnl_memory_desc_t *mask_desc);
+dnnl_status_t dnnl_primitive_attr_set_dropout(dnnl_primitive_attr_t attr, const_dnnl_memory_desc_t mask_desc);
+dnnl_status_t dnnl_primitive_attr_get_dropout_v2(const_dnnl_primitive_attr_t attr, const_dnnl_memory_desc_t *mask_desc,
+        dnnl_data_type_t *seed_dt, int *use_offset, int *use_host_scalars);
+dnnl_status_t dnnl_primitive_attr_set_dropout_v2(dnnl_primitive_attr_t attr, const_dnnl_memory_desc_t mask_desc,
+        dnnl_data_type_t seed_dt, int use_offset, int use_host_scalars);
+/* dnnl.h:661-679: stochastic rounding of DNNL_ARG_DST (bf16 / f16 / fp8 / f32 dst of ref_matmul_t) */
+dnnl_status_t dnnl_primitive_attr_set_rounding(dnnl_primitive_attr_t attr, int arg, dnnl_rounding_mode_t mode);
+dnnl_status_t dnnl_primitive_attr_get_rounding(dnnl_primitive_attr_t attr, int arg, dnnl_rounding_mode_t *mode);
 dnnl_status_t dnnl_primitive_attr_get_scratchpad_mode(const_dnnl_primitive_attr_t attr,
         dnnl_scratchpad_mode_t *mode);
 dnnl_status_t dnnl_primitive_attr_set_scales_mask(dnnl_primitive_attr_t attr, int arg, int mask);

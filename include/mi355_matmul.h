@@ -224,6 +224,22 @@ typedef struct mi355_post_op {
                              (batch, M, N); 0 on broadcast dims */
 } mi355_post_op_t;
 
+/* Dropout and stochastic rounding of ref_matmul_t (src/cpu/matmul/ref_matmul.cpp:61-67,
+ * 248-331; ref_dropout src/cpu/primitive_attr_postops.cpp:296-310;
+ * stochastic_round_fwd and the Philox generator src/common/math_utils.hpp:458-574).
+ * Floating-point src only, the generic kernel only, dst dense row-major.
+ *   dropout: after the bias and before the post-ops, element idx (its offset in
+ *   dst) is kept when philox(idx, seed[, offset]) > UINT32_MAX * p and scaled by
+ *   1 / (1 - p), else zeroed; the keep flags go to the mask.
+ *   stochastic rounding of a bf16 / f16 / fp8 dst: random bits below the dst
+ *   type's precision are added to the f32 value before truncation; the seed is
+ *   the dropout seed (0 without dropout), as in the reference's implementation. */
+#define MI355_RND_DROPOUT 1
+#define MI355_RND_DROPOUT_MASK 2
+#define MI355_RND_SEED_S64 4
+#define MI355_RND_DROPOUT_OFFSET 8
+#define MI355_RND_DST_STOCHASTIC 16
+
 typedef struct mi355_matmul_desc {
     int64_t batch, M, N, K;
     int32_t src_dt, wei_dt, dst_dt, bias_dt; /* bias_dt UNDEF = no bias */
@@ -244,7 +260,7 @@ typedef struct mi355_matmul_desc {
     int32_t impl; /* MI355_IMPL_*; AUTO picks the fastest applicable */
     int32_t wei_packing; /* MI355_WEI_PACK_* */
     int32_t dst_scale_dynamic; /* MI355_DST_DYNAMIC_* */
-    int32_t reserved;
+    int32_t rnd_flags;         /* MI355_RND_*: dropout and stochastic rounding */
 } mi355_matmul_desc_t;
 
 typedef struct mi355_matmul_args {
@@ -254,6 +270,11 @@ typedef struct mi355_matmul_args {
     const void *src_zp, *wei_zp, *dst_zp;
     const void *src_pr;
     const void *po_arg[MI355_MAX_POST_OPS]; /* binary src1 / prelu weights */
+    /* MI355_RND_DROPOUT: probability (one f32), seed (one s32 or s64), offset
+     * (one s64, with MI355_RND_DROPOUT_OFFSET), all in device memory; the mask
+     * (u8, laid out like dst) is written with MI355_RND_DROPOUT_MASK */
+    const void *dropout_p, *dropout_seed, *dropout_offset;
+    void *dropout_mask;
 } mi355_matmul_args_t;
 
 /* ---- device, memory, stream, events (engine / stream / memory_storage) --- */

@@ -68,8 +68,11 @@ class MatmulDesc(C.Structure):
         ("dst_scale_mode", C.c_int32), ("n_post_ops", C.c_int32),
         ("post_ops", PostOp * MAX_POST_OPS),
         ("impl", C.c_int32), ("wei_packing", C.c_int32),
-        ("dst_scale_dynamic", C.c_int32), ("reserved", C.c_int32),
+        ("dst_scale_dynamic", C.c_int32), ("rnd_flags", C.c_int32),
     ]
+
+
+RND_DROPOUT, RND_DROPOUT_MASK, RND_SEED_S64, RND_DROPOUT_OFFSET, RND_DST_STOCHASTIC = 1, 2, 4, 8, 16
 
 
 class MatmulArgs(C.Structure):
@@ -79,6 +82,8 @@ class MatmulArgs(C.Structure):
         ("src_zp", C.c_void_p), ("wei_zp", C.c_void_p), ("dst_zp", C.c_void_p),
         ("src_pr", C.c_void_p),
         ("po_arg", C.c_void_p * MAX_POST_OPS),
+        ("dropout_p", C.c_void_p), ("dropout_seed", C.c_void_p), ("dropout_offset", C.c_void_p),
+        ("dropout_mask", C.c_void_p),
     ]
 
 

@@ -155,6 +155,8 @@ static int impl_supported(const mi355_matmul_desc_t &d, int impl) {
     if ((d.dst_scale_dynamic == MI355_DST_DYNAMIC_FP || (d.dst_scale_dynamic && !is_f8_dt(d.dst_dt)))
             && impl != MI355_IMPL_REF)
         return MI355_UNIMPLEMENTED;
+    // dropout and stochastic rounding: generic kernel only
+    if (d.rnd_flags != 0 && impl != MI355_IMPL_REF) return MI355_UNIMPLEMENTED;
     switch (impl) {
         case MI355_IMPL_REF: return ref_supported(d);
         case MI355_IMPL_I8_MFMA: return i8_supported(d);
@@ -216,6 +218,14 @@ static int build_problem(const mi355_matmul_desc_t &d, const mi355_matmul_args_t
     P.wei_packing = d.wei_packing;
     P.dst_dynamic = d.dst_scale_dynamic;
     P.src = a.src; P.wei = a.wei; P.bias = a.bias; P.dst = a.dst;
+    P.rnd_flags = d.rnd_flags;
+    P.drop_p = a.dropout_p; P.drop_seed = a.dropout_seed; P.drop_offset = a.dropout_offset; P.drop_mask = a.dropout_mask;
+    if ((d.rnd_flags & MI355_RND_DROPOUT)
+            && (!a.dropout_p || !a.dropout_seed || ((d.rnd_flags & MI355_RND_DROPOUT_OFFSET) && !a.dropout_offset)
+                    || ((d.rnd_flags & MI355_RND_DROPOUT_MASK) && !a.dropout_mask))) {
+        set_error("missing dropout argument (probability, seed, offset or mask)");
+        return MI355_INVALID_ARGUMENTS;
+    }
     const struct { const mi355_quant_t *q; const void *p; const char *n; } need[] = {
             {&d.src_scale, a.src_scale, "src scale"}, {&d.wei_scale, a.wei_scale, "weights scale"},
             {&d.dst_scale, a.dst_scale, "dst scale"}, {&d.src_zp, a.src_zp, "src zero point"},

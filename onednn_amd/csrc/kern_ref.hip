@@ -113,6 +113,16 @@ __device__ float ref_fp_dot(const PT &P, long b, long m, long n) {
     return res;
 }
 
+// bias, dropout (ref_matmul.cpp:283-296), then the rest of the epilogue
+template <class PT>
+__device__ __forceinline__ float ref_epilogue_value(const PT &P, float v, long b, long m, long n) {
+    if (!(P.rnd_flags & MI355_RND_DROPOUT)) return epilogue_value(P, v, b, m, n);
+    if (P.bias_dt != MI355_DT_UNDEF)
+        v += load_float(P.bias_dt, P.bias, b * P.bs[0] + m * P.bs[1] + n * P.bs[2]);
+    v = dropout_f(P, v, b * P.ds[0] + m * P.ds[1] + n * P.ds[2]);
+    return epilogue_after_bias(P, v, b, m, n);
+}
+
 __global__ void __launch_bounds__(256) ref_matmul_kernel(const problem_t P_) {
     const auto &P = MI355_KERNARG_PROBLEM();
     const long total = P.B * P.M * P.N;
@@ -120,8 +130,13 @@ __global__ void __launch_bounds__(256) ref_matmul_kernel(const problem_t P_) {
             i += (long)gridDim.x * blockDim.x) {
         const long n = i % P.N, m = (i / P.N) % P.M, b = i / (P.N * P.M);
         const bool int_path = P.src_dt == MI355_DT_S8 || P.src_dt == MI355_DT_U8;
-        const float v = int_path ? ref_int_dot(P, b, m, n) : ref_fp_dot(P, b, m, n);
-        epilogue_store(P, v, b, m, n);
+        float v = int_path ? ref_int_dot(P, b, m, n) : ref_fp_dot(P, b, m, n);
+        v = ref_epilogue_value(P, v, b, m, n);
+        const long off = b * P.ds[0] + m * P.ds[1] + n * P.ds[2];
+        // the offset and the seed truncated to 32 bits, ref_matmul.cpp:322-331
+        if (P.rnd_flags & MI355_RND_DST_STOCHASTIC)
+            v = stochastic_round_f(v, (uint32_t)off, (uint32_t)dropout_seed(P), P.dst_dt);
+        store_float(P.dst_dt, v, P.dst, off);
     }
 }
 
@@ -146,7 +161,7 @@ __global__ void __launch_bounds__(256) ref_matmul_nibble_dst_kernel(const proble
 #pragma unroll 1
         for (int e = 0; e < 2; ++e) {
             const float v = int_path ? ref_int_dot(P, b, m, n + e) : ref_fp_dot(P, b, m, n + e);
-            byte |= nibble_code(P.dst_dt, epilogue_value(P, v, b, m, n + e)) << (4 * e);
+            byte |= nibble_code(P.dst_dt, ref_epilogue_value(P, v, b, m, n + e)) << (4 * e);
         }
         ((uint8_t *)P.dst)[(b * P.ds[0] + m * P.ds[1] + n) >> 1] = (uint8_t)byte;
     }
@@ -176,7 +191,7 @@ __global__ void __launch_bounds__(64) ref_matmul_dynamic_kernel(const problem_t 
         for (int e = 0; e < G; ++e) {
             const long n = ng * G + e;
             const float v = int_path ? ref_int_dot(P, b, m, n) : ref_fp_dot(P, b, m, n);
-            d[e] = epilogue_value(P, v, b, m, n);
+            d[e] = ref_epilogue_value(P, v, b, m, n);
         }
 #pragma unroll
         for (int e = 0; e < G; ++e) amax = fmaxf(amax, fabsf(d[e]));
@@ -221,6 +236,19 @@ int ref_supported(const mi355_matmul_desc_t &d) {
         if ((d.N & 1) || d.dst_stride[2] != 1 || (d.dst_stride[1] & 1) || (d.dst_stride[0] & 1)) return MI355_UNIMPLEMENTED;
     }
     if (d.wei_packing != MI355_WEI_PACK_NONE && !woq64_layout_ok(d)) return MI355_UNIMPLEMENTED;
+    if (d.rnd_flags != 0) {
+        // ref_matmul_t only (floating-point src); the element's offset in dst seeds its random
+        // number, which the reference defines for the plain row-major layout (ref_matmul.hpp:131-149)
+        if (is_int8_dt(d.src_dt)) return MI355_UNIMPLEMENTED;
+        if (d.dst_stride[2] != 1 || d.dst_stride[1] != d.N || (d.batch > 1 && d.dst_stride[0] != d.M * d.N))
+            return MI355_UNIMPLEMENTED;
+        if (d.rnd_flags & MI355_RND_DST_STOCHASTIC) {
+            const bool fp_dst = d.dst_dt == MI355_DT_F32 || d.dst_dt == MI355_DT_BF16 || d.dst_dt == MI355_DT_F16
+                    || is_f8_dt(d.dst_dt);
+            if (!fp_dst || d.dst_scale_dynamic != MI355_DST_DYNAMIC_NONE) return MI355_UNIMPLEMENTED;
+        }
+        if ((d.rnd_flags & ~MI355_RND_DST_STOCHASTIC) && !(d.rnd_flags & MI355_RND_DROPOUT)) return MI355_INVALID_ARGUMENTS;
+    }
     // dynamic dst quantization exists in ref_matmul_t only, not in the integer implementation
     if (d.dst_scale_dynamic != MI355_DST_DYNAMIC_NONE && is_int8_dt(d.src_dt)) return MI355_UNIMPLEMENTED;
     return MI355_SUCCESS;

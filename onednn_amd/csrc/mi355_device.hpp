@@ -39,6 +39,10 @@ struct problem_t {
     const void *src, *wei, *bias;
     void *dst;
     po_dev_t po[MI355_MAX_POST_OPS];
+    // dropout and stochastic rounding (generic kernel only)
+    int rnd_flags; // MI355_RND_*
+    const void *drop_p, *drop_seed, *drop_offset;
+    void *drop_mask;
 };
 
 // The problem description is the first kernel argument of every kernel.  It is
@@ -215,13 +219,98 @@ __device__ __forceinline__ float binary_f(int alg, float x, float y) {
     }
 }
 
+// ---- dropout and stochastic rounding of ref_matmul_t (src/cpu/matmul/ref_matmul.cpp:283-331)
+// Philox4x32-10 as math::philox4x32 uses it (src/common/math_utils.hpp:458-515)
+__device__ __forceinline__ uint32_t philox4x32(uint64_t idx, uint64_t seed, uint64_t offset) {
+    const uint64_t x = idx & ~(uint64_t)3;
+    uint32_t ctr[4] = {(uint32_t)offset, (uint32_t)(offset >> 32), (uint32_t)x, (uint32_t)(x >> 32)};
+    uint32_t key[2] = {(uint32_t)seed, (uint32_t)(seed >> 32)};
+#pragma unroll
+    for (int i = 0; i < 10; ++i) {
+        if (i > 0) {
+            key[0] += 0x9E3779B9u;
+            key[1] += 0xBB67AE85u;
+        }
+        const uint64_t p0 = (uint64_t)0xD2511F53u * ctr[0], p1 = (uint64_t)0xCD9E8D57u * ctr[2];
+        const uint32_t c1 = ctr[1], c3 = ctr[3];
+        ctr[0] = (uint32_t)(p1 >> 32) ^ c1 ^ key[0];
+        ctr[1] = (uint32_t)p1;
+        ctr[2] = (uint32_t)(p0 >> 32) ^ c3 ^ key[1];
+        ctr[3] = (uint32_t)p0;
+    }
+    const int w = (int)(idx & 3);
+    return w == 0 ? ctr[0] : w == 1 ? ctr[1] : w == 2 ? ctr[2] : ctr[3];
+}
+
+__device__ __forceinline__ uint32_t philox4x32_u32(uint32_t idx, uint32_t seed) {
+    const uint64_t x = idx & ~(uint32_t)3;
+    return philox4x32(((x + 3) << 32) + (x + 2), ((uint64_t)seed << 32) + seed, ((x + 1) << 32) + x);
+}
+
+template <class PT>
+__device__ __forceinline__ long dropout_seed(const PT &P) {
+    if (!(P.rnd_flags & MI355_RND_DROPOUT)) return 0;
+    return (P.rnd_flags & MI355_RND_SEED_S64) ? *(const long *)P.drop_seed : (long)*(const int *)P.drop_seed;
+}
+
+// ref_dropout, src/cpu/primitive_attr_postops.cpp:296-310; idx = the element's offset in dst
+template <class PT>
+__device__ __forceinline__ float dropout_f(const PT &P, float v, long idx) {
+    float p = *(const float *)P.drop_p;
+    const long seed = dropout_seed(P);
+    const long offset = (P.rnd_flags & MI355_RND_DROPOUT_OFFSET) ? *(const long *)P.drop_offset : 0;
+    const float inv_q = (p != 1.f) ? 1.f / (1.f - p) : 0.f;
+    const uint32_t r = offset ? philox4x32((uint64_t)idx, (uint64_t)seed, (uint64_t)offset)
+                              : philox4x32_u32((uint32_t)idx, (uint32_t)seed);
+    p = fmaxf(fminf(p, 1.f), 0.f);
+    const bool keep = (double)r > 4294967295.0 * (double)p;
+    if (P.rnd_flags & MI355_RND_DROPOUT_MASK) ((uint8_t *)P.drop_mask)[idx] = keep;
+    return keep ? v * inv_q : 0.f;
+}
+
+// math::stochastic_round_fwd, src/common/math_utils.hpp:535-574
+__device__ __forceinline__ float stochastic_round_f(float s, uint32_t idx, uint32_t seed, int dst_dt) {
+    if (s != s) return s;
+    int digits;
+    float hi, tiny;
+    switch (dst_dt) {
+        case MI355_DT_F32: digits = 24; hi = 3.40282347e38f; tiny = 1.17549435e-38f; break;
+        case MI355_DT_BF16: digits = 8; hi = 3.38953139e38f; tiny = 1.17549435e-38f; break;
+        case MI355_DT_F16: digits = 11; hi = 65504.f; tiny = 6.10351562e-05f; break;
+        case MI355_DT_F8_E5M2: digits = 3; hi = 57344.f; tiny = 6.10351562e-05f; break;
+        case MI355_DT_F8_E4M3: digits = 4; hi = 448.f; tiny = 0.015625f; break;
+        default: return __builtin_nanf("");
+    }
+    const uint32_t truncation_mask = 0xffffffffu << (24 - digits);
+    uint32_t rnd;
+    if (dst_dt == MI355_DT_BF16 || dst_dt == MI355_DT_F16)
+        rnd = (philox4x32_u32(idx >> 2, seed) >> ((idx & 3) * 8)) & 0xffu;
+    else
+        rnd = (philox4x32_u32(idx >> 1, seed) >> ((idx & 1) * 16)) & 0xffffu;
+    rnd &= ~truncation_mask;
+    float r = u2f((f2u(s) + rnd) & truncation_mask);
+    r = fminf(fmaxf(r, -hi), hi);
+    if (r > 0 && r < tiny) r = 0;
+    if (r < 0 && r > -tiny) r = 0;
+    return r;
+}
+
 // Everything after the K reduction except the store: returns the f32 value
 // that store_float() converts.
+template <class PT>
+__device__ __forceinline__ float epilogue_after_bias(const PT &P, float v, long b, long m, long n);
+
 template <class PT>
 __device__ __forceinline__ float epilogue_value(
         const PT &P, float v, long b, long m, long n) {
     if (P.bias_dt != MI355_DT_UNDEF)
         v += load_float(P.bias_dt, P.bias, b * P.bs[0] + m * P.bs[1] + n * P.bs[2]);
+    return epilogue_after_bias(P, v, b, m, n);
+}
+
+// post-ops, dst scale and dst zero point
+template <class PT>
+__device__ __forceinline__ float epilogue_after_bias(const PT &P, float v, long b, long m, long n) {
     if (P.n_po > 0) {
         float dst_old = 0.f;
         if (P.sum_dt != MI355_DT_UNDEF)

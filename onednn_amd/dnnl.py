@@ -32,6 +32,11 @@ ARG_SRC, ARG_SRC_1, ARG_DST, ARG_WEIGHTS, ARG_BIAS, ARG_SCRATCHPAD = 1, 2, 17, 3
 ARG_SRC_2 = 3
 ARG_FROM, ARG_TO = ARG_SRC, ARG_DST
 ARG_ATTR_PRECOMPUTED_REDUCTIONS, ARG_ATTR_SCALES, ARG_ATTR_ZERO_POINTS = 512, 4096, 8192
+ARG_ATTR_DROPOUT_OFFSET, ARG_ATTR_ROUNDING_SEED, ARG_ATTR_DROPOUT_MASK = 507, 508, 509
+ARG_ATTR_DROPOUT_PROBABILITY, ARG_ATTR_DROPOUT_SEED = 510, 511
+ARG_DIFF_SRC, ARG_DIFF_WEIGHTS = 129, 161
+rounding_environment, rounding_stochastic = 0, 1
+s64 = 16                               # dnnl_s64: the dropout seed / offset type
 scratchpad_library, scratchpad_user = 0, 1
 fpmath_strict, fpmath_bf16, fpmath_f16, fpmath_any = 0, 1, 2, 3
 MEMORY_ALLOCATE = C.c_void_p(-1 & (2 ** 64 - 1))
@@ -198,6 +203,13 @@ class grouped_memory:
         return out
 
 
+def zero_memory_desc():
+    """A zero memory descriptor (ndims 0: "no tensor")."""
+    h = C.c_void_p()
+    _check(lib().dnnl_memory_desc_create_with_tag(C.byref(h), 0, _dims([]), 0, 0), "memory_desc_create (zero)")
+    return memory_desc(handle=h.value)
+
+
 class host_scalar:
     """dnnl::memory of a host-side scalar (dnnl_memory_create_host_scalar): the
     value lives in the object; `value` is a numpy scalar of the storage type."""
@@ -318,6 +330,30 @@ class primitive_attr:
 
     def set_scratchpad_mode(self, mode):
         _check(lib().dnnl_primitive_attr_set_scratchpad_mode(self.h, mode), "set_scratchpad_mode")
+
+    def set_dropout(self, mask_md=None, seed_dt=None, use_offset=False, use_host_scalars=False):
+        """mask_md None: a zero descriptor (no mask is written).  seed_dt None: the first form of the call."""
+        md = mask_md if mask_md is not None else zero_memory_desc()
+        if seed_dt is None:
+            _check(lib().dnnl_primitive_attr_set_dropout(self.h, md.h), "set_dropout")
+        else:
+            _check(lib().dnnl_primitive_attr_set_dropout_v2(self.h, md.h, seed_dt, int(use_offset), int(use_host_scalars)),
+                   "set_dropout_v2")
+
+    def get_dropout(self):
+        """(mask data type, seed data type, use_offset, use_host_scalars)"""
+        mdh, dt, off, hs = C.c_void_p(), C.c_int(), C.c_int(), C.c_int()
+        _check(lib().dnnl_primitive_attr_get_dropout_v2(self.h, C.byref(mdh), C.byref(dt), C.byref(off), C.byref(hs)),
+               "get_dropout_v2")
+        return memory_desc(handle=mdh.value).data_type(), dt.value, off.value, hs.value
+
+    def set_rounding(self, arg, mode):
+        _check(lib().dnnl_primitive_attr_set_rounding(self.h, arg, mode), "set_rounding")
+
+    def get_rounding(self, arg):
+        v = C.c_int()
+        _check(lib().dnnl_primitive_attr_get_rounding(self.h, arg, C.byref(v)), "get_rounding")
+        return v.value
 
 
 class matmul_primitive_desc:

@@ -57,7 +57,7 @@ dnnl_status_t from_mi355(int st) {
 }
 
 bool dt_valid(int dt) {
-    return dt >= dnnl_f16 && dt <= dnnl_f4_e2m1 && dt != dnnl_f64 && dt != dnnl_boolean;
+    return (dt >= dnnl_f16 && dt <= dnnl_f4_e2m1 && dt != dnnl_f64 && dt != dnnl_boolean) || dt == dnnl_s64;
 }
 int dt_bits(int dt) {
     switch (dt) {
@@ -68,6 +68,7 @@ int dt_bits(int dt) {
         case dnnl_s4:
         case dnnl_u4:
         case dnnl_f4_e2m1: return 4;
+        case dnnl_s64:
         case dnnl_f64: return 64;
         default: return 8;
     }
@@ -211,6 +212,12 @@ struct dnnl_primitive_attr {
     dnnl_accumulation_mode_t acc_mode = dnnl_accumulation_mode_strict;
     dnnl_scratchpad_mode_t scratchpad_mode = dnnl_scratchpad_mode_library;
     dnnl_post_ops post_ops;
+    // dropout_t (src/common/primitive_attr.hpp:185-218): set <=> seed_dt != undef
+    dnnl_memory_desc dropout_md;
+    dnnl_data_type_t dropout_seed_dt = dnnl_data_type_undef;
+    int dropout_use_offset = 0, dropout_host_scalars = 0;
+    std::map<int, dnnl_rounding_mode_t> rounding;
+    bool with_dropout() const { return dropout_seed_dt != dnnl_data_type_undef; }
     const quant_entry_t *find(const std::map<int, quant_entry_t> &m, int arg) const {
         auto it = m.find(arg);
         return it == m.end() ? nullptr : &it->second;
@@ -284,9 +291,14 @@ namespace {
     do { \
         if (!(cond)) return dnnl_invalid_arguments; \
     } while (0)
+// ONEDNN_AMD_TRACE_UNIMPL=1 names the rule that refused a descriptor (stderr)
+static const bool g_trace_unimpl = getenv("ONEDNN_AMD_TRACE_UNIMPL") != nullptr;
 #define CHECK_UNIMPL(cond) \
     do { \
-        if (!(cond)) return dnnl_unimplemented; \
+        if (!(cond)) { \
+            if (g_trace_unimpl) fprintf(stderr, "onednn_amd: unimplemented at %s:%d: !(%s)\n", __FILE__, __LINE__, #cond); \
+            return dnnl_unimplemented; \
+        } \
     } while (0)
 #define IMPLICATION(a, b) (!(a) || (b))
 
@@ -639,6 +651,31 @@ dnnl_status_t lower(dnnl_primitive_desc &pd) {
         }
     }
     CHECK_UNIMPL(D.dst_zp.dt == MI355_DT_UNDEF || D.dst_zp.dt == MI355_DT_S32);
+    // dropout and stochastic rounding: ref_matmul_t only (ref_matmul.hpp:96-149)
+    D.rnd_flags = 0;
+    if (a.with_dropout()) {
+        CHECK_UNIMPL(first == 0);
+        D.rnd_flags |= MI355_RND_DROPOUT;
+        if (a.dropout_seed_dt == dnnl_s64) D.rnd_flags |= MI355_RND_SEED_S64;
+        if (a.dropout_use_offset) D.rnd_flags |= MI355_RND_DROPOUT_OFFSET;
+        if (a.dropout_md.dt != dnnl_data_type_undef) {
+            // the mask is laid out like dst (dropout_t::set_default_formats + similar_to)
+            const dnnl_memory_desc &mk = a.dropout_md;
+            CHECK_UNIMPL(mk.ndims == nd);
+            for (int i = 0; i < nd; ++i) CHECK_UNIMPL(mk.dims[i] == pd.dst.dims[i]);
+            if (mk.kind != dnnl_format_kind_any)
+                for (int i = 0; i < nd; ++i) CHECK_UNIMPL(mk.strides[i] == pd.dst.strides[i]);
+            D.rnd_flags |= MI355_RND_DROPOUT_MASK;
+        }
+    }
+    {
+        auto it = a.rounding.find(DNNL_ARG_DST);
+        if (it != a.rounding.end() && it->second == dnnl_rounding_mode_stochastic) {
+            CHECK_UNIMPL(first == 0);
+            D.rnd_flags |= MI355_RND_DST_STOCHASTIC;
+        }
+        for (const auto &kv : a.rounding) CHECK_UNIMPL(kv.first == DNNL_ARG_DST);
+    }
     D.fpmath_apply_to_int = a.apply_to_int;
     D.fpmath_mode = a.fpmath;
     D.dst_scale_mode = MI355_DST_SCALE_DIVIDE;
@@ -931,6 +968,10 @@ DNNL_EXPORT dnnl_status_t dnnl_memory_desc_create_with_tag(dnnl_memory_desc_t *m
         const dnnl_dims_t dims, dnnl_data_type_t data_type, dnnl_format_tag_t tag) {
     CHECK_ARG(memory_desc);
     std::unique_ptr<dnnl_memory_desc> md(new dnnl_memory_desc);
+    if (ndims == 0 || tag == dnnl_format_tag_undef) { // a zero descriptor, memory_desc.cpp:245-250
+        *memory_desc = md.release();
+        return dnnl_success;
+    }
     dnnl_status_t st = md_common(*md, ndims, dims, data_type);
     if (st) return st;
     int perm[DNNL_MAX_NDIMS];
@@ -1273,6 +1314,50 @@ DNNL_EXPORT dnnl_status_t dnnl_primitive_attr_set_accumulation_mode(dnnl_primiti
     CHECK_ARG(attr);
     CHECK_ARG(mode >= dnnl_accumulation_mode_strict && mode <= dnnl_accumulation_mode_f16);
     attr->acc_mode = mode;
+    return dnnl_success;
+}
+DNNL_EXPORT dnnl_status_t dnnl_primitive_attr_get_dropout_v2(const_dnnl_primitive_attr_t attr,
+        const_dnnl_memory_desc_t *mask_desc, dnnl_data_type_t *seed_dt, int *use_offset, int *use_host_scalars) {
+    CHECK_ARG(attr);
+    if (mask_desc) *mask_desc = &attr->dropout_md;
+    if (seed_dt) *seed_dt = attr->dropout_seed_dt;
+    if (use_offset) *use_offset = attr->dropout_use_offset;
+    if (use_host_scalars) *use_host_scalars = attr->dropout_host_scalars;
+    return dnnl_success;
+}
+DNNL_EXPORT dnnl_status_t dnnl_primitive_attr_get_dropout(const_dnnl_primitive_attr_t attr,
+        const_dnnl_memory_desc_t *mask_desc) {
+    return dnnl_primitive_attr_get_dropout_v2(attr, mask_desc, nullptr, nullptr, nullptr);
+}
+// primitive_attr_t::set_dropout, src/common/primitive_attr.cpp:423-438
+DNNL_EXPORT dnnl_status_t dnnl_primitive_attr_set_dropout_v2(dnnl_primitive_attr_t attr, const_dnnl_memory_desc_t mask_desc,
+        dnnl_data_type_t seed_dt, int use_offset, int use_host_scalars) {
+    CHECK_ARG(attr && mask_desc);
+    CHECK_ARG(mask_desc->dt == dnnl_u8 || mask_desc->dt == dnnl_data_type_undef);
+    CHECK_ARG(seed_dt == dnnl_s32 || seed_dt == dnnl_s64);
+    attr->dropout_md = *mask_desc;
+    attr->dropout_seed_dt = seed_dt;
+    attr->dropout_use_offset = use_offset != 0;
+    attr->dropout_host_scalars = use_host_scalars != 0;
+    return dnnl_success;
+}
+DNNL_EXPORT dnnl_status_t dnnl_primitive_attr_set_dropout(dnnl_primitive_attr_t attr, const_dnnl_memory_desc_t mask_desc) {
+    return dnnl_primitive_attr_set_dropout_v2(attr, mask_desc, dnnl_s32, 0, 0);
+}
+// rnd_mode_t::set / check, src/common/primitive_attr.hpp:226-258: only dst and the gradients take a non-default mode
+DNNL_EXPORT dnnl_status_t dnnl_primitive_attr_set_rounding(dnnl_primitive_attr_t attr, int arg, dnnl_rounding_mode_t mode) {
+    CHECK_ARG(attr);
+    CHECK_ARG(mode == dnnl_rounding_mode_environment || mode == dnnl_rounding_mode_stochastic);
+    if (mode != dnnl_rounding_mode_environment) {
+        CHECK_ARG(arg == DNNL_ARG_DST || arg == DNNL_ARG_DIFF_SRC || arg == DNNL_ARG_DIFF_WEIGHTS);
+        attr->rounding[arg] = mode;
+    }
+    return dnnl_success;
+}
+DNNL_EXPORT dnnl_status_t dnnl_primitive_attr_get_rounding(dnnl_primitive_attr_t attr, int arg, dnnl_rounding_mode_t *mode) {
+    CHECK_ARG(attr && mode);
+    auto it = attr->rounding.find(arg);
+    *mode = it == attr->rounding.end() ? dnnl_rounding_mode_environment : it->second;
     return dnnl_success;
 }
 DNNL_EXPORT dnnl_status_t dnnl_primitive_attr_set_scratchpad_mode(dnnl_primitive_attr_t attr,
@@ -1970,9 +2055,10 @@ DNNL_EXPORT dnnl_status_t dnnl_primitive_create(dnnl_primitive_t *primitive, con
     bool any_on_host = false;
     for (const auto *mp : {&p->pd.attr.scales, &p->pd.attr.zero_points})
         for (const auto &kv : *mp) any_on_host |= kv.second.on_host;
+    any_on_host |= p->pd.attr.with_dropout() && p->pd.attr.dropout_host_scalars;
     if (any_on_host && p->pd.kind == dnnl_matmul) {
         if (mi355_device_set((int)p->pd.engine->index) != MI355_SUCCESS) return dnnl_runtime_error;
-        const int st = mi355_mem_alloc(&p->host_scalars, 64);
+        const int st = mi355_mem_alloc(&p->host_scalars, 128); // 6 quantization slots + 3 dropout slots of 8 bytes
         if (st != MI355_SUCCESS) return from_mi355(st);
     }
     *primitive = p.release();
@@ -2161,6 +2247,36 @@ DNNL_EXPORT dnnl_status_t dnnl_primitive_execute(const_dnnl_primitive_t cprimiti
     if ((st = take_q(at.zero_points, DNNL_ARG_WEIGHTS, DNNL_ARG_ATTR_ZERO_POINTS, pd.desc.wei_zp, &A.wei_zp))) return st;
     if ((st = take_q(at.zero_points, DNNL_ARG_DST, DNNL_ARG_ATTR_ZERO_POINTS, pd.desc.dst_zp, &A.dst_zp))) return st;
     TAKE(src_pr, DNNL_ARG_ATTR_PRECOMPUTED_REDUCTIONS | DNNL_ARG_SRC, pd.desc.src_pr.dt != MI355_DT_UNDEF);
+    if (pd.desc.rnd_flags & MI355_RND_DROPOUT) {
+        // probability, seed and offset: one value each, in device memory or (use_host_scalars) host-scalar objects
+        auto take_scalar = [&](int arg, dnnl_data_type_t dt, int my_slot, const void **field) -> dnnl_status_t {
+            auto it = m.find(arg);
+            dnnl_memory_t mem = it == m.end() ? nullptr : it->second;
+            CHECK_ARG(mem && (int)mem->md.dt == (int)dt);
+            if (at.dropout_host_scalars) {
+                CHECK_ARG(mem->md.kind == dnnl_format_kind_host_scalar);
+                if (!prim->host_scalars) return dnnl_runtime_error;
+                void *dev = (char *)prim->host_scalars + 8 * my_slot;
+                order_on_device();
+                uint64_t bits = 0;
+                memcpy(&bits, mem->scalar, dt_bits(dt) / 8);
+                const int rc = mi355_mem_store_scalar(dev, bits, dt_bits(dt) / 8, stream->hip_stream);
+                if (rc != MI355_SUCCESS) return from_mi355(rc);
+                *field = dev;
+                return dnnl_success;
+            }
+            CHECK_ARG(mem->md.kind != dnnl_format_kind_host_scalar);
+            void *h = nullptr;
+            const dnnl_status_t hs = handle(arg, true, &h);
+            *field = h;
+            return hs;
+        };
+        if ((st = take_scalar(DNNL_ARG_ATTR_DROPOUT_PROBABILITY, dnnl_f32, 6, &A.dropout_p))) return st;
+        if ((st = take_scalar(DNNL_ARG_ATTR_DROPOUT_SEED, at.dropout_seed_dt, 7, &A.dropout_seed))) return st;
+        if (pd.desc.rnd_flags & MI355_RND_DROPOUT_OFFSET)
+            if ((st = take_scalar(DNNL_ARG_ATTR_DROPOUT_OFFSET, dnnl_s64, 8, &A.dropout_offset))) return st;
+        if (pd.desc.rnd_flags & MI355_RND_DROPOUT_MASK) TAKE(dropout_mask, DNNL_ARG_ATTR_DROPOUT_MASK, true);
+    }
     for (int i = 0; i < pd.desc.n_post_ops; ++i) {
         if (pd.po_arg_id[i]) {
             if ((st = handle(DNNL_ARG_ATTR_MULTIPLE_POST_OP(pd.po_entry[i]) | pd.po_arg_id[i], true, &p))) return st;

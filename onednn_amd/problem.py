@@ -134,6 +134,9 @@ class MatmulProblem:
     wei_packing: int = cabi.WEI_PACK_NONE  # `wei` stays plain here; GpuRun uploads it packed
     dst_dynamic: int = cabi.DST_DYNAMIC_NONE  # quant["dst_scale"].data is then an output (its content is ignored)
     dst_init: Optional[np.ndarray] = None   # prior dst content (sum post-op)
+    # dropout: {"p": float, "seed": int, "seed_s64": bool, "offset": int or None, "mask": bool}
+    dropout: Optional[dict] = None
+    dst_stochastic: bool = False            # stochastic rounding of dst
     name: str = ""
 
     def __post_init__(self):
@@ -182,7 +185,33 @@ class MatmulProblem:
         d.impl = self.impl
         d.wei_packing = self.wei_packing
         d.dst_scale_dynamic = self.dst_dynamic
+        d.rnd_flags = self.rnd_flags()
         return d
+
+    def rnd_flags(self):
+        f = cabi.RND_DST_STOCHASTIC if self.dst_stochastic else 0
+        if self.dropout is not None:
+            f |= cabi.RND_DROPOUT
+            if self.dropout.get("mask"):
+                f |= cabi.RND_DROPOUT_MASK
+            if self.dropout.get("seed_s64"):
+                f |= cabi.RND_SEED_S64
+            if self.dropout.get("offset") is not None:
+                f |= cabi.RND_DROPOUT_OFFSET
+        return f
+
+    def dropout_buffers(self):
+        """{args field: array} of the dropout arguments (the mask zero-filled with 0xee: every byte is written)."""
+        if self.dropout is None:
+            return {}
+        dr = self.dropout
+        seed_np = np.int64 if dr.get("seed_s64") else np.int32
+        out = {"dropout_p": np.asarray([dr["p"]], np.float32), "dropout_seed": np.asarray([dr["seed"]], seed_np)}
+        if dr.get("offset") is not None:
+            out["dropout_offset"] = np.asarray([dr["offset"]], np.int64)
+        if dr.get("mask"):
+            out["dropout_mask"] = np.full(self.dst_span(), 0xee, np.uint8)
+        return out
 
     def initial_dst(self):
         n = storage_elems(self.dst_dt, self.dst_span())
@@ -227,6 +256,9 @@ class GpuRun:
             if po.data is not None:
                 self.bufs[f"po{i}"] = cabi.DeviceBuffer.from_numpy(po.data)
                 a.po_arg[i] = self.bufs[f"po{i}"].ptr
+        for name, arr in prob.dropout_buffers().items():
+            self.bufs[name] = cabi.DeviceBuffer.from_numpy(arr)
+            setattr(a, name, self.bufs[name].ptr)
         self.args = a
         st, self.impl = cabi.query(self.desc, self.desc.impl)
         cabi.check(st)
@@ -247,6 +279,11 @@ class GpuRun:
     def result(self):
         self.sync()
         return self.bufs["dst"].to_numpy(storage_dtype(self.prob.dst_dt), self.dst_host_shape)
+
+    def dropout_mask(self):
+        """The keep flags a dropout launch wrote (u8, laid out like dst)."""
+        self.sync()
+        return self.bufs["dropout_mask"].to_numpy(np.uint8, (self.prob.dst_span(),))
 
     def dynamic_scales(self):
         """The dst scales a dynamic-quantization launch wrote (raw storage)."""

@@ -62,6 +62,10 @@ def host_args(prob: MatmulProblem, dst):
     for i, po in enumerate(prob.post_ops):
         if po.data is not None:
             a.po_arg[i] = hold(po.data)
+    for name, arr in prob.dropout_buffers().items():
+        setattr(a, name, hold(arr))
+        if name == "dropout_mask":
+            prob._oracle_mask = keep[-1]      # read back by run_oracle_dropout
     return a, keep
 
 
@@ -81,6 +85,52 @@ def run_oracle(prob: MatmulProblem, flags=0, want_ideal=False):
     if want_ideal:
         return dst, ideal, asum
     return dst
+
+
+def run_oracle_dropout(prob: MatmulProblem):
+    """(raw dst storage, the dropout mask or None)."""
+    prob._oracle_mask = None
+    dst = run_oracle(prob)
+    return dst, prob._oracle_mask
+
+
+def philox_block(ctr, key):
+    """Philox4x32-10 of the oracle: (4 counter words, 2 key words) -> 4 output words."""
+    lib = load()
+    c, k, o = (C.c_uint32 * 4)(*ctr), (C.c_uint32 * 2)(*key), (C.c_uint32 * 4)()
+    lib.oracle_philox4x32_block(c, k, o)
+    return list(o)
+
+
+def philox(idx, seed, offset):
+    lib = load()
+    lib.oracle_philox4x32.restype = C.c_uint32
+    lib.oracle_philox4x32.argtypes = [C.c_uint64] * 3
+    return lib.oracle_philox4x32(idx % 2 ** 64, seed % 2 ** 64, offset % 2 ** 64)
+
+
+def philox_u32(idx, seed):
+    lib = load()
+    lib.oracle_philox4x32_u32.restype = C.c_uint32
+    lib.oracle_philox4x32_u32.argtypes = [C.c_uint32] * 2
+    return lib.oracle_philox4x32_u32(idx % 2 ** 32, seed % 2 ** 32)
+
+
+def stochastic_round(x, idx, seed, dt):
+    lib = load()
+    lib.oracle_stochastic_round.restype = C.c_float
+    lib.oracle_stochastic_round.argtypes = [C.c_float, C.c_uint32, C.c_uint32, C.c_int]
+    return lib.oracle_stochastic_round(float(x), idx % 2 ** 32, seed % 2 ** 32, dt)
+
+
+def dropout(x, idx, p, seed, offset):
+    """(value, keep flag) of oracle_dropout."""
+    lib = load()
+    lib.oracle_dropout.restype = C.c_float
+    lib.oracle_dropout.argtypes = [C.c_float, C.c_void_p, C.c_int64, C.c_float, C.c_int64, C.c_int64]
+    mask = np.zeros(idx + 1, np.uint8)
+    v = lib.oracle_dropout(float(x), mask.ctypes.data, idx, float(p), seed, offset)
+    return v, int(mask[idx])
 
 
 def run_oracle_dynamic(prob: MatmulProblem, flags=0):

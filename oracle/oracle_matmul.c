@@ -12,6 +12,9 @@
  *                     src/cpu/matmul/ref_matmul.cpp:168-236
  *   orc_finish        bias + post-ops + dst scale + dst zero point + store
  *                     ref_matmul_int8.cpp:275-306, ref_matmul.cpp:283-331
+ *   oracle_dropout / oracle_stochastic_round / oracle_philox4x32
+ *                     ref_dropout src/cpu/primitive_attr_postops.cpp:296-310,
+ *                     math::stochastic_round_fwd, philox4x32 src/common/math_utils.hpp:458-574
  *   orc_post_ops      ref_post_ops_t::execute src/cpu/primitive_attr_postops.cpp:312-394
  *   orc_eltwise       compute_eltwise_scalar_fwd :49-87 with the formulas of
  *                     src/common/math_utils.hpp:120-430
@@ -52,6 +55,12 @@
  * there too: the scale against an exhaustive nearest-value search over the 127
  * positive e4m3 codes on constructed maxima (ties to even, both clamps), the
  * dst codes against a nearest-value search over the type's codes.
+ * Dropout and stochastic rounding (oracle_philox4x32*, oracle_dropout,
+ * oracle_stochastic_round) are pinned by tests/test_dropout_rounding.py: the
+ * Philox core against the known-answer vectors of its authors (Random123) and
+ * an independent implementation, the counter / key construction by the block
+ * structure it implies, the keep rule where it is decidable by hand, the
+ * rounding by representability, neighbourhood, limits and carry probability.
  * The ternary select post-op is pinned by tests/test_oracle_matmul.py (numpy
  * `where` on exact integer sums, three condition types).
  * Precomputed reductions (orc_int8_dot with src_pr, grouped / per-tensor src
@@ -426,6 +435,101 @@ static float orc_fp_dot(const mi355_matmul_desc_t *d,
     return res;
 }
 
+/* ------------------------------------------- dropout, stochastic rounding */
+/* Philox4x32-10 (Salmon et al., "Parallel random numbers: as easy as 1, 2, 3"), the
+ * generator of math::philox4x32(idx, seed, offset) src/common/math_utils.hpp:458-506:
+ * counter = (offset lo, offset hi, idx & ~3 lo, hi), key = seed; the word idx & 3
+ * of the output block is returned. */
+void oracle_philox4x32_block(const uint32_t *ctr_in, const uint32_t *key_in, uint32_t *out) {
+    uint32_t ctr[4] = {ctr_in[0], ctr_in[1], ctr_in[2], ctr_in[3]};
+    uint32_t key[2] = {key_in[0], key_in[1]};
+    for (int i = 0; i < 10; ++i) {
+        if (i > 0) {
+            key[0] += 0x9E3779B9u;
+            key[1] += 0xBB67AE85u;
+        }
+        const uint64_t p0 = (uint64_t)0xD2511F53u * ctr[0], p1 = (uint64_t)0xCD9E8D57u * ctr[2];
+        const uint32_t hi0 = (uint32_t)(p0 >> 32), lo0 = (uint32_t)p0;
+        const uint32_t hi1 = (uint32_t)(p1 >> 32), lo1 = (uint32_t)p1;
+        const uint32_t c1 = ctr[1], c3 = ctr[3];
+        ctr[0] = hi1 ^ c1 ^ key[0];
+        ctr[1] = lo1;
+        ctr[2] = hi0 ^ c3 ^ key[1];
+        ctr[3] = lo0;
+    }
+    for (int i = 0; i < 4; ++i) out[i] = ctr[i];
+}
+
+uint32_t oracle_philox4x32(uint64_t idx, uint64_t seed, uint64_t offset) {
+    const uint64_t x = idx & ~(uint64_t)3;
+    const uint32_t ctr[4] = {(uint32_t)offset, (uint32_t)(offset >> 32), (uint32_t)x, (uint32_t)(x >> 32)};
+    const uint32_t key[2] = {(uint32_t)seed, (uint32_t)(seed >> 32)};
+    uint32_t out[4];
+    oracle_philox4x32_block(ctr, key, out);
+    return out[idx & 3];
+}
+
+/* the 32-bit flavour, math_utils.hpp:508-515: the counter and the key are
+ * built from idx & ~3 and the seed alone (the four indices of a block share
+ * one value) */
+uint32_t oracle_philox4x32_u32(uint32_t idx, uint32_t seed) {
+    const uint64_t x = idx & ~(uint32_t)3;
+    const uint64_t idx64 = ((x + 3) << 32) + (x + 2);
+    const uint64_t off64 = ((x + 1) << 32) + x;
+    const uint64_t seed64 = ((uint64_t)seed << 32) + seed;
+    return oracle_philox4x32(idx64, seed64, off64);
+}
+
+/* ref_dropout, src/cpu/primitive_attr_postops.cpp:296-310 */
+float oracle_dropout(float src, uint8_t *mask, int64_t idx, float p, int64_t seed, int64_t offset) {
+    const float inv_q = (p != 1.f) ? 1.f / (1.f - p) : 0.f;
+    const uint32_t r = offset ? oracle_philox4x32((uint64_t)idx, (uint64_t)seed, (uint64_t)offset)
+                              : oracle_philox4x32_u32((uint32_t)idx, (uint32_t)seed);
+    p = fmaxf(fminf(p, 1.f), 0.f);
+    const uint8_t m = (double)r > (double)UINT32_MAX * (double)p;
+    if (mask) mask[idx] = m;
+    return m ? src * inv_q : 0.f;
+}
+
+/* math::stochastic_round_fwd, src/common/math_utils.hpp:535-574: `digits` =
+ * significand bits of the dst type including the hidden one. */
+float oracle_stochastic_round(float s, uint32_t idx, uint32_t seed, int dst_dt) {
+    if (s != s) return s;
+    int digits;
+    float lo, hi, tiny;
+    switch (dst_dt) {
+        case MI355_DT_F32: digits = 24; hi = 3.40282347e38f; tiny = 1.17549435e-38f; break; /* nothing is truncated */
+        case MI355_DT_BF16: digits = 8; hi = 3.38953139e38f; tiny = 1.17549435e-38f; break;
+        case MI355_DT_F16: digits = 11; hi = 65504.f; tiny = 6.10351562e-05f; break;
+        case MI355_DT_F8_E5M2: digits = 3; hi = 57344.f; tiny = 6.10351562e-05f; break;
+        case MI355_DT_F8_E4M3: digits = 4; hi = 448.f; tiny = 0.015625f; break;
+        default: return NAN;
+    }
+    lo = -hi;
+    const uint32_t truncation_mask = 0xffffffffu << (24 - digits);
+    /* two-byte types take 8 random bits, one-byte types 16 (:560-561) */
+    uint32_t rnd;
+    if (dst_dt == MI355_DT_BF16 || dst_dt == MI355_DT_F16)
+        rnd = (uint8_t)(oracle_philox4x32_u32(idx >> 2, seed) >> ((idx & 3) * 8));
+    else
+        rnd = (uint16_t)(oracle_philox4x32_u32(idx >> 1, seed) >> ((idx & 1) * 16));
+    rnd &= ~truncation_mask;
+    uint32_t su;
+    memcpy(&su, &s, 4);
+    const uint32_t ru = (su + rnd) & truncation_mask;
+    float r;
+    memcpy(&r, &ru, 4);
+    r = fminf(fmaxf(r, lo), hi);
+    if (r > 0 && r < tiny) r = 0;
+    if (r < 0 && r > -tiny) r = 0;
+    return r;
+}
+
+static int64_t orc_dropout_seed(const mi355_matmul_desc_t *d, const mi355_matmul_args_t *a) {
+    if (!(d->rnd_flags & MI355_RND_DROPOUT)) return 0;
+    return (d->rnd_flags & MI355_RND_SEED_S64) ? *(const int64_t *)a->dropout_seed : *(const int32_t *)a->dropout_seed;
+}
+
 /* ------------------------------------------------------------- epilogue */
 /* bias and post-ops: the value the dst quantization (static or dynamic) sees */
 static float orc_pre_quant(const mi355_matmul_desc_t *d,
@@ -437,6 +541,10 @@ static float orc_pre_quant(const mi355_matmul_desc_t *d,
         v += orc_load_float(d->bias_dt, a->bias,
                 b * d->bias_stride[0] + m * d->bias_stride[1]
                         + n * d->bias_stride[2]);
+    if (d->rnd_flags & MI355_RND_DROPOUT) /* ref_matmul.cpp:293-296 */
+        v = oracle_dropout(v, (d->rnd_flags & MI355_RND_DROPOUT_MASK) ? (uint8_t *)a->dropout_mask : NULL, doff,
+                *(const float *)a->dropout_p, orc_dropout_seed(d, a),
+                (d->rnd_flags & MI355_RND_DROPOUT_OFFSET) ? *(const int64_t *)a->dropout_offset : 0);
     if (d->n_post_ops > 0) {
         float dst_old = 0.f;
         for (int i = 0; i < d->n_post_ops; ++i)
@@ -469,6 +577,8 @@ static void orc_finish(const mi355_matmul_desc_t *d,
         int z = orc_load_int(MI355_DT_S32, a->dst_zp, (d->dst_zp.mask & 4) ? n : 0);
         v += (float)z;
     }
+    if (d->rnd_flags & MI355_RND_DST_STOCHASTIC) /* ref_matmul.cpp:322-331: the offset and the seed truncated to 32 bits */
+        v = oracle_stochastic_round(v, (uint32_t)doff, (uint32_t)orc_dropout_seed(d, a), d->dst_dt);
     orc_store_float(d->dst_dt, v, a->dst, doff);
 }
 

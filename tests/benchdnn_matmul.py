@@ -35,7 +35,7 @@ CUSTOM with the %engine% %impl% %name% %prb% %desc% %driver% %idx% %attr%
 %freq% print 0) with the time modifiers - 0 + and the unit modifiers K M G.
 
 Supported knobs: --dt, --stag, --wtag, --dtag (ab | ba | any), --bia-dt,
---attr-scales, --attr-zero-points, --attr-post-ops, --attr-fpmath, --impl,
+--attr-scales, --attr-zero-points, --attr-post-ops, --attr-fpmath, --attr-dropout, --attr-rounding-mode, --impl,
 --mode, --buffer-prefix, --export-buffers, --perf-template, --max-ms-per-prb,
 and 2-D problem descriptors MxK:KxN.  Policies: common, per_oc,
 per_ocic (with GxH groups), per_tensor (with GxH groups), per_dim_0, per_dim_1.
@@ -109,7 +109,8 @@ class Spec:
         parts = ["--matmul", f"--dt={self.dt}", f"--stag={self.stag}", f"--wtag={self.wtag}", f"--dtag={self.dtag}"]
         if self.bia_dt != "undef":
             parts.append(f"--bia-dt={self.bia_dt}")
-        for knob in ("attr_scales", "attr_zero_points", "attr_post_ops", "attr_fpmath"):
+        for knob in ("attr_scales", "attr_zero_points", "attr_post_ops", "attr_fpmath", "attr_dropout",
+                     "attr_rounding_mode"):
             if getattr(self, knob):
                 parts.append(f"--{knob.replace('_', '-')}={getattr(self, knob)}")
         if self.runtime_dims_masks:
@@ -129,7 +130,7 @@ def parse(argv, settings=None):
     `settings` (a dict like SETTINGS) when one is given."""
     knobs = {"dt": ["f32"], "stag": ["ab"], "wtag": ["ab"], "dtag": ["ab"], "bia_dt": ["undef"],
              "attr_scales": [""], "attr_zero_points": [""], "attr_post_ops": [""], "attr_fpmath": [""],
-             "runtime_dims_masks": [""], "impl": [""]}
+             "attr_dropout": [""], "attr_rounding_mode": [""], "runtime_dims_masks": [""], "impl": [""]}
     mode, specs = "C", []
     for a in argv:
         if a in ("--matmul", "--reset"):
@@ -260,6 +261,20 @@ def build_problem(sp, seed=7):
         fpmath = {"strict": 0, "bf16": 1, "f16": 2, "any": 3}[mode]
         apply_to_int = flag == "true"
     impl = {"": cabi.IMPL_AUTO, "ref": cabi.IMPL_REF}.get(sp.impl, cabi.IMPL_AUTO)
+    if sp.attr_dropout:
+        # PROBABILITY[:SEED[:TAG[:OFFSET[:HOST_SCALARS]]]] (doc/knobs_attr.md "--attr-dropout"); the mask is laid
+        # out like dst, so TAG only says whether there is one; host scalars are a property of the dnnl_* layer
+        f = sp.attr_dropout.split(":") + [""] * 5
+        seed = int(f[1] or 0)
+        kw["dropout"] = {"p": float(f[0]), "seed": seed, "seed_s64": not -2 ** 31 <= seed < 2 ** 31,
+                         "mask": f[2] != "undef", "offset": int(f[3]) if f[3] else None}
+    if sp.attr_rounding_mode:
+        # ARG:MODE[+...]; a matmul has dst only
+        for item in sp.attr_rounding_mode.split("+"):
+            arg, _, rmode = item.partition(":")
+            if arg != "dst" or rmode not in ("environment", "stochastic"):
+                raise ValueError(f"--attr-rounding-mode={item}")
+            kw["dst_stochastic"] = rmode == "stochastic"
     return MatmulProblem(M=M, N=N, K=K, src_dt=sdt, wei_dt=wdt, dst_dt=ddt, src=src, wei=wei, quant=quant,
                          post_ops=post_ops, apply_to_int=apply_to_int, fpmath_mode=fpmath, dst_init=dst_init,
                          impl=impl, name=sp.desc, **kw)
@@ -321,6 +336,23 @@ def api_objects(p, want_ref_impl=False, runtime_dims_masks=""):
         args[flag | arg] = dnnl.memory(dnnl.memory_desc(qdims, q.dt, tag=dnnl.tag_ab), eng, q.data)
     if p.fpmath_mode or p.apply_to_int:
         attr.set_fpmath_mode(p.fpmath_mode, p.apply_to_int)
+    if p.dropout is not None:
+        dr = p.dropout
+        mask_md = dnnl.memory_desc([p.M, p.N], cabi.DT_U8, tag=dnnl.tag_any) if dr.get("mask") else None
+        seed_dt, seed_np = (dnnl.s64, np.int64) if dr.get("seed_s64") else (cabi.DT_S32, np.int32)
+        attr.set_dropout(mask_md, seed_dt, dr.get("offset") is not None, False)
+
+        def one(dt, v, npdt):
+            return dnnl.memory(dnnl.memory_desc([1], dt, tag=dnnl.tag_a), eng, np.asarray([v], npdt))
+        args[dnnl.ARG_ATTR_DROPOUT_PROBABILITY] = one(cabi.DT_F32, dr["p"], np.float32)
+        args[dnnl.ARG_ATTR_DROPOUT_SEED] = one(seed_dt, dr["seed"], seed_np)
+        if dr.get("offset") is not None:
+            args[dnnl.ARG_ATTR_DROPOUT_OFFSET] = one(dnnl.s64, dr["offset"], np.int64)
+        if dr.get("mask"):
+            args[dnnl.ARG_ATTR_DROPOUT_MASK] = dnnl.memory(dnnl.memory_desc([p.M, p.N], cabi.DT_U8, tag=dnnl.tag_ab), eng,
+                                                           np.full(p.M * p.N, 0xee, np.uint8))
+    if p.dst_stochastic:
+        attr.set_rounding(dnnl.ARG_DST, dnnl.rounding_stochastic)
     po = dnnl.post_ops()
     for i, op in enumerate(p.post_ops):
         if op.kind == cabi.PO_ELTWISE:
@@ -488,6 +520,10 @@ def run_spec(sp, mode="C", min_times=5, max_ms=300.0, settings=None):
         transcendental = any(op.kind == cabi.PO_ELTWISE and op.alg not in (
             cabi.ELTWISE["relu"], cabi.ELTWISE["linear"], cabi.ELTWISE["clip"]) for op in p.post_ops)
         nbad, msg = compare(p, got, want, abs_sum=asum, transcendental=transcendental)
+        if not nbad and p.dropout is not None and p.dropout.get("mask"):
+            got_mask = args[dnnl.ARG_ATTR_DROPOUT_MASK].read(np.uint8)
+            nbad = int(np.count_nonzero(got_mask != p._oracle_mask))
+            msg = f"{nbad} bytes of the dropout mask differ"
         details["errors"] = nbad
         if nbad:
             return "FAILED", impl, msg

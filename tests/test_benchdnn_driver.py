@@ -87,6 +87,15 @@ LINES = [
     "--attr-scales=src:common:0.5+wei:common:0.25+dst:dynamic_mx:e8m0:1x32 --attr-post-ops=,relu 48x128:128x96",
     "--dt=f8_e4m3:f8_e4m3:bf16 --wtag=ba --runtime_dims_masks=3:3 --bia-dt=bf16 --attr-scales=src:common:0.5+wei:common:0.25 "
     "--attr-post-ops=relu+add:bf16 256x512:512x256",
+    # dropout: harness_matmul_smoke_ref:119, harness_matmul_generated_ci:302,335,417,484 (2-D analogues); stochastic
+    # rounding of dst
+    "--dt=f32 --bia-dt=undef,f32 --attr-post-ops=,relu --attr-dropout=0.5:12345678 10x30:30x20",
+    "--dt=f32 --attr-scales=src:common:2:f32 --attr-dropout=0.25:275507:any:660341:false 1x64:64x484",
+    "--dt=f32 --stag=ba --wtag=ba --attr-dropout=0.25:137415:undef:0:false,1:519230:any:0:false 1x921:921x1556",
+    "--dt=f8_e5m2:f8_e5m2:bf16 --attr-scales=src:common:0.5+wei:per_oc --attr-post-ops=clip:-0.5:8 "
+    "--attr-dropout=0.1:760263:undef:0:false 24x512:512x96",
+    "--dt=f32:f32:bf16,bf16:bf16:f16,f32:f32:f8_e4m3 --attr-rounding-mode=dst:stochastic "
+    "--attr-dropout=,0.5:77:any:5000000000 10x30:30x20",
 ]
 
 

@@ -30,7 +30,7 @@ def test_struct_layout_matches_header_sizes():
     assert C.sizeof(cabi.Quant) == 24
     assert C.sizeof(cabi.PostOp) == 56
     assert C.sizeof(cabi.MatmulDesc) == 32 + 16 + 4 * 24 + 7 * 24 + 16 + 32 * 56 + 16
-    assert C.sizeof(cabi.MatmulArgs) == 8 * (11 + 32)
+    assert C.sizeof(cabi.MatmulArgs) == 8 * (11 + 32 + 4)     # + the four dropout pointers
 
 
 def test_query_validates_without_a_device():
