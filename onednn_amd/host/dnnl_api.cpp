@@ -1607,9 +1607,23 @@ bool is_tag_3d(const dnnl_memory_desc &m, bool acb) {
                : (m.strides[0] == K * N && m.strides[1] == N && m.strides[2] == 1);
 }
 
-dnnl_status_t grouped_pd_init(dnnl_primitive_desc &pd, const dnnl_memory_desc &src, const dnnl_memory_desc &wei,
+dnnl_status_t grouped_pd_init(dnnl_primitive_desc &pd, const dnnl_memory_desc &src, const dnnl_memory_desc &wei_in,
         const dnnl_memory_desc *bias, const dnnl_memory_desc &dst_in) {
-    for (const dnnl_memory_desc *m : {&src, &wei, &dst_in}) CHECK_ARG(m->kind != dnnl_format_kind_host_scalar);
+    for (const dnnl_memory_desc *m : {&src, &wei_in, &dst_in}) CHECK_ARG(m->kind != dnnl_format_kind_host_scalar);
+    // Weights given with format_tag::any (the reference's ref_grouped_t takes abc / acb only): K-contiguous
+    // (acb) for the operand types the matrix-core tiles take, as for the plain matmul; row-major otherwise.
+    // The caller reads the layout back with dnnl_primitive_desc_query_md and reorders once.
+    dnnl_memory_desc wei = wei_in;
+    if (wei.kind == dnnl_format_kind_any && wei.ndims == 3 && !wei.grouped) {
+        const bool tiles = wei.dt == src.dt && (is_fp8(wei.dt) || wei.dt == dnnl_bf16 || wei.dt == dnnl_f16);
+        const bool both_fp8 = is_fp8(wei.dt) && is_fp8(src.dt);
+        if (tiles || both_fp8) {
+            const int acb[3] = {0, 2, 1};
+            wei.set_dense(acb);
+        } else {
+            wei.set_dense();
+        }
+    }
     if (bias) CHECK_ARG(bias->kind != dnnl_format_kind_host_scalar);
     CHECK_UNIMPL(src.grouped);
     const bool x3 = dst_in.grouped && !wei.grouped, x2 = wei.grouped && !dst_in.grouped;

@@ -238,3 +238,18 @@ def test_execute_2dx3d_on_the_matrix_cores(gpu, oracle, sdt, wdt):
     prim.execute(strm, args)
     strm.wait()
     assert np.array_equal(dst.read(np.uint8), want)
+
+
+def test_weights_with_format_any_resolve_to_the_layout_of_the_fast_kernel():
+    """Beyond the reference's ref_grouped_t (abc / acb only): `any` weights become K-contiguous (acb) for the
+    operand types the matrix-core tiles take -- what format_tag::any does for the plain matmul -- and row-major
+    otherwise; the caller reads the layout back and reorders once."""
+    eng = dnnl.engine(dnnl.gpu, 0)
+    G, total, K, N = 3, 9, 64, 16
+    for dt, strides, impl in ((BF16, [K * N, 1, K], "hip:mfma_grouped"), (cabi.DT_F8_E4M3, [K * N, 1, K], "hip:mfma_grouped"),
+                              (F32, [K * N, N, 1], "hip:ref_grouped:any")):
+        pd = dnnl.matmul_primitive_desc(eng, dnnl.grouped_memory_desc([total, K], dt, 0, G),
+                                        dnnl.memory_desc([G, K, N], dt, tag=dnnl.tag_any),
+                                        dnnl.grouped_memory_desc([total, N], F32, 0, G))
+        assert pd.impl_info_str() == impl
+        assert pd.query_md(dnnl.query_weights_md).strides() == strides
