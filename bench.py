@@ -52,6 +52,8 @@ PROFILE_OF = {
     ("g1", "any"): "grouped_nsplit_kernel_g1_deepseek_v3_prefill.md",
     ("g2", "any"): "grouped_nsplit_kernel_g2_llama4_scout_prefill.md",
     ("g3", "any"): "grouped_tile_kernel_g3_deepseek_v3_decode.md",
+    ("g4", "any"): "grouped_nsplit_kernel_g4_deepseek_v3_prefill_mxfp8.md",
+    ("g5", "any"): "grouped_nsplit_kernel_g5_deepseek_v3_prefill_mxfp4.md",
 }
 
 
@@ -263,7 +265,7 @@ def run_reorder_workloads(lib, steps, which=("r1", "r2", "r3")):
     return out
 
 
-def run_grouped_workloads(lib, steps, which=("g1", "g2", "g3")):
+def run_grouped_workloads(lib, steps, which=("g1", "g2", "g3", "g4", "g5")):
     """The grouped (mixture-of-experts) matmul on shapes of the reference's
     shapes_grouped_moe files: fp8 e4m3 operands, a scale per src row and per
     group and column, bf16 dst.  HBM-bound: the weights of every group with
@@ -317,7 +319,7 @@ def grouped_cpu_baseline(name):
     """The oracle's restatement of ref_grouped_t on the first groups and columns of the workload."""
     from oracle import binding as oracle
     from onednn_amd import configs
-    groups, N = {"g1": (16, 256), "g2": (2, 256), "g3": (64, 256)}[name]
+    groups, N = {"g1": (16, 256), "g2": (2, 256), "g3": (64, 256), "g4": (16, 256), "g5": (16, 256)}[name]
     p = configs.grouped_config(name, groups=groups, N=N)
     oracle.load()
     reps, t0 = 0, time.time()
@@ -387,10 +389,11 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=3)
-    ap.add_argument("--workload", default="c3", choices=["c1", "c2", "c3", "c4", "c5", "r1", "r2", "r3", "g1", "g2", "g3"],
+    ap.add_argument("--workload", default="c3", choices=["c1", "c2", "c3", "c4", "c5", "r1", "r2", "r3", "g1", "g2", "g3", "g4", "g5"],
                     help="c1..c5: the matmul configurations (c3 is the headline); r1..r3: the reorder "
-                         "primitive on the headline shape's tensors; g1..g3: the grouped (mixture-of-experts) "
-                         "matmul on shapes of the reference's shapes_grouped_moe files (informational)")
+                         "primitive on the headline shape's tensors; g1..g5: the grouped (mixture-of-experts) "
+                         "matmul on shapes of the reference's shapes_grouped_moe files: fp8 with row / column scales "
+                         "(g1..g3), MXFP8 (g4), MXFP4 (g5) (informational)")
     ap.add_argument("--decode-m", type=int, default=1, help="M of the c2 decode workload")
     ap.add_argument("--wtag", default="any", choices=["any", "ab", "ba"],
                     help="weights layout; any = what format_tag::any resolves to (default)")
@@ -510,15 +513,15 @@ def main():
                          "kernel": r["impl"], "kernel_ms": r["ms_per_step"]},
             "cpu_baseline": None, "others": []}), flush=True)
         return
-    if main_name in ("g1", "g2", "g3"):
+    if main_name in ("g1", "g2", "g3", "g4", "g5"):
         r = run_grouped_workloads(lib, args.steps, (main_name,))[0]
         if args.calib_copy:
             calib_copy()
         cpu = None if args.no_cpu else grouped_cpu_baseline(main_name)
         print(json.dumps({
-            "metric": "grouped fp8 matmul GB/s", "value": r["value"], "unit": "GB/s", "n_gpus": 1, "steps": args.steps,
+            "metric": "grouped %s matmul GB/s" % {"g4": "MXFP8", "g5": "MXFP4"}.get(main_name, "fp8"), "value": r["value"], "unit": "GB/s", "n_gpus": 1, "steps": args.steps,
             "warmup": args.warmup, "ms_per_step": r["ms_per_step"], "higher_is_better": True, "scaling": "weak",
-            "vs_baseline": None, "dtype": "f8_e4m3", "data": "synthetic",
+            "vs_baseline": None, "dtype": "f4_e2m1" if main_name == "g5" else "f8_e4m3", "data": "synthetic",
             "config": {"workload": r["workload"], "impl": r["impl"], "tflops": r["tflops"]},
             "roofline": {"bound": "hbm", "achieved": r["value"], "peak": PEAK_HBM_GBS, "unit": "GB/s",
                          "frac": r["frac_of_peak"], "traffic": measured_traffic(main_name)[0],

@@ -456,7 +456,9 @@ typedef struct mi355_grouped_args {
  *                          any pairing), bf16 x bf16 or f16 x f16 with
  *                          K-contiguous weights ([G][N][K], wei_stride[1] == 1,
  *                          16-byte aligned rows, K a multiple of 32 bytes),
- *                          scales without groups along K, no zero points; bias
+ *                          scales without groups along K, or -- fp8 / f4_e2m1 x
+ *                          f4_e2m1 -- e8m0 scales per 32 k on both operands (K a
+ *                          multiple of 512 bytes, N of 4); no zero points; bias
  *                          and every post-op of the list.  f32 accumulation in
  *                          the order of the hardware.
  *   "hip:ref_grouped:any"  everything else the descriptor rules allow: a thread

@@ -236,12 +236,20 @@ GROUPED_SHAPES = {
 }
 
 
+# g4 / g5: the shape of g1 with e8m0 scales per 32 k on both operands (--attr-scales=src:3:e8m0:1x32+wei:7:e8m0:32x1
+# of the same test file): MXFP8 (e4m3) and MXFP4 (e2m1) operands
+GROUPED_SHAPES["g4"] = ("DeepSeek-v3-gate/up-proj-prefill-mxfp8",) + GROUPED_SHAPES["g1"][1:]
+GROUPED_SHAPES["g5"] = ("DeepSeek-v3-gate/up-proj-prefill-mxfp4",) + GROUPED_SHAPES["g1"][1:]
+GROUPED_FORMAT = {"g1": "f8", "g2": "f8", "g3": "f8", "g4": "mxf8", "g5": "mxf4"}
+
+
 def grouped_config(name, seed=9, groups=None, N=None):
-    """One of GROUPED_SHAPES as a GroupedProblem with random fp8 operands
-    (finite e4m3 bytes over eight binades), f32 scales in [0.5, 2) and a bf16
-    dst.  `groups` / `N`: only the first groups / columns (CPU samples)."""
+    """One of GROUPED_SHAPES as a GroupedProblem with random operands (fp8: finite e4m3 bytes over eight binades;
+    fp4: random nibbles) and a bf16 dst; scales per src row and per group and column (f32 in [0.5, 2)) or, for the
+    MX formats, e8m0 scales per 32 k (2^-2 .. 2^1).  `groups` / `N`: only the first groups / columns (CPU samples)."""
     from .grouped import GroupedProblem, GroupedQuant
     label, K, n_full, sizes = GROUPED_SHAPES[name]
+    fmt = GROUPED_FORMAT[name]
     sizes = list(sizes[:groups] if groups else sizes)
     N = N or n_full
     G, total = len(sizes), int(sum(sizes))
@@ -250,17 +258,31 @@ def grouped_config(name, seed=9, groups=None, N=None):
     def fp8(shape):
         return (rng.integers(0, 2, shape, dtype=np.uint8) << 7) | rng.integers(0x20, 0x60, shape, dtype=np.uint8)
 
-    quant = {"src_scale": GroupedQuant(cabi.DT_F32, rng.uniform(0.5, 2.0, total).astype(np.float32), 0),
-             "wei_scale": GroupedQuant(cabi.DT_F32, rng.uniform(0.5, 2.0, (G, N)).astype(np.float32), 0)}
-    return GroupedProblem(pattern=cabi.GROUPED_2DX3D, sizes=sizes, K=K, N=N, src_dt=cabi.DT_F8_E4M3,
-                          wei_dt=cabi.DT_F8_E4M3, dst_dt=cabi.DT_BF16, src=fp8((total, K)), wei=fp8((G, N, K)),
-                          wei_stride=(K * N, 1, K), quant=quant, name=f"{name.upper()} {label} {total}x{K}:{G}x{K}x{N}")
+    if fmt == "mxf4":
+        dt, kb = cabi.DT_F4_E2M1, K // 2
+        src, wei = rng.integers(0, 256, (total, kb), dtype=np.uint8), rng.integers(0, 256, (G, N, kb), dtype=np.uint8)
+    else:
+        dt, kb = cabi.DT_F8_E4M3, K
+        src, wei = fp8((total, K)), fp8((G, N, K))
+    if fmt == "f8":
+        quant = {"src_scale": GroupedQuant(cabi.DT_F32, rng.uniform(0.5, 2.0, total).astype(np.float32), 0),
+                 "wei_scale": GroupedQuant(cabi.DT_F32, rng.uniform(0.5, 2.0, (G, N)).astype(np.float32), 0)}
+    else:
+        quant = {"src_scale": GroupedQuant(cabi.DT_E8M0, rng.integers(125, 129, (total, K // 32), dtype=np.uint8), 32),
+                 "wei_scale": GroupedQuant(cabi.DT_E8M0, rng.integers(125, 129, (G, K // 32, N), dtype=np.uint8), 32)}
+    return GroupedProblem(pattern=cabi.GROUPED_2DX3D, sizes=sizes, K=K, N=N, src_dt=dt, wei_dt=dt, dst_dt=cabi.DT_BF16,
+                          src=src, wei=wei, wei_stride=(K * N, 1, K), quant=quant,
+                          name=f"{name.upper()} {label} {total}x{K}:{G}x{K}x{N}")
 
 
 def grouped_bytes(p):
-    """Algorithmic HBM bytes of a grouped fp8 launch: the weights of every group
-    that has rows, src, dst, scales and offsets, each once."""
+    """Algorithmic HBM bytes of a grouped launch: the weights (and their scales) of every group that has rows, src,
+    dst, src scales and offsets, each once."""
     active = sum(1 for m in p.sizes if m)
-    es = cabi.DT_BITS[p.wei_dt] // 8
-    return (active * p.K * p.N * es + p.total * p.K * es + p.total * p.N * cabi.DT_BITS[p.dst_dt] // 8
-            + 4 * p.total + 4 * active * p.N + 8 * p.G)
+    ebits = cabi.DT_BITS[p.wei_dt]
+    total = active * p.K * p.N * ebits // 8 + p.total * p.K * ebits // 8 + p.total * p.N * cabi.DT_BITS[p.dst_dt] // 8
+    for name, rows in (("src_scale", p.total), ("wei_scale", active * p.N)):
+        q = p.quant.get(name)
+        if q is not None:
+            total += rows * (p.K // q.group_k if q.group_k else 1) * cabi.DT_BITS[q.dt] // 8
+    return total + 8 * p.G

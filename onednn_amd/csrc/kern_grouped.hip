@@ -181,14 +181,42 @@ typedef float g4f __attribute__((ext_vector_type(4)));
 typedef __bf16 g8bf __attribute__((ext_vector_type(8)));
 typedef _Float16 g8h __attribute__((ext_vector_type(8)));
 
-enum { GM_F8 = 0, GM_BF16 = 1, GM_F16 = 2 };
+enum { GM_F8 = 0, GM_BF16 = 1, GM_F16 = 2, GM_MXF8 = 3, GM_MXF4 = 4 };
+
+// GM_MXF8 / GM_MXF4: e8m0 scales per 32 consecutive k on both operands, applied by the instruction
+// (v_mfma_scale_f32_16x16x128_f8f6f4).  Lane (j, q) supplies the scale of block q of row j.  Its data
+// are, for fp8, k 16 q .. 16 q + 15 and 64 + 16 q .. 64 + 16 q + 15 (chunks q and 4 + q of the step, as
+// without scales: the instruction takes the halves of blocks q / 2 and 2 + q / 2 from it and their scales
+// from the lanes that own those blocks); for fp4 a 16-byte chunk is a block and chunks q and 4 + q feed two
+// instructions.  (Found by measurement: with a lane holding one whole fp8 block the scales came out wrong.)
+template <int MODE>
+struct gmode_t {
+    static constexpr int EBITS = (MODE == GM_BF16 || MODE == GM_F16) ? 16 : (MODE == GM_MXF4 ? 4 : 8);
+    static constexpr int SB = MODE == GM_MXF8 ? 1 : (MODE == GM_MXF4 ? 2 : 0); // scale dwords per step and row
+    static constexpr bool MX = SB != 0;
+    static constexpr int BPS = 4 * SB;                                          // blocks of 32 k per 128-byte step
+    __device__ static __forceinline__ long bytes(long elems) { return elems * EBITS / 8; }
+    // the two chunks of a step lane (j, q) ends up with
+    __device__ static __forceinline__ int chunk_lo(int q) { return q; }
+    __device__ static __forceinline__ int chunk_hi(int q) { return 4 + q; }
+    // the chunk lane (j, q) fetches (of rows j % 8 and 8 + j % 8) before the exchange
+    __device__ static __forceinline__ int chunk_fetch(int q, int half) { return q + 4 * half; }
+};
 
 // weights fragment first: the tile comes out transposed, a lane holds four
-// consecutive n (4 * (lane / 16) + e) of row lane % 16
+// consecutive n (4 * (lane / 16) + e) of row lane % 16.  sw / sa: the lane's e8m0 scale bytes (MX modes).
 template <int MODE, int FA, int FB>
-__device__ __forceinline__ g4f grouped_mma(const g8i &w, const g8i &a, g4f c) {
+__device__ __forceinline__ g4f grouped_mma(const g8i &w, const g8i &a, g4f c, const int *sw = nullptr,
+        const int *sa = nullptr) {
     if constexpr (MODE == GM_F8) {
         return __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(w, a, c, FB, FA, 0, 0, 0, 0);
+    } else if constexpr (MODE == GM_MXF8) {
+        return __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(w, a, c, FB, FA, 0, sw[0], 0, sa[0]);
+    } else if constexpr (MODE == GM_MXF4) {
+        const g8i wl = {w[0], w[1], w[2], w[3], 0, 0, 0, 0}, wh = {w[4], w[5], w[6], w[7], 0, 0, 0, 0};
+        const g8i al = {a[0], a[1], a[2], a[3], 0, 0, 0, 0}, ah = {a[4], a[5], a[6], a[7], 0, 0, 0, 0};
+        c = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(wl, al, c, 4, 4, 0, sw[0], 0, sa[0]);
+        return __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(wh, ah, c, 4, 4, 0, sw[1], 0, sa[1]);
     } else {
         const g4i wl = {w[0], w[1], w[2], w[3]}, wh = {w[4], w[5], w[6], w[7]};
         const g4i al = {a[0], a[1], a[2], a[3]}, ah = {a[4], a[5], a[6], a[7]};
@@ -206,6 +234,44 @@ __device__ __forceinline__ g4f grouped_mma(const g8i &w, const g8i &a, g4f c) {
     }
 }
 
+// what a workgroup knows about its tile (uniform over the workgroup)
+struct gtile_t {
+    long g, m_base, rows; // group, first row of the tile inside the group, rows of the group
+    long dst0, src0;      // first row of the group in dst / src
+    long n0;              // first column of the tile
+};
+
+// The weights' scales of one step for NT * 16 columns, [G][K / 32][N] with N contiguous: lane (j, q)
+// fetches the dword of columns 4 j .. 4 j + 3 of block row q (and 4 + q for fp4); the byte lane (j, q)
+// needs for fragment jn -- column 16 jn + j, block q -- sits in lane (4 jn + j / 4, q), byte j % 4.
+template <int MODE, int NT>
+struct gscale_b_t {
+    using Mo = gmode_t<MODE>;
+    const char *base; // scales of this group at the tile's first column (uniform)
+    uint32_t off;     // lane part: block row q, dword of columns
+    long N;
+    __device__ __forceinline__ void init(const grouped_dev_t &P, const gtile_t &T, long n_first, int lane) {
+        const int j = lane & 15, q = lane >> 4;
+        N = P.d.N;
+        const long kb = P.d.K / 32;
+        int jj = j < 4 * NT ? j : 4 * NT - 1;
+        long col = n_first + 4 * jj;
+        col = col <= N - 4 ? col : N - 4; // N is a multiple of 4: a dword is inside or outside as a whole
+        base = (const char *)P.a.wei_scale + T.g * kb * N;
+        off = (uint32_t)(q * N + col);
+    }
+    __device__ __forceinline__ void load(long step, int (&raw)[2]) const {
+#pragma unroll
+        for (int h = 0; h < Mo::SB; ++h) raw[h] = *(const int *)(base + (step * Mo::BPS + 4 * h) * N + off);
+    }
+    __device__ __forceinline__ void pick(const int (&raw)[2], int jn, int lane, int (&out)[2]) const {
+        const int j = lane & 15, q = lane >> 4;
+        const int from = 4 * (16 * q + 4 * jn + (j >> 2));
+#pragma unroll
+        for (int h = 0; h < Mo::SB; ++h) out[h] = (__builtin_amdgcn_ds_bpermute(from, raw[h]) >> (8 * (j & 3))) & 0xff;
+    }
+};
+
 // rows of group g that both src and dst hold, and where they start; offsets
 // that leave [0, total] or run backwards give fewer rows, never an access
 // outside the tensors
@@ -219,31 +285,24 @@ __device__ __forceinline__ long grouped_rows(const grouped_dev_t &P, long g, lon
     return n > 0 ? n : 0;
 }
 
-// what a workgroup knows about its tile (uniform over the workgroup)
-struct gtile_t {
-    long g, m_base, rows; // group, first row of the tile inside the group, rows of the group
-    long dst0, src0;      // first row of the group in dst / src
-    long n0;              // first column of the tile
-};
-
 // One wavefront's share of a tile's K walk: steps wk, wk + WK, .. of 128 bytes per
 // row for MF fragments of 16 src rows against NT fragments of 16 weights rows,
 // D steps in flight.  Leaves the MF x NT accumulators in `part`.
 template <int MODE, int FA, int FB, int MF, int NT, int D, int WK>
 __device__ __forceinline__ void grouped_walk(const grouped_dev_t &P, const gtile_t &T, g4f *part, int wk, int lane) {
-    constexpr int ES = MODE == GM_F8 ? 1 : 2; // bytes per element
+    using Mo = gmode_t<MODE>;
     const mi355_grouped_desc_t &Dd = P.d;
     const int j = lane & 15, q = lane >> 4;
-    const long row_bytes = Dd.K * ES;
+    const long row_bytes = Mo::bytes(Dd.K);
     // A load instruction fetches whole 128-byte lines: 8 rows x 8 chunks of 16
-    // bytes.  Lane (j, q) fetches chunk q + 4 (j / 8) of rows j % 8 and 8 + j % 8
-    // of a fragment; lanes j and j +- 8 then exchange one of the two so that
-    // lane (j, q) holds chunks q and 4 + q of row j.
+    // bytes.  Lane (j, q) fetches one chunk of rows j % 8 and 8 + j % 8 of a
+    // fragment; lanes j and j +- 8 then exchange one of the two so that lane
+    // (j, q) holds two chunks of row j (which ones: gmode_t).
     const int half = j >> 3;
-    const uint32_t chunk = 16 * (q + 4 * half);
-    const long pitch_b = Dd.wei_stride[2] * ES;
+    const uint32_t chunk = 16 * Mo::chunk_fetch(q, half);
+    const long pitch_b = Mo::bytes(Dd.wei_stride[2]);
     const char *abase = (const char *)P.a.src + (T.src0 + T.m_base) * row_bytes;
-    const char *bbase = (const char *)P.a.wei + (T.g * Dd.wei_stride[0] + T.n0 * Dd.wei_stride[2]) * ES;
+    const char *bbase = (const char *)P.a.wei + Mo::bytes(T.g * Dd.wei_stride[0] + T.n0 * Dd.wei_stride[2]);
     uint32_t aoff[MF][2], boff[NT][2];
 #pragma unroll
     for (int i = 0; i < MF; ++i)
@@ -261,8 +320,23 @@ __device__ __forceinline__ void grouped_walk(const grouped_dev_t &P, const gtile
             n = n < Dd.N ? n : Dd.N - 1;
             boff[jn][h] = (uint32_t)((n - T.n0) * pitch_b) + chunk;
         }
+    // MX: the src scales of row 16 i + j ([total_M][K / 32], a dword or two per step) and the weights' scales
+    const long kblocks = Dd.K / 32;
+    const char *sabase = Mo::MX ? (const char *)P.a.src_scale + (T.src0 + T.m_base) * kblocks : nullptr;
+    uint32_t saoff[MF];
+    gscale_b_t<MODE, NT> SBs;
+    if constexpr (Mo::MX) {
+#pragma unroll
+        for (int i = 0; i < MF; ++i) {
+            long m = T.m_base + 16 * i + j;
+            m = m < T.rows ? m : T.rows - 1;
+            saoff[i] = (uint32_t)((m - T.m_base) * kblocks);
+        }
+        SBs.init(P, T, T.n0, lane);
+    }
     struct stage_t {
         g4i a[MF][2], b[NT][2];
+        int sa[MF][2], sb[2];
     };
     // step_off: byte offset of the step in a row (uniform)
     auto load = [&](long step_off, uint32_t back) __attribute__((always_inline)) {
@@ -275,6 +349,14 @@ __device__ __forceinline__ void grouped_walk(const grouped_dev_t &P, const gtile
         for (int i = 0; i < MF; ++i)
 #pragma unroll
             for (int h = 0; h < 2; ++h) f.a[i][h] = *(const g4i *)(abase + step_off + (aoff[i][h] - back));
+        if constexpr (Mo::MX) {
+            const long step = step_off >> 7;
+            SBs.load(step, f.sb);
+#pragma unroll
+            for (int i = 0; i < MF; ++i)
+#pragma unroll
+                for (int h = 0; h < Mo::SB; ++h) f.sa[i][h] = *(const int *)(sabase + step * Mo::BPS + 4 * h + saoff[i]);
+        }
         return f;
     };
     // the exchange between lanes j and j +- 8 (a rotation by 8 inside each row of 16 lanes)
@@ -296,13 +378,20 @@ __device__ __forceinline__ void grouped_walk(const grouped_dev_t &P, const gtile
         for (int jn = 0; jn < NT; ++jn) acc[i][jn] = g4f {0.f, 0.f, 0.f, 0.f};
     auto compute = [&](const stage_t &f) __attribute__((always_inline)) {
         g8i a[MF];
+        int sa[MF][2];
 #pragma unroll
-        for (int i = 0; i < MF; ++i) a[i] = settle(f.a[i]);
+        for (int i = 0; i < MF; ++i) {
+            a[i] = settle(f.a[i]);
+#pragma unroll
+            for (int h = 0; h < 2; ++h) sa[i][h] = Mo::MX ? (f.sa[i][h] >> (8 * q)) & 0xff : 0; // block q (4 + q) of the step
+        }
 #pragma unroll
         for (int jn = 0; jn < NT; ++jn) {
             const g8i w = settle(f.b[jn]);
+            int sw[2] = {0, 0};
+            if constexpr (Mo::MX) SBs.pick(f.sb, jn, lane, sw);
 #pragma unroll
-            for (int i = 0; i < MF; ++i) acc[i][jn] = grouped_mma<MODE, FA, FB>(w, a[i], acc[i][jn]);
+            for (int i = 0; i < MF; ++i) acc[i][jn] = grouped_mma<MODE, FA, FB>(w, a[i], acc[i][jn], sw, sa[i]);
         }
     };
 
@@ -414,7 +503,9 @@ __device__ __forceinline__ void grouped_store_quad(const grouped_dev_t &P, const
     const mi355_grouped_desc_t &Dd = P.d;
     const long N = Dd.N;
     if (m >= T.rows || nb >= N) return;
-    const bool with_ss = Dd.src_scale_dt != MI355_DT_UNDEF, with_ws = Dd.wei_scale_dt != MI355_DT_UNDEF;
+    // scales with groups along K (the MX modes) were applied by the matrix instruction
+    const bool with_ss = Dd.src_scale_dt != MI355_DT_UNDEF && Dd.src_scale_gk <= 1;
+    const bool with_ws = Dd.wei_scale_dt != MI355_DT_UNDEF && Dd.wei_scale_gk <= 1;
     const int dbits = dt_bits(Dd.dst_dt);
     const bool vec_ok = N % 4 == 0 && ((uintptr_t)P.a.dst % 16) == 0;
     const float ss = with_ss ? load_float(Dd.src_scale_dt, P.a.src_scale, T.src0 + m) : 1.f;
@@ -525,11 +616,12 @@ __device__ __forceinline__ void grouped_walk_nsplit(const grouped_dev_t &P, cons
         int lane) {
     constexpr int CH = 4; // steps per src chunk in LDS
     static_assert(CH % D == 0, "a step's register stage must not depend on the chunk");
-    constexpr int ES = MODE == GM_F8 ? 1 : 2;
+    using Mo = gmode_t<MODE>;
     constexpr unsigned ABUF = MF * CH * 2048; // bytes of one src buffer
+    constexpr unsigned SBUF = Mo::SB * 1024;    // MX: the src scales of a chunk, 16 bytes (two of them for fp4) per row
     const mi355_grouped_desc_t &Dd = P.d;
     const int j = lane & 15, q = lane >> 4;
-    const long row_bytes = Dd.K * ES;
+    const long row_bytes = Mo::bytes(Dd.K);
     const long nfull = row_bytes / 128;
     const int tail = (int)(row_bytes % 128); // a multiple of 32
     const long nsteps = nfull + (tail != 0);
@@ -537,9 +629,9 @@ __device__ __forceinline__ void grouped_walk_nsplit(const grouped_dev_t &P, cons
 
     // ---- weights: as in grouped_walk, for this wavefront's 64 columns
     const int half = j >> 3;
-    const uint32_t chunk = 16 * (q + 4 * half);
-    const long pitch_b = Dd.wei_stride[2] * ES;
-    const char *bbase = (const char *)P.a.wei + (T.g * Dd.wei_stride[0] + T.n0 * Dd.wei_stride[2]) * ES;
+    const uint32_t chunk = 16 * Mo::chunk_fetch(q, half);
+    const long pitch_b = Mo::bytes(Dd.wei_stride[2]);
+    const char *bbase = (const char *)P.a.wei + Mo::bytes(T.g * Dd.wei_stride[0] + T.n0 * Dd.wei_stride[2]);
     uint32_t boff[NT][2];
 #pragma unroll
     for (int jn = 0; jn < NT; ++jn)
@@ -551,7 +643,10 @@ __device__ __forceinline__ void grouped_walk_nsplit(const grouped_dev_t &P, cons
         }
     struct stage_t {
         g4i b[NT][2];
+        int sb[2];
     };
+    gscale_b_t<MODE, NT> SBs;
+    if constexpr (Mo::MX) SBs.init(P, T, T.n0 + 16 * NT * wave, lane);
     // A lane whose chunk lies beyond K in the tail step fetches the step's first chunk
     // instead (the tail holds at least 32 bytes); steps beyond the last repeat it.
     const uint32_t b_back = chunk + 16 <= (uint32_t)tail ? 0 : chunk;
@@ -563,6 +658,7 @@ __device__ __forceinline__ void grouped_walk_nsplit(const grouped_dev_t &P, cons
         for (int jn = 0; jn < NT; ++jn)
 #pragma unroll
             for (int h = 0; h < 2; ++h) f.b[jn][h] = *(const g4i *)(bbase + s * 128 + (boff[jn][h] - back));
+        if constexpr (Mo::MX) SBs.load(s, f.sb);
         return f;
     };
     auto settle = [&](const g4i (&r)[2]) __attribute__((always_inline)) {
@@ -593,6 +689,16 @@ __device__ __forceinline__ void grouped_walk_nsplit(const grouped_dev_t &P, cons
         m = m < T.rows ? m : T.rows - 1; // rows beyond the group read its last one (never stored)
         a_row[x] = (uint32_t)((m - T.m_base) * row_bytes);
     }
+    // MX: wavefront 3 also brings the chunk's src scales, lane L those of row L of the tile: 16 bytes = four steps
+    // of four blocks (fp8); for fp4 (eight blocks a step) a second instruction brings the next 16
+    const long kblocks = Dd.K / 32;
+    const char *sabase = Mo::MX ? (const char *)P.a.src_scale + (T.src0 + T.m_base) * kblocks : nullptr;
+    uint32_t sa_row = 0;
+    if constexpr (Mo::MX) {
+        long m = T.m_base + lane;
+        m = m < T.rows ? m : T.rows - 1;
+        sa_row = (uint32_t)((m - T.m_base) * kblocks);
+    }
     auto issue_a = [&](long c, int which) __attribute__((always_inline)) {
         const unsigned buf = lds0 + (unsigned)which * ABUF;
 #pragma unroll
@@ -603,8 +709,16 @@ __device__ __forceinline__ void grouped_walk_nsplit(const grouped_dev_t &P, cons
             const uint32_t voff = a_row[x] + a_chunk - (s >= nfull ? a_back : 0);
             grouped_dma16(abase + s * 128, voff, buf + (unsigned)blk * 2048 + (unsigned)(inst & 1) * 1024);
         }
+        if constexpr (Mo::MX) {
+            if (wave == 3) {
+#pragma unroll
+                for (int h = 0; h < Mo::SB; ++h)
+                    grouped_dma16(sabase + c * (CH * Mo::BPS) + 16 * h, sa_row,
+                            lds0 + 2 * ABUF + (unsigned)which * SBUF + (unsigned)h * 1024);
+            }
+        }
     };
-    const unsigned a_lo = 16 * (8 * j + (q ^ (j >> 1))), a_hi = 16 * (8 * j + ((4 + q) ^ (j >> 1)));
+    const unsigned a_lo = 16 * (8 * j + (Mo::chunk_lo(q) ^ (j >> 1))), a_hi = 16 * (8 * j + (Mo::chunk_hi(q) ^ (j >> 1)));
     const bool lo_in = 16 * q + 16 <= tail, hi_in = 64 + 16 * q + 16 <= tail; // the lane's chunks in the tail step
 
     g4f acc[MF][NT];
@@ -632,7 +746,7 @@ __device__ __forceinline__ void grouped_walk_nsplit(const grouped_dev_t &P, cons
     for (long x = 0; x < nchunks; ++x) {
         // memory operations return in order: once at most the D stages of weights issued
         // after this wavefront's part of the chunk are in flight, that part has landed
-        asm volatile("s_waitcnt vmcnt(%0)" ::"n"(D * NT * 2) : "memory");
+        asm volatile("s_waitcnt vmcnt(%0)" ::"n"(D * (NT * 2 + Mo::SB)) : "memory");
         __syncthreads();
         if (x + 1 < nchunks) issue_a(chunk_at(x + 1), (x + 1) & 1); // into the buffer whose readers passed the barrier
         __builtin_amdgcn_sched_barrier(0);
@@ -649,6 +763,26 @@ __device__ __forceinline__ void grouped_walk_nsplit(const grouped_dev_t &P, cons
                     const g4i lo = *(lds_g4i_ptr_t)(size_t)(blk + a_lo), hi = *(lds_g4i_ptr_t)(size_t)(blk + a_hi);
                     a[i] = g8i {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
                 }
+                int sa[MF][2];
+#pragma unroll
+                for (int i = 0; i < MF; ++i)
+#pragma unroll
+                    for (int h = 0; h < 2; ++h) {
+                        sa[i][h] = 0;
+                        if constexpr (Mo::MX) {
+                            if (h < Mo::SB) {
+                                // row 16 i + j, the dword of this step's blocks (fp4: 0..3 and 4..7), byte q
+                                const unsigned at = lds0 + 2 * ABUF + (unsigned)(x & 1) * SBUF + (unsigned)h * 1024
+                                        + (unsigned)(16 * i + j) * 16 + (unsigned)((t * Mo::SB + h) % 4) * 4;
+                                // fp4: steps 0, 1 sit in the first 16 bytes of the row, steps 2, 3 in the second
+                                const unsigned at4 = lds0 + 2 * ABUF + (unsigned)(x & 1) * SBUF
+                                        + (unsigned)((t * 2 + h) / 4) * 1024 + (unsigned)(16 * i + j) * 16
+                                        + (unsigned)((t * 2 + h) % 4) * 4;
+                                const int raw = *(const int __attribute__((address_space(3))) *)(size_t)(Mo::SB == 2 ? at4 : at);
+                                sa[i][h] = (raw >> (8 * q)) & 0xff;
+                            }
+                        }
+                    }
                 const bool is_tail = s >= nfull;
                 if (is_tail) {
 #pragma unroll
@@ -669,8 +803,10 @@ __device__ __forceinline__ void grouped_walk_nsplit(const grouped_dev_t &P, cons
                             if (!hi_in) w[4 + e] = 0;
                         }
                     }
+                    int sw[2] = {0, 0};
+                    if constexpr (Mo::MX) SBs.pick(st[t % D].sb, jn, lane, sw);
 #pragma unroll
-                    for (int i = 0; i < MF; ++i) acc[i][jn] = grouped_mma<MODE, FA, FB>(w, a[i], acc[i][jn]);
+                    for (int i = 0; i < MF; ++i) acc[i][jn] = grouped_mma<MODE, FA, FB>(w, a[i], acc[i][jn], sw, sa[i]);
                 }
             }
             st[t % D] = load_b(step_at(x * CH + t + D));
@@ -741,22 +877,30 @@ int tile_plan(const mi355_grouped_desc_t &d) {
     const char *env = getenv("MI355_GROUPED_IMPL");
     if (env && !strcmp(env, "ref")) return 0;
     const bool f8 = f8_dt(d.src_dt) && f8_dt(d.wei_dt);
+    const bool f4 = d.src_dt == MI355_DT_F4_E2M1 && d.wei_dt == MI355_DT_F4_E2M1;
     const bool h16 = d.src_dt == d.wei_dt && (d.src_dt == MI355_DT_BF16 || d.src_dt == MI355_DT_F16);
-    if (!f8 && !h16) return 0;
-    const long es = f8 ? 1 : 2;
+    if (!f8 && !h16 && !f4) return 0;
+    const long ebits = f4 ? 4 : (f8 ? 8 : 16);
+    auto bytes = [&](long elems) { return elems * ebits / 8; };
     if (d.wei_stride[1] != 1 || d.wei_stride[2] < d.K) return 0; // K-contiguous weights only
-    if ((d.wei_stride[2] * es) % 16 != 0 || (d.wei_stride[0] * es) % 16 != 0 || (d.K * es) % 32 != 0) return 0;
-    if (d.wei_stride[2] * es > (1L << 24)) return 0; // 32-bit offsets inside a tile
-    auto k_groups = [&](int dt, long gk) { return dt != MI355_DT_UNDEF && gk > 1 && gk != d.K; };
-    if (k_groups(d.src_scale_dt, d.src_scale_gk) || k_groups(d.wei_scale_dt, d.wei_scale_gk)) return 0;
+    if (bytes(d.wei_stride[2]) % 16 != 0 || bytes(d.wei_stride[0]) % 16 != 0 || bytes(d.K) % 32 != 0 || d.K % 2 != 0) return 0;
+    if (bytes(d.wei_stride[2]) > (1L << 24)) return 0; // 32-bit offsets inside a tile
     if (d.src_zp_dt != MI355_DT_UNDEF || d.wei_zp_dt != MI355_DT_UNDEF) return 0;
+    auto k_groups = [&](int dt, long gk) { return dt != MI355_DT_UNDEF && gk > 1 && gk != d.K; };
+    const bool sg = k_groups(d.src_scale_dt, d.src_scale_gk), wg = k_groups(d.wei_scale_dt, d.wei_scale_gk);
+    // MX: e8m0 scales per 32 k on both operands of fp8 / fp4 tensors, applied by the instruction; whole
+    // 512-byte chunks of K (16 or 32 scale bytes a row), dword loads of the weights' scales along N
+    const bool mx = sg && wg && (f8 || f4) && d.src_scale_dt == MI355_DT_E8M0 && d.wei_scale_dt == MI355_DT_E8M0
+            && d.src_scale_gk == 32 && d.wei_scale_gk == 32 && bytes(d.K) % 512 == 0 && d.N % 4 == 0;
+    if ((sg || wg) && !mx) return 0;
+    if (f4 && !mx) return 0;
     const long active = d.group_count < d.total ? d.group_count : d.total;
     // Groups of a row or two: the small tiles.  Otherwise the 256-column tiles (a quarter of
     // the src traffic per byte of weights), unless they are too few to fill the device or
     // the rows are not whole lines (K not a multiple of 128 bytes: measured slower there).
     int plan = 3;
     if (d.total <= 2 * d.group_count) plan = 1;
-    else if ((d.K * es) % 128 != 0 || (d.N + 255) / 256 * active < 256) plan = 2;
+    else if (bytes(d.K) % 128 != 0 || (d.N + 255) / 256 * active < 256) plan = 2;
     if (env && !strcmp(env, "short")) plan = 1;
     if (env && !strcmp(env, "tall")) plan = 2;
     if (env && !strcmp(env, "wide")) plan = 3;
@@ -777,9 +921,16 @@ int launch_tiles(int plan, const grouped_dev_t &P, hipStream_t stream) {
         return hipGetLastError() == hipSuccess ? MI355_SUCCESS : MI355_RUNTIME_ERROR;
     };
     if (plan == 1) return go(grouped_tile_kernel<MODE, FA, FB, 1, 2, 4, 4, 1>, 1, 2, 4);
-    if (plan == 2) return go(grouped_tile_kernel<MODE, FA, FB, 3, 4, 2, 4, 2>, 3, 4, 4);
-    // two src buffers of 4 fragments x 4 steps; the accumulators fit the same space
-    return go(grouped_nsplit_kernel<MODE, FA, FB, 4, 4, 2>, 4, 4, 4);
+    // (the MX modes hold their scales too and do not fit two workgroups' registers)
+    if (plan == 2) return go(grouped_tile_kernel<MODE, FA, FB, 3, 4, 2, 4, gmode_t<MODE>::MX ? 1 : 2>, 3, 4, 4);
+    // two src buffers of 4 fragments x 4 steps (the accumulators fit the same space) + the MX scales of two chunks
+    {
+        auto kern = grouped_nsplit_kernel<MODE, FA, FB, 4, 4, 2>;
+        const int lds = 2 * 4 * 4 * 2048 + 2 * gmode_t<MODE>::SB * 1024;
+        if (const int st = ensure_dynamic_lds((const void *)kern, lds, "mfma_grouped")) return st;
+        hipLaunchKernelGGL(kern, grid, dim3(256), lds, stream, P);
+        return hipGetLastError() == hipSuccess ? MI355_SUCCESS : MI355_RUNTIME_ERROR;
+    }
 }
 
 } // namespace
@@ -865,12 +1016,22 @@ extern "C" int mi355_grouped_matmul_launch(const mi355_grouped_desc_t *d, const 
         return MI355_UNIMPLEMENTED;
     }
     // the tiles read 16 bytes at a time
-    const int plan = ((uintptr_t)a->src % 16 == 0 && (uintptr_t)a->wei % 16 == 0) ? tile_plan(*d) : 0;
+    const bool aligned = (uintptr_t)a->src % 16 == 0 && (uintptr_t)a->wei % 16 == 0
+            && (d->src_scale_gk <= 1 || ((uintptr_t)a->src_scale % 16 == 0 && (uintptr_t)a->wei_scale % 4 == 0));
+    const int plan = aligned ? tile_plan(*d) : 0;
     if (plan != 0) {
         hipStream_t s = (hipStream_t)stream;
         const int fa = d->src_dt == MI355_DT_F8_E5M2, fb = d->wei_dt == MI355_DT_F8_E5M2;
+        const bool mx = d->src_scale_dt != MI355_DT_UNDEF && d->src_scale_gk > 1;
         if (d->src_dt == MI355_DT_BF16) return launch_tiles<GM_BF16, 0, 0>(plan, P, s);
         if (d->src_dt == MI355_DT_F16) return launch_tiles<GM_F16, 0, 0>(plan, P, s);
+        if (d->src_dt == MI355_DT_F4_E2M1) return launch_tiles<GM_MXF4, 0, 0>(plan, P, s);
+        if (mx) {
+            if (!fa && !fb) return launch_tiles<GM_MXF8, 0, 0>(plan, P, s);
+            if (fa && fb) return launch_tiles<GM_MXF8, 1, 1>(plan, P, s);
+            if (fa) return launch_tiles<GM_MXF8, 1, 0>(plan, P, s);
+            return launch_tiles<GM_MXF8, 0, 1>(plan, P, s);
+        }
         if (!fa && !fb) return launch_tiles<GM_F8, 0, 0>(plan, P, s);
         if (fa && fb) return launch_tiles<GM_F8, 1, 1>(plan, P, s);
         if (fa) return launch_tiles<GM_F8, 1, 0>(plan, P, s);

@@ -36,9 +36,10 @@ def _vals(rng, dt, shape):
 
 
 def case_2dx3d(sizes, K, N, src_dt=cabi.DT_F32, wei_dt=cabi.DT_F32, dst_dt=cabi.DT_F32, wtag="abc", bias=False,
-               src_scale=None, wei_scale=None, src_zp=None, wei_zp=None, post_ops=(), seed=5):
+               src_scale=None, wei_scale=None, src_zp=None, wei_zp=None, post_ops=(), seed=5, mx=False):
     """src_scale / src_zp: None, "row" or a K group size; wei_scale / wei_zp: None, "col" or a K group size.
     post_ops: names out of relu, linear, mul_group, mul_row, mul_full, mul_grouped.
+    mx: e8m0 scales per 32 k on both operands (--attr-scales=src:3:e8m0:1x32+wei:7:e8m0:32x1).
     Returns (problem, expected float64 [total_M][N])."""
     rng = np.random.default_rng(seed)
     G, total = len(sizes), int(sum(sizes))
@@ -60,6 +61,11 @@ def case_2dx3d(sizes, K, N, src_dt=cabi.DT_F32, wei_dt=cabi.DT_F32, dst_dt=cabi.
         ws = rng.choice([0.125, 0.5, 1.0, 4.0], size=(G, kgroups(wei_scale), N))
         quant["wei_scale"] = GroupedQuant(cabi.DT_BF16, dtp.f32_to_bf16(ws.astype(np.float32)),
                                           0 if wei_scale == "col" else wei_scale)
+    if mx:
+        ss = rng.choice([0.25, 0.5, 1.0, 2.0], size=(total, K // 32))
+        ws = rng.choice([0.125, 0.5, 1.0, 4.0], size=(G, K // 32, N))
+        quant["src_scale"] = GroupedQuant(cabi.DT_E8M0, encode(cabi.DT_E8M0, ss), 32)
+        quant["wei_scale"] = GroupedQuant(cabi.DT_E8M0, encode(cabi.DT_E8M0, ws), 32)
     zs = np.zeros((total, 1))
     if src_zp is not None:
         zs = rng.integers(-3, 4, size=(total, kgroups(src_zp))).astype(np.float64)

@@ -117,6 +117,37 @@ def test_exact_data_matches_the_oracle(gpu, oracle, tile_shape, shape, tname, sd
                 assert np.array_equal(gc.logical_dst(p, got), want)
 
 
+MX_SHAPES = [
+    ([8, 8, 8, 8], 1024, 32),
+    ([10, 20, 30, 40], 1024, 36),
+    ([1, 2, 4, 8, 16], 2048, 132),
+    ([0, 1, 2, 0, 3, 0], 1024, 20),
+    ([70, 3, 129], 1024, 40),
+]
+MX_TYPES = [("mxfp8 e4m3", E4M3, E4M3), ("mxfp8 e5m2 x e4m3", E5M2, E4M3), ("mxfp4", cabi.DT_F4_E2M1, cabi.DT_F4_E2M1)]
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("shape", MX_SHAPES, ids=lambda s: f"G{len(s[0])}x{sum(s[0])}x{s[1]}x{s[2]}")
+@pytest.mark.parametrize("tname,sdt,wdt", MX_TYPES, ids=[t[0] for t in MX_TYPES])
+def test_mx_scaled_exact_data_matches_the_oracle(gpu, oracle, tile_shape, shape, tname, sdt, wdt):
+    """e8m0 scales per 32 k on both operands, applied by the scaled matrix instruction: the layout of the reference's
+    GPU tests (--attr-scales=src:3:e8m0:1x32+wei:7:e8m0:32x1).  Integers times powers of two: every order is exact."""
+    from onednn_amd import grouped
+    sizes, K, N = shape
+    for label, kw in (("plain", {}), ("bias + relu", dict(bias=True, post_ops=("relu",))),
+                      ("per-row factor", dict(post_ops=("mul_row",)))):
+        for dst_dt in (F32, BF16):
+            p, want = gc.case_2dx3d(sizes, K, N, src_dt=sdt, wei_dt=wdt, dst_dt=dst_dt, wtag="acb", mx=True, **kw)
+            assert impl_of(p) == "hip:mfma_grouped"
+            st, ref = oracle.run_oracle_grouped(p)
+            assert st == cabi.SUCCESS
+            got = grouped.run_gpu(p)
+            assert np.array_equal(got, ref), f"{p.name} {tname} {label} dst {dst_dt} ({tile_shape})"
+            if dst_dt == F32:
+                assert np.array_equal(gc.logical_dst(p, got), want)
+
+
 def random_case(rng, sizes, K, N, dt, scales=True, dst_dt=F32, active=None):
     """Random operands (fp8: random finite bytes with exponents in a band of 2^8;
     16-bit types: normal), weights [G][N][K].  Returns (problem, S, W, ss, ws) with
