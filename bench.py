@@ -300,6 +300,11 @@ def run_grouped_workloads(lib, steps, which=("g1", "g2", "g3", "g4", "g5")):
             cabi.check(lib.mi355_grouped_matmul_launch(C.byref(d), C.byref(sets[idx[0] % copies]), None))
             idx[0] += 1
 
+        t_pre = time.time()
+        while time.time() - t_pre < 0.4:     # settle the clocks (untimed), as for the other workloads
+            for _ in range(20):
+                step()
+            cabi.check(lib.mi355_stream_sync(None))
         for _ in range(3):
             step()
         ms = timer.time_ms(step, steps)
@@ -405,6 +410,10 @@ def main():
     ap.add_argument("--calib-read", action="store_true",
                     help="time a read-only kernel with the decode kernel's access shape over the C2 weights "
                          "(12 rotating copies, nothing cached) and exit: the floor of the weight stream")
+    ap.add_argument("--calib-pattern", action="store_true",
+                    help="time a read-only kernel that streams 256-row slabs the way the grouped matmul tiles do, with "
+                         "64, 128, 256 and 1024 contiguous bytes per row and load instruction, over G1's weights "
+                         "(3.76 GB) and exit: what the access shape costs by itself")
     ap.add_argument("--calib-mfma", action="store_true",
                     help="time the MFMA instructions of the GEMM kernels by themselves (registers only), with random "
                          "and with constant operand bits, and exit: the ceiling the power manager leaves")
@@ -432,6 +441,22 @@ def main():
         f"HBM={hbm.value / 2**30:.0f} GiB")
 
     main_name = args.workload
+    if args.calib_pattern:
+        K, slabs = 7168, 2048
+        buf, sink = cabi.DeviceBuffer(K * 256 * slabs), cabi.DeviceBuffer(4096)
+        cabi.check(lib.mi355_mem_set(buf.ptr, 1, C.c_size_t(K * 256 * slabs), None))
+        timer, rows = Timer(lib), []
+        for run in (64, 128, 256, 1024):
+            def step():
+                cabi.check(lib.mi355_read_pattern_kernel(buf.ptr, slabs, K, run, sink.ptr, None))
+            timer.time_ms(step, 20)
+            ms = min(timer.time_ms(step, 10) for _ in range(3))
+            gbs = K * 256 * slabs / (ms * 1e-3) / 1e9
+            rows.append({"run_bytes": run, "rows_per_instruction": 1024 // run, "ms": ms, "GBps": gbs})
+            log(f"[bench] {1024 // run:2d} rows x {run:4d} B per load instruction: {ms:.4f} ms -> {gbs:.0f} GB/s")
+        print(json.dumps({"metric": "row streaming by access shape", "unit": "GB/s", "bytes": K * 256 * slabs,
+                          "rows": rows}), flush=True)
+        return
     if args.calib_read:
         nbytes = 4096 * 14336 // 2
         bufs = [cabi.DeviceBuffer(nbytes) for _ in range(12)]

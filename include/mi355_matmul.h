@@ -487,6 +487,12 @@ int mi355_copy_kernel(void *dst, const void *src, size_t bytes, void *stream);
  * itself.  `sink` holds 4 bytes per 128 KiB and is not written in practice. */
 int mi355_read_stream_kernel(const void *src, size_t bytes, void *sink, void *stream);
 
+/* Access-shape probe for kernels that stream rows (the grouped matmul tiles): `slabs` workgroups of four
+ * wavefronts each read a slab of 256 rows x K bytes (K a multiple of 1024) of `src` once, K-major, a load
+ * instruction fetching 1024 / run rows x `run` contiguous bytes (run = 64, 128, 256 or 1024).  `sink`: 1 KiB,
+ * not written in practice. */
+int mi355_read_pattern_kernel(const void *src, int64_t slabs, int64_t K, int run, void *sink, void *stream);
+
 /* Measures what an MFMA instruction of the GEMM kernels sustains by itself:
  * 1024 workgroups x 4 wavefronts, operands and accumulators in registers, 8 or
  * 16 independent accumulator chains, `iters` rounds.  instr: 0 i32_32x32x32_i8,

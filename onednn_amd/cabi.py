@@ -150,7 +150,7 @@ KERNEL_SYMBOLS = [
     "mi355_stream_wait_event", "mi355_mem_store_scalar",
     "mi355_last_error", "mi355_matmul_query", "mi355_matmul_impl_name",
     "mi355_matmul_scratch_bytes", "mi355_matmul_launch", "mi355_matmul_launch_noalloc", "mi355_reorder_query",
-    "mi355_reorder_launch", "mi355_wei_pack_reorder_dims", "mi355_copy_kernel", "mi355_flush_kernel", "mi355_read_stream_kernel", "mi355_mfma_rate_kernel", "mi355_grouped_matmul_query",
+    "mi355_reorder_launch", "mi355_wei_pack_reorder_dims", "mi355_copy_kernel", "mi355_flush_kernel", "mi355_read_stream_kernel", "mi355_read_pattern_kernel", "mi355_mfma_rate_kernel", "mi355_grouped_matmul_query",
     "mi355_grouped_matmul_launch", "mi355_grouped_matmul_impl",
 ]
 
@@ -215,6 +215,7 @@ def load_kernels():
     lib.mi355_grouped_matmul_impl.argtypes = [C.POINTER(GroupedDesc)]
     lib.mi355_grouped_matmul_impl.restype = C.c_char_p
     lib.mi355_read_stream_kernel.argtypes = [vp, C.c_size_t, vp, vp]
+    lib.mi355_read_pattern_kernel.argtypes = [vp, C.c_int64, C.c_int64, C.c_int, vp, vp]
     lib.mi355_mfma_rate_kernel.argtypes = [C.c_int, C.c_int, vp, vp, C.POINTER(C.c_double), vp]
     lib.mi355_flush_kernel.argtypes = [vp, C.c_size_t, vp]
     _lib = lib

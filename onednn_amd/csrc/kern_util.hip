@@ -135,6 +135,47 @@ __global__ void __launch_bounds__(1024) read_stream_kernel(const uint8_t *src, u
 }
 } // namespace mi355
 
+namespace mi355 {
+// Access-shape probe for the row-streaming kernels (the grouped matmul tiles): a workgroup of four wavefronts
+// streams a slab of 256 rows x K bytes, every wavefront 64 rows, K-major; one load instruction fetches
+// 1024 / RUN rows x RUN contiguous bytes (RUN = 128: the whole lines of 8 rows, the shape of the tiles; RUN = 64:
+// half lines of 16 rows, the shape a matrix-instruction operand suggests; RUN = 1024: one row's contiguous KB).
+// Every byte is read once, non-temporally, and nothing is kept.
+template <int RUN>
+__global__ void __launch_bounds__(256) read_pattern_kernel(const uint8_t *src, long K, unsigned *sink) {
+    typedef unsigned v4u __attribute__((ext_vector_type(4)));
+    constexpr int LPR = RUN / 16, RPI = 64 / LPR; // lanes per row, rows per instruction
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const uint8_t *slab = src + ((long)blockIdx.x * 256 + wave * 64) * K;
+    const int r = lane / LPR, c = lane % LPR;
+    v4u acc = {0, 0, 0, 0};
+    for (long k = 0; k < K; k += RUN) {
+#pragma unroll
+        for (int i = 0; i < 64 / RPI; ++i)
+            acc ^= __builtin_nontemporal_load((const v4u *)(slab + (long)(i * RPI + r) * K + k + c * 16));
+    }
+    if ((acc[0] ^ acc[1] ^ acc[2] ^ acc[3]) == 0x9e3779b9u) sink[threadIdx.x] = acc[0];
+}
+} // namespace mi355
+
+extern "C" int mi355_read_pattern_kernel(const void *src, int64_t slabs, int64_t K, int run, void *sink, void *stream) {
+    if (slabs < 0 || K <= 0 || K % 1024 || ((uintptr_t)src & 15) || !sink) {
+        set_error("read pattern kernel needs a 16-byte aligned pointer, K a multiple of 1024 and a sink of 1 KiB");
+        return MI355_INVALID_ARGUMENTS;
+    }
+    if (slabs == 0) return MI355_SUCCESS;
+    const dim3 grid((unsigned)slabs), block(256);
+    hipStream_t s = (hipStream_t)stream;
+    switch (run) {
+        case 64: hipLaunchKernelGGL(read_pattern_kernel<64>, grid, block, 0, s, (const uint8_t *)src, (long)K, (unsigned *)sink); break;
+        case 128: hipLaunchKernelGGL(read_pattern_kernel<128>, grid, block, 0, s, (const uint8_t *)src, (long)K, (unsigned *)sink); break;
+        case 256: hipLaunchKernelGGL(read_pattern_kernel<256>, grid, block, 0, s, (const uint8_t *)src, (long)K, (unsigned *)sink); break;
+        case 1024: hipLaunchKernelGGL(read_pattern_kernel<1024>, grid, block, 0, s, (const uint8_t *)src, (long)K, (unsigned *)sink); break;
+        default: set_error("read pattern kernel: run must be 64, 128, 256 or 1024 bytes"); return MI355_INVALID_ARGUMENTS;
+    }
+    return hipGetLastError() == hipSuccess ? MI355_SUCCESS : MI355_RUNTIME_ERROR;
+}
+
 extern "C" int mi355_read_stream_kernel(const void *src, size_t bytes, void *sink, void *stream) {
     if (bytes % (128 << 10) || ((uintptr_t)src & 15) || !sink) {
         set_error("read stream kernel needs a 16-byte aligned pointer, a multiple of 128 KiB and a sink of 4 bytes per 128 KiB");
