@@ -113,7 +113,8 @@ typedef enum {
     dnnl_format_kind_host_scalar /* one value that lives in the memory object itself, on the host */
 } dnnl_format_kind_t;
 
-/* dnnl_types.h:175-209: only the plain tags with at most four dimensions */
+/* dnnl_types.h:175-260: the plain tags of the matmul and inner-product tensors, and the activation / weights
+ * names the reference gives them (dnnl_types.h:1096-1155) */
 typedef enum {
     dnnl_format_tag_undef = 0,
     dnnl_format_tag_any = 1,
@@ -121,9 +122,30 @@ typedef enum {
     dnnl_ab = 3,
     dnnl_abc = 4,
     dnnl_abcd = 5,
+    dnnl_abcde = 6,
     dnnl_ba = 14,
     dnnl_acb = 15,
-    dnnl_abdc = 20
+    dnnl_abdc = 20,
+    dnnl_acdb = 22,
+    dnnl_acdeb = 33,
+    dnnl_x = dnnl_a,
+    dnnl_nc = dnnl_ab,
+    dnnl_tn = dnnl_ab,
+    dnnl_nt = dnnl_ba,
+    dnnl_ncw = dnnl_abc,
+    dnnl_nwc = dnnl_acb,
+    dnnl_nchw = dnnl_abcd,
+    dnnl_nhwc = dnnl_acdb,
+    dnnl_ncdhw = dnnl_abcde,
+    dnnl_ndhwc = dnnl_acdeb,
+    dnnl_oi = dnnl_ab,
+    dnnl_io = dnnl_ba,
+    dnnl_oiw = dnnl_abc,
+    dnnl_owi = dnnl_acb,
+    dnnl_oihw = dnnl_abcd,
+    dnnl_ohwi = dnnl_acdb,
+    dnnl_oidhw = dnnl_abcde,
+    dnnl_odhwi = dnnl_acdeb
 } dnnl_format_tag_t;
 
 /* dnnl_types.h:2057-2101 */
@@ -132,10 +154,23 @@ typedef enum {
     dnnl_reorder = 1,
     dnnl_sum = 4,
     dnnl_eltwise = 7,
+    dnnl_inner_product = 10,
     dnnl_binary = 13,
     dnnl_matmul = 14,
     dnnl_prelu = 18
 } dnnl_primitive_kind_t;
+
+/* dnnl_types.h:2029-2049 */
+typedef enum {
+    dnnl_prop_kind_undef = 0,
+    dnnl_forward_training = 64,
+    dnnl_forward_inference = 96,
+    dnnl_forward = dnnl_forward_training,
+    dnnl_backward = 128,
+    dnnl_backward_data = 160,
+    dnnl_backward_weights = 192,
+    dnnl_backward_bias = 193
+} dnnl_prop_kind_t;
 
 /* dnnl_types.h:2110-2230: the eltwise and binary algorithms post-ops admit */
 typedef enum {
@@ -410,6 +445,30 @@ dnnl_status_t dnnl_matmul_primitive_desc_create(dnnl_primitive_desc_t *primitive
         const_dnnl_memory_desc_t src_desc, const_dnnl_memory_desc_t weights_desc,
         const_dnnl_memory_desc_t bias_desc, const_dnnl_memory_desc_t dst_desc,
         const_dnnl_primitive_attr_t attr);
+
+/* ---- inner product primitive descriptor: dnnl.h:2757-2762 (src/common/inner_product.cpp:188-203).
+ * src [mb, ic, spatial...] (2 to 5 dims), weights [oc, ic, spatial...], bias [oc], dst [mb, oc]:
+ * dst = src flattened to [mb, K] times weights flattened to [oc, K], transposed -- so plain weights are
+ * K-contiguous, the layout the matrix-core kernels read at full rate, and the primitive runs on the matmul
+ * kernel families (int8 with scales: src mask 0, weights mask 0 or 1, dst mask 0; f32 / bf16 / f16 / fp8
+ * without scales; sum, eltwise, binary and prelu post-ops).  src and weights must keep their reduced dims
+ * dense and in the same order in memory (nchw with oihw, nhwc with ohwi, ...): `format_tag::any` on either
+ * one resolves to the other's order.  Execute arguments: DNNL_ARG_SRC, DNNL_ARG_WEIGHTS, DNNL_ARG_BIAS,
+ * DNNL_ARG_DST and the attribute arguments of a matmul. */
+dnnl_status_t dnnl_inner_product_forward_primitive_desc_create(dnnl_primitive_desc_t *primitive_desc,
+        dnnl_engine_t engine, dnnl_prop_kind_t prop_kind, const_dnnl_memory_desc_t src_desc,
+        const_dnnl_memory_desc_t weights_desc, const_dnnl_memory_desc_t bias_desc,
+        const_dnnl_memory_desc_t dst_desc, const_dnnl_primitive_attr_t attr);
+/* dnnl.h:2781-2787, :2809-2817: the descriptors are validated as in src/common/inner_product.cpp:205-230; no
+ * implementation is offered for backward propagation (dnnl_unimplemented) */
+dnnl_status_t dnnl_inner_product_backward_data_primitive_desc_create(dnnl_primitive_desc_t *primitive_desc,
+        dnnl_engine_t engine, const_dnnl_memory_desc_t diff_src_desc, const_dnnl_memory_desc_t weights_desc,
+        const_dnnl_memory_desc_t diff_dst_desc, const_dnnl_primitive_desc_t hint_fwd_pd,
+        const_dnnl_primitive_attr_t attr);
+dnnl_status_t dnnl_inner_product_backward_weights_primitive_desc_create(dnnl_primitive_desc_t *primitive_desc,
+        dnnl_engine_t engine, const_dnnl_memory_desc_t src_desc, const_dnnl_memory_desc_t diff_weights_desc,
+        const_dnnl_memory_desc_t diff_bias_desc, const_dnnl_memory_desc_t diff_dst_desc,
+        const_dnnl_primitive_desc_t hint_fwd_pd, const_dnnl_primitive_attr_t attr);
 
 /* ---- reorder primitive descriptor: dnnl.h:1727-1731.  Execute arguments are
  * DNNL_ARG_FROM / DNNL_ARG_TO (dnnl_types.h:2553,2580) plus the scales and zero

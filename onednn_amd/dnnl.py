@@ -22,7 +22,13 @@ dims_t = C.c_int64 * MAX_NDIMS
 success, out_of_memory, invalid_arguments, unimplemented, last_impl_reached, runtime_error = range(6)
 cpu, gpu = 1, 2
 tag_any, tag_a, tag_ab, tag_abc, tag_abcd, tag_ba, tag_acb, tag_abdc = 1, 2, 3, 4, 5, 14, 15, 20
+tag_abcde, tag_acdb, tag_acdeb = 6, 22, 33
+tag_x, tag_nc, tag_ncw, tag_nwc, tag_nchw, tag_nhwc, tag_ncdhw, tag_ndhwc = 2, 3, 4, 15, 5, 22, 6, 33
+tag_oi, tag_io, tag_oiw, tag_owi, tag_oihw, tag_ohwi, tag_oidhw, tag_odhwi = 3, 14, 4, 15, 5, 22, 6, 33
 kind_sum, kind_eltwise, kind_binary, kind_matmul, kind_prelu = 4, 7, 13, 14, 18
+kind_inner_product = 10
+forward_training, forward_inference, backward_data, backward_weights = 64, 96, 160, 192
+query_primitive_kind, query_prop_kind = 2, 11
 query_impl_info_str, query_src_md, query_weights_md, query_dst_md, query_scratchpad_md = 8, 129, 131, 133, 136
 query_ndims_s32, query_dims, query_data_type, query_strides, query_memory_consumption = 256, 257, 258, 14, 6
 query_format_kind = 262
@@ -391,6 +397,22 @@ class matmul_primitive_desc:
         return d
 
 
+class inner_product_forward_primitive_desc(matmul_primitive_desc):
+    """dnnl::inner_product_forward::primitive_desc(engine, prop_kind, src_md, weights_md, bias_md, dst_md, attr)"""
+
+    def __init__(self, eng, prop_kind, src_md, weights_md, dst_md, bias_md=None, attr=None):
+        self.engine = eng
+        self.h = C.c_void_p()
+        _check(lib().dnnl_inner_product_forward_primitive_desc_create(
+            C.byref(self.h), eng.h, prop_kind, src_md.h, weights_md.h, bias_md.h if bias_md else None, dst_md.h,
+            attr.h if attr else None), "inner_product_forward_primitive_desc_create")
+
+    def query_s32(self, what):
+        v = C.c_int(0)
+        _check(lib().dnnl_primitive_desc_query(self.h, what, 0, C.byref(v)), "pd_query")
+        return v.value
+
+
 class reorder_primitive_desc(matmul_primitive_desc):
     """dnnl::reorder::primitive_desc(src_engine, src_md, dst_engine, dst_md, attr)"""
 
@@ -414,6 +436,10 @@ class matmul:
             arr[i].arg = k
             arr[i].memory = m.h
         _check(lib().dnnl_primitive_execute(self.h, strm.h, len(args), arr), "primitive_execute")
+
+
+class inner_product_forward(matmul):
+    """dnnl::inner_product_forward(pd); execute(stream, {ARG_SRC, ARG_WEIGHTS, ARG_BIAS, ARG_DST, ...})"""
 
 
 class reorder(matmul):

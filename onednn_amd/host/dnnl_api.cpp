@@ -18,6 +18,7 @@
 #include <stdlib.h>
 #include <string.h>
 
+#include <algorithm>
 #include <atomic>
 #include <chrono>
 #include <map>
@@ -233,6 +234,12 @@ struct dnnl_primitive_desc {
     dnnl_primitive_attr attr;
     mi355_matmul_desc_t desc;     // impl field = the chosen kernel family
     bool grouped = false;         // grouped (mixture-of-experts) matmul: `gdesc` instead of `desc`
+    // inner product: lowered and executed as the matmul [mb, K] x [K, oc] (src, wei, bias, dst and attr above
+    // describe that matmul); these are the tensors and the attributes the caller gave and reads back
+    bool inner_product = false;
+    int prop_kind = 96;           // dnnl_forward_inference
+    dnnl_memory_desc ip_src, ip_wei, ip_bias;
+    dnnl_primitive_attr ip_attr;
     mi355_grouped_desc_t gdesc;
     std::vector<int> impls;       // kernel families that can run it, best first
     size_t impl_pos = 0;
@@ -987,9 +994,12 @@ DNNL_EXPORT dnnl_status_t dnnl_memory_desc_create_with_tag(dnnl_memory_desc_t *m
         case dnnl_ab: CHECK_ARG(ndims == 2); break;
         case dnnl_abc: CHECK_ARG(ndims == 3); break;
         case dnnl_abcd: CHECK_ARG(ndims == 4); break;
+        case dnnl_abcde: CHECK_ARG(ndims == 5); break;
         case dnnl_ba: CHECK_ARG(ndims == 2); perm[0] = 1; perm[1] = 0; break;
         case dnnl_acb: CHECK_ARG(ndims == 3); perm[1] = 2; perm[2] = 1; break;
         case dnnl_abdc: CHECK_ARG(ndims == 4); perm[2] = 3; perm[3] = 2; break;
+        case dnnl_acdb: CHECK_ARG(ndims == 4); perm[1] = 2; perm[2] = 3; perm[3] = 1; break;
+        case dnnl_acdeb: CHECK_ARG(ndims == 5); perm[1] = 2; perm[2] = 3; perm[3] = 4; perm[4] = 1; break;
         default: return dnnl_unimplemented; // blocked layouts are not offered
     }
     md->set_dense(perm);
@@ -1875,6 +1885,182 @@ DNNL_EXPORT dnnl_status_t dnnl_matmul_primitive_desc_create(dnnl_primitive_desc_
     return dnnl_success;
 }
 
+// ---- inner product primitive descriptor
+namespace {
+// memory order of the dims of a plain tensor, outermost first (ties keep the logical order)
+void memory_order(const dnnl_memory_desc &md, int *perm) {
+    for (int i = 0; i < md.ndims; ++i) perm[i] = i;
+    std::stable_sort(perm, perm + md.ndims, [&](int a, int b) { return md.strides[a] > md.strides[b]; });
+}
+// ip_desc_init, src/common/inner_product.cpp:43-112 (the checks that do not depend on the propagation kind)
+dnnl_status_t ip_check_shapes(const dnnl_memory_desc *src, const dnnl_memory_desc *wei, const dnnl_memory_desc *bias,
+        const dnnl_memory_desc *dst) {
+    CHECK_ARG(src && wei && dst);
+    for (const dnnl_memory_desc *m : {src, wei, bias, dst})
+        if (m) CHECK_ARG(m->kind != dnnl_format_kind_host_scalar);
+    for (const dnnl_memory_desc *m : {src, wei, bias, dst})
+        if (m) CHECK_UNIMPL(!m->has_runtime());
+    CHECK_ARG(accum_dt(src->dt, wei->dt, dst->dt) != dnnl_data_type_undef);
+    CHECK_ARG(wei->nelems() != 0);
+    CHECK_ARG(src->ndims >= 2 && src->ndims <= 5);
+    CHECK_ARG(dst->ndims == 2);
+    CHECK_ARG(wei->ndims == src->ndims);
+    if (bias) CHECK_ARG(bias->ndims == 1 && bias->dims[0] == dst->dims[1]);
+    CHECK_ARG(src->dims[0] == dst->dims[0]);
+    for (int i = 1; i < src->ndims; ++i) CHECK_ARG(src->dims[i] == wei->dims[i]);
+    CHECK_ARG(dst->dims[1] == wei->dims[0]);
+    return dnnl_success;
+}
+} // namespace
+
+DNNL_EXPORT dnnl_status_t dnnl_inner_product_forward_primitive_desc_create(dnnl_primitive_desc_t *primitive_desc,
+        dnnl_engine_t engine, dnnl_prop_kind_t prop_kind, const_dnnl_memory_desc_t src_desc,
+        const_dnnl_memory_desc_t weights_desc, const_dnnl_memory_desc_t bias_desc, const_dnnl_memory_desc_t dst_desc,
+        const_dnnl_primitive_attr_t attr) {
+    CHECK_ARG(primitive_desc && engine);
+    CHECK_ARG(prop_kind == dnnl_forward_training || prop_kind == dnnl_forward_inference);
+    const dnnl_memory_desc *bias_in
+            = (bias_desc && !bias_desc->is_zero() && bias_desc->kind != dnnl_format_kind_undef) ? bias_desc : nullptr;
+    dnnl_status_t st = ip_check_shapes(src_desc, weights_desc, bias_in, dst_desc);
+    if (st) return st;
+    dnnl_memory_desc src = *src_desc, wei = *weights_desc, dst = *dst_desc, bias;
+    if (bias_in) bias = *bias_in;
+    const int nd = src.ndims;
+    for (const dnnl_memory_desc *m : {&src, &wei, &dst})
+        CHECK_UNIMPL(m->kind == dnnl_blocked || m->kind == dnnl_format_kind_any);
+    CHECK_UNIMPL(!src.grouped && !wei.grouped && !dst.grouped);
+
+    // ip_attr_check, src/common/inner_product.cpp:114-186; the data types are those of the two naive
+    // implementations (ref_inner_product.hpp:52-72, ref_inner_product_int8.hpp:52-66)
+    const bool int8 = is_int8(src.dt);
+    if (int8) {
+        CHECK_UNIMPL(wei.dt == dnnl_s8);
+        CHECK_UNIMPL(dst.dt == dnnl_f32 || dst.dt == dnnl_f16 || dst.dt == dnnl_bf16 || dst.dt == dnnl_s32
+                || is_int8(dst.dt));
+        if (bias_in)
+            CHECK_UNIMPL(bias.dt == dnnl_f32 || bias.dt == dnnl_f16 || bias.dt == dnnl_bf16 || bias.dt == dnnl_s32
+                    || is_int8(bias.dt));
+    } else {
+        CHECK_UNIMPL(src.dt == dnnl_f32 || src.dt == dnnl_bf16 || src.dt == dnnl_f16 || is_fp8(src.dt));
+        CHECK_UNIMPL(wei.dt == src.dt);
+        CHECK_UNIMPL(dst.dt == dnnl_f32 || dst.dt == src.dt);
+        if (bias_in) CHECK_UNIMPL(bias.dt == dnnl_f32 || bias.dt == src.dt);
+    }
+    dnnl_primitive_attr lowered_attr;
+    if (attr) {
+        const dnnl_primitive_attr &a = *attr;
+        CHECK_UNIMPL(a.zero_points.empty() && a.reductions.empty() && !a.with_dropout() && a.rounding.empty());
+        const bool scales_allowed = int8 || is_int8(dst.dt) || dst.dt == dnnl_s32; // the gpu-engine rule, :133-137
+        CHECK_UNIMPL(IMPLICATION(!a.scales.empty(), scales_allowed));
+        for (const auto &kv : a.scales) {
+            const quant_entry_t &q = kv.second;
+            CHECK_UNIMPL(kv.first == DNNL_ARG_SRC || kv.first == DNNL_ARG_WEIGHTS || kv.first == DNNL_ARG_DST);
+            CHECK_UNIMPL(kv.first == DNNL_ARG_WEIGHTS ? (q.mask == 0 || q.mask == 1) : q.mask == 0);
+            CHECK_UNIMPL(q.group_ndims == 0 && q.dt == dnnl_f32 && !q.is_dynamic());
+            CHECK_UNIMPL(!q.on_host);
+            CHECK_UNIMPL(int8); // the implementations read scales on the integer path only
+        }
+        for (const post_op_entry_t &e : a.post_ops.entries)
+            CHECK_UNIMPL(e.kind == dnnl_binary || e.kind == dnnl_eltwise || e.kind == dnnl_prelu || e.kind == dnnl_sum);
+        lowered_attr = a;
+        auto it = lowered_attr.scales.find(DNNL_ARG_WEIGHTS);
+        if (it != lowered_attr.scales.end() && it->second.mask == 1) it->second.mask = 2; // oc is dim 1 of [K, oc]
+    }
+
+    // format `any` (cpu_inner_product_fwd_pd_t::set_default_params, src/cpu/cpu_inner_product_pd.hpp:162-209):
+    // src and weights share one order of dims; the mb / oc dim never ends up innermost
+    int perm[DNNL_MAX_NDIMS];
+    auto outer_first = [&](int *pm) {
+        if (nd > 1 && pm[nd - 1] == 0) {
+            for (int i = nd - 1; i > 0; --i) pm[i] = pm[i - 1];
+            pm[0] = 0;
+        }
+    };
+    if (src.kind == dnnl_format_kind_any) {
+        if (wei.kind == dnnl_format_kind_any) {
+            src.set_dense();
+        } else {
+            memory_order(wei, perm);
+            outer_first(perm);
+            src.set_dense(perm);
+        }
+    }
+    if (wei.kind == dnnl_format_kind_any) {
+        memory_order(src, perm);
+        outer_first(perm);
+        wei.set_dense(perm);
+    }
+    if (dst.kind == dnnl_format_kind_any) dst.set_dense();
+    if (bias_in && bias.kind == dnnl_format_kind_any) bias.set_dense();
+    if (bias_in) CHECK_UNIMPL(bias.kind == dnnl_blocked);
+
+    // The reduced dims (ic and the spatial ones) as one K: they must be dense, and in the same order, in both
+    // tensors.  Dims of extent one do not matter.
+    int order[DNNL_MAX_NDIMS], n_inner = 0;
+    memory_order(src, perm);
+    for (int i = 0; i < nd; ++i)
+        if (perm[i] != 0 && src.dims[perm[i]] != 1) order[n_inner++] = perm[i];
+    dim_t K = 1, src_ks = 1, wei_ks = 1;
+    for (int i = 1; i < nd; ++i) K *= src.dims[i];
+    if (n_inner > 0 && K > 0) {
+        src_ks = src.strides[order[n_inner - 1]];
+        wei_ks = wei.strides[order[n_inner - 1]];
+        for (int i = 0; i + 1 < n_inner; ++i) {
+            const dim_t inner = src.dims[order[i + 1]];
+            CHECK_UNIMPL(src.strides[order[i]] == src.strides[order[i + 1]] * inner);
+            CHECK_UNIMPL(wei.strides[order[i]] == wei.strides[order[i + 1]] * inner);
+        }
+    }
+    dnnl_memory_desc src2, wei2, bias2;
+    src2.ndims = 2; src2.dt = src.dt; src2.kind = dnnl_blocked;
+    src2.dims[0] = src.dims[0]; src2.dims[1] = K;
+    src2.strides[0] = src.strides[0]; src2.strides[1] = src_ks;
+    wei2.ndims = 2; wei2.dt = wei.dt; wei2.kind = dnnl_blocked;
+    wei2.dims[0] = K; wei2.dims[1] = wei.dims[0];
+    wei2.strides[0] = wei_ks; wei2.strides[1] = wei.strides[0];
+    if (bias_in) {
+        bias2.ndims = 2; bias2.dt = bias.dt; bias2.kind = dnnl_blocked;
+        bias2.dims[0] = 1; bias2.dims[1] = bias.dims[0];
+        bias2.strides[1] = bias.strides[0]; bias2.strides[0] = bias.strides[0] * (bias.dims[0] ? bias.dims[0] : 1);
+    }
+    dnnl_primitive_desc_t mm = nullptr;
+    st = dnnl_matmul_primitive_desc_create(&mm, engine, &src2, &wei2, bias_in ? &bias2 : nullptr, &dst, &lowered_attr);
+    if (st) return st;
+    mm->inner_product = true;
+    mm->prop_kind = (int)prop_kind;
+    mm->ip_src = src; mm->ip_wei = wei;
+    if (bias_in) mm->ip_bias = bias;
+    if (attr) mm->ip_attr = *attr;
+    if (verbose_level() >= 1)
+        fprintf(stderr, "onednn_verbose,v1,primitive,create:dispatch,gpu,inner_product,%s\n", mm->impl_name.c_str());
+    *primitive_desc = mm;
+    return dnnl_success;
+}
+
+// src/common/inner_product.cpp:205-230: validated, then no implementation in the list
+DNNL_EXPORT dnnl_status_t dnnl_inner_product_backward_data_primitive_desc_create(dnnl_primitive_desc_t *primitive_desc,
+        dnnl_engine_t engine, const_dnnl_memory_desc_t diff_src_desc, const_dnnl_memory_desc_t weights_desc,
+        const_dnnl_memory_desc_t diff_dst_desc, const_dnnl_primitive_desc_t hint_fwd_pd,
+        const_dnnl_primitive_attr_t attr) {
+    (void)hint_fwd_pd; (void)attr;
+    CHECK_ARG(primitive_desc && engine);
+    dnnl_status_t st = ip_check_shapes(diff_src_desc, weights_desc, nullptr, diff_dst_desc);
+    if (st) return st;
+    return dnnl_unimplemented;
+}
+DNNL_EXPORT dnnl_status_t dnnl_inner_product_backward_weights_primitive_desc_create(
+        dnnl_primitive_desc_t *primitive_desc, dnnl_engine_t engine, const_dnnl_memory_desc_t src_desc,
+        const_dnnl_memory_desc_t diff_weights_desc, const_dnnl_memory_desc_t diff_bias_desc,
+        const_dnnl_memory_desc_t diff_dst_desc, const_dnnl_primitive_desc_t hint_fwd_pd,
+        const_dnnl_primitive_attr_t attr) {
+    (void)hint_fwd_pd; (void)attr;
+    CHECK_ARG(primitive_desc && engine);
+    const dnnl_memory_desc *b = (diff_bias_desc && !diff_bias_desc->is_zero()) ? diff_bias_desc : nullptr;
+    dnnl_status_t st = ip_check_shapes(src_desc, diff_weights_desc, b, diff_dst_desc);
+    if (st) return st;
+    return dnnl_unimplemented;
+}
+
 // ---- reorder primitive descriptor (src/common/reorder.cpp:67-170)
 DNNL_EXPORT dnnl_status_t dnnl_reorder_primitive_desc_create(dnnl_primitive_desc_t *reorder_primitive_desc,
         const_dnnl_memory_desc_t src_desc, dnnl_engine_t src_engine, const_dnnl_memory_desc_t dst_desc,
@@ -1983,7 +2169,7 @@ DNNL_EXPORT dnnl_status_t dnnl_primitive_desc_next_impl(dnnl_primitive_desc_t pd
 }
 DNNL_EXPORT dnnl_status_t dnnl_primitive_desc_get_attr(const_dnnl_primitive_desc_t pd, const_dnnl_primitive_attr_t *attr) {
     CHECK_ARG(pd && attr);
-    *attr = &pd->attr;
+    *attr = pd->inner_product ? &pd->ip_attr : &pd->attr;
     return dnnl_success;
 }
 DNNL_EXPORT dnnl_status_t dnnl_amd_primitive_desc_get_lowered(const_dnnl_primitive_desc_t pd, void *out) {
@@ -2010,6 +2196,19 @@ DNNL_EXPORT const_dnnl_memory_desc_t dnnl_primitive_desc_query_md(const_dnnl_pri
             default: return nullptr;
         }
     }
+    if (pd->inner_product) { // the tensors as the caller describes them; dst is two-dimensional either way
+        switch (what) {
+            case dnnl_query_src_md: return index == 0 ? &pd->ip_src : nullptr;
+            case dnnl_query_weights_md:
+                return index == 0 ? &pd->ip_wei : index == 1 ? (pd->with_bias ? &pd->ip_bias : &zero_md) : nullptr;
+            case dnnl_query_exec_arg_md:
+                if (index == DNNL_ARG_SRC) return &pd->ip_src;
+                if (index == DNNL_ARG_WEIGHTS) return &pd->ip_wei;
+                if (index == DNNL_ARG_BIAS) return pd->with_bias ? &pd->ip_bias : &zero_md;
+                break;
+            default: break;
+        }
+    }
     switch (what) {
         case dnnl_query_src_md: return index == 0 ? &pd->src : nullptr;
         case dnnl_query_weights_md: return index == 0 ? &pd->wei : index == 1 ? (pd->with_bias ? &pd->bias : &zero_md) : nullptr;
@@ -2032,7 +2231,9 @@ DNNL_EXPORT dnnl_status_t dnnl_primitive_desc_query(const_dnnl_primitive_desc_t 
     CHECK_ARG(pd && result);
     switch (what) {
         case dnnl_query_engine: *(dnnl_engine_t *)result = pd->engine; break;
-        case dnnl_query_primitive_kind: *(dnnl_primitive_kind_t *)result = pd->kind; break;
+        case dnnl_query_primitive_kind:
+            *(dnnl_primitive_kind_t *)result = pd->inner_product ? dnnl_inner_product : pd->kind;
+            break;
         case dnnl_query_num_of_inputs_s32:
             *(int32_t *)result = pd->kind == dnnl_reorder ? 1 : 2 + (pd->with_bias ? 1 : 0);
             break;
@@ -2041,7 +2242,7 @@ DNNL_EXPORT dnnl_status_t dnnl_primitive_desc_query(const_dnnl_primitive_desc_t 
             *(int64_t *)result = pd->attr.scratchpad_mode == dnnl_scratchpad_mode_library ? (int64_t)pd->scratch_bytes : 0;
             break;
         case dnnl_query_impl_info_str: *(const char **)result = pd->impl_name.c_str(); break;
-        case dnnl_query_prop_kind: *(int *)result = 96; break; // dnnl_forward_inference
+        case dnnl_query_prop_kind: *(int *)result = pd->prop_kind; break;
         case dnnl_query_src_md:
         case dnnl_query_weights_md:
         case dnnl_query_dst_md:
@@ -2351,8 +2552,8 @@ DNNL_EXPORT dnnl_status_t dnnl_primitive_execute(const_dnnl_primitive_t cprimiti
     if (verbose_level() >= 2) {
         mi355_stream_sync(stream->hip_stream);
         const double ms = std::chrono::duration<double, std::milli>(std::chrono::steady_clock::now() - t0).count();
-        fprintf(stderr, "onednn_verbose,v1,primitive,exec,gpu,matmul,%s,undef,src:%s wei:%s dst:%s,,%ldx%ldx%ld:%ldx%ldx%ld,%g\n",
-                pd.impl_name.c_str(), dt_name(pd.src.dt), dt_name(pd.wei.dt), dt_name(pd.dst.dt), (long)pd.desc.batch,
+        fprintf(stderr, "onednn_verbose,v1,primitive,exec,gpu,%s,%s,undef,src:%s wei:%s dst:%s,,%ldx%ldx%ld:%ldx%ldx%ld,%g\n",
+                pd.inner_product ? "inner_product" : "matmul", pd.impl_name.c_str(), dt_name(pd.src.dt), dt_name(pd.wei.dt), dt_name(pd.dst.dt), (long)pd.desc.batch,
                 (long)pd.desc.M, (long)pd.desc.K, (long)pd.desc.batch, (long)pd.desc.K, (long)pd.desc.N, ms);
     }
     return from_mi355(rc);

@@ -87,6 +87,32 @@ def run_oracle(prob: MatmulProblem, flags=0, want_ideal=False):
     return dst
 
 
+def run_oracle_inner_product(prob: MatmulProblem, src, wei):
+    """Inner product forward.  `src` / `wei` are numpy arrays (storage type of the
+    data type) of the logical shapes [mb, ic, spatial...] / [oc, ic, spatial...]:
+    views in any memory order with non-negative strides.  `prob` is the matmul
+    [mb, K] x [K, oc] that carries the data types and everything after the sum
+    (bias, scales, post-ops, dst); its own src / wei arrays are not read.
+    Returns raw dst storage."""
+    lib = load()
+    lib.oracle_inner_product_fwd.argtypes = [C.c_int, C.c_void_p, C.c_int64, C.c_void_p, C.c_void_p,
+                                             C.POINTER(cabi.MatmulDesc), C.POINTER(cabi.MatmulArgs)]
+    assert src.ndim == wei.ndim and 2 <= src.ndim <= 5 and src.shape[1:] == wei.shape[1:]
+    assert min(src.strides) >= 0 and min(wei.strides) >= 0
+    dst = prob.initial_dst()
+    desc = prob.desc()
+    args, keep = host_args(prob, dst)
+    args.src, args.wei = src.ctypes.data, wei.ctypes.data
+    dims = np.array(src.shape, np.int64)
+    ss = np.array([x // src.itemsize for x in src.strides], np.int64)
+    ws = np.array([x // wei.itemsize for x in wei.strides], np.int64)
+    st = lib.oracle_inner_product_fwd(src.ndim, dims.ctypes.data, wei.shape[0], ss.ctypes.data, ws.ctypes.data,
+                                      C.byref(desc), C.byref(args))
+    assert st == 0, f"oracle_inner_product_fwd status {st}"
+    del keep
+    return dst
+
+
 def run_oracle_dropout(prob: MatmulProblem):
     """(raw dst storage, the dropout mask or None)."""
     prob._oracle_mask = None

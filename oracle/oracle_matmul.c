@@ -27,6 +27,10 @@
  *                     ::execute src/cpu/reorder/simple_reorder.hpp:2579-2661 and
  *                     its 4-bit variants :2168-2288 (f32 -> s4/u4/f4) and
  *                     :2291-2425 (s4/u4/f4 -> f32/bf16/f16)
+ *   oracle_inner_product_fwd
+ *                     ref_inner_product_fwd_t::execute_forward src/cpu/ref_inner_product.cpp:33-100
+ *                     and ref_inner_product_int8_fwd_t::execute_forward
+ *                     src/cpu/ref_inner_product_int8.cpp:34-116
  *   orc_quant_off     quant_entry_t::get_md src/common/primitive_attr_quant.hpp:116-140
  *                     + matmul_helper_t::get_quant_off src/cpu/matmul/matmul_utils.hpp:154-173
  *
@@ -69,6 +73,11 @@
  * tests/test_oracle_pins.py against closed-form numpy expectations (the
  * formula in f32 with the reference's intermediate roundings; nstl::max / min
  * NaN semantics).
+ * The inner product (oracle_inner_product_fwd) is pinned by
+ * tests/test_inner_product.py: numpy tensordot over the flattened (ic, spatial)
+ * dims on exact data for every ndims and for permuted layouts of src and
+ * weights, the scale / bias / dst-scale order on values where a different
+ * order changes bits; bias, post-ops and the store are orc_finish.
  * Unpinned: none of the functions used by the five benchmark configurations.
  * "Parity unpinned" beyond the textbook formula: the last bits of the
  * libm-dependent eltwise algorithms (tanh, elu, exp, log, pow, gelu_erf,
@@ -852,6 +861,61 @@ int oracle_reorder(const mi355_reorder_desc_t *d, const mi355_reorder_args_t *a)
         orc_store_float(d->dst_dt, x, a->dst, dof);
     }
     return 0;
+}
+
+/* Inner product, forward: dst[mb, oc] = sum over (ic, spatial) of
+ * src[mb, ic, ...] * weights[oc, ic, ...], both tensors addressed through their
+ * own strides (ref_ip_utils::get_data_off / get_weights_off,
+ * src/cpu/ref_inner_product_utils.hpp).  `dims` are the src dims
+ * (mb, ic, then the spatial dims in the order given), the weights have oc in
+ * place of mb.  The loop over the reduced dims runs in the logical row-major
+ * order, which is the reference's ic, kd, kh, kw nest.
+ *   integer src (ref_inner_product_int8.cpp:64-106): s32 sum; d = (float)acc;
+ *     d *= src_scale[0]; d *= wei_scale[mask > 0 ? oc : 0]; bias; post-ops;
+ *     d /= dst_scale[0]; store
+ *   any other src (ref_inner_product.cpp:52-98): f32 sum of f32 products in
+ *     loop order; bias; post-ops; store
+ * `e` describes everything after the sum in matmul terms (M = mb, N = oc,
+ * batch 1): data types, bias, scales, post-ops, dst strides. */
+int oracle_inner_product_fwd(int ndims, const int64_t *dims, int64_t OC, const int64_t *src_stride,
+        const int64_t *wei_stride, const mi355_matmul_desc_t *e, const mi355_matmul_args_t *a) {
+    if (!dims || !src_stride || !wei_stride || !e || !a || ndims < 2 || ndims > 5) return MI355_INVALID_ARGUMENTS;
+    const int64_t MB = dims[0];
+    int64_t Kt = 1;
+    for (int i = 1; i < ndims; ++i) Kt *= dims[i];
+    mi355_matmul_desc_t t = *e;
+    t.dst_scale_mode = MI355_DST_SCALE_DIVIDE;
+    const int int_path = orc_src_is_int(e->src_dt);
+#pragma omp parallel for schedule(static)
+    for (int64_t mb = 0; mb < MB; ++mb)
+        for (int64_t oc = 0; oc < OC; ++oc) {
+            int acc = 0;
+            float facc = 0.f;
+            for (int64_t k = 0; k < Kt; ++k) {
+                int64_t r = k, so = mb * src_stride[0], wo = oc * wei_stride[0];
+                for (int i = ndims - 1; i >= 1; --i) {
+                    const int64_t idx = r % dims[i];
+                    r /= dims[i];
+                    so += idx * src_stride[i];
+                    wo += idx * wei_stride[i];
+                }
+                if (int_path) {
+                    acc += orc_load_int(e->src_dt, a->src, so) * orc_load_int(e->wei_dt, a->wei, wo);
+                } else {
+                    const float sv = orc_load_float(e->src_dt, a->src, so);
+                    const float wv = orc_load_float(e->wei_dt, a->wei, wo);
+                    facc += sv * wv;
+                }
+            }
+            float d = int_path ? (float)acc : facc;
+            if (int_path) {
+                if (e->src_scale.dt != MI355_DT_UNDEF) d *= orc_load_float(e->src_scale.dt, a->src_scale, 0);
+                if (e->wei_scale.dt != MI355_DT_UNDEF)
+                    d *= orc_load_float(e->wei_scale.dt, a->wei_scale, e->wei_scale.mask ? oc : 0);
+            }
+            orc_finish(&t, a, d, 0, mb, oc);
+        }
+    return MI355_SUCCESS;
 }
 
 /* ------------------------------------------------------------- grouped matmul

@@ -1,7 +1,7 @@
-"""The boundary through a compiler: two small C programs that include only
+"""The boundary through a compiler: small C programs that include only
 include/dnnl_amd.h / include/mi355_matmul.h, built with gcc against the two
-shared libraries and run on the device (a u8 x s8 -> s32 matmul checked against
-an integer loop inside the program).  Struct layouts, enum values and calling
+shared libraries and run on the device (u8 x s8 -> s32 matmuls and an inner product on
+channels-last tensors, each checked against an integer loop inside the program).  Struct layouts, enum values and calling
 conventions of the headers are what a compiled caller sees; the ctypes tests
 only check names."""
 import os
@@ -29,14 +29,15 @@ def build(name, lib):
 
 def test_headers_compile_as_c_and_link():
     # no device needed: the programs build against the headers and libraries
-    for name, lib in (("dnnl_client", "dnnl_amd"), ("mi355_client", "mi355_matmul")):
+    for name, lib in (("dnnl_client", "dnnl_amd"), ("ip_client", "dnnl_amd"), ("mi355_client", "mi355_matmul")):
         d, exe = build(name, lib)
         assert os.path.exists(exe)
         shutil.rmtree(d, ignore_errors=True)
 
 
 @pytest.mark.gpu
-@pytest.mark.parametrize("name,lib", [("dnnl_client", "dnnl_amd"), ("mi355_client", "mi355_matmul")])
+@pytest.mark.parametrize("name,lib", [("dnnl_client", "dnnl_amd"), ("ip_client", "dnnl_amd"),
+                                      ("mi355_client", "mi355_matmul")])
 def test_c_client_runs_on_the_device(gpu, name, lib):
     d, exe = build(name, lib)
     try:
