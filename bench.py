@@ -47,7 +47,7 @@ PROFILE_OF = {
     ("c2", "any", 1): "woqp_kernel_c2_m1.md", ("c2", "any", 8): "woqp_kernel_c2_m8.md",
     ("c2", "any", 32): "woqp_kernel_c2_m32.md", ("c2", "ab", 1): "woq_gemv_kernel_c2_m1_plain_ab.md",
     ("c2", "ab", 8): "woq_gemv_kernel_c2_m8_plain_ab.md", ("c2", "ab", 32): "woq_gemv_kernel_c2_m32_plain_ab.md",
-    ("r1", "any"): "reorder_direct_kernel_r1_f32_s8_8192.md", ("r2", "any"): "transpose8_kernel_r2_s8_transpose_8192.md",
+    ("r1", "any"): "reorder_rows_kernel_r1_f32_s8_8192.md", ("r2", "any"): "transpose8w_kernel_r2_s8_transpose_8192.md",
     ("r3", "any"): "pack_woq64_kernel_r3_u4_4096x14336.md",
     ("g1", "any"): "grouped_nsplit_kernel_g1_deepseek_v3_prefill.md",
     ("g2", "any"): "grouped_nsplit_kernel_g2_llama4_scout_prefill.md",

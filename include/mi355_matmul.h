@@ -381,7 +381,12 @@ typedef struct mi355_reorder_args {
 int mi355_reorder_query(const mi355_reorder_desc_t *desc);
 
 /* Enqueue the reorder on `stream` (primitive_t::execute of the reorder
- * implementations, DNNL_ARG_FROM -> DNNL_ARG_TO).  Asynchronous. */
+ * implementations, DNNL_ARG_FROM -> DNNL_ARG_TO).  Asynchronous.  Dedicated
+ * kernels serve the reorders of the matmul path (row quantization of float
+ * tensors to 8-bit types, 8-bit transposition, 4-bit weights packing), two
+ * general ones everything else; MI355_REORDER_GENERIC=1 in the environment
+ * (read once per process) keeps the row-quantization and the 128 x 128
+ * transposition kernels out, for tests and measurements. */
 int mi355_reorder_launch(const mi355_reorder_desc_t *desc,
         const mi355_reorder_args_t *args, void *stream);
 

@@ -12,7 +12,7 @@
 //   dst = saturate_and_round<dst_dt>(d) (src/cpu/simple_q10n.hpp:41-81)
 // e8m0 sources are converted without arithmetic (:2645-2655).
 //
-// Two kernels:
+// Two general kernels:
 //   direct  the unit-stride dim of dst is also unit-stride in src (or no dim
 //           is): consecutive lanes walk that dim, four elements per lane when
 //           it divides, stores packed to 2 / 4 / 8 / 16 bytes.
@@ -20,7 +20,16 @@
 //           a 64x64 tile of the two dims goes through LDS, read with lanes
 //           along the src dim and written with lanes along the dst dim, so
 //           both sides move whole cache lines.
+// and dedicated ones for what the matmul path does with a reorder:
+//   rows          quantization of activations / weights (float src, 8-bit dst,
+//                 scales per tensor or per column), data types as template
+//                 parameters, parameters fetched once per lane
+//   transpose8(w) 8-bit transposition in registers (the layout change of
+//                 int8 / fp8 weights), 64 x 64 or 128 x 128 tiles
+//   pack_woq64    4-bit weights into the packed decode layout
+// MI355_REORDER_GENERIC=1 in the environment keeps rows and transpose8w out.
 #include "kernels.hpp"
+#include "tile_epilogue.hpp" // div_by_fma
 
 namespace mi355 {
 namespace {
@@ -479,6 +488,94 @@ __global__ void __launch_bounds__(256) reorder_direct_kernel(const reorder_t R_)
     }
 }
 
+// Row quantization: float src (f32 / bf16 / f16) to an 8-bit dst (s8 / u8 /
+// e4m3 / e5m2), both unit-stride along `a`, at most one outer dim (rows), no
+// sum, no src zero point, f32 scales per tensor or per column.  This is what
+// quantizing activations or weights is, and the generic direct kernel spends
+// some 45 instructions per element on it (per-unit offsets, parameter loads
+// and data-type dispatch).  Here a workgroup owns 1024 columns -- a lane four
+// consecutive ones -- for a block of rows: the scales and, for integer dst, the
+// reciprocals of the dst scales are fetched once per lane, the data types are
+// template parameters, four rows are in flight per lane, and every load or
+// store instruction moves whole 128-byte lines.  The arithmetic is convert()'s:
+// x = src_scale * x; x = x / dst_scale + dst_zp; saturate, round to nearest
+// even.  For integer dst the division is div_by_fma where its conditions hold
+// (the IEEE quotient bit for bit where the rounding to an integer can see it).
+template <int SDT, int DDT>
+__global__ void __launch_bounds__(256) reorder_rows_kernel(const reorder_t R_, unsigned rows_per_wg) {
+    const auto &R = *(const __attribute__((address_space(4))) reorder_t *)__builtin_amdgcn_kernarg_segment_ptr();
+    typedef uint32_t u4v __attribute__((ext_vector_type(4)));
+    typedef uint32_t u2v __attribute__((ext_vector_type(2)));
+    constexpr bool INT_DST = DDT == MI355_DT_S8 || DDT == MI355_DT_U8;
+    constexpr int U = 4;
+    const unsigned a = (blockIdx.x * 256 + threadIdx.x) * 4;
+    if (a >= R.a.n) return;
+    const unsigned rows = R.n_outer ? R.outer[0].n : 1;
+    const long rs = R.n_outer ? R.outer[0].ss : 0, rd = R.n_outer ? R.outer[0].ds : 0;
+    const unsigned r0 = blockIdx.y * rows_per_wg;
+    const unsigned r1 = min(rows, r0 + rows_per_wg);
+    float s0[4], s1[4], y1[4];
+    bool fast = INT_DST;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+        s0[e] = R.qp[0] ? ((const float *)R.qp[0])[R.a.qs[0] ? a + e : 0] : 1.f;
+        s1[e] = R.qp[1] ? ((const float *)R.qp[1])[R.a.qs[1] ? a + e : 0] : 1.f;
+        y1[e] = 1.f / s1[e];
+        const float m = __builtin_fabsf(s1[e]);
+        fast = fast && m >= 0x1p-20f && m <= 0x1p20f;
+    }
+    const bool with_s0 = R.qp[0] != nullptr, with_div = R.qp[1] != nullptr || R.dst_zp != nullptr;
+    const float dzp = R.dst_zp ? (float)*(const int *)R.dst_zp : 0.f;
+    const char *src = (const char *)R.src + (long)a * (dt_bits(SDT) / 8);
+    uint8_t *dst = (uint8_t *)R.dst + a;
+    for (unsigned r = r0; r < r1; r += U) {
+        uint32_t raw[U][4];
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            const unsigned rr = min(r + u, r1 - 1); // a row past the block repeats the last one (and is not stored)
+            const char *p = src + (long)rr * rs * (dt_bits(SDT) / 8);
+            if constexpr (SDT == MI355_DT_F32) {
+                const u4v v = __builtin_nontemporal_load((const u4v *)p);
+                raw[u][0] = v.x; raw[u][1] = v.y; raw[u][2] = v.z; raw[u][3] = v.w;
+            } else {
+                const u2v v = __builtin_nontemporal_load((const u2v *)p);
+                raw[u][0] = v.x & 0xffffu; raw[u][1] = v.x >> 16; raw[u][2] = v.y & 0xffffu; raw[u][3] = v.y >> 16;
+            }
+        }
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            if (r + u >= r1) break;
+            float x[4];
+            unsigned mag = 0;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                x[e] = raw_to_float(SDT, raw[u][e]);
+                if (with_s0) x[e] = s0[e] * x[e];
+                mag = max(mag, gemm::mag_bits(x[e]));
+            }
+            if (with_div) {
+                if (fast && mag < gemm::DIV_BY_FMA_LIMIT) {
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) x[e] = gemm::div_by_fma(x[e], s1[e], y1[e]) + dzp;
+                } else {
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) x[e] = x[e] / s1[e] + dzp;
+                }
+            }
+            uint32_t w = 0;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                uint32_t b;
+                if constexpr (DDT == MI355_DT_S8) b = (uint32_t)(int)__builtin_rintf(sat(x[e], -128.f, 127.f)) & 0xffu;
+                else if constexpr (DDT == MI355_DT_U8) b = (uint32_t)(int)__builtin_rintf(sat(x[e], 0.f, 255.f)) & 0xffu;
+                else b = cvt_store_bits(DDT, x[e]) & 0xffu;
+                w |= b << (8 * e);
+            }
+            __builtin_nontemporal_store(w, (uint32_t *)(dst + (long)(r + u) * rd));
+        }
+    }
+}
+
 // 64 x 64 tile over (b, a): b has src stride 1, a has dst stride 1.  grid: x
 // over the tiles, y over the outer index.  MODE as in the direct kernel; the
 // modes other than MODE_GENERIC want the extent of a to be a multiple of four
@@ -604,6 +701,71 @@ __global__ void __launch_bounds__(256) transpose8_kernel(const reorder_t R_) {
             v.x = tile[wb * PITCH + 4 * wq]; v.y = tile[wb * PITCH + 4 * wq + 1];
             v.z = tile[wb * PITCH + 4 * wq + 2]; v.w = tile[wb * PITCH + 4 * wq + 3];
             *(uint4 *)(dst + dof + (b0 + wb) * R.b.ds + a0 + 16 * wq) = v;
+            __syncthreads();
+        }
+    }
+}
+
+// The same transposition on 128 x 128 tiles, for extents that are multiples of
+// 128 and 16-byte aligned rows: every load instruction fetches the whole
+// 128-byte lines of eight src rows and every store instruction writes the
+// whole lines of eight dst rows, so no line is touched by two workgroups
+// (with 64-byte tile rows every src line was fetched twice, by workgroups on
+// different L2s).  A thread loads 4 rows x 16 bytes, transposes the four
+// 4 x 4 blocks in registers and parks 16 dwords in LDS; dword column c of
+// tile row b sits at (c + 8 (b / 16)) % 32, which spreads a store instruction
+// over all banks and keeps the 16-byte reads aligned.
+__global__ void __launch_bounds__(256) transpose8w_kernel(const reorder_t R_) {
+    const auto &R = *(const __attribute__((address_space(4))) reorder_t *)__builtin_amdgcn_kernarg_segment_ptr();
+    __shared__ __attribute__((aligned(16))) uint32_t tile[128 * 32];
+    const unsigned tiles_b = R.b.n / 128, ntiles = (R.a.n / 128) * tiles_b;
+    const int bi = threadIdx.x & 7, ag = threadIdx.x >> 3; // read: rows 4 ag .. +3, bytes 16 bi .. +15
+    const int wq = threadIdx.x & 7, wr = threadIdx.x >> 3; // write: row wr + 32 pass, bytes 16 wq .. +15
+    const uint8_t *src = (const uint8_t *)R.src;
+    uint8_t *dst = (uint8_t *)R.dst;
+    for (unsigned o = blockIdx.y; o < R.outer_total; o += gridDim.y) {
+        long so = 0, dof = 0;
+        {
+            unsigned oo = o;
+            for (int i = 0; i < R.n_outer; ++i) {
+                const unsigned n = R.outer[i].n;
+                const unsigned q = oo / n, r = oo - q * n;
+                oo = q;
+                so += (long)r * R.outer[i].ss;
+                dof += (long)r * R.outer[i].ds;
+            }
+        }
+        for (unsigned t = blockIdx.x; t < ntiles; t += gridDim.x) {
+            const unsigned tb = t % tiles_b, ta = t / tiles_b;
+            const long a0 = (long)ta * 128, b0 = (long)tb * 128;
+            const uint8_t *p = src + so + (a0 + 4 * ag) * R.a.ss + b0 + 16 * bi;
+            typedef uint32_t u4v __attribute__((ext_vector_type(4)));
+            u4v r[4];
+#pragma unroll
+            for (int i = 0; i < 4; ++i) r[i] = __builtin_nontemporal_load((const u4v *)(p + i * R.a.ss));
+            const int col = (ag + 8 * (bi & 3)) & 31;
+#pragma unroll
+            for (int k = 0; k < 4; ++k) {
+                const uint32_t r0 = k == 0 ? r[0].x : k == 1 ? r[0].y : k == 2 ? r[0].z : r[0].w;
+                const uint32_t r1 = k == 0 ? r[1].x : k == 1 ? r[1].y : k == 2 ? r[1].z : r[1].w;
+                const uint32_t r2 = k == 0 ? r[2].x : k == 1 ? r[2].y : k == 2 ? r[2].z : r[2].w;
+                const uint32_t r3 = k == 0 ? r[3].x : k == 1 ? r[3].y : k == 2 ? r[3].z : r[3].w;
+                // byte j of r_i is element (a + i, b + 4 k + j); T_j collects byte j of the four rows
+                const uint32_t x0 = __builtin_amdgcn_perm(r1, r0, 0x05010400u), x1 = __builtin_amdgcn_perm(r1, r0, 0x07030602u);
+                const uint32_t y0 = __builtin_amdgcn_perm(r3, r2, 0x05010400u), y1 = __builtin_amdgcn_perm(r3, r2, 0x07030602u);
+                const int row = 16 * bi + 4 * k;
+                tile[(row + 0) * 32 + col] = __builtin_amdgcn_perm(y0, x0, 0x05040100u);
+                tile[(row + 1) * 32 + col] = __builtin_amdgcn_perm(y0, x0, 0x07060302u);
+                tile[(row + 2) * 32 + col] = __builtin_amdgcn_perm(y1, x1, 0x05040100u);
+                tile[(row + 3) * 32 + col] = __builtin_amdgcn_perm(y1, x1, 0x07060302u);
+            }
+            __syncthreads();
+#pragma unroll
+            for (int pass = 0; pass < 4; ++pass) {
+                const int b = wr + 32 * pass;
+                const u4v v = *(const u4v *)&tile[b * 32 + ((4 * wq + 8 * ((b >> 4) & 3)) & 31)];
+                __builtin_nontemporal_store(v, (u4v *)(dst + dof + (b0 + b) * R.b.ds + a0 + 16 * wq));
+            }
             __syncthreads();
         }
     }
@@ -900,6 +1062,9 @@ extern "C" int mi355_reorder_launch(const mi355_reorder_desc_t *desc, const mi35
     if (outer >= (1L << 31)) return MI355_UNIMPLEMENTED;
     R.outer_total = (unsigned)outer;
 
+    // MI355_REORDER_GENERIC=1 keeps the dedicated kernels (row quantization, whole-line transposition) out: for
+    // measurements and tests of the kernels behind them
+    static const bool generic_only = getenv("MI355_REORDER_GENERIC") != nullptr;
     const int dbits = dt_bits(d.dst_dt), sbits = dt_bits(d.src_dt);
     // E elements per lane along `a` as one aligned vector (several 16-byte ones
     // beyond 16 bytes): unit stride, an extent that divides, every other stride
@@ -955,12 +1120,62 @@ extern "C" int mi355_reorder_launch(const mi355_reorder_desc_t *desc, const mi35
             for (int i = 0; i < R.n_outer && qvec; ++i)
                 if (R.outer[i].qs[k] % 4) qvec = false;
         }
+        // ... and whole 128-byte lines on both sides where the extents and the row pitches allow
+        bool t8w = t8 && R.a.n % 128 == 0 && R.b.n % 128 == 0 && R.a.ss % 16 == 0 && (uintptr_t)R.src % 16 == 0
+                && !generic_only;
+        for (int i = 0; i < R.n_outer && t8w; ++i)
+            if (R.outer[i].ss % 16) t8w = false;
         const dim3 grid((unsigned)gx, gy), block(256);
-        if (t8) hipLaunchKernelGGL(transpose8_kernel, grid, block, 0, hs, R);
+        if (t8w) {
+            long gw = (long)(R.a.n / 128) * (R.b.n / 128);
+            if (gw > (1 << 20)) gw = 1 << 20;
+            hipLaunchKernelGGL(transpose8w_kernel, dim3((unsigned)gw, gy), block, 0, hs, R);
+        } else if (t8) hipLaunchKernelGGL(transpose8_kernel, grid, block, 0, hs, R);
         else if (R.a.n % 4 == 0 && simple) hipLaunchKernelGGL(reorder_tiled_kernel<MODE_SIMPLE>, grid, block, 0, hs, R);
         else if (R.a.n % 4 == 0 && qvec) hipLaunchKernelGGL(reorder_tiled_kernel<MODE_QVEC>, grid, block, 0, hs, R);
         else hipLaunchKernelGGL(reorder_tiled_kernel<MODE_GENERIC>, grid, block, 0, hs, R);
     } else {
+        // row quantization (float src, 8-bit dst, per-tensor / per-column f32 scales): the dedicated kernel
+        {
+            const bool src_ok = d.src_dt == MI355_DT_F32 || d.src_dt == MI355_DT_BF16 || d.src_dt == MI355_DT_F16;
+            const bool dst_ok = d.dst_dt == MI355_DT_S8 || d.dst_dt == MI355_DT_U8 || d.dst_dt == MI355_DT_F8_E4M3
+                    || d.dst_dt == MI355_DT_F8_E5M2;
+            const long sbytes = 4L * sbits / 8;
+            bool rows_ok = src_ok && dst_ok && d.beta == 0.f && R.n_outer <= 1 && R.a.ss == 1 && R.a.ds == 1
+                    && R.a.n % 4 == 0 && !R.qp[2] && (uintptr_t)R.src % (size_t)sbytes == 0 && (uintptr_t)R.dst % 4 == 0
+                    && !generic_only;
+            if (rows_ok && R.n_outer == 1) rows_ok = R.outer[0].ss % 4 == 0 && R.outer[0].ds % 4 == 0;
+            for (int k = 0; k < 2 && rows_ok; ++k) {
+                if (!R.qp[k]) continue;
+                rows_ok = R.qdt[k] == MI355_DT_F32 && (R.a.qs[k] == 0 || (R.a.qs[k] == 1 && R.a.qg[k] == 1))
+                        && (R.n_outer == 0 || R.outer[0].qs[k] == 0);
+            }
+            if (rows_ok) {
+                const unsigned rows = R.n_outer ? R.outer[0].n : 1;
+                const unsigned chunks = (unsigned)((R.a.n / 4 + 255) / 256);
+                // some 4096 workgroups, at least four rows (one round of loads) each
+                unsigned per = (unsigned)(((unsigned long)rows * chunks + 4095) / 4096);
+                per = per < 4 ? 4 : (per + 3) / 4 * 4;
+                const dim3 rgrid(chunks, (rows + per - 1) / per), block(256);
+                if (rgrid.y <= 65535) {
+#define MI355_ROWS_CASE(S_, D_) \
+    if (d.src_dt == S_ && d.dst_dt == D_) hipLaunchKernelGGL((reorder_rows_kernel<S_, D_>), rgrid, block, 0, hs, R, per);
+#define MI355_ROWS_SRC(S_) \
+    MI355_ROWS_CASE(S_, MI355_DT_S8) MI355_ROWS_CASE(S_, MI355_DT_U8) MI355_ROWS_CASE(S_, MI355_DT_F8_E4M3) \
+    MI355_ROWS_CASE(S_, MI355_DT_F8_E5M2)
+                    MI355_ROWS_SRC(MI355_DT_F32)
+                    MI355_ROWS_SRC(MI355_DT_BF16)
+                    MI355_ROWS_SRC(MI355_DT_F16)
+#undef MI355_ROWS_SRC
+#undef MI355_ROWS_CASE
+                    if (hipGetLastError() != hipSuccess) {
+                        set_error("reorder: launch failed");
+                        return MI355_RUNTIME_ERROR;
+                    }
+                    return MI355_SUCCESS;
+                }
+            }
+        }
         R.elems = E;
         // units of all outer indices in one grid-stride walk; enough workgroups
         // to fill the device a few times over, each lane several units

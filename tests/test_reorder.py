@@ -15,6 +15,8 @@ What pins the oracle's reorder (src/cpu/reorder/simple_reorder.hpp:2579-2661,
     (tests/gtests/internals/test_nibble.cpp:36-88) is restated in
     test_oracle_dtypes.py for pack_nibbles/unpack_nibbles, which are used here.
 """
+import os
+
 import numpy as np
 import pytest
 
@@ -154,6 +156,8 @@ def _case(name, dims, src_dt, dst_dt, seed, src_perm=None, dst_perm=None, quant=
         src = (r.standard_normal(n) * 20).astype(np.float32)
     elif src_dt == cabi.DT_BF16:
         src = dtp.f32_to_bf16((r.standard_normal(n) * 20).astype(np.float32))
+    elif src_dt == cabi.DT_F16:
+        src = (r.standard_normal(n) * 20).astype(np.float16).view(np.uint16)
     elif src_dt == cabi.DT_S8:
         src = r.integers(-128, 128, size=n).astype(np.int8)
     elif src_dt == cabi.DT_U8:
@@ -222,6 +226,10 @@ CASES = [
     lambda: _case("u8 batched acb whole tiles", (3, 64, 128), cabi.DT_U8, cabi.DT_U8, 51, dst_perm=(0, 2, 1)),
     lambda: _case("e4m3 ba->ab whole tiles", (192, 64), cabi.DT_F8_E4M3, cabi.DT_F8_E4M3, 52, src_perm=(1, 0)),
     lambda: _case("s8 ab->ba ragged", (130, 192), cabi.DT_S8, cabi.DT_S8, 53, dst_perm=(1, 0)),
+    # ... on 128 x 128 tiles (whole cache lines on both sides) where both extents are multiples of 128
+    lambda: _case("s8 ab->ba whole 128-byte lines", (256, 384), cabi.DT_S8, cabi.DT_S8, 80, dst_perm=(1, 0)),
+    lambda: _case("u8 batched acb whole 128-byte lines", (3, 128, 256), cabi.DT_U8, cabi.DT_U8, 81, dst_perm=(0, 2, 1)),
+    lambda: _case("e4m3 ba->ab whole 128-byte lines", (384, 128), cabi.DT_F8_E4M3, cabi.DT_F8_E4M3, 82, src_perm=(1, 0)),
     # tiled kernel: attribute-free, parameters constant along / consecutive along the dst-contiguous dim, generic
     lambda: _case("bf16->f32 transposed", (96, 80), cabi.DT_BF16, cabi.DT_F32, 54, dst_perm=(1, 0)),
     lambda: _case("u4 transposed", (64, 96), cabi.DT_U4, cabi.DT_U4, 55, dst_perm=(1, 0)),
@@ -275,6 +283,76 @@ def test_gpu_reorder_is_bit_exact(make):
     got = run_gpu(p)
     bad = np.flatnonzero(got != want)
     assert bad.size == 0, f"{p.name}: {bad.size} of {got.size} storage elements differ, first at {bad[:5]}"
+
+
+# Row quantization kernel (float src -> 8-bit dst, scales per tensor or per column, at most one outer dim): ragged row
+# counts, column counts that end inside a workgroup's 1024, every src / dst type it takes, and the values that leave
+# its reciprocal-based division (scales outside 2^-20 .. 2^20, huge / infinite / tiny / signed-zero values)
+ROW_CASES = [
+    lambda: _case("f32->s8 src common, dst per column, dst zp", (37, 1100), cabi.DT_F32, cabi.DT_S8, 90,
+                  quant={"src_scale": _qp(91, cabi.DT_F32, 0, (1,)), "dst_scale": _qp(92, cabi.DT_F32, 2, (1100,)),
+                         "dst_zp": _qp(93, cabi.DT_S32, 0, (1,))}),
+    lambda: _case("bf16->e4m3 common src scale", (5, 2052), cabi.DT_BF16, cabi.DT_F8_E4M3, 94,
+                  quant={"src_scale": _qp(95, cabi.DT_F32, 0, (1,), lo=0.5, hi=4.0)}),
+    lambda: _case("f16->u8 per-column src scale, dst zp", (18, 260), cabi.DT_F16, cabi.DT_U8, 96,
+                  quant={"src_scale": _qp(97, cabi.DT_F32, 2, (260,)), "dst_zp": _qp(98, cabi.DT_S32, 0, (1,))}),
+    lambda: _case("f32->e5m2 per-column dst scale", (7, 512), cabi.DT_F32, cabi.DT_F8_E5M2, 99,
+                  quant={"dst_scale": _qp(100, cabi.DT_F32, 2, (512,))}),
+    lambda: _case("f32->s8 one row", (4096,), cabi.DT_F32, cabi.DT_S8, 101,
+                  quant={"dst_scale": _qp(102, cabi.DT_F32, 0, (1,))}),
+    lambda: _case("bf16->s8 attribute-free", (9, 1024), cabi.DT_BF16, cabi.DT_S8, 103),
+    lambda: _case("f16->e4m3 batched rows merge into one outer dim", (3, 5, 256), cabi.DT_F16, cabi.DT_F8_E4M3, 104,
+                  quant={"dst_scale": _qp(105, cabi.DT_F32, 4, (256,))}),
+]
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("make", ROW_CASES, ids=[f"rows{i}" for i in range(len(ROW_CASES))])
+def test_gpu_row_quantization_is_bit_exact(make):
+    p = make()
+    assert query(p) == cabi.SUCCESS, p.name
+    want = oracle.reorder(p)
+    got = run_gpu(p)
+    bad = np.flatnonzero(got != want)
+    assert bad.size == 0, f"{p.name}: {bad.size} of {got.size} storage elements differ, first at {bad[:5]}"
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dst_dt", [cabi.DT_S8, cabi.DT_U8, cabi.DT_F8_E4M3])
+def test_gpu_row_quantization_special_values(dst_dt):
+    rows, cols = 12, 64
+    r = rng(110)
+    x = (r.standard_normal((rows, cols)) * 50).astype(np.float32)
+    special = np.array([np.inf, -np.inf, 3e38, -3e38, 1e-40, -1e-40, 0.0, -0.0, 2.0 ** 100, -(2.0 ** 99), 127.5, -128.5,
+                        0.5, 1.5, 2.5, -0.5, 1e-30, 448.0, 500.0, 57344.0], np.float32)
+    x[0, :special.size] = special
+    x[5, 3:3 + special.size] = special
+    if dst_dt == cabi.DT_F8_E4M3:
+        x[7, 9] = np.nan
+    sc = r.uniform(0.05, 2.0, size=cols).astype(np.float32)
+    sc[[1, 17, 40]] = [1e-8, 3e7, 2.0 ** -20]          # outside / at the edge of the reciprocal path's range
+    sc[[2, 18]] = [-0.75, 2.0 ** 20]
+    p = ReorderProblem(dims=(rows, cols), src_dt=cabi.DT_F32, dst_dt=dst_dt, src=x.reshape(-1),
+                       quant={"dst_scale": QuantParam(cabi.DT_F32, 2, sc)}, name="special values")
+    assert query(p) == cabi.SUCCESS
+    want = oracle.reorder(p)
+    got = run_gpu(p)
+    bad = np.flatnonzero(got != want)
+    assert bad.size == 0, f"{bad.size} of {got.size} differ, first at {bad[:8]}: got {got[bad[:8]]} want {want[bad[:8]]}"
+
+
+@pytest.mark.gpu
+def test_gpu_generic_kernels_behind_the_dedicated_ones():
+    """MI355_REORDER_GENERIC=1 (read once per process) keeps the row-quantization and whole-line transposition
+    kernels out, so the same cases run on the direct / 64 x 64 kernels they would otherwise shadow."""
+    import subprocess
+    import sys
+    env = dict(os.environ, MI355_REORDER_GENERIC="1")
+    out = subprocess.run(
+        [sys.executable, "-m", "pytest", os.path.abspath(__file__), "-q", "-m", "gpu", "-x", "-k",
+         "test_gpu_reorder_is_bit_exact or test_gpu_row_quantization"],
+        env=env, capture_output=True, text=True, timeout=600, cwd=os.path.dirname(os.path.dirname(os.path.abspath(__file__))))
+    assert out.returncode == 0, out.stdout[-3000:] + out.stderr[-2000:]
 
 
 @pytest.mark.gpu
