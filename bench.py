@@ -22,6 +22,7 @@ Workloads (the benchmark configurations):
   c2  bf16 x u4 -> bf16 decode, K=4096 N=14336, M in {1,8,32} (HBM bound)
   c4  e4m3 x e4m3 -> bf16, 4096 x 8192 x 28672, bias+gelu+add (MFMA fp8 bound)
   c5  MXFP4, M=N=K=8192 (MFMA fp4 bound)
+  h1  bf16 x bf16 -> bf16, M=N=K=8192 (MFMA bf16 bound; the unquantized matmul on the same tiles)
   c1  u8 x s8 -> f32, 256 x 1024 x 1024 (latency bound, no roofline claim)
 """
 import argparse
@@ -44,6 +45,7 @@ import numpy as np  # noqa: E402
 PROFILE_OF = {
     ("c3", "any"): "i8_gemm_kernel_c3_8192.md", ("c4", "any"): "f8_gemm_kernel_c4_4096x8192x28672.md",
     ("c5", "any"): "mxf4_gemm_kernel_c5_8192.md", ("c1", "any"): "i8_small_kernel_c1_256x1024x1024.md",
+    ("h1", "any"): "f8_gemm_kernel_h1_bf16_8192.md",
     ("c2", "any", 1): "woqp_kernel_c2_m1.md", ("c2", "any", 8): "woqp_kernel_c2_m8.md",
     ("c2", "any", 32): "woqp_kernel_c2_m32.md", ("c2", "ab", 1): "woq_gemv_kernel_c2_m1_plain_ab.md",
     ("c2", "ab", 8): "woq_gemv_kernel_c2_m8_plain_ab.md", ("c2", "ab", 32): "woq_gemv_kernel_c2_m32_plain_ab.md",
@@ -77,6 +79,7 @@ PEAK_HBM_GBS = 8000.0
 PEAK_I8_TOPS = 5000.0
 PEAK_F8_TFLOPS = 5000.0
 PEAK_F4_TFLOPS = 10100.0
+PEAK_BF16_TFLOPS = 2500.0
 
 
 def log(*a):
@@ -136,6 +139,8 @@ def build_problem(name, M=None, wtag="any"):
         return p
     if name == "c5":
         return configs.config5(wtag=mfma_tag)
+    if name == "h1":
+        return configs.config_h16(wtag=mfma_tag)
     raise ValueError(name)
 
 
@@ -151,6 +156,8 @@ def algorithmic(name, p):
         return ops, "TFLOP/s", "mfma", PEAK_F8_TFLOPS
     if name == "c5":
         return ops, "TFLOP/s", "mfma", PEAK_F4_TFLOPS
+    if name == "h1":
+        return ops, "TFLOP/s", "mfma", PEAK_BF16_TFLOPS
     return ops, "TOPS", "mfma", PEAK_I8_TOPS
 
 
@@ -361,6 +368,9 @@ def cpu_baseline(name, M=None):
     elif name == "c5":
         p = configs.config5(M=128, N=1024, K=8192)
         sample = "M=128, N=1024, K=8192 slice of the 8192^3 shape"
+    elif name == "h1":
+        p = configs.config_h16(M=128, N=1024, K=8192)
+        sample = "M=128, N=1024, K=8192 slice of the 8192^3 shape"
     else:
         p = configs.config1()
         sample = "full problem 256x1024x1024"
@@ -378,7 +388,8 @@ def cpu_baseline(name, M=None):
     # where it could be built is quoted so that the port's number is not read as the reference's speed
     probe = {"c3": "4.97 TOPS (221 ms)", "c1": "6.37 TOPS (0.084 ms)",
              "c2": {1: "4.17 GB/s (7.05 ms)", 8: "4.64 GB/s (6.39 ms)", 32: "3.16 GB/s (9.67 ms)"}.get(M or 1),
-             "c4": "no JIT implementation on that host (ref:any only)", "c5": "no CPU implementation (skipped)"}[name]
+             "c4": "no JIT implementation on that host (ref:any only)", "c5": "no CPU implementation (skipped)",
+             "h1": "not measured"}[name]
     return {"value": rate(work * reps, dt * 1e3, unit), "unit": unit, "cores": threads, "kind": "port",
             "reference_probe": {"what": "benchdnn --matmul --mode=P on the reference built with its own CMake, "
                                         "impl brg_matmul:avx10_1_512_amx, this configuration at full size",
@@ -394,7 +405,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=3)
-    ap.add_argument("--workload", default="c3", choices=["c1", "c2", "c3", "c4", "c5", "r1", "r2", "r3", "g1", "g2", "g3", "g4", "g5"],
+    ap.add_argument("--workload", default="c3", choices=["c1", "c2", "c3", "c4", "c5", "h1", "r1", "r2", "r3", "g1", "g2", "g3", "g4", "g5"],
                     help="c1..c5: the matmul configurations (c3 is the headline); r1..r3: the reorder "
                          "primitive on the headline shape's tensors; g1..g5: the grouped (mixture-of-experts) "
                          "matmul on shapes of the reference's shapes_grouped_moe files: fp8 with row / column scales "
@@ -581,7 +592,8 @@ def main():
         # (workload, M, weights tag); "ab" = row-major weights as in the reference's benchdnn line for C3: the
         # layout change then runs inside every launch
         plan = [("c2", 1, "any"), ("c2", 8, "any"), ("c2", 32, "any"), ("c3", None, "any"), ("c3", None, "ab"),
-                ("c4", None, "any"), ("c4mx", None, "any"), ("c5", None, "any"), ("c1", None, "any")]
+                ("c4", None, "any"), ("c4mx", None, "any"), ("c5", None, "any"), ("c1", None, "any"),
+                ("h1", None, "any")]
         for nm, m, wt in plan:
             if nm == main_name and wt == args.wtag and (nm != "c2" or m == args.decode_m):
                 continue
@@ -617,8 +629,8 @@ def main():
 
     metric = {"c3": "int8 matmul TOPS @8192^3", "c2": "int4 weight-only decode GB/s",
               "c4": "fp8 matmul TFLOP/s @4096x8192x28672", "c5": "MXFP4 matmul TFLOP/s @8192^3",
-              "c1": "int8 matmul TOPS @256x1024x1024"}[main_name]
-    dtype = {"c3": "s8", "c2": "bf16", "c4": "f8_e4m3", "c5": "f4_e2m1", "c1": "u8"}[main_name]
+              "c1": "int8 matmul TOPS @256x1024x1024", "h1": "bf16 matmul TFLOP/s @8192^3"}[main_name]
+    dtype = {"c3": "s8", "c2": "bf16", "c4": "f8_e4m3", "c5": "f4_e2m1", "c1": "u8", "h1": "bf16"}[main_name]
     line = {
         "metric": metric, "value": res["value"], "unit": res["unit"], "n_gpus": 1,
         "steps": args.steps, "warmup": args.warmup, "ms_per_step": res["ms_per_step"],

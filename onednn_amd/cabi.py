@@ -41,6 +41,7 @@ BINARY = {
 
 DST_SCALE_DIVIDE, DST_SCALE_RECIPROCAL = 0, 1
 IMPL_AUTO, IMPL_REF, IMPL_I8_MFMA, IMPL_F8_MFMA, IMPL_MXF4_MFMA, IMPL_WOQ_GEMV, IMPL_WOQ_PACKED = range(7)
+IMPL_H16_MFMA = 7
 NOALLOC_SCRATCH_BYTES = 8 << 20
 WEI_PACK_NONE, WEI_PACK_WOQ64 = 0, 1
 DST_DYNAMIC_NONE, DST_DYNAMIC_MX, DST_DYNAMIC_FP = 0, 1, 2

@@ -161,6 +161,7 @@ static int impl_supported(const mi355_matmul_desc_t &d, int impl) {
         case MI355_IMPL_REF: return ref_supported(d);
         case MI355_IMPL_I8_MFMA: return i8_supported(d);
         case MI355_IMPL_F8_MFMA: return f8_supported(d);
+        case MI355_IMPL_H16_MFMA: return h16_supported(d);
         case MI355_IMPL_MXF4_MFMA: return mxf4_supported(d);
         case MI355_IMPL_WOQ_GEMV: return woq_supported(d);
         case MI355_IMPL_WOQ_PACKED: return woqp_supported(d);
@@ -171,7 +172,7 @@ static int impl_supported(const mi355_matmul_desc_t &d, int impl) {
 // priority order of the implementation list (fastest first, generic last),
 // the role of an engine's impl_list_item_t[] in the reference
 static const int g_impl_order[] = {MI355_IMPL_WOQ_PACKED, MI355_IMPL_WOQ_GEMV, MI355_IMPL_I8_MFMA, MI355_IMPL_F8_MFMA,
-        MI355_IMPL_MXF4_MFMA, MI355_IMPL_REF};
+        MI355_IMPL_MXF4_MFMA, MI355_IMPL_H16_MFMA, MI355_IMPL_REF};
 
 static int choose_impl(const mi355_matmul_desc_t &d, int *chosen) {
     if (d.impl != MI355_IMPL_AUTO) {
@@ -391,6 +392,7 @@ const char *mi355_matmul_impl_name(int impl) {
         case MI355_IMPL_REF: return "hip:ref:any";
         case MI355_IMPL_I8_MFMA: return "hip:mfma_i8:gfx950";
         case MI355_IMPL_F8_MFMA: return "hip:mfma_f8:gfx950";
+        case MI355_IMPL_H16_MFMA: return "hip:mfma_h16:gfx950";
         case MI355_IMPL_MXF4_MFMA: return "hip:mfma_mxf4:gfx950";
         case MI355_IMPL_WOQ_GEMV: return "hip:woq_gemv:gfx950";
         case MI355_IMPL_WOQ_PACKED: return "hip:woq_packed:gfx950";
@@ -422,6 +424,7 @@ int mi355_matmul_scratch_bytes(const mi355_matmul_desc_t *desc, size_t *bytes) {
     switch (impl) {
         case MI355_IMPL_I8_MFMA: *bytes = i8_scratch_bytes(*desc); break;
         case MI355_IMPL_F8_MFMA: *bytes = f8_scratch_bytes(*desc); break;
+        case MI355_IMPL_H16_MFMA: *bytes = h16_scratch_bytes(*desc); break;
         case MI355_IMPL_MXF4_MFMA: *bytes = mxf4_scratch_bytes(*desc); break;
         case MI355_IMPL_WOQ_GEMV: *bytes = woq_scratch_bytes(*desc); break;
         default: break;
@@ -449,6 +452,7 @@ int mi355_matmul_launch(const mi355_matmul_desc_t *desc, const mi355_matmul_args
         case MI355_IMPL_REF: return ref_launch(P, s);
         case MI355_IMPL_I8_MFMA: return i8_launch(*desc, P, scratch, s);
         case MI355_IMPL_F8_MFMA: return f8_launch(*desc, P, scratch, s);
+        case MI355_IMPL_H16_MFMA: return h16_launch(*desc, P, scratch, s);
         case MI355_IMPL_MXF4_MFMA: return mxf4_launch(*desc, P, scratch, s);
         case MI355_IMPL_WOQ_GEMV: return woq_launch(*desc, P, scratch, s);
         case MI355_IMPL_WOQ_PACKED: return woqp_launch(*desc, P, s);

@@ -18,6 +18,14 @@
 // of one group, shorter than the memory latency (measured 175 us per 256x256
 // tile at K = 8192).  The 32x32x64 shape consumes one 64-byte stage like the
 // int8 kernel and keeps three stages in flight.
+//
+// "hip:mfma_h16" -- the same tiles for bf16 x bf16 and f16 x f16 operands
+// (ref_matmul_t's f32 sum of exact products): a 64-byte stage is 32 elements of
+// K, two v_mfma_f32_32x32x16_{bf16,f16} per fragment pair in the time of the
+// one fp8 instruction, so the data path (DMA, LDS ring, fragment reads,
+// epilogue) is shared unchanged; a lane's two 16-byte chunks of a stage feed
+// the two instructions, the same chunks for both operands, so the order in
+// which the 32 k of a stage meet does not matter.
 #include "gemm_core.hpp"
 
 namespace mi355 {
@@ -40,6 +48,8 @@ struct f8_ctx_t {};
 template <int FMT_A, int FMT_B, class G_>
 struct f8_mma_t {
     using G = G_;
+    static constexpr int ELEM_BYTES = 1;
+    static constexpr bool HOT = FMT_A == 0 && FMT_B == 0;
     static constexpr int EXTRA_DMAS = 0;
     __device__ static __forceinline__ void issue_extra(const f8_ctx_t &, int, int, int, int) {}
     static constexpr int ROWS = 4, COLS = G::WCOLS / 32, A_READS = 2, B_READS = 2;
@@ -80,6 +90,57 @@ struct f8_mma_t {
             // consecutive n of one row per accumulator quad (tile_epilogue.hpp)
             acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(
                     f.b[j], f.a[i], acc[i][j], FMT_B, FMT_A, 0, 0, 0, 0);
+    }
+};
+
+typedef __bf16 v8bf_t __attribute__((ext_vector_type(8)));
+typedef _Float16 v8h_t __attribute__((ext_vector_type(8)));
+
+// bf16 (BF16) or f16 operands: the fp8 policy's addresses and reads; a fragment
+// is its two 16-byte chunks, each the operand of one 32x32x16 instruction
+template <bool BF16, class G_>
+struct h16_mma_t {
+    using G = G_;
+    static constexpr int ELEM_BYTES = 2;
+    static constexpr bool HOT = BF16; // the whole-row bf16 epilogue chains of the fp8 family
+    static constexpr int EXTRA_DMAS = 0;
+    __device__ static __forceinline__ void issue_extra(const f8_ctx_t &, int, int, int, int) {}
+    static constexpr int ROWS = 4, COLS = G::WCOLS / 32, A_READS = 2, B_READS = 2;
+    struct frag_t {
+        v4i a[ROWS][2], b[COLS][2];
+    };
+    __device__ static __forceinline__ frag_t zero_frag() { return frag_t {}; }
+    using addr_t = typename f8_mma_t<0, 0, G_>::addr_t;
+    __device__ static __forceinline__ addr_t lane_addr(int wm, int wn, int lane) {
+        return f8_mma_t<0, 0, G_>::lane_addr(wm, wn, lane);
+    }
+    __device__ static __forceinline__ void load_b(frag_t &f, const unsigned (&S)[1], const addr_t &ad,
+            const f8_ctx_t &, int) {
+#pragma unroll
+        for (int j = 0; j < COLS; ++j) {
+            f.b[j][0] = lds_read16(S[0] + ad.b0 + j * 2048);
+            f.b[j][1] = lds_read16(S[0] + ad.b1 + j * 2048);
+        }
+    }
+    __device__ static __forceinline__ void load_a(frag_t &f, int i, const unsigned (&S)[1], const addr_t &ad,
+            const f8_ctx_t &, int) {
+        f.a[i][0] = lds_read16(S[0] + ad.a0 + i * 2048);
+        f.a[i][1] = lds_read16(S[0] + ad.a1 + i * 2048);
+    }
+    __device__ static __forceinline__ void mma_row(v16f (&acc)[ROWS][COLS], const frag_t &f, int i,
+            const f8_ctx_t &, int) {
+#pragma unroll
+        for (int h = 0; h < 2; ++h)
+#pragma unroll
+            for (int j = 0; j < COLS; ++j) {
+                // operands exchanged, as in the fp8 policy: the tile comes out transposed
+                if constexpr (BF16)
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(v8bf_t, f.b[j][h]),
+                            __builtin_bit_cast(v8bf_t, f.a[i][h]), acc[i][j], 0, 0, 0);
+                else
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(v8h_t, f.b[j][h]),
+                            __builtin_bit_cast(v8h_t, f.a[i][h]), acc[i][j], 0, 0, 0);
+            }
     }
 };
 
@@ -210,7 +271,8 @@ struct f8_conv_t {
             const long r = d * 8 + wr;
             const int chunk = wslot ^ (int)(r & 7);
             const v4u_t q = *(lds_u4_ptr_t)(size_t)(lds_part + (unsigned)(d * 1024 + lane * 16));
-            if (r < rows_left) *(v4u_t *)(dbase + r * P.ds[1] * 2 + chunk * 16) = q;
+            // written once, never read again by this launch: non-temporal
+            if (r < rows_left) __builtin_nontemporal_store(q, (v4u_t *)(dbase + r * P.ds[1] * 2 + chunk * 16));
         }
     }
     template <class PT, int C>
@@ -268,9 +330,10 @@ struct f8_conv_t {
 
 extern __shared__ __attribute__((aligned(16))) char f8_smem[];
 
-template <int FMT_A, int FMT_B, class G>
-__global__ void __launch_bounds__(G::NT) __attribute__((amdgpu_waves_per_eu(G::NW * G::WG_PER_CU / 4))) f8_gemm_kernel(const problem_t P_, const f8_extra_t X) {
-    using Mma = f8_mma_t<FMT_A, FMT_B, G>;
+template <class Mma>
+__global__ void __launch_bounds__(Mma::G::NT) __attribute__((amdgpu_waves_per_eu(Mma::G::NW * Mma::G::WG_PER_CU / 4))) f8_gemm_kernel(const problem_t P_, const f8_extra_t X) {
+    using G = typename Mma::G;
+    constexpr int EB = Mma::ELEM_BYTES;
     const auto &P = MI355_KERNARG_PROBLEM();
     char *smem = f8_smem;
     const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
@@ -279,12 +342,12 @@ __global__ void __launch_bounds__(G::NT) __attribute__((amdgpu_waves_per_eu(G::N
     const tile_pos_t tp = tile_position<G>((int)blockIdx.x, X.tiles_m, X.tiles_n);
     const long m0 = tp.m0, n0 = tp.n0;
 
-    const long lda = P.ss[1];
-    const char *A = (const char *)P.src + (P.ss[0] ? b * P.ss[0] : 0) + m0 * lda;
+    const long lda = P.ss[1] * EB; // bytes, like X.ldb and X.bt_bstride
+    const char *A = (const char *)P.src + (P.ss[0] ? b * P.ss[0] * EB : 0) + m0 * lda;
     const char *Bt = X.bt + b * X.bt_bstride + n0 * X.ldb;
 
     const long bs = P.ss[0] ? b : 0, bw = P.ws[0] ? b : 0;
-    f8_conv_t<FMT_A == 0 && FMT_B == 0> cv;
+    f8_conv_t<Mma::HOT> cv;
     cv.with_src_sc = P.src_scale.dt != MI355_DT_UNDEF;
     cv.with_wei_sc = P.wei_scale.dt != MI355_DT_UNDEF;
     cv.ssc_common = 1.f;
@@ -312,7 +375,7 @@ __global__ void __launch_bounds__(G::NT) __attribute__((amdgpu_waves_per_eu(G::N
             for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
 
     main_loop<NSTAGE, KSTEP, Mma>(acc, smem, A, Bt, lda, X.ldb, P.M - m0,
-            P.N - n0, (int)(P.K / (BKB * KSTEP)), f8_ctx_t {});
+            P.N - n0, (int)(P.K * EB / (BKB * KSTEP)), f8_ctx_t {});
 
     store_quadrant<layout32_t, G::WCOLS>(P, smem, ntab, acc, b, m0 + wm * 128, n0 + wn * G::WCOLS, wn * G::WCOLS, cv);
 }
@@ -387,10 +450,86 @@ int f8_launch(const mi355_matmul_desc_t &d, const problem_t &P, void *scratch, h
         return hipGetLastError() == hipSuccess ? MI355_SUCCESS : MI355_RUNTIME_ERROR;
     };
     const int fa = d.src_dt == MI355_DT_F8_E5M2, fb = d.wei_dt == MI355_DT_F8_E5M2;
-    if (fa && fb) return go(f8_gemm_kernel<1, 1, f8_geo_t>);
-    if (fa) return go(f8_gemm_kernel<1, 0, f8_geo_t>);
-    if (fb) return go(f8_gemm_kernel<0, 1, f8_geo_t>);
-    return go(f8_gemm_kernel<0, 0, f8_geo_t>);
+    if (fa && fb) return go(f8_gemm_kernel<f8_mma_t<1, 1, f8_geo_t>>);
+    if (fa) return go(f8_gemm_kernel<f8_mma_t<1, 0, f8_geo_t>>);
+    if (fb) return go(f8_gemm_kernel<f8_mma_t<0, 1, f8_geo_t>>);
+    return go(f8_gemm_kernel<f8_mma_t<0, 0, f8_geo_t>>);
+}
+
+// ---- bf16 / f16
+int h16_supported(const mi355_matmul_desc_t &d) {
+    if (d.src_dt != d.wei_dt || (d.src_dt != MI355_DT_BF16 && d.src_dt != MI355_DT_F16)) return MI355_UNIMPLEMENTED;
+    if (dt_bits(d.dst_dt) < 8) return MI355_UNIMPLEMENTED;
+    constexpr int KE = BKB * KSTEP / 2; // elements of K per stage
+    if (d.K < KE || d.K % KE != 0) return MI355_UNIMPLEMENTED;
+    // 16-byte row pieces: strides in multiples of eight elements
+    if (d.src_stride[2] != 1 || d.src_stride[1] % 8 != 0 || d.src_stride[0] % 8 != 0) return MI355_UNIMPLEMENTED;
+    // K-contiguous weights (what format_tag::any resolves to) are read in place; N-contiguous ones are
+    // transposed into scratch by a pre-pass of every launch
+    const bool k_major = d.wei_stride[1] == 1 && d.wei_stride[2] % 8 == 0 && d.wei_stride[0] % 8 == 0;
+    const bool n_major = d.wei_stride[2] == 1;
+    if (!k_major && !n_major) return MI355_UNIMPLEMENTED;
+    // byte offsets inside a tile are 32-bit
+    const long ldb = k_major ? d.wei_stride[2] : d.K;
+    if (d.src_stride[1] * 2 * BM >= (1L << 31) || ldb * 2 * f8_geo_t::BN >= (1L << 31)) return MI355_UNIMPLEMENTED;
+    if (!quant_absent(d.src_zp) || !quant_absent(d.wei_zp) || !quant_absent(d.src_pr)) return MI355_UNIMPLEMENTED;
+    if (!quant_absent(d.src_scale)
+            && ((d.src_scale.mask & 4) || d.src_scale.group[0] > 1 || d.src_scale.group[1] > 1))
+        return MI355_UNIMPLEMENTED;
+    if (!quant_absent(d.wei_scale)
+            && ((d.wei_scale.mask & 2) || d.wei_scale.group[0] > 1 || d.wei_scale.group[1] > 1))
+        return MI355_UNIMPLEMENTED;
+    if (d.batch > 65535) return MI355_UNIMPLEMENTED;
+    return MI355_SUCCESS;
+}
+
+size_t h16_scratch_bytes(const mi355_matmul_desc_t &d) {
+    const bool k_major = d.wei_stride[1] == 1 && d.wei_stride[2] % 8 == 0 && d.wei_stride[0] % 8 == 0;
+    const long Bw = d.wei_stride[0] ? d.batch : 1;
+    return k_major ? 0 : align_up((size_t)Bw * d.N * d.K * 2, 256);
+}
+
+int h16_launch(const mi355_matmul_desc_t &d, const problem_t &P, void *scratch, hipStream_t stream) {
+    f8_extra_t X {};
+    const size_t need = h16_scratch_bytes(d);
+    if (need > 0) {
+        if (!scratch) {
+            set_error("mfma_h16: %zu bytes of scratch required", need);
+            return MI355_INVALID_ARGUMENTS;
+        }
+        // [Bw][K][N] with N contiguous -> [Bw][N][K] with K contiguous: the reorder's tiled kernel
+        const long Bw = d.wei_stride[0] ? d.batch : 1;
+        mi355_reorder_desc_t rd {};
+        rd.ndims = 3;
+        rd.src_dt = rd.dst_dt = d.wei_dt;
+        rd.dims[0] = Bw; rd.dims[1] = d.K; rd.dims[2] = d.N;
+        rd.src_stride[0] = d.wei_stride[0]; rd.src_stride[1] = d.wei_stride[1]; rd.src_stride[2] = 1;
+        rd.dst_stride[0] = d.N * d.K; rd.dst_stride[1] = 1; rd.dst_stride[2] = d.K;
+        rd.src_scale.group[0] = rd.src_scale.group[1] = rd.dst_scale.group[0] = rd.dst_scale.group[1] = 1;
+        rd.src_zp.group[0] = rd.src_zp.group[1] = rd.dst_zp.group[0] = rd.dst_zp.group[1] = 1;
+        mi355_reorder_args_t ra {};
+        ra.src = P.wei;
+        ra.dst = scratch;
+        if (const int st = mi355_reorder_launch(&rd, &ra, stream)) return st;
+        X.bt = (const char *)scratch;
+        X.ldb = d.K * 2;
+        X.bt_bstride = Bw > 1 ? d.N * d.K * 2 : 0;
+    } else {
+        X.bt = (const char *)P.wei;
+        X.ldb = d.wei_stride[2] * 2;
+        X.bt_bstride = d.wei_stride[0] * 2;
+    }
+    X.tiles_m = (int)((d.M + BM - 1) / BM);
+    X.tiles_n = (int)((d.N + f8_geo_t::BN - 1) / f8_geo_t::BN);
+    dim3 grid((unsigned)(X.tiles_m * X.tiles_n), 1, (unsigned)d.batch);
+    constexpr int smem_bytes = NSTAGE * f8_geo_t::STAGE_BYTES + NTAB_BYTES;
+    auto go = [&](auto kern) -> int {
+        if (const int st = ensure_dynamic_lds((const void *)kern, smem_bytes, "mfma_h16")) return st;
+        hipLaunchKernelGGL(kern, grid, dim3(f8_geo_t::NT), smem_bytes, stream, P, X);
+        return hipGetLastError() == hipSuccess ? MI355_SUCCESS : MI355_RUNTIME_ERROR;
+    };
+    if (d.src_dt == MI355_DT_BF16) return go(f8_gemm_kernel<h16_mma_t<true, f8_geo_t>>);
+    return go(f8_gemm_kernel<h16_mma_t<false, f8_geo_t>>);
 }
 
 } // namespace mi355

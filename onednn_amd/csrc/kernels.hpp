@@ -21,6 +21,10 @@ int f8_supported(const mi355_matmul_desc_t &d);
 size_t f8_scratch_bytes(const mi355_matmul_desc_t &d);
 int f8_launch(const mi355_matmul_desc_t &d, const problem_t &P, void *scratch,
         hipStream_t stream);
+int h16_supported(const mi355_matmul_desc_t &d);
+size_t h16_scratch_bytes(const mi355_matmul_desc_t &d);
+int h16_launch(const mi355_matmul_desc_t &d, const problem_t &P, void *scratch,
+        hipStream_t stream);
 
 int mxf4_supported(const mi355_matmul_desc_t &d);
 size_t mxf4_scratch_bytes(const mi355_matmul_desc_t &d);

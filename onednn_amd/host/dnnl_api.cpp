@@ -763,7 +763,7 @@ dnnl_status_t lower(dnnl_primitive_desc &pd) {
 // implementation list of the HIP engine, best first (the role of
 // engine_t::get_implementation_list, src/common/engine.hpp:134-137)
 const int k_impl_list[] = {MI355_IMPL_WOQ_PACKED, MI355_IMPL_WOQ_GEMV, MI355_IMPL_I8_MFMA, MI355_IMPL_F8_MFMA, MI355_IMPL_MXF4_MFMA,
-        MI355_IMPL_REF};
+        MI355_IMPL_H16_MFMA, MI355_IMPL_REF};
 
 dnnl_status_t select_impl(dnnl_primitive_desc &pd) {
     pd.desc.impl = pd.impls[pd.impl_pos];
@@ -1833,7 +1833,7 @@ DNNL_EXPORT dnnl_status_t dnnl_matmul_primitive_desc_create(dnnl_primitive_desc_
     // format `any`: the implementation picks the layout and the caller asks
     // weights_desc() for it, as with the reference's blocked weights
     // (brgemm_matmul_utils.cpp: set_or_check_B_tag).  The MFMA GEMM families
-    // consume K-contiguous weight columns, so int8 / fp8 / fp4 weights resolve
+    // consume K-contiguous weight columns, so int8 / fp8 / fp4 / bf16 / f16 weights resolve
     // to the plain transposed tag (ba, acb, ...); everything else resolves to
     // row-major (matmul_pd_t::set_default_formats, matmul_pd.hpp:419-431).
     bool try_packed = false;
@@ -1846,7 +1846,8 @@ DNNL_EXPORT dnnl_status_t dnnl_matmul_primitive_desc_create(dnnl_primitive_desc_
         try_packed = pd->src.dt == dnnl_bf16 && (w.dt == dnnl_s4 || w.dt == dnnl_u4) && pd->attr.apply_to_int
                 && w.ndims == 2 && w.dims[1] >= 64 * 128;
         const bool mfma_operands = (is_int8(pd->src.dt) && is_int8(w.dt)) || (is_fp8(pd->src.dt) && is_fp8(w.dt))
-                || (pd->src.dt == dnnl_f4_e2m1 && w.dt == dnnl_f4_e2m1);
+                || (pd->src.dt == dnnl_f4_e2m1 && w.dt == dnnl_f4_e2m1)
+                || (pd->src.dt == w.dt && (w.dt == dnnl_bf16 || w.dt == dnnl_f16));
         if (mfma_operands && w.ndims >= 2) {
             w.strides[w.ndims - 2] = 1;
             w.strides[w.ndims - 1] = w.dims[w.ndims - 2] == 0 ? 1 : w.dims[w.ndims - 2];
