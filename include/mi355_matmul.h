@@ -170,7 +170,7 @@ enum {
     MI355_IMPL_MXF4_MFMA = 4,/* "hip:mfma_mxf4": block-scaled e2m1 MFMA GEMM */
     MI355_IMPL_WOQ_GEMV = 5, /* "hip:woq_gemv": int4/int8 weight-only decode */
     MI355_IMPL_WOQ_PACKED = 6, /* "hip:woq_packed": decode over MI355_WEI_PACK_WOQ64 weights */
-    MI355_IMPL_H16_MFMA = 7, /* "hip:mfma_h16": bf16 x bf16 / f16 x f16 MFMA GEMM, f32 accumulation */
+    MI355_IMPL_H16_MFMA = 7, /* "hip:mfma_h16": bf16 x bf16 / f16 x f16 / f32 x f32 MFMA GEMM, f32 accumulation */
     MI355_IMPL_COUNT = 8
 };
 

@@ -289,15 +289,18 @@ def grouped_bytes(p):
 
 
 def config_h16(M=8192, N=8192, K=8192, dt="bf16", seed=6, impl=cabi.IMPL_AUTO, wtag="ba"):
-    """bf16 x bf16 (or f16 x f16) -> same type, no attributes: the unquantized
+    """bf16 x bf16 (or f16 x f16, f32 x f32) -> same type, no attributes: the unquantized
     matmul next to the quantized configurations (same tiles, 16-bit operands)."""
     sv = _rng(seed, 1).standard_normal((M, K)).astype(np.float32)
     wv = _rng(seed, 2).standard_normal((K, N)).astype(np.float32)
-    if dt == "bf16":
+    if dt == "f32":
+        src, wei = sv, wv
+    elif dt == "bf16":
         src, wei = dtp.f32_to_bf16(sv.reshape(-1)).reshape(M, K), dtp.f32_to_bf16(wv.reshape(-1)).reshape(K, N)
     else:
         src, wei = sv.astype(np.float16).view(np.uint16), wv.astype(np.float16).view(np.uint16)
     if wtag == "ba":
         wei = np.ascontiguousarray(wei.T)
     return MatmulProblem(M=M, N=N, K=K, src_dt=cabi.DT_NAMES[dt], wei_dt=cabi.DT_NAMES[dt], dst_dt=cabi.DT_NAMES[dt],
-                         src=src, wei=wei, wei_stride=strides_for(wtag, 1, K, N), impl=impl, name=f"H1-{dt}")
+                         src=src, wei=wei, wei_stride=strides_for(wtag, 1, K, N), impl=impl,
+                         name=f"{'H2' if dt == 'f32' else 'H1'}-{dt}")

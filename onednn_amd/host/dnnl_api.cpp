@@ -1833,7 +1833,7 @@ DNNL_EXPORT dnnl_status_t dnnl_matmul_primitive_desc_create(dnnl_primitive_desc_
     // format `any`: the implementation picks the layout and the caller asks
     // weights_desc() for it, as with the reference's blocked weights
     // (brgemm_matmul_utils.cpp: set_or_check_B_tag).  The MFMA GEMM families
-    // consume K-contiguous weight columns, so int8 / fp8 / fp4 / bf16 / f16 weights resolve
+    // consume K-contiguous weight columns, so int8 / fp8 / fp4 / bf16 / f16 / f32 weights resolve
     // to the plain transposed tag (ba, acb, ...); everything else resolves to
     // row-major (matmul_pd_t::set_default_formats, matmul_pd.hpp:419-431).
     bool try_packed = false;
@@ -1847,7 +1847,7 @@ DNNL_EXPORT dnnl_status_t dnnl_matmul_primitive_desc_create(dnnl_primitive_desc_
                 && w.ndims == 2 && w.dims[1] >= 64 * 128;
         const bool mfma_operands = (is_int8(pd->src.dt) && is_int8(w.dt)) || (is_fp8(pd->src.dt) && is_fp8(w.dt))
                 || (pd->src.dt == dnnl_f4_e2m1 && w.dt == dnnl_f4_e2m1)
-                || (pd->src.dt == w.dt && (w.dt == dnnl_bf16 || w.dt == dnnl_f16));
+                || (pd->src.dt == w.dt && (w.dt == dnnl_bf16 || w.dt == dnnl_f16 || w.dt == dnnl_f32));
         if (mfma_operands && w.ndims >= 2) {
             w.strides[w.ndims - 2] = 1;
             w.strides[w.ndims - 1] = w.dims[w.ndims - 2] == 0 ? 1 : w.dims[w.ndims - 2];

@@ -204,8 +204,14 @@ def test_format_any_is_resolved_by_the_implementation(eng):
     pd = dnnl.matmul_primitive_desc(eng, md([2, 8, 128], "f8_e4m3"), md([2, 128, 4], "f8_e4m3", tag=dnnl.tag_any),
                                     md([2, 8, 4], "bf16"))
     assert pd.query_md(dnnl.query_weights_md).strides() == [512, 1, 128]
-    # ... and row-major for everything else
-    pd = dnnl.matmul_primitive_desc(eng, md([8, 16], "f32"), md([16, 4], "f32", tag=dnnl.tag_any), md([8, 4], "f32"))
+    # ... for the unquantized float types of the same tiles too ...
+    for dt in ("f32", "bf16", "f16"):
+        pd = dnnl.matmul_primitive_desc(eng, md([8, 16], dt), md([16, 4], dt, tag=dnnl.tag_any), md([8, 4], dt))
+        assert pd.query_md(dnnl.query_weights_md).strides() == [1, 16]
+    # ... and row-major for everything else (here: 8-bit weights that a bf16 src decompresses)
+    wo = _attr(lambda t: t.set_fpmath_mode(dnnl.fpmath_bf16, True))
+    pd = dnnl.matmul_primitive_desc(eng, md([8, 16], "bf16"), md([16, 4], "s8", tag=dnnl.tag_any), md([8, 4], "bf16"),
+                                    attr=wo)
     assert pd.query_md(dnnl.query_weights_md).strides() == [4, 1]
 
 

@@ -1,4 +1,4 @@
-"""hip:mfma_h16 -- bf16 x bf16 and f16 x f16 matmul on the matrix-core tiles
+"""hip:mfma_h16 -- bf16 x bf16, f16 x f16 and f32 x f32 matmul on the matrix-core tiles
 (ref_matmul_t's f32 sum of exact products, src/cpu/matmul/ref_matmul.cpp:168-331).
 
 Dispatch rules need no device.  On the device: data whose every partial sum is
@@ -22,6 +22,8 @@ MASK_COMMON, MASK_ROW, MASK_COL = 0, 2, 4
 
 def enc(v, dt):
     v = np.asarray(v, np.float32)
+    if dt == "f32":
+        return v
     if dt == "bf16":
         return dtp.f32_to_bf16(v.reshape(-1)).reshape(v.shape)
     return v.astype(np.float16).view(np.uint16)
@@ -58,6 +60,8 @@ def test_dispatch_rules():
     assert st == cabi.SUCCESS and impl == cabi.IMPL_H16_MFMA
     assert cabi.impl_name(impl).startswith("hip:mfma_h16")
     assert q(problem(64, 64, 64, "f16", "f16"))[1] == cabi.IMPL_H16_MFMA
+    assert q(problem(64, 64, 16, "f32", "f32"))[1] == cabi.IMPL_H16_MFMA           # f32: stages of 16 k
+    assert q(problem(64, 64, 24, "f32", "f32"))[1] == cabi.IMPL_REF
     assert q(problem(1, 8, 32, "bf16", "bf16"))[1] == cabi.IMPL_H16_MFMA          # any M, N; K in stages of 32
     assert q(problem(64, 64, 48, "bf16", "f32"))[1] == cabi.IMPL_REF              # K not a multiple of 32
     p = problem(64, 64, 64, "bf16", "f32", wtag="ab")                             # row-major weights: a layout pre-pass
@@ -83,7 +87,8 @@ SHAPES = [(256, 256, 64), (300, 200, 96), (1, 8, 32), (33, 515, 160), (512, 768,
 
 @pytest.mark.gpu
 @pytest.mark.parametrize("shape", SHAPES)
-@pytest.mark.parametrize("dt,ddt", [("bf16", "f32"), ("bf16", "bf16"), ("f16", "f16"), ("f16", "f32")])
+@pytest.mark.parametrize("dt,ddt", [("bf16", "f32"), ("bf16", "bf16"), ("f16", "f16"), ("f16", "f32"), ("f32", "f32"),
+                                    ("f32", "bf16")])
 def test_exact_data_bit_exact(gpu, oracle, shape, dt, ddt):
     M, N, K = shape
     # keep |sum| small enough for an exact 16-bit dst: |values| <= 4, K <= 1024 -> |sum| <= 16384 would not be,
@@ -96,7 +101,7 @@ def test_exact_data_bit_exact(gpu, oracle, shape, dt, ddt):
 
 
 @pytest.mark.gpu
-@pytest.mark.parametrize("dt", ["bf16", "f16"])
+@pytest.mark.parametrize("dt", ["bf16", "f16", "f32"])
 def test_exact_data_with_scales_bias_and_post_ops(gpu, oracle, dt):
     M, N, K = 130, 190, 128
     r = np.random.default_rng(5)
@@ -132,7 +137,7 @@ def test_bf16_dst_whole_row_epilogue(gpu, oracle, shape, chain):
 
 
 @pytest.mark.gpu
-@pytest.mark.parametrize("dt", ["bf16", "f16"])
+@pytest.mark.parametrize("dt", ["bf16", "f16", "f32"])
 @pytest.mark.parametrize("shape", [(300, 200, 96), (64, 130, 64), (512, 768, 1024)])
 def test_row_major_weights_take_the_layout_pre_pass(gpu, oracle, dt, shape):
     M, N, K = shape
@@ -153,13 +158,15 @@ def test_batched_exact(gpu, oracle, wei_batch, wtag):
 
 
 @pytest.mark.gpu
-@pytest.mark.parametrize("dt,ddt", [("bf16", "f32"), ("bf16", "bf16"), ("f16", "f32")])
+@pytest.mark.parametrize("dt,ddt", [("bf16", "f32"), ("bf16", "bf16"), ("f16", "f32"), ("f32", "f32")])
 def test_random_data_within_the_f32_sum_bound(gpu, oracle, dt, ddt):
     p = problem(320, 448, 2048, dt, ddt, exact=False, seed=8, bias=True)
     got, name = run_gpu(p)
     assert name.startswith("hip:mfma_h16"), name
     _, ideal, asum = oracle.run_oracle(p, want_ideal=True)
-    assert_gemm_close(p, got, ideal, asum, what=name)
+    # products of two f32 values round once each (2^-24 relative) before they are added; those of 16-bit values are exact
+    hw = np.asarray(asum, np.float64).reshape(p.M, p.N) * 2.0 ** -24 if dt == "f32" else None
+    assert_gemm_close(p, got, ideal, asum, what=name, hw=hw)
 
 
 @pytest.mark.gpu
