@@ -22,6 +22,7 @@ Workloads (the benchmark configurations):
   c2  bf16 x u4 -> bf16 decode, K=4096 N=14336, M in {1,8,32} (HBM bound)
   c4  e4m3 x e4m3 -> bf16, 4096 x 8192 x 28672, bias+gelu+add (MFMA fp8 bound)
   c5  MXFP4, M=N=K=8192 (MFMA fp4 bound)
+  m1  MXFP8 (e4m3, e8m0 scales per 32 k on both operands), M=N=K=8192 (MFMA fp8 bound)
   h1  bf16 x bf16 -> bf16, M=N=K=8192 (MFMA bf16 bound; the unquantized matmul on the same tiles)
   h2  f32 x f32 -> f32, M=N=K=8192 (MFMA f32 bound)
   c1  u8 x s8 -> f32, 256 x 1024 x 1024 (latency bound, no roofline claim)
@@ -47,6 +48,7 @@ PROFILE_OF = {
     ("c3", "any"): "i8_gemm_kernel_c3_8192.md", ("c4", "any"): "f8_gemm_kernel_c4_4096x8192x28672.md",
     ("c5", "any"): "mxf4_gemm_kernel_c5_8192.md", ("c1", "any"): "i8_small_kernel_c1_256x1024x1024.md",
     ("h1", "any"): "f8_gemm_kernel_h1_bf16_8192.md", ("h2", "any"): "f8_gemm_kernel_h2_f32_8192.md",
+    ("m1", "any"): "mxf8_gemm_kernel_m1_mxfp8_8192.md",
     ("c2", "any", 1): "woqp_kernel_c2_m1.md", ("c2", "any", 8): "woqp_kernel_c2_m8.md",
     ("c2", "any", 32): "woqp_kernel_c2_m32.md", ("c2", "ab", 1): "woq_gemv_kernel_c2_m1_plain_ab.md",
     ("c2", "ab", 8): "woq_gemv_kernel_c2_m8_plain_ab.md", ("c2", "ab", 32): "woq_gemv_kernel_c2_m32_plain_ab.md",
@@ -145,6 +147,8 @@ def build_problem(name, M=None, wtag="any"):
         return configs.config_h16(wtag=mfma_tag)
     if name == "h2":
         return configs.config_h16(dt="f32", wtag=mfma_tag)
+    if name == "m1":
+        return configs.config_mxf8(wtag=mfma_tag)
     raise ValueError(name)
 
 
@@ -156,7 +160,7 @@ def algorithmic(name, p):
         return configs.config2_bytes(p.M, p.N, p.K), "GB/s", "hbm", PEAK_HBM_GBS
     if name == "c3":
         return ops, "TOPS", "mfma", PEAK_I8_TOPS
-    if name in ("c4", "c4mx"):
+    if name in ("c4", "c4mx", "m1"):
         return ops, "TFLOP/s", "mfma", PEAK_F8_TFLOPS
     if name == "c5":
         return ops, "TFLOP/s", "mfma", PEAK_F4_TFLOPS
@@ -374,6 +378,9 @@ def cpu_baseline(name, M=None):
     elif name == "c5":
         p = configs.config5(M=128, N=1024, K=8192)
         sample = "M=128, N=1024, K=8192 slice of the 8192^3 shape"
+    elif name == "m1":
+        p = configs.config_mxf8(M=128, N=1024, K=8192)
+        sample = "M=128, N=1024, K=8192 slice of the 8192^3 shape"
     elif name in ("h1", "h2"):
         p = configs.config_h16(M=128, N=1024, K=8192, dt="f32" if name == "h2" else "bf16")
         sample = "M=128, N=1024, K=8192 slice of the 8192^3 shape"
@@ -395,7 +402,8 @@ def cpu_baseline(name, M=None):
     probe = {"c3": "4.97 TOPS (221 ms)", "c1": "6.37 TOPS (0.084 ms)",
              "c2": {1: "4.17 GB/s (7.05 ms)", 8: "4.64 GB/s (6.39 ms)", 32: "3.16 GB/s (9.67 ms)"}.get(M or 1),
              "c4": "no JIT implementation on that host (ref:any only)", "c5": "no CPU implementation (skipped)",
-             "h1": "not measured", "h2": "not measured"}[name]
+             "h1": "not measured", "h2": "not measured",
+             "m1": "no CPU implementation (skipped)"}[name]
     return {"value": rate(work * reps, dt * 1e3, unit), "unit": unit, "cores": threads, "kind": "port",
             "reference_probe": {"what": "benchdnn --matmul --mode=P on the reference built with its own CMake, "
                                         "impl brg_matmul:avx10_1_512_amx, this configuration at full size",
@@ -411,7 +419,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=3)
-    ap.add_argument("--workload", default="c3", choices=["c1", "c2", "c3", "c4", "c5", "h1", "h2", "r1", "r2", "r3", "g1", "g2", "g3", "g4", "g5"],
+    ap.add_argument("--workload", default="c3", choices=["c1", "c2", "c3", "c4", "c5", "m1", "h1", "h2", "r1", "r2", "r3", "g1", "g2", "g3", "g4", "g5"],
                     help="c1..c5: the matmul configurations (c3 is the headline); r1..r3: the reorder "
                          "primitive on the headline shape's tensors; g1..g5: the grouped (mixture-of-experts) "
                          "matmul on shapes of the reference's shapes_grouped_moe files: fp8 with row / column scales "
@@ -599,7 +607,7 @@ def main():
         # layout change then runs inside every launch
         plan = [("c2", 1, "any"), ("c2", 8, "any"), ("c2", 32, "any"), ("c3", None, "any"), ("c3", None, "ab"),
                 ("c4", None, "any"), ("c4mx", None, "any"), ("c5", None, "any"), ("c1", None, "any"),
-                ("h1", None, "any"), ("h2", None, "any")]
+                ("m1", None, "any"), ("h1", None, "any"), ("h2", None, "any")]
         for nm, m, wt in plan:
             if nm == main_name and wt == args.wtag and (nm != "c2" or m == args.decode_m):
                 continue
@@ -635,8 +643,9 @@ def main():
 
     metric = {"c3": "int8 matmul TOPS @8192^3", "c2": "int4 weight-only decode GB/s",
               "c4": "fp8 matmul TFLOP/s @4096x8192x28672", "c5": "MXFP4 matmul TFLOP/s @8192^3",
-              "c1": "int8 matmul TOPS @256x1024x1024", "h1": "bf16 matmul TFLOP/s @8192^3", "h2": "f32 matmul TFLOP/s @8192^3"}[main_name]
-    dtype = {"c3": "s8", "c2": "bf16", "c4": "f8_e4m3", "c5": "f4_e2m1", "c1": "u8", "h1": "bf16", "h2": "f32"}[main_name]
+              "c1": "int8 matmul TOPS @256x1024x1024", "h1": "bf16 matmul TFLOP/s @8192^3", "h2": "f32 matmul TFLOP/s @8192^3",
+              "m1": "MXFP8 matmul TFLOP/s @8192^3"}[main_name]
+    dtype = {"c3": "s8", "c2": "bf16", "c4": "f8_e4m3", "c5": "f4_e2m1", "c1": "u8", "h1": "bf16", "h2": "f32", "m1": "f8_e4m3"}[main_name]
     line = {
         "metric": metric, "value": res["value"], "unit": res["unit"], "n_gpus": 1,
         "steps": args.steps, "warmup": args.warmup, "ms_per_step": res["ms_per_step"],

@@ -201,6 +201,43 @@ def config5(M=8192, N=8192, K=8192, seed=5, impl=cabi.IMPL_AUTO, wtag="ba"):
                          wei_stride=strides_for(wtag, 1, K, N), quant=quant, impl=impl, name="C5")
 
 
+def mx_quantize_f8(x, axis):
+    """Block-quantize to f8_e4m3 in blocks of 32 along `axis` the OCP-MX way (the rule of the reference's tutorial
+    examples/tutorials/matmul/mxfp_matmul.cpp:155-162): scale = 2^(floor(log2 amax) - 8), 8 = the largest exponent
+    of e4m3; returns (codes, scale bytes), the scale axis last."""
+    x = np.asarray(x, dtype=np.float32)
+    xm = np.moveaxis(x, axis, -1)
+    shp = xm.shape
+    blk = xm.reshape(shp[:-1] + (shp[-1] // 32, 32))
+    amax = np.max(np.abs(blk), axis=-1)
+    with np.errstate(divide="ignore"):
+        e = np.floor(np.log2(amax)) - 8
+    e = np.where(amax > 0, e, -127.0)
+    sb = np.clip(e + 127, 0, 254).astype(np.int32)
+    scale = np.ldexp(np.float32(1.0), sb - 127).astype(np.float32)
+    q = dtp.f32_to_e4m3(np.clip(blk / scale[..., None], -448, 448).astype(np.float32).reshape(-1)).reshape(shp)
+    return np.moveaxis(q, -1, axis), sb.astype(np.uint8)
+
+
+def config_mxf8(M=8192, N=8192, K=8192, seed=7, impl=cabi.IMPL_AUTO, wtag="ba"):
+    """MXFP8: e4m3 x e4m3 -> bf16 with e8m0 scales per block of 32 along K on both operands (the dense sibling of
+    the grouped MXFP8 workload; weights K-contiguous by default)."""
+    xs = _rng(seed, 1).standard_normal((M, K), dtype=np.float32)
+    src, s_sb = mx_quantize_f8(xs, axis=1)            # scales [M][K/32]
+    del xs
+    xw = _rng(seed, 2).standard_normal((K, N), dtype=np.float32)
+    w_codes, w_sbT = mx_quantize_f8(xw, axis=0)        # [K][N] codes, scales [N][K/32]
+    del xw
+    w_sb = np.ascontiguousarray(w_sbT.T)               # layout [K/32][N]
+    wei = np.ascontiguousarray(w_codes.T) if wtag == "ba" else w_codes
+    quant = {
+        "src_scale": QuantParam(cabi.DT_E8M0, MASK_ROW | MASK_COL, s_sb, (1, 32)),
+        "wei_scale": QuantParam(cabi.DT_E8M0, MASK_ROW | MASK_COL, w_sb, (32, 1)),
+    }
+    return MatmulProblem(M=M, N=N, K=K, src_dt=cabi.DT_F8_E4M3, wei_dt=cabi.DT_F8_E4M3, dst_dt=cabi.DT_BF16,
+                         src=src, wei=wei, wei_stride=strides_for(wtag, 1, K, N), quant=quant, impl=impl, name="M1-mxfp8")
+
+
 # algorithmic work per configuration
 def config_ops(p):
     return 2 * p.batch * p.M * p.N * p.K
