@@ -1,0 +1,190 @@
+// "hip:mfma_h16" -- the same tiles for bf16 x bf16, f16 x f16 and f32 x f32 operands
+// (ref_matmul_t's f32 sum of exact products): a 64-byte stage is 32 elements of
+// K, two v_mfma_f32_32x32x16_{bf16,f16} per fragment pair in the time of the
+// one fp8 instruction, so the data path (DMA, LDS ring, fragment reads,
+// epilogue) is shared unchanged; a lane's two 16-byte chunks of a stage feed
+// the two instructions, the same chunks for both operands, so the order in
+// which the 32 k of a stage meet does not matter.
+#include "f8_family.hpp"
+
+namespace mi355 {
+namespace {
+
+typedef __bf16 v8bf_t __attribute__((ext_vector_type(8)));
+typedef _Float16 v8h_t __attribute__((ext_vector_type(8)));
+
+// bf16 (BF16) or f16 operands: the fp8 policy's addresses and reads; a fragment
+// is its two 16-byte chunks, each the operand of one 32x32x16 instruction
+template <bool BF16, class G_>
+struct h16_mma_t {
+    using G = G_;
+    static constexpr int ELEM_BYTES = 2;
+    static constexpr bool HOT = BF16; // the whole-row bf16 epilogue chains of the fp8 family
+    static constexpr int EXTRA_DMAS = 0;
+    __device__ static __forceinline__ void issue_extra(const f8_ctx_t &, int, int, int, int) {}
+    static constexpr int ROWS = 4, COLS = G::WCOLS / 32, A_READS = 2, B_READS = 2;
+    struct frag_t {
+        v4i a[ROWS][2], b[COLS][2];
+    };
+    __device__ static __forceinline__ frag_t zero_frag() { return frag_t {}; }
+    using addr_t = typename f8_mma_t<0, 0, G_>::addr_t;
+    __device__ static __forceinline__ addr_t lane_addr(int wm, int wn, int lane) {
+        return f8_mma_t<0, 0, G_>::lane_addr(wm, wn, lane);
+    }
+    __device__ static __forceinline__ void load_b(frag_t &f, const unsigned (&S)[1], const addr_t &ad,
+            const f8_ctx_t &, int) {
+#pragma unroll
+        for (int j = 0; j < COLS; ++j) {
+            f.b[j][0] = lds_read16(S[0] + ad.b0 + j * 2048);
+            f.b[j][1] = lds_read16(S[0] + ad.b1 + j * 2048);
+        }
+    }
+    __device__ static __forceinline__ void load_a(frag_t &f, int i, const unsigned (&S)[1], const addr_t &ad,
+            const f8_ctx_t &, int) {
+        f.a[i][0] = lds_read16(S[0] + ad.a0 + i * 2048);
+        f.a[i][1] = lds_read16(S[0] + ad.a1 + i * 2048);
+    }
+    __device__ static __forceinline__ void mma_row(v16f (&acc)[ROWS][COLS], const frag_t &f, int i,
+            const f8_ctx_t &, int) {
+#pragma unroll
+        for (int h = 0; h < 2; ++h)
+#pragma unroll
+            for (int j = 0; j < COLS; ++j) {
+                // operands exchanged, as in the fp8 policy: the tile comes out transposed
+                if constexpr (BF16)
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(v8bf_t, f.b[j][h]),
+                            __builtin_bit_cast(v8bf_t, f.a[i][h]), acc[i][j], 0, 0, 0);
+                else
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(v8h_t, f.b[j][h]),
+                            __builtin_bit_cast(v8h_t, f.a[i][h]), acc[i][j], 0, 0, 0);
+            }
+    }
+};
+
+// f32 x f32: a 64-byte stage is 16 elements of K, eight v_mfma_f32_32x32x2_f32 per
+// fragment pair (instruction t takes dword t of the lane's eight: k = t from the
+// lower half of the lanes, k = 8 + t from the upper one, on both operands alike).
+// Eight times the matrix-core cycles of the other policies per stage: this one
+// is bound by the f32 instruction's own rate (157 TFLOP/s), not by the data path.
+template <class G_>
+struct f32_mma_t {
+    using G = G_;
+    static constexpr int ELEM_BYTES = 4;
+    static constexpr bool HOT = false;
+    static constexpr int EXTRA_DMAS = 0;
+    __device__ static __forceinline__ void issue_extra(const f8_ctx_t &, int, int, int, int) {}
+    static constexpr int ROWS = 4, COLS = G::WCOLS / 32, A_READS = 2, B_READS = 2;
+    struct frag_t {
+        v8i a[ROWS], b[COLS];
+    };
+    __device__ static __forceinline__ frag_t zero_frag() { return frag_t {}; }
+    using base_t = f8_mma_t<0, 0, G_>;
+    using addr_t = typename base_t::addr_t;
+    __device__ static __forceinline__ addr_t lane_addr(int wm, int wn, int lane) { return base_t::lane_addr(wm, wn, lane); }
+    __device__ static __forceinline__ void load_b(frag_t &f, const unsigned (&S)[1], const addr_t &ad,
+            const f8_ctx_t &, int) {
+#pragma unroll
+        for (int j = 0; j < COLS; ++j) f.b[j] = base_t::read32(S[0] + ad.b0 + j * 2048, S[0] + ad.b1 + j * 2048);
+    }
+    __device__ static __forceinline__ void load_a(frag_t &f, int i, const unsigned (&S)[1], const addr_t &ad,
+            const f8_ctx_t &, int) {
+        f.a[i] = base_t::read32(S[0] + ad.a0 + i * 2048, S[0] + ad.a1 + i * 2048);
+    }
+    __device__ static __forceinline__ void mma_row(v16f (&acc)[ROWS][COLS], const frag_t &f, int i,
+            const f8_ctx_t &, int) {
+#pragma unroll
+        for (int t = 0; t < 8; ++t)
+#pragma unroll
+            for (int j = 0; j < COLS; ++j)
+                acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(__int_as_float(f.b[j][t]), __int_as_float(f.a[i][t]),
+                        acc[i][j], 0, 0, 0);
+    }
+};
+
+} // namespace
+
+// ---- bf16 / f16 / f32
+static bool h16_k_major(const mi355_matmul_desc_t &d) {
+    const int AL = 16 / (dt_bits(d.src_dt) / 8);
+    return d.wei_stride[1] == 1 && d.wei_stride[2] % AL == 0 && d.wei_stride[0] % AL == 0;
+}
+
+int h16_supported(const mi355_matmul_desc_t &d) {
+    if (d.src_dt != d.wei_dt || (d.src_dt != MI355_DT_BF16 && d.src_dt != MI355_DT_F16 && d.src_dt != MI355_DT_F32))
+        return MI355_UNIMPLEMENTED;
+    if (dt_bits(d.dst_dt) < 8) return MI355_UNIMPLEMENTED;
+    const int EB = dt_bits(d.src_dt) / 8;   // bytes per element
+    const int KE = BKB * KSTEP / EB, AL = 16 / EB; // elements of K per stage; elements per 16 bytes
+    if (d.K < KE || d.K % KE != 0) return MI355_UNIMPLEMENTED;
+    // 16-byte row pieces
+    if (d.src_stride[2] != 1 || d.src_stride[1] % AL != 0 || d.src_stride[0] % AL != 0) return MI355_UNIMPLEMENTED;
+    // K-contiguous weights (what format_tag::any resolves to) are read in place; N-contiguous ones are
+    // transposed into scratch by a pre-pass of every launch
+    const bool k_major = h16_k_major(d);
+    const bool n_major = d.wei_stride[2] == 1;
+    if (!k_major && !n_major) return MI355_UNIMPLEMENTED;
+    // byte offsets inside a tile are 32-bit
+    const long ldb = k_major ? d.wei_stride[2] : d.K;
+    if (d.src_stride[1] * EB * BM >= (1L << 31) || ldb * EB * f8_geo_t::BN >= (1L << 31)) return MI355_UNIMPLEMENTED;
+    if (!quant_absent(d.src_zp) || !quant_absent(d.wei_zp) || !quant_absent(d.src_pr)) return MI355_UNIMPLEMENTED;
+    if (!quant_absent(d.src_scale)
+            && ((d.src_scale.mask & 4) || d.src_scale.group[0] > 1 || d.src_scale.group[1] > 1))
+        return MI355_UNIMPLEMENTED;
+    if (!quant_absent(d.wei_scale)
+            && ((d.wei_scale.mask & 2) || d.wei_scale.group[0] > 1 || d.wei_scale.group[1] > 1))
+        return MI355_UNIMPLEMENTED;
+    if (d.batch > 65535) return MI355_UNIMPLEMENTED;
+    return MI355_SUCCESS;
+}
+
+size_t h16_scratch_bytes(const mi355_matmul_desc_t &d) {
+    const long Bw = d.wei_stride[0] ? d.batch : 1;
+    return h16_k_major(d) ? 0 : align_up((size_t)Bw * d.N * d.K * (dt_bits(d.src_dt) / 8), 256);
+}
+
+int h16_launch(const mi355_matmul_desc_t &d, const problem_t &P, void *scratch, hipStream_t stream) {
+    f8_extra_t X {};
+    const long EB = dt_bits(d.src_dt) / 8;
+    const size_t need = h16_scratch_bytes(d);
+    if (need > 0) {
+        if (!scratch) {
+            set_error("mfma_h16: %zu bytes of scratch required", need);
+            return MI355_INVALID_ARGUMENTS;
+        }
+        // [Bw][K][N] with N contiguous -> [Bw][N][K] with K contiguous: the reorder's tiled kernel
+        const long Bw = d.wei_stride[0] ? d.batch : 1;
+        mi355_reorder_desc_t rd {};
+        rd.ndims = 3;
+        rd.src_dt = rd.dst_dt = d.wei_dt;
+        rd.dims[0] = Bw; rd.dims[1] = d.K; rd.dims[2] = d.N;
+        rd.src_stride[0] = d.wei_stride[0]; rd.src_stride[1] = d.wei_stride[1]; rd.src_stride[2] = 1;
+        rd.dst_stride[0] = d.N * d.K; rd.dst_stride[1] = 1; rd.dst_stride[2] = d.K;
+        rd.src_scale.group[0] = rd.src_scale.group[1] = rd.dst_scale.group[0] = rd.dst_scale.group[1] = 1;
+        rd.src_zp.group[0] = rd.src_zp.group[1] = rd.dst_zp.group[0] = rd.dst_zp.group[1] = 1;
+        mi355_reorder_args_t ra {};
+        ra.src = P.wei;
+        ra.dst = scratch;
+        if (const int st = mi355_reorder_launch(&rd, &ra, stream)) return st;
+        X.bt = (const char *)scratch;
+        X.ldb = d.K * EB;
+        X.bt_bstride = Bw > 1 ? d.N * d.K * EB : 0;
+    } else {
+        X.bt = (const char *)P.wei;
+        X.ldb = d.wei_stride[2] * EB;
+        X.bt_bstride = d.wei_stride[0] * EB;
+    }
+    X.tiles_m = (int)((d.M + BM - 1) / BM);
+    X.tiles_n = (int)((d.N + f8_geo_t::BN - 1) / f8_geo_t::BN);
+    dim3 grid((unsigned)(X.tiles_m * X.tiles_n), 1, (unsigned)d.batch);
+    constexpr int smem_bytes = NSTAGE * f8_geo_t::STAGE_BYTES + NTAB_BYTES;
+    auto go = [&](auto kern) -> int {
+        if (const int st = ensure_dynamic_lds((const void *)kern, smem_bytes, "mfma_h16")) return st;
+        hipLaunchKernelGGL(kern, grid, dim3(f8_geo_t::NT), smem_bytes, stream, P, X);
+        return hipGetLastError() == hipSuccess ? MI355_SUCCESS : MI355_RUNTIME_ERROR;
+    };
+    if (d.src_dt == MI355_DT_BF16) return go(f8_gemm_kernel<h16_mma_t<true, f8_geo_t>>);
+    if (d.src_dt == MI355_DT_F32) return go(f8_gemm_kernel<f32_mma_t<f8_geo_t>>);
+    return go(f8_gemm_kernel<h16_mma_t<false, f8_geo_t>>);
+}
+
+} // namespace mi355
