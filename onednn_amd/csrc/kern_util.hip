@@ -70,12 +70,59 @@ __global__ void __launch_bounds__(256) transpose_bytes_tiles_kernel(const uint8_
     *(uint4 *)(out + (c0 + wc) * ld_out + r0 + 16 * wq) = v;
 }
 
+// ... and for whole 128 x 128 tiles with 16-byte aligned rows: a thread loads
+// 4 rows x 16 bytes, so every load instruction fetches the whole 128-byte lines
+// of eight rows and every store instruction writes those of eight output rows
+// (with 64-byte tile rows each input line is fetched by two workgroups, on
+// different L2s); dword column c of tile row r sits at (c + 8 (r / 16)) % 32:
+// conflict-free stores, aligned 16-byte reads.  Output written once, input read
+// once: non-temporal both ways.
+__global__ void __launch_bounds__(256) transpose_bytes_tiles128_kernel(const uint8_t *in, long ld_in, long in_bstride,
+        uint8_t *out, long ld_out, long out_bstride) {
+    typedef uint32_t u4v __attribute__((ext_vector_type(4)));
+    __shared__ __attribute__((aligned(16))) uint32_t tile[128 * 32];
+    in += blockIdx.z * in_bstride;
+    out += blockIdx.z * out_bstride;
+    const long r0 = (long)blockIdx.y * 128, c0 = (long)blockIdx.x * 128;
+    const int ci = threadIdx.x & 7, rg = threadIdx.x >> 3; // read: rows 4 rg .. +3, bytes 16 ci .. +15
+    const int wq = threadIdx.x & 7, wr = threadIdx.x >> 3; // write: output row wr + 32 pass, bytes 16 wq .. +15
+    const uint8_t *p = in + (r0 + 4 * rg) * ld_in + c0 + 16 * ci;
+    u4v q[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) q[i] = __builtin_nontemporal_load((const u4v *)(p + i * ld_in));
+    const int col = (rg + 8 * (ci & 3)) & 31;
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+        const uint32_t q0 = q[0][k], q1 = q[1][k], q2 = q[2][k], q3 = q[3][k];
+        // byte j of q_i is element (r + i, c + 4 k + j); the results collect byte j of the four rows
+        const uint32_t x0 = __builtin_amdgcn_perm(q1, q0, 0x05010400u), x1 = __builtin_amdgcn_perm(q1, q0, 0x07030602u);
+        const uint32_t y0 = __builtin_amdgcn_perm(q3, q2, 0x05010400u), y1 = __builtin_amdgcn_perm(q3, q2, 0x07030602u);
+        const int row = 16 * ci + 4 * k;
+        tile[(row + 0) * 32 + col] = __builtin_amdgcn_perm(y0, x0, 0x05040100u);
+        tile[(row + 1) * 32 + col] = __builtin_amdgcn_perm(y0, x0, 0x07060302u);
+        tile[(row + 2) * 32 + col] = __builtin_amdgcn_perm(y1, x1, 0x05040100u);
+        tile[(row + 3) * 32 + col] = __builtin_amdgcn_perm(y1, x1, 0x07060302u);
+    }
+    __syncthreads();
+#pragma unroll
+    for (int pass = 0; pass < 4; ++pass) {
+        const int c = wr + 32 * pass;
+        const u4v v = *(const u4v *)&tile[c * 32 + ((4 * wq + 8 * ((c >> 4) & 3)) & 31)];
+        __builtin_nontemporal_store(v, (u4v *)(out + (c0 + c) * ld_out + r0 + 16 * wq));
+    }
+}
+
 void transpose_bytes(const void *in, long R, long C, long ld_in, long in_bstride, void *out,
         long ld_out, long out_bstride, long batches, hipStream_t stream) {
     dim3 grid((unsigned)((C + 63) / 64), (unsigned)((R + 63) / 64), (unsigned)batches);
     const bool whole = R % 64 == 0 && C % 64 == 0 && ld_in % 4 == 0 && in_bstride % 4 == 0 && ld_out % 16 == 0
             && out_bstride % 16 == 0 && (uintptr_t)in % 4 == 0 && (uintptr_t)out % 16 == 0;
-    if (whole)
+    const bool whole128 = whole && R % 128 == 0 && C % 128 == 0 && ld_in % 16 == 0 && in_bstride % 16 == 0
+            && (uintptr_t)in % 16 == 0;
+    if (whole128)
+        hipLaunchKernelGGL(transpose_bytes_tiles128_kernel, dim3((unsigned)(C / 128), (unsigned)(R / 128), (unsigned)batches),
+                dim3(256), 0, stream, (const uint8_t *)in, ld_in, in_bstride, (uint8_t *)out, ld_out, out_bstride);
+    else if (whole)
         hipLaunchKernelGGL(transpose_bytes_tiles_kernel, grid, dim3(256), 0, stream, (const uint8_t *)in, ld_in,
                 in_bstride, (uint8_t *)out, ld_out, out_bstride);
     else
