@@ -339,8 +339,81 @@ __global__ void __launch_bounds__(NWV * 64)
         }
     };
 
+    // Two tiles of rows: a wavefront has two super-steps or more, and with one in flight at a time the memory
+    // pipeline drains while each is multiplied.  Units of half a super-step instead, the next one requested
+    // before the current one is multiplied: the same registers hold loads in flight all the time.
+    constexpr int U = SS / 2;                           // steps per unit
+    constexpr bool PIPE = MT == 2 && U % 2 == 0 && (SPG == 0 || U % (SPG ? SPG : 1) == 0);
+    constexpr int NGU = SPG ? (U / (SPG ? SPG : 1) > 0 ? U / (SPG ? SPG : 1) : 1) : 1;
+    struct unit_t {
+        v4u a[U / 2 > 0 ? U / 2 : 1][MT][2], w[U > 0 ? U : 1];
+        unsigned raw_s[NGU], raw_z[NGU];
+    };
+    auto issue_unit = [&](unit_t &u, int kbu) __attribute__((always_inline)) {
+        const int g0 = SPG ? kbu / (SPG ? SPG : 1) : kbu / X.spg;
+#pragma unroll
+        for (int gi = 0; gi < NGU; ++gi) fetch_params(u.raw_s[gi], u.raw_z[gi], g0 + gi);
+#pragma unroll
+        for (int p = 0; p < U / 2; ++p)
+#pragma unroll
+            for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+                for (int h = 0; h < 2; ++h)
+                    u.a[p][mt][h] = *(const v4u *)(X.src + (long)(kbu + 2 * p) * (KBLK * 2) + src_row_off[mt][h]);
+#pragma unroll
+        for (int i = 0; i < U; ++i)
+            u.w[i] = __builtin_nontemporal_load((const v4u *)(wlane + (long)(kbu + i) * (KBLK * CHUNK / 2)));
+    };
+    auto consume_unit = [&](unit_t &u, int kbu) __attribute__((always_inline)) {
+#pragma unroll
+        for (int p = 0; p < U / 2; ++p) {
+            v4u as[2][MT];
+#pragma unroll
+            for (int mt = 0; mt < MT; ++mt) {
+#pragma unroll
+                for (int h = 0; h < 2; ++h) stage[mt * 128 + wr_idx[h]] = u.a[p][mt][h];
+            }
+#pragma unroll
+            for (int sx = 0; sx < 2; ++sx)
+#pragma unroll
+                for (int mt = 0; mt < MT; ++mt) as[sx][mt] = stage[mt * 128 + rd_idx[sx]];
+#pragma unroll
+            for (int sx = 0; sx < 2; ++sx) {
+                const int i = 2 * p + sx;
+                compute_step(u.w[i], as[sx], SPG != 0 && i % (SPG ? SPG : 1) == 0);
+                if constexpr (SPG != 0) {
+                    if ((i + 1) % SPG == 0) flush_group(u.raw_s[i / SPG], u.raw_z[i / SPG], false);
+                }
+            }
+        }
+        if constexpr (SPG == 0) {
+            if ((kbu + U) % X.spg == 0 || kbu + U >= kb1) flush_group(u.raw_s[0], u.raw_z[0], true);
+        }
+    };
+
     int kb = kb0;
-    for (; kb + SS <= kb1; kb += SS) super_step(kb);
+    if constexpr (PIPE) {
+        if (kb + U <= kb1) {
+            unit_t ua, ub;
+            issue_unit(ua, kb);
+            while (true) {
+                const bool more_b = kb + 2 * U <= kb1;
+                if (more_b) issue_unit(ub, kb + U);
+                __builtin_amdgcn_sched_barrier(0);
+                consume_unit(ua, kb);
+                kb += U;
+                if (!more_b) break;
+                const bool more_a = kb + 2 * U <= kb1;
+                if (more_a) issue_unit(ua, kb + U);
+                __builtin_amdgcn_sched_barrier(0);
+                consume_unit(ub, kb);
+                kb += U;
+                if (!more_a) break;
+            }
+        }
+    } else {
+        for (; kb + SS <= kb1; kb += SS) super_step(kb);
+    }
     if (kb < kb1) {
         // ragged end of K: one step at a time, parameters fetched when the
         // group ends
