@@ -254,7 +254,8 @@ typedef struct mi355_matmul_desc {
     mi355_quant_t src_zp, wei_zp, dst_zp;
     mi355_quant_t src_pr; /* precomputed reductions over K of src */
     int32_t fpmath_apply_to_int; /* weight decompression switch */
-    int32_t fpmath_mode;         /* dnnl_fpmath_mode_t value, informational */
+    int32_t fpmath_mode;         /* dnnl_fpmath_mode_t value: bf16 (1), f16 (2) or any (3) let "hip:mfma_h16"
+                                    convert f32 operands to bf16 / f16 / bf16 before it multiplies them */
     int32_t dst_scale_mode;      /* MI355_DST_SCALE_* */
     int32_t n_post_ops;
     mi355_post_op_t post_ops[MI355_MAX_POST_OPS];

@@ -109,10 +109,35 @@ static bool h16_k_major(const mi355_matmul_desc_t &d) {
     return d.wei_stride[1] == 1 && d.wei_stride[2] % AL == 0 && d.wei_stride[0] % AL == 0;
 }
 
+// f32 operands under fpmath_mode bf16 / f16 / any (dnnl_fpmath_mode_t 1 / 2 / 3): the attribute allows an implicit
+// down-conversion (doc/programming_model/attributes_fpmath_mode.md), so both operands are converted into scratch by
+// two reorder launches -- the weights into the K-contiguous layout on the way -- and the 16-bit policy multiplies
+// them: eight times the matrix-core rate of the f32 instruction.  0 = no down-conversion.
+static int h16_down_dt(const mi355_matmul_desc_t &d) {
+    if (d.src_dt != MI355_DT_F32 || d.wei_dt != MI355_DT_F32) return 0;
+    if (d.fpmath_mode == 1 || d.fpmath_mode == 3) return MI355_DT_BF16;
+    if (d.fpmath_mode == 2) return MI355_DT_F16;
+    return 0;
+}
+
 int h16_supported(const mi355_matmul_desc_t &d) {
     if (d.src_dt != d.wei_dt || (d.src_dt != MI355_DT_BF16 && d.src_dt != MI355_DT_F16 && d.src_dt != MI355_DT_F32))
         return MI355_UNIMPLEMENTED;
     if (dt_bits(d.dst_dt) < 8) return MI355_UNIMPLEMENTED;
+    if (!quant_absent(d.src_zp) || !quant_absent(d.wei_zp) || !quant_absent(d.src_pr)) return MI355_UNIMPLEMENTED;
+    if (!quant_absent(d.src_scale)
+            && ((d.src_scale.mask & 4) || d.src_scale.group[0] > 1 || d.src_scale.group[1] > 1))
+        return MI355_UNIMPLEMENTED;
+    if (!quant_absent(d.wei_scale)
+            && ((d.wei_scale.mask & 2) || d.wei_scale.group[0] > 1 || d.wei_scale.group[1] > 1))
+        return MI355_UNIMPLEMENTED;
+    if (d.batch > 65535) return MI355_UNIMPLEMENTED;
+    if (h16_down_dt(d) && d.K >= 32 && d.K % 32 == 0 && d.M * d.K * 2 < (1L << 31) && d.K * 2 * f8_geo_t::BN < (1L << 31)) {
+        // the converted copies are dense: any strides the reorder takes
+        const bool src_ok = d.src_stride[2] == 1 || d.src_stride[1] == 1;
+        const bool wei_ok = d.wei_stride[2] == 1 || d.wei_stride[1] == 1;
+        if (src_ok && wei_ok) return MI355_SUCCESS;
+    }
     const int EB = dt_bits(d.src_dt) / 8;   // bytes per element
     const int KE = BKB * KSTEP / EB, AL = 16 / EB; // elements of K per stage; elements per 16 bytes
     if (d.K < KE || d.K % KE != 0) return MI355_UNIMPLEMENTED;
@@ -126,49 +151,73 @@ int h16_supported(const mi355_matmul_desc_t &d) {
     // byte offsets inside a tile are 32-bit
     const long ldb = k_major ? d.wei_stride[2] : d.K;
     if (d.src_stride[1] * EB * BM >= (1L << 31) || ldb * EB * f8_geo_t::BN >= (1L << 31)) return MI355_UNIMPLEMENTED;
-    if (!quant_absent(d.src_zp) || !quant_absent(d.wei_zp) || !quant_absent(d.src_pr)) return MI355_UNIMPLEMENTED;
-    if (!quant_absent(d.src_scale)
-            && ((d.src_scale.mask & 4) || d.src_scale.group[0] > 1 || d.src_scale.group[1] > 1))
-        return MI355_UNIMPLEMENTED;
-    if (!quant_absent(d.wei_scale)
-            && ((d.wei_scale.mask & 2) || d.wei_scale.group[0] > 1 || d.wei_scale.group[1] > 1))
-        return MI355_UNIMPLEMENTED;
-    if (d.batch > 65535) return MI355_UNIMPLEMENTED;
     return MI355_SUCCESS;
 }
 
+// whether the down-converting path runs (h16_supported's first acceptance)
+static bool h16_down(const mi355_matmul_desc_t &d) {
+    if (!h16_down_dt(d) || d.K < 32 || d.K % 32 != 0 || d.M * d.K * 2 >= (1L << 31) || d.K * 2 * f8_geo_t::BN >= (1L << 31))
+        return false;
+    return (d.src_stride[2] == 1 || d.src_stride[1] == 1) && (d.wei_stride[2] == 1 || d.wei_stride[1] == 1);
+}
+
 size_t h16_scratch_bytes(const mi355_matmul_desc_t &d) {
-    const long Bw = d.wei_stride[0] ? d.batch : 1;
+    const long Bw = d.wei_stride[0] ? d.batch : 1, Bs = d.src_stride[0] ? d.batch : 1;
+    if (h16_down(d))
+        return align_up((size_t)Bs * d.M * d.K * 2, 256) + align_up((size_t)Bw * d.N * d.K * 2, 256);
     return h16_k_major(d) ? 0 : align_up((size_t)Bw * d.N * d.K * (dt_bits(d.src_dt) / 8), 256);
 }
 
-int h16_launch(const mi355_matmul_desc_t &d, const problem_t &P, void *scratch, hipStream_t stream) {
+// [B][R][C] with the given strides -> dense [B][...] of data type `to`, rows x cols or (transposed) cols x rows
+static int h16_convert(const void *in, int from, long B, long R, long C, const int64_t *stride, bool transposed, int to,
+        void *out, hipStream_t stream) {
+    mi355_reorder_desc_t rd {};
+    rd.ndims = 3;
+    rd.src_dt = from;
+    rd.dst_dt = to;
+    rd.dims[0] = B; rd.dims[1] = R; rd.dims[2] = C;
+    rd.src_stride[0] = stride[0]; rd.src_stride[1] = stride[1]; rd.src_stride[2] = stride[2];
+    rd.dst_stride[0] = R * C;
+    rd.dst_stride[1] = transposed ? 1 : C;
+    rd.dst_stride[2] = transposed ? R : 1;
+    rd.src_scale.group[0] = rd.src_scale.group[1] = rd.dst_scale.group[0] = rd.dst_scale.group[1] = 1;
+    rd.src_zp.group[0] = rd.src_zp.group[1] = rd.dst_zp.group[0] = rd.dst_zp.group[1] = 1;
+    mi355_reorder_args_t ra {};
+    ra.src = in;
+    ra.dst = out;
+    return mi355_reorder_launch(&rd, &ra, stream);
+}
+
+int h16_launch(const mi355_matmul_desc_t &d, const problem_t &P_in, void *scratch, hipStream_t stream) {
     f8_extra_t X {};
-    const long EB = dt_bits(d.src_dt) / 8;
+    problem_t P = P_in;
+    int op_dt = d.src_dt;
     const size_t need = h16_scratch_bytes(d);
-    if (need > 0) {
-        if (!scratch) {
-            set_error("mfma_h16: %zu bytes of scratch required", need);
-            return MI355_INVALID_ARGUMENTS;
-        }
+    if (need > 0 && !scratch) {
+        set_error("mfma_h16: %zu bytes of scratch required", need);
+        return MI355_INVALID_ARGUMENTS;
+    }
+    const long Bw = d.wei_stride[0] ? d.batch : 1, Bs = d.src_stride[0] ? d.batch : 1;
+    if (h16_down(d)) {
+        op_dt = h16_down_dt(d);
+        char *a16 = (char *)scratch, *b16 = a16 + align_up((size_t)Bs * d.M * d.K * 2, 256);
+        if (const int st = h16_convert(P.src, MI355_DT_F32, Bs, d.M, d.K, d.src_stride, false, op_dt, a16, stream)) return st;
+        if (const int st = h16_convert(P.wei, MI355_DT_F32, Bw, d.K, d.N, d.wei_stride, true, op_dt, b16, stream)) return st;
+        P.src = a16;
+        P.src_dt = P.wei_dt = op_dt;
+        P.ss[0] = Bs > 1 ? d.M * d.K : 0; P.ss[1] = d.K; P.ss[2] = 1;
+        X.bt = b16;
+        X.ldb = d.K * 2;
+        X.bt_bstride = Bw > 1 ? d.N * d.K * 2 : 0;
+    } else if (need > 0) {
         // [Bw][K][N] with N contiguous -> [Bw][N][K] with K contiguous: the reorder's tiled kernel
-        const long Bw = d.wei_stride[0] ? d.batch : 1;
-        mi355_reorder_desc_t rd {};
-        rd.ndims = 3;
-        rd.src_dt = rd.dst_dt = d.wei_dt;
-        rd.dims[0] = Bw; rd.dims[1] = d.K; rd.dims[2] = d.N;
-        rd.src_stride[0] = d.wei_stride[0]; rd.src_stride[1] = d.wei_stride[1]; rd.src_stride[2] = 1;
-        rd.dst_stride[0] = d.N * d.K; rd.dst_stride[1] = 1; rd.dst_stride[2] = d.K;
-        rd.src_scale.group[0] = rd.src_scale.group[1] = rd.dst_scale.group[0] = rd.dst_scale.group[1] = 1;
-        rd.src_zp.group[0] = rd.src_zp.group[1] = rd.dst_zp.group[0] = rd.dst_zp.group[1] = 1;
-        mi355_reorder_args_t ra {};
-        ra.src = P.wei;
-        ra.dst = scratch;
-        if (const int st = mi355_reorder_launch(&rd, &ra, stream)) return st;
+        const long EB = dt_bits(d.src_dt) / 8;
+        if (const int st = h16_convert(P.wei, d.wei_dt, Bw, d.K, d.N, d.wei_stride, true, d.wei_dt, scratch, stream)) return st;
         X.bt = (const char *)scratch;
         X.ldb = d.K * EB;
         X.bt_bstride = Bw > 1 ? d.N * d.K * EB : 0;
     } else {
+        const long EB = dt_bits(d.src_dt) / 8;
         X.bt = (const char *)P.wei;
         X.ldb = d.wei_stride[2] * EB;
         X.bt_bstride = d.wei_stride[0] * EB;
@@ -182,8 +231,8 @@ int h16_launch(const mi355_matmul_desc_t &d, const problem_t &P, void *scratch, 
         hipLaunchKernelGGL(kern, grid, dim3(f8_geo_t::NT), smem_bytes, stream, P, X);
         return hipGetLastError() == hipSuccess ? MI355_SUCCESS : MI355_RUNTIME_ERROR;
     };
-    if (d.src_dt == MI355_DT_BF16) return go(f8_gemm_kernel<h16_mma_t<true, f8_geo_t>>);
-    if (d.src_dt == MI355_DT_F32) return go(f8_gemm_kernel<f32_mma_t<f8_geo_t>>);
+    if (op_dt == MI355_DT_BF16) return go(f8_gemm_kernel<h16_mma_t<true, f8_geo_t>>);
+    if (op_dt == MI355_DT_F32) return go(f8_gemm_kernel<f32_mma_t<f8_geo_t>>);
     return go(f8_gemm_kernel<h16_mma_t<false, f8_geo_t>>);
 }
 

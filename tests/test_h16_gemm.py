@@ -184,3 +184,50 @@ def test_matches_the_generic_kernel_on_a_large_shape(gpu):
     tol = np.abs(w) * 2.0 ** -7 + 64 * 2.0 ** -7 * 0.05
     assert (err <= tol).all(), f"worst {err.max()} at {err.argmax()}"
     assert (err > 0).mean() < 0.2          # most elements round to the same bf16 value
+
+
+# ------------------------------------------------------------------ f32 operands under fpmath_mode bf16 / f16 / any
+FPMATH_BF16, FPMATH_F16, FPMATH_ANY = 1, 2, 3
+
+
+def test_fpmath_dispatch_rules():
+    p = problem(64, 96, 64, "f32", "f32", wtag="ab")
+    p.fpmath_mode = FPMATH_BF16
+    st, impl = cabi.query(p.desc())
+    assert st == cabi.SUCCESS and impl == cabi.IMPL_H16_MFMA
+    assert cabi.scratch_bytes(p.desc()) == 64 * 64 * 2 + 96 * 64 * 2             # both operands as 16-bit copies
+    p.fpmath_mode = 0
+    assert cabi.scratch_bytes(p.desc()) == 96 * 64 * 4                           # strict: only the f32 layout pre-pass
+    p = problem(64, 96, 48, "f32", "f32")                                        # K = 48: f32 stages of 16, no bf16 stages of 32
+    p.fpmath_mode = FPMATH_ANY
+    assert cabi.query(p.desc())[1] == cabi.IMPL_H16_MFMA and cabi.scratch_bytes(p.desc()) == 0
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("mode", [FPMATH_BF16, FPMATH_F16, FPMATH_ANY])
+@pytest.mark.parametrize("wtag", ["ab", "ba"])
+def test_fpmath_exact_data_bit_exact(gpu, oracle, mode, wtag):
+    """values every 16-bit type holds exactly: the down-conversion changes nothing, the f32 oracle applies"""
+    p = problem(300, 200, 96, "f32", "f32", seed=21, wtag=wtag, bias=True, batch=2)
+    p.fpmath_mode = mode
+    got, name = run_gpu(p)
+    assert name.startswith("hip:mfma_h16"), name
+    assert_bit_exact(p, got, oracle.run_oracle(p), name)
+
+
+@pytest.mark.gpu
+def test_fpmath_bf16_is_the_bf16_matmul_of_the_rounded_operands(gpu):
+    """random f32 operands under fpmath bf16 give the bits of the bf16 problem whose operands are the same values
+    rounded to nearest even -- which pins the conversion and that nothing else changes"""
+    M, N, K = 192, 320, 512
+    r = np.random.default_rng(22)
+    sv = r.standard_normal((1, M, K)).astype(np.float32)
+    wv = r.standard_normal((1, K, N)).astype(np.float32)
+    pf = MatmulProblem(M=M, N=N, K=K, src_dt=cabi.DT_F32, wei_dt=cabi.DT_F32, dst_dt=cabi.DT_F32, src=sv, wei=wv,
+                       fpmath_mode=FPMATH_BF16, name="f32 under fpmath bf16")
+    pb = MatmulProblem(M=M, N=N, K=K, src_dt=cabi.DT_BF16, wei_dt=cabi.DT_BF16, dst_dt=cabi.DT_F32,
+                       src=enc(sv, "bf16"), wei=enc(wv, "bf16"), name="bf16")
+    got_f, name_f = run_gpu(pf)
+    got_b, name_b = run_gpu(pb)
+    assert name_f.startswith("hip:mfma_h16") and name_b.startswith("hip:mfma_h16")
+    assert np.array_equal(np.asarray(got_f).view(np.uint32), np.asarray(got_b).view(np.uint32))
