@@ -274,6 +274,20 @@ def test_shape_rules(eng):
     assert create(s, w, d, bias=dnnl.zero_memory_desc()) == dnnl.success         # a zero descriptor: no bias
 
 
+def test_zero_dims(eng):
+    # tests/gtests/test_inner_product_forward.cpp:260-283: an empty batch is a valid (no-op) problem, empty weights are not
+    ip_pd(eng, 0, 32, (6, 6), 48, sdt="f32", wdt="f32", stag=dnnl.tag_any, wtag=dnnl.tag_any, dtag=dnnl.tag_any)
+    assert status_of(lambda: ip_pd(eng, 2, 0, (6, 6), 48, sdt="f32", wdt="f32")) == dnnl.invalid_arguments
+
+
+def test_float_problems_run_on_the_matrix_cores(eng):
+    pd = ip_pd(eng, 128, 2048, (), 1000, sdt="bf16", wdt="bf16", ddt="bf16", wtag=dnnl.tag_any)
+    assert pd.impl_info_str().startswith("hip:mfma_h16") and pd.query_md(dnnl.query_weights_md).strides() == [2048, 1]
+    pd = ip_pd(eng, 128, 512, (7, 7), 1000, sdt="f32", wdt="f32", ddt="f32", stag=dnnl.tag_nhwc, wtag=dnnl.tag_any)
+    assert pd.impl_info_str().startswith("hip:mfma_h16")
+    assert pd.query_md(dnnl.query_weights_md).strides() == [25088, 1, 3584, 512]
+
+
 def test_data_type_rules(eng):
     un = dnnl.unimplemented
     assert status_of(lambda: ip_pd(eng, 2, 8, (), 6, sdt="s8", wdt="u8")) == un        # integer weights are s8
