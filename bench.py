@@ -510,7 +510,8 @@ def main():
     if args.calib_mfma:
         names = ["v_mfma_i32_32x32x32_i8", "v_mfma_i32_16x16x64_i8", "v_mfma_f32_32x32x64_f8f6f4 (fp8)",
                  "v_mfma_f32_16x16x128_f8f6f4 (fp8)", "v_mfma_scale_f32_32x32x64_f8f6f4 (fp4)",
-                 "v_mfma_scale_f32_16x16x128_f8f6f4 (fp4)"]
+                 "v_mfma_scale_f32_16x16x128_f8f6f4 (fp4)", "v_mfma_f32_32x32x16_bf16", "v_mfma_f32_16x16x32_bf16",
+                 "v_mfma_f32_32x32x2_f32"]
         out = cabi.DeviceBuffer(1 << 20)
         rng = np.random.default_rng(1)
         rows = []
@@ -521,6 +522,10 @@ def main():
                     else np.full(4096, 0x01010101, np.uint32)
                 if "fp8" in name:     # finite, moderate values: clear sign and top exponent bit
                     h &= np.uint32(0x3f3f3f3f)
+                elif "bf16" in name:
+                    h &= np.uint32(0x3fff3fff)
+                elif "_f32" in name and "x2_" in name:
+                    h &= np.uint32(0x3fffffff)
                 bits = cabi.DeviceBuffer.from_numpy(h)
                 ops = C.c_double(0)
                 timer = Timer(lib)

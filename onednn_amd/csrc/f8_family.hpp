@@ -2,6 +2,8 @@
 // kern_h16.hip) share: the kernel, templated over an operand policy; the fp8 policy, whose addresses and
 // fragment reads the other policies reuse; the scale handling and the compile-time epilogue chains.
 #pragma once
+#include <type_traits>
+
 #include "gemm_core.hpp"
 
 namespace mi355 {
@@ -246,6 +248,12 @@ struct f8_conv_t {
         return true;
         }
     }
+    // accumulator shapes without compile-time chains (the 16 x 16 tiles)
+    template <class PT, class Acc>
+    __device__ __forceinline__ bool hot_chain(const PT &, const epi_uniform_t &, unsigned, unsigned, const Acc &, long, long,
+            long, int) const {
+        return false;
+    }
     __device__ __forceinline__ void quad(const v4i_t &raw, float ssc, unsigned ntab, int col, float (&f)[4]) const {
 #pragma unroll
         for (int e = 0; e < 4; ++e) f[e] = __int_as_float(raw[e]);
@@ -259,6 +267,20 @@ struct f8_conv_t {
             for (int e = 0; e < 4; ++e) f[e] *= w[e];
         }
     }
+};
+
+// accumulator tile of a policy: 32 x 32 (sixteen registers) unless it declares TILE16
+template <class Mma, class = void>
+struct acc_of {
+    typedef v16f type;
+    typedef layout32_t layout;
+    static constexpr int N = 16;
+};
+template <class Mma>
+struct acc_of<Mma, std::enable_if_t<Mma::TILE16>> {
+    typedef v4f type;
+    typedef layout16_t layout;
+    static constexpr int N = 4;
 };
 
 extern __shared__ __attribute__((aligned(16))) char f8_smem[];
@@ -299,18 +321,19 @@ __global__ void __launch_bounds__(Mma::G::NT) __attribute__((amdgpu_waves_per_eu
     const unsigned ntab = (unsigned)(size_t)(__attribute__((address_space(3))) char *)smem + NSTAGE * G::STAGE_BYTES;
     fill_ntab<G::NT>(P, cv, ntab, b, n0);
 
-    v16f acc[Mma::ROWS][Mma::COLS];
+    typename acc_of<Mma>::type acc[Mma::ROWS][Mma::COLS];
 #pragma unroll
     for (int i = 0; i < Mma::ROWS; ++i)
 #pragma unroll
         for (int j = 0; j < Mma::COLS; ++j)
 #pragma unroll
-            for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
+            for (int r = 0; r < acc_of<Mma>::N; ++r) acc[i][j][r] = 0.f;
 
     main_loop<NSTAGE, KSTEP, Mma>(acc, smem, A, Bt, lda, X.ldb, P.M - m0,
             P.N - n0, (int)(P.K * EB / (BKB * KSTEP)), f8_ctx_t {});
 
-    store_quadrant<layout32_t, G::WCOLS>(P, smem, ntab, acc, b, m0 + wm * 128, n0 + wn * G::WCOLS, wn * G::WCOLS, cv);
+    store_quadrant<typename acc_of<Mma>::layout, G::WCOLS>(P, smem, ntab, acc, b, m0 + wm * 128, n0 + wn * G::WCOLS,
+            wn * G::WCOLS, cv);
 }
 
 } // namespace

@@ -1,10 +1,8 @@
 // "hip:mfma_h16" -- the same tiles for bf16 x bf16, f16 x f16 and f32 x f32 operands
 // (ref_matmul_t's f32 sum of exact products): a 64-byte stage is 32 elements of
-// K, two v_mfma_f32_32x32x16_{bf16,f16} per fragment pair in the time of the
-// one fp8 instruction, so the data path (DMA, LDS ring, fragment reads,
-// epilogue) is shared unchanged; a lane's two 16-byte chunks of a stage feed
-// the two instructions, the same chunks for both operands, so the order in
-// which the 32 k of a stage meet does not matter.
+// K, one v_mfma_f32_16x16x32_{bf16,f16} per pair of 16-row fragments, in the
+// matrix cycles of the fp8 family's instruction per stage, so the data path
+// (DMA, LDS ring, epilogue) is shared unchanged.
 #include "f8_family.hpp"
 
 namespace mi355 {
@@ -13,51 +11,55 @@ namespace {
 typedef __bf16 v8bf_t __attribute__((ext_vector_type(8)));
 typedef _Float16 v8h_t __attribute__((ext_vector_type(8)));
 
-// bf16 (BF16) or f16 operands: the fp8 policy's addresses and reads; a fragment
-// is its two 16-byte chunks, each the operand of one 32x32x16 instruction
+// bf16 (BF16) or f16 operands on the 16 x 16 x 32 instruction: a lane's one
+// 16-byte chunk of a stage (row lane % 16, chunk lane / 16) is the whole
+// operand.  The 32 x 32 x 16 shape (two instructions per fragment pair of the
+// fp8 policy's layout) costs the same matrix cycles and LDS bytes per stage, but
+// sustains 1.53 instead of 1.85 PFLOP/s on random operand bits (the clock the
+// power manager allows, `bench.py --calib-mfma`): 0.90 against 0.84 ms on
+// 8192^3, the fp8 family's whole-row bf16 epilogue included.
 template <bool BF16, class G_>
-struct h16_mma_t {
+struct h16x16_mma_t {
     using G = G_;
+    static constexpr bool TILE16 = true;
     static constexpr int ELEM_BYTES = 2;
-    static constexpr bool HOT = BF16; // the whole-row bf16 epilogue chains of the fp8 family
+    static constexpr bool HOT = false;
     static constexpr int EXTRA_DMAS = 0;
     __device__ static __forceinline__ void issue_extra(const f8_ctx_t &, int, int, int, int) {}
-    static constexpr int ROWS = 4, COLS = G::WCOLS / 32, A_READS = 2, B_READS = 2;
+    static constexpr int ROWS = 8, COLS = G::WCOLS / 16, A_READS = 1, B_READS = 1;
     struct frag_t {
-        v4i a[ROWS][2], b[COLS][2];
+        v4i a[ROWS], b[COLS];
     };
     __device__ static __forceinline__ frag_t zero_frag() { return frag_t {}; }
-    using addr_t = typename f8_mma_t<0, 0, G_>::addr_t;
+    struct addr_t {
+        unsigned a, b;
+    };
     __device__ static __forceinline__ addr_t lane_addr(int wm, int wn, int lane) {
-        return f8_mma_t<0, 0, G_>::lane_addr(wm, wn, lane);
+        const int frow = lane & 15, q = lane >> 4;
+        const int ra = wm * 128 + frow, rb = wn * G::WCOLS + frow;
+        return addr_t {(unsigned)swz(ra, q), (unsigned)(B_OFF + swz(rb, q))};
     }
     __device__ static __forceinline__ void load_b(frag_t &f, const unsigned (&S)[1], const addr_t &ad,
             const f8_ctx_t &, int) {
 #pragma unroll
-        for (int j = 0; j < COLS; ++j) {
-            f.b[j][0] = lds_read16(S[0] + ad.b0 + j * 2048);
-            f.b[j][1] = lds_read16(S[0] + ad.b1 + j * 2048);
-        }
+        for (int j = 0; j < COLS; ++j) f.b[j] = lds_read16(S[0] + ad.b + j * 1024);
     }
     __device__ static __forceinline__ void load_a(frag_t &f, int i, const unsigned (&S)[1], const addr_t &ad,
             const f8_ctx_t &, int) {
-        f.a[i][0] = lds_read16(S[0] + ad.a0 + i * 2048);
-        f.a[i][1] = lds_read16(S[0] + ad.a1 + i * 2048);
+        f.a[i] = lds_read16(S[0] + ad.a + i * 1024);
     }
-    __device__ static __forceinline__ void mma_row(v16f (&acc)[ROWS][COLS], const frag_t &f, int i,
+    __device__ static __forceinline__ void mma_row(v4f (&acc)[ROWS][COLS], const frag_t &f, int i,
             const f8_ctx_t &, int) {
 #pragma unroll
-        for (int h = 0; h < 2; ++h)
-#pragma unroll
-            for (int j = 0; j < COLS; ++j) {
-                // operands exchanged, as in the fp8 policy: the tile comes out transposed
-                if constexpr (BF16)
-                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(v8bf_t, f.b[j][h]),
-                            __builtin_bit_cast(v8bf_t, f.a[i][h]), acc[i][j], 0, 0, 0);
-                else
-                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(v8h_t, f.b[j][h]),
-                            __builtin_bit_cast(v8h_t, f.a[i][h]), acc[i][j], 0, 0, 0);
-            }
+        for (int j = 0; j < COLS; ++j) {
+            // operands exchanged: the tile comes out transposed (a lane holds four consecutive n of one row)
+            if constexpr (BF16)
+                acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(v8bf_t, f.b[j]),
+                        __builtin_bit_cast(v8bf_t, f.a[i]), acc[i][j], 0, 0, 0);
+            else
+                acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(v8h_t, f.b[j]),
+                        __builtin_bit_cast(v8h_t, f.a[i]), acc[i][j], 0, 0, 0);
+        }
     }
 };
 
@@ -231,9 +233,9 @@ int h16_launch(const mi355_matmul_desc_t &d, const problem_t &P_in, void *scratc
         hipLaunchKernelGGL(kern, grid, dim3(f8_geo_t::NT), smem_bytes, stream, P, X);
         return hipGetLastError() == hipSuccess ? MI355_SUCCESS : MI355_RUNTIME_ERROR;
     };
-    if (op_dt == MI355_DT_BF16) return go(f8_gemm_kernel<h16_mma_t<true, f8_geo_t>>);
+    if (op_dt == MI355_DT_BF16) return go(f8_gemm_kernel<h16x16_mma_t<true, f8_geo_t>>);
     if (op_dt == MI355_DT_F32) return go(f8_gemm_kernel<f32_mma_t<f8_geo_t>>);
-    return go(f8_gemm_kernel<h16_mma_t<false, f8_geo_t>>);
+    return go(f8_gemm_kernel<h16x16_mma_t<false, f8_geo_t>>);
 }
 
 } // namespace mi355

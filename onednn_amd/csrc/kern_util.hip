@@ -240,7 +240,7 @@ namespace mi355 {
 // SIMD, 8 or 16 independent accumulator chains per wavefront.  The operand bits
 // come from memory once, so the caller decides how much they toggle (the clock
 // the power manager grants depends on it).
-enum { RATE_I8_32, RATE_I8_16, RATE_F8_32, RATE_F8_16, RATE_F4_32, RATE_F4_16, RATE_COUNT };
+enum { RATE_I8_32, RATE_I8_16, RATE_F8_32, RATE_F8_16, RATE_F4_32, RATE_F4_16, RATE_BF16_32, RATE_BF16_16, RATE_F32_32, RATE_COUNT };
 
 template <int MODE>
 __global__ void __launch_bounds__(256) mfma_rate_kernel(int iters, int *out, const int *bits) {
@@ -264,6 +264,29 @@ __global__ void __launch_bounds__(256) mfma_rate_kernel(int iters, int *out, con
 #pragma unroll
             for (int j = 0; j < 16; ++j) c[j] = __builtin_amdgcn_mfma_i32_16x16x64_i8(a, b, c[j], 0, 0, 0);
         for (int j = 0; j < 16; ++j) result += c[j][0];
+    } else if (MODE == RATE_BF16_32) {
+        typedef __bf16 v8bf __attribute__((ext_vector_type(8)));
+        v16f c[8] = {};
+        for (int i = 0; i < iters; ++i)
+#pragma unroll
+            for (int j = 0; j < 8; ++j)
+                c[j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(v8bf, a), __builtin_bit_cast(v8bf, b), c[j], 0, 0, 0);
+        for (int j = 0; j < 8; ++j) result += (int)c[j][0];
+    } else if (MODE == RATE_BF16_16) {
+        typedef __bf16 v8bf __attribute__((ext_vector_type(8)));
+        v4f c[16] = {};
+        for (int i = 0; i < iters; ++i)
+#pragma unroll
+            for (int j = 0; j < 16; ++j)
+                c[j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(v8bf, a), __builtin_bit_cast(v8bf, b), c[j], 0, 0, 0);
+        for (int j = 0; j < 16; ++j) result += (int)c[j][0];
+    } else if (MODE == RATE_F32_32) {
+        v16f c[8] = {};
+        for (int i = 0; i < iters; ++i)
+#pragma unroll
+            for (int j = 0; j < 8; ++j)
+                c[j] = __builtin_amdgcn_mfma_f32_32x32x2f32(__int_as_float(a[0]), __int_as_float(b[0]), c[j], 0, 0, 0);
+        for (int j = 0; j < 8; ++j) result += (int)c[j][0];
     } else if (MODE == RATE_F8_32 || MODE == RATE_F4_32) {
         constexpr int fmt = MODE == RATE_F4_32 ? 4 : 0, sc = MODE == RATE_F4_32 ? 127 : 0;
         v16f c[8] = {};
@@ -289,12 +312,13 @@ extern "C" int mi355_mfma_rate_kernel(int instr, int iters, void *out, const voi
         void *stream) {
     constexpr int blocks = 1024;
     if (instr < 0 || instr >= RATE_COUNT || iters < 1 || !out || !bits) {
-        set_error("mfma rate kernel: instruction 0..5, out of 1 MiB, 16 KiB of operand bits");
+        set_error("mfma rate kernel: instruction 0..8, out of 1 MiB, 16 KiB of operand bits");
         return MI355_INVALID_ARGUMENTS;
     }
     static const double inst_ops[RATE_COUNT] = {2.0 * 32 * 32 * 32, 2.0 * 16 * 16 * 64, 2.0 * 32 * 32 * 64,
-            2.0 * 16 * 16 * 128, 2.0 * 32 * 32 * 64, 2.0 * 16 * 16 * 128};
-    static const int chains[RATE_COUNT] = {8, 16, 8, 16, 8, 16};
+            2.0 * 16 * 16 * 128, 2.0 * 32 * 32 * 64, 2.0 * 16 * 16 * 128, 2.0 * 32 * 32 * 16, 2.0 * 16 * 16 * 32,
+            2.0 * 32 * 32 * 2};
+    static const int chains[RATE_COUNT] = {8, 16, 8, 16, 8, 16, 8, 16, 8};
     if (ops_per_launch) *ops_per_launch = (double)blocks * 4 * iters * chains[instr] * inst_ops[instr];
     hipStream_t s = (hipStream_t)stream;
     int *o = (int *)out;
@@ -305,6 +329,9 @@ extern "C" int mi355_mfma_rate_kernel(int instr, int iters, void *out, const voi
         case RATE_F8_32: hipLaunchKernelGGL(mfma_rate_kernel<RATE_F8_32>, dim3(blocks), dim3(256), 0, s, iters, o, bp); break;
         case RATE_F8_16: hipLaunchKernelGGL(mfma_rate_kernel<RATE_F8_16>, dim3(blocks), dim3(256), 0, s, iters, o, bp); break;
         case RATE_F4_32: hipLaunchKernelGGL(mfma_rate_kernel<RATE_F4_32>, dim3(blocks), dim3(256), 0, s, iters, o, bp); break;
+        case RATE_BF16_32: hipLaunchKernelGGL(mfma_rate_kernel<RATE_BF16_32>, dim3(blocks), dim3(256), 0, s, iters, o, bp); break;
+        case RATE_BF16_16: hipLaunchKernelGGL(mfma_rate_kernel<RATE_BF16_16>, dim3(blocks), dim3(256), 0, s, iters, o, bp); break;
+        case RATE_F32_32: hipLaunchKernelGGL(mfma_rate_kernel<RATE_F32_32>, dim3(blocks), dim3(256), 0, s, iters, o, bp); break;
         default: hipLaunchKernelGGL(mfma_rate_kernel<RATE_F4_16>, dim3(blocks), dim3(256), 0, s, iters, o, bp); break;
     }
     return hipGetLastError() == hipSuccess ? MI355_SUCCESS : MI355_RUNTIME_ERROR;

@@ -121,9 +121,9 @@ def test_exact_data_with_scales_bias_and_post_ops(gpu, oracle, dt):
 @pytest.mark.gpu
 @pytest.mark.parametrize("shape", [(256, 256, 64), (300, 200, 96), (33, 520, 160), (512, 768, 1024)])
 @pytest.mark.parametrize("chain", ["none", "bias", "residual", "bias+residual"])
-def test_bf16_dst_whole_row_epilogue(gpu, oracle, shape, chain):
-    """bf16 dst with at most a bias and a bf16 residual add takes the epilogue that moves whole 128-byte rows
-    (the fp8 family's); exact sums round to bf16 the same way on both sides."""
+def test_bf16_dst_with_bias_and_residual(gpu, oracle, shape, chain):
+    """bf16 dst with a bias and / or a bf16 residual add (the transformer layer's chain): exact sums round to bf16
+    the same way on both sides."""
     M, N, K = shape
     r = np.random.default_rng(12)
     post = []
