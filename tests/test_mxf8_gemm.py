@@ -110,3 +110,36 @@ def test_random_data_within_the_matrix_core_bound(gpu, oracle, ddt):
     assert name.startswith("hip:mfma_f8"), name
     _, ideal, asum = oracle.run_oracle(p, want_ideal=True)
     assert_gemm_close(p, got, ideal, asum, what=name, hw=mx_mfma_bound(p))
+
+
+@pytest.mark.gpu
+def test_block_scales_are_exact_powers_of_two_at_full_k(gpu):
+    """A size-independent property at K = 8192 (256 blocks per row): raising every src scale byte by one doubles every
+    dst value exactly, and raising the scales of a single block of weights doubles that block's contribution --
+    checked through a problem whose other blocks are zero."""
+    M, N, K = 512, 1024, 8192
+    p1 = problem(M, N, K, exact=False, seed=31)
+    p2 = problem(M, N, K, exact=False, seed=31)
+    p2.quant["src_scale"].data = (p2.quant["src_scale"].data + 1).astype(np.uint8)
+    g1, name = run_gpu(p1)
+    g2, _ = run_gpu(p2)
+    assert name.startswith("hip:mfma_f8"), name
+    a, b = np.asarray(g1, np.float32), np.asarray(g2, np.float32)
+    assert np.isfinite(a).all() and np.array_equal(b, a * np.float32(2))
+    # one block of K alive: block 100 of the weights (k 3200 .. 3231); its scale raised by one doubles dst
+    p3 = problem(M, N, K, exact=False, seed=31)
+    w = p3.wei.reshape(1, N, K).copy()
+    keep = w[:, :, 3200:3232].copy()
+    w[:] = 0
+    w[:, :, 3200:3232] = keep
+    p3.wei = w
+    g3, _ = run_gpu(p3)
+    p3.quant["wei_scale"].data = p3.quant["wei_scale"].data.copy()
+    p3.quant["wei_scale"].data.reshape(1, K // 32, N)[:, 100, :] += 1
+    g4, _ = run_gpu(p3)
+    a, b = np.asarray(g3, np.float32), np.asarray(g4, np.float32)
+    assert np.abs(a).max() > 0 and np.array_equal(b, a * np.float32(2))
+    # ... and the scales of any other block change nothing
+    p3.quant["wei_scale"].data.reshape(1, K // 32, N)[:, 101, :] += 3
+    g5, _ = run_gpu(p3)
+    assert np.array_equal(np.asarray(g5, np.float32), b)
