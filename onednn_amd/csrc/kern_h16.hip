@@ -106,10 +106,14 @@ struct f32_mma_t {
 } // namespace
 
 // ---- bf16 / f16 / f32
-static bool h16_k_major(const mi355_matmul_desc_t &d) {
-    const int AL = 16 / (dt_bits(d.src_dt) / 8);
-    return d.wei_stride[1] == 1 && d.wei_stride[2] % AL == 0 && d.wei_stride[0] % AL == 0;
+namespace {
+// zeroes bytes [from, pitch) of every row: the K padding of an operand copy
+__global__ void __launch_bounds__(256) h16_zero_tail_kernel(uint16_t *base, long rows, long pitch16, long from16) {
+    const long per = pitch16 - from16, total = rows * per;
+    for (long i = (long)blockIdx.x * 256 + threadIdx.x; i < total; i += (long)gridDim.x * 256)
+        base[(i / per) * pitch16 + from16 + i % per] = 0;
 }
+} // namespace
 
 // f32 operands under fpmath_mode bf16 / f16 / any (dnnl_fpmath_mode_t 1 / 2 / 3): the attribute allows an implicit
 // down-conversion (doc/programming_model/attributes_fpmath_mode.md), so both operands are converted into scratch by
@@ -120,6 +124,49 @@ static int h16_down_dt(const mi355_matmul_desc_t &d) {
     if (d.fpmath_mode == 1 || d.fpmath_mode == 3) return MI355_DT_BF16;
     if (d.fpmath_mode == 2) return MI355_DT_F16;
     return 0;
+}
+
+// How a problem reaches the tiles.  An operand is read where it lies when it is K-contiguous with 16-byte aligned
+// rows and K fills whole 64-byte stages; otherwise a reorder launch copies it into scratch as dense K-contiguous
+// rows of Kp = K rounded up to whole stages (converted on the way under fpmath, transposed on the way for
+// N-contiguous weights), the padding zeroed -- so any K and any plain layout with a unit stride runs here, at the
+// price of the copy.
+struct h16_plan_t {
+    bool ok;
+    int op_dt;
+    long EB, Kp, Bs, Bw;
+    bool copy_src, copy_wei;
+    size_t off_wei, total;
+};
+
+static h16_plan_t h16_plan(const mi355_matmul_desc_t &d) {
+    h16_plan_t p {};
+    if (d.K < 1) return p;
+    p.Bs = d.src_stride[0] ? d.batch : 1;
+    p.Bw = d.wei_stride[0] ? d.batch : 1;
+    const int down = h16_down_dt(d);
+    p.op_dt = down ? down : d.src_dt;
+    p.EB = dt_bits(p.op_dt) / 8;
+    const long KE = BKB * KSTEP / p.EB, AL = 16 / p.EB;
+    p.Kp = (d.K + KE - 1) / KE * KE;
+    const bool pad = p.Kp != d.K;
+    const bool src_direct = !down && !pad && d.src_stride[2] == 1 && d.src_stride[1] % AL == 0 && d.src_stride[0] % AL == 0;
+    const bool wei_direct = !down && !pad && d.wei_stride[1] == 1 && d.wei_stride[2] % AL == 0 && d.wei_stride[0] % AL == 0;
+    p.copy_src = !src_direct;
+    p.copy_wei = !wei_direct;
+    // the copies come from the reorder's direct or tiled kernels: a unit stride on the way in
+    if (p.copy_src && d.src_stride[2] != 1 && d.src_stride[1] != 1) return p;
+    if (p.copy_wei && d.wei_stride[2] != 1 && d.wei_stride[1] != 1) return p;
+    // byte offsets inside a tile are 32-bit
+    const long lda = p.copy_src ? p.Kp : d.src_stride[1], ldb = p.copy_wei ? p.Kp : d.wei_stride[2];
+    if (lda * p.EB * BM >= (1L << 31) || ldb * p.EB * f8_geo_t::BN >= (1L << 31)) return p;
+    size_t off = 0;
+    if (p.copy_src) off += align_up((size_t)p.Bs * d.M * p.Kp * p.EB, 256);
+    p.off_wei = off;
+    if (p.copy_wei) off += align_up((size_t)p.Bw * d.N * p.Kp * p.EB, 256);
+    p.total = off;
+    p.ok = true;
+    return p;
 }
 
 int h16_supported(const mi355_matmul_desc_t &d) {
@@ -134,96 +181,81 @@ int h16_supported(const mi355_matmul_desc_t &d) {
             && ((d.wei_scale.mask & 2) || d.wei_scale.group[0] > 1 || d.wei_scale.group[1] > 1))
         return MI355_UNIMPLEMENTED;
     if (d.batch > 65535) return MI355_UNIMPLEMENTED;
-    if (h16_down_dt(d) && d.K >= 32 && d.K % 32 == 0 && d.M * d.K * 2 < (1L << 31) && d.K * 2 * f8_geo_t::BN < (1L << 31)) {
-        // the converted copies are dense: any strides the reorder takes
-        const bool src_ok = d.src_stride[2] == 1 || d.src_stride[1] == 1;
-        const bool wei_ok = d.wei_stride[2] == 1 || d.wei_stride[1] == 1;
-        if (src_ok && wei_ok) return MI355_SUCCESS;
-    }
-    const int EB = dt_bits(d.src_dt) / 8;   // bytes per element
-    const int KE = BKB * KSTEP / EB, AL = 16 / EB; // elements of K per stage; elements per 16 bytes
-    if (d.K < KE || d.K % KE != 0) return MI355_UNIMPLEMENTED;
-    // 16-byte row pieces
-    if (d.src_stride[2] != 1 || d.src_stride[1] % AL != 0 || d.src_stride[0] % AL != 0) return MI355_UNIMPLEMENTED;
-    // K-contiguous weights (what format_tag::any resolves to) are read in place; N-contiguous ones are
-    // transposed into scratch by a pre-pass of every launch
-    const bool k_major = h16_k_major(d);
-    const bool n_major = d.wei_stride[2] == 1;
-    if (!k_major && !n_major) return MI355_UNIMPLEMENTED;
-    // byte offsets inside a tile are 32-bit
-    const long ldb = k_major ? d.wei_stride[2] : d.K;
-    if (d.src_stride[1] * EB * BM >= (1L << 31) || ldb * EB * f8_geo_t::BN >= (1L << 31)) return MI355_UNIMPLEMENTED;
-    return MI355_SUCCESS;
-}
-
-// whether the down-converting path runs (h16_supported's first acceptance)
-static bool h16_down(const mi355_matmul_desc_t &d) {
-    if (!h16_down_dt(d) || d.K < 32 || d.K % 32 != 0 || d.M * d.K * 2 >= (1L << 31) || d.K * 2 * f8_geo_t::BN >= (1L << 31))
-        return false;
-    return (d.src_stride[2] == 1 || d.src_stride[1] == 1) && (d.wei_stride[2] == 1 || d.wei_stride[1] == 1);
+    return h16_plan(d).ok ? MI355_SUCCESS : MI355_UNIMPLEMENTED;
 }
 
 size_t h16_scratch_bytes(const mi355_matmul_desc_t &d) {
-    const long Bw = d.wei_stride[0] ? d.batch : 1, Bs = d.src_stride[0] ? d.batch : 1;
-    if (h16_down(d))
-        return align_up((size_t)Bs * d.M * d.K * 2, 256) + align_up((size_t)Bw * d.N * d.K * 2, 256);
-    return h16_k_major(d) ? 0 : align_up((size_t)Bw * d.N * d.K * (dt_bits(d.src_dt) / 8), 256);
+    const h16_plan_t p = h16_plan(d);
+    return p.ok ? p.total : 0;
 }
 
-// [B][R][C] with the given strides -> dense [B][...] of data type `to`, rows x cols or (transposed) cols x rows
+// [B][R][C] with the given strides -> [B][R][ld] (or, transposed, [B][C][ld]) of data type `to`, ld >= the row
+// length; the columns beyond it are zeroed
 static int h16_convert(const void *in, int from, long B, long R, long C, const int64_t *stride, bool transposed, int to,
-        void *out, hipStream_t stream) {
+        void *out, long ld, hipStream_t stream) {
+    const long rows = transposed ? C : R, cols = transposed ? R : C;
     mi355_reorder_desc_t rd {};
     rd.ndims = 3;
     rd.src_dt = from;
     rd.dst_dt = to;
     rd.dims[0] = B; rd.dims[1] = R; rd.dims[2] = C;
     rd.src_stride[0] = stride[0]; rd.src_stride[1] = stride[1]; rd.src_stride[2] = stride[2];
-    rd.dst_stride[0] = R * C;
-    rd.dst_stride[1] = transposed ? 1 : C;
-    rd.dst_stride[2] = transposed ? R : 1;
+    rd.dst_stride[0] = rows * ld;
+    rd.dst_stride[1] = transposed ? 1 : ld;
+    rd.dst_stride[2] = transposed ? ld : 1;
     rd.src_scale.group[0] = rd.src_scale.group[1] = rd.dst_scale.group[0] = rd.dst_scale.group[1] = 1;
     rd.src_zp.group[0] = rd.src_zp.group[1] = rd.dst_zp.group[0] = rd.dst_zp.group[1] = 1;
     mi355_reorder_args_t ra {};
     ra.src = in;
     ra.dst = out;
-    return mi355_reorder_launch(&rd, &ra, stream);
+    if (const int st = mi355_reorder_launch(&rd, &ra, stream)) return st;
+    if (ld > cols) {
+        const long units = dt_bits(to) / 16; // 16-bit words per element
+        const long total = B * rows * (ld - cols) * units;
+        long blocks = (total + 255) / 256;
+        if (blocks > 65535) blocks = 65535;
+        hipLaunchKernelGGL(h16_zero_tail_kernel, dim3((unsigned)blocks), dim3(256), 0, stream, (uint16_t *)out, B * rows,
+                ld * units, cols * units);
+        if (hipGetLastError() != hipSuccess) return MI355_RUNTIME_ERROR;
+    }
+    return MI355_SUCCESS;
 }
 
 int h16_launch(const mi355_matmul_desc_t &d, const problem_t &P_in, void *scratch, hipStream_t stream) {
-    f8_extra_t X {};
-    problem_t P = P_in;
-    int op_dt = d.src_dt;
-    const size_t need = h16_scratch_bytes(d);
-    if (need > 0 && !scratch) {
-        set_error("mfma_h16: %zu bytes of scratch required", need);
+    const h16_plan_t plan = h16_plan(d);
+    if (!plan.ok) {
+        set_error("mfma_h16: the problem is not one this family takes");
+        return MI355_UNIMPLEMENTED;
+    }
+    if (plan.total > 0 && !scratch) {
+        set_error("mfma_h16: %zu bytes of scratch required", plan.total);
         return MI355_INVALID_ARGUMENTS;
     }
-    const long Bw = d.wei_stride[0] ? d.batch : 1, Bs = d.src_stride[0] ? d.batch : 1;
-    if (h16_down(d)) {
-        op_dt = h16_down_dt(d);
-        char *a16 = (char *)scratch, *b16 = a16 + align_up((size_t)Bs * d.M * d.K * 2, 256);
-        if (const int st = h16_convert(P.src, MI355_DT_F32, Bs, d.M, d.K, d.src_stride, false, op_dt, a16, stream)) return st;
-        if (const int st = h16_convert(P.wei, MI355_DT_F32, Bw, d.K, d.N, d.wei_stride, true, op_dt, b16, stream)) return st;
-        P.src = a16;
-        P.src_dt = P.wei_dt = op_dt;
-        P.ss[0] = Bs > 1 ? d.M * d.K : 0; P.ss[1] = d.K; P.ss[2] = 1;
-        X.bt = b16;
-        X.ldb = d.K * 2;
-        X.bt_bstride = Bw > 1 ? d.N * d.K * 2 : 0;
-    } else if (need > 0) {
-        // [Bw][K][N] with N contiguous -> [Bw][N][K] with K contiguous: the reorder's tiled kernel
-        const long EB = dt_bits(d.src_dt) / 8;
-        if (const int st = h16_convert(P.wei, d.wei_dt, Bw, d.K, d.N, d.wei_stride, true, d.wei_dt, scratch, stream)) return st;
-        X.bt = (const char *)scratch;
-        X.ldb = d.K * EB;
-        X.bt_bstride = Bw > 1 ? d.N * d.K * EB : 0;
+    f8_extra_t X {};
+    problem_t P = P_in;
+    const long EB = plan.EB;
+    char *a_copy = (char *)scratch, *b_copy = (char *)scratch + plan.off_wei;
+    if (plan.copy_src) {
+        if (const int st = h16_convert(P.src, d.src_dt, plan.Bs, d.M, d.K, d.src_stride, false, plan.op_dt, a_copy, plan.Kp,
+                    stream))
+            return st;
+        P.src = a_copy;
+        P.ss[0] = plan.Bs > 1 ? d.M * plan.Kp : 0; P.ss[1] = plan.Kp; P.ss[2] = 1;
+    }
+    if (plan.copy_wei) {
+        if (const int st = h16_convert(P.wei, d.wei_dt, plan.Bw, d.K, d.N, d.wei_stride, true, plan.op_dt, b_copy, plan.Kp,
+                    stream))
+            return st;
+        X.bt = b_copy;
+        X.ldb = plan.Kp * EB;
+        X.bt_bstride = plan.Bw > 1 ? d.N * plan.Kp * EB : 0;
     } else {
-        const long EB = dt_bits(d.src_dt) / 8;
         X.bt = (const char *)P.wei;
         X.ldb = d.wei_stride[2] * EB;
         X.bt_bstride = d.wei_stride[0] * EB;
     }
+    P.src_dt = P.wei_dt = plan.op_dt;
+    P.K = plan.Kp; // the padding multiplies zeros by zeros
     X.tiles_m = (int)((d.M + BM - 1) / BM);
     X.tiles_n = (int)((d.N + f8_geo_t::BN - 1) / f8_geo_t::BN);
     dim3 grid((unsigned)(X.tiles_m * X.tiles_n), 1, (unsigned)d.batch);
@@ -233,8 +265,8 @@ int h16_launch(const mi355_matmul_desc_t &d, const problem_t &P_in, void *scratc
         hipLaunchKernelGGL(kern, grid, dim3(f8_geo_t::NT), smem_bytes, stream, P, X);
         return hipGetLastError() == hipSuccess ? MI355_SUCCESS : MI355_RUNTIME_ERROR;
     };
-    if (op_dt == MI355_DT_BF16) return go(f8_gemm_kernel<h16x16_mma_t<true, f8_geo_t>>);
-    if (op_dt == MI355_DT_F32) return go(f8_gemm_kernel<f32_mma_t<f8_geo_t>>);
+    if (plan.op_dt == MI355_DT_BF16) return go(f8_gemm_kernel<h16x16_mma_t<true, f8_geo_t>>);
+    if (plan.op_dt == MI355_DT_F32) return go(f8_gemm_kernel<f32_mma_t<f8_geo_t>>);
     return go(f8_gemm_kernel<h16x16_mma_t<false, f8_geo_t>>);
 }
 

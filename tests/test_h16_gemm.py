@@ -61,10 +61,12 @@ def test_dispatch_rules():
     assert cabi.impl_name(impl).startswith("hip:mfma_h16")
     assert q(problem(64, 64, 64, "f16", "f16"))[1] == cabi.IMPL_H16_MFMA
     assert q(problem(64, 64, 16, "f32", "f32"))[1] == cabi.IMPL_H16_MFMA           # f32: stages of 16 k
-    assert q(problem(64, 64, 24, "f32", "f32"))[1] == cabi.IMPL_REF
+    assert q(problem(64, 64, 24, "f32", "f32"))[1] == cabi.IMPL_H16_MFMA          # ... 24 -> 32
+    assert cabi.scratch_bytes(problem(64, 64, 24, "f32", "f32").desc()) == 2 * 64 * 32 * 4
     assert q(problem(1, 8, 32, "bf16", "bf16"))[1] == cabi.IMPL_H16_MFMA          # any M, N; K in stages of 32
-    assert q(problem(64, 64, 48, "bf16", "f32"))[1] == cabi.IMPL_REF              # K not a multiple of 32
-    p = problem(64, 64, 64, "bf16", "f32", wtag="ab")                             # row-major weights: a layout pre-pass
+    p = problem(64, 64, 48, "bf16", "f32")                                        # K not in whole stages: padded copies
+    assert q(p)[1] == cabi.IMPL_H16_MFMA and cabi.scratch_bytes(p.desc()) == 2 * 64 * 64 * 2
+    p = problem(64, 64, 64, "bf16", "f32", wtag="ab")                             # row-major weights: copied K-contiguous
     assert q(p)[1] == cabi.IMPL_H16_MFMA and cabi.scratch_bytes(p.desc()) == 64 * 64 * 2
     assert cabi.scratch_bytes(problem(64, 64, 64, "bf16", "f32").desc()) == 0
     p = problem(64, 64, 64, "bf16", "f32")
@@ -198,9 +200,11 @@ def test_fpmath_dispatch_rules():
     assert cabi.scratch_bytes(p.desc()) == 64 * 64 * 2 + 96 * 64 * 2             # both operands as 16-bit copies
     p.fpmath_mode = 0
     assert cabi.scratch_bytes(p.desc()) == 96 * 64 * 4                           # strict: only the f32 layout pre-pass
-    p = problem(64, 96, 48, "f32", "f32")                                        # K = 48: f32 stages of 16, no bf16 stages of 32
+    p = problem(64, 96, 48, "f32", "f32")                                        # K = 48: bf16 copies padded to 64
     p.fpmath_mode = FPMATH_ANY
-    assert cabi.query(p.desc())[1] == cabi.IMPL_H16_MFMA and cabi.scratch_bytes(p.desc()) == 0
+    assert cabi.query(p.desc())[1] == cabi.IMPL_H16_MFMA and cabi.scratch_bytes(p.desc()) == (64 + 96) * 64 * 2
+    p.fpmath_mode = 0                                                            # strict: f32 stages of 16, read in place
+    assert cabi.scratch_bytes(p.desc()) == 0
 
 
 @pytest.mark.gpu
@@ -231,3 +235,36 @@ def test_fpmath_bf16_is_the_bf16_matmul_of_the_rounded_operands(gpu):
     got_b, name_b = run_gpu(pb)
     assert name_f.startswith("hip:mfma_h16") and name_b.startswith("hip:mfma_h16")
     assert np.array_equal(np.asarray(got_f).view(np.uint32), np.asarray(got_b).view(np.uint32))
+
+
+# ------------------------------------------------------------------ any K, any plain layout: operand copies
+@pytest.mark.gpu
+@pytest.mark.parametrize("K", [1, 8, 33, 100, 1000])
+@pytest.mark.parametrize("dt", ["bf16", "f16", "f32"])
+@pytest.mark.parametrize("wtag", ["ab", "ba"])
+def test_any_k_exact(gpu, oracle, K, dt, wtag):
+    p = problem(130, 75, K, dt, "f32", seed=40 + K, wtag=wtag, bias=True)
+    got, name = run_gpu(p)
+    assert name.startswith("hip:mfma_h16"), name
+    assert_bit_exact(p, got, oracle.run_oracle(p), name)
+
+
+@pytest.mark.gpu
+def test_column_major_src_and_batched_odd_k(gpu, oracle):
+    M, N, K, B = 70, 90, 45, 3
+    p = problem(M, N, K, "bf16", "bf16", seed=50, batch=B, wtag="ab")
+    src = p.src.reshape(B, M, K)
+    p.src = np.ascontiguousarray(src.transpose(0, 2, 1))          # [B][K][M]: M contiguous
+    p.src_stride = (M * K, 1, M)
+    got, name = run_gpu(p)
+    assert name.startswith("hip:mfma_h16"), name
+    assert_bit_exact(p, got, oracle.run_oracle(p), name)
+
+
+@pytest.mark.gpu
+def test_fpmath_with_odd_k(gpu, oracle):
+    p = problem(64, 48, 77, "f32", "f32", seed=51, wtag="ab")
+    p.fpmath_mode = FPMATH_BF16
+    got, name = run_gpu(p)
+    assert name.startswith("hip:mfma_h16"), name
+    assert_bit_exact(p, got, oracle.run_oracle(p), name)
