@@ -132,7 +132,7 @@ static int h16_down_dt(const mi355_matmul_desc_t &d) {
 // N-contiguous weights), the padding zeroed -- so any K and any plain layout with a unit stride runs here, at the
 // price of the copy.
 struct h16_plan_t {
-    bool ok;
+    bool ok, woq;
     int op_dt;
     long EB, Kp, Bs, Bw;
     bool copy_src, copy_wei;
@@ -145,13 +145,15 @@ static h16_plan_t h16_plan(const mi355_matmul_desc_t &d) {
     p.Bs = d.src_stride[0] ? d.batch : 1;
     p.Bw = d.wei_stride[0] ? d.batch : 1;
     const int down = h16_down_dt(d);
+    p.woq = d.src_dt != d.wei_dt; // 8- or 4-bit integer weights under a 16-bit src (checked by h16_supported)
     p.op_dt = down ? down : d.src_dt;
     p.EB = dt_bits(p.op_dt) / 8;
     const long KE = BKB * KSTEP / p.EB, AL = 16 / p.EB;
     p.Kp = (d.K + KE - 1) / KE * KE;
     const bool pad = p.Kp != d.K;
     const bool src_direct = !down && !pad && d.src_stride[2] == 1 && d.src_stride[1] % AL == 0 && d.src_stride[0] % AL == 0;
-    const bool wei_direct = !down && !pad && d.wei_stride[1] == 1 && d.wei_stride[2] % AL == 0 && d.wei_stride[0] % AL == 0;
+    const bool wei_direct = !down && !pad && !p.woq && d.wei_stride[1] == 1 && d.wei_stride[2] % AL == 0
+            && d.wei_stride[0] % AL == 0;
     p.copy_src = !src_direct;
     p.copy_wei = !wei_direct;
     // the copies come from the reorder's direct or tiled kernels: a unit stride on the way in
@@ -169,10 +171,35 @@ static h16_plan_t h16_plan(const mi355_matmul_desc_t &d) {
     return p;
 }
 
+// Weight-only quantization beyond the decode kernels' 32 rows (prefill): s4 / u4 / s8 / u8 weights under a bf16 / f16
+// src with fpmath apply_to_int.  The weights' copy is written by the reorder with the weights' scales and zero points
+// as its src parameters -- (w - zp) * scale rounded to the src type, what the reference's JIT path multiplies
+// (brgemm_matmul_copy_utils.cpp:2870-2896) -- and the 16-bit tiles run without them.
+static bool h16_woq(const mi355_matmul_desc_t &d) {
+    if (d.src_dt != MI355_DT_BF16 && d.src_dt != MI355_DT_F16) return false;
+    if (d.wei_dt != MI355_DT_S4 && d.wei_dt != MI355_DT_U4 && d.wei_dt != MI355_DT_S8 && d.wei_dt != MI355_DT_U8) return false;
+    if (!d.fpmath_apply_to_int || d.wei_packing != MI355_WEI_PACK_NONE) return false;
+    if (!quant_absent(d.src_scale) || !quant_absent(d.src_zp) || !quant_absent(d.src_pr)) return false;
+    const int sdt = d.wei_scale.dt, zdt = d.wei_zp.dt;
+    if (sdt != MI355_DT_UNDEF && sdt != MI355_DT_F32 && sdt != MI355_DT_BF16 && sdt != MI355_DT_F16) return false;
+    if (zdt != MI355_DT_UNDEF && zdt != MI355_DT_S32 && zdt != MI355_DT_S8 && zdt != MI355_DT_U8 && zdt != MI355_DT_S4
+            && zdt != MI355_DT_U4)
+        return false;
+    for (const mi355_quant_t *q : {&d.wei_scale, &d.wei_zp})
+        if (q->dt != MI355_DT_UNDEF
+                && ((q->group[0] > 1 && d.K % q->group[0]) || (q->group[1] > 1 && d.N % q->group[1])))
+            return false;
+    // 4-bit weights: whole bytes along the contiguous dim
+    if (dt_bits(d.wei_dt) == 4 && ((d.wei_stride[2] == 1 ? d.N : d.K) % 2)) return false;
+    return true;
+}
+
 int h16_supported(const mi355_matmul_desc_t &d) {
+    if (dt_bits(d.dst_dt) < 8) return MI355_UNIMPLEMENTED;
+    if (d.batch > 65535) return MI355_UNIMPLEMENTED;
+    if (h16_woq(d)) return h16_plan(d).ok ? MI355_SUCCESS : MI355_UNIMPLEMENTED;
     if (d.src_dt != d.wei_dt || (d.src_dt != MI355_DT_BF16 && d.src_dt != MI355_DT_F16 && d.src_dt != MI355_DT_F32))
         return MI355_UNIMPLEMENTED;
-    if (dt_bits(d.dst_dt) < 8) return MI355_UNIMPLEMENTED;
     if (!quant_absent(d.src_zp) || !quant_absent(d.wei_zp) || !quant_absent(d.src_pr)) return MI355_UNIMPLEMENTED;
     if (!quant_absent(d.src_scale)
             && ((d.src_scale.mask & 4) || d.src_scale.group[0] > 1 || d.src_scale.group[1] > 1))
@@ -192,7 +219,8 @@ size_t h16_scratch_bytes(const mi355_matmul_desc_t &d) {
 // [B][R][C] with the given strides -> [B][R][ld] (or, transposed, [B][C][ld]) of data type `to`, ld >= the row
 // length; the columns beyond it are zeroed
 static int h16_convert(const void *in, int from, long B, long R, long C, const int64_t *stride, bool transposed, int to,
-        void *out, long ld, hipStream_t stream) {
+        void *out, long ld, hipStream_t stream, const mi355_quant_t *scale = nullptr, const void *scale_p = nullptr,
+        const mi355_quant_t *zp = nullptr, const void *zp_p = nullptr) {
     const long rows = transposed ? C : R, cols = transposed ? R : C;
     mi355_reorder_desc_t rd {};
     rd.ndims = 3;
@@ -208,6 +236,14 @@ static int h16_convert(const void *in, int from, long B, long R, long C, const i
     mi355_reorder_args_t ra {};
     ra.src = in;
     ra.dst = out;
+    if (scale && scale->dt != MI355_DT_UNDEF) {
+        rd.src_scale = *scale;
+        ra.src_scale = scale_p;
+    }
+    if (zp && zp->dt != MI355_DT_UNDEF) {
+        rd.src_zp = *zp;
+        ra.src_zp = zp_p;
+    }
     if (const int st = mi355_reorder_launch(&rd, &ra, stream)) return st;
     if (ld > cols) {
         const long units = dt_bits(to) / 16; // 16-bit words per element
@@ -244,8 +280,9 @@ int h16_launch(const mi355_matmul_desc_t &d, const problem_t &P_in, void *scratc
     }
     if (plan.copy_wei) {
         if (const int st = h16_convert(P.wei, d.wei_dt, plan.Bw, d.K, d.N, d.wei_stride, true, plan.op_dt, b_copy, plan.Kp,
-                    stream))
+                    stream, plan.woq ? &d.wei_scale : nullptr, P.wei_scale.p, plan.woq ? &d.wei_zp : nullptr, P.wei_zp.p))
             return st;
+        if (plan.woq) P.wei_scale.dt = P.wei_zp.dt = MI355_DT_UNDEF; // applied by the copy
         X.bt = b_copy;
         X.ldb = plan.Kp * EB;
         X.bt_bstride = plan.Bw > 1 ? d.N * plan.Kp * EB : 0;

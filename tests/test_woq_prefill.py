@@ -1,0 +1,91 @@
+"""Weight-only quantization beyond the decode kernels' 32 rows (prefill): bf16 src x
+s4 / u4 / s8 / u8 weights with scales and zero points along K and N, fpmath
+apply_to_int -- on hip:mfma_h16, whose weights copy is written by the reorder
+with the weights' scales and zero points as its parameters ((w - zp) * scale
+rounded to bf16: the flavour of the reference's JIT path,
+brgemm_matmul_copy_utils.cpp:2870-2896, the oracle's FLAG_WEI_BF16) and the
+16-bit tiles multiply.
+
+Exact data (small integer src, power-of-two scales: every decompressed weight
+and every partial sum is exact, in bf16 and in f32) must match the oracle bit for
+bit in either flavour; random data are held to the f32 summation bound around
+the oracle's float64 sum of the bf16-rounded weights."""
+import numpy as np
+import pytest
+
+from onednn_amd import cabi, configs
+from onednn_amd import dtypes as dtp
+from onednn_amd.problem import run_gpu
+from tests.helpers import assert_bit_exact, assert_gemm_close
+
+
+def exact(p, seed=0):
+    """small integer src; scales replaced by powers of two of the same type"""
+    r = np.random.default_rng(seed)
+    p.src = dtp.f32_to_bf16(r.integers(-4, 5, size=p.M * p.K).astype(np.float32)).reshape(p.M, p.K)
+    if "wei_scale" in p.quant:
+        q = p.quant["wei_scale"]
+        v = (2.0 ** r.integers(-6, -1, size=np.asarray(q.data).size)).astype(np.float32)
+        q.data = {cabi.DT_F32: v, cabi.DT_BF16: dtp.f32_to_bf16(v),
+                  cabi.DT_F16: v.astype(np.float16).view(np.uint16)}[q.dt].reshape(np.asarray(q.data).shape)
+    return p
+
+
+def test_dispatch_rules():
+    p = configs.woq_variant(64, 256, 256, 128)
+    st, impl = cabi.query(p.desc())
+    assert st == cabi.SUCCESS and impl == cabi.IMPL_H16_MFMA
+    assert cabi.scratch_bytes(p.desc()) == 256 * 256 * 2                       # the decompressed weights, K-contiguous
+    assert cabi.query(configs.woq_variant(32, 256, 256, 128).desc())[1] == cabi.IMPL_WOQ_GEMV   # decode sizes stay
+    p = configs.woq_variant(64, 256, 256, 128)
+    p.apply_to_int = False
+    assert cabi.query(p.desc())[1] != cabi.IMPL_H16_MFMA
+
+
+VARIANTS = [
+    dict(),                                                       # u4, bf16 scales and u4 zero points per group of 128
+    dict(wei_dt="s4", sc_dt="f32", zp_dt="s8"),
+    dict(sc_dt="f16", zp_dt="s32", zp_kind="column"),
+    dict(sc_kind="column", zp_kind="common", zp_dt="u8"),
+    dict(zp_kind="none"),
+    dict(sc_kind="none", zp_kind="none"),
+    dict(dst_dt="f32", relu_bias=True),
+]
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("kw", VARIANTS, ids=[str(i) for i in range(len(VARIANTS))])
+@pytest.mark.parametrize("shape", [(64, 256, 256, 128), (300, 192, 512, 64), (33, 130, 96, 32)])
+def test_exact_data_bit_exact(gpu, oracle, kw, shape):
+    M, N, K, G = shape
+    p = exact(configs.woq_variant(M, N, K, G, **kw), seed=M)
+    got, name = run_gpu(p)
+    assert name.startswith("hip:mfma_h16"), name
+    assert_bit_exact(p, got, oracle.run_oracle(p), name)
+    assert_bit_exact(p, got, oracle.run_oracle(p, flags=oracle.FLAG_WEI_BF16), name)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("wtag", ["ab", "ba"])
+def test_c2_shape_at_prefill_sizes(gpu, oracle, wtag):
+    """the decode configuration's tensors at M = 256 (N and K reduced): random data against the float64 sum of the
+    bf16-rounded weights"""
+    p = configs.config2(M=256, N=1024, K=1024, wtag=wtag)
+    p.dst_dt = cabi.DT_F32
+    got, name = run_gpu(p)
+    assert name.startswith("hip:mfma_h16"), name
+    _, ideal, asum = oracle.run_oracle(p, flags=oracle.FLAG_WEI_BF16, want_ideal=True)
+    assert_gemm_close(p, got, ideal, asum, what=name)
+
+
+@pytest.mark.gpu
+def test_int8_weights(gpu, oracle):
+    M, N, K = 128, 192, 256
+    r = np.random.default_rng(5)
+    p = configs.woq_variant(M, N, K, 128, sc_dt="f32", zp_dt="s8")
+    p.wei_dt = cabi.DT_S8
+    p.wei = r.integers(-128, 128, size=(K, N), dtype=np.int8)
+    p = exact(p, seed=6)
+    got, name = run_gpu(p)
+    assert name.startswith("hip:mfma_h16"), name
+    assert_bit_exact(p, got, oracle.run_oracle(p), name)
