@@ -113,6 +113,134 @@ __global__ void __launch_bounds__(256) h16_zero_tail_kernel(uint16_t *base, long
     for (long i = (long)blockIdx.x * 256 + threadIdx.x; i < total; i += (long)gridDim.x * 256)
         base[(i / per) * pitch16 + from16 + i % per] = 0;
 }
+
+// Decompression of row-major 4-bit weights [K][N] (two n per byte, low nibble = even n) into the K-contiguous 16-bit
+// copy the tiles read, [N][K]: value = (w - zp[k / gk][n]) * scale[k / gk][n], the reorder's arithmetic (integer
+// subtraction, one f32 multiplication, round to nearest even).  A workgroup owns 64 k x 256 n: a thread loads the
+// 16 bytes (32 columns) of two adjacent k rows -- eight lanes a whole 128-byte line -- with the scales and zero
+// points of its columns, packs the two k of a column into one dword and parks it in LDS at dword column
+// (k / 2) ^ 4 (n / 32) of row n, which spreads a store instruction over all banks and keeps every aligned group of
+// four columns together; the tile then leaves as whole 128-byte rows.  The generic tiled reorder took 0.36 ms for
+// 4096 x 14336 weights with grouped parameters; this kernel moves the same 29 MB in and 117 MB out.
+struct woq_dq_t {
+    const uint8_t *wei;  // [K][ldw / 2] bytes
+    uint16_t *out;       // [N][ldo]
+    const void *sc, *zp; // [K / gk or 1][N or 1], null = absent
+    long ldw, ldo;       // elements
+    int K, N;
+    int sc_dt, zp_dt;
+    int sc_gk, zp_gk;    // rows of k per parameter row; 0 = one row for all k
+    int sc_per_n, zp_per_n;
+    int signed_w, out_bf16;
+};
+
+typedef uint32_t woq_u4v __attribute__((ext_vector_type(4)));
+
+// the parameters of 32 consecutive columns into registers, 16 bytes a load (idx is a multiple of 32 and the base
+// 16-byte aligned whenever per_n is set)
+__device__ __forceinline__ void woq_scales32(float (&sc)[32], const void *p, int dt, long idx, bool per_n) {
+    if (!p || !per_n) {
+        const float v = p ? load_float(dt, p, idx) : 1.f;
+#pragma unroll
+        for (int e = 0; e < 32; ++e) sc[e] = v;
+    } else if (dt == MI355_DT_F32) {
+        const woq_u4v *q = (const woq_u4v *)((const float *)p + idx);
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+            const woq_u4v v = q[j];
+            sc[4 * j] = __uint_as_float(v.x), sc[4 * j + 1] = __uint_as_float(v.y);
+            sc[4 * j + 2] = __uint_as_float(v.z), sc[4 * j + 3] = __uint_as_float(v.w);
+        }
+    } else {
+        const woq_u4v *q = (const woq_u4v *)((const uint16_t *)p + idx);
+        const bool bf = dt == MI355_DT_BF16;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const woq_u4v v = q[j];
+            const uint32_t d[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const uint16_t lo = (uint16_t)d[i], hi = (uint16_t)(d[i] >> 16);
+                sc[8 * j + 2 * i] = bf ? __uint_as_float((uint32_t)lo << 16) : (float)__builtin_bit_cast(_Float16, lo);
+                sc[8 * j + 2 * i + 1] = bf ? __uint_as_float((uint32_t)hi << 16) : (float)__builtin_bit_cast(_Float16, hi);
+            }
+        }
+    }
+}
+
+__device__ __forceinline__ void woq_zps32(int (&zp)[32], const void *p, int dt, long idx, bool per_n) {
+    if (!p || !per_n) {
+        const int v = p ? load_int(dt, p, idx) : 0;
+#pragma unroll
+        for (int e = 0; e < 32; ++e) zp[e] = v;
+    } else if (dt == MI355_DT_S32) {
+        const woq_u4v *q = (const woq_u4v *)((const int *)p + idx);
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+            const woq_u4v v = q[j];
+            zp[4 * j] = (int)v.x, zp[4 * j + 1] = (int)v.y, zp[4 * j + 2] = (int)v.z, zp[4 * j + 3] = (int)v.w;
+        }
+    } else if (dt == MI355_DT_S8 || dt == MI355_DT_U8) {
+        const woq_u4v *q = (const woq_u4v *)((const uint8_t *)p + idx);
+        const bool sg = dt == MI355_DT_S8;
+#pragma unroll
+        for (int j = 0; j < 2; ++j) {
+            const woq_u4v v = q[j];
+            const uint32_t d[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+            for (int e = 0; e < 16; ++e) {
+                const uint32_t b = (d[e >> 2] >> (8 * (e & 3))) & 255;
+                zp[16 * j + e] = sg ? (int)(int8_t)b : (int)b;
+            }
+        }
+    } else { // s4 / u4
+        const woq_u4v v = *(const woq_u4v *)((const uint8_t *)p + idx / 2);
+        const uint32_t d[4] = {v.x, v.y, v.z, v.w};
+        const bool sg = dt == MI355_DT_S4;
+#pragma unroll
+        for (int e = 0; e < 32; ++e) {
+            const uint32_t b = (d[e >> 3] >> (4 * (e & 7))) & 15;
+            zp[e] = sg ? (int)(b ^ 8) - 8 : (int)b;
+        }
+    }
+}
+
+__global__ void __launch_bounds__(256) woq_dequant_kernel(const woq_dq_t A) {
+    typedef woq_u4v u4v;
+    __shared__ __attribute__((aligned(16))) uint32_t tile[256 * 32];
+    const int t = threadIdx.x;
+    const int k0 = blockIdx.y * 64, n0 = blockIdx.x * 256;
+    const int c = t & 7, kp = t >> 3;            // columns n0 + 32 c .. + 31, rows k0 + 2 kp and + 1
+    const int nb = n0 + 32 * c;
+    const long k = k0 + 2 * kp;
+    const u4v w0 = __builtin_nontemporal_load((const u4v *)(A.wei + (k * A.ldw + nb) / 2));
+    const u4v w1 = __builtin_nontemporal_load((const u4v *)(A.wei + ((k + 1) * A.ldw + nb) / 2));
+    float sc[32];
+    int zp[32];
+    woq_scales32(sc, A.sc, A.sc_dt, (A.sc_gk ? (k / A.sc_gk) * (long)(A.sc_per_n ? A.N : 1) : 0) + (A.sc_per_n ? nb : 0),
+            A.sc_per_n);
+    woq_zps32(zp, A.zp, A.zp_dt, (A.zp_gk ? (k / A.zp_gk) * (long)(A.zp_per_n ? A.N : 1) : 0) + (A.zp_per_n ? nb : 0),
+            A.zp_per_n);
+    const uint32_t d0[4] = {w0.x, w0.y, w0.z, w0.w}, d1[4] = {w1.x, w1.y, w1.z, w1.w};
+    const int sx = A.signed_w ? 8 : 0; // (b ^ 8) - 8 sign-extends a nibble
+#pragma unroll
+    for (int e = 0; e < 32; ++e) {
+        const int v0 = (int)(((d0[e >> 3] >> (4 * (e & 7))) & 15) ^ sx) - sx;
+        const int v1 = (int)(((d1[e >> 3] >> (4 * (e & 7))) & 15) ^ sx) - sx;
+        const float f0 = sc[e] * (float)(v0 - zp[e]), f1 = sc[e] * (float)(v1 - zp[e]);
+        const unsigned lo = A.out_bf16 ? f32_to_bf16(f0) : f32_to_f16(f0), hi = A.out_bf16 ? f32_to_bf16(f1) : f32_to_f16(f1);
+        tile[(32 * c + e) * 32 + (kp ^ (4 * c))] = lo | (hi << 16);
+    }
+    __syncthreads();
+    const int q = t & 7, r = t >> 3; // write: row r + 32 pass, dwords of the physical group q
+#pragma unroll
+    for (int pass = 0; pass < 8; ++pass) {
+        const int row = r + 32 * pass, cc = row >> 5;
+        const u4v v = *(const u4v *)&tile[row * 32 + 4 * q];
+        // physical group q of this row holds the logical dword columns 4 (q ^ cc) .. + 3, i.e. k0 + 8 (q ^ cc) .. + 7
+        __builtin_nontemporal_store(v, (u4v *)(A.out + (long)(n0 + row) * A.ldo + k0 + 8 * (q ^ cc)));
+    }
+}
 } // namespace
 
 // f32 operands under fpmath_mode bf16 / f16 / any (dnnl_fpmath_mode_t 1 / 2 / 3): the attribute allows an implicit
@@ -191,6 +319,23 @@ static bool h16_woq(const mi355_matmul_desc_t &d) {
             return false;
     // 4-bit weights: whole bytes along the contiguous dim
     if (dt_bits(d.wei_dt) == 4 && ((d.wei_stride[2] == 1 ? d.N : d.K) % 2)) return false;
+    return true;
+}
+
+// the dedicated kernel's conditions: row-major 4-bit weights of one batch, whole tiles, parameters per tensor, per
+// column, or per group of whole tiles of k and column
+static bool h16_woq_fast(const mi355_matmul_desc_t &d, const h16_plan_t &p) {
+    if (!p.woq || dt_bits(d.wei_dt) != 4 || p.Bw != 1 || p.Kp != d.K) return false;
+    if (d.wei_stride[2] != 1 || d.wei_stride[1] % 32 != 0 || d.K % 64 != 0 || d.N % 256 != 0) return false;
+    if (d.K >= (1L << 31) || d.N >= (1L << 31)) return false;
+    for (const mi355_quant_t *q : {&d.wei_scale, &d.wei_zp}) {
+        if (q->dt == MI355_DT_UNDEF) continue;
+        const int m = q->mask & 6;
+        if ((q->mask & 1) || q->group[1] != 1) return false;
+        if (m == 2) return false;                            // per k only
+        if ((m & 2) && (q->group[0] < 64 || q->group[0] % 64 != 0)) return false; // a parameter row covers whole tiles of k
+        if (dt_bits(q->dt) == 4 && (m & 4) && d.N % 2) return false;
+    }
     return true;
 }
 
@@ -278,10 +423,31 @@ int h16_launch(const mi355_matmul_desc_t &d, const problem_t &P_in, void *scratc
         P.src = a_copy;
         P.ss[0] = plan.Bs > 1 ? d.M * plan.Kp : 0; P.ss[1] = plan.Kp; P.ss[2] = 1;
     }
-    if (plan.copy_wei) {
+    if (plan.copy_wei && h16_woq_fast(d, plan) && (((uintptr_t)P.wei | (uintptr_t)P.wei_scale.p | (uintptr_t)P.wei_zp.p) & 15) == 0) {
+        woq_dq_t A {};
+        A.wei = (const uint8_t *)P.wei;
+        A.out = (uint16_t *)b_copy;
+        A.ldw = d.wei_stride[1];
+        A.ldo = plan.Kp;
+        A.K = (int)d.K; A.N = (int)d.N;
+        auto param = [&](const mi355_quant_t &q, const void *ptr, const void *&p_, int &dt, int &gk, int &per_n) {
+            p_ = q.dt != MI355_DT_UNDEF ? ptr : nullptr;
+            dt = q.dt;
+            gk = (q.mask & 2) ? (int)q.group[0] : 0;
+            per_n = (q.mask & 4) ? 1 : 0;
+        };
+        param(d.wei_scale, P.wei_scale.p, A.sc, A.sc_dt, A.sc_gk, A.sc_per_n);
+        param(d.wei_zp, P.wei_zp.p, A.zp, A.zp_dt, A.zp_gk, A.zp_per_n);
+        A.signed_w = d.wei_dt == MI355_DT_S4;
+        A.out_bf16 = plan.op_dt == MI355_DT_BF16;
+        hipLaunchKernelGGL(woq_dequant_kernel, dim3((unsigned)(d.N / 256), (unsigned)(d.K / 64)), dim3(256), 0, stream, A);
+        if (hipGetLastError() != hipSuccess) return MI355_RUNTIME_ERROR;
+    } else if (plan.copy_wei) {
         if (const int st = h16_convert(P.wei, d.wei_dt, plan.Bw, d.K, d.N, d.wei_stride, true, plan.op_dt, b_copy, plan.Kp,
                     stream, plan.woq ? &d.wei_scale : nullptr, P.wei_scale.p, plan.woq ? &d.wei_zp : nullptr, P.wei_zp.p))
             return st;
+    }
+    if (plan.copy_wei) {
         if (plan.woq) P.wei_scale.dt = P.wei_zp.dt = MI355_DT_UNDEF; // applied by the copy
         X.bt = b_copy;
         X.ldb = plan.Kp * EB;

@@ -55,8 +55,9 @@ VARIANTS = [
 
 @pytest.mark.gpu
 @pytest.mark.parametrize("kw", VARIANTS, ids=[str(i) for i in range(len(VARIANTS))])
-@pytest.mark.parametrize("shape", [(64, 256, 256, 128), (300, 192, 512, 64), (33, 130, 96, 32)])
+@pytest.mark.parametrize("shape", [(64, 256, 256, 128), (300, 192, 512, 64), (33, 130, 96, 32), (96, 512, 384, 64)])
 def test_exact_data_bit_exact(gpu, oracle, kw, shape):
+    """N in whole 256s with K in whole 64s takes the dedicated decompression kernel, everything else the reorder"""
     M, N, K, G = shape
     p = exact(configs.woq_variant(M, N, K, G, **kw), seed=M)
     got, name = run_gpu(p)
@@ -76,6 +77,20 @@ def test_c2_shape_at_prefill_sizes(gpu, oracle, wtag):
     assert name.startswith("hip:mfma_h16"), name
     _, ideal, asum = oracle.run_oracle(p, flags=oracle.FLAG_WEI_BF16, want_ideal=True)
     assert_gemm_close(p, got, ideal, asum, what=name)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("shape", [(64, 256, 256, 128), (40, 200, 96, 32)])
+def test_f16_src(gpu, oracle, shape):
+    """f16 src: the weights are decompressed to f16 (exact data, so the oracle's f32 weights are the same numbers)"""
+    M, N, K, G = shape
+    p = exact(configs.woq_variant(M, N, K, G, sc_dt="f16", zp_dt="s8", dst_dt="f32"), seed=3)
+    p.src_dt = cabi.DT_F16
+    p.src = dtp.bf16_to_f32(p.src).astype(np.float16).view(np.uint16).reshape(M, K)
+    p.fpmath_mode = 2
+    got, name = run_gpu(p)
+    assert name.startswith("hip:mfma_h16"), name
+    assert_bit_exact(p, got, oracle.run_oracle(p), name)
 
 
 @pytest.mark.gpu
