@@ -67,7 +67,7 @@ def config2(M=1, N=14336, K=4096, group=128, seed=2, impl=cabi.IMPL_AUTO, wtag="
 
 
 def woq_variant(M, N, K, group, wei_dt="u4", sc_dt="bf16", zp_dt="u4", zp_kind="grouped", sc_kind="grouped",
-                dst_dt="bf16", relu_bias=False, seed=12):
+                dst_dt="bf16", relu_bias=False, seed=12, wtag="ab"):
     """Weight-only int4 decode in the attribute combinations the reference admits
     (matmul_pd.hpp:131-226): s4 / u4 weights; f32 / bf16 / f16 scales, grouped
     along K or per column; s32 / s8 / u8 / s4 / u4 zero points, grouped, per
@@ -76,7 +76,7 @@ def woq_variant(M, N, K, group, wei_dt="u4", sc_dt="bf16", zp_dt="u4", zp_kind="
              "u8": cabi.DT_U8, "s4": cabi.DT_S4, "u4": cabi.DT_U4}
     src = dtp.f32_to_bf16(_rng(seed, 1).standard_normal((M, K)).astype(np.float32))
     codes = _rng(seed, 2).integers(0, 16, size=(K, N), dtype=np.uint8)  # raw nibbles, s4 reads them as signed
-    wei = dtp.pack_nibbles(codes)
+    wei = dtp.pack_nibbles(codes if wtag == "ab" else codes.T.copy())   # two n, or two k, per byte
     G = K // group
 
     def shaped(kind):
@@ -102,8 +102,8 @@ def woq_variant(M, N, K, group, wei_dt="u4", sc_dt="bf16", zp_dt="u4", zp_kind="
         kw["bias"] = _rng(seed, 5).uniform(-1, 1, size=N).astype(np.float32)
         kw["post_ops"] = [PostOp(kind=cabi.PO_ELTWISE, alg=cabi.ELTWISE["relu"], alpha=0.0, beta=0.0, scale=1.0)]
     return MatmulProblem(M=M, N=N, K=K, src_dt=cabi.DT_BF16, wei_dt=names[wei_dt], dst_dt=names[dst_dt], src=src,
-                         wei=wei, wei_stride=strides_for("ab", 1, K, N), quant=quant, apply_to_int=True,
-                         fpmath_mode=1, name=f"WOQ-{wei_dt}-{sc_dt}/{sc_kind}-{zp_dt}/{zp_kind}-M{M}", **kw)
+                         wei=wei, wei_stride=strides_for(wtag, 1, K, N), quant=quant, apply_to_int=True,
+                         fpmath_mode=1, name=f"WOQ-{wei_dt}-{sc_dt}/{sc_kind}-{zp_dt}/{zp_kind}-M{M}-{wtag}", **kw)
 
 
 def config3(M=8192, N=8192, K=8192, seed=3, impl=cabi.IMPL_AUTO, wtag="ab",

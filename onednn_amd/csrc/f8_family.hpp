@@ -318,7 +318,7 @@ __global__ void __launch_bounds__(Mma::G::NT) __attribute__((amdgpu_waves_per_eu
     }
     // the epilogue's per-column operands go into their LDS table now: the loads
     // hide behind the pipeline prologue
-    const unsigned ntab = (unsigned)(size_t)(__attribute__((address_space(3))) char *)smem + NSTAGE * G::STAGE_BYTES;
+    const unsigned ntab = (unsigned)(size_t)(__attribute__((address_space(3))) char *)smem + G::NSTAGE * G::STAGE_BYTES;
     fill_ntab<G::NT>(P, cv, ntab, b, n0);
 
     typename acc_of<Mma>::type acc[Mma::ROWS][Mma::COLS];
@@ -329,7 +329,7 @@ __global__ void __launch_bounds__(Mma::G::NT) __attribute__((amdgpu_waves_per_eu
 #pragma unroll
             for (int r = 0; r < acc_of<Mma>::N; ++r) acc[i][j][r] = 0.f;
 
-    main_loop<NSTAGE, KSTEP, Mma>(acc, smem, A, Bt, lda, X.ldb, P.M - m0,
+    main_loop<G::NSTAGE, KSTEP, Mma>(acc, smem, A, Bt, lda, X.ldb, P.M - m0,
             P.N - n0, (int)(P.K * EB / (BKB * KSTEP)), f8_ctx_t {});
 
     store_quadrant<typename acc_of<Mma>::layout, G::WCOLS>(P, smem, ntab, acc, b, m0 + wm * 128, n0 + wn * G::WCOLS,

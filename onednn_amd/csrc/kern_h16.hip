@@ -241,6 +241,42 @@ __global__ void __launch_bounds__(256) woq_dequant_kernel(const woq_dq_t A) {
         __builtin_nontemporal_store(v, (u4v *)(A.out + (long)(n0 + row) * A.ldo + k0 + 8 * (q ^ cc)));
     }
 }
+
+// The same for K-contiguous 4-bit weights [N][K] (two k per byte): no transposition.  A workgroup owns 256 k x 32 n;
+// thread (c = t % 8, r = t / 8) takes the dwords c, c + 8, c + 16, c + 24 of row r's 128 bytes, so that the eight
+// lanes of a row write 128 contiguous bytes with every store instruction (the reads, a quarter of the traffic, come
+// in 32-byte pieces instead).  The eight k of a dword share their parameters (groups along k are multiples of 64).
+__global__ void __launch_bounds__(256) woq_dequant_kmajor_kernel(const woq_dq_t A) {
+    const int t = threadIdx.x, c = t & 7;
+    const int n = blockIdx.y * 32 + (t >> 3);
+    if (n >= A.N) return;
+    const long k0 = (long)blockIdx.x * 256;
+    const uint32_t *row = (const uint32_t *)(A.wei + ((long)n * A.ldw + k0) / 2);
+    uint32_t d[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) d[j] = __builtin_nontemporal_load(row + c + 8 * j);
+    const int sx = A.signed_w ? 8 : 0;
+    long sg = -1, zg = -1;
+    float sc = 1.f;
+    int zp = 0;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        const long k = k0 + 8 * (c + 8 * j);
+        const long sgj = A.sc_gk ? k / A.sc_gk : 0, zgj = A.zp_gk ? k / A.zp_gk : 0;
+        if (A.sc && sgj != sg) sc = load_float(A.sc_dt, A.sc, sgj * (A.sc_per_n ? A.N : 1) + (A.sc_per_n ? n : 0)), sg = sgj;
+        if (A.zp && zgj != zg) zp = load_int(A.zp_dt, A.zp, zgj * (A.zp_per_n ? A.N : 1) + (A.zp_per_n ? n : 0)), zg = zgj;
+        uint32_t h[8];
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+            const int v = (int)(((d[j] >> (4 * e)) & 15) ^ sx) - sx;
+            const float f = sc * (float)(v - zp);
+            h[e] = A.out_bf16 ? f32_to_bf16(f) : f32_to_f16(f);
+        }
+        woq_u4v o;
+        o.x = h[0] | (h[1] << 16), o.y = h[2] | (h[3] << 16), o.z = h[4] | (h[5] << 16), o.w = h[6] | (h[7] << 16);
+        __builtin_nontemporal_store(o, (woq_u4v *)(A.out + (long)n * A.ldo + k));
+    }
+}
 } // namespace
 
 // f32 operands under fpmath_mode bf16 / f16 / any (dnnl_fpmath_mode_t 1 / 2 / 3): the attribute allows an implicit
@@ -322,21 +358,22 @@ static bool h16_woq(const mi355_matmul_desc_t &d) {
     return true;
 }
 
-// the dedicated kernel's conditions: row-major 4-bit weights of one batch, whole tiles, parameters per tensor, per
-// column, or per group of whole tiles of k and column
-static bool h16_woq_fast(const mi355_matmul_desc_t &d, const h16_plan_t &p) {
-    if (!p.woq || dt_bits(d.wei_dt) != 4 || p.Bw != 1 || p.Kp != d.K) return false;
-    if (d.wei_stride[2] != 1 || d.wei_stride[1] % 32 != 0 || d.K % 64 != 0 || d.N % 256 != 0) return false;
-    if (d.K >= (1L << 31) || d.N >= (1L << 31)) return false;
+// the dedicated kernels' conditions: 4-bit weights of one batch in whole tiles (row-major: 64 k x 256 n, returns 1;
+// K-contiguous: K in whole 256s, returns 2), parameters per tensor, per column, or per group of whole 64s of k and
+// column; 0 = the reorder
+static int h16_woq_fast(const mi355_matmul_desc_t &d, const h16_plan_t &p) {
+    if (!p.woq || dt_bits(d.wei_dt) != 4 || p.Bw != 1 || p.Kp != d.K) return 0;
+    if (d.K >= (1L << 31) || d.N >= (1L << 31)) return 0;
     for (const mi355_quant_t *q : {&d.wei_scale, &d.wei_zp}) {
         if (q->dt == MI355_DT_UNDEF) continue;
         const int m = q->mask & 6;
-        if ((q->mask & 1) || q->group[1] != 1) return false;
-        if (m == 2) return false;                            // per k only
-        if ((m & 2) && (q->group[0] < 64 || q->group[0] % 64 != 0)) return false; // a parameter row covers whole tiles of k
-        if (dt_bits(q->dt) == 4 && (m & 4) && d.N % 2) return false;
+        if ((q->mask & 1) || q->group[1] > 1) return 0;
+        if (m == 2) return 0;                                                       // per k only
+        if ((m & 2) && (q->group[0] < 64 || q->group[0] % 64 != 0)) return 0;       // whole 64s of k share a parameter
     }
-    return true;
+    if (d.wei_stride[2] == 1 && d.wei_stride[1] % 32 == 0 && d.K % 64 == 0 && d.N % 256 == 0) return 1;
+    if (d.wei_stride[1] == 1 && d.wei_stride[2] % 8 == 0 && d.K % 256 == 0 && (d.N + 31) / 32 <= 65535) return 2;
+    return 0;
 }
 
 int h16_supported(const mi355_matmul_desc_t &d) {
@@ -423,11 +460,14 @@ int h16_launch(const mi355_matmul_desc_t &d, const problem_t &P_in, void *scratc
         P.src = a_copy;
         P.ss[0] = plan.Bs > 1 ? d.M * plan.Kp : 0; P.ss[1] = plan.Kp; P.ss[2] = 1;
     }
-    if (plan.copy_wei && h16_woq_fast(d, plan) && (((uintptr_t)P.wei | (uintptr_t)P.wei_scale.p | (uintptr_t)P.wei_zp.p) & 15) == 0) {
+    const int fast = plan.copy_wei ? h16_woq_fast(d, plan) : 0;
+    const uintptr_t align = fast == 1 ? ((uintptr_t)P.wei | (uintptr_t)P.wei_scale.p | (uintptr_t)P.wei_zp.p) & 15
+                                      : (uintptr_t)P.wei & 3;
+    if (fast && align == 0) {
         woq_dq_t A {};
         A.wei = (const uint8_t *)P.wei;
         A.out = (uint16_t *)b_copy;
-        A.ldw = d.wei_stride[1];
+        A.ldw = fast == 1 ? d.wei_stride[1] : d.wei_stride[2];
         A.ldo = plan.Kp;
         A.K = (int)d.K; A.N = (int)d.N;
         auto param = [&](const mi355_quant_t &q, const void *ptr, const void *&p_, int &dt, int &gk, int &per_n) {
@@ -440,7 +480,11 @@ int h16_launch(const mi355_matmul_desc_t &d, const problem_t &P_in, void *scratc
         param(d.wei_zp, P.wei_zp.p, A.zp, A.zp_dt, A.zp_gk, A.zp_per_n);
         A.signed_w = d.wei_dt == MI355_DT_S4;
         A.out_bf16 = plan.op_dt == MI355_DT_BF16;
-        hipLaunchKernelGGL(woq_dequant_kernel, dim3((unsigned)(d.N / 256), (unsigned)(d.K / 64)), dim3(256), 0, stream, A);
+        if (fast == 1)
+            hipLaunchKernelGGL(woq_dequant_kernel, dim3((unsigned)(d.N / 256), (unsigned)(d.K / 64)), dim3(256), 0, stream, A);
+        else
+            hipLaunchKernelGGL(woq_dequant_kmajor_kernel, dim3((unsigned)(d.K / 256), (unsigned)((d.N + 31) / 32)), dim3(256),
+                    0, stream, A);
         if (hipGetLastError() != hipSuccess) return MI355_RUNTIME_ERROR;
     } else if (plan.copy_wei) {
         if (const int st = h16_convert(P.wei, d.wei_dt, plan.Bw, d.K, d.N, d.wei_stride, true, plan.op_dt, b_copy, plan.Kp,
@@ -461,6 +505,21 @@ int h16_launch(const mi355_matmul_desc_t &d, const problem_t &P_in, void *scratc
     P.K = plan.Kp; // the padding multiplies zeros by zeros
     X.tiles_m = (int)((d.M + BM - 1) / BM);
     X.tiles_n = (int)((d.N + f8_geo_t::BN - 1) / f8_geo_t::BN);
+    // Few tiles (prefill at a few hundred rows): 256 x 128 tiles of four wavefronts, two workgroups a CU, put twice
+    // the CUs to work; a wavefront's part, 128 x 64, and with it the fragments and the epilogue are the same.
+    using narrow_t = geo_t<4, 128>;
+    if (plan.op_dt != MI355_DT_F32 && (long)X.tiles_m * X.tiles_n * d.batch <= 128 && d.N > 128) {
+        X.tiles_n = (int)((d.N + narrow_t::BN - 1) / narrow_t::BN);
+        dim3 grid((unsigned)(X.tiles_m * X.tiles_n), 1, (unsigned)d.batch);
+        constexpr int smem_bytes = narrow_t::NSTAGE * narrow_t::STAGE_BYTES + NTAB_BYTES;
+        auto go = [&](auto kern) -> int {
+            if (const int st = ensure_dynamic_lds((const void *)kern, smem_bytes, "mfma_h16")) return st;
+            hipLaunchKernelGGL(kern, grid, dim3(narrow_t::NT), smem_bytes, stream, P, X);
+            return hipGetLastError() == hipSuccess ? MI355_SUCCESS : MI355_RUNTIME_ERROR;
+        };
+        if (plan.op_dt == MI355_DT_BF16) return go(f8_gemm_kernel<h16x16_mma_t<true, narrow_t>>);
+        return go(f8_gemm_kernel<h16x16_mma_t<false, narrow_t>>);
+    }
     dim3 grid((unsigned)(X.tiles_m * X.tiles_n), 1, (unsigned)d.batch);
     constexpr int smem_bytes = NSTAGE * f8_geo_t::STAGE_BYTES + NTAB_BYTES;
     auto go = [&](auto kern) -> int {

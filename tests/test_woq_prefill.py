@@ -80,6 +80,19 @@ def test_c2_shape_at_prefill_sizes(gpu, oracle, wtag):
 
 
 @pytest.mark.gpu
+@pytest.mark.parametrize("kw", VARIANTS, ids=[str(i) for i in range(len(VARIANTS))])
+@pytest.mark.parametrize("shape", [(64, 72, 512, 64), (80, 300, 768, 256), (48, 96, 192, 64)])
+def test_k_contiguous_weights(gpu, oracle, kw, shape):
+    """two k per byte: K in whole 256s takes the dedicated kernel without the transposition, the last shape the reorder"""
+    M, N, K, G = shape
+    p = exact(configs.woq_variant(M, N, K, G, wtag="ba", **kw), seed=N)
+    got, name = run_gpu(p)
+    assert name.startswith("hip:mfma_h16"), name
+    assert_bit_exact(p, got, oracle.run_oracle(p), name)
+    assert_bit_exact(p, got, oracle.run_oracle(p, flags=oracle.FLAG_WEI_BF16), name)
+
+
+@pytest.mark.gpu
 @pytest.mark.parametrize("shape", [(64, 256, 256, 128), (40, 200, 96, 32)])
 def test_f16_src(gpu, oracle, shape):
     """f16 src: the weights are decompressed to f16 (exact data, so the oracle's f32 weights are the same numbers)"""
