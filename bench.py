@@ -26,6 +26,8 @@ Workloads (the benchmark configurations):
   h1  bf16 x bf16 -> bf16, M=N=K=8192 (MFMA bf16 bound; the unquantized matmul on the same tiles)
   h2  f32 x f32 -> f32, M=N=K=8192 (MFMA f32 bound)
   c1  u8 x s8 -> f32, 256 x 1024 x 1024 (latency bound, no roofline claim)
+Among the side workloads of a default run, p2 is C2's tensors at prefill sizes (M = 512 / 2048): the step includes
+the decompression of the 4-bit weights into the bf16 copy the tiles read (MFMA bf16 bound).
 """
 import argparse
 import ctypes as C
@@ -126,6 +128,8 @@ def build_problem(name, M=None, wtag="any"):
         if wtag == "any":  # what format_tag::any resolves to for decode weights
             p.wei_packing = cabi.WEI_PACK_WOQ64
         return p
+    if name == "p2":  # C2's tensors at prefill size: the weights are decompressed into a bf16 copy inside every launch
+        return configs.config2(M=M or 2048, wtag="ab" if wtag == "any" else wtag)
     mfma_tag = "ba" if wtag == "any" else wtag
     if name == "c3":
         return configs.config3(wtag=mfma_tag)
@@ -164,7 +168,7 @@ def algorithmic(name, p):
         return ops, "TFLOP/s", "mfma", PEAK_F8_TFLOPS
     if name == "c5":
         return ops, "TFLOP/s", "mfma", PEAK_F4_TFLOPS
-    if name == "h1":
+    if name in ("h1", "p2"):
         return ops, "TFLOP/s", "mfma", PEAK_BF16_TFLOPS
     if name == "h2":
         return ops, "TFLOP/s", "mfma", PEAK_F32_TFLOPS
@@ -612,7 +616,7 @@ def main():
         # layout change then runs inside every launch
         plan = [("c2", 1, "any"), ("c2", 8, "any"), ("c2", 32, "any"), ("c3", None, "any"), ("c3", None, "ab"),
                 ("c4", None, "any"), ("c4mx", None, "any"), ("c5", None, "any"), ("c1", None, "any"),
-                ("m1", None, "any"), ("h1", None, "any"), ("h2", None, "any")]
+                ("m1", None, "any"), ("h1", None, "any"), ("h2", None, "any"), ("p2", 512, "any"), ("p2", 2048, "any")]
         for nm, m, wt in plan:
             if nm == main_name and wt == args.wtag and (nm != "c2" or m == args.decode_m):
                 continue
