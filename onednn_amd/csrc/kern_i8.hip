@@ -242,7 +242,7 @@ __global__ void __launch_bounds__(G::NT) __attribute__((amdgpu_waves_per_eu(G::N
     cv.rowsum = X.rowsum ? X.rowsum + bs * P.M : nullptr;
     cv.colsum = X.colsum ? X.colsum + bw * P.N : nullptr;
     cv.has_comp = X.rowsum != nullptr || X.colsum != nullptr || cv.a_c != 0 || WEI_U8 || P.wei_zp.dt != MI355_DT_UNDEF;
-    const unsigned ntab = (unsigned)(size_t)(__attribute__((address_space(3))) char *)smem + NSTAGE * G::STAGE_BYTES;
+    const unsigned ntab = (unsigned)(size_t)(__attribute__((address_space(3))) char *)smem + G::NSTAGE * G::STAGE_BYTES;
     fill_ntab<G::NT>(P, cv, ntab, b, n0);
 
     v4i acc[Mma::ROWS][Mma::COLS];
@@ -253,7 +253,7 @@ __global__ void __launch_bounds__(G::NT) __attribute__((amdgpu_waves_per_eu(G::N
 #pragma unroll
             for (int r = 0; r < 4; ++r) acc[i][j][r] = 0;
 
-    main_loop<NSTAGE, 1, Mma>(acc, smem, A, Bt, lda, X.ldb, P.M - m0, P.N - n0,
+    main_loop<G::NSTAGE, 1, Mma>(acc, smem, A, Bt, lda, X.ldb, P.M - m0, P.N - n0,
             (int)(P.K / BK), i8_ctx_t {});
 
     store_quadrant<layout16_t, G::WCOLS>(P, smem, ntab, acc, b, m0 + wm * 128, n0 + wn * G::WCOLS, wn * G::WCOLS, cv);
@@ -447,10 +447,11 @@ i8_plan_t make_plan(const mi355_matmul_desc_t &d) {
     // quantization)
     const long big_tiles = ((d.M + BM - 1) / BM) * ((d.N + i8_geo_t::BN - 1) / i8_geo_t::BN) * d.batch;
     p.small = !d.dst_scale_dynamic && (big_tiles < 24 || d.K % BK != 0);
-    // MI355_I8_TILES=large|small overrides the choice where both can run (for
-    // tests and tuning; read at every call)
+    // MI355_I8_TILES=large|wide|small overrides the choice where both can run (for
+    // tests and tuning; read at every call): large = the LDS tiles, 256 x 128 or
+    // 256 x 256 by the number of tiles; wide = the 256 x 256 ones
     if (const char *force = getenv("MI355_I8_TILES")) {
-        if (!strcmp(force, "large") && d.K % BK == 0) p.small = false;
+        if ((!strcmp(force, "large") || !strcmp(force, "wide")) && d.K % BK == 0) p.small = false;
         if (!strcmp(force, "small") && !d.dst_scale_dynamic) p.small = true;
     }
     // a = off_s - zs can be non-zero whenever src is u8 or has a zero point;
@@ -561,6 +562,23 @@ int i8_launch(const mi355_matmul_desc_t &d, const problem_t &P, void *scratch,
     }
     X.tiles_m = (int)((d.M + BM - 1) / BM);
     X.tiles_n = (int)((d.N + i8_geo_t::BN - 1) / i8_geo_t::BN);
+    // Up to 128 large tiles leave half of the CUs or more idle: 256 x 128 tiles of four wavefronts, two workgroups a
+    // CU, put twice as many to work (a wavefront's part, 128 x 64, its fragments and the epilogue are the same).
+    // s8 weights only, to bound the build.  MI355_I8_TILES=wide keeps the 256 x 256 tiles.
+    using narrow_t = geo_t<4, 128>;
+    const char *force = getenv("MI355_I8_TILES");
+    if (!wu && (long)X.tiles_m * X.tiles_n * d.batch <= 128 && d.N > 128 && !(force && !strcmp(force, "wide"))) {
+        X.tiles_n = (int)((d.N + narrow_t::BN - 1) / narrow_t::BN);
+        dim3 grid((unsigned)(X.tiles_m * X.tiles_n), 1, (unsigned)d.batch);
+        constexpr int smem_bytes = narrow_t::NSTAGE * narrow_t::STAGE_BYTES + NTAB_BYTES;
+        auto go = [&](auto kern) -> int {
+            if (const int st = ensure_dynamic_lds((const void *)kern, smem_bytes, "mfma_i8")) return st;
+            hipLaunchKernelGGL(kern, grid, dim3(narrow_t::NT), smem_bytes, stream, P, X);
+            return hipGetLastError() == hipSuccess ? MI355_SUCCESS : MI355_RUNTIME_ERROR;
+        };
+        if (su) return go(i8_gemm_kernel<true, false, narrow_t>);
+        return go(i8_gemm_kernel<false, false, narrow_t>);
+    }
     dim3 grid((unsigned)(X.tiles_m * X.tiles_n), 1, (unsigned)d.batch);
     constexpr int smem_bytes = NSTAGE * i8_geo_t::STAGE_BYTES + NTAB_BYTES;
     auto go = [&](auto kern) -> int {

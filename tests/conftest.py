@@ -33,10 +33,13 @@ def gpu():
     return lib
 
 
-@pytest.fixture(params=["large", "small"])
+@pytest.fixture(params=["large", "wide", "small"])
 def i8_tiles(request, monkeypatch):
-    """Runs a test once per tile geometry of hip:mfma_i8 (the 256 x 256 LDS
-    tiles and the 32 x 32 direct ones) wherever both can take the problem; by
-    itself the dispatcher would give every small test shape to the small tiles."""
+    """Runs a test once per tile geometry of hip:mfma_i8 (the LDS tiles -- "large":
+    256 x 128 when a problem has few tiles, as all test shapes do; "wide": 256 x 256
+    -- and the 32 x 32 direct ones) wherever they can take the problem; by itself
+    the dispatcher would give every small test shape to the small tiles."""
     monkeypatch.setenv("MI355_I8_TILES", request.param)
+    if request.param == "wide":   # the fp8 family's switch between the same two LDS geometries
+        monkeypatch.setenv("MI355_F8_TILES", "wide")
     return request.param

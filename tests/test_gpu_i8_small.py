@@ -110,9 +110,25 @@ def test_both_tile_geometries_against_the_oracle_with_re_biased_operands(gpu, or
         w = np.asarray(want).view(np.int8)
         assert np.mean(np.abs(w.astype(np.int32)) < 127) > 0.9      # not saturated away
     outs = []
-    for tiles in ("large", "small"):
+    for tiles in ("large", "wide", "small"):
         monkeypatch.setenv("MI355_I8_TILES", tiles)
         got, name = run_gpu(p, cabi.IMPL_I8_MFMA)
         assert_bit_exact(p, got, want, f"{name} {tiles}")
         outs.append(np.asarray(got).copy())
-    assert np.array_equal(outs[0], outs[1])
+    assert np.array_equal(outs[0], outs[1]) and np.array_equal(outs[0], outs[2])
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("src_dt", [cabi.DT_S8, cabi.DT_U8])
+def test_mid_size_problems_on_the_dispatchers_own_choice(gpu, oracle, monkeypatch, src_dt):
+    """30 large tiles (24 to 128 take the 256 x 128 LDS tiles by themselves), ragged in M and N: against the oracle, and
+    the same bits from the 256 x 256 tiles"""
+    monkeypatch.delenv("MI355_I8_TILES", raising=False)
+    p = int8_problem(1500, 1100, 192, src_dt, cabi.DT_S8, cabi.DT_S8, src_zp=7 if src_dt == cabi.DT_U8 else None,
+                     dst_scale=40.0, bias=True)
+    want = oracle.run_oracle(p)
+    got, name = run_gpu(p, cabi.IMPL_I8_MFMA)
+    assert_bit_exact(p, got, want, name)
+    monkeypatch.setenv("MI355_I8_TILES", "wide")
+    wide, name = run_gpu(p, cabi.IMPL_I8_MFMA)
+    assert np.array_equal(np.asarray(got), np.asarray(wide))
