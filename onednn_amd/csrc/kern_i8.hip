@@ -440,13 +440,16 @@ i8_plan_t make_plan(const mi355_matmul_desc_t &d) {
     p.Bw = d.wei_stride[0] ? d.batch : 1;
     p.Bs = d.src_stride[0] ? d.batch : 1;
     p.need_transpose = !(d.wei_stride[1] == 1);
-    // the small tiles when the large ones would occupy less than a tenth of the
-    // device (measured with K = 1024 and 4096: 16 large tiles take 24 / 52 us
-    // against 18 / 40 us, 32 large tiles 55 us against 74), or cannot step
-    // through K (the small tiles compute their own sums and have no dynamic dst
-    // quantization)
+    // the small tiles when the LDS tiles would occupy too little of the device
+    // (measured with K = 1024 / 4096 against the 256 x 128 tiles, which take 16.7 /
+    // 35 us for anything up to 128 large tiles: the small tiles take 14.5 / 30.3 us
+    // at 12 large tiles, 17.2 / 37.5 at 16, 22.4 / 53.5 at 20; against the
+    // 256 x 256 tiles, all there is for u8 weights, they lose from 24 on), or when
+    // the LDS tiles cannot step through K (the small tiles compute their own sums
+    // and have no dynamic dst quantization)
     const long big_tiles = ((d.M + BM - 1) / BM) * ((d.N + i8_geo_t::BN - 1) / i8_geo_t::BN) * d.batch;
-    p.small = !d.dst_scale_dynamic && (big_tiles < 24 || d.K % BK != 0);
+    const long crossover = d.wei_dt == MI355_DT_U8 ? 24 : 16;
+    p.small = !d.dst_scale_dynamic && (big_tiles < crossover || d.K % BK != 0);
     // MI355_I8_TILES=large|wide|small overrides the choice where both can run (for
     // tests and tuning; read at every call): large = the LDS tiles, 256 x 128 or
     // 256 x 256 by the number of tiles; wide = the 256 x 256 ones
