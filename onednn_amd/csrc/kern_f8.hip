@@ -273,17 +273,9 @@ int f8_launch(const mi355_matmul_desc_t &d, const problem_t &P, void *scratch, h
     // Up to 128 tiles leave half of the CUs or more idle: 256 x 128 tiles of four wavefronts, two workgroups a CU, put
     // twice as many to work (a wavefront's part, 128 x 64, its fragments and the epilogue are the same).  e4m3 x e4m3
     // only, to bound the build.  MI355_F8_TILES=wide keeps the 256 x 256 tiles.
-    using narrow_t = geo_t<4, 128>;
     const char *force = getenv("MI355_F8_TILES");
-    if (!fa && !fb && (long)X.tiles_m * X.tiles_n * d.batch <= 128 && d.N > 128 && !(force && !strcmp(force, "wide"))) {
-        X.tiles_n = (int)((d.N + narrow_t::BN - 1) / narrow_t::BN);
-        const dim3 ngrid((unsigned)(X.tiles_m * X.tiles_n), 1, (unsigned)d.batch);
-        constexpr int nsmem = narrow_t::NSTAGE * narrow_t::STAGE_BYTES + NTAB_BYTES;
-        auto kern = f8_gemm_kernel<f8_mma_t<0, 0, narrow_t>>;
-        if (const int st = ensure_dynamic_lds((const void *)kern, nsmem, "mfma_f8")) return st;
-        hipLaunchKernelGGL(kern, ngrid, dim3(narrow_t::NT), nsmem, stream, P, X);
-        return hipGetLastError() == hipSuccess ? MI355_SUCCESS : MI355_RUNTIME_ERROR;
-    }
+    if (!fa && !fb && (long)X.tiles_m * X.tiles_n * d.batch <= 128 && d.N > 128 && !(force && !strcmp(force, "wide")))
+        return f8_launch_narrow_e4m3(P, X.bt, X.ldb, X.bt_bstride, (unsigned)d.batch, stream);
     if (fa && fb) return go(f8_gemm_kernel<f8_mma_t<1, 1, f8_geo_t>>);
     if (fa) return go(f8_gemm_kernel<f8_mma_t<1, 0, f8_geo_t>>);
     if (fb) return go(f8_gemm_kernel<f8_mma_t<0, 1, f8_geo_t>>);
