@@ -443,12 +443,11 @@ i8_plan_t make_plan(const mi355_matmul_desc_t &d) {
     // the small tiles when the LDS tiles would occupy too little of the device
     // (measured with K = 1024 / 4096 against the 256 x 128 tiles, which take 16.7 /
     // 35 us for anything up to 128 large tiles: the small tiles take 14.5 / 30.3 us
-    // at 12 large tiles, 17.2 / 37.5 at 16, 22.4 / 53.5 at 20; against the
-    // 256 x 256 tiles, all there is for u8 weights, they lose from 24 on), or when
-    // the LDS tiles cannot step through K (the small tiles compute their own sums
-    // and have no dynamic dst quantization)
+    // at 12 large tiles, 17.2 / 37.5 at 16, 22.4 / 53.5 at 20), or when the LDS
+    // tiles cannot step through K (the small tiles compute their own sums and have
+    // no dynamic dst quantization)
     const long big_tiles = ((d.M + BM - 1) / BM) * ((d.N + i8_geo_t::BN - 1) / i8_geo_t::BN) * d.batch;
-    const long crossover = d.wei_dt == MI355_DT_U8 ? 24 : 16;
+    const long crossover = 16;
     p.small = !d.dst_scale_dynamic && (big_tiles < crossover || d.K % BK != 0);
     // MI355_I8_TILES=large|wide|small overrides the choice where both can run (for
     // tests and tuning; read at every call): large = the LDS tiles, 256 x 128 or
@@ -567,10 +566,10 @@ int i8_launch(const mi355_matmul_desc_t &d, const problem_t &P, void *scratch,
     X.tiles_n = (int)((d.N + i8_geo_t::BN - 1) / i8_geo_t::BN);
     // Up to 128 large tiles leave half of the CUs or more idle: 256 x 128 tiles of four wavefronts, two workgroups a
     // CU, put twice as many to work (a wavefront's part, 128 x 64, its fragments and the epilogue are the same).
-    // s8 weights only, to bound the build.  MI355_I8_TILES=wide keeps the 256 x 256 tiles.
+    // MI355_I8_TILES=wide keeps the 256 x 256 tiles.
     using narrow_t = geo_t<4, 128>;
     const char *force = getenv("MI355_I8_TILES");
-    if (!wu && (long)X.tiles_m * X.tiles_n * d.batch <= 128 && d.N > 128 && !(force && !strcmp(force, "wide"))) {
+    if ((long)X.tiles_m * X.tiles_n * d.batch <= 128 && d.N > 128 && !(force && !strcmp(force, "wide"))) {
         X.tiles_n = (int)((d.N + narrow_t::BN - 1) / narrow_t::BN);
         dim3 grid((unsigned)(X.tiles_m * X.tiles_n), 1, (unsigned)d.batch);
         constexpr int smem_bytes = narrow_t::NSTAGE * narrow_t::STAGE_BYTES + NTAB_BYTES;
@@ -579,7 +578,9 @@ int i8_launch(const mi355_matmul_desc_t &d, const problem_t &P, void *scratch,
             hipLaunchKernelGGL(kern, grid, dim3(narrow_t::NT), smem_bytes, stream, P, X);
             return hipGetLastError() == hipSuccess ? MI355_SUCCESS : MI355_RUNTIME_ERROR;
         };
+        if (su && wu) return go(i8_gemm_kernel<true, true, narrow_t>);
         if (su) return go(i8_gemm_kernel<true, false, narrow_t>);
+        if (wu) return go(i8_gemm_kernel<false, true, narrow_t>);
         return go(i8_gemm_kernel<false, false, narrow_t>);
     }
     dim3 grid((unsigned)(X.tiles_m * X.tiles_n), 1, (unsigned)d.batch);

@@ -40,9 +40,9 @@ int woq_launch(const mi355_matmul_desc_t &d, const problem_t &P, void *scratch,
 int woqp_supported(const mi355_matmul_desc_t &d);
 int woqp_launch(const mi355_matmul_desc_t &d, const problem_t &P, hipStream_t stream);
 
-// hip:mfma_f8 on 256 x 128 tiles of four wavefronts, e4m3 x e4m3 (a translation unit of its own: the build runs
+// hip:mfma_f8 on 256 x 128 tiles of four wavefronts; fa / fb: 1 = e5m2 src / weights, 0 = e4m3 (a translation unit of its own: the build runs
 // the family's instantiations side by side); bt = the weights as [N][K] bytes, K contiguous
-int f8_launch_narrow_e4m3(const problem_t &P, const char *bt, long ldb, long bt_bstride, unsigned batch, hipStream_t stream);
+int f8_launch_narrow(int fa, int fb, const problem_t &P, const char *bt, long ldb, long bt_bstride, unsigned batch, hipStream_t stream);
 
 void set_error(const char *fmt, ...);
 
