@@ -439,6 +439,9 @@ def main():
     ap.add_argument("--calib-read", action="store_true",
                     help="time a read-only kernel with the decode kernel's access shape over the C2 weights "
                          "(12 rotating copies, nothing cached) and exit: the floor of the weight stream")
+    ap.add_argument("--calib-launch", action="store_true",
+                    help="time empty launches of several grid shapes and the decode kernel's skeleton (read the C2 "
+                         "weights, sum through LDS, store) and exit: what a launch and the stream cost by themselves")
     ap.add_argument("--calib-pattern", action="store_true",
                     help="time a read-only kernel that streams 256-row slabs the way the grouped matmul tiles do, with "
                          "64, 128, 256 and 1024 contiguous bytes per row and load instruction, over G1's weights "
@@ -470,14 +473,71 @@ def main():
         f"HBM={hbm.value / 2**30:.0f} GiB")
 
     main_name = args.workload
+
+    def calib_lib():
+        """the measurement kernels (tests/bin/libmi355_calib.so, built by tests/Makefile)"""
+        path = os.path.join(os.path.dirname(os.path.abspath(__file__)), "tests", "bin", "libmi355_calib.so")
+        if not os.path.exists(path):
+            sys.exit(f"bench.py: {path} is missing: build it with `make -C tests`")
+        cl = C.CDLL(path)
+        vp = C.c_void_p
+        cl.mi355_calib_copy.argtypes = [vp, vp, C.c_size_t, vp]
+        cl.mi355_calib_empty.argtypes = [C.c_int, C.c_int, vp]
+        cl.mi355_calib_read_stream.argtypes = [vp, C.c_size_t, vp, vp]
+        cl.mi355_calib_read_reduce.argtypes = [vp, C.c_size_t, vp, vp]
+        cl.mi355_calib_read_pattern.argtypes = [vp, C.c_int64, C.c_int64, C.c_int, vp, vp]
+        cl.mi355_calib_mfma_rate.argtypes = [C.c_int, C.c_int, vp, vp, C.POINTER(C.c_double), vp]
+        return cl
+
+    def ok(rc):
+        if rc != 0:
+            raise RuntimeError(f"calibration kernel refused its arguments or failed to launch ({rc})")
+
+    if args.calib_launch:
+        # what a launch costs by itself, and what the decode kernel's skeleton (read 128 KB per workgroup, meet in
+        # LDS, store 64 values) costs over the C2 weights: back-to-back launches, HIP events around 200 of them
+        cl = calib_lib()
+        nbytes = 4096 * 14336 // 2
+        bufs = [cabi.DeviceBuffer(nbytes) for _ in range(12)]
+        out = cabi.DeviceBuffer(256 * (nbytes // (128 << 10)))
+        timer, idx, rows = Timer(lib), [0], []
+
+        def pre(step):
+            t_pre = time.time()
+            while time.time() - t_pre < 0.3:
+                for _ in range(50):
+                    step()
+                cabi.check(lib.mi355_stream_sync(None))
+
+        for label, blocks, threads in (("empty launch, 1 x 64", 1, 64), ("empty launch, 224 x 1024", 224, 1024),
+                                       ("empty launch, 224 x 512", 224, 512), ("empty launch, 1024 x 256", 1024, 256)):
+            def step():
+                ok(cl.mi355_calib_empty(blocks, threads, None))
+            pre(step)
+            runs = [timer.time_ms(step, 200) for _ in range(5)]
+            rows.append({"kernel": label, "us_avg": 1e3 * sum(runs) / 5, "us_best": 1e3 * min(runs)})
+        for label, fn in (("read 29.4 MB, nothing kept", cl.mi355_calib_read_stream),
+                          ("read 29.4 MB, sum through LDS, 64 stores per workgroup", cl.mi355_calib_read_reduce)):
+            def step():
+                ok(fn(bufs[idx[0] % 12].ptr, C.c_size_t(nbytes), out.ptr, None))
+                idx[0] += 1
+            pre(step)
+            runs = [timer.time_ms(step, 200) for _ in range(5)]
+            rows.append({"kernel": label, "us_avg": 1e3 * sum(runs) / 5, "us_best": 1e3 * min(runs)})
+        for r in rows:
+            log(f"[bench] {r['kernel']}: {r['us_avg']:.2f} us per launch (best of 5 x 200: {r['us_best']:.2f})")
+        print(json.dumps({"metric": "launch and stream skeleton of the decode kernel", "unit": "us", "rows": rows}),
+              flush=True)
+        return
     if args.calib_pattern:
+        cl = calib_lib()
         K, slabs = 7168, 2048
         buf, sink = cabi.DeviceBuffer(K * 256 * slabs), cabi.DeviceBuffer(4096)
         cabi.check(lib.mi355_mem_set(buf.ptr, 1, C.c_size_t(K * 256 * slabs), None))
         timer, rows = Timer(lib), []
         for run in (64, 128, 256, 1024):
             def step():
-                cabi.check(lib.mi355_read_pattern_kernel(buf.ptr, slabs, K, run, sink.ptr, None))
+                ok(cl.mi355_calib_read_pattern(buf.ptr, slabs, K, run, sink.ptr, None))
             timer.time_ms(step, 20)
             ms = min(timer.time_ms(step, 10) for _ in range(3))
             gbs = K * 256 * slabs / (ms * 1e-3) / 1e9
@@ -487,13 +547,14 @@ def main():
                           "rows": rows}), flush=True)
         return
     if args.calib_read:
+        cl = calib_lib()
         nbytes = 4096 * 14336 // 2
         bufs = [cabi.DeviceBuffer(nbytes) for _ in range(12)]
         sink = cabi.DeviceBuffer(4096)
         timer, idx = Timer(lib), [0]
 
         def step():
-            cabi.check(lib.mi355_read_stream_kernel(bufs[idx[0] % 12].ptr, C.c_size_t(nbytes), sink.ptr, None))
+            ok(cl.mi355_calib_read_stream(bufs[idx[0] % 12].ptr, C.c_size_t(nbytes), sink.ptr, None))
             idx[0] += 1
 
         t_pre = time.time()
@@ -512,6 +573,7 @@ def main():
         return
 
     if args.calib_mfma:
+        cl = calib_lib()
         names = ["v_mfma_i32_32x32x32_i8", "v_mfma_i32_16x16x64_i8", "v_mfma_f32_32x32x64_f8f6f4 (fp8)",
                  "v_mfma_f32_16x16x128_f8f6f4 (fp8)", "v_mfma_scale_f32_32x32x64_f8f6f4 (fp4)",
                  "v_mfma_scale_f32_16x16x128_f8f6f4 (fp4)", "v_mfma_f32_32x32x16_bf16", "v_mfma_f32_16x16x32_bf16",
@@ -535,7 +597,7 @@ def main():
                 timer = Timer(lib)
 
                 def step():
-                    cabi.check(lib.mi355_mfma_rate_kernel(instr, 20000, out.ptr, bits.ptr, C.byref(ops), None))
+                    ok(cl.mi355_calib_mfma_rate(instr, 20000, out.ptr, bits.ptr, C.byref(ops), None))
 
                 step()
                 cabi.check(lib.mi355_stream_sync(None))
@@ -549,10 +611,11 @@ def main():
         return
 
     def calib_copy():
+        cl = calib_lib()
         nbytes = 256 << 20
         a, b = cabi.DeviceBuffer(nbytes), cabi.DeviceBuffer(nbytes)
         for _ in range(3):
-            cabi.check(lib.mi355_copy_kernel(b.ptr, a.ptr, C.c_size_t(nbytes), None))
+            ok(cl.mi355_calib_copy(b.ptr, a.ptr, C.c_size_t(nbytes), None))
         cabi.check(lib.mi355_stream_sync(None))
         a.free()
         b.free()

@@ -285,6 +285,7 @@ typedef enum {
 /* opaque handles, dnnl_common_types.h / dnnl_types.h */
 typedef struct dnnl_engine *dnnl_engine_t;
 typedef struct dnnl_stream *dnnl_stream_t;
+typedef const struct dnnl_stream *const_dnnl_stream_t;
 typedef struct dnnl_memory_desc *dnnl_memory_desc_t;
 typedef const struct dnnl_memory_desc *const_dnnl_memory_desc_t;
 typedef struct dnnl_memory *dnnl_memory_t;
@@ -310,7 +311,7 @@ dnnl_status_t dnnl_engine_get_kind(dnnl_engine_t engine, dnnl_engine_kind_t *kin
 dnnl_status_t dnnl_engine_destroy(dnnl_engine_t engine);
 size_t dnnl_engine_get_count(dnnl_engine_kind_t kind);
 dnnl_status_t dnnl_stream_create(dnnl_stream_t *stream, dnnl_engine_t engine, unsigned flags);
-dnnl_status_t dnnl_stream_get_engine(dnnl_stream_t stream, dnnl_engine_t *engine);
+dnnl_status_t dnnl_stream_get_engine(const_dnnl_stream_t stream, dnnl_engine_t *engine);
 dnnl_status_t dnnl_stream_wait(dnnl_stream_t stream);
 dnnl_status_t dnnl_stream_destroy(dnnl_stream_t stream);
 

@@ -308,6 +308,22 @@ int mi355_stream_wait_event(void *stream, void *event);
 int mi355_mem_store_scalar(void *dptr, uint64_t bits, int nbytes, void *stream);
 const char *mi355_last_error(void); /* thread-local text of the last failure */
 
+/* Tuning switches for tests and measurements; no counterpart in the reference
+ * (its nearest relative is the ONEDNN_MAX_CPU_ISA family of environment
+ * controls, src/common/utils.cpp getenv_int_user).  Each switch starts from the
+ * environment variable of the same name, read once per process, and afterwards
+ * changes only through this call -- launches never read the environment:
+ *   MI355_I8_TILES     large | wide | small   tile geometry of hip:mfma_i8
+ *   MI355_F8_TILES     wide                   hip:mfma_f8 on 256 x 256 tiles
+ *   MI355_H16_TILES    wide                   hip:mfma_h16 on 256 x 256 tiles
+ *   MI355_GROUPED_IMPL ref | short | tall | wide   grouped matmul kernel
+ *   MI355_GEMM_ORDER   0..63                  tile order of the large GEMMs
+ * value NULL, "" or "auto" restores the library's own choice.  Scratch sizes
+ * do not depend on a switch, so a change between mi355_matmul_scratch_bytes
+ * and the launch is harmless; a change while launches are in progress on other
+ * threads takes effect at some launch boundary. */
+int mi355_tuning_set(const char *name, const char *value);
+
 /* ---- the matmul path ---------------------------------------------------- */
 
 /* Dispatch predicate: MI355_SUCCESS if kernel family `impl` can run `desc`
@@ -483,35 +499,6 @@ const char *mi355_grouped_matmul_impl(const mi355_grouped_desc_t *desc);
  * no access leaves the tensors whatever the offsets hold.  Buffers that are
  * not 16-byte aligned run on "hip:ref_grouped:any". */
 int mi355_grouped_matmul_launch(const mi355_grouped_desc_t *desc, const mi355_grouped_args_t *args, void *stream);
-
-/* Plain device-to-device copy kernel (one 16-byte load + store per lane), used
- * to calibrate the FETCH_SIZE / WRITE_SIZE counters against a known size. */
-int mi355_copy_kernel(void *dst, const void *src, size_t bytes, void *stream);
-
-/* Read-only kernel with the access shape of the weight-only decode kernel
- * (128 KiB per workgroup, 16 wavefronts of eight 1 KiB non-temporal runs):
- * times what streaming `bytes` (a multiple of 128 KiB) of weights costs by
- * itself.  `sink` holds 4 bytes per 128 KiB and is not written in practice. */
-int mi355_read_stream_kernel(const void *src, size_t bytes, void *sink, void *stream);
-
-/* Access-shape probe for kernels that stream rows (the grouped matmul tiles): `slabs` workgroups of four
- * wavefronts each read a slab of 256 rows x K bytes (K a multiple of 1024) of `src` once, K-major, a load
- * instruction fetching 1024 / run rows x `run` contiguous bytes (run = 64, 128, 256 or 1024).  `sink`: 1 KiB,
- * not written in practice. */
-int mi355_read_pattern_kernel(const void *src, int64_t slabs, int64_t K, int run, void *sink, void *stream);
-
-/* Measures what an MFMA instruction of the GEMM kernels sustains by itself:
- * 1024 workgroups x 4 wavefronts, operands and accumulators in registers, 8 or
- * 16 independent accumulator chains, `iters` rounds.  instr: 0 i32_32x32x32_i8,
- * 1 i32_16x16x64_i8, 2 f32_32x32x64 fp8, 3 f32_16x16x128 fp8, 4 f32_32x32x64
- * fp4, 5 f32_16x16x128 fp4.  `bits`: 16 KiB of operand bits (their toggling
- * decides the clock the power manager grants), `out`: 1 MiB.  *ops_per_launch
- * receives the operation count to divide by the measured time. */
-int mi355_mfma_rate_kernel(int instr, int iters, void *out, const void *bits, double *ops_per_launch, void *stream);
-
-/* Evict caches between timed launches: streams `bytes` of `buf` through a
- * read-modify-write kernel so a following launch sees cold L2/MALL. */
-int mi355_flush_kernel(void *buf, size_t bytes, void *stream);
 
 #ifdef __cplusplus
 }

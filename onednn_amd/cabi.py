@@ -151,7 +151,7 @@ KERNEL_SYMBOLS = [
     "mi355_stream_wait_event", "mi355_mem_store_scalar",
     "mi355_last_error", "mi355_matmul_query", "mi355_matmul_impl_name",
     "mi355_matmul_scratch_bytes", "mi355_matmul_launch", "mi355_matmul_launch_noalloc", "mi355_reorder_query",
-    "mi355_reorder_launch", "mi355_wei_pack_reorder_dims", "mi355_copy_kernel", "mi355_flush_kernel", "mi355_read_stream_kernel", "mi355_read_pattern_kernel", "mi355_mfma_rate_kernel", "mi355_grouped_matmul_query",
+    "mi355_reorder_launch", "mi355_wei_pack_reorder_dims", "mi355_tuning_set", "mi355_grouped_matmul_query",
     "mi355_grouped_matmul_launch", "mi355_grouped_matmul_impl",
 ]
 
@@ -181,6 +181,7 @@ def load_kernels():
     lib.mi355_last_error.restype = C.c_char_p
     lib.mi355_matmul_impl_name.restype = C.c_char_p
     lib.mi355_matmul_impl_name.argtypes = [C.c_int]
+    lib.mi355_tuning_set.argtypes = [C.c_char_p, C.c_char_p]
     lib.mi355_device_count.argtypes = [C.POINTER(C.c_int)]
     lib.mi355_device_set.argtypes = [C.c_int]
     lib.mi355_device_info.argtypes = [C.c_int, C.c_char_p, C.c_size_t, C.POINTER(C.c_int),
@@ -210,15 +211,10 @@ def load_kernels():
     lib.mi355_reorder_launch.argtypes = [C.POINTER(ReorderDesc), C.POINTER(ReorderArgs), vp]
     lib.mi355_wei_pack_reorder_dims.argtypes = [C.c_int, C.c_int64, C.c_int64, C.c_int64, C.c_int64,
                                                 C.POINTER(ReorderDesc)]
-    lib.mi355_copy_kernel.argtypes = [vp, vp, C.c_size_t, vp]
     lib.mi355_grouped_matmul_query.argtypes = [C.POINTER(GroupedDesc)]
     lib.mi355_grouped_matmul_launch.argtypes = [C.POINTER(GroupedDesc), C.POINTER(GroupedArgs), vp]
     lib.mi355_grouped_matmul_impl.argtypes = [C.POINTER(GroupedDesc)]
     lib.mi355_grouped_matmul_impl.restype = C.c_char_p
-    lib.mi355_read_stream_kernel.argtypes = [vp, C.c_size_t, vp, vp]
-    lib.mi355_read_pattern_kernel.argtypes = [vp, C.c_int64, C.c_int64, C.c_int, vp, vp]
-    lib.mi355_mfma_rate_kernel.argtypes = [C.c_int, C.c_int, vp, vp, C.POINTER(C.c_double), vp]
-    lib.mi355_flush_kernel.argtypes = [vp, C.c_size_t, vp]
     _lib = lib
     return lib
 
@@ -295,3 +291,26 @@ def scratch_bytes(desc):
     n = C.c_size_t(0)
     check(load_kernels().mi355_matmul_scratch_bytes(C.byref(desc), C.byref(n)))
     return n.value
+
+
+def tuning_set(name, value=None):
+    """Set one of the library's tuning switches (MI355_I8_TILES, MI355_F8_TILES, MI355_H16_TILES,
+    MI355_GROUPED_IMPL, MI355_GEMM_ORDER); None restores the library's own choice.  The switches start from the
+    environment variables of the same names, read once per process."""
+    lib = load_kernels()
+    check(lib.mi355_tuning_set(name.encode(), None if value is None else str(value).encode()))
+
+
+class tuning:
+    """with tuning("MI355_I8_TILES", "small"): ...  -- the switch is back on the library's choice afterwards."""
+
+    def __init__(self, name, value):
+        self.name, self.value = name, value
+
+    def __enter__(self):
+        tuning_set(self.name, self.value)
+        return self
+
+    def __exit__(self, *exc):
+        tuning_set(self.name, None)
+        return False

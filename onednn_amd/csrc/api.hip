@@ -5,6 +5,9 @@
 #include <stdio.h>
 #include <string.h>
 
+#include <stdlib.h>
+
+#include <atomic>
 #include <map>
 #include <mutex>
 #include <utility>
@@ -20,6 +23,54 @@ void set_error(const char *fmt, ...) {
     va_start(ap, fmt);
     vsnprintf(g_err, sizeof(g_err), fmt, ap);
     va_end(ap);
+}
+
+namespace {
+struct tune_name_t {
+    const char *name;
+    const char *values; // accepted words, blank-separated
+};
+const tune_name_t TUNE_NAMES[TUNE_COUNT] = {
+        {"MI355_I8_TILES", "large wide small"},
+        {"MI355_F8_TILES", "wide"},
+        {"MI355_H16_TILES", "wide"},
+        {"MI355_GROUPED_IMPL", "ref short tall wide"},
+        {"MI355_GEMM_ORDER", ""},
+};
+std::atomic<int> g_tune[TUNE_COUNT];
+std::once_flag g_tune_once;
+
+// word -> value; -1 = not a word of this switch.  MI355_GEMM_ORDER takes a small non-negative number.
+int tune_parse(int key, const char *v) {
+    if (!v || !*v || !strcmp(v, "auto")) return TUNE_AUTO;
+    if (key == TUNE_GEMM_ORDER) {
+        char *end = nullptr;
+        const long x = strtol(v, &end, 10);
+        return (end && *end == 0 && x >= 0 && x < 64) ? (int)x : -1;
+    }
+    static const struct {
+        const char *w;
+        int val;
+    } words[] = {{"large", TUNE_LARGE}, {"wide", TUNE_WIDE}, {"small", TUNE_SMALL}, {"ref", TUNE_REF},
+            {"short", TUNE_SHORT}, {"tall", TUNE_TALL}};
+    for (const auto &w : words) {
+        if (strcmp(v, w.w)) continue;
+        const char *hit = strstr(TUNE_NAMES[key].values, v);
+        return hit ? w.val : -1;
+    }
+    return -1;
+}
+void tune_init() {
+    for (int k = 0; k < TUNE_COUNT; ++k) {
+        const int v = tune_parse(k, getenv(TUNE_NAMES[k].name));
+        g_tune[k].store(v < 0 ? TUNE_AUTO : v, std::memory_order_relaxed);
+    }
+}
+} // namespace
+
+int tuning(tune_key_t key) {
+    std::call_once(g_tune_once, tune_init);
+    return g_tune[key].load(std::memory_order_relaxed);
 }
 
 int ensure_dynamic_lds(const void *kernel, int bytes, const char *who) {
@@ -293,6 +344,23 @@ using namespace mi355;
 extern "C" {
 
 const char *mi355_last_error(void) { return g_err; }
+
+int mi355_tuning_set(const char *name, const char *value) {
+    if (!name) return MI355_INVALID_ARGUMENTS;
+    tuning(TUNE_I8_TILES); // the environment first, once
+    for (int k = 0; k < TUNE_COUNT; ++k) {
+        if (strcmp(name, TUNE_NAMES[k].name)) continue;
+        const int v = tune_parse(k, value);
+        if (v < 0) {
+            set_error("mi355_tuning_set: %s does not take '%s'", name, value);
+            return MI355_INVALID_ARGUMENTS;
+        }
+        g_tune[k].store(v, std::memory_order_relaxed);
+        return MI355_SUCCESS;
+    }
+    set_error("mi355_tuning_set: unknown switch %s", name);
+    return MI355_INVALID_ARGUMENTS;
+}
 
 int mi355_device_count(int *count) {
     if (!count) return MI355_INVALID_ARGUMENTS;

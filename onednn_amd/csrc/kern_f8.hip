@@ -272,8 +272,7 @@ int f8_launch(const mi355_matmul_desc_t &d, const problem_t &P, void *scratch, h
     }
     // Up to 128 tiles leave half of the CUs or more idle: 256 x 128 tiles of four wavefronts, two workgroups a CU, put
     // twice as many to work (a wavefront's part, 128 x 64, its fragments and the epilogue are the same).  MI355_F8_TILES=wide keeps the 256 x 256 tiles.
-    const char *force = getenv("MI355_F8_TILES");
-    if ((long)X.tiles_m * X.tiles_n * d.batch <= 128 && d.N > 128 && !(force && !strcmp(force, "wide")))
+    if ((long)X.tiles_m * X.tiles_n * d.batch <= 128 && d.N > 128 && tuning(TUNE_F8_TILES) != TUNE_WIDE)
         return f8_launch_narrow(fa, fb, P, X.bt, X.ldb, X.bt_bstride, (unsigned)d.batch, stream);
     if (fa && fb) return go(f8_gemm_kernel<f8_mma_t<1, 1, f8_geo_t>>);
     if (fa) return go(f8_gemm_kernel<f8_mma_t<1, 0, f8_geo_t>>);

@@ -509,8 +509,9 @@ __device__ __forceinline__ void grouped_store_quad(const grouped_dev_t &P, const
     const long N = Dd.N;
     if (m >= T.rows || nb >= N) return;
     // scales with groups along K (the MX modes) were applied by the matrix instruction
-    const bool with_ss = Dd.src_scale_dt != MI355_DT_UNDEF && Dd.src_scale_gk <= 1;
-    const bool with_ws = Dd.wei_scale_dt != MI355_DT_UNDEF && Dd.wei_scale_gk <= 1;
+    // (a group that spans all of K is one scale per row / per group and column: no groups along K)
+    const bool with_ss = Dd.src_scale_dt != MI355_DT_UNDEF && (Dd.src_scale_gk <= 1 || Dd.src_scale_gk == Dd.K);
+    const bool with_ws = Dd.wei_scale_dt != MI355_DT_UNDEF && (Dd.wei_scale_gk <= 1 || Dd.wei_scale_gk == Dd.K);
     const int dbits = dt_bits(Dd.dst_dt);
     const bool vec_ok = N % 4 == 0 && ((uintptr_t)P.a.dst % 16) == 0;
     const float ss = with_ss ? load_float(Dd.src_scale_dt, P.a.src_scale, T.src0 + m) : 1.f;
@@ -887,10 +888,13 @@ constexpr gshape_t GSHAPES[4] = {{0, 0}, {16, 32}, {48, 64}, {64, 256}};
 // wavefronts (groups of a row or two: many small workgroups); 2: 48 x 64, K
 // split, two workgroups per compute unit; 3: 64 x 256, columns split, src rows
 // through LDS.  Decided on the descriptor.
-int tile_plan(const mi355_grouped_desc_t &d) {
+// *mx_out: the plan is one of the MX modes (scales inside the instruction); every other plan has
+// no groups along K (a group size of K counts as none) and applies its scales after the K sum.
+int tile_plan(const mi355_grouped_desc_t &d, bool *mx_out = nullptr) {
+    if (mx_out) *mx_out = false;
     if (d.pattern != MI355_GROUPED_2DX3D) return 0;
-    const char *env = getenv("MI355_GROUPED_IMPL");
-    if (env && !strcmp(env, "ref")) return 0;
+    const int force = tuning(TUNE_GROUPED_IMPL);
+    if (force == TUNE_REF) return 0;
     const bool f8 = f8_dt(d.src_dt) && f8_dt(d.wei_dt);
     const bool f4 = d.src_dt == MI355_DT_F4_E2M1 && d.wei_dt == MI355_DT_F4_E2M1;
     const bool h16 = d.src_dt == d.wei_dt && (d.src_dt == MI355_DT_BF16 || d.src_dt == MI355_DT_F16);
@@ -916,10 +920,11 @@ int tile_plan(const mi355_grouped_desc_t &d) {
     int plan = 3;
     if (d.total <= 2 * d.group_count) plan = 1;
     else if (bytes(d.K) % 128 != 0 || (d.N + 255) / 256 * active < 256) plan = 2;
-    if (env && !strcmp(env, "short")) plan = 1;
-    if (env && !strcmp(env, "tall")) plan = 2;
-    if (env && !strcmp(env, "wide")) plan = 3;
+    if (force == TUNE_SHORT) plan = 1;
+    if (force == TUNE_TALL) plan = 2;
+    if (force == TUNE_WIDE) plan = 3;
     if (d.total / GSHAPES[plan].bm + active > 65535) return 0;
+    if (mx_out) *mx_out = mx;
     return plan;
 }
 
@@ -1033,11 +1038,11 @@ extern "C" int mi355_grouped_matmul_launch(const mi355_grouped_desc_t *d, const 
     // the tiles read 16 bytes at a time
     const bool aligned = (uintptr_t)a->src % 16 == 0 && (uintptr_t)a->wei % 16 == 0
             && (d->src_scale_gk <= 1 || ((uintptr_t)a->src_scale % 16 == 0 && (uintptr_t)a->wei_scale % 4 == 0));
-    const int plan = aligned ? tile_plan(*d) : 0;
+    bool mx = false;
+    const int plan = aligned ? tile_plan(*d, &mx) : 0;
     if (plan != 0) {
         hipStream_t s = (hipStream_t)stream;
         const int fa = d->src_dt == MI355_DT_F8_E5M2, fb = d->wei_dt == MI355_DT_F8_E5M2;
-        const bool mx = d->src_scale_dt != MI355_DT_UNDEF && d->src_scale_gk > 1;
         if (d->src_dt == MI355_DT_BF16) return launch_tiles<GM_BF16, 0, 0>(plan, P, s);
         if (d->src_dt == MI355_DT_F16) return launch_tiles<GM_F16, 0, 0>(plan, P, s);
         if (d->src_dt == MI355_DT_F4_E2M1) return launch_tiles<GM_MXF4, 0, 0>(plan, P, s);

@@ -510,9 +510,9 @@ int h16_launch(const mi355_matmul_desc_t &d, const problem_t &P_in, void *scratc
     // Few tiles (prefill at a few hundred rows): 256 x 128 tiles of four wavefronts, two workgroups a CU, put twice
     // the CUs to work; a wavefront's part, 128 x 64, and with it the fragments and the epilogue are the same.
     using narrow_t = geo_t<4, 128>;
-    const char *force = getenv("MI355_H16_TILES"); // "wide" keeps the 256 x 256 tiles (tests, tuning)
+    // (the MI355_H16_TILES switch keeps the 256 x 256 tiles: tests, tuning)
     if (plan.op_dt != MI355_DT_F32 && (long)X.tiles_m * X.tiles_n * d.batch <= 128 && d.N > 128
-            && !(force && !strcmp(force, "wide"))) {
+            && tuning(TUNE_H16_TILES) != TUNE_WIDE) {
         X.tiles_n = (int)((d.N + narrow_t::BN - 1) / narrow_t::BN);
         dim3 grid((unsigned)(X.tiles_m * X.tiles_n), 1, (unsigned)d.batch);
         constexpr int smem_bytes = narrow_t::NSTAGE * narrow_t::STAGE_BYTES + NTAB_BYTES;

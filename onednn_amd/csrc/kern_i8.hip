@@ -449,24 +449,27 @@ i8_plan_t make_plan(const mi355_matmul_desc_t &d) {
     const long big_tiles = ((d.M + BM - 1) / BM) * ((d.N + i8_geo_t::BN - 1) / i8_geo_t::BN) * d.batch;
     const long crossover = 16;
     p.small = !d.dst_scale_dynamic && (big_tiles < crossover || d.K % BK != 0);
-    // MI355_I8_TILES=large|wide|small overrides the choice where both can run (for
-    // tests and tuning; read at every call): large = the LDS tiles, 256 x 128 or
-    // 256 x 256 by the number of tiles; wide = the 256 x 256 ones
-    if (const char *force = getenv("MI355_I8_TILES")) {
-        if ((!strcmp(force, "large") || !strcmp(force, "wide")) && d.K % BK == 0) p.small = false;
-        if (!strcmp(force, "small") && !d.dst_scale_dynamic) p.small = true;
-    }
+    // the MI355_I8_TILES switch overrides the choice where both can run (tests and
+    // tuning): large = the LDS tiles, 256 x 128 or 256 x 256 by the number of
+    // tiles; wide = the 256 x 256 ones
+    const int force = tuning(TUNE_I8_TILES);
+    if ((force == TUNE_LARGE || force == TUNE_WIDE) && d.K % BK == 0) p.small = false;
+    if (force == TUNE_SMALL && !d.dst_scale_dynamic) p.small = true;
     // a = off_s - zs can be non-zero whenever src is u8 or has a zero point;
-    // c likewise for the weights
-    p.need_colsum = !p.small && (d.src_dt == MI355_DT_U8 || !quant_absent(d.src_zp));
-    p.need_rowsum = !p.small && (d.wei_dt == MI355_DT_U8 || !quant_absent(d.wei_zp));
+    // c likewise for the weights.  The scratch layout is that of the LDS tiles
+    // whichever tiles run (the sums are 4 (M + N) bytes), so its size does not
+    // depend on the switch.
+    const bool colsum = d.src_dt == MI355_DT_U8 || !quant_absent(d.src_zp);
+    const bool rowsum = d.wei_dt == MI355_DT_U8 || !quant_absent(d.wei_zp);
+    p.need_colsum = !p.small && colsum;
+    p.need_rowsum = !p.small && rowsum;
     size_t off = 0;
     p.off_bt = off;
     if (p.need_transpose) off += align_up((size_t)p.Bw * d.N * d.K, 256);
     p.off_colsum = off;
-    if (p.need_colsum) off += align_up((size_t)p.Bw * d.N * 4, 256);
+    if (colsum) off += align_up((size_t)p.Bw * d.N * 4, 256);
     p.off_rowsum = off;
-    if (p.need_rowsum) off += align_up((size_t)p.Bs * d.M * 4, 256);
+    if (rowsum) off += align_up((size_t)p.Bs * d.M * 4, 256);
     p.total = off;
     return p;
 }
@@ -568,8 +571,7 @@ int i8_launch(const mi355_matmul_desc_t &d, const problem_t &P, void *scratch,
     // CU, put twice as many to work (a wavefront's part, 128 x 64, its fragments and the epilogue are the same).
     // MI355_I8_TILES=wide keeps the 256 x 256 tiles.
     using narrow_t = geo_t<4, 128>;
-    const char *force = getenv("MI355_I8_TILES");
-    if ((long)X.tiles_m * X.tiles_n * d.batch <= 128 && d.N > 128 && !(force && !strcmp(force, "wide"))) {
+    if ((long)X.tiles_m * X.tiles_n * d.batch <= 128 && d.N > 128 && tuning(TUNE_I8_TILES) != TUNE_WIDE) {
         X.tiles_n = (int)((d.N + narrow_t::BN - 1) / narrow_t::BN);
         dim3 grid((unsigned)(X.tiles_m * X.tiles_n), 1, (unsigned)d.batch);
         constexpr int smem_bytes = narrow_t::NSTAGE * narrow_t::STAGE_BYTES + NTAB_BYTES;

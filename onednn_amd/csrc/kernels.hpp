@@ -46,6 +46,13 @@ int f8_launch_narrow(int fa, int fb, const problem_t &P, const char *bt, long ld
 
 void set_error(const char *fmt, ...);
 
+// Tuning switches (tests and measurements force a tile geometry where several can run a problem).  Each starts from
+// the environment variable of its name, read once per process, and changes only through mi355_tuning_set: no getenv on a
+// launch path.  Values: 0 = the library's own choice.
+enum tune_key_t { TUNE_I8_TILES = 0, TUNE_F8_TILES, TUNE_H16_TILES, TUNE_GROUPED_IMPL, TUNE_GEMM_ORDER, TUNE_COUNT };
+enum { TUNE_AUTO = 0, TUNE_LARGE = 1, TUNE_WIDE = 2, TUNE_SMALL = 3, TUNE_REF = 4, TUNE_SHORT = 5, TUNE_TALL = 6 };
+int tuning(tune_key_t key);
+
 // hipFuncSetAttribute(MaxDynamicSharedMemorySize) for a kernel, once per
 // (kernel, device, size) of this process.  Safe to call from several host
 // threads.

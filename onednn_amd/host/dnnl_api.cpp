@@ -917,7 +917,7 @@ DNNL_EXPORT dnnl_status_t dnnl_stream_create(dnnl_stream_t *stream, dnnl_engine_
     *stream = new dnnl_stream {engine, s};
     return dnnl_success;
 }
-DNNL_EXPORT dnnl_status_t dnnl_stream_get_engine(dnnl_stream_t stream, dnnl_engine_t *engine) {
+DNNL_EXPORT dnnl_status_t dnnl_stream_get_engine(const_dnnl_stream_t stream, dnnl_engine_t *engine) {
     CHECK_ARG(stream && engine);
     *engine = stream->engine;
     return dnnl_success;

@@ -34,12 +34,15 @@ def gpu():
 
 
 @pytest.fixture(params=["large", "wide", "small"])
-def i8_tiles(request, monkeypatch):
+def i8_tiles(request):
     """Runs a test once per tile geometry of hip:mfma_i8 (the LDS tiles -- "large":
     256 x 128 when a problem has few tiles, as all test shapes do; "wide": 256 x 256
     -- and the 32 x 32 direct ones) wherever they can take the problem; by itself
     the dispatcher would give every small test shape to the small tiles."""
-    monkeypatch.setenv("MI355_I8_TILES", request.param)
+    from onednn_amd import cabi
+    cabi.tuning_set("MI355_I8_TILES", request.param)
     if request.param == "wide":   # the fp8 family's switch between the same two LDS geometries
-        monkeypatch.setenv("MI355_F8_TILES", "wide")
-    return request.param
+        cabi.tuning_set("MI355_F8_TILES", "wide")
+    yield request.param
+    cabi.tuning_set("MI355_I8_TILES", None)
+    cabi.tuning_set("MI355_F8_TILES", None)

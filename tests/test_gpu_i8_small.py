@@ -75,13 +75,13 @@ def test_k_4000_at_a_size_the_large_tiles_would_take(gpu, oracle):
 
 @pytest.mark.parametrize("shape", [(1, 1, 64), (1, 33, 128), (31, 1, 192), (33, 65, 256), (256, 1024, 1024)])
 @pytest.mark.parametrize("dst_dt", [cabi.DT_S32, cabi.DT_BF16, cabi.DT_U8])
-def test_small_tiles_edges_and_dst_types(gpu, oracle, monkeypatch, shape, dst_dt):
-    monkeypatch.setenv("MI355_I8_TILES", "small")
+def test_small_tiles_edges_and_dst_types(gpu, oracle, shape, dst_dt):
     M, N, K = shape
     scales = dst_dt != cabi.DT_S32
     p = int8_problem(M, N, K, cabi.DT_U8, cabi.DT_S8, dst_dt, src_zp=128, wei_zp=True, scales=scales, bias=scales,
                      dst_scale=3.1 if dst_dt == cabi.DT_U8 else None)
-    got, name = run_gpu(p, cabi.IMPL_I8_MFMA)
+    with cabi.tuning("MI355_I8_TILES", "small"):
+        got, name = run_gpu(p, cabi.IMPL_I8_MFMA)
     assert_bit_exact(p, got, oracle.run_oracle(p), name)
 
 
@@ -97,8 +97,7 @@ def test_small_tiles_batched_and_broadcast_weights(gpu, oracle, wtag, wei_batch)
 
 @pytest.mark.parametrize("src_dt,wei_dt", [(cabi.DT_U8, cabi.DT_U8), (cabi.DT_U8, cabi.DT_S8), (cabi.DT_S8, cabi.DT_U8)])
 @pytest.mark.parametrize("dst_dt", [cabi.DT_S32, cabi.DT_S8])
-def test_both_tile_geometries_against_the_oracle_with_re_biased_operands(gpu, oracle, monkeypatch, src_dt, wei_dt,
-                                                                         dst_dt):
+def test_both_tile_geometries_against_the_oracle_with_re_biased_operands(gpu, oracle, src_dt, wei_dt, dst_dt):
     # rows 128 .. 255 of a large tile belong to the wavefronts whose first
     # iteration multiplies placeholder fragments: those must be the operand's
     # zero (0x80 for u8), or u8 x u8 gains 64 * 128 * 128 per element there
@@ -111,8 +110,8 @@ def test_both_tile_geometries_against_the_oracle_with_re_biased_operands(gpu, or
         assert np.mean(np.abs(w.astype(np.int32)) < 127) > 0.9      # not saturated away
     outs = []
     for tiles in ("large", "wide", "small"):
-        monkeypatch.setenv("MI355_I8_TILES", tiles)
-        got, name = run_gpu(p, cabi.IMPL_I8_MFMA)
+        with cabi.tuning("MI355_I8_TILES", tiles):
+            got, name = run_gpu(p, cabi.IMPL_I8_MFMA)
         assert_bit_exact(p, got, want, f"{name} {tiles}")
         outs.append(np.asarray(got).copy())
     assert np.array_equal(outs[0], outs[1]) and np.array_equal(outs[0], outs[2])
@@ -120,15 +119,15 @@ def test_both_tile_geometries_against_the_oracle_with_re_biased_operands(gpu, or
 
 @pytest.mark.gpu
 @pytest.mark.parametrize("src_dt", [cabi.DT_S8, cabi.DT_U8])
-def test_mid_size_problems_on_the_dispatchers_own_choice(gpu, oracle, monkeypatch, src_dt):
+def test_mid_size_problems_on_the_dispatchers_own_choice(gpu, oracle, src_dt):
     """30 large tiles (24 to 128 take the 256 x 128 LDS tiles by themselves), ragged in M and N: against the oracle, and
     the same bits from the 256 x 256 tiles"""
-    monkeypatch.delenv("MI355_I8_TILES", raising=False)
+    cabi.tuning_set("MI355_I8_TILES", None)
     p = int8_problem(1500, 1100, 192, src_dt, cabi.DT_S8, cabi.DT_S8, src_zp=7 if src_dt == cabi.DT_U8 else None,
                      dst_scale=40.0, bias=True)
     want = oracle.run_oracle(p)
     got, name = run_gpu(p, cabi.IMPL_I8_MFMA)
     assert_bit_exact(p, got, want, name)
-    monkeypatch.setenv("MI355_I8_TILES", "wide")
-    wide, name = run_gpu(p, cabi.IMPL_I8_MFMA)
+    with cabi.tuning("MI355_I8_TILES", "wide"):
+        wide, name = run_gpu(p, cabi.IMPL_I8_MFMA)
     assert np.array_equal(np.asarray(got), np.asarray(wide))

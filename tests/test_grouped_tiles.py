@@ -59,13 +59,8 @@ EXTRAS = [
 @pytest.fixture(params=["short", "tall", "wide"])
 def tile_shape(request):
     """Forces one of the three tile shapes of the matrix-core kernel."""
-    old = os.environ.get("MI355_GROUPED_IMPL")
-    os.environ["MI355_GROUPED_IMPL"] = request.param
-    yield request.param
-    if old is None:
-        del os.environ["MI355_GROUPED_IMPL"]
-    else:
-        os.environ["MI355_GROUPED_IMPL"] = old
+    with cabi.tuning("MI355_GROUPED_IMPL", request.param):
+        yield request.param
 
 
 def impl_of(p):
@@ -91,12 +86,15 @@ def test_dispatch_rules():
     assert impl_of(p) == "hip:ref_grouped:any"
     p, _ = gc.case_2dx3d([4, 4], 64, 32, src_dt=F16, wei_dt=cabi.DT_U4, wei_scale=16, wei_zp=16)
     assert impl_of(p) == "hip:ref_grouped:any"
-    os.environ["MI355_GROUPED_IMPL"] = "ref"
-    try:
+    with cabi.tuning("MI355_GROUPED_IMPL", "ref"):
         p, _ = gc.case_2dx3d([4, 4], 64, 32, src_dt=E4M3, wei_dt=E4M3, wtag="acb")
         assert impl_of(p) == "hip:ref_grouped:any"
-    finally:
-        del os.environ["MI355_GROUPED_IMPL"]
+    # a group that spans all of K is no group: scales per row / per group and column, applied after the K sum
+    for ss, ws in ((64, "col"), ("row", 64), (64, 64)):
+        p, _ = gc.case_2dx3d([4, 4], 64, 32, src_dt=E4M3, wei_dt=E4M3, wtag="acb", src_scale=ss, wei_scale=ws)
+        assert impl_of(p) == "hip:mfma_grouped", (ss, ws)
+    with pytest.raises(Exception):
+        cabi.tuning_set("MI355_GROUPED_IMPL", "sideways")
 
 
 @pytest.mark.gpu
@@ -115,6 +113,24 @@ def test_exact_data_matches_the_oracle(gpu, oracle, tile_shape, shape, tname, sd
             assert np.array_equal(got, ref), f"{p.name} {tname} {label} dst {dst_dt} ({tile_shape})"
             if dst_dt == F32:
                 assert np.array_equal(gc.logical_dst(p, got), want)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("tname,sdt,wdt", [("e4m3", E4M3, E4M3), ("bf16", BF16, BF16)])
+@pytest.mark.parametrize("ss,ws", [("K", "col"), ("row", "K"), ("K", "K"), ("K", None), (None, "K")])
+def test_a_k_group_of_all_of_k_is_a_row_or_column_scale(gpu, oracle, tile_shape, tname, sdt, wdt, ss, ws):
+    """scales with group size K along K (attr masks 3 / 7 with groups {1,K} / {K,1}) hold one value per row /
+    per group and column: the tiles apply them after the K sum like the ungrouped ones, never through the MX path"""
+    from onednn_amd import grouped
+    sizes, K, N = [5, 0, 40, 19], 256, 72
+    kw = dict(src_scale=K if ss == "K" else ss, wei_scale=K if ws == "K" else ws)
+    p, want = gc.case_2dx3d(sizes, K, N, src_dt=sdt, wei_dt=wdt, dst_dt=F32, wtag="acb", bias=True, **kw)
+    assert impl_of(p) == "hip:mfma_grouped"
+    st, ref = oracle.run_oracle_grouped(p)
+    assert st == cabi.SUCCESS
+    got = grouped.run_gpu(p)
+    assert np.array_equal(got, ref), f"{p.name} {tname} {ss} {ws} ({tile_shape})"
+    assert np.array_equal(gc.logical_dst(p, got), want)
 
 
 MX_SHAPES = [
@@ -225,15 +241,8 @@ def test_random_data_within_the_derived_bound(gpu, tile_shape, dt):
 
 def _ref_kernel(p):
     from onednn_amd import grouped
-    old = os.environ.get("MI355_GROUPED_IMPL")
-    os.environ["MI355_GROUPED_IMPL"] = "ref"
-    try:
+    with cabi.tuning("MI355_GROUPED_IMPL", "ref"):
         return grouped.run_gpu(p)
-    finally:
-        if old is None:
-            del os.environ["MI355_GROUPED_IMPL"]
-        else:
-            os.environ["MI355_GROUPED_IMPL"] = old
 
 
 MOE = {

@@ -105,7 +105,7 @@ def test_exact_data_bit_exact(gpu, oracle, shape, dt, ddt):
 @pytest.mark.gpu
 @pytest.mark.parametrize("shape", [(300, 520, 256), (64, 256, 128), (257, 300, 64)])
 @pytest.mark.parametrize("dt,ddt", [("bf16", "f32"), ("bf16", "bf16"), ("f16", "f16")])
-def test_wide_tiles_on_small_problems(gpu, oracle, monkeypatch, shape, dt, ddt):
+def test_wide_tiles_on_small_problems(gpu, oracle, shape, dt, ddt):
     """problems of at most 128 large tiles take 256 x 128 tiles by themselves (every other test shape here but the
     f32 ones does); MI355_H16_TILES=wide puts them on the 256 x 256 tiles the large problems run on: the same bits"""
     M, N, K = shape
@@ -115,8 +115,8 @@ def test_wide_tiles_on_small_problems(gpu, oracle, monkeypatch, shape, dt, ddt):
     narrow, name = run_gpu(p)
     assert name.startswith("hip:mfma_h16"), name
     assert_bit_exact(p, narrow, want, name)
-    monkeypatch.setenv("MI355_H16_TILES", "wide")
-    wide, name = run_gpu(p)
+    with cabi.tuning("MI355_H16_TILES", "wide"):
+        wide, name = run_gpu(p)
     assert_bit_exact(p, wide, want, name + " wide")
 
 
