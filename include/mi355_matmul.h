@@ -318,10 +318,11 @@ const char *mi355_last_error(void); /* thread-local text of the last failure */
  *   MI355_H16_TILES    wide                   hip:mfma_h16 on 256 x 256 tiles
  *   MI355_GROUPED_IMPL ref | short | tall | wide   grouped matmul kernel
  *   MI355_GEMM_ORDER   0..63                  tile order of the large GEMMs
- * value NULL, "" or "auto" restores the library's own choice.  Scratch sizes
- * do not depend on a switch, so a change between mi355_matmul_scratch_bytes
- * and the launch is harmless; a change while launches are in progress on other
- * threads takes effect at some launch boundary. */
+ * value NULL, "" or "auto" restores the library's own choice.  A switch can
+ * change a problem's scratch need (the 32 x 32 int8 tiles need none, the LDS
+ * tiles want column / row sums): set it before mi355_matmul_scratch_bytes, not
+ * between that call and the launch.  A change while launches are in progress
+ * on other threads takes effect at some launch boundary. */
 int mi355_tuning_set(const char *name, const char *value);
 
 /* ---- the matmul path ---------------------------------------------------- */

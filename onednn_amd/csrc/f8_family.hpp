@@ -108,9 +108,9 @@ struct f8_conv_t {
     // flight at once; every quad is read from there, and the bf16 result is
     // written back over it (same lane, same address); at the end the part leaves
     // LDS as 16 stores of 8 whole rows.  LDS rows are 128 bytes with the eight
-    // 16-byte chunks XOR-swizzled by the row number (on the global-address side of
-    // the DMA and of the final stores), which keeps both access patterns free of
-    // bank conflicts.
+    // 16-byte chunks XOR-swizzled by bits 1-3 of the row number (on the
+    // global-address side of the DMA and of the final stores), which keeps both
+    // access patterns free of bank conflicts.
     template <bool BIAS, bool GELU, bool ADD, class PT, int C>
     __device__ __forceinline__ void hot_store(const PT &P, const epi_uniform_t &H, unsigned ntab, unsigned lds_part,
             const v16f (&acc)[4][C], long b, long m_base, long n_base, int col0) const {
@@ -122,14 +122,17 @@ struct f8_conv_t {
         const int lane = threadIdx.x & 63, lrow = lane & 31, half = lane >> 5;
         const long rows_left = P.M - m_base; // > 0, checked by the caller
         // whole-row accesses: lane -> (row d * 8 + lane / 8, chunk slot lane % 8); the slot holds
-        // the row's chunk slot ^ (row & 7)
+        // the row's chunk slot ^ ((row >> 1) & 7): a row is 32 banks, so bit 0 of the row picks
+        // the half of the 64 banks and bits 1-3 the 16-byte slot inside it -- the 8-byte accesses
+        // of the 32 rows of an accumulator tile then spread over all banks (with row & 7 they
+        // used half of them: SQ_LDS_BANK_CONFLICT was 18 % of the LDS cycles of the kernel)
         const int wr = lane >> 3, wslot = lane & 7;
         if (ADD) {
             const char *rbase = scalar_ptr(H.staged_p + (b * H.st_s0 + m_base * H.st_s1 + n_base) * 2);
 #pragma unroll
             for (int d = 0; d < 16; ++d) {
                 long r = d * 8 + wr;
-                const int chunk = wslot ^ (int)(r & 7);
+                const int chunk = wslot ^ (int)((r >> 1) & 7);
                 r = r < rows_left ? r : rows_left - 1;
                 dma16(rbase, (unsigned)(r * H.st_s1 * 2 + chunk * 16), lds_part + d * 1024);
             }
@@ -150,7 +153,7 @@ struct f8_conv_t {
             unsigned cell[4];
 #pragma unroll
             for (int g = 0; g < 4; ++g) {
-                cell[g] = lds_part + (unsigned)(r * 128 + (((4 * j + g) ^ (r & 7)) << 4) + 8 * half);
+                cell[g] = lds_part + (unsigned)(r * 128 + (((4 * j + g) ^ ((r >> 1) & 7)) << 4) + 8 * half);
                 // keeps the table reads of every tile apart: merged, the 32 columns'
                 // operands of all tiles would stay in registers
                 int col = col0 + 32 * j + 8 * g + 4 * half;
@@ -200,7 +203,7 @@ struct f8_conv_t {
 #pragma unroll
         for (int d = 0; d < 16; ++d) {
             const long r = d * 8 + wr;
-            const int chunk = wslot ^ (int)(r & 7);
+            const int chunk = wslot ^ (int)((r >> 1) & 7);
             const v4u_t q = *(lds_u4_ptr_t)(size_t)(lds_part + (unsigned)(d * 1024 + lane * 16));
             // written once, never read again by this launch: non-temporal
             if (r < rows_left) __builtin_nontemporal_store(q, (v4u_t *)(dbase + r * P.ds[1] * 2 + chunk * 16));

@@ -27,6 +27,8 @@
 // outstanding-load counter is managed by hand (a prefetch distance of
 // NSTAGE-1 stages needs "wait until at most N loads are in flight").
 #pragma once
+#include <type_traits>
+
 #include "kernels.hpp"
 #include "tile_epilogue.hpp"
 
@@ -201,6 +203,13 @@ __device__ __forceinline__ dma_plan_t<DPA, DPB> make_dma_plan(int wave, int lane
     return p;
 }
 
+// operand policies that supply load_b_one (one B^T fragment at a time) run the
+// four-wavefront loop that reads a stage ahead
+template <class Mma, class = void>
+struct reads_ahead : std::false_type {};
+template <class Mma>
+struct reads_ahead<Mma, std::enable_if_t<Mma::READS_AHEAD>> : std::true_type {};
+
 // s_waitcnt lgkmcnt(0) only
 __device__ __forceinline__ void wait_lds_reads() {
     __builtin_amdgcn_s_waitcnt(0xC07F);
@@ -338,6 +347,123 @@ __device__ __forceinline__ void main_loop_two_groups(Acc &acc, char *smem, const
     phase_barrier();
 }
 
+// Main loop for four wavefronts, one per SIMD, with the fragments of the next
+// stage read while the current one is multiplied.  A single wavefront per SIMD
+// has nobody to cover for it: whatever it waits for, the matrix core waits
+// too.  So nothing a stage's MFMAs need is requested inside that stage -- its
+// fragments were read from LDS into a second set of registers during the
+// previous stage's MFMAs (a stage's fragments are 64-80 registers; one
+// wavefront per SIMD has 512), and the only wait between two stages' MFMAs is
+// the workgroup barrier itself.
+//
+// Ring of NSTAGE slots, stage s in slot s % NSTAGE.  At the barrier of
+// iteration g
+//   every wavefront holds stage g in registers (read during iteration g-1):
+//     slot g % NSTAGE is free and takes the DMAs of stage g + NSTAGE;
+//   every wavefront's DMAs of stage g+1 have landed (each waited for its own
+//     before the barrier): it is read from LDS during this iteration;
+//   stages g+2 .. g+NSTAGE-1 stay in flight: NSTAGE-2 stages of lead, as with
+//     the ring used the plain way, at one more stage of registers.
+// The loop is unrolled by two so that the two fragment sets keep their
+// registers (the sets swap roles, not contents); an odd stage count ends with
+// one more copy of the body.  Past the last stage the DMAs are issued all the
+// same, clamped to the last stage and into a slot nobody reads again, and the
+// reads fetch whatever the next slot holds: every iteration is the same
+// straight-line code and one outstanding-load count fits all of them.
+template <int NSTAGE, class Mma, class Acc, class Ctx>
+__device__ __forceinline__ void main_loop_ahead(Acc &acc, char *smem, const char *a_tile_, const char *b_tile_,
+        long lda, long ldb, long rows_a_left, long rows_b_left, int nstages_, const Ctx &ctx) {
+    using G = typename Mma::G;
+    const char *a_tile = scalar_ptr(a_tile_), *b_tile = scalar_ptr(b_tile_);
+    const int nstages = scalar_int(nstages_);
+    constexpr int STAGE_BYTES = G::STAGE_BYTES;
+    constexpr int DPA = G::DPA, DPB = G::DPB, DPS = G::DPS;
+    constexpr int STAGE_DMAS = DPS + Mma::EXTRA_DMAS;
+    constexpr int ROWS = Mma::ROWS, COLS = Mma::COLS;
+    static_assert(NSTAGE >= 3 && (NSTAGE - 1) * STAGE_DMAS < 64, "vmcnt range");
+    const int t = threadIdx.x, lane = t & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(t >> 6);
+    const typename Mma::addr_t AD = Mma::lane_addr(G::wm(wave), G::wn(wave), lane);
+    const unsigned lds0 = (unsigned)(size_t)(__attribute__((address_space(3))) char *)smem;
+    const dma_plan_t<DPA, DPB> plan = make_dma_plan<DPA, DPB>(wave, lane, rows_a_left, rows_b_left, lda, ldb);
+
+    auto issue_part = [&](int s, int slot, int i) __attribute__((always_inline)) {
+        const long koff = (long)s * BKB;
+        const unsigned lds_stage = lds0 + slot * STAGE_BYTES;
+        if (i < DPA) dma16(a_tile + koff, plan.voff_a[i], lds_stage + plan.lds_a[i]);
+        else dma16(b_tile + koff, plan.voff_b[i - DPA], lds_stage + plan.lds_b[i - DPA]);
+        if (i == DPS - 1) Mma::issue_extra(ctx, s, slot, wave, lane);
+    };
+
+#pragma unroll
+    for (int s = 0; s < NSTAGE; ++s) {
+        const int sc = s < nstages ? s : nstages - 1;
+#pragma unroll
+        for (int i = 0; i < DPS; ++i) issue_part(sc, s, i);
+    }
+    typename Mma::frag_t f0, f1;
+    wait_vmcnt<(NSTAGE - 1) * STAGE_DMAS>();
+    phase_barrier();
+    {
+        const unsigned S[1] = {lds0};
+#pragma unroll
+        for (int j = 0; j < COLS; ++j) Mma::load_b_one(f0, j, S, AD, ctx, 0);
+#pragma unroll
+        for (int i = 0; i < ROWS; ++i) Mma::load_a(f0, i, S, AD, ctx, 0);
+    }
+
+#ifdef MI355_ABLATE_READS
+    wait_lds_reads();
+    f1 = f0; // both sets hold real operand bits
+#endif
+    int slot = 0; // of stage g
+    // iteration g: multiply `cur` (stage g), read stage g+1 into `nxt`, DMA stage g+NSTAGE
+    auto step = [&](int g, typename Mma::frag_t &cur, typename Mma::frag_t &nxt) __attribute__((always_inline)) {
+        wait_vmcnt<(NSTAGE - 2) * STAGE_DMAS>();
+        wait_lds_reads();
+        phase_barrier();
+        Mma::prepare(cur);
+        int rslot = slot + 1;
+        if (rslot == NSTAGE) rslot = 0;
+        const unsigned S[1] = {lds0 + rslot * STAGE_BYTES};
+        const int sd = g + NSTAGE < nstages ? g + NSTAGE : nstages - 1;
+#pragma unroll
+        for (int i = 0; i < ROWS; ++i) {
+            // (MI355_ABLATE_READS / MI355_ABLATE_DMA: measurement builds that leave the fragment reads / the
+            // stage loads out of the loop -- wrong results, the same MFMAs -- to price each by itself)
+#ifndef MI355_ABLATE_READS
+            Mma::load_a(nxt, i, S, AD, ctx, g + 1);
+#pragma unroll
+            for (int j = 0; j < COLS; ++j)
+                if (j * ROWS / COLS == i) Mma::load_b_one(nxt, j, S, AD, ctx, g + 1);
+#endif
+#ifndef MI355_ABLATE_DMA
+#pragma unroll
+            for (int d = 0; d < DPS; ++d)
+                if (d * ROWS / DPS == i) issue_part(sd, slot, d);
+#endif
+            Mma::mma_row(acc, cur, i, ctx, g);
+            __builtin_amdgcn_sched_barrier(0); // keeps the reads and DMAs spread between the rows
+        }
+        slot = rslot;
+    };
+    int g = 0;
+#pragma nounroll
+    for (; g + 1 < nstages; g += 2) {
+        step(g, f0, f1);
+        step(g + 1, f1, f0);
+    }
+    if (g < nstages) step(g, f0, f1);
+    // every DMA has landed (the clamped ones included) and every read is back
+    // before the ring's memory is used for something else; the wait states
+    // between the last MFMA and the first read of its result, which the compiler
+    // cannot count for an MFMA written as inline assembly
+    wait_vmcnt<0>();
+    wait_lds_reads();
+    asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");
+    phase_barrier();
+}
+
 // Main loop.  The ring holds NSTAGE stages; one iteration consumes KSTEP of
 // them (a "group": KSTEP * 64 bytes of K), so NSTAGE / KSTEP groups rotate.
 // Per group g:
@@ -366,6 +492,10 @@ __device__ __forceinline__ void main_loop(Acc &acc, char *smem, const char *a_ti
     const int ngroups = scalar_int(ngroups_);
     constexpr int NG = NSTAGE / KSTEP;           // groups in the ring
     constexpr int STAGE_BYTES = G::STAGE_BYTES, GROUP_BYTES = KSTEP * STAGE_BYTES;
+    if constexpr (NSTAGE >= 4 && KSTEP == 1 && reads_ahead<Mma>::value) {
+        main_loop_ahead<NSTAGE, Mma>(acc, smem, a_tile_, b_tile_, lda, ldb, rows_a_left, rows_b_left, ngroups_, ctx);
+        return;
+    }
     if constexpr (G::NW == 8) {
         main_loop_two_groups<NSTAGE, KSTEP, Mma>(acc, smem, a_tile_, b_tile_, lda, ldb, rows_a_left,
                 rows_b_left, ngroups_, ctx);

@@ -22,6 +22,12 @@ namespace mi355 {
 namespace {
 
 using namespace gemm;
+// 1: the loop that reads a stage ahead instead of the two-group loop.  Both pass the parity tests and measured the
+// same on the 8192^3 configuration (0.4560 against 0.4566 ms, same box): the kernel's time is set by the energy of
+// its data movement, not by how the wavefronts take turns.
+#ifndef MI355_I8_AHEAD
+#define MI355_I8_AHEAD 0
+#endif
 constexpr int BK = BKB;       // int8: one byte per K element
 using i8_geo_t = geo_t<8, 256>;
 constexpr int NSTAGE = i8_geo_t::NSTAGE;
@@ -80,15 +86,43 @@ struct i8_mma_t {
             const i8_ctx_t &, int) {
         f.a[i] = lds_read16(S[0] + ad.a + i * 1024);
     }
+    // The loop that reads a stage ahead (gemm_core.hpp): a u8 operand is
+    // re-biased in place when its stage's turn comes, and the instruction is
+    // written out with the accumulator tied to one operand -- left to itself the
+    // compiler accumulates out of place in a loop that alternates between two
+    // fragment sets and then copies accumulators around in every iteration.  (No
+    // wait states are owed inside the loop: an accumulator is next touched 31
+    // instructions later, and a VALU result may feed the following MFMA.)
+    static constexpr bool READS_AHEAD = MI355_I8_AHEAD && G::NSTAGE >= 4;
+    __device__ static __forceinline__ void load_b_one(frag_t &f, int j, const unsigned (&S)[1], const addr_t &ad,
+            const i8_ctx_t &, int) {
+        f.b[j] = lds_read16(S[0] + ad.b + j * 1024);
+    }
+    __device__ static __forceinline__ void prepare(frag_t &f) {
+        if (SRC_U8) {
+#pragma unroll
+            for (int i = 0; i < ROWS; ++i) f.a[i] ^= (int)0x80808080;
+        }
+        if (WEI_U8) {
+#pragma unroll
+            for (int j = 0; j < COLS; ++j) f.b[j] ^= (int)0x80808080;
+        }
+    }
     __device__ static __forceinline__ void mma_row(v4i (&acc)[ROWS][COLS], const frag_t &f, int i,
             const i8_ctx_t &, int) {
-        const v4i a = SRC_U8 ? (f.a[i] ^ (int)0x80808080) : f.a[i];
+        if constexpr (READS_AHEAD) {
 #pragma unroll
-        for (int j = 0; j < COLS; ++j) {
-            const v4i b = WEI_U8 ? (f.b[j] ^ (int)0x80808080) : f.b[j];
-            // operands exchanged: the tile comes out transposed, a lane holds four
-            // consecutive n of one row (tile_epilogue.hpp)
-            acc[i][j] = __builtin_amdgcn_mfma_i32_16x16x64_i8(b, a, acc[i][j], 0, 0, 0);
+            for (int j = 0; j < COLS; ++j)
+                asm volatile("v_mfma_i32_16x16x64_i8 %0, %1, %2, %0" : "+v"(acc[i][j]) : "v"(f.b[j]), "v"(f.a[i]));
+        } else {
+            const v4i a = SRC_U8 ? (f.a[i] ^ (int)0x80808080) : f.a[i];
+#pragma unroll
+            for (int j = 0; j < COLS; ++j) {
+                const v4i b = WEI_U8 ? (f.b[j] ^ (int)0x80808080) : f.b[j];
+                // operands exchanged: the tile comes out transposed, a lane holds four
+                // consecutive n of one row (tile_epilogue.hpp)
+                acc[i][j] = __builtin_amdgcn_mfma_i32_16x16x64_i8(b, a, acc[i][j], 0, 0, 0);
+            }
         }
     }
 };
@@ -456,13 +490,14 @@ i8_plan_t make_plan(const mi355_matmul_desc_t &d) {
     if ((force == TUNE_LARGE || force == TUNE_WIDE) && d.K % BK == 0) p.small = false;
     if (force == TUNE_SMALL && !d.dst_scale_dynamic) p.small = true;
     // a = off_s - zs can be non-zero whenever src is u8 or has a zero point;
-    // c likewise for the weights.  The scratch layout is that of the LDS tiles
-    // whichever tiles run (the sums are 4 (M + N) bytes), so its size does not
-    // depend on the switch.
-    const bool colsum = d.src_dt == MI355_DT_U8 || !quant_absent(d.src_zp);
-    const bool rowsum = d.wei_dt == MI355_DT_U8 || !quant_absent(d.wei_zp);
-    p.need_colsum = !p.small && colsum;
-    p.need_rowsum = !p.small && rowsum;
+    // c likewise for the weights.  The small tiles compute their own sums: a
+    // problem they run on K-contiguous weights needs no scratch at all.
+    p.need_colsum = !p.small && (d.src_dt == MI355_DT_U8 || !quant_absent(d.src_zp));
+    p.need_rowsum = !p.small && (d.wei_dt == MI355_DT_U8 || !quant_absent(d.wei_zp));
+    // where a scratch buffer exists anyway its layout is that of the LDS tiles
+    // (the sums are 4 (M + N) bytes), whichever tiles run
+    const bool colsum = p.need_colsum || (p.need_transpose && (d.src_dt == MI355_DT_U8 || !quant_absent(d.src_zp)));
+    const bool rowsum = p.need_rowsum || (p.need_transpose && (d.wei_dt == MI355_DT_U8 || !quant_absent(d.wei_zp)));
     size_t off = 0;
     p.off_bt = off;
     if (p.need_transpose) off += align_up((size_t)p.Bw * d.N * d.K, 256);

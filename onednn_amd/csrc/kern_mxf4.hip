@@ -17,15 +17,25 @@
 //
 // Scales ride along with the tile stages: per stage and operand one extra
 // direct-to-LDS load per wavefront brings the 4 scale bytes (one dword) of
-// each of its 64 rows; weights scales [K/32][N] are transposed to [N][K/32]
-// by a pre-pass so both sides look alike.
+// each of its 64 rows.  Two small pre-pass kernels of the launch put both
+// operands' scales into a stage-major order, [K/128][rows] dwords, so that this
+// load is 256 contiguous bytes: from the plain layouts (src [M][K/32] bytes, a
+// row's dword of a stage 256 bytes from the next row's at K = 8192) the same
+// load touched 64 cache lines for 256 useful bytes, and the scales made as many
+// requests to the L2 as the tiles themselves.
 #include "gemm_core.hpp"
 
 namespace mi355 {
 namespace {
 
 using namespace gemm;
-using mx_geo_t = geo_t<4, 256>;
+#ifndef MI355_MXF4_NW
+#define MI355_MXF4_NW 8
+#endif
+#ifndef MI355_MXF4_AHEAD
+#define MI355_MXF4_AHEAD 1
+#endif
+using mx_geo_t = geo_t<MI355_MXF4_NW, 256>;
 constexpr int NSTAGE = mx_geo_t::NSTAGE;
 constexpr int SCALE_OFF = NSTAGE * mx_geo_t::STAGE_BYTES; // scale ring after the tile ring
 constexpr int SCALE_STAGE = (BM + mx_geo_t::BN) * 4;      // 256 dwords A + BN dwords B
@@ -35,16 +45,19 @@ constexpr int SMEM_BYTES = SMEM_RING_BYTES + NTAB_BYTES;
 struct mxf4_extra_t {
     const char *bt;       // weights [N][K/2] bytes
     long ldb, bt_bstride; // bytes
-    const char *sa;       // src scales [M][K/32] bytes, this batch added in-kernel
-    const char *sb;       // weights scales [N][K/32] bytes (transposed copy)
+    const char *sa;       // src scales, stage-major copy: [K/128][M] dwords, this batch added in-kernel
+    const char *sb;       // weights scales, stage-major copy: [K/128][N] dwords
     long sa_bstride, sb_bstride;
+    long sa_pitch, sb_pitch; // bytes between stages: 4 M, 4 N
     int tiles_m, tiles_n;
 };
 
 struct mxf4_ctx_t {
-    const char *sa_tile, *sb_tile; // first scale byte of tile row 0
+    const char *sa_tile, *sb_tile; // scale dword of tile row 0, stage 0
+    long sa_pitch, sb_pitch;       // bytes between stages
     unsigned voff_a, voff_b;       // this lane's row offset in the scale arrays
     const char *s_tile;            // eight wavefronts: the one operand this wavefront brings
+    long s_pitch;
     unsigned voff_s;
     unsigned lds_scale0;           // LDS byte address of the scale ring
     unsigned lds0;                 // LDS byte address of the tile ring
@@ -64,17 +77,18 @@ struct mxf4_mma_t {
             int) {
         const unsigned dst = c.lds_scale0 + slot * SCALE_STAGE + wave * 256;
         if (G::NW == 4) {
-            dma4(c.sa_tile + (long)g * 4, c.voff_a, dst);
-            dma4(c.sb_tile + (long)g * 4, c.voff_b,
+            dma4(c.sa_tile + (long)g * c.sa_pitch, c.voff_a, dst);
+            dma4(c.sb_tile + (long)g * c.sb_pitch, c.voff_b,
                     c.lds_scale0 + slot * SCALE_STAGE + 1024 + (wave % BBLK) * 256);
         } else {
-            dma4(c.s_tile + (long)g * 4, c.voff_s, dst);
+            dma4(c.s_tile + (long)g * c.s_pitch, c.voff_s, dst);
         }
     }
     static constexpr int ROWS = 8, COLS = G::WCOLS / 16, A_READS = 2, B_READS = 2; // data + scale dword
+    static constexpr int SA = ROWS / 4, SB = (COLS + 3) / 4; // scale dwords: one per four fragments
     struct frag_t {
         v4i a[ROWS], b[COLS];
-        int sa[ROWS], sb[COLS];
+        int sa[SA], sb[SB];
     };
     __device__ static __forceinline__ frag_t zero_frag() { return frag_t {}; } // e2m1 zero is all-zero bits
     // LDS byte address of the scale dwords that belong to the stage at S[0]
@@ -82,43 +96,79 @@ struct mxf4_mma_t {
         const unsigned slot = (S[0] - c.lds0) / G::STAGE_BYTES;
         return c.lds_scale0 + slot * SCALE_STAGE;
     }
-    // Per-lane LDS offsets of fragment 0 (data) and of its scale dword, and the
-    // bit position of this lane's scale byte; fragment i is 16 rows further.
+    // Per-lane LDS offsets of fragment 0 (data; fragment i is 16 rows further) and of
+    // the scale dword of the lane's first group of 64 rows.  A group of 64 rows holds
+    // its stage's scales as 64 dwords, dword 4 r + q = the bytes of block q of rows r,
+    // 16 + r, 32 + r and 48 + r (the pre-pass kernels of the launch write that order):
+    // lane (r, q) of an MFMA operand reads one dword and has the scale bytes of four
+    // fragments, which the instruction picks by its op_sel bits -- a dword and a read
+    // per four fragments, nothing to shift or mask.
     struct addr_t {
-        unsigned a, b, sa, sb, shift;
+        unsigned a, b, sa, sb;
     };
     __device__ static __forceinline__ addr_t lane_addr(int wm, int wn, int lane) {
         const int frow = lane & 15, q = lane >> 4;
         const int ra = wm * 128 + frow, rb = wn * G::WCOLS + frow;
-        return addr_t {(unsigned)swz(ra, q), (unsigned)(B_OFF + swz(rb, q)), (unsigned)(ra * 4),
-                (unsigned)((256 + rb) * 4), (unsigned)(q * 8)};
+        const int cell = (frow * 4 + q) * 4;
+        return addr_t {(unsigned)swz(ra, q), (unsigned)(B_OFF + swz(rb, q)), (unsigned)(wm * 2 * 256 + cell),
+                (unsigned)(1024 + (wn * G::WCOLS / 64) * 256 + cell)};
+    }
+    static constexpr bool READS_AHEAD = MI355_MXF4_AHEAD;
+    __device__ static __forceinline__ void prepare(frag_t &) {}
+    __device__ static __forceinline__ void load_b_one(frag_t &f, int j, const unsigned (&S)[1], const addr_t &ad,
+            const mxf4_ctx_t &c, int) {
+        f.b[j] = lds_read16(S[0] + ad.b + j * 1024);
+        if (j % 4 == 0) f.sb[j / 4] = (int)lds_read4(scales(S, c) + ad.sb + (j / 4) * 256);
     }
     __device__ static __forceinline__ void load_b(frag_t &f, const unsigned (&S)[1], const addr_t &ad,
-            const mxf4_ctx_t &c, int) {
-        const unsigned sc = scales(S, c);
+            const mxf4_ctx_t &c, int g) {
 #pragma unroll
-        for (int j = 0; j < COLS; ++j) {
-            f.b[j] = lds_read16(S[0] + ad.b + j * 1024);
-            f.sb[j] = (int)((lds_read4(sc + ad.sb + j * 64) >> ad.shift) & 0xffu);
-        }
+        for (int j = 0; j < COLS; ++j) load_b_one(f, j, S, ad, c, g);
     }
     __device__ static __forceinline__ void load_a(frag_t &f, int i, const unsigned (&S)[1], const addr_t &ad,
             const mxf4_ctx_t &c, int) {
-        const unsigned sc = scales(S, c);
         f.a[i] = lds_read16(S[0] + ad.a + i * 1024);
-        f.sa[i] = (int)((lds_read4(sc + ad.sa + i * 64) >> ad.shift) & 0xffu);
+        if (i % 4 == 0) f.sa[i / 4] = (int)lds_read4(scales(S, c) + ad.sa + (i / 4) * 256);
     }
+    // The instruction is written out with the accumulator tied to one operand: left
+    // to itself the compiler accumulates out of place in the loops that alternate
+    // between fragment sets or wavefront groups and then moves accumulators through
+    // scratch memory in every iteration (one wavefront per SIMD: the accumulation
+    // registers; two: plain ones, which the epilogue can work on directly).  No
+    // wait states are owed inside the loop: an accumulator is next touched 31 or 63
+    // instructions later.  OW / OS: the byte of the scale dwords that belongs to the
+    // weights / src fragment (op_sel bit 0, op_sel_hi bit 1 of each).
+    template <int OW, int OS>
+    __device__ static __forceinline__ void mma_one(v4f &acc, const v4i &w, const v4i &s, int sw, int ss) {
+        // operands exchanged: the tile comes out transposed, a lane holds four
+        // consecutive n of one row (tile_epilogue.hpp)
+        if constexpr (G::NW == 4)
+            asm volatile("v_mfma_scale_f32_16x16x128_f8f6f4 %0, %1, %2, %0, %3, %4 op_sel:[%5,%6,0] op_sel_hi:[%7,%8,0] cbsz:4 blgp:4"
+                         : "+a"(acc)
+                         : "v"(w), "v"(s), "v"(sw), "v"(ss), "n"(OW & 1), "n"(OS & 1), "n"(OW >> 1), "n"(OS >> 1));
+        else
+            asm volatile("v_mfma_scale_f32_16x16x128_f8f6f4 %0, %1, %2, %0, %3, %4 op_sel:[%5,%6,0] op_sel_hi:[%7,%8,0] cbsz:4 blgp:4"
+                         : "+v"(acc)
+                         : "v"(w), "v"(s), "v"(sw), "v"(ss), "n"(OW & 1), "n"(OS & 1), "n"(OW >> 1), "n"(OS >> 1));
+    }
+    template <int I, int J>
+    __device__ static __forceinline__ void mma_cols(v4f (&acc)[ROWS][COLS], const frag_t &f) {
+        if constexpr (J < COLS) {
+            mma_one<J % 4, I % 4>(acc[I][J], f.b[J], f.a[I], f.sb[J / 4], f.sa[I / 4]);
+            mma_cols<I, J + 1>(acc, f);
+        }
+    }
+    template <int I>
+    __device__ static __forceinline__ void mma_rows(v4f (&acc)[ROWS][COLS], const frag_t &f, int i) {
+        if constexpr (I < ROWS) {
+            if (i == I) mma_cols<I, 0>(acc, f);
+            else mma_rows<I + 1>(acc, f, i);
+        }
+    }
+    // (i is a constant after unrolling: the chain of comparisons folds away)
     __device__ static __forceinline__ void mma_row(v4f (&acc)[ROWS][COLS], const frag_t &f, int i,
             const mxf4_ctx_t &, int) {
-        const v8i a = {f.a[i][0], f.a[i][1], f.a[i][2], f.a[i][3], 0, 0, 0, 0};
-#pragma unroll
-        for (int j = 0; j < COLS; ++j) {
-            const v8i bb = {f.b[j][0], f.b[j][1], f.b[j][2], f.b[j][3], 0, 0, 0, 0};
-            // operands exchanged: the tile comes out transposed, a lane holds four
-            // consecutive n of one row (tile_epilogue.hpp)
-            acc[i][j] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(
-                    bb, a, acc[i][j], 4, 4, 0, f.sb[j], 0, f.sa[i]);
-        }
+        mma_rows<0>(acc, f, i);
     }
 };
 
@@ -127,6 +177,62 @@ struct mxf4_conv_t {
     template <class PT>
     __device__ __forceinline__ void per_n(const PT &, long, long, float &, int &, int &) const {}
     __device__ __forceinline__ int row_data(long) const { return 0; }
+    // The configuration's own chain: the accumulators as they are -> bf16, no bias, no post-ops.  Global memory sees
+    // whole 128-byte rows only: in the accumulator layout a lane owns 8 bytes of a dst row and a wavefront-wide store
+    // touches 16 rows, 32 bytes each (the memory pipeline's cost is per line touched).  The wavefront's 128 x 64 part
+    // goes through its 16 KB share of the idle tile ring instead -- 8-byte writes at row * 128 + ((slot ^ (row / 2 & 7))
+    // << 4), which spread over all banks -- and leaves as 16 stores of 8 whole rows.
+    template <class PT>
+    __device__ __forceinline__ bool hot_chain(const PT &P, const epi_uniform_t &H, unsigned, unsigned lds_part,
+            const v4f (&acc)[8][4], long b, long m_base, long n_base, int) const {
+        typedef unsigned v2u_t __attribute__((ext_vector_type(2)));
+        typedef unsigned v4u_t __attribute__((ext_vector_type(4)));
+        typedef v2u_t __attribute__((address_space(3), may_alias)) *lds_u2_ptr_t;
+        typedef v4u_t __attribute__((address_space(3), may_alias)) *lds_u4_ptr_t;
+        typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
+        typedef float f32x2_t __attribute__((ext_vector_type(2)));
+        if (m_base >= P.M) return true; // nothing of this wavefront's part is inside dst
+        if (H.n_po != 0 || H.bias_mode != 0 || H.ds_mode != 0 || H.dzp_mode != 0 || H.dynamic || H.dst_dt != MI355_DT_BF16)
+            return false;
+        if (((uintptr_t)P.dst & 15) || (P.ds[0] % 8) || (P.ds[1] % 8)) return false;
+        const int lane = threadIdx.x & 63, lrow = lane & 15, q = lane >> 4;
+        const long rows_left = P.M - m_base;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            const int r = 16 * i + lrow;
+            bool special = false;
+#pragma unroll
+            for (int j = 0; j < 4; ++j)
+#pragma unroll
+                for (int e = 0; e < 4; ++e) special |= __builtin_amdgcn_classf(acc[i][j][e], 0x93); // NaN or subnormal
+            const bool soft = __builtin_amdgcn_ballot_w64(special) != 0;
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                v2u_t o;
+                if (!soft) {
+                    o.x = __builtin_bit_cast(unsigned, __builtin_convertvector(f32x2_t {acc[i][j][0], acc[i][j][1]}, bf16x2_t));
+                    o.y = __builtin_bit_cast(unsigned, __builtin_convertvector(f32x2_t {acc[i][j][2], acc[i][j][3]}, bf16x2_t));
+                } else {
+                    o.x = f32_to_bf16(acc[i][j][0]) | ((unsigned)f32_to_bf16(acc[i][j][1]) << 16);
+                    o.y = f32_to_bf16(acc[i][j][2]) | ((unsigned)f32_to_bf16(acc[i][j][3]) << 16);
+                }
+                // columns 16 j + 4 q ..: byte 32 j + 8 q of the row = slot 2 j + q / 2, half q % 2
+                const int slot = 2 * j + (q >> 1);
+                *(lds_u2_ptr_t)(size_t)(lds_part + (unsigned)(r * 128 + ((slot ^ ((r >> 1) & 7)) << 4) + 8 * (q & 1))) = o;
+            }
+        }
+        // (a wavefront reads back what its own lanes wrote: program order, no barrier)
+        char *dbase = (char *)P.dst + (b * P.ds[0] + m_base * P.ds[1] + n_base) * 2;
+        const int wr = lane >> 3, wslot = lane & 7;
+#pragma unroll
+        for (int d = 0; d < 16; ++d) {
+            const long r = d * 8 + wr;
+            const int chunk = wslot ^ (int)((r >> 1) & 7);
+            const v4u_t v = *(lds_u4_ptr_t)(size_t)(lds_part + (unsigned)(d * 1024 + lane * 16));
+            if (r < rows_left) __builtin_nontemporal_store(v, (v4u_t *)(dbase + r * P.ds[1] * 2 + chunk * 16));
+        }
+        return true;
+    }
     template <class PT, class Acc>
     __device__ __forceinline__ bool hot_chain(const PT &, const epi_uniform_t &, unsigned, unsigned, const Acc &, long,
             long, long, int) const {
@@ -152,23 +258,24 @@ __global__ void __launch_bounds__(G::NT) __attribute__((amdgpu_waves_per_eu(G::N
     const long m0 = tp.m0, n0 = tp.n0;
 
     const long lda = P.ss[1] / 2; // bytes per src row
-    const long kb = P.K / 32;     // scale bytes per row
     const char *A = (const char *)P.src + (P.ss[0] ? b * (P.ss[0] / 2) : 0) + m0 * lda;
     const char *Bt = X.bt + b * X.bt_bstride + n0 * X.ldb;
 
     mxf4_ctx_t ctx;
     ctx.lds0 = (unsigned)(size_t)(__attribute__((address_space(3))) char *)smem;
     ctx.lds_scale0 = (unsigned)(size_t)(__attribute__((address_space(3))) char *)smem + SCALE_OFF;
-    ctx.sa_tile = X.sa + b * X.sa_bstride + m0 * kb;
-    ctx.sb_tile = X.sb + b * X.sb_bstride + n0 * kb;
+    ctx.sa_tile = X.sa + b * X.sa_bstride + m0 * 4;
+    ctx.sb_tile = X.sb + b * X.sb_bstride + n0 * 4;
+    ctx.sa_pitch = X.sa_pitch;
+    ctx.sb_pitch = X.sb_pitch;
     {
-        long ra = (wave & 3) * 64 + lane, rb = ((wave & 3) % (G::BN / 64)) * 64 + lane;
-        if (ra > P.M - m0 - 1) ra = P.M - m0 - 1;
-        if (rb > P.N - n0 - 1) rb = P.N - n0 - 1;
-        ctx.voff_a = (unsigned)(ra * kb);
-        ctx.voff_b = (unsigned)(rb * kb);
+        // (the packed scales are padded to whole tiles of 256 rows: nothing to clamp)
+        const long ra = (wave & 3) * 64 + lane, rb = ((wave & 3) % (G::BN / 64)) * 64 + lane;
+        ctx.voff_a = (unsigned)(ra * 4);
+        ctx.voff_b = (unsigned)(rb * 4);
         const bool brings_a = __builtin_amdgcn_readfirstlane(wave) < 4; // uniform: the base stays scalar
         ctx.s_tile = brings_a ? ctx.sa_tile : ctx.sb_tile;
+        ctx.s_pitch = brings_a ? ctx.sa_pitch : ctx.sb_pitch;
         ctx.voff_s = brings_a ? ctx.voff_a : ctx.voff_b;
     }
 
@@ -207,10 +314,72 @@ __global__ void __launch_bounds__(256) transpose_nibbles_kernel(const uint8_t *i
     }
 }
 
+// e8m0 scales of `rows` rows x KB blocks of 32 k, element (r, kb) at in[r * rs + kb * ks], into the order the tile
+// kernel loads: per stage of 128 k (four blocks) and group of 64 rows 64 dwords, dword 4 r + q = the bytes of block q
+// of rows r, 16 + r, 32 + r, 48 + r of the group; groups padded to whole tiles of 256 rows (rows beyond the last
+// repeat it).  out[stage][group][64] dwords.
+// Rows contiguous in the input (weights scales [K/32][N], rs = 1): a thread per dword.
+__global__ void __launch_bounds__(256) mx_scales_rows_kernel(const uint8_t *in, long rows, long prows, long KB, long ks,
+        long in_bstride, uint32_t *out, long out_bstride) {
+    in += blockIdx.z * in_bstride;
+    out += blockIdx.z * out_bstride;
+    const long total = prows * (KB / 4);
+    for (long i = (long)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += (long)gridDim.x * blockDim.x) {
+        const long st = i / prows, w = i % prows, grp = w / 64;
+        const int cell = (int)(w % 64), r = cell >> 2, q = cell & 3;
+        uint32_t v = 0;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            long row = grp * 64 + 16 * e + r;
+            row = row < rows ? row : rows - 1;
+            v |= (uint32_t)in[(4 * st + q) * ks + row] << (8 * e);
+        }
+        out[i] = v;
+    }
+}
+// Blocks contiguous in the input (src scales [M][K/32], ks = 1): a workgroup moves 64 rows x 16 stages through LDS,
+// 64 contiguous bytes of a row in, 256 contiguous bytes of a stage and group out.
+__global__ void __launch_bounds__(256) mx_scales_blocks_kernel(const uint8_t *in, long rows, long prows, long KB, long rs,
+        long in_bstride, uint32_t *out, long out_bstride) {
+    __shared__ uint32_t tile[16][65]; // [stage][row]: the row's four block bytes of the stage
+    in += blockIdx.z * in_bstride;
+    out += blockIdx.z * out_bstride;
+    const long grp = blockIdx.x, r0 = grp * 64, q0 = (long)blockIdx.y * 16, nq = KB / 4;
+    const int t = threadIdx.x;
+    const bool aligned = ((uintptr_t)in & 3) == 0 && (rs & 3) == 0;
+    {
+        const int r = t >> 2, c = t & 3; // row, group of four stages
+        const long row = r0 + r < rows ? r0 + r : rows - 1;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            const long q = q0 + 4 * c + e;
+            const uint8_t *p = in + row * rs + 4 * q;
+            uint32_t v = 0u;
+            if (q < nq) {
+                if (aligned) v = *(const uint32_t *)p;
+                else v = (uint32_t)p[0] | ((uint32_t)p[1] << 8) | ((uint32_t)p[2] << 16) | ((uint32_t)p[3] << 24);
+            }
+            tile[4 * c + e][r] = v;
+        }
+    }
+    __syncthreads();
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+        const int st = (t >> 6) + 4 * e, cell = t & 63, r = cell >> 2, q = cell & 3;
+        if (q0 + st < nq) {
+            uint32_t v = 0;
+#pragma unroll
+            for (int k = 0; k < 4; ++k) v |= ((tile[st][16 * k + r] >> (8 * q)) & 0xffu) << (8 * k);
+            out[(q0 + st) * prows + grp * 64 + cell] = v;
+        }
+    }
+}
+
 struct mxf4_plan_t {
     bool need_transpose;
-    size_t off_bt, off_sb, total;
-    long Bw, Bsb;
+    size_t off_bt, off_sb, off_sa, total;
+    long Bw, Bsb, Bsa;
+    long pm, pn; // M, N rounded up to whole tiles
 };
 
 mxf4_plan_t make_plan(const mi355_matmul_desc_t &d) {
@@ -221,8 +390,14 @@ mxf4_plan_t make_plan(const mi355_matmul_desc_t &d) {
     size_t off = 0;
     p.off_bt = off;
     if (p.need_transpose) off += align_up((size_t)p.Bw * d.N * d.K / 2, 256);
+    // the scales in the tile kernel's order, rows padded to whole tiles
+    p.pn = (d.N + 255) / 256 * 256;
+    p.pm = (d.M + 255) / 256 * 256;
     p.off_sb = off;
-    off += align_up((size_t)p.Bsb * d.N * (d.K / 32), 256);
+    off += align_up((size_t)p.Bsb * p.pn * (d.K / 32), 256);
+    p.Bsa = ((d.src_scale.mask & 1) && d.src_stride[0]) ? d.batch : 1;
+    p.off_sa = off;
+    off += align_up((size_t)p.Bsa * p.pm * (d.K / 32), 256);
     p.total = off;
     return p;
 }
@@ -278,14 +453,25 @@ int mxf4_launch(const mi355_matmul_desc_t &d, const problem_t &P, void *scratch,
         X.ldb = d.wei_stride[2] / 2;
         X.bt_bstride = d.wei_stride[0] / 2;
     }
-    // weights scales [K/32][N] -> [N][K/32]
+    // scales into the tile kernel's order (see mx_scales_rows_kernel)
     const long kb = d.K / 32;
-    transpose_bytes(P.wei_scale.p, kb, d.N, d.N, kb * d.N, sc + plan.off_sb, kb, d.N * kb, plan.Bsb,
-            stream);
+    {
+        long blocks = (plan.pn * (kb / 4) + 255) / 256;
+        if (blocks > 65535) blocks = 65535;
+        hipLaunchKernelGGL(mx_scales_rows_kernel, dim3((unsigned)blocks, 1, (unsigned)plan.Bsb), dim3(256), 0, stream,
+                (const uint8_t *)P.wei_scale.p, d.N, plan.pn, kb, d.N, kb * d.N, (uint32_t *)(sc + plan.off_sb),
+                plan.pn * (kb / 4));
+        hipLaunchKernelGGL(mx_scales_blocks_kernel,
+                dim3((unsigned)(plan.pm / 64), (unsigned)((kb / 4 + 15) / 16), (unsigned)plan.Bsa), dim3(256), 0, stream,
+                (const uint8_t *)P.src_scale.p, d.M, plan.pm, kb, kb, d.M * kb, (uint32_t *)(sc + plan.off_sa),
+                plan.pm * (kb / 4));
+    }
     X.sb = sc + plan.off_sb;
-    X.sb_bstride = plan.Bsb > 1 ? d.N * kb : 0;
-    X.sa = (const char *)P.src_scale.p;
-    X.sa_bstride = ((d.src_scale.mask & 1) && d.src_stride[0]) ? d.M * kb : 0;
+    X.sb_bstride = plan.Bsb > 1 ? plan.pn * kb : 0;
+    X.sb_pitch = plan.pn * 4;
+    X.sa = sc + plan.off_sa;
+    X.sa_bstride = plan.Bsa > 1 ? plan.pm * kb : 0;
+    X.sa_pitch = plan.pm * 4;
     X.tiles_m = (int)((d.M + BM - 1) / BM);
     X.tiles_n = (int)((d.N + mx_geo_t::BN - 1) / mx_geo_t::BN);
     dim3 grid((unsigned)(X.tiles_m * X.tiles_n), 1, (unsigned)d.batch);
