@@ -41,11 +41,13 @@ sys.path.insert(0, ROOT)
 
 import numpy as np  # noqa: E402
 
-# HBM bytes per launch come from the rocprofv3 summaries under profiles/ (two
-# --pmc passes, FETCH_SIZE and WRITE_SIZE, each scaled by what the same counter
-# reads for the plain copy kernel moving a known 256 MiB): every summary carries
-# the line "HBM bytes per launch ...: N", which is read here, so that the figure
-# in the JSON line can only be as old as the committed profile it names.
+# `traffic` comes from the rocprofv3 summaries under profiles/ (two --pmc passes,
+# FETCH_SIZE and WRITE_SIZE, each scaled by what the same counter reads for the
+# plain copy kernel moving a known 256 MiB).  The counters sit behind the L2s:
+# they count the bytes that miss them, whether the 256 MB memory-side cache or
+# HBM then serves them.  Every summary carries the line "Bytes that miss the L2s
+# per launch ...: N", which is read here, so that the figure in the JSON line can
+# only be as old as the committed profile it names.
 PROFILE_OF = {
     ("c3", "any"): "i8_gemm_kernel_c3_8192.md", ("c4", "any"): "f8_gemm_kernel_c4_4096x8192x28672.md",
     ("c5", "any"): "mxf4_gemm_kernel_c5_8192.md", ("c1", "any"): "i8_small_kernel_c1_256x1024x1024.md",
@@ -73,7 +75,7 @@ def measured_traffic(name, wtag="any", M=None):
         return None, None
     path = os.path.join(ROOT, "profiles", fn)
     try:
-        m = re.search(r"HBM bytes per launch[^:\n]*:\s*([0-9,]+)", open(path).read())
+        m = re.search(r"(?:Bytes that miss the L2s|HBM bytes) per launch[^:\n]*:\s*([0-9,]+)", open(path).read())
     except OSError:
         return None, None
     return (int(m.group(1).replace(",", "")), "profiles/" + fn) if m else (None, "profiles/" + fn)
@@ -86,6 +88,65 @@ PEAK_F8_TFLOPS = 5000.0
 PEAK_F4_TFLOPS = 10100.0
 PEAK_BF16_TFLOPS = 2500.0
 PEAK_F32_TFLOPS = 157.3
+
+
+# the MFMA instruction each compute-bound workload runs on (index into the calibration kernel's table)
+CEILING_INSTR = {"c3": 1, "c1": 1, "c4": 2, "m1": 2, "c5": 5, "h1": 7, "h2": 8}
+
+
+def measured_ceiling(lib, name):
+    """What the workload's MFMA instruction sustains by itself on this box, now, with random operand bits
+    (registers only: tests/calib/calib_kernels.hip), in the workload's unit; for the decode workload the rate of a
+    read-only kernel with the decode kernel's access shape over the same 29.4 MB of weights.  None when the
+    calibration library is not built."""
+    from onednn_amd import cabi
+    path = os.path.join(ROOT, "tests", "bin", "libmi355_calib.so")
+    if not os.path.exists(path):
+        return None
+    cl = C.CDLL(path)
+    vp = C.c_void_p
+    timer = Timer(lib)
+    if name == "c2":
+        cl.mi355_calib_read_stream.argtypes = [vp, C.c_size_t, vp, vp]
+        nbytes = 4096 * 14336 // 2
+        bufs = [cabi.DeviceBuffer(nbytes) for _ in range(12)]
+        sink = cabi.DeviceBuffer(4096)
+        idx = [0]
+
+        def step():
+            cl.mi355_calib_read_stream(bufs[idx[0] % 12].ptr, C.c_size_t(nbytes), sink.ptr, None)
+            idx[0] += 1
+
+        timer.time_ms(step, 2000)
+        ms = min(timer.time_ms(step, 200) for _ in range(3))
+        for b in bufs:
+            b.free()
+        return {"value": nbytes / (ms * 1e-3) / 1e9, "unit": "GB/s",
+                "what": "read-only kernel with the decode kernel's access shape over the same weights, per launch"}
+    instr = CEILING_INSTR.get(name)
+    if instr is None:
+        return None
+    cl.mi355_calib_mfma_rate.argtypes = [C.c_int, C.c_int, vp, vp, C.POINTER(C.c_double), vp]
+    h = np.random.default_rng(1).integers(0, 2**32, size=4096, dtype=np.uint64).astype(np.uint32)
+    if instr in (2, 3):
+        h &= np.uint32(0x3f3f3f3f)
+    elif instr in (6, 7):
+        h &= np.uint32(0x3fff3fff)
+    elif instr == 8:
+        h &= np.uint32(0x3fffffff)
+    bits, out = cabi.DeviceBuffer.from_numpy(h), cabi.DeviceBuffer(1 << 20)
+    ops = C.c_double(0)
+
+    def step():
+        cl.mi355_calib_mfma_rate(instr, 20000, out.ptr, bits.ptr, C.byref(ops), None)
+
+    step()
+    cabi.check(lib.mi355_stream_sync(None))
+    ms = min(timer.time_ms(step, 1) for _ in range(3))
+    bits.free()
+    out.free()
+    return {"value": ops.value / (ms * 1e-3) / 1e12, "unit": "TFLOP/s",
+            "what": "the kernel's MFMA instruction by itself, registers only, random operand bits"}
 
 
 def log(*a):
@@ -672,25 +733,38 @@ def main():
         "frac": res["value"] / res["peak"], "traffic": traffic, "traffic_source": traffic_source,
         "algorithmic": res["work"], "kernel": res["impl"], "kernel_ms": res["ms_per_step"],
     }
+    # next to the published peak: what this box's matrix cores (or, for decode, its memory system) deliver to a
+    # kernel that does nothing else -- `frac` stays priced against the published peak
+    ceil = measured_ceiling(lib, main_name)
+    if ceil:
+        roofline["ceiling"] = ceil["value"]
+        roofline["ceiling_what"] = ceil["what"]
+        roofline["frac_of_ceiling"] = res["value"] / ceil["value"]
+        log(f"[bench] ceiling: {ceil['value']:.0f} {ceil['unit']} ({ceil['what']}) -> {100 * roofline['frac_of_ceiling']:.1f}% of it")
 
     others = []
     if not args.no_others:
         # (workload, M, weights tag); "ab" = row-major weights as in the reference's benchdnn line for C3: the
         # layout change then runs inside every launch
-        plan = [("c2", 1, "any"), ("c2", 8, "any"), ("c2", 32, "any"), ("c3", None, "any"), ("c3", None, "ab"),
+        plan = [("c2", 1, "any"), ("c2", 8, "any"), ("c2", 32, "any"), ("c2", 1, "ab"), ("c2", 8, "ab"), ("c2", 32, "ab"),
+                ("c3", None, "any"), ("c3", None, "ab"),
                 ("c4", None, "any"), ("c4mx", None, "any"), ("c5", None, "any"), ("c1", None, "any"),
                 ("m1", None, "any"), ("h1", None, "any"), ("h2", None, "any"), ("p2", 512, "any"), ("p2", 2048, "any")]
         for nm, m, wt in plan:
             if nm == main_name and wt == args.wtag and (nm != "c2" or m == args.decode_m):
                 continue
             try:
-                r, _ = run_gpu_workload(lib, nm, max(5, args.steps // 2), 2, m,
+                r, _ = run_gpu_workload(lib, nm, max(5, args.steps // 2) if nm != "c2" else 200, 2, m,
                                         11 if nm == "c2" else 0, wt)
                 r["frac_of_peak"] = r["value"] / r["peak"]
                 if wt != "any":
                     r["workload"] += f" (weights tag {wt})"
+                r["algorithmic"] = r["work"]
+                # the layout pre-pass of row-major weights is not in the committed counter passes of the GEMMs
+                r["traffic"], r["traffic_source"] = measured_traffic(nm, wt, m) if (nm == "c2" or wt == "any") else (None, None)
                 others.append({k: r[k] for k in ("workload", "impl", "ms_per_step", "value", "unit",
-                                                 "bound", "peak", "frac_of_peak")})
+                                                 "bound", "peak", "frac_of_peak", "algorithmic", "traffic",
+                                                 "traffic_source")})
                 log(f"[bench] {r['workload']}: {r['ms_per_step']:.4f} ms -> {r['value']:.1f} "
                     f"{r['unit']} ({100 * r['frac_of_peak']:.1f}% of {r['bound']} peak) via {r['impl']}")
             except Exception as e:  # a failing side workload must not hide the headline

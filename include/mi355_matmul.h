@@ -313,8 +313,10 @@ const char *mi355_last_error(void); /* thread-local text of the last failure */
  * controls, src/common/utils.cpp getenv_int_user).  Each switch starts from the
  * environment variable of the same name, read once per process, and afterwards
  * changes only through this call -- launches never read the environment:
- *   MI355_I8_TILES     large | wide | small   tile geometry of hip:mfma_i8
- *   MI355_F8_TILES     wide                   hip:mfma_f8 on 256 x 256 tiles
+ *   MI355_I8_TILES     large | wide | narrow | small   tile geometry of hip:mfma_i8
+ *                      (large: the LDS tiles, 256 x 128 or 256 x 256 by the tile count;
+ *                      wide: 256 x 256; narrow: 256 x 128; small: 32 x 32 without LDS)
+ *   MI355_F8_TILES     wide | narrow          hip:mfma_f8 on 256 x 256 / 256 x 128 tiles
  *   MI355_H16_TILES    wide                   hip:mfma_h16 on 256 x 256 tiles
  *   MI355_GROUPED_IMPL ref | short | tall | wide   grouped matmul kernel
  *   MI355_GEMM_ORDER   0..63                  tile order of the large GEMMs

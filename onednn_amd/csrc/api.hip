@@ -31,8 +31,8 @@ struct tune_name_t {
     const char *values; // accepted words, blank-separated
 };
 const tune_name_t TUNE_NAMES[TUNE_COUNT] = {
-        {"MI355_I8_TILES", "large wide small"},
-        {"MI355_F8_TILES", "wide"},
+        {"MI355_I8_TILES", "large wide small narrow"},
+        {"MI355_F8_TILES", "wide narrow"},
         {"MI355_H16_TILES", "wide"},
         {"MI355_GROUPED_IMPL", "ref short tall wide"},
         {"MI355_GEMM_ORDER", ""},
@@ -52,7 +52,7 @@ int tune_parse(int key, const char *v) {
         const char *w;
         int val;
     } words[] = {{"large", TUNE_LARGE}, {"wide", TUNE_WIDE}, {"small", TUNE_SMALL}, {"ref", TUNE_REF},
-            {"short", TUNE_SHORT}, {"tall", TUNE_TALL}};
+            {"short", TUNE_SHORT}, {"tall", TUNE_TALL}, {"narrow", TUNE_NARROW}};
     for (const auto &w : words) {
         if (strcmp(v, w.w)) continue;
         const char *hit = strstr(TUNE_NAMES[key].values, v);

@@ -73,6 +73,29 @@ struct f8_mma_t {
             acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(
                     f.b[j], f.a[i], acc[i][j], FMT_B, FMT_A, 0, 0, 0, 0);
     }
+    // K that ends inside a stage (gemm_core.hpp tail_step): the lane's two chunks are
+    // 2 (lane / 32) and the next one; chunks below nz are zeroed in both operands
+    // (fp8 zero is all-zero bits; both, so that no Inf or NaN among the bytes that were
+    // multiplied before meets a zero)
+    static constexpr bool K_TAIL = true;
+    __device__ static __forceinline__ void zero_tail(frag_t &f, int nz, int lane) {
+        const int c0 = (lane >> 5) * 2;
+        const bool z0 = c0 < nz, z1 = c0 + 1 < nz;
+#pragma unroll
+        for (int i = 0; i < ROWS; ++i)
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                f.a[i][e] = z0 ? 0 : f.a[i][e];
+                f.a[i][4 + e] = z1 ? 0 : f.a[i][4 + e];
+            }
+#pragma unroll
+        for (int j = 0; j < COLS; ++j)
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                f.b[j][e] = z0 ? 0 : f.b[j][e];
+                f.b[j][4 + e] = z1 ? 0 : f.b[j][4 + e];
+            }
+    }
 };
 
 // HOT: whether the kernel instantiation carries the compile-time specialised
@@ -332,8 +355,16 @@ __global__ void __launch_bounds__(Mma::G::NT) __attribute__((amdgpu_waves_per_eu
 #pragma unroll
             for (int r = 0; r < acc_of<Mma>::N; ++r) acc[i][j][r] = 0.f;
 
+    const long kbytes = P.K * EB;
     main_loop<G::NSTAGE, KSTEP, Mma>(acc, smem, A, Bt, lda, X.ldb, P.M - m0,
-            P.N - n0, (int)(P.K * EB / (BKB * KSTEP)), f8_ctx_t {});
+            P.N - n0, (int)(kbytes / (BKB * KSTEP)), f8_ctx_t {});
+    if constexpr (has_k_tail<Mma>::value) {
+        // the rest of a K that is whole 16-byte chunks but not whole stages
+        const int rem = (int)(kbytes % BKB);
+        if (rem != 0)
+            tail_step<Mma>(acc, smem, A + kbytes - BKB, Bt + kbytes - BKB, lda, X.ldb, P.M - m0, P.N - n0,
+                    (BKB - rem) / 16, (int)(kbytes / BKB), f8_ctx_t {});
+    }
 
     store_quadrant<typename acc_of<Mma>::layout, G::WCOLS>(P, smem, ntab, acc, b, m0 + wm * 128, n0 + wn * G::WCOLS,
             wn * G::WCOLS, cv);

@@ -464,6 +464,53 @@ __device__ __forceinline__ void main_loop_ahead(Acc &acc, char *smem, const char
     phase_barrier();
 }
 
+// operand policies that supply zero_tail take a K that ends inside a stage
+template <class Mma, class = void>
+struct has_k_tail : std::false_type {};
+template <class Mma>
+struct has_k_tail<Mma, std::enable_if_t<Mma::K_TAIL>> : std::true_type {};
+
+// The end of a K that does not fill its last stage, after the main loop has
+// taken the whole stages: one more stage whose 64 bytes per row are the LAST 64
+// bytes of the row -- a_win / b_win point 64 bytes before the row's end, so no
+// byte beyond the row is touched -- of which the first `nz` 16-byte chunks were
+// multiplied already and are zeroed in the fragments of both operands
+// (Mma::zero_tail; both operands hold the same k in the same place, so the
+// shift inside the stage does not matter to the products).  g_tail = the number
+// of whole stages = the tail's stage number for the policy's own loads.  Not pipelined: it
+// costs a problem with such a K a few microseconds per tile and the others
+// nothing.  The ring is idle on entry and on return.
+template <class Mma, class Acc, class Ctx>
+__device__ __forceinline__ void tail_step(Acc &acc, char *smem, const char *a_win_, const char *b_win_, long lda,
+        long ldb, long rows_a_left, long rows_b_left, int nz_, int g_tail, const Ctx &ctx) {
+    using G = typename Mma::G;
+    const char *a_win = scalar_ptr(a_win_), *b_win = scalar_ptr(b_win_);
+    const int nz = scalar_int(nz_);
+    constexpr int DPA = G::DPA, DPB = G::DPB;
+    const int t = threadIdx.x, lane = t & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(t >> 6);
+    const typename Mma::addr_t AD = Mma::lane_addr(G::wm(wave), G::wn(wave), lane);
+    const unsigned lds0 = (unsigned)(size_t)(__attribute__((address_space(3))) char *)smem;
+    const dma_plan_t<DPA, DPB> plan = make_dma_plan<DPA, DPB>(wave, lane, rows_a_left, rows_b_left, lda, ldb);
+#pragma unroll
+    for (int i = 0; i < DPA; ++i) dma16(a_win, plan.voff_a[i], lds0 + plan.lds_a[i]);
+#pragma unroll
+    for (int i = 0; i < DPB; ++i) dma16(b_win, plan.voff_b[i], lds0 + plan.lds_b[i]);
+    Mma::issue_extra(ctx, g_tail, 0, wave, lane); // what rides along with stage number g_tail (block scales)
+    wait_vmcnt<0>();
+    phase_barrier();
+    typename Mma::frag_t f;
+    const unsigned S[1] = {lds0};
+    Mma::load_b(f, S, AD, ctx, 0);
+#pragma unroll
+    for (int i = 0; i < Mma::ROWS; ++i) Mma::load_a(f, i, S, AD, ctx, 0);
+    wait_lds_reads();
+    Mma::zero_tail(f, nz, lane);
+#pragma unroll
+    for (int i = 0; i < Mma::ROWS; ++i) Mma::mma_row(acc, f, i, ctx, 0);
+    phase_barrier();
+}
+
 // Main loop.  The ring holds NSTAGE stages; one iteration consumes KSTEP of
 // them (a "group": KSTEP * 64 bytes of K), so NSTAGE / KSTEP groups rotate.
 // Per group g:

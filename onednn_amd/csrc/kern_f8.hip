@@ -189,7 +189,8 @@ f8_plan_t make_plan(const mi355_matmul_desc_t &d) {
 int f8_supported(const mi355_matmul_desc_t &d) {
     if (!is_f8_dt(d.src_dt) || !is_f8_dt(d.wei_dt)) return MI355_UNIMPLEMENTED;
     if (dt_bits(d.dst_dt) < 8) return MI355_UNIMPLEMENTED;
-    if (d.K < BKB * KSTEP || d.K % (BKB * KSTEP) != 0) return MI355_UNIMPLEMENTED;
+    // whole 16-byte chunks of K; a K that ends inside a 64-byte stage takes one unpipelined step more per tile
+    if (d.K < BKB * KSTEP || d.K % 16 != 0) return MI355_UNIMPLEMENTED;
     if (d.src_stride[2] != 1 || d.src_stride[1] % 16 != 0 || d.src_stride[0] % 16 != 0)
         return MI355_UNIMPLEMENTED;
     const bool k_major = d.wei_stride[1] == 1 && d.wei_stride[2] % 16 == 0 && d.wei_stride[0] % 16 == 0;
@@ -272,7 +273,8 @@ int f8_launch(const mi355_matmul_desc_t &d, const problem_t &P, void *scratch, h
     }
     // Up to 128 tiles leave half of the CUs or more idle: 256 x 128 tiles of four wavefronts, two workgroups a CU, put
     // twice as many to work (a wavefront's part, 128 x 64, its fragments and the epilogue are the same).  MI355_F8_TILES=wide keeps the 256 x 256 tiles.
-    if ((long)X.tiles_m * X.tiles_n * d.batch <= 128 && d.N > 128 && tuning(TUNE_F8_TILES) != TUNE_WIDE)
+    const int force = tuning(TUNE_F8_TILES); // wide / narrow: one geometry whatever the size (tests, tuning)
+    if (force == TUNE_NARROW || ((long)X.tiles_m * X.tiles_n * d.batch <= 128 && d.N > 128 && force != TUNE_WIDE))
         return f8_launch_narrow(fa, fb, P, X.bt, X.ldb, X.bt_bstride, (unsigned)d.batch, stream);
     if (fa && fb) return go(f8_gemm_kernel<f8_mma_t<1, 1, f8_geo_t>>);
     if (fa) return go(f8_gemm_kernel<f8_mma_t<1, 0, f8_geo_t>>);

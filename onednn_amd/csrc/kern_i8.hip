@@ -487,7 +487,7 @@ i8_plan_t make_plan(const mi355_matmul_desc_t &d) {
     // tuning): large = the LDS tiles, 256 x 128 or 256 x 256 by the number of
     // tiles; wide = the 256 x 256 ones
     const int force = tuning(TUNE_I8_TILES);
-    if ((force == TUNE_LARGE || force == TUNE_WIDE) && d.K % BK == 0) p.small = false;
+    if ((force == TUNE_LARGE || force == TUNE_WIDE || force == TUNE_NARROW) && d.K % BK == 0) p.small = false;
     if (force == TUNE_SMALL && !d.dst_scale_dynamic) p.small = true;
     // a = off_s - zs can be non-zero whenever src is u8 or has a zero point;
     // c likewise for the weights.  The small tiles compute their own sums: a
@@ -606,7 +606,8 @@ int i8_launch(const mi355_matmul_desc_t &d, const problem_t &P, void *scratch,
     // CU, put twice as many to work (a wavefront's part, 128 x 64, its fragments and the epilogue are the same).
     // MI355_I8_TILES=wide keeps the 256 x 256 tiles.
     using narrow_t = geo_t<4, 128>;
-    if ((long)X.tiles_m * X.tiles_n * d.batch <= 128 && d.N > 128 && tuning(TUNE_I8_TILES) != TUNE_WIDE) {
+    const int force = tuning(TUNE_I8_TILES);
+    if (force == TUNE_NARROW || ((long)X.tiles_m * X.tiles_n * d.batch <= 128 && d.N > 128 && force != TUNE_WIDE)) {
         X.tiles_n = (int)((d.N + narrow_t::BN - 1) / narrow_t::BN);
         dim3 grid((unsigned)(X.tiles_m * X.tiles_n), 1, (unsigned)d.batch);
         constexpr int smem_bytes = narrow_t::NSTAGE * narrow_t::STAGE_BYTES + NTAB_BYTES;

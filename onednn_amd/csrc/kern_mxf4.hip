@@ -165,6 +165,19 @@ struct mxf4_mma_t {
             else mma_rows<I + 1>(acc, f, i);
         }
     }
+    // K that ends inside a stage (gemm_core.hpp tail_step): the lane's chunk is block lane / 16 of the stage
+    static constexpr bool K_TAIL = true;
+    __device__ static __forceinline__ void zero_tail(frag_t &f, int nz, int lane) {
+        const bool z = (lane >> 4) < nz;
+#pragma unroll
+        for (int i = 0; i < ROWS; ++i)
+#pragma unroll
+            for (int e = 0; e < 4; ++e) f.a[i][e] = z ? 0 : f.a[i][e];
+#pragma unroll
+        for (int j = 0; j < COLS; ++j)
+#pragma unroll
+            for (int e = 0; e < 4; ++e) f.b[j][e] = z ? 0 : f.b[j][e];
+    }
     // (i is a constant after unrolling: the chain of comparisons folds away)
     __device__ static __forceinline__ void mma_row(v4f (&acc)[ROWS][COLS], const frag_t &f, int i,
             const mxf4_ctx_t &, int) {
@@ -293,6 +306,11 @@ __global__ void __launch_bounds__(G::NT) __attribute__((amdgpu_waves_per_eu(G::N
 
     main_loop<NSTAGE, 1, Mma>(acc, smem, A, Bt, lda, X.ldb, P.M - m0, P.N - n0,
             (int)(P.K / 128), ctx);
+    // the rest of a K that is whole blocks of 32 but not whole stages of 128: the row's last 64 bytes, the blocks
+    // multiplied before zeroed; the scales of those four blocks are the stage after the whole ones in the packed order
+    if (const int rem = (int)(P.K % 128))
+        tail_step<Mma>(acc, smem, A + P.K / 2 - BKB, Bt + P.K / 2 - BKB, lda, X.ldb, P.M - m0, P.N - n0,
+                (128 - rem) / 32, (int)(P.K / 128), ctx);
 
     store_quadrant<layout16_t, G::WCOLS>(P, smem, ntab, acc, b, m0 + wm * 128, n0 + wn * G::WCOLS, wn * G::WCOLS,
             mxf4_conv_t {});
@@ -323,16 +341,19 @@ __global__ void __launch_bounds__(256) mx_scales_rows_kernel(const uint8_t *in, 
         long in_bstride, uint32_t *out, long out_bstride) {
     in += blockIdx.z * in_bstride;
     out += blockIdx.z * out_bstride;
-    const long total = prows * (KB / 4);
+    const long nst = (KB + 3) / 4, total = prows * nst;
     for (long i = (long)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += (long)gridDim.x * blockDim.x) {
         const long st = i / prows, w = i % prows, grp = w / 64;
         const int cell = (int)(w % 64), r = cell >> 2, q = cell & 3;
+        // a last stage that K does not fill holds the last four blocks (the tile kernel multiplies the row's last
+        // 64 bytes there)
+        const long blk = 4 * st + 4 <= KB ? 4 * st + q : KB - 4 + q;
         uint32_t v = 0;
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
             long row = grp * 64 + 16 * e + r;
             row = row < rows ? row : rows - 1;
-            v |= (uint32_t)in[(4 * st + q) * ks + row] << (8 * e);
+            v |= (uint32_t)in[blk * ks + row] << (8 * e);
         }
         out[i] = v;
     }
@@ -344,7 +365,7 @@ __global__ void __launch_bounds__(256) mx_scales_blocks_kernel(const uint8_t *in
     __shared__ uint32_t tile[16][65]; // [stage][row]: the row's four block bytes of the stage
     in += blockIdx.z * in_bstride;
     out += blockIdx.z * out_bstride;
-    const long grp = blockIdx.x, r0 = grp * 64, q0 = (long)blockIdx.y * 16, nq = KB / 4;
+    const long grp = blockIdx.x, r0 = grp * 64, q0 = (long)blockIdx.y * 16, nq = (KB + 3) / 4;
     const int t = threadIdx.x;
     const bool aligned = ((uintptr_t)in & 3) == 0 && (rs & 3) == 0;
     {
@@ -353,7 +374,8 @@ __global__ void __launch_bounds__(256) mx_scales_blocks_kernel(const uint8_t *in
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
             const long q = q0 + 4 * c + e;
-            const uint8_t *p = in + row * rs + 4 * q;
+            // (a last stage that K does not fill: the row's last four blocks)
+            const uint8_t *p = in + row * rs + (4 * q + 4 <= KB ? 4 * q : KB - 4);
             uint32_t v = 0u;
             if (q < nq) {
                 if (aligned) v = *(const uint32_t *)p;
@@ -380,6 +402,7 @@ struct mxf4_plan_t {
     size_t off_bt, off_sb, off_sa, total;
     long Bw, Bsb, Bsa;
     long pm, pn; // M, N rounded up to whole tiles
+    long nst;
 };
 
 mxf4_plan_t make_plan(const mi355_matmul_desc_t &d) {
@@ -394,10 +417,11 @@ mxf4_plan_t make_plan(const mi355_matmul_desc_t &d) {
     p.pn = (d.N + 255) / 256 * 256;
     p.pm = (d.M + 255) / 256 * 256;
     p.off_sb = off;
-    off += align_up((size_t)p.Bsb * p.pn * (d.K / 32), 256);
+    p.nst = (d.K + 127) / 128; // stages, one scale dword per row and stage
+    off += align_up((size_t)p.Bsb * p.pn * p.nst * 4, 256);
     p.Bsa = ((d.src_scale.mask & 1) && d.src_stride[0]) ? d.batch : 1;
     p.off_sa = off;
-    off += align_up((size_t)p.Bsa * p.pm * (d.K / 32), 256);
+    off += align_up((size_t)p.Bsa * p.pm * p.nst * 4, 256);
     p.total = off;
     return p;
 }
@@ -407,7 +431,8 @@ mxf4_plan_t make_plan(const mi355_matmul_desc_t &d) {
 int mxf4_supported(const mi355_matmul_desc_t &d) {
     if (d.src_dt != MI355_DT_F4_E2M1 || d.wei_dt != MI355_DT_F4_E2M1) return MI355_UNIMPLEMENTED;
     if (dt_bits(d.dst_dt) < 8) return MI355_UNIMPLEMENTED;
-    if (d.K < 128 || d.K % 128 != 0) return MI355_UNIMPLEMENTED;
+    // whole MX blocks; a K that ends inside a stage of 128 takes one unpipelined step more per tile
+    if (d.K < 128 || d.K % 32 != 0) return MI355_UNIMPLEMENTED;
     if (d.src_stride[2] != 1 || d.src_stride[1] % 32 != 0 || d.src_stride[0] % 32 != 0)
         return MI355_UNIMPLEMENTED;
     const bool k_major = d.wei_stride[1] == 1 && d.wei_stride[2] % 32 == 0 && d.wei_stride[0] % 32 == 0;
@@ -456,21 +481,21 @@ int mxf4_launch(const mi355_matmul_desc_t &d, const problem_t &P, void *scratch,
     // scales into the tile kernel's order (see mx_scales_rows_kernel)
     const long kb = d.K / 32;
     {
-        long blocks = (plan.pn * (kb / 4) + 255) / 256;
+        long blocks = (plan.pn * plan.nst + 255) / 256;
         if (blocks > 65535) blocks = 65535;
         hipLaunchKernelGGL(mx_scales_rows_kernel, dim3((unsigned)blocks, 1, (unsigned)plan.Bsb), dim3(256), 0, stream,
                 (const uint8_t *)P.wei_scale.p, d.N, plan.pn, kb, d.N, kb * d.N, (uint32_t *)(sc + plan.off_sb),
-                plan.pn * (kb / 4));
+                plan.pn * plan.nst);
         hipLaunchKernelGGL(mx_scales_blocks_kernel,
-                dim3((unsigned)(plan.pm / 64), (unsigned)((kb / 4 + 15) / 16), (unsigned)plan.Bsa), dim3(256), 0, stream,
+                dim3((unsigned)(plan.pm / 64), (unsigned)((plan.nst + 15) / 16), (unsigned)plan.Bsa), dim3(256), 0, stream,
                 (const uint8_t *)P.src_scale.p, d.M, plan.pm, kb, kb, d.M * kb, (uint32_t *)(sc + plan.off_sa),
-                plan.pm * (kb / 4));
+                plan.pm * plan.nst);
     }
     X.sb = sc + plan.off_sb;
-    X.sb_bstride = plan.Bsb > 1 ? plan.pn * kb : 0;
+    X.sb_bstride = plan.Bsb > 1 ? plan.pn * plan.nst * 4 : 0;
     X.sb_pitch = plan.pn * 4;
     X.sa = sc + plan.off_sa;
-    X.sa_bstride = plan.Bsa > 1 ? plan.pm * kb : 0;
+    X.sa_bstride = plan.Bsa > 1 ? plan.pm * plan.nst * 4 : 0;
     X.sa_pitch = plan.pm * 4;
     X.tiles_m = (int)((d.M + BM - 1) / BM);
     X.tiles_n = (int)((d.N + mx_geo_t::BN - 1) / mx_geo_t::BN);

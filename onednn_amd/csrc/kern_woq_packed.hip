@@ -87,6 +87,16 @@ typedef const __attribute__((address_space(4))) woqp_args_t kernarg_woqp_t;
 
 __device__ __forceinline__ v8bf as_bf(const v4i &x) { return __builtin_bit_cast(v8bf, x); }
 
+// Loads through pointers of the global address space.  The kernel's pointers come out of a block of scalar
+// registers filled by inline assembly, so the compiler cannot tell that they point to global memory and would
+// emit flat loads: those count on the LDS counter as well as on the vector-memory counter, and every wait for an
+// LDS access (the activations' staging) then waits for every load in flight -- the next unit's included.
+typedef const v4u __attribute__((address_space(1))) *global_v4u_ptr_t;
+typedef const unsigned __attribute__((address_space(1))) *global_u32_ptr_t;
+__device__ __forceinline__ v4u gload16(const uint8_t *p) { return *(global_v4u_ptr_t)(uintptr_t)p; }
+__device__ __forceinline__ v4u gload16_nt(const uint8_t *p) { return __builtin_nontemporal_load((global_v4u_ptr_t)(uintptr_t)p); }
+__device__ __forceinline__ unsigned gload4(const uint8_t *p) { return *(global_u32_ptr_t)(uintptr_t)p; }
+
 // Quantization parameters are fetched as the aligned dword that holds the
 // element (no branch on the data type next to the load, so a fetch never waits
 // for its own data); the element is cut out when the group is flushed.  A row
@@ -113,7 +123,7 @@ __device__ __forceinline__ param_lane_t param_setup(const uint8_t *p, int bits, 
 }
 
 __device__ __forceinline__ unsigned param_word(const param_lane_t &L, int g) {
-    return *(const unsigned *)(L.base + g * L.pitch + L.voff);
+    return gload4(L.base + g * L.pitch + L.voff);
 }
 
 __device__ __forceinline__ unsigned param_cut(const param_lane_t &L, unsigned word) { return (word >> L.sh) & L.mask; }
@@ -294,14 +304,13 @@ __global__ void __launch_bounds__(NWV * 64)
             for (int mt = 0; mt < MT; ++mt)
 #pragma unroll
                 for (int h = 0; h < 2; ++h)
-                    a[p][mt][h] = ALDS
-                            ? *(const v4u *)(X.src + (long)(kb + 2 * p) * (KBLK * 2) + src_row_off[mt][h])
-                            : *(const v4u *)(X.src + (long)(kb + 2 * p + h) * (KBLK * 2) + src_lane_off[mt]);
+                    a[p][mt][h] = ALDS ? gload16(X.src + (long)(kb + 2 * p) * (KBLK * 2) + src_row_off[mt][h])
+                                       : gload16(X.src + (long)(kb + 2 * p + h) * (KBLK * 2) + src_lane_off[mt]);
         // the weights are read once: non-temporal loads keep them from
         // displacing the activations and parameters in the caches
 #pragma unroll
         for (int i = 0; i < SS; ++i)
-            w[i] = __builtin_nontemporal_load((const v4u *)(wlane + (long)(kb + i) * (KBLK * CHUNK / 2)));
+            w[i] = gload16_nt(wlane + (long)(kb + i) * (KBLK * CHUNK / 2));
         // every load of the super-step is in flight before its first MFMA
         __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
@@ -359,10 +368,10 @@ __global__ void __launch_bounds__(NWV * 64)
             for (int mt = 0; mt < MT; ++mt)
 #pragma unroll
                 for (int h = 0; h < 2; ++h)
-                    u.a[p][mt][h] = *(const v4u *)(X.src + (long)(kbu + 2 * p) * (KBLK * 2) + src_row_off[mt][h]);
+                    u.a[p][mt][h] = gload16(X.src + (long)(kbu + 2 * p) * (KBLK * 2) + src_row_off[mt][h]);
 #pragma unroll
         for (int i = 0; i < U; ++i)
-            u.w[i] = __builtin_nontemporal_load((const v4u *)(wlane + (long)(kbu + i) * (KBLK * CHUNK / 2)));
+            u.w[i] = gload16_nt(wlane + (long)(kbu + i) * (KBLK * CHUNK / 2));
     };
     auto consume_unit = [&](unit_t &u, int kbu) __attribute__((always_inline)) {
 #pragma unroll
@@ -434,8 +443,8 @@ __global__ void __launch_bounds__(NWV * 64)
         for (; kb < kb1; ++kb) {
             v4u a1[MT];
 #pragma unroll
-            for (int mt = 0; mt < MT; ++mt) a1[mt] = *(const v4u *)(X.src + (long)kb * (KBLK * 2) + src_lane_off[mt]);
-            const v4u w1 = __builtin_nontemporal_load((const v4u *)(wlane_tail + (long)kb * (KBLK * CHUNK / 2)));
+            for (int mt = 0; mt < MT; ++mt) a1[mt] = gload16(X.src + (long)kb * (KBLK * 2) + src_lane_off[mt]);
+            const v4u w1 = gload16_nt(wlane_tail + (long)kb * (KBLK * CHUNK / 2));
             compute_step(w1, a1, false);
             if ((kb + 1) % X.spg == 0 || kb + 1 == kb1) {
                 unsigned word_s, word_z;
@@ -472,9 +481,9 @@ __global__ void __launch_bounds__(NWV * 64)
                     : X.dst_dt == MI355_DT_BF16 ? (unsigned)f32_to_bf16(v) : (unsigned)f32_to_f16(v);
             const long off = (long)m * X.dst_ld + chunk * CHUNK + nl;
             if (X.dst_dt == MI355_DT_F32)
-                ((unsigned *)X.dst)[off] = bits;
+                ((unsigned __attribute__((address_space(1))) *)(uintptr_t)X.dst)[off] = bits;
             else
-                ((uint16_t *)X.dst)[off] = (uint16_t)bits;
+                ((uint16_t __attribute__((address_space(1))) *)(uintptr_t)X.dst)[off] = (uint16_t)bits;
         }
         return;
     } else {

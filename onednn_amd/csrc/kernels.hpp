@@ -50,7 +50,7 @@ void set_error(const char *fmt, ...);
 // the environment variable of its name, read once per process, and changes only through mi355_tuning_set: no getenv on a
 // launch path.  Values: 0 = the library's own choice.
 enum tune_key_t { TUNE_I8_TILES = 0, TUNE_F8_TILES, TUNE_H16_TILES, TUNE_GROUPED_IMPL, TUNE_GEMM_ORDER, TUNE_COUNT };
-enum { TUNE_AUTO = 0, TUNE_LARGE = 1, TUNE_WIDE = 2, TUNE_SMALL = 3, TUNE_REF = 4, TUNE_SHORT = 5, TUNE_TALL = 6 };
+enum { TUNE_AUTO = 0, TUNE_LARGE = 1, TUNE_WIDE = 2, TUNE_SMALL = 3, TUNE_REF = 4, TUNE_SHORT = 5, TUNE_TALL = 6, TUNE_NARROW = 7 };
 int tuning(tune_key_t key);
 
 // hipFuncSetAttribute(MaxDynamicSharedMemorySize) for a kernel, once per
