@@ -497,6 +497,9 @@ def main():
                          "(reported as `sustained`; 0 = skip)")
     ap.add_argument("--no-others", action="store_true", help="skip the informational configs")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--no-ceiling", action="store_true",
+                    help="skip the measurement of the ceiling (the MFMA instruction / the weight stream by itself): "
+                         "profiler runs, where its kernels would show up next to the workload's")
     ap.add_argument("--calib-read", action="store_true",
                     help="time a read-only kernel with the decode kernel's access shape over the C2 weights "
                          "(12 rotating copies, nothing cached) and exit: the floor of the weight stream")
@@ -735,7 +738,7 @@ def main():
     }
     # next to the published peak: what this box's matrix cores (or, for decode, its memory system) deliver to a
     # kernel that does nothing else -- `frac` stays priced against the published peak
-    ceil = measured_ceiling(lib, main_name)
+    ceil = None if args.no_ceiling else measured_ceiling(lib, main_name)
     if ceil:
         roofline["ceiling"] = ceil["value"]
         roofline["ceiling_what"] = ceil["what"]

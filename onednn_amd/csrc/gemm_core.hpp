@@ -8,7 +8,8 @@
 //   HBM/L2 --global_load_lds_dwordx4--> LDS ring of NSTAGE stages
 //       stage = A[256 rows][64 B of K] + B^T[256 rows][64 B of K]  (32 KB)
 //   LDS --ds_read_b128--> MFMA operands --v_mfma--> accumulators
-//   accumulators --LDS slab transpose--> fused epilogue --> wide dst stores
+//   accumulators --fused epilogue, straight from the registers (the MFMA operands are
+//       exchanged, so a lane holds four consecutive n of a row)--> dst stores
 //
 // Both operands are consumed K-contiguous ("A" rows are src rows, "B^T" rows
 // are weight columns).  Loads bypass the register file (direct-to-LDS DMA);
@@ -17,11 +18,15 @@
 // of an MFMA operand (32 or 16 consecutive rows, one chunk) is free of bank
 // conflicts; the swizzle is applied on the global-address side of the DMA.
 //
-// Pipeline per K step kt (ring slot kt % NSTAGE):
+// Pipeline per K step kt (ring slot kt % NSTAGE), in its plainest form:
 //   s_waitcnt vmcnt(..)   own DMAs of stage kt landed
 //   s_barrier             everybody's did, and everybody finished stage kt-1
 //   issue DMAs for stage kt+NSTAGE-1 into the slot stage kt-1 used
 //   ds_read + MFMA over stage kt
+// Three loops build on it: main_loop (four wavefronts, fragments read inside the
+// step), main_loop_two_groups (eight wavefronts in two groups half a step apart)
+// and main_loop_ahead (fragments of the next stage read into a second register
+// set while the current one is multiplied).
 //
 // The DMA instructions are emitted through inline assembly so that the
 // outstanding-load counter is managed by hand (a prefetch distance of
@@ -54,9 +59,12 @@ constexpr int B_OFF = BM * BKB;       // B^T tile offset inside a stage
 //   geo_t<8, 256>  128x64 per wavefront, two wavefronts per SIMD in two groups
 //                  that alternate between reading and multiplying (96 KB of
 //                  fragment reads per K step)
-// Each kernel family uses the one measured faster on its headline shape.  (A
-// 256x128 tile with two independent workgroups per CU, geo_t<4, 128>, also runs
-// through this code; it measured 10-30 % slower than either and is not built.)
+//   geo_t<4, 128>  256x128 tiles of four wavefronts, two workgroups per CU: for
+//                  problems of at most 128 large tiles, where it puts twice the
+//                  CUs to work; with every CU busy it measured 10-30 % slower
+//                  (1.5x the stage loads per MFMA; fp8 4096x8192x28672: 1.04
+//                  against 0.91 ms)
+// Each kernel family uses the one measured faster on its headline shape.
 template <int NW_, int BN_>
 struct geo_t {
     static constexpr int NW = NW_, NT = 64 * NW_, BN = BN_;
