@@ -117,3 +117,33 @@ def test_int8_weights(gpu, oracle):
     got, name = run_gpu(p)
     assert name.startswith("hip:mfma_h16"), name
     assert_bit_exact(p, got, oracle.run_oracle(p), name)
+
+
+@pytest.mark.gpu
+def test_decode_and_prefill_of_the_same_weights_differ_by_the_weight_rounding_only(gpu):
+    """M <= 32 runs the decode kernels ((w - zp) * scale kept in f32, like ref_matmul_t), M > 32 the 16-bit tiles on
+    weights decompressed and rounded to bf16 (the JIT flavour): the same src rows against the same weights differ by
+    the bf16 rounding of each dequantized weight -- at most 2^-9 relative per weight -- plus the two f32 summations'
+    own rounding.  Bounds the batch-size dependence INTEGRATION.md describes."""
+    from tests.helpers import decode_terms, gemm_bound
+    N, K = 512, 1024
+    big = configs.config2(M=64, N=N, K=K)
+    big.dst_dt = cabi.DT_F32
+    small = configs.config2(M=32, N=N, K=K)
+    small.dst_dt = cabi.DT_F32
+    src = np.asarray(big.src).reshape(64, K)
+    small.src = np.ascontiguousarray(src[:32]).reshape(np.asarray(small.src).shape)
+    for name in ("wei", "quant"):
+        setattr(small, name, getattr(big, name))        # the same weights, scales and zero points
+    g_small, n_small = run_gpu(small)
+    g_big, n_big = run_gpu(big)
+    assert n_small.startswith("hip:woq") and n_big.startswith("hip:mfma_h16"), (n_small, n_big)
+    a = np.asarray(g_small).view(np.float32).reshape(32, N).astype(np.float64)
+    b = np.asarray(g_big).view(np.float32).reshape(64, N)[:32].astype(np.float64)
+    s, wz, G, sc, _ = decode_terms(small)                                   # src [32, K], w - zp [K, N], scales [K/G, N]
+    wdeq = np.abs(wz * np.repeat(sc, G, 0))                                 # |(w - zp) * scale|
+    asum = np.abs(s) @ wdeq                                                 # sum |src| |dequantized weight|
+    tol = 2.0 ** -9 * asum + 2 * gemm_bound(K, asum)
+    err = np.abs(a - b)
+    assert (err <= tol).all(), f"worst {np.max(err / tol):.2f} of the bound"
+    assert err.max() > 0                                                    # the two flavours do differ
