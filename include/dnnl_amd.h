@@ -237,8 +237,11 @@ typedef enum {
     dnnl_query_prop_kind = 11,
     dnnl_query_strides = 14,
     dnnl_query_src_md = 129,
+    dnnl_query_diff_src_md = 130,
     dnnl_query_weights_md = 131,
+    dnnl_query_diff_weights_md = 132,
     dnnl_query_dst_md = 133,
+    dnnl_query_diff_dst_md = 134,
     dnnl_query_scratchpad_md = 136,
     dnnl_query_exec_arg_md = 255,
     dnnl_query_ndims_s32 = 256,
@@ -265,8 +268,10 @@ typedef enum {
 #define DNNL_ARG_SRC_1 2
 #define DNNL_ARG_SRC_2 3 /* dnnl_types.h:2562: the condition of a binary select post-op */
 #define DNNL_ARG_DST 17
-#define DNNL_ARG_DIFF_SRC 129     /* dnnl_types.h:2649-2652; named by the rounding-mode rule only */
+#define DNNL_ARG_DIFF_SRC 129     /* dnnl_types.h:2649-2652 */
+#define DNNL_ARG_DIFF_DST 145     /* dnnl_types.h:2676-2679 */
 #define DNNL_ARG_DIFF_WEIGHTS 161 /* dnnl_types.h:2697-2700 */
+#define DNNL_ARG_DIFF_BIAS 169    /* dnnl_types.h:2724 */
 #define DNNL_ARG_WEIGHTS 33
 #define DNNL_ARG_BIAS 41
 #define DNNL_ARG_SCRATCHPAD 80
@@ -460,8 +465,12 @@ dnnl_status_t dnnl_inner_product_forward_primitive_desc_create(dnnl_primitive_de
         dnnl_engine_t engine, dnnl_prop_kind_t prop_kind, const_dnnl_memory_desc_t src_desc,
         const_dnnl_memory_desc_t weights_desc, const_dnnl_memory_desc_t bias_desc,
         const_dnnl_memory_desc_t dst_desc, const_dnnl_primitive_attr_t attr);
-/* dnnl.h:2781-2787, :2809-2817: the descriptors are validated as in src/common/inner_product.cpp:205-230; no
- * implementation is offered for backward propagation (dnnl_unimplemented) */
+/* dnnl.h:2781-2787, :2809-2817 (src/common/inner_product.cpp:205-230; the naive implementations
+ * src/cpu/ref_inner_product.cpp:100-217): f32 / bf16 / f16 tensors, no attributes; both lower to matmuls over
+ * the tensors as they lie -- diff_src = diff_dst x weights; diff_weights = diff_dst^T x src, diff_bias = the
+ * column sums of diff_dst in the reference's order of additions.  Execute arguments: DNNL_ARG_DIFF_DST,
+ * DNNL_ARG_WEIGHTS, DNNL_ARG_DIFF_SRC / DNNL_ARG_SRC, DNNL_ARG_DIFF_DST, DNNL_ARG_DIFF_WEIGHTS,
+ * DNNL_ARG_DIFF_BIAS.  hint_fwd_pd is accepted and not needed. */
 dnnl_status_t dnnl_inner_product_backward_data_primitive_desc_create(dnnl_primitive_desc_t *primitive_desc,
         dnnl_engine_t engine, const_dnnl_memory_desc_t diff_src_desc, const_dnnl_memory_desc_t weights_desc,
         const_dnnl_memory_desc_t diff_dst_desc, const_dnnl_primitive_desc_t hint_fwd_pd,

@@ -503,6 +503,13 @@ const char *mi355_grouped_matmul_impl(const mi355_grouped_desc_t *desc);
  * not 16-byte aligned run on "hip:ref_grouped:any". */
 int mi355_grouped_matmul_launch(const mi355_grouped_desc_t *desc, const mi355_grouped_args_t *args, void *stream);
 
+/* out[c] = sum_r x[r * ld + c] over `rows` rows, added in row order in f32 and
+ * stored as out_dt (x_dt, out_dt: f32 / bf16 / f16).  The bias gradient of the
+ * inner product, with the operation order of the reference's loop
+ * (src/cpu/ref_inner_product.cpp:196-210).  Asynchronous on `stream`. */
+int mi355_colsum_launch(const void *x, int x_dt, int64_t rows, int64_t cols, int64_t ld, void *out, int out_dt,
+        void *stream);
+
 #ifdef __cplusplus
 }
 #endif

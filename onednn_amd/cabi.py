@@ -151,7 +151,7 @@ KERNEL_SYMBOLS = [
     "mi355_stream_wait_event", "mi355_mem_store_scalar",
     "mi355_last_error", "mi355_matmul_query", "mi355_matmul_impl_name",
     "mi355_matmul_scratch_bytes", "mi355_matmul_launch", "mi355_matmul_launch_noalloc", "mi355_reorder_query",
-    "mi355_reorder_launch", "mi355_wei_pack_reorder_dims", "mi355_tuning_set", "mi355_grouped_matmul_query",
+    "mi355_reorder_launch", "mi355_wei_pack_reorder_dims", "mi355_tuning_set", "mi355_colsum_launch", "mi355_grouped_matmul_query",
     "mi355_grouped_matmul_launch", "mi355_grouped_matmul_impl",
 ]
 
@@ -182,6 +182,7 @@ def load_kernels():
     lib.mi355_matmul_impl_name.restype = C.c_char_p
     lib.mi355_matmul_impl_name.argtypes = [C.c_int]
     lib.mi355_tuning_set.argtypes = [C.c_char_p, C.c_char_p]
+    lib.mi355_colsum_launch.argtypes = [vp, C.c_int, C.c_int64, C.c_int64, C.c_int64, vp, C.c_int, vp]
     lib.mi355_device_count.argtypes = [C.POINTER(C.c_int)]
     lib.mi355_device_set.argtypes = [C.c_int]
     lib.mi355_device_info.argtypes = [C.c_int, C.c_char_p, C.c_size_t, C.POINTER(C.c_int),

@@ -133,3 +133,31 @@ extern "C" int mi355_mem_store_scalar(void *dptr, uint64_t bits, int nbytes, voi
             nbytes);
     return hipGetLastError() == hipSuccess ? MI355_SUCCESS : MI355_RUNTIME_ERROR;
 }
+
+namespace mi355 {
+// out[c] = sum over r of x[r][c], r = 0, 1, ... in that order in f32 (the order of the reference's bias-gradient loop,
+// src/cpu/ref_inner_product.cpp:196-210): a thread per column, consecutive lanes consecutive columns
+__global__ void __launch_bounds__(256) colsum_kernel(const void *x, int x_dt, long rows, long cols, long ld, void *out,
+        int out_dt) {
+    const long c = (long)blockIdx.x * blockDim.x + threadIdx.x;
+    if (c >= cols) return;
+    float acc = 0.f;
+    for (long r = 0; r < rows; ++r) acc += load_float(x_dt, x, r * ld + c);
+    const uint32_t bits = cvt_store_bits(out_dt, acc);
+    if (dt_bits(out_dt) == 32) ((uint32_t *)out)[c] = bits;
+    else ((uint16_t *)out)[c] = (uint16_t)bits;
+}
+} // namespace mi355
+
+extern "C" int mi355_colsum_launch(const void *x, int x_dt, int64_t rows, int64_t cols, int64_t ld, void *out, int out_dt,
+        void *stream) {
+    auto fp = [](int dt) { return dt == MI355_DT_F32 || dt == MI355_DT_BF16 || dt == MI355_DT_F16; };
+    if ((!x && rows > 0) || !out || rows < 0 || cols < 0 || ld < cols || !fp(x_dt) || !fp(out_dt)) {
+        set_error("colsum: f32 / bf16 / f16 rows of at least `cols` elements");
+        return MI355_INVALID_ARGUMENTS;
+    }
+    if (cols == 0) return MI355_SUCCESS;
+    hipLaunchKernelGGL(colsum_kernel, dim3((unsigned)((cols + 255) / 256)), dim3(256), 0, (hipStream_t)stream, x, x_dt,
+            (long)rows, (long)cols, (long)ld, out, out_dt);
+    return hipGetLastError() == hipSuccess ? MI355_SUCCESS : MI355_RUNTIME_ERROR;
+}

@@ -30,6 +30,7 @@ kind_inner_product = 10
 forward_training, forward_inference, backward_data, backward_weights = 64, 96, 160, 192
 query_primitive_kind, query_prop_kind = 2, 11
 query_impl_info_str, query_src_md, query_weights_md, query_dst_md, query_scratchpad_md = 8, 129, 131, 133, 136
+query_diff_src_md, query_diff_weights_md, query_diff_dst_md = 130, 132, 134
 query_ndims_s32, query_dims, query_data_type, query_strides, query_memory_consumption = 256, 257, 258, 14, 6
 query_format_kind = 262
 quantization_mode_undef, quantization_mode_static_sazp, quantization_mode_dynamic_mx, quantization_mode_dynamic_fp = 0, 1, 2, 3
@@ -40,7 +41,7 @@ ARG_FROM, ARG_TO = ARG_SRC, ARG_DST
 ARG_ATTR_PRECOMPUTED_REDUCTIONS, ARG_ATTR_SCALES, ARG_ATTR_ZERO_POINTS = 512, 4096, 8192
 ARG_ATTR_DROPOUT_OFFSET, ARG_ATTR_ROUNDING_SEED, ARG_ATTR_DROPOUT_MASK = 507, 508, 509
 ARG_ATTR_DROPOUT_PROBABILITY, ARG_ATTR_DROPOUT_SEED = 510, 511
-ARG_DIFF_SRC, ARG_DIFF_WEIGHTS = 129, 161
+ARG_DIFF_SRC, ARG_DIFF_DST, ARG_DIFF_WEIGHTS, ARG_DIFF_BIAS = 129, 145, 161, 169
 rounding_environment, rounding_stochastic = 0, 1
 s64 = 16                               # dnnl_s64: the dropout seed / offset type
 scratchpad_library, scratchpad_user = 0, 1
@@ -413,6 +414,32 @@ class inner_product_forward_primitive_desc(matmul_primitive_desc):
         return v.value
 
 
+class inner_product_backward_data_primitive_desc(inner_product_forward_primitive_desc):
+    """dnnl::inner_product_backward_data::primitive_desc(engine, diff_src_md, weights_md, diff_dst_md, hint_fwd_pd,
+    attr)"""
+
+    def __init__(self, eng, diff_src_md, weights_md, diff_dst_md, hint_fwd_pd=None, attr=None):
+        self.engine = eng
+        self.h = C.c_void_p()
+        _check(lib().dnnl_inner_product_backward_data_primitive_desc_create(
+            C.byref(self.h), eng.h, diff_src_md.h, weights_md.h, diff_dst_md.h,
+            hint_fwd_pd.h if hint_fwd_pd else None, attr.h if attr else None),
+            "inner_product_backward_data_primitive_desc_create")
+
+
+class inner_product_backward_weights_primitive_desc(inner_product_forward_primitive_desc):
+    """dnnl::inner_product_backward_weights::primitive_desc(engine, src_md, diff_weights_md, diff_bias_md,
+    diff_dst_md, hint_fwd_pd, attr)"""
+
+    def __init__(self, eng, src_md, diff_weights_md, diff_dst_md, diff_bias_md=None, hint_fwd_pd=None, attr=None):
+        self.engine = eng
+        self.h = C.c_void_p()
+        _check(lib().dnnl_inner_product_backward_weights_primitive_desc_create(
+            C.byref(self.h), eng.h, src_md.h, diff_weights_md.h, diff_bias_md.h if diff_bias_md else None,
+            diff_dst_md.h, hint_fwd_pd.h if hint_fwd_pd else None, attr.h if attr else None),
+            "inner_product_backward_weights_primitive_desc_create")
+
+
 class reorder_primitive_desc(matmul_primitive_desc):
     """dnnl::reorder::primitive_desc(src_engine, src_md, dst_engine, dst_md, attr)"""
 
@@ -440,6 +467,15 @@ class matmul:
 
 class inner_product_forward(matmul):
     """dnnl::inner_product_forward(pd); execute(stream, {ARG_SRC, ARG_WEIGHTS, ARG_BIAS, ARG_DST, ...})"""
+
+
+class inner_product_backward_data(matmul):
+    """dnnl::inner_product_backward_data(pd); execute(stream, {ARG_DIFF_DST, ARG_WEIGHTS, ARG_DIFF_SRC})"""
+
+
+class inner_product_backward_weights(matmul):
+    """dnnl::inner_product_backward_weights(pd); execute(stream, {ARG_DIFF_DST, ARG_SRC, ARG_DIFF_WEIGHTS,
+    ARG_DIFF_BIAS})"""
 
 
 class reorder(matmul):

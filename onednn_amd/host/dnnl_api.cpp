@@ -240,6 +240,12 @@ struct dnnl_primitive_desc {
     int prop_kind = 96;           // dnnl_forward_inference
     dnnl_memory_desc ip_src, ip_wei, ip_bias;
     dnnl_primitive_attr ip_attr;
+    // inner product backward: dnnl_backward_data (diff_src = diff_dst x weights) or dnnl_backward_weights
+    // (diff_weights = diff_dst^T x src, diff_bias = column sums of diff_dst) lowered to a matmul whose src / weights
+    // / dst are other execute arguments; ip_src / ip_wei / ip_bias / ip_dst hold (diff_)src, (diff_)weights,
+    // diff_bias and diff_dst as the caller describes them
+    dnnl_memory_desc ip_dst;
+    bool ip_diff_bias = false;
     mi355_grouped_desc_t gdesc;
     std::vector<int> impls;       // kernel families that can run it, best first
     size_t impl_pos = 0;
@@ -2038,28 +2044,134 @@ DNNL_EXPORT dnnl_status_t dnnl_inner_product_forward_primitive_desc_create(dnnl_
     return dnnl_success;
 }
 
-// src/common/inner_product.cpp:205-230: validated, then no implementation in the list
+// Inner product, backward (src/common/inner_product.cpp:205-230; the naive implementations
+// src/cpu/ref_inner_product.cpp:100-217 and their data types, ref_inner_product.hpp:118-139, :196-218): both are
+// matmuls over the tensors as they lie.
+//   data:     diff_src[mb, k]     = sum_oc diff_dst[mb, oc] * weights[oc, k]    [mb, oc] x [oc, K]
+//   weights:  diff_weights[oc, k] = sum_mb diff_dst[mb, oc] * src[mb, k]        [oc, mb] x [mb, K], src = diff_dst^T
+//             diff_bias[oc]       = sum_mb diff_dst[mb, oc]                     column sums, in the reference's order
+// k = (ic, spatial) flattened: the reduced dims must be dense and in the same memory order in both tensors that carry
+// them, as in the forward lowering.
+namespace {
+// the flattened K of a tensor [x, ic, spatial...]: element stride of k in `ks`; false if the dims do not flatten
+bool ip_flatten(const dnnl_memory_desc &t, const int *order, int n_inner, dim_t *ks) {
+    *ks = 1;
+    if (n_inner == 0) return true;
+    *ks = t.strides[order[n_inner - 1]];
+    for (int i = 0; i + 1 < n_inner; ++i)
+        if (t.strides[order[i]] != t.strides[order[i + 1]] * t.dims[order[i + 1]]) return false;
+    return true;
+}
+dnnl_status_t ip_backward_create(dnnl_primitive_desc_t *primitive_desc, dnnl_engine_t engine, bool data,
+        const dnnl_memory_desc *x_desc /* diff_src | src */, const dnnl_memory_desc *w_desc /* weights | diff_weights */,
+        const dnnl_memory_desc *bias_in, const dnnl_memory_desc *ddst_desc, const_dnnl_primitive_attr_t attr) {
+    dnnl_memory_desc x = *x_desc, w = *w_desc, dd = *ddst_desc, bias;
+    if (bias_in) bias = *bias_in;
+    const int nd = x.ndims;
+    for (const dnnl_memory_desc *m : {&x, &w, &dd})
+        CHECK_UNIMPL(m->kind == dnnl_blocked || m->kind == dnnl_format_kind_any);
+    CHECK_UNIMPL(!x.grouped && !w.grouped && !dd.grouped);
+    // no attributes on the backward passes of the naive implementations (attr is default or absent)
+    if (attr) {
+        const dnnl_primitive_attr &a = *attr;
+        CHECK_UNIMPL(a.scales.empty() && a.zero_points.empty() && a.reductions.empty() && a.post_ops.entries.empty()
+                && !a.with_dropout() && a.rounding.empty());
+    }
+    auto fp = [](dnnl_data_type_t dt) { return dt == dnnl_f32 || dt == dnnl_bf16 || dt == dnnl_f16; };
+    if (data) { // diff_src in {f32, wei}, wei in {f32, bf16, f16}, diff_dst == wei
+        CHECK_UNIMPL(fp(w.dt) && dd.dt == w.dt && (x.dt == dnnl_f32 || x.dt == w.dt));
+    } else {    // src in {f32, bf16, f16}, diff_dst == src, diff_weights in {f32, src}, diff_bias in {f32, src}
+        CHECK_UNIMPL(fp(x.dt) && dd.dt == x.dt && (w.dt == dnnl_f32 || w.dt == x.dt));
+        if (bias_in) CHECK_UNIMPL(bias.dt == dnnl_f32 || bias.dt == x.dt);
+    }
+    // format `any`: as in the forward pass, the two tensors with reduced dims take each other's order
+    int perm[DNNL_MAX_NDIMS];
+    auto outer_first = [&](int *pm) {
+        if (nd > 1 && pm[nd - 1] == 0) {
+            for (int i = nd - 1; i > 0; --i) pm[i] = pm[i - 1];
+            pm[0] = 0;
+        }
+    };
+    if (x.kind == dnnl_format_kind_any) {
+        if (w.kind == dnnl_format_kind_any) {
+            x.set_dense();
+        } else {
+            memory_order(w, perm);
+            outer_first(perm);
+            x.set_dense(perm);
+        }
+    }
+    if (w.kind == dnnl_format_kind_any) {
+        memory_order(x, perm);
+        outer_first(perm);
+        w.set_dense(perm);
+    }
+    if (dd.kind == dnnl_format_kind_any) dd.set_dense();
+    if (bias_in && bias.kind == dnnl_format_kind_any) bias.set_dense();
+    if (bias_in) CHECK_UNIMPL(bias.kind == dnnl_blocked && bias.strides[0] == 1 && dd.strides[1] == 1);
+
+    int order[DNNL_MAX_NDIMS], n_inner = 0;
+    memory_order(x, perm);
+    for (int i = 0; i < nd; ++i)
+        if (perm[i] != 0 && x.dims[perm[i]] != 1) order[n_inner++] = perm[i];
+    dim_t K = 1, x_ks = 1, w_ks = 1;
+    for (int i = 1; i < nd; ++i) K *= x.dims[i];
+    CHECK_UNIMPL(ip_flatten(x, order, n_inner, &x_ks) && ip_flatten(w, order, n_inner, &w_ks));
+    const dim_t MB = x.dims[0], OC = w.dims[0];
+    auto md2 = [](dnnl_data_type_t dt, dim_t d0, dim_t d1, dim_t s0, dim_t s1) {
+        dnnl_memory_desc m;
+        m.ndims = 2; m.dt = dt; m.kind = dnnl_blocked;
+        m.dims[0] = d0; m.dims[1] = d1; m.strides[0] = s0; m.strides[1] = s1;
+        return m;
+    };
+    dnnl_memory_desc a2, b2, c2;
+    if (data) {
+        a2 = md2(dd.dt, MB, OC, dd.strides[0], dd.strides[1]);
+        b2 = md2(w.dt, OC, K, w.strides[0], w_ks);
+        c2 = md2(x.dt, MB, K, x.strides[0], x_ks);
+    } else {
+        a2 = md2(dd.dt, OC, MB, dd.strides[1], dd.strides[0]);
+        b2 = md2(x.dt, MB, K, x.strides[0], x_ks);
+        c2 = md2(w.dt, OC, K, w.strides[0], w_ks);
+    }
+    dnnl_primitive_desc_t mm = nullptr;
+    const dnnl_status_t st = dnnl_matmul_primitive_desc_create(&mm, engine, &a2, &b2, nullptr, &c2, nullptr);
+    if (st) return st;
+    mm->inner_product = true;
+    mm->prop_kind = data ? (int)dnnl_backward_data : (int)dnnl_backward_weights;
+    mm->ip_src = x; mm->ip_wei = w; mm->ip_dst = dd;
+    mm->ip_diff_bias = bias_in != nullptr;
+    if (bias_in) mm->ip_bias = bias;
+    if (attr) mm->ip_attr = *attr;
+    if (verbose_level() >= 1)
+        fprintf(stderr, "onednn_verbose,v1,primitive,create:dispatch,gpu,inner_product,%s\n", mm->impl_name.c_str());
+    *primitive_desc = mm;
+    return dnnl_success;
+}
+} // namespace
+
 DNNL_EXPORT dnnl_status_t dnnl_inner_product_backward_data_primitive_desc_create(dnnl_primitive_desc_t *primitive_desc,
         dnnl_engine_t engine, const_dnnl_memory_desc_t diff_src_desc, const_dnnl_memory_desc_t weights_desc,
         const_dnnl_memory_desc_t diff_dst_desc, const_dnnl_primitive_desc_t hint_fwd_pd,
         const_dnnl_primitive_attr_t attr) {
-    (void)hint_fwd_pd; (void)attr;
+    (void)hint_fwd_pd;
     CHECK_ARG(primitive_desc && engine);
     dnnl_status_t st = ip_check_shapes(diff_src_desc, weights_desc, nullptr, diff_dst_desc);
     if (st) return st;
-    return dnnl_unimplemented;
+    return ip_backward_create(primitive_desc, engine, true, diff_src_desc, weights_desc, nullptr, diff_dst_desc, attr);
 }
 DNNL_EXPORT dnnl_status_t dnnl_inner_product_backward_weights_primitive_desc_create(
         dnnl_primitive_desc_t *primitive_desc, dnnl_engine_t engine, const_dnnl_memory_desc_t src_desc,
         const_dnnl_memory_desc_t diff_weights_desc, const_dnnl_memory_desc_t diff_bias_desc,
         const_dnnl_memory_desc_t diff_dst_desc, const_dnnl_primitive_desc_t hint_fwd_pd,
         const_dnnl_primitive_attr_t attr) {
-    (void)hint_fwd_pd; (void)attr;
+    (void)hint_fwd_pd;
     CHECK_ARG(primitive_desc && engine);
-    const dnnl_memory_desc *b = (diff_bias_desc && !diff_bias_desc->is_zero()) ? diff_bias_desc : nullptr;
+    const dnnl_memory_desc *b = (diff_bias_desc && !diff_bias_desc->is_zero()
+            && diff_bias_desc->kind != dnnl_format_kind_undef) ? diff_bias_desc : nullptr;
     dnnl_status_t st = ip_check_shapes(src_desc, diff_weights_desc, b, diff_dst_desc);
     if (st) return st;
-    return dnnl_unimplemented;
+    return ip_backward_create(primitive_desc, engine, false, src_desc, diff_weights_desc, b, diff_dst_desc, attr);
 }
 
 // ---- reorder primitive descriptor (src/common/reorder.cpp:67-170)
@@ -2197,7 +2309,37 @@ DNNL_EXPORT const_dnnl_memory_desc_t dnnl_primitive_desc_query_md(const_dnnl_pri
             default: return nullptr;
         }
     }
-    if (pd->inner_product) { // the tensors as the caller describes them; dst is two-dimensional either way
+    if (pd->inner_product && pd->prop_kind == (int)dnnl_backward_data) {
+        switch (what) {
+            case dnnl_query_diff_src_md: return index == 0 ? &pd->ip_src : nullptr;
+            case dnnl_query_weights_md: return index == 0 ? &pd->ip_wei : nullptr;
+            case dnnl_query_diff_dst_md: return index == 0 ? &pd->ip_dst : nullptr;
+            case dnnl_query_src_md: case dnnl_query_dst_md: case dnnl_query_diff_weights_md: return nullptr;
+            case dnnl_query_exec_arg_md:
+                if (index == DNNL_ARG_DIFF_SRC) return &pd->ip_src;
+                if (index == DNNL_ARG_WEIGHTS) return &pd->ip_wei;
+                if (index == DNNL_ARG_DIFF_DST) return &pd->ip_dst;
+                if (index == DNNL_ARG_SCRATCHPAD) return &pd->scratchpad;
+                return nullptr;
+            default: break;
+        }
+    } else if (pd->inner_product && pd->prop_kind == (int)dnnl_backward_weights) {
+        switch (what) {
+            case dnnl_query_src_md: return index == 0 ? &pd->ip_src : nullptr;
+            case dnnl_query_diff_weights_md:
+                return index == 0 ? &pd->ip_wei : index == 1 ? (pd->ip_diff_bias ? &pd->ip_bias : &zero_md) : nullptr;
+            case dnnl_query_diff_dst_md: return index == 0 ? &pd->ip_dst : nullptr;
+            case dnnl_query_weights_md: case dnnl_query_dst_md: case dnnl_query_diff_src_md: return nullptr;
+            case dnnl_query_exec_arg_md:
+                if (index == DNNL_ARG_SRC) return &pd->ip_src;
+                if (index == DNNL_ARG_DIFF_WEIGHTS) return &pd->ip_wei;
+                if (index == DNNL_ARG_DIFF_BIAS) return pd->ip_diff_bias ? &pd->ip_bias : &zero_md;
+                if (index == DNNL_ARG_DIFF_DST) return &pd->ip_dst;
+                if (index == DNNL_ARG_SCRATCHPAD) return &pd->scratchpad;
+                return nullptr;
+            default: break;
+        }
+    } else if (pd->inner_product) { // the tensors as the caller describes them; dst is two-dimensional either way
         switch (what) {
             case dnnl_query_src_md: return index == 0 ? &pd->ip_src : nullptr;
             case dnnl_query_weights_md:
@@ -2302,6 +2444,42 @@ DNNL_EXPORT dnnl_status_t dnnl_primitive_execute(const_dnnl_primitive_t cprimiti
     for (int i = 0; i < nargs; ++i) {
         CHECK_ARG(m.find(args[i].arg) == m.end()); // duplicated argument
         m[args[i].arg] = args[i].memory;
+    }
+    // inner product backward: the matmul it lowers to takes its src / weights / dst from other arguments
+    dnnl_memory_t ip_diff_bias_mem = nullptr, ip_diff_dst_mem = nullptr;
+    if (pd0.inner_product && pd0.prop_kind != (int)dnnl_forward_training && pd0.prop_kind != (int)dnnl_forward_inference) {
+        auto get = [&](int arg) -> dnnl_memory_t {
+            auto it = m.find(arg);
+            return it == m.end() ? nullptr : it->second;
+        };
+        dnnl_memory_t dd = get(DNNL_ARG_DIFF_DST);
+        CHECK_ARG(dd);
+        ip_diff_dst_mem = dd;
+        if (pd0.prop_kind == (int)dnnl_backward_data) {
+            dnnl_memory_t ds = get(DNNL_ARG_DIFF_SRC);
+            CHECK_ARG(ds && get(DNNL_ARG_WEIGHTS));
+            m[DNNL_ARG_SRC] = dd;
+            m[DNNL_ARG_DST] = ds;
+        } else {
+            dnnl_memory_t sr = get(DNNL_ARG_SRC), dw = get(DNNL_ARG_DIFF_WEIGHTS);
+            CHECK_ARG(sr && dw);
+            ip_diff_bias_mem = get(DNNL_ARG_DIFF_BIAS);
+            CHECK_ARG(IMPLICATION(pd0.ip_diff_bias, ip_diff_bias_mem != nullptr));
+            if (pd0.ip_src.dims[0] == 0) {
+                // an empty batch: the sums over mb are empty, diff_weights and diff_bias are zeros
+                // (the loops of src/cpu/ref_inner_product.cpp:165-212 store their initial 0)
+                if (mi355_device_set((int)pd0.engine->index) != MI355_SUCCESS) return dnnl_runtime_error;
+                int rc0 = dw->handle ? mi355_mem_set(dw->handle, 0, pd0.ip_wei.size_bytes(), stream->hip_stream)
+                                     : MI355_INVALID_ARGUMENTS;
+                if (rc0 == MI355_SUCCESS && ip_diff_bias_mem && pd0.ip_diff_bias)
+                    rc0 = mi355_colsum_launch(nullptr, (int)pd0.ip_dst.dt, 0, pd0.ip_dst.dims[1], pd0.ip_dst.dims[1],
+                            ip_diff_bias_mem->handle, (int)pd0.ip_bias.dt, stream->hip_stream);
+                return from_mi355(rc0);
+            }
+            m[DNNL_ARG_SRC] = dd;
+            m[DNNL_ARG_WEIGHTS] = sr;
+            m[DNNL_ARG_DST] = dw;
+        }
     }
     std::unique_lock<std::mutex> lock(prim->scratch_mutex, std::defer_lock);
     // Called before the first use of the primitive's own device memory in this
@@ -2543,6 +2721,12 @@ DNNL_EXPORT dnnl_status_t dnnl_primitive_execute(const_dnnl_primitive_t cprimiti
                 if (pd.desc.post_ops[k].kind == MI355_PO_BINARY) B.po_arg[k] = shifted(A.po_arg[k], op[k], pd.desc.post_ops[k].dt);
             rc = mi355_matmul_launch(&pd.desc, &B, scratch, stream->hip_stream);
         }
+    }
+    if (rc == MI355_SUCCESS && ip_diff_bias_mem && pd0.ip_diff_bias) {
+        // diff_bias[oc] = sum over mb of diff_dst[mb, oc], added in the order of the rows
+        CHECK_ARG(ip_diff_bias_mem->handle && ip_diff_dst_mem->handle);
+        rc = mi355_colsum_launch(ip_diff_dst_mem->handle, (int)pd0.ip_dst.dt, pd0.ip_dst.dims[0], pd0.ip_dst.dims[1],
+                pd0.ip_dst.strides[0], ip_diff_bias_mem->handle, (int)pd0.ip_bias.dt, stream->hip_stream);
     }
     if (ordered && prim->order_event) {
         if (mi355_event_record(prim->order_event, stream->hip_stream) == MI355_SUCCESS) {

@@ -113,6 +113,57 @@ def run_oracle_inner_product(prob: MatmulProblem, src, wei):
     return dst
 
 
+def _elem_strides(a):
+    assert min(a.strides) >= 0
+    return np.array([x // a.itemsize for x in a.strides], np.int64)
+
+
+def run_oracle_inner_product_bwd_data(diff_dst, wei, dsrc_shape, dts, dsrc_order=None):
+    """diff_src of the inner product.  `diff_dst` [mb, oc] and `wei` [oc, ic, spatial...] are numpy views (storage
+    types) in any memory order; dts = (diff_src, weights, diff_dst) data type names; the result is a view of the
+    logical shape `dsrc_shape` whose memory order is `dsrc_order` (a permutation, outermost first; default plain)."""
+    lib = load()
+    lib.oracle_inner_product_bwd_data.argtypes = [C.c_int, C.c_void_p, C.c_int64, C.c_int, C.c_void_p, C.c_void_p,
+                                                  C.c_int, C.c_void_p, C.c_void_p, C.c_int, C.c_void_p, C.c_void_p]
+    from onednn_amd.problem import storage_dtype
+    nd = len(dsrc_shape)
+    order = list(dsrc_order) if dsrc_order is not None else list(range(nd))
+    store = np.zeros([dsrc_shape[i] for i in order], storage_dtype(cabi.DT_NAMES[dts[0]]))
+    out = store.transpose(np.argsort(order))
+    dims = np.array(dsrc_shape, np.int64)
+    s_o, s_w, s_d = _elem_strides(out), _elem_strides(wei), _elem_strides(diff_dst)
+    st = lib.oracle_inner_product_bwd_data(nd, dims.ctypes.data, wei.shape[0], cabi.DT_NAMES[dts[0]], s_o.ctypes.data,
+                                           store.ctypes.data, cabi.DT_NAMES[dts[1]], s_w.ctypes.data, wei.ctypes.data,
+                                           cabi.DT_NAMES[dts[2]], s_d.ctypes.data, diff_dst.ctypes.data)
+    assert st == 0, f"oracle_inner_product_bwd_data status {st}"
+    return out
+
+
+def run_oracle_inner_product_bwd_weights(diff_dst, src, dts, with_bias, dwei_order=None):
+    """(diff_weights, diff_bias or None).  `diff_dst` [mb, oc], `src` [mb, ic, spatial...]: numpy views;
+    dts = (src, diff_weights, diff_bias, diff_dst) data type names."""
+    lib = load()
+    lib.oracle_inner_product_bwd_weights.argtypes = [C.c_int, C.c_void_p, C.c_int64, C.c_int, C.c_void_p, C.c_void_p,
+                                                     C.c_int, C.c_void_p, C.c_void_p, C.c_int, C.c_void_p,
+                                                     C.c_int, C.c_void_p, C.c_void_p]
+    from onednn_amd.problem import storage_dtype
+    nd, oc = src.ndim, diff_dst.shape[1]
+    shape = (oc,) + tuple(src.shape[1:])
+    order = list(dwei_order) if dwei_order is not None else list(range(nd))
+    store = np.zeros([shape[i] for i in order], storage_dtype(cabi.DT_NAMES[dts[1]]))
+    out = store.transpose(np.argsort(order))
+    bias = np.zeros(oc, storage_dtype(cabi.DT_NAMES[dts[2]])) if with_bias else None
+    dims = np.array(src.shape, np.int64)
+    s_s, s_o, s_d = _elem_strides(src), _elem_strides(out), _elem_strides(diff_dst)
+    st = lib.oracle_inner_product_bwd_weights(nd, dims.ctypes.data, oc, cabi.DT_NAMES[dts[0]], s_s.ctypes.data,
+                                              src.ctypes.data, cabi.DT_NAMES[dts[1]], s_o.ctypes.data, store.ctypes.data,
+                                              cabi.DT_NAMES[dts[2]] if with_bias else 0,
+                                              bias.ctypes.data if with_bias else None, cabi.DT_NAMES[dts[3]],
+                                              s_d.ctypes.data, diff_dst.ctypes.data)
+    assert st == 0, f"oracle_inner_product_bwd_weights status {st}"
+    return out, bias
+
+
 def run_oracle_dropout(prob: MatmulProblem):
     """(raw dst storage, the dropout mask or None)."""
     prob._oracle_mask = None

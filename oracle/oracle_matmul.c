@@ -27,6 +27,9 @@
  *                     ::execute src/cpu/reorder/simple_reorder.hpp:2579-2661 and
  *                     its 4-bit variants :2168-2288 (f32 -> s4/u4/f4) and
  *                     :2291-2425 (s4/u4/f4 -> f32/bf16/f16)
+ *   oracle_inner_product_bwd_data, oracle_inner_product_bwd_weights
+ *                     ref_inner_product_bwd_data_t / _bwd_weights_t
+ *                     src/cpu/ref_inner_product.cpp:100-217
  *   oracle_inner_product_fwd
  *                     ref_inner_product_fwd_t::execute_forward src/cpu/ref_inner_product.cpp:33-100
  *                     and ref_inner_product_int8_fwd_t::execute_forward
@@ -78,6 +81,11 @@
  * dims on exact data for every ndims and for permuted layouts of src and
  * weights, the scale / bias / dst-scale order on values where a different
  * order changes bits; bias, post-ops and the store are orc_finish.
+ * The backward inner products (oracle_inner_product_bwd_data / _bwd_weights)
+ * are pinned there too: numpy tensordot on exact data over the other index
+ * pair for every ndims and for permuted layouts (a transposed operand or a
+ * wrong reduced index changes every element), diff_bias against a column sum
+ * and against a hand-ordered f32 sum whose bits depend on the order.
  * Unpinned: none of the functions used by the five benchmark configurations.
  * "Parity unpinned" beyond the textbook formula: the last bits of the
  * libm-dependent eltwise algorithms (tanh, elu, exp, log, pow, gelu_erf,
@@ -915,6 +923,76 @@ int oracle_inner_product_fwd(int ndims, const int64_t *dims, int64_t OC, const i
             }
             orc_finish(&t, a, d, 0, mb, oc);
         }
+    return MI355_SUCCESS;
+}
+
+/* Offset of element k (row-major index over dims[1..]) of row `row` of a tensor
+ * [x, ic, spatial...] with the given strides. */
+static int64_t orc_ip_off(int ndims, const int64_t *dims, const int64_t *stride, int64_t row, int64_t k) {
+    int64_t off = row * stride[0];
+    for (int i = ndims - 1; i >= 1; --i) {
+        off += (k % dims[i]) * stride[i];
+        k /= dims[i];
+    }
+    return off;
+}
+
+/* Inner product, backward by data (ref_inner_product_bwd_data_t::execute_backward_data,
+ * src/cpu/ref_inner_product.cpp:100-143):
+ *   diff_src[mb, ic, ...] = sum over oc, ascending, of diff_dst[mb, oc] * weights[oc, ic, ...]
+ * in f32, stored as diff_src's type.  `dims` are diff_src's dims; dd_stride are
+ * the two strides of diff_dst. */
+int oracle_inner_product_bwd_data(int ndims, const int64_t *dims, int64_t OC, int dsrc_dt, const int64_t *dsrc_stride,
+        void *diff_src, int wei_dt, const int64_t *wei_stride, const void *wei, int dd_dt, const int64_t *dd_stride,
+        const void *diff_dst) {
+    if (!dims || !dsrc_stride || !wei_stride || !dd_stride || ndims < 2 || ndims > 5) return MI355_INVALID_ARGUMENTS;
+    const int64_t MB = dims[0];
+    int64_t Kt = 1;
+    for (int i = 1; i < ndims; ++i) Kt *= dims[i];
+#pragma omp parallel for schedule(static)
+    for (int64_t mb = 0; mb < MB; ++mb)
+        for (int64_t k = 0; k < Kt; ++k) {
+            float ds = 0.f;
+            for (int64_t oc = 0; oc < OC; ++oc) {
+                const float dd = orc_load_float(dd_dt, diff_dst, mb * dd_stride[0] + oc * dd_stride[1]);
+                const float w = orc_load_float(wei_dt, wei, orc_ip_off(ndims, dims, wei_stride, oc, k));
+                ds += dd * w;
+            }
+            orc_store_float(dsrc_dt, ds, diff_src, orc_ip_off(ndims, dims, dsrc_stride, mb, k));
+        }
+    return MI355_SUCCESS;
+}
+
+/* Inner product, backward by weights (ref_inner_product_bwd_weights_t::execute_backward_weights,
+ * src/cpu/ref_inner_product.cpp:145-217):
+ *   diff_weights[oc, ic, ...] = sum over mb, ascending, of diff_dst[mb, oc] * src[mb, ic, ...]
+ *   diff_bias[oc]             = sum over mb, ascending, of diff_dst[mb, oc]       (if diff_bias != NULL)
+ * in f32, stored as the outputs' types.  `dims` are src's dims. */
+int oracle_inner_product_bwd_weights(int ndims, const int64_t *dims, int64_t OC, int src_dt, const int64_t *src_stride,
+        const void *src, int dwei_dt, const int64_t *dwei_stride, void *diff_wei, int dbias_dt, void *diff_bias,
+        int dd_dt, const int64_t *dd_stride, const void *diff_dst) {
+    if (!dims || !src_stride || !dwei_stride || !dd_stride || ndims < 2 || ndims > 5) return MI355_INVALID_ARGUMENTS;
+    const int64_t MB = dims[0];
+    int64_t Kt = 1;
+    for (int i = 1; i < ndims; ++i) Kt *= dims[i];
+#pragma omp parallel for schedule(static)
+    for (int64_t oc = 0; oc < OC; ++oc) {
+        for (int64_t k = 0; k < Kt; ++k) {
+            float dw = 0.f;
+            for (int64_t mb = 0; mb < MB; ++mb) {
+                const float dd = orc_load_float(dd_dt, diff_dst, mb * dd_stride[0] + oc * dd_stride[1]);
+                const float sv = orc_load_float(src_dt, src, orc_ip_off(ndims, dims, src_stride, mb, k));
+                dw += dd * sv;
+            }
+            orc_store_float(dwei_dt, dw, diff_wei, orc_ip_off(ndims, dims, dwei_stride, oc, k));
+        }
+        if (diff_bias) {
+            float db = 0.f;
+            for (int64_t mb = 0; mb < MB; ++mb)
+                db += orc_load_float(dd_dt, diff_dst, mb * dd_stride[0] + oc * dd_stride[1]);
+            orc_store_float(dbias_dt, db, diff_bias, oc);
+        }
+    }
     return MI355_SUCCESS;
 }
 

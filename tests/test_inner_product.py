@@ -1,5 +1,5 @@
-"""Inner product (forward) on top of the matmul kernels: dst[mb, oc] = sum over
-(ic, spatial) of src * weights, the caller of the matmul path the reference
+"""Inner product, forward (the backward passes: test_inner_product_backward.py),
+on top of the matmul kernels: dst[mb, oc] = sum over (ic, spatial) of src * weights, the caller of the matmul path the reference
 lists next to it (src/common/inner_product.cpp, src/cpu/ref_inner_product.cpp,
 src/cpu/ref_inner_product_int8.cpp).
 
@@ -335,20 +335,6 @@ def test_attribute_rules(eng):
     a.set_scales_mask(dnnl.ARG_WEIGHTS, 1)
     pd = ip_pd(eng, 2, 8, (), 6, attr=a)
     assert pd.lowered_desc().wei_scale.mask == MASK_COL
-
-
-def test_backward_is_validated_and_not_offered(eng):
-    lib = dnnl.lib()
-    import ctypes as C
-    h = C.c_void_p()
-    s, w, d = md((2, 8), "f32", dnnl.tag_ab), md((6, 8), "f32", dnnl.tag_ab), md((2, 6), "f32", dnnl.tag_ab)
-    assert lib.dnnl_inner_product_backward_data_primitive_desc_create(
-        C.byref(h), eng.h, s.h, w.h, d.h, None, None) == dnnl.unimplemented
-    assert lib.dnnl_inner_product_backward_weights_primitive_desc_create(
-        C.byref(h), eng.h, s.h, w.h, None, d.h, None, None) == dnnl.unimplemented
-    bad = md((3, 6), "f32", dnnl.tag_ab)
-    assert lib.dnnl_inner_product_backward_data_primitive_desc_create(
-        C.byref(h), eng.h, s.h, w.h, bad.h, None, None) == dnnl.invalid_arguments
 
 
 # ------------------------------------------------------------------ execution on the device
