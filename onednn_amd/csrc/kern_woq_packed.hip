@@ -91,11 +91,74 @@ __device__ __forceinline__ v8bf as_bf(const v4i &x) { return __builtin_bit_cast(
 // registers filled by inline assembly, so the compiler cannot tell that they point to global memory and would
 // emit flat loads: those count on the LDS counter as well as on the vector-memory counter, and every wait for an
 // LDS access (the activations' staging) then waits for every load in flight -- the next unit's included.
+// An address is a wavefront-uniform base (scalar registers) plus a lane's 32-bit byte offset plus a constant:
+// the form a global load takes as it is (base in a scalar pair, offset in one vector register, the constant in
+// the instruction), so stepping along K costs scalar additions only.
+typedef const uint8_t __attribute__((address_space(1))) *global_bytes_t;
 typedef const v4u __attribute__((address_space(1))) *global_v4u_ptr_t;
 typedef const unsigned __attribute__((address_space(1))) *global_u32_ptr_t;
-__device__ __forceinline__ v4u gload16(const uint8_t *p) { return *(global_v4u_ptr_t)(uintptr_t)p; }
-__device__ __forceinline__ v4u gload16_nt(const uint8_t *p) { return __builtin_nontemporal_load((global_v4u_ptr_t)(uintptr_t)p); }
-__device__ __forceinline__ unsigned gload4(const uint8_t *p) { return *(global_u32_ptr_t)(uintptr_t)p; }
+__device__ __forceinline__ global_bytes_t gaddr(const uint8_t *base, unsigned voff, int imm) {
+    return (global_bytes_t)(uintptr_t)base + voff + imm;
+}
+// Marks a base as wavefront-uniform for the compiler (a no-op on a value that is in scalar registers already):
+// without it loop strength reduction folds the lane's offset into a per-lane 64-bit pointer per stream, kept in
+// vector registers across the loop.
+__device__ __forceinline__ const uint8_t *uniform_ptr(const uint8_t *p) {
+    const uintptr_t v = (uintptr_t)p;
+    const unsigned lo = __builtin_amdgcn_readfirstlane((unsigned)v);
+    const unsigned hi = __builtin_amdgcn_readfirstlane((unsigned)(v >> 32));
+    return (const uint8_t *)(((uintptr_t)hi << 32) | lo);
+}
+// A lane's offset as a value defined where it is used: its zero-extension then stays next to the load instead of
+// being hoisted out of the loop as a 64-bit pair, and the load keeps the scalar-base form.
+__device__ __forceinline__ unsigned here(unsigned voff) {
+    asm volatile("" : "+v"(voff));
+    return voff;
+}
+__device__ __forceinline__ v4u gload16(const uint8_t *base, unsigned voff, int imm = 0) {
+    return *(global_v4u_ptr_t)gaddr(base, voff, imm);
+}
+__device__ __forceinline__ v4u gload16_nt(const uint8_t *base, unsigned voff, int imm = 0) {
+    return __builtin_nontemporal_load((global_v4u_ptr_t)gaddr(base, voff, imm));
+}
+__device__ __forceinline__ unsigned gload4(const uint8_t *base, unsigned voff) {
+    return *(global_u32_ptr_t)gaddr(base, voff, 0);
+}
+
+// The main loop's loads are written as instructions of their own and waited for by hand.  The counter of
+// outstanding loads is waited for by position from the end of the queue; where one piece of code is reached with
+// and without the next unit's loads behind the current one's, the compiler has to assume "without" and would wait
+// for the next unit as well -- no overlap of one unit's loads with the other's arithmetic.  Here the wait is picked
+// by a uniform branch on what is behind.  Between the first of these loads and the last of these waits the kernel
+// must not contain other vector-memory instructions: no spilled registers in particular (the build of this file
+// shows none).
+template <int N>
+__device__ __forceinline__ void wait_vm() {
+    asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N));
+}
+__device__ __forceinline__ void aload4(unsigned &d, const uint8_t *base, unsigned voff) {
+    asm volatile("global_load_dword %0, %1, %2" : "=&v"(d) : "v"(voff), "s"(base));
+}
+template <int IMM>
+__device__ __forceinline__ void aload16(v4u &d, const uint8_t *base, unsigned voff) {
+    asm volatile("global_load_dwordx4 %0, %1, %2 offset:%3" : "=&v"(d) : "v"(voff), "s"(base), "n"(IMM));
+}
+template <int IMM>
+__device__ __forceinline__ void aload16_nt(v4u &d, const uint8_t *base, unsigned voff) {
+    asm volatile("global_load_dwordx4 %0, %1, %2 offset:%3 nt" : "=&v"(d) : "v"(voff), "s"(base), "n"(IMM));
+}
+// a value loaded above is used only after the wait that precedes this
+template <class T>
+__device__ __forceinline__ void arrived(T &x) {
+    asm volatile("" : "+v"(x));
+}
+template <int I, int N, class F>
+__device__ __forceinline__ void static_for(F &&f) {
+    if constexpr (I < N) {
+        f(std::integral_constant<int, I> {});
+        static_for<I + 1, N>(f);
+    }
+}
 
 // Quantization parameters are fetched as the aligned dword that holds the
 // element (no branch on the data type next to the load, so a fetch never waits
@@ -123,7 +186,7 @@ __device__ __forceinline__ param_lane_t param_setup(const uint8_t *p, int bits, 
 }
 
 __device__ __forceinline__ unsigned param_word(const param_lane_t &L, int g) {
-    return gload4(L.base + g * L.pitch + L.voff);
+    return gload4(uniform_ptr(L.base + g * L.pitch), here(L.voff));
 }
 
 __device__ __forceinline__ unsigned param_cut(const param_lane_t &L, unsigned word) { return (word >> L.sh) & L.mask; }
@@ -165,7 +228,6 @@ __global__ void __launch_bounds__(NWV * 64)
                  : "=&s"(raw.lo), "=&s"(raw.hi)
                  : "s"(__builtin_amdgcn_kernarg_segment_ptr()));
     const woqp_extra_t X = __builtin_bit_cast(woqp_extra_t, raw);
-    constexpr int NGS = SPG ? SS / SPG : 1; // groups per super-step
     const int t = threadIdx.x, lane = t & 63;
     const int wave = __builtin_amdgcn_readfirstlane(t >> 6);
     const int j = lane & 15, q = lane >> 4;
@@ -175,44 +237,110 @@ __global__ void __launch_bounds__(NWV * 64)
     const int kb0 = wave * X.kbw;
     const int kb1 = kb0 + X.kbw < KB ? kb0 + X.kbw : KB;
 
-    const uint8_t *wlane = X.wei + (long)chunk * K * (CHUNK / 2) + lane * 16;
+    const uint8_t *wbase = X.wei + (long)chunk * K * (CHUNK / 2); // uniform; the lane's share starts at lane * 16
+    const unsigned wlane = (unsigned)lane * 16u;
     // MFMA rows beyond M read the last valid row: an output row depends on its
     // own src row only, and those results are never stored
-    unsigned src_lane_off[MT];
-#pragma unroll
-    for (int mt = 0; mt < MT; ++mt) {
-        const int m = mt * 16 + j < M ? mt * 16 + j : M - 1;
-        src_lane_off[mt] = (unsigned)(m * X.src_ld * 2 + q * 16);
-    }
-    // the super-step's loader: lane = row + 8 * slot over eight rows and two steps
+    constexpr bool ALDS = MT == 2;
     static_assert(SS % 2 == 0, "activations are loaded for pairs of steps");
+    // ALDS: the loader's lane = row + 8 * slot over eight rows and two steps; else the lane's operand row
     const int lr = lane & 7, lc = lane >> 3;
-    unsigned src_row_off[MT][2];
-    int wr_idx[2], rd_idx[2];
+    unsigned src_off[MT][2];
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt)
 #pragma unroll
         for (int h = 0; h < 2; ++h) {
-            const int m = mt * 16 + 8 * h + lr < M ? mt * 16 + 8 * h + lr : M - 1;
-            src_row_off[mt][h] = (unsigned)(m * X.src_ld * 2 + lc * 16);
+            const int row = ALDS ? mt * 16 + 8 * h + lr : mt * 16 + j;
+            const int m = row < M ? row : M - 1;
+            src_off[mt][h] = (unsigned)(m * X.src_ld * 2 + (ALDS ? lc : q) * 16);
         }
+    // quantization parameters: lane l fetches column l of the chunk, the
+    // columns a lane accumulates (16t + j) come from lanes 16t + j at the flush
+    const long n_param = (long)chunk * CHUNK + lane;
+    const param_lane_t Lsc = param_setup(X.sc, X.sc_bits, n_param, X.sc_grouped, N);
+    const param_lane_t Lzp = param_setup(X.zp, X.zp_bits, X.zp_common ? 0 : n_param, X.zp_grouped, N);
+    auto fetch_params = [&](unsigned &word_s, unsigned &word_z, int g) __attribute__((always_inline)) {
+        word_s = param_word(Lsc, g);
+        word_z = param_word(Lzp, g);
+    };
+
+    // A unit: the steps whose loads are issued together, before the first of them is multiplied.  One tile of
+    // rows: a super-step.  Two tiles: half a super-step, and the next unit is requested before the current one is
+    // multiplied (a wavefront has two super-steps or more there, and with one in flight at a time the memory
+    // pipeline would drain while each is multiplied): the same registers hold loads in flight all the time.
+    constexpr bool PIPE = MT == 2 && (SS / 2) % 2 == 0 && (SPG == 0 || (SS / 2) % (SPG ? SPG : 1) == 0);
+    constexpr int U = PIPE ? SS / 2 : SS;                // steps per unit
+    constexpr int NGU = SPG ? (U / (SPG ? SPG : 1) > 0 ? U / (SPG ? SPG : 1) : 1) : 1; // groups per unit
+    struct unit_t {
+        unsigned raw_s[NGU], raw_z[NGU];
+        // a[p][mt][h]: ALDS: pair p of steps, rows 8h .. 8h + 7; else step 2p + h in operand order
+        v4u a[U / 2][MT][2], w[U];
+    };
+    // Issue order: the groups' parameters (few bytes, needed last -- loads return in order, so they must not queue
+    // behind the weights), the activations, the weights; the MFMAs then follow step by step as their loads arrive.
+    //
+    // Activations.  The MFMA operand of a step is 16 rows x 64 bytes; loaded
+    // that way every instruction touches 16 half lines, the other halves are
+    // fetched again for the next step, and the launch time grows by 0.35 us per
+    // row of src.  With two tiles (ALDS) a load covers two steps of eight rows
+    // instead, whole 128-byte lines (lane = row + 8 * slot), and a pair of
+    // steps is brought into operand order through 2 KB of LDS per tile and
+    // wavefront when its turn comes: slot c of row r is stored at c ^ (r & 7),
+    // so the eight lanes that write or read together fall into eight different
+    // slots.  The detour costs 0.8 us per launch and halves the growth per row:
+    // it pays above 16 rows.
+    constexpr int NLOADS = 2 * NGU + MT * U + U; // per unit, in this order: parameters, activations, weights
+    auto issue_unit = [&](unit_t &u, int kbu) __attribute__((always_inline)) {
+        // (whole groups inside the unit: the group size is SPG)
+        const int g0 = SPG ? kbu / (SPG ? SPG : 1) : kbu / X.spg;
+        static_for<0, NGU>([&](auto GI) {
+            constexpr int gi = decltype(GI)::value;
+            aload4(u.raw_s[gi], uniform_ptr(Lsc.base + (g0 + gi) * Lsc.pitch), Lsc.voff);
+            aload4(u.raw_z[gi], uniform_ptr(Lzp.base + (g0 + gi) * Lzp.pitch), Lzp.voff);
+        });
+        const uint8_t *sb = uniform_ptr(X.src + (long)kbu * (KBLK * 2));
+        static_for<0, U / 2>([&](auto P) {
+            constexpr int p = decltype(P)::value;
+            static_for<0, MT>([&](auto MT_) {
+                constexpr int mt = decltype(MT_)::value;
+                aload16<(ALDS ? 2 * p : 2 * p) * (KBLK * 2)>(u.a[p][mt][0], sb, src_off[mt][0]);
+                aload16<(ALDS ? 2 * p : 2 * p + 1) * (KBLK * 2)>(u.a[p][mt][1], sb, src_off[mt][1]);
+            });
+        });
+        // the weights are read once: non-temporal loads keep them from
+        // displacing the activations and parameters in the caches
+        const uint8_t *wb = wbase + (long)kbu * (KBLK * CHUNK / 2);
+        static_for<0, U>([&](auto I) { // (the constant of an instruction reaches 4 KB: four steps per scalar base)
+            constexpr int i = decltype(I)::value;
+            aload16_nt<(i % 4) * (KBLK * CHUNK / 2)>(u.w[i], uniform_ptr(wb + (i / 4) * (4 * KBLK * CHUNK / 2)), wlane);
+        });
+    };
+    // The wavefront's first unit is requested before anything else is set up: the stream is what the launch waits
+    // for, the rest of the prologue (staging indices, sums, constants) runs under it.
+    unit_t ua;
+    int kb = kb0;
+    bool have_a = kb + U <= kb1;
+    if (have_a) issue_unit(ua, kb);
+    __builtin_amdgcn_sched_barrier(0);
+
+    int wr_idx[2], rd_idx[2];
 #pragma unroll
     for (int h = 0; h < 2; ++h) {
         wr_idx[h] = (8 * h + lr) * 8 + (lc ^ lr);
         rd_idx[h] = j * 8 + ((4 * h + q) ^ (j & 7));
     }
     v4u *stage = (v4u *)red4 + wave * (MT * 128);
-    constexpr bool ALDS = MT == 2;
-    // quantization parameters: lane l fetches column l of the chunk, the
-    // columns a lane accumulates (16t + j) come from lanes 16t + j at the flush
-    const long n_param = (long)chunk * CHUNK + lane;
 
     v4f acc[MT][4], rsum[MT], tot[MT][4];
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt) {
-        rsum[mt] = v4f {0.f, 0.f, 0.f, 0.f};
+        // (with whole groups inside a unit every group's first step starts its sums from a zero operand)
+        if constexpr (SPG == 0) rsum[mt] = v4f {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-        for (int tt = 0; tt < 4; ++tt) acc[mt][tt] = tot[mt][tt] = v4f {0.f, 0.f, 0.f, 0.f};
+        for (int tt = 0; tt < 4; ++tt) {
+            if constexpr (SPG == 0) acc[mt][tt] = v4f {0.f, 0.f, 0.f, 0.f};
+            tot[mt][tt] = v4f {0.f, 0.f, 0.f, 0.f};
+        }
     }
     // 0x4300 | nibble = bf16(128 + nibble).  The constant is kept in a vector
     // register: a VOP3 instruction takes one scalar operand at most, so
@@ -222,6 +350,14 @@ __global__ void __launch_bounds__(NWV * 64)
     const v4i ones = {0x3F803F80, 0x3F803F80, 0x3F803F80, 0x3F803F80};
     const unsigned flip = X.signed_w ? 0x88888888u : 0u; // s4 -> offset-binary
     const float zbase = X.signed_w ? 136.f : 128.f;
+    // s4 weights go to offset-binary before they are unpacked: a uniform branch around the exclusive-ors, so the
+    // unsigned case does not pay an instruction per dword for them
+    auto flip_signed = [&](auto &ws) __attribute__((always_inline)) {
+        if (flip != 0) {
+            asm volatile("" ::: "memory");
+            for (auto &wv : ws) wv ^= flip;
+        }
+    };
 
     // `first`: the step opens a quantization group (sums start from zero)
     auto compute_step = [&](const v4u &w, const v4u (&a)[MT], bool first) __attribute__((always_inline)) {
@@ -234,7 +370,7 @@ __global__ void __launch_bounds__(NWV * 64)
         }
 #pragma unroll
         for (int tt = 0; tt < 4; ++tt) {
-            const unsigned d = w[tt] ^ flip;
+            const unsigned d = w[tt];
             v4i b;
 #pragma unroll
             for (int u = 0; u < 4; ++u) b[u] = (int)(((d >> (4 * u)) & 0x000F000Fu) | magic);
@@ -242,13 +378,6 @@ __global__ void __launch_bounds__(NWV * 64)
             for (int mt = 0; mt < MT; ++mt)
                 acc[mt][tt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf(av[mt]), as_bf(b), first ? zero : acc[mt][tt], 0, 0, 0);
         }
-    };
-
-    const param_lane_t Lsc = param_setup(X.sc, X.sc_bits, n_param, X.sc_grouped, N);
-    const param_lane_t Lzp = param_setup(X.zp, X.zp_bits, X.zp_common ? 0 : n_param, X.zp_grouped, N);
-    auto fetch_params = [&](unsigned &word_s, unsigned &word_z, int g) __attribute__((always_inline)) {
-        word_s = param_word(Lsc, g);
-        word_z = param_word(Lzp, g);
     };
 
     // tot += scale * (acc - (128 + zp) * rowsum) for one finished group (rows
@@ -275,52 +404,35 @@ __global__ void __launch_bounds__(NWV * 64)
         }
     };
 
-    // One super-step.  Issue order: the groups' parameters (few bytes, needed
-    // last -- loads return in order, so they must not queue behind the weights),
-    // the activations, the weights; then the MFMAs step by step as their loads
-    // arrive.
-    //
-    // Activations.  The MFMA operand of a step is 16 rows x 64 bytes; loaded
-    // that way every instruction touches 16 half lines, the other halves are
-    // fetched again for the next step, and the launch time grows by 0.35 us per
-    // row of src.  With two tiles (ALDS) a load covers two steps of eight rows
-    // instead, whole 128-byte lines (lane = row + 8 * slot), and a pair of
-    // steps is brought into operand order through 2 KB of LDS per tile and
-    // wavefront when its turn comes: slot c of row r is stored at c ^ (r & 7),
-    // so the eight lanes that write or read together fall into eight different
-    // slots.  The detour costs 0.8 us per launch and halves the growth per row:
-    // it pays above 16 rows.
-    auto super_step = [&](int kb) __attribute__((always_inline)) {
-        unsigned raw_s[NGS], raw_z[NGS];
-        // (whole groups inside the super-step: the group size is SPG)
-        const int g0 = SPG ? kb / (SPG ? SPG : 1) : kb / X.spg;
-#pragma unroll
-        for (int gi = 0; gi < NGS; ++gi) fetch_params(raw_s[gi], raw_z[gi], g0 + gi);
-        // a[p][mt][h]: ALDS: pair p, rows 8h .. 8h + 7; else step 2p + h in operand order
-        v4u a[SS / 2][MT][2], w[SS];
-#pragma unroll
-        for (int p = 0; p < SS / 2; ++p)
-#pragma unroll
-            for (int mt = 0; mt < MT; ++mt)
-#pragma unroll
-                for (int h = 0; h < 2; ++h)
-                    a[p][mt][h] = ALDS ? gload16(X.src + (long)(kb + 2 * p) * (KBLK * 2) + src_row_off[mt][h])
-                                       : gload16(X.src + (long)(kb + 2 * p + h) * (KBLK * 2) + src_lane_off[mt]);
-        // the weights are read once: non-temporal loads keep them from
-        // displacing the activations and parameters in the caches
-#pragma unroll
-        for (int i = 0; i < SS; ++i)
-            w[i] = gload16_nt(wlane + (long)(kb + i) * (KBLK * CHUNK / 2));
-        // every load of the super-step is in flight before its first MFMA
-        __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-        for (int p = 0; p < SS / 2; ++p) {
+    // `behind`: the next unit's loads were issued after this unit's
+    auto consume_unit = [&](unit_t &u, int kbu, bool behind) __attribute__((always_inline)) {
+        // at most n of this unit's loads still outstanding
+        auto wait_left = [&](auto N_) __attribute__((always_inline)) {
+            constexpr int n = decltype(N_)::value;
+            if (behind) wait_vm<n + NLOADS>();
+            else wait_vm<n>();
+        };
+        if (flip != 0) { // s4 weights go to offset-binary before they are unpacked
+            wait_left(std::integral_constant<int, 0> {});
+            static_for<0, U>([&](auto I) {
+                arrived(u.w[decltype(I)::value]);
+                u.w[decltype(I)::value] ^= flip;
+            });
+        }
+        static_for<0, U / 2>([&](auto P) {
+            constexpr int p = decltype(P)::value;
             v4u as[2][MT];
+            wait_left(std::integral_constant<int, NLOADS - (2 * NGU + (p + 1) * 2 * MT)> {});
+#pragma unroll
+            for (int mt = 0; mt < MT; ++mt) {
+                arrived(u.a[p][mt][0]);
+                arrived(u.a[p][mt][1]);
+            }
             if constexpr (ALDS) {
 #pragma unroll
                 for (int mt = 0; mt < MT; ++mt) {
 #pragma unroll
-                    for (int h = 0; h < 2; ++h) stage[mt * 128 + wr_idx[h]] = a[p][mt][h];
+                    for (int h = 0; h < 2; ++h) stage[mt * 128 + wr_idx[h]] = u.a[p][mt][h];
                 }
 #pragma unroll
                 for (int sx = 0; sx < 2; ++sx)
@@ -330,98 +442,60 @@ __global__ void __launch_bounds__(NWV * 64)
 #pragma unroll
                 for (int sx = 0; sx < 2; ++sx)
 #pragma unroll
-                    for (int mt = 0; mt < MT; ++mt) as[sx][mt] = a[p][mt][sx];
+                    for (int mt = 0; mt < MT; ++mt) as[sx][mt] = u.a[p][mt][sx];
             }
-#pragma unroll
-            for (int sx = 0; sx < 2; ++sx) {
-                const int i = 2 * p + sx;
-                // with whole groups inside the super-step a group's first step
+            static_for<0, 2>([&](auto SX) {
+                constexpr int sx = decltype(SX)::value;
+                constexpr int i = 2 * p + sx;
+                wait_left(std::integral_constant<int, U - 1 - i> {});
+                arrived(u.w[i]);
+                // with whole groups inside the unit a group's first step
                 // is known at compile time and starts from a zero operand
-                compute_step(w[i], as[sx], SPG != 0 && i % (SPG ? SPG : 1) == 0);
-                if constexpr (SPG != 0) {
-                    if ((i + 1) % SPG == 0) flush_group(raw_s[i / SPG], raw_z[i / SPG], false);
-                }
-            }
-        }
-        if constexpr (SPG == 0) {
-            if ((kb + SS) % X.spg == 0 || kb + SS >= kb1) flush_group(raw_s[0], raw_z[0], true);
-        }
-    };
-
-    // Two tiles of rows: a wavefront has two super-steps or more, and with one in flight at a time the memory
-    // pipeline drains while each is multiplied.  Units of half a super-step instead, the next one requested
-    // before the current one is multiplied: the same registers hold loads in flight all the time.
-    constexpr int U = SS / 2;                           // steps per unit
-    constexpr bool PIPE = MT == 2 && U % 2 == 0 && (SPG == 0 || U % (SPG ? SPG : 1) == 0);
-    constexpr int NGU = SPG ? (U / (SPG ? SPG : 1) > 0 ? U / (SPG ? SPG : 1) : 1) : 1;
-    struct unit_t {
-        v4u a[U / 2 > 0 ? U / 2 : 1][MT][2], w[U > 0 ? U : 1];
-        unsigned raw_s[NGU], raw_z[NGU];
-    };
-    auto issue_unit = [&](unit_t &u, int kbu) __attribute__((always_inline)) {
-        const int g0 = SPG ? kbu / (SPG ? SPG : 1) : kbu / X.spg;
-#pragma unroll
-        for (int gi = 0; gi < NGU; ++gi) fetch_params(u.raw_s[gi], u.raw_z[gi], g0 + gi);
-#pragma unroll
-        for (int p = 0; p < U / 2; ++p)
-#pragma unroll
-            for (int mt = 0; mt < MT; ++mt)
-#pragma unroll
-                for (int h = 0; h < 2; ++h)
-                    u.a[p][mt][h] = gload16(X.src + (long)(kbu + 2 * p) * (KBLK * 2) + src_row_off[mt][h]);
-#pragma unroll
-        for (int i = 0; i < U; ++i)
-            u.w[i] = gload16_nt(wlane + (long)(kbu + i) * (KBLK * CHUNK / 2));
-    };
-    auto consume_unit = [&](unit_t &u, int kbu) __attribute__((always_inline)) {
-#pragma unroll
-        for (int p = 0; p < U / 2; ++p) {
-            v4u as[2][MT];
-#pragma unroll
-            for (int mt = 0; mt < MT; ++mt) {
-#pragma unroll
-                for (int h = 0; h < 2; ++h) stage[mt * 128 + wr_idx[h]] = u.a[p][mt][h];
-            }
-#pragma unroll
-            for (int sx = 0; sx < 2; ++sx)
-#pragma unroll
-                for (int mt = 0; mt < MT; ++mt) as[sx][mt] = stage[mt * 128 + rd_idx[sx]];
-#pragma unroll
-            for (int sx = 0; sx < 2; ++sx) {
-                const int i = 2 * p + sx;
                 compute_step(u.w[i], as[sx], SPG != 0 && i % (SPG ? SPG : 1) == 0);
                 if constexpr (SPG != 0) {
-                    if ((i + 1) % SPG == 0) flush_group(u.raw_s[i / SPG], u.raw_z[i / SPG], false);
+                    if constexpr ((i + 1) % (SPG ? SPG : 1) == 0) { // (the parameters came before the weights)
+                        arrived(u.raw_s[i / SPG]);
+                        arrived(u.raw_z[i / SPG]);
+                        flush_group(u.raw_s[i / SPG], u.raw_z[i / SPG], false);
+                    }
                 }
-            }
-        }
+            });
+        });
         if constexpr (SPG == 0) {
+            arrived(u.raw_s[0]);
+            arrived(u.raw_z[0]);
             if ((kbu + U) % X.spg == 0 || kbu + U >= kb1) flush_group(u.raw_s[0], u.raw_z[0], true);
         }
     };
 
-    int kb = kb0;
     if constexpr (PIPE) {
-        if (kb + U <= kb1) {
-            unit_t ua, ub;
-            issue_unit(ua, kb);
+        if (have_a) {
+            unit_t ub;
             while (true) {
                 const bool more_b = kb + 2 * U <= kb1;
                 if (more_b) issue_unit(ub, kb + U);
-                __builtin_amdgcn_sched_barrier(0);
-                consume_unit(ua, kb);
+                consume_unit(ua, kb, more_b);
                 kb += U;
                 if (!more_b) break;
                 const bool more_a = kb + 2 * U <= kb1;
                 if (more_a) issue_unit(ua, kb + U);
-                __builtin_amdgcn_sched_barrier(0);
-                consume_unit(ub, kb);
+                consume_unit(ub, kb, more_a);
                 kb += U;
                 if (!more_a) break;
             }
         }
     } else {
-        for (; kb + SS <= kb1; kb += SS) super_step(kb);
+        // (the first unit apart from the loop: as one loop with the issue at its end the 16-wavefront variants
+        // run out of their 128 registers)
+        if (have_a) {
+            consume_unit(ua, kb, false);
+            kb += U;
+        }
+        for (; kb + U <= kb1; kb += U) {
+            unit_t un;
+            issue_unit(un, kb);
+            consume_unit(un, kb, false);
+        }
     }
     if (kb < kb1) {
         // ragged end of K: one step at a time, parameters fetched when the
@@ -434,18 +508,17 @@ __global__ void __launch_bounds__(NWV * 64)
                 for (int tt = 0; tt < 4; ++tt) acc[mt][tt] = v4f {0.f, 0.f, 0.f, 0.f};
             }
         }
-        // (the lane's weights address is rebuilt here: kept from the prologue it
-        // is spilled to scratch memory across the main loop)
-        int lane_again = lane;
-        asm volatile("" : "+v"(lane_again));
-        const uint8_t *wlane_tail = X.wei + (long)chunk * K * (CHUNK / 2) + lane_again * 16;
 #pragma unroll 1
         for (; kb < kb1; ++kb) {
             v4u a1[MT];
 #pragma unroll
-            for (int mt = 0; mt < MT; ++mt) a1[mt] = gload16(X.src + (long)kb * (KBLK * 2) + src_lane_off[mt]);
-            const v4u w1 = gload16_nt(wlane_tail + (long)kb * (KBLK * CHUNK / 2));
-            compute_step(w1, a1, false);
+            for (int mt = 0; mt < MT; ++mt) {
+                const int m = mt * 16 + j < M ? mt * 16 + j : M - 1;
+                a1[mt] = gload16(X.src + (long)kb * (KBLK * 2), (unsigned)(m * X.src_ld * 2 + q * 16));
+            }
+            v4u w1[1] = {gload16_nt(wbase + (long)kb * (KBLK * CHUNK / 2), wlane)};
+            flip_signed(w1);
+            compute_step(w1[0], a1, false);
             if ((kb + 1) % X.spg == 0 || kb + 1 == kb1) {
                 unsigned word_s, word_z;
                 fetch_params(word_s, word_z, kb / X.spg);
@@ -567,7 +640,9 @@ woqp_geo_t pick_geo(int mt, long G, long K) {
     if (G % KBLK != 0) return {0, 0};
     const long spg = G / KBLK;
     if (spg <= ss_max && (spg & (spg - 1)) == 0) {
-        const int ss = (int)(4 * spg < ss_max ? 4 * spg : ss_max);
+        // (two tiles of rows and groups of 64: units of two steps -- with four, and two groups' parameters per
+        // unit, the kernel does not fit the registers of two wavefronts per SIMD)
+        const int ss = mt == 2 && spg == 2 ? 4 : (int)(4 * spg < ss_max ? 4 * spg : ss_max);
         // a group that fills the super-step is the spanning case
         return {ss, spg == ss ? 0 : (int)spg};
     }
@@ -650,7 +725,7 @@ int woqp_launch(const mi355_matmul_desc_t &d, const problem_t &P, hipStream_t st
     MI355_WOQP_CASE(8, 1, 4, 1)
     MI355_WOQP_CASE(8, 1, 8, 2)
     MI355_WOQP_CASE(8, 2, 4, 1)
-    MI355_WOQP_CASE(8, 2, 8, 2)
+    MI355_WOQP_CASE(8, 2, 4, 2)
     MI355_WOQP_CASE(8, 2, 8, 4)
     MI355_WOQP_CASE(8, 2, 8, 0)
 #undef MI355_WOQP_CASE
