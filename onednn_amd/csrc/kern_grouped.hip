@@ -145,7 +145,7 @@ __global__ void __launch_bounds__(256) grouped_2dx2d_kernel(const grouped_dev_t 
 }
 
 // ---- "hip:mfma_grouped" -- the 2Dx3D pattern on the matrix cores for fp8,
-// bf16 and f16 operands with K-contiguous weights ([G][N][K], tag acb), no
+// bf16, f16 and s8 operands with K-contiguous weights ([G][N][K], tag acb), no
 // groups along K in the scales, no zero points.
 //
 // Mixture-of-experts groups are short (tens of rows against weights of K x N
@@ -181,7 +181,10 @@ typedef float g4f __attribute__((ext_vector_type(4)));
 typedef __bf16 g8bf __attribute__((ext_vector_type(8)));
 typedef _Float16 g8h __attribute__((ext_vector_type(8)));
 
-enum { GM_F8 = 0, GM_BF16 = 1, GM_F16 = 2, GM_MXF8 = 3, GM_MXF4 = 4 };
+enum { GM_F8 = 0, GM_BF16 = 1, GM_F16 = 2, GM_MXF8 = 3, GM_MXF4 = 4, GM_I8 = 5 };
+// GM_I8: s8 x s8, the sums are s32 (kept in the accumulator registers' bits and added as integers wherever
+// partial sums meet); they turn into f32 once, after the last addition -- ref_grouped_t's `acc = f32(s32 sum)`
+// (src/cpu/matmul/ref_grouped_gemm.cpp:258-330), so the tiles agree with it bit for bit on any data.
 
 // GM_MXF8 / GM_MXF4: e8m0 scales per 32 consecutive k on both operands, applied by the instruction
 // (v_mfma_scale_f32_16x16x128_f8f6f4).  Lane (j, q) supplies the scale of block q of row j.  Its data
@@ -212,6 +215,13 @@ __device__ __forceinline__ g4f grouped_mma(const g8i &w, const g8i &a, g4f c, co
         return __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(w, a, c, FB, FA, 0, 0, 0, 0);
     } else if constexpr (MODE == GM_MXF8) {
         return __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(w, a, c, FB, FA, 0, sw[0], 0, sa[0]);
+    } else if constexpr (MODE == GM_I8) {
+        const g4i wl = {w[0], w[1], w[2], w[3]}, wh = {w[4], w[5], w[6], w[7]};
+        const g4i al = {a[0], a[1], a[2], a[3]}, ah = {a[4], a[5], a[6], a[7]};
+        g4i ci = __builtin_bit_cast(g4i, c);
+        ci = __builtin_amdgcn_mfma_i32_16x16x64_i8(wl, al, ci, 0, 0, 0);
+        ci = __builtin_amdgcn_mfma_i32_16x16x64_i8(wh, ah, ci, 0, 0, 0);
+        return __builtin_bit_cast(g4f, ci);
     } else if constexpr (MODE == GM_MXF4) {
         const g8i wl = {w[0], w[1], w[2], w[3], 0, 0, 0, 0}, wh = {w[4], w[5], w[6], w[7], 0, 0, 0, 0};
         const g8i al = {a[0], a[1], a[2], a[3], 0, 0, 0, 0}, ah = {a[4], a[5], a[6], a[7], 0, 0, 0, 0};
@@ -586,8 +596,15 @@ __global__ void __launch_bounds__(64 * NW, OCC) grouped_tile_kernel(const groupe
     for (int u = wave; u < mf * NT; u += NW) {
         const int i = u / NT, jn = u % NT;
         g4f sum = part[u * 64 + lane];
+        if constexpr (MODE == GM_I8) {
+            g4i isum = __builtin_bit_cast(g4i, sum);
 #pragma unroll
-        for (int w = 1; w < NW; ++w) sum += part[(w * mf * NT + u) * 64 + lane];
+            for (int w = 1; w < NW; ++w) isum += __builtin_bit_cast(g4i, part[(w * mf * NT + u) * 64 + lane]);
+            sum = g4f {(float)isum[0], (float)isum[1], (float)isum[2], (float)isum[3]};
+        } else {
+#pragma unroll
+            for (int w = 1; w < NW; ++w) sum += part[(w * mf * NT + u) * 64 + lane];
+        }
         grouped_store_quad(P, T, sum, T.m_base + 16 * i + j, T.n0 + 16 * jn + 4 * q);
     }
 }
@@ -866,7 +883,11 @@ __global__ void __launch_bounds__(256, 2) grouped_nsplit_kernel(const grouped_de
 #pragma nounroll
     for (int u = 0; u < mf * NT; ++u) {
         const int i = u / NT, jn = u % NT;
-        const g4f sum = *(lds_g4f_ptr_t)(size_t)(lds0 + (unsigned)((wave * mf * NT + u) * 64 + lane) * 16);
+        g4f sum = *(lds_g4f_ptr_t)(size_t)(lds0 + (unsigned)((wave * mf * NT + u) * 64 + lane) * 16);
+        if constexpr (MODE == GM_I8) {
+            const g4i isum = __builtin_bit_cast(g4i, sum);
+            sum = g4f {(float)isum[0], (float)isum[1], (float)isum[2], (float)isum[3]};
+        }
         grouped_store_quad(P, T, sum, T.m_base + 16 * i + j, T.n0 + 16 * NT * wave + 16 * jn + 4 * q);
     }
 }
@@ -898,7 +919,8 @@ int tile_plan(const mi355_grouped_desc_t &d, bool *mx_out = nullptr) {
     const bool f8 = f8_dt(d.src_dt) && f8_dt(d.wei_dt);
     const bool f4 = d.src_dt == MI355_DT_F4_E2M1 && d.wei_dt == MI355_DT_F4_E2M1;
     const bool h16 = d.src_dt == d.wei_dt && (d.src_dt == MI355_DT_BF16 || d.src_dt == MI355_DT_F16);
-    if (!f8 && !h16 && !f4) return 0;
+    const bool i8 = d.src_dt == MI355_DT_S8 && d.wei_dt == MI355_DT_S8; // (u8 src would need the weights' column sums)
+    if (!f8 && !h16 && !f4 && !i8) return 0;
     const long ebits = f4 ? 4 : (f8 ? 8 : 16);
     auto bytes = [&](long elems) { return elems * ebits / 8; };
     if (d.wei_stride[1] != 1 || d.wei_stride[2] < d.K) return 0; // K-contiguous weights only
@@ -1046,6 +1068,7 @@ extern "C" int mi355_grouped_matmul_launch(const mi355_grouped_desc_t *d, const 
         if (d->src_dt == MI355_DT_BF16) return launch_tiles<GM_BF16, 0, 0>(plan, P, s);
         if (d->src_dt == MI355_DT_F16) return launch_tiles<GM_F16, 0, 0>(plan, P, s);
         if (d->src_dt == MI355_DT_F4_E2M1) return launch_tiles<GM_MXF4, 0, 0>(plan, P, s);
+        if (d->src_dt == MI355_DT_S8) return launch_tiles<GM_I8, 0, 0>(plan, P, s);
         if (mx) {
             if (!fa && !fb) return launch_tiles<GM_MXF8, 0, 0>(plan, P, s);
             if (fa && fb) return launch_tiles<GM_MXF8, 1, 1>(plan, P, s);

@@ -1631,7 +1631,8 @@ dnnl_status_t grouped_pd_init(dnnl_primitive_desc &pd, const dnnl_memory_desc &s
     // The caller reads the layout back with dnnl_primitive_desc_query_md and reorders once.
     dnnl_memory_desc wei = wei_in;
     if (wei.kind == dnnl_format_kind_any && wei.ndims == 3 && !wei.grouped) {
-        const bool tiles = wei.dt == src.dt && (is_fp8(wei.dt) || wei.dt == dnnl_bf16 || wei.dt == dnnl_f16);
+        const bool tiles = wei.dt == src.dt
+                && (is_fp8(wei.dt) || wei.dt == dnnl_bf16 || wei.dt == dnnl_f16 || wei.dt == dnnl_s8 || wei.dt == dnnl_f4_e2m1);
         const bool both_fp8 = is_fp8(wei.dt) && is_fp8(src.dt);
         if (tiles || both_fp8) {
             const int acb[3] = {0, 2, 1};

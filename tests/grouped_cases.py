@@ -30,21 +30,26 @@ SHAPES_2DX2D = [
 NP_DT = {"f32": np.float32, "bf16": np.float32, "f16": np.float32}
 
 
-def _vals(rng, dt, shape):
+def _vals(rng, dt, shape, full_range=False):
     lo, hi = {cabi.DT_U8: (0, 15), cabi.DT_S8: (-8, 7), cabi.DT_U4: (0, 15), cabi.DT_S4: (-8, 7)}.get(dt, (-4, 4))
+    if full_range:
+        lo, hi = {cabi.DT_U8: (0, 255), cabi.DT_S8: (-128, 127)}[dt]
     return rng.integers(lo, hi + 1, size=shape).astype(np.float64)
 
 
 def case_2dx3d(sizes, K, N, src_dt=cabi.DT_F32, wei_dt=cabi.DT_F32, dst_dt=cabi.DT_F32, wtag="abc", bias=False,
-               src_scale=None, wei_scale=None, src_zp=None, wei_zp=None, post_ops=(), seed=5, mx=False):
+               src_scale=None, wei_scale=None, src_zp=None, wei_zp=None, post_ops=(), seed=5, mx=False,
+               full_range=False):
     """src_scale / src_zp: None, "row" or a K group size; wei_scale / wei_zp: None, "col" or a K group size.
     post_ops: names out of relu, linear, mul_group, mul_row, mul_full, mul_grouped.
     mx: e8m0 scales per 32 k on both operands (--attr-scales=src:3:e8m0:1x32+wei:7:e8m0:32x1).
+    full_range: 8-bit integer operands over their whole range (the expected float64 values are then exact, the
+    float32 results of kernel and oracle rounded: compare those two with each other).
     Returns (problem, expected float64 [total_M][N])."""
     rng = np.random.default_rng(seed)
     G, total = len(sizes), int(sum(sizes))
-    S = _vals(rng, src_dt, (total, K))
-    W = _vals(rng, wei_dt, (G, K, N))
+    S = _vals(rng, src_dt, (total, K), full_range)
+    W = _vals(rng, wei_dt, (G, K, N), full_range)
     quant = {}
     int_src = src_dt in (cabi.DT_S8, cabi.DT_U8)
     int_wei = wei_dt in (cabi.DT_S8, cabi.DT_U8, cabi.DT_S4, cabi.DT_U4)

@@ -1,4 +1,4 @@
-"""Grouped matmul on the matrix cores ("hip:mfma_grouped"): fp8 / bf16 / f16
+"""Grouped matmul on the matrix cores ("hip:mfma_grouped"): fp8 / bf16 / f16 / s8
 operands with K-contiguous weights.
 
   * data every type holds exactly, where any summation order gives the same
@@ -31,7 +31,7 @@ from onednn_amd.grouped import GroupedProblem, GroupedQuant
 from tests import grouped_cases as gc
 from tests.helpers import U, gemm_bound
 
-F32, BF16, F16 = cabi.DT_F32, cabi.DT_BF16, cabi.DT_F16
+F32, BF16, F16, S8, U8 = cabi.DT_F32, cabi.DT_BF16, cabi.DT_F16, cabi.DT_S8, cabi.DT_U8
 E4M3, E5M2 = cabi.DT_F8_E4M3, cabi.DT_F8_E5M2
 
 SHAPES = [
@@ -46,7 +46,7 @@ SHAPES = [
     ([8], 384, 12),
 ]
 TYPES = [("e4m3", E4M3, E4M3), ("e5m2", E5M2, E5M2), ("e4m3 x e5m2", E4M3, E5M2), ("e5m2 x e4m3", E5M2, E4M3),
-         ("bf16", BF16, BF16), ("f16", F16, F16)]
+         ("bf16", BF16, BF16), ("f16", F16, F16), ("s8", S8, S8)]
 EXTRAS = [
     ("plain", {}),
     ("row and column scales + bias", dict(src_scale="row", wei_scale="col", bias=True)),
@@ -85,6 +85,15 @@ def test_dispatch_rules():
     p, _ = gc.case_2dx3d([4, 4], 64, 32, wtag="acb")                                 # f32
     assert impl_of(p) == "hip:ref_grouped:any"
     p, _ = gc.case_2dx3d([4, 4], 64, 32, src_dt=F16, wei_dt=cabi.DT_U4, wei_scale=16, wei_zp=16)
+    assert impl_of(p) == "hip:ref_grouped:any"
+    # s8 x s8 with scales per row / per group and column; u8 src and zero points stay with the generic kernel
+    p, _ = gc.case_2dx3d([4, 4], 64, 32, src_dt=S8, wei_dt=S8, wtag="acb", src_scale="row", wei_scale="col")
+    assert impl_of(p) == "hip:mfma_grouped"
+    p, _ = gc.case_2dx3d([4, 4], 64, 32, src_dt=U8, wei_dt=S8, wtag="acb")
+    assert impl_of(p) == "hip:ref_grouped:any"
+    p, _ = gc.case_2dx3d([4, 4], 64, 32, src_dt=S8, wei_dt=S8, wtag="acb", src_zp="row")
+    assert impl_of(p) == "hip:ref_grouped:any"
+    p, _ = gc.case_2dx3d([4, 4], 64, 32, src_dt=S8, wei_dt=S8, wtag="acb", wei_scale=32)
     assert impl_of(p) == "hip:ref_grouped:any"
     with cabi.tuning("MI355_GROUPED_IMPL", "ref"):
         p, _ = gc.case_2dx3d([4, 4], 64, 32, src_dt=E4M3, wei_dt=E4M3, wtag="acb")
@@ -131,6 +140,27 @@ def test_a_k_group_of_all_of_k_is_a_row_or_column_scale(gpu, oracle, tile_shape,
     got = grouped.run_gpu(p)
     assert np.array_equal(got, ref), f"{p.name} {tname} {ss} {ws} ({tile_shape})"
     assert np.array_equal(gc.logical_dst(p, got), want)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("shape", [([8, 8, 8, 8], 64, 32), ([10, 20, 30, 40], 160, 36), ([70, 3, 129], 4096, 40),
+                                   ([1, 2, 4, 8, 16], 2880, 130), ([3] * 40, 7168, 256)],
+                         ids=lambda s: f"G{len(s[0])}x{sum(s[0])}x{s[1]}x{s[2]}")
+def test_int8_over_the_whole_range_matches_the_oracle(gpu, oracle, tile_shape, shape):
+    """s32 sums (beyond 2^24 at the larger K: the one conversion to f32 rounds), then the same f32 operations in the
+    same order as the reference's loop: bit for bit on any data."""
+    from onednn_amd import grouped
+    sizes, K, N = shape
+    for label, kw in EXTRAS:
+        for dst_dt in (F32, BF16):
+            p, want = gc.case_2dx3d(sizes, K, N, src_dt=S8, wei_dt=S8, dst_dt=dst_dt, wtag="acb", full_range=True, **kw)
+            assert impl_of(p) == "hip:mfma_grouped"
+            st, ref = oracle.run_oracle_grouped(p)
+            assert st == cabi.SUCCESS
+            got = grouped.run_gpu(p)
+            assert np.array_equal(got, ref), f"{p.name} {label} dst {dst_dt} ({tile_shape})"
+            if dst_dt == F32 and label == "plain":
+                assert np.array_equal(gc.logical_dst(p, got), want.astype(np.float32))
 
 
 MX_SHAPES = [
