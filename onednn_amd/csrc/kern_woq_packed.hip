@@ -47,6 +47,14 @@
 
 #include <type_traits>
 
+// Measurement builds (wrong results, timing only; `make EXTRA=-DMI355_WOQP_ABL=n OBJDIR=... OUT=...`): what a launch
+// costs with one part of the kernel taken out.  1: every unit reads the activations of the wavefront's first unit
+// (no activation traffic beyond the caches); 2: every unit reads the weights of the first unit (a quarter of the
+// weights' bytes); 3: no flush of the groups; 4: no LDS staging of the activations; 5: no unpacking; 6: loads,
+// waits, the sum over the wavefronts and the store only.
+#ifndef MI355_WOQP_ABL
+#define MI355_WOQP_ABL 0
+#endif
 namespace mi355 {
 namespace {
 
@@ -298,7 +306,11 @@ __global__ void __launch_bounds__(NWV * 64)
             aload4(u.raw_s[gi], uniform_ptr(Lsc.base + (g0 + gi) * Lsc.pitch), Lsc.voff);
             aload4(u.raw_z[gi], uniform_ptr(Lzp.base + (g0 + gi) * Lzp.pitch), Lzp.voff);
         });
+#if MI355_WOQP_ABL == 1
+        const uint8_t *sb = uniform_ptr(X.src + (long)kb0 * (KBLK * 2));
+#else
         const uint8_t *sb = uniform_ptr(X.src + (long)kbu * (KBLK * 2));
+#endif
         static_for<0, U / 2>([&](auto P) {
             constexpr int p = decltype(P)::value;
             static_for<0, MT>([&](auto MT_) {
@@ -309,7 +321,11 @@ __global__ void __launch_bounds__(NWV * 64)
         });
         // the weights are read once: non-temporal loads keep them from
         // displacing the activations and parameters in the caches
+#if MI355_WOQP_ABL == 2
+        const uint8_t *wb = wbase + (long)kb0 * (KBLK * CHUNK / 2);
+#else
         const uint8_t *wb = wbase + (long)kbu * (KBLK * CHUNK / 2);
+#endif
         static_for<0, U>([&](auto I) { // (the constant of an instruction reaches 4 KB: four steps per scalar base)
             constexpr int i = decltype(I)::value;
             aload16_nt<(i % 4) * (KBLK * CHUNK / 2)>(u.w[i], uniform_ptr(wb + (i / 4) * (4 * KBLK * CHUNK / 2)), wlane);
@@ -361,6 +377,11 @@ __global__ void __launch_bounds__(NWV * 64)
 
     // `first`: the step opens a quantization group (sums start from zero)
     auto compute_step = [&](const v4u &w, const v4u (&a)[MT], bool first) __attribute__((always_inline)) {
+#if MI355_WOQP_ABL == 6
+        // (timing build: the loads and waits only)
+        tot[0][0][0] += u2f(w[0] ^ w[1] ^ w[2] ^ w[3] ^ a[0][0] ^ a[MT - 1][3]);
+        return;
+#endif
         v4i av[MT];
         const v4f zero = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
@@ -373,7 +394,8 @@ __global__ void __launch_bounds__(NWV * 64)
             const unsigned d = w[tt];
             v4i b;
 #pragma unroll
-            for (int u = 0; u < 4; ++u) b[u] = (int)(((d >> (4 * u)) & 0x000F000Fu) | magic);
+            for (int u = 0; u < 4; ++u)
+                b[u] = MI355_WOQP_ABL == 5 ? (int)(d + u) : (int)(((d >> (4 * u)) & 0x000F000Fu) | magic);
 #pragma unroll
             for (int mt = 0; mt < MT; ++mt)
                 acc[mt][tt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf(av[mt]), as_bf(b), first ? zero : acc[mt][tt], 0, 0, 0);
@@ -384,6 +406,9 @@ __global__ void __launch_bounds__(NWV * 64)
     // beyond M hold the sums of row M - 1: finite, never stored).  ZERO: the
     // next step does not start the sums from zero by itself.
     auto flush_group = [&](unsigned word_s, unsigned word_z, bool zero_sums) __attribute__((always_inline)) {
+#if MI355_WOQP_ABL == 3 || MI355_WOQP_ABL == 6
+        if (word_s != 0x12345678u) return; // (timing build: practically never flushes)
+#endif
         const float s = decode_scale(X.sc_dt, param_cut(Lsc, word_s));
         const float z = decode_zp(X.zp_dt, X.zp_bits, param_cut(Lzp, word_z)) + zbase;
 #pragma unroll
@@ -428,7 +453,7 @@ __global__ void __launch_bounds__(NWV * 64)
                 arrived(u.a[p][mt][0]);
                 arrived(u.a[p][mt][1]);
             }
-            if constexpr (ALDS) {
+            if constexpr (ALDS && MI355_WOQP_ABL != 4 && MI355_WOQP_ABL != 6) {
 #pragma unroll
                 for (int mt = 0; mt < MT; ++mt) {
 #pragma unroll
