@@ -12,16 +12,17 @@ namespace {
 using namespace gemm;
 constexpr int KSTEP = 1;
 using f8_geo_t = geo_t<8, 256>;
-using mxf8_geo_t = geo_t<4, 256>; // the block-scaled variant: see mxf8_mma_t
 constexpr int NSTAGE = f8_geo_t::NSTAGE; // one stage (K = 64) per step
 
 struct f8_extra_t {
     const char *bt; // weights as [N][K] bytes, K contiguous
     long ldb, bt_bstride;
     int tiles_m, tiles_n;
-    // MX variant: e8m0 scales per 32 k, src [M][K/32], weights transposed to [N][K/32]
+    // MX variant: the e8m0 scales per 32 k of both operands, packed by a pre-pass of the launch into the order the
+    // wavefronts load them (mxf8_mma_t in kern_f8.hip); strides in bytes, nst = stages of K (a tail stage included)
     const char *sa, *sb;
     long sa_bstride, sb_bstride;
+    int nst;
 };
 
 struct f8_ctx_t {};
@@ -309,6 +310,20 @@ struct acc_of<Mma, std::enable_if_t<Mma::TILE16>> {
     static constexpr int N = 4;
 };
 
+// block-scaled policies (MX = true) bring a context of their own and LDS behind the tile ring
+template <class Mma, class = void>
+struct mx_of : std::false_type {
+    static constexpr int EXTRA_LDS = 0;
+    __device__ static __forceinline__ f8_ctx_t make_ctx(const f8_extra_t &, unsigned, long, long, long, int) { return {}; }
+};
+template <class Mma>
+struct mx_of<Mma, std::enable_if_t<Mma::MX>> : std::true_type {
+    static constexpr int EXTRA_LDS = Mma::EXTRA_LDS;
+    __device__ static __forceinline__ auto make_ctx(const f8_extra_t &X, unsigned lds0, long b, long m0, long n0, int wave) {
+        return Mma::make_ctx(X, lds0, b, m0, n0, wave);
+    }
+};
+
 extern __shared__ __attribute__((aligned(16))) char f8_smem[];
 
 template <class Mma>
@@ -329,11 +344,12 @@ __global__ void __launch_bounds__(Mma::G::NT) __attribute__((amdgpu_waves_per_eu
 
     const long bs = P.ss[0] ? b : 0, bw = P.ws[0] ? b : 0;
     f8_conv_t<Mma::HOT> cv;
-    cv.with_src_sc = P.src_scale.dt != MI355_DT_UNDEF;
-    cv.with_wei_sc = P.wei_scale.dt != MI355_DT_UNDEF;
+    // (block scales are operands of the instruction: nothing of them is left for the epilogue)
+    cv.with_src_sc = !mx_of<Mma>::value && P.src_scale.dt != MI355_DT_UNDEF;
+    cv.with_wei_sc = !mx_of<Mma>::value && P.wei_scale.dt != MI355_DT_UNDEF;
     cv.ssc_common = 1.f;
     cv.ssc_p = nullptr;
-    cv.ssc_dt = P.src_scale.dt;
+    cv.ssc_dt = mx_of<Mma>::value ? (int)MI355_DT_UNDEF : P.src_scale.dt;
     cv.bw = bw;
     if (cv.with_src_sc) {
         if (P.src_scale.mask & 2)
@@ -344,8 +360,10 @@ __global__ void __launch_bounds__(Mma::G::NT) __attribute__((amdgpu_waves_per_eu
     }
     // the epilogue's per-column operands go into their LDS table now: the loads
     // hide behind the pipeline prologue
-    const unsigned ntab = (unsigned)(size_t)(__attribute__((address_space(3))) char *)smem + G::NSTAGE * G::STAGE_BYTES;
+    const unsigned lds0 = (unsigned)(size_t)(__attribute__((address_space(3))) char *)smem;
+    const unsigned ntab = lds0 + G::NSTAGE * G::STAGE_BYTES + mx_of<Mma>::EXTRA_LDS;
     fill_ntab<G::NT>(P, cv, ntab, b, n0);
+    const auto ctx = mx_of<Mma>::make_ctx(X, lds0, b, m0, n0, __builtin_amdgcn_readfirstlane(wave));
 
     typename acc_of<Mma>::type acc[Mma::ROWS][Mma::COLS];
 #pragma unroll
@@ -357,13 +375,13 @@ __global__ void __launch_bounds__(Mma::G::NT) __attribute__((amdgpu_waves_per_eu
 
     const long kbytes = P.K * EB;
     main_loop<G::NSTAGE, KSTEP, Mma>(acc, smem, A, Bt, lda, X.ldb, P.M - m0,
-            P.N - n0, (int)(kbytes / (BKB * KSTEP)), f8_ctx_t {});
+            P.N - n0, (int)(kbytes / (BKB * KSTEP)), ctx);
     if constexpr (has_k_tail<Mma>::value) {
         // the rest of a K that is whole 16-byte chunks but not whole stages
         const int rem = (int)(kbytes % BKB);
         if (rem != 0)
             tail_step<Mma>(acc, smem, A + kbytes - BKB, Bt + kbytes - BKB, lda, X.ldb, P.M - m0, P.N - n0,
-                    (BKB - rem) / 16, (int)(kbytes / BKB), f8_ctx_t {});
+                    (BKB - rem) / 16, (int)(kbytes / BKB), ctx);
     }
 
     store_quadrant<typename acc_of<Mma>::layout, G::WCOLS>(P, smem, ntab, acc, b, m0 + wm * 128, n0 + wn * G::WCOLS,

@@ -28,140 +28,157 @@ namespace {
 // the instruction itself (v_mfma_scale_f32_32x32x64_f8f6f4): ref_matmul_t with
 // group_k = 32 -- acc = sum of a block's 32 products, acc *= 2^(ss-127),
 // acc *= 2^(ws-127), res += acc (src/cpu/matmul/ref_matmul.cpp:168-236).
-// A 64-byte stage is two blocks; lanes 0-31 supply the scale byte of the
-// stage's first block of their row, lanes 32-63 that of the second.  The scale
-// bytes ride along with the tile stages as in the MXFP4 family: one direct-to-LDS
-// dword per row and stage -- the dword that holds the stage's two bytes, so two
-// consecutive stages fetch the same one.  Four wavefronts of 128 x 128 (the
-// geometry of the MXFP4 family): with eight, the scale operands on top of the
-// fp8 policy's registers put spills into the K loop (6.5 GB of scratch writes
-// per 8192^3 launch, 0.4 PFLOP/s).
+//
+// A 64-byte stage is two blocks; the instruction takes block h's scale from the lanes 32 h .. 32 h + 31 (lane
+// l: row l % 32 of the fragment) and reads the first register halves of all lanes as k 0..31, the second halves
+// as k 32..63 -- so a lane holds the 16-byte chunks h and 2 + h of the stage, not 2 h and 2 h + 1 as in the
+// unscaled policy (established on the device: exact data with a scale of its own per block match the oracle bit
+// for bit this way and differ the other way).  Which byte of the scale register counts is picked by op_sel.
+//
+// The scales reach a wavefront the way the MXFP4 family's do: a pre-pass of the launch packs them, per stage and
+// block of rows, into the 64 dwords a wavefront loads for that stage -- dword l holds, for the lane's row l % 32 and
+// block l / 32, the bytes of the block's up to four fragments (rows +0, +32, +64, +96) -- so that one 4-byte LDS
+// read per operand and stage feeds all of a wavefront's MFMAs and no shift or mask touches the scales.  Blocks of
+// 128 rows of src (a wavefront's four fragments), of 64 columns of weights (its two).  The packed scales of a
+// stage -- 2 blocks of A, 4 of B^T, 256 bytes each -- ride along with the tile ring, one direct-to-LDS dword per
+// lane and stage for six of the eight wavefronts (the other two repeat two of them: every wavefront issues the
+// same number of loads per stage, which the loop's load counting relies on).  The geometry, loop and epilogue are
+// the unscaled kernel's (eight wavefronts, whole-row bf16 chains); a K that ends inside a stage takes the family's
+// tail step, the pre-pass giving that stage the scales of its window (K - 64 ..) with the neutral byte for the
+// block that was multiplied before.
 struct mxf8_ctx_t {
-    const char *sa_tile, *sb_tile; // first scale byte of tile row 0 of each operand
-    unsigned voff_a, voff_b;       // this lane's row offset in the scale arrays
-    unsigned lds_scale0;           // LDS byte address of the scale ring
-    unsigned lds0;                 // LDS byte address of the tile ring
+    const char *s_blk;     // packed scales of the block this wavefront brings in, stage 0
+    unsigned lds_scale0;   // LDS byte address of the scale ring
+    unsigned lds0;         // LDS byte address of the tile ring
 };
 
-// SPLIT: which 16-byte chunks of a stage a lane's register halves hold.  The
-// instruction reads the first halves of all lanes as k 0..31 and the second
-// halves as k 32..63 (lane group h: bytes 16h..16h+15 of each), while it takes
-// block h's scale from lane group h -- so for scaled operands a lane holds
-// chunks h and 2 + h (SPLIT), not the contiguous 2h, 2h + 1 that serve when
-// no scale distinguishes the blocks (established on the device: exact data
-// with a scale of its own per block match the oracle bit for bit this way and
-// differ the other way).
-template <int FMT_A, int FMT_B, bool SPLIT, class G_>
+template <int FMT_A, int FMT_B, class G_>
 struct mxf8_mma_t {
     using G = G_;
     static constexpr int ELEM_BYTES = 1;
-    static constexpr bool HOT = false;
-    static constexpr int EXTRA_DMAS = 2;
-    static constexpr int SCALE_STAGE = (BM + G::BN) * 4;
-    static_assert(G::NW == 4 && G::BN == 256, "wavefront w brings the scale dwords of rows 64 w .. 64 w + 63 of A and of B^T");
-    __device__ static __forceinline__ void issue_extra(const mxf8_ctx_t &c, int g, int slot, int wave, int) {
-        const unsigned dst = c.lds_scale0 + slot * SCALE_STAGE + wave * 256;
-        dma4(c.sa_tile + (long)(g >> 1) * 4, c.voff_a, dst);
-        dma4(c.sb_tile + (long)(g >> 1) * 4, c.voff_b, dst + BM * 4);
+    static constexpr bool HOT = FMT_A == 0 && FMT_B == 0;
+    static constexpr bool MX = true;
+    static constexpr int EXTRA_DMAS = 1;
+    static constexpr int SCALE_STAGE = 6 * 256; // two blocks of A, four of B^T
+    static constexpr int EXTRA_LDS = G::NSTAGE * SCALE_STAGE;
+    static_assert(G::NW == 8 && G::BN == 256 && BM == 256, "blocks of 128 rows / 64 columns per wavefront part");
+    typedef mxf8_ctx_t ctx_t;
+    // where wavefront `wave` puts its block inside a stage of the scale ring
+    __device__ static __forceinline__ unsigned blk_off(int wave) {
+        return wave >= 2 && wave < 6 ? 512u + (unsigned)(wave - 2) * 256u : (unsigned)(wave & 1) * 256u;
+    }
+    __device__ static __forceinline__ mxf8_ctx_t make_ctx(const f8_extra_t &X, unsigned lds0, long b, long m0, long n0,
+            int wave) {
+        mxf8_ctx_t c;
+        c.lds0 = lds0;
+        c.lds_scale0 = lds0 + G::NSTAGE * G::STAGE_BYTES;
+        const bool of_b = wave >= 2 && wave < 6;
+        const char *p = of_b ? X.sb + b * X.sb_bstride + ((n0 >> 6) + (wave - 2)) * (long)X.nst * 256
+                             : X.sa + b * X.sa_bstride + ((m0 >> 7) + (wave & 1)) * (long)X.nst * 256;
+        c.s_blk = scalar_ptr(p);
+        return c;
+    }
+    __device__ static __forceinline__ void issue_extra(const mxf8_ctx_t &c, int g, int slot, int wave, int lane) {
+        dma4(c.s_blk + (long)g * 256, (unsigned)lane * 4u, c.lds_scale0 + slot * SCALE_STAGE + blk_off(wave));
     }
     static constexpr int ROWS = 4, COLS = G::WCOLS / 32, A_READS = 3, B_READS = 3;
+    static_assert(COLS == 2, "a wavefront's part is 128 x 64");
     struct frag_t {
         v8i a[ROWS], b[COLS];
-        int sa[ROWS], sb[COLS];
+        int sa, sb; // byte i: the scale of fragment i
     };
     __device__ static __forceinline__ frag_t zero_frag() { return frag_t {}; }
     struct addr_t {
-        unsigned a0, a1, b0, b1, sa, sb, shift;
+        unsigned a0, a1, b0, b1, sa, sb;
     };
     __device__ static __forceinline__ addr_t lane_addr(int wm, int wn, int lane) {
         const int frow = lane & 31, h = lane >> 5;
-        const int c0 = SPLIT ? h : 2 * h, c1 = SPLIT ? 2 + h : 2 * h + 1;
         const int ra = wm * 128 + frow, rb = wn * G::WCOLS + frow;
-        return addr_t {(unsigned)swz(ra, c0), (unsigned)swz(ra, c1), (unsigned)(B_OFF + swz(rb, c0)),
-                (unsigned)(B_OFF + swz(rb, c1)), (unsigned)(ra * 4), (unsigned)((BM + rb) * 4), (unsigned)(h * 8)};
+        return addr_t {(unsigned)swz(ra, h), (unsigned)swz(ra, 2 + h), (unsigned)(B_OFF + swz(rb, h)),
+                (unsigned)(B_OFF + swz(rb, 2 + h)), (unsigned)(wm * 256 + lane * 4), (unsigned)(512 + wn * 256 + lane * 4)};
     }
     __device__ static __forceinline__ unsigned scales(const unsigned (&S)[1], const mxf8_ctx_t &c) {
         const unsigned slot = (S[0] - c.lds0) / G::STAGE_BYTES;
         return c.lds_scale0 + slot * SCALE_STAGE;
     }
     __device__ static __forceinline__ void load_b(frag_t &f, const unsigned (&S)[1], const addr_t &ad,
-            const mxf8_ctx_t &c, int g) {
-        const unsigned sc = scales(S, c), sh = ad.shift + 16 * (g & 1);
+            const mxf8_ctx_t &c, int) {
 #pragma unroll
-        for (int j = 0; j < COLS; ++j) {
+        for (int j = 0; j < COLS; ++j)
             f.b[j] = f8_mma_t<0, 0, G_>::read32(S[0] + ad.b0 + j * 2048, S[0] + ad.b1 + j * 2048);
-            f.sb[j] = (int)((lds_read4(sc + ad.sb + j * 128) >> sh) & 0xffu);
-        }
+        f.sb = (int)lds_read4(scales(S, c) + ad.sb);
     }
     __device__ static __forceinline__ void load_a(frag_t &f, int i, const unsigned (&S)[1], const addr_t &ad,
-            const mxf8_ctx_t &c, int g) {
-        const unsigned sc = scales(S, c), sh = ad.shift + 16 * (g & 1);
+            const mxf8_ctx_t &c, int) {
         f.a[i] = f8_mma_t<0, 0, G_>::read32(S[0] + ad.a0 + i * 2048, S[0] + ad.a1 + i * 2048);
-        f.sa[i] = (int)((lds_read4(sc + ad.sa + i * 128) >> sh) & 0xffu);
+        if (i == 0) f.sa = (int)lds_read4(scales(S, c) + ad.sa);
+    }
+    template <int I, int J>
+    __device__ static __forceinline__ void mma_one(v16f (&acc)[ROWS][COLS], const frag_t &f) {
+        // operands exchanged as in the unscaled policy: weights first
+        acc[I][J] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(f.b[J], f.a[I], acc[I][J], FMT_B, FMT_A, J, f.sb, I, f.sa);
     }
     __device__ static __forceinline__ void mma_row(v16f (&acc)[ROWS][COLS], const frag_t &f, int i,
             const mxf8_ctx_t &, int) {
+        switch (i) {
+            case 0: mma_one<0, 0>(acc, f); mma_one<0, 1>(acc, f); break;
+            case 1: mma_one<1, 0>(acc, f); mma_one<1, 1>(acc, f); break;
+            case 2: mma_one<2, 0>(acc, f); mma_one<2, 1>(acc, f); break;
+            default: mma_one<3, 0>(acc, f); mma_one<3, 1>(acc, f); break;
+        }
+    }
+    // K that ends inside a stage (gemm_core.hpp tail_step): the lane's chunks are h and 2 + h; chunks below nz
+    // are zeroed in both operands (their block's scale in the packed tail stage is the neutral byte)
+    static constexpr bool K_TAIL = true;
+    __device__ static __forceinline__ void zero_tail(frag_t &f, int nz, int lane) {
+        const int h = lane >> 5;
+        const bool z0 = h < nz, z1 = 2 + h < nz;
+#pragma unroll
+        for (int i = 0; i < ROWS; ++i)
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                f.a[i][e] = z0 ? 0 : f.a[i][e];
+                f.a[i][4 + e] = z1 ? 0 : f.a[i][4 + e];
+            }
 #pragma unroll
         for (int j = 0; j < COLS; ++j)
-            acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(
-                    f.b[j], f.a[i], acc[i][j], FMT_B, FMT_A, 0, f.sb[j], 0, f.sa[i]);
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                f.b[j][e] = z0 ? 0 : f.b[j][e];
+                f.b[j][4 + e] = z1 ? 0 : f.b[j][4 + e];
+            }
     }
 };
 
-template <class Mma>
-__global__ void __launch_bounds__(Mma::G::NT) __attribute__((amdgpu_waves_per_eu(Mma::G::NW * Mma::G::WG_PER_CU / 4))) mxf8_gemm_kernel(const problem_t P_, const f8_extra_t X) {
-    using G = typename Mma::G;
-    const auto &P = MI355_KERNARG_PROBLEM();
-    char *smem = f8_smem;
-    const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
-    const int wm = G::wm(wave), wn = G::wn(wave);
-    const long b = blockIdx.z;
-    const tile_pos_t tp = tile_position<G>((int)blockIdx.x, X.tiles_m, X.tiles_n);
-    const long m0 = tp.m0, n0 = tp.n0;
-
-    const long lda = P.ss[1];
-    const long kb = P.K / 32; // scale bytes per row
-    const char *A = (const char *)P.src + (P.ss[0] ? b * P.ss[0] : 0) + m0 * lda;
-    const char *Bt = X.bt + b * X.bt_bstride + n0 * X.ldb;
-
-    mxf8_ctx_t ctx;
-    ctx.lds0 = (unsigned)(size_t)(__attribute__((address_space(3))) char *)smem;
-    ctx.lds_scale0 = ctx.lds0 + NSTAGE * G::STAGE_BYTES;
-    ctx.sa_tile = X.sa + b * X.sa_bstride + m0 * kb;
-    ctx.sb_tile = X.sb + b * X.sb_bstride + n0 * kb;
-    {
-        long ra = wave * 64 + lane, rb = wave * 64 + lane;
-        if (ra > P.M - m0 - 1) ra = P.M - m0 - 1;
-        if (rb > P.N - n0 - 1) rb = P.N - n0 - 1;
-        ctx.voff_a = (unsigned)(ra * kb);
-        ctx.voff_b = (unsigned)(rb * kb);
+// The pre-pass: dword (block, stage g, lane l) of the packed scales holds, in byte i < frags, the scale of row
+// 32 * frags * block + 32 i + l % 32 for the stage's block l / 32 (blocks 2 g, 2 g + 1 of the row; the tail stage
+// of a K that is an odd number of blocks covers blocks kb - 2, kb - 1 and gives the first one, multiplied before,
+// the neutral byte); rows beyond the tensor and unused bytes hold the neutral byte too.  `in`: e8m0 bytes, element
+// (row, block) at row * row_stride + block * k_stride (src scales [M][K/32], weights scales [K/32][N]).
+__global__ void __launch_bounds__(256) mxf8_pack_scales_kernel(const uint8_t *in, long rows, long kb, long row_stride,
+        long k_stride, long in_bstride, uint32_t *out, long out_bstride, int nst, int frags, long nblk) {
+    const long idx = (long)blockIdx.x * 256 + threadIdx.x;
+    if (idx >= nblk * nst * 64) return;
+    const int l = (int)(idx & 63), h = l >> 5;
+    const long g = (idx >> 6) % nst, blk = (idx >> 6) / nst;
+    const long full = kb / 2;
+    const long kblk = g < full ? 2 * g + h : (h == 0 ? -1 : kb - 1);
+    const uint8_t *src = in + (long)blockIdx.y * in_bstride;
+    uint32_t word = 0;
+    for (int i = 0; i < 4; ++i) {
+        const long row = blk * 32 * frags + 32 * i + (l & 31);
+        uint32_t byte = 127;
+        if (i < frags && row < rows && kblk >= 0) byte = src[row * row_stride + kblk * k_stride];
+        word |= byte << (8 * i);
     }
-    f8_conv_t<false> cv;
-    cv.with_src_sc = cv.with_wei_sc = false; // the scales are operands of the instruction
-    cv.ssc_common = 1.f;
-    cv.ssc_p = nullptr;
-    cv.ssc_dt = MI355_DT_UNDEF;
-    cv.bw = 0;
-    const unsigned ntab = ctx.lds_scale0 + NSTAGE * Mma::SCALE_STAGE;
-    fill_ntab<G::NT>(P, cv, ntab, b, n0);
-
-    v16f acc[Mma::ROWS][Mma::COLS];
-#pragma unroll
-    for (int i = 0; i < Mma::ROWS; ++i)
-#pragma unroll
-        for (int j = 0; j < Mma::COLS; ++j)
-#pragma unroll
-            for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
-
-    main_loop<NSTAGE, KSTEP, Mma>(acc, smem, A, Bt, lda, X.ldb, P.M - m0, P.N - n0, (int)(P.K / (BKB * KSTEP)), ctx);
-
-    store_quadrant<layout32_t, G::WCOLS>(P, smem, ntab, acc, b, m0 + wm * 128, n0 + wn * G::WCOLS, wn * G::WCOLS, cv);
+    out[(long)blockIdx.y * out_bstride + idx] = word;
 }
 
 struct f8_plan_t {
     bool need_transpose, mx;
-    size_t off_sb, total;
-    long Bw, Bsb;
+    size_t off_sa, off_sb, total;
+    long Bw, Bsa, Bsb;
+    long nst, blk_a, blk_b; // MX: stages of K, blocks of 128 src rows / 64 columns
 };
 
 // MX: e8m0 scales per 32 consecutive k on both operands
@@ -177,9 +194,17 @@ f8_plan_t make_plan(const mi355_matmul_desc_t &d) {
     p.need_transpose = !(d.wei_stride[1] == 1);
     p.mx = f8_is_mx(d);
     p.Bsb = (d.wei_scale.mask & 1) ? p.Bw : 1;
+    p.Bsa = ((d.src_scale.mask & 1) && d.src_stride[0]) ? d.batch : 1;
     size_t off = p.need_transpose ? align_up((size_t)p.Bw * d.N * d.K, 256) : 0;
-    p.off_sb = off;
-    if (p.mx) off += align_up((size_t)p.Bsb * d.N * (d.K / 32), 256); // weights scales as [N][K/32]
+    if (p.mx) { // the packed scales of both operands
+        p.nst = (d.K + BKB - 1) / BKB;
+        p.blk_a = (d.M + 127) / 128 + 1; // (a tile of 256 rows reads two blocks whatever M is)
+        p.blk_b = (d.N + 255) / 256 * 4;
+        p.off_sa = off;
+        off += align_up((size_t)p.Bsa * p.blk_a * p.nst * 256, 256);
+        p.off_sb = off;
+        off += align_up((size_t)p.Bsb * p.blk_b * p.nst * 256, 256);
+    }
     p.total = off;
     return p;
 }
@@ -200,8 +225,8 @@ int f8_supported(const mi355_matmul_desc_t &d) {
     if (!quant_absent(d.src_zp) || !quant_absent(d.wei_zp) || !quant_absent(d.src_pr))
         return MI355_UNIMPLEMENTED;
     if (f8_is_mx(d)) {
-        // a stage fetches the dword that holds its two scale bytes: rows of whole dwords, static dst quantization
-        if (d.K % 128 != 0 || d.dst_scale_dynamic != MI355_DST_DYNAMIC_NONE) return MI355_UNIMPLEMENTED;
+        // whole blocks of 32 k (a K that ends inside a 64-byte stage takes the tail step), static dst quantization
+        if (d.K % 32 != 0 || d.dst_scale_dynamic != MI355_DST_DYNAMIC_NONE) return MI355_UNIMPLEMENTED;
         if (d.batch > 65535) return MI355_UNIMPLEMENTED;
         return MI355_SUCCESS;
     }
@@ -248,28 +273,33 @@ int f8_launch(const mi355_matmul_desc_t &d, const problem_t &P, void *scratch, h
     };
     const int fa = d.src_dt == MI355_DT_F8_E5M2, fb = d.wei_dt == MI355_DT_F8_E5M2;
     if (plan.mx) {
-        if (((uintptr_t)P.src_scale.p & 3) != 0) {
-            set_error("mfma_f8: MX src scales must be 4-byte aligned");
-            return MI355_INVALID_ARGUMENTS;
-        }
         const long kb = d.K / 32;
-        char *sb = (char *)scratch + plan.off_sb;
-        transpose_bytes(P.wei_scale.p, kb, d.N, d.N, kb * d.N, sb, kb, d.N * kb, plan.Bsb, stream);
+        char *sa = (char *)scratch + plan.off_sa, *sb = (char *)scratch + plan.off_sb;
+        auto pack = [&](const void *in, long rows, long row_stride, long k_stride, long in_bstride, char *out, int frags,
+                            long nblk, long batches) {
+            const long n = nblk * plan.nst * 64;
+            hipLaunchKernelGGL(mxf8_pack_scales_kernel, dim3((unsigned)((n + 255) / 256), (unsigned)batches), dim3(256), 0,
+                    stream, (const uint8_t *)in, rows, kb, row_stride, k_stride, in_bstride, (uint32_t *)out, n,
+                    (int)plan.nst, frags, nblk);
+        };
+        pack(P.src_scale.p, d.M, kb, 1, d.M * kb, sa, 4, plan.blk_a, plan.Bsa);
+        pack(P.wei_scale.p, d.N, 1, d.N, kb * d.N, sb, 2, plan.blk_b, plan.Bsb);
+        if (hipGetLastError() != hipSuccess) return MI355_RUNTIME_ERROR;
+        X.sa = sa;
         X.sb = sb;
-        X.sb_bstride = plan.Bsb > 1 ? d.N * kb : 0;
-        X.sa = (const char *)P.src_scale.p;
-        X.sa_bstride = ((d.src_scale.mask & 1) && d.src_stride[0]) ? d.M * kb : 0;
-        constexpr int mx_smem = NSTAGE * mxf8_geo_t::STAGE_BYTES + NSTAGE * (BM + mxf8_geo_t::BN) * 4 + NTAB_BYTES;
-        static_assert(mxf8_geo_t::NSTAGE == NSTAGE && mxf8_geo_t::BN == f8_geo_t::BN, "one ring depth and tile width");
+        X.sa_bstride = plan.Bsa > 1 ? plan.blk_a * plan.nst * 256 : 0;
+        X.sb_bstride = plan.Bsb > 1 ? plan.blk_b * plan.nst * 256 : 0;
+        X.nst = (int)plan.nst;
+        constexpr int mx_smem = NSTAGE * f8_geo_t::STAGE_BYTES + mxf8_mma_t<0, 0, f8_geo_t>::EXTRA_LDS + NTAB_BYTES;
         auto go_mx = [&](auto kern) -> int {
             if (const int st = ensure_dynamic_lds((const void *)kern, mx_smem, "mfma_f8")) return st;
-            hipLaunchKernelGGL(kern, grid, dim3(mxf8_geo_t::NT), mx_smem, stream, P, X);
+            hipLaunchKernelGGL(kern, grid, dim3(f8_geo_t::NT), mx_smem, stream, P, X);
             return hipGetLastError() == hipSuccess ? MI355_SUCCESS : MI355_RUNTIME_ERROR;
         };
-        if (fa && fb) return go_mx(mxf8_gemm_kernel<mxf8_mma_t<1, 1, true, mxf8_geo_t>>);
-        if (fa) return go_mx(mxf8_gemm_kernel<mxf8_mma_t<1, 0, true, mxf8_geo_t>>);
-        if (fb) return go_mx(mxf8_gemm_kernel<mxf8_mma_t<0, 1, true, mxf8_geo_t>>);
-        return go_mx(mxf8_gemm_kernel<mxf8_mma_t<0, 0, true, mxf8_geo_t>>);
+        if (fa && fb) return go_mx(f8_gemm_kernel<mxf8_mma_t<1, 1, f8_geo_t>>);
+        if (fa) return go_mx(f8_gemm_kernel<mxf8_mma_t<1, 0, f8_geo_t>>);
+        if (fb) return go_mx(f8_gemm_kernel<mxf8_mma_t<0, 1, f8_geo_t>>);
+        return go_mx(f8_gemm_kernel<mxf8_mma_t<0, 0, f8_geo_t>>);
     }
     // Up to 128 tiles leave half of the CUs or more idle: 256 x 128 tiles of four wavefronts, two workgroups a CU, put
     // twice as many to work (a wavefront's part, 128 x 64, its fragments and the epilogue are the same).  MI355_F8_TILES=wide keeps the 256 x 256 tiles.

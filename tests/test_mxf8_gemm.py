@@ -59,15 +59,19 @@ def problem(M, N, K, *, sdt="f8_e4m3", wdt="f8_e4m3", ddt="f32", wtag="ba", exac
 def test_dispatch_rules():
     st, impl = cabi.query(problem(64, 64, 128).desc())
     assert st == cabi.SUCCESS and impl == cabi.IMPL_F8_MFMA
-    assert cabi.query(problem(64, 64, 192).desc())[1] == cabi.IMPL_REF      # scale rows of whole dwords: K % 128
+    assert cabi.query(problem(64, 64, 192).desc())[1] == cabi.IMPL_F8_MFMA   # any whole number of 64-byte stages
+    assert cabi.query(problem(64, 64, 160).desc())[1] == cabi.IMPL_F8_MFMA   # ... or of blocks: half a stage more
+    assert cabi.query(problem(64, 64, 32).desc())[1] == cabi.IMPL_REF        # less than a stage
     p = problem(64, 64, 128)
     p.quant["wei_scale"] = QuantParam(cabi.DT_F32, MASK_COL, np.ones(64, np.float32))   # MX on one side only
     assert cabi.query(p.desc())[1] == cabi.IMPL_REF
-    assert cabi.scratch_bytes(problem(64, 64, 128).desc()) == 64 * 4                      # the transposed weights scales
+    # the packed scales: 256 bytes per stage (two) for two blocks of 128 src rows and four blocks of 64 columns
+    assert cabi.scratch_bytes(problem(64, 64, 128).desc()) == (2 + 4) * 2 * 256
 
 
 @pytest.mark.gpu
-@pytest.mark.parametrize("shape", [(256, 256, 128), (300, 200, 256), (1, 8, 128), (33, 515, 384), (512, 768, 1024)])
+@pytest.mark.parametrize("shape", [(256, 256, 128), (300, 200, 256), (1, 8, 128), (33, 515, 384), (512, 768, 1024),
+                                   (300, 200, 192), (129, 65, 64)])
 @pytest.mark.parametrize("sdt,wdt", [("f8_e4m3", "f8_e4m3"), ("f8_e5m2", "f8_e4m3"), ("f8_e4m3", "f8_e5m2"),
                                      ("f8_e5m2", "f8_e5m2")])
 def test_exact_data_bit_exact(gpu, oracle, shape, sdt, wdt):
@@ -86,6 +90,45 @@ def test_exact_data_batched_with_bias_and_relu(gpu, oracle, wtag):
     got, name = run_gpu(p)
     assert name.startswith("hip:mfma_f8"), name
     assert_bit_exact(p, got, oracle.run_oracle(p), name)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("K", [96, 160, 224, 1056])
+@pytest.mark.parametrize("wtag", ["ba", "ab"])
+def test_a_k_of_an_odd_number_of_blocks(gpu, oracle, K, wtag):
+    """K = 64 s + 32: the last block is multiplied by one more step over the row's last 64 bytes, with the block
+    before it (multiplied already) zeroed; every block has a scale of its own, so the tail's scale must be the last
+    block's."""
+    p = problem(300, 328, K, seed=K, wtag=wtag, batch=2 if K == 160 else 1, bias=True)
+    got, name = run_gpu(p)
+    assert name.startswith("hip:mfma_f8"), name
+    assert_bit_exact(p, got, oracle.run_oracle(p), name)
+
+
+@pytest.mark.gpu
+def test_a_long_k_of_an_odd_number_of_blocks_within_the_bound(gpu, oracle):
+    """K = 4064 (63 stages and a block), random data: within the matrix-core bound around the float64 sum."""
+    p = problem(320, 448, 4064, exact=False, seed=5)
+    got, name = run_gpu(p)
+    assert name.startswith("hip:mfma_f8"), name
+    _, ideal, asum = oracle.run_oracle(p, want_ideal=True)
+    assert_gemm_close(p, got, ideal, asum, what=name, hw=mx_mfma_bound(p))
+
+
+@pytest.mark.gpu
+def test_the_tail_ignores_the_scale_of_the_block_it_zeroes(gpu, oracle):
+    """The block ahead of the tail block is read again and zeroed: a NaN scale (e8m0 0xff) of that block belongs to
+    the step before; rows whose scales are finite stay finite."""
+    p = problem(64, 96, 160, seed=9)
+    ss = p.quant["src_scale"].data.reshape(1, 64, 5).copy()
+    ss[0, 7, 3] = 0xff                    # block 3 = k 96 .. 127 of row 7: NaN, in its own step and nowhere else
+    p.quant["src_scale"].data = ss
+    got, name = run_gpu(p)
+    want = oracle.run_oracle(p)
+    g, w = np.asarray(got, np.float32).reshape(64, 96), np.asarray(want, np.float32).reshape(64, 96)
+    assert np.isnan(g[7]).all() and np.isnan(w[7]).all()
+    keep = np.arange(64) != 7
+    assert np.array_equal(g[keep], w[keep]) and np.isfinite(g[keep]).all()
 
 
 def mx_mfma_bound(p):
