@@ -275,7 +275,14 @@ struct f8_conv_t {
         return true;
         }
     }
-    // accumulator shapes without compile-time chains (the 16 x 16 tiles)
+    // the 16 x 16 tiles of the 16-bit policies: whole rows for a plain bf16 dst (tile_epilogue.hpp)
+    template <class PT>
+    __device__ __forceinline__ bool hot_chain(const PT &P, const epi_uniform_t &H, unsigned, unsigned lds_part,
+            const v4f (&acc)[8][4], long b, long m_base, long n_base, int) const {
+        if (ssc_p || with_src_sc || with_wei_sc) return false;
+        return store_rows_bf16_tile16(P, H, lds_part, acc, b, m_base, n_base);
+    }
+    // other accumulator shapes without compile-time chains
     template <class PT, class Acc>
     __device__ __forceinline__ bool hot_chain(const PT &, const epi_uniform_t &, unsigned, unsigned, const Acc &, long, long,
             long, int) const {

@@ -847,6 +847,63 @@ __device__ __forceinline__ void dynamic_quantQ(const PT &P, int dst_dt, float (&
     }
 }
 
+// A wavefront's 128 x 64 part of a bf16 dst when nothing follows the K sum but the conversion, from accumulators of
+// 16 x 16 tiles (a lane holds four consecutive columns of a row): written to dst as whole 128-byte rows.  In the
+// accumulator layout a wavefront-wide store touches 16 rows, 8 bytes each; the part goes through the wavefront's 16 KB
+// share of the idle tile ring instead -- 8-byte writes at row * 128 + ((slot ^ (row / 2 & 7)) << 4), which spread
+// over all banks -- and leaves as 16 stores of 8 whole rows.  False: not this case, nothing was stored.
+template <class PT, class V4>
+__device__ __forceinline__ bool store_rows_bf16_tile16(const PT &P, const epi_uniform_t &H, unsigned lds_part,
+        const V4 (&acc)[8][4], long b, long m_base, long n_base) {
+    typedef unsigned v2u_t __attribute__((ext_vector_type(2)));
+    typedef unsigned v4u_t __attribute__((ext_vector_type(4)));
+    typedef v2u_t __attribute__((address_space(3), may_alias)) *lds_u2_ptr_t;
+    typedef v4u_t __attribute__((address_space(3), may_alias)) *lds_u4_ptr_t;
+    typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
+    typedef float f32x2_t __attribute__((ext_vector_type(2)));
+    if (m_base >= P.M) return true; // nothing of this wavefront's part is inside dst
+    if (H.n_po != 0 || H.bias_mode != 0 || H.ds_mode != 0 || H.dzp_mode != 0 || H.dynamic || H.dst_dt != MI355_DT_BF16)
+        return false;
+    if (((uintptr_t)P.dst & 15) || (P.ds[0] % 8) || (P.ds[1] % 8)) return false;
+    const int lane = threadIdx.x & 63, lrow = lane & 15, q = lane >> 4;
+    const long rows_left = P.M - m_base;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+        const int r = 16 * i + lrow;
+        bool special = false;
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+#pragma unroll
+            for (int e = 0; e < 4; ++e) special |= __builtin_amdgcn_classf(acc[i][j][e], 0x93); // NaN or subnormal
+        const bool soft = __builtin_amdgcn_ballot_w64(special) != 0;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            v2u_t o;
+            if (!soft) {
+                o.x = __builtin_bit_cast(unsigned, __builtin_convertvector(f32x2_t {acc[i][j][0], acc[i][j][1]}, bf16x2_t));
+                o.y = __builtin_bit_cast(unsigned, __builtin_convertvector(f32x2_t {acc[i][j][2], acc[i][j][3]}, bf16x2_t));
+            } else {
+                o.x = f32_to_bf16(acc[i][j][0]) | ((unsigned)f32_to_bf16(acc[i][j][1]) << 16);
+                o.y = f32_to_bf16(acc[i][j][2]) | ((unsigned)f32_to_bf16(acc[i][j][3]) << 16);
+            }
+            // columns 16 j + 4 q ..: byte 32 j + 8 q of the row = slot 2 j + q / 2, half q % 2
+            const int slot = 2 * j + (q >> 1);
+            *(lds_u2_ptr_t)(size_t)(lds_part + (unsigned)(r * 128 + ((slot ^ ((r >> 1) & 7)) << 4) + 8 * (q & 1))) = o;
+        }
+    }
+    // (a wavefront reads back what its own lanes wrote: program order, no barrier)
+    char *dbase = (char *)P.dst + (b * P.ds[0] + m_base * P.ds[1] + n_base) * 2;
+    const int wr = lane >> 3, wslot = lane & 7;
+#pragma unroll
+    for (int d = 0; d < 16; ++d) {
+        const long r = d * 8 + wr;
+        const int chunk = wslot ^ (int)((r >> 1) & 7);
+        const v4u_t v = *(lds_u4_ptr_t)(size_t)(lds_part + (unsigned)(d * 1024 + lane * 16));
+        if (r < rows_left) __builtin_nontemporal_store(v, (v4u_t *)(dbase + r * P.ds[1] * 2 + chunk * 16));
+    }
+    return true;
+}
+
 // The epilogue of one wavefront's 128 x WCOLS part.
 //   park      the idle tile ring: every wavefront owns 16 KB of it (the general path parks
 //             Q x 64 x 16 bytes there, the specialised chains stage their part of dst)
