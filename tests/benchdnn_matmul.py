@@ -36,7 +36,7 @@ CUSTOM with the %engine% %impl% %name% %prb% %desc% %driver% %idx% %attr%
 
 Supported knobs: --dt, --stag, --wtag, --dtag (ab | ba | any), --bia-dt,
 --attr-scales, --attr-zero-points, --attr-post-ops, --attr-fpmath, --attr-dropout, --attr-rounding-mode, --impl,
---mode, --buffer-prefix, --export-buffers, --perf-template, --max-ms-per-prb,
+--mode, --buffer-prefix, --export-buffers, --perf-template, --max-ms-per-prb, --cold-cache (none | wei | all),
 and 2-D problem descriptors MxK:KxN.  Policies: common, per_oc,
 per_ocic (with GxH groups), per_tensor (with GxH groups), per_dim_0, per_dim_1.
 """
@@ -122,7 +122,36 @@ class Spec:
 
 
 # settings of the run, not of a problem (they do not multiply the problem list)
-SETTINGS = {"buffer_prefix": "", "export_buffers": "", "perf_template": "def", "max_ms_per_prb": "300"}
+SETTINGS = {"buffer_prefix": "", "export_buffers": "", "perf_template": "def", "max_ms_per_prb": "300",
+            "cold_cache": "none"}
+# --cold-cache (tests/benchdnn/utils/cold_cache.hpp:28-45, cold_cache.cpp:60-170): the timed executions rotate over
+# copies of the weights (`wei`) or of every execution argument (`all`) so that no execution finds them in a cache;
+# as many copies as it takes to exceed the caches (here: twice the 256 MB memory-side cache), at least two and at
+# most COLD_CACHE_MAX_BUFFERS.
+COLD_CACHE_BYTES = 512 << 20
+COLD_CACHE_MAX_BUFFERS = 64
+
+
+def cold_cache_sets(args, mode):
+    """The argument dictionaries the timed executions rotate over: `args` itself plus copies of the cold arguments."""
+    if mode == "none":
+        return [args]
+    if mode not in ("wei", "all"):
+        raise ValueError(f"unknown --cold-cache mode {mode} (none, wei, all)")
+    cold = [k for k in args if (mode == "all" or k == dnnl.ARG_WEIGHTS) and isinstance(args[k], dnnl.memory)]
+    size = sum(args[k].md.get_size() for k in cold)
+    if size == 0:
+        return [args]
+    n = max(2, min(COLD_CACHE_MAX_BUFFERS, -(-COLD_CACHE_BYTES // size)))
+    sets = [args]
+    for _ in range(n - 1):
+        s = dict(args)
+        for k in cold:
+            m = args[k]
+            nbytes = m.md.get_size()
+            s[k] = dnnl.memory(m.md, m.engine, m.read(np.uint8)[:nbytes] if nbytes else None)
+        sets.append(s)
+    return sets
 
 
 def parse(argv, settings=None):
@@ -530,11 +559,14 @@ def run_spec(sp, mode="C", min_times=5, max_ms=300.0, settings=None):
     if "P" in mode:
         prim.execute(strm, args)
         strm.wait()
-        times, t_all = [], time.perf_counter()
+        sets = cold_cache_sets(args, settings["cold_cache"])
+        details["cold_cache_buffers"] = len(sets)
+        times, t_all, it = [], time.perf_counter(), 0
         while len(times) < min_times or (time.perf_counter() - t_all) * 1e3 < max_ms:
             t0 = time.perf_counter()
             for _ in range(10):
-                prim.execute(strm, args)
+                prim.execute(strm, sets[it % len(sets)])
+                it += 1
             strm.wait()
             times.append((time.perf_counter() - t0) * 1e3 / 10)
             if len(times) >= 1000:

@@ -213,6 +213,31 @@ def test_perf_template_fields_and_modifiers():
         f"2|{det['ops'] / 1e3:g}|4|matmul|4|ab|%unknown%"
 
 
+def test_cold_cache_knob_is_run_wide_and_checked():
+    settings = dict(bd.SETTINGS)
+    mode, specs = bd.parse("--mode=P --cold-cache=wei --dt=s8:s8:s32 10x30:30x20".split(), settings)
+    assert len(specs) == 1 and settings["cold_cache"] == "wei"
+    assert bd.cold_cache_sets({}, "none") == [{}]
+    with pytest.raises(ValueError):
+        bd.cold_cache_sets({}, "lukewarm")
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("cc", ["wei", "all"])
+def test_cold_cache_rotates_over_copies_and_leaves_the_result_alone(gpu, oracle, cc, capsys, monkeypatch):
+    """tests/benchdnn/utils/cold_cache.hpp:28-45: the timed executions run on copies of the weights (or of every
+    argument); the correctness pass and its verdict are those of the warm run."""
+    monkeypatch.setattr(bd, "COLD_CACHE_BYTES", 8 << 20)          # a handful of copies is enough for the test
+    line = "--matmul --dt=s8:s8:s8 --wtag=any --attr-scales=src:common:0.5+wei:per_oc 1024x1024:1024x1024"
+    settings = dict(bd.SETTINGS, cold_cache=cc, max_ms_per_prb="50")
+    _, specs = bd.parse(line.split())
+    status, impl, det = bd.run_spec(specs[0], "CP", max_ms=50.0, settings=settings)
+    assert status == "PASSED" and impl.startswith("hip:mfma_i8") and det["errors"] == 0
+    assert det["cold_cache_buffers"] >= (8 if cc == "wei" else 2) and det["min_ms"] > 0
+    assert bd.main(line.split() + ["--mode=P", f"--cold-cache={cc}", "--max-ms-per-prb=20"]) == 0
+    assert any(ln.startswith("perf,") for ln in capsys.readouterr().out.splitlines())
+
+
 @pytest.mark.gpu
 def test_main_with_buffer_files_and_a_custom_perf_template(gpu, oracle, tmp_path, capsys):
     """The 256x1024:1024x1024 benchmark line end to end: export, then correctness + performance on
