@@ -157,7 +157,9 @@ typedef enum {
     dnnl_inner_product = 10,
     dnnl_binary = 13,
     dnnl_matmul = 14,
-    dnnl_prelu = 18
+    dnnl_prelu = 18,
+    /* src/common/c_types_map.hpp:2036-2040: internal-only kinds start at 1 << 12; sdpa is the second */
+    dnnl_amd_sdpa = (1 << 12) + 1
 } dnnl_primitive_kind_t;
 
 /* dnnl_types.h:2029-2049 */
@@ -216,7 +218,10 @@ typedef enum {
     dnnl_binary_lt = 0x1fff9,
     dnnl_binary_eq = 0x1fffa,
     dnnl_binary_ne = 0x1fffb,
-    dnnl_binary_select = 0x1fffc /* ternary: dst = src2 ? dst : src1 (dnnl_post_ops_append_binary_v2) */
+    dnnl_binary_select = 0x1fffc, /* ternary: dst = src2 ? dst : src1 (dnnl_post_ops_append_binary_v2) */
+    dnnl_softmax_accurate = 0x30000, /* dnnl_types.h:2252 */
+    /* src/common/c_types_map.hpp:148-155: internal-only algorithms start at 1 << 12; a row of -inf gives zeros */
+    dnnl_amd_softmax_accurate_inf_as_zero = (1 << 12) + 2
 } dnnl_alg_kind_t;
 
 /* dnnl_types.h:2448-2458 */
@@ -265,9 +270,12 @@ typedef enum {
 
 /* execute argument ids, dnnl_types.h:2544-2784 */
 #define DNNL_ARG_SRC 1
+#define DNNL_ARG_SRC_0 1 /* dnnl_types.h:2544 */
 #define DNNL_ARG_SRC_1 2
 #define DNNL_ARG_SRC_2 3 /* dnnl_types.h:2562: the condition of a binary select post-op */
 #define DNNL_ARG_DST 17
+#define DNNL_ARG_SCALE 51 /* dnnl_types.h:2638 */
+#define DNNL_ARG_SHIFT 52 /* dnnl_types.h:2640 */
 #define DNNL_ARG_DIFF_SRC 129     /* dnnl_types.h:2649-2652 */
 #define DNNL_ARG_DIFF_DST 145     /* dnnl_types.h:2676-2679 */
 #define DNNL_ARG_DIFF_WEIGHTS 161 /* dnnl_types.h:2697-2700 */
@@ -479,6 +487,26 @@ dnnl_status_t dnnl_inner_product_backward_weights_primitive_desc_create(dnnl_pri
         dnnl_engine_t engine, const_dnnl_memory_desc_t src_desc, const_dnnl_memory_desc_t diff_weights_desc,
         const_dnnl_memory_desc_t diff_bias_desc, const_dnnl_memory_desc_t diff_dst_desc,
         const_dnnl_primitive_desc_t hint_fwd_pd, const_dnnl_primitive_attr_t attr);
+
+/* ---- scaled dot-product attention, forward.  The reference keeps this primitive internal: the C++ function
+ * sdpa_primitive_desc_create of src/common/sdpa_test_iface.hpp:23-33 (what its own tests call); this is that
+ * function with C linkage, its arguments in the same order (invert_scale as int).  4-D tensors of f32 / bf16 / f16:
+ * queries [b][h][sq][d], keys [b][hk][d][sk], values [b][hk][sk][dv], dst [b][h][sq][dv], hk == h or 1, any
+ * strides; mask (attn_mask_type 1: a tensor whose dims are 1 or the full ones; 2 / 3: causal from the top left /
+ * bottom right, src/common/sdpa_types.hpp:41-55) and scale (one value in device memory) optional.  Execute
+ * arguments (sdpa_types.hpp:30-33): queries DNNL_ARG_SRC_0, keys DNNL_ARG_SRC_1, values DNNL_ARG_SRC_2,
+ * DNNL_ARG_DST, the mask DNNL_ARG_SHIFT, the scale DNNL_ARG_SCALE.  Not offered (dnnl_unimplemented): training
+ * (stats), quantized keys / values (kq_attr, vs_attr), other attributes, 1 < hk < h. ---- */
+#define DNNL_ARG_QUERIES DNNL_ARG_SRC_0
+#define DNNL_ARG_KEYS DNNL_ARG_SRC_1
+#define DNNL_ARG_VALUES DNNL_ARG_SRC_2
+#define DNNL_ARG_ATTN_MASK DNNL_ARG_SHIFT
+dnnl_status_t dnnl_amd_sdpa_primitive_desc_create(dnnl_primitive_desc_t *primitive_desc, dnnl_engine_t engine,
+        const_dnnl_memory_desc_t query_desc, const_dnnl_memory_desc_t key_desc, const_dnnl_memory_desc_t value_desc,
+        const_dnnl_memory_desc_t dst_desc, const_dnnl_memory_desc_t mask_desc, const_dnnl_memory_desc_t scale_desc,
+        int invert_scale, dnnl_dim_t kv_head_number, int attn_mask_type, dnnl_alg_kind_t softmax_alg,
+        dnnl_prop_kind_t prop, const_dnnl_primitive_attr_t attr, const_dnnl_primitive_attr_t kq_attr,
+        const_dnnl_primitive_attr_t vs_attr, const_dnnl_memory_desc_t stats_desc);
 
 /* ---- reorder primitive descriptor: dnnl.h:1727-1731.  Execute arguments are
  * DNNL_ARG_FROM / DNNL_ARG_TO (dnnl_types.h:2553,2580) plus the scales and zero

@@ -510,6 +510,28 @@ int mi355_grouped_matmul_launch(const mi355_grouped_desc_t *desc, const mi355_gr
 int mi355_colsum_launch(const void *x, int x_dt, int64_t rows, int64_t cols, int64_t ld, void *out, int out_dt,
         void *stream);
 
+/* The row softmax between the two matmuls of scaled dot-product attention
+ * (ref_sdpa, src/gpu/intel/sdpa/ref.cl:21-84: score * scale, + mask, exp, / sum;
+ * causal masks as in micro.cl:864-878: scores of keys beyond the diagonal are
+ * -inf).  scores: dense f32 [b][h][sq][sk]; probs: the same shape in out_dt
+ * (f32 / bf16 / f16).  The exponentials are taken relative to the row's largest
+ * score, which the reference does not do: the same number wherever the
+ * reference's exp does not overflow.  A row whose scores are all -inf gives
+ * zeros (softmax_accurate_inf_as_zero) or NaN (softmax_accurate). */
+typedef struct {
+    int64_t b, h, sq, sk;
+    int out_dt;
+    int scale_dt;        /* MI355_DT_UNDEF: no scale; else one value of f32 / bf16 / f16 in device memory */
+    int invert_scale;    /* multiply by 1 / scale, the reciprocal rounded to scale_dt */
+    int mask_type;       /* 0 none, 1 buffer, 2 causal from the top left, 3 causal from the bottom right */
+    int mask_dt;         /* f32 / bf16 / f16 (mask_type 1) */
+    int inf_as_zero;
+    int64_t mask_dims[4];   /* element (b % d0, h % d1, q % d2, k % d3) */
+    int64_t mask_stride[4]; /* in elements */
+} mi355_softmax_desc_t;
+int mi355_sdpa_softmax_launch(const mi355_softmax_desc_t *desc, const void *scores, void *probs, const void *scale,
+        const void *mask, void *stream);
+
 #ifdef __cplusplus
 }
 #endif

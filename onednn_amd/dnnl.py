@@ -42,6 +42,10 @@ ARG_ATTR_PRECOMPUTED_REDUCTIONS, ARG_ATTR_SCALES, ARG_ATTR_ZERO_POINTS = 512, 40
 ARG_ATTR_DROPOUT_OFFSET, ARG_ATTR_ROUNDING_SEED, ARG_ATTR_DROPOUT_MASK = 507, 508, 509
 ARG_ATTR_DROPOUT_PROBABILITY, ARG_ATTR_DROPOUT_SEED = 510, 511
 ARG_DIFF_SRC, ARG_DIFF_DST, ARG_DIFF_WEIGHTS, ARG_DIFF_BIAS = 129, 145, 161, 169
+ARG_QUERIES, ARG_KEYS, ARG_VALUES, ARG_SCALE, ARG_ATTN_MASK = 1, 2, 3, 51, 52
+kind_sdpa = (1 << 12) + 1
+softmax_accurate, softmax_accurate_inf_as_zero = 0x30000, (1 << 12) + 2
+attn_mask_undef, attn_mask_buffer, attn_mask_top_left, attn_mask_bottom_right = 0, 1, 2, 3
 rounding_environment, rounding_stochastic = 0, 1
 s64 = 16                               # dnnl_s64: the dropout seed / offset type
 scratchpad_library, scratchpad_user = 0, 1
@@ -440,6 +444,22 @@ class inner_product_backward_weights_primitive_desc(inner_product_forward_primit
             "inner_product_backward_weights_primitive_desc_create")
 
 
+class sdpa_primitive_desc(inner_product_forward_primitive_desc):
+    """sdpa_primitive_desc_create(engine, query, key, value, dst, mask, scale, invert_scale, kv_head_number,
+    attn_mask_type, softmax_alg, prop, attr, kq_attr, vs_attr, stats) of the reference's internal test interface"""
+
+    def __init__(self, eng, q_md, k_md, v_md, dst_md, mask_md=None, scale_md=None, invert_scale=False,
+                 kv_head_number=0, attn_mask_type=0, softmax_alg=softmax_accurate, prop=forward_inference, attr=None,
+                 kq_attr=None, vs_attr=None, stats_md=None):
+        self.engine = eng
+        self.h = C.c_void_p()
+        h = lambda x: x.h if x is not None else None  # noqa: E731
+        _check(lib().dnnl_amd_sdpa_primitive_desc_create(
+            C.byref(self.h), eng.h, q_md.h, k_md.h, v_md.h, dst_md.h, h(mask_md), h(scale_md), int(invert_scale),
+            C.c_int64(kv_head_number), int(attn_mask_type), int(softmax_alg), int(prop), h(attr), h(kq_attr), h(vs_attr),
+            h(stats_md)), "sdpa_primitive_desc_create")
+
+
 class reorder_primitive_desc(matmul_primitive_desc):
     """dnnl::reorder::primitive_desc(src_engine, src_md, dst_engine, dst_md, attr)"""
 
@@ -476,6 +496,10 @@ class inner_product_backward_data(matmul):
 class inner_product_backward_weights(matmul):
     """dnnl::inner_product_backward_weights(pd); execute(stream, {ARG_DIFF_DST, ARG_SRC, ARG_DIFF_WEIGHTS,
     ARG_DIFF_BIAS})"""
+
+
+class sdpa(matmul):
+    """execute(stream, {ARG_QUERIES, ARG_KEYS, ARG_VALUES, ARG_DST, ARG_ATTN_MASK, ARG_SCALE})"""
 
 
 class reorder(matmul):

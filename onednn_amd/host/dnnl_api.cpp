@@ -246,6 +246,16 @@ struct dnnl_primitive_desc {
     // diff_bias and diff_dst as the caller describes them
     dnnl_memory_desc ip_dst;
     bool ip_diff_bias = false;
+    // scaled dot-product attention (kind == dnnl_amd_sdpa): dst = softmax(scale * Q K + mask) V as two batched
+    // matmuls around a row-softmax kernel; the scores and the probabilities live in the primitive's scratchpad
+    struct sdpa_t {
+        dnnl_memory_desc q, k, v, dst, mask, scale;
+        dnnl_memory_desc scores, probs; // dense [b][h][sq][sk]: f32, and the values' type
+        bool invert_scale = false, inf_as_zero = false;
+        int mask_type = 0;
+        std::shared_ptr<dnnl_primitive_desc> kq, vs;
+    };
+    std::shared_ptr<sdpa_t> sdpa;
     mi355_grouped_desc_t gdesc;
     std::vector<int> impls;       // kernel families that can run it, best first
     size_t impl_pos = 0;
@@ -273,6 +283,7 @@ struct dnnl_primitive_desc {
 
 struct dnnl_primitive {
     dnnl_primitive_desc pd;
+    dnnl_primitive *sdpa_kq = nullptr, *sdpa_vs = nullptr; // the two matmuls of an attention primitive
     void *scratch = nullptr; // library-mode scratchpad (device)
     std::mutex scratch_mutex;
     // runtime dims: the lowering of the last executed shapes, and the scratch
@@ -291,6 +302,8 @@ struct dnnl_primitive {
     void *last_stream = nullptr;
     bool event_recorded = false;
     ~dnnl_primitive() {
+        delete sdpa_kq;
+        delete sdpa_vs;
         if (scratch) mi355_mem_free(scratch);
         for (void *q : rt_scratch) mi355_mem_free(q);
         if (host_scalars) mi355_mem_free(host_scalars);
@@ -2175,6 +2188,100 @@ DNNL_EXPORT dnnl_status_t dnnl_inner_product_backward_weights_primitive_desc_cre
     return ip_backward_create(primitive_desc, engine, false, src_desc, diff_weights_desc, b, diff_dst_desc, attr);
 }
 
+// Scaled dot-product attention (src/common/sdpa_test_iface.hpp:23-33, sdpa_utils.hpp:51-82 for the shape rules,
+// sdpa_pd.hpp, the reference kernel src/gpu/intel/sdpa/ref.cl): forward only, 4-D tensors
+//   queries [b][h][sq][d], keys [b][hk][d][sk], values [b][hk][sk][dv], dst [b][h][sq][dv], any strides;
+//   mask [..][..][..][..] of dims 1 or the full ones; scale: one value in device memory.
+// Lowered to   scores = Q x K (f32)  ->  probs = softmax(scores * scale + mask)  ->  dst = probs x V
+// with the matmul families of this library (batch dims b, h; keys / values of one head are broadcast).
+DNNL_EXPORT dnnl_status_t dnnl_amd_sdpa_primitive_desc_create(dnnl_primitive_desc_t *primitive_desc, dnnl_engine_t engine,
+        const_dnnl_memory_desc_t query_desc, const_dnnl_memory_desc_t key_desc, const_dnnl_memory_desc_t value_desc,
+        const_dnnl_memory_desc_t dst_desc, const_dnnl_memory_desc_t mask_desc, const_dnnl_memory_desc_t scale_desc,
+        int invert_scale, dnnl_dim_t kv_head_number, int attn_mask_type, dnnl_alg_kind_t softmax_alg,
+        dnnl_prop_kind_t prop, const_dnnl_primitive_attr_t attr, const_dnnl_primitive_attr_t kq_attr,
+        const_dnnl_primitive_attr_t vs_attr, const_dnnl_memory_desc_t stats_desc) {
+    CHECK_ARG(primitive_desc && engine && query_desc && key_desc && value_desc && dst_desc);
+    const dnnl_memory_desc &q = *query_desc, &k = *key_desc, &v = *value_desc, &d = *dst_desc;
+    // sdpa_desc_check
+    const int nd = d.ndims, r = nd - 2, c = nd - 1;
+    CHECK_ARG(nd >= 2 && q.ndims == nd && k.ndims == nd && v.ndims == nd);
+    CHECK_ARG(q.dims[c] == k.dims[r] && k.dims[c] == v.dims[r] && d.dims[r] == q.dims[r] && d.dims[c] == v.dims[c]);
+    const bool with_mask = mask_desc && !mask_desc->is_zero() && mask_desc->dt != dnnl_data_type_undef;
+    const bool with_scale = scale_desc && !scale_desc->is_zero() && scale_desc->dt != dnnl_data_type_undef;
+    for (const dnnl_memory_desc *md : {&q, &k, &v, &d}) CHECK_ARG(md->kind != dnnl_format_kind_host_scalar);
+    if (with_mask) CHECK_ARG(mask_desc->kind != dnnl_format_kind_host_scalar);
+    CHECK_ARG(attn_mask_type >= 0 && attn_mask_type <= 3);
+    CHECK_ARG(prop == dnnl_forward_inference || prop == dnnl_forward_training);
+    // what this implementation takes
+    CHECK_UNIMPL(nd == 4);                                   // (as the reference kernel: ref.hpp:50-56)
+    CHECK_UNIMPL(prop == dnnl_forward_inference && !(stats_desc && !stats_desc->is_zero()));
+    for (const_dnnl_primitive_attr_t a : {attr, kq_attr, vs_attr}) {
+        if (!a) continue;                                    // no quantized keys / values, no attributes
+        CHECK_UNIMPL(a->scales.empty() && a->zero_points.empty() && a->reductions.empty() && a->post_ops.entries.empty()
+                && !a->with_dropout() && a->rounding.empty() && a->scratchpad_mode == dnnl_scratchpad_mode_library);
+    }
+    auto fp = [](dnnl_data_type_t dt) { return dt == dnnl_f32 || dt == dnnl_bf16 || dt == dnnl_f16; };
+    CHECK_UNIMPL(fp(q.dt) && k.dt == q.dt && v.dt == q.dt && fp(d.dt));
+    for (const dnnl_memory_desc *md : {&q, &k, &v, &d})
+        CHECK_UNIMPL(md->kind == dnnl_blocked && !md->has_runtime() && !md->grouped);
+    const dim_t B = q.dims[0], H = q.dims[1], Sq = q.dims[2], Sk = k.dims[3];
+    CHECK_ARG(d.dims[0] == B && d.dims[1] == H);
+    // keys and values: per head, or one head for all (both ways of grouping query heads agree on these two)
+    for (const dnnl_memory_desc *md : {&k, &v}) {
+        CHECK_ARG(md->dims[0] == B || md->dims[0] == 1);
+        CHECK_UNIMPL(md->dims[1] == H || md->dims[1] == 1);
+    }
+    CHECK_ARG(kv_head_number <= 0 || kv_head_number == k.dims[1] || k.dims[1] == 1);
+    CHECK_UNIMPL(softmax_alg == dnnl_softmax_accurate || (int)softmax_alg == dnnl_amd_softmax_accurate_inf_as_zero);
+    const int mask_type = with_mask ? (attn_mask_type == 0 ? 1 : attn_mask_type) : (attn_mask_type == 1 ? 0 : attn_mask_type);
+    if (with_mask) {
+        CHECK_UNIMPL(mask_type == 1 && mask_desc->ndims == 4 && mask_desc->kind == dnnl_blocked && fp(mask_desc->dt));
+        const dim_t full[4] = {B, H, Sq, Sk};
+        for (int i = 0; i < 4; ++i) CHECK_ARG(mask_desc->dims[i] == full[i] || mask_desc->dims[i] == 1);
+    }
+    if (with_scale) {
+        CHECK_UNIMPL(scale_desc->kind != dnnl_format_kind_host_scalar && fp(scale_desc->dt));
+        CHECK_ARG(scale_desc->nelems() == 1);
+    }
+    std::unique_ptr<dnnl_primitive_desc> pd(new dnnl_primitive_desc);
+    pd->kind = (dnnl_primitive_kind_t)dnnl_amd_sdpa;
+    pd->engine = engine;
+    pd->prop_kind = (int)prop;
+    if (attr) pd->attr = *attr;
+    auto S = std::make_shared<dnnl_primitive_desc::sdpa_t>();
+    S->q = q; S->k = k; S->v = v; S->dst = d;
+    if (with_mask) S->mask = *mask_desc;
+    if (with_scale) S->scale = *scale_desc;
+    S->invert_scale = invert_scale != 0;
+    S->inf_as_zero = (int)softmax_alg == dnnl_amd_softmax_accurate_inf_as_zero;
+    S->mask_type = mask_type;
+    const dim_t sdims[4] = {B, H, Sq, Sk};
+    for (dnnl_memory_desc *md : {&S->scores, &S->probs}) {
+        md->ndims = 4;
+        md->kind = dnnl_blocked;
+        for (int i = 0; i < 4; ++i) md->dims[i] = sdims[i];
+        md->set_dense();
+    }
+    S->scores.dt = dnnl_f32;
+    S->probs.dt = v.dt;
+    dnnl_primitive_desc_t kq = nullptr, vs = nullptr;
+    dnnl_status_t st = dnnl_matmul_primitive_desc_create(&kq, engine, &S->q, &S->k, nullptr, &S->scores, nullptr);
+    if (st) return st;
+    S->kq.reset(kq);
+    st = dnnl_matmul_primitive_desc_create(&vs, engine, &S->probs, &S->v, nullptr, &S->dst, nullptr);
+    if (st) return st;
+    S->vs.reset(vs);
+    pd->src = q; pd->wei = k; pd->dst = d;
+    pd->scratch_bytes = ((S->scores.size_bytes() + 255) & ~(size_t)255) + S->probs.size_bytes();
+    pd->scratchpad = dnnl_memory_desc(); // library mode only: nothing for the caller to provide
+    pd->impl_name = "hip:sdpa(" + kq->impl_name + "," + vs->impl_name + ")";
+    pd->sdpa = S;
+    if (verbose_level() >= 1)
+        fprintf(stderr, "onednn_verbose,v1,primitive,create:dispatch,gpu,sdpa,%s\n", pd->impl_name.c_str());
+    *primitive_desc = pd.release();
+    return dnnl_success;
+}
+
 // ---- reorder primitive descriptor (src/common/reorder.cpp:67-170)
 DNNL_EXPORT dnnl_status_t dnnl_reorder_primitive_desc_create(dnnl_primitive_desc_t *reorder_primitive_desc,
         const_dnnl_memory_desc_t src_desc, dnnl_engine_t src_engine, const_dnnl_memory_desc_t dst_desc,
@@ -2411,6 +2518,14 @@ DNNL_EXPORT dnnl_status_t dnnl_primitive_create(dnnl_primitive_t *primitive, con
         const int st = mi355_mem_alloc(&p->scratch, p->pd.scratch_bytes);
         if (st != MI355_SUCCESS) return from_mi355(st);
     }
+    if (p->pd.sdpa) {
+        dnnl_primitive_t kq = nullptr, vs = nullptr;
+        dnnl_status_t st = dnnl_primitive_create(&kq, p->pd.sdpa->kq.get());
+        if (st == dnnl_success) st = dnnl_primitive_create(&vs, p->pd.sdpa->vs.get());
+        p->sdpa_kq = kq;
+        p->sdpa_vs = vs;
+        if (st != dnnl_success) return st;
+    }
     bool any_on_host = false;
     for (const auto *mp : {&p->pd.attr.scales, &p->pd.attr.zero_points})
         for (const auto &kv : *mp) any_on_host |= kv.second.on_host;
@@ -2495,6 +2610,54 @@ DNNL_EXPORT dnnl_status_t dnnl_primitive_execute(const_dnnl_primitive_t cprimiti
         if (prim->order_event && prim->event_recorded && prim->last_stream != stream->hip_stream)
             mi355_stream_wait_event(stream->hip_stream, prim->order_event);
     };
+    if (pd0.sdpa) {
+        const dnnl_primitive_desc::sdpa_t &S = *pd0.sdpa;
+        auto get = [&](int arg) -> dnnl_memory_t {
+            auto it = m.find(arg);
+            return it == m.end() ? nullptr : it->second;
+        };
+        dnnl_memory_t q = get(DNNL_ARG_SRC_0), k = get(DNNL_ARG_SRC_1), v = get(DNNL_ARG_SRC_2), d = get(DNNL_ARG_DST);
+        dnnl_memory_t mask = get(DNNL_ARG_SHIFT), scale = get(DNNL_ARG_SCALE);
+        CHECK_ARG(q && k && v && d);
+        CHECK_ARG(IMPLICATION(S.mask_type == 1, mask && mask->handle));
+        CHECK_ARG(IMPLICATION(!S.scale.is_zero(), scale && scale->handle));
+        if (S.dst.nelems() == 0) return dnnl_success;
+        CHECK_ARG(q->handle && k->handle && v->handle && d->handle && prim->scratch);
+        if (mi355_device_set((int)pd0.engine->index) != MI355_SUCCESS) return dnnl_runtime_error;
+        order_on_device(); // the scores and probabilities belong to the primitive
+        dnnl_memory sc_mem, pr_mem;
+        sc_mem.md = S.scores; sc_mem.engine = pd0.engine; sc_mem.handle = prim->scratch;
+        pr_mem.md = S.probs; pr_mem.engine = pd0.engine;
+        pr_mem.handle = (char *)prim->scratch + ((S.scores.size_bytes() + 255) & ~(size_t)255);
+        const dnnl_exec_arg_t a1[3] = {{DNNL_ARG_SRC, q}, {DNNL_ARG_WEIGHTS, k}, {DNNL_ARG_DST, &sc_mem}};
+        dnnl_status_t st = dnnl_primitive_execute(prim->sdpa_kq, stream, 3, a1);
+        if (st != dnnl_success) return st;
+        mi355_softmax_desc_t sd;
+        memset(&sd, 0, sizeof(sd));
+        sd.b = S.scores.dims[0]; sd.h = S.scores.dims[1]; sd.sq = S.scores.dims[2]; sd.sk = S.scores.dims[3];
+        sd.out_dt = (int)S.probs.dt;
+        sd.scale_dt = S.scale.is_zero() ? (int)MI355_DT_UNDEF : (int)S.scale.dt;
+        sd.invert_scale = S.invert_scale;
+        sd.mask_type = S.mask_type;
+        sd.inf_as_zero = S.inf_as_zero;
+        if (S.mask_type == 1) {
+            sd.mask_dt = (int)S.mask.dt;
+            for (int i = 0; i < 4; ++i) {
+                sd.mask_dims[i] = S.mask.dims[i];
+                sd.mask_stride[i] = S.mask.strides[i];
+            }
+        }
+        const int rc = mi355_sdpa_softmax_launch(&sd, sc_mem.handle, pr_mem.handle, scale ? scale->handle : nullptr,
+                mask ? mask->handle : nullptr, stream->hip_stream);
+        if (rc != MI355_SUCCESS) return from_mi355(rc);
+        const dnnl_exec_arg_t a2[3] = {{DNNL_ARG_SRC, &pr_mem}, {DNNL_ARG_WEIGHTS, v}, {DNNL_ARG_DST, d}};
+        st = dnnl_primitive_execute(prim->sdpa_vs, stream, 3, a2);
+        if (prim->order_event && mi355_event_record(prim->order_event, stream->hip_stream) == MI355_SUCCESS) {
+            prim->event_recorded = true;
+            prim->last_stream = stream->hip_stream;
+        }
+        return st;
+    }
     void *rt_scratch = nullptr;
     if (pd0.runtime) {
         // executions of one primitive with runtime dims are serialised on the

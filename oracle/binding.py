@@ -164,6 +164,39 @@ def run_oracle_inner_product_bwd_weights(diff_dst, src, dts, with_bias, dwei_ord
     return out, bias
 
 
+def run_oracle_sdpa(q, k, v, dts, scale=None, invert_scale=False, mask=None, mask_type=0, dst_order=None):
+    """Scaled dot-product attention.  q [b1][b0][sq][d], k [.][.][d][sk], v [.][.][sk][dv]: numpy views (storage type
+    of dts[0]) in any memory order, the first two dims of k / v 1 or full; dts = (q/k/v, dst, scale, mask) data type
+    names; scale: a one-element array or None; mask: a 4-D view whose dims are 1 or full (mask_type 1), or None with
+    mask_type 2 / 3 for the causal masks.  Returns dst as a view of the logical shape [b1][b0][sq][dv]."""
+    lib = load()
+    i64p = C.c_void_p
+    lib.oracle_sdpa.argtypes = [i64p, C.c_int, i64p, C.c_void_p, i64p, i64p, C.c_void_p, i64p, i64p, C.c_void_p, C.c_int,
+                                i64p, C.c_void_p, C.c_int, C.c_void_p, C.c_int, C.c_int, C.c_int, i64p, i64p, C.c_void_p]
+    from onednn_amd.problem import storage_dtype
+    b1, b0, sq, d = q.shape
+    sk, dv = k.shape[3], v.shape[3]
+    assert k.shape[2] == d and v.shape[2] == sk
+    order = list(dst_order) if dst_order is not None else [0, 1, 2, 3]
+    shape = (b1, b0, sq, dv)
+    store = np.zeros([shape[i] for i in order], storage_dtype(cabi.DT_NAMES[dts[1]]))
+    out = store.transpose(np.argsort(order))
+    dims = np.array([b1, b0, sq, d, sk, dv], np.int64)
+    kd, vd = np.array(k.shape[:2], np.int64), np.array(v.shape[:2], np.int64)
+    sts = [_elem_strides(x) for x in (q, k, v, out)]
+    md = np.array(mask.shape if mask is not None else (1, 1, 1, 1), np.int64)
+    ms = _elem_strides(mask) if mask is not None else np.zeros(4, np.int64)
+    st = lib.oracle_sdpa(dims.ctypes.data, cabi.DT_NAMES[dts[0]], sts[0].ctypes.data, q.ctypes.data, kd.ctypes.data,
+                         sts[1].ctypes.data, k.ctypes.data, vd.ctypes.data, sts[2].ctypes.data, v.ctypes.data,
+                         cabi.DT_NAMES[dts[1]], sts[3].ctypes.data, store.ctypes.data,
+                         cabi.DT_NAMES[dts[2]] if scale is not None else 0,
+                         scale.ctypes.data if scale is not None else None, int(invert_scale), int(mask_type),
+                         cabi.DT_NAMES[dts[3]] if mask is not None else 0, md.ctypes.data, ms.ctypes.data,
+                         mask.ctypes.data if mask is not None else None)
+    assert st == 0, f"oracle_sdpa status {st}"
+    return out
+
+
 def run_oracle_dropout(prob: MatmulProblem):
     """(raw dst storage, the dropout mask or None)."""
     prob._oracle_mask = None

@@ -30,6 +30,7 @@
  *   oracle_inner_product_bwd_data, oracle_inner_product_bwd_weights
  *                     ref_inner_product_bwd_data_t / _bwd_weights_t
  *                     src/cpu/ref_inner_product.cpp:100-217
+ *   oracle_sdpa       ref_sdpa, src/gpu/intel/sdpa/ref.cl:21-84 (+ the causal masks of micro.cl:864-878)
  *   oracle_inner_product_fwd
  *                     ref_inner_product_fwd_t::execute_forward src/cpu/ref_inner_product.cpp:33-100
  *                     and ref_inner_product_int8_fwd_t::execute_forward
@@ -81,6 +82,9 @@
  * dims on exact data for every ndims and for permuted layouts of src and
  * weights, the scale / bias / dst-scale order on values where a different
  * order changes bits; bias, post-ops and the store are orc_finish.
+ * oracle_sdpa is pinned by tests/test_sdpa.py: a float64 numpy softmax(scale * Q K + mask) V for per-head and
+ * shared keys / values, broadcast masks, both causal masks (a transposed K, a mask added after the exponential
+ * or a diagonal off by one fail it), the inverted scale's rounding on a value where it changes the result.
  * The backward inner products (oracle_inner_product_bwd_data / _bwd_weights)
  * are pinned there too: numpy tensordot on exact data over the other index
  * pair for every ndims and for permuted layouts (a transposed operand or a
@@ -993,6 +997,68 @@ int oracle_inner_product_bwd_weights(int ndims, const int64_t *dims, int64_t OC,
             orc_store_float(dbias_dt, db, diff_bias, oc);
         }
     }
+    return MI355_SUCCESS;
+}
+
+/* Scaled dot-product attention, forward: ref_sdpa of src/gpu/intel/sdpa/ref.cl:21-84 loop by loop --
+ *   s[k] = sum_h Q[b1, b0, q, h] * K[b1 % kd0, b0 % kd1, h, k]           (f32, h ascending)
+ *   s[k] *= scale (the scale read in its type; inverted: 1.f / scale rounded back to that type)
+ *   s[k] += mask[b1 % md0, b0 % md1, q, k];  s[k] = exp(s[k]);  sum += s[k]  (k ascending)
+ *   s[k] /= sum
+ *   dst[b1, b0, q, v] = sum_k V[b1 % vd0, b0 % vd1, k, v] * s[k]          (f32, k ascending)
+ * No subtraction of the row maximum, as in the reference.  mask_type 2 / 3: the scores of keys beyond the
+ * diagonal (k > q, or k > q + sk - sq) are -inf before the exponential (src/gpu/intel/sdpa/micro.cl:864-878).
+ * The mask is indexed modulo its dims in all four positions (the reference: in the first two; the same thing
+ * for a mask whose last two dims are full).  dims: {b1, b0, sq, d, sk, dv}; strides in elements, four per tensor. */
+int oracle_sdpa(const int64_t *dims, int q_dt, const int64_t *q_st, const void *Q, const int64_t *k_dims01,
+        const int64_t *k_st, const void *K, const int64_t *v_dims01, const int64_t *v_st, const void *V, int dst_dt,
+        const int64_t *d_st, void *dst, int scale_dt, const void *scale_p, int invert_scale, int mask_type, int mask_dt,
+        const int64_t *m_dims, const int64_t *m_st, const void *mask) {
+    const int64_t B1 = dims[0], B0 = dims[1], SQ = dims[2], D = dims[3], SK = dims[4], DV = dims[5];
+    float scale = 1.f;
+    if (scale_dt != MI355_DT_UNDEF) {
+        scale = orc_load_float(scale_dt, scale_p, 0);
+        if (invert_scale) {
+            uint32_t tmp[1] = {0};
+            orc_store_float(scale_dt, 1.f / scale, tmp, 0);
+            scale = orc_load_float(scale_dt, tmp, 0);
+        }
+    }
+#pragma omp parallel for collapse(2) schedule(static)
+    for (int64_t b1 = 0; b1 < B1; ++b1)
+        for (int64_t b0 = 0; b0 < B0; ++b0) {
+            float *s = (float *)malloc(sizeof(float) * (size_t)(SK > 0 ? SK : 1));
+            for (int64_t q = 0; q < SQ; ++q) {
+                for (int64_t k = 0; k < SK; ++k) {
+                    float acc = 0.f;
+                    for (int64_t h = 0; h < D; ++h)
+                        acc += orc_load_float(q_dt, Q, b1 * q_st[0] + b0 * q_st[1] + q * q_st[2] + h * q_st[3])
+                                * orc_load_float(q_dt, K, (b1 % k_dims01[0]) * k_st[0] + (b0 % k_dims01[1]) * k_st[1]
+                                        + h * k_st[2] + k * k_st[3]);
+                    s[k] = acc;
+                }
+                float s_sum = 0.f;
+                for (int64_t k = 0; k < SK; ++k) {
+                    if (scale_dt != MI355_DT_UNDEF) s[k] *= scale;
+                    if (mask_type == 1)
+                        s[k] += orc_load_float(mask_dt, mask, (b1 % m_dims[0]) * m_st[0] + (b0 % m_dims[1]) * m_st[1]
+                                + (q % m_dims[2]) * m_st[2] + (k % m_dims[3]) * m_st[3]);
+                    if ((mask_type == 2 && k > q) || (mask_type == 3 && k > q + (SK - SQ))) s[k] = -INFINITY;
+                    s[k] = expf(s[k]);
+                    s_sum += s[k];
+                }
+                for (int64_t k = 0; k < SK; ++k) s[k] /= s_sum;
+                for (int64_t v = 0; v < DV; ++v) {
+                    float acc = 0.f;
+                    for (int64_t k = 0; k < SK; ++k)
+                        acc += orc_load_float(q_dt, V, (b1 % v_dims01[0]) * v_st[0] + (b0 % v_dims01[1]) * v_st[1]
+                                       + k * v_st[2] + v * v_st[3])
+                                * s[k];
+                    orc_store_float(dst_dt, acc, dst, b1 * d_st[0] + b0 * d_st[1] + q * d_st[2] + v * d_st[3]);
+                }
+            }
+            free(s);
+        }
     return MI355_SUCCESS;
 }
 
