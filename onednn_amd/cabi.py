@@ -151,7 +151,8 @@ KERNEL_SYMBOLS = [
     "mi355_stream_wait_event", "mi355_mem_store_scalar",
     "mi355_last_error", "mi355_matmul_query", "mi355_matmul_impl_name",
     "mi355_matmul_scratch_bytes", "mi355_matmul_launch", "mi355_matmul_launch_noalloc", "mi355_reorder_query",
-    "mi355_reorder_launch", "mi355_wei_pack_reorder_dims", "mi355_tuning_set", "mi355_colsum_launch", "mi355_grouped_matmul_query",
+    "mi355_reorder_launch", "mi355_wei_pack_reorder_dims", "mi355_tuning_set", "mi355_colsum_launch", "mi355_sdpa_softmax_launch",
+    "mi355_grouped_matmul_query",
     "mi355_grouped_matmul_launch", "mi355_grouped_matmul_impl",
 ]
 
