@@ -1,7 +1,8 @@
 """The boundary through a compiler: small C programs that include only
 include/dnnl_amd.h / include/mi355_matmul.h, built with gcc against the two
 shared libraries and run on the device (u8 x s8 -> s32 matmuls and an inner product on
-channels-last tensors, each checked against an integer loop inside the program).  Struct layouts, enum values and calling
+channels-last tensors, each checked against an integer loop inside the program; attention on f32 tensors against a
+double-precision loop).  Struct layouts, enum values and calling
 conventions of the headers are what a compiled caller sees; the ctypes tests
 only check names."""
 import os
@@ -23,25 +24,27 @@ def build(name, lib):
     exe = os.path.join(d, name)
     subprocess.check_call(["gcc", "-std=c11", "-Wall", "-Wextra", "-Werror", "-I", INC, "-o", exe,
                            os.path.join(ROOT, "tests", "c_clients", name + ".c"), "-L", LIB, "-l" + lib,
-                           "-Wl,-rpath," + LIB])
+                           "-Wl,-rpath," + LIB, "-lm"])
     return d, exe
 
 
 def test_headers_compile_as_c_and_link():
     # no device needed: the programs build against the headers and libraries
-    for name, lib in (("dnnl_client", "dnnl_amd"), ("ip_client", "dnnl_amd"), ("mi355_client", "mi355_matmul")):
+    for name, lib in (("dnnl_client", "dnnl_amd"), ("ip_client", "dnnl_amd"), ("sdpa_client", "dnnl_amd"),
+                      ("mi355_client", "mi355_matmul")):
         d, exe = build(name, lib)
         assert os.path.exists(exe)
         shutil.rmtree(d, ignore_errors=True)
 
 
 @pytest.mark.gpu
-@pytest.mark.parametrize("name,lib", [("dnnl_client", "dnnl_amd"), ("ip_client", "dnnl_amd"),
-                                      ("mi355_client", "mi355_matmul")])
-def test_c_client_runs_on_the_device(gpu, name, lib):
+@pytest.mark.parametrize("name,lib,impl", [("dnnl_client", "dnnl_amd", "hip:mfma_i8"), ("ip_client", "dnnl_amd", "hip:mfma_i8"),
+                                           ("sdpa_client", "dnnl_amd", "hip:sdpa("),
+                                           ("mi355_client", "mi355_matmul", "hip:mfma_i8")])
+def test_c_client_runs_on_the_device(gpu, name, lib, impl):
     d, exe = build(name, lib)
     try:
         out = subprocess.run([exe], capture_output=True, text=True, timeout=120)
-        assert out.returncode == 0 and out.stdout.startswith("ok hip:mfma_i8"), (out.stdout, out.stderr)
+        assert out.returncode == 0 and out.stdout.startswith("ok " + impl), (out.stdout, out.stderr)
     finally:
         shutil.rmtree(d, ignore_errors=True)
