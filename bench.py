@@ -52,7 +52,7 @@ PROFILE_OF = {
     ("c3", "any"): "i8_gemm_kernel_c3_8192.md", ("c4", "any"): "f8_gemm_kernel_c4_4096x8192x28672.md",
     ("c5", "any"): "mxf4_gemm_kernel_c5_8192.md", ("c1", "any"): "i8_small_kernel_c1_256x1024x1024.md",
     ("h1", "any"): "f8_gemm_kernel_h1_bf16_8192.md", ("h2", "any"): "f8_gemm_kernel_h2_f32_8192.md",
-    ("m1", "any"): "mxf8_gemm_kernel_m1_mxfp8_8192.md",
+    ("m1", "any"): "f8_gemm_kernel_m1_mxfp8_8192.md",
     ("c2", "any", 1): "woqp_kernel_c2_m1.md", ("c2", "any", 8): "woqp_kernel_c2_m8.md",
     ("c2", "any", 32): "woqp_kernel_c2_m32.md", ("c2", "ab", 1): "woq_gemv_kernel_c2_m1_plain_ab.md",
     ("c2", "ab", 8): "woq_gemv_kernel_c2_m8_plain_ab.md", ("c2", "ab", 32): "woq_gemv_kernel_c2_m32_plain_ab.md",
