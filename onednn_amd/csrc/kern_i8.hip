@@ -300,7 +300,7 @@ __global__ void __launch_bounds__(G::NT) __attribute__((amdgpu_waves_per_eu(G::N
 // stage loads want K in units of 64.  Here a workgroup of four wavefronts owns a
 // 32 x 32 tile, the wavefronts take every fourth 64-byte step of K, each lane
 // loads its MFMA operands (16 bytes of a src row, 16 bytes of a weights
-// column, K contiguous in both) straight from memory, one step ahead of the
+// column, K contiguous in both) straight from memory, four steps ahead of the
 // matrix cores, and a step beyond K's last 16 bytes is filled with the
 // operand's zero.  The column sums of the weights and the row sums of src that
 // the zero-point correction needs come out of two more MFMAs per operand tile
@@ -363,10 +363,10 @@ __global__ void __launch_bounds__(SNW * 64) i8_small_kernel(const problem_t P_, 
     }
     const v4i ones = {0x01010101, 0x01010101, 0x01010101, 0x01010101};
     const long nsteps = (K + 63) / 64;
-    long step = wave;
-    frag_t cur = load(step < nsteps ? step : 0);
-    for (; step < nsteps; step += SNW) {
-        const frag_t nxt = load(step + SNW < nsteps ? step + SNW : step);
+    // SD of the wavefront's steps are in flight: a launch of a few hundred tiles lasts a handful of memory
+    // latencies, and with one step ahead every step of a wavefront cost one of them
+    constexpr int SD = 4;
+    auto multiply = [&](const frag_t &cur) __attribute__((always_inline)) {
         v4i a[2], w[2];
 #pragma unroll
         for (int i = 0; i < 2; ++i) {
@@ -383,8 +383,25 @@ __global__ void __launch_bounds__(SNW * 64) i8_small_kernel(const problem_t P_, 
             cs[i] = __builtin_amdgcn_mfma_i32_16x16x64_i8(w[i], ones, cs[i], 0, 0, 0); // [e]: column 4 * (lane / 16) + e
             rs[i] = __builtin_amdgcn_mfma_i32_16x16x64_i8(ones, a[i], rs[i], 0, 0, 0); // every e: row lane % 16
         }
-        cur = nxt;
+    };
+    long step = wave;
+    frag_t st[SD];
+#pragma unroll
+    for (int d = 0; d < SD; ++d) {
+        const long sl = step + (long)d * SNW;
+        st[d] = load(sl < nsteps ? sl : 0);
     }
+    for (; step + (long)(SD - 1) * SNW < nsteps; step += (long)SD * SNW) {
+#pragma unroll
+        for (int d = 0; d < SD; ++d) {
+            multiply(st[d]);
+            const long sl = step + (long)(SD + d) * SNW;
+            if (sl < nsteps) st[d] = load(sl); // (uniform over the wavefront)
+        }
+    }
+#pragma unroll
+    for (int d = 0; d < SD; ++d)
+        if (step + (long)d * SNW < nsteps) multiply(st[d]);
 #pragma unroll
     for (int i = 0; i < 2; ++i) {
 #pragma unroll
