@@ -14,6 +14,9 @@
 // The groups' boundaries are cumulative s32 offsets in device memory.  A thread
 // finds its group by bisection; nothing is assumed about the offsets beyond
 // what keeps every access inside the tensors.
+//
+// Further down: "hip:mfma_grouped_k" (the variable-K pattern) and
+// "hip:mfma_grouped" (the variable-M pattern) on the matrix cores.
 #include "kernels.hpp"
 #include <cstdlib>
 #include <cstring>
@@ -142,6 +145,126 @@ __global__ void __launch_bounds__(256) grouped_2dx2d_kernel(const grouped_dev_t 
     for (long k = k0; k < k1; ++k)
         acc += load_float(D.src_dt, P.a.src, m + k * M) * load_float(D.wei_dt, P.a.wei, k * N + n);
     store_float(D.dst_dt, acc, P.a.dst, g * D.dst_stride[0] + m * D.dst_stride[1] + n * D.dst_stride[2]);
+}
+
+// ---- "hip:mfma_grouped_k" -- the variable-K pattern (the weights' gradient of
+// a mixture-of-experts layer: dst[g] = src[:, k0:k1] x wei[k0:k1, :]) on the
+// matrix cores.
+//
+// Both operands arrive with K outermost -- src as [total_K][M], weights as
+// [total_K][N] -- the opposite of what the 16-bit matrix instructions want (a
+// lane's elements consecutive along K).  v_mfma_f32_16x16x4_f32 takes ONE
+// element per lane and operand, lane (i, q) supplying row (column) i at k = q,
+// so the operands go from global memory to the instruction with no transpose at
+// all: a lane loads the four consecutive rows 4 i .. 4 i + 3 of k = q in one
+// instruction (16 bytes of f32, 8 of bf16 / f16, widened in registers) and each
+// of the four values feeds a different fragment.  Fragment r therefore holds the
+// rows 4 i + r of a wavefront's 64, and fragment c of the weights the columns
+// 4 j + c: in the 16 accumulators lane (j, q) finds, for each of its rows, the
+// columns 4 j .. 4 j + 3 side by side, which is one 16-byte store.  The work is
+// bound by dst (G x M x N elements written against (M + N) x total_K read) and
+// the f32 rate of the matrix cores is enough for that.
+//
+// A workgroup of four wavefronts owns 128 x 128 of one group's dst (64 x 64 a
+// wavefront) and walks the group's k range four at a time, DEPTH steps in
+// flight.  A dst stored with rows contiguous ("acb") is the same problem with
+// the operands exchanged, which the launch does.
+struct grouped_k_dev_t {
+    const void *a, *b;           // [total][MA] and [total][NB]
+    const int32_t *offsets;      // cumulative k per group
+    void *dst;
+    long MA, NB, total;
+    long dst_g, dst_ld;          // element strides of dst: group, row of A
+    int tiles_n;
+};
+
+template <int DT>
+__device__ __forceinline__ void gk_load(const void *base, long elem, bool ok, float (&out)[4]) {
+    if (DT == MI355_DT_F32) {
+        typedef float f4 __attribute__((ext_vector_type(4)));
+        f4 v = {0.f, 0.f, 0.f, 0.f};
+        if (ok) v = *(const f4 *)((const float *)base + elem);
+        out[0] = v.x, out[1] = v.y, out[2] = v.z, out[3] = v.w;
+    } else if (DT == MI355_DT_BF16) {
+        typedef unsigned u2 __attribute__((ext_vector_type(2)));
+        u2 v = {0u, 0u};
+        if (ok) v = *(const u2 *)((const uint16_t *)base + elem);
+        out[0] = u2f(v.x << 16), out[1] = u2f(v.x & 0xffff0000u);
+        out[2] = u2f(v.y << 16), out[3] = u2f(v.y & 0xffff0000u);
+    } else {
+        typedef _Float16 h4 __attribute__((ext_vector_type(4)));
+        h4 v = {0, 0, 0, 0};
+        if (ok) v = *(const h4 *)((const uint16_t *)base + elem);
+        out[0] = (float)v.x, out[1] = (float)v.y, out[2] = (float)v.z, out[3] = (float)v.w;
+    }
+}
+
+template <int DT>
+__global__ void __launch_bounds__(256) grouped_k_tile_kernel(const grouped_k_dev_t P) {
+    typedef float f4 __attribute__((ext_vector_type(4)));
+    constexpr int DEPTH = 4;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int i = lane & 15, q = lane >> 4;
+    const long g = blockIdx.y;
+    const long m_w = (long)(blockIdx.x / P.tiles_n) * 128 + (wave >> 1) * 64;
+    const long n_w = (long)(blockIdx.x % P.tiles_n) * 128 + (wave & 1) * 64;
+    long k0 = g > 0 ? (long)P.offsets[g - 1] : 0, k1 = P.offsets[g];
+    if (k0 < 0) k0 = 0;
+    if (k1 > P.total) k1 = P.total;
+    // a wavefront whose rows or columns are all outside has nothing to store
+    if (m_w >= P.MA || n_w >= P.NB) return;
+    const bool a_in = m_w + 4 * i < P.MA, b_in = n_w + 4 * i < P.NB; // (MA and NB are multiples of 4)
+
+    f4 acc[4][4];
+#pragma unroll
+    for (int r = 0; r < 4; ++r)
+#pragma unroll
+        for (int c = 0; c < 4; ++c) acc[r][c] = f4 {0.f, 0.f, 0.f, 0.f};
+
+    float av[DEPTH][4], bv[DEPTH][4];
+    auto fetch = [&](int slot, long kb) {
+        const long k = kb + q;
+        const bool ok = k < k1;
+        gk_load<DT>(P.a, k * P.MA + m_w + 4 * i, ok && a_in, av[slot]);
+        gk_load<DT>(P.b, k * P.NB + n_w + 4 * i, ok && b_in, bv[slot]);
+    };
+#pragma unroll
+    for (int s = 0; s < DEPTH; ++s) fetch(s, k0 + 4 * s); // (past the range: zeros, no loads)
+    for (long kb = k0; kb < k1; kb += 4 * DEPTH) {
+#pragma unroll
+        for (int s = 0; s < DEPTH; ++s) {
+            float a[4], b[4];
+#pragma unroll
+            for (int e = 0; e < 4; ++e) a[e] = av[s][e], b[e] = bv[s][e];
+            fetch(s, kb + 4 * (s + DEPTH));
+#pragma unroll
+            for (int r = 0; r < 4; ++r)
+#pragma unroll
+                for (int c = 0; c < 4; ++c)
+                    acc[r][c] = __builtin_amdgcn_mfma_f32_16x16x4f32(a[r], b[c], acc[r][c], 0, 0, 0);
+        }
+    }
+
+    if (!b_in) return;
+    const long col = n_w + 4 * i;
+#pragma unroll
+    for (int r = 0; r < 4; ++r)
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            const long row = m_w + 4 * (4 * q + e) + r;
+            if (row >= P.MA) continue;
+            const long off = g * P.dst_g + row * P.dst_ld + col;
+            const float v0 = acc[r][0][e], v1 = acc[r][1][e], v2 = acc[r][2][e], v3 = acc[r][3][e];
+            if (DT == MI355_DT_F32) {
+                *(f4 *)((float *)P.dst + off) = f4 {v0, v1, v2, v3};
+            } else {
+                typedef unsigned u2 __attribute__((ext_vector_type(2)));
+                u2 o;
+                o.x = (cvt_store_bits(DT, v0) & 0xffffu) | (cvt_store_bits(DT, v1) << 16);
+                o.y = (cvt_store_bits(DT, v2) & 0xffffu) | (cvt_store_bits(DT, v3) << 16);
+                *(u2 *)((uint16_t *)P.dst + off) = o;
+            }
+        }
 }
 
 // ---- "hip:mfma_grouped" -- the 2Dx3D pattern on the matrix cores for fp8,
@@ -950,6 +1073,45 @@ int tile_plan(const mi355_grouped_desc_t &d, bool *mx_out = nullptr) {
     return plan;
 }
 
+// The variable-K pattern on the matrix cores: 0 = no, 1 = dst rows are rows of src ("abc"), 2 = dst rows are
+// columns of the weights ("acb": the operands change places).
+int k_tile_plan(const mi355_grouped_desc_t &d) {
+    if (d.pattern != MI355_GROUPED_2DX2D) return 0;
+    if (tuning(TUNE_GROUPED_IMPL) == TUNE_REF) return 0;
+    if (d.src_dt != MI355_DT_F32 && d.src_dt != MI355_DT_BF16 && d.src_dt != MI355_DT_F16) return 0;
+    // a lane reads four consecutive rows (columns) and stores four consecutive dst elements
+    if (d.M % 4 != 0 || d.N % 4 != 0 || d.dst_stride[0] % 4 != 0) return 0;
+    if (d.group_count > 65535) return 0;
+    if (((d.M + 127) / 128) * ((d.N + 127) / 128) >= (1L << 31)) return 0;
+    if (d.dst_stride[2] == 1 && d.dst_stride[1] >= d.N && d.dst_stride[1] % 4 == 0) return 1;
+    if (d.dst_stride[1] == 1 && d.dst_stride[2] >= d.M && d.dst_stride[2] % 4 == 0) return 2;
+    return 0;
+}
+
+int launch_k_tiles(int plan, const grouped_dev_t &G, hipStream_t stream) {
+    const mi355_grouped_desc_t &d = G.d;
+    grouped_k_dev_t P;
+    const bool swap = plan == 2;
+    P.a = swap ? G.a.wei : G.a.src;
+    P.b = swap ? G.a.src : G.a.wei;
+    P.MA = swap ? d.N : d.M;
+    P.NB = swap ? d.M : d.N;
+    P.offsets = G.a.src_offsets;
+    P.dst = G.a.dst;
+    P.total = d.total;
+    P.dst_g = d.dst_stride[0];
+    P.dst_ld = swap ? d.dst_stride[2] : d.dst_stride[1];
+    P.tiles_n = (int)((P.NB + 127) / 128);
+    const dim3 grid((unsigned)(((P.MA + 127) / 128) * P.tiles_n), (unsigned)d.group_count);
+    if (d.src_dt == MI355_DT_F32)
+        hipLaunchKernelGGL(grouped_k_tile_kernel<MI355_DT_F32>, grid, dim3(256), 0, stream, P);
+    else if (d.src_dt == MI355_DT_BF16)
+        hipLaunchKernelGGL(grouped_k_tile_kernel<MI355_DT_BF16>, grid, dim3(256), 0, stream, P);
+    else
+        hipLaunchKernelGGL(grouped_k_tile_kernel<MI355_DT_F16>, grid, dim3(256), 0, stream, P);
+    return hipGetLastError() == hipSuccess ? MI355_SUCCESS : MI355_RUNTIME_ERROR;
+}
+
 template <int MODE, int FA, int FB>
 int launch_tiles(int plan, const grouped_dev_t &P, hipStream_t stream) {
     const mi355_grouped_desc_t &d = P.d;
@@ -1027,6 +1189,7 @@ extern "C" int mi355_grouped_matmul_query(const mi355_grouped_desc_t *d) {
 
 extern "C" const char *mi355_grouped_matmul_impl(const mi355_grouped_desc_t *d) {
     if (!d || mi355_grouped_matmul_query(d) != MI355_SUCCESS) return "";
+    if (k_tile_plan(*d) != 0) return "hip:mfma_grouped_k";
     return tile_plan(*d) != 0 ? "hip:mfma_grouped" : "hip:ref_grouped:any";
 }
 
@@ -1079,6 +1242,11 @@ extern "C" int mi355_grouped_matmul_launch(const mi355_grouped_desc_t *d, const 
         if (fa && fb) return launch_tiles<GM_F8, 1, 1>(plan, P, s);
         if (fa) return launch_tiles<GM_F8, 1, 0>(plan, P, s);
         return launch_tiles<GM_F8, 0, 1>(plan, P, s);
+    }
+    if (const int kplan = k_tile_plan(*d)) {
+        // (the tiles read and write 16 bytes at a time)
+        if ((uintptr_t)a->src % 16 == 0 && (uintptr_t)a->wei % 16 == 0 && (uintptr_t)a->dst % 16 == 0)
+            return launch_k_tiles(kplan, P, (hipStream_t)stream);
     }
     if (x3)
         hipLaunchKernelGGL(grouped_2dx3d_kernel, dim3((unsigned)blocks), dim3(256), 0, (hipStream_t)stream, P);
