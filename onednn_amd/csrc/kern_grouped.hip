@@ -161,14 +161,24 @@ __global__ void __launch_bounds__(256) grouped_2dx2d_kernel(const grouped_dev_t 
 // of the four values feeds a different fragment.  Fragment r therefore holds the
 // rows 4 i + r of a wavefront's 64, and fragment c of the weights the columns
 // 4 j + c: in the 16 accumulators lane (j, q) finds, for each of its rows, the
-// columns 4 j .. 4 j + 3 side by side, which is one 16-byte store.  The work is
-// bound by dst (G x M x N elements written against (M + N) x total_K read) and
-// the f32 rate of the matrix cores is enough for that.
+// columns 4 j .. 4 j + 3 side by side, which is one 16-byte store.  With the
+// short groups of expert routing the work is bound by dst (G x M x N elements
+// written against (M + N) x total_K read) and the f32 rate of the matrix cores
+// is enough; bf16 / f16 tensors with columns in eights go through LDS to the
+// 16-bit instructions instead (grouped_k_lds_kernel, further down).
 //
 // A workgroup of four wavefronts owns 128 x 128 of one group's dst (64 x 64 a
-// wavefront) and walks the group's k range four at a time, DEPTH steps in
+// wavefront) and walks the group's k range a step at a time, DEPTH steps in
 // flight.  A dst stored with rows contiguous ("acb") is the same problem with
 // the operands exchanged, which the launch does.
+typedef int g4i __attribute__((ext_vector_type(4)));
+typedef int g8i __attribute__((ext_vector_type(8)));
+typedef unsigned g2u __attribute__((ext_vector_type(2)));
+typedef unsigned g4u __attribute__((ext_vector_type(4)));
+typedef float g4f __attribute__((ext_vector_type(4)));
+typedef __bf16 g8bf __attribute__((ext_vector_type(8)));
+typedef _Float16 g8h __attribute__((ext_vector_type(8)));
+
 struct grouped_k_dev_t {
     const void *a, *b;           // [total][MA] and [total][NB]
     const int32_t *offsets;      // cumulative k per group
@@ -178,31 +188,84 @@ struct grouped_k_dev_t {
     int tiles_n;
 };
 
+typedef unsigned gk_u2 __attribute__((ext_vector_type(2)));
+typedef float gk_f4 __attribute__((ext_vector_type(4)));
+
+// What a lane holds of one step (4 k) of one operand of v_mfma_f32_16x16x4_f32: four consecutive rows of
+// k = kb + q, one load of 16 bytes (f32) or 8 (bf16 / f16, widened when the fragment is taken).
 template <int DT>
-__device__ __forceinline__ void gk_load(const void *base, long elem, bool ok, float (&out)[4]) {
-    if (DT == MI355_DT_F32) {
-        typedef float f4 __attribute__((ext_vector_type(4)));
-        f4 v = {0.f, 0.f, 0.f, 0.f};
-        if (ok) v = *(const f4 *)((const float *)base + elem);
-        out[0] = v.x, out[1] = v.y, out[2] = v.z, out[3] = v.w;
-    } else if (DT == MI355_DT_BF16) {
-        typedef unsigned u2 __attribute__((ext_vector_type(2)));
-        u2 v = {0u, 0u};
-        if (ok) v = *(const u2 *)((const uint16_t *)base + elem);
-        out[0] = u2f(v.x << 16), out[1] = u2f(v.x & 0xffff0000u);
-        out[2] = u2f(v.y << 16), out[3] = u2f(v.y & 0xffff0000u);
-    } else {
-        typedef _Float16 h4 __attribute__((ext_vector_type(4)));
-        h4 v = {0, 0, 0, 0};
-        if (ok) v = *(const h4 *)((const uint16_t *)base + elem);
-        out[0] = (float)v.x, out[1] = (float)v.y, out[2] = (float)v.z, out[3] = (float)v.w;
+struct gk_step_t {
+    static constexpr int NRAW = DT == MI355_DT_F32 ? 2 : 1; // 8-byte pieces
+    gk_u2 raw[NRAW];
+
+    __device__ __forceinline__ void load(const void *base, long ld, long kb, long k1, int q, long first, bool in) {
+        const long k = kb + q;
+        if (DT == MI355_DT_F32) {
+            gk_f4 v = {0.f, 0.f, 0.f, 0.f};
+            if (in && k < k1) v = *(const gk_f4 *)((const float *)base + k * ld + first);
+            raw[0] = gk_u2 {f2u(v.x), f2u(v.y)};
+            raw[NRAW - 1] = gk_u2 {f2u(v.z), f2u(v.w)};
+        } else {
+            raw[0] = gk_u2 {0u, 0u};
+            if (in && k < k1) raw[0] = *(const gk_u2 *)((const uint16_t *)base + k * ld + first);
+        }
     }
+    // the element of row (column) 4 i + r
+    __device__ __forceinline__ float frag(int r) const {
+        if (DT == MI355_DT_F32) return u2f(r == 0 ? raw[0].x : r == 1 ? raw[0].y : r == 2 ? raw[NRAW - 1].x : raw[NRAW - 1].y);
+        const unsigned w = (r & 2) ? raw[0].y : raw[0].x;
+        if (DT == MI355_DT_BF16) return u2f((r & 1) ? (w & 0xffff0000u) : (w << 16));
+        typedef _Float16 h2 __attribute__((ext_vector_type(2)));
+        const h2 h = __builtin_bit_cast(h2, w);
+        return (r & 1) ? (float)h.y : (float)h.x;
+    }
+};
+
+// Four rows (columns) of each of eight consecutive k -- raw[t] = rows 4 i .. 4 i + 3 of k = 8 q + t, two to a
+// dword -- into the eight consecutive k of row 4 i + r that v_mfma_f32_16x16x32_{bf16,f16} takes: a 4 x 8
+// transpose inside the lane, 4 v_perm_b32 a fragment.
+__device__ __forceinline__ g4u gk_frag16(const gk_u2 (&raw)[8], int r) {
+    const unsigned sel = (r & 1) ? 0x07060302u : 0x05040100u;
+    g4u o;
+#pragma unroll
+    for (int d = 0; d < 4; ++d) {
+        const unsigned lo = (r & 2) ? raw[2 * d].y : raw[2 * d].x;
+        const unsigned hi = (r & 2) ? raw[2 * d + 1].y : raw[2 * d + 1].x;
+        o[d] = __builtin_amdgcn_perm(hi, lo, sel);
+    }
+    return o;
+}
+
+// lane (j, q) of a wavefront's 64 x 64: acc[r][c][e] is row 4 (4 q + e) + r, column 4 j + c
+template <int DT>
+__device__ __forceinline__ void gk_store(const grouped_k_dev_t &P, const gk_f4 (&acc)[4][4], long g, long m_w, long n_w,
+        int j, int q) {
+    const long col = n_w + 4 * j;
+    if (col >= P.NB) return;
+#pragma unroll
+    for (int r = 0; r < 4; ++r)
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            const long row = m_w + 4 * (4 * q + e) + r;
+            if (row >= P.MA) continue;
+            const long off = g * P.dst_g + row * P.dst_ld + col;
+            const float v0 = acc[r][0][e], v1 = acc[r][1][e], v2 = acc[r][2][e], v3 = acc[r][3][e];
+            if (DT == MI355_DT_F32) {
+                *(gk_f4 *)((float *)P.dst + off) = gk_f4 {v0, v1, v2, v3};
+            } else {
+                gk_u2 o;
+                o.x = (cvt_store_bits(DT, v0) & 0xffffu) | (cvt_store_bits(DT, v1) << 16);
+                o.y = (cvt_store_bits(DT, v2) & 0xffffu) | (cvt_store_bits(DT, v3) << 16);
+                *(gk_u2 *)((uint16_t *)P.dst + off) = o;
+            }
+        }
 }
 
 template <int DT>
 __global__ void __launch_bounds__(256) grouped_k_tile_kernel(const grouped_k_dev_t P) {
-    typedef float f4 __attribute__((ext_vector_type(4)));
-    constexpr int DEPTH = 4;
+    typedef gk_f4 f4;
+    typedef gk_step_t<DT> step_t;
+    constexpr int DEPTH = 4, KSTEP = 4;
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int i = lane & 15, q = lane >> 4;
     const long g = blockIdx.y;
@@ -221,22 +284,20 @@ __global__ void __launch_bounds__(256) grouped_k_tile_kernel(const grouped_k_dev
 #pragma unroll
         for (int c = 0; c < 4; ++c) acc[r][c] = f4 {0.f, 0.f, 0.f, 0.f};
 
-    float av[DEPTH][4], bv[DEPTH][4];
-    auto fetch = [&](int slot, long kb) {
-        const long k = kb + q;
-        const bool ok = k < k1;
-        gk_load<DT>(P.a, k * P.MA + m_w + 4 * i, ok && a_in, av[slot]);
-        gk_load<DT>(P.b, k * P.NB + n_w + 4 * i, ok && b_in, bv[slot]);
+    step_t sa[DEPTH], sb[DEPTH];
+    auto fetch = [&](int slot, long kb) { // (past the range: zeros, no loads)
+        sa[slot].load(P.a, P.MA, kb, k1, q, m_w + 4 * i, a_in);
+        sb[slot].load(P.b, P.NB, kb, k1, q, n_w + 4 * i, b_in);
     };
 #pragma unroll
-    for (int s = 0; s < DEPTH; ++s) fetch(s, k0 + 4 * s); // (past the range: zeros, no loads)
-    for (long kb = k0; kb < k1; kb += 4 * DEPTH) {
+    for (int s = 0; s < DEPTH; ++s) fetch(s, k0 + KSTEP * s);
+    for (long kb = k0; kb < k1; kb += KSTEP * DEPTH) {
 #pragma unroll
         for (int s = 0; s < DEPTH; ++s) {
             float a[4], b[4];
 #pragma unroll
-            for (int e = 0; e < 4; ++e) a[e] = av[s][e], b[e] = bv[s][e];
-            fetch(s, kb + 4 * (s + DEPTH));
+            for (int e = 0; e < 4; ++e) a[e] = sa[s].frag(e), b[e] = sb[s].frag(e);
+            fetch(s, kb + KSTEP * (s + DEPTH));
 #pragma unroll
             for (int r = 0; r < 4; ++r)
 #pragma unroll
@@ -245,26 +306,7 @@ __global__ void __launch_bounds__(256) grouped_k_tile_kernel(const grouped_k_dev
         }
     }
 
-    if (!b_in) return;
-    const long col = n_w + 4 * i;
-#pragma unroll
-    for (int r = 0; r < 4; ++r)
-#pragma unroll
-        for (int e = 0; e < 4; ++e) {
-            const long row = m_w + 4 * (4 * q + e) + r;
-            if (row >= P.MA) continue;
-            const long off = g * P.dst_g + row * P.dst_ld + col;
-            const float v0 = acc[r][0][e], v1 = acc[r][1][e], v2 = acc[r][2][e], v3 = acc[r][3][e];
-            if (DT == MI355_DT_F32) {
-                *(f4 *)((float *)P.dst + off) = f4 {v0, v1, v2, v3};
-            } else {
-                typedef unsigned u2 __attribute__((ext_vector_type(2)));
-                u2 o;
-                o.x = (cvt_store_bits(DT, v0) & 0xffffu) | (cvt_store_bits(DT, v1) << 16);
-                o.y = (cvt_store_bits(DT, v2) & 0xffffu) | (cvt_store_bits(DT, v3) << 16);
-                *(u2 *)((uint16_t *)P.dst + off) = o;
-            }
-        }
+    gk_store<DT>(P, acc, g, m_w, n_w, i, q);
 }
 
 // ---- "hip:mfma_grouped" -- the 2Dx3D pattern on the matrix cores for fp8,
@@ -296,13 +338,6 @@ __global__ void __launch_bounds__(256) grouped_k_tile_kernel(const grouped_k_dev
 // block) in group order.  A workgroup finds its slot by a block-wide prefix
 // sum over the groups' row-block counts (the offsets live on the device); the
 // host sizes the grid by the upper bound total_M / BM + min(G, total_M).
-typedef int g4i __attribute__((ext_vector_type(4)));
-typedef int g8i __attribute__((ext_vector_type(8)));
-typedef unsigned g2u __attribute__((ext_vector_type(2)));
-typedef unsigned g4u __attribute__((ext_vector_type(4)));
-typedef float g4f __attribute__((ext_vector_type(4)));
-typedef __bf16 g8bf __attribute__((ext_vector_type(8)));
-typedef _Float16 g8h __attribute__((ext_vector_type(8)));
 
 enum { GM_F8 = 0, GM_BF16 = 1, GM_F16 = 2, GM_MXF8 = 3, GM_MXF4 = 4, GM_I8 = 5 };
 // GM_I8: s8 x s8, the sums are s32 (kept in the accumulator registers' bits and added as integers wherever
@@ -762,6 +797,106 @@ __device__ __forceinline__ void grouped_dma16(const void *sbase, unsigned voff, 
                  : "memory", "m0");
 }
 
+// ---- the variable-K pattern, long groups of bf16 / f16: the operands of a 128 x 128 tile go through LDS.
+//
+// Per step of 32 k the workgroup needs 32 rows of 256 bytes of each operand.  They are fetched by direct-to-LDS
+// instructions (a wavefront's instruction brings four rows, 1 KB; no registers are held while a stage is in
+// flight, so NST - 1 stages are), once per workgroup instead of once per wavefront.  A block of four rows takes
+// GK_BLOCK = 1024 + 64 bytes of LDS: lane (i, q) reads row 8 q + t, bytes 8 i .. 8 i + 7 of its wavefront's half,
+// and two blocks further on (q + 1) is 128 bytes further on in the banks, so the four q of a read share the 64
+// banks two by two, which is what 512 bytes cost anyway.  gk_frag16 transposes inside the lane.
+// Rows past the group's end are fetched from its last row (any valid address) and the lanes clear their
+// fragments' k slots past the end on both operands; columns past the tensors' edge are fetched from column 0 of
+// the tile and only reach accumulators that are not stored.
+constexpr int GK_NST = 4, GK_BLOCK = 1024 + 64, GK_OPERAND = 8 * GK_BLOCK, GK_STAGE = 2 * GK_OPERAND;
+
+template <int DT>
+__global__ void __launch_bounds__(256) grouped_k_lds_kernel(const grouped_k_dev_t P) {
+    typedef gk_f4 f4;
+    extern __shared__ __attribute__((aligned(16))) unsigned char gk_smem[];
+    const unsigned lds0 = (unsigned)(uintptr_t)gk_smem;
+    const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int i = lane & 15, q = lane >> 4;
+    const long g = blockIdx.y;
+    const long m_t = (long)(blockIdx.x / P.tiles_n) * 128, n_t = (long)(blockIdx.x % P.tiles_n) * 128;
+    const long m_w = m_t + (wave >> 1) * 64, n_w = n_t + (wave & 1) * 64;
+    long k0 = g > 0 ? (long)P.offsets[g - 1] : 0, k1 = P.offsets[g];
+    if (k0 < 0) k0 = 0;
+    if (k1 > P.total) k1 = P.total;
+
+    f4 acc[4][4];
+#pragma unroll
+    for (int r = 0; r < 4; ++r)
+#pragma unroll
+        for (int c = 0; c < 4; ++c) acc[r][c] = f4 {0.f, 0.f, 0.f, 0.f};
+
+    if (k0 < k1) {
+        // this lane's part of a block: row lane / 16 of its four, the 16 bytes of columns 8 (lane % 16) ..
+        const long ca = m_t + 8 * i < P.MA ? 8 * i : 0, cb = n_t + 8 * i < P.NB ? 8 * i : 0;
+        const unsigned char *abase = (const unsigned char *)P.a + (k0 * P.MA + m_t) * 2;
+        const unsigned char *bbase = (const unsigned char *)P.b + (k0 * P.NB + n_t) * 2;
+        const long last = k1 - 1 - k0;
+        auto issue = [&](long step) {
+            const unsigned slot = lds0 + (unsigned)(step % GK_NST) * GK_STAGE;
+#pragma unroll
+            for (int h = 0; h < 2; ++h) {
+                const int blk = 2 * wave + h;
+                long row = step * 32 + 4 * blk + q;
+                row = row < last ? row : last;
+                grouped_dma16(abase, (unsigned)((row * P.MA + ca) * 2), slot + blk * GK_BLOCK);
+                grouped_dma16(bbase, (unsigned)((row * P.NB + cb) * 2), slot + GK_OPERAND + blk * GK_BLOCK);
+            }
+        };
+        const long nsteps = (k1 - k0 + 31) / 32;
+#pragma unroll
+        for (int s = 0; s < GK_NST - 1; ++s) issue(s);
+        const unsigned a_rd = (unsigned)(2 * q * GK_BLOCK + ((wave >> 1) * 64 + 4 * i) * 2);
+        const unsigned b_rd = (unsigned)(GK_OPERAND + 2 * q * GK_BLOCK + ((wave & 1) * 64 + 4 * i) * 2);
+        for (long step = 0; step < nsteps; ++step) {
+            // this wavefront's part of the stage has landed; after the barrier everyone's has, and
+            // everyone is done reading the stage that the next instructions overwrite
+            asm volatile("s_waitcnt vmcnt(%0)" ::"n"(4 * (GK_NST - 2)) : "memory");
+            __syncthreads();
+            issue(step + GK_NST - 1);
+            const unsigned slot = (unsigned)(step % GK_NST) * GK_STAGE;
+            gk_u2 ra[8], rb[8];
+#pragma unroll
+            for (int t = 0; t < 8; ++t) {
+                const unsigned off = slot + (t >> 2) * GK_BLOCK + (t & 3) * 256;
+                ra[t] = *(const gk_u2 *)(gk_smem + a_rd + off);
+                rb[t] = *(const gk_u2 *)(gk_smem + b_rd + off);
+            }
+            g4u a[4], b[4];
+#pragma unroll
+            for (int e = 0; e < 4; ++e) a[e] = gk_frag16(ra, e), b[e] = gk_frag16(rb, e);
+            const long left = k1 - k0 - step * 32 - 8 * q; // k slots of this lane inside the group
+            if (step == nsteps - 1 && (k1 - k0) % 32 != 0) {
+#pragma unroll
+                for (int d = 0; d < 4; ++d) {
+                    const unsigned keep = left >= 2 * d + 2 ? 0xffffffffu : (left == 2 * d + 1 ? 0xffffu : 0u);
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) a[e][d] &= keep, b[e][d] &= keep;
+                }
+            }
+#pragma unroll
+            for (int r = 0; r < 4; ++r)
+#pragma unroll
+                for (int c = 0; c < 4; ++c) {
+                    if (DT == MI355_DT_BF16)
+                        acc[r][c] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(g8bf, a[r]),
+                                __builtin_bit_cast(g8bf, b[c]), acc[r][c], 0, 0, 0);
+                    else
+                        acc[r][c] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(g8h, a[r]),
+                                __builtin_bit_cast(g8h, b[c]), acc[r][c], 0, 0, 0);
+                }
+        }
+        // (the stages still in flight were fetched for nothing; they must land before the LDS is given back)
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    }
+    if (m_w >= P.MA || n_w >= P.NB) return;
+    gk_store<DT>(P, acc, g, m_w, n_w, i, q);
+}
+
 // NT: fragments of 16 columns per wavefront.  Leaves the wavefront's MF x NT accumulators in LDS at
 // lds0 + (wave * MF * NT + unit) * 1024.
 template <int MODE, int FA, int FB, int MF, int NT, int D>
@@ -1103,6 +1238,21 @@ int launch_k_tiles(int plan, const grouped_dev_t &G, hipStream_t stream) {
     P.dst_ld = swap ? d.dst_stride[2] : d.dst_stride[1];
     P.tiles_n = (int)((P.NB + 127) / 128);
     const dim3 grid((unsigned)(((P.MA + 127) / 128) * P.tiles_n), (unsigned)d.group_count);
+    // bf16 / f16 through LDS and the 16-bit instructions (measured faster at every group length) where columns
+    // can be fetched eight at a time and 32-bit offsets reach across a group; otherwise the f32 instruction
+    const bool h16 = d.src_dt != MI355_DT_F32;
+    bool lds_path = h16 && P.MA % 8 == 0 && P.NB % 8 == 0 && d.total * (P.MA > P.NB ? P.MA : P.NB) * 2 < (1L << 32);
+    if (tuning(TUNE_GROUPED_IMPL) == TUNE_SHORT) lds_path = false;
+    if (lds_path) {
+        constexpr int lds = GK_NST * GK_STAGE;
+        auto launch = [&](auto kern) {
+            if (const int st = ensure_dynamic_lds((const void *)kern, lds, "mfma_grouped_k")) return st;
+            hipLaunchKernelGGL(kern, grid, dim3(256), lds, stream, P);
+            return hipGetLastError() == hipSuccess ? (int)MI355_SUCCESS : (int)MI355_RUNTIME_ERROR;
+        };
+        return d.src_dt == MI355_DT_BF16 ? launch(grouped_k_lds_kernel<MI355_DT_BF16>)
+                                         : launch(grouped_k_lds_kernel<MI355_DT_F16>);
+    }
     if (d.src_dt == MI355_DT_F32)
         hipLaunchKernelGGL(grouped_k_tile_kernel<MI355_DT_F32>, grid, dim3(256), 0, stream, P);
     else if (d.src_dt == MI355_DT_BF16)

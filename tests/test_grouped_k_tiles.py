@@ -35,7 +35,17 @@ SHAPES = [
     ([1, 2, 3, 4, 5, 17, 64, 0, 33], 64, 128),
     ([40, 1], 260, 136),                  # 3 x 2 tiles a group
     ([5] * 70, 16, 20),
+    ([0, 31, 7], 136, 72),                # (columns in eights: the LDS variant's shapes)
+    ([40, 1, 100, 32, 65], 264, 136),
 ]
+
+
+@pytest.fixture(params=["short", "auto"])
+def variant(request):
+    """"short" keeps bf16 / f16 on the f32 instruction too; otherwise shapes with columns in eights go through LDS
+    to the 16-bit instructions."""
+    with cabi.tuning("MI355_GROUPED_IMPL", None if request.param == "auto" else request.param):
+        yield request.param
 
 
 def impl_of(p):
@@ -61,7 +71,7 @@ def test_dispatch_rules():
 @pytest.mark.parametrize("shape", SHAPES, ids=lambda s: f"G{len(s[0])}x{sum(s[0])}x{s[1]}x{s[2]}")
 @pytest.mark.parametrize("dt", [F32, BF16, F16], ids=["f32", "bf16", "f16"])
 @pytest.mark.parametrize("dtag", ["abc", "acb"])
-def test_exact_data_matches_the_oracle(gpu, oracle, shape, dt, dtag):
+def test_exact_data_matches_the_oracle(gpu, oracle, variant, shape, dt, dtag):
     from onednn_amd import grouped
     sizes, M, N = shape
     p, want = gc.case_2dx2d(sizes, M, N, dt=dt, dtag=dtag)
@@ -70,7 +80,8 @@ def test_exact_data_matches_the_oracle(gpu, oracle, shape, dt, dtag):
     assert st == cabi.SUCCESS
     got = grouped.run_gpu(p)
     assert np.array_equal(got, ref), p.name
-    assert np.array_equal(gc.logical_dst(p, got), want)
+    if np.abs(want).max() <= {F32: 2.0 ** 24, BF16: 2.0 ** 8, F16: 2.0 ** 11}[dt]:   # (dst holds the sums exactly)
+        assert np.array_equal(gc.logical_dst(p, got), want)
 
 
 def random_case(sizes, M, N, dt, dtag, seed):
@@ -99,9 +110,9 @@ def random_case(sizes, M, N, dt, dtag, seed):
 @pytest.mark.gpu
 @pytest.mark.parametrize("dt", [F32, BF16, F16], ids=["f32", "bf16", "f16"])
 @pytest.mark.parametrize("dtag", ["abc", "acb"])
-def test_random_data_within_the_derived_bound(gpu, dt, dtag):
+def test_random_data_within_the_derived_bound(gpu, variant, dt, dtag):
     from onednn_amd import grouped
-    p, want, tol = random_case([33, 0, 5, 64, 17, 1, 90, 2, 300], 196, 264, dt, dtag, seed=31)
+    p, want, tol = random_case([33, 0, 5, 64, 17, 1, 90, 2, 300], 200, 264, dt, dtag, seed=31)
     assert impl_of(p) == "hip:mfma_grouped_k"
     got = gc.logical_dst(p, grouped.run_gpu(p))
     err = np.abs(got - want)
@@ -111,7 +122,7 @@ def test_random_data_within_the_derived_bound(gpu, dt, dtag):
 
 
 @pytest.mark.gpu
-def test_weights_gradient_shape_at_full_size_against_the_reference_order_kernel(gpu):
+def test_weights_gradient_shape_at_full_size_against_the_reference_order_kernel(gpu, variant):
     """32 experts, 2048 tokens routed unevenly, hidden 2048 x intermediate 1024 in bf16: every dst element of the
     tiles against the thread-per-element kernel within the bound."""
     from onednn_amd import grouped
