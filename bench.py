@@ -63,6 +63,7 @@ PROFILE_OF = {
     ("g3", "any"): "grouped_tile_kernel_g3_deepseek_v3_decode.md",
     ("g4", "any"): "grouped_nsplit_kernel_g4_deepseek_v3_prefill_mxfp8.md",
     ("g5", "any"): "grouped_nsplit_kernel_g5_deepseek_v3_prefill_mxfp4.md",
+    ("g6", "any"): "grouped_k_lds_kernel_g6_llama4_scout_weights_gradient.md",
 }
 
 
@@ -347,7 +348,7 @@ def run_reorder_workloads(lib, steps, which=("r1", "r2", "r3")):
     return out
 
 
-def run_grouped_workloads(lib, steps, which=("g1", "g2", "g3", "g4", "g5")):
+def run_grouped_workloads(lib, steps, which=("g1", "g2", "g3", "g4", "g5", "g6")):
     """The grouped (mixture-of-experts) matmul on shapes of the reference's
     shapes_grouped_moe files: fp8 e4m3 operands, a scale per src row and per
     group and column, bf16 dst.  HBM-bound: the weights of every group with
@@ -360,7 +361,7 @@ def run_grouped_workloads(lib, steps, which=("g1", "g2", "g3", "g4", "g5")):
     timer = Timer(lib)
     for key in which:
         t0 = time.time()
-        p = configs.grouped_config(key)
+        p = configs.grouped_k_config() if key == "g6" else configs.grouped_config(key)
         d = p.desc()
         cabi.check(lib.mi355_grouped_matmul_query(C.byref(d)))
         copies = 1 if p.wei.nbytes > (1 << 30) else 3
@@ -395,7 +396,7 @@ def run_grouped_workloads(lib, steps, which=("g1", "g2", "g3", "g4", "g5")):
         impl = lib.mi355_grouped_matmul_impl(C.byref(d)).decode()
         out.append({"workload": p.name, "impl": impl, "ms_per_step": ms, "value": gbs, "unit": "GB/s", "bound": "hbm",
                     "peak": PEAK_HBM_GBS, "frac_of_peak": gbs / PEAK_HBM_GBS, "work": nbytes,
-                    "tflops": 2.0 * p.total * p.K * p.N / (ms * 1e-3) / 1e12})
+                    "tflops": 2.0 * p.total * (p.M if key == "g6" else p.K) * p.N / (ms * 1e-3) / 1e12})
         log(f"[bench] {p.name}: {ms:.4f} ms -> {gbs:.1f} GB/s ({100 * gbs / PEAK_HBM_GBS:.1f}% of hbm peak) via {impl}")
         for b in bufs:
             b.free()
@@ -406,8 +407,8 @@ def grouped_cpu_baseline(name):
     """The oracle's restatement of ref_grouped_t on the first groups and columns of the workload."""
     from oracle import binding as oracle
     from onednn_amd import configs
-    groups, N = {"g1": (16, 256), "g2": (2, 256), "g3": (64, 256), "g4": (16, 256), "g5": (16, 256)}[name]
-    p = configs.grouped_config(name, groups=groups, N=N)
+    groups, N = {"g1": (16, 256), "g2": (2, 256), "g3": (64, 256), "g4": (16, 256), "g5": (16, 256), "g6": (2, 256)}[name]
+    p = configs.grouped_k_config(groups=groups, M=1024, N=N) if name == "g6" else configs.grouped_config(name, groups=groups, N=N)
     oracle.load()
     reps, t0 = 0, time.time()
     while True:
@@ -419,7 +420,8 @@ def grouped_cpu_baseline(name):
             break
     from onednn_amd import configs as cf
     return {"value": cf.grouped_bytes(p) * reps / dt / 1e9, "unit": "GB/s", "cores": 1, "kind": "port",
-            "sample": f"the first {groups} groups and {N} columns of the workload ({p.total} rows); {reps} pass(es), "
+            "sample": f"the first {groups} groups and {N} columns of the workload ({p.total} rows"
+                      f"{' along K, 1024 rows of dst' if name == 'g6' else ''}); {reps} pass(es), "
                       f"{dt:.2f} s wall; oracle/liboracle.so, oracle_grouped_matmul (plain C restatement of "
                       "ref_grouped_t, one thread)"}
 
@@ -484,11 +486,11 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=3)
-    ap.add_argument("--workload", default="c3", choices=["c1", "c2", "c3", "c4", "c5", "m1", "h1", "h2", "r1", "r2", "r3", "g1", "g2", "g3", "g4", "g5"],
+    ap.add_argument("--workload", default="c3", choices=["c1", "c2", "c3", "c4", "c5", "m1", "h1", "h2", "r1", "r2", "r3", "g1", "g2", "g3", "g4", "g5", "g6"],
                     help="c1..c5: the matmul configurations (c3 is the headline); r1..r3: the reorder "
-                         "primitive on the headline shape's tensors; g1..g5: the grouped (mixture-of-experts) "
+                         "primitive on the headline shape's tensors; g1..g6: the grouped (mixture-of-experts) "
                          "matmul on shapes of the reference's shapes_grouped_moe files: fp8 with row / column scales "
-                         "(g1..g3), MXFP8 (g4), MXFP4 (g5) (informational)")
+                         "(g1..g3), MXFP8 (g4), MXFP4 (g5), and the variable-K pattern in bf16 (g6) (informational)")
     ap.add_argument("--decode-m", type=int, default=1, help="M of the c2 decode workload")
     ap.add_argument("--wtag", default="any", choices=["any", "ab", "ba"],
                     help="weights layout; any = what format_tag::any resolves to (default)")
@@ -699,15 +701,15 @@ def main():
                          "kernel": r["impl"], "kernel_ms": r["ms_per_step"]},
             "cpu_baseline": None, "others": []}), flush=True)
         return
-    if main_name in ("g1", "g2", "g3", "g4", "g5"):
+    if main_name in ("g1", "g2", "g3", "g4", "g5", "g6"):
         r = run_grouped_workloads(lib, args.steps, (main_name,))[0]
         if args.calib_copy:
             calib_copy()
         cpu = None if args.no_cpu else grouped_cpu_baseline(main_name)
         print(json.dumps({
-            "metric": "grouped %s matmul GB/s" % {"g4": "MXFP8", "g5": "MXFP4"}.get(main_name, "fp8"), "value": r["value"], "unit": "GB/s", "n_gpus": 1, "steps": args.steps,
+            "metric": "grouped %s matmul GB/s" % {"g4": "MXFP8", "g5": "MXFP4", "g6": "bf16 variable-K"}.get(main_name, "fp8"), "value": r["value"], "unit": "GB/s", "n_gpus": 1, "steps": args.steps,
             "warmup": args.warmup, "ms_per_step": r["ms_per_step"], "higher_is_better": True, "scaling": "weak",
-            "vs_baseline": None, "dtype": "f4_e2m1" if main_name == "g5" else "f8_e4m3", "data": "synthetic",
+            "vs_baseline": None, "dtype": {"g5": "f4_e2m1", "g6": "bf16"}.get(main_name, "f8_e4m3"), "data": "synthetic",
             "config": {"workload": r["workload"], "impl": r["impl"], "tflops": r["tflops"]},
             "roofline": {"bound": "hbm", "achieved": r["value"], "peak": PEAK_HBM_GBS, "unit": "GB/s",
                          "frac": r["frac_of_peak"], "traffic": measured_traffic(main_name)[0],

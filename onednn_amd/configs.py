@@ -312,9 +312,29 @@ def grouped_config(name, seed=9, groups=None, N=None):
                           name=f"{name.upper()} {label} {total}x{K}:{G}x{K}x{N}")
 
 
+def grouped_k_config(seed=9, groups=None, M=None, N=None):
+    """g6: the weights' gradient of g2's layer -- the variable-K pattern (the reference's shapes_grouped_2dby2d hold
+    test sizes only): src [M = 5120][total_K = 512 tokens] column-major, weights [512][N = 8192], both bf16 and
+    grouped along K by g2's routing, dst [16][5120][8192] bf16."""
+    from .grouped import GroupedProblem
+    _, m_full, n_full, sizes = GROUPED_SHAPES["g2"]
+    sizes = list(sizes[:groups] if groups else sizes)
+    M, N = M or m_full, N or n_full
+    total = int(sum(sizes))
+    rng = _rng(seed, 2)
+    src = dtp.f32_to_bf16(rng.standard_normal(total * M).astype(np.float32)).reshape(total, M)
+    wei = dtp.f32_to_bf16(rng.standard_normal(total * N).astype(np.float32)).reshape(total, N)
+    return GroupedProblem(pattern=cabi.GROUPED_2DX2D, sizes=sizes, M=M, N=N, src_dt=cabi.DT_BF16, wei_dt=cabi.DT_BF16,
+                          dst_dt=cabi.DT_BF16, src=src, wei=wei, dst_stride=(M * N, N, 1),
+                          name=f"G6 Llama4-Scout-gate/up-proj-weights-gradient {M}x{total}:{total}x{N} -> {len(sizes)}x{M}x{N}")
+
+
 def grouped_bytes(p):
     """Algorithmic HBM bytes of a grouped launch: the weights (and their scales) of every group that has rows, src,
     dst, src scales and offsets, each once."""
+    if p.pattern == cabi.GROUPED_2DX2D:
+        eb = cabi.DT_BITS[p.src_dt] // 8
+        return (p.total * (p.M + p.N) + p.G * p.M * p.N) * eb + 8 * p.G
     active = sum(1 for m in p.sizes if m)
     ebits = cabi.DT_BITS[p.wei_dt]
     total = active * p.K * p.N * ebits // 8 + p.total * p.K * ebits // 8 + p.total * p.N * cabi.DT_BITS[p.dst_dt] // 8

@@ -808,9 +808,11 @@ __device__ __forceinline__ void grouped_dma16(const void *sbase, unsigned voff, 
 // Rows past the group's end are fetched from its last row (any valid address) and the lanes clear their
 // fragments' k slots past the end on both operands; columns past the tensors' edge are fetched from column 0 of
 // the tile and only reach accumulators that are not stored.
-constexpr int GK_NST = 4, GK_BLOCK = 1024 + 64, GK_OPERAND = 8 * GK_BLOCK, GK_STAGE = 2 * GK_OPERAND;
+// NST stages: 4 for long groups; 2 where the groups are a step or two (three workgroups fit a compute unit then,
+// and what a workgroup waits for is the latency of its only fetch).
+constexpr int GK_BLOCK = 1024 + 64, GK_OPERAND = 8 * GK_BLOCK, GK_STAGE = 2 * GK_OPERAND;
 
-template <int DT>
+template <int DT, int GK_NST>
 __global__ void __launch_bounds__(256) grouped_k_lds_kernel(const grouped_k_dev_t P) {
     typedef gk_f4 f4;
     extern __shared__ __attribute__((aligned(16))) unsigned char gk_smem[];
@@ -849,15 +851,21 @@ __global__ void __launch_bounds__(256) grouped_k_lds_kernel(const grouped_k_dev_
         };
         const long nsteps = (k1 - k0 + 31) / 32;
 #pragma unroll
-        for (int s = 0; s < GK_NST - 1; ++s) issue(s);
+        for (int s = 0; s < GK_NST - 1; ++s)
+            if (s < nsteps) issue(s);
         const unsigned a_rd = (unsigned)(2 * q * GK_BLOCK + ((wave >> 1) * 64 + 4 * i) * 2);
         const unsigned b_rd = (unsigned)(GK_OPERAND + 2 * q * GK_BLOCK + ((wave & 1) * 64 + 4 * i) * 2);
         for (long step = 0; step < nsteps; ++step) {
             // this wavefront's part of the stage has landed; after the barrier everyone's has, and
             // everyone is done reading the stage that the next instructions overwrite
-            asm volatile("s_waitcnt vmcnt(%0)" ::"n"(4 * (GK_NST - 2)) : "memory");
+            // (four instructions a stage and wavefront; stages past the group's end are not fetched, so
+            // towards the end fewer are behind this one)
+            const long behind = nsteps - step - 1;
+            if (behind >= GK_NST - 2) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(4 * (GK_NST - 2)) : "memory");
+            else if (behind == 1) asm volatile("s_waitcnt vmcnt(4)" ::: "memory");
+            else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
             __syncthreads();
-            issue(step + GK_NST - 1);
+            if (step + GK_NST - 1 < nsteps) issue(step + GK_NST - 1);
             const unsigned slot = (unsigned)(step % GK_NST) * GK_STAGE;
             gk_u2 ra[8], rb[8];
 #pragma unroll
@@ -890,8 +898,6 @@ __global__ void __launch_bounds__(256) grouped_k_lds_kernel(const grouped_k_dev_
                                 __builtin_bit_cast(g8h, b[c]), acc[r][c], 0, 0, 0);
                 }
         }
-        // (the stages still in flight were fetched for nothing; they must land before the LDS is given back)
-        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     }
     if (m_w >= P.MA || n_w >= P.NB) return;
     gk_store<DT>(P, acc, g, m_w, n_w, i, q);
@@ -1244,14 +1250,16 @@ int launch_k_tiles(int plan, const grouped_dev_t &G, hipStream_t stream) {
     bool lds_path = h16 && P.MA % 8 == 0 && P.NB % 8 == 0 && d.total * (P.MA > P.NB ? P.MA : P.NB) * 2 < (1L << 32);
     if (tuning(TUNE_GROUPED_IMPL) == TUNE_SHORT) lds_path = false;
     if (lds_path) {
-        constexpr int lds = GK_NST * GK_STAGE;
-        auto launch = [&](auto kern) {
+        const bool brief = d.total <= 48 * d.group_count; // (k per group on average)
+        auto launch = [&](auto kern, int nst) {
+            const int lds = nst * GK_STAGE;
             if (const int st = ensure_dynamic_lds((const void *)kern, lds, "mfma_grouped_k")) return st;
             hipLaunchKernelGGL(kern, grid, dim3(256), lds, stream, P);
             return hipGetLastError() == hipSuccess ? (int)MI355_SUCCESS : (int)MI355_RUNTIME_ERROR;
         };
-        return d.src_dt == MI355_DT_BF16 ? launch(grouped_k_lds_kernel<MI355_DT_BF16>)
-                                         : launch(grouped_k_lds_kernel<MI355_DT_F16>);
+        if (d.src_dt == MI355_DT_BF16)
+            return brief ? launch(grouped_k_lds_kernel<MI355_DT_BF16, 2>, 2) : launch(grouped_k_lds_kernel<MI355_DT_BF16, 4>, 4);
+        return brief ? launch(grouped_k_lds_kernel<MI355_DT_F16, 2>, 2) : launch(grouped_k_lds_kernel<MI355_DT_F16, 4>, 4);
     }
     if (d.src_dt == MI355_DT_F32)
         hipLaunchKernelGGL(grouped_k_tile_kernel<MI355_DT_F32>, grid, dim3(256), 0, stream, P);
