@@ -302,6 +302,21 @@ int mi355_event_elapsed_ms(float *ms, void *start, void *stop);
 /* work enqueued on `stream` after this call starts when `event` has completed
  * (the in-order guarantee of a stream, extended across two streams) */
 int mi355_stream_wait_event(void *stream, void *event);
+/* HIP graphs for launch-bound loops (a decode step is a few microseconds of
+ * kernel behind a few microseconds of launch): every *_launch of this library
+ * enqueues kernels only -- no allocation, no memset, no copy, nothing read
+ * back -- so a stream that is being captured records it.  No counterpart in
+ * the reference (its SYCL runtimes leave this to the SYCL graph extension).
+ *   mi355_graph_capture_begin(stream)          stream: created, not NULL
+ *   ... launches on `stream` (none of them runs) ...
+ *   mi355_graph_capture_end(stream, &graph)    the instantiated graph
+ *   mi355_graph_launch(graph, stream)          all recorded launches, in order
+ * A launch's first call on a process may set a kernel attribute (dynamic LDS
+ * size): run each distinct launch once outside the capture first. */
+int mi355_graph_capture_begin(void *stream);
+int mi355_graph_capture_end(void *stream, void **graph);
+int mi355_graph_launch(void *graph, void *stream);
+int mi355_graph_destroy(void *graph);
 /* writes the low `nbytes` (1, 2, 4 or 8) of `bits` to device memory in stream
  * order, without a host copy: the value travels as a kernel argument, so the
  * call never waits for the stream (a host-side scalar of the attributes) */

@@ -149,6 +149,7 @@ KERNEL_SYMBOLS = [
     "mi355_stream_create", "mi355_stream_destroy", "mi355_stream_sync", "mi355_event_create",
     "mi355_event_destroy", "mi355_event_record", "mi355_event_sync", "mi355_event_elapsed_ms",
     "mi355_stream_wait_event", "mi355_mem_store_scalar",
+    "mi355_graph_capture_begin", "mi355_graph_capture_end", "mi355_graph_launch", "mi355_graph_destroy",
     "mi355_last_error", "mi355_matmul_query", "mi355_matmul_impl_name",
     "mi355_matmul_scratch_bytes", "mi355_matmul_launch", "mi355_matmul_launch_noalloc", "mi355_reorder_query",
     "mi355_reorder_launch", "mi355_wei_pack_reorder_dims", "mi355_tuning_set", "mi355_colsum_launch", "mi355_sdpa_softmax_launch",
@@ -204,6 +205,10 @@ def load_kernels():
     lib.mi355_event_sync.argtypes = [vp]
     lib.mi355_event_elapsed_ms.argtypes = [C.POINTER(C.c_float), vp, vp]
     lib.mi355_stream_wait_event.argtypes = [vp, vp]
+    lib.mi355_graph_capture_begin.argtypes = [vp]
+    lib.mi355_graph_capture_end.argtypes = [vp, C.POINTER(vp)]
+    lib.mi355_graph_launch.argtypes = [vp, vp]
+    lib.mi355_graph_destroy.argtypes = [vp]
     lib.mi355_mem_store_scalar.argtypes = [vp, C.c_uint64, C.c_int, vp]
     lib.mi355_matmul_query.argtypes = [C.POINTER(MatmulDesc), C.c_int, C.POINTER(C.c_int)]
     lib.mi355_matmul_scratch_bytes.argtypes = [C.POINTER(MatmulDesc), C.POINTER(C.c_size_t)]
@@ -233,6 +238,51 @@ def gpu_available():
         return False
     n = C.c_int(0)
     return lib.mi355_device_count(C.byref(n)) == SUCCESS and n.value > 0
+
+
+class Stream:
+    """A created (non-default) stream."""
+
+    def __init__(self):
+        self.lib = load_kernels()
+        p = C.c_void_p()
+        check(self.lib.mi355_stream_create(C.byref(p)))
+        self.ptr = p.value
+
+    def sync(self):
+        check(self.lib.mi355_stream_sync(self.ptr))
+
+    def destroy(self):
+        if self.ptr:
+            self.lib.mi355_stream_destroy(self.ptr)
+            self.ptr = None
+
+
+class Graph:
+    """with Graph(stream) as g: <launches on stream>  -- records them; g.launch() replays them in order."""
+
+    def __init__(self, stream):
+        self.lib, self.stream, self.exec = load_kernels(), stream, None
+
+    def __enter__(self):
+        check(self.lib.mi355_graph_capture_begin(self.stream.ptr))
+        return self
+
+    def __exit__(self, *exc):
+        p = C.c_void_p()
+        st = self.lib.mi355_graph_capture_end(self.stream.ptr, C.byref(p))
+        if exc[0] is None:
+            check(st)
+        self.exec = p.value
+        return False
+
+    def launch(self):
+        check(self.lib.mi355_graph_launch(self.exec, self.stream.ptr))
+
+    def destroy(self):
+        if self.exec:
+            self.lib.mi355_graph_destroy(self.exec)
+            self.exec = None
 
 
 class DeviceBuffer:

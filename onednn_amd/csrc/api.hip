@@ -427,6 +427,34 @@ int mi355_stream_destroy(void *stream) {
     if (!stream) return MI355_SUCCESS;
     return hip_status(hipStreamDestroy((hipStream_t)stream), "hipStreamDestroy");
 }
+int mi355_graph_capture_begin(void *stream) {
+    if (!stream) {
+        set_error("graph capture needs a created stream");
+        return MI355_INVALID_ARGUMENTS;
+    }
+    // (thread-local: what other host threads call meanwhile does not concern this capture)
+    return hip_status(hipStreamBeginCapture((hipStream_t)stream, hipStreamCaptureModeThreadLocal), "hipStreamBeginCapture");
+}
+int mi355_graph_capture_end(void *stream, void **graph) {
+    if (!stream || !graph) return MI355_INVALID_ARGUMENTS;
+    *graph = nullptr;
+    hipGraph_t g = nullptr;
+    if (const int st = hip_status(hipStreamEndCapture((hipStream_t)stream, &g), "hipStreamEndCapture")) return st;
+    hipGraphExec_t exec = nullptr;
+    const int st = hip_status(hipGraphInstantiate(&exec, g, nullptr, nullptr, 0), "hipGraphInstantiate");
+    hipGraphDestroy(g);
+    if (st) return st;
+    *graph = (void *)exec;
+    return MI355_SUCCESS;
+}
+int mi355_graph_launch(void *graph, void *stream) {
+    if (!graph) return MI355_INVALID_ARGUMENTS;
+    return hip_status(hipGraphLaunch((hipGraphExec_t)graph, (hipStream_t)stream), "hipGraphLaunch");
+}
+int mi355_graph_destroy(void *graph) {
+    if (!graph) return MI355_SUCCESS;
+    return hip_status(hipGraphExecDestroy((hipGraphExec_t)graph), "hipGraphExecDestroy");
+}
 int mi355_stream_sync(void *stream) {
     return hip_status(hipStreamSynchronize((hipStream_t)stream), "hipStreamSynchronize");
 }
