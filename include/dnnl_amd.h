@@ -327,6 +327,14 @@ dnnl_status_t dnnl_stream_create(dnnl_stream_t *stream, dnnl_engine_t engine, un
 dnnl_status_t dnnl_stream_get_engine(const_dnnl_stream_t stream, dnnl_engine_t *engine);
 dnnl_status_t dnnl_stream_wait(dnnl_stream_t stream);
 dnnl_status_t dnnl_stream_destroy(dnnl_stream_t stream);
+/* Interoperability with the caller's HIP stream: what dnnl_ocl_interop_stream_create /
+ * dnnl_ocl_interop_stream_get_command_queue (dnnl_ocl.h:220-231) and their SYCL twins (dnnl_sycl.h:154-165) are
+ * for the reference's GPU runtimes.  `hip_stream` is a hipStream_t (NULL: the default stream); the dnnl stream does
+ * not own it.  Primitives executed on it are ordered with the caller's own work on that stream and are recorded
+ * when the caller captures it into a HIP graph (execute then must not need the library-mode scratchpad to grow:
+ * use dnnl_scratchpad_mode_user, or execute once before capturing). */
+dnnl_status_t dnnl_amd_interop_stream_create(dnnl_stream_t *stream, dnnl_engine_t engine, void *hip_stream);
+dnnl_status_t dnnl_amd_interop_stream_get_hip_stream(dnnl_stream_t stream, void **hip_stream);
 
 /* ---- memory descriptors: dnnl.h:1018-1424 ---- */
 dnnl_status_t dnnl_memory_desc_create_with_strides(dnnl_memory_desc_t *memory_desc, int ndims,

@@ -106,13 +106,25 @@ class engine:
 
 
 class stream:
-    def __init__(self, eng, flags=1):
+    """hip_stream: a hipStream_t of the caller's (an integer; 0 = the default stream) to run on instead of a stream
+    of the library's own -- dnnl_amd_interop_stream_create."""
+
+    def __init__(self, eng, flags=1, hip_stream=None):
         self.engine = eng
         self.h = C.c_void_p()
-        _check(lib().dnnl_stream_create(C.byref(self.h), eng.h, C.c_uint(flags)), "stream_create")
+        if hip_stream is None:
+            _check(lib().dnnl_stream_create(C.byref(self.h), eng.h, C.c_uint(flags)), "stream_create")
+        else:
+            _check(lib().dnnl_amd_interop_stream_create(C.byref(self.h), eng.h, C.c_void_p(hip_stream)),
+                   "interop_stream_create")
 
     def wait(self):
         _check(lib().dnnl_stream_wait(self.h), "stream_wait")
+
+    def hip_stream(self):
+        p = C.c_void_p()
+        _check(lib().dnnl_amd_interop_stream_get_hip_stream(self.h, C.byref(p)), "interop_stream_get_hip_stream")
+        return p.value
 
 
 class memory_desc:
@@ -263,6 +275,12 @@ class memory:
         if data.nbytes:
             C.memmove(p, data.ctypes.data, data.nbytes)
         _check(lib().dnnl_memory_unmap_data(self.h, p), "memory_unmap_data")
+
+    def get_data_handle(self):
+        """The device pointer (dnnl_memory_get_data_handle)."""
+        p = C.c_void_p()
+        _check(lib().dnnl_memory_get_data_handle(self.h, C.byref(p)), "memory_get_data_handle")
+        return p.value
 
     def read(self, dtype):
         p = C.c_void_p()

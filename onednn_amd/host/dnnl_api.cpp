@@ -94,6 +94,7 @@ struct dnnl_engine {
 struct dnnl_stream {
     dnnl_engine_t engine;
     void *hip_stream;
+    bool owned = true; // false: the caller's stream (dnnl_amd_interop_stream_create), never destroyed here
 };
 
 struct dnnl_memory_desc {
@@ -933,7 +934,7 @@ DNNL_EXPORT dnnl_status_t dnnl_stream_create(dnnl_stream_t *stream, dnnl_engine_
     if (mi355_device_set((int)engine->index) != MI355_SUCCESS) return dnnl_runtime_error;
     void *s = nullptr;
     if (mi355_stream_create(&s) != MI355_SUCCESS) return dnnl_runtime_error;
-    *stream = new dnnl_stream {engine, s};
+    *stream = new dnnl_stream {engine, s, true};
     return dnnl_success;
 }
 DNNL_EXPORT dnnl_status_t dnnl_stream_get_engine(const_dnnl_stream_t stream, dnnl_engine_t *engine) {
@@ -947,9 +948,22 @@ DNNL_EXPORT dnnl_status_t dnnl_stream_wait(dnnl_stream_t stream) {
 }
 DNNL_EXPORT dnnl_status_t dnnl_stream_destroy(dnnl_stream_t stream) {
     if (stream) {
-        mi355_stream_destroy(stream->hip_stream);
+        if (stream->owned) mi355_stream_destroy(stream->hip_stream);
         delete stream;
     }
+    return dnnl_success;
+}
+// The interoperability pair of the reference's GPU runtimes (dnnl_ocl.h:220-231, dnnl_sycl.h:154-165) for HIP:
+// a dnnl stream over the caller's hipStream_t (a framework's current stream; NULL is the default stream), so that
+// primitives are ordered with the caller's own kernels -- and recorded when the caller captures that stream.
+DNNL_EXPORT dnnl_status_t dnnl_amd_interop_stream_create(dnnl_stream_t *stream, dnnl_engine_t engine, void *hip_stream) {
+    CHECK_ARG(stream && engine);
+    *stream = new dnnl_stream {engine, hip_stream, false};
+    return dnnl_success;
+}
+DNNL_EXPORT dnnl_status_t dnnl_amd_interop_stream_get_hip_stream(dnnl_stream_t stream, void **hip_stream) {
+    CHECK_ARG(stream && hip_stream);
+    *hip_stream = stream->hip_stream;
     return dnnl_success;
 }
 

@@ -102,3 +102,38 @@ def test_capture_needs_a_created_stream(gpu):
     assert lib.mi355_graph_capture_begin(None) == cabi.INVALID_ARGUMENTS
     assert lib.mi355_graph_launch(None, None) == cabi.INVALID_ARGUMENTS
     assert lib.mi355_graph_destroy(None) == cabi.SUCCESS
+
+
+@pytest.mark.gpu
+def test_a_primitive_on_the_callers_stream_is_ordered_and_captured_with_it(gpu):
+    """dnnl_amd_interop_stream_create: the dnnl stream is the caller's hipStream_t.  A fill enqueued on that stream by
+    the caller, then the primitive through the dnnl layer, no host synchronization between them; then the execute
+    call recorded into the caller's graph and replayed."""
+    from onednn_amd import dnnl
+    from tests.test_gpu_dnnl_api import run_through_api
+    lib = cabi.load_kernels()
+    p = configs.config3(M=256, N=256, K=512)
+    want, impl, (pd, prim, strm0, args) = run_through_api(p)      # eager, on a stream of the library's
+    assert impl.startswith("hip:mfma_i8")
+    hs = cabi.Stream()
+    strm = dnnl.stream(strm0.engine, hip_stream=hs.ptr)
+    assert strm.hip_stream() == hs.ptr
+    dst = args[dnnl.ARG_DST]
+    handle = dst.get_data_handle()
+    try:
+        cabi.check(lib.mi355_mem_set(handle, 0x55, dst.md.get_size(), hs.ptr))
+        prim.execute(strm, args)
+        strm.wait()
+        assert np.array_equal(dst.read(np.int8), want)
+
+        with cabi.Graph(hs) as g:
+            prim.execute(strm, args)
+        for _ in range(2):
+            dst.write(np.full(want.shape, 0x33, np.int8))
+            assert not np.array_equal(dst.read(np.int8), want)
+            g.launch()
+            hs.sync()
+            assert np.array_equal(dst.read(np.int8), want)
+        g.destroy()
+    finally:
+        hs.destroy()
