@@ -34,7 +34,8 @@ def build(name, lib):
 def test_headers_compile_as_c_and_link():
     # no device needed: the programs build against the headers and libraries
     for name, lib in (("dnnl_client", "dnnl_amd"), ("ip_client", "dnnl_amd"), ("sdpa_client", "dnnl_amd"),
-                      ("mi355_client", "mi355_matmul"), ("dnnl_cpp_client", "dnnl_amd")):
+                      ("mi355_client", "mi355_matmul"), ("dnnl_cpp_client", "dnnl_amd"), ("woq_cpp_client", "dnnl_amd"),
+                      ("mxfp_cpp_client", "dnnl_amd")):
         d, exe = build(name, lib)
         assert os.path.exists(exe)
         shutil.rmtree(d, ignore_errors=True)
@@ -44,6 +45,8 @@ def test_headers_compile_as_c_and_link():
 @pytest.mark.parametrize("name,lib,impl", [("dnnl_client", "dnnl_amd", "hip:mfma_i8"), ("ip_client", "dnnl_amd", "hip:mfma_i8"),
                                            ("sdpa_client", "dnnl_amd", "hip:sdpa("),
                                            ("dnnl_cpp_client", "dnnl_amd", "hip:mfma_i8"),
+                                           ("woq_cpp_client", "dnnl_amd", "hip:"),
+                                           ("mxfp_cpp_client", "dnnl_amd", "hip:"),
                                            ("mi355_client", "mi355_matmul", "hip:mfma_i8")])
 def test_c_client_runs_on_the_device(gpu, name, lib, impl):
     d, exe = build(name, lib)
