@@ -3,7 +3,8 @@ include/dnnl_amd.h / include/mi355_matmul.h, built with gcc against the two
 shared libraries and run on the device (u8 x s8 -> s32 matmuls and an inner product on
 channels-last tensors, each checked against an integer loop inside the program; attention on f32 tensors against a
 double-precision loop), and a C++ program over include/dnnl_amd.hpp written like the reference's int8 inference
-tutorial, and three more for its weight-only-quantization, MX and dynamic-quantization tutorials.  Struct layouts, enum values and calling
+tutorial, three more for its weight-only-quantization, MX and dynamic-quantization tutorials, and its inner-product example
+with the two backward primitives added.  Struct layouts, enum values and calling
 conventions of the headers are what a compiled caller sees; the ctypes tests
 only check names."""
 import os
@@ -35,7 +36,8 @@ def test_headers_compile_as_c_and_link():
     # no device needed: the programs build against the headers and libraries
     for name, lib in (("dnnl_client", "dnnl_amd"), ("ip_client", "dnnl_amd"), ("sdpa_client", "dnnl_amd"),
                       ("mi355_client", "mi355_matmul"), ("dnnl_cpp_client", "dnnl_amd"), ("woq_cpp_client", "dnnl_amd"),
-                      ("mxfp_cpp_client", "dnnl_amd"), ("quantization_cpp_client", "dnnl_amd")):
+                      ("mxfp_cpp_client", "dnnl_amd"), ("quantization_cpp_client", "dnnl_amd"),
+                      ("ip_cpp_client", "dnnl_amd")):
         d, exe = build(name, lib)
         assert os.path.exists(exe)
         shutil.rmtree(d, ignore_errors=True)
@@ -48,6 +50,7 @@ def test_headers_compile_as_c_and_link():
                                            ("woq_cpp_client", "dnnl_amd", "hip:"),
                                            ("mxfp_cpp_client", "dnnl_amd", "hip:"),
                                            ("quantization_cpp_client", "dnnl_amd", "hip:"),
+                                           ("ip_cpp_client", "dnnl_amd", "hip:"),
                                            ("mi355_client", "mi355_matmul", "hip:mfma_i8")])
 def test_c_client_runs_on_the_device(gpu, name, lib, impl):
     d, exe = build(name, lib)
