@@ -4,7 +4,7 @@ shared libraries and run on the device (u8 x s8 -> s32 matmuls and an inner prod
 channels-last tensors, each checked against an integer loop inside the program; attention on f32 tensors against a
 double-precision loop), and a C++ program over include/dnnl_amd.hpp written like the reference's int8 inference
 tutorial, three more for its weight-only-quantization, MX and dynamic-quantization tutorials, and its inner-product example
-with the two backward primitives added.  Struct layouts, enum values and calling
+with the two backward primitives added, its matmul and reorder examples.  Struct layouts, enum values and calling
 conventions of the headers are what a compiled caller sees; the ctypes tests
 only check names."""
 import os
@@ -37,7 +37,7 @@ def test_headers_compile_as_c_and_link():
     for name, lib in (("dnnl_client", "dnnl_amd"), ("ip_client", "dnnl_amd"), ("sdpa_client", "dnnl_amd"),
                       ("mi355_client", "mi355_matmul"), ("dnnl_cpp_client", "dnnl_amd"), ("woq_cpp_client", "dnnl_amd"),
                       ("mxfp_cpp_client", "dnnl_amd"), ("quantization_cpp_client", "dnnl_amd"),
-                      ("ip_cpp_client", "dnnl_amd")):
+                      ("ip_cpp_client", "dnnl_amd"), ("primitives_cpp_client", "dnnl_amd")):
         d, exe = build(name, lib)
         assert os.path.exists(exe)
         shutil.rmtree(d, ignore_errors=True)
@@ -51,6 +51,7 @@ def test_headers_compile_as_c_and_link():
                                            ("mxfp_cpp_client", "dnnl_amd", "hip:"),
                                            ("quantization_cpp_client", "dnnl_amd", "hip:"),
                                            ("ip_cpp_client", "dnnl_amd", "hip:"),
+                                           ("primitives_cpp_client", "dnnl_amd", "hip:"),
                                            ("mi355_client", "mi355_matmul", "hip:mfma_i8")])
 def test_c_client_runs_on_the_device(gpu, name, lib, impl):
     d, exe = build(name, lib)
