@@ -200,11 +200,9 @@ static int impl_supported(const mi355_matmul_desc_t &d, int impl) {
     // the ternary select post-op: generic kernel only
     for (int i = 0; i < d.n_post_ops; ++i)
         if (d.post_ops[i].kind == MI355_PO_SELECT_COND && impl != MI355_IMPL_REF) return MI355_UNIMPLEMENTED;
-    // a 4-bit dst: generic kernel only
-    if (dt_bits(d.dst_dt) < 8 && impl != MI355_IMPL_REF) return MI355_UNIMPLEMENTED;
-    // the tiles' group reduction is the MX one (32 columns, fp8 dst)
-    if ((d.dst_scale_dynamic == MI355_DST_DYNAMIC_FP || (d.dst_scale_dynamic && !is_f8_dt(d.dst_dt)))
-            && impl != MI355_IMPL_REF)
+    // a 4-bit dst: the generic kernel, and the floating-point GEMM tiles where groups of four columns are whole bytes
+    if (dt_bits(d.dst_dt) < 8 && impl != MI355_IMPL_REF
+            && !((impl == MI355_IMPL_F8_MFMA || impl == MI355_IMPL_MXF4_MFMA) && tile_nibble_dst_ok(d)))
         return MI355_UNIMPLEMENTED;
     // dropout and stochastic rounding: generic kernel only
     if (d.rnd_flags != 0 && impl != MI355_IMPL_REF) return MI355_UNIMPLEMENTED;

@@ -213,7 +213,7 @@ f8_plan_t make_plan(const mi355_matmul_desc_t &d) {
 
 int f8_supported(const mi355_matmul_desc_t &d) {
     if (!is_f8_dt(d.src_dt) || !is_f8_dt(d.wei_dt)) return MI355_UNIMPLEMENTED;
-    if (dt_bits(d.dst_dt) < 8) return MI355_UNIMPLEMENTED;
+    if (dt_bits(d.dst_dt) < 8 && !tile_nibble_dst_ok(d)) return MI355_UNIMPLEMENTED;
     // whole 16-byte chunks of K; a K that ends inside a 64-byte stage takes one unpipelined step more per tile
     if (d.K < BKB * KSTEP || d.K % 16 != 0) return MI355_UNIMPLEMENTED;
     if (d.src_stride[2] != 1 || d.src_stride[1] % 16 != 0 || d.src_stride[0] % 16 != 0)

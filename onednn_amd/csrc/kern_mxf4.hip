@@ -384,7 +384,7 @@ mxf4_plan_t make_plan(const mi355_matmul_desc_t &d) {
 
 int mxf4_supported(const mi355_matmul_desc_t &d) {
     if (d.src_dt != MI355_DT_F4_E2M1 || d.wei_dt != MI355_DT_F4_E2M1) return MI355_UNIMPLEMENTED;
-    if (dt_bits(d.dst_dt) < 8) return MI355_UNIMPLEMENTED;
+    if (dt_bits(d.dst_dt) < 8 && !tile_nibble_dst_ok(d)) return MI355_UNIMPLEMENTED;
     // whole MX blocks; a K that ends inside a stage of 128 takes one unpipelined step more per tile
     if (d.K < 128 || d.K % 32 != 0) return MI355_UNIMPLEMENTED;
     if (d.src_stride[2] != 1 || d.src_stride[1] % 32 != 0 || d.src_stride[0] % 32 != 0)

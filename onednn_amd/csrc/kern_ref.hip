@@ -143,13 +143,6 @@ __global__ void __launch_bounds__(256) ref_matmul_kernel(const problem_t P_) {
 // 4-bit dst (f4_e2m1, s4, u4) with static scales: two consecutive n share a
 // byte (low nibble first), so one thread computes both and writes the byte.
 // The host has checked: N even, unit n stride, even m / batch strides.
-__device__ __forceinline__ uint32_t nibble_code(int dt, float v) {
-    switch (dt) {
-        case MI355_DT_F4_E2M1: return f32_to_e2m1(v);
-        case MI355_DT_S4: return (uint32_t)(int)__builtin_rintf(sat(v, -8.f, 7.f)) & 0xfu;
-        default: return (uint32_t)(int)__builtin_rintf(sat(v, 0.f, 15.f)) & 0xfu;
-    }
-}
 
 __global__ void __launch_bounds__(256) ref_matmul_nibble_dst_kernel(const problem_t P_) {
     const auto &P = MI355_KERNARG_PROBLEM();

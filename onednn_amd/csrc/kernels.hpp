@@ -58,6 +58,12 @@ int tuning(tune_key_t key);
 // threads.
 int ensure_dynamic_lds(const void *kernel, int bytes, const char *who);
 
+// A 4-bit dst (f4_e2m1 / s4 / u4) in the GEMM tiles' epilogue: four consecutive columns of a row leave as two whole
+// bytes, so rows are contiguous, every group of four is whole and starts a byte.
+inline bool tile_nibble_dst_ok(const mi355_matmul_desc_t &d) {
+    return d.dst_stride[2] == 1 && d.N % 4 == 0 && d.dst_stride[1] % 4 == 0 && d.dst_stride[0] % 4 == 0;
+}
+
 // [R][C] bytes (row pitch ld_in) -> [C][R] bytes (row pitch ld_out), per batch
 void transpose_bytes(const void *in, long R, long C, long ld_in, long in_bstride, void *out,
         long ld_out, long out_bstride, long batches, hipStream_t stream);

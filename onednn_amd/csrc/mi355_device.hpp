@@ -109,6 +109,15 @@ __device__ __forceinline__ uint32_t cvt_store_bits(int dt, float v) {
     }
 }
 
+// the four bits of a 4-bit dst value (f4_e2m1, s4, u4): saturated, rounded to nearest even
+__device__ __forceinline__ uint32_t nibble_code(int dt, float v) {
+    switch (dt) {
+        case MI355_DT_F4_E2M1: return f32_to_e2m1(v);
+        case MI355_DT_S4: return (uint32_t)(int)__builtin_rintf(sat(v, -8.f, 7.f)) & 0xfu;
+        default: return (uint32_t)(int)__builtin_rintf(sat(v, 0.f, 15.f)) & 0xfu;
+    }
+}
+
 __device__ __forceinline__ void store_float(int dt, float v, void *p, long off) {
     const uint32_t bits = cvt_store_bits(dt, v);
     switch (dt) {

@@ -149,7 +149,7 @@ __device__ __forceinline__ bool vec_ok(const void *p, long s0, long s1, int bits
 
 __device__ __forceinline__ bool vec_ok_store(const void *p, long s0, long s1, int bits) {
     const int bytes4 = bits / 2; // bytes of four elements
-    return (bits == 8 || bits == 16 || bits == 32) && (((uintptr_t)p) % bytes4) == 0
+    return (bits == 4 || bits == 8 || bits == 16 || bits == 32) && (((uintptr_t)p) % bytes4) == 0
             && (s0 % 4) == 0 && (s1 % 4) == 0;
 }
 
@@ -274,7 +274,8 @@ __device__ __forceinline__ epi_uniform_t make_uniform(const PT &P, bool cols_ins
         };
         const int dd = H.dst_dt;
         if (dd != MI355_DT_S8 && dd != MI355_DT_U8 && dd != MI355_DT_BF16 && dd != MI355_DT_F32 && dd != MI355_DT_S32
-                && dd != MI355_DT_F8_E4M3 && dd != MI355_DT_F8_E5M2 && dd != MI355_DT_F16)
+                && dd != MI355_DT_F8_E4M3 && dd != MI355_DT_F8_E5M2 && dd != MI355_DT_F16 && dd != MI355_DT_F4_E2M1
+                && dd != MI355_DT_S4 && dd != MI355_DT_U4)
             H.fast = 0;
         if (H.nfast > 0 && !operand_ready(H.pf0, 0)) H.fast = 0;
         if (H.nfast > 1 && !operand_ready(H.pf1, 1)) H.fast = 0;
@@ -410,6 +411,12 @@ __device__ __forceinline__ void cvt4(int dt, const float (&v)[4], uint32_t (&w)[
             for (int e = 0; e < 4; ++e)
                 w[e] = (uint32_t)(int)__builtin_rintf(sat(v[e], -2147483648.f, 2147483520.f));
             break;
+        case MI355_DT_F4_E2M1:
+        case MI355_DT_S4:
+        case MI355_DT_U4:
+#pragma unroll
+            for (int e = 0; e < 4; ++e) w[e] = nibble_code(dt, v[e]);
+            break;
         default:
 #pragma unroll
             for (int e = 0; e < 4; ++e) w[e] = cvt_store_bits(dt, v[e]);
@@ -425,6 +432,17 @@ __device__ __forceinline__ void store4(const PT &P, int dst_vec, const float (&v
     uint32_t w[4];
     cvt4(P.dst_dt, v, w);
     const int bits = dt_bits(P.dst_dt);
+    if (bits == 4) {
+        // Two bytes, low nibble first.  The host admits a 4-bit dst only where every quad is whole and starts a
+        // byte (unit column stride, N and the other strides multiples of 4); the bytes may start at an odd address.
+        if (nvalid == 4) {
+            uint8_t *q = (uint8_t *)P.dst + (off >> 1);
+            const uint32_t lo = w[0] | (w[1] << 4), hi = w[2] | (w[3] << 4);
+            if ((uintptr_t)q & 1) q[0] = (uint8_t)lo, q[1] = (uint8_t)hi;
+            else *(uint16_t *)q = (uint16_t)(lo | (hi << 8));
+        }
+        return;
+    }
     if (nvalid == 4 && dst_vec) {
         if (bits == 8) {
             *(uint32_t *)((uint8_t *)P.dst + off) = w[0] | (w[1] << 8) | (w[2] << 16) | (w[3] << 24);
@@ -685,6 +703,21 @@ __device__ __forceinline__ void storeQ(const PT &P, const epi_uniform_t &H, cons
     uint32_t w[Q][4];
     const int dt = H.dst_dt;
     const long rowoff = b * P.ds[0] + m * P.ds[1];
+    if (dt_bits(dt) == 4) {
+        // two bytes a quad, low nibble first; rows and quads start whole bytes (checked by the host), possibly at an
+        // odd address
+#pragma unroll
+        for (int k = 0; k < Q; ++k) {
+            uint32_t c[4];
+            cvt4(dt, v[k], c);
+            const uint32_t lo = c[0] | (c[1] << 4), hi = c[2] | (c[3] << 4);
+            uint8_t *q = (uint8_t *)P.dst + ((rowoff + n[k]) >> 1);
+            if (!ok) continue;
+            if ((uintptr_t)q & 1) q[0] = (uint8_t)lo, q[1] = (uint8_t)hi;
+            else *(uint16_t *)q = (uint16_t)(lo | (hi << 8));
+        }
+        return;
+    }
     if (dt == MI355_DT_S8 || dt == MI355_DT_U8) {
         // Round first (v_rndne + the saturating v_cvt_i32_f32, NaN -> 0), clamp as
         // integers (maximum + minimum), pack the four low bytes with byte permutes: the
@@ -825,10 +858,34 @@ __device__ __forceinline__ void storeQ(const PT &P, const epi_uniform_t &H, cons
 // conversion.  All lanes take part in the cross-lane maximum, rows beyond M on
 // the data of a valid row; only the stores are masked.
 template <class Layout, int Q, class PT>
-__device__ __forceinline__ void dynamic_quantQ(const PT &P, int dst_dt, float (&v)[Q][4], long b, long m, bool ok,
-        const long (&n)[Q], int lane) {
+__device__ __forceinline__ void dynamic_quantQ(const PT &P, int dst_dt, int mode, float (&v)[Q][4], long b, long m,
+        bool ok, const long (&n)[Q], int lane) {
     constexpr int QPG = Layout::QPG;
-    const float dt_max = dst_dt == MI355_DT_F8_E4M3 ? 448.f : 57344.f;
+    const float dt_max = dst_dt == MI355_DT_F8_E4M3 ? 448.f : (dst_dt == MI355_DT_F4_E2M1 ? 6.f : 57344.f);
+    if (mode == MI355_DST_DYNAMIC_FP) {
+        // groups of 16 columns with an f8_e4m3 scale (ref_matmul.cpp:352-365, :381): the lower and the upper
+        // half of the lane's quads of 32 columns, shared with the same partner lanes
+        constexpr int HQ = QPG / 2;
+#pragma unroll
+        for (int g = 0; g < Q / HQ; ++g) {
+            float amax = 0.f;
+#pragma unroll
+            for (int kk = 0; kk < HQ; ++kk) amax = fmaxf(amax, amax4(v[g * HQ + kk]));
+            amax = Layout::group_max(amax);
+            float scale = amax / dt_max;
+            scale = fminf(scale, 448.f);
+            scale = fmaxf(scale, 0.125f);
+            const uint8_t sbyte = f32_to_e4m3(scale);
+            const float inv = 1.f / e4m3_to_f32(sbyte);
+#pragma unroll
+            for (int kk = 0; kk < HQ; ++kk)
+#pragma unroll
+                for (int e = 0; e < 4; ++e) v[g * HQ + kk][e] = fminf(fmaxf(v[g * HQ + kk][e] * inv, -dt_max), dt_max);
+            if (ok && Layout::group_leader(lane))
+                ((uint8_t *)P.dst_scale.p)[quant_off(P.dst_scale, b, m, n[g * HQ] & ~15L, P.M, P.N)] = sbyte;
+        }
+        return;
+    }
     const int em = (int)f32_to_e8m0(dt_max);
 #pragma unroll
     for (int g = 0; g < Q / QPG; ++g) {
@@ -1005,7 +1062,7 @@ __device__ __forceinline__ void store_quadrant(const PT &P, char *park, unsigned
                 }
             }
             apply_epilogueQ<Q>(H, ntab, col, v, sy);
-            if (H.dynamic) dynamic_quantQ<Layout, Q>(P, H.dst_dt, v, b, ok ? m : P.M - 1, ok, n, lane);
+            if (H.dynamic) dynamic_quantQ<Layout, Q>(P, H.dst_dt, H.dynamic, v, b, ok ? m : P.M - 1, ok, n, lane);
             storeQ<Q>(P, H, v, b, m, ok, n);
         }
         return;
@@ -1030,7 +1087,7 @@ __device__ __forceinline__ void store_quadrant(const PT &P, char *park, unsigned
         const bool okm = m < P.M;
         const long mv = okm ? m : P.M - 1;
         const row_t rd = conv.row_data(mv);
-        const float dt_max = P.dst_dt == MI355_DT_F8_E4M3 ? 448.f : 57344.f;
+        const float dt_max = P.dst_dt == MI355_DT_F8_E4M3 ? 448.f : (P.dst_dt == MI355_DT_F4_E2M1 ? 6.f : 57344.f);
         const int em = (int)f32_to_e8m0(dt_max);
 #pragma unroll 1
         for (int g = 0; g < Q / QPG; ++g) {
@@ -1053,7 +1110,31 @@ __device__ __forceinline__ void store_quadrant(const PT &P, char *park, unsigned
                     if (e >= nvalid[kk]) v[kk][e] = 0.f;
                 amax = fmaxf(amax, amax4(v[kk]));
             }
-            if (H.dynamic) {
+            if (H.dynamic == MI355_DST_DYNAMIC_FP) {
+                // groups of 16 columns with an f8_e4m3 scale (ref_matmul.cpp:352-365, :381): the lower and the
+                // upper half of this lane's quads of the 32 columns, shared with the same partner lanes.  N is a
+                // multiple of 16: a group is whole or absent
+                constexpr int HQ = QPG / 2;
+#pragma unroll
+                for (int h = 0; h < 2; ++h) {
+                    float hmax = 0.f;
+#pragma unroll
+                    for (int kk = 0; kk < HQ; ++kk) hmax = fmaxf(hmax, amax4(v[h * HQ + kk]));
+                    hmax = Layout::group_max(hmax);
+                    float scale = hmax / dt_max;
+                    scale = fminf(scale, 448.f);
+                    scale = fmaxf(scale, 0.125f);
+                    const uint8_t sbyte = f32_to_e4m3(scale);
+                    const float inv = 1.f / e4m3_to_f32(sbyte);
+#pragma unroll
+                    for (int kk = 0; kk < HQ; ++kk)
+#pragma unroll
+                        for (int e = 0; e < 4; ++e)
+                            v[h * HQ + kk][e] = fminf(fmaxf(v[h * HQ + kk][e] * inv, -dt_max), dt_max);
+                    if (okm && nvalid[h * HQ] > 0 && Layout::group_leader(lane))
+                        ((uint8_t *)P.dst_scale.p)[quant_off(P.dst_scale, b, m, nq[h * HQ] & ~15L, P.M, P.N)] = sbyte;
+                }
+            } else if (H.dynamic) {
                 // N is a multiple of 32: a group is whole or absent
                 amax = Layout::group_max(amax);
                 float inv;

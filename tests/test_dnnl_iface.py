@@ -266,19 +266,21 @@ def test_dynamic_mx_dst_scales_rules(eng):
     assert status_of(lambda: make_pd(eng, 64, 128, 256, "f8_e4m3", "f8_e4m3", "f8_e4m3", attr=mx(arg=dnnl.ARG_SRC, groups=(1, 32)))) == dnnl.unimplemented
     a = dnnl.primitive_attr()
     assert status_of(lambda: a.set_scales(dnnl.ARG_DST, 3, (1, 32), DT["e8m0"], qmode=7)) == dnnl.invalid_arguments
-    # quantization_mode::dynamic_fp (matmul.cpp:423-440): the NVFP4 flavour, f8_e4m3 scales per 1 x 16; generic kernel
+    # quantization_mode::dynamic_fp (matmul.cpp:423-440): the NVFP4 flavour, f8_e4m3 scales per 1 x 16
     def fp(mask=3, groups=(1, 16), dt=DT["f8_e4m3"]):
         return _attr(lambda t: t.set_scales(dnnl.ARG_DST, mask, groups, dt, qmode=dnnl.quantization_mode_dynamic_fp))
     for dst in ("f4_e2m1", "f8_e4m3"):
         pd = make_pd(eng, 64, 128, 256, "f8_e4m3", "f8_e4m3", dst, attr=fp())
-        assert pd.impl_info_str() == "hip:ref:any"
-    assert make_pd(eng, 64, 128, 256, "f8_e4m3", "f8_e4m3", "f4_e2m1", attr=mx()).impl_info_str() == "hip:ref:any"
+        assert pd.impl_info_str().startswith("hip:mfma_f8")
+        assert pd.next_impl() and pd.impl_info_str() == "hip:ref:any"
+    assert make_pd(eng, 64, 128, 256, "f8_e4m3", "f8_e4m3", "f4_e2m1", attr=mx()).impl_info_str().startswith("hip:mfma_f8")
     assert status_of(lambda: make_pd(eng, 64, 128, 256, "f8_e4m3", "f8_e4m3", "f4_e2m1", attr=fp(groups=(1, 32)))) == dnnl.unimplemented
     assert status_of(lambda: make_pd(eng, 64, 128, 256, "f8_e4m3", "f8_e4m3", "f4_e2m1", attr=fp(dt=DT["e8m0"]))) == dnnl.unimplemented
     assert status_of(lambda: make_pd(eng, 64, 128, 256, "f8_e4m3", "f8_e4m3", "f4_e2m1", attr=fp(mask=2, groups=()))) == dnnl.unimplemented
     assert status_of(lambda: make_pd(eng, 64, 128, 256, "f8_e4m3", "f8_e4m3", "bf16", attr=fp())) == dnnl.unimplemented
-    # a 4-bit dst without dynamic scales: generic kernel
-    assert make_pd(eng, 64, 128, 256, "f8_e4m3", "f8_e4m3", "f4_e2m1").impl_info_str() == "hip:ref:any"
+    # a 4-bit dst without dynamic scales: the tiles too (groups of four columns are whole bytes here), else generic
+    assert make_pd(eng, 64, 128, 256, "f8_e4m3", "f8_e4m3", "f4_e2m1").impl_info_str().startswith("hip:mfma_f8")
+    assert make_pd(eng, 64, 128, 254, "f8_e4m3", "f8_e4m3", "f4_e2m1").impl_info_str() == "hip:ref:any"
     assert status_of(lambda: a.set_scales(dnnl.ARG_DST, 1, (), DT["f32"], is_on_host=1)) == dnnl.invalid_arguments
     assert status_of(lambda: a.set_scales(dnnl.ARG_DST, 0, (), DT["f32"], is_on_host=1)) == dnnl.success
 

@@ -255,7 +255,7 @@ def search_dynamic_fp(d, dst_dt):
 
 def unpack_dst(raw, dst_dt, M, N):
     raw = np.asarray(raw).view(np.uint8).reshape(-1)
-    if dst_dt == cabi.DT_F4_E2M1:
+    if dst_dt in (cabi.DT_F4_E2M1, cabi.DT_S4, cabi.DT_U4):
         return np.stack([raw & 0xf, raw >> 4], axis=1).reshape(M, N)
     return raw.reshape(M, N)
 
@@ -309,8 +309,9 @@ def test_dynamic_fp_rules_of_the_descriptor():
     p = dynamic_fp(configs.config4(M=32, N=64, K=256))
     p.dst_dt = cabi.DT_F4_E2M1
     st, impl = cabi.query(p.desc())
-    assert st == cabi.SUCCESS and cabi.impl_name(impl) == "hip:ref:any"        # generic kernel only
-    assert cabi.query(p.desc(), cabi.IMPL_F8_MFMA)[0] == cabi.UNIMPLEMENTED
+    assert st == cabi.SUCCESS and cabi.impl_name(impl).startswith("hip:mfma_f8")   # the GEMM tiles take it
+    assert cabi.query(p.desc(), cabi.IMPL_REF)[0] == cabi.SUCCESS
+    assert cabi.query(p.desc(), cabi.IMPL_H16_MFMA)[0] == cabi.UNIMPLEMENTED
     q = dynamic_fp(configs.config4(M=32, N=64, K=256))
     q.dst_dt = cabi.DT_F4_E2M1
     q.quant["dst_scale"].groups = (1, 32)
@@ -319,19 +320,26 @@ def test_dynamic_fp_rules_of_the_descriptor():
     q.dst_dt = cabi.DT_F4_E2M1
     q.quant["dst_scale"].dt = cabi.DT_E8M0
     assert cabi.query(q.desc())[0] == cabi.INVALID_ARGUMENTS
-    # a 4-bit dst with a static scale: generic kernel, whole bytes per row
+    # a 4-bit dst with a static scale: the tiles where groups of four columns are whole bytes, else the generic
+    # kernel (whole bytes per row)
     s = configs.config4(M=32, N=64, K=256)
+    s.dst_dt = cabi.DT_F4_E2M1
+    st, impl = cabi.query(s.desc())
+    assert st == cabi.SUCCESS and cabi.impl_name(impl).startswith("hip:mfma_f8")
+    s = configs.config4(M=32, N=62, K=256)
+    s.post_ops = []
     s.dst_dt = cabi.DT_F4_E2M1
     st, impl = cabi.query(s.desc())
     assert st == cabi.SUCCESS and cabi.impl_name(impl) == "hip:ref:any"
     s = configs.config4(M=32, N=63, K=256)
+    s.post_ops = []
     s.dst_dt = cabi.DT_F4_E2M1
     assert cabi.query(s.desc())[0] == cabi.UNIMPLEMENTED
-    # MX scales over a 4-bit dst (an MXFP4 output): generic kernel
+    # MX scales over a 4-bit dst (an MXFP4 output)
     m = dynamic(configs.config4(M=32, N=64, K=256))
     m.dst_dt = cabi.DT_F4_E2M1
     st, impl = cabi.query(m.desc())
-    assert st == cabi.SUCCESS and cabi.impl_name(impl) == "hip:ref:any"
+    assert st == cabi.SUCCESS and cabi.impl_name(impl).startswith("hip:mfma_f8")
 
 
 @pytest.mark.gpu
@@ -358,11 +366,85 @@ def test_gpu_dynamic_fp_and_4bit_dst_are_bit_exact(gpu, oracle, dst, mode):
     p.post_ops = [PostOp(kind=cabi.PO_ELTWISE, alg=cabi.ELTWISE["relu"], alpha=0.25, scale=3.0), p.post_ops[1]]
     p.dst_dt = dst_dt
     p = make(p)
-    got, sc, name = run_gpu_dynamic(p)
+    got, sc, name = run_gpu_dynamic(p, cabi.IMPL_REF)
     want, want_sc = orc.run_oracle_dynamic(p)
     assert name == "hip:ref:any"
     assert np.array_equal(np.asarray(sc).reshape(-1), np.asarray(want_sc).reshape(-1))
     assert np.array_equal(np.asarray(got).view(np.uint8), np.asarray(want).view(np.uint8))
+
+
+def decode_dst(raw, dst_dt, M, N):
+    codes = unpack_dst(raw, dst_dt, M, N)
+    if dst_dt == cabi.DT_F4_E2M1:
+        return np.where(codes & 8, -1.0, 1.0) * E2M1[codes & 7]
+    if dst_dt == cabi.DT_S4:
+        return ((codes.astype(np.int32) ^ 8) - 8).astype(np.float64)
+    if dst_dt == cabi.DT_U4:
+        return codes.astype(np.float64)
+    f = dtp.e4m3_to_f32 if dst_dt == cabi.DT_F8_E4M3 else dtp.e5m2_to_f32
+    return f(codes.reshape(-1)).reshape(M, N).astype(np.float64)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("family", ["f8", "mxf4"])
+@pytest.mark.parametrize("mode,dst", [("fp", "f4_e2m1"), ("fp", "f8_e4m3"), ("mx", "f4_e2m1")])
+def test_gpu_gemm_tiles_quantize_dst_in_groups_of_16_and_to_4_bits(gpu, oracle, family, mode, dst):
+    """The NVFP4 flavour (f8_e4m3 scale per 16 columns) and 4-bit dst in the tiles' epilogue.  The tiles round the K
+    sum differently from the reference, so scales and codes are checked through what they mean: a scale within one
+    code of the oracle's (and equal nearly everywhere), and every element, times the scale the kernel wrote, within
+    the spacing of the dst type around the f32 result.  Partial tiles in both directions."""
+    dst_dt = {"f4_e2m1": cabi.DT_F4_E2M1, "f8_e4m3": cabi.DT_F8_E4M3}[dst]
+    G = 16 if mode == "fp" else 32
+    p = (configs.config4 if family == "f8" else configs.config5)(M=300, N=320, K=256)
+    p.dst_dt = cabi.DT_F32
+    pre = np.asarray(orc.run_oracle(p)).view(np.float32).reshape(p.M, p.N).astype(np.float64)
+    p.dst_dt = dst_dt
+    p = (dynamic_fp if mode == "fp" else dynamic)(p)
+    got, sc, name = run_gpu_dynamic(p)
+    assert name.startswith("hip:mfma_f8" if family == "f8" else "hip:mfma_mxf4")
+    _, want_sc = orc.run_oracle_dynamic(p)
+    sc = np.asarray(sc).reshape(p.M, p.N // G).astype(np.int32)
+    want_sc = np.asarray(want_sc).reshape(p.M, p.N // G).astype(np.int32)
+    assert np.all(np.abs(sc - want_sc) <= 1)
+    assert np.mean(sc == want_sc) > 0.97
+    scale = (dtp.e4m3_to_f32(sc.astype(np.uint8).reshape(-1)).reshape(sc.shape).astype(np.float64) if mode == "fp"
+             else np.exp2(sc - 127.0)).repeat(G, axis=1)
+    x = np.clip(pre / scale, -FP_MAX[dst_dt], FP_MAX[dst_dt])
+    q = decode_dst(got, dst_dt, p.M, p.N)
+    # half the distance between neighbours of the dst type at |x| (e2m1: 0.25 up to 2, 0.5 up to 4, 1 up to 6; e4m3:
+    # 2^-4 |x|, 2^-10 among the subnormals) + the tiles' own rounding of the sum, which may move x across a tie
+    half = np.maximum(0.25, 0.25 * np.abs(x)) if dst_dt == cabi.DT_F4_E2M1 else np.abs(x) / 16 + 2.0 ** -10
+    amax = np.abs(pre).reshape(p.M, p.N // G, G).max(axis=2).repeat(G, axis=1)
+    tol = half + 2e-3 * amax / scale + 1e-6
+    assert np.all(np.abs(q - x) <= tol), float(np.max(np.abs(q - x) / tol))
+    assert len(np.unique(q)) >= (10 if dst_dt == cabi.DT_F4_E2M1 else 40)      # not a degenerate result
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("family", ["f8", "mxf4"])
+@pytest.mark.parametrize("dst", ["f4_e2m1", "s4", "u4"])
+def test_gpu_gemm_tiles_store_a_4bit_dst_with_a_static_scale(gpu, oracle, family, dst):
+    """Codes against the oracle's: equal nearly everywhere, never more than one step of the type apart (the tiles
+    round the K sum differently).  Bias / post-ops as the configuration has them, a static dst scale."""
+    dst_dt = {"f4_e2m1": cabi.DT_F4_E2M1, "s4": cabi.DT_S4, "u4": cabi.DT_U4}[dst]
+    p = (configs.config4 if family == "f8" else configs.config5)(M=300, N=320, K=256)
+    p.dst_dt = cabi.DT_F32
+    pre = np.abs(np.asarray(orc.run_oracle(p)).view(np.float32).astype(np.float64))
+    p.dst_dt = dst_dt
+    p.quant["dst_scale"] = QuantParam(cabi.DT_F32, 0, np.array([np.percentile(pre, 90) / 5.0], np.float32))
+    run = GpuRun(p, None)
+    try:
+        run.launch()
+        got, name = run.result(), cabi.impl_name(run.impl)
+    finally:
+        run.free()
+    assert name.startswith("hip:mfma_f8" if family == "f8" else "hip:mfma_mxf4")
+    want = orc.run_oracle(p)
+    g, w = decode_dst(got, dst_dt, p.M, p.N), decode_dst(want, dst_dt, p.M, p.N)
+    step = np.maximum(0.5, 0.5 * np.maximum(np.abs(g), np.abs(w))) if dst_dt == cabi.DT_F4_E2M1 else 1.0
+    assert np.all(np.abs(g - w) <= step)
+    assert np.mean(g == w) > 0.97
+    assert len(np.unique(w)) >= 8
 
 
 @pytest.mark.gpu
@@ -377,7 +459,7 @@ def test_gpu_4bit_dst_with_a_static_scale_is_bit_exact(gpu, oracle, dst):
         p.dst_init = np.random.default_rng(9).integers(0, 256, size=p.M * p.N // 2).astype(np.uint8)
     p.dst_dt = {"f4_e2m1": cabi.DT_F4_E2M1, "s4": cabi.DT_S4, "u4": cabi.DT_U4}[dst]
     p.quant["dst_scale"] = QuantParam(cabi.DT_F32, 0, np.array([0.37], np.float32))
-    run = GpuRun(p, None)
+    run = GpuRun(p, cabi.IMPL_REF)
     try:
         run.launch()
         got, name = run.result(), cabi.impl_name(run.impl)
