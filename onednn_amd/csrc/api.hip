@@ -195,14 +195,15 @@ typedef int (*supported_fn)(const mi355_matmul_desc_t &);
 static int impl_supported(const mi355_matmul_desc_t &d, int impl) {
     // dynamic dst quantization: the generic kernel and the floating-point GEMM tiles
     if (d.dst_scale_dynamic != MI355_DST_DYNAMIC_NONE && impl != MI355_IMPL_REF && impl != MI355_IMPL_F8_MFMA
-            && impl != MI355_IMPL_MXF4_MFMA)
+            && impl != MI355_IMPL_MXF4_MFMA && impl != MI355_IMPL_H16_MFMA)
         return MI355_UNIMPLEMENTED;
     // the ternary select post-op: generic kernel only
     for (int i = 0; i < d.n_post_ops; ++i)
         if (d.post_ops[i].kind == MI355_PO_SELECT_COND && impl != MI355_IMPL_REF) return MI355_UNIMPLEMENTED;
     // a 4-bit dst: the generic kernel, and the floating-point GEMM tiles where groups of four columns are whole bytes
     if (dt_bits(d.dst_dt) < 8 && impl != MI355_IMPL_REF
-            && !((impl == MI355_IMPL_F8_MFMA || impl == MI355_IMPL_MXF4_MFMA) && tile_nibble_dst_ok(d)))
+            && !((impl == MI355_IMPL_F8_MFMA || impl == MI355_IMPL_MXF4_MFMA || impl == MI355_IMPL_H16_MFMA)
+                    && tile_nibble_dst_ok(d)))
         return MI355_UNIMPLEMENTED;
     // dropout and stochastic rounding: generic kernel only
     if (d.rnd_flags != 0 && impl != MI355_IMPL_REF) return MI355_UNIMPLEMENTED;
@@ -440,7 +441,7 @@ int mi355_graph_capture_end(void *stream, void **graph) {
     if (const int st = hip_status(hipStreamEndCapture((hipStream_t)stream, &g), "hipStreamEndCapture")) return st;
     hipGraphExec_t exec = nullptr;
     const int st = hip_status(hipGraphInstantiate(&exec, g, nullptr, nullptr, 0), "hipGraphInstantiate");
-    hipGraphDestroy(g);
+    (void)hipGraphDestroy(g);
     if (st) return st;
     *graph = (void *)exec;
     return MI355_SUCCESS;

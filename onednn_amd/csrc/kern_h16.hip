@@ -379,7 +379,7 @@ static int h16_woq_fast(const mi355_matmul_desc_t &d, const h16_plan_t &p) {
 }
 
 int h16_supported(const mi355_matmul_desc_t &d) {
-    if (dt_bits(d.dst_dt) < 8) return MI355_UNIMPLEMENTED;
+    if (dt_bits(d.dst_dt) < 8 && !tile_nibble_dst_ok(d)) return MI355_UNIMPLEMENTED;
     if (d.batch > 65535) return MI355_UNIMPLEMENTED;
     if (h16_woq(d)) return h16_plan(d).ok ? MI355_SUCCESS : MI355_UNIMPLEMENTED;
     if (d.src_dt != d.wei_dt || (d.src_dt != MI355_DT_BF16 && d.src_dt != MI355_DT_F16 && d.src_dt != MI355_DT_F32))

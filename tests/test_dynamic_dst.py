@@ -385,9 +385,13 @@ def decode_dst(raw, dst_dt, M, N):
     return f(codes.reshape(-1)).reshape(M, N).astype(np.float64)
 
 
+FAMILY = {"f8": (lambda **kw: configs.config4(**kw), "hip:mfma_f8"), "mxf4": (lambda **kw: configs.config5(**kw), "hip:mfma_mxf4"),
+          "h16": (lambda **kw: configs.config_h16(dt="bf16", **kw), "hip:mfma_h16")}
+
+
 @pytest.mark.gpu
-@pytest.mark.parametrize("family", ["f8", "mxf4"])
-@pytest.mark.parametrize("mode,dst", [("fp", "f4_e2m1"), ("fp", "f8_e4m3"), ("mx", "f4_e2m1")])
+@pytest.mark.parametrize("family", ["f8", "mxf4", "h16"])
+@pytest.mark.parametrize("mode,dst", [("fp", "f4_e2m1"), ("fp", "f8_e4m3"), ("mx", "f4_e2m1"), ("mx", "f8_e4m3")])
 def test_gpu_gemm_tiles_quantize_dst_in_groups_of_16_and_to_4_bits(gpu, oracle, family, mode, dst):
     """The NVFP4 flavour (f8_e4m3 scale per 16 columns) and 4-bit dst in the tiles' epilogue.  The tiles round the K
     sum differently from the reference, so scales and codes are checked through what they mean: a scale within one
@@ -395,13 +399,13 @@ def test_gpu_gemm_tiles_quantize_dst_in_groups_of_16_and_to_4_bits(gpu, oracle, 
     the spacing of the dst type around the f32 result.  Partial tiles in both directions."""
     dst_dt = {"f4_e2m1": cabi.DT_F4_E2M1, "f8_e4m3": cabi.DT_F8_E4M3}[dst]
     G = 16 if mode == "fp" else 32
-    p = (configs.config4 if family == "f8" else configs.config5)(M=300, N=320, K=256)
+    p = FAMILY[family][0](M=300, N=320, K=256)
     p.dst_dt = cabi.DT_F32
     pre = np.asarray(orc.run_oracle(p)).view(np.float32).reshape(p.M, p.N).astype(np.float64)
     p.dst_dt = dst_dt
     p = (dynamic_fp if mode == "fp" else dynamic)(p)
     got, sc, name = run_gpu_dynamic(p)
-    assert name.startswith("hip:mfma_f8" if family == "f8" else "hip:mfma_mxf4")
+    assert name.startswith(FAMILY[family][1])
     _, want_sc = orc.run_oracle_dynamic(p)
     sc = np.asarray(sc).reshape(p.M, p.N // G).astype(np.int32)
     want_sc = np.asarray(want_sc).reshape(p.M, p.N // G).astype(np.int32)
@@ -421,13 +425,13 @@ def test_gpu_gemm_tiles_quantize_dst_in_groups_of_16_and_to_4_bits(gpu, oracle, 
 
 
 @pytest.mark.gpu
-@pytest.mark.parametrize("family", ["f8", "mxf4"])
+@pytest.mark.parametrize("family", ["f8", "mxf4", "h16"])
 @pytest.mark.parametrize("dst", ["f4_e2m1", "s4", "u4"])
 def test_gpu_gemm_tiles_store_a_4bit_dst_with_a_static_scale(gpu, oracle, family, dst):
     """Codes against the oracle's: equal nearly everywhere, never more than one step of the type apart (the tiles
     round the K sum differently).  Bias / post-ops as the configuration has them, a static dst scale."""
     dst_dt = {"f4_e2m1": cabi.DT_F4_E2M1, "s4": cabi.DT_S4, "u4": cabi.DT_U4}[dst]
-    p = (configs.config4 if family == "f8" else configs.config5)(M=300, N=320, K=256)
+    p = FAMILY[family][0](M=300, N=320, K=256)
     p.dst_dt = cabi.DT_F32
     pre = np.abs(np.asarray(orc.run_oracle(p)).view(np.float32).astype(np.float64))
     p.dst_dt = dst_dt
@@ -438,7 +442,7 @@ def test_gpu_gemm_tiles_store_a_4bit_dst_with_a_static_scale(gpu, oracle, family
         got, name = run.result(), cabi.impl_name(run.impl)
     finally:
         run.free()
-    assert name.startswith("hip:mfma_f8" if family == "f8" else "hip:mfma_mxf4")
+    assert name.startswith(FAMILY[family][1])
     want = orc.run_oracle(p)
     g, w = decode_dst(got, dst_dt, p.M, p.N), decode_dst(want, dst_dt, p.M, p.N)
     step = np.maximum(0.5, 0.5 * np.maximum(np.abs(g), np.abs(w))) if dst_dt == cabi.DT_F4_E2M1 else 1.0
