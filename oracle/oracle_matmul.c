@@ -811,6 +811,12 @@ void oracle_binary(int alg, const float *x, const float *y, float *out,
  *   dst = _qz_a1b0<f32, type_o>()(d)    (:2659) = saturate + nearbyintf for
  *                                        integers, a conversion otherwise
  * e8m0 sources are converted without arithmetic (:2645-2655).
+ * Same data type on both sides and no attributes: the value moves unchanged --
+ * the reference's copy implementations (spec::direct_copy, :2064-2160, and the
+ * JIT reorder that comes first in its list) convert with qz_a1b0_t, which is a
+ * plain cast when the source type fits the destination type
+ * (simple_q10n.hpp:84-99), where the generic loop would take even an s32 -> s32
+ * copy through f32 and lose the low bits of values beyond 2^24.
  * Scale / zero-point offsets: get_quant_off over the logical index with the
  * groups on the last two dims (:2606-2640). */
 static int64_t orc_rq_off(const mi355_quant_t *q, const int64_t *idx, int ndims,
@@ -836,6 +842,9 @@ int oracle_reorder(const mi355_reorder_desc_t *d, const mi355_reorder_args_t *a)
     const int nd = d->ndims;
     int64_t total = 1;
     for (int i = 0; i < nd; ++i) total *= d->dims[i];
+    const int copy_s32 = d->src_dt == MI355_DT_S32 && d->dst_dt == MI355_DT_S32 && d->beta == 0.f
+            && d->src_scale.dt == MI355_DT_UNDEF && d->dst_scale.dt == MI355_DT_UNDEF
+            && d->src_zp.dt == MI355_DT_UNDEF && d->dst_zp.dt == MI355_DT_UNDEF;
     for (int64_t l = 0; l < total; ++l) {
         int64_t idx[MI355_REORDER_MAX_DIMS] = {0};
         int64_t rem = l, so = 0, dof = 0;
@@ -844,6 +853,10 @@ int oracle_reorder(const mi355_reorder_desc_t *d, const mi355_reorder_args_t *a)
             rem /= d->dims[i];
             so += idx[i] * d->src_stride[i];
             dof += idx[i] * d->dst_stride[i];
+        }
+        if (copy_s32) { /* (every other type survives the trip through f32 unchanged) */
+            ((int32_t *)a->dst)[dof] = ((const int32_t *)a->src)[so];
+            continue;
         }
         float x;
         if (d->src_dt == MI355_DT_E8M0) {

@@ -118,6 +118,20 @@ def test_integer_sources_subtract_as_integers_and_sum_post_op():
     assert np.array_equal(oracle.reorder(p), np.array([6, 12, 18, 24], np.float32))
 
 
+def test_an_s32_copy_keeps_every_bit():
+    """Same type, no attributes: the reference's copy implementations cast (simple_q10n.hpp:84-99); only its generic
+    loop would round 2^24 + 1 to a float on the way.  With an attribute the value does go through f32."""
+    x = np.array([[2 ** 24 + 1, -(2 ** 31), 2 ** 31 - 1, 2 ** 30 + 3, -7, 0]], dtype=np.int32)
+    p = ReorderProblem(dims=(1, 6), src_dt=cabi.DT_S32, dst_dt=cabi.DT_S32, src=x)
+    assert np.array_equal(oracle.reorder(p), x.reshape(-1))
+    t = ReorderProblem(dims=(2, 3), src_dt=cabi.DT_S32, dst_dt=cabi.DT_S32, src=x.reshape(2, 3), dst_stride=(1, 2))
+    assert np.array_equal(oracle.reorder(t), np.ascontiguousarray(x.reshape(2, 3).T).reshape(-1))
+    q = ReorderProblem(dims=(1, 6), src_dt=cabi.DT_S32, dst_dt=cabi.DT_S32, src=x,
+                       quant={"src_scale": QuantParam(cabi.DT_F32, 0, np.array([1.0], np.float32))})
+    got = oracle.reorder(q)
+    assert got[0] == 2 ** 24 and got[1] == -(2 ** 31) and got[4] == -7       # 2^24 + 1 is not a float
+
+
 def test_conversions_between_the_float_types():
     x = rng(8).standard_normal(64).astype(np.float32) * 3
     for dt, enc in ((cabi.DT_BF16, dtp.f32_to_bf16), (cabi.DT_F16, dtp.f32_to_f16_bits),
@@ -203,6 +217,9 @@ def _qp(seed, dt, mask, shape, groups=(1, 1), lo=0.05, hi=2.0):
 
 
 CASES = [
+    # s32 over its whole range: a copy or a transposition keeps every bit (values beyond 2^24 included)
+    lambda: _case("s32 copy", (19, 260), cabi.DT_S32, cabi.DT_S32, 38),
+    lambda: _case("s32 transposition", (40, 1000), cabi.DT_S32, cabi.DT_S32, 39, dst_perm=(1, 0)),
     # direct kernel, 16 / 8 elements per lane: attribute-free (one base per unit) ...
     lambda: _case("s8 copy 16 per lane", (24, 512), cabi.DT_S8, cabi.DT_S8, 40),
     lambda: _case("u8->f32 16 per lane, rows strided", (3, 40, 64), cabi.DT_U8, cabi.DT_F32, 41, src_perm=(1, 0, 2)),
