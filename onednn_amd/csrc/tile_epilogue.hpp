@@ -857,12 +857,12 @@ __device__ __forceinline__ void storeQ(const PT &P, const epi_uniform_t &H, cons
 // of every group and leaves v scaled and saturated, ready for the fp8
 // conversion.  All lanes take part in the cross-lane maximum, rows beyond M on
 // the data of a valid row; only the stores are masked.
-template <class Layout, int Q, class PT>
-__device__ __forceinline__ void dynamic_quantQ(const PT &P, int dst_dt, int mode, float (&v)[Q][4], long b, long m,
+template <class Layout, int Q, bool FP, class PT>
+__device__ __forceinline__ void dynamic_quantQ(const PT &P, int dst_dt, float (&v)[Q][4], long b, long m,
         bool ok, const long (&n)[Q], int lane) {
     constexpr int QPG = Layout::QPG;
     const float dt_max = dst_dt == MI355_DT_F8_E4M3 ? 448.f : (dst_dt == MI355_DT_F4_E2M1 ? 6.f : 57344.f);
-    if (mode == MI355_DST_DYNAMIC_FP) {
+    if (FP) {
         // groups of 16 columns with an f8_e4m3 scale (ref_matmul.cpp:352-365, :381): the lower and the upper
         // half of the lane's quads of 32 columns, shared with the same partner lanes
         constexpr int HQ = QPG / 2;
@@ -1062,7 +1062,8 @@ __device__ __forceinline__ void store_quadrant(const PT &P, char *park, unsigned
                 }
             }
             apply_epilogueQ<Q>(H, ntab, col, v, sy);
-            if (H.dynamic) dynamic_quantQ<Layout, Q>(P, H.dst_dt, H.dynamic, v, b, ok ? m : P.M - 1, ok, n, lane);
+            if (H.dynamic == MI355_DST_DYNAMIC_MX) dynamic_quantQ<Layout, Q, false>(P, H.dst_dt, v, b, ok ? m : P.M - 1, ok, n, lane);
+            else if (H.dynamic) dynamic_quantQ<Layout, Q, true>(P, H.dst_dt, v, b, ok ? m : P.M - 1, ok, n, lane);
             storeQ<Q>(P, H, v, b, m, ok, n);
         }
         return;
