@@ -119,8 +119,8 @@ __global__ void __launch_bounds__(256) h16_zero_tail_kernel(uint16_t *base, long
 // Decompression of row-major 4-bit weights [K][N] (two n per byte, low nibble = even n) into the K-contiguous 16-bit
 // copy the tiles read, [N][K]: value = (w - zp[k / gk][n]) * scale[k / gk][n], the reorder's arithmetic (integer
 // subtraction, one f32 multiplication, round to nearest even).  A workgroup owns 64 k x 256 n: a thread loads the
-// 16 bytes (32 columns) of two adjacent k rows -- eight lanes a whole 128-byte line -- with the scales and zero
-// points of its columns, packs the two k of a column into one dword and parks it in LDS at dword column
+// 16 bytes (32 columns) of two adjacent k rows -- eight lanes a whole 128-byte line -- takes the scales and zero
+// points of its columns from LDS (fetched once per workgroup), packs the two k of a column into one dword and parks it in LDS at dword column
 // (k / 2) ^ 4 (n / 32) of row n, which spreads a store instruction over all banks and keeps every aligned group of
 // four columns together; the tile then leaves as whole 128-byte rows.  The generic tiled reorder took 0.36 ms for
 // 4096 x 14336 weights with grouped parameters; this kernel moves the same 29 MB in and 117 MB out.
@@ -138,75 +138,6 @@ struct woq_dq_t {
 
 typedef uint32_t woq_u4v __attribute__((ext_vector_type(4)));
 
-// the parameters of 32 consecutive columns into registers, 16 bytes a load (idx is a multiple of 32 and the base
-// 16-byte aligned whenever per_n is set)
-__device__ __forceinline__ void woq_scales32(float (&sc)[32], const void *p, int dt, long idx, bool per_n) {
-    if (!p || !per_n) {
-        const float v = p ? load_float(dt, p, idx) : 1.f;
-#pragma unroll
-        for (int e = 0; e < 32; ++e) sc[e] = v;
-    } else if (dt == MI355_DT_F32) {
-        const woq_u4v *q = (const woq_u4v *)((const float *)p + idx);
-#pragma unroll
-        for (int j = 0; j < 8; ++j) {
-            const woq_u4v v = q[j];
-            sc[4 * j] = __uint_as_float(v.x), sc[4 * j + 1] = __uint_as_float(v.y);
-            sc[4 * j + 2] = __uint_as_float(v.z), sc[4 * j + 3] = __uint_as_float(v.w);
-        }
-    } else {
-        const woq_u4v *q = (const woq_u4v *)((const uint16_t *)p + idx);
-        const bool bf = dt == MI355_DT_BF16;
-#pragma unroll
-        for (int j = 0; j < 4; ++j) {
-            const woq_u4v v = q[j];
-            const uint32_t d[4] = {v.x, v.y, v.z, v.w};
-#pragma unroll
-            for (int i = 0; i < 4; ++i) {
-                const uint16_t lo = (uint16_t)d[i], hi = (uint16_t)(d[i] >> 16);
-                sc[8 * j + 2 * i] = bf ? __uint_as_float((uint32_t)lo << 16) : (float)__builtin_bit_cast(_Float16, lo);
-                sc[8 * j + 2 * i + 1] = bf ? __uint_as_float((uint32_t)hi << 16) : (float)__builtin_bit_cast(_Float16, hi);
-            }
-        }
-    }
-}
-
-__device__ __forceinline__ void woq_zps32(int (&zp)[32], const void *p, int dt, long idx, bool per_n) {
-    if (!p || !per_n) {
-        const int v = p ? load_int(dt, p, idx) : 0;
-#pragma unroll
-        for (int e = 0; e < 32; ++e) zp[e] = v;
-    } else if (dt == MI355_DT_S32) {
-        const woq_u4v *q = (const woq_u4v *)((const int *)p + idx);
-#pragma unroll
-        for (int j = 0; j < 8; ++j) {
-            const woq_u4v v = q[j];
-            zp[4 * j] = (int)v.x, zp[4 * j + 1] = (int)v.y, zp[4 * j + 2] = (int)v.z, zp[4 * j + 3] = (int)v.w;
-        }
-    } else if (dt == MI355_DT_S8 || dt == MI355_DT_U8) {
-        const woq_u4v *q = (const woq_u4v *)((const uint8_t *)p + idx);
-        const bool sg = dt == MI355_DT_S8;
-#pragma unroll
-        for (int j = 0; j < 2; ++j) {
-            const woq_u4v v = q[j];
-            const uint32_t d[4] = {v.x, v.y, v.z, v.w};
-#pragma unroll
-            for (int e = 0; e < 16; ++e) {
-                const uint32_t b = (d[e >> 2] >> (8 * (e & 3))) & 255;
-                zp[16 * j + e] = sg ? (int)(int8_t)b : (int)b;
-            }
-        }
-    } else { // s4 / u4
-        const woq_u4v v = *(const woq_u4v *)((const uint8_t *)p + idx / 2);
-        const uint32_t d[4] = {v.x, v.y, v.z, v.w};
-        const bool sg = dt == MI355_DT_S4;
-#pragma unroll
-        for (int e = 0; e < 32; ++e) {
-            const uint32_t b = (d[e >> 3] >> (4 * (e & 7))) & 15;
-            zp[e] = sg ? (int)(b ^ 8) - 8 : (int)b;
-        }
-    }
-}
-
 __global__ void __launch_bounds__(256) woq_dequant_kernel(const woq_dq_t A) {
     typedef woq_u4v u4v;
     __shared__ __attribute__((aligned(16))) uint32_t tile[256 * 32];
@@ -217,21 +148,61 @@ __global__ void __launch_bounds__(256) woq_dequant_kernel(const woq_dq_t A) {
     const long k = k0 + 2 * kp;
     const u4v w0 = __builtin_nontemporal_load((const u4v *)(A.wei + (k * A.ldw + nb) / 2));
     const u4v w1 = __builtin_nontemporal_load((const u4v *)(A.wei + ((k + 1) * A.ldw + nb) / 2));
+    // The 64 rows of k share their parameters (groups are whole 64s): thread t fetches those of column n0 + t once
+    // for the workgroup -- 32 threads per column block asking for the same 80 bytes each was most of what the
+    // vector-memory path had to serve.
+    __shared__ __attribute__((aligned(16))) float s_sc[256];
+    __shared__ __attribute__((aligned(16))) int s_zp[256];
+    {
+        float scv = 1.f;
+        int zpv = 0;
+        if (A.sc)
+            scv = load_float(A.sc_dt, A.sc,
+                    (A.sc_gk ? (k0 / A.sc_gk) * (long)(A.sc_per_n ? A.N : 1) : 0) + (A.sc_per_n ? n0 + t : 0));
+        if (A.zp)
+            zpv = load_int(A.zp_dt, A.zp,
+                    (A.zp_gk ? (k0 / A.zp_gk) * (long)(A.zp_per_n ? A.N : 1) : 0) + (A.zp_per_n ? n0 + t : 0));
+        s_sc[t] = scv;
+        s_zp[t] = zpv;
+    }
+    __syncthreads();
     float sc[32];
     int zp[32];
-    woq_scales32(sc, A.sc, A.sc_dt, (A.sc_gk ? (k / A.sc_gk) * (long)(A.sc_per_n ? A.N : 1) : 0) + (A.sc_per_n ? nb : 0),
-            A.sc_per_n);
-    woq_zps32(zp, A.zp, A.zp_dt, (A.zp_gk ? (k / A.zp_gk) * (long)(A.zp_per_n ? A.N : 1) : 0) + (A.zp_per_n ? nb : 0),
-            A.zp_per_n);
+#pragma unroll
+    for (int e = 0; e < 32; e += 4) {
+        const float4 a = *(const float4 *)&s_sc[32 * c + e];
+        const int4 z = *(const int4 *)&s_zp[32 * c + e];
+        sc[e] = a.x, sc[e + 1] = a.y, sc[e + 2] = a.z, sc[e + 3] = a.w;
+        zp[e] = z.x, zp[e + 1] = z.y, zp[e + 2] = z.z, zp[e + 3] = z.w;
+    }
     const uint32_t d0[4] = {w0.x, w0.y, w0.z, w0.w}, d1[4] = {w1.x, w1.y, w1.z, w1.w};
     const int sx = A.signed_w ? 8 : 0; // (b ^ 8) - 8 sign-extends a nibble
+    // bf16: v_cvt_pk_bf16_f32 rounds to nearest even like the software conversion for normal numbers, zeros and
+    // infinities; that one flushes f32 subnormals and quiets NaNs its own way, so a wavefront that meets either
+    // (class mask: s/q NaN, +-subnormal) redoes its part in software
+    bool special = false;
+    if (A.out_bf16) {
+        typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
+        typedef float f32x2_t __attribute__((ext_vector_type(2)));
 #pragma unroll
-    for (int e = 0; e < 32; ++e) {
-        const int v0 = (int)(((d0[e >> 3] >> (4 * (e & 7))) & 15) ^ sx) - sx;
-        const int v1 = (int)(((d1[e >> 3] >> (4 * (e & 7))) & 15) ^ sx) - sx;
-        const float f0 = sc[e] * (float)(v0 - zp[e]), f1 = sc[e] * (float)(v1 - zp[e]);
-        const unsigned lo = A.out_bf16 ? f32_to_bf16(f0) : f32_to_f16(f0), hi = A.out_bf16 ? f32_to_bf16(f1) : f32_to_f16(f1);
-        tile[(32 * c + e) * 32 + (kp ^ (4 * c))] = lo | (hi << 16);
+        for (int e = 0; e < 32; ++e) {
+            const int v0 = (int)(((d0[e >> 3] >> (4 * (e & 7))) & 15) ^ sx) - sx;
+            const int v1 = (int)(((d1[e >> 3] >> (4 * (e & 7))) & 15) ^ sx) - sx;
+            const float f0 = sc[e] * (float)(v0 - zp[e]), f1 = sc[e] * (float)(v1 - zp[e]);
+            special |= __builtin_amdgcn_classf(f0, 0x93) | __builtin_amdgcn_classf(f1, 0x93);
+            tile[(32 * c + e) * 32 + (kp ^ (4 * c))]
+                    = __builtin_bit_cast(unsigned, __builtin_convertvector(f32x2_t {f0, f1}, bf16x2_t));
+        }
+    }
+    if (!A.out_bf16 || __builtin_amdgcn_ballot_w64(special) != 0) {
+#pragma unroll
+        for (int e = 0; e < 32; ++e) {
+            const int v0 = (int)(((d0[e >> 3] >> (4 * (e & 7))) & 15) ^ sx) - sx;
+            const int v1 = (int)(((d1[e >> 3] >> (4 * (e & 7))) & 15) ^ sx) - sx;
+            const float f0 = sc[e] * (float)(v0 - zp[e]), f1 = sc[e] * (float)(v1 - zp[e]);
+            const unsigned lo = A.out_bf16 ? f32_to_bf16(f0) : f32_to_f16(f0), hi = A.out_bf16 ? f32_to_bf16(f1) : f32_to_f16(f1);
+            tile[(32 * c + e) * 32 + (kp ^ (4 * c))] = lo | (hi << 16);
+        }
     }
     __syncthreads();
     const int q = t & 7, r = t >> 3; // write: row r + 32 pass, dwords of the physical group q

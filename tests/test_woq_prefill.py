@@ -147,3 +147,27 @@ def test_decode_and_prefill_of_the_same_weights_differ_by_the_weight_rounding_on
     err = np.abs(a - b)
     assert (err <= tol).all(), f"worst {np.max(err / tol):.2f} of the bound"
     assert err.max() > 0                                                    # the two flavours do differ
+
+
+@pytest.mark.gpu
+def test_the_decompressed_weights_themselves(gpu):
+    """src = identity, so dst is the weights copy the launch wrote: (w - zp) * scale rounded to bf16 the way the
+    reference rounds (nearest even; f32 subnormals flush to zero, bfloat16.cpp:29-49).  A third of the scale groups
+    are f32 subnormals, so those wavefronts of the decompression kernel leave the hardware conversion for the
+    software one; the others stay on it.  Every element against numpy."""
+    M = N = K = 256
+    p = configs.woq_variant(M, N, K, 64, sc_dt="f32", zp_dt="u8")
+    p.src = dtp.f32_to_bf16(np.eye(M, dtype=np.float32).reshape(-1)).reshape(M, K)
+    sc = np.asarray(p.quant["wei_scale"].data).copy().reshape(K // 64, N)
+    sc[1] = np.float32(2.0 ** -140)                      # subnormal products (flushed by the conversion)
+    sc[2, ::2] = np.float32(3.0e-39)                     # subnormal scales next to normal ones
+    p.quant["wei_scale"].data = sc
+    st, impl = cabi.query(p.desc())
+    assert st == cabi.SUCCESS and impl == cabi.IMPL_H16_MFMA
+    got = dtp.bf16_to_f32(np.asarray(run_gpu(p)[0]).view(np.uint16).reshape(-1)).reshape(M, N)
+    codes = dtp.unpack_nibbles(np.asarray(p.wei).reshape(-1), K * N).reshape(K, N).astype(np.int32)
+    zp = np.asarray(p.quant["wei_zp"].data).reshape(K // 64, N).astype(np.int32)
+    w = ((codes - zp.repeat(64, axis=0)).astype(np.float32) * sc.repeat(64, axis=0)).astype(np.float32)
+    want = dtp.bf16_to_f32(dtp.f32_to_bf16(w.reshape(-1))).reshape(K, N)
+    assert np.array_equal(got, want)
+    assert np.all(want[64:128] == 0) and np.any(want[:64] != 0)
