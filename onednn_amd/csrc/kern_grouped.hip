@@ -241,6 +241,19 @@ template <int DT>
 __device__ __forceinline__ void gk_store(const grouped_k_dev_t &P, const gk_f4 (&acc)[4][4], long g, long m_w, long n_w,
         int j, int q) {
     const long col = n_w + 4 * j;
+    // bf16: v_cvt_pk_bf16_f32 unless the wavefront holds a NaN or an f32 subnormal, which the software conversion
+    // (the reference's: subnormals flush, NaNs are quieted its way) treats differently
+    bool hw = false;
+    if (DT == MI355_DT_BF16) {
+        bool special = false;
+#pragma unroll
+        for (int r = 0; r < 4; ++r)
+#pragma unroll
+            for (int c = 0; c < 4; ++c)
+#pragma unroll
+                for (int e = 0; e < 4; ++e) special |= __builtin_amdgcn_classf(acc[r][c][e], 0x93);
+        hw = __builtin_amdgcn_ballot_w64(special) == 0;
+    }
     if (col >= P.NB) return;
 #pragma unroll
     for (int r = 0; r < 4; ++r)
@@ -252,6 +265,13 @@ __device__ __forceinline__ void gk_store(const grouped_k_dev_t &P, const gk_f4 (
             const float v0 = acc[r][0][e], v1 = acc[r][1][e], v2 = acc[r][2][e], v3 = acc[r][3][e];
             if (DT == MI355_DT_F32) {
                 *(gk_f4 *)((float *)P.dst + off) = gk_f4 {v0, v1, v2, v3};
+            } else if (DT == MI355_DT_BF16 && hw) {
+                typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
+                typedef float f32x2_t __attribute__((ext_vector_type(2)));
+                gk_u2 o;
+                o.x = __builtin_bit_cast(unsigned, __builtin_convertvector(f32x2_t {v0, v1}, bf16x2_t));
+                o.y = __builtin_bit_cast(unsigned, __builtin_convertvector(f32x2_t {v2, v3}, bf16x2_t));
+                *(gk_u2 *)((uint16_t *)P.dst + off) = o;
             } else {
                 gk_u2 o;
                 o.x = (cvt_store_bits(DT, v0) & 0xffffu) | (cvt_store_bits(DT, v1) << 16);
