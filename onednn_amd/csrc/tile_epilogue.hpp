@@ -705,12 +705,31 @@ __device__ __forceinline__ void storeQ(const PT &P, const epi_uniform_t &H, cons
     const long rowoff = b * P.ds[0] + m * P.ds[1];
     if (dt_bits(dt) == 4) {
         // two bytes a quad, low nibble first; rows and quads start whole bytes (checked by the host), possibly at an
-        // odd address
+        // odd address.  f4_e2m1 by v_cvt_scalef32_pk_fp4_f32 (nearest even, saturating at +-6 like the software
+        // conversion: checked code for code on the device, tests/test_dynamic_dst.py) unless the wavefront holds a
+        // NaN, which the software conversion turns into +-6
+        bool hw = false;
+        if (dt == MI355_DT_F4_E2M1) {
+            bool nan = false;
+#pragma unroll
+            for (int k = 0; k < Q; ++k)
+#pragma unroll
+                for (int e = 0; e < 4; ++e) nan |= __builtin_amdgcn_classf(v[k][e], 0x3);
+            hw = __builtin_amdgcn_ballot_w64(nan) == 0;
+        }
 #pragma unroll
         for (int k = 0; k < Q; ++k) {
-            uint32_t c[4];
-            cvt4(dt, v[k], c);
-            const uint32_t lo = c[0] | (c[1] << 4), hi = c[2] | (c[3] << 4);
+            uint32_t lo, hi;
+            if (hw) {
+                unsigned r = 0;
+                r = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(r, v[k][0], v[k][1], 1.f, 0);
+                r = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(r, v[k][2], v[k][3], 1.f, 1);
+                lo = r & 0xffu, hi = (r >> 8) & 0xffu;
+            } else {
+                uint32_t c[4];
+                cvt4(dt, v[k], c);
+                lo = c[0] | (c[1] << 4), hi = c[2] | (c[3] << 4);
+            }
             uint8_t *q = (uint8_t *)P.dst + ((rowoff + n[k]) >> 1);
             if (!ok) continue;
             if ((uintptr_t)q & 1) q[0] = (uint8_t)lo, q[1] = (uint8_t)hi;

@@ -474,3 +474,39 @@ def test_gpu_4bit_dst_with_a_static_scale_is_bit_exact(gpu, oracle, dst):
     g, w = np.asarray(got).view(np.uint8), np.asarray(want).view(np.uint8)
     assert np.array_equal(g, w)
     assert len(np.unique(np.concatenate([w & 0xf, w >> 4]))) >= 8        # not a degenerate result
+
+
+@pytest.mark.gpu
+def test_gpu_the_tiles_convert_to_f4_like_the_reference(gpu, oracle):
+    """dst = I x W in f32, so every dst code is the conversion of a chosen f32 value: every midpoint between two
+    e2m1 values and its f32 neighbours (ties go to the even code), both signs, zero, subnormals, values beyond 6,
+    infinities, and random values over many binades -- the tiles (hardware conversion) against the oracle's
+    software conversion (float4 of the reference), code for code.  A NaN anywhere sends a wavefront to the software
+    path; one column block holds NaNs to cover that too."""
+    M = N = K = 256
+    r = np.random.default_rng(3)
+    mids = np.array([0.25, 0.75, 1.25, 1.75, 2.5, 3.5, 5.0, 6.0, 0.5, 1.0, 1.5, 2.0, 3.0, 4.0], np.float32)
+    near = np.concatenate([mids, np.nextafter(mids, np.float32(0)), np.nextafter(mids, np.float32(10))])
+    special = np.array([0.0, 1e-45, 1e-38, 5.9999995, 6.0000005, 7.0, 448.0, 1e30, np.inf], np.float32)
+    vals = np.concatenate([near, special])
+    vals = np.concatenate([vals, -vals])
+    W = (r.standard_normal((K, N)) * np.exp2(r.integers(-4, 4, size=(K, N)))).astype(np.float32)
+    W.reshape(-1)[:vals.size] = vals
+    W[:, 192:200] = r.choice([np.nan, 1.0, -2.5, 6.5], size=(K, 8)).astype(np.float32)
+    p = MatmulProblem(M=M, N=N, K=K, src_dt=cabi.DT_F32, wei_dt=cabi.DT_F32, dst_dt=cabi.DT_F4_E2M1,
+                      src=np.eye(M, dtype=np.float32), wei=W, name="f4-conversion")
+    run = GpuRun(p, None)
+    try:
+        run.launch()
+        got, name = run.result(), cabi.impl_name(run.impl)
+    finally:
+        run.free()
+    assert name.startswith("hip:mfma_h16")
+    want = orc.run_oracle(p)
+    g, w = unpack_dst(got, cabi.DT_F4_E2M1, M, N), unpack_dst(want, cabi.DT_F4_E2M1, M, N)
+    nan = np.isnan(W)
+    # 0 x NaN spoils the whole column of a NaN; elsewhere the codes are the conversions of W (the sign of a zero aside)
+    clean = ~nan.any(axis=0)
+    same = (g == w) | ((g & 7) == 0) & ((w & 7) == 0)
+    assert np.all(same[:, clean]), np.argwhere(~same[:, clean])[:5]
+    assert np.all((g[:, ~clean] & 7) == (w[:, ~clean] & 7))
