@@ -16,7 +16,9 @@ from tests import benchdnn_matmul as bd
 DTS = [("u8:s8:f32", "i8"), ("s8:s8:s8", "i8"), ("u8:s8:u8", "i8"), ("s8:s8:s32", "i8"), ("u8:u8:bf16", "i8"),
        ("f8_e4m3:f8_e4m3:bf16", "f8"), ("f8_e5m2:f8_e4m3:f32", "f8"), ("f8_e4m3:f8_e5m2:f8_e4m3", "f8"),
        ("bf16:bf16:bf16", "h"), ("f16:f16:f32", "h"), ("f32:f32:f32", "h"), ("bf16:bf16:f32", "h"),
-       ("bf16:u4:bf16", "woq"), ("f16:s4:f16", "woq"), ("bf16:s8:bf16", "woq")]
+       ("bf16:u4:bf16", "woq"), ("f16:s4:f16", "woq"), ("bf16:s8:bf16", "woq"),
+       ("f8_e4m3:f8_e4m3:bf16", "mx"), ("f8_e5m2:f8_e4m3:f32", "mx"), ("f4_e2m1:f4_e2m1:bf16", "mx"),
+       ("f4_e2m1:f4_e2m1:f32", "mx")]
 POST_OPS = ["relu", "linear:2:1", "add:f32", "add:bf16:per_oc", "mul:f32:per_oc", "sum", "gelu_tanh", "clip:-1:2", "tanh",
             "max:f32", "sum:0.5", "swish:1", "abs"]
 
@@ -55,6 +57,11 @@ def random_case(rnd):
             sc.append("src:common:0.5")
         if rnd.random() < 0.6:
             sc.append(rnd.choice(["wei:per_oc", "wei:common:2"]))
+    elif fam == "mx":       # e8m0 scales per 32 k on both operands
+        K = 32 * rnd.choice([1, 2, 3, 4, 5, 8, 9, 16, 17])
+        N += N % 2
+        sc.append("src:per_tensor:e8m0:1x32")
+        sc.append("wei:per_tensor:e8m0:32x1")
     elif fam == "woq":
         G = rnd.choice([32, 64, 128])
         K = max(G, (K // G) * G)
@@ -101,5 +108,5 @@ def test_random_problems_match_the_oracle(gpu, oracle, seed):
             failures.append((specs[0].repro(), impl, details if isinstance(details, str) else details.get("errors")))
     assert not failures, failures[:5]
     # the sweep reaches the tuned families, not only the generic kernel
-    for family in ("hip:mfma_i8", "hip:mfma_f8", "hip:mfma_h16", "hip:ref:any"):
+    for family in ("hip:mfma_i8", "hip:mfma_f8", "hip:mfma_h16", "hip:mfma_mxf4", "hip:ref:any"):
         assert impls.get(family, 0) > 0, impls
