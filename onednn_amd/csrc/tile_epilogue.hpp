@@ -70,6 +70,23 @@ __device__ __forceinline__ float gelu_tanh_fast(float s) {
     const float e = __builtin_amdgcn_exp2f(-2.8853900817779268f * v); // exp(-2v)
     return s * __builtin_amdgcn_rcpf(1.f + e);
 }
+// logistic(s) = 1 / (1 + exp(-s)) and swish(s) = s logistic(alpha s)
+// (math_utils.hpp logistic_fwd, swish_fwd) the same way.  Where s is negative
+// the result is exp(s) to first order, so the exponential has to be good to a
+// few ulp by itself: the rounding of the product s log2(e) (|s| 2^-24 in the
+// exponent) is recovered by an fma and applied to first order,
+// exp2(hi + lo) = exp2(hi) (1 + lo ln 2).  exp(-s) overflows to infinity where
+// the reference returns 0 outright, and the reciprocal of that is the same 0.
+__device__ __forceinline__ float logistic_fast(float s) {
+    const float c = -1.44269502162933349609375f; // -log2(e) rounded; the rest of it follows
+    const float hi = c * s;
+    float lo = __builtin_fmaf(c, s, -hi);
+    lo = __builtin_fmaf(-1.92596299e-8f, s, lo);
+    float e = __builtin_amdgcn_exp2f(hi);
+    // (outside: e is 0 or infinity, or s is not finite, and the correction would make NaN of it)
+    if (fabsf(hi) < 126.f) e = __builtin_fmaf(e, lo * 0.693147182464599609375f, e);
+    return __builtin_amdgcn_rcpf(1.f + e);
+}
 
 // x / s by two Newton corrections of x * (1 / s):
 //   q0 = x y, r0 = x - s q0 (one fma, exact), q1 = q0 + r0 y, r1 = x - s q1, q = q1 + r1 y
@@ -223,7 +240,8 @@ __device__ __forceinline__ epi_uniform_t make_uniform(const PT &P, bool cols_ins
             const bool simple_elt = r.kind == MI355_PO_ELTWISE
                     && (r.alg == MI355_ELTWISE_RELU || r.alg == MI355_ELTWISE_LINEAR
                             || r.alg == MI355_ELTWISE_GELU_TANH || r.alg == MI355_ELTWISE_CLIP
-                            || r.alg == MI355_ELTWISE_CLIP_V2);
+                            || r.alg == MI355_ELTWISE_CLIP_V2 || r.alg == MI355_ELTWISE_SWISH
+                            || r.alg == MI355_ELTWISE_LOGISTIC);
             return simple_elt || r.kind == MI355_PO_BINARY || r.kind == MI355_PO_SUM;
         };
         H.nfast = 0;
@@ -498,6 +516,16 @@ __device__ __forceinline__ void eltwiseQ_simple(int alg, float (&v)[Q][4], float
         for (int k = 0; k < Q; ++k)
 #pragma unroll
             for (int e = 0; e < 4; ++e) v[k][e] = gelu_tanh_fast(v[k][e]) * scale;
+    } else if (alg == MI355_ELTWISE_SWISH) {
+#pragma unroll
+        for (int k = 0; k < Q; ++k)
+#pragma unroll
+            for (int e = 0; e < 4; ++e) v[k][e] = v[k][e] * logistic_fast(alpha * v[k][e]) * scale;
+    } else if (alg == MI355_ELTWISE_LOGISTIC) {
+#pragma unroll
+        for (int k = 0; k < Q; ++k)
+#pragma unroll
+            for (int e = 0; e < 4; ++e) v[k][e] = logistic_fast(v[k][e]) * scale;
     } else if (alg == MI355_ELTWISE_CLIP) {
 #pragma unroll
         for (int k = 0; k < Q; ++k)

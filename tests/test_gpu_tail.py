@@ -132,6 +132,30 @@ def test_eltwise_algorithms(gpu, oracle, name, impl):
         assert ok.all(), (name, impl_name, got[~ok][:4], orc[~ok][:4])
 
 
+@pytest.mark.parametrize("name,alpha", [("swish", 1.5), ("swish", -0.75), ("logistic", 0.0)])
+def test_swish_and_logistic_on_full_tiles(gpu, oracle, name, alpha):
+    # the tile kernels evaluate these two with the hardware exponential and reciprocal; where the argument is
+    # negative the result is the exponential itself, so its accuracy shows: arguments out to +-25 (the result
+    # down to 1e-16), every element against the float64 formula on the float32 product alpha * s the reference forms
+    p, x = tc._int8_base(21, False, 0.11, M=256, N=256, K=64)
+    p.post_ops = [PostOp(kind=cabi.PO_ELTWISE, alg=cabi.ELTWISE[name], alpha=alpha, beta=0.0, scale=1.0)]
+    got_raw, impl_name = run_gpu(p)
+    assert impl_name.startswith("hip:mfma_i8"), impl_name
+    got = logical(p, got_raw).reshape(p.M, p.N)
+    x64 = x.astype(np.float64)
+    assert x64.min() < -18 and x64.max() > 18
+    with np.errstate(over="ignore"):
+        if name == "swish":
+            want = x64 / (1.0 + np.exp(-(F(alpha) * x).astype(np.float64)))
+        else:
+            want = 1.0 / (1.0 + np.exp(-x64))
+    ok = tc.ulp_close(got, want, ulps=8, atol=1e-37)
+    assert ok.all(), (impl_name, x[~ok][:4], got[~ok][:4], want[~ok][:4])
+    orc = logical(p, oracle.run_oracle(p)).reshape(p.M, p.N)
+    ok = tc.ulp_close(got, orc.astype(np.float64), ulps=12, atol=2e-37)
+    assert ok.all(), (impl_name, x[~ok][:4], got[~ok][:4], orc[~ok][:4])
+
+
 @pytest.mark.parametrize("impl", IMPLS)
 @pytest.mark.parametrize("name", tc.BINARY_TAIL)
 @pytest.mark.parametrize("operand,odt", [("per_element", "f32"), ("per_n", "f32"), ("per_m", "s8"), ("scalar", "bf16")])
