@@ -641,6 +641,139 @@ __device__ __forceinline__ void grouped_walk(const grouped_dev_t &P, const gtile
         for (int jn = 0; jn < NT; ++jn) part[((wk * MF + i) * NT + jn) * 64 + lane] = acc[i][jn];
 }
 
+// The same walk for row-major weights ([G][K][N], tag abc: a k row holds its N columns) of the 16-bit types, 64
+// columns a tile.  A column's eight consecutive k lie a row pitch apart, so a lane fetches 8 bytes -- four columns
+// 4 j .. 4 j + 3 -- of each of the rows k = 8 q .. 8 q + 7 and 32 + 8 q .. (a load instruction covers whole lines:
+// four rows x 128 bytes) and turns them inside the lane (`gk_frag16`) into the four fragments it needs: fragment
+// c holds column 4 j + c in lane (j, q).  The matrix instruction does not mind which 16 columns share a fragment;
+// the accumulators -- acc[i][c][e] is src row 16 i + j, column 16 q + 4 e + c -- are written to `part` in the
+// arrangement of the K-contiguous walk (unit q, lane (j, e), element c), so the same epilogue follows.
+template <int MODE, int MF, int D, int WK, bool NTL>
+__device__ __forceinline__ void grouped_walk_bt(const grouped_dev_t &P, const gtile_t &T, g4f *part, int wk, int lane) {
+    constexpr int NT = 4;
+    using Mo = gmode_t<MODE>;
+    static_assert(Mo::EBITS == 16, "row-major weights: bf16 / f16 only");
+    const mi355_grouped_desc_t &Dd = P.d;
+    const int j = lane & 15, q = lane >> 4, half = j >> 3;
+    const long row_bytes = 2 * Dd.K;
+    const uint32_t chunk = 16 * Mo::chunk_fetch(q, half);
+    const char *abase = (const char *)P.a.src + (T.src0 + T.m_base) * row_bytes;
+    uint32_t aoff[MF][2];
+#pragma unroll
+    for (int i = 0; i < MF; ++i)
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+            long m = T.m_base + 16 * i + 8 * h + (j & 7);
+            m = m < T.rows ? m : T.rows - 1;
+            aoff[i][h] = (uint32_t)((m - T.m_base) * row_bytes) + chunk;
+        }
+    const long pitch_b = 2 * Dd.wei_stride[1];
+    long col = T.n0 + 4 * j;
+    col = col <= Dd.N - 4 ? col : Dd.N - 4; // N is a multiple of 4; columns beyond N are never stored
+    const char *bbase = (const char *)P.a.wei + 2 * (T.g * Dd.wei_stride[0] + col) + 8 * q * pitch_b;
+    struct stage_t {
+        g4i a[MF][2];
+        gk_u2 b[2][8];
+    };
+    // k0: the step's first k (uniform)
+    auto load = [&](long k0) __attribute__((always_inline)) {
+        stage_t f;
+#pragma unroll
+        for (int h = 0; h < 2; ++h)
+#pragma unroll
+            for (int r = 0; r < 8; ++r) {
+                const gk_u2 *bp = (const gk_u2 *)(bbase + (k0 + 32 * h + r) * pitch_b);
+                f.b[h][r] = NTL ? __builtin_nontemporal_load(bp) : *bp;
+            }
+#pragma unroll
+        for (int i = 0; i < MF; ++i)
+#pragma unroll
+            for (int h = 0; h < 2; ++h) f.a[i][h] = *(const g4i *)(abase + 2 * k0 + aoff[i][h]);
+        return f;
+    };
+    auto settle = [&](const g4i (&r)[2]) __attribute__((always_inline)) {
+        g8i out;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            const int send = half ? r[0][e] : r[1][e];
+            const int recv = __builtin_amdgcn_update_dpp(0, send, 0x128 /* row_ror:8 */, 0xf, 0xf, false);
+            out[e] = half ? recv : r[0][e];
+            out[4 + e] = half ? r[1][e] : recv;
+        }
+        return out;
+    };
+    g4f acc[MF][NT];
+#pragma unroll
+    for (int i = 0; i < MF; ++i)
+#pragma unroll
+        for (int c = 0; c < NT; ++c) acc[i][c] = g4f {0.f, 0.f, 0.f, 0.f};
+    auto compute = [&](const stage_t &f) __attribute__((always_inline)) {
+        g8i a[MF];
+#pragma unroll
+        for (int i = 0; i < MF; ++i) a[i] = settle(f.a[i]);
+#pragma unroll
+        for (int c = 0; c < NT; ++c) {
+            const g4u lo = gk_frag16(f.b[0], c), hi = gk_frag16(f.b[1], c);
+            const g8i w = {(int)lo[0], (int)lo[1], (int)lo[2], (int)lo[3], (int)hi[0], (int)hi[1], (int)hi[2], (int)hi[3]};
+#pragma unroll
+            for (int i = 0; i < MF; ++i) acc[i][c] = grouped_mma<MODE, 0, 0>(w, a[i], acc[i][c]);
+        }
+    };
+
+    const long nfull = Dd.K / 64;
+    const int tail = (int)(Dd.K % 64); // a multiple of 16
+    if (nfull > wk) {
+        const long count = (nfull - wk + WK - 1) / WK;
+        const long c0 = (long)((blockIdx.x * 5u + blockIdx.y * 3u) % (unsigned long)count);
+        auto step_k0 = [&](long c) {
+            long cr = (c < count ? c : count - 1) + c0;
+            cr = cr >= count ? cr - count : cr;
+            return (wk + WK * cr) * 64;
+        };
+        stage_t st[D];
+#pragma unroll
+        for (int d = 0; d < D; ++d) st[d] = load(step_k0(d));
+        long c = 0;
+        for (; c + D <= count; c += D) {
+#pragma unroll
+            for (int d = 0; d < D; ++d) {
+                compute(st[d]);
+                st[d] = load(step_k0(c + D + d));
+                __builtin_amdgcn_sched_barrier(0);
+            }
+        }
+#pragma unroll
+        for (int d = 0; d < D; ++d)
+            if (c + d < count) compute(st[d]);
+    }
+    if (tail != 0 && wk == (int)(nfull % WK)) {
+        // k beyond K: zeros on both sides (a product with a zero operand would still be NaN against an infinity)
+        stage_t f;
+        const long k0 = nfull * 64;
+        const bool in = chunk + 16 <= (uint32_t)(2 * tail);
+#pragma unroll
+        for (int i = 0; i < MF; ++i)
+#pragma unroll
+            for (int h = 0; h < 2; ++h) {
+                f.a[i][h] = g4i {0, 0, 0, 0};
+                if (in) f.a[i][h] = *(const g4i *)(abase + 2 * k0 + aoff[i][h]);
+            }
+#pragma unroll
+        for (int h = 0; h < 2; ++h)
+#pragma unroll
+            for (int r = 0; r < 8; ++r) {
+                f.b[h][r] = gk_u2 {0u, 0u};
+                if (32 * h + 8 * q + r < tail) f.b[h][r] = *(const gk_u2 *)(bbase + (k0 + 32 * h + r) * pitch_b);
+            }
+        compute(f);
+    }
+#pragma unroll
+    for (int i = 0; i < MF; ++i)
+#pragma unroll
+        for (int e = 0; e < 4; ++e)
+            part[((wk * MF + i) * NT + q) * 64 + j + 16 * e] = g4f {acc[i][0][e], acc[i][1][e], acc[i][2][e], acc[i][3][e]};
+}
+
 // Which (group, row block) is slot `slot`: a block-wide prefix sum over the
 // groups' row-block counts.  False (for the whole workgroup) beyond the last tile.
 template <int BM, int NW>
@@ -732,7 +865,8 @@ __device__ __forceinline__ void grouped_store_quad(const grouped_dev_t &P, const
     }
 }
 
-template <int MODE, int FA, int FB, int MTMAX, int NT, int D, int NW, int OCC>
+// BT: row-major weights (`grouped_walk_bt`)
+template <int MODE, int FA, int FB, int MTMAX, int NT, int D, int NW, int OCC, bool BT = false>
 __global__ void __launch_bounds__(64 * NW, OCC) grouped_tile_kernel(const grouped_dev_t P) {
     constexpr int BM = 16 * MTMAX, BN = 16 * NT;
     extern __shared__ g4f part[]; // [wavefront][fragment row][fragment column][lane]
@@ -745,11 +879,16 @@ __global__ void __launch_bounds__(64 * NW, OCC) grouped_tile_kernel(const groupe
     const int mf = __builtin_amdgcn_readfirstlane((int)((here + 15) / 16)); // fragments of 16 rows the tile holds
 
     // ---- K: the wavefronts take the 128-byte steps in turn, each over the whole tile
-    const bool whole_lines = gmode_t<MODE>::bytes(P.d.wei_stride[2]) % 128 == 0;
+    const bool whole_lines = gmode_t<MODE>::bytes(P.d.wei_stride[BT ? 1 : 2]) % 128 == 0;
 #define MI355_GROUPED_WALK(MF_) \
     do { \
-        if (whole_lines) grouped_walk<MODE, FA, FB, MF_, NT, D, NW, true>(P, T, part, wave, lane); \
-        else grouped_walk<MODE, FA, FB, MF_, NT, D, NW, false>(P, T, part, wave, lane); \
+        if constexpr (BT) { \
+            if (whole_lines) grouped_walk_bt<MODE, MF_, D, NW, true>(P, T, part, wave, lane); \
+            else grouped_walk_bt<MODE, MF_, D, NW, false>(P, T, part, wave, lane); \
+        } else { \
+            if (whole_lines) grouped_walk<MODE, FA, FB, MF_, NT, D, NW, true>(P, T, part, wave, lane); \
+            else grouped_walk<MODE, FA, FB, MF_, NT, D, NW, false>(P, T, part, wave, lane); \
+        } \
     } while (0)
     switch (mf) {
         case 1: MI355_GROUPED_WALK(1); break;
@@ -1187,12 +1326,13 @@ bool f8_dt(int dt) { return dt == MI355_DT_F8_E4M3 || dt == MI355_DT_F8_E5M2; }
 struct gshape_t {
     int bm, bn;
 };
-constexpr gshape_t GSHAPES[4] = {{0, 0}, {16, 32}, {48, 64}, {64, 256}};
+constexpr gshape_t GSHAPES[5] = {{0, 0}, {16, 32}, {48, 64}, {64, 256}, {48, 64}};
 
 // 0: the thread-per-element kernel; 1: 16 x 32 tiles, K split between the
 // wavefronts (groups of a row or two: many small workgroups); 2: 48 x 64, K
 // split, two workgroups per compute unit; 3: 64 x 256, columns split, src rows
-// through LDS.  Decided on the descriptor.
+// through LDS; 4: 48 x 64 for row-major weights of the 16-bit types (a 16 x 64 shape with four steps in flight
+// measured the same on groups of one row).  Decided on the descriptor.
 // *mx_out: the plan is one of the MX modes (scales inside the instruction); every other plan has
 // no groups along K (a group size of K counts as none) and applies its scales after the K sum.
 int tile_plan(const mi355_grouped_desc_t &d, bool *mx_out = nullptr) {
@@ -1207,11 +1347,21 @@ int tile_plan(const mi355_grouped_desc_t &d, bool *mx_out = nullptr) {
     if (!f8 && !h16 && !f4 && !i8) return 0;
     const long ebits = f4 ? 4 : (f8 ? 8 : 16);
     auto bytes = [&](long elems) { return elems * ebits / 8; };
-    if (d.wei_stride[1] != 1 || d.wei_stride[2] < d.K) return 0; // K-contiguous weights only
+    auto k_groups = [&](int dt, long gk) { return dt != MI355_DT_UNDEF && gk > 1 && gk != d.K; };
+    const long active = d.group_count < d.total ? d.group_count : d.total;
+    if (h16 && d.wei_stride[2] == 1 && d.wei_stride[1] >= d.N && !(d.wei_stride[1] == 1 && d.wei_stride[2] >= d.K)) {
+        // row-major weights: a lane reads 8 bytes of a k row (four columns), 16 of a src row
+        if (d.N % 4 != 0 || d.wei_stride[1] % 4 != 0 || d.wei_stride[0] % 4 != 0 || d.K % 16 != 0) return 0;
+        if (d.src_zp_dt != MI355_DT_UNDEF || d.wei_zp_dt != MI355_DT_UNDEF) return 0;
+        if (k_groups(d.src_scale_dt, d.src_scale_gk) || k_groups(d.wei_scale_dt, d.wei_scale_gk)) return 0;
+        if (2 * d.K * GSHAPES[4].bm >= (1L << 32)) return 0; // 32-bit offsets of the src rows inside a tile
+        if (d.total / GSHAPES[4].bm + active > 65535) return 0;
+        return 4;
+    }
+    if (d.wei_stride[1] != 1 || d.wei_stride[2] < d.K) return 0; // otherwise K-contiguous weights only
     if (bytes(d.wei_stride[2]) % 16 != 0 || bytes(d.wei_stride[0]) % 16 != 0 || bytes(d.K) % 32 != 0 || d.K % 2 != 0) return 0;
     if (bytes(d.wei_stride[2]) > (1L << 24)) return 0; // 32-bit offsets inside a tile
     if (d.src_zp_dt != MI355_DT_UNDEF || d.wei_zp_dt != MI355_DT_UNDEF) return 0;
-    auto k_groups = [&](int dt, long gk) { return dt != MI355_DT_UNDEF && gk > 1 && gk != d.K; };
     const bool sg = k_groups(d.src_scale_dt, d.src_scale_gk), wg = k_groups(d.wei_scale_dt, d.wei_scale_gk);
     // MX: e8m0 scales per 32 k on both operands of fp8 / fp4 tensors, applied by the instruction; whole
     // 512-byte chunks of K (16 or 32 scale bytes a row), dword loads of the weights' scales along N
@@ -1219,7 +1369,6 @@ int tile_plan(const mi355_grouped_desc_t &d, bool *mx_out = nullptr) {
             && d.src_scale_gk == 32 && d.wei_scale_gk == 32 && bytes(d.K) % 512 == 0 && d.N % 4 == 0;
     if ((sg || wg) && !mx) return 0;
     if (f4 && !mx) return 0;
-    const long active = d.group_count < d.total ? d.group_count : d.total;
     // Groups of a row or two: the small tiles.  Otherwise the 256-column tiles (a quarter of
     // the src traffic per byte of weights), unless they are too few to fill the device or
     // the rows are not whole lines (K not a multiple of 128 bytes: measured slower there).
@@ -1302,6 +1451,10 @@ int launch_tiles(int plan, const grouped_dev_t &P, hipStream_t stream) {
         hipLaunchKernelGGL(kern, grid, dim3(64 * nw), lds, stream, P);
         return hipGetLastError() == hipSuccess ? MI355_SUCCESS : MI355_RUNTIME_ERROR;
     };
+    if (plan == 4) {
+        if constexpr (MODE == GM_BF16 || MODE == GM_F16) return go(grouped_tile_kernel<MODE, 0, 0, 3, 4, 2, 4, 2, true>, 3, 4, 4);
+        return MI355_RUNTIME_ERROR;
+    }
     if (plan == 1) return go(grouped_tile_kernel<MODE, FA, FB, 1, 2, 4, 4, 1>, 1, 2, 4);
     // (the MX modes hold their scales too and do not fit two workgroups' registers)
     if (plan == 2) return go(grouped_tile_kernel<MODE, FA, FB, 3, 4, 2, 4, gmode_t<MODE>::MX ? 1 : 2>, 3, 4, 4);

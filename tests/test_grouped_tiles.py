@@ -1,5 +1,5 @@
 """Grouped matmul on the matrix cores ("hip:mfma_grouped"): fp8 / bf16 / f16 / s8
-operands with K-contiguous weights.
+operands with K-contiguous weights, bf16 / f16 also with row-major ones.
 
   * data every type holds exactly, where any summation order gives the same
     bits: against the oracle (ref_grouped_t's order) bit for bit, both tile
@@ -74,7 +74,18 @@ def test_dispatch_rules():
     assert impl_of(p) == "hip:mfma_grouped"
     p, _ = gc.case_2dx3d([4, 4], 64, 32, src_dt=BF16, wei_dt=BF16, wtag="acb", src_scale="row", wei_scale="col")
     assert impl_of(p) == "hip:mfma_grouped"
-    p, _ = gc.case_2dx3d([4, 4], 64, 32, src_dt=BF16, wei_dt=BF16)                   # N-contiguous weights
+    # row-major ([G][K][N]) weights: the 16-bit types, N a multiple of 4, K of 16
+    p, _ = gc.case_2dx3d([4, 4], 64, 32, src_dt=BF16, wei_dt=BF16)
+    assert impl_of(p) == "hip:mfma_grouped"
+    p, _ = gc.case_2dx3d([4, 4], 48, 36, src_dt=F16, wei_dt=F16, src_scale="row", wei_scale="col", bias=True)
+    assert impl_of(p) == "hip:mfma_grouped"
+    p, _ = gc.case_2dx3d([4, 4], 64, 30, src_dt=BF16, wei_dt=BF16)
+    assert impl_of(p) == "hip:ref_grouped:any"
+    p, _ = gc.case_2dx3d([4, 4], 40, 32, src_dt=BF16, wei_dt=BF16)
+    assert impl_of(p) == "hip:ref_grouped:any"
+    p, _ = gc.case_2dx3d([4, 4], 64, 32, src_dt=E4M3, wei_dt=E4M3)
+    assert impl_of(p) == "hip:ref_grouped:any"
+    p, _ = gc.case_2dx3d([4, 4], 64, 32, src_dt=S8, wei_dt=S8)
     assert impl_of(p) == "hip:ref_grouped:any"
     p, _ = gc.case_2dx3d([4, 4], 64, 32, src_dt=E4M3, wei_dt=E4M3, wtag="acb", wei_scale=32)   # groups along K
     assert impl_of(p) == "hip:ref_grouped:any"
@@ -120,6 +131,27 @@ def test_exact_data_matches_the_oracle(gpu, oracle, tile_shape, shape, tname, sd
             assert st == cabi.SUCCESS
             got = grouped.run_gpu(p)
             assert np.array_equal(got, ref), f"{p.name} {tname} {label} dst {dst_dt} ({tile_shape})"
+            if dst_dt == F32:
+                assert np.array_equal(gc.logical_dst(p, got), want)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("shape", SHAPES + [([5, 50, 9], 80, 200), ([48, 48], 1040, 64)],
+                         ids=lambda s: f"G{len(s[0])}x{sum(s[0])}x{s[1]}x{s[2]}")
+@pytest.mark.parametrize("tname,dt", [("bf16", BF16), ("f16", F16)])
+def test_row_major_weights_exact_data_matches_the_oracle(gpu, oracle, shape, tname, dt):
+    """[G][K][N] weights (tag abc, the reference's default for the grouped matmul): columns gathered four to a lane
+    and transposed in registers.  Every shape of the list; the one whose N is not a multiple of 4 shows the fallback."""
+    from onednn_amd import grouped
+    sizes, K, N = shape
+    for label, kw in EXTRAS:
+        for dst_dt in (F32, BF16):
+            p, want = gc.case_2dx3d(sizes, K, N, src_dt=dt, wei_dt=dt, dst_dt=dst_dt, wtag="abc", **kw)
+            assert impl_of(p) == ("hip:mfma_grouped" if N % 4 == 0 else "hip:ref_grouped:any")
+            st, ref = oracle.run_oracle_grouped(p)
+            assert st == cabi.SUCCESS
+            got = grouped.run_gpu(p)
+            assert np.array_equal(got, ref), f"{p.name} {tname} {label} dst {dst_dt}"
             if dst_dt == F32:
                 assert np.array_equal(gc.logical_dst(p, got), want)
 
@@ -194,9 +226,9 @@ def test_mx_scaled_exact_data_matches_the_oracle(gpu, oracle, tile_shape, shape,
                 assert np.array_equal(gc.logical_dst(p, got), want)
 
 
-def random_case(rng, sizes, K, N, dt, scales=True, dst_dt=F32, active=None):
+def random_case(rng, sizes, K, N, dt, scales=True, dst_dt=F32, active=None, wtag="acb"):
     """Random operands (fp8: random finite bytes with exponents in a band of 2^8;
-    16-bit types: normal), weights [G][N][K].  Returns (problem, S, W, ss, ws) with
+    16-bit types: normal), weights [G][N][K] (`wtag` "abc": stored [G][K][N]).  Returns (problem, S, W, ss, ws) with
     the float64 values.  `active`: groups whose weights are filled (the others
     keep zeros; they have no rows)."""
     G, total = len(sizes), int(sum(sizes))
@@ -226,8 +258,11 @@ def random_case(rng, sizes, K, N, dt, scales=True, dst_dt=F32, active=None):
         ss = rng.uniform(0.5, 2.0, total).astype(np.float32)
         ws = rng.uniform(0.5, 2.0, (G, N)).astype(np.float32)
         quant = {"src_scale": GroupedQuant(F32, ss, 0), "wei_scale": GroupedQuant(F32, ws, 0)}
+    if wtag == "abc":
+        wraw = np.ascontiguousarray(np.swapaxes(wraw, 1, 2))
     p = GroupedProblem(pattern=cabi.GROUPED_2DX3D, sizes=list(sizes), K=K, N=N, src_dt=dt, wei_dt=dt, dst_dt=dst_dt,
-                       src=sraw, wei=wraw, wei_stride=(K * N, 1, K), quant=quant, name=f"random {len(sizes)} groups")
+                       src=sraw, wei=wraw, wei_stride=(K * N, 1, K) if wtag == "acb" else (K * N, N, 1), quant=quant,
+                       name=f"random {len(sizes)} groups")
     return p, S, W, ss, ws
 
 
@@ -267,6 +302,25 @@ def test_random_data_within_the_derived_bound(gpu, tile_shape, dt):
     err = np.abs(got - want)
     assert np.all(err <= tol), f"worst {np.max(err / np.maximum(tol, 1e-30)):.2f} of the bound"
     assert err.max() > 0          # the data is not of the exact kind
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dt", [BF16, F16], ids=["bf16", "f16"])
+@pytest.mark.parametrize("K,N", [(1120, 200), (2048, 768), (80, 12)])
+def test_row_major_weights_random_data_within_the_derived_bound(gpu, dt, K, N):
+    from onednn_amd import grouped
+    rng = np.random.default_rng(23)
+    sizes = [33, 0, 5, 64, 17, 1, 90, 2]
+    p, S, W, ss, ws = random_case(rng, sizes, K, N, dt, wtag="abc")
+    assert impl_of(p) == "hip:mfma_grouped"
+    want, tol = expectation(p, S, W, ss, ws, False)
+    got = gc.logical_dst(p, grouped.run_gpu(p))
+    err = np.abs(got - want)
+    assert np.all(err <= tol), f"worst {np.max(err / np.maximum(tol, 1e-30)):.2f} of the bound"
+    assert err.max() > 0
+    # and the thread-per-element kernel on the same bytes
+    ref = gc.logical_dst(p, _ref_kernel(p))
+    assert np.all(np.abs(ref - want) <= tol)
 
 
 def _ref_kernel(p):
