@@ -186,6 +186,7 @@ struct grouped_k_dev_t {
     long MA, NB, total;
     long dst_g, dst_ld;          // element strides of dst: group, row of A
     int tiles_n;
+    int run;                     // column tiles a workgroup of the LDS kernel takes in turn
 };
 
 typedef unsigned gk_u2 __attribute__((ext_vector_type(2)));
@@ -241,6 +242,8 @@ template <int DT>
 __device__ __forceinline__ void gk_store(const grouped_k_dev_t &P, const gk_f4 (&acc)[4][4], long g, long m_w, long n_w,
         int j, int q) {
     const long col = n_w + 4 * j;
+    // dst is written once and not read again by the launch: non-temporal stores, which do not take lines of the
+    // L2s (a quarter faster on a launch that writes 1.3 GB: 0.325 -> 0.25 ms)
     // bf16: v_cvt_pk_bf16_f32 unless the wavefront holds a NaN or an f32 subnormal, which the software conversion
     // (the reference's: subnormals flush, NaNs are quieted its way) treats differently
     bool hw = false;
@@ -264,19 +267,19 @@ __device__ __forceinline__ void gk_store(const grouped_k_dev_t &P, const gk_f4 (
             const long off = g * P.dst_g + row * P.dst_ld + col;
             const float v0 = acc[r][0][e], v1 = acc[r][1][e], v2 = acc[r][2][e], v3 = acc[r][3][e];
             if (DT == MI355_DT_F32) {
-                *(gk_f4 *)((float *)P.dst + off) = gk_f4 {v0, v1, v2, v3};
+                __builtin_nontemporal_store(gk_f4 {v0, v1, v2, v3}, (gk_f4 *)((float *)P.dst + off));
             } else if (DT == MI355_DT_BF16 && hw) {
                 typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
                 typedef float f32x2_t __attribute__((ext_vector_type(2)));
                 gk_u2 o;
                 o.x = __builtin_bit_cast(unsigned, __builtin_convertvector(f32x2_t {v0, v1}, bf16x2_t));
                 o.y = __builtin_bit_cast(unsigned, __builtin_convertvector(f32x2_t {v2, v3}, bf16x2_t));
-                *(gk_u2 *)((uint16_t *)P.dst + off) = o;
+                __builtin_nontemporal_store(o, (gk_u2 *)((uint16_t *)P.dst + off));
             } else {
                 gk_u2 o;
                 o.x = (cvt_store_bits(DT, v0) & 0xffffu) | (cvt_store_bits(DT, v1) << 16);
                 o.y = (cvt_store_bits(DT, v2) & 0xffffu) | (cvt_store_bits(DT, v3) << 16);
-                *(gk_u2 *)((uint16_t *)P.dst + off) = o;
+                __builtin_nontemporal_store(o, (gk_u2 *)((uint16_t *)P.dst + off));
             }
         }
 }
@@ -971,6 +974,19 @@ __device__ __forceinline__ void grouped_dma16(const void *sbase, unsigned voff, 
 // and what a workgroup waits for is the latency of its only fetch).
 constexpr int GK_BLOCK = 1024 + 64, GK_OPERAND = 8 * GK_BLOCK, GK_STAGE = 2 * GK_OPERAND;
 
+// s_waitcnt vmcnt(n) for the counts the kernel below uses (the instruction takes an immediate)
+__device__ __forceinline__ void gk_wait_vm(int n) {
+    switch (n) {
+        case 0: asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); break;
+        case 4: asm volatile("s_waitcnt vmcnt(4)" ::: "memory"); break;
+        case 8: asm volatile("s_waitcnt vmcnt(8)" ::: "memory"); break;
+        case 16: asm volatile("s_waitcnt vmcnt(16)" ::: "memory"); break;
+        case 20: asm volatile("s_waitcnt vmcnt(20)" ::: "memory"); break;
+        case 24: asm volatile("s_waitcnt vmcnt(24)" ::: "memory"); break;
+        default: asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); break;
+    }
+}
+
 template <int DT, int GK_NST>
 __global__ void __launch_bounds__(256) grouped_k_lds_kernel(const grouped_k_dev_t P) {
     typedef gk_f4 f4;
@@ -979,52 +995,74 @@ __global__ void __launch_bounds__(256) grouped_k_lds_kernel(const grouped_k_dev_
     const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int i = lane & 15, q = lane >> 4;
     const long g = blockIdx.y;
-    const long m_t = (long)(blockIdx.x / P.tiles_n) * 128, n_t = (long)(blockIdx.x % P.tiles_n) * 128;
-    const long m_w = m_t + (wave >> 1) * 64, n_w = n_t + (wave & 1) * 64;
+    // a workgroup takes a run of `run` column tiles of one row of tiles, one after the other
+    const int runs_n = (P.tiles_n + P.run - 1) / P.run;
+    const long m_t = (long)(blockIdx.x / runs_n) * 128;
+    const int tn0 = (int)(blockIdx.x % runs_n) * P.run;
+    const int count = P.tiles_n - tn0 < P.run ? P.tiles_n - tn0 : P.run;
+    const long m_w = m_t + (wave >> 1) * 64;
     long k0 = g > 0 ? (long)P.offsets[g - 1] : 0, k1 = P.offsets[g];
     if (k0 < 0) k0 = 0;
     if (k1 > P.total) k1 = P.total;
+    const long nsteps = k0 < k1 ? (k1 - k0 + 31) / 32 : 0;
 
-    f4 acc[4][4];
-#pragma unroll
-    for (int r = 0; r < 4; ++r)
-#pragma unroll
-        for (int c = 0; c < 4; ++c) acc[r][c] = f4 {0.f, 0.f, 0.f, 0.f};
-
-    if (k0 < k1) {
-        // this lane's part of a block: row lane / 16 of its four, the 16 bytes of columns 8 (lane % 16) ..
-        const long ca = m_t + 8 * i < P.MA ? 8 * i : 0, cb = n_t + 8 * i < P.NB ? 8 * i : 0;
-        const unsigned char *abase = (const unsigned char *)P.a + (k0 * P.MA + m_t) * 2;
+    // this lane's part of a block: row lane / 16 of its four, the 16 bytes of columns 8 (lane % 16) ..
+    const long ca = m_t + 8 * i < P.MA ? 8 * i : 0;
+    const unsigned char *abase = (const unsigned char *)P.a + (k0 * P.MA + m_t) * 2;
+    const long last = k1 - 1 - k0;
+    auto issue = [&](long n_t, long step) {
+        const unsigned cb = n_t + 8 * i < P.NB ? 16 * i : 0;
         const unsigned char *bbase = (const unsigned char *)P.b + (k0 * P.NB + n_t) * 2;
-        const long last = k1 - 1 - k0;
-        auto issue = [&](long step) {
-            const unsigned slot = lds0 + (unsigned)(step % GK_NST) * GK_STAGE;
+        const unsigned slot = lds0 + (unsigned)(step % GK_NST) * GK_STAGE;
 #pragma unroll
-            for (int h = 0; h < 2; ++h) {
-                const int blk = 2 * wave + h;
-                long row = step * 32 + 4 * blk + q;
-                row = row < last ? row : last;
-                grouped_dma16(abase, (unsigned)((row * P.MA + ca) * 2), slot + blk * GK_BLOCK);
-                grouped_dma16(bbase, (unsigned)((row * P.NB + cb) * 2), slot + GK_OPERAND + blk * GK_BLOCK);
-            }
-        };
-        const long nsteps = (k1 - k0 + 31) / 32;
+        for (int h = 0; h < 2; ++h) {
+            const int blk = 2 * wave + h;
+            long row = step * 32 + 4 * blk + q;
+            row = row < last ? row : last;
+            grouped_dma16(abase, (unsigned)((row * P.MA + ca) * 2), slot + blk * GK_BLOCK);
+            grouped_dma16(bbase, (unsigned)(row * P.NB * 2) + cb, slot + GK_OPERAND + blk * GK_BLOCK);
+        }
+    };
+    auto first_stages = [&](long n_t) {
 #pragma unroll
         for (int s = 0; s < GK_NST - 1; ++s)
-            if (s < nsteps) issue(s);
-        const unsigned a_rd = (unsigned)(2 * q * GK_BLOCK + ((wave >> 1) * 64 + 4 * i) * 2);
-        const unsigned b_rd = (unsigned)(GK_OPERAND + 2 * q * GK_BLOCK + ((wave & 1) * 64 + 4 * i) * 2);
+            if (s < nsteps) issue(n_t, s);
+    };
+    const unsigned a_rd = (unsigned)(2 * q * GK_BLOCK + ((wave >> 1) * 64 + 4 * i) * 2);
+    const unsigned b_rd = (unsigned)(GK_OPERAND + 2 * q * GK_BLOCK + ((wave & 1) * 64 + 4 * i) * 2);
+
+    first_stages((long)tn0 * 128);
+    int stores_behind = 0; // store instructions of this wavefront issued after the tile's first stages (-1: some)
+#pragma nounroll
+    for (int tp = 0; tp < count; ++tp) {
+        const long n_t = (long)(tn0 + tp) * 128;
+        f4 acc[4][4];
+#pragma unroll
+        for (int r = 0; r < 4; ++r)
+#pragma unroll
+            for (int c = 0; c < 4; ++c) acc[r][c] = f4 {0.f, 0.f, 0.f, 0.f};
         for (long step = 0; step < nsteps; ++step) {
             // this wavefront's part of the stage has landed; after the barrier everyone's has, and
             // everyone is done reading the stage that the next instructions overwrite
             // (four instructions a stage and wavefront; stages past the group's end are not fetched, so
             // towards the end fewer are behind this one)
             const long behind = nsteps - step - 1;
-            if (behind >= GK_NST - 2) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(4 * (GK_NST - 2)) : "memory");
-            else if (behind == 1) asm volatile("s_waitcnt vmcnt(4)" ::: "memory");
-            else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+            const int stages_behind = behind >= GK_NST - 2 ? GK_NST - 2 : (int)behind;
+            // Memory instructions complete in the order of issue, stores included: when the previous tile
+            // was a whole one, exactly 16 store instructions of this wavefront follow the first stages in the
+            // queue and need not be waited for (otherwise their number depends on the edges: wait for all)
+            if (__builtin_expect(step < GK_NST - 1 && stores_behind != 0, 0)) {
+                if (stores_behind == 16) gk_wait_vm(4 * stages_behind + 16);
+                else gk_wait_vm(0);
+            } else if (behind >= GK_NST - 2) {
+                asm volatile("s_waitcnt vmcnt(%0)" ::"n"(4 * (GK_NST - 2)) : "memory");
+            } else if (behind == 1) {
+                asm volatile("s_waitcnt vmcnt(4)" ::: "memory");
+            } else {
+                asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+            }
             __syncthreads();
-            if (step + GK_NST - 1 < nsteps) issue(step + GK_NST - 1);
+            if (step + GK_NST - 1 < nsteps) issue(n_t, step + GK_NST - 1);
             const unsigned slot = (unsigned)(step % GK_NST) * GK_STAGE;
             gk_u2 ra[8], rb[8];
 #pragma unroll
@@ -1057,9 +1095,18 @@ __global__ void __launch_bounds__(256) grouped_k_lds_kernel(const grouped_k_dev_
                                 __builtin_bit_cast(g8h, b[c]), acc[r][c], 0, 0, 0);
                 }
         }
+        // The next tile's first stages go out before this tile's stores: a compute unit's memory instructions
+        // are served in order, so a fetch issued behind 32 KB of stores waits for all of them (a workgroup a
+        // tile measured fetch + arithmetic + stores end to end, nothing hidden); this way the fetch is done by
+        // the time the stores are, and the store queue stays fed.
+        if (tp + 1 < count && nsteps > 0) {
+            __syncthreads(); // everyone has read this tile's last stage
+            first_stages(n_t + 128);
+        }
+        const long n_w = n_t + (wave & 1) * 64;
+        if (m_w < P.MA && n_w < P.NB) gk_store<DT>(P, acc, g, m_w, n_w, i, q);
+        stores_behind = m_w >= P.MA || n_w >= P.NB ? 0 : (m_w + 64 <= P.MA && n_w + 64 <= P.NB ? 16 : -1);
     }
-    if (m_w >= P.MA || n_w >= P.NB) return;
-    gk_store<DT>(P, acc, g, m_w, n_w, i, q);
 }
 
 // NT: fragments of 16 columns per wavefront.  Leaves the wavefront's MF x NT accumulators in LDS at
@@ -1412,7 +1459,9 @@ int launch_k_tiles(int plan, const grouped_dev_t &G, hipStream_t stream) {
     P.dst_g = d.dst_stride[0];
     P.dst_ld = swap ? d.dst_stride[2] : d.dst_stride[1];
     P.tiles_n = (int)((P.NB + 127) / 128);
-    const dim3 grid((unsigned)(((P.MA + 127) / 128) * P.tiles_n), (unsigned)d.group_count);
+    P.run = 1;
+    const long tiles_m = (P.MA + 127) / 128;
+    dim3 grid((unsigned)(tiles_m * P.tiles_n), (unsigned)d.group_count);
     // bf16 / f16 through LDS and the 16-bit instructions (measured faster at every group length) where columns
     // can be fetched eight at a time and 32-bit offsets reach across a group; otherwise the f32 instruction
     const bool h16 = d.src_dt != MI355_DT_F32;
@@ -1420,6 +1469,13 @@ int launch_k_tiles(int plan, const grouped_dev_t &G, hipStream_t stream) {
     if (tuning(TUNE_GROUPED_IMPL) == TUNE_SHORT) lds_path = false;
     if (lds_path) {
         const bool brief = d.total <= 48 * d.group_count; // (k per group on average)
+        // runs of up to 8 column tiles a workgroup, while some thousands of workgroups remain
+        const long tiles = tiles_m * P.tiles_n * d.group_count;
+        while (P.run < 8 && P.run * 2 <= P.tiles_n && tiles / (P.run * 2) >= 3072) P.run *= 2;
+        // (the tuning switch: "tall" a tile a workgroup, "wide" runs of 8 whatever the size)
+        if (tuning(TUNE_GROUPED_IMPL) == TUNE_TALL) P.run = 1;
+        if (tuning(TUNE_GROUPED_IMPL) == TUNE_WIDE) P.run = P.tiles_n < 8 ? P.tiles_n : 8;
+        grid.x = (unsigned)(tiles_m * ((P.tiles_n + P.run - 1) / P.run));
         auto launch = [&](auto kern, int nst) {
             const int lds = nst * GK_STAGE;
             if (const int st = ensure_dynamic_lds((const void *)kern, lds, "mfma_grouped_k")) return st;

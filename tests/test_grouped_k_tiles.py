@@ -37,13 +37,15 @@ SHAPES = [
     ([5] * 70, 16, 20),
     ([0, 31, 7], 136, 72),                # (columns in eights: the LDS variant's shapes)
     ([40, 1, 100, 32, 65], 264, 136),
+    ([40, 1, 100, 0, 65], 136, 1096),     # nine column tiles: a run of eight and one
 ]
 
 
-@pytest.fixture(params=["short", "auto"])
+@pytest.fixture(params=["short", "auto", "tall", "wide"])
 def variant(request):
     """"short" keeps bf16 / f16 on the f32 instruction too; otherwise shapes with columns in eights go through LDS
-    to the 16-bit instructions."""
+    to the 16-bit instructions, where a workgroup takes a run of column tiles: "tall" forces runs of one, "wide" of
+    eight (otherwise chosen by the number of tiles)."""
     with cabi.tuning("MI355_GROUPED_IMPL", None if request.param == "auto" else request.param):
         yield request.param
 
