@@ -243,6 +243,9 @@ def rate(work, ms, unit):
     return work / (ms * 1e-3) / 1e12
 
 
+GRAPH_REPLAY = True   # decode launches also timed as replays of a HIP graph (main() clears it under a profiler)
+
+
 def run_gpu_workload(lib, name, steps, warmup, M=None, cold_copies=0, wtag="any", sustained_s=0.0):
     """Returns dict with ms_per_step, value, unit, impl.
 
@@ -284,7 +287,7 @@ def run_gpu_workload(lib, name, steps, warmup, M=None, cold_copies=0, wtag="any"
     ms = timer.time_ms(step, steps)
     work, unit, bound, peak = algorithmic(name, p)
     graph = None
-    if stream is not None:
+    if stream is not None and GRAPH_REPLAY:
         # The same `steps` launches (over the same rotation of weight copies) recorded once and replayed: what a
         # serving loop does with a step that is a few microseconds of kernel behind a few microseconds of launch.
         with cabi.Graph(stream) as g:
@@ -518,6 +521,9 @@ def main():
                          "(reported as `sustained`; 0 = skip)")
     ap.add_argument("--no-others", action="store_true", help="skip the informational configs")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--no-graph", action="store_true",
+                    help="skip the HIP-graph replay of the decode launches (skipped by itself under rocprofv3, whose "
+                         "kernel tracing was seen to crash inside hipGraphLaunch)")
     ap.add_argument("--no-ceiling", action="store_true",
                     help="skip the measurement of the ceiling (the MFMA instruction / the weight stream by itself): "
                          "profiler runs, where its kernels would show up next to the workload's")
@@ -538,6 +544,9 @@ def main():
                     help="also launch the plain copy kernel on 256 MiB three times: the known-size "
                          "dispatch that FETCH_SIZE / WRITE_SIZE counter passes are scaled by")
     args = ap.parse_args()
+    global GRAPH_REPLAY
+    if args.no_graph or any(k.startswith("ROCPROF") for k in os.environ):
+        GRAPH_REPLAY = False
     if args.gpus != 1:
         sys.exit("bench.py: this build runs on one GPU (one-GPU boxes only); "
                  "--gpus must be 1. How the path would shard is described in the design notes; it is not built.")
