@@ -214,12 +214,14 @@ def test_execute_2dx2d(gpu, oracle, dtag):
 
 
 @pytest.mark.gpu
-@pytest.mark.parametrize("sdt,wdt", [(cabi.DT_F8_E4M3, cabi.DT_F8_E4M3), (BF16, BF16)], ids=["e4m3", "bf16"])
-def test_execute_2dx3d_on_the_matrix_cores(gpu, oracle, sdt, wdt):
+@pytest.mark.parametrize("sdt,wdt,wtag", [(cabi.DT_F8_E4M3, cabi.DT_F8_E4M3, "acb"), (BF16, BF16, "acb"), (BF16, BF16, "abc"),
+                                          (F16, F16, "abc")], ids=["e4m3", "bf16", "bf16 row-major", "f16 row-major"])
+def test_execute_2dx3d_on_the_matrix_cores(gpu, oracle, sdt, wdt, wtag):
     """The layout of the reference's GPU grouped tests (--wtag=acb, --attr-scales=src:1:f32+wei:5:f32 for fp8) goes
-    to hip:mfma_grouped; exact data, so the oracle's bits are the expectation."""
-    kw = dict(src_scale="row", wei_scale="col") if sdt != BF16 else {}
-    p, _ = gc.case_2dx3d([10, 20, 30, 40], 160, 36, src_dt=sdt, wei_dt=wdt, dst_dt=BF16, wtag="acb", bias=True,
+    to hip:mfma_grouped, and so do row-major (abc) weights of the 16-bit types; exact data, so the oracle's bits are
+    the expectation."""
+    kw = dict(src_scale="row", wei_scale="col") if sdt == cabi.DT_F8_E4M3 else {}
+    p, _ = gc.case_2dx3d([10, 20, 30, 40], 160, 36, src_dt=sdt, wei_dt=wdt, dst_dt=BF16, wtag=wtag, bias=True,
                          post_ops=("relu",), **kw)
     st, want = oracle.run_oracle_grouped(p)
     assert st == cabi.SUCCESS
