@@ -32,7 +32,7 @@ template <int FMT_A, int FMT_B, class G_>
 struct f8_mma_t {
     using G = G_;
     static constexpr int ELEM_BYTES = 1;
-    static constexpr bool HOT = FMT_A == 0 && FMT_B == 0;
+    static constexpr int HOT = FMT_A == 0 && FMT_B == 0 ? 2 : 0;
     static constexpr int EXTRA_DMAS = 0;
     __device__ static __forceinline__ void issue_extra(const f8_ctx_t &, int, int, int, int) {}
     static constexpr int ROWS = 4, COLS = G::WCOLS / 32, A_READS = 2, B_READS = 2;
@@ -100,8 +100,9 @@ struct f8_mma_t {
 };
 
 // HOT: whether the kernel instantiation carries the compile-time specialised
-// chains (e4m3 x e4m3 only: each one multiplies the code of the epilogue)
-template <bool HOT>
+// chains (e4m3 x e4m3 only: each one multiplies the code of the epilogue): 0 none, 1 the gelu_tanh / residual
+// ones, 2 the swish / gate ones as well
+template <int HOT>
 struct f8_conv_t {
     typedef float row_t;
     float ssc_common;
@@ -122,6 +123,11 @@ struct f8_conv_t {
     // unrolled over the wavefront's 4 x 2 accumulator tiles with every choice a
     // template parameter:
     //   acc * src_scale * wei_scale[n]  [+ bias[n]]  [-> gelu_tanh]  [+ bf16 residual]  -> bf16
+    // and, SW != 0 (the plain fp8 kernel only: HOT == 2), the gated feed-forward layer of the Llama family,
+    //   ...  [+ bias[n]]  -> swish  [* bf16 gate (SW == 2)]  -> bf16
+    // where ADD stands for "a staged bf16 operand".  (The SW == 0 instantiations are what the block-scaled
+    // kernel carries, and their code is kept as it was: that kernel's main loop sits at the register limit and
+    // any change to its epilogue moved spills into it, 0.55 -> 1.2 ms.)
     //
     // Global memory sees whole 128-byte rows only.  In the accumulator layout a
     // lane owns 8 bytes of a dst row and a wavefront-wide access touches 32 rows,
@@ -135,7 +141,7 @@ struct f8_conv_t {
     // 16-byte chunks XOR-swizzled by bits 1-3 of the row number (on the
     // global-address side of the DMA and of the final stores), which keeps both
     // access patterns free of bank conflicts.
-    template <bool BIAS, bool GELU, bool ADD, class PT, int C>
+    template <bool BIAS, bool GELU, bool ADD, int SW = 0, class PT, int C>
     __device__ __forceinline__ void hot_store(const PT &P, const epi_uniform_t &H, unsigned ntab, unsigned lds_part,
             const v16f (&acc)[4][C], long b, long m_base, long n_base, int col0) const {
         static_assert(C == 2, "a wavefront's part is 128 rows of 128 bytes");
@@ -198,7 +204,11 @@ struct f8_conv_t {
                     if (with_wei_sc) t *= w[e];
                     if (BIAS) t += bb[e];
                     if (GELU) t = gelu_tanh_fast(t);
-                    if (ADD) t += y[e];
+                    if (SW != 0) t = t * logistic_fast(H.pf0.alpha * t);
+                    if (ADD) {
+                        if (SW == 2) t *= y[e];
+                        else t += y[e];
+                    }
                     special |= __builtin_amdgcn_classf(t, 0x93); // NaN or subnormal: software conversion
                     x[g][e] = t;
                 }
@@ -246,6 +256,21 @@ struct f8_conv_t {
         if (!HOT || ssc_p || H.bias_mode == 2 || H.ds_mode != 0 || H.dzp_mode != 0 || H.dynamic || H.dst_dt != MI355_DT_BF16
                 || H.n_po > 2)
             return false;
+        if constexpr (HOT >= 2) {
+            // swish, alone or followed by the multiplication with a staged bf16 tensor
+            const bool swish = H.n_po >= 1 && H.pf0.kind == MI355_PO_ELTWISE && H.pf0.alg == MI355_ELTWISE_SWISH
+                    && H.pf0.scale == 1.f;
+            const bool gate = H.n_po == 2 && H.pf1.kind == MI355_PO_BINARY && H.pf1.alg == MI355_BINARY_MUL
+                    && H.staged == 1 && H.staged_dt == MI355_DT_BF16;
+            if (swish && (H.n_po == 1 || gate)) {
+                const bool with_bias = H.bias_mode == 1;
+#define MI355_F8_GATED(B, A, S) hot_store<B, false, A, S>(P, H, ntab, lds_part, acc, b, m_base, n_base, col0)
+                if (with_bias) { if (gate) MI355_F8_GATED(true, true, 2); else MI355_F8_GATED(true, false, 1); }
+                else { if (gate) MI355_F8_GATED(false, true, 2); else MI355_F8_GATED(false, false, 1); }
+#undef MI355_F8_GATED
+                return true;
+            }
+        }
         auto is_gelu = [](const po_reg_t &r) {
             return r.kind == MI355_PO_ELTWISE && r.alg == MI355_ELTWISE_GELU_TANH && r.scale == 1.f;
         };

@@ -56,7 +56,7 @@ template <int FMT_A, int FMT_B, class G_>
 struct mxf8_mma_t {
     using G = G_;
     static constexpr int ELEM_BYTES = 1;
-    static constexpr bool HOT = FMT_A == 0 && FMT_B == 0;
+    static constexpr int HOT = FMT_A == 0 && FMT_B == 0 ? 1 : 0;
     static constexpr bool MX = true;
     static constexpr int EXTRA_DMAS = 1;
     static constexpr int SCALE_STAGE = 6 * 256; // two blocks of A, four of B^T

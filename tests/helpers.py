@@ -173,7 +173,7 @@ def gemm_bound(K, abs_sum, sf=4.0):
 
 def finish_f64(p, pre):
     """bias and the post-op chain in float64 for the chains the configurations
-    use (relu, gelu_tanh, linear, binary add / mul, per element or per column).
+    use (relu, gelu_tanh, swish, linear, binary add / mul, per element or per column).
     Returns (value, lip, extra): `lip` = how much an error of the pre-bias sum is
     amplified at most, `extra` = absolute error the float32 evaluation of the
     chain itself may add (a few units in the last place per step)."""
@@ -193,6 +193,12 @@ def finish_f64(p, pre):
             v = 0.5 * x * (1 + np.tanh(0.79788458347320556640625 * x * (1 + 0.044715 * x * x)))
             lip = lip * 1.13                       # sup |gelu'| = 1.129
             extra = extra * 1.13 + 32 * U * np.maximum(np.abs(x), 1.0)
+        elif po.kind == cabi.PO_ELTWISE and po.alg == cabi.ELTWISE["swish"]:
+            x = v
+            with np.errstate(over="ignore"):
+                v = x / (1.0 + np.exp(-np.float64(np.float32(po.alpha)) * x))
+            lip = lip * 1.1                        # sup |swish'| = 1.0998 whatever alpha
+            extra = extra * 1.1 + 32 * U * np.maximum(np.abs(x), 1.0)
         elif po.kind == cabi.PO_ELTWISE and po.alg == cabi.ELTWISE["linear"]:
             v = po.alpha * v + po.beta
             lip, extra = lip * abs(po.alpha), extra * abs(po.alpha) + 2 * U * np.abs(v)

@@ -54,6 +54,25 @@ def test_config4_small(gpu, oracle, impl, wtag):
         assert_gemm_close(p, got, ideal, asum, what=name, hw=fp8_mfma_bound(p) if impl == cabi.IMPL_F8_MFMA else None)
 
 
+@pytest.mark.parametrize("chain", ["swish", "swish*gate", "swish*gate, no bias", "gate alone"])
+def test_config4_gated_feed_forward_chains(gpu, oracle, chain):
+    # the gated feed-forward layer of the Llama family on C4's tensors: swish (SiLU) in place of gelu_tanh and a
+    # multiplication by a bf16 tensor in place of the residual add.  Swish chains run the fp8 tiles' whole-row
+    # epilogue (a multiplication without an activation the rolled one); same bound as the configuration's own chain
+    for dst in (cabi.DT_BF16, cabi.DT_F32):
+        p = configs.config4(M=192, N=320, K=512)
+        p.dst_dt = dst
+        elt, gate = p.post_ops
+        elt.alg, elt.alpha = cabi.ELTWISE["swish"], 1.0
+        gate.alg = cabi.BINARY["mul"]
+        p.post_ops = {"swish": [elt], "gate alone": [gate]}.get(chain, [elt, gate])
+        if "no bias" in chain:
+            p.bias, p.bias_dt = None, cabi.DT_UNDEF
+        got, name = run_gpu(p, cabi.IMPL_F8_MFMA)
+        _, ideal, asum = oracle.run_oracle(p, want_ideal=True)
+        assert_gemm_close(p, got, ideal, asum, what=f"{name} {chain}", hw=fp8_mfma_bound(p))
+
+
 def test_config4_no_postops_f32(gpu, oracle):
     # plain scaled fp8 GEMM into f32: only the summation order differs
     p = configs.config4(M=256, N=256, K=1024)
