@@ -207,6 +207,17 @@ def build_problem(name, M=None, wtag="any"):
         p.dst_dynamic = cabi.DST_DYNAMIC_MX
         p.name = "C4-dynamic-mx-dst"
         return p
+    if name == "c4g":
+        # C4's tensors as the gated feed-forward layer of the Llama family: swish in place of gelu_tanh, the bf16
+        # tensor multiplied in place of the residual add
+        p = configs.config4(wtag=mfma_tag)
+        for po in p.post_ops:
+            if po.kind == cabi.PO_ELTWISE:
+                po.alg, po.alpha = cabi.ELTWISE["swish"], 1.0
+            if po.kind == cabi.PO_BINARY:
+                po.alg = cabi.BINARY["mul"]
+        p.name = "C4-swish-gate"
+        return p
     if name == "c5":
         return configs.config5(wtag=mfma_tag)
     if name == "h1":
@@ -226,7 +237,7 @@ def algorithmic(name, p):
         return configs.config2_bytes(p.M, p.N, p.K), "GB/s", "hbm", PEAK_HBM_GBS
     if name == "c3":
         return ops, "TOPS", "mfma", PEAK_I8_TOPS
-    if name in ("c4", "c4mx", "m1"):
+    if name in ("c4", "c4mx", "c4g", "m1"):
         return ops, "TFLOP/s", "mfma", PEAK_F8_TFLOPS
     if name == "c5":
         return ops, "TFLOP/s", "mfma", PEAK_F4_TFLOPS
@@ -784,7 +795,7 @@ def main():
         # layout change then runs inside every launch
         plan = [("c2", 1, "any"), ("c2", 8, "any"), ("c2", 32, "any"), ("c2", 1, "ab"), ("c2", 8, "ab"), ("c2", 32, "ab"),
                 ("c3", None, "any"), ("c3", None, "ab"),
-                ("c4", None, "any"), ("c4mx", None, "any"), ("c5", None, "any"), ("c1", None, "any"),
+                ("c4", None, "any"), ("c4mx", None, "any"), ("c4g", None, "any"), ("c5", None, "any"), ("c1", None, "any"),
                 ("m1", None, "any"), ("h1", None, "any"), ("h2", None, "any"), ("p2", 512, "any"), ("p2", 2048, "any")]
         for nm, m, wt in plan:
             if nm == main_name and wt == args.wtag and (nm != "c2" or m == args.decode_m):
