@@ -333,7 +333,10 @@ const char *mi355_last_error(void); /* thread-local text of the last failure */
  *                      wide: 256 x 256; narrow: 256 x 128; small: 32 x 32 without LDS)
  *   MI355_F8_TILES     wide | narrow          hip:mfma_f8 on 256 x 256 / 256 x 128 tiles
  *   MI355_H16_TILES    wide                   hip:mfma_h16 on 256 x 256 tiles
- *   MI355_GROUPED_IMPL ref | short | tall | wide   grouped matmul kernel
+ *   MI355_GROUPED_IMPL ref | short | tall | wide   grouped matmul kernel (ref: a thread per dst element;
+ *                      variable M: 16 x 32, 48 x 64 or 64 x 256 tiles; variable K: short = the f32
+ *                      instruction for 16-bit types too, tall / wide = a workgroup takes one / eight
+ *                      column tiles in turn)
  *   MI355_GEMM_ORDER   0..63                  tile order of the large GEMMs
  * value NULL, "" or "auto" restores the library's own choice.  A switch can
  * change a problem's scratch need (the 32 x 32 int8 tiles need none, the LDS
