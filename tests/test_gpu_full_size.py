@@ -73,15 +73,21 @@ def test_config3_full_size_sampled_rows_are_bit_exact(gpu, oracle):
     assert np.mean((g > 0) & (g < 127)) > 0.05
 
 
+@pytest.mark.parametrize("chain", ["gelu_tanh + residual", "swish x gate"])
 @pytest.mark.parametrize("dst", ["bf16", "f32"])
-def test_config4_full_size_sampled_rows(gpu, oracle, dst):
+def test_config4_full_size_sampled_rows(gpu, oracle, dst, chain):
     # against the oracle's float64 K-sums with bias, gelu_tanh and the residual in float64 on top:
     # bound = 4 standard deviations of the float32 summation error model (tests/helpers.py gemm_bound)
     # plus the matrix cores' fp8 alignment loss (fp8_mfma_bound), together about 0.1 on pre-activations
     # of standard deviation 90, carried through the chain; with the f32 dst nothing else is inside it,
     # the bf16 dst adds half a unit in its last place
+    # (the second chain: the gated feed-forward layer on the same tensors, the other whole-row epilogue of the kernel)
     p = configs.config4(wtag="ba")
     p.dst_dt = cabi.DT_NAMES[dst]
+    if chain == "swish x gate":
+        elt, gate = p.post_ops
+        elt.alg, elt.alpha = cabi.ELTWISE["swish"], 1.0
+        gate.alg = cabi.BINARY["mul"]
     got, name = run_gpu(p)
     assert name.startswith("hip:mfma_f8")
     rows = sample_rows(p.M, 1, 4)
