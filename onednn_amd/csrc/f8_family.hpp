@@ -125,6 +125,7 @@ struct f8_conv_t {
     //   acc * src_scale * wei_scale[n]  [+ bias[n]]  [-> gelu_tanh]  [+ bf16 residual]  -> bf16
     // and, SW != 0 (the plain fp8 kernel only: HOT == 2), the gated feed-forward layer of the Llama family,
     //   ...  [+ bias[n]]  -> swish  [* bf16 gate (SW == 2)]  -> bf16
+    //   ...  [+ bias[n]]  [-> gelu_tanh]  * bf16 gate (SW == 3: GeGLU, or a plain gate)  -> bf16
     // where ADD stands for "a staged bf16 operand".  (The SW == 0 instantiations are what the block-scaled
     // kernel carries, and their code is kept as it was: that kernel's main loop sits at the register limit and
     // any change to its epilogue moved spills into it, 0.55 -> 1.2 ms.)
@@ -204,9 +205,9 @@ struct f8_conv_t {
                     if (with_wei_sc) t *= w[e];
                     if (BIAS) t += bb[e];
                     if (GELU) t = gelu_tanh_fast(t);
-                    if (SW != 0) t = t * logistic_fast(H.pf0.alpha * t);
+                    if (SW == 1 || SW == 2) t = t * logistic_fast(H.pf0.alpha * t);
                     if (ADD) {
-                        if (SW == 2) t *= y[e];
+                        if (SW >= 2) t *= y[e];
                         else t += y[e];
                     }
                     special |= __builtin_amdgcn_classf(t, 0x93); // NaN or subnormal: software conversion
@@ -262,6 +263,19 @@ struct f8_conv_t {
                     && H.pf0.scale == 1.f;
             const bool gate = H.n_po == 2 && H.pf1.kind == MI355_PO_BINARY && H.pf1.alg == MI355_BINARY_MUL
                     && H.staged == 1 && H.staged_dt == MI355_DT_BF16;
+            // gelu_tanh, or nothing, followed by that multiplication
+            const bool gelu_first = H.n_po == 2 && H.pf0.kind == MI355_PO_ELTWISE && H.pf0.alg == MI355_ELTWISE_GELU_TANH
+                    && H.pf0.scale == 1.f;
+            const bool gate_alone = H.n_po == 1 && H.pf0.kind == MI355_PO_BINARY && H.pf0.alg == MI355_BINARY_MUL
+                    && H.staged == 0 && H.staged_dt == MI355_DT_BF16;
+            if ((gelu_first && gate) || gate_alone) {
+                const bool with_bias = H.bias_mode == 1;
+#define MI355_F8_GATED(B, G) hot_store<B, G, true, 3>(P, H, ntab, lds_part, acc, b, m_base, n_base, col0)
+                if (with_bias) { if (gelu_first) MI355_F8_GATED(true, true); else MI355_F8_GATED(true, false); }
+                else { if (gelu_first) MI355_F8_GATED(false, true); else MI355_F8_GATED(false, false); }
+#undef MI355_F8_GATED
+                return true;
+            }
             if (swish && (H.n_po == 1 || gate)) {
                 const bool with_bias = H.bias_mode == 1;
 #define MI355_F8_GATED(B, A, S) hot_store<B, false, A, S>(P, H, ntab, lds_part, acc, b, m_base, n_base, col0)

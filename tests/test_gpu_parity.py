@@ -54,17 +54,19 @@ def test_config4_small(gpu, oracle, impl, wtag):
         assert_gemm_close(p, got, ideal, asum, what=name, hw=fp8_mfma_bound(p) if impl == cabi.IMPL_F8_MFMA else None)
 
 
-@pytest.mark.parametrize("chain", ["swish", "swish*gate", "swish*gate, no bias", "gate alone"])
+@pytest.mark.parametrize("chain", ["swish", "swish*gate", "swish*gate, no bias", "gate alone", "gelu_tanh*gate",
+                                   "gelu_tanh*gate, no bias"])
 def test_config4_gated_feed_forward_chains(gpu, oracle, chain):
     # the gated feed-forward layer of the Llama family on C4's tensors: swish (SiLU) in place of gelu_tanh and a
-    # multiplication by a bf16 tensor in place of the residual add.  Swish chains run the fp8 tiles' whole-row
-    # epilogue (a multiplication without an activation the rolled one); same bound as the configuration's own chain
+    # multiplication by a bf16 tensor in place of the residual add (and gelu_tanh with that multiplication: GeGLU).
+    # All of them run the fp8 tiles' whole-row epilogue; same bound as the configuration's own chain
     for dst, M, N, alpha in ((cabi.DT_BF16, 192, 320, 1.0), (cabi.DT_F32, 192, 320, 1.0), (cabi.DT_BF16, 300, 512, 1.702),
                              (cabi.DT_BF16, 256, 256, 0.5)):
         p = configs.config4(M=M, N=N, K=512)
         p.dst_dt = dst
         elt, gate = p.post_ops
-        elt.alg, elt.alpha = cabi.ELTWISE["swish"], alpha
+        if "gelu" not in chain:
+            elt.alg, elt.alpha = cabi.ELTWISE["swish"], alpha
         gate.alg = cabi.BINARY["mul"]
         p.post_ops = {"swish": [elt], "gate alone": [gate]}.get(chain, [elt, gate])
         if "no bias" in chain:
